@@ -1,0 +1,773 @@
+"""Routines: the device-agnostic layer of ChainerX restated over the C ABI.
+
+Each function mirrors one routine of ``CX/routines/*.cc``: the same dtype promotion, broadcasting,
+output allocation and -- most importantly -- the same decomposition into kernel calls, one
+``hipcx_*`` call per ``CallKernel<...>`` of the reference.  Nothing is fused here that the
+reference does not fuse; the fused entry points live in ``chainer_amd.fused`` and are opt-in.
+"""
+import builtins as _py
+import ctypes
+
+import numpy
+
+from chainer_amd import _lib
+from chainer_amd._array import (ndarray, array, current_stream, alloc_bytes, _normalize_axis, _as_shape, _prod,
+                                contiguous_strides)
+
+# ---------------------------------------------------------------------------------------------
+# dtype rules (CX/dtype.cc:12-60, CX/routines/type_util.cc:11-46)
+# ---------------------------------------------------------------------------------------------
+_KIND = {'b': 0, 'i': 1, 'u': 2, 'f': 3}
+_CATEGORY = {0: 0, 1: 1, 2: 1, 3: 2}  # bool < int/uint < float
+
+
+def _kind(dtype):
+    return _KIND[numpy.dtype(dtype).kind]
+
+
+def promote_types(dt1, dt2):
+    dt1, dt2 = numpy.dtype(dt1), numpy.dtype(dt2)
+    k1, k2 = _kind(dt1), _kind(dt2)
+    if k1 == 0:
+        return dt2
+    if k2 == 0:
+        return dt1
+    if k1 == k2:
+        return dt1 if dt1.itemsize >= dt2.itemsize else dt2
+    if k1 == 3:
+        return dt1
+    if k2 == 3:
+        return dt2
+    if k1 == 2:
+        dt1, dt2 = dt2, dt1
+    if dt1.itemsize > dt2.itemsize:
+        return dt1
+    return numpy.dtype('int16')  # signed one level wider than uint8
+
+
+def _scalar_default_dtype(value):
+    if isinstance(value, (bool, numpy.bool_)):
+        return numpy.dtype('bool')
+    if isinstance(value, (int, numpy.integer)):
+        return numpy.dtype('int32')
+    return numpy.dtype('float32')
+
+
+def result_type(*args):
+    """ResultType over arrays and Python scalars: scalars only matter if of a higher category."""
+    arr_dt = None
+    sc_dt = None
+    for a in args:
+        if isinstance(a, ndarray):
+            arr_dt = a.dtype if arr_dt is None else promote_types(arr_dt, a.dtype)
+        else:
+            d = _scalar_default_dtype(a)
+            sc_dt = d if sc_dt is None else promote_types(sc_dt, d)
+    if arr_dt is not None:
+        if sc_dt is not None and _CATEGORY[_kind(sc_dt)] > _CATEGORY[_kind(arr_dt)]:
+            return sc_dt
+        return arr_dt
+    return sc_dt
+
+
+def _math_result_dtype(dtype):
+    return numpy.dtype(dtype) if _kind(dtype) == 3 else numpy.dtype('float32')
+
+
+def _is_scalar(x):
+    return isinstance(x, (bool, int, float, numpy.bool_, numpy.integer, numpy.floating))
+
+
+# ---------------------------------------------------------------------------------------------
+# creation
+# ---------------------------------------------------------------------------------------------
+def empty(shape, dtype='float32'):
+    return ndarray.empty(shape, dtype)
+
+
+def empty_like(a):
+    return ndarray.empty(a.shape, a.dtype)
+
+
+def full(shape, value, dtype=None):
+    if dtype is None:
+        dtype = _scalar_default_dtype(value)
+    out = ndarray.empty(shape, dtype)
+    out.fill(value)
+    return out
+
+
+def zeros(shape, dtype='float32'):
+    return full(shape, 0, dtype)
+
+
+def ones(shape, dtype='float32'):
+    return full(shape, 1, dtype)
+
+
+def zeros_like(a):
+    return zeros(a.shape, a.dtype)
+
+
+def arange(start, stop=None, step=1, dtype=None):
+    """Arange (CX/routines/creation.cc): size = ceil((stop-start)/step), then ArangeKernel."""
+    if stop is None:
+        start, stop = 0, start
+    if dtype is None:
+        dtype = result_type(start, stop, step)
+        if _kind(dtype) == 0:
+            dtype = numpy.dtype('int32')
+    if step == 0:
+        raise _lib.ChainerxError('Cannot create an arange array with 0 step size.')
+    size = _py.max(0, int(numpy.ceil((stop - start) / step)))
+    out = ndarray.empty((size,), dtype)
+    _lib.call('hipcx_arange', _lib.make_scalar(start), _lib.make_scalar(step), out.desc(), current_stream())
+    return out
+
+
+def copy(a):
+    return a.copy()
+
+
+def ascontiguousarray(a):
+    return a.as_contiguous()
+
+
+def astype(a, dtype, copy=True):
+    return a.astype(dtype, copy)
+
+
+# ---------------------------------------------------------------------------------------------
+# manipulation (views + Copy kernels)
+# ---------------------------------------------------------------------------------------------
+def reshape(a, shape):
+    return a.reshape(shape)
+
+
+def transpose(a, axes=None):
+    return a.transpose(axes)
+
+
+def broadcast_to(a, shape):
+    return a.broadcast_to(shape)
+
+
+def squeeze(a, axis=None):
+    return a.squeeze(axis)
+
+
+def split(a, indices_or_sections, axis=0):
+    """Split into views (CX/routines/manipulation.cc Split)."""
+    axis = _normalize_axis(axis, a.ndim)
+    dim = a.shape[axis]
+    if isinstance(indices_or_sections, (int, numpy.integer)):
+        n = int(indices_or_sections)
+        if n <= 0 or dim % n != 0:
+            raise _lib.DimensionError('array split does not result in an equal division')
+        step = dim // n
+        bounds = [(i * step, (i + 1) * step) for i in range(n)]
+    else:
+        idx = [_py.min(_py.max(int(i), 0), dim) for i in indices_or_sections]
+        starts = [0] + idx
+        stops = idx + [dim]
+        bounds = [(s, _py.max(s, e)) for s, e in zip(starts, stops)]
+    out = []
+    for s, e in bounds:
+        key = [slice(None)] * a.ndim
+        key[axis] = slice(s, e)
+        out.append(a[tuple(key)])
+    return out
+
+
+def concatenate(arrays, axis=0):
+    """Concatenate = Empty + one CopyKernel per input (CX/routines/manipulation.cc:415-460)."""
+    arrays = list(arrays)
+    if not arrays:
+        raise _lib.DimensionError('Need at least one array to concatenate')
+    axis = _normalize_axis(axis, arrays[0].ndim)
+    dtype = arrays[0].dtype
+    shape = list(arrays[0].shape)
+    total = 0
+    for a in arrays:
+        if a.ndim != len(shape):
+            raise _lib.DimensionError('all the input arrays must have same number of dimensions')
+        for i in range(a.ndim):
+            if i != axis and a.shape[i] != shape[i]:
+                raise _lib.DimensionError('all the input array dimensions except for the concatenation axis must match exactly')
+        total += a.shape[axis]
+        dtype = promote_types(dtype, a.dtype)
+    shape[axis] = total
+    out = ndarray.empty(shape, dtype)
+    pos = 0
+    for a in arrays:
+        key = [slice(None)] * out.ndim
+        key[axis] = slice(pos, pos + a.shape[axis])
+        _lib.call('hipcx_copy', a.desc(), out[tuple(key)].desc(), current_stream())
+        pos += a.shape[axis]
+    return out
+
+
+# ---------------------------------------------------------------------------------------------
+# elementwise
+# ---------------------------------------------------------------------------------------------
+def _broadcast_shape(s1, s2):
+    n = _py.max(len(s1), len(s2))
+    a = (1,) * (n - len(s1)) + tuple(s1)
+    b = (1,) * (n - len(s2)) + tuple(s2)
+    out = []
+    for x, y in zip(a, b):
+        if x == y or y == 1:
+            out.append(x)
+        elif x == 1:
+            out.append(y)
+        else:
+            raise _lib.DimensionError('operands could not be broadcast together with shapes %r %r' % (tuple(s1), tuple(s2)))
+    return tuple(out)
+
+
+def _binary(kernel, x1, x2, dtype, out=None):
+    """BroadcastBinary (CX/routines/routines_util.h:53-72): operands arrive equal-shaped, cast to out's dtype."""
+    shape = _broadcast_shape(x1.shape, x2.shape)
+    a = x1 if x1.shape == shape else x1.broadcast_to(shape)
+    b = x2 if x2.shape == shape else x2.broadcast_to(shape)
+    if out is None:
+        out = ndarray.empty(shape, dtype)
+    elif out.shape != shape:
+        raise _lib.DimensionError('in-place operand shape %r does not match %r' % (out.shape, shape))
+    _lib.call(kernel, a.astype(out.dtype, False).desc(), b.astype(out.dtype, False).desc(), out.desc(), current_stream())
+    return out
+
+
+def _binary_as(kernel, x1, scalar, dtype, out=None):
+    if out is None:
+        out = ndarray.empty(x1.shape, dtype)
+    _lib.call(kernel, x1.astype(out.dtype, False).desc(), _lib.make_scalar(scalar), out.desc(), current_stream())
+    return out
+
+
+def add(x1, x2, out=None):
+    if _is_scalar(x2):
+        return _binary_as('hipcx_add_as', x1, x2, result_type(x1, x2), out)
+    if _is_scalar(x1):
+        return _binary_as('hipcx_add_as', x2, x1, result_type(x1, x2), out)
+    return _binary('hipcx_add', x1, x2, result_type(x1, x2), out)
+
+
+def negative(x):
+    """Negative = Multiply(x, Scalar{-1}) (CX/routines/arithmetic.cc)."""
+    if x.dtype == numpy.dtype('bool'):
+        raise _lib.DtypeError('Cannot negate a boolean array.')
+    return _binary_as('hipcx_multiply_as', x, -1, x.dtype)
+
+
+def subtract(x1, x2, out=None):
+    dt = result_type(x1, x2)
+    if _kind(dt) == 0:
+        raise _lib.DtypeError('Boolean arguments are not supported in subtract.')
+    if _is_scalar(x2):
+        return _binary_as('hipcx_subtract_as', x1, x2, dt, out)
+    if _is_scalar(x1):
+        # Subtract(Scalar, Array) = Add(-Array, Scalar) (CX/routines/arithmetic.cc)
+        return add(negative(x2), x1)
+    return _binary('hipcx_subtract', x1, x2, dt, out)
+
+
+def multiply(x1, x2, out=None):
+    if _is_scalar(x2):
+        return _binary_as('hipcx_multiply_as', x1, x2, result_type(x1, x2), out)
+    if _is_scalar(x1):
+        return _binary_as('hipcx_multiply_as', x2, x1, result_type(x1, x2), out)
+    return _binary('hipcx_multiply', x1, x2, result_type(x1, x2), out)
+
+
+def _true_divide_dtype(*args):
+    dt = result_type(*args)
+    return dt if _kind(dt) == 3 else numpy.dtype('float32')
+
+
+def divide(x1, x2, out=None):
+    """TrueDivide: integer operands are computed in float32 (CX/routines/arithmetic.cc Divide)."""
+    dt = _true_divide_dtype(x1, x2)
+    if _is_scalar(x2):
+        return _binary_as('hipcx_divide_as', x1, x2, dt, out)
+    if _is_scalar(x1):
+        if out is None:
+            out = ndarray.empty(x2.shape, dt)
+        _lib.call('hipcx_divide_sa', _lib.make_scalar(x1), x2.astype(out.dtype, False).desc(), out.desc(), current_stream())
+        return out
+    return _binary('hipcx_divide', x1, x2, dt, out)
+
+
+def reciprocal(x):
+    """Reciprocal(x) = Scalar{1} / x (CX/routines/arithmetic.cc)."""
+    return divide(1, x)
+
+
+def _unary_math(kernel, x):
+    dt = _math_result_dtype(x.dtype)
+    xc = x.astype(dt, False)
+    out = ndarray.empty(x.shape, dt)
+    _lib.call(kernel, xc.desc(), out.desc(), current_stream())
+    return out
+
+
+def exp(x):
+    return _unary_math('hipcx_exp', x)
+
+
+def log(x):
+    return _unary_math('hipcx_log', x)
+
+
+def tanh(x):
+    return _unary_math('hipcx_tanh', x)
+
+
+def sqrt(x):
+    return _unary_math('hipcx_sqrt', x)
+
+
+def if_less_else(x1, x2, pos, neg):
+    """x1 < x2 ? pos : neg with scalar x2/pos (CX/routines/misc.cc:34-58)."""
+    dt = result_type(pos, neg)
+    out = ndarray.empty(x1.shape, dt)
+    _lib.call('hipcx_if_less_else_assa', x1.astype(dt, False).desc(), _lib.make_scalar(x2), _lib.make_scalar(pos),
+              neg.astype(dt, False).desc(), out.desc(), current_stream())
+    return out
+
+
+def if_greater_else(x1, x2, pos, neg):
+    dt = result_type(pos, neg)
+    out = ndarray.empty(x1.shape, dt)
+    _lib.call('hipcx_if_greater_else_assa', x1.astype(dt, False).desc(), _lib.make_scalar(x2), _lib.make_scalar(pos),
+              neg.astype(dt, False).desc(), out.desc(), current_stream())
+    return out
+
+
+def maximum(x1, x2):
+    """Maximum(array, scalar) = IfLessElse(x1, x2, x2, x1) (CX/routines/misc.cc:210-216)."""
+    if _is_scalar(x1):
+        x1, x2 = x2, x1
+    if _is_scalar(x2):
+        return if_less_else(x1, x2, x2, x1)
+    dt = result_type(x1, x2)
+    shape = _broadcast_shape(x1.shape, x2.shape)
+    a = x1.broadcast_to(shape).astype(dt, False)
+    b = x2.broadcast_to(shape).astype(dt, False)
+    out = ndarray.empty(shape, dt)
+    # MaximumImpl: x1 > x2 ? x1 : x2 (CX/routines/misc.cc)
+    _lib.call('hipcx_if_greater_else_aaaa', a.desc(), b.desc(), a.desc(), b.desc(), out.desc(), current_stream())
+    return out
+
+
+def minimum(x1, x2):
+    if _is_scalar(x1):
+        x1, x2 = x2, x1
+    if _is_scalar(x2):
+        return if_greater_else(x1, x2, x2, x1)
+    raise _lib.ChainerxNotImplementedError('minimum(array, array) is not on the supported path')
+
+
+def relu(x):
+    """Relu(x) = Maximum(0, x) in the math dtype of x (CX/routines/activation.cc:80-84)."""
+    return maximum(x.astype(_math_result_dtype(x.dtype), False), 0)
+
+
+def sigmoid(x):
+    """Sigmoid(x) = Reciprocal(1 + Exp(-x)): four kernels (CX/routines/activation.cc:74-78)."""
+    xc = x.astype(_math_result_dtype(x.dtype), False)
+    return reciprocal(add(exp(negative(xc)), 1))
+
+
+def _compare(kernel, x1, x2):
+    if _is_scalar(x2):
+        x2 = full((), x2, x1.dtype)
+    if (_kind(x1.dtype) == 0) != (_kind(x2.dtype) == 0):
+        raise _lib.DtypeError('Comparison of bool and non-bool dtypes is not supported.')
+    dt = promote_types(x1.dtype, x2.dtype)
+    shape = _broadcast_shape(x1.shape, x2.shape)
+    a = x1.broadcast_to(shape).astype(dt, False)
+    b = x2.broadcast_to(shape).astype(dt, False)
+    out = ndarray.empty(shape, 'bool')
+    _lib.call(kernel, a.desc(), b.desc(), out.desc(), current_stream())
+    return out
+
+
+def equal(x1, x2):
+    return _compare('hipcx_equal', x1, x2)
+
+
+def not_equal(x1, x2):
+    return _compare('hipcx_not_equal', x1, x2)
+
+
+def greater(x1, x2):
+    return _compare('hipcx_greater', x1, x2)
+
+
+def greater_equal(x1, x2):
+    return _compare('hipcx_greater_equal', x1, x2)
+
+
+# ---------------------------------------------------------------------------------------------
+# reductions
+# ---------------------------------------------------------------------------------------------
+def _sorted_axes(axis, ndim):
+    if axis is None:
+        return tuple(range(ndim))
+    if isinstance(axis, (int, numpy.integer)):
+        axis = (axis,)
+    ax = sorted(_normalize_axis(a, ndim) for a in axis)
+    if len(set(ax)) != len(ax):
+        raise _lib.DimensionError('Duplicate axis values.')
+    return tuple(ax)
+
+
+def _reduced_out(a, axes, keepdims, dtype):
+    """EmptyReduced (CX/routines/creation.cc:56-75): kept axes get stride 0."""
+    if keepdims:
+        out_shape = [1 if i in axes else d for i, d in enumerate(a.shape)]
+        inner = [d for i, d in enumerate(a.shape) if i not in axes]
+        inner_strides = list(contiguous_strides(inner, numpy.dtype(dtype).itemsize))
+        strides = []
+        for i in range(a.ndim):
+            strides.append(0 if i in axes else inner_strides.pop(0))
+        nbytes = _prod(inner) * numpy.dtype(dtype).itemsize
+        return ndarray(alloc_bytes(nbytes), 0, out_shape, strides, dtype)
+    return ndarray.empty([d for i, d in enumerate(a.shape) if i not in axes], dtype)
+
+
+def _reduce(kernel, a, axes, out):
+    n = len(axes)
+    ax = (ctypes.c_int8 * _py.max(n, 1))(*axes)
+    ws_bytes = _lib.load().hipcx_reduce_workspace_size(a.desc(), ax, n, out.desc())
+    ws = alloc_bytes(ws_bytes) if ws_bytes else None
+    _lib.call(kernel, a.desc(), ax, n, out.desc(), ctypes.c_void_p(ws.data_ptr() if ws is not None else 0), ws_bytes, current_stream())
+    return out
+
+
+def sum(a, axis=None, keepdims=False):
+    """Sum (CX/routines/reduction.cc:28-76): bool/int inputs accumulate and return int64."""
+    axes = _sorted_axes(axis, a.ndim)
+    k = _kind(a.dtype)
+    out_dtype = numpy.dtype('int64') if k in (0, 1, 2) else a.dtype
+    out = _reduced_out(a, axes, keepdims, out_dtype)
+    return _reduce('hipcx_sum', a, axes, out)
+
+
+def amax(a, axis=None, keepdims=False):
+    """AMax (CX/routines/statistics.cc:21-65)."""
+    axes = _sorted_axes(axis, a.ndim)
+    for i in axes:
+        if a.shape[i] == 0:
+            raise _lib.DimensionError('cannot compute the maximum along zero-sized axis')
+    out = _reduced_out(a, axes, keepdims, a.dtype)
+    return _reduce('hipcx_amax', a, axes, out)
+
+
+max = amax
+
+
+def argmax(a, axis=None):
+    """ArgMax (CX/routines/sorting.cc:21-52): int64 result, no keepdims."""
+    axes = _sorted_axes(axis, a.ndim)
+    for i in axes:
+        if a.shape[i] == 0:
+            raise _lib.DimensionError('cannot compute ArgMax for an empty array')
+    out = ndarray.empty([d for i, d in enumerate(a.shape) if i not in axes], 'int64')
+    return _reduce('hipcx_argmax', a, axes, out)
+
+
+def mean(a, axis=None, keepdims=False):
+    """Mean = Sum then DivideAS by the item count (CX/routines/statistics.cc:95-154)."""
+    axes = _sorted_axes(axis, a.ndim)
+    dt = a.dtype if _kind(a.dtype) == 3 else numpy.dtype('float32')
+    out = _reduced_out(a, axes, keepdims, dt)
+    _reduce('hipcx_sum', a, axes, out)
+    n = _prod([a.shape[i] for i in axes])
+    _lib.call('hipcx_divide_as', out.desc(), _lib.make_scalar(int(n)), out.desc(), current_stream())
+    return out
+
+
+def logsumexp(x, axis=None, keepdims=False):
+    """LogSumExp (CX/routines/reduction.cc:78-86): AMax, Subtract, Exp, Sum, Log, Add."""
+    xc = x.astype(_math_result_dtype(x.dtype), False)
+    axes = _sorted_axes(axis, x.ndim)
+    xmax = amax(xc, axes, True)
+    logs = log(sum(exp(subtract(xc, xmax)), axes, keepdims))
+    return add(xmax if keepdims else xmax.squeeze(axes), logs)
+
+
+def log_softmax(x, axis=None):
+    """LogSoftmax = x - LogSumExp(x, axis or 1, keepdims) (CX/routines/reduction.cc:88-92): seven kernels."""
+    xc = x.astype(_math_result_dtype(x.dtype), False)
+    return subtract(xc, logsumexp(xc, 1 if axis is None else axis, True))
+
+
+def softmax(x, axis=None):
+    """Softmax (CX/routines/reduction.cc:68-76)."""
+    xc = x.astype(_math_result_dtype(x.dtype), False)
+    axes = _sorted_axes(1 if axis is None else axis, x.ndim)
+    xmax = amax(xc, axes, True)
+    exps = exp(subtract(xc, xmax))
+    sums = sum(exps, axes, True)
+    return multiply(exps, reciprocal(sums))
+
+
+# ---------------------------------------------------------------------------------------------
+# linear algebra / connection
+# ---------------------------------------------------------------------------------------------
+def _workspace(nbytes):
+    if not nbytes:
+        return None, ctypes.c_void_p(0)
+    ws = alloc_bytes(nbytes)
+    return ws, ctypes.c_void_p(ws.data_ptr())
+
+
+def dot(a, b, out_dtype=None):
+    """Dot for 2-D operands (CX/routines/linalg.cc:27-100): k == 0 gives zeros without a kernel."""
+    if a.ndim != 2 or b.ndim != 2:
+        raise _lib.DimensionError('ChainerX dot supports only 2-dimensional arrays.')
+    if a.shape[1] != b.shape[0]:
+        raise _lib.DimensionError('Axis dimension mismatch')
+    dt = numpy.dtype(out_dtype) if out_dtype is not None else result_type(a, b)
+    m, k, n = a.shape[0], a.shape[1], b.shape[1]
+    if k == 0:
+        return zeros((m, n), dt)
+    out = ndarray.empty((m, n), dt)
+    _dot_into(a.astype(dt, False), b.astype(dt, False), out)
+    return out
+
+
+def _dot_into(a, b, out):
+    nbytes = _lib.load().hipcx_dot_workspace_size(a.desc(), b.desc(), out.desc())
+    ws, wsp = _workspace(nbytes)
+    _lib.call('hipcx_dot', a.desc(), b.desc(), out.desc(), wsp, nbytes, current_stream())
+
+
+def linear(x, w, b=None, n_batch_axes=1):
+    """Linear (CX/routines/connection.cc:322-394): DotKernel(x, w.T view) then AddKernel with a stride-0 bias."""
+    if w.ndim != 2:
+        raise _lib.DimensionError('w.ndim should be 2')
+    if b is not None and b.ndim != 1:
+        raise _lib.DimensionError('b.ndim should be 1')
+    n_batch_axes = _normalize_axis(n_batch_axes, x.ndim) if x.ndim > 0 else 0
+    dt = result_type(x, w, b) if b is not None else result_type(x, w)
+    out_dim = _prod(x.shape[:n_batch_axes])
+    m_dim, n_dim = w.shape
+    out_shape = tuple(x.shape[:n_batch_axes]) + (m_dim,)
+    if m_dim == 0 or n_dim == 0:
+        if b is not None:
+            return b.astype(dt, False).broadcast_to(out_shape)
+        return zeros(out_shape, dt)
+    x_matrix = x.reshape(out_dim, n_dim)
+    out_matrix = ndarray.empty((out_dim, m_dim), dt)
+    _dot_into(x_matrix.astype(dt, False), w.transpose().astype(dt, False), out_matrix)
+    if b is not None:
+        b_matrix = b.broadcast_to((out_dim, m_dim))
+        _lib.call('hipcx_add', out_matrix.desc(), b_matrix.astype(dt, False).desc(), out_matrix.desc(), current_stream())
+    return out_matrix.reshape(out_shape)
+
+
+def _pair(v, n=2):
+    if isinstance(v, (int, numpy.integer)):
+        return (int(v),) * n
+    v = tuple(int(i) for i in v)
+    if len(v) != n:
+        raise _lib.DimensionError('expected %d values, got %r' % (n, v))
+    return v
+
+
+def _i64(values):
+    return (ctypes.c_int64 * len(values))(*values)
+
+
+def conv_out_dim(in_dim, kernel_size, stride, pad, cover_all):
+    n = _lib.load().hipcx_conv_out_dim(in_dim, kernel_size, stride, pad, int(bool(cover_all)))
+    if n < 0:
+        raise _lib.DimensionError('Output size should be positive.')
+    return n
+
+
+def _channels_last_empty(n, c, h, w, dtype):
+    """NCHW-shaped array over NHWC memory: what the hip ConvKernel / pooling kernels return."""
+    it = numpy.dtype(dtype).itemsize
+    strides = (h * w * c * it, it, w * c * it, c * it)
+    return ndarray(alloc_bytes(n * c * h * w * it), 0, (n, c, h, w), strides, dtype)
+
+
+def conv(x, w, b=None, stride=1, pad=0, cover_all=False, out_dtype=None):
+    """Conv (CX/routines/connection.cc:140-208), 2-D only: one ConvKernel call with the bias inside."""
+    if x.ndim != 4 or w.ndim != 4:
+        raise _lib.ChainerxNotImplementedError('only 2-D convolution is on the supported path')
+    stride, pad = _pair(stride), _pair(pad)
+    if w.shape[1] != x.shape[1]:
+        raise _lib.DimensionError('Mismatched number of input channels in input %r and weights %r.' % (x.shape, w.shape))
+    if b is not None and (b.ndim != 1 or b.shape[0] != w.shape[0]):
+        raise _lib.DimensionError('Mismatched bias shape %r for weights %r.' % (b.shape, w.shape))
+    dt = numpy.dtype(out_dtype) if out_dtype is not None else (result_type(x, w, b) if b is not None else result_type(x, w))
+    oh = conv_out_dim(x.shape[2], w.shape[2], stride[0], pad[0], cover_all)
+    ow = conv_out_dim(x.shape[3], w.shape[3], stride[1], pad[1], cover_all)
+    out = _channels_last_empty(x.shape[0], w.shape[0], oh, ow, dt)
+    xc, wc = x.astype(dt, False), w.astype(dt, False)
+    bc = b.astype(dt, False) if b is not None else None
+    nbytes = _lib.load().hipcx_conv_workspace_size(xc.desc(), wc.desc(), out.desc())
+    ws, wsp = _workspace(nbytes)
+    _lib.call('hipcx_conv', xc.desc(), wc.desc(), bc.desc() if bc is not None else None, _i64(stride), _i64(pad),
+              int(bool(cover_all)), out.desc(), wsp, nbytes, current_stream())
+    return out
+
+
+def fixed_batch_norm(x, gamma, beta, mean, var, eps=2e-5, axis=None):
+    """FixedBatchNorm (CX/routines/normalization.cc:414-424 with PreprocessBatchNorm :61-101)."""
+    for a in (x, gamma, beta, mean, var):
+        if _kind(a.dtype) != 3:
+            raise _lib.DtypeError('BatchNorm only supports floating kind inputs.')
+    axes = _sorted_axes(axis, x.ndim) if axis is not None else (0,)
+    reduced_shape = tuple(1 if i in axes else d for i, d in enumerate(x.shape))
+    size = _prod(reduced_shape)
+    params = []
+    for name, a in (('Gamma', gamma), ('Beta', beta), ('Mean', mean), ('Variance', var)):
+        if a.size != size:
+            raise _lib.DimensionError('%s must have the same size as the reduced input. Actual: %d. Expected: %d.' % (name, a.size, size))
+        params.append(a.reshape(reduced_shape))
+    out = ndarray(alloc_bytes(x.nbytes), 0, x.shape, _dense_strides_like(x), x.dtype)
+    ax = (ctypes.c_int8 * len(axes))(*axes)
+    _lib.call('hipcx_fixed_batch_norm', x.desc(), params[0].desc(), params[1].desc(), params[2].desc(), params[3].desc(),
+              _lib.make_scalar(float(eps)), ax, len(axes), out.desc(), current_stream())
+    return out
+
+
+def _dense_strides_like(x):
+    """Dense strides with the same axis order as x's memory (so a channels-last input gives a channels-last output)."""
+    order = sorted(range(x.ndim), key=lambda i: (-abs(x.strides[i]), i))
+    strides = [0] * x.ndim
+    acc = x.itemsize
+    for i in reversed(order):
+        strides[i] = acc
+        acc *= _py.max(1, x.shape[i])
+    return tuple(strides)
+
+
+def max_pool(x, ksize, stride=None, pad=0, cover_all=False):
+    """MaxPool (CX/routines/pooling.cc:52-123), 2-D."""
+    if x.ndim != 4:
+        raise _lib.ChainerxNotImplementedError('only 2-D pooling is on the supported path')
+    ksize = _pair(ksize)
+    stride = ksize if stride is None else _pair(stride)
+    pad = _pair(pad)
+    oh = conv_out_dim(x.shape[2], ksize[0], stride[0], pad[0], cover_all)
+    ow = conv_out_dim(x.shape[3], ksize[1], stride[1], pad[1], cover_all)
+    out = _channels_last_empty(x.shape[0], x.shape[1], oh, ow, x.dtype)
+    _lib.call('hipcx_max_pool', x.desc(), _i64(ksize), _i64(stride), _i64(pad), int(bool(cover_all)), out.desc(), current_stream())
+    return out
+
+
+def average_pool(x, ksize, stride=None, pad=0, pad_mode='ignore'):
+    """AveragePool (CX/routines/pooling.cc:125-169), 2-D, float dtypes only."""
+    if _kind(x.dtype) != 3:
+        raise _lib.DtypeError('cannot apply average pooling to non-float arrays')
+    if x.ndim != 4:
+        raise _lib.ChainerxNotImplementedError('only 2-D pooling is on the supported path')
+    ksize = _pair(ksize)
+    stride = ksize if stride is None else _pair(stride)
+    pad = _pair(pad)
+    mode = {'zero': 1, 'ignore': 2}[pad_mode]
+    oh = conv_out_dim(x.shape[2], ksize[0], stride[0], pad[0], False)
+    ow = conv_out_dim(x.shape[3], ksize[1], stride[1], pad[1], False)
+    out = _channels_last_empty(x.shape[0], x.shape[1], oh, ow, x.dtype)
+    _lib.call('hipcx_average_pool', x.desc(), _i64(ksize), _i64(stride), _i64(pad), mode, out.desc(), current_stream())
+    return out
+
+
+# ---------------------------------------------------------------------------------------------
+# indexing
+# ---------------------------------------------------------------------------------------------
+_BOUNDS = {None: 0, 'raise': 1, 'wrap': 2, 'clip': 3}
+
+
+def take(a, indices, axis, mode=None):
+    """Take (CX/routines/indexing.cc:171-205). mode None / 'raise' raise IndexError on out-of-range ids like the
+    native backend; checking that costs one 4-byte read-back after the kernel."""
+    if _kind(indices.dtype) not in (1, 2):
+        raise _lib.DtypeError('Only arrays of integer dtype can be used as indices.')
+    axis = _normalize_axis(axis, a.ndim)
+    out_shape = a.shape[:axis] + indices.shape + a.shape[axis + 1:]
+    out = ndarray.empty(out_shape, a.dtype)
+    m = _BOUNDS[mode]
+    flag = None
+    flag_ptr = None
+    if m in (0, 1):
+        flag = zeros((1,), 'int32')
+        flag_ptr = ctypes.cast(ctypes.c_void_p(flag.data_ptr), ctypes.POINTER(ctypes.c_int32))
+    _lib.call('hipcx_take', a.desc(), indices.desc(), axis, out.desc(), m, flag_ptr, current_stream())
+    if flag is not None and int(flag.get()[0]) != 0:
+        raise _lib.ChainerxIndexError('Index is out of bounds for axis %d with size %d' % (axis, a.shape[axis]))
+    return out
+
+
+# ---------------------------------------------------------------------------------------------
+# composite routines
+# ---------------------------------------------------------------------------------------------
+def lstm(c, x):
+    """Lstm cell (CX/routines/connection.cc:396-446), equal batch sizes: gates are stride-4 views of x."""
+    if x.shape[0] > c.shape[0]:
+        raise _lib.DimensionError('The batch size of x must be equal to or less than the size of c')
+    if x.shape[1] != 4 * c.shape[1]:
+        raise _lib.DimensionError('Expected dimension at axis 1 of x to be equal 4 times dimension at axis 1 of c.')
+    if _kind(c.dtype) != 3:
+        raise _lib.DtypeError('Expected data type float')
+    if c.dtype != x.dtype:
+        raise _lib.DtypeError('Datatypes of c and x should be equal')
+    if x.shape[0] != c.shape[0]:
+        raise _lib.ChainerxNotImplementedError('ragged batches are not on the supported path')
+    xr = x.reshape((x.shape[0], x.shape[1] // 4, 4) + tuple(x.shape[2:]))
+    gates = [g.squeeze(2) for g in split(xr, 4, 2)]
+    a = tanh(gates[0])
+    i = sigmoid(gates[1])
+    f = sigmoid(gates[2])
+    o = sigmoid(gates[3])
+    new_c = add(multiply(a, i), multiply(f, c))
+    h = multiply(o, tanh(new_c))
+    return h, new_c
+
+
+def softmax_cross_entropy(x, t):
+    """Chainer's F.softmax_cross_entropy forward for chainerx arrays with the default reduce='mean', normalize=True
+    (chainer/functions/loss/softmax_cross_entropy.py:123-130): a Python-level composition, 15 kernel calls."""
+    score = log_softmax(x, 1)
+    mask = equal(t[:, None], arange(score.shape[1], dtype=t.dtype)).astype(score.dtype)
+    return multiply(sum(multiply(score, mask)), divide(-1, sum(mask)))
+
+
+# ---------------------------------------------------------------------------------------------
+# operators
+# ---------------------------------------------------------------------------------------------
+def _install_operators():
+    ndarray.__add__ = lambda self, o: add(self, o)
+    ndarray.__radd__ = lambda self, o: add(self, o)
+    ndarray.__sub__ = lambda self, o: subtract(self, o)
+    ndarray.__rsub__ = lambda self, o: subtract(o, self)
+    ndarray.__mul__ = lambda self, o: multiply(self, o)
+    ndarray.__rmul__ = lambda self, o: multiply(self, o)
+    ndarray.__truediv__ = lambda self, o: divide(self, o)
+    ndarray.__rtruediv__ = lambda self, o: divide(o, self)
+    ndarray.__neg__ = lambda self: negative(self)
+    ndarray.__iadd__ = lambda self, o: add(self, o, out=self)
+    ndarray.__isub__ = lambda self, o: subtract(self, o, out=self)
+    ndarray.__imul__ = lambda self, o: multiply(self, o, out=self)
+    ndarray.__itruediv__ = lambda self, o: divide(self, o, out=self)
+    ndarray.__eq__ = lambda self, o: equal(self, o)
+    ndarray.__ne__ = lambda self, o: not_equal(self, o)
+    ndarray.__gt__ = lambda self, o: greater(self, o)
+    ndarray.__ge__ = lambda self, o: greater_equal(self, o)
+    ndarray.__hash__ = None
+    ndarray.sum = lambda self, axis=None, keepdims=False: sum(self, axis, keepdims)
+    ndarray.max = lambda self, axis=None, keepdims=False: amax(self, axis, keepdims)
+    ndarray.argmax = lambda self, axis=None: argmax(self, axis)
+    ndarray.mean = lambda self, axis=None, keepdims=False: mean(self, axis, keepdims)
+    ndarray.dot = lambda self, o: dot(self, o)
+    ndarray.take = lambda self, indices, axis, mode=None: take(self, indices, axis, mode)
+
+
+_install_operators()

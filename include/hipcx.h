@@ -1,0 +1,185 @@
+/*
+ * hipcx.h -- C ABI of the MI355X (gfx950) kernel library behind the ChainerX `hip` backend.
+ *
+ * One entry point per ChainerX kernel class on the inference hot path.  Each function performs
+ * exactly the work of one `Backend::CallKernel<XxxKernel>(...)` in the reference and is what the
+ * `HipXxxKernel::Call` override of the `hip` backend plugin forwards to.  Paths in the comments
+ * are relative to the reference tree, `CX/` = `chainerx_cc/chainerx/`.
+ *
+ * Conventions
+ *  - Arrays are described by `hipcx_array`: `data` is the device address of element (0,...,0),
+ *    i.e. `raw_data + offset` (CX/backend_util.h:10-13); strides are in BYTES, signed, and may be
+ *    0 (broadcast / keep-dims) or permuted (transposed views), as in CX/array.h.
+ *  - dtype codes are the values of `chainerx::Dtype` (CX/dtype.h:19-29).
+ *  - Scalars follow `chainerx::Scalar` (CX/scalar.h): a kind tag plus an int64 or a double.
+ *  - Every call is asynchronous on `stream` (a `hipStream_t`, may be NULL for the default
+ *    stream), like the CUDA backend (CX/cuda/elementwise.cuh:41-47).
+ *  - Return value: 0 on success, otherwise a `hipcx_status` naming the ChainerX exception type
+ *    (CX/error.h:48-95) the plugin must throw; `hipcx_last_error()` gives the message.
+ *  - Kernels that need device scratch memory take `workspace`/`workspace_bytes`; the matching
+ *    `*_workspace_size` function tells how much.  The library itself never allocates.
+ */
+#ifndef HIPCX_H_
+#define HIPCX_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HIPCX_MAX_NDIM 10 /* CX/constant.h:6 kMaxNdim */
+
+typedef enum hipcx_dtype { /* CX/dtype.h:19-29 */
+    HIPCX_BOOL = 1,
+    HIPCX_INT8 = 2,
+    HIPCX_INT16 = 3,
+    HIPCX_INT32 = 4,
+    HIPCX_INT64 = 5,
+    HIPCX_UINT8 = 6,
+    HIPCX_FLOAT16 = 7,
+    HIPCX_FLOAT32 = 8,
+    HIPCX_FLOAT64 = 9
+} hipcx_dtype;
+
+typedef enum hipcx_status { /* CX/error.h:48-95 */
+    HIPCX_OK = 0,
+    HIPCX_CHAINERX_ERROR = 1,
+    HIPCX_DIMENSION_ERROR = 2,
+    HIPCX_DTYPE_ERROR = 3,
+    HIPCX_NOT_IMPLEMENTED_ERROR = 4,
+    HIPCX_INDEX_ERROR = 5,
+    HIPCX_BACKEND_ERROR = 6,
+    HIPCX_DEVICE_ERROR = 7
+} hipcx_status;
+
+typedef enum hipcx_scalar_kind { /* CX/dtype.h DtypeKind */
+    HIPCX_KIND_BOOL = 0,
+    HIPCX_KIND_INT = 1,
+    HIPCX_KIND_FLOAT = 3
+} hipcx_scalar_kind;
+
+typedef enum hipcx_index_bounds_mode { /* CX/array_index.h:21-26 */
+    HIPCX_BOUNDS_DEFAULT = 0,
+    HIPCX_BOUNDS_RAISE = 1,
+    HIPCX_BOUNDS_WRAP = 2,
+    HIPCX_BOUNDS_CLIP = 3
+} hipcx_index_bounds_mode;
+
+typedef enum hipcx_avg_pool_pad_mode { /* CX/routines/pooling.h:13-16 */
+    HIPCX_PAD_ZERO = 1,
+    HIPCX_PAD_IGNORE = 2
+} hipcx_avg_pool_pad_mode;
+
+typedef struct hipcx_array {
+    void* data;
+    int32_t dtype;
+    int32_t ndim;
+    int64_t shape[HIPCX_MAX_NDIM];
+    int64_t strides[HIPCX_MAX_NDIM];
+} hipcx_array;
+
+typedef struct hipcx_scalar {
+    int32_t kind; /* hipcx_scalar_kind */
+    int32_t reserved;
+    int64_t i; /* value when kind is BOOL or INT */
+    double f;  /* value when kind is FLOAT */
+} hipcx_scalar;
+
+/* ---- library ---- */
+const char* hipcx_last_error(void); /* thread-local message of the last failing call */
+int hipcx_version(void);
+int hipcx_device_count(int* count);          /* Backend::GetDeviceCount, CX/backend.h:29 */
+int hipcx_synchronize(int device_index);     /* Device::Synchronize, CX/device.h:71 */
+int hipcx_device_name(int device_index, char* buf, size_t buf_len);
+
+/* ---- elementwise arithmetic: CX/kernels/arithmetic.h ---- */
+/* Inputs must already have out's dtype (the plugin applies AsType as CX/native/kernel_regist.h:55-56 does). */
+int hipcx_add(const hipcx_array* x1, const hipcx_array* x2, const hipcx_array* out, void* stream);        /* AddKernel :11 */
+int hipcx_add_as(const hipcx_array* x1, hipcx_scalar x2, const hipcx_array* out, void* stream);           /* AddASKernel :16 */
+int hipcx_subtract(const hipcx_array* x1, const hipcx_array* x2, const hipcx_array* out, void* stream);   /* SubtractKernel :21 */
+int hipcx_subtract_as(const hipcx_array* x1, hipcx_scalar x2, const hipcx_array* out, void* stream);      /* SubtractASKernel :26 */
+int hipcx_multiply(const hipcx_array* x1, const hipcx_array* x2, const hipcx_array* out, void* stream);   /* MultiplyKernel :31 */
+int hipcx_multiply_as(const hipcx_array* x1, hipcx_scalar x2, const hipcx_array* out, void* stream);      /* MultiplyASKernel :36 */
+int hipcx_divide(const hipcx_array* x1, const hipcx_array* x2, const hipcx_array* out, void* stream);     /* DivideKernel :56 */
+int hipcx_divide_as(const hipcx_array* x1, hipcx_scalar x2, const hipcx_array* out, void* stream);        /* DivideASKernel :61 */
+int hipcx_divide_sa(hipcx_scalar x1, const hipcx_array* x2, const hipcx_array* out, void* stream);        /* DivideSAKernel :66 */
+
+/* ---- elementwise math: CX/kernels/explog.h, hyperbolic.h, misc.h ---- */
+int hipcx_exp(const hipcx_array* x, const hipcx_array* out, void* stream);   /* ExpKernel explog.h:15 */
+int hipcx_log(const hipcx_array* x, const hipcx_array* out, void* stream);   /* LogKernel explog.h:30 */
+int hipcx_tanh(const hipcx_array* x, const hipcx_array* out, void* stream);  /* TanhKernel hyperbolic.h:18 */
+int hipcx_sqrt(const hipcx_array* x, const hipcx_array* out, void* stream);  /* SqrtKernel misc.h:14 */
+/* out = x1 < x2 ? pos : neg   (ReLU is Maximum(x,0) = IfLessElse(x,0,0,x), CX/routines/misc.cc:210-216) */
+int hipcx_if_less_else_assa(const hipcx_array* x1, hipcx_scalar x2, hipcx_scalar pos, const hipcx_array* neg,
+                            const hipcx_array* out, void* stream);            /* IfLessElseASSAKernel misc.h:36 */
+int hipcx_if_greater_else_assa(const hipcx_array* x1, hipcx_scalar x2, hipcx_scalar pos, const hipcx_array* neg,
+                               const hipcx_array* out, void* stream);         /* IfGreaterElseASSAKernel misc.h:43 */
+int hipcx_if_greater_else_aaaa(const hipcx_array* x1, const hipcx_array* x2, const hipcx_array* pos, const hipcx_array* neg,
+                               const hipcx_array* out, void* stream);         /* IfGreaterElseAAAAKernel misc.h:48 */
+
+/* ---- logic: CX/kernels/logic.h (inputs share one dtype, out is bool) ---- */
+int hipcx_equal(const hipcx_array* x1, const hipcx_array* x2, const hipcx_array* out, void* stream);          /* EqualKernel :9 */
+int hipcx_not_equal(const hipcx_array* x1, const hipcx_array* x2, const hipcx_array* out, void* stream);      /* NotEqualKernel :14 */
+int hipcx_greater(const hipcx_array* x1, const hipcx_array* x2, const hipcx_array* out, void* stream);        /* GreaterKernel :19 */
+int hipcx_greater_equal(const hipcx_array* x1, const hipcx_array* x2, const hipcx_array* out, void* stream);  /* GreaterEqualKernel :24 */
+
+/* ---- creation: CX/kernels/creation.h, misc.h ---- */
+int hipcx_copy(const hipcx_array* a, const hipcx_array* out, void* stream);                       /* CopyKernel creation.h:16 (dtype-casting) */
+int hipcx_fill(const hipcx_array* out, hipcx_scalar value, void* stream);                         /* FillKernel misc.h:9 */
+int hipcx_arange(hipcx_scalar start, hipcx_scalar step, const hipcx_array* out, void* stream);    /* ArangeKernel creation.h:11 */
+
+/* ---- reductions: CX/kernels/reduction.h:18, statistics.h:13, sorting.h:9 ----
+ * `axis` is sorted, unique, non-negative (CX/kernels/reduction.h:11-18); `out` either drops the
+ * reduced axes or keeps them with extent 1.  argmax writes int64 and reproduces the native
+ * backend's tie/NaN rule bit for bit (CX/native/reduce.h:46-83 with the functor of
+ * CX/native/native_device/reduction.cc:34-61). */
+size_t hipcx_reduce_workspace_size(const hipcx_array* a, const int8_t* axis, int naxis, const hipcx_array* out);
+int hipcx_sum(const hipcx_array* a, const int8_t* axis, int naxis, const hipcx_array* out, void* workspace, size_t workspace_bytes,
+              void* stream);
+int hipcx_amax(const hipcx_array* a, const int8_t* axis, int naxis, const hipcx_array* out, void* workspace, size_t workspace_bytes,
+               void* stream);
+int hipcx_argmax(const hipcx_array* a, const int8_t* axis, int naxis, const hipcx_array* out, void* workspace,
+                 size_t workspace_bytes, void* stream);
+
+/* ---- linear algebra / connection: CX/kernels/linalg.h:15, connection.h:21 ---- */
+/* out[M,N] = a[M,K] . b[K,N]; float16/32/64; fp16 accumulates in fp32 (CX/native/native_device/dot.cc:181-227). */
+size_t hipcx_dot_workspace_size(const hipcx_array* a, const hipcx_array* b, const hipcx_array* out);
+int hipcx_dot(const hipcx_array* a, const hipcx_array* b, const hipcx_array* out, void* workspace, size_t workspace_bytes,
+              void* stream);
+/* Output extent of a convolution/pooling window (CX/routines/connection.cc:37-49). Returns -1 if not positive. */
+int64_t hipcx_conv_out_dim(int64_t in_dim, int64_t kernel_size, int64_t stride, int64_t pad, int cover_all);
+/* 2-D convolution forward, x[N,C,H,W] (any strides), w[K,C,kh,kw], optional b[K] (NULL = none),
+ * out[N,K,OH,OW] with any strides: the plugin allocates it channels-last (an NCHW *view* of NHWC
+ * memory, as the native backend's own result is: CX/native/native_device/conv.cc:78-84). */
+size_t hipcx_conv_workspace_size(const hipcx_array* x, const hipcx_array* w, const hipcx_array* out);
+int hipcx_conv(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, const int64_t* stride, const int64_t* pad,
+               int cover_all, const hipcx_array* out, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---- normalization: FixedBatchNormKernel CX/kernels/normalization.h:107 ----
+ * gamma/beta/mean/var have the keep-dims reduced shape of x over `axis`
+ * (CX/routines/normalization.cc:61-101). out has x's shape and dtype. */
+int hipcx_fixed_batch_norm(const hipcx_array* x, const hipcx_array* gamma, const hipcx_array* beta, const hipcx_array* mean,
+                           const hipcx_array* var, hipcx_scalar eps, const int8_t* axis, int naxis, const hipcx_array* out,
+                           void* stream);
+
+/* ---- pooling: CX/kernels/pooling.h:29,83 (2-D, NCHW logical layout, any strides) ---- */
+int hipcx_max_pool(const hipcx_array* x, const int64_t* kernel_size, const int64_t* stride, const int64_t* pad, int cover_all,
+                   const hipcx_array* out, void* stream);
+int hipcx_average_pool(const hipcx_array* x, const int64_t* kernel_size, const int64_t* stride, const int64_t* pad, int pad_mode,
+                       const hipcx_array* out, void* stream);
+
+/* ---- indexing: TakeKernel CX/kernels/indexing.h:17 ----
+ * `error_flag` is a device int32 the caller zeroes before the call; with mode DEFAULT/RAISE the
+ * kernel stores 1 there when an index is out of range (the native backend raises IndexError,
+ * CX/native/native_device/indexing.cc:68-74); the plugin reads it back and throws.  May be NULL,
+ * in which case out-of-range indices are wrapped as the CUDA backend does
+ * (CX/cuda/cuda_device/indexing.cu:58-66). */
+int hipcx_take(const hipcx_array* a, const hipcx_array* indices, int8_t axis, const hipcx_array* out, int mode, int32_t* error_flag,
+               void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HIPCX_H_ */
