@@ -1,0 +1,148 @@
+#!/usr/bin/env python3
+"""Headline benchmark: ResNet-50 float16 inference at batch 128 through the hip backend's kernels.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 128]
+
+A step is one forward pass of the network of chainer_amd/configs.py (53 convolutions, fixed batch
+norm, ReLU, residual adds, pooling, linear) over one synthetic batch that is already resident in
+device memory.  Every operation is one C-ABI kernel call, decomposed as the ChainerX routines do.
+One JSON line is printed; besides the contract keys it carries
+
+  roofline      the implicit-GEMM convolution kernel (the dominant one): algorithmic flops of its
+                launches in one step / their summed duration, measured with HIP events recorded on
+                the launch stream around each launch (hipcx_profile_start/stop) in extra steps run
+                after the timed region, against the dense fp16 MFMA peak.
+  cpu_baseline  the CPU oracle (a single-threaded restatement of the ChainerX native backend) on a
+                small batch of the same network, timed on this host.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+
+MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 matrix peak
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument('--gpus', type=int, default=1)
+    ap.add_argument('--steps', type=int, default=20)
+    ap.add_argument('--warmup', type=int, default=5)
+    ap.add_argument('--batch', type=int, default=128)
+    ap.add_argument('--cpu-batch', type=int, default=8, help='images for the CPU baseline (0 = skip)')
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit('bench.py: this build runs on one GPU only (inference shards trivially along the batch axis; '
+                 'no multi-GPU path is built). Run with --gpus 1.')
+
+    import torch
+    import chainer_amd as chx
+    from chainer_amd import _lib, configs as cfg
+
+    if not torch.cuda.is_available():
+        sys.exit('bench.py: no HIP device visible')
+
+    params_host = cfg.resnet50_params()
+    params = cfg.tree_map(chx.array, params_host)
+    x = chx.array(cfg.resnet50_input(batch=args.batch))
+
+    def step():
+        return cfg.resnet50_forward(chx, params, x)
+
+    for _ in range(args.warmup):
+        y = step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        y = step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / args.steps * 1e3
+    img_s = args.batch * args.steps / elapsed
+    finite = bool(np.isfinite(y.get().astype(np.float32)).all())
+
+    # ---- roofline of the dominant kernel: event-bracketed implicit-GEMM launches, extra steps ----
+    lib = _lib.load()
+    prof_steps = max(1, min(args.steps, 5))
+    _lib.check(lib.hipcx_profile_start())
+    for _ in range(prof_steps):
+        step()
+    n = ctypes.c_int64()
+    ms = ctypes.c_double()
+    flops = ctypes.c_double()
+    nbytes = ctypes.c_double()
+    _lib.check(lib.hipcx_profile_stop(ctypes.byref(n), ctypes.byref(ms), ctypes.byref(flops), ctypes.byref(nbytes)))
+    launches_per_step = n.value // prof_steps
+    avg_launch_ms = ms.value / max(n.value, 1)
+    achieved_tflops = flops.value / (ms.value * 1e-3) / 1e12 if ms.value > 0 else 0.0
+    roofline = {
+        'kernel': 'IGemmFastKernel/IGemmGenericKernel (conv + linear)',
+        'bound': 'mfma',
+        'achieved': round(achieved_tflops, 2),
+        'peak': MFMA_F16_PEAK_TFLOPS,
+        'unit': 'TFLOP/s',
+        'frac': round(achieved_tflops / MFMA_F16_PEAK_TFLOPS, 4),
+        'traffic': None,
+        'launches_per_step': launches_per_step,
+        'avg_launch_us': round(avg_launch_ms * 1e3, 2),
+        'kernel_ms_per_step': round(ms.value / prof_steps, 3),
+        'algorithmic_gflop_per_step': round(flops.value / prof_steps / 1e9, 2),
+        'algorithmic_gb_per_step': round(nbytes.value / prof_steps / 1e9, 3),
+        'achieved_gbs': round(nbytes.value / (ms.value * 1e-3) / 1e9, 1) if ms.value > 0 else 0.0,
+    }
+
+    # ---- CPU baseline: the oracle on a bounded sample of the same workload ----
+    cpu = None
+    if args.cpu_batch > 0:
+        from oracle import native as oracle
+        xs = cfg.resnet50_input(batch=args.cpu_batch)
+        t0 = time.perf_counter()
+        ref = cfg.resnet50_forward(oracle, params_host, xs)
+        cpu_s = time.perf_counter() - t0
+        got = cfg.resnet50_forward(chx, params, chx.array(xs)).get().astype(np.float64)
+        refd = ref.astype(np.float64)
+        rel = float(np.abs(got - refd).max() / max(np.abs(refd).max(), 1e-30))
+        cpu = {
+            'value': round(args.cpu_batch / cpu_s, 3),
+            'unit': 'img/s',
+            'cores': 1,
+            'kind': 'port',
+            'sample': '%d images, one forward pass of the same ResNet-50 (fp16 storage, fp32 accumulation), %.1f s'
+                      % (args.cpu_batch, cpu_s),
+            'max_rel_err_vs_gpu': rel,
+        }
+
+    out = {
+        'metric': 'ResNet-50 fp16 inference img/s @bs%d on 1 MI355X' % args.batch,
+        'value': round(img_s, 1),
+        'unit': 'img/s',
+        'n_gpus': 1,
+        'steps': args.steps,
+        'warmup': args.warmup,
+        'ms_per_step': round(ms_per_step, 3),
+        'higher_is_better': True,
+        'scaling': 'weak',
+        'vs_baseline': None,
+        'dtype': 'f16',
+        'data': 'synthetic',
+        'config': {
+            'workload': 'ResNet-50 inference, fp16 NCHW [%d,3,224,224], bottlenecks [3,4,6,3], fixed batch norm, '
+                        'one kernel call per ChainerX routine kernel (unfused)' % args.batch,
+            'batch': args.batch,
+            'residual_gamma_scale': cfg.RESNET50_RESIDUAL_GAMMA_SCALE,
+            'outputs_finite': finite,
+        },
+        'roofline': roofline,
+        'cpu_baseline': cpu,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == '__main__':
+    main()

@@ -136,6 +136,9 @@ SIGNATURES = {
     'hipcx_conv_out_dim': (ctypes.c_int64, [ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, _INT]),
     'hipcx_conv_workspace_size': (_SZ, [_A, _A, _A]),
     'hipcx_conv': (_INT, [_A, _A, _A, _I64P, _I64P, _INT, _A, _V, _SZ, _V]),
+    'hipcx_profile_start': (_INT, []),
+    'hipcx_profile_stop': (_INT, [_I64P, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double),
+                                  ctypes.POINTER(ctypes.c_double)]),
     'hipcx_fixed_batch_norm': (_INT, [_A, _A, _A, _A, _A, _S, _I8P, _INT, _A, _V]),
     'hipcx_max_pool': (_INT, [_A, _I64P, _I64P, _I64P, _INT, _A, _V]),
     'hipcx_average_pool': (_INT, [_A, _I64P, _I64P, _I64P, _INT, _A, _V]),

@@ -1,0 +1,241 @@
+"""The five benchmark/parity workloads, written once against a routine namespace ``F``.
+
+``F`` is either ``chainer_amd`` (device arrays, HIP kernels) or any module exposing the same
+routine names on numpy arrays; the parity tests pass the CPU oracle there.  The graphs follow the
+reference's example models and the Chainer functions' ``forward_chainerx`` decompositions:
+
+* mlp:       examples/mnist/train_mnist.py, chainerx_cc/examples/mnist/train_mnist.cc:48-75
+* sweep:     elementwise / reduction kernels one by one
+* cifar:     3x3 conv stack with fixed batch norm (examples/cifar)
+* resnet50:  chainerx_cc/examples/imagenet_py/resnet50.py:103-127,202-225 (stride on the first 1x1)
+* lstm_lm:   examples/ptb/train_ptb.py:28-50 with L.LSTM = Linear(x) + Linear(h) -> F.lstm
+
+Parameters and inputs are drawn from ``numpy.random.Generator(PCG64(seed))`` on the host.
+"""
+import numpy as np
+
+
+def _rng(seed):
+    return np.random.Generator(np.random.PCG64(seed))
+
+
+def _he_normal(rng, shape, dtype):
+    fan_in = int(np.prod(shape[1:]))
+    return (rng.standard_normal(shape) * np.sqrt(2.0 / fan_in)).astype(np.float32).astype(dtype)
+
+
+def _bn_params(rng, c, dtype):
+    return {
+        'gamma': rng.uniform(0.5, 1.5, c).astype(np.float32).astype(dtype),
+        'beta': (rng.standard_normal(c) * 0.1).astype(np.float32).astype(dtype),
+        'mean': (rng.standard_normal(c) * 0.1).astype(np.float32).astype(dtype),
+        'var': rng.uniform(0.5, 1.5, c).astype(np.float32).astype(dtype),
+    }
+
+
+def tree_map(fn, tree):
+    if isinstance(tree, dict):
+        return {k: tree_map(fn, v) for k, v in tree.items()}
+    if isinstance(tree, (list, tuple)):
+        return [tree_map(fn, v) for v in tree]
+    return fn(tree)
+
+
+BN_EPS = 2e-5
+
+
+def _bn(F, x, p):
+    # chainer.functions.fixed_batch_normalization on a 4-D input with 1-D parameters: axis (0, 2, 3)
+    # (chainer/functions/normalization/batch_normalization.py:832-840), eps 2e-5.
+    return F.fixed_batch_norm(x, p['gamma'], p['beta'], p['mean'], p['var'], BN_EPS, (0, 2, 3))
+
+
+# ---------------------------------------------------------------------------------------------
+# C1: MNIST-shaped MLP + softmax cross entropy (fp32, batch 100)
+# ---------------------------------------------------------------------------------------------
+def mlp_params(seed=1, dtype=np.float32, n_in=784, n_units=1000, n_out=10):
+    rng = _rng(seed)
+
+    def lecun(shape):  # N(0, 1/fan_in), Chainer's default initializer
+        return (rng.standard_normal(shape) / np.sqrt(shape[1])).astype(dtype)
+
+    return {
+        'w1': lecun((n_units, n_in)), 'b1': np.zeros(n_units, dtype),
+        'w2': lecun((n_units, n_units)), 'b2': np.zeros(n_units, dtype),
+        'w3': lecun((n_out, n_units)), 'b3': np.zeros(n_out, dtype),
+    }
+
+
+def mlp_input(seed=1, batch=100, dtype=np.float32, n_in=784, n_out=10):
+    rng = _rng(seed + 1000)
+    x = rng.random((batch, n_in)).astype(dtype)
+    t = rng.integers(0, n_out, batch).astype(np.int32)
+    return x, t
+
+
+def mlp_forward(F, p, x, t):
+    h = F.relu(F.linear(x, p['w1'], p['b1']))
+    h = F.relu(F.linear(h, p['w2'], p['b2']))
+    y = F.linear(h, p['w3'], p['b3'])
+    return y, F.softmax_cross_entropy(y, t)
+
+
+# ---------------------------------------------------------------------------------------------
+# C3: CIFAR-shaped conv net inference (fp32 NCHW, batch 256)
+# ---------------------------------------------------------------------------------------------
+CIFAR_CHANNELS = (64, 64, 128, 128, 256, 256)
+
+
+def cifar_params(seed=3, dtype=np.float32, n_out=10):
+    rng = _rng(seed)
+    p = {'convs': [], 'bns': []}
+    c_in = 3
+    for c_out in CIFAR_CHANNELS:
+        p['convs'].append(_he_normal(rng, (c_out, c_in, 3, 3), dtype))
+        p['bns'].append(_bn_params(rng, c_out, dtype))
+        c_in = c_out
+    p['fc_w'] = _he_normal(rng, (n_out, c_in), dtype)
+    p['fc_b'] = np.zeros(n_out, dtype)
+    return p
+
+
+def cifar_input(seed=3, batch=256, dtype=np.float32):
+    return _rng(seed + 1000).standard_normal((batch, 3, 32, 32)).astype(dtype)
+
+
+def cifar_forward(F, p, x):
+    h = x
+    for i, (w, bn) in enumerate(zip(p['convs'], p['bns'])):
+        h = F.relu(_bn(F, F.conv(h, w, None, 1, 1), bn))
+        if i % 2 == 1:
+            h = F.max_pool(h, 2, 2, 0)
+    h = F.average_pool(h, h.shape[2], 1, 0, 'zero')  # global average pooling
+    return F.linear(h, p['fc_w'], p['fc_b'])
+
+
+# ---------------------------------------------------------------------------------------------
+# C4: ResNet-50 inference (fp16 NCHW, batch 128)
+# ---------------------------------------------------------------------------------------------
+RESNET50_BLOCKS = (3, 4, 6, 3)
+
+
+RESNET50_RESIDUAL_GAMMA_SCALE = 0.25
+
+
+def resnet50_params(seed=4, dtype=np.float16, n_out=1000, residual_gamma_scale=RESNET50_RESIDUAL_GAMMA_SCALE):
+    """He-normal filters and batch-norm statistics drawn as for the CIFAR net.  One deviation: gamma of the last
+    batch norm of every residual branch is scaled by `residual_gamma_scale`.  With statistics that are drawn at random
+    instead of measured, nothing normalises the residual stream: its magnitude grows ~1.4x per block and passes the
+    float16 maximum in stage 4 (on the CPU oracle as well); the scale keeps every activation below ~100."""
+    rng = _rng(seed)
+    p = {'conv1': _he_normal(rng, (64, 3, 7, 7), dtype), 'bn1': _bn_params(rng, 64, dtype), 'stages': []}
+    c_in = 64
+    for si, n_blocks in enumerate(RESNET50_BLOCKS):
+        mid = 64 * 2 ** si
+        c_out = 4 * mid
+        stage = []
+        for bi in range(n_blocks):
+            blk = {
+                'conv1': _he_normal(rng, (mid, c_in, 1, 1), dtype), 'bn1': _bn_params(rng, mid, dtype),
+                'conv2': _he_normal(rng, (mid, mid, 3, 3), dtype), 'bn2': _bn_params(rng, mid, dtype),
+                'conv3': _he_normal(rng, (c_out, mid, 1, 1), dtype), 'bn3': _bn_params(rng, c_out, dtype),
+            }
+            g3 = blk['bn3']['gamma'].astype(np.float32) * np.float32(residual_gamma_scale)
+            blk['bn3']['gamma'] = g3.astype(dtype)
+            if bi == 0:
+                blk['conv4'] = _he_normal(rng, (c_out, c_in, 1, 1), dtype)
+                blk['bn4'] = _bn_params(rng, c_out, dtype)
+            stage.append(blk)
+            c_in = c_out
+        p['stages'].append(stage)
+    p['fc_w'] = _he_normal(rng, (n_out, c_in), dtype)
+    p['fc_b'] = np.zeros(n_out, dtype)
+    return p
+
+
+def resnet50_input(seed=4, batch=128, dtype=np.float16, size=224):
+    return _rng(seed + 1000).standard_normal((batch, 3, size, size)).astype(np.float32).astype(dtype)
+
+
+def _bottleneck(F, blk, x, stride):
+    h = F.relu(_bn(F, F.conv(x, blk['conv1'], None, stride, 0), blk['bn1']))
+    h = F.relu(_bn(F, F.conv(h, blk['conv2'], None, 1, 1), blk['bn2']))
+    h = _bn(F, F.conv(h, blk['conv3'], None, 1, 0), blk['bn3'])
+    if 'conv4' in blk:
+        sc = _bn(F, F.conv(x, blk['conv4'], None, stride, 0), blk['bn4'])
+    else:
+        sc = x
+    return F.relu(F.add(h, sc))
+
+
+def resnet50_forward(F, p, x):
+    h = F.relu(_bn(F, F.conv(x, p['conv1'], None, 2, 3), p['bn1']))
+    h = F.max_pool(h, 3, 2, 1, False)  # 112 -> 56
+    for si, stage in enumerate(p['stages']):
+        for bi, blk in enumerate(stage):
+            h = _bottleneck(F, blk, h, 2 if (bi == 0 and si > 0) else 1)
+    h = F.average_pool(h, h.shape[2], 1, 0, 'zero')
+    return F.linear(h, p['fc_w'], p['fc_b'])
+
+
+def resnet50_flops(batch=128, size=224):
+    """Multiply-add count x2 of every conv and the final linear layer."""
+    total = 0
+
+    def conv(c_in, c_out, k, hw_out):
+        return 2 * c_in * c_out * k * k * hw_out * hw_out
+
+    hw = size // 2
+    total += conv(3, 64, 7, hw)
+    hw = hw // 2
+    c_in = 64
+    for si, n_blocks in enumerate(RESNET50_BLOCKS):
+        mid = 64 * 2 ** si
+        c_out = 4 * mid
+        for bi in range(n_blocks):
+            if bi == 0 and si > 0:
+                hw //= 2
+            total += conv(c_in, mid, 1, hw) + conv(mid, mid, 3, hw) + conv(mid, c_out, 1, hw)
+            if bi == 0:
+                total += conv(c_in, c_out, 1, hw)
+            c_in = c_out
+    total += 2 * c_in * 1000
+    return total * batch
+
+
+# ---------------------------------------------------------------------------------------------
+# C5: 2-layer LSTM language model inference (fp32, batch 128, seq 35)
+# ---------------------------------------------------------------------------------------------
+def lstm_lm_params(seed=5, dtype=np.float32, vocab=10000, units=650):
+    rng = _rng(seed)
+
+    def u(shape):
+        return rng.uniform(-0.05, 0.05, shape).astype(dtype)
+
+    p = {'embed': u((vocab, units)), 'layers': [], 'out_w': u((vocab, units)), 'out_b': u((vocab,))}
+    for _ in range(2):
+        p['layers'].append({'up_w': u((4 * units, units)), 'up_b': u((4 * units,)), 'lat_w': u((4 * units, units))})
+    return p
+
+
+def lstm_lm_input(seed=5, batch=128, seq=35, vocab=10000):
+    return _rng(seed + 1000).integers(0, vocab, (batch, seq)).astype(np.int32)
+
+
+def lstm_lm_forward(F, p, ids, zeros):
+    """Runs the sequence; returns log-probabilities of the last step and the final (h, c) of both layers.
+    ``zeros(shape, dtype)`` makes the initial state on the same backend as ``F``."""
+    batch, seq = ids.shape
+    units = p['embed'].shape[1]
+    dtype = p['embed'].dtype
+    hs = [zeros((batch, units), dtype) for _ in range(2)]
+    cs = [zeros((batch, units), dtype) for _ in range(2)]
+    y = None
+    for t in range(seq):
+        x = F.take(p['embed'], ids[:, t], 0)
+        for li, layer in enumerate(p['layers']):
+            gates = F.add(F.linear(x, layer['up_w'], layer['up_b']), F.linear(hs[li], layer['lat_w']))
+            hs[li], cs[li] = F.lstm(cs[li], gates)
+            x = hs[li]
+        y = F.linear(x, p['out_w'], p['out_b'])
+    return F.log_softmax(y, 1), hs, cs

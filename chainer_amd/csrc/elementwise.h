@@ -20,7 +20,7 @@
 
 namespace hipcx {
 
-constexpr int kEwMaxOperands = 5;  // out + up to 4 inputs
+constexpr int kEwMaxOperands = 6;  // out + up to 5 inputs
 constexpr int kEwThreads = 256;
 constexpr int kEwUnroll = 4;
 
@@ -193,7 +193,12 @@ __global__ __launch_bounds__(kEwThreads) void EwKernel(EwArgs<Op::kNumIn + 1> ar
             CIn b = NIN > 1 ? static_cast<CIn>(in[u][NIN > 1 ? 1 : 0].v[e]) : CIn{};
             CIn c = NIN > 2 ? static_cast<CIn>(in[u][NIN > 2 ? 2 : 0].v[e]) : CIn{};
             CIn d = NIN > 3 ? static_cast<CIn>(in[u][NIN > 3 ? 3 : 0].v[e]) : CIn{};
-            o.v[e] = static_cast<Out>(op(a, b, c, d, index0 + e));
+            if constexpr (NIN > 4) {
+                CIn f = static_cast<CIn>(in[u][4].v[e]);
+                o.v[e] = static_cast<Out>(op.Apply5(a, b, c, d, f));
+            } else {
+                o.v[e] = static_cast<Out>(op(a, b, c, d, index0 + e));
+            }
         }
         char* q = args.ptr[0] + off[u][0];
         if (VEC > 1) {

@@ -1,0 +1,255 @@
+// 2-D MaxPool / AveragePool forward (CX/kernels/pooling.h:29,83) on an NCHW-shaped array with
+// arbitrary strides.  The native backend materialises the windows (Im2Col) and reduces them
+// (CX/native/native_device/pool.cc:69-94, 252-302); here every output is computed directly.
+//
+//  - max: identity is lowest / -inf, padding never wins, NaN propagates (AMax rule,
+//    CX/native/native_device/statistics.cc:38-42).
+//  - average: float16 sums accumulate in float, are rounded to float16 and then divided in
+//    float16 arithmetic, as Sum followed by Divide does; the divisor is the window size ('zero')
+//    or the number of in-image taps ('ignore').
+//
+// Channels-last data is processed VEC channels per thread with 16-byte accesses; any other
+// layout one element per thread, with the thread order following the output's fastest axis.
+#include "common.h"
+
+namespace hipcx {
+namespace {
+
+struct PoolArgs {
+    const void* x;
+    void* out;
+    int N, C, H, W, OH, OW;
+    int kh, kw, sh, sw, ph, pw;
+    int64_t xsN, xsC, xsH, xsW;  // elements
+    int64_t osN, osC, osH, osW;
+    int pad_mode;  // average only
+    int w_fastest;  // thread order: 1 = ow fastest (channels-first memory), 0 = channel fastest
+};
+
+template <typename T, int N>
+struct alignas(sizeof(T) * N) PVec {
+    T v[N];
+};
+
+template <typename T>
+__device__ __forceinline__ T Lowest() {
+    if constexpr (std::is_same<T, half_t>::value) {
+        return static_cast<half_t>(-__builtin_huge_valf());
+    } else if constexpr (std::is_floating_point<T>::value) {
+        return -__builtin_huge_val();
+    } else if constexpr (std::is_same<T, bool>::value) {
+        return false;
+    } else {
+        return std::numeric_limits<T>::lowest();
+    }
+}
+
+template <typename T>
+__device__ __forceinline__ bool IsNanT(T v) {
+    if constexpr (std::is_same<T, half_t>::value || std::is_floating_point<T>::value) {
+        return v != v;
+    } else {
+        return false;
+    }
+}
+
+template <typename T, int VEC, bool IS_MAX>
+__global__ __launch_bounds__(256) void PoolKernel(PoolArgs p, int64_t total) {
+    using C = compute_t<T>;
+    const T* x = static_cast<const T*>(p.x);
+    T* out = static_cast<T*>(p.out);
+    const int cvecs = p.C / VEC;
+    for (int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; idx < total;
+         idx += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+        int cv, ow, oh;
+        int64_t n;
+        int64_t t = idx;
+        if (p.w_fastest) {
+            ow = static_cast<int>(t % p.OW);
+            t /= p.OW;
+            oh = static_cast<int>(t % p.OH);
+            t /= p.OH;
+            cv = static_cast<int>(t % cvecs);
+            n = t / cvecs;
+        } else {
+            cv = static_cast<int>(t % cvecs);
+            t /= cvecs;
+            ow = static_cast<int>(t % p.OW);
+            t /= p.OW;
+            oh = static_cast<int>(t % p.OH);
+            n = t / p.OH;
+        }
+        const int c0 = cv * VEC;
+        const int h0 = oh * p.sh - p.ph;
+        const int w0 = ow * p.sw - p.pw;
+        const int hs = h0 < 0 ? 0 : h0;
+        const int ws = w0 < 0 ? 0 : w0;
+        const int he = h0 + p.kh < p.H ? h0 + p.kh : p.H;
+        const int we = w0 + p.kw < p.W ? w0 + p.kw : p.W;
+        const T* xb = x + n * p.xsN + static_cast<int64_t>(c0) * p.xsC;
+        PVec<T, VEC> res;
+        if constexpr (IS_MAX) {
+            T acc[VEC];
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) acc[e] = Lowest<T>();
+            for (int ih = hs; ih < he; ++ih) {
+                for (int iw = ws; iw < we; ++iw) {
+                    const T* q = xb + ih * p.xsH + iw * p.xsW;
+                    PVec<T, VEC> v;
+                    if constexpr (VEC > 1) {
+                        v = *reinterpret_cast<const PVec<T, VEC>*>(q);
+                    } else {
+                        v.v[0] = *q;
+                    }
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) {
+                        if (IsNanT(v.v[e]) || acc[e] < v.v[e]) acc[e] = v.v[e];
+                    }
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) res.v[e] = acc[e];
+        } else {
+            C acc[VEC];
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) acc[e] = C(0);
+            for (int ih = hs; ih < he; ++ih) {
+                for (int iw = ws; iw < we; ++iw) {
+                    const T* q = xb + ih * p.xsH + iw * p.xsW;
+                    PVec<T, VEC> v;
+                    if constexpr (VEC > 1) {
+                        v = *reinterpret_cast<const PVec<T, VEC>*>(q);
+                    } else {
+                        v.v[0] = *q;
+                    }
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) acc[e] += static_cast<C>(v.v[e]);
+                }
+            }
+            // divisor in T arithmetic (CX/native/native_device/pool.cc:191-250)
+            C div;
+            if (p.pad_mode == HIPCX_PAD_ZERO) {
+                div = static_cast<C>(static_cast<T>(static_cast<C>(p.kh * p.kw)));
+            } else {
+                int hcnt = (h0 + p.kh < p.H ? h0 + p.kh : p.H) - hs;
+                int wcnt = (w0 + p.kw < p.W ? w0 + p.kw : p.W) - ws;
+                div = static_cast<C>(static_cast<T>(static_cast<C>(hcnt) * static_cast<C>(wcnt)));
+            }
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                T s = static_cast<T>(acc[e]);  // Sum rounds to the array dtype first
+                res.v[e] = static_cast<T>(static_cast<C>(s) / div);
+            }
+        }
+        T* o = out + n * p.osN + static_cast<int64_t>(c0) * p.osC + oh * p.osH + ow * p.osW;
+        if constexpr (VEC > 1) {
+            *reinterpret_cast<PVec<T, VEC>*>(o) = res;
+        } else {
+            *o = res.v[0];
+        }
+    }
+}
+
+int64_t ElemStride(const hipcx_array* a, int axis) {
+    int64_t it = ItemSize(a->dtype);
+    HIPCX_REQUIRE(a->strides[axis] % it == 0, HIPCX_NOT_IMPLEMENTED_ERROR, "byte strides must be multiples of the item size");
+    return a->strides[axis] / it;
+}
+
+bool Aligned(const void* p, int64_t bytes) { return reinterpret_cast<uintptr_t>(p) % bytes == 0; }
+
+template <typename T, bool IS_MAX>
+void RunPool(PoolArgs p, hipStream_t stream) {
+    constexpr int VEC = 16 / sizeof(T);
+    bool vec_ok = p.xsC == 1 && p.osC == 1 && p.C % VEC == 0 && Aligned(p.x, 16) && Aligned(p.out, 16) && p.xsN % VEC == 0 &&
+                  p.xsH % VEC == 0 && p.xsW % VEC == 0 && p.osN % VEC == 0 && p.osH % VEC == 0 && p.osW % VEC == 0;
+    int64_t total = static_cast<int64_t>(p.N) * p.OH * p.OW * (vec_ok ? p.C / VEC : p.C);
+    if (total == 0) return;
+    // thread order follows the output's fastest axis
+    int64_t a_c = p.osC < 0 ? -p.osC : p.osC, a_w = p.osW < 0 ? -p.osW : p.osW;
+    p.w_fastest = (!vec_ok && a_w < a_c) ? 1 : 0;
+    int64_t blocks = (total + 255) / 256;
+    int64_t cap = static_cast<int64_t>(NumCUs()) * 32;
+    if (blocks > cap) blocks = cap;
+    if (vec_ok) {
+        hipLaunchKernelGGL((PoolKernel<T, VEC, IS_MAX>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, p, total);
+    } else {
+        hipLaunchKernelGGL((PoolKernel<T, 1, IS_MAX>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, p, total);
+    }
+    CheckLaunch("pool");
+}
+
+PoolArgs MakeArgs(const hipcx_array* x, const int64_t* ksize, const int64_t* stride, const int64_t* pad, int cover_all,
+                  const hipcx_array* out) {
+    ValidateArray(x, "x");
+    ValidateArray(out, "out");
+    HIPCX_REQUIRE(x->ndim == 4 && out->ndim == 4, HIPCX_NOT_IMPLEMENTED_ERROR, "hip pooling supports 2 spatial dimensions");
+    HIPCX_REQUIRE(x->dtype == out->dtype, HIPCX_DTYPE_ERROR, "out must have x's dtype");
+    HIPCX_REQUIRE(ksize && stride && pad, HIPCX_CHAINERX_ERROR, "null window parameters");
+    HIPCX_REQUIRE(ksize[0] > 0 && ksize[1] > 0 && stride[0] > 0 && stride[1] > 0 && pad[0] >= 0 && pad[1] >= 0, HIPCX_DIMENSION_ERROR,
+                  "invalid kernel size, stride or pad");
+    int64_t oh = hipcx_conv_out_dim(x->shape[2], ksize[0], stride[0], pad[0], cover_all);
+    int64_t ow = hipcx_conv_out_dim(x->shape[3], ksize[1], stride[1], pad[1], cover_all);
+    HIPCX_REQUIRE(oh > 0 && ow > 0, HIPCX_DIMENSION_ERROR, "Output size should be positive.");
+    HIPCX_REQUIRE(out->shape[0] == x->shape[0] && out->shape[1] == x->shape[1] && out->shape[2] == oh && out->shape[3] == ow,
+                  HIPCX_DIMENSION_ERROR, "out has the wrong shape " + ShapeStr(out));
+    for (int i = 0; i < 4; ++i) HIPCX_REQUIRE(x->shape[i] < (1LL << 31), HIPCX_NOT_IMPLEMENTED_ERROR, "extent too large");
+    PoolArgs p{};
+    p.x = x->data;
+    p.out = out->data;
+    p.N = static_cast<int>(x->shape[0]);
+    p.C = static_cast<int>(x->shape[1]);
+    p.H = static_cast<int>(x->shape[2]);
+    p.W = static_cast<int>(x->shape[3]);
+    p.OH = static_cast<int>(oh);
+    p.OW = static_cast<int>(ow);
+    p.kh = static_cast<int>(ksize[0]);
+    p.kw = static_cast<int>(ksize[1]);
+    p.sh = static_cast<int>(stride[0]);
+    p.sw = static_cast<int>(stride[1]);
+    p.ph = static_cast<int>(pad[0]);
+    p.pw = static_cast<int>(pad[1]);
+    p.xsN = ElemStride(x, 0);
+    p.xsC = ElemStride(x, 1);
+    p.xsH = ElemStride(x, 2);
+    p.xsW = ElemStride(x, 3);
+    p.osN = ElemStride(out, 0);
+    p.osC = ElemStride(out, 1);
+    p.osH = ElemStride(out, 2);
+    p.osW = ElemStride(out, 3);
+    p.pad_mode = HIPCX_PAD_ZERO;
+    return p;
+}
+
+}  // namespace
+}  // namespace hipcx
+
+using namespace hipcx;
+
+extern "C" {
+
+int hipcx_max_pool(const hipcx_array* x, const int64_t* kernel_size, const int64_t* stride, const int64_t* pad, int cover_all,
+                   const hipcx_array* out, void* stream) {
+    return Guard([&] {
+        PoolArgs p = MakeArgs(x, kernel_size, stride, pad, cover_all, out);
+        VisitDtype(x->dtype, [&](auto tag) {
+            using T = typename decltype(tag)::type;
+            RunPool<T, true>(p, AsStream(stream));
+        });
+    });
+}
+
+int hipcx_average_pool(const hipcx_array* x, const int64_t* kernel_size, const int64_t* stride, const int64_t* pad, int pad_mode,
+                       const hipcx_array* out, void* stream) {
+    return Guard([&] {
+        HIPCX_REQUIRE(pad_mode == HIPCX_PAD_ZERO || pad_mode == HIPCX_PAD_IGNORE, HIPCX_CHAINERX_ERROR, "invalid pad mode");
+        HIPCX_REQUIRE(x != nullptr && IsFloatDtype(x->dtype), HIPCX_DTYPE_ERROR, "cannot apply average pooling to non-float arrays");
+        PoolArgs p = MakeArgs(x, kernel_size, stride, pad, 0, out);
+        p.pad_mode = pad_mode;
+        VisitFloatDtype(x->dtype, [&](auto tag) {
+            using T = typename decltype(tag)::type;
+            RunPool<T, false>(p, AsStream(stream));
+        });
+    });
+}
+}

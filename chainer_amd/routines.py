@@ -225,13 +225,31 @@ def _broadcast_shape(s1, s2):
     return tuple(out)
 
 
+LAYOUT_FOLLOWS_INPUT = False
+
+
+def _empty_for(x, shape, dtype):
+    """Output allocation of the elementwise routines.  ChainerX routines call Empty(shape): C-contiguous.  With
+    LAYOUT_FOLLOWS_INPUT (opt-in) a dense input's axis order is kept instead, so channels-last data stays channels-last."""
+    if LAYOUT_FOLLOWS_INPUT and isinstance(x, ndarray) and x.shape == tuple(shape) and 0 not in x.strides:
+        dtype = numpy.dtype(dtype)
+        order = sorted(range(x.ndim), key=lambda i: (-abs(x.strides[i]), i))
+        strides = [0] * x.ndim
+        acc = dtype.itemsize
+        for i in reversed(order):
+            strides[i] = acc
+            acc *= _py.max(1, x.shape[i])
+        return ndarray(alloc_bytes(acc), 0, x.shape, strides, dtype)
+    return ndarray.empty(shape, dtype)
+
+
 def _binary(kernel, x1, x2, dtype, out=None):
     """BroadcastBinary (CX/routines/routines_util.h:53-72): operands arrive equal-shaped, cast to out's dtype."""
     shape = _broadcast_shape(x1.shape, x2.shape)
     a = x1 if x1.shape == shape else x1.broadcast_to(shape)
     b = x2 if x2.shape == shape else x2.broadcast_to(shape)
     if out is None:
-        out = ndarray.empty(shape, dtype)
+        out = _empty_for(x1, shape, dtype)
     elif out.shape != shape:
         raise _lib.DimensionError('in-place operand shape %r does not match %r' % (out.shape, shape))
     _lib.call(kernel, a.astype(out.dtype, False).desc(), b.astype(out.dtype, False).desc(), out.desc(), current_stream())
@@ -240,7 +258,7 @@ def _binary(kernel, x1, x2, dtype, out=None):
 
 def _binary_as(kernel, x1, scalar, dtype, out=None):
     if out is None:
-        out = ndarray.empty(x1.shape, dtype)
+        out = _empty_for(x1, x1.shape, dtype)
     _lib.call(kernel, x1.astype(out.dtype, False).desc(), _lib.make_scalar(scalar), out.desc(), current_stream())
     return out
 
@@ -330,7 +348,7 @@ def sqrt(x):
 def if_less_else(x1, x2, pos, neg):
     """x1 < x2 ? pos : neg with scalar x2/pos (CX/routines/misc.cc:34-58)."""
     dt = result_type(pos, neg)
-    out = ndarray.empty(x1.shape, dt)
+    out = _empty_for(x1, x1.shape, dt)
     _lib.call('hipcx_if_less_else_assa', x1.astype(dt, False).desc(), _lib.make_scalar(x2), _lib.make_scalar(pos),
               neg.astype(dt, False).desc(), out.desc(), current_stream())
     return out
@@ -590,10 +608,23 @@ def conv_out_dim(in_dim, kernel_size, stride, pad, cover_all):
 
 
 def _channels_last_empty(n, c, h, w, dtype):
-    """NCHW-shaped array over NHWC memory: what the hip ConvKernel / pooling kernels return."""
+    """NCHW-shaped array over NHWC memory (the layout the native backend's own conv result has)."""
     it = numpy.dtype(dtype).itemsize
     strides = (h * w * c * it, it, w * c * it, c * it)
     return ndarray(alloc_bytes(n * c * h * w * it), 0, (n, c, h, w), strides, dtype)
+
+
+def _is_channels_last(x):
+    return x.ndim == 4 and x.strides[1] == x.itemsize and x.shape[1] > 1 and (x.shape[2] * x.shape[3] > 1)
+
+
+def _spatial_out(x, n, c, h, w, dtype):
+    """Output of the kernels that allocate their own result (Conv, MaxPool, AveragePool).  C-contiguous NCHW, like the
+    CUDA backend's (CX/cuda/cuda_conv.cc:311); channels-last when the opt-in LAYOUT_FOLLOWS_INPUT mode is on and the
+    input already is."""
+    if LAYOUT_FOLLOWS_INPUT and (_is_channels_last(x) or x.shape[1] < 8):
+        return _channels_last_empty(n, c, h, w, dtype)
+    return ndarray.empty((n, c, h, w), dtype)
 
 
 def conv(x, w, b=None, stride=1, pad=0, cover_all=False, out_dtype=None):
@@ -608,7 +639,7 @@ def conv(x, w, b=None, stride=1, pad=0, cover_all=False, out_dtype=None):
     dt = numpy.dtype(out_dtype) if out_dtype is not None else (result_type(x, w, b) if b is not None else result_type(x, w))
     oh = conv_out_dim(x.shape[2], w.shape[2], stride[0], pad[0], cover_all)
     ow = conv_out_dim(x.shape[3], w.shape[3], stride[1], pad[1], cover_all)
-    out = _channels_last_empty(x.shape[0], w.shape[0], oh, ow, dt)
+    out = _spatial_out(x, x.shape[0], w.shape[0], oh, ow, dt)
     xc, wc = x.astype(dt, False), w.astype(dt, False)
     bc = b.astype(dt, False) if b is not None else None
     nbytes = _lib.load().hipcx_conv_workspace_size(xc.desc(), wc.desc(), out.desc())
@@ -658,7 +689,7 @@ def max_pool(x, ksize, stride=None, pad=0, cover_all=False):
     pad = _pair(pad)
     oh = conv_out_dim(x.shape[2], ksize[0], stride[0], pad[0], cover_all)
     ow = conv_out_dim(x.shape[3], ksize[1], stride[1], pad[1], cover_all)
-    out = _channels_last_empty(x.shape[0], x.shape[1], oh, ow, x.dtype)
+    out = _spatial_out(x, x.shape[0], x.shape[1], oh, ow, x.dtype)
     _lib.call('hipcx_max_pool', x.desc(), _i64(ksize), _i64(stride), _i64(pad), int(bool(cover_all)), out.desc(), current_stream())
     return out
 
@@ -675,7 +706,7 @@ def average_pool(x, ksize, stride=None, pad=0, pad_mode='ignore'):
     mode = {'zero': 1, 'ignore': 2}[pad_mode]
     oh = conv_out_dim(x.shape[2], ksize[0], stride[0], pad[0], False)
     ow = conv_out_dim(x.shape[3], ksize[1], stride[1], pad[1], False)
-    out = _channels_last_empty(x.shape[0], x.shape[1], oh, ow, x.dtype)
+    out = _spatial_out(x, x.shape[0], x.shape[1], oh, ow, x.dtype)
     _lib.call('hipcx_average_pool', x.desc(), _i64(ksize), _i64(stride), _i64(pad), mode, out.desc(), current_stream())
     return out
 

@@ -157,6 +157,13 @@ size_t hipcx_conv_workspace_size(const hipcx_array* x, const hipcx_array* w, con
 int hipcx_conv(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, const int64_t* stride, const int64_t* pad,
                int cover_all, const hipcx_array* out, void* workspace, size_t workspace_bytes, void* stream);
 
+/* Measurement aid (no counterpart in the reference): between start and stop every implicit-GEMM launch made by
+ * hipcx_dot / hipcx_conv from the calling process is bracketed by a pair of HIP events on its stream.  stop waits for them
+ * and returns the number of launches, the sum of their durations, and their algorithmic flops (2 per multiply-add) and
+ * bytes (each operand once).  Not thread-safe; one profiling window at a time. */
+int hipcx_profile_start(void);
+int hipcx_profile_stop(int64_t* launches, double* total_ms, double* flops, double* bytes);
+
 /* ---- normalization: FixedBatchNormKernel CX/kernels/normalization.h:107 ----
  * gamma/beta/mean/var have the keep-dims reduced shape of x over `axis`
  * (CX/routines/normalization.cc:61-101). out has x's shape and dtype. */

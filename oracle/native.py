@@ -1,0 +1,475 @@
+"""Parity oracle: the ChainerX *native* (CPU) backend restated with numpy + ``liboracle.so``.
+
+TEST INFRASTRUCTURE ONLY.  Importers: ``tests/``, ``__graft_entry__.smoke()`` and the
+``cpu_baseline`` leg of ``bench.py``.  The product package ``chainer_amd`` never imports this.
+
+Each function follows the reference routine + native kernel named in its docstring (paths relative
+to the reference tree, ``CX/`` = ``chainerx_cc/chainerx/``), including the order of floating point
+operations wherever the native backend fixes one: every elementwise op rounds to the array dtype
+(float16 through float32, as ``chainerx::Float16`` does), reductions use the native pairwise tree,
+Dot/Conv accumulate with one fused multiply-add per term in (i, l, j) order.
+
+How each function is pinned (golden vectors of the reference's own tests, closed forms, brute
+force) is recorded in ``tests/test_oracle_pins.py``; functions whose bit pattern only a compiled
+reference run could pin say "parity unpinned (bit level)" below -- their tolerance-level behaviour
+is still pinned.
+"""
+import ctypes
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, 'liboracle.so')
+_lib = None
+
+_f32p = ctypes.POINTER(ctypes.c_float)
+_f64p = ctypes.POINTER(ctypes.c_double)
+_i64p = ctypes.POINTER(ctypes.c_int64)
+_u16p = ctypes.POINTER(ctypes.c_uint16)
+_i64 = ctypes.c_int64
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            raise ImportError('oracle/liboracle.so is not built: run `make -C oracle`')
+        _lib = ctypes.CDLL(_LIB_PATH)
+    return _lib
+
+
+def _ptr(a, ctype):
+    return a.ctypes.data_as(ctype)
+
+
+def _c(a, dtype=None):
+    return np.ascontiguousarray(a, dtype=dtype)
+
+
+# ---------------------------------------------------------------------------------------------
+# float16 (CX/float16.cc:27-89,161-193)
+# ---------------------------------------------------------------------------------------------
+def float_to_half_bits(x):
+    x = _c(x, np.float32)
+    out = np.empty(x.shape, np.uint16)
+    lib().oracle_float_to_half(_ptr(x, _f32p), _ptr(out, _u16p), _i64(x.size))
+    return out
+
+
+def half_bits_to_float(h):
+    h = _c(h, np.uint16)
+    out = np.empty(h.shape, np.float32)
+    lib().oracle_half_to_float(_ptr(h, _u16p), _ptr(out, _f32p), _i64(h.size))
+    return out
+
+
+# ---------------------------------------------------------------------------------------------
+# elementwise (CX/native/native_device/{arithmetic,exp_log,hyperbolic,misc,logic,copy,fill}.cc)
+# numpy applies exactly one IEEE rounding per operation in the array dtype, float16 via float32,
+# which is the native functors' arithmetic (CX/arithmetic_ops.h:7-25, CX/float16.h operators).
+# ---------------------------------------------------------------------------------------------
+def astype(x, dtype):
+    """CopyKernel: static_cast<Out>(in) (copy.cc:21-35)."""
+    with np.errstate(all='ignore'):
+        return np.asarray(x).astype(dtype)
+
+
+def _scalar_as(value, dtype):
+    return np.asarray(value).astype(dtype)[()]
+
+
+def add(x1, x2):
+    x1, x2 = np.asarray(x1), np.asarray(x2)
+    if x1.dtype == np.bool_ and x2.dtype == np.bool_:
+        return x1 | x2
+    with np.errstate(all='ignore'):
+        return x1 + x2
+
+
+def subtract(x1, x2):
+    with np.errstate(all='ignore'):
+        return np.asarray(x1) - np.asarray(x2)
+
+
+def multiply(x1, x2):
+    x1, x2 = np.asarray(x1), np.asarray(x2)
+    if x1.dtype == np.bool_ and x2.dtype == np.bool_:
+        return x1 & x2
+    with np.errstate(all='ignore'):
+        return x1 * x2
+
+
+def divide(x1, x2):
+    """DivideKernel on floats (routine TrueDivide casts ints to float32 first, CX/routines/arithmetic.cc:395-417)."""
+    x1, x2 = np.asarray(x1), np.asarray(x2)
+    with np.errstate(all='ignore'):
+        return x1 / x2
+
+
+def exp(x):
+    with np.errstate(all='ignore'):
+        return np.exp(x)
+
+
+def log(x):
+    with np.errstate(all='ignore'):
+        return np.log(x)
+
+
+def tanh(x):
+    return np.tanh(x)
+
+
+def sqrt(x):
+    with np.errstate(all='ignore'):
+        return np.sqrt(x)
+
+
+def if_less_else(x1, x2, pos, neg):
+    """x1 < x2 ? pos : neg (misc.cc:39-61); x2 and pos are scalars cast to the dtype."""
+    x1 = np.asarray(x1)
+    dt = np.asarray(neg).dtype
+    return np.where(x1 < _scalar_as(x2, dt), _scalar_as(pos, dt), neg).astype(dt)
+
+
+def relu(x):
+    """Relu = Maximum(0, x) = IfLessElse(x, 0, 0, x) (CX/routines/activation.cc:80-84, misc.cc:210-216)."""
+    return if_less_else(x, 0, 0, x)
+
+
+def sigmoid(x):
+    """Reciprocal(1 + Exp(-x)) as four kernels: MultiplyAS(-1), Exp, AddAS(1), DivideSA(1) (activation.cc:74-78)."""
+    x = np.asarray(x)
+    one = _scalar_as(1, x.dtype)
+    with np.errstate(all='ignore'):
+        neg = x * _scalar_as(-1, x.dtype)
+        e = np.exp(neg)
+        return one / (e + one)
+
+
+def equal(x1, x2):
+    return np.asarray(x1) == np.asarray(x2)
+
+
+# ---------------------------------------------------------------------------------------------
+# reductions (CX/native/reduce.h:46-83 order)
+# ---------------------------------------------------------------------------------------------
+def _rows(a, axes):
+    """Moves the reduced axes last (kept in their own order: the native iterator walks the reduced axes in C order,
+    CX/reduction_kernel_arg.cc:19-144) and flattens to [n_out, reduce_len]."""
+    a = np.asarray(a)
+    axes = tuple(sorted(ax % a.ndim for ax in axes))
+    keep = [i for i in range(a.ndim) if i not in axes]
+    t = a.transpose(keep + list(axes))
+    out_shape = tuple(a.shape[i] for i in keep)
+    red = int(np.prod([a.shape[i] for i in axes], dtype=np.int64)) if axes else 1
+    return np.ascontiguousarray(t).reshape(-1, red), out_shape, axes
+
+
+def _axes_of(a, axis):
+    if axis is None:
+        return tuple(range(np.asarray(a).ndim))
+    if isinstance(axis, (int, np.integer)):
+        return (int(axis),)
+    return tuple(axis)
+
+
+def _restore(out, out_shape, a, axes, keepdims):
+    out = out.reshape(out_shape)
+    if keepdims:
+        shape = [1 if i in axes else d for i, d in enumerate(np.asarray(a).shape)]
+        out = out.reshape(shape)
+    return out
+
+
+def sum(a, axis=None, keepdims=False):
+    """NativeSumKernel (reduction.cc:96-119): int/bool inputs accumulate in int64 (CX/routines/reduction.cc:34-49),
+    float16 accumulates in float32 and rounds once, float32/64 accumulate in their own type, pairwise order.
+    parity unpinned (bit level) for float data: the order is derived from the source; integer-valued data pins it exactly."""
+    a = np.asarray(a)
+    rows, out_shape, axes = _rows(a, _axes_of(a, axis))
+    n, length = rows.shape
+    L = lib()
+    if a.dtype.kind in 'biu':
+        r = _c(rows, np.int64)
+        out = np.empty(n, np.int64)
+        L.oracle_sum_i64(_ptr(r, _i64p), _i64(n), _i64(length), _ptr(out, _i64p))
+    elif a.dtype == np.float32:
+        out = np.empty(n, np.float32)
+        L.oracle_sum_f32(_ptr(rows, _f32p), _i64(n), _i64(length), _ptr(out, _f32p))
+    elif a.dtype == np.float64:
+        out = np.empty(n, np.float64)
+        L.oracle_sum_f64(_ptr(rows, _f64p), _i64(n), _i64(length), _ptr(out, _f64p))
+    elif a.dtype == np.float16:
+        bits = rows.view(np.uint16)
+        ob = np.empty(n, np.uint16)
+        L.oracle_sum_f16(_ptr(bits, _u16p), _i64(n), _i64(length), _ptr(ob, _u16p))
+        out = ob.view(np.float16)
+    else:
+        raise TypeError(a.dtype)
+    return _restore(out, out_shape, a, axes, keepdims)
+
+
+def amax(a, axis=None, keepdims=False):
+    """NativeAMaxKernel (statistics.cc:27-48): NaN-propagating maximum, identity lowest / -inf."""
+    a = np.asarray(a)
+    rows, out_shape, axes = _rows(a, _axes_of(a, axis))
+    n, length = rows.shape
+    L = lib()
+    if a.dtype.kind == 'f' and a.dtype != np.float64:
+        r = _c(rows, np.float32)  # float16 -> float32 is exact and order preserving
+        out = np.empty(n, np.float32)
+        L.oracle_amax_f32(_ptr(r, _f32p), _i64(n), _i64(length), _ptr(out, _f32p))
+        out = out.astype(a.dtype)
+    elif a.dtype == np.float64:
+        out = np.empty(n, np.float64)
+        L.oracle_amax_f64(_ptr(rows, _f64p), _i64(n), _i64(length), _ptr(out, _f64p))
+    else:
+        r = _c(rows, np.int64)
+        lowest = 0 if a.dtype.kind in 'bu' else int(np.iinfo(a.dtype).min)
+        out = np.empty(n, np.int64)
+        L.oracle_amax_i64(_ptr(r, _i64p), _i64(n), _i64(length), _i64(lowest), _ptr(out, _i64p))
+        out = out.astype(a.dtype)
+    return _restore(out, out_shape, a, axes, keepdims)
+
+
+def argmax(a, axis=None):
+    """NativeArgMaxKernel (reduction.cc:34-61) through the pairwise tree: the earlier index wins a tie inside a
+    32-element block (and in the tail), the later block wins a tie between blocks; NaN never replaces and a leading
+    NaN is never replaced.  The index counts positions in the C-order flattening of the reduced axes."""
+    a = np.asarray(a)
+    rows, out_shape, axes = _rows(a, _axes_of(a, axis))
+    n, length = rows.shape
+    r = _c(rows, np.float64)
+    out = np.empty(n, np.int64)
+    lib().oracle_argmax(_ptr(r, _f64p), _i64(n), _i64(length), _ptr(out, _i64p))
+    return out.reshape(out_shape)
+
+
+def mean(a, axis=None, keepdims=False):
+    """Mean = SumKernel into the float result dtype, then DivideASKernel by the count (CX/routines/statistics.cc:95-154)."""
+    a = np.asarray(a)
+    dt = a.dtype if a.dtype.kind == 'f' else np.dtype(np.float32)
+    axes = _axes_of(a, axis)
+    n = int(np.prod([a.shape[i] for i in axes], dtype=np.int64))
+    s = sum(a.astype(dt), axis, keepdims)
+    return (s / _scalar_as(n, dt)).astype(dt)
+
+
+def logsumexp(x, axis=None, keepdims=False):
+    """CX/routines/reduction.cc:78-86."""
+    x = np.asarray(x)
+    axes = _axes_of(x, axis)
+    xmax = amax(x, axes, True)
+    logs = log(sum(exp(subtract(x, xmax)), axes, keepdims))
+    return add(xmax if keepdims else xmax.reshape(logs.shape), logs)
+
+
+def log_softmax(x, axis=None):
+    """x - LogSumExp(x, axis or 1, keepdims=True) (CX/routines/reduction.cc:88-92)."""
+    x = np.asarray(x)
+    return subtract(x, logsumexp(x, 1 if axis is None else axis, True))
+
+
+# ---------------------------------------------------------------------------------------------
+# dot / linear / conv
+# ---------------------------------------------------------------------------------------------
+def dot(a, b):
+    """NativeDotKernel without BLAS (dot.cc:181-227).  parity unpinned (bit level): exact fp32 bit patterns follow the
+    (i, l, j) fmaf order read from the source; the reference's literal vectors and integer-valued matrices pin the rest."""
+    a, b = np.asarray(a), np.asarray(b)
+    assert a.ndim == 2 and b.ndim == 2 and a.shape[1] == b.shape[0] and a.dtype == b.dtype
+    m, k = a.shape
+    n = b.shape[1]
+    L = lib()
+    ac, bc = _c(a), _c(b)
+    if a.dtype == np.float32:
+        out = np.empty((m, n), np.float32)
+        L.oracle_dot_f32(_ptr(ac, _f32p), _ptr(bc, _f32p), _ptr(out, _f32p), _i64(m), _i64(k), _i64(n))
+    elif a.dtype == np.float64:
+        out = np.empty((m, n), np.float64)
+        L.oracle_dot_f64(_ptr(ac, _f64p), _ptr(bc, _f64p), _ptr(out, _f64p), _i64(m), _i64(k), _i64(n))
+    elif a.dtype == np.float16:
+        ob = np.empty((m, n), np.uint16)
+        rc = L.oracle_dot_f16(_ptr(ac.view(np.uint16), _u16p), _ptr(bc.view(np.uint16), _u16p), _ptr(ob, _u16p), _i64(m), _i64(k), _i64(n))
+        assert rc == 0
+        out = ob.view(np.float16)
+    else:
+        raise TypeError(a.dtype)
+    return out
+
+
+def linear(x, w, b=None):
+    """Linear (CX/routines/connection.cc:322-394): Dot(x, w.T) then AddKernel with the broadcast bias."""
+    x, w = np.asarray(x), np.asarray(w)
+    x2 = x.reshape(x.shape[0], -1)
+    y = dot(x2, np.ascontiguousarray(w.T))
+    if b is not None:
+        y = add(y, np.broadcast_to(b, y.shape))
+    return y
+
+
+def conv_out_dim(in_dim, k, s, p, cover_all):
+    """GetConvOutDim (CX/routines/connection.cc:37-49)."""
+    num = in_dim + 2 * p - k + (s - 1 if cover_all else 0)
+    if num < 0:
+        raise ValueError('Output size should be positive.')
+    return num // s + 1
+
+
+def _pair(v):
+    return (int(v), int(v)) if isinstance(v, (int, np.integer)) else (int(v[0]), int(v[1]))
+
+
+def conv(x, w, b=None, stride=1, pad=0, cover_all=False):
+    """NativeConvKernel (conv.cc:41-89); returns contiguous NCHW values."""
+    x, w = np.asarray(x), np.asarray(w)
+    assert x.dtype == w.dtype
+    N, C, H, W = x.shape
+    K, C2, R, S = w.shape
+    assert C == C2
+    sh, sw = _pair(stride)
+    ph, pw = _pair(pad)
+    OH = conv_out_dim(H, R, sh, ph, cover_all)
+    OW = conv_out_dim(W, S, sw, pw, cover_all)
+    L = lib()
+    xc, wc = _c(x), _c(w)
+    bc = _c(b, x.dtype) if b is not None else None
+    args = [_i64(v) for v in (N, C, H, W, K, R, S, sh, sw, ph, pw, OH, OW)]
+    if x.dtype == np.float32:
+        out = np.empty((N, K, OH, OW), np.float32)
+        rc = L.oracle_conv_f32(_ptr(xc, _f32p), _ptr(wc, _f32p), _ptr(bc, _f32p) if bc is not None else None, _ptr(out, _f32p), *args)
+    elif x.dtype == np.float64:
+        out = np.empty((N, K, OH, OW), np.float64)
+        rc = L.oracle_conv_f64(_ptr(xc, _f64p), _ptr(wc, _f64p), _ptr(bc, _f64p) if bc is not None else None, _ptr(out, _f64p), *args)
+    elif x.dtype == np.float16:
+        ob = np.empty((N, K, OH, OW), np.uint16)
+        rc = L.oracle_conv_f16(_ptr(xc.view(np.uint16), _u16p), _ptr(wc.view(np.uint16), _u16p),
+                               _ptr(bc.view(np.uint16), _u16p) if bc is not None else None, _ptr(ob, _u16p), *args)
+        out = ob.view(np.float16)
+    else:
+        raise TypeError(x.dtype)
+    assert rc == 0
+    return out
+
+
+# ---------------------------------------------------------------------------------------------
+# normalization / pooling / indexing
+# ---------------------------------------------------------------------------------------------
+def fixed_batch_norm(x, gamma, beta, mean, var, eps=2e-5, axis=None):
+    """GenericFixedBatchNormKernel (CX/routines/normalization.cc:251-264 -> ApplyGenericBatchNorm :113-153):
+    interm dtype = promotion of the five operands; inv_std = 1 / sqrt(var + eps);
+    out = ((x - mean) * inv_std) * gamma + beta, one rounding per operation in the interm dtype, cast back to x's."""
+    x = np.asarray(x)
+    axes = (0,) if axis is None else tuple(sorted(_axes_of(x, axis)))
+    red_shape = tuple(1 if i in axes else d for i, d in enumerate(x.shape))
+    dt = np.result_type(x.dtype, *[np.asarray(p).dtype for p in (gamma, beta, mean, var)])
+    g, b, m, v = [np.asarray(p).reshape(red_shape).astype(dt) for p in (gamma, beta, mean, var)]
+    xc = x.astype(dt)
+    with np.errstate(all='ignore'):
+        inv_std = _scalar_as(1, dt) / np.sqrt(v + _scalar_as(eps, dt))
+        out = (xc - m) * inv_std * g + b
+    return out.astype(x.dtype)
+
+
+def _windows(x, ksize, stride, pad, cover_all, pad_value):
+    """Im2Col (CX/native/im2col.cc:82-149): [N,C,kh,kw,OH,OW] with `pad_value` outside the image."""
+    N, C, H, W = x.shape
+    kh, kw = ksize
+    sh, sw = stride
+    ph, pw = pad
+    OH = conv_out_dim(H, kh, sh, ph, cover_all)
+    OW = conv_out_dim(W, kw, sw, pw, cover_all)
+    eh = sh - 1 if cover_all else 0
+    ew = sw - 1 if cover_all else 0
+    padded = np.full((N, C, H + 2 * ph + eh, W + 2 * pw + ew), pad_value, x.dtype)
+    padded[:, :, ph:ph + H, pw:pw + W] = x
+    col = np.empty((N, C, kh, kw, OH, OW), x.dtype)
+    for r in range(kh):
+        for s in range(kw):
+            col[:, :, r, s] = padded[:, :, r:r + sh * OH:sh, s:s + sw * OW:sw]
+    return col
+
+
+def _lowest(dtype):
+    dtype = np.dtype(dtype)
+    if dtype.kind == 'f':
+        return -np.inf
+    if dtype.kind == 'b':
+        return False
+    return np.iinfo(dtype).min
+
+
+def max_pool(x, ksize, stride=None, pad=0, cover_all=False):
+    """NativeMaxPoolKernel (pool.cc:69-94): Im2Col padded with lowest/-inf, then AMax over the window axes."""
+    x = np.asarray(x)
+    ksize = _pair(ksize)
+    stride = ksize if stride is None else _pair(stride)
+    col = _windows(x, ksize, stride, _pair(pad), cover_all, _lowest(x.dtype))
+    return amax(col, (2, 3))
+
+
+def average_pool(x, ksize, stride=None, pad=0, pad_mode='ignore'):
+    """NativeAveragePoolKernel (pool.cc:252-302): zero-padded Im2Col, SumKernel over the window, then DivideAS by the
+    window size ('zero') or Divide by the per-position count of in-image taps ('ignore', :197-250)."""
+    x = np.asarray(x)
+    ksize = _pair(ksize)
+    stride = ksize if stride is None else _pair(stride)
+    pad = _pair(pad)
+    col = _windows(x, ksize, stride, pad, False, 0)
+    s = sum(col, (2, 3))
+    if pad_mode == 'zero':
+        with np.errstate(all='ignore'):
+            return (s / _scalar_as(ksize[0] * ksize[1], x.dtype)).astype(x.dtype)
+    widths = None
+    for i in range(2):
+        d, k, st, p = x.shape[2 + i], ksize[i], stride[i], pad[i]
+        n_out = conv_out_dim(d, k, st, p, False)
+        start = np.arange(n_out).astype(x.dtype) * _scalar_as(st, x.dtype) - _scalar_as(p, x.dtype)
+        end = start + _scalar_as(k, x.dtype)
+        w = (np.minimum(end, _scalar_as(d, x.dtype)) - np.maximum(start, _scalar_as(0, x.dtype))).astype(x.dtype)
+        widths = w if widths is None else (widths[:, None] * w[None, :]).astype(x.dtype)
+    with np.errstate(all='ignore'):
+        return (s / widths).astype(x.dtype)
+
+
+def take(a, indices, axis, mode=None):
+    """NativeTakeKernel (indexing.cc:31-103): mode None/'raise' raise IndexError when out of range."""
+    a = np.asarray(a)
+    idx = np.asarray(indices).astype(np.int64)
+    dim = a.shape[axis]
+    if mode in (None, 'raise'):
+        if ((idx < -dim) | (idx >= dim)).any():
+            raise IndexError('Index is out of bounds for axis %d with size %d' % (axis, dim))
+        idx = np.where(idx < 0, idx + dim, idx)
+    elif mode == 'wrap':
+        idx = np.where(idx < 0, dim - ((-idx + dim - 1) % dim + 1), idx % dim)
+    elif mode == 'clip':
+        idx = np.clip(idx, 0, dim - 1)
+    else:
+        raise ValueError(mode)
+    return np.take(a, idx, axis=axis)
+
+
+def lstm(c, x):
+    """Lstm (CX/routines/connection.cc:396-446): gate k of unit j sits at column 4j+k."""
+    c, x = np.asarray(c), np.asarray(x)
+    g = x.reshape(x.shape[0], x.shape[1] // 4, 4)
+    a = tanh(g[:, :, 0])
+    i = sigmoid(g[:, :, 1])
+    f = sigmoid(g[:, :, 2])
+    o = sigmoid(g[:, :, 3])
+    new_c = add(multiply(a, i), multiply(f, c))
+    h = multiply(o, tanh(new_c))
+    return h, new_c
+
+
+def softmax_cross_entropy(x, t):
+    """chainer/functions/loss/softmax_cross_entropy.py:123-130 (reduce='mean', normalize=True)."""
+    x, t = np.asarray(x), np.asarray(t)
+    score = log_softmax(x, 1)
+    mask = (t[:, None] == np.arange(score.shape[1], dtype=t.dtype)).astype(score.dtype)
+    num = sum(multiply(score, mask))
+    den = sum(mask)
+    return multiply(num, divide(_scalar_as(-1, score.dtype), den))
