@@ -76,34 +76,62 @@ __global__ __launch_bounds__(256) void BnChannelsLastKernel(const T* __restrict_
     }
 }
 
-// ---- channels-first: x, out = [rows = N*C, L] dense rows; row r uses channel r % C ----
+// ---- channels-first: x, out dense [N*C rows, L]; row r uses channel r % C ----
+// The array is walked as one flat run of 16-byte vectors, whatever L is.  A block covers kSpan
+// consecutive elements, i.e. a handful of rows: it first derives (mean, inv_std, gamma, beta) for
+// those rows into LDS, one row per thread, then every element looks its row's parameters up there.
+constexpr int kBnFlatThreads = 256;
+constexpr int kBnFlatUnroll = 4;
+
 template <typename T, int VEC>
-__global__ __launch_bounds__(256) void BnChannelsFirstKernel(const T* __restrict__ x, T* __restrict__ out, const T* __restrict__ gamma,
-                                                             const T* __restrict__ beta, const T* __restrict__ mean,
-                                                             const T* __restrict__ var, compute_t<T> eps, int C_, int64_t L,
-                                                             int64_t pstride) {
+__global__ __launch_bounds__(kBnFlatThreads) void BnChannelsFirstKernel(const T* __restrict__ x, T* __restrict__ out,
+                                                                        const T* __restrict__ gamma, const T* __restrict__ beta,
+                                                                        const T* __restrict__ mean, const T* __restrict__ var,
+                                                                        compute_t<T> eps, int C_, int64_t L, int64_t pstride,
+                                                                        int64_t total, int max_rows) {
     using C = compute_t<T>;
-    const int64_t row = blockIdx.y;
-    const int ch = static_cast<int>(row % C_);
-    const C m = static_cast<C>(mean[ch * pstride]);
-    const C is = InvStd<C>(static_cast<C>(var[ch * pstride]), eps);
-    const C g = static_cast<C>(gamma[ch * pstride]);
-    const C b = static_cast<C>(beta[ch * pstride]);
-    const T* xr = x + row * L;
-    T* orow = out + row * L;
-    const int64_t lvecs = L / VEC;
-    for (int64_t v = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; v < lvecs; v += static_cast<int64_t>(gridDim.x) * blockDim.x) {
-        Vec<T, VEC> in = *reinterpret_cast<const Vec<T, VEC>*>(xr + v * VEC);
+    constexpr int64_t kSpan = static_cast<int64_t>(kBnFlatThreads) * kBnFlatUnroll * VEC;
+    extern __shared__ __align__(16) char bn_lds[];
+    C* prm = reinterpret_cast<C*>(bn_lds);  // [max_rows][4]
+    const int64_t e0 = static_cast<int64_t>(blockIdx.x) * kSpan;
+    const int64_t row_first = e0 / L;
+    for (int r = threadIdx.x; r < max_rows; r += kBnFlatThreads) {
+        int ch = static_cast<int>((row_first + r) % C_);
+        prm[r * 4 + 0] = static_cast<C>(mean[ch * pstride]);
+        prm[r * 4 + 1] = InvStd<C>(static_cast<C>(var[ch * pstride]), eps);
+        prm[r * 4 + 2] = static_cast<C>(gamma[ch * pstride]);
+        prm[r * 4 + 3] = static_cast<C>(beta[ch * pstride]);
+    }
+    __syncthreads();
+    Vec<T, VEC> in[kBnFlatUnroll];
+    int64_t idx[kBnFlatUnroll];
+#pragma unroll
+    for (int u = 0; u < kBnFlatUnroll; ++u) {
+        idx[u] = e0 + (static_cast<int64_t>(u) * kBnFlatThreads + threadIdx.x) * VEC;
+        if (idx[u] < total) in[u] = *reinterpret_cast<const Vec<T, VEC>*>(x + idx[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < kBnFlatUnroll; ++u) {
+        if (idx[u] >= total) continue;
+        int64_t row = idx[u] / L;
+        int col = static_cast<int>(idx[u] - row * L);
+        int r = static_cast<int>(row - row_first);
         Vec<T, VEC> o;
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
-            C t = static_cast<C>(in.v[e]) - m;
-            t = t * is;
-            t = t * g;
-            t = t + b;
+            if (col >= L) {  // the vector crosses into the next row(s)
+                col -= static_cast<int>(L);
+                ++r;
+            }
+            const C* q = prm + r * 4;
+            C t = static_cast<C>(in[u].v[e]) - q[0];
+            t = t * q[1];
+            t = t * q[2];
+            t = t + q[3];
             o.v[e] = static_cast<T>(t);
+            ++col;
         }
-        *reinterpret_cast<Vec<T, VEC>*>(orow + v * VEC) = o;
+        *reinterpret_cast<Vec<T, VEC>*>(out + idx[u]) = o;
     }
 }
 
@@ -155,7 +183,7 @@ void RunBn(const hipcx_array* x, const hipcx_array* const params[4], hipcx_scala
     const T* g = reinterpret_cast<const T*>(p.ptr[2]);
     const T* b = reinterpret_cast<const T*>(p.ptr[3]);
     const T* m = reinterpret_cast<const T*>(p.ptr[4]);
-    const T* v = reinterpret_cast<const T*>(p.ptr[5]);
+    const T* v_ = reinterpret_cast<const T*>(p.ptr[5]);
 
     // channels-last: [P, C] with parameters (0, it); a single pixel row gives ndim == 1.
     if (p.ndim <= 2 && p.ndim >= 1) {
@@ -184,7 +212,7 @@ void RunBn(const hipcx_array* x, const hipcx_array* const params[4], hipcx_scala
             int64_t cap = static_cast<int64_t>(NumCUs()) * 16 / gy + 1;
             int gx = static_cast<int>(want < cap ? want : cap);
             if (gx < 1) gx = 1;
-            hipLaunchKernelGGL((BnChannelsLastKernel<T, VEC>), dim3(gx, gy), dim3(threads), 0, stream, xp, op, g, b, m, v, eps, P, cvecs,
+            hipLaunchKernelGGL((BnChannelsLastKernel<T, VEC>), dim3(gx, gy), dim3(threads), 0, stream, xp, op, g, b, m, v_, eps, P, cvecs,
                                x_row, o_row, tpb_c, tpb_p);
             CheckLaunch("fixed_batch_norm(channels-last)");
             return;
@@ -200,22 +228,24 @@ void RunBn(const hipcx_array* x, const hipcx_array* const params[4], hipcx_scala
         for (int i = 2; i < 6; ++i) {
             ok = ok && p.strides[i][li] == 0 && p.strides[i][ci] == ps && (p.ndim == 2 || p.strides[i][0] == 0);
         }
-        ok = ok && ps % it == 0 && Nn * Cn < 65536 * 32767LL;
+        ok = ok && ps % it == 0 && Cn < (1LL << 31);
         if (ok) {
-            bool vec_ok = L % VEC == 0 && Aligned(xp, 16) && Aligned(op, 16);
-            int64_t rows = Nn * Cn;
-            // gridDim.y is limited to 65535: fold the excess into a loop-free split is not needed for the shapes met here
-            if (rows <= 65535) {
-                int64_t lv = vec_ok ? L / VEC : L;
-                int gx = static_cast<int>((lv + 255) / 256);
-                if (gx > 64) gx = 64;
-                if (gx < 1) gx = 1;
+            int64_t total = Nn * Cn * L;
+            bool vec_ok = total % VEC == 0 && Aligned(xp, 16) && Aligned(op, 16);
+            int v = vec_ok ? VEC : 1;
+            int64_t span = static_cast<int64_t>(kBnFlatThreads) * kBnFlatUnroll * v;
+            int64_t max_rows = span / L + 2;  // rows a span can touch
+            int64_t lds = max_rows * 4 * static_cast<int64_t>(sizeof(C));
+            int64_t blocks = (total + span - 1) / span;
+            if (lds <= 48 * 1024 && blocks < (1LL << 31)) {
                 if (vec_ok) {
-                    hipLaunchKernelGGL((BnChannelsFirstKernel<T, VEC>), dim3(gx, static_cast<unsigned>(rows)), dim3(256), 0, stream, xp, op,
-                                       g, b, m, v, eps, static_cast<int>(Cn), L, ps / it);
+                    hipLaunchKernelGGL((BnChannelsFirstKernel<T, VEC>), dim3(static_cast<unsigned>(blocks)), dim3(kBnFlatThreads),
+                                       static_cast<size_t>(lds), stream, xp, op, g, b, m, v_, eps, static_cast<int>(Cn), L, ps / it, total,
+                                       static_cast<int>(max_rows));
                 } else {
-                    hipLaunchKernelGGL((BnChannelsFirstKernel<T, 1>), dim3(gx, static_cast<unsigned>(rows)), dim3(256), 0, stream, xp, op, g,
-                                       b, m, v, eps, static_cast<int>(Cn), L, ps / it);
+                    hipLaunchKernelGGL((BnChannelsFirstKernel<T, 1>), dim3(static_cast<unsigned>(blocks)), dim3(kBnFlatThreads),
+                                       static_cast<size_t>(lds), stream, xp, op, g, b, m, v_, eps, static_cast<int>(Cn), L, ps / it, total,
+                                       static_cast<int>(max_rows));
                 }
                 CheckLaunch("fixed_batch_norm(channels-first)");
                 return;

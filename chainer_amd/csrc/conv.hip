@@ -2,10 +2,12 @@
 // implicit-GEMM core.  The arithmetic contract is the native backend's: products of the stored
 // values accumulated in fp32 (fp64 for float64) and rounded once to the output dtype
 // (CX/native/native_device/dot.cc:181-227, conv.cc:41-89).
+#include <cstdlib>
 #include <utility>
 #include <vector>
 
 #include "igemm.h"
+#include "igemm_pipe.h"
 #include "layout_kernels.h"
 
 namespace hipcx {
@@ -54,7 +56,30 @@ void LaunchShape(IGemmArgs<T> p, bool fast16, bool fast8, hipStream_t stream) {
     double bytes = sizeof(T) * (static_cast<double>(p.N) * p.C_logical * p.H_logical * p.W_logical +
                                 static_cast<double>(p.K) * p.R * p.S * p.C_logical + static_cast<double>(p.M) * p.K);
     ProfileScope prof(stream, flops, bytes);
-    if (fast16) {
+    // the pipelined kernel indexes x and w with 32-bit element offsets
+    double x_elems = static_cast<double>(p.N) * (p.xsN > 0 ? p.xsN : 1);
+    bool fits32 = x_elems < 2147483647.0 && static_cast<double>(p.K) * p.wsK < 2147483647.0;
+    static const bool use_pipe = [] { const char* e = getenv("HIPCX_IGEMM_PIPE"); return e != nullptr && e[0] == '1'; }();
+    if ((fast16 || fast8) && fits32 && use_pipe) {
+        constexpr int lds_bytes = PipeLdsBytes<T, WM, WN, PM>();
+        if (fast16) {
+            auto kern = IGemmPipeKernel<T, WM, WN, 16, PM>;
+            static bool configured = false;
+            if (!configured) {
+                HIPCX_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes));
+                configured = true;
+            }
+            hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, p);
+        } else {
+            auto kern = IGemmPipeKernel<T, WM, WN, 8, PM>;
+            static bool configured = false;
+            if (!configured) {
+                HIPCX_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes));
+                configured = true;
+            }
+            hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, p);
+        }
+    } else if (fast16) {
         hipLaunchKernelGGL((IGemmFastKernel<T, WM, WN, 16, PM>), grid, block, 0, stream, p);
     } else if (fast8) {
         hipLaunchKernelGGL((IGemmFastKernel<T, WM, WN, 8, PM>), grid, block, 0, stream, p);
@@ -97,6 +122,17 @@ void LaunchIGemmImpl(IGemmArgs<T> p, hipStream_t stream) {
     } else {
         p.out_vec = (p.osC == 1 && p.K % 4 == 0 && Aligned(p.out, sizeof(T) * 4) && p.osN % 4 == 0 && p.osH % 4 == 0 &&
                      p.osW % 4 == 0) ? 1 : 0;
+    }
+    {
+        const int epv = 16 / static_cast<int>(sizeof(T));
+        int64_t ohw = static_cast<int64_t>(p.OH) * p.OW;
+        if (pm) {
+            p.out_wide = (p.osW == 1 && (p.OH == 1 || p.osH == p.OW) && ohw % epv == 0 && Aligned(p.out, 16) && p.osN % epv == 0 &&
+                          p.osC % epv == 0) ? 1 : 0;
+        } else {
+            p.out_wide = (p.osC == 1 && p.K % epv == 0 && Aligned(p.out, 16) && p.osN % epv == 0 && p.osH % epv == 0 &&
+                          p.osW % epv == 0) ? 1 : 0;
+        }
     }
     bool fast16 = FastOk(p, 16);
     bool fast8 = !fast16 && FastOk(p, 8);

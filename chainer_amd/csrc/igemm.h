@@ -38,6 +38,7 @@ struct IGemmArgs {
     int Kg;                      // R*S*C
     int tiles_m, tiles_n;
     int out_vec;                 // 1 if the 4 accumulators a lane holds per group can be stored as one vector
+    int out_wide;                // 1 if 16-byte runs along the output's contiguous axis can be stored (pipelined kernel)
 };
 
 constexpr int kRowBytes = 128;           // bytes of the reduction axis per tile row
@@ -47,12 +48,9 @@ using half8_t = __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16;
 using float4_t = __attribute__((__vector_size__(4 * sizeof(float)))) float;
 using float16_t = __attribute__((__vector_size__(16 * sizeof(float)))) float;
 
-struct alignas(16) Bytes16 {
-    uint32_t v[4];
-};
-struct alignas(8) Bytes8 {
-    uint32_t v[2];
-};
+// 16- and 8-byte chunks as native vector types, so that arrays of them are promoted to registers
+using Bytes16 = __attribute__((ext_vector_type(4))) unsigned int;
+using Bytes8 = __attribute__((ext_vector_type(2))) unsigned int;
 template <int LB>
 struct BytesOf;
 template <>
@@ -83,19 +81,19 @@ __device__ __forceinline__ void MfmaTile(const Bytes16& a, const Bytes16& b, flo
 
 template <>
 __device__ __forceinline__ void MfmaTile<half_t>(const Bytes16& a, const Bytes16& b, float16_t& acc) {
-    half8_t av = *reinterpret_cast<const half8_t*>(&a);
-    half8_t bv = *reinterpret_cast<const half8_t*>(&b);
+    half8_t av = __builtin_bit_cast(half8_t, a);
+    half8_t bv = __builtin_bit_cast(half8_t, b);
     acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(av, bv, acc, 0, 0, 0);
 }
 
 template <>
 __device__ __forceinline__ void MfmaTile<float>(const Bytes16& a, const Bytes16& b, float16_t& acc) {
-    const float* af = reinterpret_cast<const float*>(&a);
-    const float* bf = reinterpret_cast<const float*>(&b);
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af[t], bf[t], acc, 0, 0, 0);
-    }
+    float4_t af = __builtin_bit_cast(float4_t, a);
+    float4_t bf = __builtin_bit_cast(float4_t, b);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af[0], bf[0], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af[1], bf[1], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af[2], bf[2], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af[3], bf[3], acc, 0, 0, 0);
 }
 
 // One K step over the LDS tile: every wave multiplies its 64 channels x 64 pixels.
@@ -315,13 +313,13 @@ __global__ __launch_bounds__(64 * WM * WN) void IGemmFastKernel(IGemmArgs<T> p) 
             int ih = ih0[i] + r;
             int iw = iw0[i] + s;
             bool ok = kvalid && ih >= 0 && ih < p.H && iw >= 0 && iw < p.W;
-            Chunk v = {};
+            Chunk v = Chunk(0);
             if (ok) v = *reinterpret_cast<const Chunk*>(p.x + xbase[i] + ih * p.xsH + iw * p.xsW + c);
             xreg[i] = v;
         }
 #pragma unroll
         for (int i = 0; i < WCH; ++i) {
-            Chunk v = {};
+            Chunk v = Chunk(0);
             if (kvalid && wvalid[i]) v = *reinterpret_cast<const Chunk*>(wrow[i] + kk);
             wreg[i] = v;
         }

@@ -1,0 +1,591 @@
+// Reductions: Sum (CX/kernels/reduction.h:18), AMax (statistics.h:13), ArgMax (sorting.h:9).
+//
+// Order of operations.  The native backend reduces every output element with one fixed tree
+// (CX/native/reduce.h:46-83): elements are taken in groups of four, (e0.e1).(e2.e3); eight groups
+// are folded serially into a 32-element chunk; chunks are merged by a binary counter, which is a
+// balanced binary tree over aligned runs of chunks, the later operand being the accumulator; the
+// last chunk also takes the up-to-3 leftover elements and any groups short of a full chunk.
+// Both kernels below evaluate exactly that tree, so
+//   * ArgMax returns the native backend's index for every input, ties and NaNs included
+//     (earlier index wins inside a chunk, later chunk wins between chunks, a NaN never replaces
+//     and a leading NaN is never replaced: CX/native/native_device/reduction.cc:34-61);
+//   * Sum carries the native backend's rounding sequence (float16 accumulates in float,
+//     reduction.cc:105), so float results agree bit for bit;
+//   * AMax propagates NaN (statistics.cc:38-42).
+//
+// RowReduceKernel: the reduced axes form one contiguous run (a "row").  Lane <-> group of four
+// (one 16-byte load), 8 lanes <-> chunk, then wave shuffles, an LDS tree and, for rows split
+// over several blocks, a second pass over per-block partials in the workspace.
+// GenericReduceKernel: any strides; one thread per output element runs the reference loop
+// literally.  Consecutive threads take consecutive outputs, so reducing over outer axes of a
+// dense array (a "column" reduction) is coalesced.
+#include "common.h"
+
+namespace hipcx {
+namespace {
+
+constexpr int kMaxDims = HIPCX_MAX_NDIM;
+constexpr int kRowThreads = 256;
+constexpr int kElemsPerIter = kRowThreads * 4;  // 1024 elements = 32 chunks = 4 nodes (one per wave)
+constexpr int kMaxNodes = 256;                  // LDS nodes per block -> span <= 65536 elements
+constexpr int kMaxPartials = 1024;              // blocks per row handled by the finalize pass
+
+// ---------------------------------------------------------------------------------------------
+// Reduction functors.  Acc is what travels through the tree.
+//   Identity()            impl.Identity() of the reference
+//   Map(in, index)        impl.MapIn
+//   Reduce(next, acc)     impl.Reduce(next, accum), additionally a no-op when `next` is the padding value Empty()
+//   kSerialFold           whether the 8 groups of a chunk must be folded strictly in order (floating point addition)
+// ---------------------------------------------------------------------------------------------
+template <typename In_, typename Out_>
+struct SumImpl {
+    using In = In_;
+    using Out = Out_;
+    using Acc = std::conditional_t<std::is_same<Out_, half_t>::value, float, Out_>;
+    static constexpr bool kSerialFold = true;
+    static constexpr bool kHasIndex = false;
+    __device__ static Acc Identity() { return Acc(0); }
+    __device__ static Acc Empty() { return Acc(0); }  // x + 0 == x for every x a chunk can produce (never -0)
+    __device__ static Acc Map(In v, int64_t) {
+        if constexpr (std::is_same<In, half_t>::value) {
+            return static_cast<Acc>(static_cast<float>(v));
+        } else {
+            return static_cast<Acc>(v);
+        }
+    }
+    __device__ static void Reduce(Acc next, Acc& acc) { acc += next; }
+    __device__ static void MaskLaterNan(Acc&, bool) {}
+    __device__ static Out MapOut(Acc a) {
+        if constexpr (std::is_same<Out, half_t>::value) {
+            return static_cast<half_t>(a);
+        } else {
+            return static_cast<Out>(a);
+        }
+    }
+    __device__ static Acc Shfl(Acc a, int src) { return __shfl(a, src); }
+};
+
+template <typename T>
+__device__ __forceinline__ T LowestOrInf() {
+    if constexpr (std::is_same<T, half_t>::value) {
+        return static_cast<half_t>(-__builtin_huge_valf());
+    } else if constexpr (std::is_same<T, float>::value) {
+        return -__builtin_huge_valf();
+    } else if constexpr (std::is_same<T, double>::value) {
+        return -__builtin_huge_val();
+    } else if constexpr (std::is_same<T, bool>::value) {
+        return false;
+    } else {
+        return std::numeric_limits<T>::lowest();
+    }
+}
+
+template <typename T>
+__device__ __forceinline__ bool IsNanV(T v) {
+    if constexpr (std::is_same<T, half_t>::value || std::is_floating_point<T>::value) {
+        return v != v;
+    } else {
+        return false;
+    }
+}
+
+template <typename T>
+struct AMaxImpl {
+    using In = T;
+    using Out = T;
+    // half values are compared as floats (exact and order preserving); bool as int
+    using Acc = std::conditional_t<std::is_same<T, half_t>::value, float, std::conditional_t<std::is_same<T, bool>::value, int, T>>;
+    static constexpr bool kSerialFold = false;
+    static constexpr bool kHasIndex = false;
+    __device__ static Acc Identity() { return static_cast<Acc>(LowestOrInf<T>()); }
+    __device__ static Acc Empty() { return Identity(); }
+    __device__ static Acc Map(In v, int64_t) { return static_cast<Acc>(v); }
+    __device__ static void Reduce(Acc next, Acc& acc) {
+        if (IsNanV(next) || acc < next) acc = next;
+    }
+    __device__ static void MaskLaterNan(Acc&, bool) {}
+    __device__ static Out MapOut(Acc a) { return static_cast<Out>(a); }
+    __device__ static Acc Shfl(Acc a, int src) { return __shfl(a, src); }
+};
+
+template <typename V>
+struct MaxIdx {
+    V v;
+    int64_t i;  // < 0: empty / identity
+};
+
+template <typename T>
+struct ArgMaxImpl {
+    using In = T;
+    using Out = int64_t;
+    using V = std::conditional_t<std::is_same<T, half_t>::value, float, std::conditional_t<std::is_same<T, bool>::value, int, T>>;
+    using Acc = MaxIdx<V>;
+    static constexpr bool kSerialFold = false;
+    static constexpr bool kHasIndex = true;
+    __device__ static Acc Identity() { return Acc{V(0), -1}; }
+    __device__ static Acc Empty() { return Acc{V(0), -1}; }
+    __device__ static Acc Map(In v, int64_t index) { return Acc{static_cast<V>(v), index}; }
+    __device__ static void Reduce(Acc next, Acc& acc) {
+        if (next.i < 0) return;
+        if (acc.i < 0 || acc.v < next.v) acc = next;
+    }
+    // Inside a chunk a NaN operand other than the very first never replaces the accumulator; turning
+    // it into padding makes the in-chunk fold associative, so it can run as a shuffle tree.
+    __device__ static void MaskLaterNan(Acc& a, bool is_first) {
+        if (!is_first && IsNanV(a.v)) a.i = -1;
+    }
+    __device__ static Out MapOut(Acc a) { return a.i; }
+    __device__ static Acc Shfl(Acc a, int src) {
+        Acc r;
+        r.v = __shfl(a.v, src);
+        r.i = __shfl(a.i, src);
+        return r;
+    }
+};
+
+// ---------------------------------------------------------------------------------------------
+// Geometry shared by both kernels
+// ---------------------------------------------------------------------------------------------
+struct ReduceGeom {
+    const char* in;
+    char* out;
+    int n_keep;   // kept (output) axes after squashing
+    int n_red;    // reduced axes after squashing
+    int64_t keep_shape[kMaxDims];
+    int64_t keep_in_stride[kMaxDims];   // bytes
+    int64_t keep_out_stride[kMaxDims];  // bytes
+    int64_t red_shape[kMaxDims];
+    int64_t red_stride[kMaxDims];  // bytes
+    int64_t n_out;                 // product of keep_shape
+    int64_t red_len;               // product of red_shape
+};
+
+__device__ __forceinline__ void OutOffsets(const ReduceGeom& g, int64_t o, int64_t& in_off, int64_t& out_off) {
+    in_off = 0;
+    out_off = 0;
+    for (int d = g.n_keep - 1; d >= 0; --d) {
+        int64_t q = o / g.keep_shape[d];
+        int64_t r = o - q * g.keep_shape[d];
+        o = q;
+        in_off += r * g.keep_in_stride[d];
+        out_off += r * g.keep_out_stride[d];
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Row kernel
+// ---------------------------------------------------------------------------------------------
+template <typename Impl, bool ALIGNED>
+__global__ __launch_bounds__(kRowThreads) void RowReduceKernel(ReduceGeom g, int64_t span, int blocks_per_row, void* partials) {
+    using In = typename Impl::In;
+    using Acc = typename Impl::Acc;
+    __shared__ Acc nodes[kMaxNodes];
+
+    const int64_t row = blockIdx.x / blocks_per_row;
+    const int blk = blockIdx.x - static_cast<int>(row * blocks_per_row);
+    int64_t in_off, out_off;
+    OutOffsets(g, row, in_off, out_off);
+    const In* x = reinterpret_cast<const In*>(g.in + in_off);
+
+    const int64_t L = g.red_len;
+    const int64_t G = L / 4;                          // full groups
+    const int64_t k_last = G > 0 ? (G - 1) / 8 : 0;   // chunk that also takes the tail
+    const int64_t e_begin = static_cast<int64_t>(blk) * span;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int seg_lane = lane & 7;
+    const int iters = static_cast<int>(span / kElemsPerIter);
+
+    for (int it = 0; it < iters; ++it) {
+        const int64_t grp = e_begin / 4 + static_cast<int64_t>(it) * kRowThreads + tid;
+        const int64_t chunk = grp >> 3;
+        Acc gv = Impl::Empty();
+        if (grp < G) {
+            In e[4];
+            if (ALIGNED) {
+                struct alignas(sizeof(In) * 4) In4 {
+                    In v[4];
+                };
+                In4 q = *reinterpret_cast<const In4*>(x + grp * 4);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) e[j] = q.v[j];
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) e[j] = x[grp * 4 + j];
+            }
+            // (e0 . e1) . (e2 . e3): the later element is `next`
+            Acc p0 = Impl::Map(e[0], grp * 4);
+            Impl::Reduce(Impl::Map(e[1], grp * 4 + 1), p0);
+            Acc p1 = Impl::Map(e[2], grp * 4 + 2);
+            Impl::Reduce(Impl::Map(e[3], grp * 4 + 3), p1);
+            Impl::Reduce(p1, p0);
+            gv = p0;
+        }
+        // ---- fold the 8 groups of a chunk into the segment leader ----
+        Acc acc;
+        if (Impl::kSerialFold) {
+            acc = Impl::Identity();
+            Impl::Reduce(gv, acc);
+#pragma unroll
+            for (int j = 1; j < 8; ++j) {
+                Acc o = Impl::Shfl(gv, (lane & ~7) + j);
+                Impl::Reduce(o, acc);
+            }
+        } else {
+            Impl::MaskLaterNan(gv, seg_lane == 0);
+            acc = Impl::Identity();
+            Impl::Reduce(gv, acc);  // lane-local start: Identity . group
+#pragma unroll
+            for (int s = 1; s < 8; s <<= 1) {
+                Acc o = Impl::Shfl(acc, lane + s);  // the later operand
+                Impl::Reduce(o, acc);
+            }
+        }
+        // ---- the last chunk also folds the leftover elements, in order ----
+        if (seg_lane == 0 && chunk == k_last) {
+            for (int64_t i = G * 4; i < L; ++i) Impl::Reduce(Impl::Map(x[i], i), acc);
+        }
+        if (chunk > k_last) acc = Impl::Empty();
+        // ---- 8 chunk results per wave -> one node: balanced tree, the later operand is the accumulator ----
+#pragma unroll
+        for (int s = 8; s < 64; s <<= 1) {
+            Acc later = Impl::Shfl(acc, lane + s);
+            Impl::Reduce(acc, later);
+            acc = later;
+        }
+        if (lane == 0) nodes[it * 4 + wave] = acc;
+    }
+    __syncthreads();
+    const int n_nodes = iters * 4;  // a power of two
+    for (int s = 1; s < n_nodes; s <<= 1) {
+        for (int i = tid; (2 * i + 1) * s < n_nodes; i += kRowThreads) {
+            Acc earlier = nodes[2 * i * s];
+            Acc later = nodes[2 * i * s + s];
+            Impl::Reduce(earlier, later);
+            nodes[2 * i * s] = later;
+        }
+        __syncthreads();
+    }
+    if (tid == 0) {
+        if (blocks_per_row == 1) {
+            *reinterpret_cast<typename Impl::Out*>(g.out + out_off) = Impl::MapOut(nodes[0]);
+        } else {
+            reinterpret_cast<Acc*>(partials)[row * blocks_per_row + blk] = nodes[0];
+        }
+    }
+}
+
+// second pass: tree over the per-block partials of each row (blocks_per_row <= kMaxPartials)
+template <typename Impl>
+__global__ __launch_bounds__(kRowThreads) void RowFinalizeKernel(ReduceGeom g, int blocks_per_row, const void* partials) {
+    using Acc = typename Impl::Acc;
+    __shared__ Acc nodes[kMaxPartials];
+    const int64_t row = blockIdx.x;
+    const int tid = threadIdx.x;
+    int n = 1;
+    while (n < blocks_per_row) n <<= 1;
+    const Acc* src = reinterpret_cast<const Acc*>(partials) + row * blocks_per_row;
+    for (int i = tid; i < n; i += kRowThreads) nodes[i] = i < blocks_per_row ? src[i] : Impl::Empty();
+    __syncthreads();
+    for (int s = 1; s < n; s <<= 1) {
+        for (int i = tid; (2 * i + 1) * s < n; i += kRowThreads) {
+            Acc earlier = nodes[2 * i * s];
+            Acc later = nodes[2 * i * s + s];
+            Impl::Reduce(earlier, later);
+            nodes[2 * i * s] = later;
+        }
+        __syncthreads();
+    }
+    if (tid == 0) {
+        int64_t in_off, out_off;
+        OutOffsets(g, row, in_off, out_off);
+        *reinterpret_cast<typename Impl::Out*>(g.out + out_off) = Impl::MapOut(nodes[0]);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Generic kernel: the reference loop, one output per thread
+// ---------------------------------------------------------------------------------------------
+template <typename Impl>
+__global__ __launch_bounds__(256) void GenericReduceKernel(ReduceGeom g) {
+    using In = typename Impl::In;
+    using Acc = typename Impl::Acc;
+    const int64_t o = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (o >= g.n_out) return;
+    int64_t in_off, out_off;
+    OutOffsets(g, o, in_off, out_off);
+    const char* base = g.in + in_off;
+
+    // odometer over the reduced axes (C order)
+    int64_t cnt[kMaxDims];
+    for (int d = 0; d < g.n_red; ++d) cnt[d] = 0;
+    int64_t off = 0;
+    int64_t i = 0;
+    auto next_elem = [&]() -> Acc {
+        Acc a = Impl::Map(*reinterpret_cast<const In*>(base + off), i);
+        ++i;
+        for (int d = g.n_red - 1; d >= 0; --d) {
+            off += g.red_stride[d];
+            if (++cnt[d] < g.red_shape[d]) break;
+            off -= g.red_stride[d] * g.red_shape[d];
+            cnt[d] = 0;
+        }
+        return a;
+    };
+
+    const int64_t len = g.red_len;
+    const int64_t main_len = len - (len % 4);
+    Acc accum = Impl::Identity();
+    Acc tree[48];
+    while (i < main_len) {
+        if (i != 0 && i % 32 == 0) {
+            int lvl = 0;
+            for (int64_t k = i >> 1; k % 32 == 0; k >>= 1, ++lvl) Impl::Reduce(tree[lvl], accum);
+            tree[lvl] = accum;
+            accum = Impl::Identity();
+        }
+        Acc p0 = next_elem();
+        Impl::Reduce(next_elem(), p0);
+        Acc p1 = next_elem();
+        Impl::Reduce(next_elem(), p1);
+        Impl::Reduce(p1, p0);
+        Impl::Reduce(p0, accum);
+    }
+    while (i < len) Impl::Reduce(next_elem(), accum);
+    {
+        int lvl = 0;
+        for (int64_t k = (len / 4 - 1) / 8; k > 0; k >>= 1, ++lvl) {
+            if (k & 1) Impl::Reduce(tree[lvl], accum);
+        }
+    }
+    *reinterpret_cast<typename Impl::Out*>(g.out + out_off) = Impl::MapOut(accum);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------------------------------
+struct ReducePlan {
+    ReduceGeom g;
+    bool row_path = false;
+    bool aligned = false;
+    int64_t span = 0;
+    int blocks_per_row = 1;
+    size_t acc_size = 0;
+};
+
+ReduceGeom MakeGeom(const hipcx_array* a, const int8_t* axis, int naxis, const hipcx_array* out) {
+    ValidateArray(a, "a");
+    ValidateArray(out, "out");
+    bool red[kMaxDims] = {};
+    int prev = -1;
+    for (int i = 0; i < naxis; ++i) {
+        HIPCX_REQUIRE(axis[i] >= 0 && axis[i] < a->ndim, HIPCX_DIMENSION_ERROR, "reduction axis out of range");
+        HIPCX_REQUIRE(axis[i] > prev, HIPCX_DIMENSION_ERROR, "reduction axes must be sorted and unique");
+        prev = axis[i];
+        red[axis[i]] = true;
+    }
+    // out either keeps the reduced axes with extent 1 or drops them (CX/shape.cc:34-37)
+    bool keepdims = out->ndim == a->ndim && naxis > 0;
+    if (keepdims) {
+        for (int d = 0; d < a->ndim; ++d) {
+            int64_t expect = red[d] ? 1 : a->shape[d];
+            if (out->shape[d] != expect) {
+                keepdims = false;
+                break;
+            }
+        }
+    }
+    if (!keepdims) {
+        HIPCX_REQUIRE(out->ndim == a->ndim - naxis, HIPCX_DIMENSION_ERROR, "out has the wrong number of dimensions for this reduction");
+        int j = 0;
+        for (int d = 0; d < a->ndim; ++d) {
+            if (red[d]) continue;
+            HIPCX_REQUIRE(out->shape[j] == a->shape[d], HIPCX_DIMENSION_ERROR, "out has the wrong shape for this reduction");
+            ++j;
+        }
+    }
+    ReduceGeom g{};
+    g.in = static_cast<const char*>(a->data);
+    g.out = static_cast<char*>(out->data);
+    g.n_out = 1;
+    g.red_len = 1;
+    int j = 0;
+    for (int d = 0; d < a->ndim; ++d) {
+        if (red[d]) {
+            g.red_len *= a->shape[d];
+            if (a->shape[d] == 1) continue;
+            int n = g.n_red;
+            if (n > 0 && g.red_stride[n - 1] == a->shape[d] * a->strides[d]) {  // walks on as one run
+                g.red_shape[n - 1] *= a->shape[d];
+                g.red_stride[n - 1] = a->strides[d];
+            } else {
+                g.red_shape[n] = a->shape[d];
+                g.red_stride[n] = a->strides[d];
+                ++g.n_red;
+            }
+        } else {
+            int64_t ostride = keepdims ? out->strides[d] : out->strides[j];
+            ++j;
+            g.n_out *= a->shape[d];
+            if (a->shape[d] == 1) continue;
+            int n = g.n_keep;
+            if (n > 0 && g.keep_in_stride[n - 1] == a->shape[d] * a->strides[d] && g.keep_out_stride[n - 1] == a->shape[d] * ostride) {
+                g.keep_shape[n - 1] *= a->shape[d];
+                g.keep_in_stride[n - 1] = a->strides[d];
+                g.keep_out_stride[n - 1] = ostride;
+            } else {
+                g.keep_shape[n] = a->shape[d];
+                g.keep_in_stride[n] = a->strides[d];
+                g.keep_out_stride[n] = ostride;
+                ++g.n_keep;
+            }
+        }
+    }
+    return g;
+}
+
+ReducePlan MakePlan(const hipcx_array* a, const int8_t* axis, int naxis, const hipcx_array* out, size_t acc_size) {
+    ReducePlan pl;
+    pl.g = MakeGeom(a, axis, naxis, out);
+    pl.acc_size = acc_size;
+    const ReduceGeom& g = pl.g;
+    const int64_t it = ItemSize(a->dtype);
+    // Row path: one contiguous run of at least 256 elements, short enough for 32-bit-safe bookkeeping.
+    if (g.n_red == 1 && g.red_stride[0] == it && g.red_len >= 256 && g.red_len < (1LL << 40) && g.n_out < (1LL << 31)) {
+        pl.row_path = true;
+        int64_t L = g.red_len;
+        int64_t span = kElemsPerIter;
+        while (span < L && span < static_cast<int64_t>(kMaxNodes) * 256) span <<= 1;
+        // few long rows: split rows over more blocks so that the whole chip is busy
+        int64_t target_blocks = static_cast<int64_t>(NumCUs()) * 8;
+        while (span > 4 * kElemsPerIter && g.n_out * ((L + span - 1) / span) < target_blocks && (L + span / 2 - 1) / (span / 2) <= kMaxPartials) {
+            span >>= 1;
+        }
+        int64_t bpr = (L + span - 1) / span;
+        if (bpr > kMaxPartials || g.n_out * bpr >= (1LL << 31)) {
+            pl.row_path = false;
+        } else {
+            pl.span = span;
+            pl.blocks_per_row = static_cast<int>(bpr);
+            bool al = reinterpret_cast<uintptr_t>(g.in) % (4 * it) == 0;
+            for (int d = 0; d < g.n_keep; ++d) al = al && g.keep_in_stride[d] % (4 * it) == 0;
+            pl.aligned = al;
+        }
+    }
+    return pl;
+}
+
+size_t WorkspaceBytes(const ReducePlan& pl) {
+    if (!pl.row_path || pl.blocks_per_row == 1) return 0;
+    return static_cast<size_t>(pl.g.n_out) * pl.blocks_per_row * pl.acc_size;
+}
+
+template <typename Impl>
+void Run(const hipcx_array* a, const int8_t* axis, int naxis, const hipcx_array* out, void* workspace, size_t workspace_bytes,
+         hipStream_t stream) {
+    ReducePlan pl = MakePlan(a, axis, naxis, out, sizeof(typename Impl::Acc));
+    const ReduceGeom& g = pl.g;
+    if (g.n_out == 0) return;
+    if (pl.row_path) {
+        size_t need = WorkspaceBytes(pl);
+        HIPCX_REQUIRE(need == 0 || (workspace != nullptr && workspace_bytes >= need), HIPCX_CHAINERX_ERROR,
+                      "reduction workspace too small: need " + std::to_string(need) + " bytes");
+        HIPCX_REQUIRE(need == 0 || reinterpret_cast<uintptr_t>(workspace) % 16 == 0, HIPCX_CHAINERX_ERROR,
+                      "workspace must be 16-byte aligned");
+        dim3 grid(static_cast<unsigned>(g.n_out * pl.blocks_per_row)), block(kRowThreads);
+        if (pl.aligned) {
+            hipLaunchKernelGGL((RowReduceKernel<Impl, true>), grid, block, 0, stream, g, pl.span, pl.blocks_per_row, workspace);
+        } else {
+            hipLaunchKernelGGL((RowReduceKernel<Impl, false>), grid, block, 0, stream, g, pl.span, pl.blocks_per_row, workspace);
+        }
+        CheckLaunch("row_reduce");
+        if (pl.blocks_per_row > 1) {
+            hipLaunchKernelGGL((RowFinalizeKernel<Impl>), dim3(static_cast<unsigned>(g.n_out)), block, 0, stream, g, pl.blocks_per_row,
+                               workspace);
+            CheckLaunch("row_reduce_finalize");
+        }
+        return;
+    }
+    int64_t blocks = (g.n_out + 255) / 256;
+    HIPCX_REQUIRE(blocks < (1LL << 31), HIPCX_NOT_IMPLEMENTED_ERROR, "too many outputs for one launch");
+    hipLaunchKernelGGL((GenericReduceKernel<Impl>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, g);
+    CheckLaunch("generic_reduce");
+}
+
+}  // namespace
+}  // namespace hipcx
+
+using namespace hipcx;
+
+extern "C" {
+
+// Upper bound over the three reductions (they share one query): partials are at most 16 bytes each.
+size_t hipcx_reduce_workspace_size(const hipcx_array* a, const int8_t* axis, int naxis, const hipcx_array* out) {
+    try {
+        if (a == nullptr || out == nullptr) return 0;
+        ReducePlan pl = MakePlan(a, axis, naxis, out, 16);
+        return WorkspaceBytes(pl);
+    } catch (...) {
+        return 0;
+    }
+}
+
+int hipcx_sum(const hipcx_array* a, const int8_t* axis, int naxis, const hipcx_array* out, void* workspace, size_t workspace_bytes,
+              void* stream) {
+    return Guard([&] {
+        ValidateArray(a, "a");
+        ValidateArray(out, "out");
+        hipStream_t st = AsStream(stream);
+        const int in = a->dtype, od = out->dtype;
+        // Out dtypes the routines produce: the input's float dtype, int64 for bool/int/uint inputs,
+        // float32/float64 for Mean of integers (CX/routines/reduction.cc:34-49, statistics.cc:111-116).
+        auto for_out = [&](auto in_tag) {
+            using In = typename decltype(in_tag)::type;
+            switch (od) {
+                case HIPCX_INT64: Run<SumImpl<In, int64_t>>(a, axis, naxis, out, workspace, workspace_bytes, st); break;
+                case HIPCX_FLOAT16: Run<SumImpl<In, half_t>>(a, axis, naxis, out, workspace, workspace_bytes, st); break;
+                case HIPCX_FLOAT32: Run<SumImpl<In, float>>(a, axis, naxis, out, workspace, workspace_bytes, st); break;
+                case HIPCX_FLOAT64: Run<SumImpl<In, double>>(a, axis, naxis, out, workspace, workspace_bytes, st); break;
+                default:
+                    throw Error(HIPCX_NOT_IMPLEMENTED_ERROR, std::string("hip sum: unsupported output dtype ") + DtypeName(od));
+            }
+        };
+        VisitDtype(in, for_out);
+    });
+}
+
+int hipcx_amax(const hipcx_array* a, const int8_t* axis, int naxis, const hipcx_array* out, void* workspace, size_t workspace_bytes,
+               void* stream) {
+    return Guard([&] {
+        ValidateArray(a, "a");
+        ValidateArray(out, "out");
+        HIPCX_REQUIRE(a->dtype == out->dtype, HIPCX_DTYPE_ERROR, "amax: out must have a's dtype");
+        for (int i = 0; i < naxis; ++i) {
+            HIPCX_REQUIRE(axis[i] >= 0 && axis[i] < a->ndim && a->shape[axis[i]] > 0, HIPCX_DIMENSION_ERROR,
+                          "cannot compute the maximum along zero-sized axis");
+        }
+        VisitDtype(a->dtype, [&](auto tag) {
+            using T = typename decltype(tag)::type;
+            Run<AMaxImpl<T>>(a, axis, naxis, out, workspace, workspace_bytes, AsStream(stream));
+        });
+    });
+}
+
+int hipcx_argmax(const hipcx_array* a, const int8_t* axis, int naxis, const hipcx_array* out, void* workspace, size_t workspace_bytes,
+                 void* stream) {
+    return Guard([&] {
+        ValidateArray(a, "a");
+        ValidateArray(out, "out");
+        HIPCX_REQUIRE(out->dtype == HIPCX_INT64, HIPCX_DTYPE_ERROR, "argmax: out must be int64");
+        for (int i = 0; i < naxis; ++i) {
+            HIPCX_REQUIRE(axis[i] >= 0 && axis[i] < a->ndim && a->shape[axis[i]] > 0, HIPCX_DIMENSION_ERROR,
+                          "cannot compute ArgMax for an empty array");
+        }
+        VisitDtype(a->dtype, [&](auto tag) {
+            using T = typename decltype(tag)::type;
+            Run<ArgMaxImpl<T>>(a, axis, naxis, out, workspace, workspace_bytes, AsStream(stream));
+        });
+    });
+}
+}

@@ -1,0 +1,197 @@
+// Take (gather along one axis), CX/kernels/indexing.h:17.
+//
+//   out[l..., i..., r...] = a[l..., index[i...], r...]          (CX/native/native_device/indexing.cc:31-103)
+//
+// A pure copy, so results are bit-exact for every dtype; the kernel is instantiated per element
+// size, not per dtype.  Index handling follows the native backend: negative indices count from
+// the end; RAISE / DEFAULT flag an out-of-range index through `error_flag` (the caller turns it
+// into IndexError), WRAP is Python's modulo, CLIP clamps to [0, dim).  When rows of `a` and
+// `out` are dense and 16-byte aligned (the embedding case), a thread moves 16 bytes.
+#include "common.h"
+
+namespace hipcx {
+namespace {
+
+struct DimGroup {
+    int n;
+    int64_t shape[HIPCX_MAX_NDIM];
+    int64_t stride_a[HIPCX_MAX_NDIM];  // bytes in the source (a or indices)
+    int64_t stride_o[HIPCX_MAX_NDIM];  // bytes in out
+    int64_t total;
+};
+
+struct TakeArgs {
+    const char* a;
+    const char* idx;
+    char* out;
+    DimGroup left, index, right;  // index.stride_a are the strides of the indices array
+    int64_t axis_dim;
+    int64_t axis_stride;  // bytes
+    int idx_dtype;
+    int mode;
+    int32_t* error_flag;
+    int64_t total;  // work items: elements, or 16-byte vectors on the row path
+    int64_t right_vecs;  // row path: 16-byte vectors per row
+};
+
+__device__ __forceinline__ void Decompose(const DimGroup& g, int64_t i, int64_t& off_a, int64_t& off_o) {
+    for (int d = g.n - 1; d >= 0; --d) {
+        int64_t q = i / g.shape[d];
+        int64_t r = i - q * g.shape[d];
+        i = q;
+        off_a += r * g.stride_a[d];
+        off_o += r * g.stride_o[d];
+    }
+}
+
+__device__ __forceinline__ int64_t LoadIndex(const char* p, int dtype) {
+    switch (dtype) {
+        case HIPCX_INT8: return *reinterpret_cast<const int8_t*>(p);
+        case HIPCX_INT16: return *reinterpret_cast<const int16_t*>(p);
+        case HIPCX_INT32: return *reinterpret_cast<const int32_t*>(p);
+        case HIPCX_UINT8: return *reinterpret_cast<const uint8_t*>(p);
+        default: return *reinterpret_cast<const int64_t*>(p);
+    }
+}
+
+__device__ __forceinline__ int64_t ResolveIndex(int64_t index, int64_t dim, int mode, int32_t* error_flag) {
+    if (mode == HIPCX_BOUNDS_CLIP) {
+        return index < 0 ? 0 : (index >= dim ? dim - 1 : index);
+    }
+    if (mode == HIPCX_BOUNDS_WRAP || error_flag == nullptr) {
+        if (index < 0) return dim - ((-index + dim - 1) % dim + 1);
+        return index % dim;
+    }
+    if (index < -dim || index >= dim) {
+        *error_flag = 1;
+        return 0;  // stay in bounds; the caller discards the result
+    }
+    return index < 0 ? index + dim : index;
+}
+
+// ROWS: dense right part moved as 16-byte vectors, no left axes, out rows dense.
+template <int BYTES, bool ROWS>
+__global__ __launch_bounds__(256) void TakeKernel(TakeArgs t) {
+    struct alignas(BYTES) Elem {
+        char b[BYTES];
+    };
+    for (int64_t w = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; w < t.total;
+         w += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+        if (ROWS) {
+            int64_t i = w / t.right_vecs;
+            int64_t v = w - i * t.right_vecs;
+            int64_t ioff = 0, unused = 0;
+            Decompose(t.index, i, ioff, unused);
+            int64_t index = ResolveIndex(LoadIndex(t.idx + ioff, t.idx_dtype), t.axis_dim, t.mode, t.error_flag);
+            *reinterpret_cast<Elem*>(t.out + w * BYTES) = *reinterpret_cast<const Elem*>(t.a + index * t.axis_stride + v * BYTES);
+        } else {
+            int64_t r = w % t.right.total;
+            int64_t rest = w / t.right.total;
+            int64_t i = rest % t.index.total;
+            int64_t l = rest / t.index.total;
+            int64_t a_off = 0, o_off = 0, ioff = 0;
+            Decompose(t.left, l, a_off, o_off);
+            Decompose(t.right, r, a_off, o_off);
+            Decompose(t.index, i, ioff, o_off);
+            int64_t index = ResolveIndex(LoadIndex(t.idx + ioff, t.idx_dtype), t.axis_dim, t.mode, t.error_flag);
+            *reinterpret_cast<Elem*>(t.out + o_off) = *reinterpret_cast<const Elem*>(t.a + a_off + index * t.axis_stride);
+        }
+    }
+}
+
+bool DenseGroup(const DimGroup& g, const int64_t* strides, int64_t itemsize) {
+    int64_t expect = itemsize;
+    for (int d = g.n - 1; d >= 0; --d) {
+        if (g.shape[d] != 1 && strides[d] != expect) return false;
+        expect *= g.shape[d];
+    }
+    return true;
+}
+
+}  // namespace
+}  // namespace hipcx
+
+using namespace hipcx;
+
+extern "C" int hipcx_take(const hipcx_array* a, const hipcx_array* indices, int8_t axis, const hipcx_array* out, int mode,
+                          int32_t* error_flag, void* stream) {
+    return Guard([&] {
+        ValidateArray(a, "a");
+        ValidateArray(indices, "indices");
+        ValidateArray(out, "out");
+        HIPCX_REQUIRE(axis >= 0 && axis < a->ndim, HIPCX_DIMENSION_ERROR, "take: axis out of range");
+        HIPCX_REQUIRE(indices->dtype == HIPCX_INT8 || indices->dtype == HIPCX_INT16 || indices->dtype == HIPCX_INT32 ||
+                              indices->dtype == HIPCX_INT64 || indices->dtype == HIPCX_UINT8,
+                      HIPCX_DTYPE_ERROR, "Only arrays of integer dtype can be used as indices.");
+        HIPCX_REQUIRE(out->dtype == a->dtype, HIPCX_DTYPE_ERROR, "take: out must have a's dtype");
+        HIPCX_REQUIRE(mode >= HIPCX_BOUNDS_DEFAULT && mode <= HIPCX_BOUNDS_CLIP, HIPCX_CHAINERX_ERROR, "take: invalid bounds mode");
+        HIPCX_REQUIRE(out->ndim == a->ndim - 1 + indices->ndim, HIPCX_DIMENSION_ERROR, "take: out has the wrong number of dimensions");
+        TakeArgs t{};
+        t.a = static_cast<const char*>(a->data);
+        t.idx = static_cast<const char*>(indices->data);
+        t.out = static_cast<char*>(out->data);
+        t.axis_dim = a->shape[axis];
+        t.axis_stride = a->strides[axis];
+        t.idx_dtype = indices->dtype;
+        t.mode = mode;
+        t.error_flag = error_flag;
+        t.left.total = t.index.total = t.right.total = 1;
+        int o = 0;
+        for (int d = 0; d < axis; ++d, ++o) {
+            HIPCX_REQUIRE(out->shape[o] == a->shape[d], HIPCX_DIMENSION_ERROR, "take: out has the wrong shape");
+            t.left.shape[t.left.n] = a->shape[d];
+            t.left.stride_a[t.left.n] = a->strides[d];
+            t.left.stride_o[t.left.n] = out->strides[o];
+            t.left.total *= a->shape[d];
+            ++t.left.n;
+        }
+        for (int d = 0; d < indices->ndim; ++d, ++o) {
+            HIPCX_REQUIRE(out->shape[o] == indices->shape[d], HIPCX_DIMENSION_ERROR, "take: out has the wrong shape");
+            t.index.shape[t.index.n] = indices->shape[d];
+            t.index.stride_a[t.index.n] = indices->strides[d];
+            t.index.stride_o[t.index.n] = out->strides[o];
+            t.index.total *= indices->shape[d];
+            ++t.index.n;
+        }
+        for (int d = axis + 1; d < a->ndim; ++d, ++o) {
+            HIPCX_REQUIRE(out->shape[o] == a->shape[d], HIPCX_DIMENSION_ERROR, "take: out has the wrong shape");
+            t.right.shape[t.right.n] = a->shape[d];
+            t.right.stride_a[t.right.n] = a->strides[d];
+            t.right.stride_o[t.right.n] = out->strides[o];
+            t.right.total *= a->shape[d];
+            ++t.right.n;
+        }
+        int64_t total = t.left.total * t.index.total * t.right.total;
+        if (total == 0) return;
+        HIPCX_REQUIRE(t.axis_dim > 0, HIPCX_INDEX_ERROR, "take: cannot take from an axis of extent 0");
+        const int64_t it = ItemSize(a->dtype);
+        hipStream_t st = AsStream(stream);
+        int64_t cap = static_cast<int64_t>(NumCUs()) * 32;
+
+        // embedding-style rows
+        int64_t row_bytes = t.right.total * it;
+        bool rows = t.left.total == 1 && row_bytes % 16 == 0 && row_bytes > 0 && DenseGroup(t.right, t.right.stride_a, it) &&
+                    DenseGroup(t.right, t.right.stride_o, it) && t.axis_stride % 16 == 0 && reinterpret_cast<uintptr_t>(t.a) % 16 == 0 &&
+                    reinterpret_cast<uintptr_t>(t.out) % 16 == 0 && IsContiguous(out);
+        if (rows) {
+            t.right_vecs = row_bytes / 16;
+            t.total = t.index.total * t.right_vecs;
+            int64_t blocks = (t.total + 255) / 256;
+            if (blocks > cap) blocks = cap;
+            hipLaunchKernelGGL((TakeKernel<16, true>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st, t);
+            CheckLaunch("take(rows)");
+            return;
+        }
+        t.total = total;
+        int64_t blocks = (total + 255) / 256;
+        if (blocks > cap) blocks = cap;
+        dim3 grid(static_cast<unsigned>(blocks)), block(256);
+        switch (it) {
+            case 1: hipLaunchKernelGGL((TakeKernel<1, false>), grid, block, 0, st, t); break;
+            case 2: hipLaunchKernelGGL((TakeKernel<2, false>), grid, block, 0, st, t); break;
+            case 4: hipLaunchKernelGGL((TakeKernel<4, false>), grid, block, 0, st, t); break;
+            default: hipLaunchKernelGGL((TakeKernel<8, false>), grid, block, 0, st, t); break;
+        }
+        CheckLaunch("take");
+    });
+}
