@@ -1,0 +1,124 @@
+"""Dot / Linear / Conv forward (MFMA implicit GEMM) against the CPU oracle: 1e-5 relative for float32, 2e-2 for float16
+(products of the stored values, float32 accumulation, one rounding), 1e-12 for float64."""
+import numpy as np
+import pytest
+
+from oracle import native as O
+from helpers import assert_close, channels_last, padded, upload_view
+from test_oracle_pins import CONV_GRID
+
+pytestmark = pytest.mark.gpu
+
+DT = [('float32', 1e-5), ('float16', 2e-2), ('float64', 1e-12)]
+
+CONV_CASES = [
+    # N,C,H,W,K,R,S,stride,pad,cover_all
+    (2, 3, 9, 8, 4, 3, 3, (2, 1), (1, 2), False),
+    (2, 16, 8, 8, 32, 3, 3, 1, 1, False),
+    (3, 64, 7, 7, 64, 1, 1, 1, 0, False),
+    (2, 64, 14, 14, 256, 1, 1, 2, 0, False),
+    (2, 32, 10, 10, 24, 3, 3, 2, 1, True),
+    (1, 3, 32, 32, 64, 7, 7, 2, 3, False),
+    (2, 8, 5, 5, 130, 3, 3, 1, 1, False),
+    (1, 24, 6, 6, 70, 1, 1, 1, 0, False),
+    (4, 128, 9, 9, 128, 3, 3, 1, 1, False),
+    (2, 20, 6, 7, 9, 2, 3, (1, 2), (0, 1), True),
+]
+
+
+@pytest.mark.parametrize('dt,tol', DT)
+def test_conv_layouts_and_shapes(dt, tol):
+    import chainer_amd as chx
+    rng = np.random.default_rng(0)
+    for (N, C, H, W, K, R, S, st, pd, cv) in CONV_CASES:
+        x = rng.standard_normal((N, C, H, W)).astype(dt)
+        w = (rng.standard_normal((K, C, R, S)) / np.sqrt(C * R * S)).astype(dt)
+        b = rng.standard_normal(K).astype(dt)
+        ref = O.conv(x, w, b, st, pd, cv)
+        what = '%s %s' % (dt, (N, C, H, W, K, R, S, st, pd, cv))
+        for lay, X in (('nchw', chx.array(x)), ('nhwc', channels_last(chx, x))):
+            y = chx.conv(X, chx.array(w), chx.array(b), st, pd, cv)
+            assert y.shape == ref.shape and y.dtype == ref.dtype
+            assert_close(y.get(), ref, tol, 'conv %s %s' % (lay, what))
+        y = chx.conv(channels_last(chx, x), chx.array(w), None, st, pd, cv)
+        assert_close(y.get(), O.conv(x, w, None, st, pd, cv), tol, 'conv without bias ' + what)
+
+
+@pytest.mark.parametrize('xs,ws,bias,stride,pad', CONV_GRID)
+@pytest.mark.parametrize('cover_all', [False, True])
+def test_conv_reference_grid(xs, ws, bias, stride, pad, cover_all):
+    """The 2-D rows of the reference's own parameter grid (test_connection.py:183-203), padded (non-contiguous) x."""
+    import chainer_amd as chx
+    rng = np.random.default_rng(1)
+    for dt, tol in DT:
+        x = padded(xs, rng.standard_normal(xs), 1, dt)
+        w = (rng.standard_normal(ws) / np.sqrt(np.prod(ws[1:]))).astype(dt)
+        b = rng.standard_normal(ws[0]).astype(dt) if bias else None
+        y = chx.conv(upload_view(chx, x), chx.array(w), chx.array(b) if bias else None, stride, pad, cover_all)
+        assert_close(y.get(), O.conv(x, w, b, stride, pad, cover_all), tol)
+
+
+@pytest.mark.parametrize('dt,tol', DT)
+def test_dot_and_linear(dt, tol):
+    import chainer_amd as chx
+    rng = np.random.default_rng(2)
+    for (m, k, n) in [(100, 784, 1000), (7, 33, 5), (128, 650, 2600), (64, 64, 64), (1, 1, 1), (130, 100, 70), (3, 2000, 3)]:
+        a = rng.standard_normal((m, k)).astype(dt)
+        b = (rng.standard_normal((k, n)) / np.sqrt(k)).astype(dt)
+        ref = O.dot(a, b)
+        what = '%s %s' % (dt, (m, k, n))
+        assert_close(chx.dot(chx.array(a), chx.array(b)).get(), ref, tol, 'dot ' + what)
+        bt = chx.array(np.ascontiguousarray(b.T)).T  # the W^T view Linear passes (strides (item, item*K))
+        assert_close(chx.dot(chx.array(a), bt).get(), ref, tol, 'dot with transposed-view b ' + what)
+        at = chx.array(np.ascontiguousarray(a.T)).T
+        assert_close(chx.dot(at, bt).get(), ref, tol, 'dot with both operands transposed views ' + what)
+        bias = rng.standard_normal(n).astype(dt)
+        wt = np.ascontiguousarray(b.T)
+        assert_close(chx.linear(chx.array(a), chx.array(wt), chx.array(bias)).get(), O.linear(a, wt, bias), tol, 'linear ' + what)
+    ap = padded((5, 9), rng.standard_normal((5, 9)), 1, dt)
+    bp = padded((9, 4), rng.standard_normal((9, 4)), 2, dt)
+    assert_close(chx.dot(upload_view(chx, ap), upload_view(chx, bp)).get(), O.dot(ap, bp), tol, 'padded operands')
+
+
+def test_dot_integer_valued_is_exact():
+    import chainer_amd as chx
+    rng = np.random.default_rng(3)
+    for dt in ('float32', 'float16', 'float64'):
+        a = rng.integers(-3, 4, (70, 90)).astype(dt)
+        b = rng.integers(-3, 4, (90, 50)).astype(dt)
+        got = chx.dot(chx.array(a), chx.array(b)).get()
+        assert np.array_equal(got.astype(np.int64), a.astype(np.int64) @ b.astype(np.int64))
+
+
+def test_dot_conv_edge_cases_and_errors():
+    import chainer_amd as chx
+    z = chx.dot(chx.zeros((3, 0), 'float32'), chx.zeros((0, 4), 'float32')).get()
+    assert z.shape == (3, 4) and not z.any()  # k == 0 -> zeros (CX/routines/linalg.cc:59-61)
+    assert chx.dot(chx.zeros((0, 5), 'float32'), chx.zeros((5, 4), 'float32')).shape == (0, 4)
+    with pytest.raises(chx.DimensionError):
+        chx.dot(chx.zeros((3, 4), 'float32'), chx.zeros((5, 4), 'float32'))
+    with pytest.raises(chx.DimensionError):
+        chx.conv(chx.zeros((1, 3, 4, 4), 'float32'), chx.zeros((2, 4, 3, 3), 'float32'))
+    with pytest.raises(chx.DimensionError):
+        chx.conv(chx.zeros((1, 3, 2, 2), 'float32'), chx.zeros((2, 3, 5, 5), 'float32'))  # output size not positive
+    assert chx.conv(chx.zeros((0, 3, 4, 4), 'float32'), chx.zeros((2, 3, 3, 3), 'float32')).shape == (0, 2, 2, 2)
+
+
+def test_conv_linearity_at_resnet_layer_size():
+    """Size-independent property at a real layer shape (fp16 [32,256,14,14] * [256,256,3,3]): conv(x, w1 + w2) matches
+    conv(x, w1) + conv(x, w2) to rounding, and a delta filter reproduces the input."""
+    import chainer_amd as chx
+    rng = np.random.default_rng(4)
+    x = rng.standard_normal((32, 256, 14, 14)).astype('float16')
+    w1 = (rng.standard_normal((256, 256, 3, 3)) / 48).astype('float16')
+    w2 = (rng.standard_normal((256, 256, 3, 3)) / 48).astype('float16')
+    X = chx.array(x)
+    y1 = chx.conv(X, chx.array(w1), None, 1, 1).get().astype(np.float64)
+    y2 = chx.conv(X, chx.array(w2), None, 1, 1).get().astype(np.float64)
+    w12 = (w1.astype(np.float32) + w2.astype(np.float32)).astype('float16')
+    y12 = chx.conv(X, chx.array(w12), None, 1, 1).get().astype(np.float64)
+    scale = np.abs(y1 + y2).max()
+    assert np.abs(y12 - (y1 + y2)).max() / scale < 2e-2
+    delta = np.zeros((256, 256, 3, 3), 'float16')
+    delta[np.arange(256), np.arange(256), 1, 1] = 1
+    assert np.array_equal(chx.conv(X, chx.array(delta), None, 1, 1).get(), x)

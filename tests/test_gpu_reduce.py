@@ -1,0 +1,121 @@
+"""Sum / AMax / ArgMax / log_softmax against the CPU oracle.
+
+Bar: ArgMax and AMax bit-exact (including the native backend's tie and NaN rules); Sum bit-exact as well, because the
+kernels reproduce the native pairwise tree (integers are exact in any order); log_softmax within the float tolerance."""
+import numpy as np
+import pytest
+
+from oracle import native as O
+from helpers import assert_close, assert_exact, padded, upload_view
+
+pytestmark = pytest.mark.gpu
+
+SHAPES_AXES = [((5, 70), 1), ((5, 70), 0), ((5, 70), None), ((3, 4, 5), (0, 2)), ((3, 4, 5), 1), ((7, 300), 1), ((4, 1024), 1),
+               ((3, 4100), 1), ((2, 70000), 1), ((6,), 0), ((2, 3, 1500), (1, 2)), ((1, 65536 * 3 + 5), 1), ((300, 9), 0),
+               ((2, 2, 2, 2), (1, 3)), ((3, 33), 1), ((3, 35), 1), ((3, 3), 1)]
+DTYPES = ['float32', 'float64', 'float16', 'int32', 'int64', 'int8', 'uint8', 'bool', 'int16']
+
+
+def rand(rng, shape, dt):
+    if dt == 'bool':
+        return rng.random(shape) > 0.7
+    if dt.startswith('float'):
+        return rng.standard_normal(shape).astype(dt)
+    return rng.integers(0 if dt == 'uint8' else -100, 100, shape).astype(dt)
+
+
+@pytest.mark.parametrize('dt', DTYPES)
+def test_reductions_match_oracle(dt):
+    import chainer_amd as chx
+    rng = np.random.default_rng(0)
+    for shape, axis in SHAPES_AXES:
+        x = rand(rng, shape, dt)
+        X = chx.array(x)
+        what = '%s %s axis=%s' % (dt, shape, axis)
+        for keep in (False, True):
+            assert_exact(chx.sum(X, axis, keep).get(), O.sum(x, axis, keep), 'sum ' + what)
+            assert_exact(chx.amax(X, axis, keep).get(), O.amax(x, axis, keep), 'amax ' + what)
+        assert_exact(chx.argmax(X, axis).get(), O.argmax(x, axis), 'argmax ' + what)
+    if dt != 'bool':  # strided views
+        x = (rng.standard_normal((6, 2100)) * 10).astype(dt)
+        X = chx.array(x)
+        assert_exact(chx.sum(X.T, 0).get(), O.sum(x.T, 0), 'sum of a transposed view')
+        assert_exact(chx.argmax(X[:, 3:2051], 1).get(), O.argmax(x[:, 3:2051], 1), 'argmax of a slice')
+        assert_exact(chx.argmax(X[:, ::2], 1).get(), O.argmax(x[:, ::2], 1), 'argmax with a step')
+        xp = padded((3, 4, 5), rand(rng, (3, 4, 5), dt), 1, dt)
+        assert_exact(chx.amax(upload_view(chx, xp), (0, 2)).get(), O.amax(xp, (0, 2)), 'amax padded')
+
+
+@pytest.mark.parametrize('length', [10, 64, 100, 1000, 4096, 70000])
+def test_argmax_ties_and_nans_bit_exact(length):
+    """Rows full of ties and NaNs: the index must be the one the native backend's pairwise tree selects."""
+    import chainer_amd as chx
+    rng = np.random.default_rng(length)
+    for trial in range(6):
+        x = rng.integers(0, 4, (5, length)).astype('float32')
+        if trial >= 2:
+            x[rng.random((5, length)) < (0.02 if trial < 4 else 0.5)] = np.nan
+        if trial == 5:
+            x[:, 0] = np.nan
+        X = chx.array(x)
+        assert_exact(chx.argmax(X, 1).get(), O.argmax(x, 1), 'argmax rows t=%d' % trial)
+        assert_exact(chx.amax(X, 1).get(), O.amax(x, 1), 'amax rows t=%d' % trial)
+        xt = np.ascontiguousarray(x.T)
+        assert_exact(chx.argmax(chx.array(xt), 0).get(), O.argmax(xt, 0), 'argmax columns t=%d' % trial)
+    xz = np.array([[-0.0, 0.0, 0.0, -0.0]], 'float32')
+    assert_exact(chx.argmax(chx.array(xz), 1).get(), O.argmax(xz, 1), 'signed zeros')
+
+
+@pytest.mark.parametrize('dt,tol', [('float32', 1e-5), ('float64', 1e-12), ('float16', 2e-2)])
+def test_log_softmax_mean_softmax(dt, tol):
+    import chainer_amd as chx
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal((37, 1000)).astype(dt)
+    X = chx.array(x)
+    assert_close(chx.log_softmax(X, 1).get(), O.log_softmax(x, 1), tol, 'log_softmax')
+    assert_close(chx.mean(X, 1).get(), O.mean(x, 1), tol, 'mean')
+    sm = chx.softmax(X, 1).get().astype(np.float64)
+    assert np.abs(sm.sum(1) - 1).max() < (2e-2 if dt == 'float16' else 1e-5)
+    xi = rng.integers(-5, 5, (6, 7)).astype('int32')
+    assert_close(chx.mean(chx.array(xi), 0).get(), O.mean(xi, 0), 1e-6, 'mean of ints is float32')
+
+
+def test_softmax_cross_entropy():
+    import chainer_amd as chx
+    rng = np.random.default_rng(2)
+    t = rng.integers(0, 10, 100).astype('int32')
+    y = rng.standard_normal((100, 10)).astype('float32')
+    assert_close(chx.softmax_cross_entropy(chx.array(y), chx.array(t)).get(), O.softmax_cross_entropy(y, t), 1e-5)
+
+
+@pytest.mark.parametrize('shape', [(4096, 4096), (64, 1048576)])
+def test_sweep_shapes_full_size(shape):
+    """The elementwise/reduction sweep at its real sizes: argmax/amax bit-exact, sum bit-exact, log_softmax 1e-5,
+    plus the size-independent properties (rows of exp(log_softmax) sum to 1; argmax indexes the max)."""
+    import chainer_amd as chx
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal(shape).astype('float32')
+    X = chx.array(x)
+    am = chx.argmax(X, 1).get()
+    assert_exact(am, O.argmax(x, 1), 'argmax')
+    assert_exact(chx.amax(X, 1).get(), O.amax(x, 1), 'amax')
+    assert np.array_equal(x[np.arange(shape[0]), am], x.max(1))
+    assert_exact(chx.sum(X, 1).get(), O.sum(x, 1), 'sum')
+    ls = chx.log_softmax(X, 1)
+    assert_close(ls.get(), O.log_softmax(x, 1), 1e-5, 'log_softmax')
+    rows = chx.sum(chx.exp(ls), 1).get()
+    assert np.abs(rows - 1).max() < 1e-4
+    assert_exact(chx.sum(X, 0).get(), O.sum(x, 0), 'column sum')
+
+
+def test_reduction_errors_and_empty():
+    import chainer_amd as chx
+    X = chx.array(np.zeros((2, 3), np.float32))
+    with pytest.raises(chx.DimensionError):
+        chx.sum(X, 2)
+    with pytest.raises(chx.DimensionError):
+        chx.argmax(X, -3)
+    with pytest.raises(chx.DimensionError):
+        chx.argmax(chx.zeros((2, 0, 3), 'float32'), 1)  # "cannot compute the argmax of an empty array" (routines/sorting.cc)
+    assert chx.sum(chx.zeros((2, 0, 3), 'float32'), 1).get().tolist() == [[0, 0, 0], [0, 0, 0]]
+    assert chx.argmax(chx.zeros((2, 0, 3), 'float32'), 2).get().shape == (2, 0)

@@ -1,0 +1,511 @@
+"""Pins of the CPU oracle (oracle/native.py + oracle/native_oracle.c).
+
+The oracle is only trusted as far as it is pinned here.  Kinds of pin used, per function:
+
+  R  literal input/expected vectors held by the reference's own tests (tests/golden/reference_vectors.json and
+     the literals of tests/chainerx_tests/unit_tests/routines_tests/test_sorting.py:11-29, expected = numpy.argmax)
+  X  the reference's own float16.cc compiled from the reference tree into oracle/_ref (when present)
+  C  closed form / invariant in float64 or exact integer arithmetic
+  L  an independent library routine (numpy, scipy)
+  B  brute-force loops on small inputs, written from the definition of the operation (not from the oracle's code)
+
+What stays "parity unpinned" at bit level (tolerance level is pinned): the float summation order of Sum, the float
+bit patterns of the naive Dot, and ArgMax's tie rule between different 32-element blocks -- all three are derived from
+the reference's source (CX/native/reduce.h:46-83, CX/native/native_device/dot.cc:181-227) and no vector held by the
+reference distinguishes them from other orders.
+"""
+import ctypes
+import itertools
+import json
+import math
+import os
+
+import numpy as np
+import pytest
+import scipy.special
+
+from oracle import native as O
+from helpers import padded, assert_close, assert_exact
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+GOLDEN = json.load(open(os.path.join(HERE, 'golden', 'reference_vectors.json')))['cases']
+REF_F16 = os.path.join(os.path.dirname(HERE), 'oracle', '_ref', 'libcxfloat16.so')
+
+
+def build_input(spec, dtype):
+    shape = spec['shape']
+    pad = spec.get('padding', 0)
+    if 'linear' in spec:
+        start, step = spec['linear']
+        return padded(shape, None, pad, dtype, start, step)
+    return padded(shape, spec['data'], pad, dtype)
+
+
+def norm_axis(axis):
+    return None if axis is None else tuple(axis)
+
+
+def run_golden(F, case, to_dev=lambda a: a, to_host=np.asarray):
+    """Evaluates one golden case with routine namespace F; shared by the CPU (oracle) and GPU (hip) golden tests."""
+    dt = np.dtype(case['dtype'])
+    op = case['op']
+    if op in ('sum', 'amax'):
+        x = build_input(case['input'], dt)
+        axis = norm_axis(case['axis'])
+        axis = None if axis is None else tuple(a % x.ndim for a in axis)
+        out = getattr(F, op)(to_dev(x), axis, case['keepdims'])
+    elif op == 'argmax':
+        x = build_input(case['input'], dt)
+        axis = norm_axis(case['axis'])
+        out = F.argmax(to_dev(x), None if axis is None else axis[0])
+    elif op == 'dot':
+        out = F.dot(to_dev(build_input(case['a'], dt)), to_dev(build_input(case['b'], dt)))
+    elif op == 'take':
+        a = build_input(case['input'], dt)
+        idx = np.asarray(case['indices']['data'], np.int64).reshape(case['indices']['shape'])
+        out = F.take(to_dev(a), to_dev(idx), case['axis'], case['mode'])
+    elif op in ('add', 'subtract', 'multiply', 'divide'):
+        out = getattr(F, op)(to_dev(build_input(case['a'], dt)), to_dev(build_input(case['b'], dt)))
+    elif op.endswith('_scalar'):
+        a = to_dev(build_input(case['a'], dt))
+        s = case['scalar']
+        name = op[:-len('_scalar')]
+        if F is O:
+            out = getattr(F, name)(a, np.asarray(s, dt))
+        else:
+            out = getattr(F, name)(a, s)
+    else:
+        raise AssertionError('unknown golden op %s' % op)
+    return to_host(out)
+
+
+@pytest.mark.parametrize('case', GOLDEN, ids=[c['name'] for c in GOLDEN])
+def test_oracle_matches_reference_vectors(case):
+    """R: every literal vector the reference's C++ tests hold for these kernels (cite in the JSON)."""
+    got = run_golden(O, case)
+    exp = np.asarray(case['expected'])
+    shape = tuple(case.get('expected_shape', got.shape))
+    assert got.shape == shape
+    assert np.array_equal(got.reshape(-1).astype(np.float64), exp.reshape(-1).astype(np.float64))
+
+
+# ---------------------------------------------------------------------------------------------
+# float16
+# ---------------------------------------------------------------------------------------------
+def _f32_samples():
+    rng = np.random.default_rng(16)
+    bits = rng.integers(0, 2 ** 32, 1 << 20, dtype=np.uint64).astype(np.uint32)
+    rand = bits.view(np.float32)
+    near_half = np.arange(0, 1 << 16, dtype=np.uint16).view(np.float16).astype(np.float32)
+    # neighbours of every representable half and of every rounding midpoint
+    mids = (near_half[:-1].astype(np.float64) + near_half[1:].astype(np.float64)) / 2
+    with np.errstate(all='ignore'):
+        mids = mids[np.isfinite(mids)].astype(np.float32)
+    edge = np.concatenate([near_half, np.nextafter(near_half, np.float32(np.inf)), np.nextafter(near_half, np.float32(-np.inf)),
+                           mids, np.nextafter(mids, np.float32(np.inf)), np.nextafter(mids, np.float32(-np.inf)),
+                           np.array([65504, 65519.99, 65520, 65536, 1e-8, 5.96e-8, 2.98e-8, 2.9802322e-8, 2.9802326e-8, 6.1e-5], np.float32)])
+    return np.concatenate([rand, edge, -edge])
+
+
+def test_float16_conversions_match_numpy():
+    """L: numpy's float16 uses the same npy_floatbits_to_halfbits algorithm the reference says it borrowed
+    (CX/float16.cc:24-26).  Exhaustive half->float, 1.5M sampled/edge float->half."""
+    allh = np.arange(1 << 16, dtype=np.uint16)
+    assert_exact(O.half_bits_to_float(allh), allh.view(np.float16).astype(np.float32))
+    x = _f32_samples()
+    got = O.float_to_half_bits(x)
+    with np.errstate(all='ignore'):
+        ref = x.astype(np.float16).view(np.uint16)
+    nan = np.isnan(x)
+    assert np.array_equal(got[~nan], ref[~nan])
+    assert (((got[nan] & 0x7c00) == 0x7c00) & ((got[nan] & 0x3ff) != 0)).all()  # NaN stays NaN
+    assert np.array_equal(got[nan] & 0x8000, ref[nan] & 0x8000)
+
+
+def test_float16_literals_of_reference_test():
+    """R: CX/float16_test.cc:60-73 (zeros), :102-110 (infinities), :132-157 (round-to-nearest-even of 1 + 3*2^-11)."""
+    f = np.array([0.0, -0.0, np.inf, -np.inf], np.float32)
+    assert O.float_to_half_bits(f).tolist() == [0x0000, 0x8000, 0x7c00, 0xfc00]
+    back = O.half_bits_to_float(np.array([0x0000, 0x8000, 0x7c00, 0xfc00], np.uint16))
+    assert back[0] == 0 and not np.signbit(back[0]) and back[1] == 0 and np.signbit(back[1])
+    assert back[2] == np.inf and back[3] == -np.inf
+    # a value exactly between mantissas 1 and 2 rounds to the even one (2)
+    tie = np.array([1.0 + 1.5 * 2.0 ** -10], np.float32)
+    assert int(O.float_to_half_bits(tie)[0]) & 0x3ff == 0x2
+    for bit in range(0x7c01, 0x8000, 37):  # NaN payloads stay NaN (:113-121)
+        assert np.isnan(O.half_bits_to_float(np.array([bit, bit | 0x8000], np.uint16))).all()
+
+
+@pytest.mark.skipif(not os.path.exists(REF_F16), reason='oracle/_ref/libcxfloat16.so not built (needs the reference tree)')
+def test_float16_matches_compiled_reference():
+    """X: chainerx::Float16 itself, compiled from the reference's float16.cc by oracle/Makefile."""
+    ref = ctypes.CDLL(REF_F16)
+    i64 = ctypes.c_int64
+    u16p, f32p = ctypes.POINTER(ctypes.c_uint16), ctypes.POINTER(ctypes.c_float)
+    allh = np.arange(1 << 16, dtype=np.uint16)
+    out = np.empty(allh.size, np.float32)
+    ref.ref_half_to_float(allh.ctypes.data_as(u16p), out.ctypes.data_as(f32p), i64(allh.size))
+    assert_exact(O.half_bits_to_float(allh), out)
+    x = np.ascontiguousarray(_f32_samples())
+    hb = np.empty(x.size, np.uint16)
+    ref.ref_float_to_half(x.ctypes.data_as(f32p), hb.ctypes.data_as(u16p), i64(x.size))
+    assert np.array_equal(O.float_to_half_bits(x), hb)
+    # Float16 arithmetic (operator+ and operator* via float) against the oracle's elementwise add / multiply
+    rng = np.random.default_rng(7)
+    a = rng.integers(0, 1 << 16, 1 << 18).astype(np.uint16)
+    b = rng.integers(0, 1 << 16, 1 << 18).astype(np.uint16)
+    for name, fn in (('ref_half_add', O.add), ('ref_half_mul', O.multiply)):
+        r = np.empty(a.size, np.uint16)
+        getattr(ref, name)(a.ctypes.data_as(u16p), b.ctypes.data_as(u16p), r.ctypes.data_as(u16p), i64(a.size))
+        got = fn(a.view(np.float16), b.view(np.float16))
+        both_nan = np.isnan(got) & np.isnan(r.view(np.float16))
+        assert (both_nan | (got.view(np.uint16) == r)).all(), name
+
+
+# ---------------------------------------------------------------------------------------------
+# elementwise
+# ---------------------------------------------------------------------------------------------
+def test_elementwise_single_rounding():
+    """C: each op is one IEEE operation in the array dtype; for float32 the float64 result rounded once is the same
+    thing (a double holds the exact sum/product of two floats)."""
+    rng = np.random.default_rng(1)
+    a = rng.standard_normal(4096).astype(np.float32) * 100
+    b = rng.standard_normal(4096).astype(np.float32)
+    assert_exact(O.add(a, b), (a.astype(np.float64) + b.astype(np.float64)).astype(np.float32))
+    assert_exact(O.subtract(a, b), (a.astype(np.float64) - b.astype(np.float64)).astype(np.float32))
+    assert_exact(O.multiply(a, b), (a.astype(np.float64) * b.astype(np.float64)).astype(np.float32))
+    # float16: Float16(float(a) op float(b))
+    ah, bh = a.astype(np.float16), b.astype(np.float16)
+    assert_exact(O.add(ah, bh), (ah.astype(np.float32) + bh.astype(np.float32)).astype(np.float16))
+    assert_exact(O.multiply(ah, bh), (ah.astype(np.float32) * bh.astype(np.float32)).astype(np.float16))
+    # bool: Add is OR, Multiply is AND (CX/arithmetic_ops.h:18-24)
+    p, q = rng.random(64) > 0.5, rng.random(64) > 0.5
+    assert np.array_equal(O.add(p, q), p | q) and np.array_equal(O.multiply(p, q), p & q)
+
+
+def test_relu_select_and_nan():
+    """C: IfLessElse(x, 0, 0, x): negative -> 0, NaN < 0 is false so NaN passes through (misc.cc:39-61)."""
+    x = np.array([-1.5, -0.0, 0.0, 2.0, np.nan, -np.inf, np.inf], np.float32)
+    got = O.relu(x)
+    assert np.array_equal(got[[0, 2, 3, 5, 6]], np.array([0, 0, 2, 0, np.inf], np.float32))
+    assert np.isnan(got[4]) and got[1] == 0
+    xi = np.array([-3, 0, 7], np.int8)
+    assert_exact(O.relu(xi), np.array([0, 0, 7], np.int8))
+
+
+def test_math_functions_within_ulps():
+    """L: exp/log/tanh/sqrt are libm calls in the reference (CX/numeric.h:55-87); compare with float64 libm."""
+    rng = np.random.default_rng(2)
+    x = (rng.standard_normal(20000) * 3).astype(np.float32)
+    for name in ('exp', 'tanh'):
+        ref = getattr(np, name)(x.astype(np.float64))
+        got = getattr(O, name)(x).astype(np.float64)
+        assert np.abs(got - ref).max() <= 2 * np.spacing(np.abs(ref).astype(np.float32)).max()
+    xp = np.abs(x) + np.float32(1e-3)
+    assert_close(O.log(xp), np.log(xp.astype(np.float64)).astype(np.float32), 1e-6)
+    assert_exact(O.sqrt(xp), np.sqrt(xp.astype(np.float64)).astype(np.float32))  # sqrt is correctly rounded
+    assert_close(O.sigmoid(x), scipy.special.expit(x.astype(np.float64)).astype(np.float32), 1e-6)
+
+
+# ---------------------------------------------------------------------------------------------
+# reductions
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize('dtype', ['float32', 'float64', 'float16', 'int32', 'int8', 'uint8', 'bool'])
+@pytest.mark.parametrize('shape,axis', [((5, 70), 1), ((5, 70), 0), ((3, 4, 5), (0, 2)), ((2, 1031), None), ((2, 3, 150), (1, 2))])
+def test_sum_integer_valued_is_exact(dtype, shape, axis):
+    """C: with small integer values every partial sum is exact, whatever the order; int/bool inputs sum to int64
+    (CX/routines/reduction.cc:34-49)."""
+    rng = np.random.default_rng(3)
+    x = rng.integers(0, 2, shape).astype(dtype) if dtype == 'bool' else rng.integers(0 if dtype == 'uint8' else -4, 5, shape).astype(dtype)
+    got = O.sum(x, axis)
+    ref = x.astype(np.int64).sum(axis)
+    assert got.dtype == (np.int64 if np.dtype(dtype).kind in 'biu' else np.dtype(dtype))
+    assert np.array_equal(got.astype(np.int64), ref)
+    assert O.sum(x, axis, True).shape == x.astype(np.int64).sum(axis, keepdims=True).shape
+
+
+def test_sum_float_within_pairwise_bound():
+    """C: |pairwise sum - exact| <= eps * (log2(n)+8) * sum|x| (any 4x8xtree order obeys it; a serial sum of 1M terms
+    would not, in general).  fp16 accumulates in float32 and rounds once (reduction.cc:105)."""
+    rng = np.random.default_rng(4)
+    for n in (7, 32, 33, 1000, 65536, 1 << 20):
+        x = rng.standard_normal((3, n)).astype(np.float32)
+        got = O.sum(x, 1).astype(np.float64)
+        exact = np.array([math.fsum(r) for r in x.astype(np.float64)])
+        bound = np.finfo(np.float32).eps * (math.log2(n) + 8) * np.abs(x).astype(np.float64).sum(1)
+        assert (np.abs(got - exact) <= bound).all(), n
+    xh = rng.standard_normal((4, 5000)).astype(np.float16)
+    exact = np.array([math.fsum(r) for r in xh.astype(np.float64)])
+    got = O.sum(xh, 1)
+    assert got.dtype == np.float16
+    assert np.abs(got.astype(np.float64) - exact).max() <= np.abs(exact).max() * 2.0 ** -10 + 0.05
+
+
+def test_amax_matches_numpy_and_propagates_nan():
+    """L + C: order independent; NaN propagates (statistics.cc:38-42) like numpy.max."""
+    rng = np.random.default_rng(5)
+    for dt in ('float32', 'float64', 'float16', 'int16', 'uint8', 'int64'):
+        x = (rng.standard_normal((6, 7, 40)) * 50).astype(dt)
+        for axis in (0, 2, (0, 2), None):
+            assert_exact(O.amax(x, axis), np.asarray(x.max(axis)))
+    x = rng.standard_normal((5, 100)).astype(np.float32)
+    x[1, 3] = np.nan
+    x[4, 99] = np.nan
+    with np.errstate(all='ignore'):
+        assert_exact(O.amax(x, 1), x.max(1))
+
+
+SORTING_LITERALS = [  # tests/chainerx_tests/unit_tests/routines_tests/test_sorting.py:11-29, valid params
+    (np.asarray(0), None), (np.asarray(-1), None), (np.asarray(float('inf')), None), (np.asarray(float('nan')), None),
+    (np.asarray(-float('inf')), None), (np.asarray([4, 1, 4, 1]), None), (np.asarray([4, 1, 4, 1]), 0),
+    (np.asarray([[4, 4, 1, 1], [4, 1, 4, 1]]), 0), (np.asarray([[4, 4, 1, 1], [4, 1, 4, 1]]).T, 1), (np.asarray([-2, -3, -1]), 0),
+    (np.asarray([-0.0, +0.0, +0.0, -0.0]), None), (np.asarray([[True, True, False, False], [True, False, True, False]]), 0),
+    (np.ones((2, 3)), 1), (np.ones((2, 3)), -2),
+]
+
+
+@pytest.mark.parametrize('x,axis', SORTING_LITERALS, ids=[str(i) for i in range(len(SORTING_LITERALS))])
+def test_argmax_reference_literals(x, axis):
+    """R: the reference's argmax test takes numpy.argmax as the expected value on these inputs."""
+    for dt in ([x.dtype] if x.dtype == np.bool_ else [np.float32, np.float64, np.float16, np.int32]):
+        if np.dtype(dt).kind != 'f' and not np.isfinite(np.asarray(x, np.float64)).all():
+            continue
+        xa = x.astype(dt)
+        got = O.argmax(xa, axis)
+        assert got.dtype == np.int64
+        assert np.array_equal(got, np.argmax(xa, axis))
+
+
+def test_argmax_tie_free_and_in_block_ties():
+    """C: without ties the answer is unique (= numpy.argmax); ties inside one 32-element block and in the <=3-element
+    tail resolve to the first index like numpy (reduce.h:28-31,65,69-72).  The rule between blocks is unpinned."""
+    rng = np.random.default_rng(6)
+    for n in (1, 5, 31, 32, 33, 100, 4096, 70001):
+        x = rng.permutation(n * 3).reshape(3, n).astype(np.float32)
+        assert np.array_equal(O.argmax(x, 1), x.argmax(1))
+        assert np.array_equal(O.argmax(x.T.copy(), 0), x.argmax(1))
+    x = rng.integers(0, 3, (200, 32)).astype(np.float32)  # many ties, single block
+    assert np.array_equal(O.argmax(x, 1), x.argmax(1))
+    x = rng.integers(0, 3, (200, 35)).astype(np.float32)
+    x[:, :32] -= 10  # maximum lives in the 3-element tail
+    assert np.array_equal(O.argmax(x, 1), x.argmax(1))
+
+
+def test_argmax_nan_rule():
+    """C from the functor (reduction.cc:44-52): replace iff accum.argmax < 0 or accum.max < next.max, so a NaN never
+    replaces a number, and a leading NaN is never replaced (inside one block, where visiting order is index order)."""
+    x = np.array([[1, np.nan, 3, 2], [np.nan, 5, 6, 7], [np.nan, np.nan, np.nan, np.nan]], np.float32)
+    assert O.argmax(x, 1).tolist() == [2, 0, 0]
+
+
+def test_log_softmax_matches_scipy():
+    rng = np.random.default_rng(8)
+    for dt, tol in (('float32', 2e-6), ('float64', 1e-14)):
+        x = (rng.standard_normal((37, 1000)) * 4).astype(dt)
+        ref = scipy.special.log_softmax(x.astype(np.float64), axis=1)
+        got = O.log_softmax(x, 1)
+        assert got.dtype == np.dtype(dt)
+        assert np.abs(got - ref).max() / np.abs(ref).max() <= tol
+        assert np.allclose(np.exp(got.astype(np.float64)).sum(1), 1, atol=1e-5)  # rows are distributions
+        assert_close(O.log_softmax(x + np.asarray(3, dt), 1), got, 1e-5 if dt == 'float32' else 1e-12)  # shift invariance
+
+
+def test_softmax_cross_entropy_closed_form():
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal((100, 10)).astype(np.float32)
+    t = rng.integers(0, 10, 100).astype(np.int32)
+    ref = -scipy.special.log_softmax(x.astype(np.float64), axis=1)[np.arange(100), t].mean()
+    assert abs(float(O.softmax_cross_entropy(x, t)) - ref) <= 1e-6 * abs(ref)
+
+
+# ---------------------------------------------------------------------------------------------
+# dot / conv
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize('dtype,tol', [('float32', 2e-6), ('float64', 1e-14), ('float16', 2e-3)])
+def test_dot_matches_float64_matmul(dtype, tol):
+    """L: numpy float64 matmul; integer-valued operands give the exact result."""
+    rng = np.random.default_rng(10)
+    for m, k, n in ((7, 33, 5), (64, 64, 64), (100, 784, 50), (1, 1, 1)):
+        a = rng.standard_normal((m, k)).astype(dtype)
+        b = (rng.standard_normal((k, n)) / np.sqrt(k)).astype(dtype)
+        ref = a.astype(np.float64) @ b.astype(np.float64)
+        got = O.dot(a, b)
+        assert got.dtype == np.dtype(dtype)
+        assert np.abs(got - ref).max() / max(np.abs(ref).max(), 1e-30) <= tol
+        ai = rng.integers(-3, 4, (m, k)).astype(dtype)
+        bi = rng.integers(-3, 4, (k, n)).astype(dtype)
+        assert np.array_equal(O.dot(ai, bi).astype(np.int64), ai.astype(np.int64) @ bi.astype(np.int64))
+
+
+def brute_conv(x, w, b, stride, pad, cover_all):
+    """Definition of the cross-correlation (float64), out extent from the definition of cover_all: the last window must
+    cover the last padded input element (chainer.utils.conv.get_conv_outsize)."""
+    N, C, H, W = x.shape
+    K, _, R, S = w.shape
+    sh, sw = stride
+    ph, pw = pad
+
+    def out_dim(d, k, s, p):
+        if cover_all:
+            return (d + 2 * p - k + s - 1) // s + 1
+        return (d + 2 * p - k) // s + 1
+    OH, OW = out_dim(H, R, sh, ph), out_dim(W, S, sw, pw)
+    out = np.zeros((N, K, OH, OW))
+    x = x.astype(np.float64)
+    w = w.astype(np.float64)
+    for n, k, oh, ow in itertools.product(range(N), range(K), range(OH), range(OW)):
+        acc = 0.0
+        for c, r, s in itertools.product(range(C), range(R), range(S)):
+            ih, iw = oh * sh - ph + r, ow * sw - pw + s
+            if 0 <= ih < H and 0 <= iw < W:
+                acc += x[n, c, ih, iw] * w[k, c, r, s]
+        out[n, k, oh, ow] = acc + (float(b[k]) if b is not None else 0.0)
+    return out
+
+
+CONV_GRID = [  # the 2-D rows of the reference's grid, tests/.../routines_tests/test_connection.py:183-203
+    ((2, 3, 4, 4), (2, 3, 3, 3), False, (2, 2), (2, 0)),
+    ((2, 3, 4, 4), (2, 3, 3, 3), True, (1, 1), (0, 0)),
+    ((1, 3, 4, 4), (2, 3, 3, 3), True, (1, 2), (1, 1)),
+    ((1, 3, 4, 4), (2, 3, 3, 3), True, (2, 2), (2, 0)),
+    ((2, 5, 7, 6), (4, 5, 1, 1), True, (2, 2), (0, 0)),
+    ((1, 2, 9, 9), (3, 2, 7, 7), False, (2, 2), (3, 3)),
+]
+
+
+@pytest.mark.parametrize('xs,ws,bias,stride,pad', CONV_GRID)
+@pytest.mark.parametrize('cover_all', [False, True])
+@pytest.mark.parametrize('dtype,tol', [('float32', 2e-6), ('float64', 1e-14), ('float16', 2e-3)])
+def test_conv_matches_brute_force(xs, ws, bias, stride, pad, cover_all, dtype, tol):
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal(xs).astype(dtype)
+    w = (rng.standard_normal(ws) / np.sqrt(np.prod(ws[1:]))).astype(dtype)
+    b = rng.standard_normal(ws[0]).astype(dtype) if bias else None
+    ref = brute_conv(x, w, b, stride, pad, cover_all)
+    got = O.conv(x, w, b, stride, pad, cover_all)
+    assert got.shape == ref.shape and got.dtype == np.dtype(dtype)
+    assert np.abs(got - ref).max() / np.abs(ref).max() <= tol
+
+
+def test_conv_out_dim_formula():
+    """C: CX/routines/connection.cc:37-49."""
+    assert O.conv_out_dim(224, 7, 2, 3, False) == 112
+    assert O.conv_out_dim(112, 3, 2, 1, False) == 56
+    assert O.conv_out_dim(112, 3, 2, 0, False) == 55
+    assert O.conv_out_dim(112, 3, 2, 0, True) == 56
+    assert O.conv_out_dim(4, 3, 2, 2, False) == 3
+    with pytest.raises(ValueError):
+        O.conv_out_dim(2, 5, 1, 0, False)
+
+
+def test_linear_is_dot_with_transposed_weight_plus_bias():
+    rng = np.random.default_rng(12)
+    x = rng.standard_normal((9, 4, 5)).astype(np.float32)
+    w = rng.standard_normal((7, 20)).astype(np.float32)
+    b = rng.standard_normal(7).astype(np.float32)
+    ref = x.reshape(9, 20).astype(np.float64) @ w.T.astype(np.float64) + b
+    assert_close(O.linear(x, w, b), ref.astype(np.float32), 2e-6)
+
+
+# ---------------------------------------------------------------------------------------------
+# normalization / pooling / indexing / lstm
+# ---------------------------------------------------------------------------------------------
+BN_GRID = [  # tests/.../routines_tests/test_normalization.py:50-58 (<= 4-D rows)
+    ((3, 2), (2,), None), ((5, 4, 3, 2), (4, 3, 2), None), ((5, 4, 3, 2), (4, 3, 2), (0,)), ((5, 4, 3, 2), (4,), (0, 2, 3)),
+]
+
+
+@pytest.mark.parametrize('xs,rs,axis', BN_GRID)
+@pytest.mark.parametrize('dtype,tol', [('float32', 2e-6), ('float64', 1e-14), ('float16', 4e-3)])
+def test_fixed_batch_norm_closed_form(xs, rs, axis, dtype, tol):
+    rng = np.random.default_rng(13)
+    x = rng.standard_normal(xs).astype(dtype)
+    g, b, m = [rng.standard_normal(rs).astype(dtype) for _ in range(3)]
+    v = rng.uniform(0.5, 1.5, rs).astype(dtype)
+    axes = (0,) if axis is None else axis
+    red = tuple(1 if i in axes else d for i, d in enumerate(xs))
+    g64, b64, m64, v64 = [p.astype(np.float64).reshape(red) for p in (g, b, m, v)]
+    ref = (x.astype(np.float64) - m64) / np.sqrt(v64 + 2e-5) * g64 + b64
+    got = O.fixed_batch_norm(x, g, b, m, v, 2e-5, axis)
+    assert got.dtype == np.dtype(dtype) and got.shape == x.shape
+    assert np.abs(got - ref).max() / np.abs(ref).max() <= tol
+
+
+POOL_GRID = [  # 2-D rows of tests/.../routines_tests/test_pooling.py:15-27,121-133
+    ((2, 3, 4, 4), (3, 3), (1, 1), (0, 0)), ((2, 3, 4, 4), (3, 3), None, (0, 0)), ((1, 3, 4, 4), (3, 3), (1, 2), (1, 1)),
+    ((1, 3, 4, 4), (3, 3), (2, 2), (2, 0)), ((2, 4, 9, 8), (3, 2), (2, 1), (1, 0)),
+]
+
+
+def brute_pool(x, ksize, stride, pad, cover_all, mode):
+    N, C, H, W = x.shape
+    kh, kw = ksize
+    sh, sw = stride if stride is not None else ksize
+    ph, pw = pad
+    ex_h = sh - 1 if cover_all else 0
+    ex_w = sw - 1 if cover_all else 0
+    OH = (H + 2 * ph - kh + ex_h) // sh + 1
+    OW = (W + 2 * pw - kw + ex_w) // sw + 1
+    out = np.zeros((N, C, OH, OW))
+    for n, c, oh, ow in itertools.product(range(N), range(C), range(OH), range(OW)):
+        vals = []
+        for r, s in itertools.product(range(kh), range(kw)):
+            ih, iw = oh * sh - ph + r, ow * sw - pw + s
+            if 0 <= ih < H and 0 <= iw < W:
+                vals.append(float(x[n, c, ih, iw]))
+        if mode == 'max':
+            out[n, c, oh, ow] = max(vals) if vals else -np.inf
+        elif mode == 'zero':
+            out[n, c, oh, ow] = sum(vals) / (kh * kw)
+        else:
+            out[n, c, oh, ow] = sum(vals) / len(vals) if vals else np.nan
+    return out
+
+
+@pytest.mark.parametrize('xs,ksize,stride,pad', POOL_GRID)
+@pytest.mark.parametrize('dtype', ['float32', 'float64', 'float16'])
+def test_pooling_matches_brute_force(xs, ksize, stride, pad, dtype):
+    rng = np.random.default_rng(14)
+    x = rng.standard_normal(xs).astype(dtype)
+    for cover_all in (False, True):
+        ref = brute_pool(x, ksize, stride, pad, cover_all, 'max')
+        got = O.max_pool(x, ksize, stride, pad, cover_all)
+        assert got.dtype == x.dtype and np.array_equal(got.astype(np.float64), ref)  # max is exact
+    tol = {'float32': 2e-6, 'float64': 1e-14, 'float16': 3e-3}[dtype]
+    for mode in ('zero', 'ignore'):
+        ref = brute_pool(x, ksize, stride, pad, False, mode)
+        got = O.average_pool(x, ksize, stride, pad, mode).astype(np.float64)
+        fin = np.isfinite(ref)
+        assert np.abs(got[fin] - ref[fin]).max() <= tol * max(1.0, np.abs(ref[fin]).max())
+
+
+def test_take_modes():
+    """L + B: numpy.take for in-range / wrap / clip; out-of-range raises in the default mode (indexing.cc:68-74)."""
+    rng = np.random.default_rng(15)
+    a = rng.integers(-100, 100, (6, 5, 4)).astype(np.int16)
+    idx = rng.integers(-5, 5, (3, 2))
+    for axis in (0, 1, 2):
+        dim = a.shape[axis]
+        ii = np.clip(idx, -dim, dim - 1)
+        assert_exact(O.take(a, ii, axis), np.take(a, ii, axis=axis))
+        big = idx * 7
+        assert_exact(O.take(a, big, axis, 'wrap'), np.take(a, big, axis=axis, mode='wrap'))
+        assert_exact(O.take(a, big, axis, 'clip'), np.take(a, np.clip(big, 0, dim - 1), axis=axis))
+    with pytest.raises(IndexError):
+        O.take(a, np.array([6]), 0)
+    with pytest.raises(IndexError):
+        O.take(a, np.array([-7]), 0, 'raise')
+
+
+def test_lstm_closed_form():
+    """C: gate k of unit j at column 4j+k; a=tanh, i,f,o=sigmoid; c' = a*i + f*c; h = o*tanh(c') (connection.cc:396-446)."""
+    rng = np.random.default_rng(17)
+    c = rng.standard_normal((5, 6))
+    x = rng.standard_normal((5, 24))
+    a, i, f, o = [x[:, k::4] for k in range(4)]
+    sig = scipy.special.expit
+    c_ref = np.tanh(a) * sig(i) + sig(f) * c
+    h_ref = sig(o) * np.tanh(c_ref)
+    for dt, tol in (('float64', 1e-14), ('float32', 1e-6)):
+        h, cn = O.lstm(c.astype(dt), x.astype(dt))
+        assert np.abs(h - h_ref).max() <= tol and np.abs(cn - c_ref).max() <= tol
