@@ -1,0 +1,637 @@
+// ChainerX backend plugin `hip`: the Backend/Device pair and the kernel classes that forward to
+// the C ABI of libhipcx.so (include/hipcx.h).
+//
+// Build inside a ChainerX checkout (it needs libchainerx's headers and its abseil/gsl-lite), e.g.
+//   hipcc -std=c++14 -fPIC -shared -I<chainerx_cc> -I<abseil> -I<gsl-lite>/include -I<repo>/include \
+//         hip_backend.cc -L<repo>/chainer_amd -lhipcx -lchainerx -o $CHAINERX_PATH/backends/hip.so
+// The file name is the backend name: chainerx.get_device('hip:0') loads it through
+// Context::GetBackend (chainerx/context.cc:84-111), which looks up the two extern "C" functions at
+// the bottom of this file.
+//
+// Every kernel below follows the conventions of the reference's own backends
+// (chainerx/native/kernel_regist.h:15-70, chainerx/cuda/kernel_regist.h:15-17): check devices, make
+// the device current, cast inputs to out's dtype with AsType, honour strides/offset, launch
+// asynchronously on the default stream.  Nothing is registered from the native backend's registry:
+// its kernels would dereference device pointers on the host.
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <map>
+#include <memory>
+#include <mutex>
+#include <string>
+#include <tuple>
+#include <utility>
+#include <vector>
+
+#include <absl/types/optional.h>
+
+#include "chainerx/array.h"
+#include "chainerx/axes.h"
+#include "chainerx/backend.h"
+#include "chainerx/backend_util.h"
+#include "chainerx/context.h"
+#include "chainerx/device.h"
+#include "chainerx/dims.h"
+#include "chainerx/dtype.h"
+#include "chainerx/error.h"
+#include "chainerx/kernel_registry.h"
+#include "chainerx/kernels/arithmetic.h"
+#include "chainerx/kernels/connection.h"
+#include "chainerx/kernels/creation.h"
+#include "chainerx/kernels/explog.h"
+#include "chainerx/kernels/hyperbolic.h"
+#include "chainerx/kernels/indexing.h"
+#include "chainerx/kernels/linalg.h"
+#include "chainerx/kernels/logic.h"
+#include "chainerx/kernels/misc.h"
+#include "chainerx/kernels/normalization.h"
+#include "chainerx/kernels/pooling.h"
+#include "chainerx/kernels/reduction.h"
+#include "chainerx/kernels/sorting.h"
+#include "chainerx/kernels/statistics.h"
+#include "chainerx/native/native_backend.h"
+#include "chainerx/routines/connection.h"
+#include "chainerx/routines/creation.h"
+#include "chainerx/scalar.h"
+#include "chainerx/shape.h"
+
+#include "hipcx.h"
+
+namespace chainerx {
+namespace hip {
+namespace {
+
+void CheckHip(hipError_t e, const char* what) {
+    if (e != hipSuccess) throw BackendError{what, ": ", hipGetErrorString(e)};
+}
+
+// hipcx_status -> the ChainerX exception class named by it (chainerx/error.h:48-95).
+void Check(int status) {
+    if (status == HIPCX_OK) return;
+    std::string msg = hipcx_last_error();
+    switch (status) {
+        case HIPCX_DIMENSION_ERROR: throw DimensionError{msg};
+        case HIPCX_DTYPE_ERROR: throw DtypeError{msg};
+        case HIPCX_NOT_IMPLEMENTED_ERROR: throw NotImplementedError{msg};
+        case HIPCX_INDEX_ERROR: throw IndexError{msg};
+        case HIPCX_BACKEND_ERROR: throw BackendError{msg};
+        case HIPCX_DEVICE_ERROR: throw DeviceError{msg};
+        default: throw ChainerxError{msg};
+    }
+}
+
+class SetDeviceScope {
+public:
+    explicit SetDeviceScope(int index) {
+        CheckHip(hipGetDevice(&prev_), "hipGetDevice");
+        if (prev_ != index) CheckHip(hipSetDevice(index), "hipSetDevice");
+        index_ = index;
+    }
+    ~SetDeviceScope() {
+        if (prev_ != index_) (void)hipSetDevice(prev_);
+    }
+    SetDeviceScope(const SetDeviceScope&) = delete;
+    SetDeviceScope& operator=(const SetDeviceScope&) = delete;
+
+private:
+    int prev_{0};
+    int index_{0};
+};
+
+// Array -> hipcx_array: data = raw_data + offset (chainerx/backend_util.h:10-13), byte strides as they are.
+hipcx_array ToC(const Array& a) {
+    hipcx_array c{};
+    c.data = internal::GetRawOffsetData(a);
+    c.dtype = static_cast<int32_t>(a.dtype());  // same numeric codes (chainerx/dtype.h:19-29)
+    c.ndim = a.ndim();
+    for (int8_t i = 0; i < a.ndim(); ++i) {
+        c.shape[i] = a.shape()[i];
+        c.strides[i] = a.strides()[i];
+    }
+    return c;
+}
+
+hipcx_scalar ToC(Scalar s) {
+    hipcx_scalar c{};
+    switch (s.kind()) {
+        case DtypeKind::kBool:
+            c.kind = HIPCX_KIND_BOOL;
+            c.i = static_cast<bool>(s) ? 1 : 0;
+            break;
+        case DtypeKind::kInt:
+        case DtypeKind::kUInt:
+            c.kind = HIPCX_KIND_INT;
+            c.i = static_cast<int64_t>(s);
+            break;
+        default:
+            c.kind = HIPCX_KIND_FLOAT;
+            c.f = static_cast<double>(s);
+            break;
+    }
+    return c;
+}
+
+std::vector<int8_t> ToC(const Axes& axes) { return std::vector<int8_t>(axes.begin(), axes.end()); }
+
+// Caching device allocator: power-of-two-ish size classes of 512-byte units, free blocks kept per
+// class, everything released and the request retried once when hipMalloc fails.  Buffers are
+// shared_ptr<void> whose deleter hands the block back; the pool outlives its buffers through a
+// shared_ptr held by each deleter, and the deleter never throws.
+class MemoryPool : public std::enable_shared_from_this<MemoryPool> {
+public:
+    explicit MemoryPool(int device_index) : device_index_{device_index} {}
+    ~MemoryPool() { FreeAll(); }
+
+    std::shared_ptr<void> Allocate(size_t bytesize) {
+        if (bytesize == 0) return nullptr;  // native does the same (native_device/memory.cc:14-19)
+        size_t size = RoundUp(bytesize);
+        void* ptr = nullptr;
+        {
+            std::lock_guard<std::mutex> lock{mutex_};
+            auto it = free_.find(size);
+            if (it != free_.end() && !it->second.empty()) {
+                ptr = it->second.back();
+                it->second.pop_back();
+            }
+        }
+        if (ptr == nullptr) {
+            SetDeviceScope scope{device_index_};
+            hipError_t e = hipMalloc(&ptr, size);
+            if (e != hipSuccess) {
+                (void)hipGetLastError();
+                FreeAll();
+                CheckHip(hipMalloc(&ptr, size), "hipMalloc");
+            }
+        }
+        std::shared_ptr<MemoryPool> self = shared_from_this();
+        return std::shared_ptr<void>{ptr, [self, size](void* p) noexcept { self->Release(p, size); }};
+    }
+
+private:
+    static size_t RoundUp(size_t n) {
+        constexpr size_t kUnit = 512;
+        size_t units = (n + kUnit - 1) / kUnit;
+        size_t cls = 1;
+        while (cls < units) cls += (cls < 8 ? 1 : cls / 8);  // 12.5 % steps above 4 KiB
+        return cls * kUnit;
+    }
+    void Release(void* p, size_t size) noexcept {
+        try {
+            std::lock_guard<std::mutex> lock{mutex_};
+            free_[size].push_back(p);
+        } catch (...) {
+            (void)hipFree(p);
+        }
+    }
+    void FreeAll() noexcept {
+        std::lock_guard<std::mutex> lock{mutex_};
+        for (auto& kv : free_) {
+            for (void* p : kv.second) (void)hipFree(p);
+        }
+        free_.clear();
+    }
+
+    int device_index_;
+    std::mutex mutex_;
+    std::map<size_t, std::vector<void*>> free_;
+};
+
+class HipBackend;
+
+class HipDevice : public Device {
+public:
+    HipDevice(Backend& backend, int index) : Device{backend, index}, pool_{std::make_shared<MemoryPool>(index)} {}
+
+    std::shared_ptr<void> Allocate(size_t bytesize) override { return pool_->Allocate(bytesize); }
+
+    std::shared_ptr<void> MakeDataFromForeignPointer(const std::shared_ptr<void>& data) override {
+        if (data == nullptr) return data;
+        hipPointerAttribute_t attr{};
+        SetDeviceScope scope{index()};
+        hipError_t e = hipPointerGetAttributes(&attr, data.get());
+        if (e != hipSuccess || attr.device != index()) {
+            (void)hipGetLastError();
+            throw ChainerxError{"Memory is not a HIP allocation of device ", name()};
+        }
+        return data;
+    }
+
+    void MemoryCopyFrom(void* dst, const void* src, size_t bytesize, Device& src_device) override {
+        if (bytesize == 0) return;
+        SetDeviceScope scope{index()};
+        if (&src_device == this || dynamic_cast<HipDevice*>(&src_device) != nullptr) {
+            CheckHip(hipMemcpyAsync(dst, src, bytesize, hipMemcpyDeviceToDevice, nullptr), "hipMemcpyAsync");
+        } else {  // native (host) source: blocking, like the CUDA backend (cuda/cuda_device/memory.cc:94-110)
+            CheckHip(hipMemcpy(dst, src, bytesize, hipMemcpyHostToDevice), "hipMemcpy");
+        }
+    }
+
+    void MemoryCopyTo(void* dst, const void* src, size_t bytesize, Device& dst_device) override {
+        if (bytesize == 0) return;
+        SetDeviceScope scope{index()};
+        if (&dst_device == this || dynamic_cast<HipDevice*>(&dst_device) != nullptr) {
+            CheckHip(hipMemcpyAsync(dst, src, bytesize, hipMemcpyDeviceToDevice, nullptr), "hipMemcpyAsync");
+        } else {
+            CheckHip(hipMemcpy(dst, src, bytesize, hipMemcpyDeviceToHost), "hipMemcpy");
+        }
+    }
+
+    std::shared_ptr<void> TransferDataFrom(Device& src_device, const std::shared_ptr<void>& src_ptr, size_t offset, size_t bytesize) override {
+        std::shared_ptr<void> dst = Allocate(bytesize);
+        MemoryCopyFrom(dst.get(), static_cast<const uint8_t*>(src_ptr.get()) + offset, bytesize, src_device);
+        return dst;
+    }
+
+    std::shared_ptr<void> TransferDataTo(Device& dst_device, const std::shared_ptr<void>& src_ptr, size_t offset, size_t bytesize) override {
+        std::shared_ptr<void> dst = dst_device.Allocate(bytesize);
+        MemoryCopyTo(dst.get(), static_cast<const uint8_t*>(src_ptr.get()) + offset, bytesize, dst_device);
+        return dst;
+    }
+
+    std::shared_ptr<void> FromHostMemory(const std::shared_ptr<void>& src_ptr, size_t bytesize) override {
+        std::shared_ptr<void> dst = Allocate(bytesize);
+        if (bytesize != 0) {
+            SetDeviceScope scope{index()};
+            CheckHip(hipMemcpy(dst.get(), src_ptr.get(), bytesize, hipMemcpyHostToDevice), "hipMemcpy");
+        }
+        return dst;
+    }
+
+    void Synchronize() override { Check(hipcx_synchronize(index())); }
+
+private:
+    std::shared_ptr<MemoryPool> pool_;
+};
+
+}  // namespace
+
+class HipBackend : public Backend {
+public:
+    using Backend::Backend;
+
+    std::string GetName() const override { return "hip"; }
+
+    int GetDeviceCount() const override {
+        int n = 0;
+        Check(hipcx_device_count(&n));
+        return n;
+    }
+
+    // Transfers inside the backend and to/from the native (host) backend, like cuda/cuda_backend.cc:49-59.
+    bool SupportsTransfer(Device& src_device, Device& dst_device) override {
+        Backend& src = src_device.backend();
+        Backend& dst = dst_device.backend();
+        if (&src == this) return &dst == this || nullptr != dynamic_cast<native::NativeBackend*>(&dst);
+        if (&dst == this) return nullptr != dynamic_cast<native::NativeBackend*>(&src);
+        return false;
+    }
+
+    static KernelRegistry& GetGlobalKernelRegistry() {
+        static KernelRegistry* global_kernel_registry = new KernelRegistry{};
+        return *global_kernel_registry;
+    }
+
+protected:
+    KernelRegistry& GetParentKernelRegistry() override { return GetGlobalKernelRegistry(); }
+
+private:
+    std::unique_ptr<Device> CreateDevice(int index) override {
+        int n = GetDeviceCount();
+        if (index < 0 || index >= n) throw std::out_of_range{"The index number (= " + std::to_string(index) + ") is out of range"};
+        return std::make_unique<HipDevice>(*this, index);
+    }
+};
+
+namespace {
+
+#define HIPCX_REGISTER_KERNEL(key_kernel_cls, kernel_cls) \
+    static chainerx::internal::KernelRegistrar<chainerx::hip::HipBackend, key_kernel_cls, kernel_cls> s_hip_backend_kernel_##kernel_cls{};
+
+Array Cast(const Array& a, Dtype dtype) { return a.dtype() == dtype ? a : a.AsType(dtype); }
+
+// ---- elementwise: (x1, x2, out), (x1, Scalar, out), (Scalar, x2, out), (x, out) ----
+#define HIPCX_BINARY_KERNEL(Name, entry)                                                  \
+    class Hip##Name##Kernel : public Name##Kernel {                                       \
+    public:                                                                               \
+        void Call(const Array& x1, const Array& x2, const Array& out) override {          \
+            Device& device = x1.device();                                                 \
+            device.CheckDevicesCompatible(x1, x2, out);                                   \
+            SetDeviceScope scope{device.index()};                                         \
+            hipcx_array a = ToC(Cast(x1, out.dtype())), b = ToC(Cast(x2, out.dtype())), o = ToC(out); \
+            Check(entry(&a, &b, &o, nullptr));                                            \
+        }                                                                                 \
+    };                                                                                    \
+    HIPCX_REGISTER_KERNEL(Name##Kernel, Hip##Name##Kernel)
+
+#define HIPCX_BINARY_AS_KERNEL(Name, entry)                                               \
+    class Hip##Name##Kernel : public Name##Kernel {                                       \
+    public:                                                                               \
+        void Call(const Array& x1, Scalar x2, const Array& out) override {                \
+            Device& device = x1.device();                                                 \
+            device.CheckDevicesCompatible(x1, out);                                       \
+            SetDeviceScope scope{device.index()};                                         \
+            hipcx_array a = ToC(Cast(x1, out.dtype())), o = ToC(out);                     \
+            Check(entry(&a, ToC(x2), &o, nullptr));                                       \
+        }                                                                                 \
+    };                                                                                    \
+    HIPCX_REGISTER_KERNEL(Name##Kernel, Hip##Name##Kernel)
+
+#define HIPCX_UNARY_KERNEL(Name, entry)                                                   \
+    class Hip##Name##Kernel : public Name##Kernel {                                       \
+    public:                                                                               \
+        void Call(const Array& x, const Array& out) override {                            \
+            Device& device = x.device();                                                  \
+            device.CheckDevicesCompatible(x, out);                                        \
+            SetDeviceScope scope{device.index()};                                         \
+            hipcx_array a = ToC(Cast(x, out.dtype())), o = ToC(out);                      \
+            Check(entry(&a, &o, nullptr));                                                \
+        }                                                                                 \
+    };                                                                                    \
+    HIPCX_REGISTER_KERNEL(Name##Kernel, Hip##Name##Kernel)
+
+HIPCX_BINARY_KERNEL(Add, hipcx_add)
+HIPCX_BINARY_KERNEL(Subtract, hipcx_subtract)
+HIPCX_BINARY_KERNEL(Multiply, hipcx_multiply)
+HIPCX_BINARY_KERNEL(Divide, hipcx_divide)
+HIPCX_BINARY_AS_KERNEL(AddAS, hipcx_add_as)
+HIPCX_BINARY_AS_KERNEL(SubtractAS, hipcx_subtract_as)
+HIPCX_BINARY_AS_KERNEL(MultiplyAS, hipcx_multiply_as)
+HIPCX_BINARY_AS_KERNEL(DivideAS, hipcx_divide_as)
+HIPCX_UNARY_KERNEL(Exp, hipcx_exp)
+HIPCX_UNARY_KERNEL(Log, hipcx_log)
+HIPCX_UNARY_KERNEL(Tanh, hipcx_tanh)
+HIPCX_UNARY_KERNEL(Sqrt, hipcx_sqrt)
+
+class HipDivideSAKernel : public DivideSAKernel {
+public:
+    void Call(Scalar x1, const Array& x2, const Array& out) override {
+        Device& device = x2.device();
+        device.CheckDevicesCompatible(x2, out);
+        SetDeviceScope scope{device.index()};
+        hipcx_array b = ToC(Cast(x2, out.dtype())), o = ToC(out);
+        Check(hipcx_divide_sa(ToC(x1), &b, &o, nullptr));
+    }
+};
+HIPCX_REGISTER_KERNEL(DivideSAKernel, HipDivideSAKernel)
+
+// Comparisons: the operands share one dtype (promoted here as native/native_device/logic.cc does), out is bool.
+#define HIPCX_COMPARE_KERNEL(Name, entry)                                                 \
+    class Hip##Name##Kernel : public Name##Kernel {                                       \
+    public:                                                                               \
+        void Call(const Array& x1, const Array& x2, const Array& out) override {          \
+            Device& device = x1.device();                                                 \
+            device.CheckDevicesCompatible(x1, x2, out);                                   \
+            SetDeviceScope scope{device.index()};                                         \
+            Dtype dtype = PromoteTypes(x1.dtype(), x2.dtype());                           \
+            hipcx_array a = ToC(Cast(x1, dtype)), b = ToC(Cast(x2, dtype)), o = ToC(out); \
+            Check(entry(&a, &b, &o, nullptr));                                            \
+        }                                                                                 \
+    };                                                                                    \
+    HIPCX_REGISTER_KERNEL(Name##Kernel, Hip##Name##Kernel)
+
+HIPCX_COMPARE_KERNEL(Equal, hipcx_equal)
+HIPCX_COMPARE_KERNEL(NotEqual, hipcx_not_equal)
+HIPCX_COMPARE_KERNEL(Greater, hipcx_greater)
+HIPCX_COMPARE_KERNEL(GreaterEqual, hipcx_greater_equal)
+
+#define HIPCX_SELECT_ASSA_KERNEL(Name, entry)                                                          \
+    class Hip##Name##Kernel : public Name##Kernel {                                                    \
+    public:                                                                                            \
+        void Call(const Array& x1, Scalar x2, Scalar pos, const Array& neg, const Array& out) override { \
+            Device& device = x1.device();                                                              \
+            device.CheckDevicesCompatible(x1, neg, out);                                               \
+            SetDeviceScope scope{device.index()};                                                      \
+            hipcx_array a = ToC(Cast(x1, out.dtype())), n = ToC(Cast(neg, out.dtype())), o = ToC(out); \
+            Check(entry(&a, ToC(x2), ToC(pos), &n, &o, nullptr));                                      \
+        }                                                                                              \
+    };                                                                                                 \
+    HIPCX_REGISTER_KERNEL(Name##Kernel, Hip##Name##Kernel)
+
+HIPCX_SELECT_ASSA_KERNEL(IfLessElseASSA, hipcx_if_less_else_assa)        // ReLU = Maximum(x, 0), routines/misc.cc:210-216
+HIPCX_SELECT_ASSA_KERNEL(IfGreaterElseASSA, hipcx_if_greater_else_assa)  // Minimum(x, scalar)
+
+class HipIfGreaterElseAAAAKernel : public IfGreaterElseAAAAKernel {
+public:
+    void Call(const Array& x1, const Array& x2, const Array& pos, const Array& neg, const Array& out) override {
+        Device& device = x1.device();
+        device.CheckDevicesCompatible(x1, x2, pos, neg, out);
+        SetDeviceScope scope{device.index()};
+        Dtype dt = out.dtype();
+        hipcx_array a = ToC(Cast(x1, dt)), b = ToC(Cast(x2, dt)), p = ToC(Cast(pos, dt)), n = ToC(Cast(neg, dt)), o = ToC(out);
+        Check(hipcx_if_greater_else_aaaa(&a, &b, &p, &n, &o, nullptr));
+    }
+};
+HIPCX_REGISTER_KERNEL(IfGreaterElseAAAAKernel, HipIfGreaterElseAAAAKernel)
+
+// ---- creation ----
+class HipCopyKernel : public CopyKernel {
+public:
+    void Call(const Array& a, const Array& out) override {
+        Device& device = a.device();
+        device.CheckDevicesCompatible(a, out);
+        SetDeviceScope scope{device.index()};
+        hipcx_array ca = ToC(a), o = ToC(out);  // the kernel casts: every (In, Out) dtype pair
+        Check(hipcx_copy(&ca, &o, nullptr));
+    }
+};
+HIPCX_REGISTER_KERNEL(CopyKernel, HipCopyKernel)
+
+class HipFillKernel : public FillKernel {
+public:
+    void Call(const Array& out, Scalar value) override {
+        SetDeviceScope scope{out.device().index()};
+        hipcx_array o = ToC(out);
+        Check(hipcx_fill(&o, ToC(value), nullptr));
+    }
+};
+HIPCX_REGISTER_KERNEL(FillKernel, HipFillKernel)
+
+class HipArangeKernel : public ArangeKernel {
+public:
+    void Call(Scalar start, Scalar step, const Array& out) override {
+        SetDeviceScope scope{out.device().index()};
+        hipcx_array o = ToC(out);
+        Check(hipcx_arange(ToC(start), ToC(step), &o, nullptr));
+    }
+};
+HIPCX_REGISTER_KERNEL(ArangeKernel, HipArangeKernel)
+
+// ---- reductions ----
+using ReduceEntry = int (*)(const hipcx_array*, const int8_t*, int, const hipcx_array*, void*, size_t, void*);
+
+void CallReduce(ReduceEntry entry, const Array& a, const Axes& axis, const Array& out) {
+    Device& device = a.device();
+    device.CheckDevicesCompatible(a, out);
+    SetDeviceScope scope{device.index()};
+    hipcx_array ca = ToC(a), o = ToC(out);
+    std::vector<int8_t> ax = ToC(axis);
+    size_t ws_bytes = hipcx_reduce_workspace_size(&ca, ax.data(), static_cast<int>(ax.size()), &o);
+    std::shared_ptr<void> ws = device.Allocate(ws_bytes);  // returned to the pool after the launch: stream order keeps it safe
+    Check(entry(&ca, ax.data(), static_cast<int>(ax.size()), &o, ws.get(), ws_bytes, nullptr));
+}
+
+class HipSumKernel : public SumKernel {
+public:
+    void Call(const Array& a, const Axes& axis, const Array& out) override { CallReduce(hipcx_sum, a, axis, out); }
+};
+HIPCX_REGISTER_KERNEL(SumKernel, HipSumKernel)
+
+class HipAMaxKernel : public AMaxKernel {
+public:
+    void Call(const Array& a, const Axes& axis, const Array& out) override { CallReduce(hipcx_amax, a, axis, out); }
+};
+HIPCX_REGISTER_KERNEL(AMaxKernel, HipAMaxKernel)
+
+class HipArgMaxKernel : public ArgMaxKernel {
+public:
+    void Call(const Array& a, const Axes& axis, const Array& out) override { CallReduce(hipcx_argmax, a, axis, out); }
+};
+HIPCX_REGISTER_KERNEL(ArgMaxKernel, HipArgMaxKernel)
+
+// ---- dot / conv ----
+class HipDotKernel : public DotKernel {
+public:
+    void Call(const Array& a, const Array& b, const Array& out) override {
+        Device& device = a.device();
+        device.CheckDevicesCompatible(a, b, out);
+        SetDeviceScope scope{device.index()};
+        hipcx_array ca = ToC(Cast(a, out.dtype())), cb = ToC(Cast(b, out.dtype())), o = ToC(out);
+        size_t ws_bytes = hipcx_dot_workspace_size(&ca, &cb, &o);
+        std::shared_ptr<void> ws = device.Allocate(ws_bytes);
+        Check(hipcx_dot(&ca, &cb, &o, ws.get(), ws_bytes, nullptr));
+    }
+};
+HIPCX_REGISTER_KERNEL(DotKernel, HipDotKernel)
+
+int64_t OutDim(int64_t in, int64_t k, int64_t s, int64_t p, bool cover_all) {
+    int64_t n = hipcx_conv_out_dim(in, k, s, p, cover_all ? 1 : 0);
+    if (n <= 0) throw DimensionError{"Output size should be positive."};
+    return n;
+}
+
+class HipConvKernel : public ConvKernel {
+public:
+    Array Call(const Array& x, const Array& w, const absl::optional<Array>& b, const Dims& stride, const Dims& pad, bool cover_all,
+               Dtype out_dtype, const absl::optional<Array>& out) override {
+        if (out.has_value()) throw NotImplementedError{"Passing out as an argument is not yet supported."};  // like native conv.cc:52-55
+        if (x.ndim() != 4) throw NotImplementedError{"hip conv supports 2 spatial dimensions."};
+        Device& device = x.device();
+        device.CheckDevicesCompatible(x, w);
+        if (b.has_value()) device.CheckDevicesCompatible(*b);
+        SetDeviceScope scope{device.index()};
+        Shape out_shape{x.shape()[0], w.shape()[0], OutDim(x.shape()[2], w.shape()[2], stride[0], pad[0], cover_all),
+                        OutDim(x.shape()[3], w.shape()[3], stride[1], pad[1], cover_all)};
+        Array y = Empty(out_shape, out_dtype, device);  // C-contiguous NCHW, like cuda/cuda_conv.cc:311
+        Array xc = Cast(x, out_dtype), wc = Cast(w, out_dtype);
+        hipcx_array cx = ToC(xc), cw = ToC(wc), cy = ToC(y), cb{};
+        if (b.has_value()) cb = ToC(Cast(*b, out_dtype));
+        int64_t st[2] = {stride[0], stride[1]}, pd[2] = {pad[0], pad[1]};
+        size_t ws_bytes = hipcx_conv_workspace_size(&cx, &cw, &cy);
+        std::shared_ptr<void> ws = device.Allocate(ws_bytes);
+        Check(hipcx_conv(&cx, &cw, b.has_value() ? &cb : nullptr, st, pd, cover_all ? 1 : 0, &cy, ws.get(), ws_bytes, nullptr));
+        return y;
+    }
+};
+HIPCX_REGISTER_KERNEL(ConvKernel, HipConvKernel)
+
+// ---- fixed batch norm ----
+class HipFixedBatchNormKernel : public FixedBatchNormKernel {
+public:
+    Array Call(const Array& x, const Array& gamma, const Array& beta, const Array& mean, const Array& var, Scalar eps, const Axes& axis,
+               const absl::optional<Array>& out) override {
+        if (out.has_value()) throw NotImplementedError{"Passing out as an argument is not yet supported."};
+        Device& device = x.device();
+        device.CheckDevicesCompatible(x, gamma, beta, mean, var);
+        SetDeviceScope scope{device.index()};
+        Array y = EmptyLike(x, device);
+        hipcx_array cx = ToC(x), cg = ToC(gamma), cb = ToC(beta), cm = ToC(mean), cv = ToC(var), cy = ToC(y);
+        std::vector<int8_t> ax = ToC(axis);
+        Check(hipcx_fixed_batch_norm(&cx, &cg, &cb, &cm, &cv, ToC(eps), ax.data(), static_cast<int>(ax.size()), &cy, nullptr));
+        return y;
+    }
+};
+HIPCX_REGISTER_KERNEL(FixedBatchNormKernel, HipFixedBatchNormKernel)
+
+// ---- pooling (forward only: the states are inert) ----
+class HipMaxPoolGradState : public MaxPoolGradState {};
+class HipAveragePoolGradState : public AveragePoolGradState {};
+
+Shape PoolOutShape(const Array& x, const Dims& k, const Dims& s, const Dims& p, bool cover_all) {
+    if (x.ndim() != 4) throw NotImplementedError{"hip pooling supports 2 spatial dimensions."};
+    return Shape{x.shape()[0], x.shape()[1], OutDim(x.shape()[2], k[0], s[0], p[0], cover_all), OutDim(x.shape()[3], k[1], s[1], p[1], cover_all)};
+}
+
+class HipMaxPoolKernel : public MaxPoolKernel {
+public:
+    std::tuple<Array, std::unique_ptr<MaxPoolGradState>> Call(const Array& x, Dims kernel_size, Dims stride, Dims pad, bool cover_all,
+                                                             bool return_state, const absl::optional<Array>& out) override {
+        if (out.has_value()) throw NotImplementedError{"Passing out as an argument is not yet supported."};
+        Device& device = x.device();
+        SetDeviceScope scope{device.index()};
+        Array y = Empty(PoolOutShape(x, kernel_size, stride, pad, cover_all), x.dtype(), device);
+        hipcx_array cx = ToC(x), cy = ToC(y);
+        int64_t k[2] = {kernel_size[0], kernel_size[1]}, s[2] = {stride[0], stride[1]}, p[2] = {pad[0], pad[1]};
+        Check(hipcx_max_pool(&cx, k, s, p, cover_all ? 1 : 0, &cy, nullptr));
+        std::unique_ptr<MaxPoolGradState> state = return_state ? std::make_unique<HipMaxPoolGradState>() : nullptr;
+        return std::make_tuple(std::move(y), std::move(state));
+    }
+};
+HIPCX_REGISTER_KERNEL(MaxPoolKernel, HipMaxPoolKernel)
+
+class HipAveragePoolKernel : public AveragePoolKernel {
+public:
+    std::tuple<Array, std::unique_ptr<AveragePoolGradState>> Call(const Array& x, const Dims& kernel_size, const Dims& stride, const Dims& pad,
+                                                                 AveragePoolPadMode pad_mode, bool return_state,
+                                                                 const absl::optional<Array>& out) override {
+        if (out.has_value()) throw NotImplementedError{"Passing out as an argument is not yet supported."};
+        Device& device = x.device();
+        SetDeviceScope scope{device.index()};
+        Array y = Empty(PoolOutShape(x, kernel_size, stride, pad, false), x.dtype(), device);
+        hipcx_array cx = ToC(x), cy = ToC(y);
+        int64_t k[2] = {kernel_size[0], kernel_size[1]}, s[2] = {stride[0], stride[1]}, p[2] = {pad[0], pad[1]};
+        int mode = pad_mode == AveragePoolPadMode::kZero ? HIPCX_PAD_ZERO : HIPCX_PAD_IGNORE;
+        Check(hipcx_average_pool(&cx, k, s, p, mode, &cy, nullptr));
+        std::unique_ptr<AveragePoolGradState> state = return_state ? std::make_unique<HipAveragePoolGradState>() : nullptr;
+        return std::make_tuple(std::move(y), std::move(state));
+    }
+};
+HIPCX_REGISTER_KERNEL(AveragePoolKernel, HipAveragePoolKernel)
+
+// ---- take ----
+class HipTakeKernel : public TakeKernel {
+public:
+    void Call(const Array& a, const Array& indices, int8_t axis, const Array& out, IndexBoundsMode mode) override {
+        Device& device = a.device();
+        device.CheckDevicesCompatible(a, indices, out);
+        SetDeviceScope scope{device.index()};
+        hipcx_array ca = ToC(a), ci = ToC(indices), co = ToC(out);
+        int m = HIPCX_BOUNDS_DEFAULT;
+        switch (mode) {
+            case IndexBoundsMode::kRaise: m = HIPCX_BOUNDS_RAISE; break;
+            case IndexBoundsMode::kWrap: m = HIPCX_BOUNDS_WRAP; break;
+            case IndexBoundsMode::kClip: m = HIPCX_BOUNDS_CLIP; break;
+            default: break;
+        }
+        bool checks = m == HIPCX_BOUNDS_DEFAULT || m == HIPCX_BOUNDS_RAISE;
+        std::shared_ptr<void> flag = checks ? device.Allocate(sizeof(int32_t)) : nullptr;
+        if (checks) CheckHip(hipMemsetAsync(flag.get(), 0, sizeof(int32_t), nullptr), "hipMemsetAsync");
+        Check(hipcx_take(&ca, &ci, axis, &co, m, static_cast<int32_t*>(flag.get()), nullptr));
+        if (checks) {  // native raises IndexError on an out-of-range index (native_device/indexing.cc:68-74)
+            int32_t host = 0;
+            CheckHip(hipMemcpy(&host, flag.get(), sizeof(int32_t), hipMemcpyDeviceToHost), "hipMemcpy");
+            if (host != 0) throw IndexError{"Index is out of bounds for axis ", static_cast<int>(axis), " with size ", a.shape()[axis]};
+        }
+    }
+};
+HIPCX_REGISTER_KERNEL(TakeKernel, HipTakeKernel)
+
+}  // namespace
+}  // namespace hip
+}  // namespace chainerx
+
+// NOLINTNEXTLINE(cppcoreguidelines-owning-memory)
+extern "C" chainerx::Backend* CreateBackend(chainerx::Context& ctx) { return new chainerx::hip::HipBackend{ctx}; }
+
+// NOLINTNEXTLINE(cppcoreguidelines-owning-memory)
+extern "C" void DestroyBackend(chainerx::Backend* backend) { delete backend; }
