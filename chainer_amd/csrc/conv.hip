@@ -2,6 +2,7 @@
 // implicit-GEMM core.  The arithmetic contract is the native backend's: products of the stored
 // values accumulated in fp32 (fp64 for float64) and rounded once to the output dtype
 // (CX/native/native_device/dot.cc:181-227, conv.cc:41-89).
+#include <algorithm>
 #include <cstdlib>
 #include <utility>
 #include <vector>
@@ -9,6 +10,7 @@
 #include "igemm.h"
 #include "igemm_pipe.h"
 #include "layout_kernels.h"
+#include "nchw_conv.h"
 
 namespace hipcx {
 namespace {
@@ -90,6 +92,8 @@ void LaunchShape(IGemmArgs<T> p, bool fast16, bool fast8, hipStream_t stream) {
     }
     CheckLaunch("igemm");
 }
+
+size_t RoundUpTo(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 bool Aligned(const void* ptr, int64_t bytes) { return reinterpret_cast<uintptr_t>(ptr) % bytes == 0; }
 
@@ -187,6 +191,137 @@ int64_t ElemStride(const hipcx_array* a, int axis, const char* name) {
     HIPCX_REQUIRE(a->strides[axis] % it == 0, HIPCX_NOT_IMPLEMENTED_ERROR,
                   std::string(name) + ": byte strides must be multiples of the item size");
     return a->strides[axis] / it;
+}
+
+
+// ---- float16 NCHW-native path (nchw_conv.h) ----
+struct NchwPlan {
+    bool ok = false;
+    int taps = 1, npx = 1, ck = 32, wpx = 4, wch = 1, maxi = 1;
+    int nrow = 0, nslot = 0;
+    size_t wp_bytes = 0;
+    int lds_bytes = 0;
+};
+
+NchwPlan PlanNchw(const hipcx_array* x, const hipcx_array* w, const hipcx_array* out, const int64_t* stride, const int64_t* pad) {
+    NchwPlan pl;
+    static const bool enabled = [] { const char* e = getenv("HIPCX_CONV_NCHW"); return e == nullptr || e[0] != '0'; }();
+    if (!enabled || x->dtype != HIPCX_FLOAT16) return pl;
+    if (!IsContiguous(x) || !IsContiguous(out)) return pl;
+    const int64_t N = x->shape[0], C = x->shape[1], H = x->shape[2], W = x->shape[3];
+    const int64_t K = w->shape[0], R = w->shape[2], S = w->shape[3];
+    const int64_t OH = out->shape[2], OW = out->shape[3];
+    if (N * C * H * W * 2 >= (1LL << 31) || N * K * OH * OW * 2 >= (1LL << 31) || K * C * R * S * 2 >= (1LL << 31)) return pl;
+    if (reinterpret_cast<uintptr_t>(x->data) % 16 != 0 || reinterpret_cast<uintptr_t>(out->data) % 8 != 0) return pl;
+    const bool is1 = R == 1 && S == 1 && pad[0] == 0 && pad[1] == 0 && stride[0] == stride[1];
+    const bool is3 = R == 3 && S == 3 && pad[0] == 1 && pad[1] == 1 && stride[0] == 1 && stride[1] == 1;
+    if (!is1 && !is3) return pl;
+    const int64_t P = OH * OW;
+    auto pick = [](int64_t n) { return n % 8 == 0 ? 8 : n % 4 == 0 ? 4 : n % 2 == 0 ? 2 : 1; };
+    if (is1) {
+        if (C % 32 != 0) return pl;
+        pl.taps = 1;
+        pl.ck = 32;
+        pl.npx = stride[0] == 1 ? pick(P) : 1;
+        if (K <= 64) {
+            pl.wpx = 4, pl.wch = 1;
+            pl.maxi = pl.npx >= 4 ? 1 : pl.npx == 2 ? 2 : 4;
+        } else {
+            pl.wpx = 2, pl.wch = 2;
+            pl.maxi = pl.npx >= 2 ? 1 : 2;
+        }
+        pl.nslot = 64 * pl.wpx;
+    } else {
+        if (C % 16 != 0) return pl;
+        pl.taps = 9;
+        pl.ck = 16;
+        pl.npx = pick(W);
+        pl.wpx = 4, pl.wch = 1;
+        pl.maxi = pl.npx >= 4 ? 1 : pl.npx == 2 ? 2 : 4;
+        const int64_t BM = 256;
+        int64_t rows = (BM + W - 2) / W + 1;
+        int64_t cross = (BM + P - 2) / P;
+        pl.nrow = static_cast<int>(rows + 2 * cross + 2);
+        pl.nslot = pl.nrow * static_cast<int>(W + 2);
+        int64_t items = static_cast<int64_t>(pl.nrow) * (W / pl.npx) * (pl.ck / 8);
+        if (items > static_cast<int64_t>(pl.maxi) * 256) return pl;
+    }
+    const int cg = pl.ck / 8;
+    const int bn = 64 * pl.wch;
+    pl.lds_bytes = 2 * (cg * pl.nslot * 16 + pl.taps * cg * bn * 16) + pl.npx * 16;
+    if (pl.lds_bytes > 160 * 1024) return pl;
+    pl.wp_bytes = RoundUpTo(static_cast<size_t>(K) * C * R * S * 2, 256);
+    pl.ok = true;
+    return pl;
+}
+
+template <int TAPS, int WPX, int WCH, int CK, int NPX, int MAXI>
+void LaunchNchwKernel(const NchwConvArgs& a, int lds_bytes, hipStream_t stream) {
+    auto kern = NchwConvKernel<TAPS, WPX, WCH, CK, NPX, MAXI>;
+    static int configured = 0;
+    if (lds_bytes > configured) {
+        HIPCX_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes));
+        configured = lds_bytes;
+    }
+    int64_t total = static_cast<int64_t>(a.tiles_m) * a.tiles_n;
+    dim3 grid(static_cast<unsigned>((total + 7) / 8 * 8)), block(64 * WPX * WCH);
+    hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, a);
+    CheckLaunch("nchw_conv");
+}
+
+void RunNchw(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, const NchwPlan& pl, const int64_t* stride,
+             const hipcx_array* out, char* workspace, hipStream_t stream) {
+    NchwConvArgs a{};
+    a.x = static_cast<const half_t*>(x->data);
+    a.wp = reinterpret_cast<const half_t*>(workspace);
+    a.bias = b ? static_cast<const half_t*>(b->data) : nullptr;
+    a.bias_stride = b ? b->strides[0] / 2 : 0;
+    a.out = static_cast<half_t*>(out->data);
+    a.N = static_cast<int>(x->shape[0]);
+    a.C = static_cast<int>(x->shape[1]);
+    a.H = static_cast<int>(x->shape[2]);
+    a.W = static_cast<int>(x->shape[3]);
+    a.K = static_cast<int>(w->shape[0]);
+    a.OH = static_cast<int>(out->shape[2]);
+    a.OW = static_cast<int>(out->shape[3]);
+    a.stride = static_cast<int>(stride[0]);
+    a.P = a.OH * a.OW;
+    a.M = a.N * a.P;
+    const int BM = 64 * pl.wpx, BN = 64 * pl.wch;
+    a.tiles_m = (a.M + BM - 1) / BM;
+    a.tiles_n = (a.K + BN - 1) / BN;
+    a.nrow = pl.nrow;
+    a.nslot = pl.nslot;
+    a.x_bytes = static_cast<unsigned>(static_cast<int64_t>(a.N) * a.C * a.H * a.W * 2);
+    const int RS = static_cast<int>(w->shape[2] * w->shape[3]);
+    a.wp_bytes = static_cast<unsigned>(static_cast<int64_t>(a.K) * a.C * RS * 2);
+    a.vec_out = a.P % 4 == 0 ? 1 : 0;
+    {
+        int64_t groups = static_cast<int64_t>(a.C / 8) * RS * a.K;
+        hipLaunchKernelGGL(NchwRepackFiltersKernel, dim3(static_cast<unsigned>((groups + 255) / 256)), dim3(256), 0, stream,
+                           static_cast<const half_t*>(w->data), reinterpret_cast<half_t*>(workspace), a.K, a.C, RS,
+                           static_cast<int>(w->shape[3]), w->strides[0] / 2, w->strides[1] / 2, w->strides[2] / 2, w->strides[3] / 2);
+        CheckLaunch("nchw_repack_filters");
+    }
+    double flops = 2.0 * a.M * a.K * RS * a.C;
+    double bytes = 2.0 * (static_cast<double>(a.N) * a.C * a.H * a.W + static_cast<double>(a.K) * RS * a.C + static_cast<double>(a.M) * a.K);
+    ProfileScope prof(stream, flops, bytes);
+    const int key = pl.taps * 1000 + pl.wpx * 100 + pl.npx * 10 + pl.maxi;
+    switch (key) {
+        case 1000 + 400 + 80 + 1: LaunchNchwKernel<1, 4, 1, 32, 8, 1>(a, pl.lds_bytes, stream); break;
+        case 1000 + 400 + 40 + 1: LaunchNchwKernel<1, 4, 1, 32, 4, 1>(a, pl.lds_bytes, stream); break;
+        case 1000 + 400 + 20 + 2: LaunchNchwKernel<1, 4, 1, 32, 2, 2>(a, pl.lds_bytes, stream); break;
+        case 1000 + 400 + 10 + 4: LaunchNchwKernel<1, 4, 1, 32, 1, 4>(a, pl.lds_bytes, stream); break;
+        case 1000 + 200 + 80 + 1: LaunchNchwKernel<1, 2, 2, 32, 8, 1>(a, pl.lds_bytes, stream); break;
+        case 1000 + 200 + 40 + 1: LaunchNchwKernel<1, 2, 2, 32, 4, 1>(a, pl.lds_bytes, stream); break;
+        case 1000 + 200 + 20 + 1: LaunchNchwKernel<1, 2, 2, 32, 2, 1>(a, pl.lds_bytes, stream); break;
+        case 1000 + 200 + 10 + 2: LaunchNchwKernel<1, 2, 2, 32, 1, 2>(a, pl.lds_bytes, stream); break;
+        case 9000 + 400 + 80 + 1: LaunchNchwKernel<9, 4, 1, 16, 8, 1>(a, pl.lds_bytes, stream); break;
+        case 9000 + 400 + 40 + 1: LaunchNchwKernel<9, 4, 1, 16, 4, 1>(a, pl.lds_bytes, stream); break;
+        case 9000 + 400 + 20 + 2: LaunchNchwKernel<9, 4, 1, 16, 2, 2>(a, pl.lds_bytes, stream); break;
+        case 9000 + 400 + 10 + 4: LaunchNchwKernel<9, 4, 1, 16, 1, 4>(a, pl.lds_bytes, stream); break;
+        default: throw Error(HIPCX_CHAINERX_ERROR, "nchw conv: no kernel for plan " + std::to_string(key));
+    }
 }
 
 // How a convolution is staged.  The MFMA kernel wants the reduction axis (r, s, c) contiguous in
@@ -431,7 +566,10 @@ size_t hipcx_conv_workspace_size(const hipcx_array* x, const hipcx_array* w, con
         // report the full-plane size
         int64_t one[2] = {1, 1}, zero[2] = {0, 0};
         ConvPlan pl = PlanConv(x, w, one, zero);
-        return pl.x_bytes + pl.w_bytes;
+        size_t need = pl.x_bytes + pl.w_bytes;
+        // the NCHW-native float16 path needs room for the packed filters only; report the larger of the two
+        if (x->dtype == HIPCX_FLOAT16) need = std::max(need, RoundUpTo(static_cast<size_t>(TotalSize(w)) * 2, 256));
+        return need;
     } catch (...) {
         return 0;
     }
@@ -443,6 +581,14 @@ int hipcx_conv(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b,
         CheckConv(x, w, b, stride, pad, cover_all, out);
         if (TotalSize(out) == 0) return;
         hipStream_t st = AsStream(stream);
+        NchwPlan npl = PlanNchw(x, w, out, stride, pad);
+        if (npl.ok) {
+            HIPCX_REQUIRE(workspace != nullptr && workspace_bytes >= npl.wp_bytes, HIPCX_CHAINERX_ERROR,
+                          "conv workspace too small: need " + std::to_string(npl.wp_bytes) + " bytes");
+            HIPCX_REQUIRE(reinterpret_cast<uintptr_t>(workspace) % 16 == 0, HIPCX_CHAINERX_ERROR, "workspace must be 16-byte aligned");
+            RunNchw(x, w, b, npl, stride, out, static_cast<char*>(workspace), st);
+            return;
+        }
         ConvPlan pl = PlanConv(x, w, stride, pad);
         size_t need = pl.x_bytes + pl.w_bytes;
         if (need > 0) {

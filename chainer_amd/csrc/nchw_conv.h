@@ -1,0 +1,356 @@
+// Convolution forward for float16 activations that are C-contiguous NCHW on both sides -- the layout every
+// ChainerX routine allocates -- without a layout-conversion pass.
+//
+//   out[n, k, oh, ow] = bias[k] + sum_{c, r, s} x[n, c, oh*stride - pad + r, ow*stride - pad + s] * w[k, c, r, s]
+//
+// Supported geometries: 1x1 (any stride, no padding) and 3x3 (stride 1, padding 1).
+//
+// Work decomposition.  Output pixels are flattened to m = (n*OH + oh)*OW + ow; a workgroup owns BM consecutive
+// pixels x BN output channels and loops over the input channels in chunks of CK.  For every chunk
+//   * the activations the tile needs (for 3x3: its rows plus one halo row above and below, all columns) are
+//     loaded with buffer loads of NPX consecutive pixels from 8 channel planes, transposed in registers and written
+//     to LDS as 16-byte groups of 8 channels per pixel: patch[channel group][slot] (slot = pixel position in a
+//     zero-bordered patch whose rows are W+2 slots wide, with an all-zero row between images);
+//   * the filters of the chunk arrive pre-packed ([C/8][R*S][K][8], see NchwRepackFilters) and are copied to LDS as
+//     weights[channel group][tap][BN] 16-byte groups.
+// Both LDS arrays are exactly the operand layout of v_mfma_f32_32x32x16_f16 (lane = row/column, 8 consecutive
+// reduction indices per lane), so a fragment is one conflict-free ds_read_b128 of consecutive 16-byte groups, and
+// a 3x3 tap is a constant slot offset into the same patch: the patch is written once and read nine times.
+// Two LDS stages; global loads of chunk i+1 are in flight while chunk i is multiplied; one barrier per chunk.
+// All addresses are computed once per workgroup; inside the channel loop only a scalar offset advances, and
+// out-of-range loads are served as zeros by the buffer bounds check instead of branches.
+//
+// Accumulator orientation: pixels are MFMA rows, output channels MFMA columns, so a lane ends up with 4
+// consecutive pixels of one channel -- an 8-byte store into NCHW memory.
+#pragma once
+
+#include "common.h"
+#include "igemm.h"
+
+namespace hipcx {
+
+struct NchwConvArgs {
+    const half_t* x;
+    const half_t* wp;    // packed filters [C/8][taps][K][8]
+    const half_t* bias;  // may be null
+    half_t* out;
+    int N, C, H, W;  // input
+    int K;           // output channels
+    int OH, OW;      // output plane
+    int stride;      // spatial stride (1x1 only; 3x3 runs with 1)
+    int M;           // N*OH*OW
+    int P;           // OH*OW
+    int tiles_m, tiles_n;
+    int nrow;   // 3x3: rows of the LDS patch (upper bound over tiles)
+    int nslot;  // slots per channel group in the LDS patch
+    int64_t bias_stride;
+    unsigned x_bytes, wp_bytes;
+    int vec_out;  // P % 4 == 0: a lane's 4 consecutive pixels share an image and are 8-byte aligned
+};
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t MakeRsrc(const void* ptr, unsigned bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(ptr), 0, static_cast<int>(bytes), 0x00020000);
+}
+
+// NPX pixels (NPX * 2 bytes) of one channel plane as dwords.
+template <int NPX>
+struct PixVec {
+    static constexpr int DW = NPX >= 2 ? NPX / 2 : 1;
+    unsigned d[DW];
+};
+
+template <int NPX>
+__device__ __forceinline__ PixVec<NPX> BufLoad(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
+    PixVec<NPX> v;
+    if constexpr (NPX == 8) {
+        Bytes16 t = __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0);
+        v.d[0] = t.x;
+        v.d[1] = t.y;
+        v.d[2] = t.z;
+        v.d[3] = t.w;
+    } else if constexpr (NPX == 4) {
+        Bytes8 t = __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 0);
+        v.d[0] = t.x;
+        v.d[1] = t.y;
+    } else if constexpr (NPX == 2) {
+        v.d[0] = __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0);
+    } else {
+        v.d[0] = __builtin_amdgcn_raw_buffer_load_b16(r, voff, soff, 0);  // zero-extended
+    }
+    return v;
+}
+
+// 8 channel planes x NPX pixels -> NPX groups of 8 channels (16 bytes each).
+template <int NPX>
+__device__ __forceinline__ void Transpose8(const PixVec<NPX> (&in)[8], Bytes16 (&out)[NPX]) {
+#pragma unroll
+    for (int e = 0; e < NPX; ++e) {
+        unsigned dw[4];
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            if constexpr (NPX == 1) {
+                dw[d] = in[2 * d].d[0] | (in[2 * d + 1].d[0] << 16);
+            } else {
+                unsigned a = in[2 * d].d[e / 2], b = in[2 * d + 1].d[e / 2];
+                dw[d] = (e & 1) ? __builtin_amdgcn_perm(b, a, 0x07060302u) : __builtin_amdgcn_perm(b, a, 0x05040100u);
+            }
+        }
+        out[e] = Bytes16{dw[0], dw[1], dw[2], dw[3]};
+    }
+}
+
+template <int TAPS, int WPX, int WCH, int CK, int NPX, int MAXI>
+__global__ __launch_bounds__(64 * WPX * WCH) void NchwConvKernel(NchwConvArgs p) {
+    constexpr int PW = 2, CW = 2;  // wave tile: 64 pixels x 64 channels
+    constexpr int NT = 64 * WPX * WCH;
+    constexpr int BM = 32 * PW * WPX;
+    constexpr int BN = 32 * CW * WCH;
+    constexpr int CG = CK / 8;    // 16-byte channel groups per chunk
+    constexpr int KS = CK / 16;   // MFMA reduction steps per chunk and tap
+    constexpr int WITEMS = TAPS * CG * BN;
+    constexpr int WPT = (WITEMS + NT - 1) / NT;
+
+    extern __shared__ __align__(16) char lds[];
+    const int patch_bytes = CG * p.nslot * 16;
+    const int stage_bytes = patch_bytes + WITEMS * 16;
+    const int dump_off = 2 * stage_bytes;  // NPX * 16 bytes that absorb the writes of idle load slots
+
+    int tile_m, tile_n;
+    if (!TileOf(p.tiles_m, p.tiles_n, tile_m, tile_n)) return;
+    const int m0 = tile_m * BM;
+    const int n0 = tile_n * BN;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wpx = wave % WPX;
+    const int wch = wave / WPX;
+    const int lr = lane & 31;
+    const int g = lane >> 5;
+    const int HW = p.H * p.W;
+    const int W2 = p.W + 2;
+
+    // ---- patch geometry (3x3): first patch row of this tile in "padded row" coordinates n*(H+2) + h + 1 ----
+    int base_row = 0, last_row = 0;
+    if constexpr (TAPS == 9) {
+        int m_last = min(m0 + BM, p.M) - 1;
+        int nf = m0 / p.P, hf = (m0 - nf * p.P) / p.W;
+        int nl = m_last / p.P, hl = (m_last - nl * p.P) / p.W;
+        base_row = nf * (p.H + 2) + hf;          // one above the first output row
+        last_row = nl * (p.H + 2) + hl + 2;      // one below the last output row
+    }
+
+    // ---- activation load slots of this thread ----
+    int xvoff[MAXI];  // byte offset of (n, channel group base, first pixel) in x; out of range for idle slots
+    int xlds[MAXI];   // byte offset of the first pixel's group inside a stage
+#pragma unroll
+    for (int i = 0; i < MAXI; ++i) {
+        int it = tid + i * NT;
+        bool valid;
+        int voff = 0, loff = 0;
+        if constexpr (TAPS == 9) {
+            const int wchunks = p.W / NPX;
+            const int per_cg = p.nrow * wchunks;
+            int cg = it / per_cg;
+            int q = it - cg * per_cg;
+            int pr = q / wchunks;
+            int wc = q - pr * wchunks;
+            int grow = base_row + pr;
+            int n = grow / (p.H + 2);
+            int hh = grow - n * (p.H + 2) - 1;
+            valid = cg < CG && grow <= last_row && n < p.N && hh >= 0 && hh < p.H;
+            voff = (((n * p.C + cg * 8) * p.H + hh) * p.W + wc * NPX) * 2;
+            loff = (cg * p.nslot + pr * W2 + wc * NPX + 1) * 16;
+        } else {
+            constexpr int per_cg = BM / NPX;
+            int cg = it / per_cg;
+            int q = it - cg * per_cg;
+            int m = m0 + q * NPX;
+            valid = cg < CG && m < p.M;
+            int n = m / p.P;
+            int pix = m - n * p.P;
+            int oh = pix / p.OW;
+            int ow = pix - oh * p.OW;
+            voff = (((n * p.C + cg * 8) * p.H + oh * p.stride) * p.W + ow * p.stride) * 2;
+            loff = (cg * p.nslot + q * NPX) * 16;
+        }
+        xvoff[i] = valid ? voff : 0x7fffffff;  // beyond the buffer: the load returns zeros
+        xlds[i] = valid ? loff : -1;           // idle slots write into the dump area
+    }
+    // ---- filter load slots ----
+    int wvoff[WPT];
+    int wlds[WPT];
+#pragma unroll
+    for (int i = 0; i < WPT; ++i) {
+        int wi = tid + i * NT;
+        int cg = wi / (TAPS * BN);
+        int rest = wi - cg * (TAPS * BN);
+        int tap = rest / BN;
+        int kl = rest - tap * BN;
+        bool valid = wi < WITEMS && n0 + kl < p.K;
+        wvoff[i] = valid ? ((cg * TAPS + tap) * p.K + n0 + kl) * 16 : 0x7fffffff;
+        wlds[i] = wi < WITEMS ? patch_bytes + wi * 16 : -1;
+    }
+
+    const __amdgpu_buffer_rsrc_t xr = MakeRsrc(p.x, p.x_bytes);
+    const __amdgpu_buffer_rsrc_t wr = MakeRsrc(p.wp, p.wp_bytes);
+
+    PixVec<NPX> xreg[MAXI][8];
+    Bytes16 wreg[WPT];
+    auto load_chunk = [&](int ci) {
+        const int xs = ci * CK * HW * 2;
+#pragma unroll
+        for (int i = 0; i < MAXI; ++i) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) xreg[i][j] = BufLoad<NPX>(xr, xvoff[i], xs + j * HW * 2);
+        }
+        const int ws = ci * (CG * TAPS) * p.K * 16;
+#pragma unroll
+        for (int i = 0; i < WPT; ++i) wreg[i] = __builtin_amdgcn_raw_buffer_load_b128(wr, wvoff[i], ws, 0);
+    };
+    auto store_chunk = [&](char* stage) {
+#pragma unroll
+        for (int i = 0; i < MAXI; ++i) {
+            Bytes16 t[NPX];
+            Transpose8<NPX>(xreg[i], t);
+            char* dst = xlds[i] >= 0 ? stage + xlds[i] : lds + dump_off;
+#pragma unroll
+            for (int e = 0; e < NPX; ++e) *reinterpret_cast<Bytes16*>(dst + e * 16) = t[e];
+        }
+#pragma unroll
+        for (int i = 0; i < WPT; ++i) {
+            if (wlds[i] >= 0) *reinterpret_cast<Bytes16*>(stage + wlds[i]) = wreg[i];
+        }
+    };
+
+    // ---- fragment addresses ----
+    int aoff[PW];  // byte offset of this lane's pixel group (channel group g) inside a stage, tap (0,0) of a 3x3 = slot - W2 - 1
+#pragma unroll
+    for (int a = 0; a < PW; ++a) {
+        int m = m0 + (wpx * PW + a) * 32 + lr;
+        int slot;
+        if constexpr (TAPS == 9) {
+            int mm = m < p.M ? m : p.M - 1;
+            int n = mm / p.P;
+            int pix = mm - n * p.P;
+            int h = pix / p.W;
+            int w = pix - h * p.W;
+            slot = (n * (p.H + 2) + h + 1 - base_row) * W2 + w + 1;
+            slot -= W2 + 1;  // tap (r, s) adds r * W2 + s
+        } else {
+            slot = (wpx * PW + a) * 32 + lr;
+        }
+        aoff[a] = (g * p.nslot + slot) * 16;
+    }
+    const int boff = patch_bytes + (g * TAPS * BN + wch * CW * 32 + lr) * 16;
+    const int a_ks = 2 * p.nslot * 16;  // advance of one 16-channel reduction step in the patch
+
+    float16_t acc[PW][CW];
+#pragma unroll
+    for (int a = 0; a < PW; ++a) {
+#pragma unroll
+        for (int b = 0; b < CW; ++b) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.f;
+        }
+    }
+
+    auto compute = [&](const char* stage) {
+#pragma unroll
+        for (int tap = 0; tap < TAPS; ++tap) {
+            const int toff = TAPS == 9 ? ((tap / 3) * W2 + (tap % 3)) * 16 : 0;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                Bytes16 af[PW], bf[CW];
+#pragma unroll
+                for (int a = 0; a < PW; ++a) af[a] = *reinterpret_cast<const Bytes16*>(stage + aoff[a] + toff + ks * a_ks);
+#pragma unroll
+                for (int b = 0; b < CW; ++b) {
+                    bf[b] = *reinterpret_cast<const Bytes16*>(stage + boff + ((ks * 2 * TAPS + tap) * BN + b * 32) * 16);
+                }
+#pragma unroll
+                for (int a = 0; a < PW; ++a) {
+#pragma unroll
+                    for (int b = 0; b < CW; ++b) MfmaTile<half_t>(af[a], bf[b], acc[a][b]);
+                }
+            }
+        }
+    };
+
+    // ---- pipeline ----
+    load_chunk(0);
+    if constexpr (TAPS == 9) {  // borders of both patches must read as zero; nothing ever writes them
+        for (int off = tid * 16; off < 2 * stage_bytes; off += NT * 16) *reinterpret_cast<Bytes16*>(lds + off) = Bytes16(0);
+        __syncthreads();
+    }
+    store_chunk(lds);
+    __syncthreads();
+    const int nchunks = p.C / CK;
+    for (int ci = 0; ci < nchunks; ++ci) {
+        char* cur = lds + (ci & 1) * stage_bytes;
+        char* nxt = lds + ((ci + 1) & 1) * stage_bytes;
+        const bool more = ci + 1 < nchunks;
+        if (more) load_chunk(ci + 1);
+        compute(cur);
+        if (more) store_chunk(nxt);
+        __syncthreads();
+    }
+
+    // ---- epilogue: lane holds channel column lr of each 32-wide sub-tile, pixel rows 8*(v/4) + 4*g + v%4 ----
+#pragma unroll
+    for (int b = 0; b < CW; ++b) {
+        int n = n0 + (wch * CW + b) * 32 + lr;
+        if (n >= p.K) continue;
+        float bias = p.bias != nullptr ? static_cast<float>(p.bias[n * p.bias_stride]) : 0.f;
+#pragma unroll
+        for (int a = 0; a < PW; ++a) {
+#pragma unroll
+            for (int vq = 0; vq < 4; ++vq) {
+                int m = m0 + (wpx * PW + a) * 32 + vq * 8 + g * 4;
+                if (m >= p.M) continue;
+                float v[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = acc[a][b][vq * 4 + e] + bias;
+                if (p.vec_out) {
+                    int img = m / p.P;
+                    int pix = m - img * p.P;
+                    struct alignas(8) Out4 {
+                        half_t e[4];
+                    } pack;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) pack.e[e] = static_cast<half_t>(v[e]);
+                    *reinterpret_cast<Out4*>(p.out + (static_cast<int64_t>(img) * p.K + n) * p.P + pix) = pack;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        int me = m + e;
+                        if (me >= p.M) continue;
+                        int img = me / p.P;
+                        int pix = me - img * p.P;
+                        p.out[(static_cast<int64_t>(img) * p.K + n) * p.P + pix] = static_cast<half_t>(v[e]);
+                    }
+                }
+            }
+        }
+    }
+}
+
+// w[K][C][R][S] (element strides wsK, wsC, wsR, wsS) -> wp[C/8][R*S][K][8].
+__global__ __launch_bounds__(256) void NchwRepackFiltersKernel(const half_t* w, half_t* wp, int K, int C, int RS, int S, int64_t wsK,
+                                                               int64_t wsC, int64_t wsR, int64_t wsS) {
+    int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;  // one 16-byte group each
+    int64_t total = static_cast<int64_t>(C / 8) * RS * K;
+    if (idx >= total) return;
+    int k = static_cast<int>(idx % K);
+    int64_t t = idx / K;
+    int tap = static_cast<int>(t % RS);
+    int cg = static_cast<int>(t / RS);
+    int r = tap / S, s = tap - r * S;
+    struct alignas(16) G {
+        half_t e[8];
+    } grp;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) grp.e[j] = w[k * wsK + (cg * 8 + j) * wsC + r * wsR + s * wsS];
+    *reinterpret_cast<G*>(wp + idx * 8) = grp;
+}
+
+}  // namespace hipcx
