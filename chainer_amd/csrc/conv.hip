@@ -212,7 +212,7 @@ NchwPlan PlanNchw(const hipcx_array* x, const hipcx_array* w, const hipcx_array*
     const int64_t K = w->shape[0], R = w->shape[2], S = w->shape[3];
     const int64_t OH = out->shape[2], OW = out->shape[3];
     if (N * C * H * W * 2 >= (1LL << 31) || N * K * OH * OW * 2 >= (1LL << 31) || K * C * R * S * 2 >= (1LL << 31)) return pl;
-    if (reinterpret_cast<uintptr_t>(x->data) % 16 != 0 || reinterpret_cast<uintptr_t>(out->data) % 8 != 0) return pl;
+    if (reinterpret_cast<uintptr_t>(x->data) % 16 != 0 || reinterpret_cast<uintptr_t>(out->data) % 16 != 0) return pl;
     const bool is1 = R == 1 && S == 1 && pad[0] == 0 && pad[1] == 0 && stride[0] == stride[1];
     const bool is3 = R == 3 && S == 3 && pad[0] == 1 && pad[1] == 1 && stride[0] == 1 && stride[1] == 1;
     if (!is1 && !is3) return pl;
@@ -249,6 +249,7 @@ NchwPlan PlanNchw(const hipcx_array* x, const hipcx_array* w, const hipcx_array*
     const int cg = pl.ck / 8;
     const int bn = 64 * pl.wch;
     pl.lds_bytes = 2 * (cg * pl.nslot * 16 + pl.taps * cg * bn * 16) + pl.npx * 16;
+    pl.lds_bytes = std::max(pl.lds_bytes, bn * (64 * pl.wpx * 2 + 16));  // the epilogue's [channel][pixel] staging tile
     if (pl.lds_bytes > 160 * 1024) return pl;
     pl.wp_bytes = RoundUpTo(static_cast<size_t>(K) * C * R * S * 2, 256);
     pl.ok = true;
@@ -295,7 +296,7 @@ void RunNchw(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, c
     a.x_bytes = static_cast<unsigned>(static_cast<int64_t>(a.N) * a.C * a.H * a.W * 2);
     const int RS = static_cast<int>(w->shape[2] * w->shape[3]);
     a.wp_bytes = static_cast<unsigned>(static_cast<int64_t>(a.K) * a.C * RS * 2);
-    a.vec_out = a.P % 4 == 0 ? 1 : 0;
+    a.out_ev = a.P % 8 == 0 ? 8 : a.P % 4 == 0 ? 4 : a.P % 2 == 0 ? 2 : 1;
     {
         int64_t groups = static_cast<int64_t>(a.C / 8) * RS * a.K;
         hipLaunchKernelGGL(NchwRepackFiltersKernel, dim3(static_cast<unsigned>((groups + 255) / 256)), dim3(256), 0, stream,

@@ -45,7 +45,7 @@ struct NchwConvArgs {
     int nslot;  // slots per channel group in the LDS patch
     int64_t bias_stride;
     unsigned x_bytes, wp_bytes;
-    int vec_out;  // P % 4 == 0: a lane's 4 consecutive pixels share an image and are 8-byte aligned
+    int out_ev;   // pixels per output store: the largest of 8, 4, 2, 1 that divides P (a run then stays inside one image)
 };
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t MakeRsrc(const void* ptr, unsigned bytes) {
@@ -254,25 +254,32 @@ __global__ __launch_bounds__(64 * WPX * WCH) void NchwConvKernel(NchwConvArgs p)
         }
     }
 
+    // One channel chunk out of a stage.  Fragments are double-buffered by hand: the reads of step i+1 are issued
+    // before the MFMAs of step i, and the scheduling groups keep that order in the instruction stream.
     auto compute = [&](const char* stage) {
-#pragma unroll
-        for (int tap = 0; tap < TAPS; ++tap) {
+        constexpr int NSTEP = TAPS * KS;
+        Bytes16 af[2][PW], bf[2][CW];
+        auto read_frags = [&](int st, Bytes16(&fa)[PW], Bytes16(&fb)[CW]) {
+            const int tap = st / KS, ks = st % KS;
             const int toff = TAPS == 9 ? ((tap / 3) * W2 + (tap % 3)) * 16 : 0;
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                Bytes16 af[PW], bf[CW];
+            for (int a = 0; a < PW; ++a) fa[a] = *reinterpret_cast<const Bytes16*>(stage + aoff[a] + toff + ks * a_ks);
 #pragma unroll
-                for (int a = 0; a < PW; ++a) af[a] = *reinterpret_cast<const Bytes16*>(stage + aoff[a] + toff + ks * a_ks);
-#pragma unroll
-                for (int b = 0; b < CW; ++b) {
-                    bf[b] = *reinterpret_cast<const Bytes16*>(stage + boff + ((ks * 2 * TAPS + tap) * BN + b * 32) * 16);
-                }
-#pragma unroll
-                for (int a = 0; a < PW; ++a) {
-#pragma unroll
-                    for (int b = 0; b < CW; ++b) MfmaTile<half_t>(af[a], bf[b], acc[a][b]);
-                }
+            for (int b = 0; b < CW; ++b) {
+                fb[b] = *reinterpret_cast<const Bytes16*>(stage + boff + ((ks * 2 * TAPS + tap) * BN + b * 32) * 16);
             }
+        };
+        read_frags(0, af[0], bf[0]);
+#pragma unroll
+        for (int st = 0; st < NSTEP; ++st) {
+            if (st + 1 < NSTEP) read_frags(st + 1, af[(st + 1) & 1], bf[(st + 1) & 1]);
+#pragma unroll
+            for (int a = 0; a < PW; ++a) {
+#pragma unroll
+                for (int b = 0; b < CW; ++b) MfmaTile<half_t>(af[st & 1][a], bf[st & 1][b], acc[a][b]);
+            }
+            if (st + 1 < NSTEP) __builtin_amdgcn_sched_group_barrier(0x100, PW + CW, 0);  // DS reads of the next step
+            __builtin_amdgcn_sched_group_barrier(0x008, PW * CW, 0);                      // MFMAs of this step
         }
     };
 
@@ -295,42 +302,68 @@ __global__ __launch_bounds__(64 * WPX * WCH) void NchwConvKernel(NchwConvArgs p)
         __syncthreads();
     }
 
-    // ---- epilogue: lane holds channel column lr of each 32-wide sub-tile, pixel rows 8*(v/4) + 4*g + v%4 ----
+    // ---- epilogue ----
+    // A lane holds channel column lr of each 32-wide sub-tile and pixel rows 8*(v/4) + 4*g + v%4.  The tile is
+    // regrouped through LDS as [channel][pixel] (the last barrier of the loop has retired every stage read), so that
+    // consecutive lanes store consecutive pixel runs of one channel plane: whole cache lines per instruction.
+    constexpr int OPITCH = BM * 2 + 16;  // bytes per channel row
 #pragma unroll
     for (int b = 0; b < CW; ++b) {
-        int n = n0 + (wch * CW + b) * 32 + lr;
-        if (n >= p.K) continue;
-        float bias = p.bias != nullptr ? static_cast<float>(p.bias[n * p.bias_stride]) : 0.f;
+        const int row = (wch * CW + b) * 32 + lr;
+        const int n = n0 + row;
+        float bias = (p.bias != nullptr && n < p.K) ? static_cast<float>(p.bias[n * p.bias_stride]) : 0.f;
 #pragma unroll
         for (int a = 0; a < PW; ++a) {
 #pragma unroll
             for (int vq = 0; vq < 4; ++vq) {
-                int m = m0 + (wpx * PW + a) * 32 + vq * 8 + g * 4;
-                if (m >= p.M) continue;
-                float v[4];
+                const int col = (wpx * PW + a) * 32 + vq * 8 + g * 4;
+                struct alignas(8) Out4 {
+                    half_t e[4];
+                } pack;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) v[e] = acc[a][b][vq * 4 + e] + bias;
-                if (p.vec_out) {
-                    int img = m / p.P;
-                    int pix = m - img * p.P;
-                    struct alignas(8) Out4 {
-                        half_t e[4];
-                    } pack;
+                for (int e = 0; e < 4; ++e) pack.e[e] = static_cast<half_t>(acc[a][b][vq * 4 + e] + bias);
+                *reinterpret_cast<Out4*>(lds + row * OPITCH + col * 2) = pack;
+            }
+        }
+    }
+    __syncthreads();
+    auto store_rows = [&](auto ev_tag) {
+        constexpr int EV = decltype(ev_tag)::value;  // pixels per store
+        constexpr int CPR = BM / EV;                 // chunks per channel row
+        static_assert(NT % CPR == 0 || CPR % NT == 0, "a thread keeps one pixel column");
+        constexpr int COLS_PER_THREAD = CPR > NT ? CPR / NT : 1;
+        constexpr int ROW_STEP = CPR > NT ? 1 : NT / CPR;
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) pack.e[e] = static_cast<half_t>(v[e]);
-                    *reinterpret_cast<Out4*>(p.out + (static_cast<int64_t>(img) * p.K + n) * p.P + pix) = pack;
+        for (int cj = 0; cj < COLS_PER_THREAD; ++cj) {
+            const int cc = (tid % (CPR > NT ? NT : CPR)) + cj * NT;
+            const int m = m0 + cc * EV;
+            if (m >= p.M) continue;
+            const int img = m / p.P;
+            const int pix = m - img * p.P;
+            half_t* obase = p.out + static_cast<int64_t>(img) * p.K * p.P + pix;
+            for (int row = (CPR > NT ? 0 : tid / CPR); row < BN; row += ROW_STEP) {
+                const int n = n0 + row;
+                if (n >= p.K) break;
+                const char* src = lds + row * OPITCH + cc * EV * 2;
+                half_t* dst = obase + static_cast<int64_t>(n) * p.P;
+                if constexpr (EV == 8) {
+                    *reinterpret_cast<Bytes16*>(dst) = *reinterpret_cast<const Bytes16*>(src);
+                } else if constexpr (EV == 4) {
+                    *reinterpret_cast<Bytes8*>(dst) = *reinterpret_cast<const Bytes8*>(src);
+                } else if constexpr (EV == 2) {
+                    *reinterpret_cast<unsigned*>(dst) = *reinterpret_cast<const unsigned*>(src);
                 } else {
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        int me = m + e;
-                        if (me >= p.M) continue;
-                        int img = me / p.P;
-                        int pix = me - img * p.P;
-                        p.out[(static_cast<int64_t>(img) * p.K + n) * p.P + pix] = static_cast<half_t>(v[e]);
-                    }
+                    *dst = *reinterpret_cast<const half_t*>(src);
                 }
             }
         }
+    };
+    // EV consecutive pixels never straddle an image and are EV*2-byte aligned when P % EV == 0 (m0 % EV == 0 always)
+    switch (p.out_ev) {
+        case 8: store_rows(std::integral_constant<int, 8>{}); break;
+        case 4: store_rows(std::integral_constant<int, 4>{}); break;
+        case 2: store_rows(std::integral_constant<int, 2>{}); break;
+        default: store_rows(std::integral_constant<int, 1>{}); break;
     }
 }
 
