@@ -217,7 +217,10 @@ NchwPlan PlanNchw(const hipcx_array* x, const hipcx_array* w, const hipcx_array*
     const bool is3 = R == 3 && S == 3 && pad[0] == 1 && pad[1] == 1 && stride[0] == 1 && stride[1] == 1;
     if (!is1 && !is3) return pl;
     const int64_t P = OH * OW;
-    auto pick = [](int64_t n) { return n % 8 == 0 ? 8 : n % 4 == 0 ? 4 : n % 2 == 0 ? 2 : 1; };
+    // Pixels per activation load.  Wider loads would be fewer, but a thread's transposed 16-byte groups go to LDS
+    // NPX slots apart from its neighbour's, and beyond a 32-byte lane stride those writes serialise on LDS banks
+    // (measured: 16 clk per wave instruction at 32 bytes, 32 at 64, 64 at 128).
+    auto pick = [](int64_t n) { return n % 2 == 0 ? 2 : 1; };
     if (is1) {
         if (C % 32 != 0) return pl;
         pl.taps = 1;
@@ -225,10 +228,10 @@ NchwPlan PlanNchw(const hipcx_array* x, const hipcx_array* w, const hipcx_array*
         pl.npx = stride[0] == 1 ? pick(P) : 1;
         if (K <= 64) {
             pl.wpx = 4, pl.wch = 1;
-            pl.maxi = pl.npx >= 4 ? 1 : pl.npx == 2 ? 2 : 4;
+            pl.maxi = pl.npx == 2 ? 2 : 4;
         } else {
             pl.wpx = 2, pl.wch = 2;
-            pl.maxi = pl.npx >= 2 ? 1 : 2;
+            pl.maxi = pl.npx == 2 ? 1 : 2;
         }
         pl.nslot = 64 * pl.wpx;
     } else {
@@ -237,13 +240,13 @@ NchwPlan PlanNchw(const hipcx_array* x, const hipcx_array* w, const hipcx_array*
         pl.ck = 16;
         pl.npx = pick(W);
         pl.wpx = 4, pl.wch = 1;
-        pl.maxi = pl.npx >= 4 ? 1 : pl.npx == 2 ? 2 : 4;
         const int64_t BM = 256;
         int64_t rows = (BM + W - 2) / W + 1;
         int64_t cross = (BM + P - 2) / P;
         pl.nrow = static_cast<int>(rows + 2 * cross + 2);
         pl.nslot = pl.nrow * static_cast<int>(W + 2);
         int64_t items = static_cast<int64_t>(pl.nrow) * (W / pl.npx) * (pl.ck / 8);
+        pl.maxi = items <= 512 ? 2 : 4;
         if (items > static_cast<int64_t>(pl.maxi) * 256) return pl;
     }
     const int cg = pl.ck / 8;
@@ -309,17 +312,13 @@ void RunNchw(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, c
     ProfileScope prof(stream, flops, bytes);
     const int key = pl.taps * 1000 + pl.wpx * 100 + pl.npx * 10 + pl.maxi;
     switch (key) {
-        case 1000 + 400 + 80 + 1: LaunchNchwKernel<1, 4, 1, 32, 8, 1>(a, pl.lds_bytes, stream); break;
-        case 1000 + 400 + 40 + 1: LaunchNchwKernel<1, 4, 1, 32, 4, 1>(a, pl.lds_bytes, stream); break;
         case 1000 + 400 + 20 + 2: LaunchNchwKernel<1, 4, 1, 32, 2, 2>(a, pl.lds_bytes, stream); break;
         case 1000 + 400 + 10 + 4: LaunchNchwKernel<1, 4, 1, 32, 1, 4>(a, pl.lds_bytes, stream); break;
-        case 1000 + 200 + 80 + 1: LaunchNchwKernel<1, 2, 2, 32, 8, 1>(a, pl.lds_bytes, stream); break;
-        case 1000 + 200 + 40 + 1: LaunchNchwKernel<1, 2, 2, 32, 4, 1>(a, pl.lds_bytes, stream); break;
         case 1000 + 200 + 20 + 1: LaunchNchwKernel<1, 2, 2, 32, 2, 1>(a, pl.lds_bytes, stream); break;
         case 1000 + 200 + 10 + 2: LaunchNchwKernel<1, 2, 2, 32, 1, 2>(a, pl.lds_bytes, stream); break;
-        case 9000 + 400 + 80 + 1: LaunchNchwKernel<9, 4, 1, 16, 8, 1>(a, pl.lds_bytes, stream); break;
-        case 9000 + 400 + 40 + 1: LaunchNchwKernel<9, 4, 1, 16, 4, 1>(a, pl.lds_bytes, stream); break;
         case 9000 + 400 + 20 + 2: LaunchNchwKernel<9, 4, 1, 16, 2, 2>(a, pl.lds_bytes, stream); break;
+        case 9000 + 400 + 20 + 4: LaunchNchwKernel<9, 4, 1, 16, 2, 4>(a, pl.lds_bytes, stream); break;
+        case 9000 + 400 + 10 + 2: LaunchNchwKernel<9, 4, 1, 16, 1, 2>(a, pl.lds_bytes, stream); break;
         case 9000 + 400 + 10 + 4: LaunchNchwKernel<9, 4, 1, 16, 1, 4>(a, pl.lds_bytes, stream); break;
         default: throw Error(HIPCX_CHAINERX_ERROR, "nchw conv: no kernel for plan " + std::to_string(key));
     }
