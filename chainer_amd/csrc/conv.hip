@@ -300,7 +300,11 @@ void RunNchw(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, c
     const int RS = static_cast<int>(w->shape[2] * w->shape[3]);
     a.wp_bytes = static_cast<unsigned>(static_cast<int64_t>(a.K) * a.C * RS * 2);
     a.out_ev = a.P % 8 == 0 ? 8 : a.P % 4 == 0 ? 4 : a.P % 2 == 0 ? 2 : 1;
-    {
+    const bool w_dense = w->strides[1] == 2 && w->strides[0] == static_cast<int64_t>(a.C) * 2 && reinterpret_cast<uintptr_t>(w->data) % 16 == 0;
+    if (RS == 1 && w_dense) {
+        a.w_direct = 1;
+        a.wp = static_cast<const half_t*>(w->data);
+    } else {
         int64_t groups = static_cast<int64_t>(a.C / 8) * RS * a.K;
         hipLaunchKernelGGL(NchwRepackFiltersKernel, dim3(static_cast<unsigned>((groups + 255) / 256)), dim3(256), 0, stream,
                            static_cast<const half_t*>(w->data), reinterpret_cast<half_t*>(workspace), a.K, a.C, RS,

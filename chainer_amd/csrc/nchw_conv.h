@@ -31,7 +31,7 @@ namespace hipcx {
 
 struct NchwConvArgs {
     const half_t* x;
-    const half_t* wp;    // packed filters [C/8][taps][K][8]
+    const half_t* wp;    // packed filters [C/8][taps][K][8]; or, with w_direct, the caller's dense [K][C] 1x1 filters
     const half_t* bias;  // may be null
     half_t* out;
     int N, C, H, W;  // input
@@ -45,6 +45,7 @@ struct NchwConvArgs {
     int nslot;  // slots per channel group in the LDS patch
     int64_t bias_stride;
     unsigned x_bytes, wp_bytes;
+    int w_direct;  // 1x1 only: read the filter bank in place (a row's 8 consecutive channels are one 16-byte group already)
     int out_ev;   // pixels per output store: the largest of 8, 4, 2, 1 that divides P (a run then stays inside one image)
 };
 
@@ -187,7 +188,11 @@ __global__ __launch_bounds__(64 * WPX * WCH) void NchwConvKernel(NchwConvArgs p)
         int tap = rest / BN;
         int kl = rest - tap * BN;
         bool valid = wi < WITEMS && n0 + kl < p.K;
-        wvoff[i] = valid ? ((cg * TAPS + tap) * p.K + n0 + kl) * 16 : 0x7fffffff;
+        if (TAPS == 1 && p.w_direct) {
+            wvoff[i] = valid ? ((n0 + kl) * p.C + cg * 8) * 2 : 0x7fffffff;
+        } else {
+            wvoff[i] = valid ? ((cg * TAPS + tap) * p.K + n0 + kl) * 16 : 0x7fffffff;
+        }
         wlds[i] = wi < WITEMS ? patch_bytes + wi * 16 : -1;
     }
 
@@ -203,7 +208,7 @@ __global__ __launch_bounds__(64 * WPX * WCH) void NchwConvKernel(NchwConvArgs p)
 #pragma unroll
             for (int j = 0; j < 8; ++j) xreg[i][j] = BufLoad<NPX>(xr, xvoff[i], xs + j * HW * 2);
         }
-        const int ws = ci * (CG * TAPS) * p.K * 16;
+        const int ws = (TAPS == 1 && p.w_direct) ? ci * CK * 2 : ci * (CG * TAPS) * p.K * 16;
 #pragma unroll
         for (int i = 0; i < WPT; ++i) wreg[i] = __builtin_amdgcn_raw_buffer_load_b128(wr, wvoff[i], ws, 0);
     };

@@ -150,6 +150,65 @@ __global__ __launch_bounds__(256) void PoolKernel(PoolArgs p, int64_t total) {
     }
 }
 
+
+// Max pooling with horizontal stride 2 over dense NCHW rows: a thread produces EPV/2 adjacent outputs of one row from
+// two aligned 16-byte loads per input row (columns [2*ow0 - EPV, 2*ow0 + EPV)), instead of kh*kw scalar loads per
+// output.  Requires W % EPV == 0, OW % (EPV/2) == 0, pw <= EPV and kw <= pw + 2 (then every tap falls inside the two
+// chunks), which covers the 3x3/2 pad 1 and 2x2/2 pad 0 windows.
+template <typename T>
+__global__ __launch_bounds__(256) void MaxPoolRowsS2Kernel(PoolArgs p, int64_t total) {
+    constexpr int EPV = 16 / sizeof(T);
+    constexpr int VO = EPV / 2;
+    const T* x = static_cast<const T*>(p.x);
+    T* out = static_cast<T*>(p.out);
+    const int ovecs = p.OW / VO;
+    for (int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; idx < total;
+         idx += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+        int ov = static_cast<int>(idx % ovecs);
+        int64_t t = idx / ovecs;
+        int oh = static_cast<int>(t % p.OH);
+        int64_t plane = t / p.OH;  // n * C + c
+        const T* xp = x + plane * p.H * p.W;
+        const int ow0 = ov * VO;
+        const int col0 = 2 * ow0 - EPV;  // first column of the left chunk
+        T acc[VO];
+#pragma unroll
+        for (int e = 0; e < VO; ++e) acc[e] = Lowest<T>();
+        const int h0 = oh * p.sh - p.ph;
+        for (int r = 0; r < p.kh; ++r) {
+            int ih = h0 + r;
+            if (ih < 0 || ih >= p.H) continue;
+            const T* row = xp + static_cast<int64_t>(ih) * p.W;
+            T win[2 * EPV];
+            PVec<T, EPV> lo, hi;
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) lo.v[e] = hi.v[e] = Lowest<T>();
+            if (col0 >= 0) lo = *reinterpret_cast<const PVec<T, EPV>*>(row + col0);
+            if (col0 + EPV < p.W) hi = *reinterpret_cast<const PVec<T, EPV>*>(row + col0 + EPV);
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) {
+                win[e] = lo.v[e];
+                win[EPV + e] = hi.v[e];
+            }
+#pragma unroll
+            for (int e = 0; e < VO; ++e) {
+#pragma unroll
+                for (int s = 0; s < 2 * EPV; ++s) {  // taps of output e: window columns EPV + 2e - pw + [0, kw)
+                    int rel = s - (EPV + 2 * e - p.pw);
+                    if (rel >= 0 && rel < p.kw) {
+                        T v = win[s];
+                        if (IsNanT(v) || acc[e] < v) acc[e] = v;
+                    }
+                }
+            }
+        }
+        PVec<T, VO> res;
+#pragma unroll
+        for (int e = 0; e < VO; ++e) res.v[e] = acc[e];
+        *reinterpret_cast<PVec<T, VO>*>(out + (plane * p.OH + oh) * p.OW + ow0) = res;
+    }
+}
+
 int64_t ElemStride(const hipcx_array* a, int axis) {
     int64_t it = ItemSize(a->dtype);
     HIPCX_REQUIRE(a->strides[axis] % it == 0, HIPCX_NOT_IMPLEMENTED_ERROR, "byte strides must be multiples of the item size");
@@ -160,6 +219,23 @@ bool Aligned(const void* p, int64_t bytes) { return reinterpret_cast<uintptr_t>(
 
 template <typename T, bool IS_MAX>
 void RunPool(PoolArgs p, hipStream_t stream) {
+    if constexpr (IS_MAX && sizeof(T) <= 8) {
+        constexpr int EPV = 16 / sizeof(T);
+        constexpr int VO = EPV / 2;
+        bool dense_in = p.xsW == 1 && p.xsH == p.W && p.xsC == static_cast<int64_t>(p.H) * p.W && p.xsN == p.xsC * p.C;
+        bool dense_out = p.osW == 1 && p.osH == p.OW && p.osC == static_cast<int64_t>(p.OH) * p.OW && p.osN == p.osC * p.C;
+        if (VO >= 1 && dense_in && dense_out && p.sw == 2 && p.W % EPV == 0 && p.OW % VO == 0 && p.pw <= EPV && p.kw <= p.pw + 2 &&
+            Aligned(p.x, 16) && Aligned(p.out, sizeof(T) * VO) && 2 * (p.OW - 1) - p.pw + p.kw <= p.W + p.pw) {
+            int64_t total = static_cast<int64_t>(p.N) * p.C * p.OH * (p.OW / VO);
+            if (total == 0) return;
+            int64_t blocks = (total + 255) / 256;
+            int64_t cap = static_cast<int64_t>(NumCUs()) * 32;
+            if (blocks > cap) blocks = cap;
+            hipLaunchKernelGGL((MaxPoolRowsS2Kernel<T>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, p, total);
+            CheckLaunch("max_pool_rows");
+            return;
+        }
+    }
     constexpr int VEC = 16 / sizeof(T);
     bool vec_ok = p.xsC == 1 && p.osC == 1 && p.C % VEC == 0 && Aligned(p.x, 16) && Aligned(p.out, 16) && p.xsN % VEC == 0 &&
                   p.xsH % VEC == 0 && p.xsW % VEC == 0 && p.osN % VEC == 0 && p.osH % VEC == 0 && p.osW % VEC == 0;
