@@ -36,11 +36,19 @@ def main():
     ap.add_argument('--warmup', type=int, default=5)
     ap.add_argument('--batch', type=int, default=128)
     ap.add_argument('--eager', action='store_true', help='time eager launches instead of a HIP graph replay')
+    ap.add_argument('--ops', nargs='?', const='sweep,mlp,cifar,resnet_layers,lstm', default=None,
+                    help='instead of the headline step, print per-operation roofline lines (chainer_amd.bench_ops) with a CPU baseline column')
     ap.add_argument('--cpu-batch', type=int, default=8, help='images for the CPU baseline (0 = skip)')
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit('bench.py: this build runs on one GPU only (inference shards trivially along the batch axis; '
                  'no multi-GPU path is built). Run with --gpus 1.')
+
+    if args.ops is not None:
+        from chainer_amd import bench_ops
+        from oracle import native as oracle  # CPU baseline column only
+        bench_ops.run(args.ops.split(','), cpu=oracle)
+        return
 
     import torch
     import chainer_amd as chx

@@ -1,0 +1,245 @@
+#!/usr/bin/env python3
+"""Per-operation and per-workload measurements of the hip kernels against the MI355X rooflines.
+
+    python -m chainer_amd.bench_ops [--section sweep,mlp,cifar,resnet_layers,lstm]
+    python bench.py --ops [sections]        (the same, plus a CPU baseline column)
+
+Every figure is device time between two events recorded on the launch stream around `iters` back-to-back calls
+(after warm-up), divided by `iters`.  Bandwidth figures divide the *algorithmic* bytes of the operation (each operand
+once, no temporaries) by that time; the fraction is taken against the published peaks (8 TB/s HBM, 2.5 PFLOP/s dense
+fp16 MFMA, 157.3 TFLOP/s fp32 MFMA).  Chains of kernels (log_softmax = 7 launches, softmax_cross_entropy, the LSTM
+cell) are timed as the chain and priced against the bytes a single fused pass would move.
+
+`run(sections, cpu=namespace)` additionally times each operation on a CPU implementation of the same routine names that
+the caller passes in (bench.py passes its single-threaded restatement of the ChainerX native backend; bounded sample
+sizes) for the "next to the native backend" column.  This module itself only knows the hip kernels.  Output: one JSON
+object per line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+HBM_PEAK = 8000.0  # GB/s
+MFMA_PEAK = {'float16': 2500.0, 'float32': 157.3}  # TFLOP/s
+
+
+def device_time(fn, iters=20, warmup=5):
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    e1.synchronize()
+    return e0.elapsed_time(e1) / iters * 1e-3  # seconds
+
+
+def graph_time(fn, iters=20):
+    """Seconds per replay of `fn` captured into a HIP graph (launch overhead of its kernels removed)."""
+    import torch
+    fn()
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        fn()
+    g.replay()
+    torch.cuda.synchronize()
+    return device_time(g.replay, iters, 3)
+
+
+def cpu_time(fn, min_s=0.2):
+    fn()
+    t0 = time.perf_counter()
+    n = 0
+    while True:
+        fn()
+        n += 1
+        dt = time.perf_counter() - t0
+        if dt > min_s:
+            return dt / n
+
+
+def emit(**kw):
+    print(json.dumps(kw), flush=True)
+
+
+def bw_row(section, name, shape, seconds, nbytes, launches=1, cpu_s=None, note=None):
+    row = dict(section=section, op=name, shape=list(shape), us=round(seconds * 1e6, 2), launches=launches,
+               algorithmic_MB=round(nbytes / 1e6, 2), GBps=round(nbytes / seconds / 1e9, 1),
+               hbm_frac=round(nbytes / seconds / 1e9 / HBM_PEAK, 4))
+    if cpu_s is not None:
+        row['cpu_native_1core_us'] = round(cpu_s * 1e6, 1)
+    if note:
+        row['note'] = note
+    emit(**row)
+
+
+def section_sweep(chx, oracle, with_cpu):
+    """Config 2: elementwise / reduction sweep, float32 [4096,4096] and [64,1048576]."""
+    rng = np.random.default_rng(2)
+    for shape in ((4096, 4096), (64, 1048576)):
+        x = rng.standard_normal(shape).astype(np.float32)
+        b = rng.standard_normal(shape[1]).astype(np.float32)
+        X, B = chx.array(x), chx.array(b)
+        n, s = x.size, 4
+        rows = shape[0]
+        small = x[:max(1, rows // 64)] if with_cpu else None  # CPU sample: 1/64 of the rows, scaled back up
+        scale = rows / max(1, rows // 64)
+        ops = [
+            ('x+b', lambda: chx.add(X, B), 2 * n * s + b.nbytes, 1, (lambda: oracle.add(small, b)) if with_cpu else None),
+            ('x*b', lambda: chx.multiply(X, B), 2 * n * s + b.nbytes, 1, (lambda: oracle.multiply(small, b)) if with_cpu else None),
+            ('exp', lambda: chx.exp(X), 2 * n * s, 1, (lambda: oracle.exp(small)) if with_cpu else None),
+            ('tanh', lambda: chx.tanh(X), 2 * n * s, 1, (lambda: oracle.tanh(small)) if with_cpu else None),
+            ('sum axis1', lambda: chx.sum(X, 1), n * s + rows * s, 1, (lambda: oracle.sum(small, 1)) if with_cpu else None),
+            ('max axis1', lambda: chx.amax(X, 1), n * s + rows * s, 1, (lambda: oracle.amax(small, 1)) if with_cpu else None),
+            ('argmax axis1', lambda: chx.argmax(X, 1), n * s + rows * 8, 1, (lambda: oracle.argmax(small, 1)) if with_cpu else None),
+            ('log_softmax axis1', lambda: chx.log_softmax(X, 1), (2 if shape[1] * s <= 65536 else 3) * n * s, 7,
+             (lambda: oracle.log_softmax(small, 1)) if with_cpu else None),
+        ]
+        for name, fn, nbytes, launches, cfn in ops:
+            t = device_time(fn)
+            cpu = cpu_time(cfn) * scale if cfn is not None else None
+            note = None
+            if launches > 1:
+                note = ('7 kernel launches as the ChainerX routine decomposes it (moves 8*N*4 bytes: ceiling %.0f%% of the '
+                        'fused-ideal figure used here)' % (100.0 * nbytes / (8 * n * s)))
+            bw_row('sweep', name, shape, t, nbytes, launches, cpu, note)
+
+
+def section_mlp(chx, oracle, with_cpu):
+    """Config 1: MNIST-shaped MLP forward + softmax cross entropy, float32 batch 100 (launch-latency bound)."""
+    from chainer_amd import configs as cfg
+    p = cfg.mlp_params()
+    x, t = cfg.mlp_input()
+    pd = cfg.tree_map(chx.array, p)
+    X, T = chx.array(x), chx.array(t)
+    fn = lambda: cfg.mlp_forward(chx, pd, X, T)
+    eager = device_time(fn)
+    graph = graph_time(fn)
+    flops = 2 * 100 * (784 * 1000 + 1000 * 1000 + 1000 * 10)
+    row = dict(section='mlp', op='forward+loss', batch=100, eager_us=round(eager * 1e6, 1), graph_replay_us=round(graph * 1e6, 1),
+               kernel_launches=3 + 3 + 2 + 15, GFLOP=round(flops / 1e9, 4), TFLOPs_graph=round(flops / graph / 1e12, 2))
+    if with_cpu:
+        row['cpu_native_1core_us'] = round(cpu_time(lambda: cfg.mlp_forward(oracle, p, x, t)) * 1e6, 1)
+    emit(**row)
+
+
+def section_cifar(chx, oracle, with_cpu):
+    """Config 3: CIFAR-shaped convnet inference, float32 batch 256."""
+    from chainer_amd import configs as cfg
+    p = cfg.cifar_params()
+    x = cfg.cifar_input()
+    pd = cfg.tree_map(chx.array, p)
+    X = chx.array(x)
+    fn = lambda: cfg.cifar_forward(chx, pd, X)
+    eager = device_time(fn, 10, 3)
+    graph = graph_time(fn, 10)
+    flops = 78.22e9
+    row = dict(section='cifar', op='forward', batch=256, dtype='float32', eager_ms=round(eager * 1e3, 3),
+               graph_replay_ms=round(graph * 1e3, 3), img_per_s=round(256 / graph, 1), TFLOPs=round(flops / graph / 1e12, 2),
+               fp32_mfma_frac=round(flops / graph / 1e12 / MFMA_PEAK['float32'], 4))
+    if with_cpu:
+        xs = x[:2]
+        row['cpu_native_1core_img_per_s'] = round(2 / cpu_time(lambda: cfg.cifar_forward(oracle, p, xs), 1.0), 3)
+    emit(**row)
+
+
+RESNET_LAYERS = [  # N, C, H, W, K, R, S, stride, pad, occurrences in ResNet-50
+    (128, 3, 224, 224, 64, 7, 7, 2, 3, 1),
+    (128, 64, 56, 56, 64, 1, 1, 1, 0, 1), (128, 64, 56, 56, 64, 3, 3, 1, 1, 3), (128, 64, 56, 56, 256, 1, 1, 1, 0, 4),
+    (128, 256, 56, 56, 64, 1, 1, 1, 0, 2), (128, 256, 56, 56, 128, 1, 1, 2, 0, 1), (128, 256, 56, 56, 512, 1, 1, 2, 0, 1),
+    (128, 128, 28, 28, 128, 3, 3, 1, 1, 4), (128, 128, 28, 28, 512, 1, 1, 1, 0, 4), (128, 512, 28, 28, 128, 1, 1, 1, 0, 3),
+    (128, 512, 28, 28, 256, 1, 1, 2, 0, 1), (128, 512, 28, 28, 1024, 1, 1, 2, 0, 1), (128, 256, 14, 14, 256, 3, 3, 1, 1, 6),
+    (128, 256, 14, 14, 1024, 1, 1, 1, 0, 6), (128, 1024, 14, 14, 256, 1, 1, 1, 0, 5), (128, 1024, 14, 14, 512, 1, 1, 2, 0, 1),
+    (128, 1024, 14, 14, 2048, 1, 1, 2, 0, 1), (128, 512, 7, 7, 512, 3, 3, 1, 1, 3), (128, 512, 7, 7, 2048, 1, 1, 1, 0, 3),
+    (128, 2048, 7, 7, 512, 1, 1, 1, 0, 2),
+]
+
+
+def section_resnet_layers(chx, oracle, with_cpu):
+    """Config 4 layer by layer: every distinct convolution (float16 NCHW in and out), and the bandwidth-bound kernels at
+    the largest activation shape."""
+    rng = np.random.default_rng(4)
+    total = 0.0
+    for (N, C, H, W, K, R, S, st, pd, cnt) in RESNET_LAYERS:
+        x = rng.standard_normal((N, C, H, W)).astype(np.float16)
+        w = (rng.standard_normal((K, C, R, S)) / np.sqrt(C * R * S)).astype(np.float16)
+        X, Wd = chx.array(x), chx.array(w)
+        OH = (H + 2 * pd - R) // st + 1
+        flops = 2.0 * N * OH * OH * K * C * R * S
+        nbytes = 2.0 * (x.size + w.size + N * K * OH * OH)
+        t = device_time(lambda: chx.conv(X, Wd, None, st, pd), 10, 3)
+        total += t * cnt
+        emit(section='resnet_layers', op='conv', shape=[N, C, H, W], filters=[K, C, R, S], stride=st, pad=pd, count=cnt,
+             us=round(t * 1e6, 1), TFLOPs=round(flops / t / 1e12, 1), mfma_frac=round(flops / t / 1e12 / MFMA_PEAK['float16'], 4),
+             GBps=round(nbytes / t / 1e9, 1), hbm_frac=round(nbytes / t / 1e9 / HBM_PEAK, 4),
+             bound='hbm' if nbytes / 8e12 > flops / 2.5e15 else 'mfma')
+    emit(section='resnet_layers', op='all convolutions of one forward pass', ms=round(total * 1e3, 3), TFLOPs=round(987.6e9 / total / 1e12, 1))
+    shape = (128, 256, 56, 56)
+    x = rng.standard_normal(shape).astype(np.float16)
+    X, Y = chx.array(x), chx.array(x)
+    prm = [chx.array(rng.uniform(0.5, 1.5, shape[1]).astype(np.float16)) for _ in range(4)]
+    n = x.size * 2
+    bw_row('resnet_layers', 'fixed_batch_norm', shape, device_time(lambda: chx.fixed_batch_norm(X, *prm, 2e-5, (0, 2, 3))), 2 * n)
+    bw_row('resnet_layers', 'relu', shape, device_time(lambda: chx.relu(X)), 2 * n)
+    bw_row('resnet_layers', 'add (residual)', shape, device_time(lambda: chx.add(X, Y)), 3 * n)
+    xp = chx.array(rng.standard_normal((128, 64, 112, 112)).astype(np.float16))
+    bw_row('resnet_layers', 'max_pool 3x3/2 pad 1', (128, 64, 112, 112), device_time(lambda: chx.max_pool(xp, 3, 2, 1)), xp.nbytes * 1.25)
+    xa = chx.array(rng.standard_normal((128, 2048, 7, 7)).astype(np.float16))
+    bw_row('resnet_layers', 'average_pool 7x7 (global)', (128, 2048, 7, 7), device_time(lambda: chx.average_pool(xa, 7, 1, 0, 'zero')),
+           xa.nbytes + 128 * 2048 * 2)
+
+
+def section_lstm(chx, oracle, with_cpu):
+    """Config 5: 2-layer LSTM language model inference, float32, batch 128, 35 steps, vocabulary 10000."""
+    from chainer_amd import configs as cfg
+    p = cfg.lstm_lm_params()
+    ids = cfg.lstm_lm_input()
+    pd = cfg.tree_map(chx.array, p)
+    I = chx.array(ids)
+    fn = lambda: cfg.lstm_lm_forward(chx, pd, I, chx.zeros)
+    eager = device_time(fn, 3, 1)
+    flops = 60.57e9 + 58.24e9
+    row = dict(section='lstm', op='35-step forward', batch=128, eager_ms=round(eager * 1e3, 2), TFLOPs=round(flops / eager / 1e12, 2),
+               tokens_per_s=round(128 * 35 / eager, 0),
+               note='take with the default bounds mode reads a flag back every step (the native backend raises IndexError), so '
+                    'the sequence is not graph-captured')
+    emit(**row)
+    W = pd['embed']
+    t = device_time(lambda: chx.take(W, I, 0, 'wrap'))
+    bw_row('lstm', 'take [10000,650] rows by [128,35] ids', (128, 35, 650), t, 2 * 128 * 35 * 650 * 4 + ids.nbytes)
+    if with_cpu:
+        ids2 = ids[:, :1]
+        emit(section='lstm', op='cpu native 1 core, one time step', ms=round(cpu_time(lambda: cfg.lstm_lm_forward(oracle, p, ids2, np.zeros), 1.0) * 1e3, 1))
+
+
+SECTIONS = {'sweep': section_sweep, 'mlp': section_mlp, 'cifar': section_cifar, 'resnet_layers': section_resnet_layers, 'lstm': section_lstm}
+
+
+def run(sections, cpu=None):
+    import chainer_amd as chx
+    if not chx.device_available():
+        sys.exit('bench_ops: no HIP device visible')
+    for name in sections:
+        SECTIONS[name](chx, cpu, cpu is not None)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument('--section', default=','.join(SECTIONS))
+    args = ap.parse_args()
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    if root not in sys.path:
+        sys.path.insert(0, root)
+    run(args.section.split(','))
+
+
+if __name__ == '__main__':
+    main()
