@@ -178,6 +178,31 @@ def resnet50_forward(F, p, x):
     return F.linear(h, p['fc_w'], p['fc_b'])
 
 
+def _conv_bn_act(F, x, w, stride, pad, bn, residual=None, relu=True):
+    """conv -> fixed batch norm -> (+ residual) -> ReLU through the fused entry point when `F` has one, else composed."""
+    if hasattr(F, 'conv_bn_act'):
+        return F.conv_bn_act(x, w, None, stride, pad, False, (bn['gamma'], bn['beta'], bn['mean'], bn['var']), BN_EPS, residual, relu)
+    h = _bn(F, F.conv(x, w, None, stride, pad), bn)
+    if residual is not None:
+        h = F.add(h, residual)
+    return F.relu(h) if relu else h
+
+
+def resnet50_forward_fused(F, p, x):
+    """The same network with every conv -> batch norm (-> add) -> ReLU group issued as one fused call."""
+    h = _conv_bn_act(F, x, p['conv1'], 2, 3, p['bn1'])
+    h = F.max_pool(h, 3, 2, 1, False)
+    for si, stage in enumerate(p['stages']):
+        for bi, blk in enumerate(stage):
+            stride = 2 if (bi == 0 and si > 0) else 1
+            sc = _conv_bn_act(F, h, blk['conv4'], stride, 0, blk['bn4'], relu=False) if 'conv4' in blk else h
+            t = _conv_bn_act(F, h, blk['conv1'], stride, 0, blk['bn1'])
+            t = _conv_bn_act(F, t, blk['conv2'], 1, 1, blk['bn2'])
+            h = _conv_bn_act(F, t, blk['conv3'], 1, 0, blk['bn3'], residual=sc, relu=True)
+    h = F.average_pool(h, h.shape[2], 1, 0, 'zero')
+    return F.linear(h, p['fc_w'], p['fc_b'])
+
+
 def resnet50_flops(batch=128, size=224):
     """Multiply-add count x2 of every conv and the final linear layer."""
     total = 0

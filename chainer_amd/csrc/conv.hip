@@ -251,7 +251,7 @@ NchwPlan PlanNchw(const hipcx_array* x, const hipcx_array* w, const hipcx_array*
     }
     const int cg = pl.ck / 8;
     const int bn = 64 * pl.wch;
-    pl.lds_bytes = 2 * (cg * pl.nslot * 16 + pl.taps * cg * bn * 16) + pl.npx * 16;
+    pl.lds_bytes = 2 * (cg * pl.nslot * 16 + cg * (pl.taps * bn * 16 + (pl.taps == 1 ? 64 : 0))) + pl.npx * 16;
     pl.lds_bytes = std::max(pl.lds_bytes, bn * (64 * pl.wpx * 2 + 16));  // the epilogue's [channel][pixel] staging tile
     if (pl.lds_bytes > 160 * 1024) return pl;
     pl.wp_bytes = RoundUpTo(static_cast<size_t>(K) * C * R * S * 2, 256);
@@ -273,9 +273,29 @@ void LaunchNchwKernel(const NchwConvArgs& a, int lds_bytes, hipStream_t stream) 
     CheckLaunch("nchw_conv");
 }
 
+// Fused tail of hipcx_conv_bn_act as the kernel wants it.
+struct FusedTail {
+    const half_t* gamma = nullptr;
+    const half_t* beta = nullptr;
+    const half_t* mean = nullptr;
+    const half_t* var = nullptr;
+    int64_t stride = 0;
+    float eps = 0.f;
+    const half_t* residual = nullptr;
+    int relu = 0;
+};
+
 void RunNchw(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, const NchwPlan& pl, const int64_t* stride,
-             const hipcx_array* out, char* workspace, hipStream_t stream) {
+             const hipcx_array* out, char* workspace, hipStream_t stream, const FusedTail& tail = FusedTail{}) {
     NchwConvArgs a{};
+    a.bn_gamma = tail.gamma;
+    a.bn_beta = tail.beta;
+    a.bn_mean = tail.mean;
+    a.bn_var = tail.var;
+    a.bn_stride = tail.stride;
+    a.bn_eps = tail.eps;
+    a.residual = tail.residual;
+    a.relu = tail.relu;
     a.x = static_cast<const half_t*>(x->data);
     a.wp = reinterpret_cast<const half_t*>(workspace);
     a.bias = b ? static_cast<const half_t*>(b->data) : nullptr;
@@ -301,7 +321,9 @@ void RunNchw(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, c
     a.wp_bytes = static_cast<unsigned>(static_cast<int64_t>(a.K) * a.C * RS * 2);
     a.out_ev = a.P % 8 == 0 ? 8 : a.P % 4 == 0 ? 4 : a.P % 2 == 0 ? 2 : 1;
     const bool w_dense = w->strides[1] == 2 && w->strides[0] == static_cast<int64_t>(a.C) * 2 && reinterpret_cast<uintptr_t>(w->data) % 16 == 0;
-    if (RS == 1 && w_dense) {
+    static const bool direct_ok = [] { const char* e = getenv("HIPCX_W_DIRECT"); return e == nullptr || e[0] != '0'; }();
+    // in-place rows are read in 64-byte pieces a whole row apart; beyond 1024 input channels the packed copy is cheaper
+    if (RS == 1 && w_dense && direct_ok && a.C <= 1024) {
         a.w_direct = 1;
         a.wp = static_cast<const half_t*>(w->data);
     } else {
@@ -607,6 +629,91 @@ int hipcx_conv(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b,
             RunConv<float>(x, w, b, pl, out, ws, st);
         } else {
             RunConv<double>(x, w, b, pl, out, ws, st);
+        }
+    });
+}
+
+// Channel stride (elements) of a batch-norm parameter holding one value per output channel: a vector [K] or the
+// keep-dims shape [1, K, 1, 1].  Returns false for anything else.
+static bool BnParamStride(const hipcx_array* a, int64_t K, int dtype, int64_t* stride) {
+    if (a == nullptr || a->dtype != dtype) return false;
+    int64_t it = ItemSize(dtype);
+    if (a->ndim == 1 && a->shape[0] == K && a->strides[0] % it == 0) {
+        *stride = a->strides[0] / it;
+        return true;
+    }
+    if (a->ndim == 4 && a->shape[0] == 1 && a->shape[1] == K && a->shape[2] == 1 && a->shape[3] == 1 && a->strides[1] % it == 0) {
+        *stride = a->strides[1] / it;
+        return true;
+    }
+    return false;
+}
+
+int hipcx_conv_bn_act(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, const int64_t* stride, const int64_t* pad,
+                      int cover_all, const hipcx_array* gamma, const hipcx_array* beta, const hipcx_array* mean, const hipcx_array* var,
+                      hipcx_scalar eps, const hipcx_array* residual, int relu, const hipcx_array* out, void* workspace,
+                      size_t workspace_bytes, void* stream) {
+    return Guard([&] {
+        CheckConv(x, w, b, stride, pad, cover_all, out);
+        const bool has_bn = gamma != nullptr || beta != nullptr || mean != nullptr || var != nullptr;
+        const int64_t K = w->shape[0];
+        int64_t sg = 0, sb = 0, sm = 0, sv = 0;
+        if (has_bn) {
+            HIPCX_REQUIRE(BnParamStride(gamma, K, out->dtype, &sg) && BnParamStride(beta, K, out->dtype, &sb) &&
+                              BnParamStride(mean, K, out->dtype, &sm) && BnParamStride(var, K, out->dtype, &sv),
+                          HIPCX_DIMENSION_ERROR, "batch-norm parameters must have one value of out's dtype per output channel ([K] or [1,K,1,1])");
+        }
+        if (residual != nullptr) {
+            ValidateArray(residual, "residual");
+            HIPCX_REQUIRE(SameShape(residual, out) && residual->dtype == out->dtype, HIPCX_DIMENSION_ERROR,
+                          "residual must have out's shape and dtype");
+        }
+        if (TotalSize(out) == 0) return;
+        hipStream_t st = AsStream(stream);
+        NchwPlan npl = PlanNchw(x, w, out, stride, pad);
+        const bool same_stride = !has_bn || (sg == sb && sg == sm && sg == sv);
+        const bool res_ok = residual == nullptr || (IsContiguous(residual) && reinterpret_cast<uintptr_t>(residual->data) % 16 == 0);
+        if (npl.ok && same_stride && res_ok) {
+            HIPCX_REQUIRE(workspace != nullptr && workspace_bytes >= npl.wp_bytes, HIPCX_CHAINERX_ERROR,
+                          "conv workspace too small: need " + std::to_string(npl.wp_bytes) + " bytes");
+            HIPCX_REQUIRE(reinterpret_cast<uintptr_t>(workspace) % 16 == 0, HIPCX_CHAINERX_ERROR, "workspace must be 16-byte aligned");
+            FusedTail tail;
+            if (has_bn) {
+                tail.gamma = static_cast<const half_t*>(gamma->data);
+                tail.beta = static_cast<const half_t*>(beta->data);
+                tail.mean = static_cast<const half_t*>(mean->data);
+                tail.var = static_cast<const half_t*>(var->data);
+                tail.stride = sg;
+                tail.eps = static_cast<float>(eps.kind == HIPCX_KIND_FLOAT ? eps.f : static_cast<double>(eps.i));
+            }
+            tail.residual = residual ? static_cast<const half_t*>(residual->data) : nullptr;
+            tail.relu = relu ? 1 : 0;
+            RunNchw(x, w, b, npl, stride, out, static_cast<char*>(workspace), st, tail);
+            return;
+        }
+        // Any other dtype / layout / geometry: the same result from the separate kernels, in place on `out`.
+        auto check = [](int status) {
+            if (status != HIPCX_OK) throw Error(status, hipcx_last_error());
+        };
+        check(hipcx_conv(x, w, b, stride, pad, cover_all, out, workspace, workspace_bytes, stream));
+        if (has_bn) {
+            auto keepdims = [&](const hipcx_array* a, int64_t stride_elems) {
+                hipcx_array v{};
+                v.data = a->data;
+                v.dtype = a->dtype;
+                v.ndim = 4;
+                v.shape[0] = 1, v.shape[1] = K, v.shape[2] = 1, v.shape[3] = 1;
+                v.strides[1] = stride_elems * ItemSize(a->dtype);
+                return v;
+            };
+            hipcx_array g4 = keepdims(gamma, sg), b4 = keepdims(beta, sb), m4 = keepdims(mean, sm), v4 = keepdims(var, sv);
+            const int8_t axis[3] = {0, 2, 3};
+            check(hipcx_fixed_batch_norm(out, &g4, &b4, &m4, &v4, eps, axis, 3, out, stream));
+        }
+        if (residual != nullptr) check(hipcx_add(out, residual, out, stream));
+        if (relu) {
+            hipcx_scalar zero{HIPCX_KIND_INT, 0, 0, 0.0};
+            check(hipcx_if_less_else_assa(out, zero, zero, out, out, stream));
         }
     });
 }

@@ -46,12 +46,45 @@ struct NchwConvArgs {
     int64_t bias_stride;
     unsigned x_bytes, wp_bytes;
     int w_direct;  // 1x1 only: read the filter bank in place (a row's 8 consecutive channels are one 16-byte group already)
+    // Optional fused tail (all null / 0 for a plain convolution): fixed batch normalisation over the output channels,
+    // a residual addend of out's shape (dense NCHW) and ReLU.
+    const half_t* bn_gamma;
+    const half_t* bn_beta;
+    const half_t* bn_mean;
+    const half_t* bn_var;
+    int64_t bn_stride;  // element stride of the four parameter vectors
+    float bn_eps;
+    const half_t* residual;
+    int relu;
     int out_ev;   // pixels per output store: the largest of 8, 4, 2, 1 that divides P (a run then stays inside one image)
 };
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t MakeRsrc(const void* ptr, unsigned bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(ptr), 0, static_cast<int>(bytes), 0x00020000);
 }
+
+template <int N>
+struct alignas(2 * N) PVecH {
+    half_t e[N];
+};
+template <int N>
+struct RawVec;
+template <>
+struct RawVec<8> {
+    using type = Bytes16;
+};
+template <>
+struct RawVec<4> {
+    using type = Bytes8;
+};
+template <>
+struct RawVec<2> {
+    using type = unsigned;
+};
+template <>
+struct RawVec<1> {
+    using type = unsigned short;
+};
 
 // NPX pixels (NPX * 2 bytes) of one channel plane as dwords.
 template <int NPX>
@@ -110,10 +143,13 @@ __global__ __launch_bounds__(64 * WPX * WCH) void NchwConvKernel(NchwConvArgs p)
     constexpr int KS = CK / 16;   // MFMA reduction steps per chunk and tap
     constexpr int WITEMS = TAPS * CG * BN;
     constexpr int WPT = (WITEMS + NT - 1) / NT;
+    // bytes of one channel group's filters in LDS; the 1x1 layout is padded by 64 bytes so that lanes that differ in the
+    // channel group (the order in which filters read in place are loaded) fall on different banks
+    constexpr int WCGP = TAPS * BN * 16 + (TAPS == 1 ? 64 : 0);
 
     extern __shared__ __align__(16) char lds[];
     const int patch_bytes = CG * p.nslot * 16;
-    const int stage_bytes = patch_bytes + WITEMS * 16;
+    const int stage_bytes = patch_bytes + CG * WCGP;
     const int dump_off = 2 * stage_bytes;  // NPX * 16 bytes that absorb the writes of idle load slots
 
     int tile_m, tile_n;
@@ -183,17 +219,24 @@ __global__ __launch_bounds__(64 * WPX * WCH) void NchwConvKernel(NchwConvArgs p)
 #pragma unroll
     for (int i = 0; i < WPT; ++i) {
         int wi = tid + i * NT;
-        int cg = wi / (TAPS * BN);
-        int rest = wi - cg * (TAPS * BN);
-        int tap = rest / BN;
-        int kl = rest - tap * BN;
+        int cg, tap, kl;
+        if (TAPS == 1 && p.w_direct) {  // consecutive lanes walk a filter row: 64 contiguous bytes per row and chunk
+            kl = wi / CG;
+            cg = wi - kl * CG;
+            tap = 0;
+        } else {  // packed filters: consecutive lanes walk the output channels of one (group, tap)
+            cg = wi / (TAPS * BN);
+            int rest = wi - cg * (TAPS * BN);
+            tap = rest / BN;
+            kl = rest - tap * BN;
+        }
         bool valid = wi < WITEMS && n0 + kl < p.K;
         if (TAPS == 1 && p.w_direct) {
             wvoff[i] = valid ? ((n0 + kl) * p.C + cg * 8) * 2 : 0x7fffffff;
         } else {
             wvoff[i] = valid ? ((cg * TAPS + tap) * p.K + n0 + kl) * 16 : 0x7fffffff;
         }
-        wlds[i] = wi < WITEMS ? patch_bytes + wi * 16 : -1;
+        wlds[i] = wi < WITEMS ? patch_bytes + cg * WCGP + (tap * BN + kl) * 16 : -1;
     }
 
     const __amdgpu_buffer_rsrc_t xr = MakeRsrc(p.x, p.x_bytes);
@@ -246,7 +289,7 @@ __global__ __launch_bounds__(64 * WPX * WCH) void NchwConvKernel(NchwConvArgs p)
         }
         aoff[a] = (g * p.nslot + slot) * 16;
     }
-    const int boff = patch_bytes + (g * TAPS * BN + wch * CW * 32 + lr) * 16;
+    const int boff = patch_bytes + g * WCGP + (wch * CW * 32 + lr) * 16;
     const int a_ks = 2 * p.nslot * 16;  // advance of one 16-channel reduction step in the patch
 
     float16_t acc[PW][CW];
@@ -271,7 +314,7 @@ __global__ __launch_bounds__(64 * WPX * WCH) void NchwConvKernel(NchwConvArgs p)
             for (int a = 0; a < PW; ++a) fa[a] = *reinterpret_cast<const Bytes16*>(stage + aoff[a] + toff + ks * a_ks);
 #pragma unroll
             for (int b = 0; b < CW; ++b) {
-                fb[b] = *reinterpret_cast<const Bytes16*>(stage + boff + ((ks * 2 * TAPS + tap) * BN + b * 32) * 16);
+                fb[b] = *reinterpret_cast<const Bytes16*>(stage + boff + ks * 2 * WCGP + (tap * BN + b * 32) * 16);
             }
         };
         read_frags(0, af[0], bf[0]);
@@ -312,32 +355,61 @@ __global__ __launch_bounds__(64 * WPX * WCH) void NchwConvKernel(NchwConvArgs p)
     // regrouped through LDS as [channel][pixel] (the last barrier of the loop has retired every stage read), so that
     // consecutive lanes store consecutive pixel runs of one channel plane: whole cache lines per instruction.
     constexpr int OPITCH = BM * 2 + 16;  // bytes per channel row
+    // The fused tail is compiled as separate straight-line variants (no per-element branches in the plain convolution).
+    auto stage_tile = [&](auto bn_tag, auto relu_tag) {
+        constexpr bool BN = decltype(bn_tag)::value;
+        constexpr bool RELU = decltype(relu_tag)::value;
 #pragma unroll
-    for (int b = 0; b < CW; ++b) {
-        const int row = (wch * CW + b) * 32 + lr;
-        const int n = n0 + row;
-        float bias = (p.bias != nullptr && n < p.K) ? static_cast<float>(p.bias[n * p.bias_stride]) : 0.f;
+        for (int b = 0; b < CW; ++b) {
+            const int row = (wch * CW + b) * 32 + lr;
+            const int n = n0 + row;
+            float bias = (p.bias != nullptr && n < p.K) ? static_cast<float>(p.bias[n * p.bias_stride]) : 0.f;
+            // batch norm in the reference's association order, ((v - mean) * inv_std) * gamma + beta, evaluated in float
+            float bn_mean = 0.f, bn_inv = 1.f, bn_gamma = 1.f, bn_beta = 0.f;
+            if (BN && n < p.K) {
+                bn_mean = static_cast<float>(p.bn_mean[n * p.bn_stride]);
+                bn_inv = 1.0f / sqrtf(static_cast<float>(p.bn_var[n * p.bn_stride]) + p.bn_eps);
+                bn_gamma = static_cast<float>(p.bn_gamma[n * p.bn_stride]);
+                bn_beta = static_cast<float>(p.bn_beta[n * p.bn_stride]);
+            }
 #pragma unroll
-        for (int a = 0; a < PW; ++a) {
+            for (int a = 0; a < PW; ++a) {
 #pragma unroll
-            for (int vq = 0; vq < 4; ++vq) {
-                const int col = (wpx * PW + a) * 32 + vq * 8 + g * 4;
-                struct alignas(8) Out4 {
-                    half_t e[4];
-                } pack;
+                for (int vq = 0; vq < 4; ++vq) {
+                    const int col = (wpx * PW + a) * 32 + vq * 8 + g * 4;
+                    PVecH<4> pack;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) pack.e[e] = static_cast<half_t>(acc[a][b][vq * 4 + e] + bias);
-                *reinterpret_cast<Out4*>(lds + row * OPITCH + col * 2) = pack;
+                    for (int e = 0; e < 4; ++e) {
+                        float v = acc[a][b][vq * 4 + e] + bias;
+                        if (BN) v = ((v - bn_mean) * bn_inv) * bn_gamma + bn_beta;
+                        if (RELU) v = v < 0.f ? 0.f : v;  // NaN < 0 is false: NaN passes, like IfLessElse(x, 0, 0, x)
+                        pack.e[e] = static_cast<half_t>(v);
+                    }
+                    *reinterpret_cast<PVecH<4>*>(lds + row * OPITCH + col * 2) = pack;
+                }
             }
         }
+    };
+    using True = std::integral_constant<bool, true>;
+    using False = std::integral_constant<bool, false>;
+    const bool has_bn = p.bn_gamma != nullptr;
+    const bool relu_here = p.relu && p.residual == nullptr;  // with a residual, ReLU follows the addition
+    if (has_bn) {
+        if (relu_here) stage_tile(True{}, True{});
+        else stage_tile(True{}, False{});
+    } else {
+        if (relu_here) stage_tile(False{}, True{});
+        else stage_tile(False{}, False{});
     }
     __syncthreads();
-    auto store_rows = [&](auto ev_tag) {
+    auto store_rows = [&](auto ev_tag, auto res_tag) {
         constexpr int EV = decltype(ev_tag)::value;  // pixels per store
+        constexpr bool RES = decltype(res_tag)::value;
         constexpr int CPR = BM / EV;                 // chunks per channel row
         static_assert(NT % CPR == 0 || CPR % NT == 0, "a thread keeps one pixel column");
         constexpr int COLS_PER_THREAD = CPR > NT ? CPR / NT : 1;
         constexpr int ROW_STEP = CPR > NT ? 1 : NT / CPR;
+        using Raw = typename RawVec<EV>::type;  // one LDS read and one global store of EV * 2 bytes
 #pragma unroll
         for (int cj = 0; cj < COLS_PER_THREAD; ++cj) {
             const int cc = (tid % (CPR > NT ? NT : CPR)) + cj * NT;
@@ -345,30 +417,37 @@ __global__ __launch_bounds__(64 * WPX * WCH) void NchwConvKernel(NchwConvArgs p)
             if (m >= p.M) continue;
             const int img = m / p.P;
             const int pix = m - img * p.P;
-            half_t* obase = p.out + static_cast<int64_t>(img) * p.K * p.P + pix;
+            const int64_t obase = static_cast<int64_t>(img) * p.K * p.P + pix;
             for (int row = (CPR > NT ? 0 : tid / CPR); row < BN; row += ROW_STEP) {
                 const int n = n0 + row;
                 if (n >= p.K) break;
-                const char* src = lds + row * OPITCH + cc * EV * 2;
-                half_t* dst = obase + static_cast<int64_t>(n) * p.P;
-                if constexpr (EV == 8) {
-                    *reinterpret_cast<Bytes16*>(dst) = *reinterpret_cast<const Bytes16*>(src);
-                } else if constexpr (EV == 4) {
-                    *reinterpret_cast<Bytes8*>(dst) = *reinterpret_cast<const Bytes8*>(src);
-                } else if constexpr (EV == 2) {
-                    *reinterpret_cast<unsigned*>(dst) = *reinterpret_cast<const unsigned*>(src);
-                } else {
-                    *dst = *reinterpret_cast<const half_t*>(src);
+                const int64_t o = obase + static_cast<int64_t>(n) * p.P;
+                Raw raw = *reinterpret_cast<const Raw*>(lds + row * OPITCH + cc * EV * 2);
+                if constexpr (RES) {  // y = relu(bn(conv) + residual): the addend is read with the same coalesced runs
+                    PVecH<EV> v = __builtin_bit_cast(PVecH<EV>, raw);
+                    PVecH<EV> r = __builtin_bit_cast(PVecH<EV>, *reinterpret_cast<const Raw*>(p.residual + o));
+#pragma unroll
+                    for (int e = 0; e < EV; ++e) {
+                        float t = static_cast<float>(v.e[e]) + static_cast<float>(r.e[e]);
+                        if (p.relu) t = t < 0.f ? 0.f : t;
+                        v.e[e] = static_cast<half_t>(t);
+                    }
+                    raw = __builtin_bit_cast(Raw, v);
                 }
+                *reinterpret_cast<Raw*>(p.out + o) = raw;
             }
         }
     };
     // EV consecutive pixels never straddle an image and are EV*2-byte aligned when P % EV == 0 (m0 % EV == 0 always)
+    auto store_ev = [&](auto ev_tag) {
+        if (p.residual != nullptr) store_rows(ev_tag, True{});
+        else store_rows(ev_tag, False{});
+    };
     switch (p.out_ev) {
-        case 8: store_rows(std::integral_constant<int, 8>{}); break;
-        case 4: store_rows(std::integral_constant<int, 4>{}); break;
-        case 2: store_rows(std::integral_constant<int, 2>{}); break;
-        default: store_rows(std::integral_constant<int, 1>{}); break;
+        case 8: store_ev(std::integral_constant<int, 8>{}); break;
+        case 4: store_ev(std::integral_constant<int, 4>{}); break;
+        case 2: store_ev(std::integral_constant<int, 2>{}); break;
+        default: store_ev(std::integral_constant<int, 1>{}); break;
     }
 }
 

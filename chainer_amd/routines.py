@@ -649,6 +649,31 @@ def conv(x, w, b=None, stride=1, pad=0, cover_all=False, out_dtype=None):
     return out
 
 
+def conv_bn_act(x, w, b=None, stride=1, pad=0, cover_all=False, bn=None, eps=2e-5, residual=None, relu=False):
+    """Opt-in fused block: relu(fixed_batch_norm(conv(x, w, b), *bn, eps, axis=(0, 2, 3)) + residual) in one kernel call.
+    `bn` is None or (gamma, beta, mean, var), one value per output channel.  Not part of the ChainerX routine surface:
+    the reference issues these as separate kernels (which `conv`, `fixed_batch_norm`, `add`, `relu` here do as well)."""
+    if x.ndim != 4 or w.ndim != 4:
+        raise _lib.ChainerxNotImplementedError('only 2-D convolution is on the supported path')
+    stride, pad = _pair(stride), _pair(pad)
+    if w.shape[1] != x.shape[1]:
+        raise _lib.DimensionError('Mismatched number of input channels in input %r and weights %r.' % (x.shape, w.shape))
+    dt = result_type(x, w)
+    oh = conv_out_dim(x.shape[2], w.shape[2], stride[0], pad[0], cover_all)
+    ow = conv_out_dim(x.shape[3], w.shape[3], stride[1], pad[1], cover_all)
+    out = _spatial_out(x, x.shape[0], w.shape[0], oh, ow, dt)
+    xc, wc = x.astype(dt, False), w.astype(dt, False)
+    bc = b.astype(dt, False) if b is not None else None
+    prm = [a.astype(dt, False).desc() for a in bn] if bn is not None else [None] * 4
+    res = residual.astype(dt, False) if residual is not None else None
+    nbytes = _lib.load().hipcx_conv_workspace_size(xc.desc(), wc.desc(), out.desc())
+    ws, wsp = _workspace(nbytes)
+    _lib.call('hipcx_conv_bn_act', xc.desc(), wc.desc(), bc.desc() if bc is not None else None, _i64(stride), _i64(pad),
+              int(bool(cover_all)), prm[0], prm[1], prm[2], prm[3], _lib.make_scalar(float(eps)),
+              res.desc() if res is not None else None, int(bool(relu)), out.desc(), wsp, nbytes, current_stream())
+    return out
+
+
 def fixed_batch_norm(x, gamma, beta, mean, var, eps=2e-5, axis=None):
     """FixedBatchNorm (CX/routines/normalization.cc:414-424 with PreprocessBatchNorm :61-101)."""
     for a in (x, gamma, beta, mean, var):

@@ -157,6 +157,19 @@ size_t hipcx_conv_workspace_size(const hipcx_array* x, const hipcx_array* w, con
 int hipcx_conv(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, const int64_t* stride, const int64_t* pad,
                int cover_all, const hipcx_array* out, void* workspace, size_t workspace_bytes, void* stream);
 
+/* Opt-in fused entry.  No single kernel of the reference corresponds to it: it is the composition
+ *   ConvKernel -> FixedBatchNormKernel over the output channels (axis (0,2,3), CX/routines/normalization.cc:113-153)
+ *   -> AddKernel with `residual` -> IfLessElseASSAKernel(x, 0, 0, x) (ReLU, CX/routines/misc.cc:210-216)
+ * that Chainer's conv-bn-relu blocks issue as separate kernel calls; here the tail runs in the convolution's epilogue,
+ * in float on the float accumulator, and `out` is written once.  gamma/beta/mean/var are all NULL (no batch norm) or
+ * hold one value of out's dtype per output channel ([K] or [1,K,1,1]); `residual` may be NULL; `relu` is 0 or 1.
+ * Layouts or dtypes the fused kernel does not take are served by the separate kernels run in place on `out`.
+ * Workspace as for hipcx_conv. */
+int hipcx_conv_bn_act(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, const int64_t* stride, const int64_t* pad,
+                      int cover_all, const hipcx_array* gamma, const hipcx_array* beta, const hipcx_array* mean, const hipcx_array* var,
+                      hipcx_scalar eps, const hipcx_array* residual, int relu, const hipcx_array* out, void* workspace,
+                      size_t workspace_bytes, void* stream);
+
 /* Measurement aid (no counterpart in the reference): between start and stop every implicit-GEMM launch made by
  * hipcx_dot / hipcx_conv from the calling process is bracketed by a pair of HIP events on its stream.  stop waits for them
  * and returns the number of launches, the sum of their durations, and their algorithmic flops (2 per multiply-add) and
