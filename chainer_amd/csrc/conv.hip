@@ -11,6 +11,7 @@
 #include "igemm_pipe.h"
 #include "layout_kernels.h"
 #include "nchw_conv.h"
+#include "stem_conv.h"
 
 namespace hipcx {
 namespace {
@@ -350,6 +351,79 @@ void RunNchw(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, c
     }
 }
 
+
+// ---- float16 7x7/2 stem path (stem_conv.h) ----
+struct StemPlan {
+    bool ok = false;
+    int rowp = 0, copyb = 0, lds_bytes = 0, ksteps = 0;
+    size_t wp_bytes = 0;
+};
+
+StemPlan PlanStem(const hipcx_array* x, const hipcx_array* w, const hipcx_array* out, const int64_t* stride, const int64_t* pad) {
+    StemPlan pl;
+    static const bool enabled = [] { const char* e = getenv("HIPCX_CONV_STEM"); return e == nullptr || e[0] != '0'; }();
+    if (!enabled || x->dtype != HIPCX_FLOAT16 || !IsContiguous(x) || !IsContiguous(out)) return pl;
+    const int64_t N = x->shape[0], C = x->shape[1], H = x->shape[2], W = x->shape[3];
+    const int64_t K = w->shape[0], OH = out->shape[2], OW = out->shape[3];
+    if (C != 3 || K != 64 || w->shape[2] != 7 || w->shape[3] != 7) return pl;
+    if (stride[0] != 2 || stride[1] != 2 || pad[0] != 3 || pad[1] != 3) return pl;
+    if (W % 8 != 0 || OW * 2 != W || OW % 8 != 0 || 2 * OW > 256 || OH != (H - 1) / 2 + 1) return pl;
+    if (N * C * H * W * 2 >= (1LL << 31) || N * K * OH * OW * 2 >= (1LL << 31)) return pl;
+    if (reinterpret_cast<uintptr_t>(x->data) % 16 != 0 || reinterpret_cast<uintptr_t>(out->data) % 16 != 0) return pl;
+    pl.ksteps = static_cast<int>((C * 7 + 1) / 2);
+    pl.rowp = static_cast<int>(W / 8 * 16);
+    int need = static_cast<int>(C * 9 + 3) * pl.rowp;
+    pl.copyb = need + ((64 - need % 256) + 256) % 256;  // copies 64 bytes apart modulo 256: neighbouring lanes hit different banks
+    pl.lds_bytes = std::max(4 * pl.copyb, 64 * (static_cast<int>(OW) * 4 + 16));
+    if (pl.lds_bytes > 160 * 1024) return pl;
+    pl.wp_bytes = static_cast<size_t>(pl.ksteps) * 2 * 64 * 16;
+    pl.ok = true;
+    return pl;
+}
+
+void RunStem(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, const StemPlan& pl, const hipcx_array* out, char* workspace,
+             hipStream_t stream, const FusedTail& tail = FusedTail{}) {
+    StemConvArgs a{};
+    a.x = static_cast<const half_t*>(x->data);
+    a.wp = reinterpret_cast<const half_t*>(workspace);
+    a.bias = b ? static_cast<const half_t*>(b->data) : nullptr;
+    a.bias_stride = b ? b->strides[0] / 2 : 0;
+    a.out = static_cast<half_t*>(out->data);
+    a.N = static_cast<int>(x->shape[0]);
+    a.H = static_cast<int>(x->shape[2]);
+    a.W = static_cast<int>(x->shape[3]);
+    a.OH = static_cast<int>(out->shape[2]);
+    a.OW = static_cast<int>(out->shape[3]);
+    a.x_bytes = static_cast<unsigned>(static_cast<int64_t>(a.N) * 3 * a.H * a.W * 2);
+    a.wp_bytes = static_cast<unsigned>(pl.wp_bytes);
+    a.rowp = pl.rowp;
+    a.copyb = pl.copyb;
+    a.bn_gamma = tail.gamma;
+    a.bn_beta = tail.beta;
+    a.bn_mean = tail.mean;
+    a.bn_var = tail.var;
+    a.bn_stride = tail.stride;
+    a.bn_eps = tail.eps;
+    a.relu = tail.relu;
+    int groups = pl.ksteps * 2 * 64;
+    hipLaunchKernelGGL(StemRepackFiltersKernel, dim3((groups + 255) / 256), dim3(256), 0, stream, static_cast<const half_t*>(w->data),
+                       reinterpret_cast<half_t*>(workspace), 3, pl.ksteps, w->strides[0] / 2, w->strides[1] / 2, w->strides[2] / 2,
+                       w->strides[3] / 2);
+    CheckLaunch("stem_repack_filters");
+    const double M = static_cast<double>(a.N) * a.OH * a.OW;
+    ProfileScope prof(stream, 2.0 * M * 64 * 3 * 49,
+                      2.0 * (static_cast<double>(a.N) * 3 * a.H * a.W + 64.0 * 3 * 49 + M * 64));
+    auto kern = StemConv7x7s2Kernel<3>;
+    static int configured = 0;
+    if (pl.lds_bytes > configured) {
+        HIPCX_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, pl.lds_bytes));
+        configured = pl.lds_bytes;
+    }
+    int blocks = a.N * ((a.OH + 1) / 2);
+    hipLaunchKernelGGL(kern, dim3(blocks), dim3(256), pl.lds_bytes, stream, a);
+    CheckLaunch("stem_conv");
+}
+
 // How a convolution is staged.  The MFMA kernel wants the reduction axis (r, s, c) contiguous in
 // both operands, i.e. channels-last activations and [K][R][S][C] filters.  Activations that are not
 // channels-last (the C-contiguous NCHW arrays ChainerX routines allocate) are gathered into a
@@ -594,7 +668,7 @@ size_t hipcx_conv_workspace_size(const hipcx_array* x, const hipcx_array* w, con
         ConvPlan pl = PlanConv(x, w, one, zero);
         size_t need = pl.x_bytes + pl.w_bytes;
         // the NCHW-native float16 path needs room for the packed filters only; report the larger of the two
-        if (x->dtype == HIPCX_FLOAT16) need = std::max(need, RoundUpTo(static_cast<size_t>(TotalSize(w)) * 2, 256));
+        if (x->dtype == HIPCX_FLOAT16) need = std::max(need, RoundUpTo(static_cast<size_t>(TotalSize(w)) * 2, 256) + 8192);  // packed filters, padded taps
         return need;
     } catch (...) {
         return 0;
@@ -613,6 +687,11 @@ int hipcx_conv(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b,
                           "conv workspace too small: need " + std::to_string(npl.wp_bytes) + " bytes");
             HIPCX_REQUIRE(reinterpret_cast<uintptr_t>(workspace) % 16 == 0, HIPCX_CHAINERX_ERROR, "workspace must be 16-byte aligned");
             RunNchw(x, w, b, npl, stride, out, static_cast<char*>(workspace), st);
+            return;
+        }
+        StemPlan spl = PlanStem(x, w, out, stride, pad);
+        if (spl.ok && workspace != nullptr && workspace_bytes >= spl.wp_bytes && reinterpret_cast<uintptr_t>(workspace) % 16 == 0) {
+            RunStem(x, w, b, spl, out, static_cast<char*>(workspace), st);
             return;
         }
         ConvPlan pl = PlanConv(x, w, stride, pad);
@@ -673,22 +752,28 @@ int hipcx_conv_bn_act(const hipcx_array* x, const hipcx_array* w, const hipcx_ar
         NchwPlan npl = PlanNchw(x, w, out, stride, pad);
         const bool same_stride = !has_bn || (sg == sb && sg == sm && sg == sv);
         const bool res_ok = residual == nullptr || (IsContiguous(residual) && reinterpret_cast<uintptr_t>(residual->data) % 16 == 0);
+        FusedTail tail;
+        if (has_bn) {
+            tail.gamma = static_cast<const half_t*>(gamma->data);
+            tail.beta = static_cast<const half_t*>(beta->data);
+            tail.mean = static_cast<const half_t*>(mean->data);
+            tail.var = static_cast<const half_t*>(var->data);
+            tail.stride = sg;
+            tail.eps = static_cast<float>(eps.kind == HIPCX_KIND_FLOAT ? eps.f : static_cast<double>(eps.i));
+        }
+        tail.residual = residual ? static_cast<const half_t*>(residual->data) : nullptr;
+        tail.relu = relu ? 1 : 0;
+        const bool ws_aligned = reinterpret_cast<uintptr_t>(workspace) % 16 == 0;
         if (npl.ok && same_stride && res_ok) {
             HIPCX_REQUIRE(workspace != nullptr && workspace_bytes >= npl.wp_bytes, HIPCX_CHAINERX_ERROR,
                           "conv workspace too small: need " + std::to_string(npl.wp_bytes) + " bytes");
-            HIPCX_REQUIRE(reinterpret_cast<uintptr_t>(workspace) % 16 == 0, HIPCX_CHAINERX_ERROR, "workspace must be 16-byte aligned");
-            FusedTail tail;
-            if (has_bn) {
-                tail.gamma = static_cast<const half_t*>(gamma->data);
-                tail.beta = static_cast<const half_t*>(beta->data);
-                tail.mean = static_cast<const half_t*>(mean->data);
-                tail.var = static_cast<const half_t*>(var->data);
-                tail.stride = sg;
-                tail.eps = static_cast<float>(eps.kind == HIPCX_KIND_FLOAT ? eps.f : static_cast<double>(eps.i));
-            }
-            tail.residual = residual ? static_cast<const half_t*>(residual->data) : nullptr;
-            tail.relu = relu ? 1 : 0;
+            HIPCX_REQUIRE(ws_aligned, HIPCX_CHAINERX_ERROR, "workspace must be 16-byte aligned");
             RunNchw(x, w, b, npl, stride, out, static_cast<char*>(workspace), st, tail);
+            return;
+        }
+        StemPlan spl = PlanStem(x, w, out, stride, pad);
+        if (spl.ok && same_stride && residual == nullptr && workspace != nullptr && workspace_bytes >= spl.wp_bytes && ws_aligned) {
+            RunStem(x, w, b, spl, out, static_cast<char*>(workspace), st, tail);
             return;
         }
         // Any other dtype / layout / geometry: the same result from the separate kernels, in place on `out`.

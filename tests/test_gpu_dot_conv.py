@@ -23,6 +23,8 @@ CONV_CASES = [
     (1, 24, 6, 6, 70, 1, 1, 1, 0, False),
     (4, 128, 9, 9, 128, 3, 3, 1, 1, False),
     (2, 20, 6, 7, 9, 2, 3, (1, 2), (0, 1), True),
+    (2, 3, 64, 64, 64, 7, 7, 2, 3, False),   # ImageNet stem geometry (dedicated float16 kernel)
+    (1, 3, 30, 48, 64, 7, 7, 2, 3, False),   # same with an odd number of output rows
 ]
 
 

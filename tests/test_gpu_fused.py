@@ -20,7 +20,7 @@ def ref_block(x, w, b, stride, pad, bn, residual, relu):
 
 CASES = [  # N, C, H, W, K, R, stride, pad
     (2, 64, 8, 8, 64, 1, 1, 0), (3, 32, 14, 14, 128, 1, 2, 0), (2, 16, 12, 12, 32, 3, 1, 1), (4, 64, 7, 7, 256, 1, 1, 0),
-    (2, 128, 7, 7, 128, 3, 1, 1), (1, 3, 20, 20, 16, 7, 2, 3), (2, 24, 6, 6, 40, 3, 2, 1),
+    (2, 128, 7, 7, 128, 3, 1, 1), (1, 3, 20, 20, 16, 7, 2, 3), (2, 24, 6, 6, 40, 3, 2, 1), (2, 3, 32, 32, 64, 7, 2, 3),
 ]
 
 
