@@ -247,7 +247,7 @@ def lstm_lm_input(seed=5, batch=128, seq=35, vocab=10000):
     return _rng(seed + 1000).integers(0, vocab, (batch, seq)).astype(np.int32)
 
 
-def lstm_lm_forward(F, p, ids, zeros):
+def lstm_lm_forward(F, p, ids, zeros, take_mode=None):
     """Runs the sequence; returns log-probabilities of the last step and the final (h, c) of both layers.
     ``zeros(shape, dtype)`` makes the initial state on the same backend as ``F``."""
     batch, seq = ids.shape
@@ -257,7 +257,7 @@ def lstm_lm_forward(F, p, ids, zeros):
     cs = [zeros((batch, units), dtype) for _ in range(2)]
     y = None
     for t in range(seq):
-        x = F.take(p['embed'], ids[:, t], 0)
+        x = F.take(p['embed'], ids[:, t], 0, take_mode)
         for li, layer in enumerate(p['layers']):
             gates = F.add(F.linear(x, layer['up_w'], layer['up_b']), F.linear(hs[li], layer['lat_w']))
             hs[li], cs[li] = F.lstm(cs[li], gates)

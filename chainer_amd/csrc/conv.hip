@@ -12,6 +12,7 @@
 #include "layout_kernels.h"
 #include "nchw_conv.h"
 #include "stem_conv.h"
+#include "small_dot.h"
 
 namespace hipcx {
 namespace {
@@ -141,13 +142,59 @@ void LaunchIGemmImpl(IGemmArgs<T> p, hipStream_t stream) {
     }
     bool fast16 = FastOk(p, 16);
     bool fast8 = !fast16 && FastOk(p, 8);
-    if (p.K <= 64) {
+    // Small problems (batch-sized matrix products such as Linear on 100-128 rows): at 128x128 the grid would leave most of
+    // the 256 CUs idle, so they run as one-wave 64x64 tiles instead.
+    const int64_t big_tiles = ((p.M + 127) / 128) * ((p.K + 127) / 128);
+    if (big_tiles < 128 && p.M * static_cast<int64_t>(p.K) >= 64 * 64) {
+        if (pm) LaunchShape<T, 1, 1, true>(p, fast16, fast8, stream);
+        else LaunchShape<T, 1, 1, false>(p, fast16, fast8, stream);
+    } else if (p.K <= 64) {
         if (pm) LaunchShape<T, 4, 1, true>(p, fast16, fast8, stream);
         else LaunchShape<T, 4, 1, false>(p, fast16, fast8, stream);
     } else {
         if (pm) LaunchShape<T, 2, 2, true>(p, fast16, fast8, stream);
         else LaunchShape<T, 2, 2, false>(p, fast16, fast8, stream);
     }
+}
+
+
+// Small-output matrix products (small_dot.h).  Returns false when the problem does not qualify.
+template <typename T>
+bool TrySmallDot(const hipcx_array* a, const hipcx_array* b, const hipcx_array* out, hipStream_t stream) {
+    static const bool enabled = [] { const char* e = getenv("HIPCX_SMALL_DOT"); return e == nullptr || e[0] != '0'; }();
+    if (!enabled) return false;
+    const int64_t M = a->shape[0], K = a->shape[1], N = b->shape[1];
+    const int64_t it = sizeof(T);
+    if (((M + 127) / 128) * ((N + 127) / 128) >= 128 || K < 64) return false;
+    for (const hipcx_array* x : {a, b, out}) {
+        if (x->strides[0] < 0 || x->strides[1] < 0 || x->strides[0] % it || x->strides[1] % it) return false;
+    }
+    SmallDotArgs p{};
+    p.a = a->data;
+    p.b = b->data;
+    p.out = out->data;
+    p.M = static_cast<int>(M);
+    p.N = static_cast<int>(N);
+    p.K = static_cast<int>(K);
+    p.a_row = a->strides[0] / it;
+    p.a_k = a->strides[1] / it;
+    p.b_k = b->strides[0] / it;
+    p.b_col = b->strides[1] / it;
+    p.o_row = out->strides[0] / it;
+    p.o_col = out->strides[1] / it;
+    int64_t a_span = ((M - 1) * p.a_row + (K - 1) * p.a_k + 1) * it, b_span = ((K - 1) * p.b_k + (N - 1) * p.b_col + 1) * it;
+    if (a_span >= (1LL << 31) || b_span >= (1LL << 31)) return false;
+    p.a_bytes = static_cast<unsigned>(a_span);
+    p.b_bytes = static_cast<unsigned>(b_span);
+    auto dword_ok = [&](const void* ptr, int64_t line_stride) { return reinterpret_cast<uintptr_t>(ptr) % 4 == 0 && (line_stride * it) % 4 == 0; };
+    p.a_vec = (p.a_k == 1 && dword_ok(a->data, p.a_row)) ? 1 : 0;
+    p.b_vec = (p.b_k == 1 && dword_ok(b->data, p.b_col)) ? 1 : 0;
+    p.tiles_n = static_cast<int>((N + 31) / 32);
+    int64_t blocks = ((M + 31) / 32) * p.tiles_n;
+    ProfileScope prof(stream, 2.0 * M * N * K, static_cast<double>(it) * (M * K + K * N + M * N));
+    hipLaunchKernelGGL((SmallDotKernel<T>), dim3(static_cast<unsigned>(blocks)), dim3(512), 0, stream, p);
+    CheckLaunch("small_dot");
+    return true;
 }
 
 // float64 (no MFMA path yet): one thread per output element, fma in reduction order.
@@ -862,10 +909,12 @@ int hipcx_dot(const hipcx_array* a, const hipcx_array* b, const hipcx_array* out
             p.Kg = static_cast<int>(k);
         };
         if (out->dtype == HIPCX_FLOAT16) {
+            if (TrySmallDot<half_t>(a, b, out, st)) return;
             IGemmArgs<half_t> p{};
             fill(p);
             LaunchIGemmImpl(p, st);
         } else if (out->dtype == HIPCX_FLOAT32) {
+            if (TrySmallDot<float>(a, b, out, st)) return;
             IGemmArgs<float> p{};
             fill(p);
             LaunchIGemmImpl(p, st);

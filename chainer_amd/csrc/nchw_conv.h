@@ -16,7 +16,8 @@
 // Both LDS arrays are exactly the operand layout of v_mfma_f32_32x32x16_f16 (lane = row/column, 8 consecutive
 // reduction indices per lane), so a fragment is one conflict-free ds_read_b128 of consecutive 16-byte groups, and
 // a 3x3 tap is a constant slot offset into the same patch: the patch is written once and read nine times.
-// Two LDS stages; global loads of chunk i+1 are in flight while chunk i is multiplied; one barrier per chunk.
+// Two LDS stages; chunk i+1 is written to LDS and the loads of chunk i+2 are issued before chunk i is multiplied;
+// one barrier per chunk.
 // All addresses are computed once per workgroup; inside the channel loop only a scalar offset advances, and
 // out-of-range loads are served as zeros by the buffer bounds check instead of branches.
 //
@@ -332,21 +333,25 @@ __global__ __launch_bounds__(64 * WPX * WCH) void NchwConvKernel(NchwConvArgs p)
     };
 
     // ---- pipeline ----
+    // Stage (ci & 1) holds chunk ci.  At the top of iteration ci the registers hold chunk ci+1, loaded one whole
+    // iteration ago: they go to the other stage (free since the barrier that ended iteration ci-1), the loads of chunk
+    // ci+2 are issued into the same registers, and only then chunk ci is multiplied.  No wave ever waits for a load it
+    // has just issued, and the LDS writes of one wave overlap the MFMAs of the others.
+    const int nchunks = p.C / CK;
     load_chunk(0);
     if constexpr (TAPS == 9) {  // borders of both patches must read as zero; nothing ever writes them
         for (int off = tid * 16; off < 2 * stage_bytes; off += NT * 16) *reinterpret_cast<Bytes16*>(lds + off) = Bytes16(0);
         __syncthreads();
     }
     store_chunk(lds);
+    if (nchunks > 1) load_chunk(1);
     __syncthreads();
-    const int nchunks = p.C / CK;
     for (int ci = 0; ci < nchunks; ++ci) {
         char* cur = lds + (ci & 1) * stage_bytes;
         char* nxt = lds + ((ci + 1) & 1) * stage_bytes;
-        const bool more = ci + 1 < nchunks;
-        if (more) load_chunk(ci + 1);
+        if (ci + 1 < nchunks) store_chunk(nxt);
+        if (ci + 2 < nchunks) load_chunk(ci + 2);
         compute(cur);
-        if (more) store_chunk(nxt);
         __syncthreads();
     }
 
