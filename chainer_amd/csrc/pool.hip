@@ -155,7 +155,7 @@ __global__ __launch_bounds__(256) void PoolKernel(PoolArgs p, int64_t total) {
 // two aligned 16-byte loads per input row (columns [2*ow0 - EPV, 2*ow0 + EPV)), instead of kh*kw scalar loads per
 // output.  Requires W % EPV == 0, OW % (EPV/2) == 0, pw <= EPV and kw <= pw + 2 (then every tap falls inside the two
 // chunks), which covers the 3x3/2 pad 1 and 2x2/2 pad 0 windows.
-template <typename T>
+template <typename T, int KW, int PW>
 __global__ __launch_bounds__(256) void MaxPoolRowsS2Kernel(PoolArgs p, int64_t total) {
     constexpr int EPV = 16 / sizeof(T);
     constexpr int VO = EPV / 2;
@@ -193,12 +193,9 @@ __global__ __launch_bounds__(256) void MaxPoolRowsS2Kernel(PoolArgs p, int64_t t
 #pragma unroll
             for (int e = 0; e < VO; ++e) {
 #pragma unroll
-                for (int s = 0; s < 2 * EPV; ++s) {  // taps of output e: window columns EPV + 2e - pw + [0, kw)
-                    int rel = s - (EPV + 2 * e - p.pw);
-                    if (rel >= 0 && rel < p.kw) {
-                        T v = win[s];
-                        if (IsNanT(v) || acc[e] < v) acc[e] = v;
-                    }
+                for (int t = 0; t < KW; ++t) {  // taps of output e: window columns EPV + 2e - PW + [0, KW)
+                    T v = win[EPV + 2 * e - PW + t];
+                    if (IsNanT(v) || acc[e] < v) acc[e] = v;
                 }
             }
         }
@@ -206,6 +203,35 @@ __global__ __launch_bounds__(256) void MaxPoolRowsS2Kernel(PoolArgs p, int64_t t
 #pragma unroll
         for (int e = 0; e < VO; ++e) res.v[e] = acc[e];
         *reinterpret_cast<PVec<T, VO>*>(out + (plane * p.OH + oh) * p.OW + ow0) = res;
+    }
+}
+
+// Global average pooling over dense NCHW planes (window = whole plane, no padding): a workgroup copies 256 consecutive
+// planes (one contiguous run) into LDS with 16-byte loads, then each thread sums one plane.  Sum in the compute type,
+// rounded to T, then divided in T arithmetic, like Sum followed by Divide.
+template <typename T>
+__global__ __launch_bounds__(256) void GlobalAvgPoolKernel(const T* x, T* out, int64_t planes, int hw) {
+    using C = compute_t<T>;
+    extern __shared__ __align__(16) char lds[];
+    const int64_t p0 = static_cast<int64_t>(blockIdx.x) * 256;
+    const int64_t np = planes - p0 < 256 ? planes - p0 : 256;
+    const int64_t bytes = np * hw * static_cast<int64_t>(sizeof(T));
+    const char* src = reinterpret_cast<const char*>(x + p0 * hw);
+    for (int64_t off = static_cast<int64_t>(threadIdx.x) * 16; off < bytes; off += 256 * 16) {
+        if (off + 16 <= bytes) {
+            *reinterpret_cast<PVec<unsigned, 4>*>(lds + off) = *reinterpret_cast<const PVec<unsigned, 4>*>(src + off);
+        } else {
+            for (int64_t b = off; b < bytes; ++b) lds[b] = src[b];
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x < np) {
+        const T* pl = reinterpret_cast<const T*>(lds) + threadIdx.x * hw;
+        C acc = C(0);
+        for (int i = 0; i < hw; ++i) acc += static_cast<C>(pl[i]);
+        T s = static_cast<T>(acc);
+        C div = static_cast<C>(static_cast<T>(static_cast<C>(hw)));
+        out[p0 + threadIdx.x] = static_cast<T>(static_cast<C>(s) / div);
     }
 }
 
@@ -231,8 +257,30 @@ void RunPool(PoolArgs p, hipStream_t stream) {
             int64_t blocks = (total + 255) / 256;
             int64_t cap = static_cast<int64_t>(NumCUs()) * 32;
             if (blocks > cap) blocks = cap;
-            hipLaunchKernelGGL((MaxPoolRowsS2Kernel<T>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, p, total);
-            CheckLaunch("max_pool_rows");
+            if (p.kw == 3 && p.pw == 1) {
+                hipLaunchKernelGGL((MaxPoolRowsS2Kernel<T, 3, 1>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, p, total);
+                CheckLaunch("max_pool_rows");
+                return;
+            }
+            if (p.kw == 2 && p.pw == 0) {
+                hipLaunchKernelGGL((MaxPoolRowsS2Kernel<T, 2, 0>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, p, total);
+                CheckLaunch("max_pool_rows");
+                return;
+            }
+        }
+    }
+    if constexpr (!IS_MAX) {
+        bool dense_in = p.xsW == 1 && p.xsH == p.W && p.xsC == static_cast<int64_t>(p.H) * p.W && p.xsN == p.xsC * p.C;
+        bool dense_out = p.osC == 1 && p.osN == p.C;  // [N, C, 1, 1]
+        int hw = p.H * p.W;
+        if (dense_in && dense_out && p.kh == p.H && p.kw == p.W && p.ph == 0 && p.pw == 0 && p.OH == 1 && p.OW == 1 &&
+            256 * hw * static_cast<int>(sizeof(T)) <= 64 * 1024 && Aligned(p.x, 16)) {
+            int64_t planes = static_cast<int64_t>(p.N) * p.C;
+            if (planes == 0) return;
+            int lds_bytes = 256 * hw * static_cast<int>(sizeof(T));
+            hipLaunchKernelGGL((GlobalAvgPoolKernel<T>), dim3(static_cast<unsigned>((planes + 255) / 256)), dim3(256), lds_bytes, stream,
+                               static_cast<const T*>(p.x), static_cast<T*>(p.out), planes, hw);
+            CheckLaunch("global_avg_pool");
             return;
         }
     }
