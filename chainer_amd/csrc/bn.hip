@@ -103,6 +103,7 @@ __global__ __launch_bounds__(kBnFlatThreads) void BnChannelsFirstKernel(const T*
         prm[r * 4 + 3] = static_cast<C>(beta[ch * pstride]);
     }
     __syncthreads();
+    const bool rows_hold_whole_vectors = L % VEC == 0;
     Vec<T, VEC> in[kBnFlatUnroll];
     int64_t idx[kBnFlatUnroll];
 #pragma unroll
@@ -117,19 +118,31 @@ __global__ __launch_bounds__(kBnFlatThreads) void BnChannelsFirstKernel(const T*
         int col = static_cast<int>(idx[u] - row * L);
         int r = static_cast<int>(row - row_first);
         Vec<T, VEC> o;
+        if (rows_hold_whole_vectors) {  // L % VEC == 0: one parameter set per vector
+            const C q0 = prm[r * 4 + 0], q1 = prm[r * 4 + 1], q2 = prm[r * 4 + 2], q3 = prm[r * 4 + 3];
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) {
-            if (col >= L) {  // the vector crosses into the next row(s)
-                col -= static_cast<int>(L);
-                ++r;
+            for (int e = 0; e < VEC; ++e) {
+                C t = static_cast<C>(in[u].v[e]) - q0;
+                t = t * q1;
+                t = t * q2;
+                t = t + q3;
+                o.v[e] = static_cast<T>(t);
             }
-            const C* q = prm + r * 4;
-            C t = static_cast<C>(in[u].v[e]) - q[0];
-            t = t * q[1];
-            t = t * q[2];
-            t = t + q[3];
-            o.v[e] = static_cast<T>(t);
-            ++col;
+        } else {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                if (col >= L) {  // the vector crosses into the next row(s)
+                    col -= static_cast<int>(L);
+                    ++r;
+                }
+                const C* q = prm + r * 4;
+                C t = static_cast<C>(in[u].v[e]) - q[0];
+                t = t * q[1];
+                t = t * q[2];
+                t = t + q[3];
+                o.v[e] = static_cast<T>(t);
+                ++col;
+            }
         }
         *reinterpret_cast<Vec<T, VEC>*>(out + idx[u]) = o;
     }
