@@ -27,6 +27,10 @@ import numpy as np
 sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
 
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 matrix peak
+# HBM bytes per convolution launch (fetch + write, averaged over the 53 convolutions of one step), from two rocprofv3
+# --pmc runs (FETCH_SIZE, WRITE_SIZE) scaled by what the same counters read for a 128 MiB copy kernel (x1.999, x1.000):
+# profiles/resnet50_conv_hbm_traffic.txt.  The algorithmic figure is 101 MB per launch.
+CONV_HBM_TRAFFIC_BYTES_PER_LAUNCH = 112.1e6
 
 
 def main():
@@ -127,7 +131,7 @@ def main():
         'peak': MFMA_F16_PEAK_TFLOPS,
         'unit': 'TFLOP/s',
         'frac': round(achieved_tflops / MFMA_F16_PEAK_TFLOPS, 4),
-        'traffic': None,
+        'traffic': CONV_HBM_TRAFFIC_BYTES_PER_LAUNCH if args.batch == 128 else None,
         'launches_per_step': launches_per_step,
         'avg_launch_us': round(avg_launch_ms * 1e3, 2),
         'kernel_ms_per_step': round(ms.value / prof_steps, 3),

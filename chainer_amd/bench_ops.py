@@ -222,7 +222,14 @@ def section_lstm(chx, oracle, with_cpu):
         emit(section='lstm', op='cpu native 1 core, one time step', ms=round(cpu_time(lambda: cfg.lstm_lm_forward(oracle, p, ids2, np.zeros), 1.0) * 1e3, 1))
 
 
-SECTIONS = {'sweep': section_sweep, 'mlp': section_mlp, 'cifar': section_cifar, 'resnet_layers': section_resnet_layers, 'lstm': section_lstm}
+def section_copy(chx, oracle, with_cpu):
+    """A plain copy of known size (128 MiB read + 128 MiB written): the calibration point for HBM traffic counters."""
+    x = chx.array(np.zeros(64 * 1024 * 1024, np.float16))
+    t = device_time(lambda: chx.copy(x), 10, 3)
+    bw_row('copy', 'copy float16 [67108864]', (64 * 1024 * 1024,), t, 2 * x.nbytes)
+
+
+SECTIONS = {'copy': section_copy, 'sweep': section_sweep, 'mlp': section_mlp, 'cifar': section_cifar, 'resnet_layers': section_resnet_layers, 'lstm': section_lstm}
 
 
 def run(sections, cpu=None):
@@ -235,7 +242,7 @@ def run(sections, cpu=None):
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument('--section', default=','.join(SECTIONS))
+    ap.add_argument('--section', default=','.join(k for k in SECTIONS if k != 'copy'))
     args = ap.parse_args()
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     if root not in sys.path:
