@@ -277,6 +277,11 @@ NchwPlan PlanNchw(const hipcx_array* x, const hipcx_array* w, const hipcx_array*
         if (K <= 64) {
             pl.wpx = 4, pl.wch = 1;
             pl.maxi = pl.npx == 2 ? 2 : 4;
+        } else if (K >= 256 && pl.npx == 1) {
+            // single-pixel gathers (strided or odd-sized planes) are the expensive part of a tile: 128 pixels x 256 channels with
+            // 8 waves gathers and transposes each activation tile once for 256 output channels instead of 128
+            pl.wpx = 2, pl.wch = 4;
+            pl.maxi = 1;
         } else {
             pl.wpx = 2, pl.wch = 2;
             pl.maxi = pl.npx == 2 ? 1 : 2;
@@ -367,6 +372,7 @@ void RunNchw(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, c
     a.x_bytes = static_cast<unsigned>(static_cast<int64_t>(a.N) * a.C * a.H * a.W * 2);
     const int RS = static_cast<int>(w->shape[2] * w->shape[3]);
     a.wp_bytes = static_cast<unsigned>(static_cast<int64_t>(a.K) * a.C * RS * 2);
+    a.pair_load = (pl.taps == 1 && pl.npx == 1 && a.stride == 2 && a.W % 2 == 0) ? 1 : 0;
     a.out_ev = a.P % 8 == 0 ? 8 : a.P % 4 == 0 ? 4 : a.P % 2 == 0 ? 2 : 1;
     const bool w_dense = w->strides[1] == 2 && w->strides[0] == static_cast<int64_t>(a.C) * 2 && reinterpret_cast<uintptr_t>(w->data) % 16 == 0;
     static const bool direct_ok = [] { const char* e = getenv("HIPCX_W_DIRECT"); return e == nullptr || e[0] != '0'; }();
@@ -389,6 +395,7 @@ void RunNchw(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, c
         case 1000 + 400 + 20 + 2: LaunchNchwKernel<1, 4, 1, 32, 2, 2>(a, pl.lds_bytes, stream); break;
         case 1000 + 400 + 10 + 4: LaunchNchwKernel<1, 4, 1, 32, 1, 4>(a, pl.lds_bytes, stream); break;
         case 1000 + 200 + 20 + 1: LaunchNchwKernel<1, 2, 2, 32, 2, 1>(a, pl.lds_bytes, stream); break;
+        case 1000 + 200 + 10 + 1: LaunchNchwKernel<1, 2, 4, 32, 1, 1>(a, pl.lds_bytes, stream); break;
         case 1000 + 200 + 10 + 2: LaunchNchwKernel<1, 2, 2, 32, 1, 2>(a, pl.lds_bytes, stream); break;
         case 9000 + 400 + 20 + 2: LaunchNchwKernel<9, 4, 1, 16, 2, 2>(a, pl.lds_bytes, stream); break;
         case 9000 + 400 + 20 + 4: LaunchNchwKernel<9, 4, 1, 16, 2, 4>(a, pl.lds_bytes, stream); break;

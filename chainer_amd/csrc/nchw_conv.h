@@ -46,6 +46,7 @@ struct NchwConvArgs {
     int nslot;  // slots per channel group in the LDS patch
     int64_t bias_stride;
     unsigned x_bytes, wp_bytes;
+    int pair_load;  // NPX == 1 only: every wanted pixel sits at an even element offset with a readable odd neighbour (stride 2, even W)
     int w_direct;  // 1x1 only: read the filter bank in place (a row's 8 consecutive channels are one 16-byte group already)
     // Optional fused tail (all null / 0 for a plain convolution): fixed batch normalisation over the output channels,
     // a residual addend of out's shape (dense NCHW) and ReLU.
@@ -124,7 +125,7 @@ __device__ __forceinline__ void Transpose8(const PixVec<NPX> (&in)[8], Bytes16 (
 #pragma unroll
         for (int d = 0; d < 4; ++d) {
             if constexpr (NPX == 1) {
-                dw[d] = in[2 * d].d[0] | (in[2 * d + 1].d[0] << 16);
+                dw[d] = __builtin_amdgcn_perm(in[2 * d + 1].d[0], in[2 * d].d[0], 0x05040100u);  // low halves (the high ones may hold a neighbour)
             } else {
                 unsigned a = in[2 * d].d[e / 2], b = in[2 * d + 1].d[e / 2];
                 dw[d] = (e & 1) ? __builtin_amdgcn_perm(b, a, 0x07060302u) : __builtin_amdgcn_perm(b, a, 0x05040100u);
@@ -250,7 +251,15 @@ __global__ __launch_bounds__(64 * WPX * WCH) void NchwConvKernel(NchwConvArgs p)
 #pragma unroll
         for (int i = 0; i < MAXI; ++i) {
 #pragma unroll
-            for (int j = 0; j < 8; ++j) xreg[i][j] = BufLoad<NPX>(xr, xvoff[i], xs + j * HW * 2);
+            for (int j = 0; j < 8; ++j) {
+                if (NPX == 1 && p.pair_load) {
+                    // strided gather: read the aligned dword that holds the wanted pixel in its low half.  Neighbouring
+                    // lanes then read neighbouring dwords (coalesced), where 2-byte loads 4 bytes apart are handled lane by lane.
+                    xreg[i][j].d[0] = __builtin_amdgcn_raw_buffer_load_b32(xr, xvoff[i], xs + j * HW * 2, 0);
+                } else {
+                    xreg[i][j] = BufLoad<NPX>(xr, xvoff[i], xs + j * HW * 2);
+                }
+            }
         }
         const int ws = (TAPS == 1 && p.w_direct) ? ci * CK * 2 : ci * (CG * TAPS) * p.K * 16;
 #pragma unroll
