@@ -276,16 +276,16 @@ NchwPlan PlanNchw(const hipcx_array* x, const hipcx_array* w, const hipcx_array*
         pl.npx = stride[0] == 1 ? pick(P) : 1;
         if (K <= 64) {
             pl.wpx = 4, pl.wch = 1;
-            pl.maxi = pl.npx == 2 ? 2 : 4;
         } else if (K >= 256 && pl.npx == 1) {
             // single-pixel gathers (strided or odd-sized planes) are the expensive part of a tile: 128 pixels x 256 channels with
             // 8 waves gathers and transposes each activation tile once for 256 output channels instead of 128
             pl.wpx = 2, pl.wch = 4;
-            pl.maxi = 1;
+            // too few such tiles to occupy the chip (deep layers at small batch x plane): halve the pixel extent
+            if (((N * P + 127) / 128) * ((K + 255) / 256) < 128) pl.wpx = 1;
         } else {
             pl.wpx = 2, pl.wch = 2;
-            pl.maxi = pl.npx == 2 ? 1 : 2;
         }
+        pl.maxi = std::max(1, pl.ck / 8 / (pl.npx * pl.wch));  // 64*wpx/npx pixel runs x ck/8 channel groups over 64*wpx*wch threads
         pl.nslot = 64 * pl.wpx;
     } else {
         if (C % 16 != 0) return pl;
@@ -390,19 +390,23 @@ void RunNchw(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, c
     double flops = 2.0 * a.M * a.K * RS * a.C;
     double bytes = 2.0 * (static_cast<double>(a.N) * a.C * a.H * a.W + static_cast<double>(a.K) * RS * a.C + static_cast<double>(a.M) * a.K);
     ProfileScope prof(stream, flops, bytes);
-    const int key = pl.taps * 1000 + pl.wpx * 100 + pl.npx * 10 + pl.maxi;
+    const int key = (pl.ck / 16) * 100000 + pl.taps * 10000 + pl.wpx * 1000 + pl.wch * 100 + pl.npx * 10 + pl.maxi;
+#define HIPCX_NCHW_CASE(TAPS, WPX, WCH, CK, NPX, MAXI) \
+    case (CK / 16) * 100000 + TAPS * 10000 + WPX * 1000 + WCH * 100 + NPX * 10 + MAXI: LaunchNchwKernel<TAPS, WPX, WCH, CK, NPX, MAXI>(a, pl.lds_bytes, stream); break;
     switch (key) {
-        case 1000 + 400 + 20 + 2: LaunchNchwKernel<1, 4, 1, 32, 2, 2>(a, pl.lds_bytes, stream); break;
-        case 1000 + 400 + 10 + 4: LaunchNchwKernel<1, 4, 1, 32, 1, 4>(a, pl.lds_bytes, stream); break;
-        case 1000 + 200 + 20 + 1: LaunchNchwKernel<1, 2, 2, 32, 2, 1>(a, pl.lds_bytes, stream); break;
-        case 1000 + 200 + 10 + 1: LaunchNchwKernel<1, 2, 4, 32, 1, 1>(a, pl.lds_bytes, stream); break;
-        case 1000 + 200 + 10 + 2: LaunchNchwKernel<1, 2, 2, 32, 1, 2>(a, pl.lds_bytes, stream); break;
-        case 9000 + 400 + 20 + 2: LaunchNchwKernel<9, 4, 1, 16, 2, 2>(a, pl.lds_bytes, stream); break;
-        case 9000 + 400 + 20 + 4: LaunchNchwKernel<9, 4, 1, 16, 2, 4>(a, pl.lds_bytes, stream); break;
-        case 9000 + 400 + 10 + 2: LaunchNchwKernel<9, 4, 1, 16, 1, 2>(a, pl.lds_bytes, stream); break;
-        case 9000 + 400 + 10 + 4: LaunchNchwKernel<9, 4, 1, 16, 1, 4>(a, pl.lds_bytes, stream); break;
+        HIPCX_NCHW_CASE(1, 4, 1, 32, 2, 2)
+        HIPCX_NCHW_CASE(1, 4, 1, 32, 1, 4)
+        HIPCX_NCHW_CASE(1, 2, 2, 32, 2, 1)
+        HIPCX_NCHW_CASE(1, 2, 2, 32, 1, 2)
+        HIPCX_NCHW_CASE(1, 2, 4, 32, 1, 1)
+        HIPCX_NCHW_CASE(1, 1, 4, 32, 1, 1)
+        HIPCX_NCHW_CASE(9, 4, 1, 16, 2, 2)
+        HIPCX_NCHW_CASE(9, 4, 1, 16, 2, 4)
+        HIPCX_NCHW_CASE(9, 4, 1, 16, 1, 2)
+        HIPCX_NCHW_CASE(9, 4, 1, 16, 1, 4)
         default: throw Error(HIPCX_CHAINERX_ERROR, "nchw conv: no kernel for plan " + std::to_string(key));
     }
+#undef HIPCX_NCHW_CASE
 }
 
 

@@ -25,6 +25,12 @@ CONV_CASES = [
     (2, 20, 6, 7, 9, 2, 3, (1, 2), (0, 1), True),
     (2, 3, 64, 64, 64, 7, 7, 2, 3, False),   # ImageNet stem geometry (dedicated float16 kernel)
     (1, 3, 30, 48, 64, 7, 7, 2, 3, False),   # same with an odd number of output rows
+    # 1x1 tile shapes of the float16 NCHW kernel: 128x128 tiles with pixel pairs / single pixels, 128x256 and 64x256 tiles
+    (2, 64, 8, 8, 128, 1, 1, 1, 0, False),
+    (3, 32, 7, 7, 128, 1, 1, 1, 0, False),
+    (2, 32, 8, 8, 256, 1, 1, 1, 0, False),
+    (16, 32, 46, 46, 512, 1, 1, 2, 0, False),
+    (2, 64, 7, 7, 320, 1, 1, 1, 0, False),
 ]
 
 
