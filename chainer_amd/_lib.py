@@ -137,6 +137,9 @@ SIGNATURES = {
     'hipcx_conv_workspace_size': (_SZ, [_A, _A, _A]),
     'hipcx_conv': (_INT, [_A, _A, _A, _I64P, _I64P, _INT, _A, _V, _SZ, _V]),
     'hipcx_conv_bn_act': (_INT, [_A, _A, _A, _I64P, _I64P, _INT, _A, _A, _A, _A, _S, _A, _INT, _A, _V, _SZ, _V]),
+    'hipcx_log_softmax_workspace_size': (_SZ, [_A]),
+    'hipcx_log_softmax': (_INT, [_A, _A, _V, _SZ, _V]),
+    'hipcx_lstm_cell': (_INT, [_A, _A, _A, _A, _V]),
     'hipcx_profile_start': (_INT, []),
     'hipcx_profile_stop': (_INT, [_I64P, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double),
                                   ctypes.POINTER(ctypes.c_double)]),

@@ -102,12 +102,16 @@ def section_sweep(chx, oracle, with_cpu):
             ('argmax axis1', lambda: chx.argmax(X, 1), n * s + rows * 8, 1, (lambda: oracle.argmax(small, 1)) if with_cpu else None),
             ('log_softmax axis1', lambda: chx.log_softmax(X, 1), (2 if shape[1] * s <= 65536 else 3) * n * s, 7,
              (lambda: oracle.log_softmax(small, 1)) if with_cpu else None),
+            ('log_softmax axis1, fused opt-in entry', lambda: chx.log_softmax_fused(X, 1), (2 if shape[1] * s <= 65536 else 3) * n * s,
+             1 if shape[1] * s <= 65536 else 2, None),
         ]
         for name, fn, nbytes, launches, cfn in ops:
             t = device_time(fn)
             cpu = cpu_time(cfn) * scale if cfn is not None else None
             note = None
-            if launches > 1:
+            if 'fused' in name:
+                note = 'hipcx_log_softmax: one read + one write for rows up to 64 KiB, two reads + one write beyond; not the drop-in kernel boundary'
+            elif launches > 1:
                 note = ('7 kernel launches as the ChainerX routine decomposes it (moves 8*N*4 bytes: ceiling %.0f%% of the '
                         'fused-ideal figure used here)' % (100.0 * nbytes / (8 * n * s)))
             bw_row('sweep', name, shape, t, nbytes, launches, cpu, note)
@@ -214,6 +218,10 @@ def section_lstm(chx, oracle, with_cpu):
                     'bounds mode reads an error flag back every step (the native backend raises IndexError) and cannot be captured; '
                     'results are identical for in-range ids')
     emit(**row)
+    fused = graph_time(lambda: cfg.lstm_lm_forward(chx, pd, I, chx.zeros, 'wrap', True), 5)
+    emit(section='lstm', op='35-step forward, fused opt-in Lstm cell and LogSoftmax', batch=128, graph_replay_ms=round(fused * 1e3, 2),
+         TFLOPs_graph=round(flops / fused / 1e12, 2), tokens_per_s_graph=round(128 * 35 / fused, 0), kernel_launches=35 * 14 + 1,
+         note='hipcx_lstm_cell and hipcx_log_softmax replace the ~25-kernel cell and the 7-kernel LogSoftmax chains; not the drop-in kernel boundary')
     W = pd['embed']
     t = device_time(lambda: chx.take(W, I, 0, 'wrap'))
     bw_row('lstm', 'take [10000,650] rows by [128,35] ids', (128, 35, 650), t, 2 * 128 * 35 * 650 * 4 + ids.nbytes)

@@ -247,9 +247,12 @@ def lstm_lm_input(seed=5, batch=128, seq=35, vocab=10000):
     return _rng(seed + 1000).integers(0, vocab, (batch, seq)).astype(np.int32)
 
 
-def lstm_lm_forward(F, p, ids, zeros, take_mode=None):
+def lstm_lm_forward(F, p, ids, zeros, take_mode=None, fused=False):
     """Runs the sequence; returns log-probabilities of the last step and the final (h, c) of both layers.
-    ``zeros(shape, dtype)`` makes the initial state on the same backend as ``F``."""
+    ``zeros(shape, dtype)`` makes the initial state on the same backend as ``F``.  ``fused`` takes the opt-in one-kernel
+    Lstm cell and LogSoftmax (``F.lstm_fused``, ``F.log_softmax_fused``) instead of the routine chains."""
+    lstm = F.lstm_fused if fused else F.lstm
+    log_softmax = F.log_softmax_fused if fused else F.log_softmax
     batch, seq = ids.shape
     units = p['embed'].shape[1]
     dtype = p['embed'].dtype
@@ -260,7 +263,7 @@ def lstm_lm_forward(F, p, ids, zeros, take_mode=None):
         x = F.take(p['embed'], ids[:, t], 0, take_mode)
         for li, layer in enumerate(p['layers']):
             gates = F.add(F.linear(x, layer['up_w'], layer['up_b']), F.linear(hs[li], layer['lat_w']))
-            hs[li], cs[li] = F.lstm(cs[li], gates)
+            hs[li], cs[li] = lstm(cs[li], gates)
             x = hs[li]
         y = F.linear(x, p['out_w'], p['out_b'])
-    return F.log_softmax(y, 1), hs, cs
+    return log_softmax(y, 1), hs, cs

@@ -522,6 +522,22 @@ def log_softmax(x, axis=None):
     return subtract(xc, logsumexp(xc, 1 if axis is None else axis, True))
 
 
+def log_softmax_fused(x, axis=None):
+    """Opt-in: LogSoftmax (CX/routines/reduction.cc:88-92) through hipcx_log_softmax -- one or two kernels instead of seven.
+    Arrays the fused kernel does not take (ndim != 2, another axis, strided rows) go through log_softmax."""
+    xc = x.astype(_math_result_dtype(x.dtype), False)
+    ax = 1 if axis is None else axis
+    axes = _sorted_axes(ax, x.ndim)
+    it = xc.dtype.itemsize
+    if xc.ndim != 2 or axes != (1,) or (xc.shape[1] > 1 and xc.strides[1] != it) or xc.strides[0] < 0:
+        return log_softmax(x, axis)
+    out = ndarray.empty(xc.shape, xc.dtype)
+    nbytes = _lib.load().hipcx_log_softmax_workspace_size(xc.desc())
+    ws, wsp = _workspace(nbytes)
+    _lib.call('hipcx_log_softmax', xc.desc(), out.desc(), wsp, nbytes, current_stream())
+    return out
+
+
 def softmax(x, axis=None):
     """Softmax (CX/routines/reduction.cc:68-76)."""
     xc = x.astype(_math_result_dtype(x.dtype), False)
@@ -785,6 +801,16 @@ def lstm(c, x):
     o = sigmoid(gates[3])
     new_c = add(multiply(a, i), multiply(f, c))
     h = multiply(o, tanh(new_c))
+    return h, new_c
+
+
+def lstm_fused(c, x):
+    """Opt-in: the Lstm cell through hipcx_lstm_cell -- one kernel instead of ~25; same checks and errors as lstm."""
+    if c.ndim != 2 or x.ndim != 2:
+        return lstm(c, x)
+    h = ndarray.empty(c.shape, c.dtype)
+    new_c = ndarray.empty(c.shape, c.dtype)
+    _lib.call('hipcx_lstm_cell', c.desc(), x.desc(), h.desc(), new_c.desc(), current_stream())
     return h, new_c
 
 

@@ -170,6 +170,22 @@ int hipcx_conv_bn_act(const hipcx_array* x, const hipcx_array* w, const hipcx_ar
                       hipcx_scalar eps, const hipcx_array* residual, int relu, const hipcx_array* out, void* workspace,
                       size_t workspace_bytes, void* stream);
 
+/* Opt-in fused entries for two routine chains.  No single kernel of the reference corresponds to either.
+ *
+ * hipcx_log_softmax: LogSoftmax along axis 1 of a 2-D array (CX/routines/reduction.cc:78-92: AMaxKernel, SubtractKernel,
+ *   ExpKernel, SumKernel, LogKernel, AddKernel, SubtractKernel -- 5 reads and 3 writes of the array) as one read and one
+ *   write when a row is at most 64 KiB, two reads and one write otherwise (then `workspace` must hold
+ *   hipcx_log_softmax_workspace_size(x) bytes).  Same float operations as the chain (max with AMax's NaN rule, exp(x - max),
+ *   sum, max + log(sum), x - that); only the order of the row sum differs.  x and out: same shape and float dtype, unit
+ *   stride along axis 1, any non-negative row stride.
+ * hipcx_lstm_cell: the Lstm routine (CX/routines/connection.cc:396-446) for equal batch sizes: gate k of unit j is column
+ *   4j+k of x[B,4H]; a = tanh(g0), i, f, o = 1/(1+exp(-g)) (CX/routines/activation.cc:74-78); c_out = a*i + f*c;
+ *   h_out = o*tanh(c_out).  Same operations in the same order as the ~25 separate kernels: bit-identical for float32/float64
+ *   (float16 rounds once instead of after every kernel).  Errors as the routine raises them (DimensionError, DtypeError). */
+size_t hipcx_log_softmax_workspace_size(const hipcx_array* x);
+int hipcx_log_softmax(const hipcx_array* x, const hipcx_array* out, void* workspace, size_t workspace_bytes, void* stream);
+int hipcx_lstm_cell(const hipcx_array* c, const hipcx_array* x, const hipcx_array* h_out, const hipcx_array* c_out, void* stream);
+
 /* Measurement aid (no counterpart in the reference): between start and stop every implicit-GEMM launch made by
  * hipcx_dot / hipcx_conv from the calling process is bracketed by a pair of HIP events on its stream.  stop waits for them
  * and returns the number of launches, the sum of their durations, and their algorithmic flops (2 per multiply-add) and
