@@ -137,6 +137,22 @@ SIGNATURES = {
     'hipcx_conv_workspace_size': (_SZ, [_A, _A, _A]),
     'hipcx_conv': (_INT, [_A, _A, _A, _I64P, _I64P, _INT, _A, _V, _SZ, _V]),
     'hipcx_conv_bn_act': (_INT, [_A, _A, _A, _I64P, _I64P, _INT, _A, _A, _A, _A, _S, _A, _INT, _A, _V, _SZ, _V]),
+    'hipcx_amin': (_INT, [_A, _I8P, _INT, _A, _V, _SZ, _V]),
+    'hipcx_argmin': (_INT, [_A, _I8P, _INT, _A, _V, _SZ, _V]),
+    'hipcx_all': (_INT, [_A, _I8P, _INT, _A, _V, _SZ, _V]),
+    'hipcx_any': (_INT, [_A, _I8P, _INT, _A, _V, _SZ, _V]),
+    'hipcx_unary': (_INT, [_INT, _A, _A, _V]),
+    'hipcx_predicate': (_INT, [_INT, _A, _A, _V]),
+    'hipcx_logical': (_INT, [_INT, _A, _A, _A, _V]),
+    'hipcx_power': (_INT, [_A, _A, _A, _V]),
+    'hipcx_power_as': (_INT, [_A, _S, _A, _V]),
+    'hipcx_power_sa': (_INT, [_S, _A, _A, _V]),
+    'hipcx_fmod': (_INT, [_A, _A, _A, _V]),
+    'hipcx_arctan2': (_INT, [_A, _A, _A, _V]),
+    'hipcx_where': (_INT, [_A, _A, _A, _A, _V]),
+    'hipcx_where_aas': (_INT, [_A, _A, _S, _A, _V]),
+    'hipcx_where_asa': (_INT, [_A, _S, _A, _A, _V]),
+    'hipcx_where_ass': (_INT, [_A, _S, _S, _A, _V]),
     'hipcx_log_softmax_workspace_size': (_SZ, [_A]),
     'hipcx_log_softmax': (_INT, [_A, _A, _V, _SZ, _V]),
     'hipcx_lstm_cell': (_INT, [_A, _A, _A, _A, _V]),

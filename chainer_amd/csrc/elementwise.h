@@ -113,14 +113,25 @@ __device__ __forceinline__ compute_t<T> LoadAs(const char* p) {
     return static_cast<compute_t<T>>(*reinterpret_cast<const T*>(p));
 }
 
+// Type of the first input: Op::In0 when the op declares one (a bool condition in front of numeric operands), else Op::In.
+template <typename Op, typename = void>
+struct FirstInOf {
+    using type = typename Op::In;
+};
+template <typename Op>
+struct FirstInOf<Op, std::void_t<typename Op::In0>> {
+    using type = typename Op::In0;
+};
+
 // Op interface:
-//   using In = ...; using Out = ...; static constexpr int kNumIn = n;
+//   using In = ...; using Out = ...; static constexpr int kNumIn = n;  (optionally using In0 = ... for the first input)
 //   __device__ compute_t<Out> operator()(compute_t<In> a, compute_t<In> b, compute_t<In> c, compute_t<In> d, int64_t index) const
 // `index` is the C-order position in the *normalised* iteration space; only ops that ask for it
 // (kNeedsIndex) get a meaningful value, and those are launched on contiguous outputs.
 template <typename Op, int VEC, typename IdxT>
 __global__ __launch_bounds__(kEwThreads) void EwKernel(EwArgs<Op::kNumIn + 1> args, Op op) {
     using In = typename Op::In;
+    using In0 = typename FirstInOf<Op>::type;
     using Out = typename Op::Out;
     using CIn = compute_t<In>;
     constexpr int NIN = Op::kNumIn;
@@ -159,13 +170,22 @@ __global__ __launch_bounds__(kEwThreads) void EwKernel(EwArgs<Op::kNumIn + 1> ar
 
     // loads first (all unrolled iterations in flight), then compute + store
     Vec<In, VEC> in[kEwUnroll][NIN > 0 ? NIN : 1];
+    Vec<In0, VEC> in0[kEwUnroll];
 #pragma unroll
     for (int u = 0; u < kEwUnroll; ++u) {
         if (!live[u]) continue;
 #pragma unroll
         for (int i = 0; i < NIN; ++i) {
             const char* p = args.ptr[i + 1] + off[u][i + 1];
-            if (VEC > 1) {
+            if (i == 0) {
+                if (VEC > 1 && args.col_stride[1] != 0) {
+                    in0[u] = *reinterpret_cast<const Vec<In0, VEC>*>(p);
+                } else {
+                    In0 s = *reinterpret_cast<const In0*>(p);
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) in0[u].v[e] = s;
+                }
+            } else if (VEC > 1) {
                 if (args.col_stride[i + 1] != 0) {
                     in[u][i] = *reinterpret_cast<const Vec<In, VEC>*>(p);
                 } else {
@@ -189,7 +209,7 @@ __global__ __launch_bounds__(kEwThreads) void EwKernel(EwArgs<Op::kNumIn + 1> ar
         }
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
-            CIn a = NIN > 0 ? static_cast<CIn>(in[u][0].v[e]) : CIn{};
+            CIn a = NIN > 0 ? static_cast<CIn>(in0[u].v[e]) : CIn{};
             CIn b = NIN > 1 ? static_cast<CIn>(in[u][NIN > 1 ? 1 : 0].v[e]) : CIn{};
             CIn c = NIN > 2 ? static_cast<CIn>(in[u][NIN > 2 ? 2 : 0].v[e]) : CIn{};
             CIn d = NIN > 3 ? static_cast<CIn>(in[u][NIN > 3 ? 3 : 0].v[e]) : CIn{};

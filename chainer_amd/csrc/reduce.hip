@@ -81,6 +81,21 @@ __device__ __forceinline__ T LowestOrInf() {
 }
 
 template <typename T>
+__device__ __forceinline__ T MaxOrInf() {
+    if constexpr (std::is_same<T, half_t>::value) {
+        return static_cast<half_t>(__builtin_huge_valf());
+    } else if constexpr (std::is_same<T, float>::value) {
+        return __builtin_huge_valf();
+    } else if constexpr (std::is_same<T, double>::value) {
+        return __builtin_huge_val();
+    } else if constexpr (std::is_same<T, bool>::value) {
+        return true;
+    } else {
+        return std::numeric_limits<T>::max();
+    }
+}
+
+template <typename T>
 __device__ __forceinline__ bool IsNanV(T v) {
     if constexpr (std::is_same<T, half_t>::value || std::is_floating_point<T>::value) {
         return v != v;
@@ -89,7 +104,8 @@ __device__ __forceinline__ bool IsNanV(T v) {
     }
 }
 
-template <typename T>
+// MIN: AMin (identity MaxOrInf, `accum > next`), the mirror image of AMax (native/native_device/statistics.cc:27-73).
+template <typename T, bool MIN = false>
 struct AMaxImpl {
     using In = T;
     using Out = T;
@@ -97,11 +113,11 @@ struct AMaxImpl {
     using Acc = std::conditional_t<std::is_same<T, half_t>::value, float, std::conditional_t<std::is_same<T, bool>::value, int, T>>;
     static constexpr bool kSerialFold = false;
     static constexpr bool kHasIndex = false;
-    __device__ static Acc Identity() { return static_cast<Acc>(LowestOrInf<T>()); }
+    __device__ static Acc Identity() { return static_cast<Acc>(MIN ? MaxOrInf<T>() : LowestOrInf<T>()); }
     __device__ static Acc Empty() { return Identity(); }
     __device__ static Acc Map(In v, int64_t) { return static_cast<Acc>(v); }
     __device__ static void Reduce(Acc next, Acc& acc) {
-        if (IsNanV(next) || acc < next) acc = next;
+        if (IsNanV(next) || (MIN ? acc > next : acc < next)) acc = next;
     }
     __device__ static void MaskLaterNan(Acc&, bool) {}
     __device__ static Out MapOut(Acc a) { return static_cast<Out>(a); }
@@ -114,7 +130,8 @@ struct MaxIdx {
     int64_t i;  // < 0: empty / identity
 };
 
-template <typename T>
+// MIN: ArgMin (`accum.min > next.min`), the mirror image of ArgMax (native/native_device/reduction.cc:34-92).
+template <typename T, bool MIN = false>
 struct ArgMaxImpl {
     using In = T;
     using Out = int64_t;
@@ -127,7 +144,7 @@ struct ArgMaxImpl {
     __device__ static Acc Map(In v, int64_t index) { return Acc{static_cast<V>(v), index}; }
     __device__ static void Reduce(Acc next, Acc& acc) {
         if (next.i < 0) return;
-        if (acc.i < 0 || acc.v < next.v) acc = next;
+        if (acc.i < 0 || (MIN ? acc.v > next.v : acc.v < next.v)) acc = next;
     }
     // Inside a chunk a NaN operand other than the very first never replaces the accumulator; turning
     // it into padding makes the in-chunk fold associative, so it can run as a shuffle tree.
@@ -141,6 +158,23 @@ struct ArgMaxImpl {
         r.i = __shfl(a.i, src);
         return r;
     }
+};
+
+// All / Any over bool inputs (native/native_device/logic.cc: the routine casts the input to bool first).
+template <bool ALL>
+struct AllAnyImpl {
+    using In = bool;
+    using Out = bool;
+    using Acc = int;
+    static constexpr bool kSerialFold = false;
+    static constexpr bool kHasIndex = false;
+    __device__ static Acc Identity() { return ALL ? 1 : 0; }
+    __device__ static Acc Empty() { return Identity(); }
+    __device__ static Acc Map(In v, int64_t) { return v ? 1 : 0; }
+    __device__ static void Reduce(Acc next, Acc& acc) { acc = ALL ? (acc & next) : (acc | next); }
+    __device__ static void MaskLaterNan(Acc&, bool) {}
+    __device__ static Out MapOut(Acc a) { return a != 0; }
+    __device__ static Acc Shfl(Acc a, int src) { return __shfl(a, src); }
 };
 
 // ---------------------------------------------------------------------------------------------
@@ -586,6 +620,60 @@ int hipcx_argmax(const hipcx_array* a, const int8_t* axis, int naxis, const hipc
             using T = typename decltype(tag)::type;
             Run<ArgMaxImpl<T>>(a, axis, naxis, out, workspace, workspace_bytes, AsStream(stream));
         });
+    });
+}
+
+int hipcx_amin(const hipcx_array* a, const int8_t* axis, int naxis, const hipcx_array* out, void* workspace, size_t workspace_bytes,
+               void* stream) {
+    return Guard([&] {
+        ValidateArray(a, "a");
+        ValidateArray(out, "out");
+        HIPCX_REQUIRE(a->dtype == out->dtype, HIPCX_DTYPE_ERROR, "amin: out must have a's dtype");
+        for (int i = 0; i < naxis; ++i) {
+            HIPCX_REQUIRE(axis[i] >= 0 && axis[i] < a->ndim && a->shape[axis[i]] > 0, HIPCX_DIMENSION_ERROR,
+                          "cannot compute the minimum along zero-sized axis");
+        }
+        VisitDtype(a->dtype, [&](auto tag) {
+            using T = typename decltype(tag)::type;
+            Run<AMaxImpl<T, true>>(a, axis, naxis, out, workspace, workspace_bytes, AsStream(stream));
+        });
+    });
+}
+
+int hipcx_argmin(const hipcx_array* a, const int8_t* axis, int naxis, const hipcx_array* out, void* workspace, size_t workspace_bytes,
+                 void* stream) {
+    return Guard([&] {
+        ValidateArray(a, "a");
+        ValidateArray(out, "out");
+        HIPCX_REQUIRE(out->dtype == HIPCX_INT64, HIPCX_DTYPE_ERROR, "argmin: out must be int64");
+        for (int i = 0; i < naxis; ++i) {
+            HIPCX_REQUIRE(axis[i] >= 0 && axis[i] < a->ndim && a->shape[axis[i]] > 0, HIPCX_DIMENSION_ERROR,
+                          "cannot compute ArgMin for an empty array");
+        }
+        VisitDtype(a->dtype, [&](auto tag) {
+            using T = typename decltype(tag)::type;
+            Run<ArgMaxImpl<T, true>>(a, axis, naxis, out, workspace, workspace_bytes, AsStream(stream));
+        });
+    });
+}
+
+int hipcx_all(const hipcx_array* a, const int8_t* axis, int naxis, const hipcx_array* out, void* workspace, size_t workspace_bytes,
+              void* stream) {
+    return Guard([&] {
+        ValidateArray(a, "a");
+        ValidateArray(out, "out");
+        HIPCX_REQUIRE(a->dtype == HIPCX_BOOL && out->dtype == HIPCX_BOOL, HIPCX_DTYPE_ERROR, "all: a and out must be bool (cast with hipcx_copy first)");
+        Run<AllAnyImpl<true>>(a, axis, naxis, out, workspace, workspace_bytes, AsStream(stream));
+    });
+}
+
+int hipcx_any(const hipcx_array* a, const int8_t* axis, int naxis, const hipcx_array* out, void* workspace, size_t workspace_bytes,
+              void* stream) {
+    return Guard([&] {
+        ValidateArray(a, "a");
+        ValidateArray(out, "out");
+        HIPCX_REQUIRE(a->dtype == HIPCX_BOOL && out->dtype == HIPCX_BOOL, HIPCX_DTYPE_ERROR, "any: a and out must be bool (cast with hipcx_copy first)");
+        Run<AllAnyImpl<false>>(a, axis, naxis, out, workspace, workspace_bytes, AsStream(stream));
     });
 }
 }

@@ -32,11 +32,13 @@ template <>
 struct SmallDotTraits<float> {
     static constexpr int KG = 8;  // k values one "group step" of a wave consumes (4 MFMAs x 2)
     static constexpr int PER_LANE = 4;
+    static constexpr int STEPS_IN_FLIGHT = 6;
 };
 template <>
 struct SmallDotTraits<half_t> {
     static constexpr int KG = 16;  // one MFMA
     static constexpr int PER_LANE = 8;
+    static constexpr int STEPS_IN_FLIGHT = 4;
 };
 
 // PER_LANE consecutive-k elements of one operand row/column as raw dwords; `contig`: k is the unit-stride axis.
@@ -65,6 +67,29 @@ __device__ __forceinline__ Bytes16 LoadRun(__amdgpu_buffer_rsrc_t r, const T* ba
         v.y = pk(e[2], e[3]);
         v.z = pk(e[4], e[5]);
         v.w = pk(e[6], e[7]);
+    }
+    return v;
+}
+
+// The same run when k is the unit-stride axis, without a branch: lines beyond the operand come back as zeros from the
+// buffer bounds check, elements beyond kend (they belong to the next line) are masked.  Loads written this way can all be
+// issued before the first one is waited for.
+template <typename T>
+__device__ __forceinline__ Bytes16 LoadRunContig(__amdgpu_buffer_rsrc_t r, int64_t line_off, int k, int kend, bool line_ok) {
+    constexpr int PL = SmallDotTraits<T>::PER_LANE;
+    const int off = line_ok && k < kend ? static_cast<int>((line_off + k) * static_cast<int64_t>(sizeof(T))) : 0x7fffffff;
+    Bytes16 v = __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0);
+    const int c = kend - k;  // valid elements of the run (>= PL for all but the last run of a line)
+    if constexpr (sizeof(T) == 4) {
+        v.y = c > 1 ? v.y : 0u;
+        v.z = c > 2 ? v.z : 0u;
+        v.w = c > 3 ? v.w : 0u;
+    } else {
+        auto m = [c](int d) { return c > 2 * d + 1 ? 0xffffffffu : (c > 2 * d ? 0x0000ffffu : 0u); };
+        v.x &= m(0);
+        v.y &= m(1);
+        v.z &= m(2);
+        v.w &= m(3);
     }
     return v;
 }
@@ -103,17 +128,32 @@ __global__ __launch_bounds__(512) void SmallDotKernel(SmallDotArgs p) {
     float16_t acc;
 #pragma unroll
     for (int v = 0; v < 16; ++v) acc[v] = 0.f;
-    // two group steps in flight
-    for (int k = k_begin; k < k_end; k += 2 * KG) {
-        Bytes16 av[2], bv[2];
+    // U group steps in flight: a wave's share of K is short (K / 8), and every round trip to L2 it spends is exposed
+    constexpr int U = SmallDotTraits<T>::STEPS_IN_FLIGHT;
+    if (a_contig && b_contig) {  // Linear's x and W^T: every operand load is one branch-free 16-byte buffer load
+        for (int k = k_begin; k < k_end; k += U * KG) {
+            Bytes16 av[U], bv[U];
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
-            int kk = k + u * KG + g * PL;
-            av[u] = LoadRun<T>(ar, a, a_off, p.a_k, kk, k_end, m_ok, a_contig);
-            bv[u] = LoadRun<T>(br, b, b_off, p.b_k, kk, k_end, n_ok, b_contig);
+            for (int u = 0; u < U; ++u) {
+                int kk = k + u * KG + g * PL;
+                av[u] = LoadRunContig<T>(ar, a_off, kk, k_end, m_ok);
+                bv[u] = LoadRunContig<T>(br, b_off, kk, k_end, n_ok);
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) MfmaTile<T>(av[u], bv[u], acc);
         }
+    } else {
+        for (int k = k_begin; k < k_end; k += 2 * KG) {
+            Bytes16 av[2], bv[2];
 #pragma unroll
-        for (int u = 0; u < 2; ++u) MfmaTile<T>(av[u], bv[u], acc);
+            for (int u = 0; u < 2; ++u) {
+                int kk = k + u * KG + g * PL;
+                av[u] = LoadRun<T>(ar, a, a_off, p.a_k, kk, k_end, m_ok, a_contig);
+                bv[u] = LoadRun<T>(br, b, b_off, p.b_k, kk, k_end, n_ok, b_contig);
+            }
+#pragma unroll
+            for (int u = 0; u < 2; ++u) MfmaTile<T>(av[u], bv[u], acc);
+        }
     }
     // lane holds column lr, rows 8*(v/4) + 4*g + v%4
 #pragma unroll

@@ -427,6 +427,237 @@ def greater_equal(x1, x2):
     return _compare('hipcx_greater_equal', x1, x2)
 
 
+def less(x1, x2):
+    """Less(x1, x2) = Greater(x2, x1) (CX/routines/logic.h:33)."""
+    return greater(x2, x1)
+
+
+def less_equal(x1, x2):
+    """LessEqual(x1, x2) = GreaterEqual(x2, x1) (CX/routines/logic.h:38)."""
+    return greater_equal(x2, x1)
+
+
+# Op codes of include/hipcx.h (enum hipcx_unary_op / hipcx_predicate_op / hipcx_logical_op).
+_UNARY_CODES = {name: i + 1 for i, name in enumerate(
+    ['erf', 'expm1', 'exp2', 'log10', 'log2', 'log1p', 'sinh', 'cosh', 'arcsinh', 'arccosh', 'sin', 'cos', 'tan', 'arcsin',
+     'arccos', 'arctan', 'ceil', 'floor', 'square', 'absolute', 'sign'])}
+_PRED_CODES = {'logical_not': 1, 'isnan': 2, 'isinf': 3, 'isfinite': 4}
+_LOGICAL_CODES = {'logical_and': 1, 'logical_or': 2, 'logical_xor': 3}
+
+
+def _float_unary(name, x):
+    """Unary math routines: the result dtype is x's float dtype, float32 for other kinds (GetMathResultDtype)."""
+    dt = _math_result_dtype(x.dtype)
+    out = ndarray.empty(x.shape, dt)
+    _lib.call('hipcx_unary', _UNARY_CODES[name], x.astype(dt, False).desc(), out.desc(), current_stream())
+    return out
+
+
+def erf(x):
+    return _float_unary('erf', x)
+
+
+def expm1(x):
+    return _float_unary('expm1', x)
+
+
+def exp2(x):
+    return _float_unary('exp2', x)
+
+
+def log10(x):
+    return _float_unary('log10', x)
+
+
+def log2(x):
+    return _float_unary('log2', x)
+
+
+def log1p(x):
+    return _float_unary('log1p', x)
+
+
+def sinh(x):
+    return _float_unary('sinh', x)
+
+
+def cosh(x):
+    return _float_unary('cosh', x)
+
+
+def arcsinh(x):
+    return _float_unary('arcsinh', x)
+
+
+def arccosh(x):
+    return _float_unary('arccosh', x)
+
+
+def sin(x):
+    return _float_unary('sin', x)
+
+
+def cos(x):
+    return _float_unary('cos', x)
+
+
+def tan(x):
+    return _float_unary('tan', x)
+
+
+def arcsin(x):
+    return _float_unary('arcsin', x)
+
+
+def arccos(x):
+    return _float_unary('arccos', x)
+
+
+def arctan(x):
+    return _float_unary('arctan', x)
+
+
+def ceil(x):
+    return _float_unary('ceil', x)
+
+
+def floor(x):
+    return _float_unary('floor', x)
+
+
+def _numeric_unary(name, x, message):
+    if x.dtype == numpy.dtype('bool'):
+        raise _lib.DtypeError(message)
+    out = ndarray.empty(x.shape, x.dtype)
+    _lib.call('hipcx_unary', _UNARY_CODES[name], x.desc(), out.desc(), current_stream())
+    return out
+
+
+def square(x):
+    """Square (CX/routines/misc.cc:141-150)."""
+    return _numeric_unary('square', x, "Square operation don't support Boolean type")
+
+
+def absolute(x):
+    """Absolute (CX/routines/misc.cc:185-192)."""
+    return _numeric_unary('absolute', x, 'Absolute does not support boolean array')
+
+
+def fabs(x):
+    """Fabs (CX/routines/misc.cc:194-199): Absolute into the math result dtype."""
+    return absolute(x.astype(_math_result_dtype(x.dtype), False))
+
+
+def sign(x):
+    """Sign (CX/routines/misc.cc:201-208); the kernel visits numeric dtypes only."""
+    return _numeric_unary('sign', x, 'bool dtype is not supported by this kernel')
+
+
+def _predicate(name, x):
+    out = ndarray.empty(x.shape, 'bool')
+    _lib.call('hipcx_predicate', _PRED_CODES[name], x.desc(), out.desc(), current_stream())
+    return out
+
+
+def logical_not(x):
+    return _predicate('logical_not', x)
+
+
+def isnan(x):
+    return _predicate('isnan', x)
+
+
+def isinf(x):
+    return _predicate('isinf', x)
+
+
+def isfinite(x):
+    return _predicate('isfinite', x)
+
+
+def _logical(name, x1, x2):
+    """LogicBinary (CX/routines/logic.cc:36-41): bool with non-bool is a DtypeError; the kernel promotes the operands."""
+    if (_kind(x1.dtype) == 0) != (_kind(x2.dtype) == 0):
+        raise _lib.DtypeError('Comparison of bool and non-bool dtypes is not supported.')
+    dt = promote_types(x1.dtype, x2.dtype)
+    shape = _broadcast_shape(x1.shape, x2.shape)
+    a = x1.broadcast_to(shape).astype(dt, False)
+    b = x2.broadcast_to(shape).astype(dt, False)
+    out = ndarray.empty(shape, 'bool')
+    _lib.call('hipcx_logical', _LOGICAL_CODES[name], a.desc(), b.desc(), out.desc(), current_stream())
+    return out
+
+
+def logical_and(x1, x2):
+    return _logical('logical_and', x1, x2)
+
+
+def logical_or(x1, x2):
+    return _logical('logical_or', x1, x2)
+
+
+def logical_xor(x1, x2):
+    return _logical('logical_xor', x1, x2)
+
+
+def _arithmetic_dtype(x1, x2):
+    """GetArithmeticResultDtype (CX/routines/arithmetic.cc:28-61): bool operands are refused."""
+    k1 = _kind(_scalar_default_dtype(x1)) if _is_scalar(x1) else _kind(x1.dtype)
+    k2 = _kind(_scalar_default_dtype(x2)) if _is_scalar(x2) else _kind(x2.dtype)
+    if k1 == 0 or k2 == 0:
+        raise _lib.DtypeError('Boolean arguments are not allowed in arithmetic functions.')
+    return result_type(x1, x2)
+
+
+def power(x1, x2):
+    """Power (CX/routines/arithmetic.cc:487-491)."""
+    dt = _arithmetic_dtype(x1, x2)
+    if _is_scalar(x2):
+        return _binary_as('hipcx_power_as', x1, x2, dt)
+    if _is_scalar(x1):
+        out = ndarray.empty(x2.shape, dt)
+        _lib.call('hipcx_power_sa', _lib.make_scalar(x1), x2.astype(dt, False).desc(), out.desc(), current_stream())
+        return out
+    return _binary('hipcx_power', x1, x2, dt)
+
+
+def fmod(x1, x2):
+    """Fmod (CX/routines/arithmetic.cc:607); the kernel visits float dtypes only."""
+    dt = _arithmetic_dtype(x1, x2)
+    if _kind(dt) != 3:
+        raise _lib.DtypeError('floating point dtype required, got %s' % dt)
+    return _binary('hipcx_fmod', x1, x2, dt)
+
+
+def arctan2(x1, x2):
+    """Arctan2 (CX/routines/trigonometric.cc:150-151): computed in the math result dtype of the operands."""
+    return _binary('hipcx_arctan2', x1, x2, _math_result_dtype(result_type(x1, x2)))
+
+
+def where(condition, x, y):
+    """Where (CX/routines/indexing.cc:207-298): out dtype = ResultType(x, y); a non-bool condition is cast to bool."""
+    cond = condition.astype('bool', False)
+    dt = result_type(x, y)
+    xs, ys = _is_scalar(x), _is_scalar(y)
+    shape = cond.shape
+    if not xs:
+        shape = _broadcast_shape(shape, x.shape)
+    if not ys:
+        shape = _broadcast_shape(shape, y.shape)
+    out = ndarray.empty(shape, dt)
+    c = cond.broadcast_to(shape)
+    if xs and ys:
+        _lib.call('hipcx_where_ass', c.desc(), _lib.make_scalar(x), _lib.make_scalar(y), out.desc(), current_stream())
+    elif ys:
+        _lib.call('hipcx_where_aas', c.desc(), x.broadcast_to(shape).astype(dt, False).desc(), _lib.make_scalar(y), out.desc(), current_stream())
+    elif xs:
+        _lib.call('hipcx_where_asa', c.desc(), _lib.make_scalar(x), y.broadcast_to(shape).astype(dt, False).desc(), out.desc(), current_stream())
+    else:
+        _lib.call('hipcx_where', c.desc(), x.broadcast_to(shape).astype(dt, False).desc(), y.broadcast_to(shape).astype(dt, False).desc(),
+                  out.desc(), current_stream())
+    return out
+
+
 # ---------------------------------------------------------------------------------------------
 # reductions
 # ---------------------------------------------------------------------------------------------
@@ -494,6 +725,43 @@ def argmax(a, axis=None):
             raise _lib.DimensionError('cannot compute ArgMax for an empty array')
     out = ndarray.empty([d for i, d in enumerate(a.shape) if i not in axes], 'int64')
     return _reduce('hipcx_argmax', a, axes, out)
+
+
+def amin(a, axis=None, keepdims=False):
+    """AMin (CX/routines/statistics.cc:66-79)."""
+    axes = _sorted_axes(axis, a.ndim)
+    for i in axes:
+        if a.shape[i] == 0:
+            raise _lib.DimensionError('cannot compute the minimum along zero-sized axis')
+    out = _reduced_out(a, axes, keepdims, a.dtype)
+    return _reduce('hipcx_amin', a, axes, out)
+
+
+min = amin
+
+
+def argmin(a, axis=None):
+    """ArgMin (CX/routines/sorting.cc:54-85): int64 result, no keepdims."""
+    axes = _sorted_axes(axis, a.ndim)
+    for i in axes:
+        if a.shape[i] == 0:
+            raise _lib.DimensionError('cannot compute ArgMin for an empty array')
+    out = ndarray.empty([d for i, d in enumerate(a.shape) if i not in axes], 'int64')
+    return _reduce('hipcx_argmin', a, axes, out)
+
+
+def all(a, axis=None, keepdims=False):
+    """All (CX/routines/logic.cc:79-87); the kernel casts the input to bool first (native/native_device/logic.cc)."""
+    axes = _sorted_axes(axis, a.ndim)
+    out = _reduced_out(a, axes, keepdims, 'bool')
+    return _reduce('hipcx_all', a.astype('bool', False), axes, out)
+
+
+def any(a, axis=None, keepdims=False):
+    """Any (CX/routines/logic.cc:89-97)."""
+    axes = _sorted_axes(axis, a.ndim)
+    out = _reduced_out(a, axes, keepdims, 'bool')
+    return _reduce('hipcx_any', a.astype('bool', False), axes, out)
 
 
 def mean(a, axis=None, keepdims=False):

@@ -130,6 +130,48 @@ int hipcx_copy(const hipcx_array* a, const hipcx_array* out, void* stream);     
 int hipcx_fill(const hipcx_array* out, hipcx_scalar value, void* stream);                         /* FillKernel misc.h:9 */
 int hipcx_arange(hipcx_scalar start, hipcx_scalar step, const hipcx_array* out, void* stream);    /* ArangeKernel creation.h:11 */
 
+/* ---- further elementwise kernels ----
+ * hipcx_unary: out = f(x), x.dtype == out.dtype.  Float dtypes only (float16 as Float16(f(float(x))), CX/numeric.h:59-83) for
+ *   ErfKernel explog.h:10, Expm1Kernel :20, Exp2Kernel :25, Log10Kernel :35, Log2Kernel :40, Log1pKernel :45,
+ *   SinhKernel hyperbolic.h:8, CoshKernel :13, ArcsinhKernel :23, ArccoshKernel :28,
+ *   SinKernel trigonometric.h:8, CosKernel :13, TanKernel :18, ArcsinKernel :23, ArccosKernel :28, ArctanKernel :33,
+ *   CeilKernel rounding.h:8, FloorKernel :13;
+ *   numeric dtypes for SquareKernel misc.h:19 (x*x), AbsKernel :24, SignKernel :29 (NaN passes; CX/numeric.h:33-57). */
+enum hipcx_unary_op {
+    HIPCX_UNARY_ERF = 1, HIPCX_UNARY_EXPM1, HIPCX_UNARY_EXP2, HIPCX_UNARY_LOG10, HIPCX_UNARY_LOG2, HIPCX_UNARY_LOG1P,
+    HIPCX_UNARY_SINH, HIPCX_UNARY_COSH, HIPCX_UNARY_ARCSINH, HIPCX_UNARY_ARCCOSH,
+    HIPCX_UNARY_SIN, HIPCX_UNARY_COS, HIPCX_UNARY_TAN, HIPCX_UNARY_ARCSIN, HIPCX_UNARY_ARCCOS, HIPCX_UNARY_ARCTAN,
+    HIPCX_UNARY_CEIL, HIPCX_UNARY_FLOOR,
+    HIPCX_UNARY_SQUARE, HIPCX_UNARY_ABS, HIPCX_UNARY_SIGN
+};
+int hipcx_unary(int op, const hipcx_array* x, const hipcx_array* out, void* stream);
+
+/* bool out = p(x), any x dtype: LogicalNotKernel logic.h:29 (!x), IsNanKernel :59, IsInfKernel :64, IsFiniteKernel :69
+ * (integers and bool are never NaN / Inf, CX/numeric.h:17-31). */
+enum hipcx_predicate_op { HIPCX_PRED_LOGICAL_NOT = 1, HIPCX_PRED_ISNAN, HIPCX_PRED_ISINF, HIPCX_PRED_ISFINITE };
+int hipcx_predicate(int op, const hipcx_array* x, const hipcx_array* out, void* stream);
+
+/* bool out = x1 op x2 on the truth values, operands of one dtype: LogicalAndKernel logic.h:34, LogicalOrKernel :39,
+ * LogicalXorKernel :44 (!x1 != !x2). */
+enum hipcx_logical_op { HIPCX_LOGICAL_AND = 1, HIPCX_LOGICAL_OR, HIPCX_LOGICAL_XOR };
+int hipcx_logical(int op, const hipcx_array* x1, const hipcx_array* x2, const hipcx_array* out, void* stream);
+
+/* PowerKernel arithmetic.h:71, PowerASKernel :76, PowerSAKernel :81: numeric dtypes; integers by repeated squaring with
+ * wrap-around, negative integer exponents give 0 except for bases 1 and -1 (CX/numeric.h:85-135); floats through pow.
+ * FmodKernel arithmetic.h:107 and Arctan2Kernel trigonometric.h:38: float dtypes. */
+int hipcx_power(const hipcx_array* x1, const hipcx_array* x2, const hipcx_array* out, void* stream);
+int hipcx_power_as(const hipcx_array* x1, hipcx_scalar x2, const hipcx_array* out, void* stream);
+int hipcx_power_sa(hipcx_scalar x1, const hipcx_array* x2, const hipcx_array* out, void* stream);
+int hipcx_fmod(const hipcx_array* x1, const hipcx_array* x2, const hipcx_array* out, void* stream);
+int hipcx_arctan2(const hipcx_array* x1, const hipcx_array* x2, const hipcx_array* out, void* stream);
+
+/* WhereKernel indexing.h:22, WhereAASKernel :27, WhereASAKernel :32, WhereASSKernel :37: out = condition ? x : y with a bool
+ * condition array and x / y of out's dtype, arrays or scalars (native/native_device/indexing.cc:194-283). */
+int hipcx_where(const hipcx_array* condition, const hipcx_array* x, const hipcx_array* y, const hipcx_array* out, void* stream);
+int hipcx_where_aas(const hipcx_array* condition, const hipcx_array* x, hipcx_scalar y, const hipcx_array* out, void* stream);
+int hipcx_where_asa(const hipcx_array* condition, hipcx_scalar x, const hipcx_array* y, const hipcx_array* out, void* stream);
+int hipcx_where_ass(const hipcx_array* condition, hipcx_scalar x, hipcx_scalar y, const hipcx_array* out, void* stream);
+
 /* ---- reductions: CX/kernels/reduction.h:18, statistics.h:13, sorting.h:9 ----
  * `axis` is sorted, unique, non-negative (CX/kernels/reduction.h:11-18); `out` either drops the
  * reduced axes or keeps them with extent 1.  argmax writes int64 and reproduces the native
@@ -142,6 +184,19 @@ int hipcx_amax(const hipcx_array* a, const int8_t* axis, int naxis, const hipcx_
                void* stream);
 int hipcx_argmax(const hipcx_array* a, const int8_t* axis, int naxis, const hipcx_array* out, void* workspace,
                  size_t workspace_bytes, void* stream);
+
+/* AMinKernel statistics.h:20 (identity MaxOrInf, NaN-propagating, native/native_device/statistics.cc:52-73); ArgMinKernel
+ * sorting.h:14 (same tie/NaN rule as argmax with the comparison mirrored, native/native_device/reduction.cc:65-92);
+ * AllKernel / AnyKernel logic.h:49,54 over bool arrays (the routine casts other dtypes to bool first,
+ * native/native_device/logic.cc NativeAllKernel / NativeAnyKernel).  Workspace as for hipcx_sum. */
+int hipcx_amin(const hipcx_array* a, const int8_t* axis, int naxis, const hipcx_array* out, void* workspace, size_t workspace_bytes,
+               void* stream);
+int hipcx_argmin(const hipcx_array* a, const int8_t* axis, int naxis, const hipcx_array* out, void* workspace,
+                 size_t workspace_bytes, void* stream);
+int hipcx_all(const hipcx_array* a, const int8_t* axis, int naxis, const hipcx_array* out, void* workspace, size_t workspace_bytes,
+              void* stream);
+int hipcx_any(const hipcx_array* a, const int8_t* axis, int naxis, const hipcx_array* out, void* workspace, size_t workspace_bytes,
+              void* stream);
 
 /* ---- linear algebra / connection: CX/kernels/linalg.h:15, connection.h:21 ---- */
 /* out[M,N] = a[M,K] . b[K,N]; float16/32/64; fp16 accumulates in fp32 (CX/native/native_device/dot.cc:181-227). */

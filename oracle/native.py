@@ -126,6 +126,195 @@ def sqrt(x):
         return np.sqrt(x)
 
 
+def _float_unary(fn, x):
+    """Float16(f(float(x))) for float16, f in the array's own precision otherwise (CX/numeric.h:59-83 over std::f).
+    Pinned as a library routine (numpy / scipy follow the same libm definitions); tolerance-level parity only."""
+    x = np.asarray(x)
+    with np.errstate(all='ignore'):
+        if x.dtype == np.float16:
+            return fn(x.astype(np.float32)).astype(np.float16)
+        return fn(x).astype(x.dtype)
+
+
+def erf(x):
+    from scipy import special
+    return _float_unary(special.erf, x)
+
+
+def expm1(x):
+    return _float_unary(np.expm1, x)
+
+
+def exp2(x):
+    return _float_unary(np.exp2, x)
+
+
+def log10(x):
+    return _float_unary(np.log10, x)
+
+
+def log2(x):
+    return _float_unary(np.log2, x)
+
+
+def log1p(x):
+    return _float_unary(np.log1p, x)
+
+
+def sinh(x):
+    return _float_unary(np.sinh, x)
+
+
+def cosh(x):
+    return _float_unary(np.cosh, x)
+
+
+def arcsinh(x):
+    return _float_unary(np.arcsinh, x)
+
+
+def arccosh(x):
+    return _float_unary(np.arccosh, x)
+
+
+def sin(x):
+    return _float_unary(np.sin, x)
+
+
+def cos(x):
+    return _float_unary(np.cos, x)
+
+
+def tan(x):
+    return _float_unary(np.tan, x)
+
+
+def arcsin(x):
+    return _float_unary(np.arcsin, x)
+
+
+def arccos(x):
+    return _float_unary(np.arccos, x)
+
+
+def arctan(x):
+    return _float_unary(np.arctan, x)
+
+
+def ceil(x):
+    return _float_unary(np.ceil, x)
+
+
+def floor(x):
+    return _float_unary(np.floor, x)
+
+
+def square(x):
+    """SquareKernel: out = x * x in the array dtype, integers wrap (native/native_device/misc.cc)."""
+    x = np.asarray(x)
+    with np.errstate(all='ignore'):
+        return (x * x).astype(x.dtype)
+
+
+def absolute(x):
+    """AbsKernel: std::abs, identity for uint8 (CX/numeric.h:40-57); abs(lowest) wraps to lowest."""
+    x = np.asarray(x)
+    with np.errstate(all='ignore'):
+        return np.abs(x).astype(x.dtype)
+
+
+def sign(x):
+    """SignKernel: NaN passes, else (0 < x) - (x < 0) (CX/numeric.h:33-38)."""
+    x = np.asarray(x)
+    r = ((x > 0).astype(np.int8) - (x < 0).astype(np.int8)).astype(x.dtype)
+    if x.dtype.kind == 'f':
+        r = np.where(np.isnan(x), x, r).astype(x.dtype)
+    return r
+
+
+def logical_not(x):
+    return ~np.asarray(x).astype(bool)
+
+
+def isnan(x):
+    x = np.asarray(x)
+    return np.isnan(x) if x.dtype.kind == 'f' else np.zeros(x.shape, bool)
+
+
+def isinf(x):
+    x = np.asarray(x)
+    return np.isinf(x) if x.dtype.kind == 'f' else np.zeros(x.shape, bool)
+
+
+def isfinite(x):
+    x = np.asarray(x)
+    return np.isfinite(x) if x.dtype.kind == 'f' else np.ones(x.shape, bool)
+
+
+def logical_and(x1, x2):
+    return np.asarray(x1).astype(bool) & np.asarray(x2).astype(bool)
+
+
+def logical_or(x1, x2):
+    return np.asarray(x1).astype(bool) | np.asarray(x2).astype(bool)
+
+
+def logical_xor(x1, x2):
+    """!x1 != !x2 (native/native_device/logic.cc NativeLogicalXorKernel)."""
+    return np.asarray(x1).astype(bool) ^ np.asarray(x2).astype(bool)
+
+
+def power(x1, x2):
+    """chainerx::Power (CX/numeric.h:85-135) on operands already cast to one dtype: integers by repeated squaring with
+    wrap-around, a negative exponent gives +-1 for bases 1 / -1 and 0 otherwise; floats through pow."""
+    x1, x2 = np.broadcast_arrays(np.asarray(x1), np.asarray(x2))
+    dt = x1.dtype
+    with np.errstate(all='ignore'):
+        if dt.kind == 'f':
+            if dt == np.float16:
+                return np.power(x1.astype(np.float32), x2.astype(np.float32)).astype(np.float16)
+            return np.power(x1, x2).astype(dt)
+        out = np.ones(x1.shape, dt)
+        base = x1.copy()
+        e = np.where(x2 > 0, x2, 0).astype(np.uint64)
+        while (e > 0).any():
+            out = np.where((e & np.uint64(1)) != 0, out * base, out).astype(dt)
+            base = (base * base).astype(dt)
+            e = e >> np.uint64(1)
+        if dt.kind == 'i':
+            neg = x2 < 0
+            odd = (x2 & 1) != 0
+            special = np.where(x1 == 1, 1, np.where(x1 == -1, np.where(odd, -1, 1), 0)).astype(dt)
+            out = np.where(neg, special, out).astype(dt)
+        return out
+
+
+def fmod(x1, x2):
+    """FmodKernel: std::fmod, float16 through float."""
+    x1, x2 = np.asarray(x1), np.asarray(x2)
+    with np.errstate(all='ignore'):
+        if x1.dtype == np.float16:
+            return np.fmod(x1.astype(np.float32), x2.astype(np.float32)).astype(np.float16)
+        return np.fmod(x1, x2).astype(x1.dtype)
+
+
+def arctan2(x1, x2):
+    x1, x2 = np.asarray(x1), np.asarray(x2)
+    with np.errstate(all='ignore'):
+        if x1.dtype == np.float16:
+            return np.arctan2(x1.astype(np.float32), x2.astype(np.float32)).astype(np.float16)
+        return np.arctan2(x1, x2).astype(x1.dtype)
+
+
+def where(condition, x, y, dtype):
+    """WhereKernel family (native/native_device/indexing.cc:194-283): condition cast to bool, x / y cast to the out dtype."""
+    c = np.asarray(condition).astype(bool)
+    dt = np.dtype(dtype)
+    xa = _scalar_as(x, dt) if np.isscalar(x) else np.asarray(x).astype(dt)
+    ya = _scalar_as(y, dt) if np.isscalar(y) else np.asarray(y).astype(dt)
+    return np.where(c, xa, ya).astype(dt)
+
+
 def if_less_else(x1, x2, pos, neg):
     """x1 < x2 ? pos : neg (misc.cc:39-61); x2 and pos are scalars cast to the dtype."""
     x1 = np.asarray(x1)
@@ -245,6 +434,38 @@ def argmax(a, axis=None):
     out = np.empty(n, np.int64)
     lib().oracle_argmax(_ptr(r, _f64p), _i64(n), _i64(length), _ptr(out, _i64p))
     return out.reshape(out_shape)
+
+
+def amin(a, axis=None, keepdims=False):
+    """NativeAMinKernel (statistics.cc:52-73) is AMax with the comparison mirrored: through an order-reversing exact map
+    (negation for floats, bitwise complement for integers) the same pairwise tree and NaN rule apply."""
+    a = np.asarray(a)
+    if a.dtype.kind == 'f':
+        return -amax(-a, axis, keepdims)
+    if a.dtype.kind == 'b':
+        return ~amax(~a, axis, keepdims)
+    wide = ~a.astype(np.int64)
+    return (~amax(wide, axis, keepdims)).astype(a.dtype)
+
+
+def argmin(a, axis=None):
+    """NativeArgMinKernel (reduction.cc:65-92): ArgMax's accumulator with `accum.min > next.min`."""
+    a = np.asarray(a)
+    if a.dtype.kind == 'f':
+        return argmax(-a.astype(np.float64), axis)
+    return argmax(-(a.astype(np.float64)), axis)
+
+
+def all(a, axis=None, keepdims=False):
+    """NativeAllKernel (logic.cc): input cast to bool, accum && next; order independent."""
+    a = np.asarray(a).astype(bool)
+    return np.all(a, axis=axis if axis is None or isinstance(axis, int) else tuple(axis), keepdims=keepdims)
+
+
+def any(a, axis=None, keepdims=False):
+    """NativeAnyKernel (logic.cc): input cast to bool, accum || next; order independent."""
+    a = np.asarray(a).astype(bool)
+    return np.any(a, axis=axis if axis is None or isinstance(axis, int) else tuple(axis), keepdims=keepdims)
 
 
 def mean(a, axis=None, keepdims=False):

@@ -49,15 +49,15 @@ def run_golden(F, case, to_dev=lambda a: a, to_host=np.asarray):
     """Evaluates one golden case with routine namespace F; shared by the CPU (oracle) and GPU (hip) golden tests."""
     dt = np.dtype(case['dtype'])
     op = case['op']
-    if op in ('sum', 'amax'):
+    if op in ('sum', 'amax', 'amin'):
         x = build_input(case['input'], dt)
         axis = norm_axis(case['axis'])
         axis = None if axis is None else tuple(a % x.ndim for a in axis)
         out = getattr(F, op)(to_dev(x), axis, case['keepdims'])
-    elif op == 'argmax':
+    elif op in ('argmax', 'argmin'):
         x = build_input(case['input'], dt)
         axis = norm_axis(case['axis'])
-        out = F.argmax(to_dev(x), None if axis is None else axis[0])
+        out = getattr(F, op)(to_dev(x), None if axis is None else axis[0])
     elif op == 'dot':
         out = F.dot(to_dev(build_input(case['a'], dt)), to_dev(build_input(case['b'], dt)))
     elif op == 'take':
@@ -509,3 +509,49 @@ def test_lstm_closed_form():
     for dt, tol in (('float64', 1e-14), ('float32', 1e-6)):
         h, cn = O.lstm(c.astype(dt), x.astype(dt))
         assert np.abs(h - h_ref).max() <= tol and np.abs(cn - c_ref).max() <= tol
+
+
+def test_power_integer_rule_brute_force():
+    """B: chainerx::Power on integers (CX/numeric.h:85-125) equals exact integer exponentiation reduced modulo 2^bits for
+    non-negative exponents, and the 1 / -1 / 0 rule for negative ones -- checked for every int8 base against Python's pow."""
+    bases = np.arange(-128, 128, dtype=np.int8)
+    for e in range(-4, 12):
+        got = O.power(bases, np.full(bases.shape, e, np.int8))
+        if e < 0:
+            exp = np.array([1 if b == 1 else ((-1 if e % 2 else 1) if b == -1 else 0) for b in bases.tolist()], np.int8)
+        else:
+            exp = np.array([((pow(b, e) + 128) % 256) - 128 for b in bases.tolist()], np.int8)
+        assert np.array_equal(got, exp), e
+    ub = np.arange(0, 256, dtype=np.uint8)
+    for e in range(0, 10):
+        assert np.array_equal(O.power(ub, np.full(ub.shape, e, np.uint8)), np.array([pow(b, e) % 256 for b in ub.tolist()], np.uint8))
+
+
+def test_amin_argmin_mirror_amax_argmax():
+    """C: minimum = -maximum of the negated data with the same tree, so tie-free data must agree with numpy, a NaN
+    propagates, and the ArgMin literals of the reference (array_test.cc:1436-1454, in the golden file) hold."""
+    rng = np.random.default_rng(31)
+    x = rng.standard_normal((9, 777)).astype(np.float32)
+    assert np.array_equal(O.amin(x, 1), x.min(axis=1))
+    assert np.array_equal(O.argmin(x, 1), x.argmin(axis=1))
+    xi = rng.integers(-2 ** 62, 2 ** 62, (5, 99))
+    assert np.array_equal(O.amin(xi, 1), xi.min(axis=1))
+    for dt in ('int8', 'uint8', 'bool'):
+        xs = (rng.integers(0, 2, (4, 50)) if dt == 'bool' else rng.integers(0, 100, (4, 50))).astype(dt)
+        assert np.array_equal(O.amin(xs, 1), xs.min(axis=1)) and O.amin(xs, 1).dtype == xs.dtype
+    x[3, 5] = np.nan
+    assert np.isnan(O.amin(x, 1)[3]) and not np.isnan(O.amin(x, 1)[2])
+    # earlier index wins a tie inside a block, like argmax
+    t = np.array([[3.0, 1.0, 1.0, 2.0]], np.float32)
+    assert O.argmin(t, 1)[0] == 1
+
+
+def test_sign_abs_where_literals():
+    """C: closed forms.  Sign: NaN passes, zero of either sign gives zero; Abs wraps at the lowest integer; Where selects."""
+    x = np.array([-2.5, -0.0, 0.0, 3.0, np.nan, -np.inf], np.float32)
+    s = O.sign(x)
+    assert np.array_equal(s[:4], [-1, 0, 0, 1]) and np.isnan(s[4]) and s[5] == -1
+    assert np.array_equal(O.absolute(np.array([-128, -1, 127], np.int8)), np.array([-128, 1, 127], np.int8))
+    assert np.array_equal(O.absolute(np.array([200, 3], np.uint8)), np.array([200, 3], np.uint8))
+    assert np.array_equal(O.where(np.array([1, 0, 2]), np.array([1, 2, 3]), 9, 'int32'), np.array([1, 9, 3], np.int32))
+    assert np.array_equal(O.logical_xor(np.array([0, 2, 0, 5]), np.array([0, 0, 3, 7])), [False, True, True, False])
