@@ -48,8 +48,10 @@
 #include "chainerx/kernels/normalization.h"
 #include "chainerx/kernels/pooling.h"
 #include "chainerx/kernels/reduction.h"
+#include "chainerx/kernels/rounding.h"
 #include "chainerx/kernels/sorting.h"
 #include "chainerx/kernels/statistics.h"
+#include "chainerx/kernels/trigonometric.h"
 #include "chainerx/native/native_backend.h"
 #include "chainerx/routines/connection.h"
 #include "chainerx/routines/creation.h"
@@ -424,6 +426,145 @@ public:
 };
 HIPCX_REGISTER_KERNEL(IfGreaterElseAAAAKernel, HipIfGreaterElseAAAAKernel)
 
+// ---- further elementwise kernels: one C entry per family, selected by an op code ----
+#define HIPCX_UNARY_CODE_KERNEL(Name, code)                                               \
+    class Hip##Name##Kernel : public Name##Kernel {                                       \
+    public:                                                                               \
+        void Call(const Array& x, const Array& out) override {                            \
+            Device& device = x.device();                                                  \
+            device.CheckDevicesCompatible(x, out);                                        \
+            SetDeviceScope scope{device.index()};                                         \
+            hipcx_array a = ToC(Cast(x, out.dtype())), o = ToC(out);                      \
+            Check(hipcx_unary(code, &a, &o, nullptr));                                    \
+        }                                                                                 \
+    };                                                                                    \
+    HIPCX_REGISTER_KERNEL(Name##Kernel, Hip##Name##Kernel)
+
+HIPCX_UNARY_CODE_KERNEL(Erf, HIPCX_UNARY_ERF)
+HIPCX_UNARY_CODE_KERNEL(Expm1, HIPCX_UNARY_EXPM1)
+HIPCX_UNARY_CODE_KERNEL(Exp2, HIPCX_UNARY_EXP2)
+HIPCX_UNARY_CODE_KERNEL(Log10, HIPCX_UNARY_LOG10)
+HIPCX_UNARY_CODE_KERNEL(Log2, HIPCX_UNARY_LOG2)
+HIPCX_UNARY_CODE_KERNEL(Log1p, HIPCX_UNARY_LOG1P)
+HIPCX_UNARY_CODE_KERNEL(Sinh, HIPCX_UNARY_SINH)
+HIPCX_UNARY_CODE_KERNEL(Cosh, HIPCX_UNARY_COSH)
+HIPCX_UNARY_CODE_KERNEL(Arcsinh, HIPCX_UNARY_ARCSINH)
+HIPCX_UNARY_CODE_KERNEL(Arccosh, HIPCX_UNARY_ARCCOSH)
+HIPCX_UNARY_CODE_KERNEL(Sin, HIPCX_UNARY_SIN)
+HIPCX_UNARY_CODE_KERNEL(Cos, HIPCX_UNARY_COS)
+HIPCX_UNARY_CODE_KERNEL(Tan, HIPCX_UNARY_TAN)
+HIPCX_UNARY_CODE_KERNEL(Arcsin, HIPCX_UNARY_ARCSIN)
+HIPCX_UNARY_CODE_KERNEL(Arccos, HIPCX_UNARY_ARCCOS)
+HIPCX_UNARY_CODE_KERNEL(Arctan, HIPCX_UNARY_ARCTAN)
+HIPCX_UNARY_CODE_KERNEL(Ceil, HIPCX_UNARY_CEIL)
+HIPCX_UNARY_CODE_KERNEL(Floor, HIPCX_UNARY_FLOOR)
+HIPCX_UNARY_CODE_KERNEL(Square, HIPCX_UNARY_SQUARE)
+HIPCX_UNARY_CODE_KERNEL(Abs, HIPCX_UNARY_ABS)
+HIPCX_UNARY_CODE_KERNEL(Sign, HIPCX_UNARY_SIGN)
+
+// bool out = p(x): the input keeps its dtype
+#define HIPCX_PREDICATE_KERNEL(Name, code)                                                \
+    class Hip##Name##Kernel : public Name##Kernel {                                       \
+    public:                                                                               \
+        void Call(const Array& x, const Array& out) override {                            \
+            Device& device = x.device();                                                  \
+            device.CheckDevicesCompatible(x, out);                                        \
+            SetDeviceScope scope{device.index()};                                         \
+            hipcx_array a = ToC(x), o = ToC(out);                                         \
+            Check(hipcx_predicate(code, &a, &o, nullptr));                                \
+        }                                                                                 \
+    };                                                                                    \
+    HIPCX_REGISTER_KERNEL(Name##Kernel, Hip##Name##Kernel)
+
+HIPCX_PREDICATE_KERNEL(LogicalNot, HIPCX_PRED_LOGICAL_NOT)
+HIPCX_PREDICATE_KERNEL(IsNan, HIPCX_PRED_ISNAN)
+HIPCX_PREDICATE_KERNEL(IsInf, HIPCX_PRED_ISINF)
+HIPCX_PREDICATE_KERNEL(IsFinite, HIPCX_PRED_ISFINITE)
+
+#define HIPCX_LOGICAL_KERNEL(Name, code)                                                  \
+    class Hip##Name##Kernel : public Name##Kernel {                                       \
+    public:                                                                               \
+        void Call(const Array& x1, const Array& x2, const Array& out) override {          \
+            Device& device = x1.device();                                                 \
+            device.CheckDevicesCompatible(x1, x2, out);                                   \
+            SetDeviceScope scope{device.index()};                                         \
+            Dtype dtype = PromoteTypes(x1.dtype(), x2.dtype());                           \
+            hipcx_array a = ToC(Cast(x1, dtype)), b = ToC(Cast(x2, dtype)), o = ToC(out); \
+            Check(hipcx_logical(code, &a, &b, &o, nullptr));                              \
+        }                                                                                 \
+    };                                                                                    \
+    HIPCX_REGISTER_KERNEL(Name##Kernel, Hip##Name##Kernel)
+
+HIPCX_LOGICAL_KERNEL(LogicalAnd, HIPCX_LOGICAL_AND)
+HIPCX_LOGICAL_KERNEL(LogicalOr, HIPCX_LOGICAL_OR)
+HIPCX_LOGICAL_KERNEL(LogicalXor, HIPCX_LOGICAL_XOR)
+
+HIPCX_BINARY_KERNEL(Power, hipcx_power)
+HIPCX_BINARY_AS_KERNEL(PowerAS, hipcx_power_as)
+HIPCX_BINARY_KERNEL(Fmod, hipcx_fmod)
+HIPCX_BINARY_KERNEL(Arctan2, hipcx_arctan2)
+
+class HipPowerSAKernel : public PowerSAKernel {
+public:
+    void Call(Scalar x1, const Array& x2, const Array& out) override {
+        Device& device = x2.device();
+        device.CheckDevicesCompatible(x2, out);
+        SetDeviceScope scope{device.index()};
+        hipcx_array b = ToC(Cast(x2, out.dtype())), o = ToC(out);
+        Check(hipcx_power_sa(ToC(x1), &b, &o, nullptr));
+    }
+};
+HIPCX_REGISTER_KERNEL(PowerSAKernel, HipPowerSAKernel)
+
+// Where: the condition is cast to bool, x / y to out's dtype (native/native_device/indexing.cc:194-283)
+class HipWhereKernel : public WhereKernel {
+public:
+    void Call(const Array& condition, const Array& x, const Array& y, const Array& out) override {
+        Device& device = condition.device();
+        device.CheckDevicesCompatible(condition, x, y, out);
+        SetDeviceScope scope{device.index()};
+        hipcx_array c = ToC(Cast(condition, Dtype::kBool)), a = ToC(Cast(x, out.dtype())), b = ToC(Cast(y, out.dtype())), o = ToC(out);
+        Check(hipcx_where(&c, &a, &b, &o, nullptr));
+    }
+};
+HIPCX_REGISTER_KERNEL(WhereKernel, HipWhereKernel)
+
+class HipWhereAASKernel : public WhereAASKernel {
+public:
+    void Call(const Array& condition, const Array& x, Scalar y, const Array& out) override {
+        Device& device = condition.device();
+        device.CheckDevicesCompatible(condition, x, out);
+        SetDeviceScope scope{device.index()};
+        hipcx_array c = ToC(Cast(condition, Dtype::kBool)), a = ToC(Cast(x, out.dtype())), o = ToC(out);
+        Check(hipcx_where_aas(&c, &a, ToC(y), &o, nullptr));
+    }
+};
+HIPCX_REGISTER_KERNEL(WhereAASKernel, HipWhereAASKernel)
+
+class HipWhereASAKernel : public WhereASAKernel {
+public:
+    void Call(const Array& condition, Scalar x, const Array& y, const Array& out) override {
+        Device& device = condition.device();
+        device.CheckDevicesCompatible(condition, y, out);
+        SetDeviceScope scope{device.index()};
+        hipcx_array c = ToC(Cast(condition, Dtype::kBool)), b = ToC(Cast(y, out.dtype())), o = ToC(out);
+        Check(hipcx_where_asa(&c, ToC(x), &b, &o, nullptr));
+    }
+};
+HIPCX_REGISTER_KERNEL(WhereASAKernel, HipWhereASAKernel)
+
+class HipWhereASSKernel : public WhereASSKernel {
+public:
+    void Call(const Array& condition, Scalar x, Scalar y, const Array& out) override {
+        Device& device = condition.device();
+        device.CheckDevicesCompatible(condition, out);
+        SetDeviceScope scope{device.index()};
+        hipcx_array c = ToC(Cast(condition, Dtype::kBool)), o = ToC(out);
+        Check(hipcx_where_ass(&c, ToC(x), ToC(y), &o, nullptr));
+    }
+};
+HIPCX_REGISTER_KERNEL(WhereASSKernel, HipWhereASSKernel)
+
 // ---- creation ----
 class HipCopyKernel : public CopyKernel {
 public:
@@ -488,6 +629,31 @@ public:
     void Call(const Array& a, const Axes& axis, const Array& out) override { CallReduce(hipcx_argmax, a, axis, out); }
 };
 HIPCX_REGISTER_KERNEL(ArgMaxKernel, HipArgMaxKernel)
+
+class HipAMinKernel : public AMinKernel {
+public:
+    void Call(const Array& a, const Axes& axis, const Array& out) override { CallReduce(hipcx_amin, a, axis, out); }
+};
+HIPCX_REGISTER_KERNEL(AMinKernel, HipAMinKernel)
+
+class HipArgMinKernel : public ArgMinKernel {
+public:
+    void Call(const Array& a, const Axes& axis, const Array& out) override { CallReduce(hipcx_argmin, a, axis, out); }
+};
+HIPCX_REGISTER_KERNEL(ArgMinKernel, HipArgMinKernel)
+
+// All / Any reduce truth values: other dtypes are cast to bool first (native/native_device/logic.cc)
+class HipAllKernel : public AllKernel {
+public:
+    void Call(const Array& a, const Axes& axis, const Array& out) override { CallReduce(hipcx_all, Cast(a, Dtype::kBool), axis, out); }
+};
+HIPCX_REGISTER_KERNEL(AllKernel, HipAllKernel)
+
+class HipAnyKernel : public AnyKernel {
+public:
+    void Call(const Array& a, const Axes& axis, const Array& out) override { CallReduce(hipcx_any, Cast(a, Dtype::kBool), axis, out); }
+};
+HIPCX_REGISTER_KERNEL(AnyKernel, HipAnyKernel)
 
 // ---- dot / conv ----
 class HipDotKernel : public DotKernel {
