@@ -127,19 +127,36 @@ __global__ __launch_bounds__(NT) void LogSoftmaxRowKernel(const T* x, T* out, in
 // segments, then rewrites its own segment ----
 constexpr int kSegThreads = 256;
 
+// A segment is walked in packs of 16 bytes when rows start on 16-byte boundaries (seg_len is a multiple of the pack size).
+template <typename T, typename F>
+__device__ __forceinline__ void ForSegment(const T* xr, int64_t lo, int64_t hi, int vec_ok, F&& f) {
+    constexpr int V = 16 / sizeof(T);
+    if (vec_ok) {
+        const int64_t full = lo + (hi - lo) / V * V;
+        for (int64_t e = lo + static_cast<int64_t>(threadIdx.x) * V; e < full; e += kSegThreads * V) {
+            Pack<T, V> p = *reinterpret_cast<const Pack<T, V>*>(xr + e);
+#pragma unroll
+            for (int j = 0; j < V; ++j) f(e + j, p.e[j]);
+        }
+        for (int64_t e = full + threadIdx.x; e < hi; e += kSegThreads) f(e, xr[e]);
+    } else {
+        for (int64_t e = lo + threadIdx.x; e < hi; e += kSegThreads) f(e, xr[e]);
+    }
+}
+
 template <typename T>
 __global__ __launch_bounds__(kSegThreads) void LogSoftmaxPartialKernel(const T* x, compute_t<T>* part, int64_t n, int64_t x_row, int64_t seg_len,
-                                                                       int nseg) {
+                                                                       int nseg, int vec_ok) {
     using C = compute_t<T>;
     __shared__ C scratch[kSegThreads / 64];
     const int row = blockIdx.x / nseg, seg = blockIdx.x - row * nseg;
     const T* xr = x + static_cast<int64_t>(row) * x_row;
     const int64_t lo = seg * seg_len, hi = min(n, lo + seg_len);
     C m = -INFINITY;
-    for (int64_t e = lo + threadIdx.x; e < hi; e += kSegThreads) m = MaxNan(m, static_cast<C>(xr[e]));
+    ForSegment<T>(xr, lo, hi, vec_ok, [&](int64_t, T v) { m = MaxNan(m, static_cast<C>(v)); });
     m = BlockReduce<C, kSegThreads, true>(m, scratch);
     C s = 0;
-    for (int64_t e = lo + threadIdx.x; e < hi; e += kSegThreads) s += ExpOf<C>(static_cast<C>(xr[e]) - m);
+    ForSegment<T>(xr, lo, hi, vec_ok, [&](int64_t, T v) { s += ExpOf<C>(static_cast<C>(v) - m); });  // second walk hits L2
     s = BlockReduce<C, kSegThreads, false>(s, scratch);
     // a segment of -inf only: its terms are exp(-inf - rowmax) = 0 unless the whole row is -inf (then 0 * exp(NaN) = NaN below,
     // which is what the chain gives for such a row)
@@ -152,8 +169,9 @@ __global__ __launch_bounds__(kSegThreads) void LogSoftmaxPartialKernel(const T* 
 
 template <typename T>
 __global__ __launch_bounds__(kSegThreads) void LogSoftmaxApplyKernel(const T* x, T* out, const compute_t<T>* part, int64_t n, int64_t x_row,
-                                                                     int64_t o_row, int64_t seg_len, int nseg) {
+                                                                     int64_t o_row, int64_t seg_len, int nseg, int vec_ok) {
     using C = compute_t<T>;
+    constexpr int V = 16 / sizeof(T);
     __shared__ C scratch[kSegThreads / 64];
     const int row = blockIdx.x / nseg, seg = blockIdx.x - row * nseg;
     const C* pr = part + 2 * static_cast<int64_t>(row) * nseg;
@@ -170,7 +188,18 @@ __global__ __launch_bounds__(kSegThreads) void LogSoftmaxApplyKernel(const T* x,
     const T* xr = x + static_cast<int64_t>(row) * x_row;
     T* orow = out + static_cast<int64_t>(row) * o_row;
     const int64_t lo = seg * seg_len, hi = min(n, lo + seg_len);
-    for (int64_t e = lo + threadIdx.x; e < hi; e += kSegThreads) orow[e] = static_cast<T>(static_cast<C>(xr[e]) - lse);
+    if (vec_ok) {
+        const int64_t full = lo + (hi - lo) / V * V;
+        for (int64_t e = lo + static_cast<int64_t>(threadIdx.x) * V; e < full; e += kSegThreads * V) {
+            Pack<T, V> p = *reinterpret_cast<const Pack<T, V>*>(xr + e);
+#pragma unroll
+            for (int j = 0; j < V; ++j) p.e[j] = static_cast<T>(static_cast<C>(p.e[j]) - lse);
+            *reinterpret_cast<Pack<T, V>*>(orow + e) = p;
+        }
+        for (int64_t e = full + threadIdx.x; e < hi; e += kSegThreads) orow[e] = static_cast<T>(static_cast<C>(xr[e]) - lse);
+    } else {
+        for (int64_t e = lo + threadIdx.x; e < hi; e += kSegThreads) orow[e] = static_cast<T>(static_cast<C>(xr[e]) - lse);
+    }
 }
 
 constexpr int64_t kRowInRegisters = 16384 * 4;  // bytes of a row the register kernel holds (256 threads x 16 packs x 16 bytes)
@@ -223,10 +252,10 @@ void RunLogSoftmax(const hipcx_array* x, const hipcx_array* out, const LsmShape&
         auto* part = static_cast<compute_t<T>*>(workspace);
         const unsigned blocks = static_cast<unsigned>(sh.rows * nseg);
         hipLaunchKernelGGL(LogSoftmaxPartialKernel<T>, dim3(blocks), dim3(kSegThreads), 0, stream, xp, part, sh.n, sh.x_row, seg_len,
-                           static_cast<int>(nseg));
+                           static_cast<int>(nseg), vec_ok);
         CheckLaunch("log_softmax_partial");
         hipLaunchKernelGGL(LogSoftmaxApplyKernel<T>, dim3(blocks), dim3(kSegThreads), 0, stream, xp, op, part, sh.n, sh.x_row, sh.o_row, seg_len,
-                           static_cast<int>(nseg));
+                           static_cast<int>(nseg), vec_ok);
     }
     CheckLaunch("log_softmax");
 }
