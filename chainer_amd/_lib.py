@@ -147,6 +147,9 @@ SIGNATURES = {
     'hipcx_power': (_INT, [_A, _A, _A, _V]),
     'hipcx_power_as': (_INT, [_A, _S, _A, _V]),
     'hipcx_power_sa': (_INT, [_S, _A, _A, _V]),
+    'hipcx_binary': (_INT, [_INT, _A, _A, _A, _V]),
+    'hipcx_binary_as': (_INT, [_INT, _A, _S, _A, _V]),
+    'hipcx_binary_sa': (_INT, [_INT, _S, _A, _A, _V]),
     'hipcx_fmod': (_INT, [_A, _A, _A, _V]),
     'hipcx_arctan2': (_INT, [_A, _A, _A, _V]),
     'hipcx_where': (_INT, [_A, _A, _A, _A, _V]),

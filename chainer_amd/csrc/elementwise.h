@@ -178,7 +178,7 @@ __global__ __launch_bounds__(kEwThreads) void EwKernel(EwArgs<Op::kNumIn + 1> ar
         for (int i = 0; i < NIN; ++i) {
             const char* p = args.ptr[i + 1] + off[u][i + 1];
             if (i == 0) {
-                if (VEC > 1 && args.col_stride[1] != 0) {
+                if (VEC > 1 && args.col_stride[NOPS > 1 ? 1 : 0] != 0) {
                     in0[u] = *reinterpret_cast<const Vec<In0, VEC>*>(p);
                 } else {
                     In0 s = *reinterpret_cast<const In0*>(p);

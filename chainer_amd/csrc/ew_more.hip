@@ -177,6 +177,83 @@ struct FloatBinaryOp {
     }
 };
 
+// FloorDivide / Mod (native/native_device/arithmetic.cc:107-139, 260-295): integers floor towards -inf and give 0 for a zero
+// divisor (Mod also for a zero dividend); floats follow fmod with the sign fixed up (Mod by zero is NaN).
+template <typename C>
+__device__ __forceinline__ C FloorDivideOf(C x, C y) {
+    if constexpr (std::is_same<C, bool>::value) {
+        return x;  // never launched
+    } else if constexpr (std::is_integral<C>::value) {
+        if (y == 0) return 0;
+        if constexpr (std::is_unsigned<C>::value) {
+            return x / y;
+        } else {
+            using W = std::conditional_t<sizeof(C) == 8, int64_t, int32_t>;
+            if (y == C(-1)) return static_cast<C>(W(0) - static_cast<W>(x));  // avoids the trapping lowest / -1
+            W q = static_cast<W>(x) / static_cast<W>(y), r = static_cast<W>(x) % static_cast<W>(y);
+            return static_cast<C>(q - ((y >= 0 ? r : -r) < 0 ? 1 : 0));
+        }
+    } else {
+        C rem = std::is_same<C, float>::value ? fmodf(x, y) : fmod(x, y);
+        return (x - rem) / y - (((rem < 0 && y > 0) || (rem > 0 && y < 0)) ? C(1) : C(0));
+    }
+}
+
+template <typename C>
+__device__ __forceinline__ C ModOf(C x, C y) {
+    if constexpr (std::is_same<C, bool>::value) {
+        return x;  // never launched
+    } else if constexpr (std::is_integral<C>::value) {
+        if (x == 0 || y == 0) return 0;
+        if constexpr (std::is_unsigned<C>::value) {
+            return x % y;
+        } else {
+            if (y == C(-1)) return 0;
+            int64_t r = static_cast<int64_t>(x) % static_cast<int64_t>(y);
+            if ((r > 0 && y < 0) || (r < 0 && y > 0)) r += y;
+            return static_cast<C>(r);
+        }
+    } else {
+        if (y == C(0)) return static_cast<C>(__builtin_nanf(""));
+        C r = std::is_same<C, float>::value ? fmodf(x, y) : fmod(x, y);
+        if ((r > 0 && y < 0) || (r < 0 && y > 0)) return y + r;
+        return r;
+    }
+}
+
+// op: hipcx_binary_op; kind 0: array op array, 1: array op scalar, 2: scalar op array
+template <typename T, int OP, int KIND>
+struct BinaryCodeOp {
+    using In = T;
+    using Out = T;
+    static constexpr int kNumIn = KIND == 0 ? 2 : 1;
+    static constexpr bool kNeedsIndex = false;
+    compute_t<T> scalar;
+    __device__ __forceinline__ compute_t<T> operator()(compute_t<T> a, compute_t<T> b, compute_t<T>, compute_t<T>, int64_t) const {
+        using C = compute_t<T>;
+        const C x = KIND == 2 ? scalar : a;
+        const C y = KIND == 0 ? b : (KIND == 1 ? scalar : a);
+        if constexpr (OP == HIPCX_BINARY_FLOOR_DIVIDE) {
+            return FloorDivideOf<C>(x, y);
+        } else if constexpr (OP == HIPCX_BINARY_MOD) {
+            return ModOf<C>(x, y);
+        } else if constexpr (std::is_integral<C>::value) {
+            if constexpr (OP == HIPCX_BINARY_BITWISE_AND) return static_cast<C>(x & y);
+            if constexpr (OP == HIPCX_BINARY_BITWISE_OR) return static_cast<C>(x | y);
+            if constexpr (OP == HIPCX_BINARY_BITWISE_XOR) return static_cast<C>(x ^ y);
+            // shifts run in the promoted type (int for the narrow types), as `x1 << x2` does in C++; counts outside
+            // [0, width) are undefined there and masked here
+            using W = std::conditional_t<sizeof(C) == 8, int64_t, int32_t>;
+            using UW = std::make_unsigned_t<W>;
+            const int cnt = static_cast<int>(y) & (sizeof(W) * 8 - 1);
+            if constexpr (OP == HIPCX_BINARY_LEFT_SHIFT) return static_cast<C>(static_cast<UW>(static_cast<W>(x)) << cnt);
+            if constexpr (OP == HIPCX_BINARY_RIGHT_SHIFT) return static_cast<C>(static_cast<W>(x) >> cnt);
+        } else {
+            return x;  // bitwise ops and shifts on floats are rejected on the host
+        }
+    }
+};
+
 // Where: out = condition ? x : y (CX/native/native_device/indexing.cc:173-236); x and/or y may be scalars.
 // kind 0: AAA, 1: AAS (y scalar), 2: ASA (x scalar), 3: ASS.
 template <typename T, int KIND>
@@ -205,6 +282,51 @@ void RunUnaryOp(const hipcx_array* x, const hipcx_array* out, void* stream, Visi
     });
 }
 
+}  // namespace
+}  // namespace hipcx
+
+namespace hipcx {
+namespace {
+void CheckBinaryDtype(int op, int dtype) {
+    switch (op) {
+        case HIPCX_BINARY_FLOOR_DIVIDE:
+        case HIPCX_BINARY_MOD:
+            HIPCX_REQUIRE(dtype != HIPCX_BOOL, HIPCX_DTYPE_ERROR, "bool dtype is not supported by this kernel");
+            break;
+        case HIPCX_BINARY_BITWISE_AND:
+        case HIPCX_BINARY_BITWISE_OR:
+        case HIPCX_BINARY_BITWISE_XOR:
+            HIPCX_REQUIRE(!IsFloatDtype(dtype), HIPCX_DTYPE_ERROR, "Bitwise operations don't support Float types");
+            break;
+        case HIPCX_BINARY_LEFT_SHIFT:
+        case HIPCX_BINARY_RIGHT_SHIFT:
+            HIPCX_REQUIRE(!IsFloatDtype(dtype) && dtype != HIPCX_BOOL, HIPCX_DTYPE_ERROR, "Shift operations don't support Float or Bool types");
+            break;
+        default: throw Error(HIPCX_CHAINERX_ERROR, "unknown binary op code " + std::to_string(op));
+    }
+}
+
+template <int KIND>
+void RunBinaryCode(int op, const EwPlan& p, int dtype, const hipcx_scalar* scalar, hipStream_t stream) {
+    CheckBinaryDtype(op, dtype);
+    VisitDtype(dtype, [&](auto tag) {
+        using T = typename decltype(tag)::type;
+        auto launch = [&](auto opc) {
+            BinaryCodeOp<T, decltype(opc)::value, KIND> f;
+            f.scalar = scalar != nullptr ? static_cast<compute_t<T>>(ScalarTo<T>(*scalar)) : compute_t<T>{};
+            LaunchElementwise(p, f, stream);
+        };
+        switch (op) {
+            case HIPCX_BINARY_FLOOR_DIVIDE: launch(std::integral_constant<int, HIPCX_BINARY_FLOOR_DIVIDE>{}); break;
+            case HIPCX_BINARY_MOD: launch(std::integral_constant<int, HIPCX_BINARY_MOD>{}); break;
+            case HIPCX_BINARY_BITWISE_AND: launch(std::integral_constant<int, HIPCX_BINARY_BITWISE_AND>{}); break;
+            case HIPCX_BINARY_BITWISE_OR: launch(std::integral_constant<int, HIPCX_BINARY_BITWISE_OR>{}); break;
+            case HIPCX_BINARY_BITWISE_XOR: launch(std::integral_constant<int, HIPCX_BINARY_BITWISE_XOR>{}); break;
+            case HIPCX_BINARY_LEFT_SHIFT: launch(std::integral_constant<int, HIPCX_BINARY_LEFT_SHIFT>{}); break;
+            default: launch(std::integral_constant<int, HIPCX_BINARY_RIGHT_SHIFT>{}); break;
+        }
+    });
+}
 }  // namespace
 }  // namespace hipcx
 
@@ -320,6 +442,31 @@ int hipcx_power_sa(hipcx_scalar x1, const hipcx_array* x2, const hipcx_array* ou
             op.scalar = static_cast<compute_t<T>>(ScalarTo<T>(x1));
             LaunchElementwise(p, op, AsStream(stream));
         });
+    });
+}
+
+int hipcx_binary(int op, const hipcx_array* x1, const hipcx_array* x2, const hipcx_array* out, void* stream) {
+    return Guard([&] {
+        EwPlan p = MakeEwPlan({out, x1, x2});
+        HIPCX_REQUIRE(x1->dtype == out->dtype && x2->dtype == out->dtype, HIPCX_DTYPE_ERROR,
+                      "operand dtype differs from out dtype (cast with hipcx_copy first)");
+        RunBinaryCode<0>(op, p, out->dtype, nullptr, AsStream(stream));
+    });
+}
+
+int hipcx_binary_as(int op, const hipcx_array* x1, hipcx_scalar x2, const hipcx_array* out, void* stream) {
+    return Guard([&] {
+        EwPlan p = MakeEwPlan({out, x1});
+        HIPCX_REQUIRE(x1->dtype == out->dtype, HIPCX_DTYPE_ERROR, "x1 dtype differs from out dtype (cast with hipcx_copy first)");
+        RunBinaryCode<1>(op, p, out->dtype, &x2, AsStream(stream));
+    });
+}
+
+int hipcx_binary_sa(int op, hipcx_scalar x1, const hipcx_array* x2, const hipcx_array* out, void* stream) {
+    return Guard([&] {
+        EwPlan p = MakeEwPlan({out, x2});
+        HIPCX_REQUIRE(x2->dtype == out->dtype, HIPCX_DTYPE_ERROR, "x2 dtype differs from out dtype (cast with hipcx_copy first)");
+        RunBinaryCode<2>(op, p, out->dtype, &x1, AsStream(stream));
     });
 }
 

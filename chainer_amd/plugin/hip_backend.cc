@@ -37,6 +37,7 @@
 #include "chainerx/error.h"
 #include "chainerx/kernel_registry.h"
 #include "chainerx/kernels/arithmetic.h"
+#include "chainerx/kernels/binary.h"
 #include "chainerx/kernels/connection.h"
 #include "chainerx/kernels/creation.h"
 #include "chainerx/kernels/explog.h"
@@ -515,6 +516,65 @@ public:
     }
 };
 HIPCX_REGISTER_KERNEL(PowerSAKernel, HipPowerSAKernel)
+
+// FloorDivide / Mod / bitwise / shift families: (x1, x2, out), (x1, Scalar, out), (Scalar, x2, out) with an op code
+#define HIPCX_BINARY_CODE_KERNEL(Name, code)                                              \
+    class Hip##Name##Kernel : public Name##Kernel {                                       \
+    public:                                                                               \
+        void Call(const Array& x1, const Array& x2, const Array& out) override {          \
+            Device& device = x1.device();                                                 \
+            device.CheckDevicesCompatible(x1, x2, out);                                   \
+            SetDeviceScope scope{device.index()};                                         \
+            hipcx_array a = ToC(Cast(x1, out.dtype())), b = ToC(Cast(x2, out.dtype())), o = ToC(out); \
+            Check(hipcx_binary(code, &a, &b, &o, nullptr));                               \
+        }                                                                                 \
+    };                                                                                    \
+    HIPCX_REGISTER_KERNEL(Name##Kernel, Hip##Name##Kernel)
+
+#define HIPCX_BINARY_CODE_AS_KERNEL(Name, code)                                           \
+    class Hip##Name##Kernel : public Name##Kernel {                                       \
+    public:                                                                               \
+        void Call(const Array& x1, Scalar x2, const Array& out) override {                \
+            Device& device = x1.device();                                                 \
+            device.CheckDevicesCompatible(x1, out);                                       \
+            SetDeviceScope scope{device.index()};                                         \
+            hipcx_array a = ToC(Cast(x1, out.dtype())), o = ToC(out);                     \
+            Check(hipcx_binary_as(code, &a, ToC(x2), &o, nullptr));                       \
+        }                                                                                 \
+    };                                                                                    \
+    HIPCX_REGISTER_KERNEL(Name##Kernel, Hip##Name##Kernel)
+
+#define HIPCX_BINARY_CODE_SA_KERNEL(Name, code)                                           \
+    class Hip##Name##Kernel : public Name##Kernel {                                       \
+    public:                                                                               \
+        void Call(Scalar x1, const Array& x2, const Array& out) override {                \
+            Device& device = x2.device();                                                 \
+            device.CheckDevicesCompatible(x2, out);                                       \
+            SetDeviceScope scope{device.index()};                                         \
+            hipcx_array b = ToC(Cast(x2, out.dtype())), o = ToC(out);                     \
+            Check(hipcx_binary_sa(code, ToC(x1), &b, &o, nullptr));                       \
+        }                                                                                 \
+    };                                                                                    \
+    HIPCX_REGISTER_KERNEL(Name##Kernel, Hip##Name##Kernel)
+
+HIPCX_BINARY_CODE_KERNEL(FloorDivide, HIPCX_BINARY_FLOOR_DIVIDE)
+HIPCX_BINARY_CODE_AS_KERNEL(FloorDivideAS, HIPCX_BINARY_FLOOR_DIVIDE)
+HIPCX_BINARY_CODE_SA_KERNEL(FloorDivideSA, HIPCX_BINARY_FLOOR_DIVIDE)
+HIPCX_BINARY_CODE_KERNEL(ModAA, HIPCX_BINARY_MOD)
+HIPCX_BINARY_CODE_AS_KERNEL(ModAS, HIPCX_BINARY_MOD)
+HIPCX_BINARY_CODE_SA_KERNEL(ModSA, HIPCX_BINARY_MOD)
+HIPCX_BINARY_CODE_KERNEL(BitwiseAnd, HIPCX_BINARY_BITWISE_AND)
+HIPCX_BINARY_CODE_AS_KERNEL(BitwiseAndAS, HIPCX_BINARY_BITWISE_AND)
+HIPCX_BINARY_CODE_KERNEL(BitwiseOr, HIPCX_BINARY_BITWISE_OR)
+HIPCX_BINARY_CODE_AS_KERNEL(BitwiseOrAS, HIPCX_BINARY_BITWISE_OR)
+HIPCX_BINARY_CODE_KERNEL(BitwiseXor, HIPCX_BINARY_BITWISE_XOR)
+HIPCX_BINARY_CODE_AS_KERNEL(BitwiseXorAS, HIPCX_BINARY_BITWISE_XOR)
+HIPCX_BINARY_CODE_KERNEL(LeftShiftAA, HIPCX_BINARY_LEFT_SHIFT)
+HIPCX_BINARY_CODE_AS_KERNEL(LeftShiftAS, HIPCX_BINARY_LEFT_SHIFT)
+HIPCX_BINARY_CODE_SA_KERNEL(LeftShiftSA, HIPCX_BINARY_LEFT_SHIFT)
+HIPCX_BINARY_CODE_KERNEL(RightShiftAA, HIPCX_BINARY_RIGHT_SHIFT)
+HIPCX_BINARY_CODE_AS_KERNEL(RightShiftAS, HIPCX_BINARY_RIGHT_SHIFT)
+HIPCX_BINARY_CODE_SA_KERNEL(RightShiftSA, HIPCX_BINARY_RIGHT_SHIFT)
 
 // Where: the condition is cast to bool, x / y to out's dtype (native/native_device/indexing.cc:194-283)
 class HipWhereKernel : public WhereKernel {

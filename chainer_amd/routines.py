@@ -634,6 +634,81 @@ def arctan2(x1, x2):
     return _binary('hipcx_arctan2', x1, x2, _math_result_dtype(result_type(x1, x2)))
 
 
+_BINARY_CODES = {'floor_divide': 1, 'mod': 2, 'bitwise_and': 3, 'bitwise_or': 4, 'bitwise_xor': 5, 'left_shift': 6, 'right_shift': 7}
+
+
+def _binary_code(name, x1, x2, dtype):
+    """array op array (broadcast), array op scalar, scalar op array through hipcx_binary / _as / _sa."""
+    code = _BINARY_CODES[name]
+    if _is_scalar(x2):
+        out = ndarray.empty(x1.shape, dtype)
+        _lib.call('hipcx_binary_as', code, x1.astype(dtype, False).desc(), _lib.make_scalar(x2), out.desc(), current_stream())
+        return out
+    if _is_scalar(x1):
+        out = ndarray.empty(x2.shape, dtype)
+        _lib.call('hipcx_binary_sa', code, _lib.make_scalar(x1), x2.astype(dtype, False).desc(), out.desc(), current_stream())
+        return out
+    shape = _broadcast_shape(x1.shape, x2.shape)
+    out = ndarray.empty(shape, dtype)
+    _lib.call('hipcx_binary', code, x1.broadcast_to(shape).astype(dtype, False).desc(), x2.broadcast_to(shape).astype(dtype, False).desc(),
+              out.desc(), current_stream())
+    return out
+
+
+def floor_divide(x1, x2):
+    """FloorDivide (CX/routines/arithmetic.cc:305-311)."""
+    return _binary_code('floor_divide', x1, x2, _arithmetic_dtype(x1, x2))
+
+
+def mod(x1, x2):
+    """Mod (CX/routines/arithmetic.cc:568-572)."""
+    return _binary_code('mod', x1, x2, _arithmetic_dtype(x1, x2))
+
+
+remainder = mod
+
+
+def _operand_kind(x):
+    return _kind(_scalar_default_dtype(x)) if _is_scalar(x) else _kind(x.dtype)
+
+
+def _bitwise(name, x1, x2):
+    """BitwiseAnd / Or / Xor (CX/routines/binary.cc:19-23,125-159): float operands are refused; Scalar op Array swaps."""
+    if _operand_kind(x1) == 3 or _operand_kind(x2) == 3:
+        raise _lib.DtypeError("Bitwise operations don't support Float types")
+    if _is_scalar(x1):
+        x1, x2 = x2, x1
+    return _binary_code(name, x1, x2, result_type(x1, x2))
+
+
+def bitwise_and(x1, x2):
+    return _bitwise('bitwise_and', x1, x2)
+
+
+def bitwise_or(x1, x2):
+    return _bitwise('bitwise_or', x1, x2)
+
+
+def bitwise_xor(x1, x2):
+    return _bitwise('bitwise_xor', x1, x2)
+
+
+def _shift(name, x1, x2):
+    """LeftShift / RightShift (CX/routines/binary.cc:32-36,161-189): integer operands only; the result has x1's dtype,
+    int64 when x1 is a scalar."""
+    if _operand_kind(x1) in (0, 3) or _operand_kind(x2) in (0, 3):
+        raise _lib.DtypeError("Shift operations don't support Float or Bool types")
+    return _binary_code(name, x1, x2, numpy.dtype('int64') if _is_scalar(x1) else x1.dtype)
+
+
+def left_shift(x1, x2):
+    return _shift('left_shift', x1, x2)
+
+
+def right_shift(x1, x2):
+    return _shift('right_shift', x1, x2)
+
+
 def where(condition, x, y):
     """Where (CX/routines/indexing.cc:207-298): out dtype = ResultType(x, y); a non-bool condition is cast to bool."""
     cond = condition.astype('bool', False)

@@ -165,6 +165,23 @@ int hipcx_power_sa(hipcx_scalar x1, const hipcx_array* x2, const hipcx_array* ou
 int hipcx_fmod(const hipcx_array* x1, const hipcx_array* x2, const hipcx_array* out, void* stream);
 int hipcx_arctan2(const hipcx_array* x1, const hipcx_array* x2, const hipcx_array* out, void* stream);
 
+/* Integer-flavoured binary kernels, operands and out of one dtype; _as takes x2 as a scalar, _sa takes x1 as a scalar:
+ *   FloorDivideKernel arithmetic.h:41, FloorDivideASKernel :46, FloorDivideSAKernel :51 and ModAAKernel :86, ModASKernel :93,
+ *   ModSAKernel :100 -- numeric dtypes; integers round towards -inf and give 0 for a zero divisor, float Mod by zero is NaN
+ *   (native/native_device/arithmetic.cc:107-139, 260-295);
+ *   BitwiseAndKernel binary.h:11, BitwiseAndASKernel :16, BitwiseOrKernel :21, BitwiseOrASKernel :26, BitwiseXorKernel :31,
+ *   BitwiseXorASKernel :36 -- bool and integer dtypes;
+ *   LeftShiftAAKernel binary.h:41, LeftShiftASKernel :46, LeftShiftSAKernel :51, RightShiftAAKernel :56, RightShiftASKernel :61,
+ *   RightShiftSAKernel :66 -- integer dtypes, evaluated in the promoted type as `x1 << x2` is in C++; a count outside
+ *   [0, width of the promoted type) is undefined in the reference and is masked to that width here. */
+enum hipcx_binary_op {
+    HIPCX_BINARY_FLOOR_DIVIDE = 1, HIPCX_BINARY_MOD, HIPCX_BINARY_BITWISE_AND, HIPCX_BINARY_BITWISE_OR, HIPCX_BINARY_BITWISE_XOR,
+    HIPCX_BINARY_LEFT_SHIFT, HIPCX_BINARY_RIGHT_SHIFT
+};
+int hipcx_binary(int op, const hipcx_array* x1, const hipcx_array* x2, const hipcx_array* out, void* stream);
+int hipcx_binary_as(int op, const hipcx_array* x1, hipcx_scalar x2, const hipcx_array* out, void* stream);
+int hipcx_binary_sa(int op, hipcx_scalar x1, const hipcx_array* x2, const hipcx_array* out, void* stream);
+
 /* WhereKernel indexing.h:22, WhereAASKernel :27, WhereASAKernel :32, WhereASSKernel :37: out = condition ? x : y with a bool
  * condition array and x / y of out's dtype, arrays or scalars (native/native_device/indexing.cc:194-283). */
 int hipcx_where(const hipcx_array* condition, const hipcx_array* x, const hipcx_array* y, const hipcx_array* out, void* stream);

@@ -289,6 +289,63 @@ def power(x1, x2):
         return out
 
 
+def floor_divide(x1, x2):
+    """native::FloorDivide (native/native_device/arithmetic.cc:107-139): integers floor towards -inf, 0 for a zero divisor;
+    floats (x - fmod(x, y)) / y minus one when the remainder and the divisor disagree in sign; float16 through float."""
+    x1, x2 = np.broadcast_arrays(np.asarray(x1), np.asarray(x2))
+    dt = x1.dtype
+    with np.errstate(all='ignore'):
+        if dt.kind in 'iu':
+            safe = np.where(x2 == 0, 1, x2).astype(dt)
+            return np.where(x2 == 0, 0, np.floor_divide(x1, safe)).astype(dt)
+        ct = np.float32 if dt == np.float16 else dt
+        x, y = x1.astype(ct), x2.astype(ct)
+        rem = np.fmod(x, y)
+        fix = ((rem < 0) & (y > 0)) | ((rem > 0) & (y < 0))
+        return (((x - rem) / y).astype(ct) - fix.astype(ct)).astype(dt)
+
+
+def mod(x1, x2):
+    """Mod (native/native_device/arithmetic.cc:260-295): result takes the divisor's sign; integers give 0 when either operand
+    is 0, floats NaN for a zero divisor; float16 through float."""
+    x1, x2 = np.broadcast_arrays(np.asarray(x1), np.asarray(x2))
+    dt = x1.dtype
+    with np.errstate(all='ignore'):
+        if dt.kind in 'iu':
+            safe = np.where(x2 == 0, 1, x2).astype(dt)
+            return np.where((x1 == 0) | (x2 == 0), 0, np.mod(x1, safe)).astype(dt)
+        ct = np.float32 if dt == np.float16 else dt
+        x, y = x1.astype(ct), x2.astype(ct)
+        r = np.fmod(x, y)
+        fix = ((r > 0) & (y < 0)) | ((r < 0) & (y > 0))
+        r = np.where(fix, (y + r).astype(ct), r)
+        return np.where(y == 0, np.nan, r).astype(dt)
+
+
+def bitwise_and(x1, x2):
+    return np.bitwise_and(np.asarray(x1), np.asarray(x2))
+
+
+def bitwise_or(x1, x2):
+    return np.bitwise_or(np.asarray(x1), np.asarray(x2))
+
+
+def bitwise_xor(x1, x2):
+    return np.bitwise_xor(np.asarray(x1), np.asarray(x2))
+
+
+def left_shift(x1, x2):
+    """`x1 << x2` in the promoted type, narrowed back (counts within the type's width)."""
+    x1, x2 = np.asarray(x1), np.asarray(x2)
+    wide = np.left_shift(x1.astype(np.int64), x2.astype(np.int64))
+    return wide.astype(x1.dtype)
+
+
+def right_shift(x1, x2):
+    x1, x2 = np.asarray(x1), np.asarray(x2)
+    return np.right_shift(x1.astype(np.int64), x2.astype(np.int64)).astype(x1.dtype)
+
+
 def fmod(x1, x2):
     """FmodKernel: std::fmod, float16 through float."""
     x1, x2 = np.asarray(x1), np.asarray(x2)

@@ -222,3 +222,57 @@ def test_amin_argmin_nan_rule():
     assert_exact(chx.amin(X, 1).get(), O.amin(x, 1), 'amin with NaN')
     assert_exact(chx.argmin(X, 1).get(), O.argmin(x, 1), 'argmin with NaN and ties')
     assert np.isnan(chx.amin(X, 1).get()[1])
+
+
+@pytest.mark.parametrize('dt', NUMERIC)
+def test_floor_divide_mod(dt):
+    import chainer_amd as chx
+    rng = np.random.default_rng(29)
+    x, y = rand(rng, (23, 77), dt), rand(rng, (23, 77), dt)
+    y[0, :5] = 0  # zero divisors
+    x[1, :5] = 0
+    X, Y = chx.array(x), chx.array(y)
+    s = 3 if np.dtype(dt).kind != 'f' else 2.5
+    sv = np.asarray(s, dt)
+    with np.errstate(all='ignore'):
+        for name in ('floor_divide', 'mod'):
+            f, g = getattr(chx, name), getattr(O, name)
+            assert_exact(f(X, Y).get(), g(x, y), name)
+            assert_exact(f(X, s).get(), g(x, sv), name + ' AS')
+            assert_exact(f(s, Y).get(), g(sv, y), name + ' SA')
+            assert_exact(f(X.T[::2], Y.T[::2]).get(), g(x.T[::2], y.T[::2]), name + ' views')
+            assert_exact(f(X, Y[:1]).get(), g(x, np.broadcast_to(y[:1], x.shape)), name + ' broadcast')
+    with pytest.raises(chx.DtypeError):
+        chx.floor_divide(chx.array(np.ones(3, bool)), chx.array(np.ones(3, bool)))
+
+
+@pytest.mark.parametrize('dt', ['bool', 'int8', 'int16', 'int32', 'int64', 'uint8'])
+def test_bitwise_and_shifts(dt):
+    import chainer_amd as chx
+    rng = np.random.default_rng(30)
+    x, y = rand(rng, (19, 65), dt), rand(rng, (19, 65), dt)
+    X, Y = chx.array(x), chx.array(y)
+    for name in ('bitwise_and', 'bitwise_or', 'bitwise_xor'):
+        f, g = getattr(chx, name), getattr(O, name)
+        assert_exact(f(X, Y).get(), g(x, y), name)
+        assert_exact(f(X[::2, 1::3], Y[::2, 1::3]).get(), g(x[::2, 1::3], y[::2, 1::3]), name + ' views')
+        sc = True if dt == 'bool' else 5
+        assert_exact(f(X, sc).get(), g(x, np.asarray(sc, dt)), name + ' AS')
+        assert_exact(f(sc, X).get(), g(x, np.asarray(sc, dt)), name + ' SA swaps')
+    with pytest.raises(chx.DtypeError):
+        chx.bitwise_and(chx.array(np.ones(3, 'float32')), chx.array(np.ones(3, 'float32')))
+    if dt == 'bool':
+        with pytest.raises(chx.DtypeError):
+            chx.left_shift(X, Y)
+        return
+    bits = np.dtype(dt).itemsize * 8
+    cnt = rng.integers(0, bits, (19, 65)).astype(dt)
+    Cn = chx.array(cnt)
+    assert_exact(chx.left_shift(X, Cn).get(), O.left_shift(x, cnt), 'left_shift')
+    assert_exact(chx.right_shift(X, Cn).get(), O.right_shift(x, cnt), 'right_shift')
+    assert_exact(chx.left_shift(X, 3).get(), O.left_shift(x, np.asarray(3, dt)), 'left_shift AS')
+    assert_exact(chx.right_shift(X, 2).get(), O.right_shift(x, np.asarray(2, dt)), 'right_shift AS')
+    got = chx.left_shift(3, Cn)  # Scalar << Array is int64
+    assert got.dtype == np.int64
+    assert_exact(got.get(), O.left_shift(np.full(cnt.shape, 3, np.int64), cnt.astype(np.int64)), 'left_shift SA')
+    assert_exact(chx.right_shift(-1000, Cn).get(), O.right_shift(np.full(cnt.shape, -1000, np.int64), cnt.astype(np.int64)), 'right_shift SA')

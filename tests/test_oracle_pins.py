@@ -555,3 +555,25 @@ def test_sign_abs_where_literals():
     assert np.array_equal(O.absolute(np.array([200, 3], np.uint8)), np.array([200, 3], np.uint8))
     assert np.array_equal(O.where(np.array([1, 0, 2]), np.array([1, 2, 3]), 9, 'int32'), np.array([1, 9, 3], np.int32))
     assert np.array_equal(O.logical_xor(np.array([0, 2, 0, 5]), np.array([0, 0, 3, 7])), [False, True, True, False])
+
+
+def test_floor_divide_mod_brute_force():
+    """B: for every pair of int8 values the oracle equals Python's // and % (floor semantics, sign of the divisor), with the
+    reference's conventions for zero operands (native/native_device/arithmetic.cc:107-139, 260-295); floats against
+    math.floor(x / y) and Python's % on exactly representable operands."""
+    a = np.arange(-128, 128, dtype=np.int8)
+    x, y = np.meshgrid(a, a, indexing='ij')
+    keep = ~((x == -128) & (y == -1))  # lowest / -1 overflows in the reference as well
+    xs, ys = x[keep], y[keep]
+    fd = np.array([0 if q == 0 else p // q for p, q in zip(xs.tolist(), ys.tolist())], np.int8)
+    md = np.array([0 if (p == 0 or q == 0) else p % q for p, q in zip(xs.tolist(), ys.tolist())], np.int8)
+    assert np.array_equal(O.floor_divide(xs, ys), fd)
+    assert np.array_equal(O.mod(xs, ys), md)
+    u = np.arange(0, 256, dtype=np.uint8)
+    ux, uy = [v.reshape(-1) for v in np.meshgrid(u, u, indexing='ij')]
+    assert np.array_equal(O.floor_divide(ux, uy), np.array([0 if q == 0 else p // q for p, q in zip(ux.tolist(), uy.tolist())], np.uint8))
+    f = np.array([-7.5, -3.0, -0.5, 0.0, 0.5, 2.25, 7.0, 10.75], np.float32)
+    fx, fy = [v.reshape(-1) for v in np.meshgrid(f, f[f != 0], indexing='ij')]
+    assert np.array_equal(O.floor_divide(fx, fy), np.array([np.floor(p / q) for p, q in zip(fx.tolist(), fy.tolist())], np.float32))
+    assert np.array_equal(O.mod(fx, fy), np.array([p % q for p, q in zip(fx.tolist(), fy.tolist())], np.float32))
+    assert np.isnan(O.mod(np.float32([1.0]), np.float32([0.0]))[0])
