@@ -156,6 +156,13 @@ SIGNATURES = {
     'hipcx_where_aas': (_INT, [_A, _A, _S, _A, _V]),
     'hipcx_where_asa': (_INT, [_A, _S, _A, _A, _V]),
     'hipcx_where_ass': (_INT, [_A, _S, _S, _A, _V]),
+    'hipcx_add_at': (_INT, [_A, _A, ctypes.c_int8, _A, _A, _INT, ctypes.POINTER(ctypes.c_int32), _V]),
+    'hipcx_identity': (_INT, [_A, _V]),
+    'hipcx_eye': (_INT, [ctypes.c_int64, _A, _V]),
+    'hipcx_tri': (_INT, [ctypes.c_int64, _A, _V]),
+    'hipcx_linspace': (_INT, [ctypes.c_double, ctypes.c_double, _A, _V]),
+    'hipcx_diagflat': (_INT, [_A, ctypes.c_int64, _A, _V]),
+    'hipcx_cumsum': (_INT, [_A, ctypes.c_int8, _A, _V]),
     'hipcx_log_softmax_workspace_size': (_SZ, [_A]),
     'hipcx_log_softmax': (_INT, [_A, _A, _V, _SZ, _V]),
     'hipcx_lstm_cell': (_INT, [_A, _A, _A, _A, _V]),

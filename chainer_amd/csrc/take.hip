@@ -99,6 +99,39 @@ __global__ __launch_bounds__(256) void TakeKernel(TakeArgs t) {
     }
 }
 
+// AddAt: out[l..., index[i...], r...] += b[l..., i..., r...] on top of a copy of `a` (indexing.cc:107-190).  One thread
+// owns one (l, r) position and walks the indices in C order, so contributions to the same element are added in the
+// reference's order (float results are bit-identical; float16 rounds after every addition, as Float16::operator+= does).
+// In TakeArgs terms: `a` is the accumulated array (with the axis), `out` is b (with the index axes).
+template <typename T>
+__global__ __launch_bounds__(256) void AddAtKernel(TakeArgs t) {
+    const int64_t w = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (w >= t.total) return;
+    const int64_t r = w % t.right.total;
+    const int64_t l = w / t.right.total;
+    int64_t acc_off = 0, b_off = 0;
+    Decompose(t.left, l, acc_off, b_off);
+    Decompose(t.right, r, acc_off, b_off);
+    char* acc_base = const_cast<char*>(t.a) + acc_off;
+    for (int64_t i = 0; i < t.index.total; ++i) {
+        int64_t ioff = 0, bo = b_off;
+        Decompose(t.index, i, ioff, bo);
+        const int64_t index = ResolveIndex(LoadIndex(t.idx + ioff, t.idx_dtype), t.axis_dim, t.mode, t.error_flag);
+        T* dst = reinterpret_cast<T*>(acc_base + index * t.axis_stride);
+        const T bv = *reinterpret_cast<const T*>(t.out + bo);
+        if constexpr (std::is_same<T, bool>::value) {
+            *dst = *dst || bv;
+        } else if constexpr (std::is_same<T, half_t>::value) {
+            *dst = static_cast<half_t>(static_cast<float>(*dst) + static_cast<float>(bv));
+        } else if constexpr (std::is_integral<T>::value) {
+            using U = std::make_unsigned_t<T>;
+            *dst = static_cast<T>(static_cast<U>(static_cast<U>(*dst) + static_cast<U>(bv)));
+        } else {
+            *dst = *dst + bv;
+        }
+    }
+}
+
 bool DenseGroup(const DimGroup& g, const int64_t* strides, int64_t itemsize) {
     int64_t expect = itemsize;
     for (int d = g.n - 1; d >= 0; --d) {
@@ -193,5 +226,71 @@ extern "C" int hipcx_take(const hipcx_array* a, const hipcx_array* indices, int8
             default: hipLaunchKernelGGL((TakeKernel<8, false>), grid, block, 0, st, t); break;
         }
         CheckLaunch("take");
+    });
+}
+
+
+extern "C" int hipcx_copy(const hipcx_array* a, const hipcx_array* out, void* stream);
+
+extern "C" int hipcx_add_at(const hipcx_array* a, const hipcx_array* indices, int8_t axis, const hipcx_array* b, const hipcx_array* out, int mode,
+                            int32_t* error_flag, void* stream) {
+    int st = hipcx_copy(a, out, stream);  // out starts as a copy of a (same dtype: checked below before anything is added)
+    if (st != HIPCX_OK) return st;
+    return Guard([&] {
+        ValidateArray(indices, "indices");
+        ValidateArray(b, "b");
+        HIPCX_REQUIRE(axis >= 0 && axis < a->ndim, HIPCX_DIMENSION_ERROR, "add_at: axis out of range");
+        HIPCX_REQUIRE(indices->dtype == HIPCX_INT8 || indices->dtype == HIPCX_INT16 || indices->dtype == HIPCX_INT32 ||
+                              indices->dtype == HIPCX_INT64 || indices->dtype == HIPCX_UINT8,
+                      HIPCX_DTYPE_ERROR, "Only arrays of integer dtype can be used as indices.");
+        HIPCX_REQUIRE(out->dtype == a->dtype && b->dtype == a->dtype, HIPCX_DTYPE_ERROR, "add_at: a, b and out must share a dtype");
+        HIPCX_REQUIRE(mode >= HIPCX_BOUNDS_DEFAULT && mode <= HIPCX_BOUNDS_CLIP, HIPCX_CHAINERX_ERROR, "add_at: invalid bounds mode");
+        HIPCX_REQUIRE(SameShape(a, out), HIPCX_DIMENSION_ERROR, "add_at: out must have a's shape");
+        HIPCX_REQUIRE(b->ndim == a->ndim - 1 + indices->ndim, HIPCX_DIMENSION_ERROR, "add_at: b has the wrong number of dimensions");
+        TakeArgs t{};
+        t.a = static_cast<const char*>(out->data);
+        t.idx = static_cast<const char*>(indices->data);
+        t.out = static_cast<char*>(b->data);
+        t.axis_dim = out->shape[axis];
+        t.axis_stride = out->strides[axis];
+        t.idx_dtype = indices->dtype;
+        t.mode = mode;
+        t.error_flag = error_flag;
+        t.left.total = t.index.total = t.right.total = 1;
+        int o = 0;
+        for (int d = 0; d < axis; ++d, ++o) {
+            HIPCX_REQUIRE(b->shape[o] == out->shape[d], HIPCX_DIMENSION_ERROR, "add_at: b has the wrong shape");
+            t.left.shape[t.left.n] = out->shape[d];
+            t.left.stride_a[t.left.n] = out->strides[d];
+            t.left.stride_o[t.left.n] = b->strides[o];
+            t.left.total *= out->shape[d];
+            ++t.left.n;
+        }
+        for (int d = 0; d < indices->ndim; ++d, ++o) {
+            HIPCX_REQUIRE(b->shape[o] == indices->shape[d], HIPCX_DIMENSION_ERROR, "add_at: b has the wrong shape");
+            t.index.shape[t.index.n] = indices->shape[d];
+            t.index.stride_a[t.index.n] = indices->strides[d];
+            t.index.stride_o[t.index.n] = b->strides[o];
+            t.index.total *= indices->shape[d];
+            ++t.index.n;
+        }
+        for (int d = axis + 1; d < out->ndim; ++d, ++o) {
+            HIPCX_REQUIRE(b->shape[o] == out->shape[d], HIPCX_DIMENSION_ERROR, "add_at: b has the wrong shape");
+            t.right.shape[t.right.n] = out->shape[d];
+            t.right.stride_a[t.right.n] = out->strides[d];
+            t.right.stride_o[t.right.n] = b->strides[o];
+            t.right.total *= out->shape[d];
+            ++t.right.n;
+        }
+        t.total = t.left.total * t.right.total;
+        if (t.total == 0 || t.index.total == 0) return;
+        HIPCX_REQUIRE(t.axis_dim > 0, HIPCX_INDEX_ERROR, "add_at: cannot index an axis of extent 0");
+        HIPCX_REQUIRE((t.total + 255) / 256 < (1LL << 31), HIPCX_NOT_IMPLEMENTED_ERROR, "add_at: problem too large for one launch");
+        dim3 grid(static_cast<unsigned>((t.total + 255) / 256)), block(256);
+        VisitDtype(out->dtype, [&](auto tag) {
+            using T = typename decltype(tag)::type;
+            hipLaunchKernelGGL(AddAtKernel<T>, grid, block, 0, AsStream(stream), t);
+        });
+        CheckLaunch("add_at");
     });
 }

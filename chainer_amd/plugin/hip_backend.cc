@@ -852,6 +852,108 @@ public:
 };
 HIPCX_REGISTER_KERNEL(TakeKernel, HipTakeKernel)
 
+int ToC(IndexBoundsMode mode) {
+    switch (mode) {
+        case IndexBoundsMode::kRaise: return HIPCX_BOUNDS_RAISE;
+        case IndexBoundsMode::kWrap: return HIPCX_BOUNDS_WRAP;
+        case IndexBoundsMode::kClip: return HIPCX_BOUNDS_CLIP;
+        default: return HIPCX_BOUNDS_DEFAULT;
+    }
+}
+
+class HipAddAtKernel : public AddAtKernel {
+public:
+    void Call(const Array& a, const Array& indices, int8_t axis, const Array& b, const Array& out, IndexBoundsMode mode) override {
+        Device& device = a.device();
+        device.CheckDevicesCompatible(a, indices, b, out);
+        SetDeviceScope scope{device.index()};
+        hipcx_array ca = ToC(a), ci = ToC(indices), cb = ToC(Cast(b, a.dtype())), co = ToC(out);
+        int m = ToC(mode);
+        bool checks = m == HIPCX_BOUNDS_DEFAULT || m == HIPCX_BOUNDS_RAISE;
+        std::shared_ptr<void> flag = checks ? device.Allocate(sizeof(int32_t)) : nullptr;
+        if (checks) CheckHip(hipMemsetAsync(flag.get(), 0, sizeof(int32_t), nullptr), "hipMemsetAsync");
+        Check(hipcx_add_at(&ca, &ci, axis, &cb, &co, m, static_cast<int32_t*>(flag.get()), nullptr));
+        if (checks) {
+            int32_t host = 0;
+            CheckHip(hipMemcpy(&host, flag.get(), sizeof(int32_t), hipMemcpyDeviceToHost), "hipMemcpy");
+            if (host != 0) throw IndexError{"Index is out of bounds for axis ", static_cast<int>(axis), " with size ", a.shape()[axis]};
+        }
+    }
+};
+HIPCX_REGISTER_KERNEL(AddAtKernel, HipAddAtKernel)
+
+// ---- creation patterns, Cumsum, Nansum ----
+class HipIdentityKernel : public IdentityKernel {
+public:
+    void Call(const Array& out) override {
+        SetDeviceScope scope{out.device().index()};
+        hipcx_array o = ToC(out);
+        Check(hipcx_identity(&o, nullptr));
+    }
+};
+HIPCX_REGISTER_KERNEL(IdentityKernel, HipIdentityKernel)
+
+class HipEyeKernel : public EyeKernel {
+public:
+    void Call(int64_t k, const Array& out) override {
+        SetDeviceScope scope{out.device().index()};
+        hipcx_array o = ToC(out);
+        Check(hipcx_eye(k, &o, nullptr));
+    }
+};
+HIPCX_REGISTER_KERNEL(EyeKernel, HipEyeKernel)
+
+class HipTriKernel : public TriKernel {
+public:
+    void Call(int64_t k, const Array& out) override {
+        SetDeviceScope scope{out.device().index()};
+        hipcx_array o = ToC(out);
+        Check(hipcx_tri(k, &o, nullptr));
+    }
+};
+HIPCX_REGISTER_KERNEL(TriKernel, HipTriKernel)
+
+class HipLinspaceKernel : public LinspaceKernel {
+public:
+    void Call(double start, double stop, const Array& out) override {
+        SetDeviceScope scope{out.device().index()};
+        hipcx_array o = ToC(out);
+        Check(hipcx_linspace(start, stop, &o, nullptr));
+    }
+};
+HIPCX_REGISTER_KERNEL(LinspaceKernel, HipLinspaceKernel)
+
+class HipDiagflatKernel : public DiagflatKernel {
+public:
+    void Call(const Array& v, int64_t k, const Array& out) override {
+        Device& device = v.device();
+        device.CheckDevicesCompatible(v, out);
+        SetDeviceScope scope{device.index()};
+        hipcx_array cv = ToC(v), o = ToC(out);
+        Check(hipcx_diagflat(&cv, k, &o, nullptr));
+    }
+};
+HIPCX_REGISTER_KERNEL(DiagflatKernel, HipDiagflatKernel)
+
+class HipCumsumKernel : public CumsumKernel {
+public:
+    void Call(const Array& a, int8_t axis, const Array& out) override {
+        Device& device = a.device();
+        device.CheckDevicesCompatible(a, out);
+        SetDeviceScope scope{device.index()};
+        hipcx_array ca = ToC(a), o = ToC(out);
+        Check(hipcx_cumsum(&ca, axis, &o, nullptr));
+    }
+};
+HIPCX_REGISTER_KERNEL(CumsumKernel, HipCumsumKernel)
+
+// the routine has already replaced NaNs by zeros (CX/routines/reduction.cc:151); the native NansumKernel is its SumKernel
+class HipNansumKernel : public NansumKernel {
+public:
+    void Call(const Array& a, const Axes& axis, const Array& out) override { CallReduce(hipcx_sum, a, axis, out); }
+};
+HIPCX_REGISTER_KERNEL(NansumKernel, HipNansumKernel)
+
 }  // namespace
 }  // namespace hip
 }  // namespace chainerx

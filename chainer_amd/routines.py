@@ -125,6 +125,80 @@ def arange(start, stop=None, step=1, dtype=None):
     return out
 
 
+def identity(n, dtype='float32'):
+    """Identity (CX/routines/creation.cc:178-189)."""
+    if n < 0:
+        raise _lib.DimensionError('Negative dimensions are not allowed')
+    out = ndarray.empty((n, n), dtype)
+    if n:
+        _lib.call('hipcx_identity', out.desc(), current_stream())
+    return out
+
+
+def eye(n, m=None, k=0, dtype='float64'):
+    """Eye (CX/routines/creation.cc:191-211)."""
+    m = n if m is None else m
+    if n < 0 or m < 0:
+        raise _lib.DimensionError('Negative dimensions are not allowed')
+    out = ndarray.empty((n, m), dtype)
+    if n * m:
+        _lib.call('hipcx_eye', int(k or 0), out.desc(), current_stream())
+    return out
+
+
+def tri(n, m=None, k=0, dtype='float32'):
+    """Tri (CX/routines/creation.cc:410-432)."""
+    m = n if m is None else m
+    if n < 0 or m < 0:
+        raise _lib.DimensionError('Negative dimensions are not allowed')
+    out = ndarray.empty((n, m), dtype)
+    if n * m:
+        _lib.call('hipcx_tri', int(k or 0), out.desc(), current_stream())
+    return out
+
+
+def linspace(start, stop, num=50, endpoint=True, dtype='float32'):
+    """Linspace (CX/routines/creation.cc:313-339)."""
+    if num < 0:
+        raise _lib.ChainerxError('Number of samples, %d, must be non-negative' % num)
+    out = ndarray.empty((num,), dtype)
+    if num > 0:
+        a, b = float(start), float(stop)
+        if not endpoint:
+            b = a + (b - a) * (num - 1) / num
+        _lib.call('hipcx_linspace', a, b, out.desc(), current_stream())
+    return out
+
+
+def diag(v, k=0):
+    """Diag (CX/routines/creation.cc:260-293): a 1-D v becomes the k-th diagonal of a square matrix; a 2-D v gives a view
+    of its k-th diagonal."""
+    if v.ndim == 1:
+        n = v.shape[0] + abs(k)
+        out = ndarray.empty((n, n), v.dtype)
+        if n:
+            _lib.call('hipcx_diagflat', v.desc(), int(k), out.desc(), current_stream())
+        return out
+    if v.ndim == 2:
+        rows, cols = v.shape
+        n = _py.min(rows, cols)
+        if k >= 0:
+            offset = k * v.strides[1]
+            if cols <= k + n - 1:
+                n = _py.max(0, cols - k)
+        else:
+            offset = -k * v.strides[0]
+            if rows <= -k + n - 1:
+                n = _py.max(0, rows + k)
+        return ndarray(v._buf, v._offset + offset, (n,), (v.strides[0] + v.strides[1],), v.dtype)
+    raise _lib.DimensionError('Input must be 1D or 2D.')
+
+
+def diagflat(v, k=0):
+    """Diagflat (CX/routines/creation.cc:307-310)."""
+    return diag(v.reshape((_prod(v.shape),)), k)
+
+
 def copy(a):
     return a.copy()
 
@@ -839,6 +913,25 @@ def any(a, axis=None, keepdims=False):
     return _reduce('hipcx_any', a.astype('bool', False), axes, out)
 
 
+def cumsum(a, axis=None):
+    """Cumsum (CX/routines/reduction.cc:103-134): over the flattened array when axis is None; bool / integer inputs give int64."""
+    if axis is None:
+        a = a.reshape((_prod(a.shape),))
+        axis = 0
+    else:
+        axis = _normalize_axis(axis, a.ndim)
+    out = ndarray.empty(a.shape, 'int64' if _kind(a.dtype) in (0, 1, 2) else a.dtype)
+    if _prod(a.shape):
+        _lib.call('hipcx_cumsum', a.desc(), axis, out.desc(), current_stream())
+    return out
+
+
+def nansum(a, axis=None, keepdims=False):
+    """Nansum (CX/routines/reduction.cc:149-170): Where(IsNan(a), 0, a), then the sum kernel (the native NansumKernel is its
+    SumKernel, native/native_device/reduction.cc:146-167)."""
+    return sum(where(isnan(a), 0, a), axis, keepdims)
+
+
 def mean(a, axis=None, keepdims=False):
     """Mean = Sum then DivideAS by the item count (CX/routines/statistics.cc:95-154)."""
     axes = _sorted_axes(axis, a.ndim)
@@ -1116,6 +1209,27 @@ def take(a, indices, axis, mode=None):
         flag = zeros((1,), 'int32')
         flag_ptr = ctypes.cast(ctypes.c_void_p(flag.data_ptr), ctypes.POINTER(ctypes.c_int32))
     _lib.call('hipcx_take', a.desc(), indices.desc(), axis, out.desc(), m, flag_ptr, current_stream())
+    if flag is not None and int(flag.get()[0]) != 0:
+        raise _lib.ChainerxIndexError('Index is out of bounds for axis %d with size %d' % (axis, a.shape[axis]))
+    return out
+
+
+def add_at(a, indices, axis, b, mode=None):
+    """AddAt kernel call as Take's backward issues it (CX/routines/indexing.cc:147-169): a copy of a with b added at the
+    indexed positions of `axis`; repeated indices accumulate in index order."""
+    if _kind(indices.dtype) not in (1, 2):
+        raise _lib.DtypeError('Only arrays of integer dtype can be used as indices.')
+    axis = _normalize_axis(axis, a.ndim)
+    if b.shape != a.shape[:axis] + indices.shape + a.shape[axis + 1:]:
+        raise _lib.DimensionError('b has the wrong shape')
+    out = ndarray.empty(a.shape, a.dtype)
+    m = _BOUNDS[mode]
+    flag = None
+    flag_ptr = None
+    if m in (0, 1):
+        flag = zeros((1,), 'int32')
+        flag_ptr = ctypes.cast(ctypes.c_void_p(flag.data_ptr), ctypes.POINTER(ctypes.c_int32))
+    _lib.call('hipcx_add_at', a.desc(), indices.desc(), axis, b.astype(a.dtype, False).desc(), out.desc(), m, flag_ptr, current_stream())
     if flag is not None and int(flag.get()[0]) != 0:
         raise _lib.ChainerxIndexError('Index is out of bounds for axis %d with size %d' % (axis, a.shape[axis]))
     return out

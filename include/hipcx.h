@@ -287,6 +287,26 @@ int hipcx_average_pool(const hipcx_array* x, const int64_t* kernel_size, const i
 int hipcx_take(const hipcx_array* a, const hipcx_array* indices, int8_t axis, const hipcx_array* out, int mode, int32_t* error_flag,
                void* stream);
 
+/* AddAtKernel indexing.h:12 -- out = a, then out[l..., indices[i...], r...] += b[l..., i..., r...] along `axis`, the indices
+ * walked in C order so that repeated indices accumulate in the reference's order (native/native_device/indexing.cc:107-190);
+ * bounds modes and error_flag as for hipcx_take.  a, b and out share a dtype. */
+int hipcx_add_at(const hipcx_array* a, const hipcx_array* indices, int8_t axis, const hipcx_array* b, const hipcx_array* out, int mode,
+                 int32_t* error_flag, void* stream);
+
+/* Creation kernels (native/native_device/fill.cc): IdentityKernel creation.h:24, EyeKernel(k) :31, TriKernel(k) :50 fill a
+ * C-contiguous 2-D out with the 0/1 pattern; LinspaceKernel :43 writes (start*(n-1-i) + stop*i)/(n-1) evaluated in double;
+ * DiagflatKernel :38 places the 1-D v on the k-th diagonal of a zeroed square out. */
+int hipcx_identity(const hipcx_array* out, void* stream);
+int hipcx_eye(int64_t k, const hipcx_array* out, void* stream);
+int hipcx_tri(int64_t k, const hipcx_array* out, void* stream);
+int hipcx_linspace(double start, double stop, const hipcx_array* out, void* stream);
+int hipcx_diagflat(const hipcx_array* v, int64_t k, const hipcx_array* out, void* stream);
+
+/* CumsumKernel reduction.h:23 -- inclusive prefix sums along `axis`, added serially in index order as native::Scan does
+ * (CX/native/reduce.h:98-113): float results carry the native backend's bits.  out: a's float dtype, int64 for bool and
+ * integer inputs (CX/routines/reduction.cc:115-127); float16 accumulates in float and rounds every prefix. */
+int hipcx_cumsum(const hipcx_array* a, int8_t axis, const hipcx_array* out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -525,6 +525,90 @@ def any(a, axis=None, keepdims=False):
     return np.any(a, axis=axis if axis is None or isinstance(axis, int) else tuple(axis), keepdims=keepdims)
 
 
+def cumsum(a, axis=None):
+    """NativeCumsumKernel (reduction.cc:121-144) over native::Scan (reduce.h:98-113): strictly serial prefix sums in the
+    accumulator type (float for float16 with every prefix rounded on output, int64 for bool / integer inputs)."""
+    a = np.asarray(a)
+    if axis is None:
+        a = a.reshape(-1)
+        axis = 0
+    if a.dtype.kind in 'biu':
+        return np.cumsum(a.astype(np.int64), axis=axis)
+    acc_t = np.float32 if a.dtype == np.float16 else a.dtype
+    moved = np.moveaxis(a, axis, -1)
+    out = np.empty(moved.shape, a.dtype)
+    acc = np.zeros(moved.shape[:-1], acc_t)
+    with np.errstate(all='ignore'):
+        for j in range(moved.shape[-1]):
+            acc = (acc + moved[..., j].astype(acc_t)).astype(acc_t)
+            out[..., j] = acc.astype(a.dtype)
+    return np.moveaxis(out, -1, axis)
+
+
+def nansum(a, axis=None, keepdims=False):
+    """Nansum routine (CX/routines/reduction.cc:149-170): NaNs replaced by 0, then the Sum kernel."""
+    a = np.asarray(a)
+    if a.dtype.kind == 'f':
+        a = np.where(np.isnan(a), a.dtype.type(0), a)
+    return sum(a, axis, keepdims)
+
+
+def add_at(a, indices, axis, b, mode=None):
+    """NativeAddAtKernel (indexing.cc:107-190): copy of a, then for every index in C order out[.., index, ..] += b[.., i, ..]
+    in the array dtype (float16 rounds after every addition, integers wrap, bool saturates to True)."""
+    a, indices, b = np.asarray(a), np.asarray(indices), np.asarray(b)
+    axis = axis % a.ndim
+    dim = a.shape[axis]
+    out = np.moveaxis(a.copy(), axis, 0)
+    nleft = axis
+    bm = np.moveaxis(b.reshape(a.shape[:axis] + (-1,) + a.shape[axis + 1:]), nleft, 0)
+    with np.errstate(all='ignore'):
+        for i, index in enumerate(indices.reshape(-1).tolist()):
+            if mode in (None, 'raise'):
+                if index < -dim or index >= dim:
+                    raise IndexError('Index %d is out of bounds for axis %d with size %d' % (index, axis, dim))
+                if index < 0:
+                    index += dim
+            elif mode == 'wrap':
+                index = dim - ((-index + dim - 1) % dim + 1) if index < 0 else index % dim
+            else:
+                index = max(0, min(index, dim - 1))
+            if a.dtype == np.bool_:
+                out[index] = out[index] | bm[i]
+            elif a.dtype == np.float16:
+                out[index] = (out[index].astype(np.float32) + bm[i].astype(np.float32)).astype(np.float16)
+            else:
+                out[index] = (out[index] + bm[i]).astype(a.dtype)
+    return np.moveaxis(out, 0, axis)
+
+
+def identity(n, dtype):
+    return np.identity(n, dtype)
+
+
+def eye(n, m, k, dtype):
+    return np.eye(n, m, k, dtype)
+
+
+def tri(n, m, k, dtype):
+    return np.tri(n, m, k, dtype)
+
+
+def linspace(start, stop, num, endpoint, dtype):
+    """NativeLinspaceKernel (fill.cc): (start*(n-1-i) + stop*i)/(n-1) in double, cast to the dtype."""
+    start, stop = float(start), float(stop)
+    if not endpoint:
+        stop = start + (stop - start) * (num - 1) / num
+    i = np.arange(num, dtype=np.float64)
+    v = np.full(num, start) if num == 1 else (start * (num - 1 - i) + stop * i) / (num - 1)
+    with np.errstate(all='ignore'):
+        return v.astype(dtype)
+
+
+def diagflat(v, k):
+    return np.diagflat(np.asarray(v), k)
+
+
 def mean(a, axis=None, keepdims=False):
     """Mean = SumKernel into the float result dtype, then DivideASKernel by the count (CX/routines/statistics.cc:95-154)."""
     a = np.asarray(a)

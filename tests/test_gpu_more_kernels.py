@@ -276,3 +276,76 @@ def test_bitwise_and_shifts(dt):
     assert got.dtype == np.int64
     assert_exact(got.get(), O.left_shift(np.full(cnt.shape, 3, np.int64), cnt.astype(np.int64)), 'left_shift SA')
     assert_exact(chx.right_shift(-1000, Cn).get(), O.right_shift(np.full(cnt.shape, -1000, np.int64), cnt.astype(np.int64)), 'right_shift SA')
+
+
+@pytest.mark.parametrize('dt', ALL)
+def test_creation_patterns(dt):
+    import chainer_amd as chx
+    for n in (0, 1, 5, 33):
+        assert_exact(chx.identity(n, dt).get(), O.identity(n, dt), 'identity %d' % n)
+    for (n, m, k) in [(4, 4, 0), (5, 7, 2), (7, 5, -3), (6, 6, 9), (6, 6, -9), (1, 9, 3), (40, 37, 1)]:
+        assert_exact(chx.eye(n, m, k, dt).get(), O.eye(n, m, k, dt), 'eye %r' % ((n, m, k),))
+        assert_exact(chx.tri(n, m, k, dt).get(), O.tri(n, m, k, dt), 'tri %r' % ((n, m, k),))
+    rng = np.random.default_rng(31)
+    v = rand(rng, (6,), dt)
+    for k in (0, 2, -3):
+        assert_exact(chx.diagflat(chx.array(v), k).get(), O.diagflat(v, k), 'diagflat k=%d' % k)
+    v2 = rand(rng, (2, 3), dt)
+    assert_exact(chx.diagflat(chx.array(v2)[:, ::-1], 1).get(), O.diagflat(v2[:, ::-1], 1), 'diagflat of a view')
+    m2 = rand(rng, (5, 7), dt)
+    for k in (0, 2, -1, 6, -5):
+        assert_exact(chx.diag(chx.array(m2), k).get(), np.diag(m2, k), 'diag view k=%d' % k)
+    if dt != 'bool':
+        for (a, b, num, ep) in [(0, 10, 11, True), (-3, 7.5, 50, True), (2, -2, 9, False), (5, 5, 1, True), (0, 1, 4097, True)]:
+            assert_exact(chx.linspace(a, b, num, ep, dt).get(), O.linspace(a, b, num, ep, dt), 'linspace %r' % ((a, b, num, ep),))
+    assert chx.linspace(0, 1, 0).shape == (0,)
+    with pytest.raises(chx.DimensionError):
+        chx.eye(-1)
+
+
+@pytest.mark.parametrize('dt', ALL)
+def test_cumsum_nansum(dt):
+    import chainer_amd as chx
+    rng = np.random.default_rng(32)
+    for shape, axis in [((7, 130), 1), ((7, 130), 0), ((4, 5, 6), 1), ((3, 4, 5), None), ((2000,), 0), ((5, 9), -1)]:
+        x = rand(rng, shape, dt)
+        got = chx.cumsum(chx.array(x), axis).get()
+        assert_exact(got, O.cumsum(x, axis), 'cumsum %r axis %r (serial order: bit-exact)' % (shape, axis))
+    xv = rand(rng, (9, 40), dt)
+    assert_exact(chx.cumsum(chx.array(xv).T[::2], 1).get(), O.cumsum(xv.T[::2], 1), 'cumsum of a view')
+    if np.dtype(dt).kind == 'f':
+        x = rand(rng, (6, 300), dt)
+        x[x > 15] = np.nan
+        assert np.isnan(x).any()
+        assert_close(chx.nansum(chx.array(x), 1).get(), O.nansum(x, 1), None, 'nansum')
+        assert_close(chx.nansum(chx.array(x)).get(), O.nansum(x), None, 'nansum all axes')
+
+
+@pytest.mark.parametrize('dt', ALL)
+def test_add_at(dt):
+    import chainer_amd as chx
+    rng = np.random.default_rng(33)
+    a = rand(rng, (5, 6, 7), dt)
+    for axis, ishape in [(0, (4,)), (1, (3, 2)), (2, (9,)), (1, (1,))]:
+        dim = a.shape[axis]
+        idx = rng.integers(-dim, dim, ishape)  # repeated and negative indices
+        b = rand(rng, a.shape[:axis] + ishape + a.shape[axis + 1:], dt)
+        got = chx.add_at(chx.array(a), chx.array(idx), axis, chx.array(b)).get()
+        assert_exact(got, O.add_at(a, idx, axis, b), 'add_at axis %d %r' % (axis, ishape))
+        big = idx * 5
+        for mode in ('wrap', 'clip'):
+            assert_exact(chx.add_at(chx.array(a), chx.array(big.astype('int32')), axis, chx.array(b), mode).get(),
+                         O.add_at(a, big, axis, b, mode), 'add_at %s' % mode)
+    # views on both sides
+    idx = np.array([1, 1, 0, 3])
+    b = rand(rng, (5, 4, 7), dt)
+    got = chx.add_at(chx.array(a)[:, ::-1], chx.array(idx), 1, chx.array(b)[::-1]).get()
+    assert_exact(got, O.add_at(a[:, ::-1], idx, 1, b[::-1]), 'add_at views')
+    with pytest.raises(chx.ChainerxIndexError):
+        chx.add_at(chx.array(a), chx.array(np.array([6])), 1, chx.array(rand(rng, (5, 1, 7), dt)))
+    # the embedding gradient: many rows scattered into a table
+    if dt == 'float32':
+        table = np.zeros((50, 16), dt)
+        ids = rng.integers(0, 50, (300,))
+        g = rng.standard_normal((300, 16)).astype(dt)
+        assert_exact(chx.add_at(chx.array(table), chx.array(ids), 0, chx.array(g)).get(), O.add_at(table, ids, 0, g), 'embedding gradient')

@@ -577,3 +577,28 @@ def test_floor_divide_mod_brute_force():
     assert np.array_equal(O.floor_divide(fx, fy), np.array([np.floor(p / q) for p, q in zip(fx.tolist(), fy.tolist())], np.float32))
     assert np.array_equal(O.mod(fx, fy), np.array([p % q for p, q in zip(fx.tolist(), fy.tolist())], np.float32))
     assert np.isnan(O.mod(np.float32([1.0]), np.float32([0.0]))[0])
+
+
+def test_cumsum_add_at_closed_forms():
+    """C: on integer-valued data any order is exact, so Cumsum must equal numpy.cumsum and AddAt numpy.add.at; the last
+    prefix of a float Cumsum is the strictly serial sum (CX/native/reduce.h:98-113), checked against a Python loop."""
+    rng = np.random.default_rng(34)
+    x = rng.integers(-50, 50, (6, 40)).astype(np.float32)
+    assert np.array_equal(O.cumsum(x, 1), np.cumsum(x, axis=1))
+    assert O.cumsum(np.array([True, True, False]), 0).dtype == np.int64
+    y = rng.standard_normal(500).astype(np.float32)
+    acc = np.float32(0)
+    for v in y:
+        acc = np.float32(acc + v)
+    assert O.cumsum(y, 0)[-1] == acc
+    a = rng.integers(-9, 9, (4, 5, 3)).astype(np.int32)
+    idx = np.array([[0, 4], [4, -1]])
+    b = rng.integers(-9, 9, (4, 2, 2, 3)).astype(np.int32)
+    ref = a.copy()
+    np.add.at(ref, (slice(None), idx % 5), b)
+    assert np.array_equal(O.add_at(a, idx, 1, b), ref)
+    with pytest.raises(IndexError):
+        O.add_at(a, np.array([5]), 1, b[:, :1, 0])
+    # Linspace closed form: endpoints exact, interior from the reference's expression
+    assert np.array_equal(O.linspace(0, 10, 11, True, 'float32'), np.arange(11, dtype=np.float32))
+    assert O.linspace(2, 3, 1, True, 'float64')[0] == 2.0
