@@ -30,7 +30,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 matrix peak
 # HBM bytes per convolution launch (fetch + write, averaged over the 53 convolutions of one step), from two rocprofv3
 # --pmc runs (FETCH_SIZE, WRITE_SIZE) scaled by what the same counters read for a 128 MiB copy kernel (x1.999, x1.000):
 # profiles/resnet50_conv_hbm_traffic.txt.  The algorithmic figure is 101 MB per launch.
-CONV_HBM_TRAFFIC_BYTES_PER_LAUNCH = 112.1e6
+CONV_HBM_TRAFFIC_BYTES_PER_LAUNCH = 111.1e6
 
 
 def main():

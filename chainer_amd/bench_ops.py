@@ -27,18 +27,24 @@ HBM_PEAK = 8000.0  # GB/s
 MFMA_PEAK = {'float16': 2500.0, 'float32': 157.3}  # TFLOP/s
 
 
-def device_time(fn, iters=20, warmup=5):
+def device_time(fn, iters=20, warmup=5, rounds=3):
+    """Seconds per call: HIP events around `iters` back-to-back calls, best of `rounds` (a round that happens to grow the
+    allocator's pool or to load a code object is not the kernel's time)."""
     import torch
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(iters):
-        fn()
-    e1.record()
-    e1.synchronize()
-    return e0.elapsed_time(e1) / iters * 1e-3  # seconds
+    best = None
+    for _ in range(rounds):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(iters):
+            fn()
+        e1.record()
+        e1.synchronize()
+        t = e0.elapsed_time(e1) / iters * 1e-3
+        best = t if best is None else min(best, t)
+    return best
 
 
 def graph_time(fn, iters=20):
