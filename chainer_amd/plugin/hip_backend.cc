@@ -15,7 +15,9 @@
 // its kernels would dereference device pointers on the host.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cstdint>
+#include <limits>
 #include <map>
 #include <memory>
 #include <mutex>
@@ -56,6 +58,12 @@
 #include "chainerx/native/native_backend.h"
 #include "chainerx/routines/connection.h"
 #include "chainerx/routines/creation.h"
+#include "chainerx/routines/indexing.h"
+#include "chainerx/routines/logic.h"
+#include "chainerx/routines/manipulation.h"
+#include "chainerx/native/tensor_dot.h"
+#include "chainerx/array_index.h"
+#include "chainerx/slice.h"
 #include "chainerx/scalar.h"
 #include "chainerx/shape.h"
 
@@ -779,9 +787,25 @@ public:
 };
 HIPCX_REGISTER_KERNEL(FixedBatchNormKernel, HipFixedBatchNormKernel)
 
-// ---- pooling (forward only: the states are inert) ----
-class HipMaxPoolGradState : public MaxPoolGradState {};
-class HipAveragePoolGradState : public AveragePoolGradState {};
+// ---- pooling: the states keep what the gradient kernels recompute from ----
+class HipMaxPoolGradState : public MaxPoolGradState {
+public:
+    HipMaxPoolGradState(Array x, bool cover_all) : x_{std::move(x)}, cover_all_{cover_all} {}
+    const Array& x() const { return x_; }
+    bool cover_all() const { return cover_all_; }
+
+private:
+    Array x_;
+    bool cover_all_;
+};
+class HipAveragePoolGradState : public AveragePoolGradState {
+public:
+    explicit HipAveragePoolGradState(Array x) : x_{std::move(x)} {}
+    const Array& x() const { return x_; }
+
+private:
+    Array x_;
+};
 
 Shape PoolOutShape(const Array& x, const Dims& k, const Dims& s, const Dims& p, bool cover_all) {
     if (x.ndim() != 4) throw NotImplementedError{"hip pooling supports 2 spatial dimensions."};
@@ -799,7 +823,7 @@ public:
         hipcx_array cx = ToC(x), cy = ToC(y);
         int64_t k[2] = {kernel_size[0], kernel_size[1]}, s[2] = {stride[0], stride[1]}, p[2] = {pad[0], pad[1]};
         Check(hipcx_max_pool(&cx, k, s, p, cover_all ? 1 : 0, &cy, nullptr));
-        std::unique_ptr<MaxPoolGradState> state = return_state ? std::make_unique<HipMaxPoolGradState>() : nullptr;
+        std::unique_ptr<MaxPoolGradState> state = return_state ? std::make_unique<HipMaxPoolGradState>(x, cover_all) : nullptr;
         return std::make_tuple(std::move(y), std::move(state));
     }
 };
@@ -818,11 +842,141 @@ public:
         int64_t k[2] = {kernel_size[0], kernel_size[1]}, s[2] = {stride[0], stride[1]}, p[2] = {pad[0], pad[1]};
         int mode = pad_mode == AveragePoolPadMode::kZero ? HIPCX_PAD_ZERO : HIPCX_PAD_IGNORE;
         Check(hipcx_average_pool(&cx, k, s, p, mode, &cy, nullptr));
-        std::unique_ptr<AveragePoolGradState> state = return_state ? std::make_unique<HipAveragePoolGradState>() : nullptr;
+        std::unique_ptr<AveragePoolGradState> state = return_state ? std::make_unique<HipAveragePoolGradState>(x) : nullptr;
         return std::make_tuple(std::move(y), std::move(state));
     }
 };
 HIPCX_REGISTER_KERNEL(AveragePoolKernel, HipAveragePoolKernel)
+
+// ---- backward / training kernels: compositions over the kernels above, the way the native backend composes them ----
+// Im2Col (CX/native/im2col.cc:82-149) with the gather done by one strided Copy kernel per kernel offset.
+Array HipIm2Col(const Array& x, const Dims& k, const Dims& s, const Dims& p, bool cover_all, Scalar pad_value) {
+    if (x.ndim() != 4) throw NotImplementedError{"hip backward kernels support 2 spatial dimensions."};
+    Device& device = x.device();
+    int64_t oh = OutDim(x.shape()[2], k[0], s[0], p[0], cover_all), ow = OutDim(x.shape()[3], k[1], s[1], p[1], cover_all);
+    Shape padded_shape{x.shape()[0], x.shape()[1], x.shape()[2] + 2 * p[0] + (cover_all ? s[0] - 1 : 0),
+                       x.shape()[3] + 2 * p[1] + (cover_all ? s[1] - 1 : 0)};
+    Array padded = Full(padded_shape, pad_value, x.dtype(), device);
+    device.backend().CallKernel<CopyKernel>(x, padded.At({Slice{}, Slice{}, Slice{p[0], p[0] + x.shape()[2]}, Slice{p[1], p[1] + x.shape()[3]}}));
+    Array col = Empty(Shape{x.shape()[0], x.shape()[1], k[0], k[1], oh, ow}, x.dtype(), device);
+    for (int64_t r = 0; r < k[0]; ++r) {
+        for (int64_t q = 0; q < k[1]; ++q) {
+            device.backend().CallKernel<CopyKernel>(
+                    padded.At({Slice{}, Slice{}, Slice{r, r + s[0] * oh, s[0]}, Slice{q, q + s[1] * ow, s[1]}}),
+                    col.At({Slice{}, Slice{}, ArrayIndex{r}, ArrayIndex{q}}));
+        }
+    }
+    return col;
+}
+
+// Col2Im (CX/native/col2im.cc:76-122): in-place strided Add kernels in the reference's (r, s) order.
+Array HipCol2Im(const Array& col, const Dims& s, const Dims& p, const Dims& out_size) {
+    Device& device = col.device();
+    int64_t kh = col.shape()[2], kw = col.shape()[3], h = col.shape()[4], w = col.shape()[5];
+    Array padded = Zeros(Shape{col.shape()[0], col.shape()[1], out_size[0] + 2 * p[0] + s[0] - 1, out_size[1] + 2 * p[1] + s[1] - 1},
+                         col.dtype(), device);
+    for (int64_t r = 0; r < kh; ++r) {
+        for (int64_t q = 0; q < kw; ++q) {
+            Array view = padded.At({Slice{}, Slice{}, Slice{r, r + s[0] * h, s[0]}, Slice{q, q + s[1] * w, s[1]}});
+            device.backend().CallKernel<AddKernel>(view, col.At({Slice{}, Slice{}, ArrayIndex{r}, ArrayIndex{q}}), view);
+        }
+    }
+    return padded.At({Slice{}, Slice{}, Slice{p[0], p[0] + out_size[0]}, Slice{p[1], p[1] + out_size[1]}});
+}
+
+class HipConvGradWeightKernel : public ConvGradWeightKernel {
+public:
+    Array Call(Dtype w_dtype, const Shape& w_shape, const Array& x, const Array& gy, const Dims& stride, const Dims& pad, bool cover_all,
+               const absl::optional<Array>& out) override {
+        if (out.has_value()) throw NotImplementedError{"Passing out as an argument is not yet supported."};
+        SetDeviceScope scope{x.device().index()};
+        Array col = HipIm2Col(x, Dims{w_shape[2], w_shape[3]}, stride, pad, cover_all, 0);
+        return native::TensorDot(gy, col, Axes{0, 2, 3}, Axes{0, 4, 5}, w_dtype);  // dispatches DotKernel on this backend
+    }
+};
+HIPCX_REGISTER_KERNEL(ConvGradWeightKernel, HipConvGradWeightKernel)
+
+class HipConvTransposeKernel : public ConvTransposeKernel {
+public:
+    Array Call(const Array& x, const Array& w, const absl::optional<Array>& b, const Dims& stride, const Dims& pad, const Dims& out_size,
+               Dtype out_dtype, const absl::optional<Array>& out) override {
+        if (out.has_value()) throw NotImplementedError{"Passing out as an argument is not yet supported."};
+        if (x.ndim() != 4) throw NotImplementedError{"hip convolution supports 2 spatial dimensions."};
+        SetDeviceScope scope{x.device().index()};
+        Array col = native::TensorDot(w, x, Axes{0}, Axes{1}, out_dtype);  // [C_out, kh, kw, N, H, W]
+        Array actual_out = HipCol2Im(col.Transpose(Axes{3, 0, 1, 2, 4, 5}), stride, pad, out_size);
+        if (b.has_value()) {
+            actual_out += b->AsType(out_dtype, false).Reshape(Shape{1, b->shape()[0], 1, 1});
+        }
+        return actual_out;
+    }
+};
+HIPCX_REGISTER_KERNEL(ConvTransposeKernel, HipConvTransposeKernel)
+
+// Batch normalisation in training mode and its gradient are routine compositions in the reference
+// (CX/routines/normalization.cc:155-250); registering the generic kernels runs them on this backend's kernels.
+HIPCX_REGISTER_KERNEL(BatchNormKernel, GenericBatchNormKernel)
+HIPCX_REGISTER_KERNEL(BatchNormGradKernel, GenericBatchNormGradKernel)
+
+class HipMaxPoolGradKernel : public MaxPoolGradKernel {
+public:
+    std::tuple<Array, std::unique_ptr<MaxPoolGradGradState>> Call(const Array& gout, const Dims& kernel_size, const Dims& stride, const Dims& pad,
+                                                                 const std::shared_ptr<MaxPoolGradState>& state, bool return_state,
+                                                                 const absl::optional<Array>& gx) override {
+        if (gx.has_value()) throw NotImplementedError{"Passing gx as an argument is not yet supported."};
+        if (return_state) throw NotImplementedError{"hip MaxPoolGradGrad is not implemented."};
+        auto& st = dynamic_cast<HipMaxPoolGradState&>(*state);
+        const Array& x = st.x();
+        Device& device = x.device();
+        SetDeviceScope scope{device.index()};
+        Scalar lowest = GetKind(x.dtype()) == DtypeKind::kFloat ? Scalar{-std::numeric_limits<double>::infinity()} : Scalar{0};
+        Array col = HipIm2Col(x, kernel_size, stride, pad, st.cover_all(), lowest);
+        Array indices = col.ArgMax(Axes{2, 3});  // the native tie rule picks the position inside a window
+        // every output position owns its own slots of the col, so the AddAt of the native kernel degenerates to a select
+        int64_t kt = kernel_size[0] * kernel_size[1];
+        Shape lifted{gout.shape()[0], gout.shape()[1], 1, 1, gout.shape()[2], gout.shape()[3]};
+        Array taps = Arange(kt, Dtype::kInt64, device).Reshape(Shape{1, 1, kernel_size[0], kernel_size[1], 1, 1});
+        Array gcol = Where(Equal(indices.Reshape(lifted), taps), gout.Reshape(lifted), Scalar{0, GetKind(gout.dtype())});
+        Array actual_gx = HipCol2Im(gcol, stride, pad, Dims{x.shape()[2], x.shape()[3]});
+        return std::make_tuple(std::move(actual_gx), std::unique_ptr<MaxPoolGradGradState>{});
+    }
+};
+HIPCX_REGISTER_KERNEL(MaxPoolGradKernel, HipMaxPoolGradKernel)
+
+class HipAveragePoolGradKernel : public AveragePoolGradKernel {
+public:
+    Array Call(const Array& gout, const Dims& kernel_size, const Dims& stride, const Dims& pad, AveragePoolPadMode pad_mode,
+               const std::shared_ptr<AveragePoolGradState>& state, const absl::optional<Array>& gx) override {
+        if (gx.has_value()) throw NotImplementedError{"Passing gx as an argument is not yet supported."};
+        auto& st = dynamic_cast<HipAveragePoolGradState&>(*state);
+        const Array& x = st.x();
+        Device& device = x.device();
+        SetDeviceScope scope{device.index()};
+        Shape gcol_shape{gout.shape()[0], gout.shape()[1], kernel_size[0], kernel_size[1], gout.shape()[2], gout.shape()[3]};
+        Shape lifted{gout.shape()[0], gout.shape()[1], 1, 1, gout.shape()[2], gout.shape()[3]};
+        Dims out_size{x.shape()[2], x.shape()[3]};
+        if (pad_mode == AveragePoolPadMode::kZero) {
+            Array actual_gx = HipCol2Im(gout.Reshape(lifted).BroadcastTo(gcol_shape), stride, pad, out_size).Copy();
+            actual_gx /= Scalar{kernel_size[0] * kernel_size[1]};
+            return actual_gx;
+        }
+        // per-position count of in-image taps (CX/native/native_device/pool.cc:197-250), built on the host: it is tiny
+        std::vector<double> widths(static_cast<size_t>(gout.shape()[2] * gout.shape()[3]));
+        for (int64_t i = 0; i < gout.shape()[2]; ++i) {
+            double wi = static_cast<double>(std::min(i * stride[0] - pad[0] + kernel_size[0], x.shape()[2]) - std::max<int64_t>(i * stride[0] - pad[0], 0));
+            for (int64_t j = 0; j < gout.shape()[3]; ++j) {
+                double wj = static_cast<double>(std::min(j * stride[1] - pad[1] + kernel_size[1], x.shape()[3]) - std::max<int64_t>(j * stride[1] - pad[1], 0));
+                widths[static_cast<size_t>(i * gout.shape()[3] + j)] = wi * wj;
+            }
+        }
+        Shape w_shape{gout.shape()[2], gout.shape()[3]};
+        Array w_host = internal::FromHostData(w_shape, Dtype::kFloat64, std::shared_ptr<void>(widths.data(), [](void*) {}),
+                                              Strides{w_shape, Dtype::kFloat64}, 0, GetDefaultContext().GetNativeBackend().GetDevice(0));
+        Array w_dev = w_host.ToDevice(device).AsType(gout.dtype(), false);
+        return HipCol2Im((gout / w_dev).Reshape(lifted).BroadcastTo(gcol_shape), stride, pad, out_size);
+    }
+};
+HIPCX_REGISTER_KERNEL(AveragePoolGradKernel, HipAveragePoolGradKernel)
 
 // ---- take ----
 class HipTakeKernel : public TakeKernel {

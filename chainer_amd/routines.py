@@ -1236,6 +1236,427 @@ def add_at(a, indices, axis, b, mode=None):
 
 
 # ---------------------------------------------------------------------------------------------
+# backward / training kernels, composed from the kernels above exactly as the reference's native backend composes them
+# (Im2Col / Col2Im as strided Copy / Add kernel calls, TensorDot as transposes + Dot)
+# ---------------------------------------------------------------------------------------------
+def _copy_into(dst_view, src):
+    _lib.call('hipcx_copy', src.desc(), dst_view.desc(), current_stream())
+
+
+def im2col(x, ksize, stride, pad, cover_all=False, pad_value=0):
+    """native_internal::Im2Col (CX/native/im2col.cc:82-149): a padded copy of x, then one strided Copy per kernel offset into
+    col[N, C, kh, kw, oh, ow]."""
+    n, c, h, w = x.shape
+    kh, kw = ksize
+    sh, sw = stride
+    ph, pw = pad
+    oh = conv_out_dim(h, kh, sh, ph, cover_all)
+    ow = conv_out_dim(w, kw, sw, pw, cover_all)
+    hp = h + 2 * ph + (sh - 1 if cover_all else 0)
+    wp = w + 2 * pw + (sw - 1 if cover_all else 0)
+    xp = full((n, c, hp, wp), pad_value, x.dtype)
+    _copy_into(xp[:, :, ph:ph + h, pw:pw + w], x)
+    col = ndarray.empty((n, c, kh, kw, oh, ow), x.dtype)
+    for r in range(kh):
+        for q in range(kw):
+            _copy_into(col[:, :, r, q], xp[:, :, r:r + sh * oh:sh, q:q + sw * ow:sw])
+    return col
+
+
+def col2im(col, stride, pad, out_size):
+    """native_internal::Col2Im (CX/native/col2im.cc:76-122): zeros of the padded size, then for every kernel offset in (r, s)
+    order an in-place strided Add -- the accumulation order of the reference -- and a view without the padding."""
+    n, c, kh, kw, h, w = col.shape
+    sh, sw = stride
+    ph, pw = pad
+    oh, ow = out_size
+    padded = zeros((n, c, oh + 2 * ph + sh - 1, ow + 2 * pw + sw - 1), col.dtype)
+    for r in range(kh):
+        for q in range(kw):
+            view = padded[:, :, r:r + sh * h:sh, q:q + sw * w:sw]
+            _lib.call('hipcx_add', view.desc(), col[:, :, r, q].desc(), view.desc(), current_stream())
+    return padded[:, :, ph:ph + oh, pw:pw + ow]
+
+
+def tensordot(a, b, a_axes, b_axes, out_dtype=None):
+    """TensorDot (CX/native/tensor_dot.cc:63-99): reduced axes of a rolled last, of b rolled first, reshape to 2-D, Dot."""
+    a_axes = [ax % a.ndim for ax in a_axes]
+    b_axes = [ax % b.ndim for ax in b_axes]
+    a_keep = [i for i in range(a.ndim) if i not in a_axes]
+    b_keep = [i for i in range(b.ndim) if i not in b_axes]
+    red = _prod([a.shape[i] for i in a_axes])
+    a2 = a.transpose(a_keep + a_axes).reshape((_prod([a.shape[i] for i in a_keep]), red))
+    b2 = b.transpose(b_axes + b_keep).reshape((red, _prod([b.shape[i] for i in b_keep])))
+    out = dot(a2, b2, out_dtype)
+    return out.reshape(tuple(a.shape[i] for i in a_keep) + tuple(b.shape[i] for i in b_keep))
+
+
+def conv_grad_weight(w_dtype, w_shape, x, gy, stride=1, pad=0, cover_all=False):
+    """ConvGradWeightKernel as the native backend runs it (CX/native/native_device/conv.cc:91-124): Im2Col(x), then
+    TensorDot(gy, col) over the batch and the output positions -> gw[K, C, kh, kw]."""
+    if x.ndim != 4:
+        raise _lib.ChainerxNotImplementedError('only 2-D convolution is on the supported path')
+    col = im2col(x, tuple(w_shape[2:]), _pair(stride), _pair(pad), cover_all, 0)
+    return tensordot(gy, col, (0, 2, 3), (0, 4, 5), w_dtype)
+
+
+def conv_transpose(x, w, b=None, stride=1, pad=0, out_size=None, out_dtype=None):
+    """ConvTranspose (CX/routines/connection.cc:214-320) over the native kernel (CX/native/native_device/conv.cc:126-160):
+    col = TensorDot(w, x) over the input channels, batch axis rolled first, Col2Im, bias added in place.  w: [C_in, C_out, kh, kw]."""
+    if x.ndim != 4:
+        raise _lib.ChainerxNotImplementedError('only 2-D convolution is on the supported path')
+    stride, pad = _pair(stride), _pair(pad)
+    if w.shape[0] != x.shape[1]:
+        raise _lib.DimensionError('Mismatched number of input channels in input of shape %r and filter of shape %r' % (x.shape, w.shape))
+    if b is not None and (b.ndim != 1 or b.shape[0] != w.shape[1]):
+        raise _lib.DimensionError('Mismatched bias shape %r for weights %r.' % (b.shape, w.shape))
+    kh, kw = w.shape[2:]
+    cover_all = False
+    if out_size is None:  # GetConvTransposeOutDim with cover_all = false (CX/routines/connection.cc:51-56)
+        out_size = tuple(st * (d - 1) + k - 2 * p for d, k, st, p in zip(x.shape[2:], (kh, kw), stride, pad))
+        if _py.min(out_size) < 0:
+            raise _lib.DimensionError('Inconsistent dimensions. Output dimension would be negative.')
+    else:
+        out_size = _pair(out_size)
+        if _py.min(out_size) < 0:
+            raise _lib.DimensionError('All output sizes must be non-negative.')
+        cover_all = _py.any(d != conv_out_dim(o, k, st, p, False) for d, o, k, st, p in zip(x.shape[2:], out_size, (kh, kw), stride, pad))
+    for d, o, k, st, p in zip(x.shape[2:], out_size, (kh, kw), stride, pad):
+        if d != conv_out_dim(o, k, st, p, cover_all):
+            raise _lib.DimensionError('Output dims %r are incosistent.' % (tuple(out_size),))
+    dt = numpy.dtype(out_dtype) if out_dtype is not None else (result_type(x, w, b) if b is not None else result_type(x, w))
+    oh = conv_out_dim(x.shape[2], w.shape[2], stride[0], pad[0], cover_all)
+    ow = conv_out_dim(x.shape[3], w.shape[3], stride[1], pad[1], cover_all)
+    out = _spatial_out(x, x.shape[0], w.shape[0], oh, ow, dt)
+    xc, wc = x.astype(dt, False), w.astype(dt, False)
+    bc = b.astype(dt, False) if b is not None else None
+    nbytes = _lib.load().hipcx_conv_workspace_size(xc.desc(), wc.desc(), out.desc())
+    ws, wsp = _workspace(nbytes)
+    _lib.call('hipcx_conv', xc.desc(), wc.desc(), bc.desc() if bc is not None else None, _i64(stride), _i64(pad),
+              int(bool(cover_all)), out.desc(), wsp, nbytes, current_stream())
+    return out
+
+
+def conv_bn_act(x, w, b=None, stride=1, pad=0, cover_all=False, bn=None, eps=2e-5, residual=None, relu=False):
+    """Opt-in fused block: relu(fixed_batch_norm(conv(x, w, b), *bn, eps, axis=(0, 2, 3)) + residual) in one kernel call.
+    `bn` is None or (gamma, beta, mean, var), one value per output channel.  Not part of the ChainerX routine surface:
+    the reference issues these as separate kernels (which `conv`, `fixed_batch_norm`, `add`, `relu` here do as well)."""
+    if x.ndim != 4 or w.ndim != 4:
+        raise _lib.ChainerxNotImplementedError('only 2-D convolution is on the supported path')
+    stride, pad = _pair(stride), _pair(pad)
+    if w.shape[1] != x.shape[1]:
+        raise _lib.DimensionError('Mismatched number of input channels in input %r and weights %r.' % (x.shape, w.shape))
+    dt = result_type(x, w)
+    oh = conv_out_dim(x.shape[2], w.shape[2], stride[0], pad[0], cover_all)
+    ow = conv_out_dim(x.shape[3], w.shape[3], stride[1], pad[1], cover_all)
+    out = _spatial_out(x, x.shape[0], w.shape[0], oh, ow, dt)
+    xc, wc = x.astype(dt, False), w.astype(dt, False)
+    bc = b.astype(dt, False) if b is not None else None
+    prm = [a.astype(dt, False).desc() for a in bn] if bn is not None else [None] * 4
+    res = residual.astype(dt, False) if residual is not None else None
+    nbytes = _lib.load().hipcx_conv_workspace_size(xc.desc(), wc.desc(), out.desc())
+    ws, wsp = _workspace(nbytes)
+    _lib.call('hipcx_conv_bn_act', xc.desc(), wc.desc(), bc.desc() if bc is not None else None, _i64(stride), _i64(pad),
+              int(bool(cover_all)), prm[0], prm[1], prm[2], prm[3], _lib.make_scalar(float(eps)),
+              res.desc() if res is not None else None, int(bool(relu)), out.desc(), wsp, nbytes, current_stream())
+    return out
+
+
+def fixed_batch_norm(x, gamma, beta, mean, var, eps=2e-5, axis=None):
+    """FixedBatchNorm (CX/routines/normalization.cc:414-424 with PreprocessBatchNorm :61-101)."""
+    for a in (x, gamma, beta, mean, var):
+        if _kind(a.dtype) != 3:
+            raise _lib.DtypeError('BatchNorm only supports floating kind inputs.')
+    axes = _sorted_axes(axis, x.ndim) if axis is not None else (0,)
+    reduced_shape = tuple(1 if i in axes else d for i, d in enumerate(x.shape))
+    size = _prod(reduced_shape)
+    params = []
+    for name, a in (('Gamma', gamma), ('Beta', beta), ('Mean', mean), ('Variance', var)):
+        if a.size != size:
+            raise _lib.DimensionError('%s must have the same size as the reduced input. Actual: %d. Expected: %d.' % (name, a.size, size))
+        params.append(a.reshape(reduced_shape))
+    out = ndarray(alloc_bytes(x.nbytes), 0, x.shape, _dense_strides_like(x), x.dtype)
+    ax = (ctypes.c_int8 * len(axes))(*axes)
+    _lib.call('hipcx_fixed_batch_norm', x.desc(), params[0].desc(), params[1].desc(), params[2].desc(), params[3].desc(),
+              _lib.make_scalar(float(eps)), ax, len(axes), out.desc(), current_stream())
+    return out
+
+
+def _dense_strides_like(x):
+    """Dense strides with the same axis order as x's memory (so a channels-last input gives a channels-last output)."""
+    order = sorted(range(x.ndim), key=lambda i: (-abs(x.strides[i]), i))
+    strides = [0] * x.ndim
+    acc = x.itemsize
+    for i in reversed(order):
+        strides[i] = acc
+        acc *= _py.max(1, x.shape[i])
+    return tuple(strides)
+
+
+def max_pool(x, ksize, stride=None, pad=0, cover_all=False):
+    """MaxPool (CX/routines/pooling.cc:52-123), 2-D."""
+    if x.ndim != 4:
+        raise _lib.ChainerxNotImplementedError('only 2-D pooling is on the supported path')
+    ksize = _pair(ksize)
+    stride = ksize if stride is None else _pair(stride)
+    pad = _pair(pad)
+    oh = conv_out_dim(x.shape[2], ksize[0], stride[0], pad[0], cover_all)
+    ow = conv_out_dim(x.shape[3], ksize[1], stride[1], pad[1], cover_all)
+    out = _spatial_out(x, x.shape[0], x.shape[1], oh, ow, x.dtype)
+    _lib.call('hipcx_max_pool', x.desc(), _i64(ksize), _i64(stride), _i64(pad), int(bool(cover_all)), out.desc(), current_stream())
+    return out
+
+
+def average_pool(x, ksize, stride=None, pad=0, pad_mode='ignore'):
+    """AveragePool (CX/routines/pooling.cc:125-169), 2-D, float dtypes only."""
+    if _kind(x.dtype) != 3:
+        raise _lib.DtypeError('cannot apply average pooling to non-float arrays')
+    if x.ndim != 4:
+        raise _lib.ChainerxNotImplementedError('only 2-D pooling is on the supported path')
+    ksize = _pair(ksize)
+    stride = ksize if stride is None else _pair(stride)
+    pad = _pair(pad)
+    mode = {'zero': 1, 'ignore': 2}[pad_mode]
+    oh = conv_out_dim(x.shape[2], ksize[0], stride[0], pad[0], False)
+    ow = conv_out_dim(x.shape[3], ksize[1], stride[1], pad[1], False)
+    out = _spatial_out(x, x.shape[0], x.shape[1], oh, ow, x.dtype)
+    _lib.call('hipcx_average_pool', x.desc(), _i64(ksize), _i64(stride), _i64(pad), mode, out.desc(), current_stream())
+    return out
+
+
+# ---------------------------------------------------------------------------------------------
+# indexing
+# ---------------------------------------------------------------------------------------------
+_BOUNDS = {None: 0, 'raise': 1, 'wrap': 2, 'clip': 3}
+
+
+def take(a, indices, axis, mode=None):
+    """Take (CX/routines/indexing.cc:171-205). mode None / 'raise' raise IndexError on out-of-range ids like the
+    native backend; checking that costs one 4-byte read-back after the kernel."""
+    if _kind(indices.dtype) not in (1, 2):
+        raise _lib.DtypeError('Only arrays of integer dtype can be used as indices.')
+    axis = _normalize_axis(axis, a.ndim)
+    out_shape = a.shape[:axis] + indices.shape + a.shape[axis + 1:]
+    out = ndarray.empty(out_shape, a.dtype)
+    m = _BOUNDS[mode]
+    flag = None
+    flag_ptr = None
+    if m in (0, 1):
+        flag = zeros((1,), 'int32')
+        flag_ptr = ctypes.cast(ctypes.c_void_p(flag.data_ptr), ctypes.POINTER(ctypes.c_int32))
+    _lib.call('hipcx_take', a.desc(), indices.desc(), axis, out.desc(), m, flag_ptr, current_stream())
+    if flag is not None and int(flag.get()[0]) != 0:
+        raise _lib.ChainerxIndexError('Index is out of bounds for axis %d with size %d' % (axis, a.shape[axis]))
+    return out
+
+
+def add_at(a, indices, axis, b, mode=None):
+    """AddAt kernel call as Take's backward issues it (CX/routines/indexing.cc:147-169): a copy of a with b added at the
+    indexed positions of `axis`; repeated indices accumulate in index order."""
+    if _kind(indices.dtype) not in (1, 2):
+        raise _lib.DtypeError('Only arrays of integer dtype can be used as indices.')
+    axis = _normalize_axis(axis, a.ndim)
+    if b.shape != a.shape[:axis] + indices.shape + a.shape[axis + 1:]:
+        raise _lib.DimensionError('b has the wrong shape')
+    out = ndarray.empty(a.shape, a.dtype)
+    m = _BOUNDS[mode]
+    flag = None
+    flag_ptr = None
+    if m in (0, 1):
+        flag = zeros((1,), 'int32')
+        flag_ptr = ctypes.cast(ctypes.c_void_p(flag.data_ptr), ctypes.POINTER(ctypes.c_int32))
+    _lib.call('hipcx_add_at', a.desc(), indices.desc(), axis, b.astype(a.dtype, False).desc(), out.desc(), m, flag_ptr, current_stream())
+    if flag is not None and int(flag.get()[0]) != 0:
+        raise _lib.ChainerxIndexError('Index is out of bounds for axis %d with size %d' % (axis, a.shape[axis]))
+    return out
+
+
+# ---------------------------------------------------------------------------------------------
+# backward / training kernels, composed from the kernels above exactly as the reference's native backend composes them
+# (Im2Col / Col2Im as strided Copy / Add kernel calls, TensorDot as transposes + Dot)
+# ---------------------------------------------------------------------------------------------
+def _copy_into(dst_view, src):
+    _lib.call('hipcx_copy', src.desc(), dst_view.desc(), current_stream())
+
+
+def im2col(x, ksize, stride, pad, cover_all=False, pad_value=0):
+    """native_internal::Im2Col (CX/native/im2col.cc:82-149): a padded copy of x, then one strided Copy per kernel offset into
+    col[N, C, kh, kw, oh, ow]."""
+    n, c, h, w = x.shape
+    kh, kw = ksize
+    sh, sw = stride
+    ph, pw = pad
+    oh = conv_out_dim(h, kh, sh, ph, cover_all)
+    ow = conv_out_dim(w, kw, sw, pw, cover_all)
+    hp = h + 2 * ph + (sh - 1 if cover_all else 0)
+    wp = w + 2 * pw + (sw - 1 if cover_all else 0)
+    xp = full((n, c, hp, wp), pad_value, x.dtype)
+    _copy_into(xp[:, :, ph:ph + h, pw:pw + w], x)
+    col = ndarray.empty((n, c, kh, kw, oh, ow), x.dtype)
+    for r in range(kh):
+        for q in range(kw):
+            _copy_into(col[:, :, r, q], xp[:, :, r:r + sh * oh:sh, q:q + sw * ow:sw])
+    return col
+
+
+def col2im(col, stride, pad, out_size):
+    """native_internal::Col2Im (CX/native/col2im.cc:76-122): zeros of the padded size, then for every kernel offset in (r, s)
+    order an in-place strided Add -- the accumulation order of the reference -- and a view without the padding."""
+    n, c, kh, kw, h, w = col.shape
+    sh, sw = stride
+    ph, pw = pad
+    oh, ow = out_size
+    padded = zeros((n, c, oh + 2 * ph + sh - 1, ow + 2 * pw + sw - 1), col.dtype)
+    for r in range(kh):
+        for q in range(kw):
+            view = padded[:, :, r:r + sh * h:sh, q:q + sw * w:sw]
+            _lib.call('hipcx_add', view.desc(), col[:, :, r, q].desc(), view.desc(), current_stream())
+    return padded[:, :, ph:ph + oh, pw:pw + ow]
+
+
+def tensordot(a, b, a_axes, b_axes, out_dtype=None):
+    """TensorDot (CX/native/tensor_dot.cc:63-99): reduced axes of a rolled last, of b rolled first, reshape to 2-D, Dot."""
+    a_axes = [ax % a.ndim for ax in a_axes]
+    b_axes = [ax % b.ndim for ax in b_axes]
+    a_keep = [i for i in range(a.ndim) if i not in a_axes]
+    b_keep = [i for i in range(b.ndim) if i not in b_axes]
+    red = _prod([a.shape[i] for i in a_axes])
+    a2 = a.transpose(a_keep + a_axes).reshape((_prod([a.shape[i] for i in a_keep]), red))
+    b2 = b.transpose(b_axes + b_keep).reshape((red, _prod([b.shape[i] for i in b_keep])))
+    out = dot(a2, b2, out_dtype)
+    return out.reshape(tuple(a.shape[i] for i in a_keep) + tuple(b.shape[i] for i in b_keep))
+
+
+def conv_grad_weight(w_dtype, w_shape, x, gy, stride=1, pad=0, cover_all=False):
+    """ConvGradWeightKernel as the native backend runs it (CX/native/native_device/conv.cc:91-124): Im2Col(x), then
+    TensorDot(gy, col) over the batch and the output positions -> gw[K, C, kh, kw]."""
+    if x.ndim != 4:
+        raise _lib.ChainerxNotImplementedError('only 2-D convolution is on the supported path')
+    col = im2col(x, tuple(w_shape[2:]), _pair(stride), _pair(pad), cover_all, 0)
+    return tensordot(gy, col, (0, 2, 3), (0, 4, 5), w_dtype)
+
+
+def conv_transpose(x, w, b=None, stride=1, pad=0, out_size=None, out_dtype=None):
+    """ConvTranspose (CX/routines/connection.cc:214-320) over the native kernel (CX/native/native_device/conv.cc:126-160):
+    col = TensorDot(w, x) over the input channels, batch axis rolled first, Col2Im, bias added in place.  w: [C_in, C_out, kh, kw]."""
+    if x.ndim != 4:
+        raise _lib.ChainerxNotImplementedError('only 2-D convolution is on the supported path')
+    stride, pad = _pair(stride), _pair(pad)
+    if w.shape[0] != x.shape[1]:
+        raise _lib.DimensionError('Mismatched number of input channels in input of shape %r and filter of shape %r' % (x.shape, w.shape))
+    kh, kw = w.shape[2:]
+    if out_size is None:  # GetConvTransposeOutDim with cover_all = false (CX/routines/connection.cc:51-56)
+        out_size = tuple(st * (d - 1) + k - 2 * p for d, k, st, p in zip(x.shape[2:], (kh, kw), stride, pad))
+    else:
+        out_size = _pair(out_size)
+        for d, o, k, st, p in zip(x.shape[2:], out_size, (kh, kw), stride, pad):
+            if d != conv_out_dim(o, k, st, p, False) and d != conv_out_dim(o, k, st, p, True):
+                raise _lib.DimensionError('Output dims %r is incosistent.' % (out_size,))
+    dt = numpy.dtype(out_dtype) if out_dtype is not None else (result_type(x, w, b) if b is not None else result_type(x, w))
+    col = tensordot(w, x, (0,), (1,), dt)                 # [C_out, kh, kw, N, H, W]
+    col = col.transpose((3, 0, 1, 2, 4, 5))                # batch axis rolled to the top
+    out = col2im(col, stride, pad, out_size)
+    if b is not None:
+        bb = b.astype(dt, False).reshape((1, -1, 1, 1)).broadcast_to(out.shape)
+        _lib.call('hipcx_add', out.desc(), bb.desc(), out.desc(), current_stream())
+    return out
+
+
+def var(a, axis=None, keepdims=False):
+    """Var (CX/routines/statistics.cc:147-154): Mean of the squared deviation from the (keepdims) Mean."""
+    axes = _sorted_axes(axis, a.ndim)
+    dt = a.dtype if _kind(a.dtype) == 3 else numpy.dtype('float32')
+    diff = subtract(a.astype(dt), mean(a, axes, True))
+    return mean(multiply(diff, diff), axes, keepdims)
+
+
+def batch_norm(x, gamma, beta, running_mean, running_var, eps=2e-5, decay=0.9, axis=None):
+    """BatchNorm in training mode through GenericBatchNormKernel (CX/routines/normalization.cc:155-193): batch Mean / Var in the
+    promoted dtype, ApplyGenericBatchNorm, then the running statistics are updated in place (the variance with the n/(n-1)
+    correction).  Returns (out, state) with state = (x_mean, x_inv_std, beta dtype) for batch_norm_grad."""
+    if _py.any(_kind(t.dtype) != 3 for t in (x, gamma, beta, running_mean, running_var)):
+        raise _lib.DtypeError('BatchNorm requires floating point arrays')
+    axes = _sorted_axes((0,) + tuple(range(2, x.ndim)) if axis is None else axis, x.ndim)
+    red_shape = tuple(1 if i in axes else d for i, d in enumerate(x.shape))
+    interm = result_type(x, gamma, beta)
+    xc = x.astype(interm, False)
+    x_mean = mean(xc, axes, True)
+    x_var = var(xc, axes, True)
+    g, bt = gamma.reshape(red_shape).astype(interm, False), beta.reshape(red_shape).astype(interm, False)
+    inv_std = reciprocal(sqrt(add(x_var, eps)))
+    out = add(multiply(multiply(subtract(xc, x_mean), inv_std), g), bt).astype(x.dtype, False)
+    n = _prod(x.shape) // _py.max(1, _prod(gamma.shape))
+    inv_decay = 1.0 - float(decay)
+    rm, rv = running_mean.reshape(red_shape), running_var.reshape(red_shape)
+    multiply(rm, decay, out=rm)
+    add(rm, multiply(x_mean, inv_decay).astype(rm.dtype, False), out=rm)
+    multiply(rv, decay, out=rv)
+    add(rv, multiply(x_var, inv_decay * (float(n) / _py.max(n - 1, 1))).astype(rv.dtype, False), out=rv)
+    return out, (x_mean, inv_std, beta.dtype)
+
+
+def batch_norm_grad(x, gamma, gout, state, axis=None):
+    """GenericBatchNormGradKernel (CX/routines/normalization.cc:195-250): returns (gx, ggamma, gbeta)."""
+    x_mean, x_inv_std, beta_dtype = state
+    axes = _sorted_axes((0,) + tuple(range(2, x.ndim)) if axis is None else axis, x.ndim)
+    red_shape = tuple(1 if i in axes else d for i, d in enumerate(x.shape))
+    interm = x_mean.dtype
+    n = _prod(x.shape) // _py.max(1, _prod(gamma.shape))
+    inv_n = 1.0 / n
+    gc = gout.astype(interm, False)
+    x_hat = multiply(subtract(x.astype(interm, False), x_mean), x_inv_std)
+    ggamma = sum(multiply(gc, x_hat), axes, True)
+    gbeta = sum(gc, axes, True)
+    g = gamma.reshape(red_shape).astype(interm, False)
+    gx = multiply(multiply(g, x_inv_std), subtract(gc, multiply(add(multiply(x_hat, ggamma), gbeta), inv_n)))
+    return (gx.astype(x.dtype, False), ggamma.astype(gamma.dtype, False).reshape(gamma.shape),
+            gbeta.astype(beta_dtype, False).reshape(gamma.shape))
+
+
+def max_pool_grad(x, gout, ksize, stride=None, pad=0, cover_all=False):
+    """MaxPoolGradKernel after the native backend (CX/native/native_device/pool.cc:97-143): Im2Col with -inf padding, ArgMax over
+    the kernel axes (its tie rule picks the position), gout placed at that kernel offset of an otherwise zero col, Col2Im."""
+    ksize = _pair(ksize)
+    stride = ksize if stride is None else _pair(stride)
+    pad = _pair(pad)
+    lowest = -numpy.inf if _kind(x.dtype) == 3 else (0 if x.dtype == numpy.dtype('bool') else int(numpy.iinfo(x.dtype).min))
+    col = im2col(x, ksize, stride, pad, cover_all, lowest)            # [N, C, kh, kw, oh, ow]
+    indices = argmax(col, (2, 3))                                     # [N, C, oh, ow]
+    if indices.shape != gout.shape:
+        raise _lib.DimensionError('gout has the wrong shape')
+    # Every output position owns its own kt slots of the flat col, so the reference's AddAt at (index + offset) writes each
+    # slot at most once: the same values come out of a select against the kernel offsets, which runs in parallel.
+    taps = arange(0, ksize[0] * ksize[1], 1, dtype='int64').reshape((1, 1) + ksize + (1, 1))
+    n, c, oh, ow = gout.shape
+    full_shape = (n, c) + ksize + (oh, ow)
+    hit = equal(indices.reshape((n, c, 1, 1, oh, ow)).broadcast_to(full_shape), taps.broadcast_to(full_shape))
+    gcol = where(hit, gout.reshape((n, c, 1, 1, oh, ow)).broadcast_to(full_shape), 0)
+    return col2im(gcol, stride, pad, x.shape[2:])
+
+
+def average_pool_grad(x, gout, ksize, stride=None, pad=0, pad_mode='ignore'):
+    """AveragePoolGradKernel as the native backend runs it (CX/native/native_device/pool.cc:304-346): gout (divided by the
+    per-window width first in 'ignore' mode) broadcast over the kernel axes, Col2Im, and in 'zero' mode a division by the
+    window size afterwards."""
+    ksize = _pair(ksize)
+    stride = ksize if stride is None else _pair(stride)
+    pad = _pair(pad)
+    n, c, oh, ow = gout.shape
+    g = gout
+    if pad_mode == 'ignore':
+        def widths(dim, k, st, p, count):  # GetPadModeIgnorePoolingWidths (pool.cc:197-250)
+            return numpy.array([_py.min(i * st - p + k, dim) - _py.max(i * st - p, 0) for i in range(count)], x.dtype)
+        wi = numpy.outer(widths(x.shape[2], ksize[0], stride[0], pad[0], oh), widths(x.shape[3], ksize[1], stride[1], pad[1], ow))
+        g = divide(gout, array(wi.astype(x.dtype)))
+    gcol = g.reshape((n, c, 1, 1, oh, ow)).broadcast_to((n, c, ksize[0], ksize[1], oh, ow))
+    gx = col2im(gcol, stride, pad, x.shape[2:])
+    if pad_mode == 'zero':
+        gx = gx.copy()
+        _lib.call('hipcx_divide_as', gx.desc(), _lib.make_scalar(ksize[0] * ksize[1]), gx.desc(), current_stream())
+    return gx
+
+
+# ---------------------------------------------------------------------------------------------
 # composite routines
 # ---------------------------------------------------------------------------------------------
 def lstm(c, x):

@@ -796,6 +796,141 @@ def average_pool(x, ksize, stride=None, pad=0, pad_mode='ignore'):
         return (s / widths).astype(x.dtype)
 
 
+def _col2im(col, stride, pad, out_size):
+    """native_internal::Col2Im (CX/native/col2im.cc:22-122): zero array of the padded size, `+=` per kernel offset in (r, s)
+    order, every addition rounded to the array dtype (float16 through float), padding cut off."""
+    n, c, kh, kw, h, w = col.shape
+    sh, sw = stride
+    ph, pw = pad
+    oh, ow = out_size
+    padded = np.zeros((n, c, oh + 2 * ph + sh - 1, ow + 2 * pw + sw - 1), col.dtype)
+    with np.errstate(all='ignore'):
+        for r in range(kh):
+            for q in range(kw):
+                view = padded[:, :, r:r + sh * h:sh, q:q + sw * w:sw]
+                view[...] = add(view, col[:, :, r, q])
+    return padded[:, :, ph:ph + oh, pw:pw + ow]
+
+
+def _tensordot(a, b, a_axes, b_axes):
+    """TensorDot (CX/native/tensor_dot.cc:63-99): roll, reshape to 2-D, native Dot."""
+    a, b = np.asarray(a), np.asarray(b)
+    a_keep = [i for i in range(a.ndim) if i not in a_axes]
+    b_keep = [i for i in range(b.ndim) if i not in b_axes]
+    red = int(np.prod([a.shape[i] for i in a_axes], dtype=np.int64))
+    a2 = a.transpose(a_keep + list(a_axes)).reshape(-1, red)
+    b2 = b.transpose(list(b_axes) + b_keep).reshape(red, -1)
+    return dot(a2, b2).reshape(tuple(a.shape[i] for i in a_keep) + tuple(b.shape[i] for i in b_keep))
+
+
+def conv_grad_weight(w_shape, x, gy, stride=1, pad=0, cover_all=False):
+    """NativeConvGradWeightKernel (conv.cc:91-124): Im2Col(x) then TensorDot(gy, col) over batch and output positions."""
+    x, gy = np.asarray(x), np.asarray(gy)
+    col = _windows(x, tuple(w_shape[2:]), _pair(stride), _pair(pad), cover_all, 0)
+    return _tensordot(gy, col, (0, 2, 3), (0, 4, 5))
+
+
+def conv_transpose(x, w, b=None, stride=1, pad=0, out_size=None):
+    """NativeConvTransposeKernel (conv.cc:126-160): TensorDot(w, x) over the input channels, batch axis first, Col2Im, bias."""
+    x, w = np.asarray(x), np.asarray(w)
+    stride, pad = _pair(stride), _pair(pad)
+    kh, kw = w.shape[2:]
+    if out_size is None:
+        out_size = tuple(st * (d - 1) + k - 2 * p for d, k, st, p in zip(x.shape[2:], (kh, kw), stride, pad))
+    col = _tensordot(w, x, (0,), (1,)).transpose(3, 0, 1, 2, 4, 5)
+    out = np.ascontiguousarray(_col2im(np.ascontiguousarray(col), stride, pad, _pair(out_size)))
+    if b is not None:
+        out = add(out, np.broadcast_to(np.asarray(b).reshape(1, -1, 1, 1), out.shape))
+    return out
+
+
+def var(a, axis=None, keepdims=False):
+    """Var (CX/routines/statistics.cc:147-154)."""
+    a = np.asarray(a)
+    axes = _axes_of(a, axis)
+    diff = subtract(a, np.broadcast_to(mean(a, axes, True), a.shape))
+    return mean(multiply(diff, diff), axes, keepdims)
+
+
+def batch_norm(x, gamma, beta, running_mean, running_var, eps=2e-5, decay=0.9, axis=None):
+    """GenericBatchNormKernel (CX/routines/normalization.cc:155-193), operands of one float dtype.  Returns
+    (out, new_running_mean, new_running_var, (x_mean, x_inv_std))."""
+    x = np.asarray(x)
+    dt = x.dtype
+    axes = tuple(sorted(a % x.ndim for a in ((0,) + tuple(range(2, x.ndim)) if axis is None else axis)))
+    red = tuple(1 if i in axes else d for i, d in enumerate(x.shape))
+    x_mean = mean(x, axes, True)
+    x_var = var(x, axes, True)
+    g, bt = np.asarray(gamma).reshape(red), np.asarray(beta).reshape(red)
+    B = lambda v: np.broadcast_to(v, x.shape)
+    inv_std = divide(_scalar_as(1, dt), sqrt(add(x_var, _scalar_as(eps, dt))))
+    out = add(multiply(multiply(subtract(x, B(x_mean)), B(inv_std)), B(g)), B(bt))
+    n = x.size // max(1, np.asarray(gamma).size)
+    inv_decay = 1.0 - float(decay)
+    rm = add(multiply(np.asarray(running_mean).reshape(red), _scalar_as(decay, dt)), multiply(x_mean, _scalar_as(inv_decay, dt)))
+    rv = add(multiply(np.asarray(running_var).reshape(red), _scalar_as(decay, dt)),
+             multiply(x_var, _scalar_as(inv_decay * (float(n) / max(n - 1, 1)), dt)))
+    shp = np.asarray(gamma).shape
+    return out, rm.reshape(shp), rv.reshape(shp), (x_mean, inv_std)
+
+
+def batch_norm_grad(x, gamma, gout, state, axis=None):
+    """GenericBatchNormGradKernel (CX/routines/normalization.cc:195-250): (gx, ggamma, gbeta)."""
+    x, gout = np.asarray(x), np.asarray(gout)
+    dt = x.dtype
+    x_mean, x_inv_std = state
+    axes = tuple(sorted(a % x.ndim for a in ((0,) + tuple(range(2, x.ndim)) if axis is None else axis)))
+    red = tuple(1 if i in axes else d for i, d in enumerate(x.shape))
+    B = lambda v: np.broadcast_to(v, x.shape)
+    n = x.size // max(1, np.asarray(gamma).size)
+    x_hat = multiply(subtract(x, B(x_mean)), B(x_inv_std))
+    ggamma = sum(multiply(gout, x_hat), axes, True)
+    gbeta = sum(gout, axes, True)
+    g = np.asarray(gamma).reshape(red)
+    inner = multiply(add(multiply(x_hat, B(ggamma)), B(gbeta)), _scalar_as(1.0 / n, dt))
+    gx = multiply(B(multiply(g, x_inv_std)), subtract(gout, inner))
+    shp = np.asarray(gamma).shape
+    return gx, ggamma.reshape(shp), gbeta.reshape(shp)
+
+
+def max_pool_grad(x, gout, ksize, stride=None, pad=0, cover_all=False):
+    """NativeMaxPoolGradKernel (pool.cc:97-143): ArgMax of the -inf padded windows (native tie rule), gout added at that
+    kernel offset of a zero col, Col2Im."""
+    x, gout = np.asarray(x), np.asarray(gout)
+    ksize = _pair(ksize)
+    stride = ksize if stride is None else _pair(stride)
+    pad = _pair(pad)
+    col = _windows(x, ksize, stride, pad, cover_all, _lowest(x.dtype))
+    idx = argmax(col, (2, 3))
+    taps = np.arange(ksize[0] * ksize[1]).reshape(1, 1, ksize[0], ksize[1], 1, 1)
+    gcol = np.where(idx[:, :, None, None] == taps, gout[:, :, None, None], np.zeros((), x.dtype)).astype(x.dtype)
+    return np.ascontiguousarray(_col2im(gcol, stride, pad, x.shape[2:]))
+
+
+def average_pool_grad(x, gout, ksize, stride=None, pad=0, pad_mode='ignore'):
+    """NativeAveragePoolGradKernel (pool.cc:304-346)."""
+    x, gout = np.asarray(x), np.asarray(gout)
+    ksize = _pair(ksize)
+    stride = ksize if stride is None else _pair(stride)
+    pad = _pair(pad)
+    n, c, oh, ow = gout.shape
+    g = gout
+    if pad_mode == 'ignore':
+        widths = None
+        for i in range(2):
+            d, k, st, p = x.shape[2 + i], ksize[i], stride[i], pad[i]
+            start = np.arange(gout.shape[2 + i]).astype(x.dtype) * _scalar_as(st, x.dtype) - _scalar_as(p, x.dtype)
+            end = start + _scalar_as(k, x.dtype)
+            w = (np.minimum(end, _scalar_as(d, x.dtype)) - np.maximum(start, _scalar_as(0, x.dtype))).astype(x.dtype)
+            widths = w if widths is None else (widths[:, None] * w[None, :]).astype(x.dtype)
+        g = divide(gout, np.broadcast_to(widths, gout.shape))
+    gcol = np.broadcast_to(g[:, :, None, None], (n, c, ksize[0], ksize[1], oh, ow))
+    gx = np.ascontiguousarray(_col2im(gcol, stride, pad, x.shape[2:]))
+    if pad_mode == 'zero':
+        gx = divide(gx, _scalar_as(ksize[0] * ksize[1], x.dtype))
+    return gx
+
+
 def take(a, indices, axis, mode=None):
     """NativeTakeKernel (indexing.cc:31-103): mode None/'raise' raise IndexError when out of range."""
     a = np.asarray(a)

@@ -1,0 +1,130 @@
+"""The backward / training kernels (ConvGradWeight, ConvTranspose, BatchNorm + BatchNormGrad, MaxPoolGrad, AveragePoolGrad),
+composed on the device from the forward kernels the way the reference's native backend composes them, against the CPU oracle.
+
+Bar: 1e-5 relative float32, 2e-2 float16, 1e-12 float64 for everything that goes through Dot; the pooling gradients add in
+the reference's order and are held to the same tolerances."""
+import numpy as np
+import pytest
+
+from oracle import native as O
+from helpers import assert_close, assert_exact
+
+pytestmark = pytest.mark.gpu
+
+DT = [('float32', 1e-5), ('float16', 2e-2), ('float64', 1e-12)]
+CONV_CASES = [  # N, C, H, W, K, kh, kw, stride, pad, cover_all
+    (2, 3, 9, 8, 4, 3, 3, (2, 1), (1, 2), False), (2, 16, 8, 8, 32, 3, 3, 1, 1, False), (3, 64, 7, 7, 64, 1, 1, 1, 0, False),
+    (2, 32, 10, 10, 24, 3, 3, 2, 1, True), (1, 3, 20, 20, 8, 7, 7, 2, 3, False), (2, 20, 6, 7, 9, 2, 3, (1, 2), (0, 1), False),
+    (4, 8, 12, 12, 16, 1, 1, 2, 0, False),
+]
+
+
+@pytest.mark.parametrize('dt,tol', DT)
+def test_conv_grad_weight_and_transpose(dt, tol):
+    import chainer_amd as chx
+    rng = np.random.default_rng(50)
+    for (N, C, H, W, K, kh, kw, st, pd, cv) in CONV_CASES:
+        x = rng.standard_normal((N, C, H, W)).astype(dt)
+        w = (rng.standard_normal((K, C, kh, kw)) / np.sqrt(C * kh * kw)).astype(dt)
+        y_shape = O.conv(x.astype('float32'), w.astype('float32'), None, st, pd, cv).shape
+        gy = (rng.standard_normal(y_shape) / np.sqrt(K)).astype(dt)
+        what = '%s %r' % (dt, (N, C, H, W, K, kh, kw, st, pd, cv))
+        gw = chx.conv_grad_weight(dt, w.shape, chx.array(x), chx.array(gy), st, pd, cv)
+        assert gw.shape == w.shape and gw.dtype == np.dtype(dt)
+        assert_close(gw.get(), O.conv_grad_weight(w.shape, x, gy, st, pd, cv), tol, 'conv_grad_weight ' + what)
+        gx = chx.conv_transpose(chx.array(gy), chx.array(w), None, st, pd, (H, W))
+        assert gx.shape == x.shape
+        assert_close(gx.get(), O.conv_transpose(gy, w, None, st, pd, (H, W)), tol, 'conv_transpose ' + what)
+        b = rng.standard_normal(C).astype(dt)
+        assert_close(chx.conv_transpose(chx.array(gy), chx.array(w), chx.array(b), st, pd, (H, W)).get(),
+                     O.conv_transpose(gy, w, b, st, pd, (H, W)), tol, 'conv_transpose + bias ' + what)
+    # default output size and the shape checks of the routine
+    gy = rng.standard_normal((2, 4, 5, 5)).astype(dt)
+    w = rng.standard_normal((4, 3, 3, 3)).astype(dt)
+    out = chx.conv_transpose(chx.array(gy), chx.array(w), None, 2, 1)
+    assert out.shape == (2, 3, 9, 9)
+    assert_close(out.get(), O.conv_transpose(gy, w, None, 2, 1), tol, 'default out_size')
+    with pytest.raises(chx.DimensionError):
+        chx.conv_transpose(chx.array(gy), chx.array(w[:3]), None, 2, 1)
+    with pytest.raises(chx.DimensionError):
+        chx.conv_transpose(chx.array(gy), chx.array(w), None, 2, 1, (20, 20))
+
+
+def test_conv_backward_is_the_adjoint_on_the_device():
+    """<conv(x, w), gy> = <x, conv_transpose(gy, w)> = <w, conv_grad_weight(x, gy)> with all three evaluated on the device."""
+    import chainer_amd as chx
+    rng = np.random.default_rng(51)
+    x = rng.standard_normal((4, 16, 14, 14)).astype('float32')
+    w = (rng.standard_normal((32, 16, 3, 3)) / 12).astype('float32')
+    X, Wd = chx.array(x), chx.array(w)
+    y = chx.conv(X, Wd, None, 1, 1)
+    gy = rng.standard_normal(y.shape).astype('float32')
+    G = chx.array(gy)
+    lhs = float((y.get().astype(np.float64) * gy).sum())
+    gx = chx.conv_transpose(G, Wd, None, 1, 1, (14, 14)).get().astype(np.float64)
+    gw = chx.conv_grad_weight('float32', w.shape, X, G, 1, 1).get().astype(np.float64)
+    assert abs((x * gx).sum() - lhs) <= 1e-4 * abs(lhs) + 1e-3
+    assert abs((w * gw).sum() - lhs) <= 1e-4 * abs(lhs) + 1e-3
+
+
+@pytest.mark.parametrize('dt,tol', DT)
+def test_batch_norm_training_and_grad(dt, tol):
+    import chainer_amd as chx
+    rng = np.random.default_rng(52)
+    for shape in [(8, 6, 5, 4), (16, 3, 7, 7), (32, 10)]:
+        C = shape[1]
+        x = (rng.standard_normal(shape) * 2 + 0.5).astype(dt)
+        gamma, beta = rng.uniform(0.5, 1.5, C).astype(dt), (rng.standard_normal(C) * 0.1).astype(dt)
+        rm, rv = (rng.standard_normal(C) * 0.1).astype(dt), rng.uniform(0.5, 1.5, C).astype(dt)
+        axis = (0,) if len(shape) == 2 else None
+        RM, RV = chx.array(rm), chx.array(rv)
+        out, state = chx.batch_norm(chx.array(x), chx.array(gamma), chx.array(beta), RM, RV, 2e-5, 0.9, axis)
+        o_ref, rm_ref, rv_ref, st_ref = O.batch_norm(x, gamma, beta, rm, rv, 2e-5, 0.9, axis)
+        assert_close(out.get(), o_ref, tol, 'batch_norm out %s %r' % (dt, shape))
+        assert_close(RM.get(), rm_ref, tol, 'running mean (updated in place)')
+        assert_close(RV.get(), rv_ref, tol, 'running var (updated in place)')
+        gout = rng.standard_normal(shape).astype(dt)
+        gx, gg, gb = chx.batch_norm_grad(chx.array(x), chx.array(gamma), chx.array(gout), state, axis)
+        gx_ref, gg_ref, gb_ref = O.batch_norm_grad(x, gamma, gout, st_ref, axis)
+        gtol = tol * (50 if dt == 'float16' else 20)  # the gradient cancels terms of size |gout| * n
+        assert_close(gx.get(), gx_ref, gtol, 'batch_norm gx')
+        assert_close(gg.get(), gg_ref, gtol, 'batch_norm ggamma')
+        assert_close(gb.get(), gb_ref, gtol, 'batch_norm gbeta')
+    with pytest.raises(chx.DtypeError):
+        chx.batch_norm(chx.array(np.zeros((2, 3), 'int32')), chx.array(np.ones(3, 'float32')), chx.array(np.ones(3, 'float32')),
+                       chx.array(np.ones(3, 'float32')), chx.array(np.ones(3, 'float32')), axis=(0,))
+
+
+POOL_CASES = [((2, 3, 7, 6), (3, 3), (2, 2), (1, 1), False), ((1, 2, 5, 5), (2, 3), (1, 2), (0, 1), True), ((2, 4, 8, 8), (2, 2), (2, 2), (0, 0), False),
+              ((2, 8, 14, 14), (3, 3), (2, 2), (1, 1), False), ((3, 5, 9, 9), (3, 3), (1, 1), (1, 1), False)]
+
+
+@pytest.mark.parametrize('dt,tol', DT)
+def test_pool_grads(dt, tol):
+    import chainer_amd as chx
+    rng = np.random.default_rng(53)
+    for (shape, k, s, p, cv) in POOL_CASES:
+        x = rng.integers(-4, 5, shape).astype(dt)  # ties inside windows: the ArgMax tie rule decides
+        y_shape = O.max_pool(x, k, s, p, cv).shape
+        g = rng.standard_normal(y_shape).astype(dt)
+        gx = chx.max_pool_grad(chx.array(x), chx.array(g), k, s, p, cv)
+        assert gx.shape == x.shape
+        if dt == 'float16':
+            assert_close(gx.get(), O.max_pool_grad(x, g, k, s, p, cv), tol, 'max_pool_grad %r' % (shape,))
+        else:  # same additions in the same order
+            assert_exact(gx.get(), O.max_pool_grad(x, g, k, s, p, cv), 'max_pool_grad %r' % (shape,))
+        if not cv:
+            xf = rng.standard_normal(shape).astype(dt)
+            for mode in ('zero', 'ignore'):
+                ya = O.average_pool(xf, k, s, p, mode)
+                ga = rng.standard_normal(ya.shape).astype(dt)
+                got = chx.average_pool_grad(chx.array(xf), chx.array(ga), k, s, p, mode)
+                assert_close(got.get(), O.average_pool_grad(xf, ga, k, s, p, mode), tol, 'average_pool_grad %s %r' % (mode, shape))
+
+
+def test_var_routine():
+    import chainer_amd as chx
+    rng = np.random.default_rng(54)
+    x = rng.standard_normal((6, 5, 40)).astype('float32')
+    assert_close(chx.var(chx.array(x), (0, 2)).get(), O.var(x, (0, 2)), 1e-5, 'var')
+    assert_close(chx.var(chx.array(x), 1, True).get(), O.var(x, 1, True), 1e-5, 'var keepdims')

@@ -602,3 +602,101 @@ def test_cumsum_add_at_closed_forms():
     # Linspace closed form: endpoints exact, interior from the reference's expression
     assert np.array_equal(O.linspace(0, 10, 11, True, 'float32'), np.arange(11, dtype=np.float32))
     assert O.linspace(2, 3, 1, True, 'float64')[0] == 2.0
+
+
+# ---------------------------------------------------------------------------------------------
+# backward / training kernels
+# ---------------------------------------------------------------------------------------------
+BACKWARD_CONV_CASES = [  # N, C, H, W, K, kh, kw, stride, pad, cover_all
+    (2, 3, 6, 5, 4, 3, 3, (1, 1), (1, 1), False), (1, 2, 7, 7, 3, 3, 2, (2, 1), (0, 1), False),
+    (2, 4, 5, 6, 2, 1, 1, (2, 2), (0, 0), False), (1, 3, 6, 6, 2, 3, 3, (2, 2), (1, 1), True),
+]
+
+
+@pytest.mark.parametrize('case', BACKWARD_CONV_CASES)
+def test_conv_backward_adjoint_identities(case):
+    """C: convolution is bilinear, so <conv(x, w), gy> = <x, conv_transpose(gy, w)> = <w, conv_grad_weight(x, gy)> exactly (up to
+    float64 rounding).  A transposed operand, a flipped kernel or a wrong stride / pad offset breaks the identity."""
+    N, C, H, W, K, kh, kw, st, pd, cv = case
+    rng = np.random.default_rng(41)
+    x = rng.standard_normal((N, C, H, W))
+    w = rng.standard_normal((K, C, kh, kw))
+    y = O.conv(x, w, None, st, pd, cv)
+    gy = rng.standard_normal(y.shape)
+    lhs = float((y * gy).sum())
+    gx = O.conv_transpose(gy, w, None, st, pd, (H, W))
+    assert gx.shape == x.shape
+    assert abs(float((x * gx).sum()) - lhs) <= 1e-10 * max(1.0, abs(lhs))
+    gw = O.conv_grad_weight(w.shape, x, gy, st, pd, cv)
+    assert gw.shape == w.shape
+    assert abs(float((w * gw).sum()) - lhs) <= 1e-10 * max(1.0, abs(lhs))
+    if not cv:  # default out_size is the inverse of GetConvOutDim (CX/routines/connection.cc:51-56)
+        exp = tuple(s * (d - 1) + k - 2 * p for d, k, s, p in zip(y.shape[2:], (kh, kw), st, pd))
+        assert O.conv_transpose(gy, w, None, st, pd).shape[2:] == exp
+    b = rng.standard_normal(C)
+    assert np.allclose(O.conv_transpose(gy, w, b, st, pd, (H, W)), gx + b.reshape(1, -1, 1, 1), rtol=0, atol=1e-12)
+
+
+def test_pool_backward_brute_force_and_adjoint():
+    """B + C: MaxPoolGrad against a loop that routes every gout element to the first maximum of its window (the native ArgMax
+    tie rule inside one window); AveragePoolGrad through the adjoint identity <avg_pool(x), g> = <x, avg_pool_grad(g)>."""
+    rng = np.random.default_rng(42)
+    for (shape, k, s, p, cv) in [((2, 3, 7, 6), (3, 3), (2, 2), (1, 1), False), ((1, 2, 5, 5), (2, 3), (1, 2), (0, 1), True),
+                                 ((2, 1, 6, 6), (3, 3), (3, 3), (0, 0), False)]:
+        x = rng.integers(-3, 4, shape).astype(np.float64)  # ties on purpose
+        y = O.max_pool(x, k, s, p, cv)
+        g = rng.standard_normal(y.shape)
+        ref = np.zeros_like(x)
+        N, C, H, W = shape
+        for n in range(N):
+            for c in range(C):
+                for oh in range(y.shape[2]):
+                    for ow in range(y.shape[3]):
+                        best, pos = -np.inf, None
+                        for r in range(k[0]):
+                            for q in range(k[1]):
+                                ih, iw = oh * s[0] - p[0] + r, ow * s[1] - p[1] + q
+                                v = x[n, c, ih, iw] if 0 <= ih < H and 0 <= iw < W else -np.inf
+                                if pos is None or v > best:
+                                    best, pos = v, (ih, iw)
+                        if 0 <= pos[0] < H and 0 <= pos[1] < W:
+                            ref[n, c, pos[0], pos[1]] += g[n, c, oh, ow]
+        assert np.allclose(O.max_pool_grad(x, g, k, s, p, cv), ref, rtol=0, atol=1e-12)
+    for mode in ('zero', 'ignore'):
+        for (shape, k, s, p) in [((2, 3, 7, 6), (3, 3), (2, 2), (1, 1)), ((1, 2, 8, 8), (2, 2), (2, 2), (0, 0)), ((1, 1, 5, 7), (3, 2), (1, 2), (1, 0))]:
+            x = rng.standard_normal(shape)
+            y = O.average_pool(x, k, s, p, mode)
+            g = rng.standard_normal(y.shape)
+            gx = O.average_pool_grad(x, g, k, s, p, mode)
+            assert abs(float((y * g).sum()) - float((x * gx).sum())) <= 1e-10
+
+
+def test_batch_norm_training_closed_forms():
+    """C: normalised output has per-channel mean beta and variance gamma^2 * var/(var+eps); running statistics follow
+    decay * old + (1 - decay) * batch (variance with n/(n-1)); the gradients agree with central differences in float64."""
+    rng = np.random.default_rng(43)
+    x = rng.standard_normal((4, 3, 5, 2)) * 2 + 1
+    gamma, beta = rng.uniform(0.5, 1.5, 3), rng.standard_normal(3)
+    rm, rv = rng.standard_normal(3), rng.uniform(0.5, 1.5, 3)
+    eps, decay = 2e-5, 0.9
+    out, nrm, nrv, state = O.batch_norm(x, gamma, beta, rm, rv, eps, decay)
+    m, v = x.mean(axis=(0, 2, 3)), x.var(axis=(0, 2, 3))
+    assert np.allclose(out.mean(axis=(0, 2, 3)), beta, atol=1e-12)
+    assert np.allclose(out.var(axis=(0, 2, 3)), gamma ** 2 * v / (v + eps), atol=1e-12)
+    n = 4 * 5 * 2
+    assert np.allclose(nrm, decay * rm + (1 - decay) * m, atol=1e-14)
+    assert np.allclose(nrv, decay * rv + (1 - decay) * v * n / (n - 1), atol=1e-14)
+    gout = rng.standard_normal(x.shape)
+    gx, gg, gb = O.batch_norm_grad(x, gamma, gout, state)
+    loss = lambda xx, g_, b_: float((O.batch_norm(xx, g_, b_, rm, rv, eps, decay)[0] * gout).sum())
+    h = 1e-6
+    for idx in [(0, 0, 0, 0), (3, 2, 4, 1), (1, 1, 2, 0)]:
+        xp, xm = x.copy(), x.copy()
+        xp[idx] += h
+        xm[idx] -= h
+        assert abs((loss(xp, gamma, beta) - loss(xm, gamma, beta)) / (2 * h) - gx[idx]) <= 1e-6
+    for c in range(3):
+        e = np.zeros(3)
+        e[c] = h
+        assert abs((loss(x, gamma + e, beta) - loss(x, gamma - e, beta)) / (2 * h) - gg[c]) <= 1e-6
+        assert abs((loss(x, gamma, beta + e) - loss(x, gamma, beta - e)) / (2 * h) - gb[c]) <= 1e-6
