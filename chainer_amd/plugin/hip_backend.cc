@@ -710,6 +710,20 @@ public:
 };
 HIPCX_REGISTER_KERNEL(ArgMinKernel, HipArgMinKernel)
 
+// the routines have already replaced NaNs by -inf / +inf (CX/routines/sorting.cc:96); the native NanArgMax / NanArgMin functors
+// are those of ArgMax / ArgMin (native/native_device/reduction.cc:171-226)
+class HipNanArgMaxKernel : public NanArgMaxKernel {
+public:
+    void Call(const Array& a, const Axes& axis, const Array& out) override { CallReduce(hipcx_argmax, a, axis, out); }
+};
+HIPCX_REGISTER_KERNEL(NanArgMaxKernel, HipNanArgMaxKernel)
+
+class HipNanArgMinKernel : public NanArgMinKernel {
+public:
+    void Call(const Array& a, const Axes& axis, const Array& out) override { CallReduce(hipcx_argmin, a, axis, out); }
+};
+HIPCX_REGISTER_KERNEL(NanArgMinKernel, HipNanArgMinKernel)
+
 // All / Any reduce truth values: other dtypes are cast to bool first (native/native_device/logic.cc)
 class HipAllKernel : public AllKernel {
 public:

@@ -899,6 +899,17 @@ def argmin(a, axis=None):
     return _reduce('hipcx_argmin', a, axes, out)
 
 
+def nanargmax(a, axis=None):
+    """NanArgMax (CX/routines/sorting.cc:93-126): NaNs replaced by -inf, then the ArgMax kernel (the native NanArgMaxKernel is
+    its ArgMax functor, native/native_device/reduction.cc:171-198)."""
+    return argmax(where(isnan(a), float('-inf'), a), axis)
+
+
+def nanargmin(a, axis=None):
+    """NanArgMin (CX/routines/sorting.cc): NaNs replaced by +inf, then the ArgMin kernel."""
+    return argmin(where(isnan(a), float('inf'), a), axis)
+
+
 def all(a, axis=None, keepdims=False):
     """All (CX/routines/logic.cc:79-87); the kernel casts the input to bool first (native/native_device/logic.cc)."""
     axes = _sorted_axes(axis, a.ndim)
@@ -1632,6 +1643,21 @@ def max_pool_grad(x, gout, ksize, stride=None, pad=0, cover_all=False):
     hit = equal(indices.reshape((n, c, 1, 1, oh, ow)).broadcast_to(full_shape), taps.broadcast_to(full_shape))
     gcol = where(hit, gout.reshape((n, c, 1, 1, oh, ow)).broadcast_to(full_shape), 0)
     return col2im(gcol, stride, pad, x.shape[2:])
+
+
+def max_pool_grad_grad(x, ggx, ksize, stride=None, pad=0, cover_all=False):
+    """MaxPoolGradGradKernel after the native backend (CX/native/native_device/pool.cc:147-177): the element of every window
+    of ggx at the position where x had its maximum -- Im2Col(ggx) with the kernel axes last, flattened, Take at index + offset."""
+    ksize = _pair(ksize)
+    stride = ksize if stride is None else _pair(stride)
+    pad = _pair(pad)
+    lowest = -numpy.inf if _kind(x.dtype) == 3 else (0 if x.dtype == numpy.dtype('bool') else int(numpy.iinfo(x.dtype).min))
+    indices = argmax(im2col(x, ksize, stride, pad, cover_all, lowest), (2, 3))
+    kt = ksize[0] * ksize[1]
+    total = _prod(indices.shape)
+    offset = arange(0, total * kt, kt, dtype='int64').reshape(indices.shape)
+    col = im2col(ggx, ksize, stride, pad, cover_all, lowest).transpose((0, 1, 4, 5, 2, 3))
+    return take(col.reshape((total * kt,)), add(indices, offset), 0, 'raise')
 
 
 def average_pool_grad(x, gout, ksize, stride=None, pad=0, pad_mode='ignore'):

@@ -513,6 +513,17 @@ def argmin(a, axis=None):
     return argmax(-(a.astype(np.float64)), axis)
 
 
+def nanargmax(a, axis=None):
+    """NanArgMax routine (CX/routines/sorting.cc:93-126): NaN -> -inf, then ArgMax."""
+    a = np.asarray(a)
+    return argmax(np.where(np.isnan(a), -np.inf, a).astype(a.dtype) if a.dtype.kind == 'f' else a, axis)
+
+
+def nanargmin(a, axis=None):
+    a = np.asarray(a)
+    return argmin(np.where(np.isnan(a), np.inf, a).astype(a.dtype) if a.dtype.kind == 'f' else a, axis)
+
+
 def all(a, axis=None, keepdims=False):
     """NativeAllKernel (logic.cc): input cast to bool, accum && next; order independent."""
     a = np.asarray(a).astype(bool)
@@ -905,6 +916,18 @@ def max_pool_grad(x, gout, ksize, stride=None, pad=0, cover_all=False):
     taps = np.arange(ksize[0] * ksize[1]).reshape(1, 1, ksize[0], ksize[1], 1, 1)
     gcol = np.where(idx[:, :, None, None] == taps, gout[:, :, None, None], np.zeros((), x.dtype)).astype(x.dtype)
     return np.ascontiguousarray(_col2im(gcol, stride, pad, x.shape[2:]))
+
+
+def max_pool_grad_grad(x, ggx, ksize, stride=None, pad=0, cover_all=False):
+    """NativeMaxPoolGradGradKernel (pool.cc:147-177): ggx's window element at the ArgMax position of x's window."""
+    x, ggx = np.asarray(x), np.asarray(ggx)
+    ksize = _pair(ksize)
+    stride = ksize if stride is None else _pair(stride)
+    pad = _pair(pad)
+    idx = argmax(_windows(x, ksize, stride, pad, cover_all, _lowest(x.dtype)), (2, 3))
+    col = _windows(ggx, ksize, stride, pad, cover_all, _lowest(x.dtype)).transpose(0, 1, 4, 5, 2, 3)
+    flat = col.reshape(col.shape[:4] + (-1,))
+    return np.take_along_axis(flat, idx[..., None], axis=-1)[..., 0]
 
 
 def average_pool_grad(x, gout, ksize, stride=None, pad=0, pad_mode='ignore'):

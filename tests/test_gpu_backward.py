@@ -128,3 +128,23 @@ def test_var_routine():
     x = rng.standard_normal((6, 5, 40)).astype('float32')
     assert_close(chx.var(chx.array(x), (0, 2)).get(), O.var(x, (0, 2)), 1e-5, 'var')
     assert_close(chx.var(chx.array(x), 1, True).get(), O.var(x, 1, True), 1e-5, 'var keepdims')
+
+
+def test_max_pool_grad_grad_and_nanarg():
+    import chainer_amd as chx
+    rng = np.random.default_rng(55)
+    for (shape, k, s, p, cv) in POOL_CASES:
+        x = rng.integers(-4, 5, shape).astype('float32')
+        ggx = rng.standard_normal(shape).astype('float32')
+        got = chx.max_pool_grad_grad(chx.array(x), chx.array(ggx), k, s, p, cv)
+        assert_exact(got.get(), O.max_pool_grad_grad(x, ggx, k, s, p, cv), 'max_pool_grad_grad %r' % (shape,))
+    # for tie-free x the double gradient of the gradient's own input is the pooled value itself
+    xt = rng.standard_normal((2, 3, 8, 8)).astype('float32')
+    assert_exact(chx.max_pool_grad_grad(chx.array(xt), chx.array(xt), 2, 2, 0).get(), O.max_pool(xt, 2, 2, 0), 'ggx = x gives max_pool(x)')
+    a = rng.standard_normal((5, 200)).astype('float32')
+    a[0, 3] = np.nan
+    a[1, :] = np.nan
+    a[2, 0] = np.nan
+    assert_exact(chx.nanargmax(chx.array(a), 1).get(), O.nanargmax(a, 1), 'nanargmax')
+    assert_exact(chx.nanargmin(chx.array(a), 1).get(), O.nanargmin(a, 1), 'nanargmin')
+    assert chx.nanargmax(chx.array(a), 1).get()[0] == np.nanargmax(a[0]) and chx.nanargmin(chx.array(a), 1).get()[2] == np.nanargmin(a[2])
