@@ -192,6 +192,34 @@ bool TrySmallDot(const hipcx_array* a, const hipcx_array* b, const hipcx_array* 
     p.tiles_n = static_cast<int>((N + 31) / 32);
     int64_t blocks = ((M + 31) / 32) * p.tiles_n;
     ProfileScope prof(stream, 2.0 * M * N * K, static_cast<double>(it) * (M * K + K * N + M * N));
+    static const bool rows_ok = [] { const char* e = getenv("HIPCX_SMALL_DOT_ROWS"); return e == nullptr || e[0] != '0'; }();
+    // whole-line loads regrouped through LDS pay off once the product is large enough to be bandwidth-bound (measured: the
+    // 10000-column projection of the language model gains 15 %, the 2600- and 1000-column layers lose 10 %)
+    if (rows_ok && p.a_vec && p.b_vec && 2.0 * M * N * K >= 1e9) {
+        // Waves per workgroup = ways K is split: the choice that leaves the busiest SIMD the least matrix work
+        // (wave-tiles are dealt over 4 SIMDs per CU; a wave's share is whole 128-byte steps).
+        const int64_t steps = (K * it + 127) / 128;
+        const int64_t simds = static_cast<int64_t>(NumCUs()) * 4;
+        int best_nw = 1;
+        int64_t best_cost = -1;
+        for (int nw : {1, 2, 3, 4, 6, 8}) {
+            if (nw > steps) break;
+            int64_t rounds = (blocks * nw + simds - 1) / simds;
+            int64_t cost = rounds * ((steps + nw - 1) / nw) * 8 + nw;  // + the partial-sum pass
+            if (best_cost < 0 || cost < best_cost) best_cost = cost, best_nw = nw;
+        }
+        p.nw = best_nw;
+        const int lds_bytes = best_nw * 2 * 32 * 144;
+        static const bool configured = [] {
+            HIPCX_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(SmallDotRowsKernel<T>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                8 * 2 * 32 * 144));
+            return true;
+        }();
+        (void)configured;
+        hipLaunchKernelGGL((SmallDotRowsKernel<T>), dim3(static_cast<unsigned>(blocks)), dim3(64 * best_nw), lds_bytes, stream, p);
+        CheckLaunch("small_dot_rows");
+        return true;
+    }
     hipLaunchKernelGGL((SmallDotKernel<T>), dim3(static_cast<unsigned>(blocks)), dim3(512), 0, stream, p);
     CheckLaunch("small_dot");
     return true;
