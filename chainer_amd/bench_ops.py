@@ -236,6 +236,45 @@ def section_lstm(chx, oracle, with_cpu):
         emit(section='lstm', op='cpu native 1 core, one time step', ms=round(cpu_time(lambda: cfg.lstm_lm_forward(oracle, p, ids2, np.zeros), 1.0) * 1e3, 1))
 
 
+def section_backward(chx, oracle, with_cpu):
+    """Backward / training kernels at ResNet-50 layer shapes (float16, batch 32): compositions of the forward kernels, so the
+    figures are those of Im2Col / Col2Im copies plus one matrix product -- functional, not tuned."""
+    rng = np.random.default_rng(6)
+    n, c, k, hw = 32, 256, 256, 14
+    x = chx.array(rng.standard_normal((n, c, hw, hw)).astype(np.float16))
+    w = chx.array((rng.standard_normal((k, c, 3, 3)) / np.sqrt(9 * c)).astype(np.float16))
+    gy = chx.array(rng.standard_normal((n, k, hw, hw)).astype(np.float16))
+    flops = 2.0 * n * hw * hw * k * c * 9
+    for name, fn in (('conv_grad_weight 3x3', lambda: chx.conv_grad_weight('float16', w.shape, x, gy, 1, 1)),
+                     ('conv_transpose 3x3', lambda: chx.conv_transpose(gy, w, None, 1, 1, (hw, hw))),
+                     ('conv 3x3 (forward, for scale)', lambda: chx.conv(x, w, None, 1, 1))):
+        t = device_time(fn, 5, 2)
+        emit(section='backward', op=name, shape=[n, c, hw, hw, k], us=round(t * 1e6, 1), TFLOPs=round(flops / t / 1e12, 2),
+             fp16_mfma_frac=round(flops / t / 1e12 / MFMA_PEAK['float16'], 4))
+    shape = (32, 256, 56, 56)
+    xb = chx.array(rng.standard_normal(shape).astype(np.float16))
+    gb = chx.array(rng.standard_normal(shape).astype(np.float16))
+    prm = [chx.array(rng.uniform(0.5, 1.5, 256).astype(np.float16)) for _ in range(2)]
+    rm, rv = chx.array(np.zeros(256, np.float16)), chx.array(np.ones(256, np.float16))
+    nbytes = xb.nbytes
+    out_state = []
+    t = device_time(lambda: out_state.__setitem__(slice(None), [chx.batch_norm(xb, prm[0], prm[1], rm, rv)]), 5, 2)
+    bw_row('backward', 'batch_norm (training forward, routine composition)', shape, t, 3 * nbytes, 20,
+           note='algorithmic bytes: two reads (statistics, normalise) and one write')
+    state = out_state[0][1]
+    t = device_time(lambda: chx.batch_norm_grad(xb, prm[0], gb, state), 5, 2)
+    bw_row('backward', 'batch_norm_grad (routine composition)', shape, t, 5 * nbytes, 12,
+           note='algorithmic bytes: x and gout read twice, gx written')
+    xp = chx.array(rng.standard_normal((32, 64, 112, 112)).astype(np.float16))
+    gp = chx.array(rng.standard_normal((32, 64, 56, 56)).astype(np.float16))
+    t = device_time(lambda: chx.max_pool_grad(xp, gp, 3, 2, 1), 5, 2)
+    bw_row('backward', 'max_pool_grad 3x3/2 pad 1', (32, 64, 112, 112), t, 2 * xp.nbytes + gp.nbytes)
+    xa = chx.array(rng.standard_normal((128, 2048, 7, 7)).astype(np.float16))
+    ga = chx.array(rng.standard_normal((128, 2048, 1, 1)).astype(np.float16))
+    t = device_time(lambda: chx.average_pool_grad(xa, ga, 7, 1, 0, 'zero'), 5, 2)
+    bw_row('backward', 'average_pool_grad 7x7 (global)', (128, 2048, 7, 7), t, xa.nbytes + ga.nbytes)
+
+
 def section_copy(chx, oracle, with_cpu):
     """A plain copy of known size (128 MiB read + 128 MiB written): the calibration point for HBM traffic counters."""
     x = chx.array(np.zeros(64 * 1024 * 1024, np.float16))
@@ -243,7 +282,7 @@ def section_copy(chx, oracle, with_cpu):
     bw_row('copy', 'copy float16 [67108864]', (64 * 1024 * 1024,), t, 2 * x.nbytes)
 
 
-SECTIONS = {'copy': section_copy, 'sweep': section_sweep, 'mlp': section_mlp, 'cifar': section_cifar, 'resnet_layers': section_resnet_layers, 'lstm': section_lstm}
+SECTIONS = {'copy': section_copy, 'sweep': section_sweep, 'mlp': section_mlp, 'cifar': section_cifar, 'resnet_layers': section_resnet_layers, 'lstm': section_lstm, 'backward': section_backward}
 
 
 def run(sections, cpu=None):

@@ -192,6 +192,10 @@ struct ReduceGeom {
     int64_t red_stride[kMaxDims];  // bytes
     int64_t n_out;                 // product of keep_shape
     int64_t red_len;               // product of red_shape
+    // Row kernel: the reduced sequence is red_len / seg_len dense runs of seg_len elements, seg_stride bytes apart
+    // (one run: seg_len == red_len).  Reducing N and H*W of an NCHW array for each channel is the two-level case.
+    int64_t seg_len;
+    int64_t seg_stride;
 };
 
 __device__ __forceinline__ void OutOffsets(const ReduceGeom& g, int64_t o, int64_t& in_off, int64_t& out_off) {
@@ -219,7 +223,13 @@ __global__ __launch_bounds__(kRowThreads) void RowReduceKernel(ReduceGeom g, int
     const int blk = blockIdx.x - static_cast<int>(row * blocks_per_row);
     int64_t in_off, out_off;
     OutOffsets(g, row, in_off, out_off);
-    const In* x = reinterpret_cast<const In*>(g.in + in_off);
+    const char* xbase = g.in + in_off;
+    // address of element i of the reduced sequence; groups of four never straddle a run (seg_len % 4 == 0 when there are several)
+    auto at = [&](int64_t i) -> const In* {
+        if (g.seg_stride == 0) return reinterpret_cast<const In*>(xbase) + i;  // one run (uniform branch): no division
+        const int64_t sidx = i / g.seg_len;
+        return reinterpret_cast<const In*>(xbase + sidx * g.seg_stride) + (i - sidx * g.seg_len);
+    };
 
     const int64_t L = g.red_len;
     const int64_t G = L / 4;                          // full groups
@@ -241,12 +251,13 @@ __global__ __launch_bounds__(kRowThreads) void RowReduceKernel(ReduceGeom g, int
                 struct alignas(sizeof(In) * 4) In4 {
                     In v[4];
                 };
-                In4 q = *reinterpret_cast<const In4*>(x + grp * 4);
+                In4 q = *reinterpret_cast<const In4*>(at(grp * 4));
 #pragma unroll
                 for (int j = 0; j < 4; ++j) e[j] = q.v[j];
             } else {
+                const In* xp = at(grp * 4);
 #pragma unroll
-                for (int j = 0; j < 4; ++j) e[j] = x[grp * 4 + j];
+                for (int j = 0; j < 4; ++j) e[j] = xp[j];
             }
             // (e0 . e1) . (e2 . e3): the later element is `next`
             Acc p0 = Impl::Map(e[0], grp * 4);
@@ -278,7 +289,7 @@ __global__ __launch_bounds__(kRowThreads) void RowReduceKernel(ReduceGeom g, int
         }
         // ---- the last chunk also folds the leftover elements, in order ----
         if (seg_lane == 0 && chunk == k_last) {
-            for (int64_t i = G * 4; i < L; ++i) Impl::Reduce(Impl::Map(x[i], i), acc);
+            for (int64_t i = G * 4; i < L; ++i) Impl::Reduce(Impl::Map(*at(i), i), acc);
         }
         if (chunk > k_last) acc = Impl::Empty();
         // ---- 8 chunk results per wave -> one node: balanced tree, the later operand is the accumulator ----
@@ -485,8 +496,13 @@ ReducePlan MakePlan(const hipcx_array* a, const int8_t* axis, int naxis, const h
     pl.acc_size = acc_size;
     const ReduceGeom& g = pl.g;
     const int64_t it = ItemSize(a->dtype);
-    // Row path: one contiguous run of at least 256 elements, short enough for 32-bit-safe bookkeeping.
-    if (g.n_red == 1 && g.red_stride[0] == it && g.red_len >= 256 && g.red_len < (1LL << 40) && g.n_out < (1LL << 31)) {
+    // Row path: one contiguous run of at least 256 elements -- or several such runs of a multiple of four elements at a
+    // constant pitch (e.g. the (0, 2, 3) axes of an NCHW array) -- short enough for 32-bit-safe bookkeeping.
+    const bool one_run = g.n_red == 1 && g.red_stride[0] == it;
+    const bool runs = g.n_red == 2 && g.red_stride[1] == it && g.red_shape[1] % 4 == 0 && g.red_stride[0] > 0;
+    pl.g.seg_len = runs ? g.red_shape[1] : g.red_len;
+    pl.g.seg_stride = runs ? g.red_stride[0] : 0;
+    if ((one_run || runs) && g.red_len >= 256 && g.red_len < (1LL << 40) && g.n_out < (1LL << 31)) {
         pl.row_path = true;
         int64_t L = g.red_len;
         int64_t span = kElemsPerIter;
@@ -504,6 +520,7 @@ ReducePlan MakePlan(const hipcx_array* a, const int8_t* axis, int naxis, const h
             pl.blocks_per_row = static_cast<int>(bpr);
             bool al = reinterpret_cast<uintptr_t>(g.in) % (4 * it) == 0;
             for (int d = 0; d < g.n_keep; ++d) al = al && g.keep_in_stride[d] % (4 * it) == 0;
+            al = al && g.seg_stride % (4 * it) == 0;
             pl.aligned = al;
         }
     }

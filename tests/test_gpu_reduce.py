@@ -119,3 +119,27 @@ def test_reduction_errors_and_empty():
         chx.argmax(chx.zeros((2, 0, 3), 'float32'), 1)  # "cannot compute the argmax of an empty array" (routines/sorting.cc)
     assert chx.sum(chx.zeros((2, 0, 3), 'float32'), 1).get().tolist() == [[0, 0, 0], [0, 0, 0]]
     assert chx.argmax(chx.zeros((2, 0, 3), 'float32'), 2).get().shape == (2, 0)
+
+
+@pytest.mark.parametrize('dt', ['float32', 'float16', 'int32', 'float64'])
+def test_reduce_over_batch_and_plane_of_nchw(dt):
+    """Axes (0, 2, 3) of a dense NCHW array: runs of H*W elements at a constant pitch per channel (batch-norm statistics, bias
+    gradients).  Same pairwise tree over the flattened (n, h, w) sequence as the native backend, so sums stay bit-exact."""
+    import chainer_amd as chx
+    rng = np.random.default_rng(77)
+    for shape in [(8, 6, 12, 12), (32, 16, 14, 14), (3, 5, 7, 8), (2, 4, 6, 6), (5, 3, 2, 128), (4, 7, 9, 9)]:
+        if np.dtype(dt).kind == 'f':
+            x = rng.standard_normal(shape).astype(dt)
+        else:
+            x = rng.integers(-100, 100, shape).astype(dt)
+        X = chx.array(x)
+        what = '%s %r' % (dt, shape)
+        assert_exact(chx.sum(X, (0, 2, 3)).get(), O.sum(x, (0, 2, 3)), 'sum ' + what)
+        assert_exact(chx.sum(X, (0, 2, 3), True).get(), O.sum(x, (0, 2, 3), True), 'sum keepdims ' + what)
+        assert_exact(chx.amax(X, (0, 2, 3)).get(), O.amax(x, (0, 2, 3)), 'amax ' + what)
+        assert_exact(chx.amin(X, (0, 2, 3)).get(), O.amin(x, (0, 2, 3)), 'amin ' + what)
+        # a sliced batch axis keeps the pitch constant; a sliced plane breaks the runs (generic path)
+        assert_exact(chx.sum(X[::2], (0, 2, 3)).get(), O.sum(x[::2], (0, 2, 3)), 'sum of every second image ' + what)
+        assert_exact(chx.sum(X[:, :, ::2], (0, 2, 3)).get(), O.sum(x[:, :, ::2], (0, 2, 3)), 'sum of a strided plane ' + what)
+    big = rng.standard_normal((16, 8, 56, 56)).astype(dt) if np.dtype(dt).kind == 'f' else rng.integers(-100, 100, (16, 8, 56, 56)).astype(dt)
+    assert_exact(chx.sum(chx.array(big), (0, 2, 3)).get(), O.sum(big, (0, 2, 3)), 'rows split over several workgroups')
