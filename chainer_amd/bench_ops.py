@@ -238,7 +238,8 @@ def section_lstm(chx, oracle, with_cpu):
 
 def section_backward(chx, oracle, with_cpu):
     """Backward / training kernels at ResNet-50 layer shapes (float16, batch 32): compositions of the forward kernels, so the
-    figures are those of Im2Col / Col2Im copies plus one matrix product -- functional, not tuned."""
+    figures are those of Im2Col / Col2Im copies plus one matrix product -- functional, not tuned.  Timed as HIP-graph replays
+    (each composition is 10-25 kernel launches; issued eagerly from Python it would be host-bound)."""
     rng = np.random.default_rng(6)
     n, c, k, hw = 32, 256, 256, 14
     x = chx.array(rng.standard_normal((n, c, hw, hw)).astype(np.float16))
@@ -248,7 +249,7 @@ def section_backward(chx, oracle, with_cpu):
     for name, fn in (('conv_grad_weight 3x3', lambda: chx.conv_grad_weight('float16', w.shape, x, gy, 1, 1)),
                      ('conv_transpose 3x3', lambda: chx.conv_transpose(gy, w, None, 1, 1, (hw, hw))),
                      ('conv 3x3 (forward, for scale)', lambda: chx.conv(x, w, None, 1, 1))):
-        t = device_time(fn, 5, 2)
+        t = graph_time(fn, 5)
         emit(section='backward', op=name, shape=[n, c, hw, hw, k], us=round(t * 1e6, 1), TFLOPs=round(flops / t / 1e12, 2),
              fp16_mfma_frac=round(flops / t / 1e12 / MFMA_PEAK['float16'], 4))
     shape = (32, 256, 56, 56)
@@ -258,20 +259,21 @@ def section_backward(chx, oracle, with_cpu):
     rm, rv = chx.array(np.zeros(256, np.float16)), chx.array(np.ones(256, np.float16))
     nbytes = xb.nbytes
     out_state = []
-    t = device_time(lambda: out_state.__setitem__(slice(None), [chx.batch_norm(xb, prm[0], prm[1], rm, rv)]), 5, 2)
+    out_state[:] = [chx.batch_norm(xb, prm[0], prm[1], rm, rv)]
+    t = graph_time(lambda: chx.batch_norm(xb, prm[0], prm[1], rm, rv), 5)
     bw_row('backward', 'batch_norm (training forward, routine composition)', shape, t, 3 * nbytes, 20,
            note='algorithmic bytes: two reads (statistics, normalise) and one write')
     state = out_state[0][1]
-    t = device_time(lambda: chx.batch_norm_grad(xb, prm[0], gb, state), 5, 2)
+    t = graph_time(lambda: chx.batch_norm_grad(xb, prm[0], gb, state), 5)
     bw_row('backward', 'batch_norm_grad (routine composition)', shape, t, 5 * nbytes, 12,
            note='algorithmic bytes: x and gout read twice, gx written')
     xp = chx.array(rng.standard_normal((32, 64, 112, 112)).astype(np.float16))
     gp = chx.array(rng.standard_normal((32, 64, 56, 56)).astype(np.float16))
-    t = device_time(lambda: chx.max_pool_grad(xp, gp, 3, 2, 1), 5, 2)
+    t = graph_time(lambda: chx.max_pool_grad(xp, gp, 3, 2, 1), 5)
     bw_row('backward', 'max_pool_grad 3x3/2 pad 1', (32, 64, 112, 112), t, 2 * xp.nbytes + gp.nbytes)
     xa = chx.array(rng.standard_normal((128, 2048, 7, 7)).astype(np.float16))
     ga = chx.array(rng.standard_normal((128, 2048, 1, 1)).astype(np.float16))
-    t = device_time(lambda: chx.average_pool_grad(xa, ga, 7, 1, 0, 'zero'), 5, 2)
+    t = graph_time(lambda: chx.average_pool_grad(xa, ga, 7, 1, 0, 'zero'), 5)
     bw_row('backward', 'average_pool_grad 7x7 (global)', (128, 2048, 7, 7), t, xa.nbytes + ga.nbytes)
 
 

@@ -889,17 +889,58 @@ int hipcx_conv_bn_act(const hipcx_array* x, const hipcx_array* w, const hipcx_ar
     });
 }
 
+namespace {
+// The MFMA kernels read both operands with the reduction index k as the unit-stride axis, rows 16-byte aligned.  An operand
+// laid out otherwise (a plain row-major b, a transposed a, odd pitches) is first copied into that layout -- one pass over
+// the operand instead of an element-gather kernel for the whole product.
+struct DotStaging {
+    bool a = false, b = false;
+    int64_t kpad = 0;       // staged row pitch, elements (k rounded up to 16 bytes)
+    size_t a_bytes = 0, b_bytes = 0;
+};
+
+bool OperandIsFast(const void* ptr, int64_t line_stride_bytes, int64_t k_stride_bytes, int64_t k, int64_t it) {
+    // 8-byte granules are enough for the fast kernel (its 16-byte variant is picked when everything is 16-byte aligned)
+    return k_stride_bytes == it && reinterpret_cast<uintptr_t>(ptr) % 8 == 0 && line_stride_bytes % 8 == 0 && line_stride_bytes >= 0 &&
+           (k * it) % 8 == 0;
+}
+
+DotStaging PlanDotStaging(const hipcx_array* a, const hipcx_array* b, const hipcx_array* out) {
+    DotStaging st;
+    if (a == nullptr || b == nullptr || out == nullptr || a->ndim != 2 || b->ndim != 2) return st;
+    if (out->dtype != HIPCX_FLOAT16 && out->dtype != HIPCX_FLOAT32) return st;
+    static const bool enabled = [] { const char* e = getenv("HIPCX_DOT_STAGE"); return e == nullptr || e[0] != '0'; }();
+    const int64_t it = ItemSize(out->dtype);
+    const int64_t m = a->shape[0], k = a->shape[1], n = b->shape[1];
+    if (!enabled || m == 0 || n == 0 || k == 0) return st;
+    const bool a_fast = OperandIsFast(a->data, a->strides[0], a->strides[1], k, it);
+    const bool b_fast = OperandIsFast(b->data, b->strides[1], b->strides[0], k, it);
+    if (a_fast && b_fast) return st;
+    // worth it only when the product is large against the copies; small outputs have their own kernel (any layout)
+    if (2.0 * m * n * k < 2e8) return st;
+    if (((m + 127) / 128) * ((n + 127) / 128) < 128 && k >= 64) return st;
+    const int64_t epv = 16 / it;
+    st.kpad = (k + epv - 1) / epv * epv;
+    // a changed pitch on one side needs the same (zero-padded) k extent on the other
+    st.a = !a_fast || st.kpad != k;
+    st.b = !b_fast || st.kpad != k;
+    st.a_bytes = st.a ? RoundUpTo(static_cast<size_t>(m * st.kpad * it), 256) : 0;
+    st.b_bytes = st.b ? RoundUpTo(static_cast<size_t>(n * st.kpad * it), 256) : 0;
+    return st;
+}
+}  // namespace
+
 size_t hipcx_dot_workspace_size(const hipcx_array* a, const hipcx_array* b, const hipcx_array* out) {
-    (void)a;
-    (void)b;
-    (void)out;
-    return 0;
+    try {
+        DotStaging st = PlanDotStaging(a, b, out);
+        return st.a_bytes + st.b_bytes;
+    } catch (...) {
+        return 0;
+    }
 }
 
 int hipcx_dot(const hipcx_array* a, const hipcx_array* b, const hipcx_array* out, void* workspace, size_t workspace_bytes,
               void* stream) {
-    (void)workspace;
-    (void)workspace_bytes;
     return Guard([&] {
         ValidateArray(a, "a");
         ValidateArray(b, "b");
@@ -947,6 +988,39 @@ int hipcx_dot(const hipcx_array* a, const hipcx_array* b, const hipcx_array* out
             p.M = m;
             p.Kg = static_cast<int>(k);
         };
+        // operands in another layout than the MFMA kernels read are staged in the workspace first
+        hipcx_array a_st = *a, b_st = *b;
+        if (out->dtype == a->dtype && out->dtype == b->dtype) {
+            DotStaging plan = PlanDotStaging(a, b, out);
+            if (plan.a || plan.b) {
+                HIPCX_REQUIRE(workspace != nullptr && workspace_bytes >= plan.a_bytes + plan.b_bytes, HIPCX_CHAINERX_ERROR,
+                              "dot: workspace of " + std::to_string(plan.a_bytes + plan.b_bytes) + " bytes required (hipcx_dot_workspace_size)");
+                HIPCX_REQUIRE(reinterpret_cast<uintptr_t>(workspace) % 16 == 0, HIPCX_CHAINERX_ERROR, "workspace must be 16-byte aligned");
+                const int64_t it = ItemSize(out->dtype);
+                char* ws = static_cast<char*>(workspace);
+                auto stage = [&](const hipcx_array* src, bool transposed, int64_t lines, char* dst, hipcx_array& view) {
+                    // lines = rows of a, or columns of b; the staged matrix is [lines][kpad]
+                    const int64_t sl = src->strides[transposed ? 1 : 0] / it, sk = src->strides[transposed ? 0 : 1] / it;
+                    HIPCX_REQUIRE(src->strides[0] % it == 0 && src->strides[1] % it == 0, HIPCX_NOT_IMPLEMENTED_ERROR,
+                                  "dot: byte strides must be multiples of the item size");
+                    if (out->dtype == HIPCX_FLOAT16) {
+                        StageMatrix<half_t>(static_cast<const half_t*>(src->data), sl, sk, reinterpret_cast<half_t*>(dst), plan.kpad, lines, k, st);
+                    } else {
+                        StageMatrix<float>(static_cast<const float*>(src->data), sl, sk, reinterpret_cast<float*>(dst), plan.kpad, lines, k, st);
+                    }
+                    view.data = dst;
+                    view.shape[transposed ? 1 : 0] = lines;
+                    view.shape[transposed ? 0 : 1] = plan.kpad;
+                    view.strides[transposed ? 1 : 0] = plan.kpad * it;
+                    view.strides[transposed ? 0 : 1] = it;
+                };
+                if (plan.a) stage(a, false, m, ws, a_st);
+                if (plan.b) stage(b, true, n, ws + plan.a_bytes, b_st);
+                k = plan.kpad;
+            }
+        }
+        a = &a_st;
+        b = &b_st;
         if (out->dtype == HIPCX_FLOAT16) {
             if (TrySmallDot<half_t>(a, b, out, st)) return;
             IGemmArgs<half_t> p{};

@@ -97,4 +97,39 @@ inline void LaunchToChannelsLast(const ToChannelsLastArgs& a, hipStream_t stream
     CheckLaunch("to_channels_last");
 }
 
+// dst[r][c] (dense, row pitch dst_pitch elements, columns c >= cols zero-filled up to dst_pitch) = src[r * sr + c * sc]:
+// brings a matrix operand whose reduction axis is not the unit-stride one into the layout the MFMA kernels read.
+// 64x64 tiles through LDS; reads walk the source's faster axis, writes walk dst rows.
+template <typename T>
+__global__ __launch_bounds__(256) void StageMatrixKernel(const T* src, int64_t sr, int64_t sc, T* dst, int64_t dst_pitch, int rows, int cols,
+                                                         int read_rows_fast) {
+    constexpr int TILE = 64;
+    __shared__ T tile[TILE][TILE + 2];
+    const int r0 = blockIdx.y * TILE, c0 = blockIdx.x * TILE;
+    const int tid = threadIdx.x;
+    for (int e = tid; e < TILE * TILE; e += 256) {
+        // consecutive threads take consecutive rows when the source is contiguous along r, consecutive columns otherwise
+        const int rl = read_rows_fast ? e % TILE : e / TILE;
+        const int cl = read_rows_fast ? e / TILE : e % TILE;
+        const int r = r0 + rl, c = c0 + cl;
+        tile[rl][cl] = (r < rows && c < cols) ? src[r * sr + c * sc] : T(0);
+    }
+    __syncthreads();
+    for (int e = tid; e < TILE * TILE; e += 256) {
+        const int rl = e / TILE, cl = e % TILE;
+        const int r = r0 + rl, c = c0 + cl;
+        if (r < rows && c < dst_pitch) dst[r * dst_pitch + c] = tile[rl][cl];
+    }
+}
+
+template <typename T>
+void StageMatrix(const T* src, int64_t sr, int64_t sc, T* dst, int64_t dst_pitch, int64_t rows, int64_t cols, hipStream_t stream) {
+    const int64_t asr = sr < 0 ? -sr : sr, asc = sc < 0 ? -sc : sc;
+    dim3 grid(static_cast<unsigned>((dst_pitch + 63) / 64), static_cast<unsigned>((rows + 63) / 64));
+    HIPCX_REQUIRE(grid.y < 65536, HIPCX_NOT_IMPLEMENTED_ERROR, "matrix operand has too many rows to stage in one launch");
+    hipLaunchKernelGGL((StageMatrixKernel<T>), grid, dim3(256), 0, stream, src, sr, sc, dst, dst_pitch, static_cast<int>(rows),
+                       static_cast<int>(cols), asr < asc ? 1 : 0);
+    CheckLaunch("stage_matrix");
+}
+
 }  // namespace hipcx

@@ -1303,12 +1303,27 @@ def tensordot(a, b, a_axes, b_axes, out_dtype=None):
 
 
 def conv_grad_weight(w_dtype, w_shape, x, gy, stride=1, pad=0, cover_all=False):
-    """ConvGradWeightKernel as the native backend runs it (CX/native/native_device/conv.cc:91-124): Im2Col(x), then
-    TensorDot(gy, col) over the batch and the output positions -> gw[K, C, kh, kw]."""
+    """ConvGradWeightKernel after the native backend (CX/native/native_device/conv.cc:91-124): Im2Col(x), then TensorDot(gy, col)
+    over the batch and the output positions -> gw[K, C, kh, kw].  The same two matrices meet in the same Dot; only the col is
+    laid out [C, kh, kw, N, oh, ow] so that both Dot operands have the reduction index (n, oh, ow) as their unit-stride axis
+    (the MFMA kernel's layout) and no transposed copy of the col is needed."""
     if x.ndim != 4:
         raise _lib.ChainerxNotImplementedError('only 2-D convolution is on the supported path')
-    col = im2col(x, tuple(w_shape[2:]), _pair(stride), _pair(pad), cover_all, 0)
-    return tensordot(gy, col, (0, 2, 3), (0, 4, 5), w_dtype)
+    (kh, kw), (sh, sw), (ph, pw) = tuple(w_shape[2:]), _pair(stride), _pair(pad)
+    n, c, h, w = x.shape
+    oh = conv_out_dim(h, kh, sh, ph, cover_all)
+    ow = conv_out_dim(w, kw, sw, pw, cover_all)
+    if gy.shape != (n, w_shape[0], oh, ow):
+        raise _lib.DimensionError('gy has the wrong shape')
+    xp = zeros((n, c, h + 2 * ph + (sh - 1 if cover_all else 0), w + 2 * pw + (sw - 1 if cover_all else 0)), x.dtype)
+    _copy_into(xp[:, :, ph:ph + h, pw:pw + w], x)
+    col_t = ndarray.empty((c, kh, kw, n, oh, ow), x.dtype)
+    for r in range(kh):
+        for q in range(kw):
+            _copy_into(col_t[:, r, q], xp[:, :, r:r + sh * oh:sh, q:q + sw * ow:sw].transpose((1, 0, 2, 3)))
+    gy_t = gy.transpose((1, 0, 2, 3)).reshape((w_shape[0], n * oh * ow))
+    gw = dot(gy_t, col_t.reshape((c * kh * kw, n * oh * ow)).T, w_dtype)
+    return gw.reshape(tuple(w_shape))
 
 
 def conv_transpose(x, w, b=None, stride=1, pad=0, out_size=None, out_dtype=None):
@@ -1564,8 +1579,13 @@ def conv_transpose(x, w, b=None, stride=1, pad=0, out_size=None, out_dtype=None)
             if d != conv_out_dim(o, k, st, p, False) and d != conv_out_dim(o, k, st, p, True):
                 raise _lib.DimensionError('Output dims %r is incosistent.' % (out_size,))
     dt = numpy.dtype(out_dtype) if out_dtype is not None else (result_type(x, w, b) if b is not None else result_type(x, w))
-    col = tensordot(w, x, (0,), (1,), dt)                 # [C_out, kh, kw, N, H, W]
-    col = col.transpose((3, 0, 1, 2, 4, 5))                # batch axis rolled to the top
+    # TensorDot(w, x) over the input channels; x goes in channels-last so that both Dot operands have the reduction index as
+    # their unit-stride axis
+    n, ci, h, wd = x.shape
+    w2 = w.transpose((1, 2, 3, 0)).reshape((w.shape[1] * kh * kw, ci))
+    x2 = x.transpose((0, 2, 3, 1)).reshape((n * h * wd, ci))
+    col = dot(w2, x2.T, dt).reshape((w.shape[1], kh, kw, n, h, wd))   # [C_out, kh, kw, N, H, W]
+    col = col.transpose((3, 0, 1, 2, 4, 5))                            # batch axis rolled to the top
     out = col2im(col, stride, pad, out_size)
     if b is not None:
         bb = b.astype(dt, False).reshape((1, -1, 1, 1)).broadcast_to(out.shape)

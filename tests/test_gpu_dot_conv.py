@@ -130,3 +130,25 @@ def test_conv_linearity_at_resnet_layer_size():
     delta = np.zeros((256, 256, 3, 3), 'float16')
     delta[np.arange(256), np.arange(256), 1, 1] = 1
     assert np.array_equal(chx.conv(X, chx.array(delta), None, 1, 1).get(), x)
+
+
+@pytest.mark.parametrize('dt,tol', DT)
+def test_dot_operand_layouts_large(dt, tol):
+    """Products large enough for the tiled MFMA kernel with every operand layout Dot accepts without a copy in the reference
+    (native/native_device/dot.cc:51-77): row-major and transposed views on either side, odd reduction lengths, padded pitches."""
+    import chainer_amd as chx
+    rng = np.random.default_rng(9)
+    for (m, k, n) in [(1200, 100, 1800), (1200, 101, 1800), (1500, 64, 1300)]:
+        a = (rng.standard_normal((m, k)) / np.sqrt(k)).astype(dt)
+        b = rng.standard_normal((k, n)).astype(dt)
+        ref = O.dot(a, b)
+        A_row, B_row = chx.array(a), chx.array(b)
+        A_t = chx.array(np.ascontiguousarray(a.T)).T          # unit stride along m
+        B_t = chx.array(np.ascontiguousarray(b.T)).T          # unit stride along k
+        for la, A in (('a row-major', A_row), ('a transposed view', A_t)):
+            for lb, B in (('b row-major', B_row), ('b transposed view', B_t)):
+                assert_close(chx.dot(A, B).get(), ref, tol, 'dot %s %s, %s, %s' % (dt, (m, k, n), la, lb))
+        # padded parents: pitches that are no multiple of the row length
+        ap = padded((m, k), a, 1, dt)
+        bp = padded((k, n), b, 1, dt)
+        assert_close(chx.dot(upload_view(chx, ap), upload_view(chx, bp)).get(), ref, tol, 'dot of padded operands %r' % ((m, k, n),))
