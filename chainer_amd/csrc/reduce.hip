@@ -408,6 +408,100 @@ __global__ __launch_bounds__(256) void GenericReduceKernel(ReduceGeom g) {
 }
 
 // ---------------------------------------------------------------------------------------------
+// Column kernels: one strided reduced axis, few outputs against its length (sums over the batch axis, bias gradients).
+// The reduced sequence is cut into `nslices` aligned slices of 2^level 32-element blocks.  Pass 1: one thread per
+// (slice, output), outputs fastest (coalesced for an inner kept axis), runs the reference loop over its slice -- whose
+// result is exactly the node the sequential binary counter would hold for those blocks.  Pass 2: one thread per output
+// pushes the slice nodes through the counter, then walks on through the blocks after the last slice (at least one is
+// always left, so the tail and the final fold happen exactly where the reference has them).
+// ---------------------------------------------------------------------------------------------
+template <typename Impl>
+__global__ __launch_bounds__(256) void ColumnSliceKernel(ReduceGeom g, int level, int nslices, void* partials) {
+    using In = typename Impl::In;
+    using Acc = typename Impl::Acc;
+    const int64_t t = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (t >= g.n_out * nslices) return;
+    const int64_t slice = t / g.n_out;
+    const int64_t o = t - slice * g.n_out;
+    int64_t in_off, out_off;
+    OutOffsets(g, o, in_off, out_off);
+    const int64_t stride = g.red_stride[0];
+    const int64_t count = static_cast<int64_t>(32) << level;
+    const int64_t i_begin = slice * count;
+    const char* ptr = g.in + in_off + i_begin * stride;
+    Acc accum = Impl::Identity();
+    Acc tree[32];
+    for (int64_t r = 0; r < count; r += 4) {
+        if (r != 0 && r % 32 == 0) {
+            int lvl = 0;
+            for (int64_t k = r >> 1; k % 32 == 0; k >>= 1, ++lvl) Impl::Reduce(tree[lvl], accum);
+            tree[lvl] = accum;
+            accum = Impl::Identity();
+        }
+        const int64_t i = i_begin + r;
+        Acc p0 = Impl::Map(*reinterpret_cast<const In*>(ptr), i);
+        Impl::Reduce(Impl::Map(*reinterpret_cast<const In*>(ptr + stride), i + 1), p0);
+        Acc p1 = Impl::Map(*reinterpret_cast<const In*>(ptr + 2 * stride), i + 2);
+        Impl::Reduce(Impl::Map(*reinterpret_cast<const In*>(ptr + 3 * stride), i + 3), p1);
+        Impl::Reduce(p1, p0);
+        Impl::Reduce(p0, accum);
+        ptr += 4 * stride;
+    }
+    for (int lvl = 0; lvl < level; ++lvl) Impl::Reduce(tree[lvl], accum);  // 2^level blocks: every lower level is pending
+    reinterpret_cast<Acc*>(partials)[slice * g.n_out + o] = accum;
+}
+
+template <typename Impl>
+__global__ __launch_bounds__(256) void ColumnFinishKernel(ReduceGeom g, int level, int nslices, const void* partials) {
+    using In = typename Impl::In;
+    using Acc = typename Impl::Acc;
+    const int64_t o = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (o >= g.n_out) return;
+    int64_t in_off, out_off;
+    OutOffsets(g, o, in_off, out_off);
+    const int64_t stride = g.red_stride[0];
+    const Acc* part = reinterpret_cast<const Acc*>(partials);
+    Acc tree[48];
+    Acc accum;
+    for (int s = 0; s < nslices; ++s) {  // the boundary merges of the reference at the end of every slice
+        accum = part[static_cast<int64_t>(s) * g.n_out + o];
+        int lvl = level;
+        for (int t = s; t & 1; t >>= 1, ++lvl) Impl::Reduce(tree[lvl], accum);
+        tree[lvl] = accum;
+    }
+    const int64_t len = g.red_len;
+    const int64_t main_len = len - (len % 4);
+    const int64_t i0 = static_cast<int64_t>(nslices) * (static_cast<int64_t>(32) << level);
+    const char* ptr = g.in + in_off + i0 * stride;
+    int64_t i = i0;
+    accum = Impl::Identity();
+    while (i < main_len) {
+        if (i != i0 && i % 32 == 0) {
+            int lvl = 0;
+            for (int64_t k = i >> 1; k % 32 == 0; k >>= 1, ++lvl) Impl::Reduce(tree[lvl], accum);
+            tree[lvl] = accum;
+            accum = Impl::Identity();
+        }
+        Acc p0 = Impl::Map(*reinterpret_cast<const In*>(ptr), i);
+        Impl::Reduce(Impl::Map(*reinterpret_cast<const In*>(ptr + stride), i + 1), p0);
+        Acc p1 = Impl::Map(*reinterpret_cast<const In*>(ptr + 2 * stride), i + 2);
+        Impl::Reduce(Impl::Map(*reinterpret_cast<const In*>(ptr + 3 * stride), i + 3), p1);
+        Impl::Reduce(p1, p0);
+        Impl::Reduce(p0, accum);
+        ptr += 4 * stride;
+        i += 4;
+    }
+    for (; i < len; ++i, ptr += stride) Impl::Reduce(Impl::Map(*reinterpret_cast<const In*>(ptr), i), accum);
+    {
+        int lvl = 0;
+        for (int64_t k = (len / 4 - 1) / 8; k > 0; k >>= 1, ++lvl) {
+            if (k & 1) Impl::Reduce(tree[lvl], accum);
+        }
+    }
+    *reinterpret_cast<typename Impl::Out*>(g.out + out_off) = Impl::MapOut(accum);
+}
+
+// ---------------------------------------------------------------------------------------------
 // Host side
 // ---------------------------------------------------------------------------------------------
 struct ReducePlan {
@@ -417,6 +511,9 @@ struct ReducePlan {
     int64_t span = 0;
     int blocks_per_row = 1;
     size_t acc_size = 0;
+    bool column_path = false;
+    int col_level = 0;    // a slice is 2^col_level blocks of 32 elements
+    int col_slices = 0;
 };
 
 ReduceGeom MakeGeom(const hipcx_array* a, const int8_t* axis, int naxis, const hipcx_array* out) {
@@ -524,10 +621,36 @@ ReducePlan MakePlan(const hipcx_array* a, const int8_t* axis, int naxis, const h
             pl.aligned = al;
         }
     }
+    // Column path: one strided reduced axis that is long against the number of outputs (one thread per output would walk it alone).
+    if (!pl.row_path && g.n_red == 1 && g.red_len >= 512 && g.n_out > 0 && g.n_out < (1LL << 28)) {
+        const int64_t main_len = g.red_len - g.red_len % 4;
+        const int64_t nblocks = (main_len + 31) / 32;
+        // Serial work of the longest thread: a slice in pass 1 (times the rounds the chip needs for all slice threads), then
+        // in pass 2 the slice nodes plus the blocks behind the last slice.  Take the slice size that minimises it.
+        const int64_t resident = static_cast<int64_t>(NumCUs()) * 2048;
+        int best_level = -1;
+        int64_t best_cost = g.red_len;  // the generic kernel's: one thread walks everything
+        for (int level = 0; level < 24; ++level) {
+            const int64_t slices = (nblocks - 1) >> level;  // at least one block stays behind the last slice
+            if (slices < 2) break;
+            if (slices > (1 << 20) || g.n_out * slices >= (1LL << 36)) continue;
+            const int64_t slice_len = static_cast<int64_t>(32) << level;
+            const int64_t rounds = (g.n_out * slices + resident - 1) / resident;
+            const int64_t left = g.red_len - slices * slice_len;
+            const int64_t cost = slice_len * rounds + slices + left;
+            if (cost < best_cost) best_cost = cost, best_level = level;
+        }
+        if (best_level >= 0 && 2 * best_cost <= g.red_len) {
+            pl.column_path = true;
+            pl.col_level = best_level;
+            pl.col_slices = static_cast<int>((nblocks - 1) >> best_level);
+        }
+    }
     return pl;
 }
 
 size_t WorkspaceBytes(const ReducePlan& pl) {
+    if (pl.column_path) return static_cast<size_t>(pl.g.n_out) * pl.col_slices * pl.acc_size;
     if (!pl.row_path || pl.blocks_per_row == 1) return 0;
     return static_cast<size_t>(pl.g.n_out) * pl.blocks_per_row * pl.acc_size;
 }
@@ -556,6 +679,20 @@ void Run(const hipcx_array* a, const int8_t* axis, int naxis, const hipcx_array*
                                workspace);
             CheckLaunch("row_reduce_finalize");
         }
+        return;
+    }
+    if (pl.column_path) {
+        size_t need = WorkspaceBytes(pl);
+        HIPCX_REQUIRE(workspace != nullptr && workspace_bytes >= need, HIPCX_CHAINERX_ERROR,
+                      "reduction workspace too small: need " + std::to_string(need) + " bytes");
+        HIPCX_REQUIRE(reinterpret_cast<uintptr_t>(workspace) % 16 == 0, HIPCX_CHAINERX_ERROR, "workspace must be 16-byte aligned");
+        const int64_t threads = g.n_out * pl.col_slices;
+        hipLaunchKernelGGL((ColumnSliceKernel<Impl>), dim3(static_cast<unsigned>((threads + 255) / 256)), dim3(256), 0, stream, g, pl.col_level,
+                           pl.col_slices, workspace);
+        CheckLaunch("column_reduce_slices");
+        hipLaunchKernelGGL((ColumnFinishKernel<Impl>), dim3(static_cast<unsigned>((g.n_out + 255) / 256)), dim3(256), 0, stream, g, pl.col_level,
+                           pl.col_slices, workspace);
+        CheckLaunch("column_reduce_finish");
         return;
     }
     int64_t blocks = (g.n_out + 255) / 256;

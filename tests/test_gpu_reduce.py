@@ -143,3 +143,39 @@ def test_reduce_over_batch_and_plane_of_nchw(dt):
         assert_exact(chx.sum(X[:, :, ::2], (0, 2, 3)).get(), O.sum(x[:, :, ::2], (0, 2, 3)), 'sum of a strided plane ' + what)
     big = rng.standard_normal((16, 8, 56, 56)).astype(dt) if np.dtype(dt).kind == 'f' else rng.integers(-100, 100, (16, 8, 56, 56)).astype(dt)
     assert_exact(chx.sum(chx.array(big), (0, 2, 3)).get(), O.sum(big, (0, 2, 3)), 'rows split over several workgroups')
+
+
+@pytest.mark.parametrize('dt', ['float32', 'float16', 'int32', 'float64', 'bool'])
+def test_reduce_over_a_long_strided_axis(dt):
+    """A long reduced axis that is not the contiguous one (sums over the batch axis, bias gradients of a linear layer): the
+    sequence is cut into aligned slices that run in parallel and are merged through the native backend's binary counter, so every
+    result stays bit-identical to the sequential tree -- including the tie and NaN choices of ArgMax / ArgMin."""
+    import chainer_amd as chx
+    rng = np.random.default_rng(91)
+    cases = [((4096, 512), 0), ((100003, 64), 0), ((5000, 33), 0), ((513, 7), 0), ((1027, 300), 0), ((640, 3), 0), ((20001, 3, 5), 0),
+             ((4, 9002, 6), 1), ((2049, 1), 0), ((70000, 2), 0)]
+    for shape, axis in cases:
+        if dt == 'bool':
+            x = rng.random(shape) > 0.5
+        elif np.dtype(dt).kind == 'f':
+            x = rng.integers(0, 6, shape).astype(dt) if shape[0] == 5000 else rng.standard_normal(shape).astype(dt)
+            if shape[0] == 1027:
+                x[rng.random(shape) < 0.01] = np.nan
+        else:
+            x = rng.integers(-100, 100, shape).astype(dt)
+        X = chx.array(x)
+        what = '%s %r axis=%d' % (dt, shape, axis)
+        assert_exact(chx.sum(X, axis).get(), O.sum(x, axis), 'sum ' + what)
+        assert_exact(chx.sum(X, axis, True).get(), O.sum(x, axis, True), 'sum keepdims ' + what)
+        assert_exact(chx.amax(X, axis).get(), O.amax(x, axis), 'amax ' + what)
+        assert_exact(chx.amin(X, axis).get(), O.amin(x, axis), 'amin ' + what)
+        assert_exact(chx.argmax(X, axis).get(), O.argmax(x, axis), 'argmax ' + what)
+        assert_exact(chx.argmin(X, axis).get(), O.argmin(x, axis), 'argmin ' + what)
+        if dt == 'bool':
+            assert_exact(chx.all(X, axis).get(), O.all(x, axis), 'all ' + what)
+            assert_exact(chx.any(X, axis).get(), O.any(x, axis), 'any ' + what)
+    if dt != 'bool':  # a transposed view: the reduced axis is the contiguous one of the base array's other axis
+        x = rng.standard_normal((48, 3000)).astype(dt) if np.dtype(dt).kind == 'f' else rng.integers(-100, 100, (48, 3000)).astype(dt)
+        X = chx.array(x)
+        assert_exact(chx.sum(X[:, ::3].T, 1).get(), O.sum(x[:, ::3].T, 1), 'sum over the strided axis of a view')
+        assert_exact(chx.sum(X[:, ::3], 1).get(), O.sum(x[:, ::3], 1), 'sum over a stepped axis')
