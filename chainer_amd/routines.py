@@ -1476,27 +1476,6 @@ def take(a, indices, axis, mode=None):
     return out
 
 
-def add_at(a, indices, axis, b, mode=None):
-    """AddAt kernel call as Take's backward issues it (CX/routines/indexing.cc:147-169): a copy of a with b added at the
-    indexed positions of `axis`; repeated indices accumulate in index order."""
-    if _kind(indices.dtype) not in (1, 2):
-        raise _lib.DtypeError('Only arrays of integer dtype can be used as indices.')
-    axis = _normalize_axis(axis, a.ndim)
-    if b.shape != a.shape[:axis] + indices.shape + a.shape[axis + 1:]:
-        raise _lib.DimensionError('b has the wrong shape')
-    out = ndarray.empty(a.shape, a.dtype)
-    m = _BOUNDS[mode]
-    flag = None
-    flag_ptr = None
-    if m in (0, 1):
-        flag = zeros((1,), 'int32')
-        flag_ptr = ctypes.cast(ctypes.c_void_p(flag.data_ptr), ctypes.POINTER(ctypes.c_int32))
-    _lib.call('hipcx_add_at', a.desc(), indices.desc(), axis, b.astype(a.dtype, False).desc(), out.desc(), m, flag_ptr, current_stream())
-    if flag is not None and int(flag.get()[0]) != 0:
-        raise _lib.ChainerxIndexError('Index is out of bounds for axis %d with size %d' % (axis, a.shape[axis]))
-    return out
-
-
 # ---------------------------------------------------------------------------------------------
 # backward / training kernels, composed from the kernels above exactly as the reference's native backend composes them
 # (Im2Col / Col2Im as strided Copy / Add kernel calls, TensorDot as transposes + Dot)
@@ -1736,6 +1715,216 @@ def lstm_fused(c, x):
     new_c = ndarray.empty(c.shape, c.dtype)
     _lib.call('hipcx_lstm_cell', c.desc(), x.desc(), h.desc(), new_c.desc(), current_stream())
     return h, new_c
+
+
+def stack(arrays, axis=0):
+    """Stack = Empty + one CopyKernel per input into a view of the new axis (CX/routines/manipulation.cc Stack)."""
+    arrays = list(arrays)
+    if not arrays:
+        raise _lib.DimensionError('Need at least one array to stack')
+    first = arrays[0]
+    axis = _normalize_axis(axis, first.ndim + 1)
+    dtype = first.dtype
+    for a in arrays:
+        if a.shape != first.shape:
+            raise _lib.DimensionError('All arrays need to have the same shape')
+        dtype = promote_types(dtype, a.dtype)
+    out = ndarray.empty(first.shape[:axis] + (len(arrays),) + first.shape[axis:], dtype)
+    for i, a in enumerate(arrays):
+        key = [slice(None)] * out.ndim
+        key[axis] = i
+        _lib.call('hipcx_copy', a.desc(), out[tuple(key)].desc(), current_stream())
+    return out
+
+
+def clipped_relu(x, z):
+    """ClippedRelu = Minimum(Maximum(0, x), z) (CX/routines/activation.cc:51-55)."""
+    return minimum(maximum(x.astype(_math_result_dtype(x.dtype), False), 0), z)
+
+
+def crelu(x, axis=1):
+    """CRelu = Relu(Concatenate({x, -x}, axis)) (CX/routines/activation.cc:57-64)."""
+    xc = x.astype(_math_result_dtype(x.dtype), False)
+    return relu(concatenate([xc, negative(xc)], axis))
+
+
+def elu(x, alpha=1.0):
+    """Elu = Where(x > 0, x, alpha * Expm1(x)) (CX/routines/activation.cc:66-72)."""
+    xc = x.astype(_math_result_dtype(x.dtype), False)
+    return where(greater(xc, zeros((), xc.dtype)), xc, multiply(expm1(xc), alpha))
+
+
+def leaky_relu(x, slope=0.2):
+    """LeakyRelu = Where(x >= 0, x, slope * x) (CX/routines/activation.cc:86-92)."""
+    xc = x.astype(_math_result_dtype(x.dtype), False)
+    return where(greater_equal(xc, zeros((), xc.dtype)), xc, multiply(xc, slope))
+
+
+def softplus(x, beta=1.0):
+    """Softplus = (Maximum(beta*x, 0) + Log1p(Exp(-Fabs(beta*x)))) / beta (CX/routines/activation.cc:151-158)."""
+    xc = x.astype(_math_result_dtype(x.dtype), False)
+    bx = multiply(xc, beta)
+    return multiply(add(maximum(bx, 0), log1p(exp(negative(fabs(bx))))), 1.0 / beta)
+
+
+def _extract_gates(x, n_splits, axis):
+    """ExtractGates (CX/routines/activation.cc:30-46): axis 1 -> [B, n, H] (gate-major), axis 2 -> [B, H, n] (unit-major)."""
+    rest = tuple(x.shape[2:])
+    if axis == 1:
+        xr = x.reshape((x.shape[0], n_splits, x.shape[1] // n_splits) + rest)
+    else:
+        xr = x.reshape((x.shape[0], x.shape[1] // n_splits, n_splits) + rest)
+    return [g.squeeze(axis) for g in split(xr, n_splits, axis)]
+
+
+def tree_lstm(*arrays):
+    """TreeLstm(c_1..c_n, x) -> (c, h); gates of x are gate-major: a, i, o, f_1..f_n (CX/routines/activation.cc:94-121)."""
+    arrays = list(arrays)
+    n_ary = len(arrays) - 1
+    gates = _extract_gates(arrays[-1], 3 + n_ary, 1)
+    a = tanh(gates[0])
+    i = sigmoid(gates[1])
+    o = sigmoid(gates[2])
+    fs = [sigmoid(f) for f in gates[3:]]
+    acc = multiply(arrays[0], fs[0])
+    for k in range(1, n_ary):
+        acc = add(acc, multiply(arrays[k], fs[k]))
+    c = add(multiply(a, i), acc)
+    h = multiply(o, tanh(c))
+    return c, h
+
+
+def slstm(c_prev1, c_prev2, x1, x2):
+    """SLstm -> (c, h); gates are unit-major a, i, f, o (CX/routines/activation.cc:123-149)."""
+    a1, i1, f1, o1 = _extract_gates(x1, 4, 2)
+    a2, i2, f2, o2 = _extract_gates(x2, 4, 2)
+    a1, i1, f1 = tanh(a1), sigmoid(i1), sigmoid(f1)
+    a2, i2, f2 = tanh(a2), sigmoid(i2), sigmoid(f2)
+    o = sigmoid(add(o1, o2))
+    c = add(add(add(multiply(a1, i1), multiply(a2, i2)), multiply(f1, c_prev1)), multiply(f2, c_prev2))
+    h = multiply(o, tanh(c))
+    return c, h
+
+
+# ---------------------------------------------------------------------------------------------
+# n-step recurrent networks: the composition every backend but cuDNN's runs (CX/routines/n_step_rnn.cc:360-429)
+# ---------------------------------------------------------------------------------------------
+def _stack_weight(ws):
+    """StackWeight (CX/routines/n_step_rnn.cc:41-54): row u*len(ws) + g of the result is row u of ws[g]."""
+    w = stack(ws, 1)
+    return w.reshape((w.shape[0] * w.shape[1],) + tuple(w.shape[2:]))
+
+
+def _gru_impl(x, h, c, ws, bs, activation):
+    xw = concatenate([ws[0], ws[1], ws[2]], 0)
+    hw = concatenate([ws[3], ws[4], ws[5]], 0)
+    xb = concatenate([bs[0], bs[1], bs[2]], 0)
+    hb = concatenate([bs[3], bs[4], bs[5]], 0)
+    gx = split(linear(x, xw, xb), 3, 1)
+    gh = split(linear(h, hw, hb), 3, 1)
+    r = sigmoid(add(gx[0], gh[0]))
+    z = sigmoid(add(gx[1], gh[1]))
+    h_bar = tanh(add(gx[2], multiply(r, gh[2])))
+    return [add(multiply(subtract(1, z), h_bar), multiply(z, h))]
+
+
+def _lstm_impl(x, h, c, ws, bs, activation, cell=None):
+    xw = _stack_weight([ws[2], ws[0], ws[1], ws[3]])
+    hw = _stack_weight([ws[6], ws[4], ws[5], ws[7]])
+    xb = _stack_weight([bs[2], bs[0], bs[1], bs[3]])
+    hb = _stack_weight([bs[6], bs[4], bs[5], bs[7]])
+    lstm_in = add(linear(x, xw, xb), linear(h, hw, hb))
+    return list((cell or lstm)(c, lstm_in))
+
+
+def _lstm_impl_fused(x, h, c, ws, bs, activation):
+    return _lstm_impl(x, h, c, ws, bs, activation, cell=lstm_fused)
+
+
+def _rnn_impl(x, h, c, ws, bs, activation):
+    rnn_in = add(linear(x, ws[0], bs[0]), linear(h, ws[1], bs[1]))
+    return [tanh(rnn_in) if activation == 'tanh' else relu(rnn_in)]
+
+
+def _one_directional_loop(impl, xs, h, c, ws, bs, activation):
+    h = h.reshape((h.shape[1], h.shape[2]))
+    if c is not None:
+        c = c.reshape(h.shape)
+    h_list = []
+    for x in xs:
+        if x.shape[0] > h.shape[0]:
+            raise _lib.DimensionError('The batch size of x must be equal to or less than the size of state')
+        h_split = split(h, [x.shape[0], h.shape[0]], 0)
+        if c is not None:
+            c_split = split(c, [x.shape[0], c.shape[0]], 0)
+            h_c = impl(x, h_split[0], c_split[0], ws, bs, activation)
+            c_split[0] = h_c[1]
+            c = concatenate(c_split, 0)
+        else:
+            h_c = impl(x, h_split[0], None, ws, bs, activation)
+        h_list.append(h_c[0])
+        h_split[0] = h_c[0]
+        h = concatenate(h_split, 0)
+    return ([h] if c is None else [h, c]), h_list
+
+
+def _n_step_rnn_impl(impl, n_layers, hx, cx, ws, bs, xs, bidirectional, activation=None):
+    direction = 2 if bidirectional else 1
+    hx_list = split(hx, hx.shape[0], 0)
+    cx_list = split(cx, cx.shape[0], 0) if cx is not None else [None] * hx.shape[0]
+    xs_next = list(xs)
+    hy, cy = [], []
+    for layer in range(n_layers):
+        xs = xs_next
+        idx = direction * layer
+        state, h_forward = _one_directional_loop(impl, xs, hx_list[idx], cx_list[idx], ws[idx], bs[idx], activation)
+        hy.append(state[0])
+        if cx is not None:
+            cy.append(state[1])
+        if bidirectional:
+            idx += 1
+            state, h_backward = _one_directional_loop(impl, xs[::-1], hx_list[idx], cx_list[idx], ws[idx], bs[idx], activation)
+            h_backward = h_backward[::-1]
+            xs_next = [concatenate([f, b], 1) for f, b in zip(h_forward, h_backward)]
+            hy.append(state[0])
+            if cx is not None:
+                cy.append(state[1])
+        else:
+            xs_next = h_forward
+    if cx is not None:
+        return stack(hy, 0), stack(cy, 0), xs_next
+    return stack(hy, 0), xs_next
+
+
+def n_step_lstm(n_layers, hx, cx, ws, bs, xs, fused=False):
+    """NStepLstm (CX/routines/n_step_rnn.cc:434-443) -> (hy, cy, ys).  ws[layer] / bs[layer] hold the eight matrices / vectors in
+    cuDNN order: input, forget, cell, output for x, then the same for h.  `fused` (opt-in) runs each cell through hipcx_lstm_cell."""
+    return _n_step_rnn_impl(_lstm_impl_fused if fused else _lstm_impl, n_layers, hx, cx, ws, bs, xs, False)
+
+
+def n_step_bilstm(n_layers, hx, cx, ws, bs, xs, fused=False):
+    """NStepBiLstm (CX/routines/n_step_rnn.cc:445-454): ws[2*layer + direction]."""
+    return _n_step_rnn_impl(_lstm_impl_fused if fused else _lstm_impl, n_layers, hx, cx, ws, bs, xs, True)
+
+
+def n_step_gru(n_layers, hx, ws, bs, xs):
+    """NStepGru (CX/routines/n_step_rnn.cc:456-465) -> (hy, ys); six matrices per layer: reset, update, candidate for x, then h."""
+    return _n_step_rnn_impl(_gru_impl, n_layers, hx, None, ws, bs, xs, False)
+
+
+def n_step_bigru(n_layers, hx, ws, bs, xs):
+    """NStepBiGru (CX/routines/n_step_rnn.cc:467-476)."""
+    return _n_step_rnn_impl(_gru_impl, n_layers, hx, None, ws, bs, xs, True)
+
+
+def n_step_rnn(n_layers, hx, ws, bs, xs, activation='tanh'):
+    """NStepRnn (CX/routines/n_step_rnn.cc:478-487) -> (hy, ys); activation 'tanh' or 'relu'."""
+    return _n_step_rnn_impl(_rnn_impl, n_layers, hx, None, ws, bs, xs, False, activation)
+
+
+def n_step_birnn(n_layers, hx, ws, bs, xs, activation='tanh'):
+    """NStepBiRnn (CX/routines/n_step_rnn.cc:489-498)."""
+    return _n_step_rnn_impl(_rnn_impl, n_layers, hx, None, ws, bs, xs, True, activation)
 
 
 def softmax_cross_entropy(x, t):

@@ -985,6 +985,174 @@ def lstm(c, x):
     return h, new_c
 
 
+def _math(x):
+    """GetMathResultDtype: float dtypes stay, everything else computes in float32 (CX/routines/type_util.h)."""
+    x = np.asarray(x)
+    return x if x.dtype.kind == 'f' else x.astype(np.float32)
+
+
+def clipped_relu(x, z):
+    """Minimum(Maximum(0, x), z) = IfGreaterElse(max, z, z, max) (CX/routines/activation.cc:51-55, misc.cc)."""
+    m = relu(_math(x))
+    zz = _scalar_as(z, m.dtype)
+    return np.where(m > zz, zz, m).astype(m.dtype)
+
+
+def crelu(x, axis=1):
+    """Relu(Concatenate({x, -x}, axis)) (CX/routines/activation.cc:57-64)."""
+    x = _math(x)
+    return relu(np.concatenate([x, multiply(x, _scalar_as(-1, x.dtype))], axis))
+
+
+def elu(x, alpha=1.0):
+    """Where(x > 0, x, alpha * Expm1(x)) (CX/routines/activation.cc:66-72)."""
+    x = _math(x)
+    return where(x > 0, x, multiply(expm1(x), _scalar_as(alpha, x.dtype)), x.dtype)
+
+
+def leaky_relu(x, slope=0.2):
+    """Where(x >= 0, x, slope * x) (CX/routines/activation.cc:86-92)."""
+    x = _math(x)
+    return where(x >= 0, x, multiply(x, _scalar_as(slope, x.dtype)), x.dtype)
+
+
+def softplus(x, beta=1.0):
+    """(Maximum(beta*x, 0) + Log1p(Exp(-Fabs(beta*x)))) * (1/beta) (CX/routines/activation.cc:151-158)."""
+    x = _math(x)
+    bx = multiply(x, _scalar_as(beta, x.dtype))
+    neg_abs = multiply(absolute(bx), _scalar_as(-1, x.dtype))
+    return multiply(add(relu(bx), log1p(exp(neg_abs))), _scalar_as(1.0 / beta, x.dtype))
+
+
+def tree_lstm(*arrays):
+    """TreeLstm(c_1..c_n, x) -> (c, h), gate-major gates a, i, o, f_1..f_n (CX/routines/activation.cc:94-121)."""
+    cs, x = [np.asarray(a) for a in arrays[:-1]], np.asarray(arrays[-1])
+    n = 3 + len(cs)
+    g = x.reshape((x.shape[0], n, x.shape[1] // n) + x.shape[2:])
+    a, i, o = tanh(g[:, 0]), sigmoid(g[:, 1]), sigmoid(g[:, 2])
+    fs = [sigmoid(g[:, 3 + k]) for k in range(len(cs))]
+    acc = multiply(cs[0], fs[0])
+    for k in range(1, len(cs)):
+        acc = add(acc, multiply(cs[k], fs[k]))
+    c = add(multiply(a, i), acc)
+    return c, multiply(o, tanh(c))
+
+
+def slstm(c_prev1, c_prev2, x1, x2):
+    """SLstm -> (c, h), unit-major gates a, i, f, o (CX/routines/activation.cc:123-149)."""
+    def gates(x):
+        x = np.asarray(x)
+        g = x.reshape((x.shape[0], x.shape[1] // 4, 4) + x.shape[2:])
+        return g[:, :, 0], g[:, :, 1], g[:, :, 2], g[:, :, 3]
+    a1, i1, f1, o1 = gates(x1)
+    a2, i2, f2, o2 = gates(x2)
+    a1, i1, f1 = tanh(a1), sigmoid(i1), sigmoid(f1)
+    a2, i2, f2 = tanh(a2), sigmoid(i2), sigmoid(f2)
+    o = sigmoid(add(o1, o2))
+    c = add(add(add(multiply(a1, i1), multiply(a2, i2)), multiply(f1, c_prev1)), multiply(f2, c_prev2))
+    return c, multiply(o, tanh(c))
+
+
+def _stack_weight(ws):
+    """StackWeight (CX/routines/n_step_rnn.cc:41-54)."""
+    w = np.stack([np.asarray(a) for a in ws], 1)
+    return w.reshape((w.shape[0] * w.shape[1],) + w.shape[2:])
+
+
+def _gru_step(x, h, c, ws, bs, activation):
+    """GruImpl (CX/routines/n_step_rnn.cc:56-86)."""
+    gx = linear(x, np.concatenate(ws[0:3], 0), np.concatenate(bs[0:3], 0))
+    gh = linear(h, np.concatenate(ws[3:6], 0), np.concatenate(bs[3:6], 0))
+    u = gx.shape[1] // 3
+    r = sigmoid(add(gx[:, :u], gh[:, :u]))
+    z = sigmoid(add(gx[:, u:2 * u], gh[:, u:2 * u]))
+    h_bar = tanh(add(gx[:, 2 * u:], multiply(r, gh[:, 2 * u:])))
+    one_minus_z = add(multiply(z, _scalar_as(-1, z.dtype)), _scalar_as(1, z.dtype))  # Subtract(Scalar, Array) = Add(-Array, Scalar)
+    return [add(multiply(one_minus_z, h_bar), multiply(z, h))]
+
+
+def _lstm_step(x, h, c, ws, bs, activation):
+    """LstmImpl (CX/routines/n_step_rnn.cc:88-110): cuDNN order i, f, c, o becomes the Lstm routine's a, i, f, o."""
+    xw = _stack_weight([ws[2], ws[0], ws[1], ws[3]])
+    hw = _stack_weight([ws[6], ws[4], ws[5], ws[7]])
+    xb = _stack_weight([bs[2], bs[0], bs[1], bs[3]])
+    hb = _stack_weight([bs[6], bs[4], bs[5], bs[7]])
+    return list(lstm(c, add(linear(x, xw, xb), linear(h, hw, hb))))
+
+
+def _rnn_step(x, h, c, ws, bs, activation):
+    """RnnImpl (CX/routines/n_step_rnn.cc:112-139)."""
+    s = add(linear(x, ws[0], bs[0]), linear(h, ws[1], bs[1]))
+    return [tanh(s) if activation == 'tanh' else relu(s)]
+
+
+def _one_direction(step, xs, h, c, ws, bs, activation):
+    """OneDirectionalLoop (CX/routines/n_step_rnn.cc:141-194): only the first len(x) rows of the state advance."""
+    h = np.array(h)
+    c = None if c is None else np.array(c)
+    hs = []
+    for x in xs:
+        n = x.shape[0]
+        if n > h.shape[0]:
+            raise ValueError('The batch size of x must be equal to or less than the size of state')
+        out = step(x, h[:n], None if c is None else c[:n], ws, bs, activation)
+        hs.append(out[0])
+        h = np.concatenate([out[0], h[n:]], 0)
+        if c is not None:
+            c = np.concatenate([out[1], c[n:]], 0)
+    return h, c, hs
+
+
+def _n_step(step, n_layers, hx, cx, ws, bs, xs, bidirectional, activation=None):
+    """NStepRnnImpl, the non-cuDNN branch (CX/routines/n_step_rnn.cc:360-429)."""
+    d = 2 if bidirectional else 1
+    hx = np.asarray(hx)
+    cx = None if cx is None else np.asarray(cx)
+    xs = [np.asarray(x) for x in xs]
+    hy, cy = [], []
+    for layer in range(n_layers):
+        i = d * layer
+        h, c, fw = _one_direction(step, xs, hx[i], None if cx is None else cx[i], ws[i], bs[i], activation)
+        hy.append(h)
+        cy.append(c)
+        if bidirectional:
+            i += 1
+            h, c, bw = _one_direction(step, xs[::-1], hx[i], None if cx is None else cx[i], ws[i], bs[i], activation)
+            bw = bw[::-1]
+            hy.append(h)
+            cy.append(c)
+            xs = [np.concatenate([f, b], 1) for f, b in zip(fw, bw)]
+        else:
+            xs = fw
+    if cx is not None:
+        return np.stack(hy, 0), np.stack(cy, 0), xs
+    return np.stack(hy, 0), xs
+
+
+def n_step_lstm(n_layers, hx, cx, ws, bs, xs):
+    return _n_step(_lstm_step, n_layers, hx, cx, ws, bs, xs, False)
+
+
+def n_step_bilstm(n_layers, hx, cx, ws, bs, xs):
+    return _n_step(_lstm_step, n_layers, hx, cx, ws, bs, xs, True)
+
+
+def n_step_gru(n_layers, hx, ws, bs, xs):
+    return _n_step(_gru_step, n_layers, hx, None, ws, bs, xs, False)
+
+
+def n_step_bigru(n_layers, hx, ws, bs, xs):
+    return _n_step(_gru_step, n_layers, hx, None, ws, bs, xs, True)
+
+
+def n_step_rnn(n_layers, hx, ws, bs, xs, activation='tanh'):
+    return _n_step(_rnn_step, n_layers, hx, None, ws, bs, xs, False, activation)
+
+
+def n_step_birnn(n_layers, hx, ws, bs, xs, activation='tanh'):
+    return _n_step(_rnn_step, n_layers, hx, None, ws, bs, xs, True, activation)
+
+
 def softmax_cross_entropy(x, t):
     """chainer/functions/loss/softmax_cross_entropy.py:123-130 (reduce='mean', normalize=True)."""
     x, t = np.asarray(x), np.asarray(t)

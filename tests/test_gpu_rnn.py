@@ -1,0 +1,99 @@
+"""Activations composed from other routines and the n-step recurrent family, device against the CPU oracle.
+
+Both sides run the same sequence of kernels in the same order (the reference's composition); the only differences are the
+libm-class functions (exp, tanh, log1p), so float32 agrees to 1e-5 relative and float16 to 2e-2."""
+import numpy as np
+import pytest
+
+from oracle import native as O
+from helpers import assert_close
+from test_oracle_pins import _rnn_problem
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize('dt', ['float32', 'float16', 'float64'])
+def test_composed_activations(dt):
+    import chainer_amd as chx
+    rng = np.random.default_rng(3)
+    x = (rng.standard_normal((5, 8, 3)) * 3).astype(dt)
+    x[0, 0, 0] = 0
+    x[0, 1, 0] = np.nan
+    X = chx.array(x)
+    assert_close(chx.clipped_relu(X, 2.5).get(), O.clipped_relu(x, 2.5), what='clipped_relu')
+    assert_close(chx.crelu(X, 1).get(), O.crelu(x, 1), what='crelu axis 1')
+    assert_close(chx.crelu(X, 2).get(), O.crelu(x, 2), what='crelu axis 2')
+    assert_close(chx.elu(X, 0.7).get(), O.elu(x, 0.7), what='elu')
+    assert_close(chx.leaky_relu(X, 0.1).get(), O.leaky_relu(x, 0.1), what='leaky_relu')
+    assert_close(chx.softplus(X, 1.7).get(), O.softplus(x, 1.7), what='softplus')
+    c1, c2, c3 = rng.standard_normal((3, 6, 10)).astype(dt)
+    g2 = rng.standard_normal((6, 50)).astype(dt)
+    g3 = rng.standard_normal((6, 60)).astype(dt)
+    for got, ref in zip(chx.tree_lstm(chx.array(c1), chx.array(c2), chx.array(g2)), O.tree_lstm(c1, c2, g2)):
+        assert_close(got.get(), ref, what='tree_lstm 2-ary')
+    for got, ref in zip(chx.tree_lstm(chx.array(c1), chx.array(c2), chx.array(c3), chx.array(g3)), O.tree_lstm(c1, c2, c3, g3)):
+        assert_close(got.get(), ref, what='tree_lstm 3-ary')
+    x1, x2 = rng.standard_normal((2, 6, 40)).astype(dt)
+    for got, ref in zip(chx.slstm(chx.array(c1), chx.array(c2), chx.array(x1), chx.array(x2)), O.slstm(c1, c2, x1, x2)):
+        assert_close(got.get(), ref, what='slstm')
+    xi = np.arange(-3, 4, dtype=np.int32)
+    assert_close(chx.elu(chx.array(xi)).get(), O.elu(xi), what='elu of integers computes in float32')
+
+
+def _upload(chx, ws, bs, xs, hx, cx):
+    W = [[chx.array(m) for m in layer] for layer in ws]
+    B = [[chx.array(v) for v in layer] for layer in bs]
+    return W, B, [chx.array(x) for x in xs], chx.array(hx), chx.array(cx)
+
+
+CASES = [('lstm', 1, False, None), ('lstm', 2, False, None), ('lstm', 2, True, None), ('gru', 1, False, None), ('gru', 2, True, None),
+         ('rnn', 2, False, 'tanh'), ('rnn', 1, True, 'relu'), ('rnn', 2, True, 'tanh')]
+
+
+@pytest.mark.parametrize('kind,n_layers,bidirectional,activation', CASES)
+def test_n_step_family_matches_oracle(kind, n_layers, bidirectional, activation):
+    import chainer_amd as chx
+    rng = np.random.default_rng(11)
+    for in_size, units, lengths in [(4, 3, (5, 3, 3, 1)), (40, 64, (6, 6, 6, 6, 6, 6, 6, 6)), (17, 33, (4, 2))]:
+        ws, bs, seqs, xs, hx, cx = _rnn_problem(rng, kind, n_layers, bidirectional, in_size, units, lengths)
+        W, B, X, HX, CX = _upload(chx, ws, bs, xs, hx, cx)
+        what = '%s layers=%d bi=%s units=%d' % (kind, n_layers, bidirectional, units)
+        if kind == 'lstm':
+            ref = (O.n_step_bilstm if bidirectional else O.n_step_lstm)(n_layers, hx, cx, ws, bs, xs)
+            for fused in (False, True):
+                got = (chx.n_step_bilstm if bidirectional else chx.n_step_lstm)(n_layers, HX, CX, W, B, X, fused=fused)
+                assert_close(got[0].get(), ref[0], what='hy ' + what)
+                assert_close(got[1].get(), ref[1], what='cy ' + what)
+                assert len(got[2]) == len(ref[2])
+                for t, (y, r) in enumerate(zip(got[2], ref[2])):
+                    assert_close(y.get(), r, what='ys[%d] %s fused=%s' % (t, what, fused))
+            continue
+        if kind == 'gru':
+            ref = (O.n_step_bigru if bidirectional else O.n_step_gru)(n_layers, hx, ws, bs, xs)
+            got = (chx.n_step_bigru if bidirectional else chx.n_step_gru)(n_layers, HX, W, B, X)
+        else:
+            ref = (O.n_step_birnn if bidirectional else O.n_step_rnn)(n_layers, hx, ws, bs, xs, activation)
+            got = (chx.n_step_birnn if bidirectional else chx.n_step_rnn)(n_layers, HX, W, B, X, activation)
+        assert_close(got[0].get(), ref[0], what='hy ' + what)
+        assert len(got[1]) == len(ref[1])
+        for t, (y, r) in enumerate(zip(got[1], ref[1])):
+            assert_close(y.get(), r, what='ys[%d] %s' % (t, what))
+
+
+def test_n_step_lstm_float16_and_errors():
+    import chainer_amd as chx
+    rng = np.random.default_rng(12)
+    ws, bs, seqs, xs, hx, cx = _rnn_problem(rng, 'lstm', 2, False, 24, 32, (5, 5, 4, 2))
+    h = lambda tree: [[a.astype(np.float16) for a in layer] for layer in tree]
+    ws, bs = h(ws), h(bs)
+    xs = [x.astype(np.float16) for x in xs]
+    hx, cx = hx.astype(np.float16), cx.astype(np.float16)
+    W, B, X, HX, CX = _upload(chx, ws, bs, xs, hx, cx)
+    ref = O.n_step_lstm(2, hx, cx, ws, bs, xs)
+    got = chx.n_step_lstm(2, HX, CX, W, B, X)
+    assert_close(got[0].get(), ref[0], what='hy float16')
+    assert_close(got[1].get(), ref[1], what='cy float16')
+    for y, r in zip(got[2], ref[2]):
+        assert_close(y.get(), r, what='ys float16')
+    with pytest.raises(chx.DimensionError):  # a batch larger than the state
+        chx.n_step_lstm(2, HX[:, :3], CX[:, :3], W, B, X)

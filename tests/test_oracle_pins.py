@@ -700,3 +700,139 @@ def test_batch_norm_training_closed_forms():
         e[c] = h
         assert abs((loss(x, gamma + e, beta) - loss(x, gamma - e, beta)) / (2 * h) - gg[c]) <= 1e-6
         assert abs((loss(x, gamma, beta + e) - loss(x, gamma, beta - e)) / (2 * h) - gb[c]) <= 1e-6
+
+
+# ---------------------------------------------------------------------------------------------
+# activations built from other routines, and the n-step recurrent family: textbook formulas in float64
+# ---------------------------------------------------------------------------------------------
+def _sig(v):
+    return 1.0 / (1.0 + np.exp(-v))
+
+
+def test_composed_activations_closed_forms():
+    rng = np.random.default_rng(5)
+    x = (rng.standard_normal((4, 6, 3)) * 3).astype(np.float32)
+    x64 = x.astype(np.float64)
+    assert np.allclose(O.clipped_relu(x, 2.5), np.clip(x64, 0, 2.5), rtol=1e-6)
+    assert np.allclose(O.crelu(x, 1), np.concatenate([np.maximum(x64, 0), np.maximum(-x64, 0)], 1), rtol=1e-6)
+    assert O.crelu(x, 2).shape == (4, 6, 6)
+    assert np.allclose(O.elu(x, 0.7), np.where(x64 > 0, x64, 0.7 * (np.exp(x64) - 1)), rtol=1e-5, atol=1e-6)
+    assert np.allclose(O.leaky_relu(x, 0.1), np.where(x64 >= 0, x64, 0.1 * x64), rtol=1e-6)
+    assert np.allclose(O.softplus(x, 1.7), np.log1p(np.exp(1.7 * x64)) / 1.7, rtol=1e-5, atol=1e-6)
+    assert O.elu(np.arange(-2, 3, dtype=np.int32)).dtype == np.float32  # integers compute in float32
+    # TreeLstm with two children: gates are laid out gate-major (a | i | o | f1 | f2), unlike Lstm's unit-major layout
+    c1, c2 = rng.standard_normal((2, 3, 5)).astype(np.float32)
+    g = rng.standard_normal((3, 25)).astype(np.float32)
+    a, i, o, f1, f2 = [g[:, k * 5:(k + 1) * 5].astype(np.float64) for k in range(5)]
+    c_ref = np.tanh(a) * _sig(i) + c1 * _sig(f1) + c2 * _sig(f2)
+    c, h = O.tree_lstm(c1, c2, g)
+    assert np.allclose(c, c_ref, rtol=1e-5, atol=1e-6) and np.allclose(h, _sig(o) * np.tanh(c_ref), rtol=1e-5, atol=1e-6)
+    # SLstm: unit-major gates (column 4*u + k), output gate from the sum of both inputs
+    x1, x2 = rng.standard_normal((2, 3, 20)).astype(np.float32)
+    ga = [x1[:, k::4].astype(np.float64) for k in range(4)]
+    gb = [x2[:, k::4].astype(np.float64) for k in range(4)]
+    c_ref = np.tanh(ga[0]) * _sig(ga[1]) + np.tanh(gb[0]) * _sig(gb[1]) + _sig(ga[2]) * c1 + _sig(gb[2]) * c2
+    c, h = O.slstm(c1, c2, x1, x2)
+    assert np.allclose(c, c_ref, rtol=1e-5, atol=1e-6)
+    assert np.allclose(h, _sig(ga[3] + gb[3]) * np.tanh(c_ref), rtol=1e-5, atol=1e-6)
+
+
+def _rnn_problem(rng, kind, n_layers, bidirectional, in_size=4, units=3, lengths=(5, 3, 3, 1)):
+    """Random parameters and a batch of sequences sorted by decreasing length, time-major like the reference takes them."""
+    nw = {'lstm': 8, 'gru': 6, 'rnn': 2}[kind]
+    d = 2 if bidirectional else 1
+    ws, bs = [], []
+    for layer in range(n_layers):
+        for _ in range(d):
+            isz = in_size if layer == 0 else units * d
+            ws.append([rng.uniform(-0.6, 0.6, (units, isz if j < nw // 2 else units)).astype(np.float32) for j in range(nw)])
+            bs.append([rng.uniform(-0.3, 0.3, (units,)).astype(np.float32) for j in range(nw)])
+    seqs = [rng.standard_normal((n, in_size)).astype(np.float32) for n in lengths]
+    xs = [np.stack([s[t] for s in seqs if len(s) > t]) for t in range(max(lengths))]
+    hx = rng.standard_normal((n_layers * d, len(lengths), units)).astype(np.float32)
+    cx = rng.standard_normal((n_layers * d, len(lengths), units)).astype(np.float32)
+    return ws, bs, seqs, xs, hx, cx
+
+
+def _textbook_cell(kind, x, h, c, w, b, activation):
+    """One step of one sequence, written from the gate equations (cuDNN / Chainer parameter order), float64."""
+    w = [m.astype(np.float64) for m in w]
+    b = [v.astype(np.float64) for v in b]
+    if kind == 'lstm':
+        i = _sig(w[0] @ x + b[0] + w[4] @ h + b[4])
+        f = _sig(w[1] @ x + b[1] + w[5] @ h + b[5])
+        g = np.tanh(w[2] @ x + b[2] + w[6] @ h + b[6])
+        o = _sig(w[3] @ x + b[3] + w[7] @ h + b[7])
+        c = f * c + i * g
+        return o * np.tanh(c), c
+    if kind == 'gru':
+        r = _sig(w[0] @ x + b[0] + w[3] @ h + b[3])
+        z = _sig(w[1] @ x + b[1] + w[4] @ h + b[4])
+        n = np.tanh(w[2] @ x + b[2] + r * (w[5] @ h + b[5]))
+        return (1 - z) * n + z * h, None
+    s = w[0] @ x + b[0] + w[1] @ h + b[1]
+    return (np.tanh(s) if activation == 'tanh' else np.maximum(s, 0)), None
+
+
+def _textbook_n_step(kind, n_layers, bidirectional, ws, bs, seqs, hx, cx, activation='tanh'):
+    """Every sequence on its own, in float64: layer by layer, forward in time and (bidirectional) backward from its own last step."""
+    d = 2 if bidirectional else 1
+    units = hx.shape[2]
+    hy = np.zeros(hx.shape)
+    cy = np.zeros(hx.shape)
+    outs = []
+    for bi, seq in enumerate(seqs):
+        inp = seq.astype(np.float64)
+        for layer in range(n_layers):
+            per_dir = []
+            for di in range(d):
+                idx = layer * d + di
+                h = hx[idx, bi].astype(np.float64)
+                c = cx[idx, bi].astype(np.float64)
+                hs = np.zeros((len(inp), units))
+                order = range(len(inp)) if di == 0 else range(len(inp) - 1, -1, -1)
+                for t in order:
+                    h, c_new = _textbook_cell(kind, inp[t], h, c, ws[idx], bs[idx], activation)
+                    c = c_new if c_new is not None else c
+                    hs[t] = h
+                hy[idx, bi] = h
+                cy[idx, bi] = c
+                per_dir.append(hs)
+            inp = np.concatenate(per_dir, 1)
+        outs.append(inp)
+    T = max(len(s) for s in seqs)
+    ys = [np.stack([o[t] for o in outs if len(o) > t]) for t in range(T)]
+    return hy, cy, ys
+
+
+@pytest.mark.parametrize('kind,n_layers,bidirectional,activation', [
+    ('lstm', 1, False, None), ('lstm', 2, False, None), ('lstm', 2, True, None), ('gru', 1, False, None), ('gru', 2, True, None),
+    ('rnn', 2, False, 'tanh'), ('rnn', 1, True, 'relu'), ('rnn', 2, True, 'tanh')])
+def test_n_step_rnn_family_matches_textbook_recurrences(kind, n_layers, bidirectional, activation):
+    """Pins the parameter order (which matrix feeds which gate), the stacking of gate rows, the handling of shrinking batches and
+    the direction / layer wiring: a swapped gate, a transposed weight or a state row advanced past its sequence's end fails."""
+    rng = np.random.default_rng(len(kind) * 100 + n_layers * 10 + int(bidirectional))
+    ws, bs, seqs, xs, hx, cx = _rnn_problem(rng, kind, n_layers, bidirectional)
+    hy_ref, cy_ref, ys_ref = _textbook_n_step(kind, n_layers, bidirectional, ws, bs, seqs, hx, cx, activation or 'tanh')
+    if kind == 'lstm':
+        fn = O.n_step_bilstm if bidirectional else O.n_step_lstm
+        hy, cy, ys = fn(n_layers, hx, cx, ws, bs, xs)
+        assert np.allclose(cy, cy_ref, rtol=2e-5, atol=2e-6)
+    elif kind == 'gru':
+        fn = O.n_step_bigru if bidirectional else O.n_step_gru
+        hy, ys = fn(n_layers, hx, ws, bs, xs)
+    else:
+        fn = O.n_step_birnn if bidirectional else O.n_step_rnn
+        hy, ys = fn(n_layers, hx, ws, bs, xs, activation)
+    assert hy.dtype == np.float32 and hy.shape == hx.shape
+    assert np.allclose(hy, hy_ref, rtol=2e-5, atol=2e-6)
+    assert len(ys) == len(ys_ref)
+    for y, r in zip(ys, ys_ref):
+        assert y.shape == r.shape and np.allclose(y, r, rtol=2e-5, atol=2e-6)
+
+
+def test_n_step_rejects_a_growing_batch():
+    rng = np.random.default_rng(0)
+    ws, bs, seqs, xs, hx, cx = _rnn_problem(rng, 'rnn', 1, False)
+    with pytest.raises(ValueError):
+        O.n_step_rnn(1, hx[:, :2], ws, bs, xs)
