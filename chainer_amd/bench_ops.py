@@ -228,6 +228,22 @@ def section_lstm(chx, oracle, with_cpu):
     emit(section='lstm', op='35-step forward, fused opt-in Lstm cell and LogSoftmax', batch=128, graph_replay_ms=round(fused * 1e3, 2),
          TFLOPs_graph=round(flops / fused / 1e12, 2), tokens_per_s_graph=round(128 * 35 / fused, 0), kernel_launches=35 * 14 + 1,
          note='hipcx_lstm_cell and hipcx_log_softmax replace the ~25-kernel cell and the 7-kernel LogSoftmax chains; not the drop-in kernel boundary')
+    # NStepLstm at the same size: 2 layers x 35 steps, batch 128, 650 units (float32)
+    rng = np.random.default_rng(5)
+    u = 650
+    ws = [[chx.array(rng.uniform(-0.05, 0.05, (u, u)).astype(np.float32)) for _ in range(8)] for _ in range(2)]
+    bs = [[chx.array(rng.uniform(-0.05, 0.05, (u,)).astype(np.float32)) for _ in range(8)] for _ in range(2)]
+    xs = [chx.array(rng.standard_normal((128, u)).astype(np.float32)) for _ in range(35)]
+    hx = chx.zeros((2, 128, u), 'float32')
+    cx = chx.zeros((2, 128, u), 'float32')
+    nflops = 2 * 35 * 2 * 2.0 * 128 * u * 4 * u
+    composed = graph_time(lambda: chx.n_step_lstm(2, hx, cx, ws, bs, xs), 5)
+    hoisted = graph_time(lambda: chx.n_step_lstm(2, hx, cx, ws, bs, xs, fused=True), 5)
+    emit(section='lstm', op='n_step_lstm 2 layers x 35 steps, as the reference composes it', batch=128, units=u,
+         graph_replay_ms=round(composed * 1e3, 2), TFLOPs_graph=round(nflops / composed / 1e12, 2),
+         note='the composition restacks the eight gate matrices at every time step')
+    emit(section='lstm', op='n_step_lstm 2 layers x 35 steps, opt-in: weights stacked once, one input Dot per layer, fused cell', batch=128,
+         units=u, graph_replay_ms=round(hoisted * 1e3, 2), TFLOPs_graph=round(nflops / hoisted / 1e12, 2))
     W = pd['embed']
     t = device_time(lambda: chx.take(W, I, 0, 'wrap'))
     bw_row('lstm', 'take [10000,650] rows by [128,35] ids', (128, 35, 650), t, 2 * 128 * 35 * 650 * 4 + ids.nbytes)

@@ -1846,7 +1846,39 @@ def _rnn_impl(x, h, c, ws, bs, activation):
     return [tanh(rnn_in) if activation == 'tanh' else relu(rnn_in)]
 
 
+def _lstm_direction_fused(xs, h, c, ws, bs):
+    """One layer and direction of an LSTM with the loop-invariant work hoisted (opt-in): the gate rows are stacked once instead of
+    once per time step, the input projection of all time steps is one Dot over the concatenated batch, and each step is
+    Dot(h, hw) + Add + one hipcx_lstm_cell call.  State rows beyond a step's batch keep their values, as in the composed loop."""
+    h = h.reshape((h.shape[1], h.shape[2]))
+    c = c.reshape(h.shape)
+    xw = _stack_weight([ws[2], ws[0], ws[1], ws[3]])
+    hw = _stack_weight([ws[6], ws[4], ws[5], ws[7]])
+    xb = _stack_weight([bs[2], bs[0], bs[1], bs[3]])
+    hb = _stack_weight([bs[6], bs[4], bs[5], bs[7]])
+    sizes = [x.shape[0] for x in xs]
+    if _py.max(sizes) > h.shape[0]:
+        raise _lib.DimensionError('The batch size of x must be equal to or less than the size of state')
+    gx_all = linear(concatenate(xs, 0) if len(xs) > 1 else xs[0], xw, xb)
+    h_list = []
+    pos = 0
+    for n in sizes:
+        gx = gx_all[pos:pos + n]
+        pos += n
+        full = n == h.shape[0]
+        h_n, c_n = lstm_fused(c if full else c[:n], add(gx, linear(h if full else h[:n], hw, hb)))
+        h_list.append(h_n)
+        if full:
+            h, c = h_n, c_n
+        else:
+            h = concatenate([h_n, h[n:]], 0)
+            c = concatenate([c_n, c[n:]], 0)
+    return [h, c], h_list
+
+
 def _one_directional_loop(impl, xs, h, c, ws, bs, activation):
+    if impl is _lstm_impl_fused:
+        return _lstm_direction_fused(xs, h, c, ws, bs)
     h = h.reshape((h.shape[1], h.shape[2]))
     if c is not None:
         c = c.reshape(h.shape)
