@@ -273,7 +273,7 @@ int64_t ElemStride(const hipcx_array* a, int axis, const char* name) {
 // ---- float16 NCHW-native path (nchw_conv.h) ----
 struct NchwPlan {
     bool ok = false;
-    int taps = 1, npx = 1, ck = 32, wpx = 4, wch = 1, maxi = 1;
+    int taps = 1, npx = 1, ck = 32, wpx = 4, wch = 1, maxi = 1, ksplit = 1;
     int nrow = 0, nslot = 0;
     size_t wp_bytes = 0;
     int lds_bytes = 0;
@@ -321,35 +321,46 @@ NchwPlan PlanNchw(const hipcx_array* x, const hipcx_array* w, const hipcx_array*
         pl.ck = 16;
         pl.npx = pick(W);
         pl.wpx = 4, pl.wch = 1;
-        const int64_t BM = 256;
+        const int64_t BM = 64 * pl.wpx;
         int64_t rows = (BM + W - 2) / W + 1;
         int64_t cross = (BM + P - 2) / P;
         pl.nrow = static_cast<int>(rows + 2 * cross + 2);
         pl.nslot = pl.nrow * static_cast<int>(W + 2);
         int64_t items = static_cast<int64_t>(pl.nrow) * (W / pl.npx) * (pl.ck / 8);
-        pl.maxi = items <= 512 ? 2 : 4;
-        if (items > static_cast<int64_t>(pl.maxi) * 256) return pl;
+        const int64_t nt = 64 * pl.wpx;
+        pl.maxi = items <= 2 * nt ? 2 : 4;
+        if (items > pl.maxi * nt) return pl;
     }
     const int cg = pl.ck / 8;
     const int bn = 64 * pl.wch;
-    pl.lds_bytes = 2 * (cg * pl.nslot * 16 + cg * (pl.taps * bn * 16 + (pl.taps == 1 ? 64 : 0))) + pl.npx * 16;
+    const int stage_bytes = cg * pl.nslot * 16 + cg * (pl.taps * bn * 16 + (pl.taps == 1 ? 64 : 0));
+    // At most one tile per compute unit: a second group of waves takes every other channel chunk (twice the loads in flight).
+    static const bool ksplit_ok = [] { const char* e = getenv("HIPCX_CONV_KSPLIT"); return e == nullptr || e[0] != '0'; }();
+    const int64_t tiles = ((N * P + 64 * pl.wpx - 1) / (64 * pl.wpx)) * ((K + bn - 1) / bn);
+    const int64_t nchunks = C / pl.ck;
+    const bool ksplit_built = (pl.taps == 9 && pl.wpx == 4) || (pl.taps == 1 && pl.wpx * pl.wch <= 4 && pl.wch > 1);
+    if (ksplit_ok && ksplit_built && tiles <= NumCUs() && nchunks >= 4 && nchunks % 2 == 0 && 4 * stage_bytes + pl.npx * 16 <= 160 * 1024) {
+        pl.ksplit = 2;
+    }
+    pl.lds_bytes = pl.ksplit * 2 * stage_bytes + pl.npx * 16;
     pl.lds_bytes = std::max(pl.lds_bytes, bn * (64 * pl.wpx * 2 + 16));  // the epilogue's [channel][pixel] staging tile
+    if (pl.ksplit > 1) pl.lds_bytes = std::max(pl.lds_bytes, 64 * pl.wpx * pl.wch * 64 * 4);  // the second group's accumulators
     if (pl.lds_bytes > 160 * 1024) return pl;
     pl.wp_bytes = RoundUpTo(static_cast<size_t>(K) * C * R * S * 2, 256);
     pl.ok = true;
     return pl;
 }
 
-template <int TAPS, int WPX, int WCH, int CK, int NPX, int MAXI>
+template <int TAPS, int WPX, int WCH, int CK, int NPX, int MAXI, int KSPLIT = 1>
 void LaunchNchwKernel(const NchwConvArgs& a, int lds_bytes, hipStream_t stream) {
-    auto kern = NchwConvKernel<TAPS, WPX, WCH, CK, NPX, MAXI>;
+    auto kern = NchwConvKernel<TAPS, WPX, WCH, CK, NPX, MAXI, KSPLIT>;
     static int configured = 0;
     if (lds_bytes > configured) {
         HIPCX_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes));
         configured = lds_bytes;
     }
     int64_t total = static_cast<int64_t>(a.tiles_m) * a.tiles_n;
-    dim3 grid(static_cast<unsigned>((total + 7) / 8 * 8)), block(64 * WPX * WCH);
+    dim3 grid(static_cast<unsigned>((total + 7) / 8 * 8)), block(64 * WPX * WCH * KSPLIT);
     hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, a);
     CheckLaunch("nchw_conv");
 }
@@ -418,7 +429,7 @@ void RunNchw(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, c
     double flops = 2.0 * a.M * a.K * RS * a.C;
     double bytes = 2.0 * (static_cast<double>(a.N) * a.C * a.H * a.W + static_cast<double>(a.K) * RS * a.C + static_cast<double>(a.M) * a.K);
     ProfileScope prof(stream, flops, bytes);
-    const int key = (pl.ck / 16) * 100000 + pl.taps * 10000 + pl.wpx * 1000 + pl.wch * 100 + pl.npx * 10 + pl.maxi;
+    const int key = (pl.ksplit - 1) * 1000000 + (pl.ck / 16) * 100000 + pl.taps * 10000 + pl.wpx * 1000 + pl.wch * 100 + pl.npx * 10 + pl.maxi;
 #define HIPCX_NCHW_CASE(TAPS, WPX, WCH, CK, NPX, MAXI) \
     case (CK / 16) * 100000 + TAPS * 10000 + WPX * 1000 + WCH * 100 + NPX * 10 + MAXI: LaunchNchwKernel<TAPS, WPX, WCH, CK, NPX, MAXI>(a, pl.lds_bytes, stream); break;
     switch (key) {
@@ -432,6 +443,16 @@ void RunNchw(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, c
         HIPCX_NCHW_CASE(9, 4, 1, 16, 2, 4)
         HIPCX_NCHW_CASE(9, 4, 1, 16, 1, 2)
         HIPCX_NCHW_CASE(9, 4, 1, 16, 1, 4)
+#define HIPCX_NCHW_SPLIT_CASE(TAPS, WPX, WCH, CK, NPX, MAXI) \
+    case 1000000 + (CK / 16) * 100000 + TAPS * 10000 + WPX * 1000 + WCH * 100 + NPX * 10 + MAXI: LaunchNchwKernel<TAPS, WPX, WCH, CK, NPX, MAXI, 2>(a, pl.lds_bytes, stream); break;
+        HIPCX_NCHW_SPLIT_CASE(1, 2, 2, 32, 2, 1)
+        HIPCX_NCHW_SPLIT_CASE(1, 2, 2, 32, 1, 2)
+        HIPCX_NCHW_SPLIT_CASE(1, 1, 4, 32, 1, 1)
+        HIPCX_NCHW_SPLIT_CASE(9, 4, 1, 16, 2, 2)
+        HIPCX_NCHW_SPLIT_CASE(9, 4, 1, 16, 2, 4)
+        HIPCX_NCHW_SPLIT_CASE(9, 4, 1, 16, 1, 2)
+        HIPCX_NCHW_SPLIT_CASE(9, 4, 1, 16, 1, 4)
+#undef HIPCX_NCHW_SPLIT_CASE
         default: throw Error(HIPCX_CHAINERX_ERROR, "nchw conv: no kernel for plan " + std::to_string(key));
     }
 #undef HIPCX_NCHW_CASE
@@ -889,6 +910,8 @@ int hipcx_conv_bn_act(const hipcx_array* x, const hipcx_array* w, const hipcx_ar
     });
 }
 
+}  // extern "C"
+
 namespace {
 // The MFMA kernels read both operands with the reduction index k as the unit-stride axis, rows 16-byte aligned.  An operand
 // laid out otherwise (a plain row-major b, a transposed a, odd pitches) is first copied into that layout -- one pass over
@@ -929,6 +952,8 @@ DotStaging PlanDotStaging(const hipcx_array* a, const hipcx_array* b, const hipc
     return st;
 }
 }  // namespace
+
+extern "C" {
 
 size_t hipcx_dot_workspace_size(const hipcx_array* a, const hipcx_array* b, const hipcx_array* out) {
     try {

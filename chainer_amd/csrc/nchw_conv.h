@@ -135,10 +135,14 @@ __device__ __forceinline__ void Transpose8(const PixVec<NPX> (&in)[8], Bytes16 (
     }
 }
 
-template <int TAPS, int WPX, int WCH, int CK, int NPX, int MAXI>
-__global__ __launch_bounds__(64 * WPX * WCH) void NchwConvKernel(NchwConvArgs p) {
+// KSPLIT = 2: a second set of WPX * WCH waves works on the same tile and takes every other channel chunk through LDS stages of
+// its own; the two accumulator sets are added through LDS before the epilogue.  For grids with at most one tile per compute unit
+// (7x7 planes, small batches) this doubles the waves and the loads in flight per unit, which is what bounds those layers.
+template <int TAPS, int WPX, int WCH, int CK, int NPX, int MAXI, int KSPLIT = 1>
+__global__ __launch_bounds__(64 * WPX * WCH * KSPLIT) void NchwConvKernel(NchwConvArgs p) {
     constexpr int PW = 2, CW = 2;  // wave tile: 64 pixels x 64 channels
-    constexpr int NT = 64 * WPX * WCH;
+    constexpr int NT = 64 * WPX * WCH;       // threads of one reduction group
+    constexpr int NT_ALL = NT * KSPLIT;
     constexpr int BM = 32 * PW * WPX;
     constexpr int BN = 32 * CW * WCH;
     constexpr int CG = CK / 8;    // 16-byte channel groups per chunk
@@ -152,13 +156,16 @@ __global__ __launch_bounds__(64 * WPX * WCH) void NchwConvKernel(NchwConvArgs p)
     extern __shared__ __align__(16) char lds[];
     const int patch_bytes = CG * p.nslot * 16;
     const int stage_bytes = patch_bytes + CG * WCGP;
-    const int dump_off = 2 * stage_bytes;  // NPX * 16 bytes that absorb the writes of idle load slots
+    const int dump_off = KSPLIT * 2 * stage_bytes;  // NPX * 16 bytes that absorb the writes of idle load slots
 
     int tile_m, tile_n;
     if (!TileOf(p.tiles_m, p.tiles_n, tile_m, tile_n)) return;
     const int m0 = tile_m * BM;
     const int n0 = tile_n * BN;
-    const int tid = threadIdx.x;
+    const int tid_all = threadIdx.x;
+    const int kg = KSPLIT > 1 ? __builtin_amdgcn_readfirstlane(tid_all / NT) : 0;  // reduction group of this wave
+    const int tid = tid_all - kg * NT;                                             // thread index inside the group
+    char* const glds = lds + kg * 2 * stage_bytes;                                 // the group's two stages
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int wpx = wave % WPX;
@@ -246,7 +253,8 @@ __global__ __launch_bounds__(64 * WPX * WCH) void NchwConvKernel(NchwConvArgs p)
 
     PixVec<NPX> xreg[MAXI][8];
     Bytes16 wreg[WPT];
-    auto load_chunk = [&](int ci) {
+    auto load_chunk = [&](int gi) {  // gi: chunk number inside this group; the groups interleave chunks
+        const int ci = gi * KSPLIT + kg;
         const int xs = ci * CK * HW * 2;
 #pragma unroll
         for (int i = 0; i < MAXI; ++i) {
@@ -346,22 +354,49 @@ __global__ __launch_bounds__(64 * WPX * WCH) void NchwConvKernel(NchwConvArgs p)
     // iteration ago: they go to the other stage (free since the barrier that ended iteration ci-1), the loads of chunk
     // ci+2 are issued into the same registers, and only then chunk ci is multiplied.  No wave ever waits for a load it
     // has just issued, and the LDS writes of one wave overlap the MFMAs of the others.
-    const int nchunks = p.C / CK;
+    const int nchunks = p.C / CK / KSPLIT;  // per group; the host only picks KSPLIT when it divides the chunk count
     load_chunk(0);
-    if constexpr (TAPS == 9) {  // borders of both patches must read as zero; nothing ever writes them
-        for (int off = tid * 16; off < 2 * stage_bytes; off += NT * 16) *reinterpret_cast<Bytes16*>(lds + off) = Bytes16(0);
+    if constexpr (TAPS == 9) {  // borders of all patches must read as zero; nothing ever writes them
+        for (int off = tid_all * 16; off < KSPLIT * 2 * stage_bytes; off += NT_ALL * 16) *reinterpret_cast<Bytes16*>(lds + off) = Bytes16(0);
         __syncthreads();
     }
-    store_chunk(lds);
+    store_chunk(glds);
     if (nchunks > 1) load_chunk(1);
     __syncthreads();
     for (int ci = 0; ci < nchunks; ++ci) {
-        char* cur = lds + (ci & 1) * stage_bytes;
-        char* nxt = lds + ((ci + 1) & 1) * stage_bytes;
+        char* cur = glds + (ci & 1) * stage_bytes;
+        char* nxt = glds + ((ci + 1) & 1) * stage_bytes;
         if (ci + 1 < nchunks) store_chunk(nxt);
         if (ci + 2 < nchunks) load_chunk(ci + 2);
         compute(cur);
         __syncthreads();
+    }
+
+    // ---- the second group hands its sums over (the loop's last barrier has retired every stage read) ----
+    if constexpr (KSPLIT > 1) {
+        float* red = reinterpret_cast<float*>(lds);  // [PW * CW * 16][NT]: consecutive lanes, consecutive words
+        if (kg == 1) {
+#pragma unroll
+            for (int a = 0; a < PW; ++a) {
+#pragma unroll
+                for (int b = 0; b < CW; ++b) {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) red[((a * CW + b) * 16 + v) * NT + tid] = acc[a][b][v];
+                }
+            }
+        }
+        __syncthreads();
+        if (kg == 0) {
+#pragma unroll
+            for (int a = 0; a < PW; ++a) {
+#pragma unroll
+                for (int b = 0; b < CW; ++b) {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) acc[a][b][v] += red[((a * CW + b) * 16 + v) * NT + tid];
+                }
+            }
+        }
+        __syncthreads();  // the staging tile below reuses this memory
     }
 
     // ---- epilogue ----
@@ -408,31 +443,33 @@ __global__ __launch_bounds__(64 * WPX * WCH) void NchwConvKernel(NchwConvArgs p)
     using False = std::integral_constant<bool, false>;
     const bool has_bn = p.bn_gamma != nullptr;
     const bool relu_here = p.relu && p.residual == nullptr;  // with a residual, ReLU follows the addition
-    if (has_bn) {
-        if (relu_here) stage_tile(True{}, True{});
-        else stage_tile(True{}, False{});
-    } else {
-        if (relu_here) stage_tile(False{}, True{});
-        else stage_tile(False{}, False{});
+    if (kg == 0) {
+        if (has_bn) {
+            if (relu_here) stage_tile(True{}, True{});
+            else stage_tile(True{}, False{});
+        } else {
+            if (relu_here) stage_tile(False{}, True{});
+            else stage_tile(False{}, False{});
+        }
     }
     __syncthreads();
     auto store_rows = [&](auto ev_tag, auto res_tag) {
         constexpr int EV = decltype(ev_tag)::value;  // pixels per store
         constexpr bool RES = decltype(res_tag)::value;
         constexpr int CPR = BM / EV;                 // chunks per channel row
-        static_assert(NT % CPR == 0 || CPR % NT == 0, "a thread keeps one pixel column");
-        constexpr int COLS_PER_THREAD = CPR > NT ? CPR / NT : 1;
-        constexpr int ROW_STEP = CPR > NT ? 1 : NT / CPR;
+        static_assert(NT_ALL % CPR == 0 || CPR % NT_ALL == 0, "a thread keeps one pixel column");
+        constexpr int COLS_PER_THREAD = CPR > NT_ALL ? CPR / NT_ALL : 1;
+        constexpr int ROW_STEP = CPR > NT_ALL ? 1 : NT_ALL / CPR;
         using Raw = typename RawVec<EV>::type;  // one LDS read and one global store of EV * 2 bytes
 #pragma unroll
         for (int cj = 0; cj < COLS_PER_THREAD; ++cj) {
-            const int cc = (tid % (CPR > NT ? NT : CPR)) + cj * NT;
+            const int cc = (tid_all % (CPR > NT_ALL ? NT_ALL : CPR)) + cj * NT_ALL;
             const int m = m0 + cc * EV;
             if (m >= p.M) continue;
             const int img = m / p.P;
             const int pix = m - img * p.P;
             const int64_t obase = static_cast<int64_t>(img) * p.K * p.P + pix;
-            for (int row = (CPR > NT ? 0 : tid / CPR); row < BN; row += ROW_STEP) {
+            for (int row = (CPR > NT_ALL ? 0 : tid_all / CPR); row < BN; row += ROW_STEP) {
                 const int n = n0 + row;
                 if (n >= p.K) break;
                 const int64_t o = obase + static_cast<int64_t>(n) * p.P;

@@ -15,7 +15,7 @@ DT = [('float32', 1e-5), ('float16', 2e-2), ('float64', 1e-12)]
 def test_fixed_batch_norm(dt, tol):
     import chainer_amd as chx
     rng = np.random.default_rng(0)
-    for shape in [(2, 16, 5, 7), (3, 64, 8, 8), (2, 5, 3, 3), (1, 8, 1, 1)]:
+    for shape in [(2, 16, 5, 7), (3, 64, 8, 8), (2, 5, 3, 3), (1, 8, 1, 1), (4, 32, 14, 14), (8, 64, 7, 7), (3, 2000, 2, 2), (2, 700, 1, 3), (2, 3, 70, 70)]:
         C = shape[1]
         x = rng.standard_normal(shape).astype(dt)
         g = rng.uniform(0.5, 1.5, C).astype(dt)

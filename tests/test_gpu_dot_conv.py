@@ -31,6 +31,14 @@ CONV_CASES = [
     (2, 32, 8, 8, 256, 1, 1, 1, 0, False),
     (16, 32, 46, 46, 512, 1, 1, 2, 0, False),
     (2, 64, 7, 7, 320, 1, 1, 1, 0, False),
+    # at most one tile per compute unit and an even number (>= 4) of channel chunks: two wave groups split the reduction
+    (2, 256, 7, 7, 512, 1, 1, 1, 0, False),
+    (2, 128, 14, 14, 128, 1, 1, 1, 0, False),
+    (3, 128, 7, 7, 128, 1, 1, 1, 0, False),
+    (2, 64, 7, 7, 128, 3, 3, 1, 1, False),
+    (3, 64, 14, 14, 64, 3, 3, 1, 1, False),
+    (1, 64, 56, 56, 64, 3, 3, 1, 1, False),
+    (5, 96, 7, 7, 70, 3, 3, 1, 1, False),
 ]
 
 
@@ -152,3 +160,17 @@ def test_dot_operand_layouts_large(dt, tol):
         ap = padded((m, k), a, 1, dt)
         bp = padded((k, n), b, 1, dt)
         assert_close(chx.dot(upload_view(chx, ap), upload_view(chx, bp)).get(), ref, tol, 'dot of padded operands %r' % ((m, k, n),))
+
+
+@pytest.mark.parametrize('N,C,H,K', [(8, 16, 56, 192), (16, 16, 28, 384), (32, 16, 14, 704), (64, 16, 7, 1344), (2, 32, 7, 128), (3, 16, 14, 64),
+                                     (2, 16, 28, 64), (1, 16, 56, 64)])
+def test_conv3x3_float16_tile_variants(N, C, H, K):
+    """3x3 / stride 1 / pad 1 on dense float16 NCHW, from grids of several hundred 256-pixel tiles down to a single partial tile,
+    for even (pixel pairs) and odd (single pixels) plane widths."""
+    import chainer_amd as chx
+    rng = np.random.default_rng(N * 100 + H)
+    x = rng.standard_normal((N, C, H, H)).astype('float16')
+    w = (rng.standard_normal((K, C, 3, 3)) / np.sqrt(C * 9)).astype('float16')
+    b = rng.standard_normal(K).astype('float16')
+    y = chx.conv(chx.array(x), chx.array(w), chx.array(b), 1, 1)
+    assert_close(y.get(), O.conv(x, w, b, 1, 1, False), 2e-2, 'conv3x3 %r' % ((N, C, H, K),))
