@@ -76,29 +76,40 @@ __global__ __launch_bounds__(256) void StemConv7x7s2Kernel(StemConvArgs p) {
 #pragma unroll
         for (int k = 0; k < 4; ++k) *reinterpret_cast<Bytes16*>(lds + k * p.copyb + NROW * p.rowp + off) = Bytes16(0);
     }
-    const int items = NROW * ch;
-    for (int it = tid; it < items; it += 256) {
-        int rr = it / ch;
-        int j = it - rr * ch;
-        int c = rr / 9;
-        int ihl = rr - c * 9;
-        int ih = 2 * oh0 - 3 + ihl;
-        bool row_ok = ih >= 0 && ih < p.H;
-        int base = (((n * C + c) * p.H + ih) * p.W + j * 8) * 2;
-        Bytes16 g1 = __builtin_amdgcn_raw_buffer_load_b128(xr, row_ok ? base : 0x7fffffff, 0, 0);
-        Bytes8 g0 = __builtin_amdgcn_raw_buffer_load_b64(xr, (row_ok && j > 0) ? base - 8 : 0x7fffffff, 0, 0);
-        Bytes8 g2 = __builtin_amdgcn_raw_buffer_load_b64(xr, (row_ok && j + 1 < ch) ? base + 16 : 0x7fffffff, 0, 0);
-        // d[i] holds input pixels 8*j - 8 + 2*i, +1 of this row (i = 2 .. 9)
-        unsigned d[10] = {0, 0, g0.x, g0.y, g1.x, g1.y, g1.z, g1.w, g2.x, g2.y};
-        char* dst = lds + rr * p.rowp + j * 16;
+    // Thread (tr, tj) stages 16-byte chunk tj (+32 per pass) of rows tr, tr + 8, ...: no divisions by run-time values, and all
+    // loads of a pass are issued before the first is used.
+    constexpr int kRowsPerThread = (NROW + 7) / 8;
+    const int tj = tid & 31, tr = tid >> 5;
+    for (int j = tj; j < ch; j += 32) {
+        Bytes16 g1[kRowsPerThread];
+        Bytes8 g0[kRowsPerThread], g2[kRowsPerThread];
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {  // copy k, chunk j = padded pixels 8*j + 2*k .. +7 = input pixels 8*j + 2*k - 3 .. +4
-            Bytes16 v;
-            v.x = __builtin_amdgcn_alignbit(d[3 + k], d[2 + k], 16);
-            v.y = __builtin_amdgcn_alignbit(d[4 + k], d[3 + k], 16);
-            v.z = __builtin_amdgcn_alignbit(d[5 + k], d[4 + k], 16);
-            v.w = __builtin_amdgcn_alignbit(d[6 + k], d[5 + k], 16);
-            *reinterpret_cast<Bytes16*>(dst + k * p.copyb) = v;
+        for (int u = 0; u < kRowsPerThread; ++u) {
+            const int rr = tr + 8 * u;
+            const int c = rr / 9;
+            const int ih = 2 * oh0 - 3 + (rr - c * 9);
+            const bool row_ok = rr < NROW && ih >= 0 && ih < p.H;
+            const int base = (((n * C + c) * p.H + ih) * p.W + j * 8) * 2;
+            g1[u] = __builtin_amdgcn_raw_buffer_load_b128(xr, row_ok ? base : 0x7fffffff, 0, 0);
+            g0[u] = __builtin_amdgcn_raw_buffer_load_b64(xr, (row_ok && j > 0) ? base - 8 : 0x7fffffff, 0, 0);
+            g2[u] = __builtin_amdgcn_raw_buffer_load_b64(xr, (row_ok && j + 1 < ch) ? base + 16 : 0x7fffffff, 0, 0);
+        }
+#pragma unroll
+        for (int u = 0; u < kRowsPerThread; ++u) {
+            const int rr = tr + 8 * u;
+            if (rr >= NROW) continue;
+            // d[i] holds input pixels 8*j - 8 + 2*i, +1 of this row (i = 2 .. 9)
+            unsigned d[10] = {0, 0, g0[u].x, g0[u].y, g1[u].x, g1[u].y, g1[u].z, g1[u].w, g2[u].x, g2[u].y};
+            char* dst = lds + rr * p.rowp + j * 16;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {  // copy k, chunk j = padded pixels 8*j + 2*k .. +7 = input pixels 8*j + 2*k - 3 .. +4
+                Bytes16 v;
+                v.x = __builtin_amdgcn_alignbit(d[3 + k], d[2 + k], 16);
+                v.y = __builtin_amdgcn_alignbit(d[4 + k], d[3 + k], 16);
+                v.z = __builtin_amdgcn_alignbit(d[5 + k], d[4 + k], 16);
+                v.w = __builtin_amdgcn_alignbit(d[6 + k], d[5 + k], 16);
+                *reinterpret_cast<Bytes16*>(dst + k * p.copyb) = v;
+            }
         }
     }
 
@@ -108,8 +119,8 @@ __global__ __launch_bounds__(256) void StemConv7x7s2Kernel(StemConvArgs p) {
     for (int s = 0; s < MAXSUB; ++s) {
         int q = (sub0 + 2 * s) * 32 + lr;
         if (q >= npix) q = npix - 1;  // rows of the MFMA that are never stored
-        int orow = q / p.OW;
-        int ow = q - orow * p.OW;
+        int orow = q >= p.OW ? 1 : 0;  // the tile holds two output rows
+        int ow = q - (orow ? p.OW : 0);
         abase[s] = (ow & 3) * p.copyb + 2 * orow * p.rowp + (ow >> 2) * 16;
     }
     int poff[KSTEPS];  // staged row of this lane's filter row (c, r) in each step
@@ -174,11 +185,13 @@ __global__ __launch_bounds__(256) void StemConv7x7s2Kernel(StemConvArgs p) {
     }
     __syncthreads();
     const int cpr = npix / 8;  // 16-byte chunks per channel row (OW % 8 == 0)
-    for (int id = tid; id < K * cpr; id += 256) {
-        int row = id / cpr;
-        int cc = id - row * cpr;
-        Bytes16 v = *reinterpret_cast<const Bytes16*>(lds + row * opitch + cc * 16);
-        *reinterpret_cast<Bytes16*>(p.out + ((static_cast<int64_t>(n) * K + row) * p.OH + oh0) * p.OW + cc * 8) = v;
+    for (int cc = tj; cc < cpr; cc += 32) {
+        half_t* dst = p.out + (static_cast<int64_t>(n) * K * p.OH + oh0) * p.OW + cc * 8;
+#pragma unroll 4
+        for (int row = tr; row < K; row += 8) {
+            Bytes16 v = *reinterpret_cast<const Bytes16*>(lds + row * opitch + cc * 16);
+            *reinterpret_cast<Bytes16*>(dst + static_cast<int64_t>(row) * p.OH * p.OW) = v;
+        }
     }
 }
 
