@@ -88,7 +88,7 @@ __global__ __launch_bounds__(kBnFlatThreads) void BnChannelsFirstKernel(const T*
                                                                         const T* __restrict__ gamma, const T* __restrict__ beta,
                                                                         const T* __restrict__ mean, const T* __restrict__ var,
                                                                         compute_t<T> eps, int C_, int64_t L, int64_t pstride,
-                                                                        int64_t total, int max_rows) {
+                                                                        int64_t total, int max_rows, int stream_in) {
     using C = compute_t<T>;
     constexpr int64_t kSpan = static_cast<int64_t>(kBnFlatThreads) * kBnFlatUnroll * VEC;
     extern __shared__ __align__(16) char bn_lds[];
@@ -109,7 +109,10 @@ __global__ __launch_bounds__(kBnFlatThreads) void BnChannelsFirstKernel(const T*
 #pragma unroll
     for (int u = 0; u < kBnFlatUnroll; ++u) {
         idx[u] = e0 + (static_cast<int64_t>(u) * kBnFlatThreads + threadIdx.x) * VEC;
-        if (idx[u] < total) in[u] = *reinterpret_cast<const Vec<T, VEC>*>(x + idx[u]);
+        if (idx[u] < total) {
+            const char* src = reinterpret_cast<const char*>(x + idx[u]);
+            in[u] = stream_in ? LoadStreaming<Vec<T, VEC>>(src) : *reinterpret_cast<const Vec<T, VEC>*>(src);
+        }
     }
 #pragma unroll
     for (int u = 0; u < kBnFlatUnroll; ++u) {
@@ -250,15 +253,16 @@ void RunBn(const hipcx_array* x, const hipcx_array* const params[4], hipcx_scala
             int64_t max_rows = span / L + 2;  // rows a span can touch
             int64_t lds = max_rows * 4 * static_cast<int64_t>(sizeof(C));
             int64_t blocks = (total + span - 1) / span;
+            const int stream_in = vec_ok && total * it > StreamingThresholdBytes() ? 1 : 0;
             if (lds <= 48 * 1024 && blocks < (1LL << 31)) {
                 if (vec_ok) {
                     hipLaunchKernelGGL((BnChannelsFirstKernel<T, VEC>), dim3(static_cast<unsigned>(blocks)), dim3(kBnFlatThreads),
                                        static_cast<size_t>(lds), stream, xp, op, g, b, m, v_, eps, static_cast<int>(Cn), L, ps / it, total,
-                                       static_cast<int>(max_rows));
+                                       static_cast<int>(max_rows), stream_in);
                 } else {
                     hipLaunchKernelGGL((BnChannelsFirstKernel<T, 1>), dim3(static_cast<unsigned>(blocks)), dim3(kBnFlatThreads),
                                        static_cast<size_t>(lds), stream, xp, op, g, b, m, v_, eps, static_cast<int>(Cn), L, ps / it, total,
-                                       static_cast<int>(max_rows));
+                                       static_cast<int>(max_rows), stream_in);
                 }
                 CheckLaunch("fixed_batch_norm(channels-first)");
                 return;

@@ -1,4 +1,6 @@
 // Library-wide state: last-error string, device queries.
+#include <cstdlib>
+#include <cstdint>
 #include "common.h"
 
 namespace hipcx {
@@ -8,6 +10,15 @@ thread_local std::string g_last_error;
 }
 
 void SetLastError(const std::string& msg) { g_last_error = msg; }
+
+int64_t StreamingThresholdBytes() {
+    static const int64_t bytes = [] {
+        const char* e = getenv("HIPCX_STREAM_MB");
+        int64_t mb = e != nullptr ? atoll(e) : 75;
+        return mb <= 0 ? INT64_MAX : mb * 1000000;
+    }();
+    return bytes;
+}
 
 int NumCUs() {
     static thread_local int cached_dev = -1;

@@ -101,7 +101,21 @@ struct EwArgs {
     int64_t cols;   // elements
     int64_t cvecs;  // cols / VEC
     int64_t nvec;   // rows * cvecs
+    int stream_in;  // inputs are too large to stay in the last-level cache: load them without allocating there
 };
+
+// A 16-byte vector load that does not allocate in the caches (other sizes: a plain load).  A tensor larger than the memory-side
+// cache that is read front to back with allocating loads evicts its own tail -- the part the producer left there -- before reaching it.
+template <typename V>
+__device__ __forceinline__ V LoadStreaming(const char* p) {
+    if constexpr (sizeof(V) == 16) {
+        typedef unsigned Raw16 __attribute__((ext_vector_type(4)));
+        Raw16 r = __builtin_nontemporal_load(reinterpret_cast<const Raw16*>(p));
+        return __builtin_bit_cast(V, r);
+    } else {
+        return *reinterpret_cast<const V*>(p);
+    }
+}
 
 template <typename T, int N>
 struct alignas(sizeof(T) * N) Vec {
@@ -171,32 +185,40 @@ __global__ __launch_bounds__(kEwThreads) void EwKernel(EwArgs<Op::kNumIn + 1> ar
     // loads first (all unrolled iterations in flight), then compute + store
     Vec<In, VEC> in[kEwUnroll][NIN > 0 ? NIN : 1];
     Vec<In0, VEC> in0[kEwUnroll];
+    auto load_all = [&](auto stream_tag) {
+        constexpr bool STREAM = decltype(stream_tag)::value;
 #pragma unroll
-    for (int u = 0; u < kEwUnroll; ++u) {
-        if (!live[u]) continue;
+        for (int u = 0; u < kEwUnroll; ++u) {
+            if (!live[u]) continue;
 #pragma unroll
-        for (int i = 0; i < NIN; ++i) {
-            const char* p = args.ptr[i + 1] + off[u][i + 1];
-            if (i == 0) {
-                if (VEC > 1 && args.col_stride[NOPS > 1 ? 1 : 0] != 0) {
-                    in0[u] = *reinterpret_cast<const Vec<In0, VEC>*>(p);
+            for (int i = 0; i < NIN; ++i) {
+                const char* p = args.ptr[i + 1] + off[u][i + 1];
+                if (i == 0) {
+                    if (VEC > 1 && args.col_stride[NOPS > 1 ? 1 : 0] != 0) {
+                        in0[u] = STREAM ? LoadStreaming<Vec<In0, VEC>>(p) : *reinterpret_cast<const Vec<In0, VEC>*>(p);
+                    } else {
+                        In0 s = *reinterpret_cast<const In0*>(p);
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e) in0[u].v[e] = s;
+                    }
+                } else if (VEC > 1) {
+                    if (args.col_stride[i + 1] != 0) {
+                        in[u][i] = STREAM ? LoadStreaming<Vec<In, VEC>>(p) : *reinterpret_cast<const Vec<In, VEC>*>(p);
+                    } else {
+                        In s = *reinterpret_cast<const In*>(p);
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e) in[u][i].v[e] = s;
+                    }
                 } else {
-                    In0 s = *reinterpret_cast<const In0*>(p);
-#pragma unroll
-                    for (int e = 0; e < VEC; ++e) in0[u].v[e] = s;
+                    in[u][i].v[0] = *reinterpret_cast<const In*>(p);
                 }
-            } else if (VEC > 1) {
-                if (args.col_stride[i + 1] != 0) {
-                    in[u][i] = *reinterpret_cast<const Vec<In, VEC>*>(p);
-                } else {
-                    In s = *reinterpret_cast<const In*>(p);
-#pragma unroll
-                    for (int e = 0; e < VEC; ++e) in[u][i].v[e] = s;
-                }
-            } else {
-                in[u][i].v[0] = *reinterpret_cast<const In*>(p);
             }
         }
+    };
+    if (VEC > 1 && args.stream_in) {
+        load_all(std::integral_constant<bool, true>{});
+    } else {
+        load_all(std::integral_constant<bool, false>{});
     }
 #pragma unroll
     for (int u = 0; u < kEwUnroll; ++u) {
@@ -255,6 +277,7 @@ inline void LaunchEwVec(const EwPlan& p, const Op& op, hipStream_t stream) {
     a.cols = cols;
     a.cvecs = cols / VEC;
     a.nvec = rows * a.cvecs;
+    a.stream_in = a.nvec * VEC * static_cast<int64_t>(sizeof(typename Op::In)) > StreamingThresholdBytes() ? 1 : 0;
     int64_t per_block = static_cast<int64_t>(kEwThreads) * kEwUnroll;
     int64_t blocks = (a.nvec + per_block - 1) / per_block;
     HIPCX_REQUIRE(blocks <= 0x7fffffffLL, HIPCX_NOT_IMPLEMENTED_ERROR, "array too large for one launch");
