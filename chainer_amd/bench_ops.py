@@ -253,9 +253,10 @@ def section_lstm(chx, oracle, with_cpu):
 
 
 def section_backward(chx, oracle, with_cpu):
-    """Backward / training kernels at ResNet-50 layer shapes (float16, batch 32): compositions of the forward kernels, so the
-    figures are those of Im2Col / Col2Im copies plus one matrix product -- functional, not tuned.  Timed as HIP-graph replays
-    (each composition is 10-25 kernel launches; issued eagerly from Python it would be host-bound)."""
+    """Backward / training kernels at ResNet-50 layer shapes (float16, batch 32).  The convolution and batch-norm gradients are
+    compositions of the forward kernels (Im2Col / Col2Im copies plus one matrix product; reductions and elementwise kernels) --
+    functional, not tuned; the pooling gradients have kernels of their own.  Timed as HIP-graph replays (a composition is 10-25
+    kernel launches; issued eagerly from Python it would be host-bound)."""
     rng = np.random.default_rng(6)
     n, c, k, hw = 32, 256, 256, 14
     x = chx.array(rng.standard_normal((n, c, hw, hw)).astype(np.float16))
@@ -286,7 +287,8 @@ def section_backward(chx, oracle, with_cpu):
     xp = chx.array(rng.standard_normal((32, 64, 112, 112)).astype(np.float16))
     gp = chx.array(rng.standard_normal((32, 64, 56, 56)).astype(np.float16))
     t = graph_time(lambda: chx.max_pool_grad(xp, gp, 3, 2, 1), 5)
-    bw_row('backward', 'max_pool_grad 3x3/2 pad 1', (32, 64, 112, 112), t, 2 * xp.nbytes + gp.nbytes)
+    bw_row('backward', 'max_pool_grad 3x3/2 pad 1', (32, 64, 112, 112), t, 2 * xp.nbytes + gp.nbytes, 2,
+           note='window ArgMax kernel + gather kernel; bits of the Im2Col / ArgMax / Col2Im composition')
     xa = chx.array(rng.standard_normal((128, 2048, 7, 7)).astype(np.float16))
     ga = chx.array(rng.standard_normal((128, 2048, 1, 1)).astype(np.float16))
     t = graph_time(lambda: chx.average_pool_grad(xa, ga, 7, 1, 0, 'zero'), 5)

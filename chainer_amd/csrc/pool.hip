@@ -345,6 +345,234 @@ PoolArgs MakeArgs(const hipcx_array* x, const int64_t* ksize, const int64_t* str
     return p;
 }
 
+// ---------------------------------------------------------------------------------------------
+// Gradients (CX/kernels/pooling.h:47-107).  The native backend scatters through Col2Im: a zeroed padded image receives, for
+// every kernel offset in (r, s) order, one strided in-place Add (CX/native/col2im.cc:76-122).  Here every input position
+// gathers its contributions in that same (r, s) order with the same rounding after every addition, so the result has the bits
+// of the composition.
+// ---------------------------------------------------------------------------------------------
+struct PoolGradArgs {
+    const void* x;     // max only
+    const void* gout;
+    void* gx;
+    int N, C, H, W, OH, OW;
+    int kh, kw, sh, sw, ph, pw;
+    int64_t xsN, xsC, xsH, xsW;  // elements
+    int64_t gsN, gsC, gsH, gsW;  // gout
+    int64_t dsN, dsC, dsH, dsW;  // gx
+    int pad_mode;
+    int w_fastest;
+    int* win_index;  // max only: ArgMax of every window, dense [N, C, OH, OW]
+};
+
+template <typename V>
+struct WinBest {
+    V v;
+    int i;  // < 0: empty
+};
+
+template <typename V>
+__device__ __forceinline__ void WinReduce(WinBest<V> next, WinBest<V>& acc) {  // ArgMax's rule: a later element must be strictly larger
+    if (next.i < 0) return;
+    if (acc.i < 0 || acc.v < next.v) acc = next;
+}
+
+// ArgMax over the kh x kw window of output (oh, ow) as the native backend computes it: the reduction loop of CX/native/reduce.h:46-83
+// over the Im2Col'ed window, whose out-of-image taps hold the lowest value (CX/native/native_device/pool.cc:97-113).
+template <typename T>
+__device__ int WindowArgMax(const PoolGradArgs& p, const T* xb, int oh, int ow) {
+    using V = std::conditional_t<std::is_same<T, half_t>::value, float, std::conditional_t<std::is_same<T, bool>::value, int, T>>;
+    using B = WinBest<V>;
+    const int h0 = oh * p.sh - p.ph, w0 = ow * p.sw - p.pw;
+    const int len = p.kh * p.kw;
+    int i = 0, r = 0, q = 0;
+    auto next_elem = [&]() -> B {
+        const int ih = h0 + r, iw = w0 + q;
+        T v = (ih >= 0 && ih < p.H && iw >= 0 && iw < p.W) ? xb[ih * p.xsH + iw * p.xsW] : Lowest<T>();
+        B b{static_cast<V>(v), i};
+        ++i;
+        if (++q == p.kw) q = 0, ++r;
+        return b;
+    };
+    const int main_len = len - (len % 4);
+    B accum{V(0), -1};
+    if (main_len <= 32) {  // one block of the tree: groups of four, then the tail (every usual window)
+        while (i < main_len) {
+            B p0 = next_elem();
+            WinReduce(next_elem(), p0);
+            B p1 = next_elem();
+            WinReduce(next_elem(), p1);
+            WinReduce(p1, p0);
+            WinReduce(p0, accum);
+        }
+        while (i < len) WinReduce(next_elem(), accum);
+        return accum.i;
+    }
+    B tree[26];
+    while (i < main_len) {
+        if (i != 0 && i % 32 == 0) {
+            int lvl = 0;
+            for (int k = i >> 1; k % 32 == 0; k >>= 1, ++lvl) WinReduce(tree[lvl], accum);
+            tree[lvl] = accum;
+            accum = B{V(0), -1};
+        }
+        B p0 = next_elem();
+        WinReduce(next_elem(), p0);
+        B p1 = next_elem();
+        WinReduce(next_elem(), p1);
+        WinReduce(p1, p0);
+        WinReduce(p0, accum);
+    }
+    while (i < len) WinReduce(next_elem(), accum);
+    int lvl = 0;
+    for (int k = (len / 4 - 1) / 8; k > 0; k >>= 1, ++lvl) {
+        if (k & 1) WinReduce(tree[lvl], accum);
+    }
+    return accum.i;
+}
+
+template <typename T, typename IdxT>
+__global__ __launch_bounds__(256) void WindowArgMaxKernel(PoolGradArgs p, IdxT total) {
+    const T* x = static_cast<const T*>(p.x);
+    for (IdxT idx = static_cast<IdxT>(blockIdx.x) * blockDim.x + threadIdx.x; idx < total; idx += static_cast<IdxT>(gridDim.x) * blockDim.x) {
+        IdxT t = idx;
+        const int ow = static_cast<int>(t % p.OW);
+        t /= p.OW;
+        const int oh = static_cast<int>(t % p.OH);
+        t /= p.OH;
+        const int c = static_cast<int>(t % p.C);
+        const int64_t n = static_cast<int64_t>(t / p.C);
+        p.win_index[idx] = WindowArgMax<T>(p, x + n * p.xsN + static_cast<int64_t>(c) * p.xsC, oh, ow);
+    }
+}
+
+template <typename T, bool IS_MAX, typename IdxT>
+__global__ __launch_bounds__(256) void PoolGradKernel(PoolGradArgs p, IdxT total) {
+    using C = compute_t<T>;
+    const T* gout = static_cast<const T*>(p.gout);
+    T* gx = static_cast<T*>(p.gx);
+    for (IdxT idx = static_cast<IdxT>(blockIdx.x) * blockDim.x + threadIdx.x; idx < total; idx += static_cast<IdxT>(gridDim.x) * blockDim.x) {
+        int c, w, h;
+        int64_t n;
+        IdxT t = idx;
+        if (p.w_fastest) {
+            w = static_cast<int>(t % p.W);
+            t /= p.W;
+            h = static_cast<int>(t % p.H);
+            t /= p.H;
+            c = static_cast<int>(t % p.C);
+            n = static_cast<int64_t>(t / p.C);
+        } else {
+            c = static_cast<int>(t % p.C);
+            t /= p.C;
+            w = static_cast<int>(t % p.W);
+            t /= p.W;
+            h = static_cast<int>(t % p.H);
+            n = static_cast<int64_t>(t / p.H);
+        }
+        const int* wb = IS_MAX ? p.win_index + (n * p.C + c) * (static_cast<int64_t>(p.OH) * p.OW) : nullptr;
+        const T* gb = gout + n * p.gsN + static_cast<int64_t>(c) * p.gsC;
+        const int y = h + p.ph, xq = w + p.pw;
+        T acc = T(0);
+        // windows (i, j) that cover this position, walked with the kernel offset r = y - i * sh (and q) ascending
+        int i_hi = y / p.sh, j_hi = xq / p.sw;
+        if (i_hi > p.OH - 1) i_hi = p.OH - 1;
+        if (j_hi > p.OW - 1) j_hi = p.OW - 1;
+        for (int i = i_hi; i >= 0; --i) {
+            const int r = y - i * p.sh;
+            if (r >= p.kh) break;
+            for (int j = j_hi; j >= 0; --j) {
+                const int q = xq - j * p.sw;
+                if (q >= p.kw) break;
+                T g = gb[i * p.gsH + j * p.gsW];
+                if constexpr (IS_MAX) {
+                    if (wb[i * p.OW + j] != r * p.kw + q) continue;
+                } else if (p.pad_mode == HIPCX_PAD_IGNORE) {  // gout / width first, in T arithmetic (pool.cc:197-250, 304-346)
+                    const int h0 = i * p.sh - p.ph, w0 = j * p.sw - p.pw;
+                    const int hcnt = (h0 + p.kh < p.H ? h0 + p.kh : p.H) - (h0 < 0 ? 0 : h0);
+                    const int wcnt = (w0 + p.kw < p.W ? w0 + p.kw : p.W) - (w0 < 0 ? 0 : w0);
+                    const T width = static_cast<T>(static_cast<C>(static_cast<T>(static_cast<C>(hcnt))) * static_cast<C>(static_cast<T>(static_cast<C>(wcnt))));
+                    g = static_cast<T>(static_cast<C>(g) / static_cast<C>(width));
+                }
+                acc = static_cast<T>(static_cast<C>(acc) + static_cast<C>(g));
+            }
+        }
+        if (!IS_MAX && p.pad_mode == HIPCX_PAD_ZERO) {
+            acc = static_cast<T>(static_cast<C>(acc) / static_cast<C>(static_cast<T>(static_cast<C>(p.kh * p.kw))));
+        }
+        gx[n * p.dsN + static_cast<int64_t>(c) * p.dsC + h * p.dsH + w * p.dsW] = acc;
+    }
+}
+
+PoolGradArgs MakeGradArgs(const hipcx_array* x, const hipcx_array* gout, const int64_t* ksize, const int64_t* stride, const int64_t* pad,
+                          int cover_all, const hipcx_array* gx) {
+    ValidateArray(gout, "gout");
+    ValidateArray(gx, "gx");
+    if (x != nullptr) ValidateArray(x, "x");
+    HIPCX_REQUIRE(gx->ndim == 4 && gout->ndim == 4 && (x == nullptr || x->ndim == 4), HIPCX_NOT_IMPLEMENTED_ERROR,
+                  "hip pooling supports 2 spatial dimensions");
+    HIPCX_REQUIRE(gout->dtype == gx->dtype && (x == nullptr || x->dtype == gx->dtype), HIPCX_DTYPE_ERROR, "x, gout and gx must share a dtype");
+    HIPCX_REQUIRE(x == nullptr || SameShape(x, gx), HIPCX_DIMENSION_ERROR, "gx must have x's shape");
+    HIPCX_REQUIRE(ksize && stride && pad, HIPCX_CHAINERX_ERROR, "null window parameters");
+    HIPCX_REQUIRE(ksize[0] > 0 && ksize[1] > 0 && stride[0] > 0 && stride[1] > 0 && pad[0] >= 0 && pad[1] >= 0, HIPCX_DIMENSION_ERROR,
+                  "invalid kernel size, stride or pad");
+    int64_t oh = hipcx_conv_out_dim(gx->shape[2], ksize[0], stride[0], pad[0], cover_all);
+    int64_t ow = hipcx_conv_out_dim(gx->shape[3], ksize[1], stride[1], pad[1], cover_all);
+    HIPCX_REQUIRE(gout->shape[0] == gx->shape[0] && gout->shape[1] == gx->shape[1] && gout->shape[2] == oh && gout->shape[3] == ow,
+                  HIPCX_DIMENSION_ERROR, "gout has the wrong shape " + ShapeStr(gout));
+    for (int i = 0; i < 4; ++i) HIPCX_REQUIRE(gx->shape[i] < (1LL << 31), HIPCX_NOT_IMPLEMENTED_ERROR, "extent too large");
+    HIPCX_REQUIRE(ksize[0] * ksize[1] < (1LL << 24) && ksize[0] < (1 << 20) && ksize[1] < (1 << 20), HIPCX_NOT_IMPLEMENTED_ERROR, "window too large");
+    PoolGradArgs p{};
+    p.x = x ? x->data : nullptr;
+    p.gout = gout->data;
+    p.gx = gx->data;
+    p.N = static_cast<int>(gx->shape[0]);
+    p.C = static_cast<int>(gx->shape[1]);
+    p.H = static_cast<int>(gx->shape[2]);
+    p.W = static_cast<int>(gx->shape[3]);
+    p.OH = static_cast<int>(oh);
+    p.OW = static_cast<int>(ow);
+    p.kh = static_cast<int>(ksize[0]);
+    p.kw = static_cast<int>(ksize[1]);
+    p.sh = static_cast<int>(stride[0]);
+    p.sw = static_cast<int>(stride[1]);
+    p.ph = static_cast<int>(pad[0]);
+    p.pw = static_cast<int>(pad[1]);
+    if (x != nullptr) p.xsN = ElemStride(x, 0), p.xsC = ElemStride(x, 1), p.xsH = ElemStride(x, 2), p.xsW = ElemStride(x, 3);
+    p.gsN = ElemStride(gout, 0), p.gsC = ElemStride(gout, 1), p.gsH = ElemStride(gout, 2), p.gsW = ElemStride(gout, 3);
+    p.dsN = ElemStride(gx, 0), p.dsC = ElemStride(gx, 1), p.dsH = ElemStride(gx, 2), p.dsW = ElemStride(gx, 3);
+    p.pad_mode = HIPCX_PAD_ZERO;
+    int64_t a_c = p.dsC < 0 ? -p.dsC : p.dsC, a_w = p.dsW < 0 ? -p.dsW : p.dsW;
+    p.w_fastest = a_w < a_c ? 1 : 0;
+    return p;
+}
+
+template <typename T, bool IS_MAX>
+void RunPoolGrad(const PoolGradArgs& p, hipStream_t stream) {
+    const int64_t total = static_cast<int64_t>(p.N) * p.C * p.H * p.W;
+    const int64_t windows = static_cast<int64_t>(p.N) * p.C * p.OH * p.OW;
+    if (total == 0) return;
+    const int64_t cap = static_cast<int64_t>(NumCUs()) * 64;
+    auto grid_for = [&](int64_t n) { int64_t b = (n + 255) / 256; return dim3(static_cast<unsigned>(b > cap ? cap : (b < 1 ? 1 : b))); };
+    const bool narrow = total + cap * 256 < (1LL << 31) && windows + cap * 256 < (1LL << 31);  // 32-bit index arithmetic
+    if constexpr (IS_MAX) {
+        if (windows > 0) {
+            if (narrow) {
+                hipLaunchKernelGGL((WindowArgMaxKernel<T, unsigned>), grid_for(windows), dim3(256), 0, stream, p, static_cast<unsigned>(windows));
+            } else {
+                hipLaunchKernelGGL((WindowArgMaxKernel<T, int64_t>), grid_for(windows), dim3(256), 0, stream, p, windows);
+            }
+            CheckLaunch("window_argmax");
+        }
+    }
+    if (narrow) {
+        hipLaunchKernelGGL((PoolGradKernel<T, IS_MAX, unsigned>), grid_for(total), dim3(256), 0, stream, p, static_cast<unsigned>(total));
+    } else {
+        hipLaunchKernelGGL((PoolGradKernel<T, IS_MAX, int64_t>), grid_for(total), dim3(256), 0, stream, p, total);
+    }
+    CheckLaunch("pool_grad");
+}
+
 }  // namespace
 }  // namespace hipcx
 
@@ -373,6 +601,48 @@ int hipcx_average_pool(const hipcx_array* x, const int64_t* kernel_size, const i
         VisitFloatDtype(x->dtype, [&](auto tag) {
             using T = typename decltype(tag)::type;
             RunPool<T, false>(p, AsStream(stream));
+        });
+    });
+}
+
+size_t hipcx_max_pool_grad_workspace_size(const hipcx_array* gout) {
+    if (gout == nullptr || gout->ndim != 4) return 0;
+    int64_t n = 1;
+    for (int i = 0; i < 4; ++i) n *= gout->shape[i] > 0 ? gout->shape[i] : 0;
+    return static_cast<size_t>(n) * sizeof(int);
+}
+
+int hipcx_max_pool_grad(const hipcx_array* x, const hipcx_array* gout, const int64_t* kernel_size, const int64_t* stride,
+                        const int64_t* pad, int cover_all, const hipcx_array* gx, void* workspace, size_t workspace_bytes, void* stream) {
+    return Guard([&] {
+        HIPCX_REQUIRE(x != nullptr, HIPCX_CHAINERX_ERROR, "null array x");
+        PoolGradArgs p = MakeGradArgs(x, gout, kernel_size, stride, pad, cover_all, gx);
+        const size_t need = hipcx_max_pool_grad_workspace_size(gout);
+        HIPCX_REQUIRE(need == 0 || (workspace != nullptr && workspace_bytes >= need), HIPCX_CHAINERX_ERROR,
+                      "max_pool_grad workspace too small: need " + std::to_string(need) + " bytes");
+        HIPCX_REQUIRE(reinterpret_cast<uintptr_t>(workspace) % 4 == 0, HIPCX_CHAINERX_ERROR, "workspace must be 4-byte aligned");
+        p.win_index = static_cast<int*>(workspace);
+        VisitDtype(gx->dtype, [&](auto tag) {
+            using T = typename decltype(tag)::type;
+            if constexpr (std::is_same<T, bool>::value) {
+                throw Error(HIPCX_DTYPE_ERROR, "max_pool_grad: bool arrays are not supported");
+            } else {
+                RunPoolGrad<T, true>(p, AsStream(stream));
+            }
+        });
+    });
+}
+
+int hipcx_average_pool_grad(const hipcx_array* gout, const int64_t* kernel_size, const int64_t* stride, const int64_t* pad, int pad_mode,
+                            const hipcx_array* gx, void* stream) {
+    return Guard([&] {
+        HIPCX_REQUIRE(pad_mode == HIPCX_PAD_ZERO || pad_mode == HIPCX_PAD_IGNORE, HIPCX_CHAINERX_ERROR, "invalid pad mode");
+        HIPCX_REQUIRE(gx != nullptr && IsFloatDtype(gx->dtype), HIPCX_DTYPE_ERROR, "cannot apply average pooling to non-float arrays");
+        PoolGradArgs p = MakeGradArgs(nullptr, gout, kernel_size, stride, pad, 0, gx);
+        p.pad_mode = pad_mode;
+        VisitFloatDtype(gx->dtype, [&](auto tag) {
+            using T = typename decltype(tag)::type;
+            RunPoolGrad<T, false>(p, AsStream(stream));
         });
     });
 }

@@ -942,16 +942,16 @@ public:
         auto& st = dynamic_cast<HipMaxPoolGradState&>(*state);
         const Array& x = st.x();
         Device& device = x.device();
+        device.CheckDevicesCompatible(x, gout);
         SetDeviceScope scope{device.index()};
-        Scalar lowest = GetKind(x.dtype()) == DtypeKind::kFloat ? Scalar{-std::numeric_limits<double>::infinity()} : Scalar{0};
-        Array col = HipIm2Col(x, kernel_size, stride, pad, st.cover_all(), lowest);
-        Array indices = col.ArgMax(Axes{2, 3});  // the native tie rule picks the position inside a window
-        // every output position owns its own slots of the col, so the AddAt of the native kernel degenerates to a select
-        int64_t kt = kernel_size[0] * kernel_size[1];
-        Shape lifted{gout.shape()[0], gout.shape()[1], 1, 1, gout.shape()[2], gout.shape()[3]};
-        Array taps = Arange(kt, Dtype::kInt64, device).Reshape(Shape{1, 1, kernel_size[0], kernel_size[1], 1, 1});
-        Array gcol = Where(Equal(indices.Reshape(lifted), taps), gout.Reshape(lifted), Scalar{0, GetKind(gout.dtype())});
-        Array actual_gx = HipCol2Im(gcol, stride, pad, Dims{x.shape()[2], x.shape()[3]});
+        // one kernel with the bits of the native Im2Col / ArgMax / AddAt / Col2Im sequence (native/native_device/pool.cc:97-143)
+        Array actual_gx = Empty(x.shape(), x.dtype(), device);
+        const Array& g = gout.dtype() == x.dtype() ? gout : gout.AsType(x.dtype());
+        hipcx_array cx = ToC(x), cg = ToC(g), cgx = ToC(actual_gx);
+        int64_t k[2] = {kernel_size[0], kernel_size[1]}, s[2] = {stride[0], stride[1]}, p[2] = {pad[0], pad[1]};
+        size_t ws_bytes = hipcx_max_pool_grad_workspace_size(&cg);
+        std::shared_ptr<void> ws = device.Allocate(ws_bytes);
+        Check(hipcx_max_pool_grad(&cx, &cg, k, s, p, st.cover_all() ? 1 : 0, &cgx, ws.get(), ws_bytes, nullptr));
         return std::make_tuple(std::move(actual_gx), std::unique_ptr<MaxPoolGradGradState>{});
     }
 };
@@ -965,29 +965,16 @@ public:
         auto& st = dynamic_cast<HipAveragePoolGradState&>(*state);
         const Array& x = st.x();
         Device& device = x.device();
+        device.CheckDevicesCompatible(x, gout);
         SetDeviceScope scope{device.index()};
-        Shape gcol_shape{gout.shape()[0], gout.shape()[1], kernel_size[0], kernel_size[1], gout.shape()[2], gout.shape()[3]};
-        Shape lifted{gout.shape()[0], gout.shape()[1], 1, 1, gout.shape()[2], gout.shape()[3]};
-        Dims out_size{x.shape()[2], x.shape()[3]};
-        if (pad_mode == AveragePoolPadMode::kZero) {
-            Array actual_gx = HipCol2Im(gout.Reshape(lifted).BroadcastTo(gcol_shape), stride, pad, out_size).Copy();
-            actual_gx /= Scalar{kernel_size[0] * kernel_size[1]};
-            return actual_gx;
-        }
-        // per-position count of in-image taps (CX/native/native_device/pool.cc:197-250), built on the host: it is tiny
-        std::vector<double> widths(static_cast<size_t>(gout.shape()[2] * gout.shape()[3]));
-        for (int64_t i = 0; i < gout.shape()[2]; ++i) {
-            double wi = static_cast<double>(std::min(i * stride[0] - pad[0] + kernel_size[0], x.shape()[2]) - std::max<int64_t>(i * stride[0] - pad[0], 0));
-            for (int64_t j = 0; j < gout.shape()[3]; ++j) {
-                double wj = static_cast<double>(std::min(j * stride[1] - pad[1] + kernel_size[1], x.shape()[3]) - std::max<int64_t>(j * stride[1] - pad[1], 0));
-                widths[static_cast<size_t>(i * gout.shape()[3] + j)] = wi * wj;
-            }
-        }
-        Shape w_shape{gout.shape()[2], gout.shape()[3]};
-        Array w_host = internal::FromHostData(w_shape, Dtype::kFloat64, std::shared_ptr<void>(widths.data(), [](void*) {}),
-                                              Strides{w_shape, Dtype::kFloat64}, 0, GetDefaultContext().GetNativeBackend().GetDevice(0));
-        Array w_dev = w_host.ToDevice(device).AsType(gout.dtype(), false);
-        return HipCol2Im((gout / w_dev).Reshape(lifted).BroadcastTo(gcol_shape), stride, pad, out_size);
+        // one kernel with the bits of the native broadcast / Col2Im / Divide sequence (native/native_device/pool.cc:304-346)
+        Array actual_gx = Empty(x.shape(), x.dtype(), device);
+        const Array& g = gout.dtype() == x.dtype() ? gout : gout.AsType(x.dtype());
+        hipcx_array cg = ToC(g), cgx = ToC(actual_gx);
+        int64_t k[2] = {kernel_size[0], kernel_size[1]}, s[2] = {stride[0], stride[1]}, p[2] = {pad[0], pad[1]};
+        int mode = pad_mode == AveragePoolPadMode::kZero ? HIPCX_PAD_ZERO : HIPCX_PAD_IGNORE;
+        Check(hipcx_average_pool_grad(&cg, k, s, p, mode, &cgx, nullptr));
+        return actual_gx;
     }
 };
 HIPCX_REGISTER_KERNEL(AveragePoolGradKernel, HipAveragePoolGradKernel)

@@ -1408,12 +1408,30 @@ def batch_norm_grad(x, gamma, gout, state, axis=None):
             gbeta.astype(beta_dtype, False).reshape(gamma.shape))
 
 
+# True: pooling gradients run as the native backend's Im2Col / ArgMax / Col2Im composition instead of the dedicated kernels (tests
+# compare the two bit for bit).
+COMPOSE_POOL_GRADIENTS = False
+
+
 def max_pool_grad(x, gout, ksize, stride=None, pad=0, cover_all=False):
     """MaxPoolGradKernel after the native backend (CX/native/native_device/pool.cc:97-143): Im2Col with -inf padding, ArgMax over
     the kernel axes (its tie rule picks the position), gout placed at that kernel offset of an otherwise zero col, Col2Im."""
     ksize = _pair(ksize)
     stride = ksize if stride is None else _pair(stride)
     pad = _pair(pad)
+    if x.ndim == 4 and x.dtype != numpy.dtype('bool') and gout.dtype == x.dtype and not COMPOSE_POOL_GRADIENTS:
+        # one kernel: every input position gathers, in kernel-offset order, gout of the windows whose ArgMax it is -- the bits
+        # of the composition below
+        oh = conv_out_dim(x.shape[2], ksize[0], stride[0], pad[0], cover_all)
+        ow = conv_out_dim(x.shape[3], ksize[1], stride[1], pad[1], cover_all)
+        if gout.shape != (x.shape[0], x.shape[1], oh, ow):
+            raise _lib.DimensionError('gout has the wrong shape')
+        gx = ndarray.empty(x.shape, x.dtype)
+        nbytes = _lib.load().hipcx_max_pool_grad_workspace_size(gout.desc())
+        ws, wsp = _workspace(nbytes)
+        _lib.call('hipcx_max_pool_grad', x.desc(), gout.desc(), _i64(ksize), _i64(stride), _i64(pad), int(bool(cover_all)), gx.desc(),
+                  wsp, nbytes, current_stream())
+        return gx
     lowest = -numpy.inf if _kind(x.dtype) == 3 else (0 if x.dtype == numpy.dtype('bool') else int(numpy.iinfo(x.dtype).min))
     col = im2col(x, ksize, stride, pad, cover_all, lowest)            # [N, C, kh, kw, oh, ow]
     indices = argmax(col, (2, 3))                                     # [N, C, oh, ow]
@@ -1452,6 +1470,11 @@ def average_pool_grad(x, gout, ksize, stride=None, pad=0, pad_mode='ignore'):
     stride = ksize if stride is None else _pair(stride)
     pad = _pair(pad)
     n, c, oh, ow = gout.shape
+    if x.ndim == 4 and _kind(x.dtype) == 3 and gout.dtype == x.dtype and not COMPOSE_POOL_GRADIENTS:
+        gx = ndarray.empty(x.shape, x.dtype)
+        _lib.call('hipcx_average_pool_grad', gout.desc(), _i64(ksize), _i64(stride), _i64(pad), {'zero': 1, 'ignore': 2}[pad_mode],
+                  gx.desc(), current_stream())
+        return gx
     g = gout
     if pad_mode == 'ignore':
         def widths(dim, k, st, p, count):  # GetPadModeIgnorePoolingWidths (pool.cc:197-250)

@@ -278,6 +278,17 @@ int hipcx_max_pool(const hipcx_array* x, const int64_t* kernel_size, const int64
 int hipcx_average_pool(const hipcx_array* x, const int64_t* kernel_size, const int64_t* stride, const int64_t* pad, int pad_mode,
                        const hipcx_array* out, void* stream);
 
+/* ---- pooling gradients: MaxPoolGradKernel CX/kernels/pooling.h:47-65, AveragePoolGradKernel CX/kernels/pooling.h:95-107 ----
+ * x is the forward input the reference keeps in its grad state; gx has x's shape.  Results carry the bits of the native
+ * backend's Im2Col / ArgMax / Col2Im composition (CX/native/native_device/pool.cc:97-143, 304-346): contributions are added in
+ * kernel-offset order with one rounding per addition, and the window maximum is chosen by ArgMax's tie and NaN rule.
+ * `workspace`: device memory of hipcx_max_pool_grad_workspace_size(gout) bytes (the ArgMax of every window, one int each). */
+size_t hipcx_max_pool_grad_workspace_size(const hipcx_array* gout);
+int hipcx_max_pool_grad(const hipcx_array* x, const hipcx_array* gout, const int64_t* kernel_size, const int64_t* stride,
+                        const int64_t* pad, int cover_all, const hipcx_array* gx, void* workspace, size_t workspace_bytes, void* stream);
+int hipcx_average_pool_grad(const hipcx_array* gout, const int64_t* kernel_size, const int64_t* stride, const int64_t* pad, int pad_mode,
+                            const hipcx_array* gx, void* stream);
+
 /* ---- indexing: TakeKernel CX/kernels/indexing.h:17 ----
  * `error_flag` is a device int32 the caller zeroes before the call; with mode DEFAULT/RAISE the
  * kernel stores 1 there when an index is out of range (the native backend raises IndexError,

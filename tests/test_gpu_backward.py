@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 
 from oracle import native as O
-from helpers import assert_close, assert_exact
+from helpers import assert_close, assert_exact, channels_last
 
 pytestmark = pytest.mark.gpu
 
@@ -148,3 +148,42 @@ def test_max_pool_grad_grad_and_nanarg():
     assert_exact(chx.nanargmax(chx.array(a), 1).get(), O.nanargmax(a, 1), 'nanargmax')
     assert_exact(chx.nanargmin(chx.array(a), 1).get(), O.nanargmin(a, 1), 'nanargmin')
     assert chx.nanargmax(chx.array(a), 1).get()[0] == np.nanargmax(a[0]) and chx.nanargmin(chx.array(a), 1).get()[2] == np.nanargmin(a[2])
+
+
+@pytest.mark.parametrize('dt', ['float32', 'float16', 'float64', 'int32'])
+def test_pool_gradient_kernels_have_the_bits_of_the_composition(dt):
+    """hipcx_max_pool_grad / hipcx_average_pool_grad against the Im2Col / ArgMax / Col2Im composition on the device: same
+    additions in the same order, same ArgMax choice among ties and NaNs (a 7x7 window crosses the 32-element block of the
+    reduction tree), for dense, channels-last and overlapping / non-overlapping windows."""
+    import chainer_amd as chx
+    from chainer_amd import routines
+    rng = np.random.default_rng(61)
+    cases = POOL_CASES + [((2, 3, 20, 20), 7, 3, 3, False), ((1, 2, 15, 15), 7, 1, 0, False), ((2, 4, 9, 11), (3, 2), (1, 2), (1, 0), True),
+                          ((3, 5, 12, 12), 3, 2, 1, False), ((2, 8, 56, 56), 3, 2, 1, False)]
+    for (shape, k, s, p, cv) in cases:
+        x = rng.integers(-3, 4, shape).astype(dt)
+        if np.dtype(dt).kind == 'f':
+            x[rng.random(shape) < 0.05] = np.nan
+        y_shape = O.max_pool(np.nan_to_num(x), k, s, p, cv).shape
+        g = rng.standard_normal(y_shape).astype(dt) if np.dtype(dt).kind == 'f' else rng.integers(-50, 50, y_shape).astype(dt)
+        for lay in ('nchw', 'nhwc'):
+            X = chx.array(x) if lay == 'nchw' else channels_last(chx, x)
+            G = chx.array(g) if lay == 'nchw' else channels_last(chx, g)
+            got = chx.max_pool_grad(X, G, k, s, p, cv).get()
+            routines.COMPOSE_POOL_GRADIENTS = True
+            try:
+                ref = chx.max_pool_grad(X, G, k, s, p, cv).get()
+            finally:
+                routines.COMPOSE_POOL_GRADIENTS = False
+            assert_exact(got, ref, 'max_pool_grad %s %s %r' % (dt, lay, (shape, k, s, p, cv)))
+        if np.dtype(dt).kind == 'f' and not cv:
+            for mode in ('zero', 'ignore'):
+                got = chx.average_pool_grad(chx.array(x), chx.array(g), k, s, p, mode).get()
+                routines.COMPOSE_POOL_GRADIENTS = True
+                try:
+                    ref = chx.average_pool_grad(chx.array(x), chx.array(g), k, s, p, mode).get()
+                finally:
+                    routines.COMPOSE_POOL_GRADIENTS = False
+                assert_exact(got, ref, 'average_pool_grad %s %s %r' % (dt, mode, (shape, k, s, p)))
+    with pytest.raises(chx.DimensionError):
+        chx.max_pool_grad(chx.zeros((1, 1, 4, 4), dt), chx.zeros((1, 1, 3, 3), dt), 2, 2, 0)
