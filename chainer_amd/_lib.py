@@ -170,6 +170,9 @@ SIGNATURES = {
     'hipcx_profile_stop': (_INT, [_I64P, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double),
                                   ctypes.POINTER(ctypes.c_double)]),
     'hipcx_fixed_batch_norm': (_INT, [_A, _A, _A, _A, _A, _S, _I8P, _INT, _A, _V]),
+    'hipcx_batch_norm_workspace_size': (_SZ, [_A, _I8P, _INT]),
+    'hipcx_batch_norm': (_INT, [_A, _A, _A, _A, _A, _S, _S, _I8P, _INT, _A, _A, _A, _V, _SZ, _V]),
+    'hipcx_batch_norm_grad': (_INT, [_A, _A, _A, _A, _A, _I8P, _INT, _A, _A, _A, _V, _SZ, _V]),
     'hipcx_max_pool': (_INT, [_A, _I64P, _I64P, _I64P, _INT, _A, _V]),
     'hipcx_average_pool': (_INT, [_A, _I64P, _I64P, _I64P, _INT, _A, _V]),
     'hipcx_max_pool_grad_workspace_size': (_SZ, [_A]),

@@ -253,9 +253,9 @@ def section_lstm(chx, oracle, with_cpu):
 
 
 def section_backward(chx, oracle, with_cpu):
-    """Backward / training kernels at ResNet-50 layer shapes (float16, batch 32).  The convolution and batch-norm gradients are
-    compositions of the forward kernels (Im2Col / Col2Im copies plus one matrix product; reductions and elementwise kernels) --
-    functional, not tuned; the pooling gradients have kernels of their own.  Timed as HIP-graph replays (a composition is 10-25
+    """Backward / training kernels at ResNet-50 layer shapes (float16, batch 32).  The convolution gradients are compositions of
+    the forward kernels (Im2Col / Col2Im copies plus one matrix product) -- functional, not tuned; batch normalisation, its
+    gradient and the pooling gradients have kernels of their own.  Timed as HIP-graph replays (a composition is 10-25
     kernel launches; issued eagerly from Python it would be host-bound)."""
     rng = np.random.default_rng(6)
     n, c, k, hw = 32, 256, 256, 14
@@ -278,11 +278,11 @@ def section_backward(chx, oracle, with_cpu):
     out_state = []
     out_state[:] = [chx.batch_norm(xb, prm[0], prm[1], rm, rv)]
     t = graph_time(lambda: chx.batch_norm(xb, prm[0], prm[1], rm, rv), 5)
-    bw_row('backward', 'batch_norm (training forward, routine composition)', shape, t, 3 * nbytes, 20,
-           note='algorithmic bytes: two reads (statistics, normalise) and one write')
+    bw_row('backward', 'batch_norm (training forward)', shape, t, 4 * nbytes, 5,
+           note='algorithmic bytes: three reads (sum, centred sum of squares, normalise) and one write')
     state = out_state[0][1]
     t = graph_time(lambda: chx.batch_norm_grad(xb, prm[0], gb, state), 5)
-    bw_row('backward', 'batch_norm_grad (routine composition)', shape, t, 5 * nbytes, 12,
+    bw_row('backward', 'batch_norm_grad', shape, t, 5 * nbytes, 5,
            note='algorithmic bytes: x and gout read twice, gx written')
     xp = chx.array(rng.standard_normal((32, 64, 112, 112)).astype(np.float16))
     gp = chx.array(rng.standard_normal((32, 64, 56, 56)).astype(np.float16))

@@ -1,0 +1,450 @@
+// BatchNorm in training mode and its gradient (BatchNormKernel / BatchNormGradKernel, CX/kernels/normalization.h:32-61) for the
+// layout every ChainerX routine hands over: x dense [N, C, L] (L = product of the spatial extents) normalised over every axis but
+// the channel axis, all arrays of one float dtype.
+//
+// The reference's generic kernels are routine compositions (CX/routines/normalization.cc:155-250): Mean, Var = Mean((x - mean)^2),
+// 1 / sqrt(var + eps), five elementwise passes, four in-place updates of the running statistics -- about twenty launches that read
+// or write the tensor a dozen times.  Here: two statistics passes (sum, then centred sum of squares: the two-pass variance of the
+// reference, not E[x^2] - mean^2), one per-channel finish, one normalising pass.  Arithmetic runs in float (double for float64)
+// with one rounding per stored value, so float16 results are at least as accurate as the composition's; agreement with it is to
+// tolerance, not to the bit.
+//
+// Statistics: grid (C, S).  Block (c, s) walks images s, s + S, ... of channel c with 16-byte loads, reduces over the block and
+// stores one partial; the finish kernel adds a channel's S partials in order (deterministic).
+#include "elementwise.h"
+
+namespace hipcx {
+namespace {
+
+constexpr int kBnTrainThreads = 256;
+
+inline size_t RoundUpTo(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+template <typename C>
+__device__ __forceinline__ C BlockSum(C v, C* lds) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_down(v, o);
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    __syncthreads();  // lds may still be read by a previous call
+    if (lane == 0) lds[wave] = v;
+    __syncthreads();
+    C r = C(0);
+    if (threadIdx.x == 0) {
+        for (int w = 0; w < kBnTrainThreads / 64; ++w) r += lds[w];
+    }
+    return r;  // valid in thread 0
+}
+
+struct BnStatArgs {
+    const void* x;
+    const void* g;        // gradient pass only
+    const void* mean;     // compute-type vector [C] (workspace)
+    const void* inv_std;  // compute-type vector [C] (gradient pass)
+    void* partial;        // compute-type [C][S][2]
+    int N, C;
+    int64_t L;
+    int S;
+};
+
+// MODE 0: sum x.  MODE 1: sum (x - mean)^2.  MODE 2: sum g and sum g * (x - mean) * inv_std.
+template <typename T, int MODE, int VEC>
+__global__ __launch_bounds__(kBnTrainThreads) void BnStatKernel(BnStatArgs p) {
+    using C = compute_t<T>;
+    __shared__ C lds[kBnTrainThreads / 64];
+    const int c = blockIdx.x, s = blockIdx.y;
+    const T* x = static_cast<const T*>(p.x);
+    const T* g = static_cast<const T*>(p.g);
+    C m = C(0), is = C(1);
+    if (MODE >= 1) m = static_cast<const C*>(p.mean)[c];
+    if (MODE == 2) is = static_cast<const C*>(p.inv_std)[c];
+    C a0 = C(0), a1 = C(0);
+    const int64_t lv = p.L / VEC;
+    for (int n = s; n < p.N; n += p.S) {
+        const int64_t base = (static_cast<int64_t>(n) * p.C + c) * p.L;
+        for (int64_t v = threadIdx.x; v < lv; v += kBnTrainThreads) {
+            Vec<T, VEC> xv = *reinterpret_cast<const Vec<T, VEC>*>(x + base + v * VEC);
+            Vec<T, VEC> gv;
+            if (MODE == 2) gv = *reinterpret_cast<const Vec<T, VEC>*>(g + base + v * VEC);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                C xe = static_cast<C>(xv.v[e]);
+                if (MODE == 0) {
+                    a0 += xe;
+                } else if (MODE == 1) {
+                    C d = xe - m;
+                    a0 += d * d;
+                } else {
+                    C ge = static_cast<C>(gv.v[e]);
+                    a0 += ge;
+                    a1 += ge * ((xe - m) * is);
+                }
+            }
+        }
+    }
+    C r0 = BlockSum<C>(a0, lds);
+    C r1 = MODE == 2 ? BlockSum<C>(a1, lds) : C(0);
+    if (threadIdx.x == 0) {
+        C* out = static_cast<C*>(p.partial) + (static_cast<int64_t>(c) * p.S + s) * 2;
+        out[0] = r0;
+        out[1] = r1;
+    }
+}
+
+struct BnFinishArgs {
+    const void* partial;
+    void* mean;     // compute-type [C]
+    void* inv_std;  // compute-type [C]
+    void* mean_out;     // T, stride in elements
+    void* inv_std_out;  // T
+    void* running_mean;
+    void* running_var;
+    int64_t mo_stride, io_stride, rm_stride, rv_stride;
+    int C, S;
+    double count;  // N * L
+    double eps, decay;
+};
+
+// STEP 0: mean from the sums.  STEP 1: variance -> inv_std, state outputs, running statistics (CX/routines/normalization.cc:176-191).
+template <typename T, int STEP>
+__global__ __launch_bounds__(256) void BnFinishKernel(BnFinishArgs p) {
+    using C = compute_t<T>;
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= p.C) return;
+    const C* part = static_cast<const C*>(p.partial) + static_cast<int64_t>(c) * p.S * 2;
+    C sum = C(0);
+    for (int s = 0; s < p.S; ++s) sum += part[s * 2];
+    const C n = static_cast<C>(p.count);
+    if (STEP == 0) {
+        static_cast<C*>(p.mean)[c] = sum / n;
+        return;
+    }
+    const C mean = static_cast<const C*>(p.mean)[c];
+    const C var = sum / n;
+    C inv_std;
+    if constexpr (std::is_same<C, float>::value) {
+        inv_std = 1.0f / sqrtf(var + static_cast<float>(p.eps));
+    } else {
+        inv_std = 1.0 / sqrt(var + p.eps);
+    }
+    static_cast<C*>(p.inv_std)[c] = inv_std;
+    static_cast<T*>(p.mean_out)[c * p.mo_stride] = static_cast<T>(mean);
+    static_cast<T*>(p.inv_std_out)[c * p.io_stride] = static_cast<T>(inv_std);
+    const C decay = static_cast<C>(p.decay);
+    const C inv_decay = static_cast<C>(1.0 - p.decay);
+    const C adjust = static_cast<C>(p.count / (p.count - 1.0 > 1.0 ? p.count - 1.0 : 1.0));
+    T* rm = static_cast<T*>(p.running_mean) + c * p.rm_stride;
+    T* rv = static_cast<T*>(p.running_var) + c * p.rv_stride;
+    *rm = static_cast<T>(static_cast<C>(*rm) * decay + inv_decay * mean);
+    *rv = static_cast<T>(static_cast<C>(*rv) * decay + inv_decay * adjust * var);
+}
+
+struct BnApplyArgs {
+    const void* x;
+    const void* g;  // gradient only
+    void* out;
+    const void* mean;     // compute-type [C]
+    const void* inv_std;  // compute-type [C]
+    const void* gamma;    // T
+    const void* beta;     // T (forward only)
+    const void* partial;  // gradient: [C][S][2]
+    void* ggamma;         // gradient outputs, T
+    void* gbeta;
+    int64_t gamma_stride, beta_stride, gg_stride, gb_stride;
+    int C, S;
+    int64_t L, total;
+    double count;
+};
+
+// Gradient finish: ggamma = sum g * x_hat, gbeta = sum g, one thread per channel; leaves both as compute-type values at partial[c][0].
+template <typename T>
+__global__ __launch_bounds__(256) void BnGradFinishKernel(BnApplyArgs p) {
+    using C = compute_t<T>;
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= p.C) return;
+    C* part = const_cast<C*>(static_cast<const C*>(p.partial)) + static_cast<int64_t>(c) * p.S * 2;
+    C sg = C(0), sgx = C(0);
+    for (int s = 0; s < p.S; ++s) {
+        sg += part[s * 2];
+        sgx += part[s * 2 + 1];
+    }
+    part[0] = sg;
+    part[1] = sgx;
+    static_cast<T*>(p.gbeta)[c * p.gb_stride] = static_cast<T>(sg);
+    static_cast<T*>(p.ggamma)[c * p.gg_stride] = static_cast<T>(sgx);
+}
+
+// GRAD false: out = ((x - mean) * inv_std) * gamma + beta.
+// GRAD true:  gx = (gamma * inv_std) * (g - (x_hat * ggamma + gbeta) / count)   (CX/routines/normalization.cc:232-246).
+template <typename T, bool GRAD, int VEC>
+__global__ __launch_bounds__(256) void BnApplyKernel(BnApplyArgs p) {
+    using C = compute_t<T>;
+    const T* x = static_cast<const T*>(p.x);
+    const T* g = static_cast<const T*>(p.g);
+    T* out = static_cast<T*>(p.out);
+    const int64_t nvec = p.total / VEC;
+    const int64_t lv = p.L / VEC;
+    const C inv_n = static_cast<C>(1.0 / p.count);
+    for (int64_t v = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; v < nvec; v += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+        const int c = static_cast<int>((v / lv) % p.C);
+        const C m = static_cast<const C*>(p.mean)[c];
+        const C is = static_cast<const C*>(p.inv_std)[c];
+        const C ga = static_cast<C>(static_cast<const T*>(p.gamma)[c * p.gamma_stride]);
+        Vec<T, VEC> xv = *reinterpret_cast<const Vec<T, VEC>*>(x + v * VEC);
+        Vec<T, VEC> o;
+        if constexpr (GRAD) {
+            const C* part = static_cast<const C*>(p.partial) + static_cast<int64_t>(c) * p.S * 2;
+            const C gbeta = part[0], ggamma = part[1];
+            Vec<T, VEC> gv = *reinterpret_cast<const Vec<T, VEC>*>(g + v * VEC);
+            const C scale = ga * is;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                C x_hat = (static_cast<C>(xv.v[e]) - m) * is;
+                o.v[e] = static_cast<T>(scale * (static_cast<C>(gv.v[e]) - (x_hat * ggamma + gbeta) * inv_n));
+            }
+        } else {
+            const C be = static_cast<C>(static_cast<const T*>(p.beta)[c * p.beta_stride]);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) o.v[e] = static_cast<T>(((static_cast<C>(xv.v[e]) - m) * is) * ga + be);
+        }
+        *reinterpret_cast<Vec<T, VEC>*>(out + v * VEC) = o;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------------------------
+struct BnTrainGeom {
+    int N = 0, C = 0, S = 1;
+    int64_t L = 1;
+    size_t csize = 4;  // bytes of the compute type
+};
+
+// x must be dense C-order with ndim >= 2 and the reduction must run over every axis but 1.
+BnTrainGeom MakeGeom(const hipcx_array* x, const int8_t* axis, int naxis) {
+    ValidateArray(x, "x");
+    HIPCX_REQUIRE(IsFloatDtype(x->dtype), HIPCX_DTYPE_ERROR, "BatchNorm only supports floating kind inputs.");
+    HIPCX_REQUIRE(x->ndim >= 2 && IsContiguous(x), HIPCX_NOT_IMPLEMENTED_ERROR, "hip batch_norm: x must be C-contiguous with at least 2 axes");
+    HIPCX_REQUIRE(naxis == x->ndim - 1, HIPCX_NOT_IMPLEMENTED_ERROR, "hip batch_norm: the statistics must run over every axis but axis 1");
+    for (int i = 0; i < naxis; ++i) {
+        int want = i == 0 ? 0 : i + 1;
+        HIPCX_REQUIRE(axis[i] == want, HIPCX_NOT_IMPLEMENTED_ERROR, "hip batch_norm: the statistics must run over every axis but axis 1");
+    }
+    BnTrainGeom g;
+    HIPCX_REQUIRE(x->shape[0] < (1LL << 31) && x->shape[1] < (1LL << 16) * 32, HIPCX_NOT_IMPLEMENTED_ERROR, "hip batch_norm: extent too large");
+    g.N = static_cast<int>(x->shape[0]);
+    g.C = static_cast<int>(x->shape[1]);
+    for (int d = 2; d < x->ndim; ++d) g.L *= x->shape[d];
+    g.csize = x->dtype == HIPCX_FLOAT64 ? 8 : 4;
+    int want = (4 * NumCUs() + g.C - 1) / (g.C > 0 ? g.C : 1);
+    g.S = want < 1 ? 1 : (want > g.N ? (g.N > 0 ? g.N : 1) : want);
+    if (g.S > 65535) g.S = 65535;
+    return g;
+}
+
+size_t TrainWorkspace(const BnTrainGeom& g) {
+    // mean [C], inv_std [C], partials [C][S][2]
+    return RoundUpTo(static_cast<size_t>(g.C) * g.csize, 16) * 2 + static_cast<size_t>(g.C) * g.S * 2 * g.csize;
+}
+
+// A per-channel vector: shape [C] or the keep-dims shape of x; returns its element stride along the channel axis.
+int64_t ChannelStride(const hipcx_array* a, const hipcx_array* x, const char* name) {
+    ValidateArray(a, name);
+    HIPCX_REQUIRE(a->dtype == x->dtype, HIPCX_NOT_IMPLEMENTED_ERROR, std::string(name) + ": must have x's dtype on the hip backend");
+    const int64_t it = ItemSize(a->dtype);
+    if (a->ndim == 1) {
+        HIPCX_REQUIRE(a->shape[0] == x->shape[1], HIPCX_DIMENSION_ERROR, std::string(name) + " must have one value per channel");
+        return a->strides[0] / it;
+    }
+    HIPCX_REQUIRE(a->ndim == x->ndim, HIPCX_DIMENSION_ERROR, std::string(name) + " must have the keep-dims reduced shape of x");
+    for (int d = 0; d < x->ndim; ++d) {
+        HIPCX_REQUIRE(a->shape[d] == (d == 1 ? x->shape[1] : 1), HIPCX_DIMENSION_ERROR, std::string(name) + " must have the keep-dims reduced shape of x");
+    }
+    return a->strides[1] / it;
+}
+
+template <typename T, int MODE>
+void LaunchStat(const BnStatArgs& a, bool vec, hipStream_t stream) {
+    constexpr int VEC = 16 / sizeof(T);
+    dim3 grid(static_cast<unsigned>(a.C), static_cast<unsigned>(a.S));
+    if (vec) {
+        hipLaunchKernelGGL((BnStatKernel<T, MODE, VEC>), grid, dim3(kBnTrainThreads), 0, stream, a);
+    } else {
+        hipLaunchKernelGGL((BnStatKernel<T, MODE, 1>), grid, dim3(kBnTrainThreads), 0, stream, a);
+    }
+    CheckLaunch("batch_norm statistics");
+}
+
+template <typename T, bool GRAD>
+void LaunchApply(const BnApplyArgs& a, bool vec, hipStream_t stream) {
+    constexpr int VEC = 16 / sizeof(T);
+    int64_t nvec = a.total / (vec ? VEC : 1);
+    int64_t blocks = (nvec + 255) / 256;
+    int64_t cap = static_cast<int64_t>(NumCUs()) * 32;
+    if (blocks > cap) blocks = cap;
+    if (blocks < 1) blocks = 1;
+    if (vec) {
+        hipLaunchKernelGGL((BnApplyKernel<T, GRAD, VEC>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, a);
+    } else {
+        hipLaunchKernelGGL((BnApplyKernel<T, GRAD, 1>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, a);
+    }
+    CheckLaunch("batch_norm apply");
+}
+
+void CheckWorkspace(void* workspace, size_t workspace_bytes, size_t need) {
+    HIPCX_REQUIRE(workspace != nullptr && workspace_bytes >= need, HIPCX_CHAINERX_ERROR,
+                  "batch_norm workspace too small: need " + std::to_string(need) + " bytes");
+    HIPCX_REQUIRE(reinterpret_cast<uintptr_t>(workspace) % 16 == 0, HIPCX_CHAINERX_ERROR, "workspace must be 16-byte aligned");
+}
+
+}  // namespace
+}  // namespace hipcx
+
+using namespace hipcx;
+
+extern "C" {
+
+size_t hipcx_batch_norm_workspace_size(const hipcx_array* x, const int8_t* axis, int naxis) {
+    try {
+        if (x == nullptr) return 0;
+        return TrainWorkspace(MakeGeom(x, axis, naxis));
+    } catch (...) {
+        return 0;
+    }
+}
+
+int hipcx_batch_norm(const hipcx_array* x, const hipcx_array* gamma, const hipcx_array* beta, const hipcx_array* running_mean,
+                     const hipcx_array* running_var, hipcx_scalar eps, hipcx_scalar decay, const int8_t* axis, int naxis,
+                     const hipcx_array* out, const hipcx_array* mean_out, const hipcx_array* inv_std_out, void* workspace,
+                     size_t workspace_bytes, void* stream) {
+    return Guard([&] {
+        BnTrainGeom g = MakeGeom(x, axis, naxis);
+        ValidateArray(out, "out");
+        HIPCX_REQUIRE(out->dtype == x->dtype && SameShape(x, out) && IsContiguous(out), HIPCX_NOT_IMPLEMENTED_ERROR,
+                      "hip batch_norm: out must be C-contiguous with x's shape and dtype");
+        BnFinishArgs f{};
+        BnApplyArgs a{};
+        a.gamma_stride = ChannelStride(gamma, x, "gamma");
+        a.beta_stride = ChannelStride(beta, x, "beta");
+        f.rm_stride = ChannelStride(running_mean, x, "running_mean");
+        f.rv_stride = ChannelStride(running_var, x, "running_var");
+        f.mo_stride = ChannelStride(mean_out, x, "mean_out");
+        f.io_stride = ChannelStride(inv_std_out, x, "inv_std_out");
+        const int64_t total = static_cast<int64_t>(g.N) * g.C * g.L;
+        if (total == 0) return;
+        CheckWorkspace(workspace, workspace_bytes, TrainWorkspace(g));
+        char* ws = static_cast<char*>(workspace);
+        const size_t vec_bytes = RoundUpTo(static_cast<size_t>(g.C) * g.csize, 16);
+        void* mean_c = ws;
+        void* inv_c = ws + vec_bytes;
+        void* partial = ws + 2 * vec_bytes;
+        hipStream_t st = AsStream(stream);
+        const bool vec = (g.L * ItemSize(x->dtype)) % 16 == 0 && reinterpret_cast<uintptr_t>(x->data) % 16 == 0 &&
+                         reinterpret_cast<uintptr_t>(out->data) % 16 == 0;
+        BnStatArgs s{};
+        s.x = x->data;
+        s.mean = mean_c;
+        s.inv_std = inv_c;
+        s.partial = partial;
+        s.N = g.N, s.C = g.C, s.L = g.L, s.S = g.S;
+        f.partial = partial;
+        f.mean = mean_c;
+        f.inv_std = inv_c;
+        f.mean_out = mean_out->data;
+        f.inv_std_out = inv_std_out->data;
+        f.running_mean = running_mean->data;
+        f.running_var = running_var->data;
+        f.C = g.C, f.S = g.S;
+        f.count = static_cast<double>(g.N) * static_cast<double>(g.L);
+        f.eps = ScalarTo<double>(eps);
+        f.decay = ScalarTo<double>(decay);
+        a.x = x->data;
+        a.out = out->data;
+        a.mean = mean_c;
+        a.inv_std = inv_c;
+        a.gamma = gamma->data;
+        a.beta = beta->data;
+        a.C = g.C, a.S = g.S, a.L = g.L, a.total = total;
+        a.count = f.count;
+        const unsigned cblocks = static_cast<unsigned>((g.C + 255) / 256);
+        VisitFloatDtype(x->dtype, [&](auto tag) {
+            using T = typename decltype(tag)::type;
+            LaunchStat<T, 0>(s, vec, st);
+            hipLaunchKernelGGL((BnFinishKernel<T, 0>), dim3(cblocks), dim3(256), 0, st, f);
+            LaunchStat<T, 1>(s, vec, st);
+            hipLaunchKernelGGL((BnFinishKernel<T, 1>), dim3(cblocks), dim3(256), 0, st, f);
+            CheckLaunch("batch_norm finish");
+            LaunchApply<T, false>(a, vec, st);
+        });
+    });
+}
+
+int hipcx_batch_norm_grad(const hipcx_array* x, const hipcx_array* gamma, const hipcx_array* gout, const hipcx_array* mean,
+                          const hipcx_array* inv_std, const int8_t* axis, int naxis, const hipcx_array* gx, const hipcx_array* ggamma,
+                          const hipcx_array* gbeta, void* workspace, size_t workspace_bytes, void* stream) {
+    return Guard([&] {
+        BnTrainGeom g = MakeGeom(x, axis, naxis);
+        ValidateArray(gout, "gout");
+        ValidateArray(gx, "gx");
+        HIPCX_REQUIRE(gout->dtype == x->dtype && SameShape(x, gout) && IsContiguous(gout), HIPCX_NOT_IMPLEMENTED_ERROR,
+                      "hip batch_norm_grad: gout must be C-contiguous with x's shape and dtype");
+        HIPCX_REQUIRE(gx->dtype == x->dtype && SameShape(x, gx) && IsContiguous(gx), HIPCX_NOT_IMPLEMENTED_ERROR,
+                      "hip batch_norm_grad: gx must be C-contiguous with x's shape and dtype");
+        BnApplyArgs a{};
+        a.gamma_stride = ChannelStride(gamma, x, "gamma");
+        a.gg_stride = ChannelStride(ggamma, x, "ggamma");
+        a.gb_stride = ChannelStride(gbeta, x, "gbeta");
+        const int64_t mean_stride = ChannelStride(mean, x, "mean");
+        const int64_t inv_stride = ChannelStride(inv_std, x, "inv_std");
+        const int64_t total = static_cast<int64_t>(g.N) * g.C * g.L;
+        if (total == 0) return;
+        CheckWorkspace(workspace, workspace_bytes, TrainWorkspace(g));
+        char* ws = static_cast<char*>(workspace);
+        const size_t vec_bytes = RoundUpTo(static_cast<size_t>(g.C) * g.csize, 16);
+        void* mean_c = ws;
+        void* inv_c = ws + vec_bytes;
+        void* partial = ws + 2 * vec_bytes;
+        hipStream_t st = AsStream(stream);
+        const bool vec = (g.L * ItemSize(x->dtype)) % 16 == 0 && reinterpret_cast<uintptr_t>(x->data) % 16 == 0 &&
+                         reinterpret_cast<uintptr_t>(gout->data) % 16 == 0 && reinterpret_cast<uintptr_t>(gx->data) % 16 == 0;
+        // the state arrives in the array dtype: widen it into the workspace vectors the kernels read
+        hipcx_array mc{}, ic{};
+        const int cdtype = x->dtype == HIPCX_FLOAT64 ? HIPCX_FLOAT64 : HIPCX_FLOAT32;
+        mc.data = mean_c, mc.dtype = cdtype, mc.ndim = 1, mc.shape[0] = g.C, mc.strides[0] = static_cast<int64_t>(g.csize);
+        ic = mc;
+        ic.data = inv_c;
+        hipcx_array m1{}, i1{};
+        m1.data = mean->data, m1.dtype = mean->dtype, m1.ndim = 1, m1.shape[0] = g.C, m1.strides[0] = mean_stride * ItemSize(mean->dtype);
+        i1.data = inv_std->data, i1.dtype = inv_std->dtype, i1.ndim = 1, i1.shape[0] = g.C, i1.strides[0] = inv_stride * ItemSize(inv_std->dtype);
+        int rc = hipcx_copy(&m1, &mc, stream);
+        if (rc == HIPCX_OK) rc = hipcx_copy(&i1, &ic, stream);
+        HIPCX_REQUIRE(rc == HIPCX_OK, HIPCX_CHAINERX_ERROR, std::string("batch_norm_grad: widening the state failed: ") + hipcx_last_error());
+        BnStatArgs s{};
+        s.x = x->data;
+        s.g = gout->data;
+        s.mean = mean_c;
+        s.inv_std = inv_c;
+        s.partial = partial;
+        s.N = g.N, s.C = g.C, s.L = g.L, s.S = g.S;
+        a.x = x->data;
+        a.g = gout->data;
+        a.out = gx->data;
+        a.mean = mean_c;
+        a.inv_std = inv_c;
+        a.gamma = gamma->data;
+        a.partial = partial;
+        a.ggamma = ggamma->data;
+        a.gbeta = gbeta->data;
+        a.C = g.C, a.S = g.S, a.L = g.L, a.total = total;
+        a.count = static_cast<double>(g.N) * static_cast<double>(g.L);
+        const unsigned cblocks = static_cast<unsigned>((g.C + 255) / 256);
+        VisitFloatDtype(x->dtype, [&](auto tag) {
+            using T = typename decltype(tag)::type;
+            LaunchStat<T, 2>(s, vec, st);
+            hipLaunchKernelGGL((BnGradFinishKernel<T>), dim3(cblocks), dim3(256), 0, st, a);
+            CheckLaunch("batch_norm_grad finish");
+            LaunchApply<T, true>(a, vec, st);
+        });
+    });
+}
+
+}  // extern "C"

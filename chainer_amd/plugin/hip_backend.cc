@@ -927,10 +927,79 @@ public:
 };
 HIPCX_REGISTER_KERNEL(ConvTransposeKernel, HipConvTransposeKernel)
 
-// Batch normalisation in training mode and its gradient are routine compositions in the reference
-// (CX/routines/normalization.cc:155-250); registering the generic kernels runs them on this backend's kernels.
-HIPCX_REGISTER_KERNEL(BatchNormKernel, GenericBatchNormKernel)
-HIPCX_REGISTER_KERNEL(BatchNormGradKernel, GenericBatchNormGradKernel)
+// Batch normalisation in training mode and its gradient.  The reference's generic kernels are routine compositions
+// (CX/routines/normalization.cc:155-250); they run on this backend's kernels as they are and remain the path for everything the
+// dedicated kernels do not take (a non-contiguous x, mixed dtypes, other axis sets).  The state handed to the gradient is the
+// generic one (batch mean, 1 / sqrt(var + eps), dtype of beta), so either gradient kernel can consume either forward's state.
+namespace {
+bool HipBatchNormApplies(const Array& x, const Axes& axis, std::initializer_list<const Array*> others) {
+    if (x.ndim() < 2 || !x.IsContiguous() || x.GetTotalSize() == 0) return false;
+    if (static_cast<int8_t>(axis.size()) != x.ndim() - 1) return false;
+    for (int8_t i = 0; i < static_cast<int8_t>(axis.size()); ++i) {
+        if (axis[i] != (i == 0 ? 0 : i + 1)) return false;
+    }
+    for (const Array* a : others) {
+        if (a->dtype() != x.dtype()) return false;
+    }
+    return true;
+}
+}  // namespace
+
+class HipBatchNormKernel : public GenericBatchNormKernel {
+public:
+    std::tuple<Array, std::unique_ptr<BatchNormGradState>> Call(const Array& x, const Array& gamma, const Array& beta, const Array& running_mean,
+                                                               const Array& running_var, Scalar eps, Scalar decay, const Axes& axis,
+                                                               bool return_state, const absl::optional<Array>& out) override {
+        if (out.has_value() || !HipBatchNormApplies(x, axis, {&gamma, &beta, &running_mean, &running_var})) {
+            return GenericBatchNormKernel::Call(x, gamma, beta, running_mean, running_var, eps, decay, axis, return_state, out);
+        }
+        Device& device = x.device();
+        device.CheckDevicesCompatible(x, gamma, beta, running_mean, running_var);
+        SetDeviceScope scope{device.index()};
+        Array y = Empty(x.shape(), x.dtype(), device);
+        Array x_mean = Empty(gamma.shape(), x.dtype(), device);
+        Array x_inv_std = Empty(gamma.shape(), x.dtype(), device);
+        hipcx_array cx = ToC(x), cg = ToC(gamma), cb = ToC(beta), crm = ToC(running_mean), crv = ToC(running_var), cy = ToC(y),
+                    cm = ToC(x_mean), ci = ToC(x_inv_std);
+        std::vector<int8_t> ax = ToC(axis);
+        size_t ws_bytes = hipcx_batch_norm_workspace_size(&cx, ax.data(), static_cast<int>(ax.size()));
+        std::shared_ptr<void> ws = device.Allocate(ws_bytes);
+        Check(hipcx_batch_norm(&cx, &cg, &cb, &crm, &crv, ToC(eps), ToC(decay), ax.data(), static_cast<int>(ax.size()), &cy, &cm, &ci,
+                               ws.get(), ws_bytes, nullptr));
+        std::unique_ptr<BatchNormGradState> state =
+                return_state ? std::make_unique<GenericBatchNormGradState>(std::move(x_mean), std::move(x_inv_std), beta.dtype()) : nullptr;
+        return std::make_tuple(std::move(y), std::move(state));
+    }
+};
+HIPCX_REGISTER_KERNEL(BatchNormKernel, HipBatchNormKernel)
+
+class HipBatchNormGradKernel : public GenericBatchNormGradKernel {
+public:
+    std::tuple<Array, Array, Array> Call(const Array& x, const Array& gamma, const Array& gout, Scalar eps, const Axes& axis,
+                                         const std::shared_ptr<BatchNormGradState>& state, const absl::optional<Array>& gx,
+                                         const absl::optional<Array>& ggamma, const absl::optional<Array>& gbeta) override {
+        auto* st = dynamic_cast<GenericBatchNormGradState*>(state.get());
+        if (st == nullptr || gx.has_value() || ggamma.has_value() || gbeta.has_value() || !gout.IsContiguous() ||
+            st->beta_dtype() != x.dtype() || !HipBatchNormApplies(x, axis, {&gamma, &gout, &st->x_mean(), &st->x_inv_std()})) {
+            return GenericBatchNormGradKernel::Call(x, gamma, gout, eps, axis, state, gx, ggamma, gbeta);
+        }
+        Device& device = x.device();
+        device.CheckDevicesCompatible(x, gamma, gout);
+        SetDeviceScope scope{device.index()};
+        Array actual_gx = Empty(x.shape(), x.dtype(), device);
+        Array actual_ggamma = Empty(gamma.shape(), x.dtype(), device);
+        Array actual_gbeta = Empty(gamma.shape(), x.dtype(), device);
+        hipcx_array cx = ToC(x), cg = ToC(gamma), cgo = ToC(gout), cm = ToC(st->x_mean()), ci = ToC(st->x_inv_std()), cgx = ToC(actual_gx),
+                    cgg = ToC(actual_ggamma), cgb = ToC(actual_gbeta);
+        std::vector<int8_t> ax = ToC(axis);
+        size_t ws_bytes = hipcx_batch_norm_workspace_size(&cx, ax.data(), static_cast<int>(ax.size()));
+        std::shared_ptr<void> ws = device.Allocate(ws_bytes);
+        Check(hipcx_batch_norm_grad(&cx, &cg, &cgo, &cm, &ci, ax.data(), static_cast<int>(ax.size()), &cgx, &cgg, &cgb, ws.get(), ws_bytes,
+                                    nullptr));
+        return std::make_tuple(std::move(actual_gx), std::move(actual_ggamma), std::move(actual_gbeta));
+    }
+};
+HIPCX_REGISTER_KERNEL(BatchNormGradKernel, HipBatchNormGradKernel)
 
 class HipMaxPoolGradKernel : public MaxPoolGradKernel {
 public:

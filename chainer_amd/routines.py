@@ -1365,6 +1365,16 @@ def var(a, axis=None, keepdims=False):
     return mean(multiply(diff, diff), axes, keepdims)
 
 
+# True: BatchNorm (training) and its gradient run as the reference's routine compositions instead of the dedicated kernels.
+COMPOSE_BATCH_NORM = False
+
+
+def _bn_kernel_applies(x, axes, others):
+    """The dedicated kernels take a C-contiguous x reduced over every axis but 1, with every other array in x's dtype."""
+    return (not COMPOSE_BATCH_NORM and x.ndim >= 2 and tuple(axes) == (0,) + tuple(range(2, x.ndim)) and x.is_contiguous
+            and _py.all(a.dtype == x.dtype for a in others))
+
+
 def batch_norm(x, gamma, beta, running_mean, running_var, eps=2e-5, decay=0.9, axis=None):
     """BatchNorm in training mode through GenericBatchNormKernel (CX/routines/normalization.cc:155-193): batch Mean / Var in the
     promoted dtype, ApplyGenericBatchNorm, then the running statistics are updated in place (the variance with the n/(n-1)
@@ -1374,6 +1384,18 @@ def batch_norm(x, gamma, beta, running_mean, running_var, eps=2e-5, decay=0.9, a
     axes = _sorted_axes((0,) + tuple(range(2, x.ndim)) if axis is None else axis, x.ndim)
     red_shape = tuple(1 if i in axes else d for i, d in enumerate(x.shape))
     interm = result_type(x, gamma, beta)
+    if _bn_kernel_applies(x, axes, (gamma, beta, running_mean, running_var)) and x.size > 0:
+        # the dedicated kernels: two statistics passes, a per-channel finish, one normalising pass
+        out = ndarray.empty(x.shape, x.dtype)
+        x_mean = ndarray.empty(red_shape, x.dtype)
+        inv_std = ndarray.empty(red_shape, x.dtype)
+        ax = (ctypes.c_int8 * len(axes))(*axes)
+        nbytes = _lib.load().hipcx_batch_norm_workspace_size(x.desc(), ax, len(axes))
+        ws, wsp = _workspace(nbytes)
+        _lib.call('hipcx_batch_norm', x.desc(), gamma.reshape(red_shape).desc(), beta.reshape(red_shape).desc(),
+                  running_mean.reshape(red_shape).desc(), running_var.reshape(red_shape).desc(), _lib.make_scalar(float(eps)),
+                  _lib.make_scalar(float(decay)), ax, len(axes), out.desc(), x_mean.desc(), inv_std.desc(), wsp, nbytes, current_stream())
+        return out, (x_mean, inv_std, beta.dtype)
     xc = x.astype(interm, False)
     x_mean = mean(xc, axes, True)
     x_var = var(xc, axes, True)
@@ -1396,6 +1418,18 @@ def batch_norm_grad(x, gamma, gout, state, axis=None):
     axes = _sorted_axes((0,) + tuple(range(2, x.ndim)) if axis is None else axis, x.ndim)
     red_shape = tuple(1 if i in axes else d for i, d in enumerate(x.shape))
     interm = x_mean.dtype
+    if (_bn_kernel_applies(x, axes, (gamma, gout, x_mean, x_inv_std)) and gout.shape == x.shape and gout.is_contiguous
+            and numpy.dtype(beta_dtype) == x.dtype and x.size > 0):
+        gx = ndarray.empty(x.shape, x.dtype)
+        ggamma = ndarray.empty(gamma.shape, x.dtype)
+        gbeta = ndarray.empty(gamma.shape, x.dtype)
+        ax = (ctypes.c_int8 * len(axes))(*axes)
+        nbytes = _lib.load().hipcx_batch_norm_workspace_size(x.desc(), ax, len(axes))
+        ws, wsp = _workspace(nbytes)
+        _lib.call('hipcx_batch_norm_grad', x.desc(), gamma.reshape(red_shape).desc(), gout.desc(), x_mean.reshape(red_shape).desc(),
+                  x_inv_std.reshape(red_shape).desc(), ax, len(axes), gx.desc(), ggamma.reshape(red_shape).desc(),
+                  gbeta.reshape(red_shape).desc(), wsp, nbytes, current_stream())
+        return gx, ggamma, gbeta
     n = _prod(x.shape) // _py.max(1, _prod(gamma.shape))
     inv_n = 1.0 / n
     gc = gout.astype(interm, False)

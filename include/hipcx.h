@@ -272,6 +272,21 @@ int hipcx_fixed_batch_norm(const hipcx_array* x, const hipcx_array* gamma, const
                            const hipcx_array* var, hipcx_scalar eps, const int8_t* axis, int naxis, const hipcx_array* out,
                            void* stream);
 
+/* ---- training-mode normalization: BatchNormKernel CX/kernels/normalization.h:32-47, BatchNormGradKernel :49-61 ----
+ * For x C-contiguous with ndim >= 2 and `axis` = every axis but 1 (anything else: HIPCX_NOT_IMPLEMENTED_ERROR, and the caller
+ * runs the reference's routine composition, CX/routines/normalization.cc:155-250).  gamma / beta / running_* / mean_out /
+ * inv_std_out / ggamma / gbeta hold one value per channel, shaped [C] or as the keep-dims reduction of x, in x's dtype.
+ * hipcx_batch_norm writes out, the batch mean and 1 / sqrt(var + eps) (the state the gradient needs) and updates running_mean /
+ * running_var in place (decay, and n / max(n - 1, 1) on the variance).  Both need hipcx_batch_norm_workspace_size bytes. */
+size_t hipcx_batch_norm_workspace_size(const hipcx_array* x, const int8_t* axis, int naxis);
+int hipcx_batch_norm(const hipcx_array* x, const hipcx_array* gamma, const hipcx_array* beta, const hipcx_array* running_mean,
+                     const hipcx_array* running_var, hipcx_scalar eps, hipcx_scalar decay, const int8_t* axis, int naxis,
+                     const hipcx_array* out, const hipcx_array* mean_out, const hipcx_array* inv_std_out, void* workspace,
+                     size_t workspace_bytes, void* stream);
+int hipcx_batch_norm_grad(const hipcx_array* x, const hipcx_array* gamma, const hipcx_array* gout, const hipcx_array* mean,
+                          const hipcx_array* inv_std, const int8_t* axis, int naxis, const hipcx_array* gx, const hipcx_array* ggamma,
+                          const hipcx_array* gbeta, void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---- pooling: CX/kernels/pooling.h:29,83 (2-D, NCHW logical layout, any strides) ---- */
 int hipcx_max_pool(const hipcx_array* x, const int64_t* kernel_size, const int64_t* stride, const int64_t* pad, int cover_all,
                    const hipcx_array* out, void* stream);

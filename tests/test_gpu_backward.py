@@ -187,3 +187,63 @@ def test_pool_gradient_kernels_have_the_bits_of_the_composition(dt):
                 assert_exact(got, ref, 'average_pool_grad %s %s %r' % (dt, mode, (shape, k, s, p)))
     with pytest.raises(chx.DimensionError):
         chx.max_pool_grad(chx.zeros((1, 1, 4, 4), dt), chx.zeros((1, 1, 3, 3), dt), 2, 2, 0)
+
+
+@pytest.mark.parametrize('dt,tol', [('float32', 1e-5), ('float16', 2e-2), ('float64', 1e-12)])
+def test_batch_norm_kernels_against_the_composition(dt, tol):
+    """hipcx_batch_norm / hipcx_batch_norm_grad against the reference's routine composition on the device and against the oracle:
+    plane sizes that are and are not whole 16-byte vectors, one image, one channel, 2-D input, a large-mean input (the two-pass
+    variance must not cancel), running statistics updated in place; a non-contiguous x takes the composition."""
+    import chainer_amd as chx
+    from chainer_amd import routines
+    rng = np.random.default_rng(71)
+    shapes = [(8, 16, 14, 14), (4, 3, 7, 7), (1, 5, 6, 4), (6, 1, 3, 3), (32, 10), (2, 4, 3, 5, 2)]
+    if dt != 'float16':
+        # 50176 elements per channel: the float16 composition (like the native backend) overflows its Sum of squares there and
+        # returns inf statistics, while the kernel accumulates in float -- a case where the two differ on purpose
+        shapes.append((64, 32, 28, 28))
+    for shape in shapes:
+        C = shape[1]
+        x = (rng.standard_normal(shape) * 2 + (5 if shape == (4, 3, 7, 7) else 0)).astype(dt)
+        gamma = rng.uniform(0.5, 1.5, C).astype(dt)
+        beta = rng.standard_normal(C).astype(dt)
+        rm0, rv0 = rng.standard_normal(C).astype(dt), rng.uniform(0.5, 1.5, C).astype(dt)
+        gout = rng.standard_normal(shape).astype(dt)
+        res = {}
+        for mode in ('kernel', 'composition'):
+            routines.COMPOSE_BATCH_NORM = mode == 'composition'
+            try:
+                RM, RV = chx.array(rm0), chx.array(rv0)
+                out, state = chx.batch_norm(chx.array(x), chx.array(gamma), chx.array(beta), RM, RV, 2e-5, 0.9)
+                gx, gg, gb = chx.batch_norm_grad(chx.array(x), chx.array(gamma), chx.array(gout), state)
+                res[mode] = [out.get(), RM.get(), RV.get(), state[0].get(), state[1].get(), gx.get(), gg.get(), gb.get()]
+            finally:
+                routines.COMPOSE_BATCH_NORM = False
+        names = ['out', 'running_mean', 'running_var', 'mean', 'inv_std']
+        for name, a, b in zip(names, res['kernel'], res['composition']):
+            assert_close(a, b, tol, 'batch_norm %s %s %r kernel vs composition' % (name, dt, shape))
+        # gradients against the closed form in float64; the sums cancel, so errors are measured against the size of their terms
+        red = (0,) + tuple(range(2, x.ndim))
+        bshape = (1, C) + (1,) * (x.ndim - 2)
+        x64, g64 = x.astype(np.float64), gout.astype(np.float64)
+        m64 = x64.mean(red, keepdims=True)
+        is64 = 1.0 / np.sqrt(x64.var(red, keepdims=True) + 2e-5)
+        xh = (x64 - m64) * is64
+        gb64, gg64 = g64.sum(red), (g64 * xh).sum(red)
+        gx64 = gamma.astype(np.float64).reshape(bshape) * is64 * (g64 - (xh * gg64.reshape(bshape) + gb64.reshape(bshape)) / (x.size // C))
+        gx, gg, gb = res['kernel'][5:8]
+        t = 4 * tol
+        assert gx.dtype == x.dtype and gg.shape == (C,) and gb.shape == (C,)
+        assert np.all(np.abs(gb.astype(np.float64) - gb64) <= t * np.abs(g64).sum(red) + 1e-30), 'gbeta %s %r' % (dt, shape)
+        assert np.all(np.abs(gg.astype(np.float64) - gg64) <= t * np.abs(g64 * xh).sum(red) + 1e-30), 'ggamma %s %r' % (dt, shape)
+        assert np.abs(gx.astype(np.float64) - gx64).max() <= t * np.abs(gx64).max() + t * 1e-2, 'gx %s %r' % (dt, shape)
+        o_ref, rm_ref, rv_ref, st_ref = O.batch_norm(x, gamma, beta, rm0.copy(), rv0.copy(), 2e-5, 0.9)
+        assert_close(res['kernel'][0], o_ref, tol, 'batch_norm out vs oracle %s %r' % (dt, shape))
+        assert_close(res['kernel'][1], rm_ref, tol, 'running_mean vs oracle')
+        assert_close(res['kernel'][2], rv_ref, tol, 'running_var vs oracle')
+    # a channels-last view is not C-contiguous: the composition runs and agrees
+    x = rng.standard_normal((4, 8, 5, 5)).astype(dt)
+    X = channels_last(chx, x)
+    g1, b1 = np.ones(8, dt), np.zeros(8, dt)
+    out, _ = chx.batch_norm(X, chx.array(g1), chx.array(b1), chx.array(b1.copy()), chx.array(g1.copy()))
+    assert_close(out.get(), O.batch_norm(x, g1, b1, b1.copy(), g1.copy(), 2e-5, 0.9)[0], tol, 'channels-last input')
