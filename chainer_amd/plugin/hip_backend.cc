@@ -917,6 +917,14 @@ public:
         if (out.has_value()) throw NotImplementedError{"Passing out as an argument is not yet supported."};
         if (x.ndim() != 4) throw NotImplementedError{"hip convolution supports 2 spatial dimensions."};
         SetDeviceScope scope{x.device().index()};
+        const int64_t kh = w.shape()[2], kw = w.shape()[3];
+        if (stride[0] == 1 && stride[1] == 1 && pad[0] <= kh - 1 && pad[1] <= kw - 1 && GetKind(out_dtype) == DtypeKind::kFloat &&
+            out_size[0] == x.shape()[2] - 1 + kh - 2 * pad[0] && out_size[1] == x.shape()[3] - 1 + kw - 2 * pad[1]) {
+            // stride 1: a forward convolution with the filters flipped in both spatial axes, channel axes swapped, padding k - 1 - p
+            Array w_flipped = Flip(w, Axes{2, 3}).Transpose(Axes{1, 0, 2, 3}).Copy();
+            return x.device().backend().CallKernel<ConvKernel>(x, w_flipped, b, Dims{1, 1}, Dims{kh - 1 - pad[0], kw - 1 - pad[1]}, false,
+                                                               out_dtype, absl::nullopt);
+        }
         Array col = native::TensorDot(w, x, Axes{0}, Axes{1}, out_dtype);  // [C_out, kh, kw, N, H, W]
         Array actual_out = HipCol2Im(col.Transpose(Axes{3, 0, 1, 2, 4, 5}), stride, pad, out_size);
         if (b.has_value()) {

@@ -1326,6 +1326,10 @@ def conv_grad_weight(w_dtype, w_shape, x, gy, stride=1, pad=0, cover_all=False):
     return gw.reshape(tuple(w_shape))
 
 
+# True: ConvTranspose always runs as the native backend's TensorDot + Col2Im composition.
+COMPOSE_CONV_TRANSPOSE = False
+
+
 def conv_transpose(x, w, b=None, stride=1, pad=0, out_size=None, out_dtype=None):
     """ConvTranspose (CX/routines/connection.cc:214-320) over the native kernel (CX/native/native_device/conv.cc:126-160):
     col = TensorDot(w, x) over the input channels, batch axis rolled first, Col2Im, bias added in place.  w: [C_in, C_out, kh, kw]."""
@@ -1343,6 +1347,13 @@ def conv_transpose(x, w, b=None, stride=1, pad=0, out_size=None, out_dtype=None)
             if d != conv_out_dim(o, k, st, p, False) and d != conv_out_dim(o, k, st, p, True):
                 raise _lib.DimensionError('Output dims %r is incosistent.' % (out_size,))
     dt = numpy.dtype(out_dtype) if out_dtype is not None else (result_type(x, w, b) if b is not None else result_type(x, w))
+    if (not COMPOSE_CONV_TRANSPOSE and stride == (1, 1) and pad[0] <= kh - 1 and pad[1] <= kw - 1 and _kind(dt) == 3
+            and tuple(out_size) == tuple(d - 1 + k - 2 * p for d, k, p in zip(x.shape[2:], (kh, kw), pad))):
+        # At stride 1 the transposed convolution is a forward convolution with the filters flipped in both spatial axes, their
+        # channel axes swapped and the padding k - 1 - p: one MFMA convolution instead of Dot + kh*kw strided additions.  The
+        # sums run in another order than the composition's (float accumulation, one rounding), equal to tolerance.
+        w_flipped = w[:, :, ::-1, ::-1].transpose((1, 0, 2, 3)).copy()
+        return conv(x, w_flipped, b, 1, (kh - 1 - pad[0], kw - 1 - pad[1]), False, dt)
     # TensorDot(w, x) over the input channels; x goes in channels-last so that both Dot operands have the reduction index as
     # their unit-stride axis
     n, ci, h, wd = x.shape
