@@ -178,6 +178,7 @@ SIGNATURES = {
     'hipcx_max_pool_grad_workspace_size': (_SZ, [_A]),
     'hipcx_max_pool_grad': (_INT, [_A, _A, _I64P, _I64P, _I64P, _INT, _A, _V, _SZ, _V]),
     'hipcx_average_pool_grad': (_INT, [_A, _I64P, _I64P, _I64P, _INT, _A, _V]),
+    'hipcx_max_pool_grad_grad': (_INT, [_A, _A, _I64P, _I64P, _I64P, _INT, _A, _V]),
     'hipcx_take': (_INT, [_A, _A, ctypes.c_int8, _A, _INT, ctypes.POINTER(ctypes.c_int32), _V]),
 }
 

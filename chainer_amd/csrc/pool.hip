@@ -446,6 +446,31 @@ __global__ __launch_bounds__(256) void WindowArgMaxKernel(PoolGradArgs p, IdxT t
     }
 }
 
+// MaxPoolGradGrad (CX/native/native_device/pool.cc:147-177): the element of every window of ggx at the position where x has its
+// ArgMax; a position in the padding reads the lowest value, as the Im2Col of the native kernel fills it.  gout/gs* describe ggx here
+// and gx/ds* the output [N, C, OH, OW].
+template <typename T, typename IdxT>
+__global__ __launch_bounds__(256) void MaxPoolGradGradKernel(PoolGradArgs p, IdxT total) {
+    const T* x = static_cast<const T*>(p.x);
+    const T* ggx = static_cast<const T*>(p.gout);
+    T* ggout = static_cast<T*>(p.gx);
+    for (IdxT idx = static_cast<IdxT>(blockIdx.x) * blockDim.x + threadIdx.x; idx < total; idx += static_cast<IdxT>(gridDim.x) * blockDim.x) {
+        IdxT t = idx;
+        const int ow = static_cast<int>(t % p.OW);
+        t /= p.OW;
+        const int oh = static_cast<int>(t % p.OH);
+        t /= p.OH;
+        const int c = static_cast<int>(t % p.C);
+        const int64_t n = static_cast<int64_t>(t / p.C);
+        const int best = WindowArgMax<T>(p, x + n * p.xsN + static_cast<int64_t>(c) * p.xsC, oh, ow);
+        const int r = best / p.kw, q = best - r * p.kw;
+        const int ih = oh * p.sh - p.ph + r, iw = ow * p.sw - p.pw + q;
+        T v = Lowest<T>();
+        if (ih >= 0 && ih < p.H && iw >= 0 && iw < p.W) v = ggx[n * p.gsN + static_cast<int64_t>(c) * p.gsC + ih * p.gsH + iw * p.gsW];
+        ggout[n * p.dsN + static_cast<int64_t>(c) * p.dsC + oh * p.dsH + ow * p.dsW] = v;
+    }
+}
+
 template <typename T, bool IS_MAX, typename IdxT>
 __global__ __launch_bounds__(256) void PoolGradKernel(PoolGradArgs p, IdxT total) {
     using C = compute_t<T>;
@@ -644,6 +669,40 @@ int hipcx_average_pool_grad(const hipcx_array* gout, const int64_t* kernel_size,
             using T = typename decltype(tag)::type;
             RunPoolGrad<T, false>(p, AsStream(stream));
         });
+    });
+}
+
+int hipcx_max_pool_grad_grad(const hipcx_array* x, const hipcx_array* ggx, const int64_t* kernel_size, const int64_t* stride,
+                             const int64_t* pad, int cover_all, const hipcx_array* ggout, void* stream) {
+    return Guard([&] {
+        HIPCX_REQUIRE(x != nullptr && ggx != nullptr, HIPCX_CHAINERX_ERROR, "null array");
+        // the geometry helper wants (x, window-shaped array, image-shaped array): here the image-shaped one is ggx
+        PoolGradArgs p = MakeGradArgs(x, ggout, kernel_size, stride, pad, cover_all, ggx);
+        // swap roles: gout/gs* <- ggx (image), gx/ds* <- ggout (windows)
+        std::swap(p.gsN, p.dsN);
+        std::swap(p.gsC, p.dsC);
+        std::swap(p.gsH, p.dsH);
+        std::swap(p.gsW, p.dsW);
+        p.gout = ggx->data;
+        p.gx = ggout->data;
+        const int64_t windows = static_cast<int64_t>(p.N) * p.C * p.OH * p.OW;
+        if (windows == 0) return;
+        const int64_t cap = static_cast<int64_t>(NumCUs()) * 64;
+        int64_t blocks = (windows + 255) / 256;
+        if (blocks > cap) blocks = cap;
+        VisitDtype(x->dtype, [&](auto tag) {
+            using T = typename decltype(tag)::type;
+            if constexpr (std::is_same<T, bool>::value) {
+                throw Error(HIPCX_DTYPE_ERROR, "max_pool_grad_grad: bool arrays are not supported");
+            } else if (windows + cap * 256 < (1LL << 31)) {
+                hipLaunchKernelGGL((MaxPoolGradGradKernel<T, unsigned>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, AsStream(stream), p,
+                                   static_cast<unsigned>(windows));
+            } else {
+                hipLaunchKernelGGL((MaxPoolGradGradKernel<T, int64_t>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, AsStream(stream), p,
+                                   windows);
+            }
+        });
+        CheckLaunch("max_pool_grad_grad");
     });
 }
 }

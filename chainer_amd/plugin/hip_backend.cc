@@ -812,6 +812,14 @@ private:
     Array x_;
     bool cover_all_;
 };
+class HipMaxPoolGradGradState : public MaxPoolGradGradState {
+public:
+    explicit HipMaxPoolGradGradState(Array x) : x_{std::move(x)} {}
+    const Array& x() const { return x_; }
+
+private:
+    Array x_;
+};
 class HipAveragePoolGradState : public AveragePoolGradState {
 public:
     explicit HipAveragePoolGradState(Array x) : x_{std::move(x)} {}
@@ -1015,7 +1023,6 @@ public:
                                                                  const std::shared_ptr<MaxPoolGradState>& state, bool return_state,
                                                                  const absl::optional<Array>& gx) override {
         if (gx.has_value()) throw NotImplementedError{"Passing gx as an argument is not yet supported."};
-        if (return_state) throw NotImplementedError{"hip MaxPoolGradGrad is not implemented."};
         auto& st = dynamic_cast<HipMaxPoolGradState&>(*state);
         const Array& x = st.x();
         Device& device = x.device();
@@ -1029,10 +1036,31 @@ public:
         size_t ws_bytes = hipcx_max_pool_grad_workspace_size(&cg);
         std::shared_ptr<void> ws = device.Allocate(ws_bytes);
         Check(hipcx_max_pool_grad(&cx, &cg, k, s, p, st.cover_all() ? 1 : 0, &cgx, ws.get(), ws_bytes, nullptr));
-        return std::make_tuple(std::move(actual_gx), std::unique_ptr<MaxPoolGradGradState>{});
+        std::unique_ptr<MaxPoolGradGradState> grad_grad_state = return_state ? std::make_unique<HipMaxPoolGradGradState>(x) : nullptr;
+        return std::make_tuple(std::move(actual_gx), std::move(grad_grad_state));
     }
 };
 HIPCX_REGISTER_KERNEL(MaxPoolGradKernel, HipMaxPoolGradKernel)
+
+class HipMaxPoolGradGradKernel : public MaxPoolGradGradKernel {
+public:
+    Array Call(const Array& ggx, const Dims& kernel_size, const Dims& stride, const Dims& pad, bool cover_all,
+               const std::shared_ptr<MaxPoolGradGradState>& state, const absl::optional<Array>& ggout) override {
+        if (ggout.has_value()) throw NotImplementedError{"Passing ggout as an argument is not yet supported."};
+        auto& st = dynamic_cast<HipMaxPoolGradGradState&>(*state);
+        const Array& x = st.x();
+        Device& device = x.device();
+        device.CheckDevicesCompatible(x, ggx);
+        SetDeviceScope scope{device.index()};
+        Array actual_ggout = Empty(PoolOutShape(x, kernel_size, stride, pad, cover_all), x.dtype(), device);
+        const Array& g = ggx.dtype() == x.dtype() ? ggx : ggx.AsType(x.dtype());
+        hipcx_array cx = ToC(x), cg = ToC(g), co = ToC(actual_ggout);
+        int64_t k[2] = {kernel_size[0], kernel_size[1]}, s[2] = {stride[0], stride[1]}, p[2] = {pad[0], pad[1]};
+        Check(hipcx_max_pool_grad_grad(&cx, &cg, k, s, p, cover_all ? 1 : 0, &co, nullptr));
+        return actual_ggout;
+    }
+};
+HIPCX_REGISTER_KERNEL(MaxPoolGradGradKernel, HipMaxPoolGradGradKernel)
 
 class HipAveragePoolGradKernel : public AveragePoolGradKernel {
 public:

@@ -1498,6 +1498,13 @@ def max_pool_grad_grad(x, ggx, ksize, stride=None, pad=0, cover_all=False):
     ksize = _pair(ksize)
     stride = ksize if stride is None else _pair(stride)
     pad = _pair(pad)
+    if x.ndim == 4 and x.dtype != numpy.dtype('bool') and ggx.dtype == x.dtype and ggx.shape == x.shape and not COMPOSE_POOL_GRADIENTS:
+        oh = conv_out_dim(x.shape[2], ksize[0], stride[0], pad[0], cover_all)
+        ow = conv_out_dim(x.shape[3], ksize[1], stride[1], pad[1], cover_all)
+        ggout = ndarray.empty((x.shape[0], x.shape[1], oh, ow), x.dtype)
+        _lib.call('hipcx_max_pool_grad_grad', x.desc(), ggx.desc(), _i64(ksize), _i64(stride), _i64(pad), int(bool(cover_all)),
+                  ggout.desc(), current_stream())
+        return ggout
     lowest = -numpy.inf if _kind(x.dtype) == 3 else (0 if x.dtype == numpy.dtype('bool') else int(numpy.iinfo(x.dtype).min))
     indices = argmax(im2col(x, ksize, stride, pad, cover_all, lowest), (2, 3))
     kt = ksize[0] * ksize[1]

@@ -301,6 +301,10 @@ int hipcx_average_pool(const hipcx_array* x, const int64_t* kernel_size, const i
 size_t hipcx_max_pool_grad_workspace_size(const hipcx_array* gout);
 int hipcx_max_pool_grad(const hipcx_array* x, const hipcx_array* gout, const int64_t* kernel_size, const int64_t* stride,
                         const int64_t* pad, int cover_all, const hipcx_array* gx, void* workspace, size_t workspace_bytes, void* stream);
+/* MaxPoolGradGradKernel CX/kernels/pooling.h:66-76: ggout[window] = ggx at the ArgMax position of x in that window (a position in
+ * the padding gives the lowest value, as the native Im2Col fills it); ggx has x's shape, ggout the pooled shape. */
+int hipcx_max_pool_grad_grad(const hipcx_array* x, const hipcx_array* ggx, const int64_t* kernel_size, const int64_t* stride,
+                             const int64_t* pad, int cover_all, const hipcx_array* ggout, void* stream);
 int hipcx_average_pool_grad(const hipcx_array* gout, const int64_t* kernel_size, const int64_t* stride, const int64_t* pad, int pad_mode,
                             const hipcx_array* gx, void* stream);
 

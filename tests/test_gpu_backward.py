@@ -179,6 +179,15 @@ def test_pool_gradient_kernels_have_the_bits_of_the_composition(dt):
             finally:
                 routines.COMPOSE_POOL_GRADIENTS = False
             assert_exact(got, ref, 'max_pool_grad %s %s %r' % (dt, lay, (shape, k, s, p, cv)))
+            ggx = rng.standard_normal(shape).astype(dt) if np.dtype(dt).kind == 'f' else rng.integers(-50, 50, shape).astype(dt)
+            GGX = chx.array(ggx) if lay == 'nchw' else channels_last(chx, ggx)
+            got = chx.max_pool_grad_grad(X, GGX, k, s, p, cv).get()
+            routines.COMPOSE_POOL_GRADIENTS = True
+            try:
+                ref = chx.max_pool_grad_grad(X, GGX, k, s, p, cv).get()
+            finally:
+                routines.COMPOSE_POOL_GRADIENTS = False
+            assert_exact(got, ref, 'max_pool_grad_grad %s %s %r' % (dt, lay, (shape, k, s, p, cv)))
         if np.dtype(dt).kind == 'f' and not cv:
             for mode in ('zero', 'ignore'):
                 got = chx.average_pool_grad(chx.array(x), chx.array(g), k, s, p, mode).get()
