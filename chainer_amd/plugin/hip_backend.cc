@@ -1084,6 +1084,70 @@ public:
 };
 HIPCX_REGISTER_KERNEL(AveragePoolGradKernel, HipAveragePoolGradKernel)
 
+// ---- linear algebra: Solve, Inverse, Cholesky (the LAPACK-backed kernels of the native backend, native_device/linalg.cc) ----
+namespace {
+// A zeroed device int32 for LAPACK's `info`, and the check that turns a non-zero value into the reference's ChainerxError.
+std::shared_ptr<void> NewInfoFlag(Device& device) {
+    std::shared_ptr<void> flag = device.Allocate(sizeof(int32_t));
+    CheckHip(hipMemsetAsync(flag.get(), 0, sizeof(int32_t), nullptr), "hipMemsetAsync");
+    return flag;
+}
+void ThrowIfInfo(const std::shared_ptr<void>& flag, const char* what) {
+    int32_t host = 0;
+    CheckHip(hipMemcpy(&host, flag.get(), sizeof(int32_t), hipMemcpyDeviceToHost), "hipMemcpy");
+    if (host != 0) throw ChainerxError{"Unsuccessful ", what, " execution. Info = ", host};
+}
+}  // namespace
+
+class HipSolveKernel : public SolveKernel {
+public:
+    void Call(const Array& a, const Array& b, const Array& out) override {
+        Device& device = a.device();
+        device.CheckDevicesCompatible(a, b, out);
+        SetDeviceScope scope{device.index()};
+        if (out.dtype() == Dtype::kFloat16) throw DtypeError{"Half-precision (float16) is not supported by solve"};
+        hipcx_array ca = ToC(a), cb = ToC(b), co = ToC(out);
+        size_t ws_bytes = hipcx_solve_workspace_size(&ca);
+        std::shared_ptr<void> ws = device.Allocate(ws_bytes);
+        std::shared_ptr<void> flag = NewInfoFlag(device);
+        Check(hipcx_solve(&ca, &cb, &co, ws.get(), ws_bytes, static_cast<int32_t*>(flag.get()), nullptr));
+        ThrowIfInfo(flag, "gesv (Solve)");
+    }
+};
+HIPCX_REGISTER_KERNEL(SolveKernel, HipSolveKernel)
+
+class HipInverseKernel : public InverseKernel {
+public:
+    void Call(const Array& a, const Array& out) override {
+        Device& device = a.device();
+        device.CheckDevicesCompatible(a, out);
+        SetDeviceScope scope{device.index()};
+        if (out.dtype() == Dtype::kFloat16) throw DtypeError{"Half-precision (float16) is not supported by inverse"};
+        hipcx_array ca = ToC(a), co = ToC(out);
+        size_t ws_bytes = hipcx_solve_workspace_size(&ca);
+        std::shared_ptr<void> ws = device.Allocate(ws_bytes);
+        std::shared_ptr<void> flag = NewInfoFlag(device);
+        Check(hipcx_inverse(&ca, &co, ws.get(), ws_bytes, static_cast<int32_t*>(flag.get()), nullptr));
+        ThrowIfInfo(flag, "getrf (LU)");
+    }
+};
+HIPCX_REGISTER_KERNEL(InverseKernel, HipInverseKernel)
+
+class HipCholeskyKernel : public CholeskyKernel {
+public:
+    void Call(const Array& a, const Array& out) override {
+        Device& device = a.device();
+        device.CheckDevicesCompatible(a, out);
+        SetDeviceScope scope{device.index()};
+        if (out.dtype() == Dtype::kFloat16) throw DtypeError{"Half-precision (float16) is not supported by cholesky"};
+        hipcx_array ca = ToC(a), co = ToC(out);
+        std::shared_ptr<void> flag = NewInfoFlag(device);
+        Check(hipcx_cholesky(&ca, &co, static_cast<int32_t*>(flag.get()), nullptr));
+        ThrowIfInfo(flag, "potrf (Cholesky)");
+    }
+};
+HIPCX_REGISTER_KERNEL(CholeskyKernel, HipCholeskyKernel)
+
 // ---- take ----
 class HipTakeKernel : public TakeKernel {
 public:

@@ -1200,6 +1200,72 @@ def average_pool(x, ksize, stride=None, pad=0, pad_mode='ignore'):
 
 
 # ---------------------------------------------------------------------------------------------
+# linear algebra (CX/routines/linalg.cc): solve, inv, cholesky
+# ---------------------------------------------------------------------------------------------
+def _check_square(a):
+    if a.ndim != 2:
+        raise _lib.DimensionError('ChainerX linear algebra routines only support 2-dimensional arrays.')
+    if a.shape[0] != a.shape[1]:
+        raise _lib.DimensionError('Matrix is not square.')
+
+
+def _linalg_flag():
+    flag = zeros((1,), 'int32')
+    return flag, ctypes.cast(ctypes.c_void_p(flag.data_ptr), ctypes.POINTER(ctypes.c_int32))
+
+
+def _raise_if_flagged(flag, what):
+    info = int(flag.get()[0])
+    if info != 0:
+        raise _lib.ChainerxError('Unsuccessful %s execution. Info = %d' % (what, info))
+
+
+def solve(a, b):
+    """Solve (CX/routines/linalg.cc:121-163): x with a @ x = b, b a vector or a matrix; dtype = ResultType(a, b)."""
+    _check_square(a)
+    dt = result_type(a, b)
+    if dt == numpy.dtype('float16'):
+        raise _lib.DtypeError('Half-precision (float16) is not supported by solve')
+    if _kind(dt) != 3:
+        dt = numpy.dtype('float32') if dt.itemsize < 8 else numpy.dtype('float64')
+    out = ndarray.empty(b.shape, dt)
+    nbytes = _lib.load().hipcx_solve_workspace_size(a.desc())
+    ws, wsp = _workspace(nbytes)
+    flag, flag_ptr = _linalg_flag()
+    _lib.call('hipcx_solve', a.desc(), b.desc(), out.desc(), wsp, nbytes, flag_ptr, current_stream())
+    _raise_if_flagged(flag, 'gesv (Solve)')
+    return out
+
+
+def inv(a):
+    """Inverse (CX/routines/linalg.cc:165-192), in the math dtype of a."""
+    _check_square(a)
+    dt = _math_result_dtype(a.dtype)
+    if dt == numpy.dtype('float16'):
+        raise _lib.DtypeError('Half-precision (float16) is not supported by inverse')
+    out = ndarray.empty(a.shape, dt)
+    nbytes = _lib.load().hipcx_solve_workspace_size(a.desc())
+    ws, wsp = _workspace(nbytes)
+    flag, flag_ptr = _linalg_flag()
+    _lib.call('hipcx_inverse', a.desc(), out.desc(), wsp, nbytes, flag_ptr, current_stream())
+    _raise_if_flagged(flag, 'getrf (LU)')
+    return out
+
+
+def cholesky(a):
+    """Cholesky (CX/routines/linalg.cc:415-450): the lower factor L of a = L @ L.T, read from a's lower triangle."""
+    _check_square(a)
+    dt = _math_result_dtype(a.dtype)
+    if dt == numpy.dtype('float16'):
+        raise _lib.DtypeError('Half-precision (float16) is not supported by cholesky')
+    out = ndarray.empty(a.shape, dt)
+    flag, flag_ptr = _linalg_flag()
+    _lib.call('hipcx_cholesky', a.desc(), out.desc(), flag_ptr, current_stream())
+    _raise_if_flagged(flag, 'potrf (Cholesky)')
+    return out
+
+
+# ---------------------------------------------------------------------------------------------
 # indexing
 # ---------------------------------------------------------------------------------------------
 _BOUNDS = {None: 0, 'raise': 1, 'wrap': 2, 'clip': 3}

@@ -272,6 +272,17 @@ int hipcx_fixed_batch_norm(const hipcx_array* x, const hipcx_array* gamma, const
                            const hipcx_array* var, hipcx_scalar eps, const int8_t* axis, int naxis, const hipcx_array* out,
                            void* stream);
 
+/* ---- linear algebra: SolveKernel, InverseKernel, CholeskyKernel CX/kernels/linalg.h:20-43 (float32 / float64, 2-D) ----
+ * The native backend calls LAPACK gesv / getrf + getri / potrf (CX/native/native_device/linalg.cc:280-347, 560-600); these entries
+ * agree with it to rounding.  `out` is C-contiguous; a (and b) are cast to out's dtype.  `error_flag`: a device int32 the caller
+ * zeroes; a singular / not positive definite matrix stores LAPACK's `info` (1-based position) there and the reference's
+ * ChainerxError is the caller's to raise.  Workspace: hipcx_solve_workspace_size(a) bytes for solve and inverse. */
+size_t hipcx_solve_workspace_size(const hipcx_array* a);
+int hipcx_solve(const hipcx_array* a, const hipcx_array* b, const hipcx_array* out, void* workspace, size_t workspace_bytes,
+                int32_t* error_flag, void* stream);
+int hipcx_inverse(const hipcx_array* a, const hipcx_array* out, void* workspace, size_t workspace_bytes, int32_t* error_flag, void* stream);
+int hipcx_cholesky(const hipcx_array* a, const hipcx_array* out, int32_t* error_flag, void* stream);
+
 /* ---- training-mode normalization: BatchNormKernel CX/kernels/normalization.h:32-47, BatchNormGradKernel :49-61 ----
  * For x C-contiguous with ndim >= 2 and `axis` = every axis but 1 (anything else: HIPCX_NOT_IMPLEMENTED_ERROR, and the caller
  * runs the reference's routine composition, CX/routines/normalization.cc:155-250).  gamma / beta / running_* / mean_out /

@@ -1153,6 +1153,34 @@ def n_step_birnn(n_layers, hx, ws, bs, xs, activation='tanh'):
     return _n_step(_rnn_step, n_layers, hx, None, ws, bs, xs, True, activation)
 
 
+def _linalg_dtype(*arrays):
+    dt = np.result_type(*[np.asarray(a).dtype for a in arrays])
+    if dt == np.float16:
+        raise TypeError('Half-precision (float16) is not supported')
+    return dt if dt.kind == 'f' else (np.dtype(np.float32) if dt.itemsize < 8 else np.dtype(np.float64))
+
+
+def solve(a, b):
+    """SolveKernel: LAPACK gesv in the result dtype (CX/native/native_device/linalg.cc:280-311) -- numpy.linalg.solve is the same
+    routine.  Raises numpy.linalg.LinAlgError where the native backend throws ChainerxError (info != 0)."""
+    dt = _linalg_dtype(a, b)
+    return np.linalg.solve(np.asarray(a).astype(dt), np.asarray(b).astype(dt)).astype(dt)
+
+
+def inv(a):
+    """InverseKernel: getrf + getri (CX/native/native_device/linalg.cc:313-347)."""
+    dt = _linalg_dtype(a)
+    a = np.asarray(a).astype(dt)
+    return np.linalg.inv(a).astype(dt) if a.size else a.copy()
+
+
+def cholesky(a):
+    """CholeskyKernel: potrf on the lower triangle, strict upper triangle zero (CX/native/native_device/linalg.cc:560-600)."""
+    dt = _linalg_dtype(a)
+    a = np.asarray(a).astype(dt)
+    return np.linalg.cholesky(np.tril(a) + np.tril(a, -1).T).astype(dt) if a.size else a.copy()
+
+
 def softmax_cross_entropy(x, t):
     """chainer/functions/loss/softmax_cross_entropy.py:123-130 (reduce='mean', normalize=True)."""
     x, t = np.asarray(x), np.asarray(t)

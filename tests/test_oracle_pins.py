@@ -836,3 +836,27 @@ def test_n_step_rejects_a_growing_batch():
     ws, bs, seqs, xs, hx, cx = _rnn_problem(rng, 'rnn', 1, False)
     with pytest.raises(ValueError):
         O.n_step_rnn(1, hx[:, :2], ws, bs, xs)
+
+
+def test_linalg_identities():
+    """solve / inv / cholesky reduce to LAPACK routines through numpy; pinned by what defines them: a @ x = b, inv(a) @ a = I,
+    L @ L.T = a with L lower triangular and only a's lower triangle read."""
+    rng = np.random.default_rng(9)
+    for n in (1, 2, 7, 40):
+        a = rng.standard_normal((n, n)) + n * np.eye(n)
+        b = rng.standard_normal((n, 3))
+        for dt, tol in (('float64', 1e-11), ('float32', 2e-4)):
+            x = O.solve(a.astype(dt), b.astype(dt))
+            assert x.dtype == np.dtype(dt) and np.abs(a @ x - b).max() <= tol * n
+            assert np.abs(O.solve(a.astype(dt), b[:, 0].astype(dt)) - x[:, 0]).max() <= tol
+            assert np.abs(O.inv(a.astype(dt)) @ a - np.eye(n)).max() <= tol * n
+            spd = (a @ a.T).astype(dt)
+            lower = O.cholesky(spd)
+            assert np.array_equal(lower, np.tril(lower)) and np.abs(lower @ lower.T - spd).max() <= tol * np.abs(spd).max() * n
+            garbage_above = np.tril(spd) + np.triu(rng.standard_normal((n, n)).astype(dt), 1)
+            assert np.array_equal(O.cholesky(garbage_above), lower)
+    assert O.solve(np.eye(2, dtype=np.int32), np.ones(2, np.int32)).dtype == np.float32
+    with pytest.raises(np.linalg.LinAlgError):
+        O.solve(np.zeros((2, 2)), np.ones(2))
+    with pytest.raises(np.linalg.LinAlgError):
+        O.cholesky(-np.eye(2))
