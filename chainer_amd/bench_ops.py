@@ -295,6 +295,27 @@ def section_backward(chx, oracle, with_cpu):
     bw_row('backward', 'average_pool_grad 7x7 (global)', (128, 2048, 7, 7), t, xa.nbytes + ga.nbytes)
 
 
+def section_train(chx, oracle, with_cpu):
+    """ResNet-50 training step (forward with batch statistics, hand-written backward, SGD) in float16 -- the kernel sequence of the
+    reference's ImageNet example without its autograd bookkeeping.  Not the headline metric: it shows the backward set end to end."""
+    import copy
+    from chainer_amd import configs as cfg
+    F = cfg.DeviceTrainOps(chx)
+    p0 = cfg.resnet50_params()
+    for batch in (32, 128):
+        x = chx.array(cfg.resnet50_input(batch=batch))
+        t = chx.array(np.random.default_rng(8).integers(0, 1000, batch).astype(np.int32))
+        pd = cfg.tree_map(chx.array, copy.deepcopy(p0))
+        step = lambda: cfg.resnet50_train_step(F, pd, x, t, 0.0)  # lr 0: the timed steps do not walk the weights into overflow
+        eager = device_time(step, 2, 1, 1)
+        graph = graph_time(step, 3)
+        flops = 3.0 * cfg.resnet50_flops(batch)
+        emit(section='train', op='ResNet-50 training step, float16', batch=batch, eager_ms=round(eager * 1e3, 2),
+             graph_replay_ms=round(graph * 1e3, 2), img_per_s_graph=round(batch / graph, 1), TFLOPs_graph=round(flops / graph / 1e12, 1),
+             note='3x the forward flops (forward, data gradient, weight gradient); eager time includes ~1500 Python-issued kernel calls')
+        del pd
+
+
 def section_copy(chx, oracle, with_cpu):
     """A plain copy of known size (128 MiB read + 128 MiB written): the calibration point for HBM traffic counters."""
     x = chx.array(np.zeros(64 * 1024 * 1024, np.float16))
@@ -302,7 +323,7 @@ def section_copy(chx, oracle, with_cpu):
     bw_row('copy', 'copy float16 [67108864]', (64 * 1024 * 1024,), t, 2 * x.nbytes)
 
 
-SECTIONS = {'copy': section_copy, 'sweep': section_sweep, 'mlp': section_mlp, 'cifar': section_cifar, 'resnet_layers': section_resnet_layers, 'lstm': section_lstm, 'backward': section_backward}
+SECTIONS = {'copy': section_copy, 'sweep': section_sweep, 'mlp': section_mlp, 'cifar': section_cifar, 'resnet_layers': section_resnet_layers, 'lstm': section_lstm, 'backward': section_backward, 'train': section_train}
 
 
 def run(sections, cpu=None):

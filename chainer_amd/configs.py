@@ -122,7 +122,7 @@ RESNET50_BLOCKS = (3, 4, 6, 3)
 RESNET50_RESIDUAL_GAMMA_SCALE = 0.25
 
 
-def resnet50_params(seed=4, dtype=np.float16, n_out=1000, residual_gamma_scale=RESNET50_RESIDUAL_GAMMA_SCALE):
+def resnet50_params(seed=4, dtype=np.float16, n_out=1000, residual_gamma_scale=RESNET50_RESIDUAL_GAMMA_SCALE, blocks=None):
     """He-normal filters and batch-norm statistics drawn as for the CIFAR net.  One deviation: gamma of the last
     batch norm of every residual branch is scaled by `residual_gamma_scale`.  With statistics that are drawn at random
     instead of measured, nothing normalises the residual stream: its magnitude grows ~1.4x per block and passes the
@@ -130,7 +130,7 @@ def resnet50_params(seed=4, dtype=np.float16, n_out=1000, residual_gamma_scale=R
     rng = _rng(seed)
     p = {'conv1': _he_normal(rng, (64, 3, 7, 7), dtype), 'bn1': _bn_params(rng, 64, dtype), 'stages': []}
     c_in = 64
-    for si, n_blocks in enumerate(RESNET50_BLOCKS):
+    for si, n_blocks in enumerate(blocks or RESNET50_BLOCKS):
         mid = 64 * 2 ** si
         c_out = 4 * mid
         stage = []
@@ -201,6 +201,117 @@ def resnet50_forward_fused(F, p, x):
             h = _conv_bn_act(F, t, blk['conv3'], 1, 0, blk['bn3'], residual=sc, relu=True)
     h = F.average_pool(h, h.shape[2], 1, 0, 'zero')
     return F.linear(h, p['fc_w'], p['fc_b'])
+
+
+# ---------------------------------------------------------------------------------------------
+# ResNet-50 training step: forward in training mode, the backward pass written out from the backward kernels, SGD.
+# This is the kernel sequence the reference's ImageNet example issues through autograd
+# (chainerx_cc/examples/imagenet_py/train_imagenet.py with resnet50.py); autograd itself is outside the backend.
+# `F` supplies the kernels: DeviceTrainOps below for the device, an adapter over the CPU oracle in the tests.
+# ---------------------------------------------------------------------------------------------
+class DeviceTrainOps:
+    """The call shapes resnet50_train_step uses, over the chainer_amd routines."""
+
+    def __init__(self, chx):
+        self.c = chx
+        for name in ('conv', 'relu', 'max_pool', 'average_pool', 'linear', 'log_softmax', 'exp', 'add', 'subtract', 'multiply', 'sum',
+                     'max_pool_grad', 'average_pool_grad', 'conv_transpose', 'dot', 'batch_norm_grad'):
+            setattr(self, name, getattr(chx, name))
+        self.array = chx.array
+        self.get = lambda a: a.get()
+
+    def conv_grad_weight(self, w, x, gy, stride, pad):
+        return self.c.conv_grad_weight(w.dtype, w.shape, x, gy, stride, pad)
+
+    def batch_norm(self, x, gamma, beta, rm, rv):
+        return self.c.batch_norm(x, gamma, beta, rm, rv, BN_EPS, 0.9)
+
+    def relu_grad(self, y, g):
+        return self.c.where(self.c.greater(y, 0), g, 0)
+
+    def onehot(self, t, n, dtype):
+        return self.c.equal(t[:, None], self.c.arange(n, dtype=t.dtype)).astype(dtype)
+
+    def scale(self, a, s):
+        return self.c.multiply(a, s)
+
+
+def _unit_forward(F, x, w, bn, stride, pad, relu):
+    """conv -> batch norm (batch statistics, running statistics updated in place) -> optional ReLU; returns (y, saved)."""
+    c = F.conv(x, w, None, stride, pad)
+    b, state = F.batch_norm(c, bn['gamma'], bn['beta'], bn['mean'], bn['var'])
+    y = F.relu(b) if relu else b
+    return y, (x, w, bn, stride, pad, c, state, y if relu else None)
+
+
+def _unit_backward(F, saved, gy, grads, need_gx=True):
+    x, w, bn, stride, pad, c, state, y = saved
+    g = F.relu_grad(y, gy) if y is not None else gy
+    gc, ggamma, gbeta = F.batch_norm_grad(c, bn['gamma'], g, state)
+    grads.append((bn, 'gamma', ggamma))
+    grads.append((bn, 'beta', gbeta))
+    grads.append((w, None, F.conv_grad_weight(w, x, gc, stride, pad)))
+    return F.conv_transpose(gc, w, None, stride, pad, x.shape[2:]) if need_gx else None
+
+
+def resnet50_train_step(F, p, x, t, lr=0.01):
+    """One SGD step on softmax cross entropy (mean over the batch); updates `p` in place and returns the loss array."""
+    n = x.shape[0]
+    # ---- forward ----
+    h0, s_stem = _unit_forward(F, x, p['conv1'], p['bn1'], 2, 3, True)
+    h = F.max_pool(h0, 3, 2, 1, False)
+    tape = []
+    for si, stage in enumerate(p['stages']):
+        for bi, blk in enumerate(stage):
+            stride = 2 if (bi == 0 and si > 0) else 1
+            a, s1 = _unit_forward(F, h, blk['conv1'], blk['bn1'], stride, 0, True)
+            b, s2 = _unit_forward(F, a, blk['conv2'], blk['bn2'], 1, 1, True)
+            c, s3 = _unit_forward(F, b, blk['conv3'], blk['bn3'], 1, 0, False)
+            if 'conv4' in blk:
+                sc, s4 = _unit_forward(F, h, blk['conv4'], blk['bn4'], stride, 0, False)
+            else:
+                sc, s4 = h, None
+            out = F.relu(F.add(c, sc))
+            tape.append((s1, s2, s3, s4, out))
+            h = out
+    pooled = F.average_pool(h, h.shape[2], 1, 0, 'zero')
+    feat = pooled.reshape((n, -1))
+    logits = F.linear(feat, p['fc_w'], p['fc_b'])
+    logp = F.log_softmax(logits, 1)
+    onehot = F.onehot(t, logits.shape[1], logp.dtype)
+    loss = F.scale(F.sum(F.multiply(logp, onehot)), -1.0 / n)
+    # ---- backward ----
+    grads = []  # (container, key or None for the array itself, gradient)
+    dlogits = F.scale(F.subtract(F.exp(logp), onehot), 1.0 / n)
+    g_fc_w = F.dot(dlogits.T, feat)
+    g_fc_b = F.sum(dlogits, 0)
+    gh = F.average_pool_grad(h, F.dot(dlogits, p['fc_w']).reshape(pooled.shape), h.shape[2], 1, 0, 'zero')
+    for (s1, s2, s3, s4, out) in reversed(tape):
+        g = F.relu_grad(out, gh)
+        gb = _unit_backward(F, s3, g, grads)
+        ga = _unit_backward(F, s2, gb, grads)
+        gx = _unit_backward(F, s1, ga, grads)
+        gh = F.add(gx, _unit_backward(F, s4, g, grads) if s4 is not None else g)
+    g0 = F.max_pool_grad(h0, gh, 3, 2, 1)
+    _unit_backward(F, s_stem, g0, grads, need_gx=False)
+    # ---- SGD ----
+    updates = {}
+    for container, key, g in grads:
+        if key is None:
+            updates[id(container)] = F.subtract(container, F.scale(g, lr))
+        else:
+            container[key] = F.subtract(container[key], F.scale(g.reshape(container[key].shape), lr))
+
+    def swap(tree):  # filters are values of dicts: replace them where they live
+        for k, v in (tree.items() if isinstance(tree, dict) else enumerate(tree)):
+            if isinstance(v, (dict, list)):
+                swap(v)
+            elif id(v) in updates:
+                tree[k] = updates[id(v)]
+    swap(p)
+    p['fc_w'] = F.subtract(p['fc_w'], F.scale(g_fc_w, lr))
+    p['fc_b'] = F.subtract(p['fc_b'], F.scale(g_fc_b, lr))
+    return loss
 
 
 def resnet50_flops(batch=128, size=224):

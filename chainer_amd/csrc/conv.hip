@@ -54,7 +54,9 @@ void LaunchShape(IGemmArgs<T> p, bool fast16, bool fast8, hipStream_t stream) {
     int64_t total = static_cast<int64_t>(p.tiles_m) * p.tiles_n;
     HIPCX_REQUIRE(total < (1LL << 30), HIPCX_NOT_IMPLEMENTED_ERROR, "problem too large for one launch");
     int per = static_cast<int>((total + 7) / 8);
-    dim3 grid(per * 8), block(64 * WM * WN);
+    static const bool pipe_env = [] { const char* e = getenv("HIPCX_IGEMM_PIPE"); return e != nullptr && e[0] == '1'; }();
+    if (PM || pipe_env || !(fast16 || fast8) || p.partial == nullptr) p.ksplit = 1;  // only the simple fast kernel splits the reduction
+    dim3 grid(per * 8, p.ksplit > 1 ? p.ksplit : 1), block(64 * WM * WN);
     // algorithmic work of this launch: 2 flops per multiply-add; every operand byte moved once
     double flops = 2.0 * static_cast<double>(p.M) * p.K * p.R * p.S * p.C_logical;
     double bytes = sizeof(T) * (static_cast<double>(p.N) * p.C_logical * p.H_logical * p.W_logical +
@@ -93,6 +95,12 @@ void LaunchShape(IGemmArgs<T> p, bool fast16, bool fast8, hipStream_t stream) {
         hipLaunchKernelGGL((IGemmGenericKernel<T, WM, WN, PM>), grid, block, 0, stream, p, x_row_fast, w_row_fast);
     }
     CheckLaunch("igemm");
+    if (p.ksplit > 1) {
+        int64_t blocks = (p.M * p.K + 255) / 256;
+        int64_t cap = static_cast<int64_t>(NumCUs()) * 16;
+        hipLaunchKernelGGL((SplitKReduceKernel<T>), dim3(static_cast<unsigned>(blocks > cap ? cap : blocks)), dim3(256), 0, stream, p);
+        CheckLaunch("igemm split reduction");
+    }
 }
 
 size_t RoundUpTo(size_t v, size_t a) { return (v + a - 1) / a * a; }
@@ -145,7 +153,9 @@ void LaunchIGemmImpl(IGemmArgs<T> p, hipStream_t stream) {
     // Small problems (batch-sized matrix products such as Linear on 100-128 rows): at 128x128 the grid would leave most of
     // the 256 CUs idle, so they run as one-wave 64x64 tiles instead.
     const int64_t big_tiles = ((p.M + 127) / 128) * ((p.K + 127) / 128);
-    if (big_tiles < 128 && p.M * static_cast<int64_t>(p.K) >= 64 * 64) {
+    if (p.ksplit > 1 && !pm && (fast16 || fast8)) {
+        LaunchShape<T, 2, 2, false>(p, fast16, fast8, stream);
+    } else if (big_tiles < 128 && p.M * static_cast<int64_t>(p.K) >= 64 * 64) {
         if (pm) LaunchShape<T, 1, 1, true>(p, fast16, fast8, stream);
         else LaunchShape<T, 1, 1, false>(p, fast16, fast8, stream);
     } else if (p.K <= 64) {
@@ -953,12 +963,33 @@ DotStaging PlanDotStaging(const hipcx_array* a, const hipcx_array* b, const hipc
 }
 }  // namespace
 
+namespace {
+// Matrix products with few 128x128 output tiles and a long reduction axis (weight gradients: M x N = filters, reduction = batch x
+// pixels): slices of the reduction run as separate workgroups.  Returns the number of slices (1: no split).
+int PlanSplitK(int64_t m, int64_t n, int64_t k, int dtype) {
+    static const bool enabled = [] { const char* e = getenv("HIPCX_DOT_SPLITK"); return e == nullptr || e[0] != '0'; }();
+    if (!enabled || (dtype != HIPCX_FLOAT16 && dtype != HIPCX_FLOAT32)) return 1;
+    const int64_t tiles = ((m + 127) / 128) * ((n + 127) / 128);
+    const int64_t steps = k * ItemSize(dtype) / 128;  // reduction steps of 128 bytes per row
+    if (k < 4096 || tiles * 2 > NumCUs() || m * n < 64 * 64 || steps < 16) return 1;
+    int64_t s = (2 * NumCUs() + tiles - 1) / tiles;
+    if (s > steps / 24) s = steps / 24;  // a slice of fewer steps costs more in partial sums than it gains
+    if (s > 64) s = 64;
+    return s < 2 ? 1 : static_cast<int>(s);
+}
+size_t SplitKBytes(int64_t m, int64_t n, int slices) { return slices > 1 ? static_cast<size_t>(slices) * m * n * sizeof(float) : 0; }
+}  // namespace
+
 extern "C" {
 
 size_t hipcx_dot_workspace_size(const hipcx_array* a, const hipcx_array* b, const hipcx_array* out) {
     try {
         DotStaging st = PlanDotStaging(a, b, out);
-        return st.a_bytes + st.b_bytes;
+        size_t split = 0;
+        if (a != nullptr && b != nullptr && out != nullptr && a->ndim == 2 && b->ndim == 2) {
+            split = SplitKBytes(a->shape[0], b->shape[1], PlanSplitK(a->shape[0], b->shape[1], a->shape[1], out->dtype));
+        }
+        return RoundUpTo(st.a_bytes + st.b_bytes, 256) + split;
     } catch (...) {
         return 0;
     }
@@ -1046,15 +1077,36 @@ int hipcx_dot(const hipcx_array* a, const hipcx_array* b, const hipcx_array* out
         }
         a = &a_st;
         b = &b_st;
+        // few output tiles over a long reduction axis, both operands laid out for the MFMA kernel: split the reduction
+        int slices = 1;
+        float* partial = nullptr;
+        {
+            const int64_t it = ItemSize(out->dtype);
+            const int planned = PlanSplitK(m, n, a->shape[1], out->dtype);
+            if (planned > 1 && OperandIsFast(a->data, a->strides[0], a->strides[1], k, it) &&
+                OperandIsFast(b->data, b->strides[1], b->strides[0], k, it) && out->strides[0] >= 0 && out->strides[1] >= 0) {
+                DotStaging plan = PlanDotStaging(a, b, out);  // nothing is staged for operands in this layout
+                const size_t offset = RoundUpTo(plan.a_bytes + plan.b_bytes, 256);
+                const size_t need = offset + SplitKBytes(m, n, planned);
+                if (workspace != nullptr && workspace_bytes >= need && reinterpret_cast<uintptr_t>(workspace) % 16 == 0) {
+                    slices = planned;
+                    partial = reinterpret_cast<float*>(static_cast<char*>(workspace) + offset);
+                }
+            }
+        }
         if (out->dtype == HIPCX_FLOAT16) {
-            if (TrySmallDot<half_t>(a, b, out, st)) return;
+            if (slices == 1 && TrySmallDot<half_t>(a, b, out, st)) return;
             IGemmArgs<half_t> p{};
             fill(p);
+            p.ksplit = slices;
+            p.partial = partial;
             LaunchIGemmImpl(p, st);
         } else if (out->dtype == HIPCX_FLOAT32) {
-            if (TrySmallDot<float>(a, b, out, st)) return;
+            if (slices == 1 && TrySmallDot<float>(a, b, out, st)) return;
             IGemmArgs<float> p{};
             fill(p);
+            p.ksplit = slices;
+            p.partial = partial;
             LaunchIGemmImpl(p, st);
         } else {
             IGemmArgs<double> p{};

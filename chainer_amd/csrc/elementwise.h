@@ -137,6 +137,12 @@ struct FirstInOf<Op, std::void_t<typename Op::In0>> {
     using type = typename Op::In0;
 };
 
+// Ops that set `static constexpr bool kNarrowVectors = true` are also instantiated for 8- and 4-byte vectors.
+template <typename Op, typename = void>
+struct HasNarrowVectors : std::false_type {};
+template <typename Op>
+struct HasNarrowVectors<Op, std::enable_if_t<Op::kNarrowVectors>> : std::true_type {};
+
 // Op interface:
 //   using In = ...; using Out = ...; static constexpr int kNumIn = n;  (optionally using In0 = ... for the first input)
 //   __device__ compute_t<Out> operator()(compute_t<In> a, compute_t<In> b, compute_t<In> c, compute_t<In> d, int64_t index) const
@@ -318,8 +324,18 @@ inline void LaunchElementwise(const EwPlan& p, const Op& op, hipStream_t stream)
         }
         return true;
     };
-    // Two instantiations per op keep the code object small: full 16-byte vectors, or scalars.
+    // Two instantiations per op keep the code object small: full 16-byte vectors, or scalars.  Ops that declare
+    // kNarrowVectors (plain copies: the strided copies of Im2Col, transposes and staging) also get 8- and 4-byte vectors, for
+    // rows that are not whole 16-byte multiples (14x14 and 7x7 planes of float16).
     if (kMaxVec > 1 && fits(kMaxVec)) return LaunchEwVec<Op, kMaxVec>(p, op, stream);
+    if constexpr (HasNarrowVectors<Op>::value) {
+        if constexpr (kMaxVec >= 4) {
+            if (fits(kMaxVec / 2)) return LaunchEwVec<Op, kMaxVec / 2>(p, op, stream);
+        }
+        if constexpr (kMaxVec >= 8) {
+            if (fits(kMaxVec / 4)) return LaunchEwVec<Op, kMaxVec / 4>(p, op, stream);
+        }
+    }
     return LaunchEwVec<Op, 1>(p, op, stream);
 }
 

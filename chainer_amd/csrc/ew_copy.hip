@@ -14,6 +14,7 @@ struct CastOp {
     using Out = TOut;
     static constexpr int kNumIn = 1;
     static constexpr bool kNeedsIndex = false;
+    static constexpr bool kNarrowVectors = std::is_same<TIn, TOut>::value && sizeof(TIn) <= 4;  // plain copies
     __device__ __forceinline__ compute_t<TOut> operator()(compute_t<TIn> a, compute_t<TIn>, compute_t<TIn>, compute_t<TIn>, int64_t) const {
         if constexpr (std::is_same<TOut, bool>::value) {
             return a != compute_t<TIn>{};

@@ -39,6 +39,10 @@ struct IGemmArgs {
     int tiles_m, tiles_n;
     int out_vec;                 // 1 if the 4 accumulators a lane holds per group can be stored as one vector
     int out_wide;                // 1 if 16-byte runs along the output's contiguous axis can be stored (pipelined kernel)
+    // Split reduction (matrix products with few output tiles and a long reduction axis, e.g. weight gradients): grid.y slices of
+    // the reduction steps, each storing float partial sums [ksplit][M][K]; SplitKReduceKernel adds them up.  0 or 1: off.
+    int ksplit;
+    float* partial;
 };
 
 constexpr int kRowBytes = 128;           // bytes of the reduction axis per tile row
@@ -170,6 +174,44 @@ __device__ __forceinline__ void StoreTile(const IGemmArgs<T>& p, int m0, int n0,
                 }
             }
         }
+    }
+}
+
+// Split reduction: the accumulators go out as floats, partial[slice][m][n], in StoreTile's orientation.
+template <typename T>
+__device__ __forceinline__ void StorePartial(const IGemmArgs<T>& p, int m0, int n0, int wm, int wn, int lane, float16_t (&acc)[2][2], int slice) {
+    const int lr = lane & 31;
+    const int g = lane >> 5;
+#pragma unroll
+    for (int tj = 0; tj < 2; ++tj) {
+        int64_t m = static_cast<int64_t>(m0) + wm * 64 + tj * 32 + lr;
+        if (m >= p.M) continue;
+        float* o = p.partial + (static_cast<int64_t>(slice) * p.M + m) * p.K;
+#pragma unroll
+        for (int ti = 0; ti < 2; ++ti) {
+#pragma unroll
+            for (int vq = 0; vq < 4; ++vq) {
+                int n = n0 + wn * 64 + ti * 32 + vq * 8 + g * 4;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    if (n + e < p.K) o[n + e] = acc[ti][tj][vq * 4 + e];
+                }
+            }
+        }
+    }
+}
+
+// out[m][n] = sum over slices of partial[slice][m][n] (+ bias), for outputs addressed as out + m * osN + n * osC (matrix products).
+template <typename T>
+__global__ __launch_bounds__(256) void SplitKReduceKernel(IGemmArgs<T> p) {
+    const int64_t total = p.M * p.K;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < total; i += static_cast<int64_t>(gridDim.x) * 256) {
+        float sum = 0.f;
+        for (int sl = 0; sl < p.ksplit; ++sl) sum += p.partial[static_cast<int64_t>(sl) * total + i];
+        const int64_t m = i / p.K;
+        const int n = static_cast<int>(i - m * p.K);
+        if (p.bias != nullptr) sum += static_cast<float>(p.bias[n * p.bias_stride]);
+        p.out[m * p.osN + static_cast<int64_t>(n) * p.osC] = static_cast<T>(sum);
     }
 }
 
@@ -345,13 +387,22 @@ __global__ __launch_bounds__(64 * WM * WN) void IGemmFastKernel(IGemmArgs<T> p) 
         }
     }
 
-    load_tile(0);
-    for (int kt = 0; kt < nk; ++kt) {
+    int kt_begin = 0, kt_end = nk;
+    if (p.ksplit > 1) {
+        kt_begin = static_cast<int>(static_cast<int64_t>(nk) * blockIdx.y / p.ksplit);
+        kt_end = static_cast<int>(static_cast<int64_t>(nk) * (blockIdx.y + 1) / p.ksplit);
+    }
+    if (kt_begin < kt_end) load_tile(kt_begin);
+    for (int kt = kt_begin; kt < kt_end; ++kt) {
         store_tile();
         __syncthreads();
-        if (kt + 1 < nk) load_tile(kt + 1);
+        if (kt + 1 < kt_end) load_tile(kt + 1);
         ComputeTile<T, PM>(ldsX, ldsW, wm, wn, lane, acc);
         __syncthreads();
+    }
+    if (p.ksplit > 1) {
+        if constexpr (!PM) StorePartial<T>(p, m0, n0, wm, wn, lane, acc, blockIdx.y);
+        return;
     }
     if (PM) {
         StoreTilePM<T>(p, m0, n0, wm, wn, lane, acc);

@@ -174,3 +174,19 @@ def test_conv3x3_float16_tile_variants(N, C, H, K):
     b = rng.standard_normal(K).astype('float16')
     y = chx.conv(chx.array(x), chx.array(w), chx.array(b), 1, 1)
     assert_close(y.get(), O.conv(x, w, b, 1, 1, False), 2e-2, 'conv3x3 %r' % ((N, C, H, K),))
+
+
+@pytest.mark.parametrize('dt,tol', [('float32', 1e-5), ('float16', 2e-2)])
+def test_dot_long_reduction_few_tiles(dt, tol):
+    """Few output tiles over a long reduction axis (the weight-gradient shape): slices of the reduction run as separate workgroups
+    and are summed in float.  Operands as the callers hand them over: a row-major, b the transposed view of a row-major [N, K]."""
+    import chainer_amd as chx
+    rng = np.random.default_rng(12)
+    for (m, k, n) in [(128, 8192, 256), (200, 5000, 130), (64, 16384, 64), (256, 4096, 576), (70, 6000, 300)]:
+        a = rng.standard_normal((m, k)).astype(dt)
+        bt = (rng.standard_normal((n, k)) / np.sqrt(k)).astype(dt)
+        ref = O.dot(a, np.ascontiguousarray(bt.T))
+        got = chx.dot(chx.array(a), chx.array(bt).T)
+        assert_close(got.get(), ref, tol, 'dot %s %r' % (dt, (m, k, n)))
+        out_t = chx.dot(chx.array(bt), chx.array(a).T)  # the same product transposed: [n, m]
+        assert_close(out_t.get(), ref.T.copy(), tol, 'dot transposed %s %r' % (dt, (m, k, n)))

@@ -142,3 +142,33 @@ def test_two_sgd_steps_match_the_oracle():
     assert np.allclose(ld, lo, rtol=1e-5, atol=1e-6), (ld, lo)
     for k in po:
         assert_close(pd[k].get(), po[k], 2e-5, 'parameter %s after two steps' % k)
+
+
+def test_resnet_training_step_matches_the_oracle():
+    """One SGD step of a bottleneck ResNet (one block per stage, 64x64 images) through configs.resnet50_train_step: conv / batch
+    norm (batch statistics) / ReLU / pooling / linear forward, every backward kernel, the update.  Device against oracle."""
+    import copy
+    import chainer_amd as chx
+    from chainer_amd import configs as cfg
+    p0 = cfg.resnet50_params(seed=7, dtype=np.float32, n_out=10, blocks=(1, 1, 1, 1))
+    rng = np.random.default_rng(70)
+    x = rng.standard_normal((8, 3, 64, 64)).astype('float32')
+    t = rng.integers(0, 10, 8).astype('int32')
+    po = copy.deepcopy(p0)
+    pd = cfg.tree_map(chx.array, copy.deepcopy(p0))
+    loss_o = float(np.asarray(cfg.resnet50_train_step(OracleOps, po, x, t, 0.05)))
+    loss_d = float(cfg.resnet50_train_step(cfg.DeviceTrainOps(chx), pd, chx.array(x), chx.array(t), 0.05).get())
+    assert abs(loss_d - loss_o) <= 1e-4 * abs(loss_o), (loss_d, loss_o)
+
+    def compare(a, b, path):
+        if isinstance(a, dict):
+            for k in a:
+                compare(a[k], b[k], path + '/' + str(k))
+        elif isinstance(a, list):
+            for i, (u, v) in enumerate(zip(a, b)):
+                compare(u, v, path + '/' + str(i))
+        else:
+            assert_close(a.get(), np.asarray(b), 2e-3, 'parameter %s after one step' % path)
+    compare(pd, po, '')
+    changed = np.abs(np.asarray(po['conv1']) - p0['conv1']).max()
+    assert changed > 0, 'the step must have updated the first filters'
