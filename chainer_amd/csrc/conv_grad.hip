@@ -1,0 +1,220 @@
+// ConvGradWeightKernel (CX/kernels/connection.h:34-49) for dense NCHW float16 / float32 / float64 arrays.
+//
+// The native backend computes gw = TensorDot(gy, Im2Col(x)) over the batch and the output positions
+// (CX/native/native_device/conv.cc:91-124).  Same product here, with both operands written once in the layout the MFMA matrix
+// kernel reads -- the reduction index (n, oh, ow) as the unit-stride axis:
+//     gy_t[k][n][oh][ow]            (one transposing copy of gy)
+//     col_t[c][r][s][n][oh][ow]     (Im2Col in one launch instead of kh*kw strided copies of a padded image)
+// and then gw[k][(c, r, s)] = Dot(gy_t, col_t^T), which for these shapes (few output tiles, long reduction) runs with the
+// reduction split over workgroups.
+#include "common.h"
+
+namespace hipcx {
+namespace {
+
+struct GradWeightArgs {
+    const void* x;
+    const void* gy;
+    void* col_t;
+    void* gy_t;
+    int N, C, H, W, K, kh, kw, OH, OW, sh, sw, ph, pw;
+};
+
+template <typename T, int VEC>
+struct alignas(sizeof(T) * VEC) GVec {
+    T v[VEC];
+};
+
+// One thread: VEC consecutive ow of one (c, r, s, n, oh).
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void Im2ColTKernel(GradWeightArgs p, int64_t total) {
+    const T* x = static_cast<const T*>(p.x);
+    T* col = static_cast<T*>(p.col_t);
+    const int owv = p.OW / VEC;
+    for (int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; idx < total; idx += static_cast<int64_t>(gridDim.x) * 256) {
+        int64_t t = idx;
+        const int wv = static_cast<int>(t % owv);
+        t /= owv;
+        const int oh = static_cast<int>(t % p.OH);
+        t /= p.OH;
+        const int n = static_cast<int>(t % p.N);
+        t /= p.N;
+        const int s = static_cast<int>(t % p.kw);
+        t /= p.kw;
+        const int r = static_cast<int>(t % p.kh);
+        const int c = static_cast<int>(t / p.kh);
+        const int ih = oh * p.sh - p.ph + r;
+        GVec<T, VEC> out;
+        const T* row = x + ((static_cast<int64_t>(n) * p.C + c) * p.H + ih) * p.W;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            const int iw = (wv * VEC + e) * p.sw - p.pw + s;
+            out.v[e] = (ih >= 0 && ih < p.H && iw >= 0 && iw < p.W) ? row[iw] : T(0);
+        }
+        *reinterpret_cast<GVec<T, VEC>*>(col + idx * VEC) = out;  // idx enumerates the vectors of col_t in memory order
+    }
+}
+
+// gy_t[k][n][p] = gy[n][k][p], VEC consecutive p per thread.
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void TransposeNKKernel(GradWeightArgs p, int64_t total) {
+    const T* gy = static_cast<const T*>(p.gy);
+    T* gt = static_cast<T*>(p.gy_t);
+    const int64_t pv = static_cast<int64_t>(p.OH) * p.OW / VEC;
+    for (int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; idx < total; idx += static_cast<int64_t>(gridDim.x) * 256) {
+        int64_t t = idx;
+        const int64_t v = t % pv;
+        t /= pv;
+        const int n = static_cast<int>(t % p.N);
+        const int k = static_cast<int>(t / p.N);
+        *reinterpret_cast<GVec<T, VEC>*>(gt + idx * VEC) =
+                *reinterpret_cast<const GVec<T, VEC>*>(gy + ((static_cast<int64_t>(n) * p.K + k) * pv + v) * VEC);
+    }
+}
+
+int WidestVec(int64_t extent, int64_t item, const void* a, const void* b) {
+    int v = static_cast<int>(16 / item);
+    while (v > 1 && (extent % v != 0 || reinterpret_cast<uintptr_t>(a) % (v * item) != 0 || reinterpret_cast<uintptr_t>(b) % (v * item) != 0)) v /= 2;
+    return v;
+}
+
+struct GradWeightPlan {
+    GradWeightArgs a{};
+    size_t col_bytes = 0, gyt_bytes = 0;
+    hipcx_array gy_t{}, col_view{};  // Dot operands: [K, NP] and the [NP, C*kh*kw] view of col_t
+};
+
+size_t RoundUp256(size_t v) { return (v + 255) / 256 * 256; }
+
+GradWeightPlan PlanGradWeight(const hipcx_array* x, const hipcx_array* gy, const hipcx_array* gw, const int64_t* stride, const int64_t* pad,
+                              int cover_all) {
+    ValidateArray(x, "x");
+    ValidateArray(gy, "gy");
+    ValidateArray(gw, "gw");
+    HIPCX_REQUIRE(x->ndim == 4 && gy->ndim == 4 && gw->ndim == 4, HIPCX_NOT_IMPLEMENTED_ERROR, "hip convolution supports 2 spatial dimensions");
+    HIPCX_REQUIRE(IsFloatDtype(gw->dtype) && x->dtype == gw->dtype && gy->dtype == gw->dtype, HIPCX_DTYPE_ERROR,
+                  "conv_grad_weight: x and gy must have gw's floating point dtype (cast with hipcx_copy first)");
+    HIPCX_REQUIRE(IsContiguous(x) && IsContiguous(gy) && IsContiguous(gw), HIPCX_NOT_IMPLEMENTED_ERROR,
+                  "hip conv_grad_weight: x, gy and gw must be C-contiguous");
+    HIPCX_REQUIRE(stride && pad && stride[0] > 0 && stride[1] > 0 && pad[0] >= 0 && pad[1] >= 0, HIPCX_DIMENSION_ERROR, "invalid stride or pad");
+    HIPCX_REQUIRE(gw->shape[1] == x->shape[1], HIPCX_DIMENSION_ERROR, "conv_grad_weight: gw and x disagree on the input channels");
+    const int64_t oh = hipcx_conv_out_dim(x->shape[2], gw->shape[2], stride[0], pad[0], cover_all);
+    const int64_t ow = hipcx_conv_out_dim(x->shape[3], gw->shape[3], stride[1], pad[1], cover_all);
+    HIPCX_REQUIRE(gy->shape[0] == x->shape[0] && gy->shape[1] == gw->shape[0] && gy->shape[2] == oh && gy->shape[3] == ow, HIPCX_DIMENSION_ERROR,
+                  "gy has the wrong shape " + ShapeStr(gy));
+    for (int i = 0; i < 4; ++i) {
+        HIPCX_REQUIRE(x->shape[i] < (1LL << 31) && gw->shape[i] < (1LL << 31) && gy->shape[i] < (1LL << 31), HIPCX_NOT_IMPLEMENTED_ERROR, "extent too large");
+    }
+    GradWeightPlan pl;
+    GradWeightArgs& a = pl.a;
+    a.x = x->data;
+    a.gy = gy->data;
+    a.N = static_cast<int>(x->shape[0]), a.C = static_cast<int>(x->shape[1]), a.H = static_cast<int>(x->shape[2]), a.W = static_cast<int>(x->shape[3]);
+    a.K = static_cast<int>(gw->shape[0]), a.kh = static_cast<int>(gw->shape[2]), a.kw = static_cast<int>(gw->shape[3]);
+    a.OH = static_cast<int>(oh), a.OW = static_cast<int>(ow);
+    a.sh = static_cast<int>(stride[0]), a.sw = static_cast<int>(stride[1]), a.ph = static_cast<int>(pad[0]), a.pw = static_cast<int>(pad[1]);
+    const int64_t it = ItemSize(gw->dtype);
+    const int64_t np = static_cast<int64_t>(a.N) * a.OH * a.OW;
+    const int64_t ckk = static_cast<int64_t>(a.C) * a.kh * a.kw;
+    pl.col_bytes = RoundUp256(static_cast<size_t>(ckk * np * it));
+    pl.gyt_bytes = RoundUp256(static_cast<size_t>(a.K * np * it));
+    pl.gy_t.dtype = gw->dtype, pl.gy_t.ndim = 2;
+    pl.gy_t.shape[0] = a.K, pl.gy_t.shape[1] = np;
+    pl.gy_t.strides[0] = np * it, pl.gy_t.strides[1] = it;
+    pl.col_view.dtype = gw->dtype, pl.col_view.ndim = 2;
+    pl.col_view.shape[0] = np, pl.col_view.shape[1] = ckk;
+    pl.col_view.strides[0] = it, pl.col_view.strides[1] = np * it;
+    return pl;
+}
+
+hipcx_array GwAsMatrix(const hipcx_array* gw) {
+    hipcx_array m{};
+    m.data = gw->data, m.dtype = gw->dtype, m.ndim = 2;
+    m.shape[0] = gw->shape[0];
+    m.shape[1] = gw->shape[1] * gw->shape[2] * gw->shape[3];
+    m.strides[1] = ItemSize(gw->dtype);
+    m.strides[0] = m.shape[1] * m.strides[1];
+    return m;
+}
+
+template <typename T>
+void RunLayouts(const GradWeightArgs& a, hipStream_t stream) {
+    const int64_t cap = static_cast<int64_t>(NumCUs()) * 32;
+    auto grid = [&](int64_t n) { int64_t b = (n + 255) / 256; return dim3(static_cast<unsigned>(b > cap ? cap : (b < 1 ? 1 : b))); };
+    {
+        const int v = WidestVec(a.OW, sizeof(T), a.col_t, a.col_t);
+        const int64_t total = static_cast<int64_t>(a.C) * a.kh * a.kw * a.N * a.OH * (a.OW / v);
+        switch (v) {
+            case 8: hipLaunchKernelGGL((Im2ColTKernel<T, (sizeof(T) <= 2 ? 8 : 1)>), grid(total), dim3(256), 0, stream, a, total); break;
+            case 4: hipLaunchKernelGGL((Im2ColTKernel<T, (sizeof(T) <= 4 ? 4 : 1)>), grid(total), dim3(256), 0, stream, a, total); break;
+            case 2: hipLaunchKernelGGL((Im2ColTKernel<T, 2>), grid(total), dim3(256), 0, stream, a, total); break;
+            default: hipLaunchKernelGGL((Im2ColTKernel<T, 1>), grid(total), dim3(256), 0, stream, a, total); break;
+        }
+        CheckLaunch("im2col (weight gradient)");
+    }
+    {
+        const int64_t plane = static_cast<int64_t>(a.OH) * a.OW;
+        const int v = WidestVec(plane, sizeof(T), a.gy, a.gy_t);
+        const int64_t total = static_cast<int64_t>(a.K) * a.N * (plane / v);
+        switch (v) {
+            case 8: hipLaunchKernelGGL((TransposeNKKernel<T, (sizeof(T) <= 2 ? 8 : 1)>), grid(total), dim3(256), 0, stream, a, total); break;
+            case 4: hipLaunchKernelGGL((TransposeNKKernel<T, (sizeof(T) <= 4 ? 4 : 1)>), grid(total), dim3(256), 0, stream, a, total); break;
+            case 2: hipLaunchKernelGGL((TransposeNKKernel<T, 2>), grid(total), dim3(256), 0, stream, a, total); break;
+            default: hipLaunchKernelGGL((TransposeNKKernel<T, 1>), grid(total), dim3(256), 0, stream, a, total); break;
+        }
+        CheckLaunch("gy transpose (weight gradient)");
+    }
+}
+
+}  // namespace
+}  // namespace hipcx
+
+using namespace hipcx;
+
+extern "C" {
+
+size_t hipcx_conv_grad_weight_workspace_size(const hipcx_array* x, const hipcx_array* gy, const hipcx_array* gw, const int64_t* stride,
+                                             const int64_t* pad, int cover_all) {
+    try {
+        if (x == nullptr || gy == nullptr || gw == nullptr) return 0;
+        GradWeightPlan pl = PlanGradWeight(x, gy, gw, stride, pad, cover_all);
+        hipcx_array out = GwAsMatrix(gw);
+        return pl.col_bytes + pl.gyt_bytes + hipcx_dot_workspace_size(&pl.gy_t, &pl.col_view, &out);
+    } catch (...) {
+        return 0;
+    }
+}
+
+int hipcx_conv_grad_weight(const hipcx_array* x, const hipcx_array* gy, const int64_t* stride, const int64_t* pad, int cover_all,
+                           const hipcx_array* gw, void* workspace, size_t workspace_bytes, void* stream) {
+    return Guard([&] {
+        GradWeightPlan pl = PlanGradWeight(x, gy, gw, stride, pad, cover_all);
+        hipcx_array out = GwAsMatrix(gw);
+        if (out.shape[0] == 0 || out.shape[1] == 0) return;
+        if (pl.gy_t.shape[1] == 0) {  // an empty batch or plane: the sum over nothing
+            hipcx_scalar zero{HIPCX_KIND_INT, 0, 0, 0.0};
+            int rc = hipcx_fill(gw, zero, stream);
+            HIPCX_REQUIRE(rc == HIPCX_OK, rc, hipcx_last_error());
+            return;
+        }
+        const size_t dot_bytes = hipcx_dot_workspace_size(&pl.gy_t, &pl.col_view, &out);
+        const size_t need = pl.col_bytes + pl.gyt_bytes + dot_bytes;
+        HIPCX_REQUIRE(workspace != nullptr && workspace_bytes >= need, HIPCX_CHAINERX_ERROR,
+                      "conv_grad_weight workspace too small: need " + std::to_string(need) + " bytes");
+        HIPCX_REQUIRE(reinterpret_cast<uintptr_t>(workspace) % 16 == 0, HIPCX_CHAINERX_ERROR, "workspace must be 16-byte aligned");
+        char* ws = static_cast<char*>(workspace);
+        pl.a.col_t = ws;
+        pl.a.gy_t = ws + pl.col_bytes;
+        pl.col_view.data = pl.a.col_t;
+        pl.gy_t.data = pl.a.gy_t;
+        hipStream_t st = AsStream(stream);
+        VisitFloatDtype(gw->dtype, [&](auto tag) {
+            using T = typename decltype(tag)::type;
+            RunLayouts<T>(pl.a, st);
+        });
+        int rc = hipcx_dot(&pl.gy_t, &pl.col_view, &out, ws + pl.col_bytes + pl.gyt_bytes, dot_bytes, stream);
+        HIPCX_REQUIRE(rc == HIPCX_OK, rc, hipcx_last_error());
+    });
+}
+
+}  // extern "C"

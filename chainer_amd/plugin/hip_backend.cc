@@ -911,7 +911,21 @@ public:
     Array Call(Dtype w_dtype, const Shape& w_shape, const Array& x, const Array& gy, const Dims& stride, const Dims& pad, bool cover_all,
                const absl::optional<Array>& out) override {
         if (out.has_value()) throw NotImplementedError{"Passing out as an argument is not yet supported."};
-        SetDeviceScope scope{x.device().index()};
+        Device& device = x.device();
+        device.CheckDevicesCompatible(x, gy);
+        SetDeviceScope scope{device.index()};
+        if (x.ndim() == 4 && GetKind(w_dtype) == DtypeKind::kFloat) {
+            // one entry: Im2Col and the gy transpose as one kernel each, then the matrix product (split over the reduction)
+            Array xc = AsContiguous(x.dtype() == w_dtype ? x : x.AsType(w_dtype));
+            Array gc = AsContiguous(gy.dtype() == w_dtype ? gy : gy.AsType(w_dtype));
+            Array gw = Empty(w_shape, w_dtype, device);
+            hipcx_array cx = ToC(xc), cg = ToC(gc), cw = ToC(gw);
+            int64_t st[2] = {stride[0], stride[1]}, pd[2] = {pad[0], pad[1]};
+            size_t ws_bytes = hipcx_conv_grad_weight_workspace_size(&cx, &cg, &cw, st, pd, cover_all ? 1 : 0);
+            std::shared_ptr<void> ws = device.Allocate(ws_bytes);
+            Check(hipcx_conv_grad_weight(&cx, &cg, st, pd, cover_all ? 1 : 0, &cw, ws.get(), ws_bytes, nullptr));
+            return gw;
+        }
         Array col = HipIm2Col(x, Dims{w_shape[2], w_shape[3]}, stride, pad, cover_all, 0);
         return native::TensorDot(gy, col, Axes{0, 2, 3}, Axes{0, 4, 5}, w_dtype);  // dispatches DotKernel on this backend
     }

@@ -1368,6 +1368,10 @@ def tensordot(a, b, a_axes, b_axes, out_dtype=None):
     return out.reshape(tuple(a.shape[i] for i in a_keep) + tuple(b.shape[i] for i in b_keep))
 
 
+# True: ConvGradWeight runs as strided copies + Dot issued from here instead of through hipcx_conv_grad_weight.
+COMPOSE_CONV_GRAD_WEIGHT = False
+
+
 def conv_grad_weight(w_dtype, w_shape, x, gy, stride=1, pad=0, cover_all=False):
     """ConvGradWeightKernel after the native backend (CX/native/native_device/conv.cc:91-124): Im2Col(x), then TensorDot(gy, col)
     over the batch and the output positions -> gw[K, C, kh, kw].  The same two matrices meet in the same Dot; only the col is
@@ -1381,6 +1385,16 @@ def conv_grad_weight(w_dtype, w_shape, x, gy, stride=1, pad=0, cover_all=False):
     ow = conv_out_dim(w, kw, sw, pw, cover_all)
     if gy.shape != (n, w_shape[0], oh, ow):
         raise _lib.DimensionError('gy has the wrong shape')
+    wdt = numpy.dtype(w_dtype)
+    if not COMPOSE_CONV_GRAD_WEIGHT and _kind(wdt) == 3 and tuple(w_shape[:2]) == (gy.shape[1], c):
+        # one entry: Im2Col and the gy transpose as one kernel each, then the matrix product
+        xc, gc = x.astype(wdt, False).as_contiguous(), gy.astype(wdt, False).as_contiguous()
+        gw = ndarray.empty(tuple(w_shape), wdt)
+        st, pd = _i64((sh, sw)), _i64((ph, pw))
+        nbytes = _lib.load().hipcx_conv_grad_weight_workspace_size(xc.desc(), gc.desc(), gw.desc(), st, pd, int(bool(cover_all)))
+        ws, wsp = _workspace(nbytes)
+        _lib.call('hipcx_conv_grad_weight', xc.desc(), gc.desc(), st, pd, int(bool(cover_all)), gw.desc(), wsp, nbytes, current_stream())
+        return gw
     xp = zeros((n, c, h + 2 * ph + (sh - 1 if cover_all else 0), w + 2 * pw + (sw - 1 if cover_all else 0)), x.dtype)
     _copy_into(xp[:, :, ph:ph + h, pw:pw + w], x)
     col_t = ndarray.empty((c, kh, kw, n, oh, ow), x.dtype)

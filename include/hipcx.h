@@ -272,6 +272,14 @@ int hipcx_fixed_batch_norm(const hipcx_array* x, const hipcx_array* gamma, const
                            const hipcx_array* var, hipcx_scalar eps, const int8_t* axis, int naxis, const hipcx_array* out,
                            void* stream);
 
+/* ---- ConvGradWeightKernel CX/kernels/connection.h:34-49 (2-D, C-contiguous NCHW x and gy in gw's float dtype) ----
+ * gw[k, c, r, s] = sum over n, oh, ow of gy[n, k, oh, ow] * x[n, c, oh*stride - pad + r, ow*stride - pad + s]: the native
+ * backend's TensorDot(gy, Im2Col(x)) (CX/native/native_device/conv.cc:91-124), equal to tolerance (float accumulation). */
+size_t hipcx_conv_grad_weight_workspace_size(const hipcx_array* x, const hipcx_array* gy, const hipcx_array* gw, const int64_t* stride,
+                                             const int64_t* pad, int cover_all);
+int hipcx_conv_grad_weight(const hipcx_array* x, const hipcx_array* gy, const int64_t* stride, const int64_t* pad, int cover_all,
+                           const hipcx_array* gw, void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---- linear algebra: SolveKernel, InverseKernel, CholeskyKernel CX/kernels/linalg.h:20-43 (float32 / float64, 2-D) ----
  * The native backend calls LAPACK gesv / getrf + getri / potrf (CX/native/native_device/linalg.cc:280-347, 560-600); these entries
  * agree with it to rounding.  `out` is C-contiguous; a (and b) are cast to out's dtype.  `error_flag`: a device int32 the caller

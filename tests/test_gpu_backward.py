@@ -35,6 +35,15 @@ def test_conv_grad_weight_and_transpose(dt, tol):
         gw = chx.conv_grad_weight(dt, w.shape, chx.array(x), chx.array(gy), st, pd, cv)
         assert gw.shape == w.shape and gw.dtype == np.dtype(dt)
         assert_close(gw.get(), O.conv_grad_weight(w.shape, x, gy, st, pd, cv), tol, 'conv_grad_weight ' + what)
+        from chainer_amd import routines
+        routines.COMPOSE_CONV_GRAD_WEIGHT = True
+        try:  # the same product issued as strided copies + Dot from the routine layer
+            gw_c = chx.conv_grad_weight(dt, w.shape, chx.array(x), chx.array(gy), st, pd, cv)
+        finally:
+            routines.COMPOSE_CONV_GRAD_WEIGHT = False
+        assert_close(gw_c.get(), O.conv_grad_weight(w.shape, x, gy, st, pd, cv), tol, 'conv_grad_weight (composed) ' + what)
+        gw_v = chx.conv_grad_weight(dt, w.shape, channels_last(chx, x), chx.array(gy), st, pd, cv)  # a non-contiguous x is copied first
+        assert_close(gw_v.get(), O.conv_grad_weight(w.shape, x, gy, st, pd, cv), tol, 'conv_grad_weight (channels-last x) ' + what)
         gx = chx.conv_transpose(chx.array(gy), chx.array(w), None, st, pd, (H, W))
         assert gx.shape == x.shape
         assert_close(gx.get(), O.conv_transpose(gy, w, None, st, pd, (H, W)), tol, 'conv_transpose ' + what)
