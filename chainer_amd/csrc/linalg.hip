@@ -150,6 +150,130 @@ __global__ __launch_bounds__(256) void IdentityFillKernel(T* out, int n) {
     out[e] = (e / n == e % n) ? T(1) : T(0);
 }
 
+// Symmetric eigendecomposition by cyclic Jacobi rotations, one workgroup.  s: [n, n] row-major, symmetric on entry, destroyed
+// (its diagonal converges to the eigenvalues); v: [n, n] accumulates the rotations (eigenvectors as columns); w: the eigenvalues in
+// ascending order, with the columns of v permuted to match (LAPACK syevd's order, CX/native/native_device/linalg.cc:602-660).
+// A sweep visits all pairs in n - 1 rounds of n / 2 disjoint pairs (round-robin pairing), so the rotations of a round apply in
+// parallel: first to the columns of s and v, then to the rows of s.
+template <typename T>
+__global__ __launch_bounds__(kLinalgThreads) void JacobiEighKernel(T* s, T* v, T* w, int n, int compute_v, int64_t v_row, int64_t v_col,
+                                                                   int64_t w_stride, T* v_scratch) {
+    extern __shared__ __align__(16) char eigh_lds[];
+    T* cs = reinterpret_cast<T*>(eigh_lds);             // [half][2]: cosine, sine of the round's rotations
+    int* pq = reinterpret_cast<int*>(cs + 2 * ((n + 1) / 2));  // [half][2]: the pairs
+    __shared__ T red[kLinalgThreads / 64];
+    __shared__ T off_norm, total_norm;
+    const int tid = threadIdx.x;
+    const int np = n + (n & 1);  // players of the round-robin schedule (one dummy when n is odd)
+    const int half = np / 2;
+    const int m = np - 1;
+    for (int64_t e = tid; e < static_cast<int64_t>(n) * n; e += kLinalgThreads) v_scratch[e] = (e / n == e % n) ? T(1) : T(0);
+    __syncthreads();
+    auto block_sum = [&](T x) -> T {
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) x += __shfl_down(x, o);
+        __syncthreads();
+        if ((tid & 63) == 0) red[tid >> 6] = x;
+        __syncthreads();
+        T r = T(0);
+        for (int k = 0; k < kLinalgThreads / 64; ++k) r += red[k];
+        return r;  // every thread adds the same partials
+    };
+    {
+        T acc = T(0);
+        for (int64_t e = tid; e < static_cast<int64_t>(n) * n; e += kLinalgThreads) acc += s[e] * s[e];
+        T t = block_sum(acc);
+        if (tid == 0) total_norm = t;
+        __syncthreads();
+    }
+    const T eps = std::is_same<T, float>::value ? T(4e-7) : T(1e-15);  // relative off-diagonal norm at which rounding dominates
+    for (int sweep = 0; sweep < 60; ++sweep) {
+        T acc = T(0);
+        for (int64_t e = tid; e < static_cast<int64_t>(n) * n; e += kLinalgThreads) {
+            if (e / n != e % n) acc += s[e] * s[e];
+        }
+        T t = block_sum(acc);
+        if (tid == 0) off_norm = t;
+        __syncthreads();
+        if (!(off_norm > eps * eps * total_norm)) break;  // uniform: every thread reads the same value
+        for (int round = 0; round < m; ++round) {
+            // the round's rotations
+            for (int i = tid; i < half; i += kLinalgThreads) {
+                int p = i == 0 ? m : (round + i) % m;
+                int q = i == 0 ? round % m : (round - i + m) % m;
+                if (p > q) { int t2 = p; p = q; q = t2; }
+                T c = T(1), sn = T(0);
+                if (q < n) {
+                    const T apq = s[static_cast<int64_t>(p) * n + q];
+                    if (apq != T(0)) {
+                        const T app = s[static_cast<int64_t>(p) * n + p], aqq = s[static_cast<int64_t>(q) * n + q];
+                        const T tau = (aqq - app) / (T(2) * apq);
+                        const T root = std::is_same<T, float>::value ? T(sqrtf(static_cast<float>(T(1) + tau * tau))) : T(sqrt(static_cast<double>(T(1) + tau * tau)));
+                        const T tt = (tau >= T(0) ? T(1) : T(-1)) / ((tau >= T(0) ? tau : -tau) + root);
+                        c = T(1) / (std::is_same<T, float>::value ? T(sqrtf(static_cast<float>(T(1) + tt * tt))) : T(sqrt(static_cast<double>(T(1) + tt * tt))));
+                        sn = tt * c;
+                    }
+                } else {
+                    q = -1;  // the dummy player: no rotation
+                }
+                cs[2 * i] = c, cs[2 * i + 1] = sn;
+                pq[2 * i] = p, pq[2 * i + 1] = q;
+            }
+            __syncthreads();
+            // columns of s and of v: x[:, p], x[:, q] <- c x[:, p] - s x[:, q], s x[:, p] + c x[:, q]
+            for (int64_t e = tid; e < static_cast<int64_t>(half) * n; e += kLinalgThreads) {
+                const int r = static_cast<int>(e / half), i = static_cast<int>(e % half);  // neighbours share a row of s
+                const int p = pq[2 * i], q = pq[2 * i + 1];
+                if (q < 0) continue;
+                const T c = cs[2 * i], sn = cs[2 * i + 1];
+                T* sp = s + static_cast<int64_t>(r) * n;
+                const T a = sp[p], b = sp[q];
+                sp[p] = c * a - sn * b;
+                sp[q] = sn * a + c * b;
+                T* vp = v_scratch + static_cast<int64_t>(r) * n;
+                const T va = vp[p], vb = vp[q];
+                vp[p] = c * va - sn * vb;
+                vp[q] = sn * va + c * vb;
+            }
+            __syncthreads();
+            // rows of s
+            for (int64_t e = tid; e < static_cast<int64_t>(half) * n; e += kLinalgThreads) {
+                const int i = static_cast<int>(e / n), r = static_cast<int>(e % n);
+                const int p = pq[2 * i], q = pq[2 * i + 1];
+                if (q < 0) continue;
+                const T c = cs[2 * i], sn = cs[2 * i + 1];
+                const T a = s[static_cast<int64_t>(p) * n + r], b = s[static_cast<int64_t>(q) * n + r];
+                s[static_cast<int64_t>(p) * n + r] = c * a - sn * b;
+                s[static_cast<int64_t>(q) * n + r] = sn * a + c * b;
+            }
+            __syncthreads();
+        }
+    }
+    // ascending order: rank of every diagonal entry (ties by index), then scatter
+    for (int i = tid; i < n; i += kLinalgThreads) {
+        const T wi = s[static_cast<int64_t>(i) * n + i];
+        int rank = 0;
+        for (int j = 0; j < n; ++j) {
+            const T wj = s[static_cast<int64_t>(j) * n + j];
+            if (wj < wi || (wj == wi && j < i)) ++rank;
+        }
+        w[rank * w_stride] = wi;
+        if (compute_v) {
+            for (int r = 0; r < n; ++r) v[r * v_row + rank * v_col] = v_scratch[static_cast<int64_t>(r) * n + i];
+        }
+    }
+}
+
+// s[i][j] <- a read from the chosen triangle (upper: a[min][max], lower: a[max][min]), cast is the caller's.
+template <typename T>
+__global__ __launch_bounds__(256) void SymmetrizeKernel(const T* a, int64_t a_row, int64_t a_col, T* s, int n, int upper) {
+    const int64_t e = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (e >= static_cast<int64_t>(n) * n) return;
+    const int i = static_cast<int>(e / n), j = static_cast<int>(e % n);
+    const int lo = i < j ? i : j, hi = i < j ? j : i;
+    s[e] = upper ? a[lo * a_row + hi * a_col] : a[hi * a_row + lo * a_col];
+}
+
 void CheckSquare(const hipcx_array* a, const char* name) {
     ValidateArray(a, name);
     HIPCX_REQUIRE(a->ndim == 2, HIPCX_DIMENSION_ERROR, "ChainerX linear algebra routines only support 2-dimensional arrays.");
@@ -266,6 +390,50 @@ int hipcx_cholesky(const hipcx_array* a, const hipcx_array* out, int32_t* error_
                                static_cast<int>(n), error_flag);
         }
         CheckLaunch("cholesky");
+    });
+}
+
+size_t hipcx_syevd_workspace_size(const hipcx_array* a) {
+    if (a == nullptr || a->ndim != 2 || a->shape[0] < 0) return 0;
+    return static_cast<size_t>(a->shape[0]) * static_cast<size_t>(a->shape[0]) * 8 * 2;  // the working copy and the rotations
+}
+
+int hipcx_syevd(const hipcx_array* a, const hipcx_array* w, const hipcx_array* v, char uplo, int compute_v, void* workspace,
+                size_t workspace_bytes, void* stream) {
+    return Guard([&] {
+        CheckSquare(a, "a");
+        ValidateArray(w, "w");
+        ValidateArray(v, "v");
+        CheckLinalgDtype(a->dtype, "eigh");
+        HIPCX_REQUIRE(uplo == 'U' || uplo == 'u' || uplo == 'L' || uplo == 'l', HIPCX_CHAINERX_ERROR, "eigh: uplo must be 'U' or 'L'");
+        HIPCX_REQUIRE(w->dtype == a->dtype && v->dtype == a->dtype, HIPCX_DTYPE_ERROR, "eigh: w and v must have a's dtype");
+        const int64_t n = a->shape[0];
+        HIPCX_REQUIRE(w->ndim == 1 && w->shape[0] == n, HIPCX_DIMENSION_ERROR, "eigh: w must have one entry per row of a");
+        HIPCX_REQUIRE(!compute_v || (v->ndim == 2 && v->shape[0] == n && v->shape[1] == n), HIPCX_DIMENSION_ERROR, "eigh: v must have a's shape");
+        if (n == 0) return;
+        HIPCX_REQUIRE(n <= 4096, HIPCX_NOT_IMPLEMENTED_ERROR, "hip eigh: matrix too large for the one-workgroup Jacobi kernel");
+        const int64_t it = ItemSize(a->dtype);
+        const size_t need = static_cast<size_t>(n * n * it) * 2;
+        HIPCX_REQUIRE(workspace != nullptr && workspace_bytes >= need, HIPCX_CHAINERX_ERROR, "eigh workspace too small");
+        HIPCX_REQUIRE(reinterpret_cast<uintptr_t>(workspace) % 16 == 0, HIPCX_CHAINERX_ERROR, "workspace must be 16-byte aligned");
+        const int upper = (uplo == 'U' || uplo == 'u') ? 1 : 0;
+        const unsigned blocks = static_cast<unsigned>((n * n + 255) / 256);
+        const size_t lds = static_cast<size_t>((n + 1) / 2) * (2 * it + 2 * sizeof(int)) + 16;
+        hipStream_t st = AsStream(stream);
+        char* ws = static_cast<char*>(workspace);
+        auto run = [&](auto tag) {
+            using T = decltype(tag);
+            T* s = reinterpret_cast<T*>(ws);
+            T* vs = reinterpret_cast<T*>(ws + n * n * it);
+            hipLaunchKernelGGL(SymmetrizeKernel<T>, dim3(blocks), dim3(256), 0, st, static_cast<const T*>(a->data), a->strides[0] / it,
+                               a->strides[1] / it, s, static_cast<int>(n), upper);
+            hipLaunchKernelGGL(JacobiEighKernel<T>, dim3(1), dim3(kLinalgThreads), lds, st, s, static_cast<T*>(v->data),
+                               static_cast<T*>(w->data), static_cast<int>(n), compute_v ? 1 : 0, compute_v ? v->strides[0] / it : 0,
+                               compute_v ? v->strides[1] / it : 0, w->strides[0] / it, vs);
+        };
+        if (a->dtype == HIPCX_FLOAT32) run(float{});
+        else run(double{});
+        CheckLaunch("eigh");
     });
 }
 

@@ -1098,7 +1098,7 @@ public:
 };
 HIPCX_REGISTER_KERNEL(AveragePoolGradKernel, HipAveragePoolGradKernel)
 
-// ---- linear algebra: Solve, Inverse, Cholesky (the LAPACK-backed kernels of the native backend, native_device/linalg.cc) ----
+// ---- linear algebra: Solve, Inverse, Cholesky, Syevd (the LAPACK-backed kernels of the native backend, native_device/linalg.cc) ----
 namespace {
 // A zeroed device int32 for LAPACK's `info`, and the check that turns a non-zero value into the reference's ChainerxError.
 std::shared_ptr<void> NewInfoFlag(Device& device) {
@@ -1161,6 +1161,21 @@ public:
     }
 };
 HIPCX_REGISTER_KERNEL(CholeskyKernel, HipCholeskyKernel)
+
+class HipSyevdKernel : public SyevdKernel {
+public:
+    void Call(const Array& a, const Array& w, const Array& v, char uplo, bool compute_v) override {
+        Device& device = a.device();
+        device.CheckDevicesCompatible(a, w, v);
+        SetDeviceScope scope{device.index()};
+        if (a.dtype() == Dtype::kFloat16) throw DtypeError{"Half-precision (float16) is not supported by eigen decomposition"};
+        hipcx_array ca = ToC(a), cw = ToC(w), cv = ToC(v);
+        size_t ws_bytes = hipcx_syevd_workspace_size(&ca);
+        std::shared_ptr<void> ws = device.Allocate(ws_bytes);
+        Check(hipcx_syevd(&ca, &cw, &cv, uplo, compute_v ? 1 : 0, ws.get(), ws_bytes, nullptr));
+    }
+};
+HIPCX_REGISTER_KERNEL(SyevdKernel, HipSyevdKernel)
 
 // ---- take ----
 class HipTakeKernel : public TakeKernel {

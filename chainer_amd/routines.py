@@ -1200,7 +1200,7 @@ def average_pool(x, ksize, stride=None, pad=0, pad_mode='ignore'):
 
 
 # ---------------------------------------------------------------------------------------------
-# linear algebra (CX/routines/linalg.cc): solve, inv, cholesky
+# linear algebra (CX/routines/linalg.cc): solve, inv, cholesky, eigh, eigvalsh
 # ---------------------------------------------------------------------------------------------
 def _check_square(a):
     if a.ndim != 2:
@@ -1263,6 +1263,34 @@ def cholesky(a):
     _lib.call('hipcx_cholesky', a.desc(), out.desc(), flag_ptr, current_stream())
     _raise_if_flagged(flag, 'potrf (Cholesky)')
     return out
+
+
+def _syevd(a, uplo, compute_v):
+    _check_square(a)
+    if not isinstance(uplo, str) or len(uplo) != 1:
+        raise TypeError('UPLO must be a one-character string')
+    if uplo.upper() not in ('U', 'L'):
+        raise _lib.ChainerxError("UPLO argument must be 'L' or 'U'.")
+    if a.dtype == numpy.dtype('float16'):
+        raise _lib.DtypeError('Half-precision (float16) is not supported by eigen decomposition')
+    if _kind(a.dtype) != 3:
+        raise _lib.DtypeError('Eigen decomposition needs a floating-point matrix')
+    w = ndarray.empty((a.shape[0],), a.dtype)
+    v = ndarray.empty(a.shape, a.dtype)
+    nbytes = _lib.load().hipcx_syevd_workspace_size(a.desc())
+    ws, wsp = _workspace(nbytes)
+    _lib.call('hipcx_syevd', a.desc(), w.desc(), v.desc(), uplo.encode(), 1 if compute_v else 0, wsp, nbytes, current_stream())
+    return w, v
+
+
+def eigh(a, UPLO='L'):
+    """Eigh (CX/routines/linalg.cc:452-495): (w, v) with a @ v = v * w, w ascending, a read from its UPLO triangle."""
+    return _syevd(a, UPLO, True)
+
+
+def eigvalsh(a, UPLO='L'):
+    """Eigvalsh (CX/routines/linalg.cc:497-511): the eigenvalues alone."""
+    return _syevd(a, UPLO, False)[0]
 
 
 # ---------------------------------------------------------------------------------------------

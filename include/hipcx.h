@@ -291,6 +291,16 @@ int hipcx_solve(const hipcx_array* a, const hipcx_array* b, const hipcx_array* o
 int hipcx_inverse(const hipcx_array* a, const hipcx_array* out, void* workspace, size_t workspace_bytes, int32_t* error_flag, void* stream);
 int hipcx_cholesky(const hipcx_array* a, const hipcx_array* out, int32_t* error_flag, void* stream);
 
+/* ---- SyevdKernel CX/kernels/linalg.h:45-48 (float32 / float64, a 2-D and square) ----
+ * Eigenvalues w (ascending) and, when compute_v, eigenvectors v (as columns) of the symmetric matrix held in a's `uplo` triangle
+ * ('U' / 'L', either case; the other triangle is never read), as LAPACK syevd gives them to the native backend
+ * (CX/native/native_device/linalg.cc:602-660).  Cyclic Jacobi rotations in one workgroup: eigenvalues agree with LAPACK's to
+ * rounding, eigenvectors up to the sign of each column (and up to a rotation inside an eigenspace of a repeated eigenvalue).
+ * w: [n], v: [n, n], any strides, a's dtype.  Workspace: hipcx_syevd_workspace_size(a) bytes.  n <= 4096. */
+size_t hipcx_syevd_workspace_size(const hipcx_array* a);
+int hipcx_syevd(const hipcx_array* a, const hipcx_array* w, const hipcx_array* v, char uplo, int compute_v, void* workspace,
+                size_t workspace_bytes, void* stream);
+
 /* ---- training-mode normalization: BatchNormKernel CX/kernels/normalization.h:32-47, BatchNormGradKernel :49-61 ----
  * For x C-contiguous with ndim >= 2 and `axis` = every axis but 1 (anything else: HIPCX_NOT_IMPLEMENTED_ERROR, and the caller
  * runs the reference's routine composition, CX/routines/normalization.cc:155-250).  gamma / beta / running_* / mean_out /

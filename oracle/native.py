@@ -1181,6 +1181,24 @@ def cholesky(a):
     return np.linalg.cholesky(np.tril(a) + np.tril(a, -1).T).astype(dt) if a.size else a.copy()
 
 
+def eigh(a, uplo='L'):
+    """SyevdKernel with compute_v: LAPACK syevd on the `uplo` triangle of the row-major matrix, eigenvalues ascending, eigenvectors
+    as columns (CX/native/native_device/linalg.cc:602-660; routine CX/routines/linalg.cc:452-495) -- numpy.linalg.eigh calls the same
+    driver.  Only floating-point input (VisitFloatingPointDtype)."""
+    a = np.asarray(a)
+    if a.dtype.kind != 'f' or a.dtype == np.float16:
+        raise TypeError('eigh needs float32 / float64')
+    if a.size == 0:
+        return np.empty((0,), a.dtype), a.copy()
+    w, v = np.linalg.eigh(a, UPLO=uplo.upper())
+    return w.astype(a.dtype), v.astype(a.dtype)
+
+
+def eigvalsh(a, uplo='L'):
+    """SyevdKernel without compute_v (CX/routines/linalg.cc:497-511)."""
+    return eigh(a, uplo)[0]
+
+
 def softmax_cross_entropy(x, t):
     """chainer/functions/loss/softmax_cross_entropy.py:123-130 (reduce='mean', normalize=True)."""
     x, t = np.asarray(x), np.asarray(t)

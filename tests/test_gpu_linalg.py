@@ -1,4 +1,4 @@
-"""Solve / Inverse / Cholesky against the CPU oracle (LAPACK through numpy, as the native backend calls it).
+"""Solve / Inverse / Cholesky / Eigh against the CPU oracle (LAPACK through numpy, as the native backend calls it).
 
 The device kernels use another operation order than LAPACK's blocked routines, so agreement is to rounding: errors are measured
 against the conditioning-free residuals (a @ x - b, inv(a) @ a - I, L @ L.T - a) as well as against the oracle's values."""
@@ -66,3 +66,66 @@ def test_linalg_errors_and_empty():
         chx.solve(chx.zeros((2, 2), 'float16'), chx.zeros((2,), 'float16'))
     assert chx.inv(chx.zeros((0, 0), 'float32')).shape == (0, 0)
     assert chx.solve(chx.zeros((0, 0), 'float32'), chx.zeros((0, 2), 'float32')).shape == (0, 2)
+
+
+@pytest.mark.parametrize('dt,tol', [('float32', 2e-5), ('float64', 1e-12)])
+def test_eigh(dt, tol):
+    """Eigenvalues against the oracle's (LAPACK syevd); eigenvectors through what defines them (a @ v = v * w, orthonormal
+    columns) and, for well separated spectra, against the oracle's up to the sign of each column -- the comparison the reference's
+    own test makes (tests/chainerx_tests/unit_tests/routines_tests/test_linalg.py:510-539)."""
+    import chainer_amd as chx
+    rng = np.random.default_rng(4)
+    for n in (1, 2, 3, 8, 33, 64, 129, 200):
+        a = rng.standard_normal((n, n)).astype(dt)
+        a = ((a + a.T) / 2 + 1e-3 * np.eye(n)).astype(dt)
+        scale = max(np.abs(a).max() * n ** 0.5, 1.0)
+        for uplo in ('u', 'L'):
+            noise = rng.standard_normal((n, n)).astype(dt)
+            spoiled = np.triu(a) + np.tril(noise, -1) if uplo.upper() == 'U' else np.tril(a) + np.triu(noise, 1)
+            w, v = chx.eigh(chx.array(spoiled), uplo)
+            assert w.shape == (n,) and v.shape == (n, n) and w.dtype == np.dtype(dt) and v.dtype == np.dtype(dt)
+            w, v = w.get(), v.get()
+            w_ref, v_ref = O.eigh(a, uplo)
+            assert np.all(np.diff(w) >= 0), 'ascending order'
+            assert np.abs(w - w_ref).max() <= tol * scale * n ** 0.5, 'eigenvalues n=%d' % n
+            a64, v64 = a.astype(np.float64), v.astype(np.float64)
+            assert np.abs(a64 @ v64 - v64 * w).max() <= tol * scale * n ** 0.5, 'a v = v w, n=%d' % n
+            assert np.abs(v64.T @ v64 - np.eye(n)).max() <= tol * n, 'orthonormal n=%d' % n
+            only_w = chx.eigvalsh(chx.array(spoiled), uplo).get()
+            assert np.array_equal(only_w, w)
+    # a prescribed, well separated spectrum: eigenvectors agree with LAPACK's up to sign
+    n = 12
+    q, _ = np.linalg.qr(rng.standard_normal((n, n)))
+    d = np.arange(1, n + 1, dtype=np.float64)
+    a = ((q * d) @ q.T)
+    a = ((a + a.T) / 2).astype(dt)
+    w, v = chx.eigh(chx.array(a))
+    w_ref, v_ref = O.eigh(a)
+    assert_close(w.get(), w_ref, tol * 100, 'prescribed spectrum')
+    assert np.abs(np.abs(v.get()) - np.abs(v_ref)).max() <= tol * 1000
+    # a transposed view and a diagonal matrix (no rotation at all: the values are only sorted)
+    wt = chx.eigvalsh(chx.array(a).T, 'U').get()
+    assert_close(wt, w_ref, tol * 100, 'transposed view reads the other triangle of the same symmetric matrix')
+    dg = np.diag(np.array([3., -1., 2., -1.], dt))
+    w, v = chx.eigh(chx.array(dg))
+    assert np.array_equal(w.get(), np.array([-1., -1., 2., 3.], dt))
+    assert np.array_equal(np.abs(v.get()), np.eye(4, dtype=dt)[:, [1, 3, 2, 0]])
+
+
+def test_eigh_errors_and_empty():
+    import chainer_amd as chx
+    w, v = chx.eigh(chx.zeros((0, 0), 'float32'))
+    assert w.shape == (0,) and v.shape == (0, 0)
+    with pytest.raises(chx.DimensionError):
+        chx.eigh(chx.zeros((2, 3), 'float32'))
+    with pytest.raises(chx.DimensionError):
+        chx.eigvalsh(chx.zeros((2, 2, 2), 'float32'))
+    with pytest.raises(chx.DtypeError):
+        chx.eigh(chx.zeros((2, 2), 'float16'))
+    with pytest.raises(chx.DtypeError):
+        chx.eigh(chx.zeros((2, 2), 'int32'))
+    with pytest.raises(chx.ChainerxError):
+        chx.eigh(chx.zeros((2, 2), 'float32'), 'X')
+    with pytest.raises(TypeError):
+        chx.eigh(chx.zeros((2, 2), 'float32'), None)
+

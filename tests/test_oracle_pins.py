@@ -860,3 +860,31 @@ def test_linalg_identities():
         O.solve(np.zeros((2, 2)), np.ones(2))
     with pytest.raises(np.linalg.LinAlgError):
         O.cholesky(-np.eye(2))
+
+
+def test_eigh_identities():
+    """eigh / eigvalsh reduce to LAPACK syevd through numpy; pinned by what defines them: a known spectrum (a = q diag(d) q.T) is
+    recovered in ascending order, a @ v = v * w with orthonormal columns, and only the chosen triangle is read."""
+    rng = np.random.default_rng(10)
+    for n in (1, 2, 6, 30):
+        q, _ = np.linalg.qr(rng.standard_normal((n, n)))
+        d = np.sort(rng.standard_normal(n) * 3)
+        a = (q * d) @ q.T
+        a = (a + a.T) / 2
+        for dt, tol in (('float64', 1e-12), ('float32', 1e-5)):
+            ad = a.astype(dt)
+            for uplo in ('U', 'l'):
+                w, v = O.eigh(ad, uplo)
+                assert w.dtype == np.dtype(dt) and v.dtype == np.dtype(dt)
+                assert np.abs(w - d).max() <= tol * n * 10
+                assert np.abs(ad.astype(np.float64) @ v - v * w).max() <= tol * n * 10
+                assert np.abs(v.T.astype(np.float64) @ v - np.eye(n)).max() <= tol * n * 10
+                noise = rng.standard_normal((n, n)).astype(dt)
+                spoiled = np.triu(ad) + np.tril(noise, -1) if uplo.upper() == 'U' else np.tril(ad) + np.triu(noise, 1)
+                assert np.array_equal(O.eigvalsh(spoiled, uplo), w)
+    # a matrix whose two triangles differ: each triangle defines its own symmetric matrix
+    m = np.array([[2., 1.], [0., 2.]])
+    assert np.allclose(O.eigvalsh(m, 'U'), [1., 3.]) and np.allclose(O.eigvalsh(m, 'L'), [2., 2.])
+    with pytest.raises(TypeError):
+        O.eigh(np.eye(2, dtype=np.int32))
+
