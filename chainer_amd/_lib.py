@@ -179,6 +179,8 @@ SIGNATURES = {
     'hipcx_cholesky': (_INT, [_A, _A, ctypes.POINTER(ctypes.c_int32), _V]),
     'hipcx_syevd_workspace_size': (_SZ, [_A]),
     'hipcx_syevd': (_INT, [_A, _A, _A, ctypes.c_char, _INT, _V, _SZ, _V]),
+    'hipcx_qr_workspace_size': (_SZ, [_A]),
+    'hipcx_qr': (_INT, [_A, _A, _A, _A, _INT, _V, _SZ, _V]),
     'hipcx_conv_grad_weight_workspace_size': (_SZ, [_A, _A, _A, _I64P, _I64P, _INT]),
     'hipcx_conv_grad_weight': (_INT, [_A, _A, _I64P, _I64P, _INT, _A, _V, _SZ, _V]),
     'hipcx_max_pool': (_INT, [_A, _I64P, _I64P, _I64P, _INT, _A, _V]),

@@ -274,6 +274,120 @@ __global__ __launch_bounds__(256) void SymmetrizeKernel(const T* a, int64_t a_ro
     s[e] = upper ? a[lo * a_row + hi * a_col] : a[hi * a_row + lo * a_col];
 }
 
+// y[i][c] -= tau * v[i] * (sum over i of v[i] * y[i][c]) for rows i in [j, m) and columns c in [c_begin, c_end): the Householder
+// reflector H = I - tau v v^T with v[j] = 1 and v[i > j] = w[i][j] (LAPACK's storage), applied from the left.  Whole workgroup,
+// 64 columns at a time with 16 row groups whose partial sums meet in LDS.
+template <typename T>
+__device__ void ApplyReflector(const T* w, int n, int j, int m, T tau, T* y, int64_t y_row, int64_t y_col, int c_begin, int c_end, T* part) {
+    const int tid = threadIdx.x, tx = tid & 63, ty = tid >> 6;
+    constexpr int kGroups = kLinalgThreads / 64;
+    for (int c0 = c_begin; c0 < c_end; c0 += 64) {  // uniform bounds: every thread reaches every barrier
+        const int c = c0 + tx;
+        T acc = T(0);
+        if (c < c_end) {
+            for (int i = j + ty; i < m; i += kGroups) {
+                const T vi = i == j ? T(1) : w[static_cast<int64_t>(i) * n + j];
+                acc += vi * y[i * y_row + c * y_col];
+            }
+        }
+        part[ty * 64 + tx] = acc;
+        __syncthreads();
+        T total = T(0);
+#pragma unroll
+        for (int g = 0; g < kGroups; ++g) total += part[g * 64 + tx];
+        total *= tau;
+        if (c < c_end) {
+            for (int i = j + ty; i < m; i += kGroups) {
+                const T vi = i == j ? T(1) : w[static_cast<int64_t>(i) * n + j];
+                y[i * y_row + c * y_col] -= vi * total;
+            }
+        }
+        __syncthreads();
+    }
+}
+
+template <typename T>
+__device__ inline T SqrtT(T x) {
+    return std::is_same<T, float>::value ? T(sqrtf(static_cast<float>(x))) : T(sqrt(static_cast<double>(x)));
+}
+
+// Householder QR in place, LAPACK geqrf's result: R on and above the diagonal of w ([m, n] row-major), the reflector vectors below
+// it (v[j] = 1 implied), tau[j] their scalars; reflector j is larfg's: beta = -sign(alpha) * norm(column), tau = (beta - alpha) /
+// beta, v = x / (alpha - beta), tau = 0 where the column is already zero below the diagonal.
+template <typename T>
+__global__ __launch_bounds__(kLinalgThreads) void HouseholderQrKernel(T* w, int m, int n, T* tau, int64_t tau_stride) {
+    __shared__ T part[kLinalgThreads];
+    __shared__ T red[kLinalgThreads / 64];
+    __shared__ T sh_tau, sh_scale, sh_beta;
+    const int tid = threadIdx.x;
+    const int k = m < n ? m : n;
+    for (int j = 0; j < k; ++j) {
+        T acc = T(0);
+        for (int i = j + 1 + tid; i < m; i += kLinalgThreads) {
+            const T x = w[static_cast<int64_t>(i) * n + j];
+            acc += x * x;
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) acc += __shfl_down(acc, o);
+        if ((tid & 63) == 0) red[tid >> 6] = acc;
+        __syncthreads();
+        if (tid == 0) {
+            T xnorm2 = T(0);
+            for (int g = 0; g < kLinalgThreads / 64; ++g) xnorm2 += red[g];
+            const T alpha = w[static_cast<int64_t>(j) * n + j];
+            if (xnorm2 == T(0)) {
+                sh_tau = T(0), sh_scale = T(0), sh_beta = alpha;
+            } else {
+                const T norm = SqrtT(alpha * alpha + xnorm2);
+                const T beta = alpha >= T(0) ? -norm : norm;
+                sh_tau = (beta - alpha) / beta;
+                sh_scale = T(1) / (alpha - beta);
+                sh_beta = beta;
+            }
+            tau[j * tau_stride] = sh_tau;
+        }
+        __syncthreads();
+        const T t = sh_tau;
+        if (t != T(0)) {  // uniform
+            const T scale = sh_scale;
+            for (int i = j + 1 + tid; i < m; i += kLinalgThreads) w[static_cast<int64_t>(i) * n + j] *= scale;
+            if (tid == 0) w[static_cast<int64_t>(j) * n + j] = sh_beta;
+            __syncthreads();
+            ApplyReflector(w, n, j, m, t, w, static_cast<int64_t>(n), int64_t{1}, j + 1, n, part);
+        }
+        __syncthreads();
+    }
+}
+
+// q[m, mc] = H_0 H_1 ... H_{k-1} applied to the first mc columns of the identity (LAPACK orgqr), reflectors read from w / tau.
+template <typename T>
+__global__ __launch_bounds__(kLinalgThreads) void FormQKernel(const T* w, int m, int n, const T* tau, int64_t tau_stride, T* q, int64_t q_row,
+                                                              int64_t q_col, int mc) {
+    __shared__ T part[kLinalgThreads];
+    const int tid = threadIdx.x;
+    const int k = m < n ? m : n;
+    for (int64_t e = tid; e < static_cast<int64_t>(m) * mc; e += kLinalgThreads) {
+        const int64_t i = e / mc, c = e % mc;
+        q[i * q_row + c * q_col] = i == c ? T(1) : T(0);
+    }
+    __syncthreads();
+    for (int j = k - 1; j >= 0; --j) {
+        const T t = tau[j * tau_stride];
+        if (t != T(0)) ApplyReflector(w, n, j, m, t, q, q_row, q_col, j, mc, part);  // columns before j are still the identity's
+    }
+}
+
+// r[i][c] = w[i][c] on and above the diagonal, 0 below (rows i < r_rows); or, raw, r[c][i] = w[i][c] (the column-major factored matrix)
+template <typename T>
+__global__ __launch_bounds__(256) void ExtractRKernel(const T* w, int m, int n, T* r, int64_t r_row, int64_t r_col, int r_rows, int raw) {
+    const int64_t e = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    const int64_t rows = raw ? m : r_rows;
+    if (e >= rows * n) return;
+    const int64_t i = e / n, c = e % n;
+    if (raw) r[c * r_row + i * r_col] = w[e];
+    else r[i * r_row + c * r_col] = (c >= i && i < m) ? w[i * n + c] : T(0);
+}
+
 void CheckSquare(const hipcx_array* a, const char* name) {
     ValidateArray(a, name);
     HIPCX_REQUIRE(a->ndim == 2, HIPCX_DIMENSION_ERROR, "ChainerX linear algebra routines only support 2-dimensional arrays.");
@@ -434,6 +548,76 @@ int hipcx_syevd(const hipcx_array* a, const hipcx_array* w, const hipcx_array* v
         if (a->dtype == HIPCX_FLOAT32) run(float{});
         else run(double{});
         CheckLaunch("eigh");
+    });
+}
+
+size_t hipcx_qr_workspace_size(const hipcx_array* a) {
+    if (a == nullptr || a->ndim != 2 || a->shape[0] < 0 || a->shape[1] < 0) return 0;
+    return static_cast<size_t>(a->shape[0]) * static_cast<size_t>(a->shape[1]) * 8 + 256;  // the factored copy
+}
+
+int hipcx_qr(const hipcx_array* a, const hipcx_array* q, const hipcx_array* r, const hipcx_array* tau, int mode, void* workspace,
+             size_t workspace_bytes, void* stream) {
+    return Guard([&] {
+        ValidateArray(a, "a");
+        ValidateArray(r, "r");
+        ValidateArray(tau, "tau");
+        HIPCX_REQUIRE(a->ndim == 2, HIPCX_DIMENSION_ERROR, "ChainerX linear algebra routines only support 2-dimensional arrays.");
+        HIPCX_REQUIRE(mode >= HIPCX_QR_REDUCED && mode <= HIPCX_QR_RAW, HIPCX_CHAINERX_ERROR, "Invalid QR mode");
+        const int dtype = r->dtype;
+        CheckLinalgDtype(dtype, "QR decomposition");
+        const int64_t m = a->shape[0], n = a->shape[1], k = std::min(m, n);
+        HIPCX_REQUIRE(m < (1LL << 15) && n < (1LL << 15), HIPCX_NOT_IMPLEMENTED_ERROR, "hip linear algebra: matrix too large");
+        HIPCX_REQUIRE(tau->dtype == dtype && tau->ndim == 1 && tau->shape[0] == k, HIPCX_DIMENSION_ERROR, "qr: tau must hold min(m, n) values of r's dtype");
+        const bool want_q = mode == HIPCX_QR_REDUCED || mode == HIPCX_QR_COMPLETE;
+        const int64_t mc = (mode == HIPCX_QR_COMPLETE && m > n) ? m : k;
+        const int64_t r_rows = mode == HIPCX_QR_RAW ? n : (want_q ? mc : k), r_cols = mode == HIPCX_QR_RAW ? m : n;
+        HIPCX_REQUIRE(r->ndim == 2 && r->shape[0] == r_rows && r->shape[1] == r_cols, HIPCX_DIMENSION_ERROR, "qr: r has the wrong shape for this mode");
+        if (want_q) {
+            ValidateArray(q, "q");
+            HIPCX_REQUIRE(q->dtype == dtype && q->ndim == 2 && q->shape[0] == m && q->shape[1] == mc, HIPCX_DIMENSION_ERROR,
+                          "qr: q has the wrong shape or dtype for this mode");
+        }
+        const int64_t it = ItemSize(dtype);
+        hipStream_t st = AsStream(stream);
+        if (m == 0 || n == 0) {
+            // nothing to factor; a complete q of an [m, 0] matrix is the identity
+            if (want_q && m > 0 && mc > 0) {
+                auto fill = [&](auto tag) {
+                    using T = decltype(tag);
+                    hipLaunchKernelGGL(FormQKernel<T>, dim3(1), dim3(kLinalgThreads), 0, st, static_cast<const T*>(nullptr), static_cast<int>(m), 0,
+                                       static_cast<const T*>(nullptr), int64_t{1}, static_cast<T*>(q->data), q->strides[0] / it, q->strides[1] / it,
+                                       static_cast<int>(mc));
+                };
+                if (dtype == HIPCX_FLOAT32) fill(float{});
+                else fill(double{});
+                CheckLaunch("qr");
+            }
+            return;
+        }
+        const size_t need = static_cast<size_t>(m * n * it);
+        HIPCX_REQUIRE(workspace != nullptr && workspace_bytes >= need, HIPCX_CHAINERX_ERROR, "qr workspace too small");
+        HIPCX_REQUIRE(reinterpret_cast<uintptr_t>(workspace) % 16 == 0, HIPCX_CHAINERX_ERROR, "workspace must be 16-byte aligned");
+        hipcx_array w_desc = Dense2D(workspace, dtype, m, n);
+        CopyInto(a, &w_desc, stream, "qr");  // cast + gather into the dense working copy
+        auto run = [&](auto tag) {
+            using T = decltype(tag);
+            T* w = static_cast<T*>(workspace);
+            T* tau_p = static_cast<T*>(tau->data);
+            const int64_t tau_stride = k > 1 ? tau->strides[0] / it : 1;
+            hipLaunchKernelGGL(HouseholderQrKernel<T>, dim3(1), dim3(kLinalgThreads), 0, st, w, static_cast<int>(m), static_cast<int>(n), tau_p, tau_stride);
+            if (want_q) {
+                hipLaunchKernelGGL(FormQKernel<T>, dim3(1), dim3(kLinalgThreads), 0, st, w, static_cast<int>(m), static_cast<int>(n), tau_p, tau_stride,
+                                   static_cast<T*>(q->data), q->strides[0] / it, q->strides[1] / it, static_cast<int>(mc));
+            }
+            const int raw = mode == HIPCX_QR_RAW ? 1 : 0;
+            const int64_t total = (raw ? m : r_rows) * n;
+            hipLaunchKernelGGL(ExtractRKernel<T>, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, st, w, static_cast<int>(m),
+                               static_cast<int>(n), static_cast<T*>(r->data), r->strides[0] / it, r->strides[1] / it, static_cast<int>(r_rows), raw);
+        };
+        if (dtype == HIPCX_FLOAT32) run(float{});
+        else run(double{});
+        CheckLaunch("qr");
     });
 }
 

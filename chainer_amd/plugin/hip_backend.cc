@@ -1098,7 +1098,7 @@ public:
 };
 HIPCX_REGISTER_KERNEL(AveragePoolGradKernel, HipAveragePoolGradKernel)
 
-// ---- linear algebra: Solve, Inverse, Cholesky, Syevd (the LAPACK-backed kernels of the native backend, native_device/linalg.cc) ----
+// ---- linear algebra: Solve, Inverse, Cholesky, Syevd, Qr (the LAPACK-backed kernels of the native backend, native_device/linalg.cc) ----
 namespace {
 // A zeroed device int32 for LAPACK's `info`, and the check that turns a non-zero value into the reference's ChainerxError.
 std::shared_ptr<void> NewInfoFlag(Device& device) {
@@ -1176,6 +1176,30 @@ public:
     }
 };
 HIPCX_REGISTER_KERNEL(SyevdKernel, HipSyevdKernel)
+
+class HipQrKernel : public QrKernel {
+public:
+    void Call(const Array& a, const Array& q, const Array& r, const Array& tau, QrMode mode) override {
+        Device& device = a.device();
+        device.CheckDevicesCompatible(a, q, r, tau);
+        SetDeviceScope scope{device.index()};
+        if (a.dtype() == Dtype::kFloat16) throw DtypeError{"Half-precision (float16) is not supported by QR decomposition"};
+        int code = HIPCX_QR_REDUCED;
+        switch (mode) {
+            case QrMode::kReduced: code = HIPCX_QR_REDUCED; break;
+            case QrMode::kComplete: code = HIPCX_QR_COMPLETE; break;
+            case QrMode::kR: code = HIPCX_QR_R; break;
+            case QrMode::kRaw: code = HIPCX_QR_RAW; break;
+            default: throw ChainerxError{"Invalid QR mode"};
+        }
+        hipcx_array ca = ToC(a), cq = ToC(q), cr = ToC(r), ct = ToC(tau);
+        size_t ws_bytes = hipcx_qr_workspace_size(&ca);
+        std::shared_ptr<void> ws = device.Allocate(ws_bytes);
+        const bool want_q = mode == QrMode::kReduced || mode == QrMode::kComplete;
+        Check(hipcx_qr(&ca, want_q ? &cq : nullptr, &cr, &ct, code, ws.get(), ws_bytes, nullptr));
+    }
+};
+HIPCX_REGISTER_KERNEL(QrKernel, HipQrKernel)
 
 // ---- take ----
 class HipTakeKernel : public TakeKernel {

@@ -1200,7 +1200,7 @@ def average_pool(x, ksize, stride=None, pad=0, pad_mode='ignore'):
 
 
 # ---------------------------------------------------------------------------------------------
-# linear algebra (CX/routines/linalg.cc): solve, inv, cholesky, eigh, eigvalsh
+# linear algebra (CX/routines/linalg.cc): solve, inv, cholesky, eigh, eigvalsh, qr
 # ---------------------------------------------------------------------------------------------
 def _check_square(a):
     if a.ndim != 2:
@@ -1291,6 +1291,44 @@ def eigh(a, UPLO='L'):
 def eigvalsh(a, UPLO='L'):
     """Eigvalsh (CX/routines/linalg.cc:497-511): the eigenvalues alone."""
     return _syevd(a, UPLO, False)[0]
+
+
+_QR_MODES = {'reduced': 0, 'complete': 1, 'r': 2, 'raw': 3}
+
+
+def qr(a, mode='reduced'):
+    """Qr (CX/routines/linalg.cc:333-413; mode strings CX/python/routines.cc:450-477): (q, r) for 'reduced' / 'complete', r for
+    'r', (h, tau) for 'raw' (h = the factored matrix, transposed: LAPACK's column-major result)."""
+    if a.ndim != 2:
+        raise _lib.DimensionError('ChainerX linear algebra routines only support 2-dimensional arrays.')
+    if mode not in _QR_MODES:
+        raise ValueError("mode must be 'reduced', 'complete', 'r', or 'raw'")
+    if a.dtype == numpy.dtype('float16'):
+        raise _lib.DtypeError('Half-precision (float16) is not supported by QR decomposition')
+    if _kind(a.dtype) != 3:
+        raise _lib.DtypeError('QR decomposition needs a floating-point matrix')
+    m, n = a.shape
+    k = _py.min(m, n)
+    dt = a.dtype
+    tau = ndarray.empty((k,), dt)
+    q = None
+    if mode == 'reduced':
+        q, r = ndarray.empty((m, k), dt), ndarray.empty((k, n), dt)
+    elif mode == 'complete':
+        q, r = ndarray.empty((m, m), dt), ndarray.empty((m, n), dt)
+    elif mode == 'r':
+        r = ndarray.empty((k, n), dt)
+    else:
+        r = ndarray.empty((n, m), dt)
+    nbytes = _lib.load().hipcx_qr_workspace_size(a.desc())
+    ws, wsp = _workspace(nbytes)
+    _lib.call('hipcx_qr', a.desc(), q.desc() if q is not None else None, r.desc(), tau.desc(), _QR_MODES[mode], wsp, nbytes,
+              current_stream())
+    if mode == 'r':
+        return r
+    if mode == 'raw':
+        return r, tau
+    return q, r
 
 
 # ---------------------------------------------------------------------------------------------

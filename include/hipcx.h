@@ -301,6 +301,17 @@ size_t hipcx_syevd_workspace_size(const hipcx_array* a);
 int hipcx_syevd(const hipcx_array* a, const hipcx_array* w, const hipcx_array* v, char uplo, int compute_v, void* workspace,
                 size_t workspace_bytes, void* stream);
 
+/* ---- QrKernel CX/kernels/linalg.h:38-41, modes CX/routines/linalg.h:22-28 (float32 / float64; a 2-D [m, n], cast to r's dtype) ----
+ * Householder QR with LAPACK geqrf's reflectors (beta = -sign(alpha) * norm) and orgqr's Q, as the native backend calls them
+ * (CX/native/native_device/linalg.cc:349-430): values and signs agree with it to rounding.  k = min(m, n).
+ *   HIPCX_QR_REDUCED : q [m, k], r [k, n] upper triangular          HIPCX_QR_COMPLETE : q [m, m], r [m, n]
+ *   HIPCX_QR_R       : r [k, n] alone (q ignored)                   HIPCX_QR_RAW      : r [n, m] = the factored matrix in column-major
+ * order (R and the reflector vectors), q ignored.  tau [k] receives the reflector scalars in every mode. */
+enum hipcx_qr_mode { HIPCX_QR_REDUCED = 0, HIPCX_QR_COMPLETE = 1, HIPCX_QR_R = 2, HIPCX_QR_RAW = 3 };
+size_t hipcx_qr_workspace_size(const hipcx_array* a);
+int hipcx_qr(const hipcx_array* a, const hipcx_array* q, const hipcx_array* r, const hipcx_array* tau, int mode, void* workspace,
+             size_t workspace_bytes, void* stream);
+
 /* ---- training-mode normalization: BatchNormKernel CX/kernels/normalization.h:32-47, BatchNormGradKernel :49-61 ----
  * For x C-contiguous with ndim >= 2 and `axis` = every axis but 1 (anything else: HIPCX_NOT_IMPLEMENTED_ERROR, and the caller
  * runs the reference's routine composition, CX/routines/normalization.cc:155-250).  gamma / beta / running_* / mean_out /

@@ -1199,6 +1199,15 @@ def eigvalsh(a, uplo='L'):
     return eigh(a, uplo)[0]
 
 
+def qr(a, mode='reduced'):
+    """QrKernel: LAPACK geqrf, then orgqr for 'reduced' / 'complete' (CX/native/native_device/linalg.cc:349-430; shapes per mode
+    CX/routines/linalg.cc:333-366) -- numpy.linalg.qr drives the same two routines.  Returns (q, r), r for 'r', (h, tau) for 'raw'."""
+    a = np.asarray(a)
+    if a.dtype.kind != 'f' or a.dtype == np.float16:
+        raise TypeError('qr needs float32 / float64')
+    return np.linalg.qr(a, mode=mode)
+
+
 def softmax_cross_entropy(x, t):
     """chainer/functions/loss/softmax_cross_entropy.py:123-130 (reduce='mean', normalize=True)."""
     x, t = np.asarray(x), np.asarray(t)

@@ -129,3 +129,64 @@ def test_eigh_errors_and_empty():
     with pytest.raises(TypeError):
         chx.eigh(chx.zeros((2, 2), 'float32'), None)
 
+
+@pytest.mark.parametrize('dt,tol', [('float32', 2e-5), ('float64', 1e-12)])
+def test_qr(dt, tol):
+    """Every mode against the oracle (LAPACK geqrf / orgqr): the reflector convention is LAPACK's, so values agree including signs;
+    plus the defining identities against float64."""
+    import chainer_amd as chx
+    rng = np.random.default_rng(5)
+    for m, n in ((1, 1), (2, 2), (5, 5), (7, 3), (3, 7), (1, 6), (6, 1), (64, 64), (130, 70), (70, 130), (300, 200)):
+        a = rng.standard_normal((m, n)).astype(dt)
+        k = min(m, n)
+        bound = tol * max(m, n)
+        q, r = chx.qr(chx.array(a))
+        q_ref, r_ref = O.qr(a)
+        assert q.shape == q_ref.shape and r.shape == r_ref.shape and q.dtype == np.dtype(dt) and r.dtype == np.dtype(dt)
+        q, r = q.get(), r.get()
+        assert np.array_equal(r, np.triu(r))
+        assert np.abs(q.astype(np.float64) @ r - a).max() <= bound, 'q r = a for %r' % ((m, n),)
+        assert np.abs(q.T.astype(np.float64) @ q - np.eye(k)).max() <= bound
+        assert np.abs(q - q_ref).max() <= bound * 10 and np.abs(r - r_ref).max() <= bound * 10, 'values and signs %r' % ((m, n),)
+        qc, rc = chx.qr(chx.array(a), 'complete')
+        qc_ref, rc_ref = O.qr(a, 'complete')
+        assert qc.shape == (m, m) and rc.shape == (m, n)
+        qc, rc = qc.get(), rc.get()
+        assert np.abs(qc.astype(np.float64) @ rc - a).max() <= bound
+        assert np.abs(qc.T.astype(np.float64) @ qc - np.eye(m)).max() <= bound
+        assert np.abs(qc - qc_ref).max() <= bound * 10 and np.abs(rc - rc_ref).max() <= bound * 10
+        assert np.abs(chx.qr(chx.array(a), 'r').get() - r_ref).max() <= bound * 10
+        h, tau = chx.qr(chx.array(a), 'raw')
+        h_ref, tau_ref = O.qr(a, 'raw')
+        assert h.shape == (n, m) and tau.shape == (k,)
+        assert np.abs(h.get() - h_ref).max() <= bound * 10 and np.abs(tau.get() - tau_ref).max() <= bound * 10
+    # a transposed view; columns that are already zero below the diagonal (tau = 0, no reflection)
+    a = rng.standard_normal((6, 4)).astype(dt)
+    q, r = chx.qr(chx.array(a).T)
+    q_ref, r_ref = O.qr(a.T)
+    assert_close(q.get(), q_ref, tol * 100, 'transposed view q')
+    assert_close(r.get(), r_ref, tol * 100, 'transposed view r')
+    tri = np.triu(rng.standard_normal((5, 5))).astype(dt)
+    q, r = chx.qr(chx.array(tri))
+    assert np.array_equal(q.get(), np.eye(5, dtype=dt)) and np.array_equal(r.get(), tri)
+
+
+def test_qr_errors_and_empty():
+    import chainer_amd as chx
+    for shape in ((0, 0), (0, 3), (3, 0)):
+        for mode in ('reduced', 'complete', 'r', 'raw'):
+            ref = O.qr(np.zeros(shape, 'float32'), mode)
+            got = chx.qr(chx.zeros(shape, 'float32'), mode)
+            ref = ref if isinstance(ref, tuple) else (ref,)
+            got = got if isinstance(got, tuple) else (got,)
+            for g, e in zip(got, ref):
+                assert g.shape == e.shape and np.array_equal(g.get(), e), (shape, mode)
+    with pytest.raises(ValueError):
+        chx.qr(chx.zeros((2, 2), 'float32'), 'full')
+    with pytest.raises(chx.DimensionError):
+        chx.qr(chx.zeros((2, 2, 2), 'float32'))
+    with pytest.raises(chx.DtypeError):
+        chx.qr(chx.zeros((2, 2), 'float16'))
+    with pytest.raises(chx.DtypeError):
+        chx.qr(chx.zeros((2, 2), 'int32'))
+

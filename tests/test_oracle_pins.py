@@ -888,3 +888,38 @@ def test_eigh_identities():
     with pytest.raises(TypeError):
         O.eigh(np.eye(2, dtype=np.int32))
 
+
+def test_qr_identities():
+    """qr reduces to LAPACK geqrf / orgqr through numpy; pinned by what defines the factorisation: q @ r = a, orthonormal columns,
+    r upper triangular with the shapes of each mode, and the raw form (reflector vectors + tau) rebuilding the same q by the
+    Householder product H_0 H_1 ... with H_j = I - tau_j v_j v_j^T."""
+    rng = np.random.default_rng(11)
+    for m, n in ((1, 1), (4, 4), (7, 3), (3, 7), (20, 12)):
+        a = rng.standard_normal((m, n))
+        k = min(m, n)
+        for dt, tol in (('float64', 1e-12), ('float32', 1e-5)):
+            ad = a.astype(dt)
+            q, r = O.qr(ad)
+            assert q.shape == (m, k) and r.shape == (k, n) and q.dtype == np.dtype(dt)
+            assert np.abs(q.astype(np.float64) @ r - ad).max() <= tol * 10 and np.array_equal(r, np.triu(r))
+            assert np.abs(q.T.astype(np.float64) @ q - np.eye(k)).max() <= tol * 10
+            qc, rc = O.qr(ad, 'complete')
+            assert qc.shape == (m, m) and rc.shape == (m, n)
+            assert np.abs(qc.astype(np.float64) @ rc - ad).max() <= tol * 10
+            assert np.abs(qc.T.astype(np.float64) @ qc - np.eye(m)).max() <= tol * 10
+            assert np.abs(qc[:, :k] - q).max() <= tol * 10 and np.abs(rc[:k] - r).max() <= tol * 10
+            assert np.abs(O.qr(ad, 'r') - r).max() <= tol * 10
+            h, tau = O.qr(ad, 'raw')
+            assert h.shape == (n, m) and tau.shape == (k,)
+            f = h.T.astype(np.float64)
+            assert np.abs(np.triu(f)[:k] - r).max() <= tol * 10
+            prod = np.eye(m)
+            for j in range(k):
+                v = np.zeros(m)
+                v[j] = 1
+                v[j + 1:] = f[j + 1:, j]
+                prod = prod @ (np.eye(m) - tau[j] * np.outer(v, v))
+            assert np.abs(prod[:, :k] - q).max() <= tol * 100
+    with pytest.raises(TypeError):
+        O.qr(np.eye(2, dtype=np.int64))
+
