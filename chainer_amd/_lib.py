@@ -181,6 +181,8 @@ SIGNATURES = {
     'hipcx_syevd': (_INT, [_A, _A, _A, ctypes.c_char, _INT, _V, _SZ, _V]),
     'hipcx_qr_workspace_size': (_SZ, [_A]),
     'hipcx_qr': (_INT, [_A, _A, _A, _A, _INT, _V, _SZ, _V]),
+    'hipcx_svd_workspace_size': (_SZ, [_A]),
+    'hipcx_svd': (_INT, [_A, _A, _A, _A, _INT, _INT, _V, _SZ, _V]),
     'hipcx_conv_grad_weight_workspace_size': (_SZ, [_A, _A, _A, _I64P, _I64P, _INT]),
     'hipcx_conv_grad_weight': (_INT, [_A, _A, _I64P, _I64P, _INT, _A, _V, _SZ, _V]),
     'hipcx_max_pool': (_INT, [_A, _I64P, _I64P, _I64P, _INT, _A, _V]),

@@ -388,6 +388,199 @@ __global__ __launch_bounds__(256) void ExtractRKernel(const T* w, int m, int n, 
     else r[i * r_row + c * r_col] = (c >= i && i < m) ? w[i * n + c] : T(0);
 }
 
+// Singular value decomposition by one-sided Jacobi rotations (Hestenes), one workgroup.  g: [M, N] row-major with M >= N, destroyed:
+// its columns are rotated in pairs until they are mutually orthogonal, then their norms are the singular values and the normalised
+// columns the left vectors; v: [N, N] accumulates the rotations (right vectors as columns).  Results leave in descending order of
+// the singular value: s[rank], tall(i, rank) = g[i][j] / sigma_j, sq(i, rank) = v[i][j], both addressed through (row, col)
+// element strides so that the caller decides which of u / vt each one is and how it is transposed.  Columns whose singular value
+// is zero are left for the completion kernel; *first_fill receives the number of columns that are final.
+template <typename T>
+__global__ __launch_bounds__(kLinalgThreads) void JacobiSvdKernel(T* g, int M, int N, T* v, T* sigma, int* rank, T* s_out, int64_t s_stride,
+                                                                  T* tall, int64_t tall_row, int64_t tall_col, T* sq, int64_t sq_row,
+                                                                  int64_t sq_col, int compute_uv, int* first_fill) {
+    constexpr int kGroups = kLinalgThreads / 64;
+    __shared__ T part[3 * kLinalgThreads];
+    __shared__ T cs[2 * 64];
+    __shared__ int rotated, zeros;
+    const int tid = threadIdx.x, tx = tid & 63, ty = tid >> 6;
+    const int np = N + (N & 1), half = np / 2, rounds = np - 1;
+    if (compute_uv) {
+        for (int64_t e = tid; e < static_cast<int64_t>(N) * N; e += kLinalgThreads) v[e] = (e / N == e % N) ? T(1) : T(0);
+    }
+    const T tol = SqrtT(static_cast<T>(M)) * (std::is_same<T, float>::value ? T(1.2e-7) : T(2.3e-16));
+    __syncthreads();
+    for (int sweep = 0; sweep < 60; ++sweep) {
+        if (tid == 0) rotated = 0;
+        __syncthreads();
+        for (int round = 0; round < rounds; ++round) {
+            for (int c0 = 0; c0 < half; c0 += 64) {  // uniform bounds
+                const int idx = c0 + tx;
+                int p = 0, q = -1;
+                if (idx < half) {
+                    p = idx == 0 ? rounds : (round + idx) % rounds;
+                    q = idx == 0 ? round % rounds : (round - idx + rounds) % rounds;
+                    if (p > q) { const int t2 = p; p = q; q = t2; }
+                    if (q >= N) q = -1;  // the dummy player of an odd N
+                }
+                T alpha = T(0), beta = T(0), gamma = T(0);
+                if (q >= 0) {
+                    for (int i = ty; i < M; i += kGroups) {
+                        const T a = g[static_cast<int64_t>(i) * N + p], b = g[static_cast<int64_t>(i) * N + q];
+                        alpha += a * a, beta += b * b, gamma += a * b;
+                    }
+                }
+                part[ty * 64 + tx] = alpha;
+                part[kLinalgThreads + ty * 64 + tx] = beta;
+                part[2 * kLinalgThreads + ty * 64 + tx] = gamma;
+                __syncthreads();
+                if (ty == 0) {
+                    alpha = beta = gamma = T(0);
+#pragma unroll
+                    for (int k2 = 0; k2 < kGroups; ++k2) {
+                        alpha += part[k2 * 64 + tx];
+                        beta += part[kLinalgThreads + k2 * 64 + tx];
+                        gamma += part[2 * kLinalgThreads + k2 * 64 + tx];
+                    }
+                    T c = T(1), sn = T(0);
+                    const T abs_gamma = gamma >= T(0) ? gamma : -gamma;
+                    if (q >= 0 && abs_gamma > tol * SqrtT(alpha * beta) && abs_gamma > T(0)) {
+                        const T zeta = (beta - alpha) / (T(2) * gamma);
+                        const T tt = (zeta >= T(0) ? T(1) : T(-1)) / ((zeta >= T(0) ? zeta : -zeta) + SqrtT(T(1) + zeta * zeta));
+                        c = T(1) / SqrtT(T(1) + tt * tt);
+                        sn = c * tt;
+                        rotated = 1;  // every writer stores the same value
+                    }
+                    cs[2 * tx] = c, cs[2 * tx + 1] = sn;
+                }
+                __syncthreads();
+                const T c = cs[2 * tx], sn = cs[2 * tx + 1];
+                if (q >= 0 && sn != T(0)) {
+                    for (int i = ty; i < M; i += kGroups) {
+                        T* row = g + static_cast<int64_t>(i) * N;
+                        const T a = row[p], b = row[q];
+                        row[p] = c * a - sn * b;
+                        row[q] = sn * a + c * b;
+                    }
+                    if (compute_uv) {
+                        for (int i = ty; i < N; i += kGroups) {
+                            T* row = v + static_cast<int64_t>(i) * N;
+                            const T a = row[p], b = row[q];
+                            row[p] = c * a - sn * b;
+                            row[q] = sn * a + c * b;
+                        }
+                    }
+                }
+                __syncthreads();
+            }
+        }
+        const int any = rotated;
+        __syncthreads();
+        if (!any) break;
+    }
+    // singular values: the column norms
+    for (int j = tid; j < N; j += kLinalgThreads) {
+        T acc = T(0);
+        for (int i = 0; i < M; ++i) {
+            const T x = g[static_cast<int64_t>(i) * N + j];
+            acc += x * x;
+        }
+        sigma[j] = SqrtT(acc);
+    }
+    if (tid == 0) zeros = 0;
+    __syncthreads();
+    T sigma_max = T(0);
+    for (int j = 0; j < N; ++j) sigma_max = sigma[j] > sigma_max ? sigma[j] : sigma_max;
+    const T floor_value = sigma_max * T(1e-30);
+    for (int j = tid; j < N; j += kLinalgThreads) {
+        const T sj = sigma[j];
+        int r = 0;
+        for (int l = 0; l < N; ++l) {
+            const T sl = sigma[l];
+            if (sl > sj || (sl == sj && l < j)) ++r;
+        }
+        rank[j] = r;
+        s_out[r * s_stride] = sj;
+        if (!(sj > floor_value)) atomicAdd(&zeros, 1);
+    }
+    __syncthreads();
+    if (tid == 0) *first_fill = N - zeros;
+    if (!compute_uv) return;
+    for (int64_t e = tid; e < static_cast<int64_t>(M) * N; e += kLinalgThreads) {
+        const int64_t i = e / N, j = e % N;
+        const T sj = sigma[j];
+        tall[i * tall_row + rank[j] * tall_col] = sj > floor_value ? g[e] / sj : T(0);
+    }
+    for (int64_t e = tid; e < static_cast<int64_t>(N) * N; e += kLinalgThreads) {
+        const int64_t i = e / N, j = e % N;
+        sq[i * sq_row + rank[j] * sq_col] = v[e];
+    }
+}
+
+// Columns [*first_fill, cols) of tall ([M, cols], (row, col) element strides) become an orthonormal completion of the columns
+// before them: unit vectors e_0, e_1, ... are orthogonalised against everything present (classical Gram-Schmidt, twice) and kept
+// when enough of them is left; each candidate is tried once, which always suffices (the squared residuals of all candidates add
+// up to the number of missing columns).
+template <typename T>
+__global__ __launch_bounds__(kLinalgThreads) void CompleteBasisKernel(T* tall, int64_t tall_row, int64_t tall_col, int M, int cols,
+                                                                      const int* first_fill, T* dots) {
+    __shared__ T red[kLinalgThreads / 64];
+    __shared__ T sh_norm2;
+    const int tid = threadIdx.x;
+    int cand = 0;
+    const T keep = T(1) / (T(4) * static_cast<T>(M));
+    for (int col = *first_fill; col < cols; ++col) {
+        bool done = false;
+        while (!done && cand < M) {  // uniform: cand, col and the norm are the same in every thread
+            for (int i = tid; i < M; i += kLinalgThreads) tall[i * tall_row + col * tall_col] = i == cand ? T(1) : T(0);
+            __syncthreads();
+            for (int pass = 0; pass < 2; ++pass) {
+                for (int e = tid; e < col; e += kLinalgThreads) {
+                    T acc = T(0);
+                    for (int i = 0; i < M; ++i) acc += tall[i * tall_row + e * tall_col] * tall[i * tall_row + col * tall_col];
+                    dots[e] = acc;
+                }
+                __syncthreads();
+                for (int i = tid; i < M; i += kLinalgThreads) {
+                    T acc = T(0);
+                    for (int e = 0; e < col; ++e) acc += tall[i * tall_row + e * tall_col] * dots[e];
+                    tall[i * tall_row + col * tall_col] -= acc;
+                }
+                __syncthreads();
+            }
+            T acc = T(0);
+            for (int i = tid; i < M; i += kLinalgThreads) {
+                const T x = tall[i * tall_row + col * tall_col];
+                acc += x * x;
+            }
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) acc += __shfl_down(acc, o);
+            if ((tid & 63) == 0) red[tid >> 6] = acc;
+            __syncthreads();
+            if (tid == 0) {
+                T t = T(0);
+                for (int k2 = 0; k2 < kLinalgThreads / 64; ++k2) t += red[k2];
+                sh_norm2 = t;
+            }
+            __syncthreads();
+            const T norm2 = sh_norm2;
+            if (norm2 >= keep) {
+                const T inv = T(1) / SqrtT(norm2);
+                for (int i = tid; i < M; i += kLinalgThreads) tall[i * tall_row + col * tall_col] *= inv;
+                done = true;
+            }
+            ++cand;
+            __syncthreads();
+        }
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void StridedIdentityKernel(T* out, int64_t row, int64_t col, int n) {
+    const int64_t e = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (e >= static_cast<int64_t>(n) * n) return;
+    out[(e / n) * row + (e % n) * col] = (e / n == e % n) ? T(1) : T(0);
+}
+
 void CheckSquare(const hipcx_array* a, const char* name) {
     ValidateArray(a, name);
     HIPCX_REQUIRE(a->ndim == 2, HIPCX_DIMENSION_ERROR, "ChainerX linear algebra routines only support 2-dimensional arrays.");
@@ -618,6 +811,103 @@ int hipcx_qr(const hipcx_array* a, const hipcx_array* q, const hipcx_array* r, c
         if (dtype == HIPCX_FLOAT32) run(float{});
         else run(double{});
         CheckLaunch("qr");
+    });
+}
+
+size_t hipcx_svd_workspace_size(const hipcx_array* a) {
+    if (a == nullptr || a->ndim != 2 || a->shape[0] < 0 || a->shape[1] < 0) return 0;
+    const size_t big = static_cast<size_t>(std::max(a->shape[0], a->shape[1])), small = static_cast<size_t>(std::min(a->shape[0], a->shape[1]));
+    // the working copy, the accumulated rotations, singular values + ranks + projections, the count of final columns
+    return (big * small + small * small + 2 * small + big) * 8 + 8 * 256;
+}
+
+int hipcx_svd(const hipcx_array* a, const hipcx_array* u, const hipcx_array* s, const hipcx_array* vt, int full_matrices, int compute_uv,
+              void* workspace, size_t workspace_bytes, void* stream) {
+    return Guard([&] {
+        ValidateArray(a, "a");
+        ValidateArray(s, "s");
+        HIPCX_REQUIRE(a->ndim == 2, HIPCX_DIMENSION_ERROR, "ChainerX linear algebra routines only support 2-dimensional arrays.");
+        const int dtype = a->dtype;
+        CheckLinalgDtype(dtype, "SVD");
+        const int64_t m = a->shape[0], n = a->shape[1], k = std::min(m, n);
+        HIPCX_REQUIRE(s->dtype == dtype && s->ndim == 1 && s->shape[0] == k, HIPCX_DIMENSION_ERROR, "svd: s must hold min(m, n) values of a's dtype");
+        if (compute_uv) {
+            ValidateArray(u, "u");
+            ValidateArray(vt, "vt");
+            HIPCX_REQUIRE(u->dtype == dtype && u->ndim == 2 && u->shape[0] == m && u->shape[1] == (full_matrices ? m : k), HIPCX_DIMENSION_ERROR,
+                          "svd: u has the wrong shape or dtype");
+            HIPCX_REQUIRE(vt->dtype == dtype && vt->ndim == 2 && vt->shape[1] == n && vt->shape[0] == (full_matrices ? n : k), HIPCX_DIMENSION_ERROR,
+                          "svd: vt has the wrong shape or dtype");
+        }
+        const int64_t it = ItemSize(dtype);
+        hipStream_t st = AsStream(stream);
+        if (m == 0 || n == 0) {
+            // the native backend's rule (CX/native/native_device/linalg.cc:445-452): full u and vt of an empty matrix are identities
+            if (compute_uv && full_matrices) {
+                auto fill = [&](auto tag) {
+                    using T = decltype(tag);
+                    for (const hipcx_array* o : {u, vt}) {
+                        const int64_t side = o->shape[0];
+                        if (side == 0) continue;
+                        hipLaunchKernelGGL(StridedIdentityKernel<T>, dim3(static_cast<unsigned>((side * side + 255) / 256)), dim3(256), 0, st,
+                                           static_cast<T*>(o->data), o->strides[0] / it, o->strides[1] / it, static_cast<int>(side));
+                    }
+                };
+                if (dtype == HIPCX_FLOAT32) fill(float{});
+                else fill(double{});
+                CheckLaunch("svd");
+            }
+            return;
+        }
+        const bool transposed = m < n;
+        const int64_t M = std::max(m, n), N = k;
+        HIPCX_REQUIRE(M <= 4096, HIPCX_NOT_IMPLEMENTED_ERROR, "hip svd: matrix too large for the one-workgroup Jacobi kernel");
+        HIPCX_REQUIRE(workspace != nullptr && workspace_bytes >= hipcx_svd_workspace_size(a), HIPCX_CHAINERX_ERROR, "svd workspace too small");
+        HIPCX_REQUIRE(reinterpret_cast<uintptr_t>(workspace) % 16 == 0, HIPCX_CHAINERX_ERROR, "workspace must be 16-byte aligned");
+        char* ws = static_cast<char*>(workspace);
+        size_t off = 0;
+        auto take = [&](size_t bytes) { char* p = ws + off; off += (bytes + 255) / 256 * 256; return p; };
+        // the size above counts 8 bytes per element for either dtype; its 8 * 256 bytes of slack cover the 256-alignment of each block
+        char* g_mem = take(static_cast<size_t>(M * N) * it);
+        char* v_mem = take(static_cast<size_t>(N * N) * it);
+        char* sigma_mem = take(static_cast<size_t>(N) * it);
+        char* dots_mem = take(static_cast<size_t>(M) * it);
+        char* rank_mem = take(static_cast<size_t>(N) * sizeof(int) + sizeof(int));
+        HIPCX_REQUIRE(off <= workspace_bytes, HIPCX_CHAINERX_ERROR, "svd workspace too small");
+        hipcx_array g_desc = Dense2D(g_mem, dtype, M, N);
+        hipcx_array src = *a;
+        if (transposed) {
+            std::swap(src.shape[0], src.shape[1]);
+            std::swap(src.strides[0], src.strides[1]);
+        }
+        CopyInto(&src, &g_desc, stream, "svd");
+        auto run = [&](auto tag) {
+            using T = decltype(tag);
+            T* tall = nullptr;
+            T* sq = nullptr;
+            int64_t tall_row = 0, tall_col = 0, sq_row = 0, sq_col = 0, tall_cols = N;
+            if (compute_uv) {
+                if (!transposed) {
+                    tall = static_cast<T*>(u->data), tall_row = u->strides[0] / it, tall_col = u->strides[1] / it, tall_cols = u->shape[1];
+                    sq = static_cast<T*>(vt->data), sq_row = vt->strides[1] / it, sq_col = vt->strides[0] / it;
+                } else {
+                    tall = static_cast<T*>(vt->data), tall_row = vt->strides[1] / it, tall_col = vt->strides[0] / it, tall_cols = vt->shape[0];
+                    sq = static_cast<T*>(u->data), sq_row = u->strides[0] / it, sq_col = u->strides[1] / it;
+                }
+            }
+            int* rank = reinterpret_cast<int*>(rank_mem);
+            int* first_fill = rank + N;
+            hipLaunchKernelGGL(JacobiSvdKernel<T>, dim3(1), dim3(kLinalgThreads), 0, st, reinterpret_cast<T*>(g_mem), static_cast<int>(M),
+                               static_cast<int>(N), reinterpret_cast<T*>(v_mem), reinterpret_cast<T*>(sigma_mem), rank, static_cast<T*>(s->data),
+                               k > 1 ? s->strides[0] / it : 1, tall, tall_row, tall_col, sq, sq_row, sq_col, compute_uv ? 1 : 0, first_fill);
+            if (compute_uv) {
+                hipLaunchKernelGGL(CompleteBasisKernel<T>, dim3(1), dim3(kLinalgThreads), 0, st, tall, tall_row, tall_col, static_cast<int>(M),
+                                   static_cast<int>(tall_cols), first_fill, reinterpret_cast<T*>(dots_mem));
+            }
+        };
+        if (dtype == HIPCX_FLOAT32) run(float{});
+        else run(double{});
+        CheckLaunch("svd");
     });
 }
 

@@ -1098,7 +1098,7 @@ public:
 };
 HIPCX_REGISTER_KERNEL(AveragePoolGradKernel, HipAveragePoolGradKernel)
 
-// ---- linear algebra: Solve, Inverse, Cholesky, Syevd, Qr (the LAPACK-backed kernels of the native backend, native_device/linalg.cc) ----
+// ---- linear algebra: Solve, Inverse, Cholesky, Syevd, Qr, Svd (the LAPACK-backed kernels of the native backend, native_device/linalg.cc) ----
 namespace {
 // A zeroed device int32 for LAPACK's `info`, and the check that turns a non-zero value into the reference's ChainerxError.
 std::shared_ptr<void> NewInfoFlag(Device& device) {
@@ -1200,6 +1200,23 @@ public:
     }
 };
 HIPCX_REGISTER_KERNEL(QrKernel, HipQrKernel)
+
+class HipSvdKernel : public SvdKernel {
+public:
+    void Call(const Array& a, const Array& u, const Array& s, const Array& vt, bool full_matrices, bool compute_uv) override {
+        Device& device = a.device();
+        device.CheckDevicesCompatible(a, u, s, vt);
+        SetDeviceScope scope{device.index()};
+        if (a.dtype() == Dtype::kFloat16) throw DtypeError{"Half-precision (float16) is not supported by SVD"};
+        hipcx_array ca = ToC(a), cu = ToC(u), cs = ToC(s), cvt = ToC(vt);
+        size_t ws_bytes = hipcx_svd_workspace_size(&ca);
+        std::shared_ptr<void> ws = device.Allocate(ws_bytes);
+        // without compute_uv the routine hands over placeholders of shape (0,) (routines/linalg.cc:216-218): the entry ignores them
+        Check(hipcx_svd(&ca, compute_uv ? &cu : nullptr, &cs, compute_uv ? &cvt : nullptr, full_matrices ? 1 : 0, compute_uv ? 1 : 0, ws.get(),
+                        ws_bytes, nullptr));
+    }
+};
+HIPCX_REGISTER_KERNEL(SvdKernel, HipSvdKernel)
 
 // ---- take ----
 class HipTakeKernel : public TakeKernel {

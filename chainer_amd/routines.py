@@ -1200,7 +1200,7 @@ def average_pool(x, ksize, stride=None, pad=0, pad_mode='ignore'):
 
 
 # ---------------------------------------------------------------------------------------------
-# linear algebra (CX/routines/linalg.cc): solve, inv, cholesky, eigh, eigvalsh, qr
+# linear algebra (CX/routines/linalg.cc): solve, inv, cholesky, eigh, eigvalsh, qr, svd, pinv
 # ---------------------------------------------------------------------------------------------
 def _check_square(a):
     if a.ndim != 2:
@@ -1329,6 +1329,40 @@ def qr(a, mode='reduced'):
     if mode == 'raw':
         return r, tau
     return q, r
+
+
+def svd(a, full_matrices=True, compute_uv=True):
+    """Svd (CX/routines/linalg.cc:194-301; defaults CX/python/routines.cc:429-443): (u, s, vt) with a = u @ diag(s) @ vt, s
+    descending; s alone without compute_uv."""
+    if a.ndim != 2:
+        raise _lib.DimensionError('ChainerX linear algebra routines only support 2-dimensional arrays.')
+    if a.dtype == numpy.dtype('float16'):
+        raise _lib.DtypeError('Half-precision (float16) is not supported by SVD')
+    if _kind(a.dtype) != 3:
+        raise _lib.DtypeError('SVD needs a floating-point matrix')
+    m, n = a.shape
+    k = _py.min(m, n)
+    dt = a.dtype
+    s = ndarray.empty((k,), dt)
+    u = vt = None
+    if compute_uv:
+        u = ndarray.empty((m, m if full_matrices else k), dt)
+        vt = ndarray.empty((n if full_matrices else k, n), dt)
+    nbytes = _lib.load().hipcx_svd_workspace_size(a.desc())
+    ws, wsp = _workspace(nbytes)
+    _lib.call('hipcx_svd', a.desc(), u.desc() if compute_uv else None, s.desc(), vt.desc() if compute_uv else None,
+              1 if full_matrices else 0, 1 if compute_uv else 0, wsp, nbytes, current_stream())
+    return (u, s, vt) if compute_uv else s
+
+
+def pinv(a, rcond=1e-15):
+    """PseudoInverse (CX/routines/linalg.cc:303-331): vt.T @ diag(1 / s, 0 where s <= rcond * max(s)) @ u.T from the reduced SVD."""
+    u, s, vt = svd(a, full_matrices=False, compute_uv=True)
+    if a.size == 0:
+        return copy(a.T)
+    cutoff = multiply(amax(s), float(numpy.float32(rcond)))
+    sinv = where(less_equal(s, cutoff), 0, reciprocal(s))
+    return dot(multiply(vt.T, sinv), u.T)
 
 
 # ---------------------------------------------------------------------------------------------

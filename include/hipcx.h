@@ -312,6 +312,16 @@ size_t hipcx_qr_workspace_size(const hipcx_array* a);
 int hipcx_qr(const hipcx_array* a, const hipcx_array* q, const hipcx_array* r, const hipcx_array* tau, int mode, void* workspace,
              size_t workspace_bytes, void* stream);
 
+/* ---- SvdKernel CX/kernels/linalg.h:33-36 (float32 / float64; a 2-D [m, n]; k = min(m, n)) ----
+ * a = u @ diag(s) @ vt with s descending, as LAPACK gesdd gives it to the native backend (CX/native/native_device/linalg.cc:432-503):
+ * u [m, k] and vt [k, n], or, full_matrices, u [m, m] and vt [n, n]; without compute_uv only s [k] is written (u, vt ignored).
+ * One-sided Jacobi rotations in one workgroup: singular values agree with LAPACK's to rounding; singular vectors up to a common
+ * sign of u[:, i] and vt[i, :] (and a rotation inside the space of a repeated value; the columns that complete a full u / vt, or
+ * that belong to zero singular values, are some orthonormal basis of the same space).  max(m, n) <= 4096. */
+size_t hipcx_svd_workspace_size(const hipcx_array* a);
+int hipcx_svd(const hipcx_array* a, const hipcx_array* u, const hipcx_array* s, const hipcx_array* vt, int full_matrices, int compute_uv,
+              void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---- training-mode normalization: BatchNormKernel CX/kernels/normalization.h:32-47, BatchNormGradKernel :49-61 ----
  * For x C-contiguous with ndim >= 2 and `axis` = every axis but 1 (anything else: HIPCX_NOT_IMPLEMENTED_ERROR, and the caller
  * runs the reference's routine composition, CX/routines/normalization.cc:155-250).  gamma / beta / running_* / mean_out /

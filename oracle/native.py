@@ -1208,6 +1208,27 @@ def qr(a, mode='reduced'):
     return np.linalg.qr(a, mode=mode)
 
 
+def svd(a, full_matrices=True, compute_uv=True):
+    """SvdKernel: LAPACK gesdd, job 'A' / 'S' / 'N' (CX/native/native_device/linalg.cc:432-503; shapes CX/routines/linalg.cc:194-228)
+    -- numpy.linalg.svd calls the same driver.  Full u / vt of an empty matrix are identities (:445-452)."""
+    a = np.asarray(a)
+    if a.dtype.kind != 'f' or a.dtype == np.float16:
+        raise TypeError('svd needs float32 / float64')
+    return np.linalg.svd(a, full_matrices=full_matrices, compute_uv=compute_uv)
+
+
+def pinv(a, rcond=1e-15):
+    """PseudoInverse (CX/routines/linalg.cc:303-331): from the reduced SVD, singular values <= rcond * max(s) dropped; rcond is a
+    C float in the binding (CX/python/routines.cc:444-448)."""
+    a = np.asarray(a)
+    u, s, vt = svd(a, full_matrices=False)
+    if a.size == 0:
+        return a.T.copy()
+    cutoff = (np.float32(rcond) * s.max()).astype(a.dtype)
+    sinv = np.where(s <= cutoff, 0, 1 / s).astype(a.dtype)
+    return ((vt.T * sinv) @ u.T).astype(a.dtype)
+
+
 def softmax_cross_entropy(x, t):
     """chainer/functions/loss/softmax_cross_entropy.py:123-130 (reduce='mean', normalize=True)."""
     x, t = np.asarray(x), np.asarray(t)

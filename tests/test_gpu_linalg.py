@@ -1,4 +1,4 @@
-"""Solve / Inverse / Cholesky / Eigh against the CPU oracle (LAPACK through numpy, as the native backend calls it).
+"""Solve / Inverse / Cholesky / Eigh / Qr / Svd / Pinv against the CPU oracle (LAPACK through numpy, as the native backend calls it).
 
 The device kernels use another operation order than LAPACK's blocked routines, so agreement is to rounding: errors are measured
 against the conditioning-free residuals (a @ x - b, inv(a) @ a - I, L @ L.T - a) as well as against the oracle's values."""
@@ -189,4 +189,80 @@ def test_qr_errors_and_empty():
         chx.qr(chx.zeros((2, 2), 'float16'))
     with pytest.raises(chx.DtypeError):
         chx.qr(chx.zeros((2, 2), 'int32'))
+
+
+@pytest.mark.parametrize('dt,tol', [('float32', 2e-5), ('float64', 1e-12)])
+def test_svd_pinv(dt, tol):
+    """Singular values against the oracle's (LAPACK gesdd); the factors through what defines them (reconstruction, orthonormal
+    columns / rows in every shape, full and reduced) and, for a well separated spectrum, against the oracle's up to the common sign
+    of u[:, i] and vt[i, :]; pinv against the oracle and the Moore-Penrose conditions."""
+    import chainer_amd as chx
+    rng = np.random.default_rng(6)
+    for m, n in ((1, 1), (2, 2), (5, 5), (7, 3), (3, 7), (1, 6), (6, 1), (64, 64), (130, 40), (40, 130), (200, 150)):
+        a = rng.standard_normal((m, n)).astype(dt)
+        k = min(m, n)
+        bound = tol * max(m, n)
+        s_ref = O.svd(a, compute_uv=False)
+        s_only = chx.svd(chx.array(a), compute_uv=False)
+        assert s_only.shape == (k,) and s_only.dtype == np.dtype(dt)
+        assert np.abs(s_only.get() - s_ref).max() <= bound * 4, 'singular values %r' % ((m, n),)
+        for full in (True, False):
+            u, s, vt = chx.svd(chx.array(a), full_matrices=full)
+            assert u.shape == (m, m if full else k) and s.shape == (k,) and vt.shape == (n if full else k, n)
+            u, s, vt = u.get().astype(np.float64), s.get(), vt.get().astype(np.float64)
+            assert np.array_equal(s, s_only.get()) and np.all(np.diff(s) <= 0)
+            assert np.abs((u[:, :k] * s) @ vt[:k] - a).max() <= bound * 4, 'u s vt = a %r full=%r' % ((m, n), full)
+            assert np.abs(u.T @ u - np.eye(u.shape[1])).max() <= bound * 4, 'u orthonormal %r full=%r' % ((m, n), full)
+            assert np.abs(vt @ vt.T - np.eye(vt.shape[0])).max() <= bound * 4, 'vt orthonormal %r full=%r' % ((m, n), full)
+        p = chx.pinv(chx.array(a))
+        assert p.shape == (n, m) and p.dtype == np.dtype(dt)
+        cond = s_ref[0] / s_ref[-1]
+        assert np.abs(p.get() - O.pinv(a)).max() <= bound * 10 * cond / s_ref[-1], 'pinv %r' % ((m, n),)
+    # a prescribed, well separated spectrum: vectors agree with LAPACK's up to sign; a transposed view gives the transposed factors
+    m, n, k = 9, 6, 6
+    qu, _ = np.linalg.qr(rng.standard_normal((m, m)))
+    qv, _ = np.linalg.qr(rng.standard_normal((n, n)))
+    d = np.arange(k, 0, -1).astype(np.float64)
+    a = ((qu[:, :k] * d) @ qv.T).astype(dt)
+    u, s, vt = chx.svd(chx.array(a), full_matrices=False)
+    u_ref, s_ref, vt_ref = O.svd(a, full_matrices=False)
+    assert_close(s.get(), s_ref, tol * 100, 'prescribed spectrum')
+    sign = np.sign((u.get() * u_ref).sum(0))
+    assert np.abs(u.get() * sign - u_ref).max() <= tol * 1000 and np.abs(vt.get() * sign[:, None] - vt_ref).max() <= tol * 1000
+    ut, st, vtt = chx.svd(chx.array(a).T, full_matrices=False)
+    assert_close(st.get(), s_ref, tol * 100, 'transposed view')
+    assert np.abs((ut.get().astype(np.float64) * st.get()) @ vtt.get() - a.T).max() <= tol * 100
+    # rank deficiency: zero singular values, and the factors still orthonormal (their columns come from the completion)
+    low = (rng.standard_normal((8, 2)) @ rng.standard_normal((2, 5))).astype(dt)
+    low[:, 4] = 0
+    for mat in (low, low.T.copy(), np.zeros((4, 3), dt)):
+        u, s, vt = chx.svd(chx.array(mat))
+        u, s, vt = u.get().astype(np.float64), s.get(), vt.get().astype(np.float64)
+        kk = min(mat.shape)
+        assert np.abs(s - O.svd(mat, compute_uv=False)).max() <= tol * 100
+        assert np.abs((u[:, :kk] * s) @ vt[:kk] - mat).max() <= tol * 100
+        assert np.abs(u.T @ u - np.eye(u.shape[0])).max() <= tol * 100 and np.abs(vt @ vt.T - np.eye(vt.shape[0])).max() <= tol * 100
+    # pinv drops what rcond says
+    dg = np.diag(np.array([2., 1e-3, 4.], dt))
+    assert_close(chx.pinv(chx.array(dg), rcond=1e-2).get(), O.pinv(dg, rcond=1e-2), tol * 10, 'pinv rcond')
+
+
+def test_svd_errors_and_empty():
+    import chainer_amd as chx
+    for shape in ((0, 0), (0, 3), (3, 0)):
+        for full in (True, False):
+            ref = O.svd(np.zeros(shape, 'float32'), full_matrices=full)
+            got = chx.svd(chx.zeros(shape, 'float32'), full_matrices=full)
+            for g, e in zip(got, ref):
+                assert g.shape == e.shape and np.array_equal(g.get(), e), (shape, full)
+        assert chx.svd(chx.zeros(shape, 'float32'), compute_uv=False).shape == (0,)
+        assert chx.pinv(chx.zeros(shape, 'float32')).shape == shape[::-1]
+    with pytest.raises(chx.DimensionError):
+        chx.svd(chx.zeros((2, 2, 2), 'float32'))
+    with pytest.raises(chx.DimensionError):
+        chx.pinv(chx.zeros((2,), 'float32'))
+    with pytest.raises(chx.DtypeError):
+        chx.svd(chx.zeros((2, 2), 'float16'))
+    with pytest.raises(chx.DtypeError):
+        chx.pinv(chx.zeros((2, 2), 'int64'))
 

@@ -923,3 +923,35 @@ def test_qr_identities():
     with pytest.raises(TypeError):
         O.qr(np.eye(2, dtype=np.int64))
 
+
+def test_svd_pinv_identities():
+    """svd reduces to LAPACK gesdd through numpy; pinned by a prescribed decomposition (orthogonal factors and singular values
+    chosen first, recovered afterwards), by u diag(s) vt = a with orthonormal factors in both shapes, and pinv by the four
+    Moore-Penrose conditions and by the explicit inverse of a rank-deficient diagonal matrix."""
+    rng = np.random.default_rng(12)
+    for m, n in ((1, 1), (5, 5), (8, 3), (3, 8), (20, 13)):
+        k = min(m, n)
+        qu, _ = np.linalg.qr(rng.standard_normal((m, m)))
+        qv, _ = np.linalg.qr(rng.standard_normal((n, n)))
+        d = np.sort(rng.uniform(0.5, 4.0, k))[::-1]
+        a = (qu[:, :k] * d) @ qv[:, :k].T
+        for dt, tol in (('float64', 1e-12), ('float32', 1e-5)):
+            ad = a.astype(dt)
+            assert np.abs(O.svd(ad, compute_uv=False) - d).max() <= tol * 10
+            for full in (True, False):
+                u, s, vt = O.svd(ad, full_matrices=full)
+                assert u.shape == (m, m if full else k) and s.shape == (k,) and vt.shape == (n if full else k, n)
+                assert u.dtype == np.dtype(dt) and np.all(np.diff(s) <= 0) and np.abs(s - d).max() <= tol * 10
+                assert np.abs((u[:, :k].astype(np.float64) * s) @ vt[:k] - ad).max() <= tol * 20
+                assert np.abs(u.T.astype(np.float64) @ u - np.eye(u.shape[1])).max() <= tol * 20
+                assert np.abs(vt.astype(np.float64) @ vt.T - np.eye(vt.shape[0])).max() <= tol * 20
+            p = O.pinv(ad).astype(np.float64)
+            assert p.shape == (n, m)
+            for lhs, rhs in ((a @ p @ a, a), (p @ a @ p, p), ((a @ p).T, a @ p), ((p @ a).T, p @ a)):
+                assert np.abs(lhs - rhs).max() <= tol * 200
+    assert np.array_equal(O.pinv(np.diag([2., 0., 4.])), np.diag([0.5, 0., 0.25]))
+    assert np.allclose(O.pinv(np.diag([2., 1e-3, 4.]), rcond=1e-2), np.diag([0.5, 0., 0.25]))
+    u, s, vt = O.svd(np.zeros((0, 3), 'float32'))
+    assert u.shape == (0, 0) and s.shape == (0,) and np.array_equal(vt, np.eye(3, dtype='float32'))
+    assert O.pinv(np.zeros((0, 3))).shape == (3, 0)
+
