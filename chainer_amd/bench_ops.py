@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Per-operation and per-workload measurements of the hip kernels against the MI355X rooflines.
 
-    python -m chainer_amd.bench_ops [--section sweep,mlp,cifar,resnet_layers,lstm]
+    python -m chainer_amd.bench_ops [--section sweep,mlp,cifar,resnet_layers,lstm,backward,train,linalg]
     python bench.py --ops [sections]        (the same, plus a CPU baseline column)
 
 Every figure is device time between two events recorded on the launch stream around `iters` back-to-back calls
@@ -316,6 +316,32 @@ def section_train(chx, oracle, with_cpu):
         del pd
 
 
+def section_linalg(chx, oracle, with_cpu):
+    """Dense decompositions (float32; one workgroup per matrix: functional kernels, latency-bound).  The CPU column is LAPACK through
+    numpy, which is what the native backend calls."""
+    rng = np.random.default_rng(8)
+    for n in (64, 256):
+        a = (rng.standard_normal((n, n)) + np.sqrt(n) * np.eye(n)).astype(np.float32)
+        sym = ((a + a.T) / 2).astype(np.float32)
+        spd = (a @ a.T).astype(np.float32)
+        b = rng.standard_normal((n, 8)).astype(np.float32)
+        A, S, P, B = chx.array(a), chx.array(sym), chx.array(spd), chx.array(b)
+        cases = (('solve (8 right-hand sides)', lambda: chx.solve(A, B), lambda: oracle.solve(a, b), 2 / 3 * n ** 3),
+                 ('inv', lambda: chx.inv(A), lambda: oracle.inv(a), 2.0 * n ** 3),
+                 ('cholesky', lambda: chx.cholesky(P), lambda: oracle.cholesky(spd), n ** 3 / 3),
+                 ('qr reduced', lambda: chx.qr(A), lambda: oracle.qr(a), 8 / 3 * n ** 3),
+                 ('eigh', lambda: chx.eigh(S), lambda: oracle.eigh(sym), None),
+                 ('svd full', lambda: chx.svd(A), lambda: oracle.svd(a), None))
+        for name, fn, cpu_fn, flops in cases:
+            t = device_time(fn, 3, 1)
+            row = dict(section='linalg', op=name, shape=[n, n], dtype='float32', us=round(t * 1e6, 1))
+            if flops is not None:
+                row['GFLOPs'] = round(flops / t / 1e9, 2)
+            if with_cpu:
+                row['cpu_us'] = round(cpu_time(cpu_fn) * 1e6, 1)
+            emit(**row)
+
+
 def section_copy(chx, oracle, with_cpu):
     """A plain copy of known size (128 MiB read + 128 MiB written): the calibration point for HBM traffic counters."""
     x = chx.array(np.zeros(64 * 1024 * 1024, np.float16))
@@ -323,7 +349,7 @@ def section_copy(chx, oracle, with_cpu):
     bw_row('copy', 'copy float16 [67108864]', (64 * 1024 * 1024,), t, 2 * x.nbytes)
 
 
-SECTIONS = {'copy': section_copy, 'sweep': section_sweep, 'mlp': section_mlp, 'cifar': section_cifar, 'resnet_layers': section_resnet_layers, 'lstm': section_lstm, 'backward': section_backward, 'train': section_train}
+SECTIONS = {'copy': section_copy, 'sweep': section_sweep, 'mlp': section_mlp, 'cifar': section_cifar, 'resnet_layers': section_resnet_layers, 'lstm': section_lstm, 'backward': section_backward, 'train': section_train, 'linalg': section_linalg}
 
 
 def run(sections, cpu=None):

@@ -243,8 +243,10 @@ __global__ __launch_bounds__(kLinalgThreads) void JacobiEighKernel(T* s, T* v, T
                 if (q < 0) continue;
                 const T c = cs[2 * i], sn = cs[2 * i + 1];
                 const T a = s[static_cast<int64_t>(p) * n + r], b = s[static_cast<int64_t>(q) * n + r];
-                s[static_cast<int64_t>(p) * n + r] = c * a - sn * b;
-                s[static_cast<int64_t>(q) * n + r] = sn * a + c * b;
+                // the rotated pair's own off-diagonal entry is zero by construction: storing the exact zero keeps rounding noise of the
+                // size of the eigenvalues out of the off-diagonal part, which is what lets the sweeps converge to the threshold
+                s[static_cast<int64_t>(p) * n + r] = r == q ? T(0) : c * a - sn * b;
+                s[static_cast<int64_t>(q) * n + r] = r == p ? T(0) : sn * a + c * b;
             }
             __syncthreads();
         }
