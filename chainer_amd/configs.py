@@ -226,8 +226,10 @@ class DeviceTrainOps:
     def batch_norm(self, x, gamma, beta, rm, rv):
         return self.c.batch_norm(x, gamma, beta, rm, rv, BN_EPS, 0.9)
 
-    def relu_grad(self, y, g):
-        return self.c.where(self.c.greater(y, 0), g, 0)
+    def relu_grad(self, x, g):
+        """Gradient of Relu(x) = Maximum(0, x) as the reference's backward issues it: IfLessElse(x, 0, 0, g) on the input of the
+        activation (chainerx/routines/misc.cc:34-58, 210-216), one kernel."""
+        return self.c.if_less_else(x, 0, 0, g)
 
     def onehot(self, t, n, dtype):
         return self.c.equal(t[:, None], self.c.arange(n, dtype=t.dtype)).astype(dtype)
@@ -241,12 +243,12 @@ def _unit_forward(F, x, w, bn, stride, pad, relu):
     c = F.conv(x, w, None, stride, pad)
     b, state = F.batch_norm(c, bn['gamma'], bn['beta'], bn['mean'], bn['var'])
     y = F.relu(b) if relu else b
-    return y, (x, w, bn, stride, pad, c, state, y if relu else None)
+    return y, (x, w, bn, stride, pad, c, state, b if relu else None)
 
 
 def _unit_backward(F, saved, gy, grads, need_gx=True):
-    x, w, bn, stride, pad, c, state, y = saved
-    g = F.relu_grad(y, gy) if y is not None else gy
+    x, w, bn, stride, pad, c, state, pre = saved
+    g = F.relu_grad(pre, gy) if pre is not None else gy
     gc, ggamma, gbeta = F.batch_norm_grad(c, bn['gamma'], g, state)
     grads.append((bn, 'gamma', ggamma))
     grads.append((bn, 'beta', gbeta))
@@ -271,9 +273,9 @@ def resnet50_train_step(F, p, x, t, lr=0.01):
                 sc, s4 = _unit_forward(F, h, blk['conv4'], blk['bn4'], stride, 0, False)
             else:
                 sc, s4 = h, None
-            out = F.relu(F.add(c, sc))
-            tape.append((s1, s2, s3, s4, out))
-            h = out
+            pre = F.add(c, sc)
+            h = F.relu(pre)
+            tape.append((s1, s2, s3, s4, pre))
     pooled = F.average_pool(h, h.shape[2], 1, 0, 'zero')
     feat = pooled.reshape((n, -1))
     logits = F.linear(feat, p['fc_w'], p['fc_b'])
@@ -286,8 +288,8 @@ def resnet50_train_step(F, p, x, t, lr=0.01):
     g_fc_w = F.dot(dlogits.T, feat)
     g_fc_b = F.sum(dlogits, 0)
     gh = F.average_pool_grad(h, F.dot(dlogits, p['fc_w']).reshape(pooled.shape), h.shape[2], 1, 0, 'zero')
-    for (s1, s2, s3, s4, out) in reversed(tape):
-        g = F.relu_grad(out, gh)
+    for (s1, s2, s3, s4, pre) in reversed(tape):
+        g = F.relu_grad(pre, gh)
         gb = _unit_backward(F, s3, g, grads)
         ga = _unit_backward(F, s2, gb, grads)
         gx = _unit_backward(F, s1, ga, grads)

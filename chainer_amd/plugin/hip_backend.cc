@@ -947,6 +947,22 @@ public:
             return x.device().backend().CallKernel<ConvKernel>(x, w_flipped, b, Dims{1, 1}, Dims{kh - 1 - pad[0], kw - 1 - pad[1]}, false,
                                                                out_dtype, absl::nullopt);
         }
+        if (kh == 1 && kw == 1 && pad[0] == 0 && pad[1] == 0 && GetKind(out_dtype) == DtypeKind::kFloat && x.GetTotalSize() > 0) {
+            // a 1x1 filter at any stride: every input pixel lands on one output pixel, so the result is a 1x1 forward convolution
+            // (channel axes of w swapped) scattered to every stride-th pixel of a zero-filled output
+            Array y1 = x.device().backend().CallKernel<ConvKernel>(x, w.Transpose(Axes{1, 0, 2, 3}).Copy(), absl::nullopt, Dims{1, 1},
+                                                                   Dims{0, 0}, false, out_dtype, absl::nullopt);
+            Array actual_out = Zeros(Shape{x.shape()[0], w.shape()[1], out_size[0], out_size[1]}, out_dtype, x.device());
+            // cover_all sizes: the last input row / column may fall outside the output
+            const int64_t hh = std::min(x.shape()[2], (out_size[0] + stride[0] - 1) / stride[0]);
+            const int64_t ww = std::min(x.shape()[3], (out_size[1] + stride[1] - 1) / stride[1]);
+            Array view = actual_out.At({Slice{}, Slice{}, Slice{0, hh * stride[0], stride[0]}, Slice{0, ww * stride[1], stride[1]}});
+            x.device().backend().CallKernel<CopyKernel>(y1.At({Slice{}, Slice{}, Slice{0, hh}, Slice{0, ww}}), view);
+            if (b.has_value()) {
+                actual_out += b->AsType(out_dtype, false).Reshape(Shape{1, b->shape()[0], 1, 1});
+            }
+            return actual_out;
+        }
         Array col = native::TensorDot(w, x, Axes{0}, Axes{1}, out_dtype);  // [C_out, kh, kw, N, H, W]
         Array actual_out = HipCol2Im(col.Transpose(Axes{3, 0, 1, 2, 4, 5}), stride, pad, out_size);
         if (b.has_value()) {

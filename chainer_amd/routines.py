@@ -1534,9 +1534,22 @@ def conv_transpose(x, w, b=None, stride=1, pad=0, out_size=None, out_dtype=None)
         # sums run in another order than the composition's (float accumulation, one rounding), equal to tolerance.
         w_flipped = w[:, :, ::-1, ::-1].transpose((1, 0, 2, 3)).copy()
         return conv(x, w_flipped, b, 1, (kh - 1 - pad[0], kw - 1 - pad[1]), False, dt)
+    n, ci, h, wd = x.shape
+    if not COMPOSE_CONV_TRANSPOSE and (kh, kw) == (1, 1) and pad == (0, 0) and _kind(dt) == 3 and x.size > 0:
+        # A 1x1 filter at any stride: every input pixel lands on exactly one output pixel (Col2Im adds one strided plane into
+        # zeros), so the result is a 1x1 forward convolution with the channel axes of w swapped, scattered to every stride-th
+        # pixel of a zero-filled output.
+        y1 = conv(x, w.transpose((1, 0, 2, 3)).copy(), None, 1, 0, False, dt)
+        out = zeros((n, w.shape[1]) + tuple(out_size), dt)
+        view = out[:, :, ::stride[0], ::stride[1]]
+        hh, ww = _py.min(h, view.shape[2]), _py.min(wd, view.shape[3])  # cover_all sizes: the last input row / column falls outside
+        _lib.call('hipcx_copy', y1[:, :, :hh, :ww].desc(), view[:, :, :hh, :ww].desc(), current_stream())
+        if b is not None:
+            bb = b.astype(dt, False).reshape((1, -1, 1, 1)).broadcast_to(out.shape)
+            _lib.call('hipcx_add', out.desc(), bb.desc(), out.desc(), current_stream())
+        return out
     # TensorDot(w, x) over the input channels; x goes in channels-last so that both Dot operands have the reduction index as
     # their unit-stride axis
-    n, ci, h, wd = x.shape
     w2 = w.transpose((1, 2, 3, 0)).reshape((w.shape[1] * kh * kw, ci))
     x2 = x.transpose((0, 2, 3, 1)).reshape((n * h * wd, ci))
     col = dot(w2, x2.T, dt).reshape((w.shape[1], kh, kw, n, h, wd))   # [C_out, kh, kw, N, H, W]

@@ -34,8 +34,8 @@ class OracleOps:
     batch_norm_grad = staticmethod(O.batch_norm_grad)
 
     @staticmethod
-    def relu_grad(y, g):
-        return np.where(y > 0, g, np.zeros((), g.dtype)).astype(g.dtype)
+    def relu_grad(x, g):
+        return O.if_less_else(x, 0, 0, g)
 
     @staticmethod
     def dot(a, b):
@@ -69,8 +69,8 @@ class DeviceOps:
     def batch_norm(self, x, gamma, beta, rm, rv):
         return self.c.batch_norm(x, gamma, beta, rm, rv, 2e-5, 0.9)
 
-    def relu_grad(self, y, g):
-        return self.c.where(self.c.greater(y, 0), g, 0)
+    def relu_grad(self, x, g):
+        return self.c.if_less_else(x, 0, 0, g)
 
     def onehot(self, t, n, dtype):
         return self.c.equal(t[:, None], self.c.arange(n, dtype=t.dtype)).astype(dtype)
@@ -107,12 +107,12 @@ def train_steps(F, p, x, t, steps=2, lr=0.05):
         gh = F.dot(dlogits, p['w3'])
         ga2 = gh.reshape(a2.shape)
         gr2 = F.average_pool_grad(r2, ga2, r2.shape[2], 1, 0, 'zero')
-        gc2 = F.relu_grad(r2, gr2)
+        gc2 = F.relu_grad(c2, gr2)
         gw2 = F.conv_grad_weight(p['w2'], m1, gc2, 2, 1)
         gb2 = F.sum(gc2, (0, 2, 3))
         gm1 = F.conv_transpose(gc2, p['w2'], None, 2, 1, m1.shape[2:])
         gr1 = F.max_pool_grad(r1, gm1, 2, 2, 0)
-        gb1 = F.relu_grad(r1, gr1)
+        gb1 = F.relu_grad(b1, gr1)
         gc1, ggamma, gbeta = F.batch_norm_grad(c1, p['gamma'], gb1, bn_state)
         gw1 = F.conv_grad_weight(p['w1'], x, gc1, 1, 1)
         # SGD
