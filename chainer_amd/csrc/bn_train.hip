@@ -58,26 +58,29 @@ __global__ __launch_bounds__(kBnTrainThreads) void BnStatKernel(BnStatArgs p) {
     if (MODE >= 1) m = static_cast<const C*>(p.mean)[c];
     if (MODE == 2) is = static_cast<const C*>(p.inv_std)[c];
     C a0 = C(0), a1 = C(0);
-    const int64_t lv = p.L / VEC;
-    for (int n = s; n < p.N; n += p.S) {
-        const int64_t base = (static_cast<int64_t>(n) * p.C + c) * p.L;
-        for (int64_t v = threadIdx.x; v < lv; v += kBnTrainThreads) {
-            Vec<T, VEC> xv = *reinterpret_cast<const Vec<T, VEC>*>(x + base + v * VEC);
-            Vec<T, VEC> gv;
-            if (MODE == 2) gv = *reinterpret_cast<const Vec<T, VEC>*>(g + base + v * VEC);
+    // The slice's images n = s, s + S, ... times the plane's vectors form one index space shared out over the threads, so that
+    // planes shorter than the workgroup (14x14, 7x7) keep every lane busy.  32-bit index arithmetic: the host checks N * L < 2^31.
+    const uint32_t lv = static_cast<uint32_t>(p.L / VEC);
+    const uint32_t images = static_cast<uint32_t>((p.N - s + p.S - 1) / p.S);
+    const uint32_t items = images * lv;
+    for (uint32_t idx = threadIdx.x; idx < items; idx += kBnTrainThreads) {
+        const uint32_t j = idx / lv, v = idx - j * lv;
+        const int64_t base = (static_cast<int64_t>(s + j * p.S) * p.C + c) * p.L + static_cast<int64_t>(v) * VEC;
+        Vec<T, VEC> xv = *reinterpret_cast<const Vec<T, VEC>*>(x + base);
+        Vec<T, VEC> gv;
+        if (MODE == 2) gv = *reinterpret_cast<const Vec<T, VEC>*>(g + base);
 #pragma unroll
-            for (int e = 0; e < VEC; ++e) {
-                C xe = static_cast<C>(xv.v[e]);
-                if (MODE == 0) {
-                    a0 += xe;
-                } else if (MODE == 1) {
-                    C d = xe - m;
-                    a0 += d * d;
-                } else {
-                    C ge = static_cast<C>(gv.v[e]);
-                    a0 += ge;
-                    a1 += ge * ((xe - m) * is);
-                }
+        for (int e = 0; e < VEC; ++e) {
+            C xe = static_cast<C>(xv.v[e]);
+            if (MODE == 0) {
+                a0 += xe;
+            } else if (MODE == 1) {
+                C d = xe - m;
+                a0 += d * d;
+            } else {
+                C ge = static_cast<C>(gv.v[e]);
+                a0 += ge;
+                a1 += ge * ((xe - m) * is);
             }
         }
     }
@@ -182,29 +185,56 @@ __global__ __launch_bounds__(256) void BnApplyKernel(BnApplyArgs p) {
     const T* g = static_cast<const T*>(p.g);
     T* out = static_cast<T*>(p.out);
     const int64_t nvec = p.total / VEC;
-    const int64_t lv = p.L / VEC;
     const C inv_n = static_cast<C>(1.0 / p.count);
+    // The array is one contiguous run of [N][C] planes of L elements, cut into vectors without regard to the planes: when VEC does
+    // not divide L a vector can hold the end of one plane and the start of the next (never more: the host keeps VEC <= L), and
+    // its elements pick the constants of their own channel.  32-bit index arithmetic: the host checks total < 2^31.
+    const uint32_t L = static_cast<uint32_t>(p.L);
+    const bool planes_split = (L % VEC) != 0;
     for (int64_t v = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; v < nvec; v += static_cast<int64_t>(gridDim.x) * blockDim.x) {
-        const int c = static_cast<int>((v / lv) % p.C);
+        const uint32_t first = static_cast<uint32_t>(v) * VEC;
+        const uint32_t plane = first / L;
+        const uint32_t within = first - plane * L;
+        const int c = static_cast<int>(plane % static_cast<uint32_t>(p.C));
+        const int c2 = c + 1 == p.C ? 0 : c + 1;
+        const bool split = planes_split && within + VEC > L;
+        const int split_at = split ? static_cast<int>(L - within) : VEC;  // elements from split_at on belong to channel c2
         const C m = static_cast<const C*>(p.mean)[c];
         const C is = static_cast<const C*>(p.inv_std)[c];
         const C ga = static_cast<C>(static_cast<const T*>(p.gamma)[c * p.gamma_stride]);
+        C m2 = m, is2 = is, ga2 = ga;
+        if (split) {
+            m2 = static_cast<const C*>(p.mean)[c2];
+            is2 = static_cast<const C*>(p.inv_std)[c2];
+            ga2 = static_cast<C>(static_cast<const T*>(p.gamma)[c2 * p.gamma_stride]);
+        }
         Vec<T, VEC> xv = *reinterpret_cast<const Vec<T, VEC>*>(x + v * VEC);
         Vec<T, VEC> o;
         if constexpr (GRAD) {
             const C* part = static_cast<const C*>(p.partial) + static_cast<int64_t>(c) * p.S * 2;
             const C gbeta = part[0], ggamma = part[1];
+            C gbeta2 = gbeta, ggamma2 = ggamma;
+            if (split) {
+                const C* part2 = static_cast<const C*>(p.partial) + static_cast<int64_t>(c2) * p.S * 2;
+                gbeta2 = part2[0], ggamma2 = part2[1];
+            }
             Vec<T, VEC> gv = *reinterpret_cast<const Vec<T, VEC>*>(g + v * VEC);
-            const C scale = ga * is;
+            const C scale = ga * is, scale2 = ga2 * is2;
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
-                C x_hat = (static_cast<C>(xv.v[e]) - m) * is;
-                o.v[e] = static_cast<T>(scale * (static_cast<C>(gv.v[e]) - (x_hat * ggamma + gbeta) * inv_n));
+                const bool second = e >= split_at;
+                C x_hat = (static_cast<C>(xv.v[e]) - (second ? m2 : m)) * (second ? is2 : is);
+                o.v[e] = static_cast<T>((second ? scale2 : scale) *
+                                        (static_cast<C>(gv.v[e]) - (x_hat * (second ? ggamma2 : ggamma) + (second ? gbeta2 : gbeta)) * inv_n));
             }
         } else {
             const C be = static_cast<C>(static_cast<const T*>(p.beta)[c * p.beta_stride]);
+            const C be2 = split ? static_cast<C>(static_cast<const T*>(p.beta)[c2 * p.beta_stride]) : be;
 #pragma unroll
-            for (int e = 0; e < VEC; ++e) o.v[e] = static_cast<T>(((static_cast<C>(xv.v[e]) - m) * is) * ga + be);
+            for (int e = 0; e < VEC; ++e) {
+                const bool second = e >= split_at;
+                o.v[e] = static_cast<T>(((static_cast<C>(xv.v[e]) - (second ? m2 : m)) * (second ? is2 : is)) * (second ? ga2 : ga) + (second ? be2 : be));
+            }
         }
         *reinterpret_cast<Vec<T, VEC>*>(out + v * VEC) = o;
     }
@@ -262,12 +292,37 @@ int64_t ChannelStride(const hipcx_array* a, const hipcx_array* x, const char* na
     return a->strides[1] / it;
 }
 
+// Widths of the two kernel families.  The statistics kernels read whole planes of one channel, so their vectors must divide the
+// plane (16, 8 or one element's bytes); the element-wise kernels cut the contiguous array into 16-byte vectors wherever the planes
+// fall, as long as a vector is not longer than a plane.
+struct BnWidths {
+    int stat;    // elements per vector in the statistics kernels: full, half or 1
+    bool apply;  // full vectors in the element-wise kernels
+};
+
+BnWidths PickWidths(int64_t L, int64_t total, int64_t item, std::initializer_list<const void*> pointers) {
+    const int64_t full = 16 / item;
+    auto aligned = [&](int64_t bytes) {
+        for (const void* ptr : pointers) {
+            if (ptr != nullptr && reinterpret_cast<uintptr_t>(ptr) % bytes != 0) return false;
+        }
+        return true;
+    };
+    BnWidths w{1, false};
+    if (L % full == 0 && aligned(16)) w.stat = static_cast<int>(full);
+    else if (full >= 4 && L % (full / 2) == 0 && aligned(8)) w.stat = static_cast<int>(full / 2);
+    w.apply = total % full == 0 && L >= full && aligned(16);
+    return w;
+}
+
 template <typename T, int MODE>
-void LaunchStat(const BnStatArgs& a, bool vec, hipStream_t stream) {
+void LaunchStat(const BnStatArgs& a, int width, hipStream_t stream) {
     constexpr int VEC = 16 / sizeof(T);
     dim3 grid(static_cast<unsigned>(a.C), static_cast<unsigned>(a.S));
-    if (vec) {
+    if (width == VEC) {
         hipLaunchKernelGGL((BnStatKernel<T, MODE, VEC>), grid, dim3(kBnTrainThreads), 0, stream, a);
+    } else if (VEC >= 4 && width == VEC / 2) {
+        hipLaunchKernelGGL((BnStatKernel<T, MODE, (VEC >= 4 ? VEC / 2 : 1)>), grid, dim3(kBnTrainThreads), 0, stream, a);
     } else {
         hipLaunchKernelGGL((BnStatKernel<T, MODE, 1>), grid, dim3(kBnTrainThreads), 0, stream, a);
     }
@@ -338,8 +393,8 @@ int hipcx_batch_norm(const hipcx_array* x, const hipcx_array* gamma, const hipcx
         void* inv_c = ws + vec_bytes;
         void* partial = ws + 2 * vec_bytes;
         hipStream_t st = AsStream(stream);
-        const bool vec = (g.L * ItemSize(x->dtype)) % 16 == 0 && reinterpret_cast<uintptr_t>(x->data) % 16 == 0 &&
-                         reinterpret_cast<uintptr_t>(out->data) % 16 == 0;
+        HIPCX_REQUIRE(total < (int64_t{1} << 31), HIPCX_NOT_IMPLEMENTED_ERROR, "hip batch_norm: array too large for the dedicated kernels");
+        const BnWidths widths = PickWidths(g.L, total, ItemSize(x->dtype), {x->data, out->data});
         BnStatArgs s{};
         s.x = x->data;
         s.mean = mean_c;
@@ -368,12 +423,12 @@ int hipcx_batch_norm(const hipcx_array* x, const hipcx_array* gamma, const hipcx
         const unsigned cblocks = static_cast<unsigned>((g.C + 255) / 256);
         VisitFloatDtype(x->dtype, [&](auto tag) {
             using T = typename decltype(tag)::type;
-            LaunchStat<T, 0>(s, vec, st);
+            LaunchStat<T, 0>(s, widths.stat, st);
             hipLaunchKernelGGL((BnFinishKernel<T, 0>), dim3(cblocks), dim3(256), 0, st, f);
-            LaunchStat<T, 1>(s, vec, st);
+            LaunchStat<T, 1>(s, widths.stat, st);
             hipLaunchKernelGGL((BnFinishKernel<T, 1>), dim3(cblocks), dim3(256), 0, st, f);
             CheckLaunch("batch_norm finish");
-            LaunchApply<T, false>(a, vec, st);
+            LaunchApply<T, false>(a, widths.apply, st);
         });
     });
 }
@@ -404,8 +459,8 @@ int hipcx_batch_norm_grad(const hipcx_array* x, const hipcx_array* gamma, const 
         void* inv_c = ws + vec_bytes;
         void* partial = ws + 2 * vec_bytes;
         hipStream_t st = AsStream(stream);
-        const bool vec = (g.L * ItemSize(x->dtype)) % 16 == 0 && reinterpret_cast<uintptr_t>(x->data) % 16 == 0 &&
-                         reinterpret_cast<uintptr_t>(gout->data) % 16 == 0 && reinterpret_cast<uintptr_t>(gx->data) % 16 == 0;
+        HIPCX_REQUIRE(total < (int64_t{1} << 31), HIPCX_NOT_IMPLEMENTED_ERROR, "hip batch_norm_grad: array too large for the dedicated kernels");
+        const BnWidths widths = PickWidths(g.L, total, ItemSize(x->dtype), {x->data, gout->data, gx->data});
         // the state arrives in the array dtype: widen it into the workspace vectors the kernels read
         hipcx_array mc{}, ic{};
         const int cdtype = x->dtype == HIPCX_FLOAT64 ? HIPCX_FLOAT64 : HIPCX_FLOAT32;
@@ -439,10 +494,10 @@ int hipcx_batch_norm_grad(const hipcx_array* x, const hipcx_array* gamma, const 
         const unsigned cblocks = static_cast<unsigned>((g.C + 255) / 256);
         VisitFloatDtype(x->dtype, [&](auto tag) {
             using T = typename decltype(tag)::type;
-            LaunchStat<T, 2>(s, vec, st);
+            LaunchStat<T, 2>(s, widths.stat, st);
             hipLaunchKernelGGL((BnGradFinishKernel<T>), dim3(cblocks), dim3(256), 0, st, a);
             CheckLaunch("batch_norm_grad finish");
-            LaunchApply<T, true>(a, vec, st);
+            LaunchApply<T, true>(a, widths.apply, st);
         });
     });
 }

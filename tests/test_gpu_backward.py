@@ -220,7 +220,8 @@ def test_batch_norm_kernels_against_the_composition(dt, tol):
     import chainer_amd as chx
     from chainer_amd import routines
     rng = np.random.default_rng(71)
-    shapes = [(8, 16, 14, 14), (4, 3, 7, 7), (1, 5, 6, 4), (6, 1, 3, 3), (32, 10), (2, 4, 3, 5, 2)]
+    shapes = [(8, 16, 14, 14), (4, 3, 7, 7), (1, 5, 6, 4), (6, 1, 3, 3), (32, 10), (2, 4, 3, 5, 2), (16, 8, 7, 7), (3, 24, 14, 14),
+              (5, 7, 3, 3)]
     if dt != 'float16':
         # 50176 elements per channel: the float16 composition (like the native backend) overflows its Sum of squares there and
         # returns inf statistics, while the kernel accumulates in float -- a case where the two differ on purpose
