@@ -66,7 +66,8 @@ void LaunchShape(IGemmArgs<T> p, bool fast16, bool fast8, hipStream_t stream) {
     double x_elems = static_cast<double>(p.N) * (p.xsN > 0 ? p.xsN : 1);
     bool fits32 = x_elems < 2147483647.0 && static_cast<double>(p.K) * p.wsK < 2147483647.0;
     static const bool use_pipe = [] { const char* e = getenv("HIPCX_IGEMM_PIPE"); return e != nullptr && e[0] == '1'; }();
-    if ((fast16 || fast8) && fits32 && use_pipe) {
+    HIPCX_REQUIRE(p.batch == 0 || ((fast16 || fast8) && !PM), HIPCX_NOT_IMPLEMENTED_ERROR, "batched products need operands in the MFMA layout");
+    if ((fast16 || fast8) && fits32 && use_pipe && p.batch == 0) {
         constexpr int lds_bytes = PipeLdsBytes<T, WM, WN, PM>();
         if (fast16) {
             auto kern = IGemmPipeKernel<T, WM, WN, 16, PM>;
@@ -979,6 +980,64 @@ int PlanSplitK(int64_t m, int64_t n, int64_t k, int dtype) {
 }
 size_t SplitKBytes(int64_t m, int64_t n, int slices) { return slices > 1 ? static_cast<size_t>(slices) * m * n * sizeof(float) : 0; }
 }  // namespace
+
+// out[m][n] = sum over b < batch, k < depth of a[b][m][k] * bt[b][n][k]: one matrix product per batch entry, accumulated.  Rows of a_b
+// and bt_b are dense along k; a_row / bt_row are their row strides and a_slice / bt_slice the distances between batch entries, in
+// elements.  out is row-major [m][n].  Float partial sums go to `partial` when BatchedProductSlices(...) > 1
+// (BatchedProductPartialBytes bytes).  float16 / float32; the operands must satisfy the MFMA kernel's 8-byte granularity.
+int BatchedProductSlices(int64_t m, int64_t n, int64_t depth, int batch, int dtype) {
+    const int64_t it = ItemSize(dtype);
+    const int64_t steps_per = (depth * it + 127) / 128;
+    const int planned = PlanSplitK(m, n, depth * batch, dtype);
+    const int64_t steps = steps_per * batch;
+    return planned > steps ? static_cast<int>(steps) : planned;
+}
+
+size_t BatchedProductPartialBytes(int64_t m, int64_t n, int64_t depth, int batch, int dtype) {
+    return SplitKBytes(m, n, BatchedProductSlices(m, n, depth, batch, dtype));
+}
+
+bool BatchedProductApplies(const void* a, int64_t a_row, int64_t a_slice, const void* bt, int64_t bt_row, int64_t bt_slice, int64_t depth,
+                           const void* out, int dtype) {
+    if (dtype != HIPCX_FLOAT16 && dtype != HIPCX_FLOAT32) return false;
+    const int64_t epc = 16 / ItemSize(dtype);  // 16-byte granules throughout
+    return depth % epc == 0 && a_row % epc == 0 && a_slice % epc == 0 && bt_row % epc == 0 && bt_slice % epc == 0 && Aligned(a, 16) &&
+           Aligned(bt, 16) && Aligned(out, 16);
+}
+
+void LaunchBatchedProduct(int dtype, const void* a, int64_t a_row, int64_t a_slice, const void* bt, int64_t bt_row, int64_t bt_slice, int64_t m,
+                          int64_t n, int64_t depth, int batch, void* out, float* partial, hipStream_t stream) {
+    auto run = [&](auto tag) {
+        using T = decltype(tag);
+        IGemmArgs<T> p{};
+        p.x = static_cast<const T*>(a);
+        p.w = static_cast<const T*>(bt);
+        p.out = static_cast<T*>(out);
+        p.N = static_cast<int>(m);
+        p.C = static_cast<int>(depth);
+        p.H = p.W = 1;
+        p.K = static_cast<int>(n);
+        p.R = p.S = 1;
+        p.OH = p.OW = 1;
+        p.stride_h = p.stride_w = 1;
+        p.xsN = a_row, p.xsC = 1;
+        p.wsK = bt_row, p.wsC = 1;
+        p.wsR = p.wsS = depth;
+        p.osN = n, p.osC = 1;
+        p.M = m;
+        p.Kg = static_cast<int>(depth);
+        p.batch = batch;
+        p.x_slice = a_slice, p.w_slice = bt_slice;
+        p.ksplit = partial != nullptr ? BatchedProductSlices(m, n, depth, batch, dtype) : 1;
+        p.partial = p.ksplit > 1 ? partial : nullptr;
+        // the work accounting of the launch sees the whole reduction
+        p.C_logical = static_cast<int>(std::min<int64_t>(depth * batch, 0x7fffffff));
+        p.H_logical = p.W_logical = 1;
+        LaunchIGemmImpl(p, stream);
+    };
+    if (dtype == HIPCX_FLOAT16) run(half_t{});
+    else run(float{});
+}
 
 extern "C" {
 

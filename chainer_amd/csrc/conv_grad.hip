@@ -171,6 +171,30 @@ void RunLayouts(const GradWeightArgs& a, hipStream_t stream) {
 
 using namespace hipcx;
 
+// conv.hip: accumulated batch of matrix products on the MFMA kernel
+int BatchedProductSlices(int64_t m, int64_t n, int64_t depth, int batch, int dtype);
+size_t BatchedProductPartialBytes(int64_t m, int64_t n, int64_t depth, int batch, int dtype);
+bool BatchedProductApplies(const void* a, int64_t a_row, int64_t a_slice, const void* bt, int64_t bt_row, int64_t bt_slice, int64_t depth,
+                           const void* out, int dtype);
+void LaunchBatchedProduct(int dtype, const void* a, int64_t a_row, int64_t a_slice, const void* bt, int64_t bt_row, int64_t bt_slice, int64_t m,
+                          int64_t n, int64_t depth, int batch, void* out, float* partial, hipStream_t stream);
+
+namespace {
+// A 1x1 filter at stride 1 without padding: gw[k][c] = sum over images of gy_n [K, pixels] @ x_n [C, pixels]^T, which the MFMA kernel
+// reads from gy and x where they lie (rows along the pixels, one matrix per image) -- no Im2Col, no transposed copy of gy.
+// Taken when the planes are whole 16-byte granules and long enough to fill reduction steps (14x14 planes in float16 are 8-byte
+// granules and 3 1/16 steps long: measured no faster than the Im2Col route).
+bool DirectPointwise(const GradWeightPlan& pl, const hipcx_array* x, const hipcx_array* gy, const hipcx_array* gw) {
+    static const bool enabled = [] { const char* e = getenv("HIPCX_GRAD_WEIGHT_DIRECT"); return e == nullptr || e[0] != '0'; }();
+    const GradWeightArgs& a = pl.a;
+    if (!enabled || a.kh != 1 || a.kw != 1 || a.sh != 1 || a.sw != 1 || a.ph != 0 || a.pw != 0 || a.OH != a.H || a.OW != a.W) return false;
+    const int64_t pixels = static_cast<int64_t>(a.H) * a.W;
+    if (pixels < 256 || a.N < 1) return false;
+    return BatchedProductApplies(gy->data, pixels, static_cast<int64_t>(a.K) * pixels, x->data, pixels, static_cast<int64_t>(a.C) * pixels, pixels,
+                                 gw->data, gw->dtype);
+}
+}  // namespace
+
 extern "C" {
 
 size_t hipcx_conv_grad_weight_workspace_size(const hipcx_array* x, const hipcx_array* gy, const hipcx_array* gw, const int64_t* stride,
@@ -179,6 +203,9 @@ size_t hipcx_conv_grad_weight_workspace_size(const hipcx_array* x, const hipcx_a
         if (x == nullptr || gy == nullptr || gw == nullptr) return 0;
         GradWeightPlan pl = PlanGradWeight(x, gy, gw, stride, pad, cover_all);
         hipcx_array out = GwAsMatrix(gw);
+        if (DirectPointwise(pl, x, gy, gw)) {
+            return BatchedProductPartialBytes(pl.a.K, pl.a.C, static_cast<int64_t>(pl.a.H) * pl.a.W, pl.a.N, gw->dtype) + 256;
+        }
         return pl.col_bytes + pl.gyt_bytes + hipcx_dot_workspace_size(&pl.gy_t, &pl.col_view, &out);
     } catch (...) {
         return 0;
@@ -195,6 +222,17 @@ int hipcx_conv_grad_weight(const hipcx_array* x, const hipcx_array* gy, const in
             hipcx_scalar zero{HIPCX_KIND_INT, 0, 0, 0.0};
             int rc = hipcx_fill(gw, zero, stream);
             HIPCX_REQUIRE(rc == HIPCX_OK, rc, hipcx_last_error());
+            return;
+        }
+        if (DirectPointwise(pl, x, gy, gw)) {
+            const int64_t pixels = static_cast<int64_t>(pl.a.H) * pl.a.W;
+            const size_t partial_bytes = BatchedProductPartialBytes(pl.a.K, pl.a.C, pixels, pl.a.N, gw->dtype);
+            HIPCX_REQUIRE(partial_bytes == 0 || (workspace != nullptr && workspace_bytes >= partial_bytes), HIPCX_CHAINERX_ERROR,
+                          "conv_grad_weight workspace too small: need " + std::to_string(partial_bytes) + " bytes");
+            HIPCX_REQUIRE(reinterpret_cast<uintptr_t>(workspace) % 16 == 0, HIPCX_CHAINERX_ERROR, "workspace must be 16-byte aligned");
+            LaunchBatchedProduct(gw->dtype, gy->data, pixels, static_cast<int64_t>(pl.a.K) * pixels, x->data, pixels,
+                                 static_cast<int64_t>(pl.a.C) * pixels, pl.a.K, pl.a.C, pixels, pl.a.N, gw->data,
+                                 partial_bytes ? static_cast<float*>(workspace) : nullptr, AsStream(stream));
             return;
         }
         const size_t dot_bytes = hipcx_dot_workspace_size(&pl.gy_t, &pl.col_view, &out);

@@ -43,6 +43,11 @@ struct IGemmArgs {
     // the reduction steps, each storing float partial sums [ksplit][M][K]; SplitKReduceKernel adds them up.  0 or 1: off.
     int ksplit;
     float* partial;
+    // Batched reduction (fast kernel only): out = sum over b < batch of x_b @ w_b^T with x_b = x + b * x_slice and
+    // w_b = w + b * w_slice (elements).  The reduction steps of all batches form one sequence, which is what ksplit slices.
+    // 0: off.  Weight gradients of 1x1 convolutions read gy and x in place this way (one [channels, pixels] matrix per image).
+    int batch;
+    int64_t x_slice, w_slice;
 };
 
 constexpr int kRowBytes = 128;           // bytes of the reduction axis per tile row
@@ -331,6 +336,13 @@ __global__ __launch_bounds__(64 * WM * WN) void IGemmFastKernel(IGemmArgs<T> p) 
 
     Chunk xreg[XCH], wreg[WCH];
     auto load_tile = [&](int kt) {
+        int64_t x_off = 0, w_off = 0;
+        if (p.batch > 0) {
+            const int b = kt / nk;
+            kt -= b * nk;
+            x_off = b * p.x_slice;
+            w_off = b * p.w_slice;
+        }
         const int kbase = kt * BKE;
         const int kk = kbase + kc * EPC;
         const bool kvalid = kk < p.Kg;
@@ -356,13 +368,13 @@ __global__ __launch_bounds__(64 * WM * WN) void IGemmFastKernel(IGemmArgs<T> p) 
             int iw = iw0[i] + s;
             bool ok = kvalid && ih >= 0 && ih < p.H && iw >= 0 && iw < p.W;
             Chunk v = Chunk(0);
-            if (ok) v = *reinterpret_cast<const Chunk*>(p.x + xbase[i] + ih * p.xsH + iw * p.xsW + c);
+            if (ok) v = *reinterpret_cast<const Chunk*>(p.x + x_off + xbase[i] + ih * p.xsH + iw * p.xsW + c);
             xreg[i] = v;
         }
 #pragma unroll
         for (int i = 0; i < WCH; ++i) {
             Chunk v = Chunk(0);
-            if (kvalid && wvalid[i]) v = *reinterpret_cast<const Chunk*>(wrow[i] + kk);
+            if (kvalid && wvalid[i]) v = *reinterpret_cast<const Chunk*>(wrow[i] + w_off + kk);
             wreg[i] = v;
         }
     };
@@ -387,10 +399,11 @@ __global__ __launch_bounds__(64 * WM * WN) void IGemmFastKernel(IGemmArgs<T> p) 
         }
     }
 
-    int kt_begin = 0, kt_end = nk;
+    const int steps = p.batch > 0 ? nk * p.batch : nk;
+    int kt_begin = 0, kt_end = steps;
     if (p.ksplit > 1) {
-        kt_begin = static_cast<int>(static_cast<int64_t>(nk) * blockIdx.y / p.ksplit);
-        kt_end = static_cast<int>(static_cast<int64_t>(nk) * (blockIdx.y + 1) / p.ksplit);
+        kt_begin = static_cast<int>(static_cast<int64_t>(steps) * blockIdx.y / p.ksplit);
+        kt_end = static_cast<int>(static_cast<int64_t>(steps) * (blockIdx.y + 1) / p.ksplit);
     }
     if (kt_begin < kt_end) load_tile(kt_begin);
     for (int kt = kt_begin; kt < kt_end; ++kt) {

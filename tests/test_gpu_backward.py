@@ -18,6 +18,10 @@ CONV_CASES = [  # N, C, H, W, K, kh, kw, stride, pad, cover_all
     (4, 8, 12, 12, 16, 1, 1, 2, 0, False),
     # 1x1 filters at a stride: ConvTranspose runs as a 1x1 convolution scattered into a zero-filled output
     (2, 16, 13, 9, 8, 1, 1, (2, 3), 0, False), (2, 8, 10, 10, 8, 1, 1, 2, 0, True), (2, 256, 14, 14, 512, 1, 1, 2, 0, False),
+    # 1x1 filters at stride 1 on planes of whole 16-byte granules: ConvGradWeight reads gy and x in place, one matrix product per
+    # image accumulated (one slice; a split reduction; a last reduction step that is partly past the plane; float32-only granules)
+    (3, 32, 16, 16, 48, 1, 1, 1, 0, False), (16, 64, 28, 28, 256, 1, 1, 1, 0, False), (2, 200, 28, 28, 72, 1, 1, 1, 0, False),
+    (2, 24, 18, 18, 40, 1, 1, 1, 0, False),
     # stride 1: ConvTranspose runs as a forward convolution with flipped filters (padding k - 1 - p)
     (2, 6, 7, 9, 10, 2, 3, 1, (0, 1), False), (2, 8, 9, 9, 12, 5, 5, 1, 2, False), (2, 16, 6, 6, 16, 3, 3, 1, 0, False),
     (4, 64, 14, 14, 128, 3, 3, 1, 1, False), (2, 128, 7, 7, 256, 1, 1, 1, 0, False), (2, 5, 6, 6, 7, 3, 3, 1, 2, False),
