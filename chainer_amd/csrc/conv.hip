@@ -97,7 +97,7 @@ void LaunchShape(IGemmArgs<T> p, bool fast16, bool fast8, hipStream_t stream) {
     }
     CheckLaunch("igemm");
     if (p.ksplit > 1) {
-        int64_t blocks = (p.M * p.K + 255) / 256;
+        int64_t blocks = (p.M * p.K + 63) / 64;  // 64 outputs per workgroup
         int64_t cap = static_cast<int64_t>(NumCUs()) * 16;
         hipLaunchKernelGGL((SplitKReduceKernel<T>), dim3(static_cast<unsigned>(blocks > cap ? cap : blocks)), dim3(256), 0, stream, p);
         CheckLaunch("igemm split reduction");
@@ -975,7 +975,8 @@ int PlanSplitK(int64_t m, int64_t n, int64_t k, int dtype) {
     if (k < 4096 || tiles * 2 > NumCUs() || m * n < 64 * 64 || steps < 16) return 1;
     int64_t s = (2 * NumCUs() + tiles - 1) / tiles;
     if (s > steps / 24) s = steps / 24;  // a slice of fewer steps costs more in partial sums than it gains
-    if (s > 64) s = 64;
+    static const int64_t max_slices = [] { const char* e = getenv("HIPCX_DOT_SPLITK_MAX"); int v = e ? atoi(e) : 0; return v >= 2 && v <= 1024 ? v : 64; }();
+    if (s > max_slices) s = max_slices;
     return s < 2 ? 1 : static_cast<int>(s);
 }
 size_t SplitKBytes(int64_t m, int64_t n, int slices) { return slices > 1 ? static_cast<size_t>(slices) * m * n * sizeof(float) : 0; }

@@ -209,14 +209,34 @@ __device__ __forceinline__ void StorePartial(const IGemmArgs<T>& p, int m0, int 
 // out[m][n] = sum over slices of partial[slice][m][n] (+ bias), for outputs addressed as out + m * osN + n * osC (matrix products).
 template <typename T>
 __global__ __launch_bounds__(256) void SplitKReduceKernel(IGemmArgs<T> p) {
+    // 64 outputs per workgroup, the slices dealt out over its four waves (four independent loads in flight per lane), the four
+    // partial sums joined through LDS: the loop over the slices is a chain of memory latencies otherwise.
+    __shared__ float part[4][64];
     const int64_t total = p.M * p.K;
-    for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < total; i += static_cast<int64_t>(gridDim.x) * 256) {
-        float sum = 0.f;
-        for (int sl = 0; sl < p.ksplit; ++sl) sum += p.partial[static_cast<int64_t>(sl) * total + i];
-        const int64_t m = i / p.K;
-        const int n = static_cast<int>(i - m * p.K);
-        if (p.bias != nullptr) sum += static_cast<float>(p.bias[n * p.bias_stride]);
-        p.out[m * p.osN + static_cast<int64_t>(n) * p.osC] = static_cast<T>(sum);
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    for (int64_t base = static_cast<int64_t>(blockIdx.x) * 64; base < total; base += static_cast<int64_t>(gridDim.x) * 64) {
+        const int64_t i = base + tx;
+        float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+        if (i < total) {
+            int sl = ty;
+            for (; sl + 12 < p.ksplit; sl += 16) {
+                s0 += p.partial[static_cast<int64_t>(sl) * total + i];
+                s1 += p.partial[static_cast<int64_t>(sl + 4) * total + i];
+                s2 += p.partial[static_cast<int64_t>(sl + 8) * total + i];
+                s3 += p.partial[static_cast<int64_t>(sl + 12) * total + i];
+            }
+            for (; sl < p.ksplit; sl += 4) s0 += p.partial[static_cast<int64_t>(sl) * total + i];
+        }
+        part[ty][tx] = (s0 + s1) + (s2 + s3);
+        __syncthreads();
+        if (ty == 0 && i < total) {
+            float sum = (part[0][tx] + part[1][tx]) + (part[2][tx] + part[3][tx]);
+            const int64_t m = i / p.K;
+            const int n = static_cast<int>(i - m * p.K);
+            if (p.bias != nullptr) sum += static_cast<float>(p.bias[n * p.bias_stride]);
+            p.out[m * p.osN + static_cast<int64_t>(n) * p.osC] = static_cast<T>(sum);
+        }
+        __syncthreads();
     }
 }
 

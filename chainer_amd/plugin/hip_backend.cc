@@ -979,7 +979,7 @@ HIPCX_REGISTER_KERNEL(ConvTransposeKernel, HipConvTransposeKernel)
 // generic one (batch mean, 1 / sqrt(var + eps), dtype of beta), so either gradient kernel can consume either forward's state.
 namespace {
 bool HipBatchNormApplies(const Array& x, const Axes& axis, std::initializer_list<const Array*> others) {
-    if (x.ndim() < 2 || !x.IsContiguous() || x.GetTotalSize() == 0) return false;
+    if (x.ndim() < 2 || !x.IsContiguous() || x.GetTotalSize() == 0 || x.GetTotalSize() >= (int64_t{1} << 31)) return false;
     if (static_cast<int8_t>(axis.size()) != x.ndim() - 1) return false;
     for (int8_t i = 0; i < static_cast<int8_t>(axis.size()); ++i) {
         if (axis[i] != (i == 0 ? 0 : i + 1)) return false;

@@ -1574,8 +1574,9 @@ COMPOSE_BATCH_NORM = False
 
 
 def _bn_kernel_applies(x, axes, others):
-    """The dedicated kernels take a C-contiguous x reduced over every axis but 1, with every other array in x's dtype."""
-    return (not COMPOSE_BATCH_NORM and x.ndim >= 2 and tuple(axes) == (0,) + tuple(range(2, x.ndim)) and x.is_contiguous
+    """The dedicated kernels take a C-contiguous x of fewer than 2^31 elements reduced over every axis but 1, with every other array
+    in x's dtype."""
+    return (not COMPOSE_BATCH_NORM and x.ndim >= 2 and tuple(axes) == (0,) + tuple(range(2, x.ndim)) and x.is_contiguous and x.size < 2 ** 31
             and _py.all(a.dtype == x.dtype for a in others))
 
 

@@ -266,3 +266,13 @@ def test_svd_errors_and_empty():
     with pytest.raises(chx.DtypeError):
         chx.pinv(chx.zeros((2, 2), 'int64'))
 
+
+def test_one_workgroup_limits():
+    """Matrices beyond what the one-workgroup kernels take are refused before anything is launched."""
+    import chainer_amd as chx
+    big = chx.zeros((4097, 4097), 'float32')
+    with pytest.raises(chx.ChainerxNotImplementedError):
+        chx.eigh(big)
+    with pytest.raises(chx.ChainerxNotImplementedError):
+        chx.svd(big)
+
