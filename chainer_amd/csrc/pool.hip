@@ -471,38 +471,55 @@ __global__ __launch_bounds__(256) void MaxPoolGradGradKernel(PoolGradArgs p, Idx
     }
 }
 
-template <typename T, bool IS_MAX, typename IdxT>
+// SMALL: the window is at most twice the stride along both axes, so a position is covered by at most 2 x 2 windows; their gradients
+// and indices are then loaded up front, independent of each other, and accumulated in the same order as the general loop visits them.
+template <typename T, bool IS_MAX, typename IdxT, bool SMALL = false>
 __global__ __launch_bounds__(256) void PoolGradKernel(PoolGradArgs p, IdxT total) {
     using C = compute_t<T>;
     const T* gout = static_cast<const T*>(p.gout);
     T* gx = static_cast<T*>(p.gx);
-    for (IdxT idx = static_cast<IdxT>(blockIdx.x) * blockDim.x + threadIdx.x; idx < total; idx += static_cast<IdxT>(gridDim.x) * blockDim.x) {
-        int c, w, h;
-        int64_t n;
-        IdxT t = idx;
-        if (p.w_fastest) {
-            w = static_cast<int>(t % p.W);
-            t /= p.W;
-            h = static_cast<int>(t % p.H);
-            t /= p.H;
-            c = static_cast<int>(t % p.C);
-            n = static_cast<int64_t>(t / p.C);
-        } else {
-            c = static_cast<int>(t % p.C);
-            t /= p.C;
-            w = static_cast<int>(t % p.W);
-            t /= p.W;
-            h = static_cast<int>(t % p.H);
-            n = static_cast<int64_t>(t / p.H);
-        }
+    // strides that are powers of two (the usual 1 and 2) divide by a shift; -1: a real division
+    const int sh_shift = (p.sh & (p.sh - 1)) == 0 ? __builtin_ctz(p.sh) : -1;
+    const int sw_shift = (p.sw & (p.sw - 1)) == 0 ? __builtin_ctz(p.sw) : -1;
+    auto pixel = [&](int64_t n, int c, int h, int w) {
         const int* wb = IS_MAX ? p.win_index + (n * p.C + c) * (static_cast<int64_t>(p.OH) * p.OW) : nullptr;
         const T* gb = gout + n * p.gsN + static_cast<int64_t>(c) * p.gsC;
         const int y = h + p.ph, xq = w + p.pw;
         T acc = T(0);
         // windows (i, j) that cover this position, walked with the kernel offset r = y - i * sh (and q) ascending
-        int i_hi = y / p.sh, j_hi = xq / p.sw;
+        int i_hi = sh_shift >= 0 ? y >> sh_shift : y / p.sh, j_hi = sw_shift >= 0 ? xq >> sw_shift : xq / p.sw;
         if (i_hi > p.OH - 1) i_hi = p.OH - 1;
         if (j_hi > p.OW - 1) j_hi = p.OW - 1;
+        if constexpr (SMALL) {
+            T g4[4];
+            bool ok4[4];
+#pragma unroll
+            for (int a = 0; a < 2; ++a) {
+#pragma unroll
+                for (int b = 0; b < 2; ++b) {
+                    const int i = i_hi - a, j = j_hi - b;
+                    const int r = y - i * p.sh, q = xq - j * p.sw;
+                    bool ok = i >= 0 && j >= 0 && r < p.kh && q < p.kw;
+                    const int ic = ok ? i : 0, jc = ok ? j : 0;
+                    T g = gb[ic * p.gsH + jc * p.gsW];
+                    if constexpr (IS_MAX) {
+                        ok = ok && wb[ic * p.OW + jc] == r * p.kw + q;
+                    } else if (p.pad_mode == HIPCX_PAD_IGNORE) {
+                        const int h0 = ic * p.sh - p.ph, w0 = jc * p.sw - p.pw;
+                        const int hcnt = (h0 + p.kh < p.H ? h0 + p.kh : p.H) - (h0 < 0 ? 0 : h0);
+                        const int wcnt = (w0 + p.kw < p.W ? w0 + p.kw : p.W) - (w0 < 0 ? 0 : w0);
+                        const T width = static_cast<T>(static_cast<C>(static_cast<T>(static_cast<C>(hcnt))) * static_cast<C>(static_cast<T>(static_cast<C>(wcnt))));
+                        g = static_cast<T>(static_cast<C>(g) / static_cast<C>(width));
+                    }
+                    g4[a * 2 + b] = g;
+                    ok4[a * 2 + b] = ok;
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                if (ok4[e]) acc = static_cast<T>(static_cast<C>(acc) + static_cast<C>(g4[e]));
+            }
+        } else
         for (int i = i_hi; i >= 0; --i) {
             const int r = y - i * p.sh;
             if (r >= p.kh) break;
@@ -526,6 +543,27 @@ __global__ __launch_bounds__(256) void PoolGradKernel(PoolGradArgs p, IdxT total
             acc = static_cast<T>(static_cast<C>(acc) / static_cast<C>(static_cast<T>(static_cast<C>(p.kh * p.kw))));
         }
         gx[n * p.dsN + static_cast<int64_t>(c) * p.dsC + h * p.dsH + w * p.dsW] = acc;
+    };
+    for (IdxT idx = static_cast<IdxT>(blockIdx.x) * blockDim.x + threadIdx.x; idx < total; idx += static_cast<IdxT>(gridDim.x) * blockDim.x) {
+        int c, w, h;
+        int64_t n;
+        IdxT t = idx;
+        if (p.w_fastest) {
+            w = static_cast<int>(t % p.W);
+            t /= p.W;
+            h = static_cast<int>(t % p.H);
+            t /= p.H;
+            c = static_cast<int>(t % p.C);
+            n = static_cast<int64_t>(t / p.C);
+        } else {
+            c = static_cast<int>(t % p.C);
+            t /= p.C;
+            w = static_cast<int>(t % p.W);
+            t /= p.W;
+            h = static_cast<int>(t % p.H);
+            n = static_cast<int64_t>(t / p.H);
+        }
+        pixel(n, c, h, w);
     }
 }
 
@@ -590,10 +628,14 @@ void RunPoolGrad(const PoolGradArgs& p, hipStream_t stream) {
             CheckLaunch("window_argmax");
         }
     }
-    if (narrow) {
-        hipLaunchKernelGGL((PoolGradKernel<T, IS_MAX, unsigned>), grid_for(total), dim3(256), 0, stream, p, static_cast<unsigned>(total));
+    const bool small = p.kh <= 2 * p.sh && p.kw <= 2 * p.sw && p.OH > 0 && p.OW > 0;
+    const dim3 grid = grid_for(total);
+    if (narrow && small) {
+        hipLaunchKernelGGL((PoolGradKernel<T, IS_MAX, unsigned, true>), grid, dim3(256), 0, stream, p, static_cast<unsigned>(total));
+    } else if (narrow) {
+        hipLaunchKernelGGL((PoolGradKernel<T, IS_MAX, unsigned>), grid, dim3(256), 0, stream, p, static_cast<unsigned>(total));
     } else {
-        hipLaunchKernelGGL((PoolGradKernel<T, IS_MAX, int64_t>), grid_for(total), dim3(256), 0, stream, p, total);
+        hipLaunchKernelGGL((PoolGradKernel<T, IS_MAX, int64_t>), grid, dim3(256), 0, stream, p, total);
     }
     CheckLaunch("pool_grad");
 }
