@@ -282,7 +282,7 @@ def section_backward(chx, oracle, with_cpu):
            note='algorithmic bytes: three reads (sum, centred sum of squares, normalise) and one write')
     state = out_state[0][1]
     t = graph_time(lambda: chx.batch_norm_grad(xb, prm[0], gb, state), 5)
-    bw_row('backward', 'batch_norm_grad', shape, t, 5 * nbytes, 5,
+    bw_row('backward', 'batch_norm_grad', shape, t, 5 * nbytes, 3,
            note='algorithmic bytes: x and gout read twice, gx written')
     xp = chx.array(rng.standard_normal((32, 64, 112, 112)).astype(np.float16))
     gp = chx.array(rng.standard_normal((32, 64, 56, 56)).astype(np.float16))

@@ -35,6 +35,14 @@ __device__ __forceinline__ C BlockSum(C v, C* lds) {
     return r;  // valid in thread 0
 }
 
+// The per-channel state (mean, 1 / std): compute-type vectors in the workspace (forward), or the caller's arrays in the array dtype
+// with an element stride (gradient: the state BatchNorm handed out) -- read in place, so the gradient needs no widening copies.
+template <typename T>
+__device__ __forceinline__ compute_t<T> LoadState(const void* ptr, int c, int in_array_dtype, int64_t stride) {
+    using C = compute_t<T>;
+    return in_array_dtype ? static_cast<C>(static_cast<const T*>(ptr)[c * stride]) : static_cast<const C*>(ptr)[c];
+}
+
 struct BnStatArgs {
     const void* x;
     const void* g;        // gradient pass only
@@ -44,6 +52,8 @@ struct BnStatArgs {
     int N, C;
     int64_t L;
     int S;
+    int state_in_array_dtype;  // see LoadState
+    int64_t mean_stride, inv_stride;
 };
 
 // MODE 0: sum x.  MODE 1: sum (x - mean)^2.  MODE 2: sum g and sum g * (x - mean) * inv_std.
@@ -55,8 +65,8 @@ __global__ __launch_bounds__(kBnTrainThreads) void BnStatKernel(BnStatArgs p) {
     const T* x = static_cast<const T*>(p.x);
     const T* g = static_cast<const T*>(p.g);
     C m = C(0), is = C(1);
-    if (MODE >= 1) m = static_cast<const C*>(p.mean)[c];
-    if (MODE == 2) is = static_cast<const C*>(p.inv_std)[c];
+    if (MODE >= 1) m = LoadState<T>(p.mean, c, p.state_in_array_dtype, p.mean_stride);
+    if (MODE == 2) is = LoadState<T>(p.inv_std, c, p.state_in_array_dtype, p.inv_stride);
     C a0 = C(0), a1 = C(0);
     // The slice's images n = s, s + S, ... times the plane's vectors form one index space shared out over the threads, so that
     // planes shorter than the workgroup (14x14, 7x7) keep every lane busy.  32-bit index arithmetic: the host checks N * L < 2^31.
@@ -156,6 +166,8 @@ struct BnApplyArgs {
     int C, S;
     int64_t L, total;
     double count;
+    int state_in_array_dtype;  // see LoadState
+    int64_t mean_stride, inv_stride;
 };
 
 // Gradient finish: ggamma = sum g * x_hat, gbeta = sum g, one thread per channel; leaves both as compute-type values at partial[c][0].
@@ -199,13 +211,13 @@ __global__ __launch_bounds__(256) void BnApplyKernel(BnApplyArgs p) {
         const int c2 = c + 1 == p.C ? 0 : c + 1;
         const bool split = planes_split && within + VEC > L;
         const int split_at = split ? static_cast<int>(L - within) : VEC;  // elements from split_at on belong to channel c2
-        const C m = static_cast<const C*>(p.mean)[c];
-        const C is = static_cast<const C*>(p.inv_std)[c];
+        const C m = LoadState<T>(p.mean, c, p.state_in_array_dtype, p.mean_stride);
+        const C is = LoadState<T>(p.inv_std, c, p.state_in_array_dtype, p.inv_stride);
         const C ga = static_cast<C>(static_cast<const T*>(p.gamma)[c * p.gamma_stride]);
         C m2 = m, is2 = is, ga2 = ga;
         if (split) {
-            m2 = static_cast<const C*>(p.mean)[c2];
-            is2 = static_cast<const C*>(p.inv_std)[c2];
+            m2 = LoadState<T>(p.mean, c2, p.state_in_array_dtype, p.mean_stride);
+            is2 = LoadState<T>(p.inv_std, c2, p.state_in_array_dtype, p.inv_stride);
             ga2 = static_cast<C>(static_cast<const T*>(p.gamma)[c2 * p.gamma_stride]);
         }
         Vec<T, VEC> xv = *reinterpret_cast<const Vec<T, VEC>*>(x + v * VEC);
@@ -455,36 +467,28 @@ int hipcx_batch_norm_grad(const hipcx_array* x, const hipcx_array* gamma, const 
         CheckWorkspace(workspace, workspace_bytes, TrainWorkspace(g));
         char* ws = static_cast<char*>(workspace);
         const size_t vec_bytes = RoundUpTo(static_cast<size_t>(g.C) * g.csize, 16);
-        void* mean_c = ws;
-        void* inv_c = ws + vec_bytes;
-        void* partial = ws + 2 * vec_bytes;
+        void* partial = ws + 2 * vec_bytes;  // the same layout as the forward's workspace; the state vectors before it stay unused here
         hipStream_t st = AsStream(stream);
         HIPCX_REQUIRE(total < (int64_t{1} << 31), HIPCX_NOT_IMPLEMENTED_ERROR, "hip batch_norm_grad: array too large for the dedicated kernels");
         const BnWidths widths = PickWidths(g.L, total, ItemSize(x->dtype), {x->data, gout->data, gx->data});
-        // the state arrives in the array dtype: widen it into the workspace vectors the kernels read
-        hipcx_array mc{}, ic{};
-        const int cdtype = x->dtype == HIPCX_FLOAT64 ? HIPCX_FLOAT64 : HIPCX_FLOAT32;
-        mc.data = mean_c, mc.dtype = cdtype, mc.ndim = 1, mc.shape[0] = g.C, mc.strides[0] = static_cast<int64_t>(g.csize);
-        ic = mc;
-        ic.data = inv_c;
-        hipcx_array m1{}, i1{};
-        m1.data = mean->data, m1.dtype = mean->dtype, m1.ndim = 1, m1.shape[0] = g.C, m1.strides[0] = mean_stride * ItemSize(mean->dtype);
-        i1.data = inv_std->data, i1.dtype = inv_std->dtype, i1.ndim = 1, i1.shape[0] = g.C, i1.strides[0] = inv_stride * ItemSize(inv_std->dtype);
-        int rc = hipcx_copy(&m1, &mc, stream);
-        if (rc == HIPCX_OK) rc = hipcx_copy(&i1, &ic, stream);
-        HIPCX_REQUIRE(rc == HIPCX_OK, HIPCX_CHAINERX_ERROR, std::string("batch_norm_grad: widening the state failed: ") + hipcx_last_error());
+        HIPCX_REQUIRE(mean->dtype == x->dtype && inv_std->dtype == x->dtype, HIPCX_NOT_IMPLEMENTED_ERROR,
+                      "hip batch_norm_grad: the state must have x's dtype");
         BnStatArgs s{};
         s.x = x->data;
         s.g = gout->data;
-        s.mean = mean_c;
-        s.inv_std = inv_c;
+        s.mean = mean->data;  // the state as BatchNorm handed it out, read in place
+        s.inv_std = inv_std->data;
+        s.state_in_array_dtype = 1;
+        s.mean_stride = mean_stride, s.inv_stride = inv_stride;
         s.partial = partial;
         s.N = g.N, s.C = g.C, s.L = g.L, s.S = g.S;
         a.x = x->data;
         a.g = gout->data;
         a.out = gx->data;
-        a.mean = mean_c;
-        a.inv_std = inv_c;
+        a.mean = mean->data;
+        a.inv_std = inv_std->data;
+        a.state_in_array_dtype = 1;
+        a.mean_stride = mean_stride, a.inv_stride = inv_stride;
         a.gamma = gamma->data;
         a.partial = partial;
         a.ggamma = ggamma->data;
