@@ -56,7 +56,9 @@ void LaunchShape(IGemmArgs<T> p, bool fast16, bool fast8, hipStream_t stream) {
     int per = static_cast<int>((total + 7) / 8);
     static const bool pipe_env = [] { const char* e = getenv("HIPCX_IGEMM_PIPE"); return e != nullptr && e[0] == '1'; }();
     if (PM || pipe_env || !(fast16 || fast8) || p.partial == nullptr) p.ksplit = 1;  // only the simple fast kernel splits the reduction
-    dim3 grid(per * 8, p.ksplit > 1 ? p.ksplit : 1), block(64 * WM * WN);
+    dim3 grid(per * 8, 1), block(64 * WM * WN);
+    if (p.ksplit > 1 && total > 65535) p.ksplit = 1;  // never planned for that many tiles; the grid's y extent could not hold them
+    if (p.ksplit > 1) grid = dim3(p.ksplit, static_cast<unsigned>(total));  // slices along x: see IGemmFastKernel
     // algorithmic work of this launch: 2 flops per multiply-add; every operand byte moved once
     double flops = 2.0 * static_cast<double>(p.M) * p.K * p.R * p.S * p.C_logical;
     double bytes = sizeof(T) * (static_cast<double>(p.N) * p.C_logical * p.H_logical * p.W_logical +
@@ -975,7 +977,7 @@ int PlanSplitK(int64_t m, int64_t n, int64_t k, int dtype) {
     if (k < 4096 || tiles * 2 > NumCUs() || m * n < 64 * 64 || steps < 16) return 1;
     int64_t s = (2 * NumCUs() + tiles - 1) / tiles;
     if (s > steps / 24) s = steps / 24;  // a slice of fewer steps costs more in partial sums than it gains
-    static const int64_t max_slices = [] { const char* e = getenv("HIPCX_DOT_SPLITK_MAX"); int v = e ? atoi(e) : 0; return v >= 2 && v <= 1024 ? v : 64; }();
+    static const int64_t max_slices = [] { const char* e = getenv("HIPCX_DOT_SPLITK_MAX"); int v = e ? atoi(e) : 0; return v >= 2 && v <= 1024 ? v : 256; }();
     if (s > max_slices) s = max_slices;
     return s < 2 ? 1 : static_cast<int>(s);
 }

@@ -39,7 +39,7 @@ struct IGemmArgs {
     int tiles_m, tiles_n;
     int out_vec;                 // 1 if the 4 accumulators a lane holds per group can be stored as one vector
     int out_wide;                // 1 if 16-byte runs along the output's contiguous axis can be stored (pipelined kernel)
-    // Split reduction (matrix products with few output tiles and a long reduction axis, e.g. weight gradients): grid.y slices of
+    // Split reduction (matrix products with few output tiles and a long reduction axis, e.g. weight gradients): grid.x slices of
     // the reduction steps, each storing float partial sums [ksplit][M][K]; SplitKReduceKernel adds them up.  0 or 1: off.
     int ksplit;
     float* partial;
@@ -310,7 +310,17 @@ __global__ __launch_bounds__(64 * WM * WN) void IGemmFastKernel(IGemmArgs<T> p) 
     char* ldsW = lds + BM * kLdsRow;
 
     int tile_m, tile_n;
-    if (!TileOf(p.tiles_m, p.tiles_n, tile_m, tile_n)) return;
+    unsigned slice = 0;
+    if (p.ksplit > 1) {
+        // Split reduction: grid (slices, tiles).  Workgroup ids go round-robin to the 8 XCDs with x as the fast index, so the
+        // slices of one tile spread over all of them -- with the tiles along x, a product of one or two tiles would keep one
+        // or two XCDs (a quarter of the chip) busy however many slices it has.
+        slice = blockIdx.x;
+        tile_n = static_cast<int>(blockIdx.y) % p.tiles_n;
+        tile_m = static_cast<int>(blockIdx.y) / p.tiles_n;
+    } else if (!TileOf(p.tiles_m, p.tiles_n, tile_m, tile_n)) {
+        return;
+    }
     const int m0 = tile_m * BM;
     const int n0 = tile_n * BN;
     const int tid = threadIdx.x;
@@ -422,8 +432,8 @@ __global__ __launch_bounds__(64 * WM * WN) void IGemmFastKernel(IGemmArgs<T> p) 
     const int steps = p.batch > 0 ? nk * p.batch : nk;
     int kt_begin = 0, kt_end = steps;
     if (p.ksplit > 1) {
-        kt_begin = static_cast<int>(static_cast<int64_t>(steps) * blockIdx.y / p.ksplit);
-        kt_end = static_cast<int>(static_cast<int64_t>(steps) * (blockIdx.y + 1) / p.ksplit);
+        kt_begin = static_cast<int>(static_cast<int64_t>(steps) * slice / p.ksplit);
+        kt_end = static_cast<int>(static_cast<int64_t>(steps) * (slice + 1) / p.ksplit);
     }
     if (kt_begin < kt_end) load_tile(kt_begin);
     for (int kt = kt_begin; kt < kt_end; ++kt) {
@@ -434,7 +444,7 @@ __global__ __launch_bounds__(64 * WM * WN) void IGemmFastKernel(IGemmArgs<T> p) 
         __syncthreads();
     }
     if (p.ksplit > 1) {
-        if constexpr (!PM) StorePartial<T>(p, m0, n0, wm, wn, lane, acc, blockIdx.y);
+        if constexpr (!PM) StorePartial<T>(p, m0, n0, wm, wn, lane, acc, slice);
         return;
     }
     if (PM) {
