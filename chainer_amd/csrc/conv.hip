@@ -976,7 +976,8 @@ int PlanSplitK(int64_t m, int64_t n, int64_t k, int dtype) {
     const int64_t steps = k * ItemSize(dtype) / 128;  // reduction steps of 128 bytes per row
     if (k < 4096 || tiles * 2 > NumCUs() || m * n < 64 * 64 || steps < 16) return 1;
     int64_t s = (2 * NumCUs() + tiles - 1) / tiles;
-    if (s > steps / 24) s = steps / 24;  // a slice of fewer steps costs more in partial sums than it gains
+    static const int64_t min_steps = [] { const char* e = getenv("HIPCX_DOT_SPLITK_MINSTEPS"); int v = e ? atoi(e) : 0; return v >= 1 && v <= 4096 ? v : 8; }();
+    if (s > steps / min_steps) s = steps / min_steps;  // a slice of fewer steps costs more in partial sums than it gains
     static const int64_t max_slices = [] { const char* e = getenv("HIPCX_DOT_SPLITK_MAX"); int v = e ? atoi(e) : 0; return v >= 2 && v <= 1024 ? v : 256; }();
     if (s > max_slices) s = max_slices;
     return s < 2 ? 1 : static_cast<int>(s);
