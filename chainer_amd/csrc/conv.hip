@@ -974,7 +974,7 @@ int PlanSplitK(int64_t m, int64_t n, int64_t k, int dtype) {
     if (!enabled || (dtype != HIPCX_FLOAT16 && dtype != HIPCX_FLOAT32)) return 1;
     const int64_t tiles = ((m + 127) / 128) * ((n + 127) / 128);
     const int64_t steps = k * ItemSize(dtype) / 128;  // reduction steps of 128 bytes per row
-    if (k < 4096 || tiles * 2 > NumCUs() || m * n < 64 * 64 || steps < 16) return 1;
+    if (k < 4096 || tiles > NumCUs() || m * n < 64 * 64 || steps < 16) return 1;  // up to one tile per compute unit: a second workgroup per unit still hides latency
     int64_t s = (2 * NumCUs() + tiles - 1) / tiles;
     static const int64_t min_steps = [] { const char* e = getenv("HIPCX_DOT_SPLITK_MINSTEPS"); int v = e ? atoi(e) : 0; return v >= 1 && v <= 4096 ? v : 8; }();
     if (s > steps / min_steps) s = steps / min_steps;  // a slice of fewer steps costs more in partial sums than it gains
