@@ -31,18 +31,7 @@ __global__ __launch_bounds__(256) void Im2ColTKernel(GradWeightArgs p, int64_t t
     const T* x = static_cast<const T*>(p.x);
     T* col = static_cast<T*>(p.col_t);
     const int owv = p.OW / VEC;
-    for (int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; idx < total; idx += static_cast<int64_t>(gridDim.x) * 256) {
-        int64_t t = idx;
-        const int wv = static_cast<int>(t % owv);
-        t /= owv;
-        const int oh = static_cast<int>(t % p.OH);
-        t /= p.OH;
-        const int n = static_cast<int>(t % p.N);
-        t /= p.N;
-        const int s = static_cast<int>(t % p.kw);
-        t /= p.kw;
-        const int r = static_cast<int>(t % p.kh);
-        const int c = static_cast<int>(t / p.kh);
+    auto emit = [&](int64_t idx, int wv, int oh, int n, int s, int r, int c) {
         const int ih = oh * p.sh - p.ph + r;
         GVec<T, VEC> out;
         const T* row = x + ((static_cast<int64_t>(n) * p.C + c) * p.H + ih) * p.W;
@@ -52,6 +41,38 @@ __global__ __launch_bounds__(256) void Im2ColTKernel(GradWeightArgs p, int64_t t
             out.v[e] = (ih >= 0 && ih < p.H && iw >= 0 && iw < p.W) ? row[iw] : T(0);
         }
         *reinterpret_cast<GVec<T, VEC>*>(col + idx * VEC) = out;  // idx enumerates the vectors of col_t in memory order
+    };
+    if (total < (int64_t{1} << 31)) {  // the usual case: five 32-bit divisions per vector instead of five 64-bit ones
+        const uint32_t n_total = static_cast<uint32_t>(total), step = gridDim.x * 256u;
+        for (uint32_t idx = blockIdx.x * 256u + threadIdx.x; idx < n_total; idx += step) {
+            uint32_t t = idx;
+            const uint32_t wv = t % static_cast<uint32_t>(owv);
+            t /= static_cast<uint32_t>(owv);
+            const uint32_t oh = t % static_cast<uint32_t>(p.OH);
+            t /= static_cast<uint32_t>(p.OH);
+            const uint32_t n = t % static_cast<uint32_t>(p.N);
+            t /= static_cast<uint32_t>(p.N);
+            const uint32_t s2 = t % static_cast<uint32_t>(p.kw);
+            t /= static_cast<uint32_t>(p.kw);
+            const uint32_t r = t % static_cast<uint32_t>(p.kh);
+            emit(idx, static_cast<int>(wv), static_cast<int>(oh), static_cast<int>(n), static_cast<int>(s2), static_cast<int>(r),
+                 static_cast<int>(t / static_cast<uint32_t>(p.kh)));
+            if (idx + step < idx) break;  // the next index would wrap
+        }
+        return;
+    }
+    for (int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; idx < total; idx += static_cast<int64_t>(gridDim.x) * 256) {
+        int64_t t = idx;
+        const int wv = static_cast<int>(t % owv);
+        t /= owv;
+        const int oh = static_cast<int>(t % p.OH);
+        t /= p.OH;
+        const int n = static_cast<int>(t % p.N);
+        t /= p.N;
+        const int s2 = static_cast<int>(t % p.kw);
+        t /= p.kw;
+        const int r = static_cast<int>(t % p.kh);
+        emit(idx, wv, oh, n, s2, r, static_cast<int>(t / p.kh));
     }
 }
 
@@ -61,6 +82,19 @@ __global__ __launch_bounds__(256) void TransposeNKKernel(GradWeightArgs p, int64
     const T* gy = static_cast<const T*>(p.gy);
     T* gt = static_cast<T*>(p.gy_t);
     const int64_t pv = static_cast<int64_t>(p.OH) * p.OW / VEC;
+    if (total < (int64_t{1} << 31)) {  // 32-bit index arithmetic
+        const uint32_t n_total = static_cast<uint32_t>(total), step = gridDim.x * 256u, pv32 = static_cast<uint32_t>(pv);
+        for (uint32_t idx = blockIdx.x * 256u + threadIdx.x; idx < n_total; idx += step) {
+            uint32_t t = idx / pv32;
+            const uint32_t v = idx - t * pv32;
+            const uint32_t k = t / static_cast<uint32_t>(p.N);
+            const uint32_t n = t - k * static_cast<uint32_t>(p.N);
+            *reinterpret_cast<GVec<T, VEC>*>(gt + static_cast<int64_t>(idx) * VEC) =
+                    *reinterpret_cast<const GVec<T, VEC>*>(gy + ((static_cast<int64_t>(n) * p.K + k) * pv + v) * VEC);
+            if (idx + step < idx) break;  // the next index would wrap
+        }
+        return;
+    }
     for (int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; idx < total; idx += static_cast<int64_t>(gridDim.x) * 256) {
         int64_t t = idx;
         const int64_t v = t % pv;
