@@ -164,10 +164,19 @@ __global__ __launch_bounds__(256) void MaxPoolRowsS2Kernel(PoolArgs p, int64_t t
     const int ovecs = p.OW / VO;
     for (int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; idx < total;
          idx += static_cast<int64_t>(gridDim.x) * blockDim.x) {
-        int ov = static_cast<int>(idx % ovecs);
-        int64_t t = idx / ovecs;
-        int oh = static_cast<int>(t % p.OH);
-        int64_t plane = t / p.OH;  // n * C + c
+        int ov, oh;
+        int64_t plane;  // n * C + c
+        if (total < (int64_t{1} << 31)) {  // 32-bit index arithmetic (uniform branch)
+            const uint32_t i = static_cast<uint32_t>(idx), t = i / static_cast<uint32_t>(ovecs), pl = t / static_cast<uint32_t>(p.OH);
+            ov = static_cast<int>(i - t * static_cast<uint32_t>(ovecs));
+            oh = static_cast<int>(t - pl * static_cast<uint32_t>(p.OH));
+            plane = pl;
+        } else {
+            ov = static_cast<int>(idx % ovecs);
+            const int64_t t = idx / ovecs;
+            oh = static_cast<int>(t % p.OH);
+            plane = t / p.OH;
+        }
         const T* xp = x + plane * p.H * p.W;
         const int ow0 = ov * VO;
         const int col0 = 2 * ow0 - EPV;  // first column of the left chunk
