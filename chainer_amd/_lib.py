@@ -129,6 +129,7 @@ SIGNATURES = {
     'hipcx_arange': (_INT, [_S, _S, _A, _V]),
     'hipcx_reduce_workspace_size': (_SZ, [_A, _I8P, _INT, _A]),
     'hipcx_sum': (_INT, [_A, _I8P, _INT, _A, _V, _SZ, _V]),
+    'hipcx_sum_static_scratch': (_INT, [_A, _I8P, _INT, _A, _V]),
     'hipcx_amax': (_INT, [_A, _I8P, _INT, _A, _V, _SZ, _V]),
     'hipcx_argmax': (_INT, [_A, _I8P, _INT, _A, _V, _SZ, _V]),
     'hipcx_dot_workspace_size': (_SZ, [_A, _A, _A]),

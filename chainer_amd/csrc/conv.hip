@@ -1109,9 +1109,12 @@ int hipcx_dot(const hipcx_array* a, const hipcx_array* b, const hipcx_array* out
         };
         // operands in another layout than the MFMA kernels read are staged in the workspace first
         hipcx_array a_st = *a, b_st = *b;
+        const int64_t k_given = k;  // the reduction extent the workspace query saw (staging may pad it)
+        size_t staged_bytes = 0;    // the front of the workspace that holds staged operands
         if (out->dtype == a->dtype && out->dtype == b->dtype) {
             DotStaging plan = PlanDotStaging(a, b, out);
             if (plan.a || plan.b) {
+                staged_bytes = plan.a_bytes + plan.b_bytes;
                 HIPCX_REQUIRE(workspace != nullptr && workspace_bytes >= plan.a_bytes + plan.b_bytes, HIPCX_CHAINERX_ERROR,
                               "dot: workspace of " + std::to_string(plan.a_bytes + plan.b_bytes) + " bytes required (hipcx_dot_workspace_size)");
                 HIPCX_REQUIRE(reinterpret_cast<uintptr_t>(workspace) % 16 == 0, HIPCX_CHAINERX_ERROR, "workspace must be 16-byte aligned");
@@ -1145,11 +1148,11 @@ int hipcx_dot(const hipcx_array* a, const hipcx_array* b, const hipcx_array* out
         float* partial = nullptr;
         {
             const int64_t it = ItemSize(out->dtype);
-            const int planned = PlanSplitK(m, n, a->shape[1], out->dtype);
+            // slices from the extent the workspace query planned with; the partial sums lie behind the staged operands
+            const int planned = PlanSplitK(m, n, k_given, out->dtype);
             if (planned > 1 && OperandIsFast(a->data, a->strides[0], a->strides[1], k, it) &&
                 OperandIsFast(b->data, b->strides[1], b->strides[0], k, it) && out->strides[0] >= 0 && out->strides[1] >= 0) {
-                DotStaging plan = PlanDotStaging(a, b, out);  // nothing is staged for operands in this layout
-                const size_t offset = RoundUpTo(plan.a_bytes + plan.b_bytes, 256);
+                const size_t offset = RoundUpTo(staged_bytes, 256);
                 const size_t need = offset + SplitKBytes(m, n, planned);
                 if (workspace != nullptr && workspace_bytes >= need && reinterpret_cast<uintptr_t>(workspace) % 16 == 0) {
                     slices = planned;

@@ -237,10 +237,11 @@ size_t hipcx_conv_grad_weight_workspace_size(const hipcx_array* x, const hipcx_a
         if (x == nullptr || gy == nullptr || gw == nullptr) return 0;
         GradWeightPlan pl = PlanGradWeight(x, gy, gw, stride, pad, cover_all);
         hipcx_array out = GwAsMatrix(gw);
-        if (DirectPointwise(pl, x, gy, gw)) {
-            return BatchedProductPartialBytes(pl.a.K, pl.a.C, static_cast<int64_t>(pl.a.H) * pl.a.W, pl.a.N, gw->dtype) + 256;
-        }
-        return pl.col_bytes + pl.gyt_bytes + hipcx_dot_workspace_size(&pl.gy_t, &pl.col_view, &out);
+        // Which path the call takes depends on the alignment of the data pointers, which a caller sizing its workspace from
+        // descriptors alone may not have yet: the answer covers both.
+        const size_t direct = BatchedProductPartialBytes(pl.a.K, pl.a.C, static_cast<int64_t>(pl.a.H) * pl.a.W, pl.a.N, gw->dtype) + 256;
+        const size_t staged = pl.col_bytes + pl.gyt_bytes + hipcx_dot_workspace_size(&pl.gy_t, &pl.col_view, &out);
+        return std::max(direct, staged);
     } catch (...) {
         return 0;
     }

@@ -19,7 +19,13 @@
 // GenericReduceKernel: any strides; one thread per output element runs the reference loop
 // literally.  Consecutive threads take consecutive outputs, so reducing over outer axes of a
 // dense array (a "column" reduction) is coalesced.
+#include <mutex>
+
 #include "common.h"
+
+// Device memory for the partial results of hipcx_sum_static_scratch: part of the code object, so every device the library
+// runs on holds its own copy (at its own address) from the moment the module is loaded until the process ends.
+static __device__ __align__(256) __attribute__((used)) unsigned char scratch[HIPCX_STATIC_SCRATCH_BYTES];
 
 namespace hipcx {
 namespace {
@@ -701,6 +707,25 @@ void Run(const hipcx_array* a, const int8_t* axis, int naxis, const hipcx_array*
     CheckLaunch("generic_reduce");
 }
 
+// The device address of `scratch` on the current device.  In host code the array's name is only a handle for this lookup,
+// never an address a kernel may be given.  Looked up once per device, with that device current.
+void* StaticScratchAddress() {
+    constexpr int kMaxDevices = 64;
+    static std::mutex mu;
+    static void* address[kMaxDevices] = {};
+    int dev = 0;
+    HIPCX_CHECK_HIP(hipGetDevice(&dev));
+    HIPCX_REQUIRE(dev >= 0 && dev < kMaxDevices, HIPCX_DEVICE_ERROR, "device index beyond the static scratch table");
+    std::lock_guard<std::mutex> lock(mu);
+    if (address[dev] == nullptr) {
+        void* ptr = nullptr;
+        HIPCX_CHECK_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        HIPCX_REQUIRE(ptr != nullptr, HIPCX_BACKEND_ERROR, "hipGetSymbolAddress returned a null address for the static scratch");
+        address[dev] = ptr;
+    }
+    return address[dev];
+}
+
 }  // namespace
 }  // namespace hipcx
 
@@ -741,6 +766,26 @@ int hipcx_sum(const hipcx_array* a, const int8_t* axis, int naxis, const hipcx_a
         };
         VisitDtype(in, for_out);
     });
+}
+
+// hipcx_sum for callers that can neither allocate a workspace nor have one allocated for them: the per-block / per-slice
+// partial results go to the library's own static device array.  Same kernels and launch plan as hipcx_sum, hence the same bits.
+// Every partial is written before it is read, so nothing has to be cleared between calls; calls that overlap on one device
+// (different streams or threads) share the array and race.
+int hipcx_sum_static_scratch(const hipcx_array* a, const int8_t* axis, int naxis, const hipcx_array* out, void* stream) {
+    int status = Guard([&] {
+        ValidateArray(a, "a");
+        ValidateArray(out, "out");
+        const size_t need = hipcx_reduce_workspace_size(a, axis, naxis, out);
+        HIPCX_REQUIRE(need <= HIPCX_STATIC_SCRATCH_BYTES, HIPCX_CHAINERX_ERROR,
+                      "sum_static_scratch: this reduction needs " + std::to_string(need) + " bytes of partial results, the static scratch holds " +
+                              std::to_string(static_cast<size_t>(HIPCX_STATIC_SCRATCH_BYTES)) + "; use hipcx_sum with a workspace");
+    });
+    if (status != HIPCX_OK) return status;
+    void* ptr = nullptr;
+    status = Guard([&] { ptr = StaticScratchAddress(); });
+    if (status != HIPCX_OK) return status;
+    return hipcx_sum(a, axis, naxis, out, ptr, HIPCX_STATIC_SCRATCH_BYTES, stream);
 }
 
 int hipcx_amax(const hipcx_array* a, const int8_t* axis, int naxis, const hipcx_array* out, void* workspace, size_t workspace_bytes,

@@ -58,7 +58,7 @@ __device__ __forceinline__ int64_t ResolveIndex(int64_t index, int64_t dim, int 
     if (mode == HIPCX_BOUNDS_CLIP) {
         return index < 0 ? 0 : (index >= dim ? dim - 1 : index);
     }
-    if (mode == HIPCX_BOUNDS_WRAP || error_flag == nullptr) {
+    if (mode == HIPCX_BOUNDS_WRAP) {
         if (index < 0) return dim - ((-index + dim - 1) % dim + 1);
         return index % dim;
     }
@@ -158,6 +158,8 @@ extern "C" int hipcx_take(const hipcx_array* a, const hipcx_array* indices, int8
                       HIPCX_DTYPE_ERROR, "Only arrays of integer dtype can be used as indices.");
         HIPCX_REQUIRE(out->dtype == a->dtype, HIPCX_DTYPE_ERROR, "take: out must have a's dtype");
         HIPCX_REQUIRE(mode >= HIPCX_BOUNDS_DEFAULT && mode <= HIPCX_BOUNDS_CLIP, HIPCX_CHAINERX_ERROR, "take: invalid bounds mode");
+        HIPCX_REQUIRE(error_flag != nullptr || mode == HIPCX_BOUNDS_WRAP || mode == HIPCX_BOUNDS_CLIP, HIPCX_CHAINERX_ERROR,
+                      "take: the default and raise bounds modes report out-of-range indices through error_flag, which is null");
         HIPCX_REQUIRE(out->ndim == a->ndim - 1 + indices->ndim, HIPCX_DIMENSION_ERROR, "take: out has the wrong number of dimensions");
         TakeArgs t{};
         t.a = static_cast<const char*>(a->data);
@@ -234,9 +236,9 @@ extern "C" int hipcx_copy(const hipcx_array* a, const hipcx_array* out, void* st
 
 extern "C" int hipcx_add_at(const hipcx_array* a, const hipcx_array* indices, int8_t axis, const hipcx_array* b, const hipcx_array* out, int mode,
                             int32_t* error_flag, void* stream) {
-    int st = hipcx_copy(a, out, stream);  // out starts as a copy of a (same dtype: checked below before anything is added)
-    if (st != HIPCX_OK) return st;
     return Guard([&] {
+        ValidateArray(a, "a");
+        ValidateArray(out, "out");
         ValidateArray(indices, "indices");
         ValidateArray(b, "b");
         HIPCX_REQUIRE(axis >= 0 && axis < a->ndim, HIPCX_DIMENSION_ERROR, "add_at: axis out of range");
@@ -245,6 +247,8 @@ extern "C" int hipcx_add_at(const hipcx_array* a, const hipcx_array* indices, in
                       HIPCX_DTYPE_ERROR, "Only arrays of integer dtype can be used as indices.");
         HIPCX_REQUIRE(out->dtype == a->dtype && b->dtype == a->dtype, HIPCX_DTYPE_ERROR, "add_at: a, b and out must share a dtype");
         HIPCX_REQUIRE(mode >= HIPCX_BOUNDS_DEFAULT && mode <= HIPCX_BOUNDS_CLIP, HIPCX_CHAINERX_ERROR, "add_at: invalid bounds mode");
+        HIPCX_REQUIRE(error_flag != nullptr || mode == HIPCX_BOUNDS_WRAP || mode == HIPCX_BOUNDS_CLIP, HIPCX_CHAINERX_ERROR,
+                      "add_at: the default and raise bounds modes report out-of-range indices through error_flag, which is null");
         HIPCX_REQUIRE(SameShape(a, out), HIPCX_DIMENSION_ERROR, "add_at: out must have a's shape");
         HIPCX_REQUIRE(b->ndim == a->ndim - 1 + indices->ndim, HIPCX_DIMENSION_ERROR, "add_at: b has the wrong number of dimensions");
         TakeArgs t{};
@@ -283,9 +287,13 @@ extern "C" int hipcx_add_at(const hipcx_array* a, const hipcx_array* indices, in
             ++t.right.n;
         }
         t.total = t.left.total * t.right.total;
-        if (t.total == 0 || t.index.total == 0) return;
-        HIPCX_REQUIRE(t.axis_dim > 0, HIPCX_INDEX_ERROR, "add_at: cannot index an axis of extent 0");
+        const bool nothing_to_add = t.total == 0 || t.index.total == 0;
+        HIPCX_REQUIRE(nothing_to_add || t.axis_dim > 0, HIPCX_INDEX_ERROR, "add_at: cannot index an axis of extent 0");
         HIPCX_REQUIRE((t.total + 255) / 256 < (1LL << 31), HIPCX_NOT_IMPLEMENTED_ERROR, "add_at: problem too large for one launch");
+        // every argument is accepted: only now is out written, first as a copy of a
+        int copied = hipcx_copy(a, out, stream);
+        HIPCX_REQUIRE(copied == HIPCX_OK, copied, hipcx_last_error());
+        if (nothing_to_add) return;
         dim3 grid(static_cast<unsigned>((t.total + 255) / 256)), block(256);
         VisitDtype(out->dtype, [&](auto tag) {
             using T = typename decltype(tag)::type;

@@ -215,6 +215,15 @@ int hipcx_all(const hipcx_array* a, const int8_t* axis, int naxis, const hipcx_a
 int hipcx_any(const hipcx_array* a, const int8_t* axis, int naxis, const hipcx_array* out, void* workspace, size_t workspace_bytes,
               void* stream);
 
+/* hipcx_sum without a workspace argument.  No counterpart in the reference: it is for callers that cannot allocate device
+ * memory (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc) and so cannot provide the workspace
+ * hipcx_sum asks for.  The partial results live in a static device array of HIPCX_STATIC_SCRATCH_BYTES inside the library (one
+ * copy per device, held until the process ends); the call allocates and frees nothing.  Reductions whose
+ * hipcx_reduce_workspace_size exceeds that are refused with HIPCX_CHAINERX_ERROR.  Results are bit-identical to hipcx_sum's.
+ * Calls that overlap on one device share the array and race: issue them on one stream, or serialise them. */
+#define HIPCX_STATIC_SCRATCH_BYTES (4u << 20)
+int hipcx_sum_static_scratch(const hipcx_array* a, const int8_t* axis, int naxis, const hipcx_array* out, void* stream);
+
 /* ---- linear algebra / connection: CX/kernels/linalg.h:15, connection.h:21 ---- */
 /* out[M,N] = a[M,K] . b[K,N]; float16/32/64; fp16 accumulates in fp32 (CX/native/native_device/dot.cc:181-227). */
 size_t hipcx_dot_workspace_size(const hipcx_array* a, const hipcx_array* b, const hipcx_array* out);
@@ -361,9 +370,9 @@ int hipcx_average_pool_grad(const hipcx_array* gout, const int64_t* kernel_size,
 /* ---- indexing: TakeKernel CX/kernels/indexing.h:17 ----
  * `error_flag` is a device int32 the caller zeroes before the call; with mode DEFAULT/RAISE the
  * kernel stores 1 there when an index is out of range (the native backend raises IndexError,
- * CX/native/native_device/indexing.cc:68-74); the plugin reads it back and throws.  May be NULL,
- * in which case out-of-range indices are wrapped as the CUDA backend does
- * (CX/cuda/cuda_device/indexing.cu:58-66). */
+ * CX/native/native_device/indexing.cc:68-74); the plugin reads it back and throws.  It may be NULL
+ * only for the WRAP and CLIP modes; DEFAULT/RAISE without it is refused with HIPCX_CHAINERX_ERROR
+ * (no silent wrapping).  Nothing is written to `out` by a call that is refused. */
 int hipcx_take(const hipcx_array* a, const hipcx_array* indices, int8_t axis, const hipcx_array* out, int mode, int32_t* error_flag,
                void* stream);
 

@@ -190,3 +190,23 @@ def test_dot_long_reduction_few_tiles(dt, tol):
         assert_close(got.get(), ref, tol, 'dot %s %r' % (dt, (m, k, n)))
         out_t = chx.dot(chx.array(bt), chx.array(a).T)  # the same product transposed: [n, m]
         assert_close(out_t.get(), ref.T.copy(), tol, 'dot transposed %s %r' % (dt, (m, k, n)))
+
+
+@pytest.mark.parametrize('dt,tol', [('float32', 1e-5), ('float16', 2e-2)])
+def test_dot_staged_operands_with_split_reduction(dt, tol):
+    """128 to 256 output tiles over a reduction of 4096 or more with an operand that is not laid out along the reduction axis:
+    the operand is staged in the workspace and the reduction is split as well, so the float partial sums must lie behind the
+    staged copy, not on top of it.  Too large for the serial oracle loop: checked against the float64 product of the stored
+    values (the oracle's own result lies within the same bound of it)."""
+    import chainer_amd as chx
+    rng = np.random.default_rng(21)
+    for (m, k, n) in [(1536, 4096, 1536), (2048, 4096, 1024), (1536, 4100, 1300)]:
+        a = rng.standard_normal((m, k)).astype(dt)
+        b = (rng.standard_normal((k, n)) / np.sqrt(k)).astype(dt)
+        ref = (a.astype(np.float64) @ b.astype(np.float64)).astype(dt)
+        A_row, B_row = chx.array(a), chx.array(b)
+        A_t = chx.array(np.ascontiguousarray(a.T)).T
+        B_t = chx.array(np.ascontiguousarray(b.T)).T
+        for la, A in (('a row-major', A_row), ('a transposed view', A_t)):
+            for lb, B in (('b row-major', B_row), ('b transposed view', B_t)):
+                assert_close(chx.dot(A, B).get(), ref, tol, 'dot %s %r, %s, %s' % (dt, (m, k, n), la, lb))
