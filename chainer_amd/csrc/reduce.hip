@@ -25,7 +25,7 @@
 
 // Device memory for the partial results of hipcx_sum_static_scratch: part of the code object, so every device the library
 // runs on holds its own copy (at its own address) from the moment the module is loaded until the process ends.
-static __device__ __align__(256) __attribute__((used)) unsigned char scratch[HIPCX_STATIC_SCRATCH_BYTES];
+static __device__ __align__(256) unsigned char scratch[HIPCX_STATIC_SCRATCH_BYTES];
 
 namespace hipcx {
 namespace {
