@@ -424,6 +424,14 @@ void RunNchw(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, c
     a.x_bytes = static_cast<unsigned>(static_cast<int64_t>(a.N) * a.C * a.H * a.W * 2);
     const int RS = static_cast<int>(w->shape[2] * w->shape[3]);
     a.wp_bytes = static_cast<unsigned>(static_cast<int64_t>(a.K) * a.C * RS * 2);
+    a.div_P = FastDiv(a.P);
+    a.div_W = FastDiv(a.W);
+    a.div_OW = FastDiv(a.OW);
+    a.div_H2 = FastDiv(a.H + 2);
+    if (pl.taps == 9) {
+        a.div_wchunks = FastDiv(a.W / pl.npx);
+        a.div_percg = FastDiv(pl.nrow * (a.W / pl.npx));
+    }
     a.pair_load = (pl.taps == 1 && pl.npx == 1 && a.stride == 2 && a.W % 2 == 0) ? 1 : 0;
     a.out_ev = a.P % 8 == 0 ? 8 : a.P % 4 == 0 ? 4 : a.P % 2 == 0 ? 2 : 1;
     const bool w_dense = w->strides[1] == 2 && w->strides[0] == static_cast<int64_t>(a.C) * 2 && reinterpret_cast<uintptr_t>(w->data) % 16 == 0;

@@ -16,8 +16,9 @@
 // Both LDS arrays are exactly the operand layout of v_mfma_f32_32x32x16_f16 (lane = row/column, 8 consecutive
 // reduction indices per lane), so a fragment is one conflict-free ds_read_b128 of consecutive 16-byte groups, and
 // a 3x3 tap is a constant slot offset into the same patch: the patch is written once and read nine times.
-// Two LDS stages; chunk i+1 is written to LDS and the loads of chunk i+2 are issued before chunk i is multiplied;
-// one barrier per chunk.
+// Two LDS stages and a software pipeline laid out by hand: while chunk i is multiplied out of one stage, the registers that
+// hold chunk i+1 are transposed and written to the other stage and refilled with chunk i+2, one such operation after each
+// MFMA, and the operand fragments of the step after the next are read (three rotating fragment sets); one barrier per chunk.
 // All addresses are computed once per workgroup; inside the channel loop only a scalar offset advances, and
 // out-of-range loads are served as zeros by the buffer bounds check instead of branches.
 //
@@ -29,6 +30,21 @@
 #include "igemm.h"
 
 namespace hipcx {
+
+// Division of a non-negative int below 2^31 by a positive constant chosen on the host: q = (mulhi(n, mul) + n) >> shift.
+struct FastDiv {
+    unsigned mul = 1, shift = 0;
+    FastDiv() = default;
+    explicit FastDiv(int d) {
+        unsigned l = 0;
+        while ((1ull << l) < static_cast<unsigned long long>(d)) ++l;
+        mul = static_cast<unsigned>(((1ull << 32) * ((1ull << l) - static_cast<unsigned long long>(d))) / static_cast<unsigned long long>(d)) + 1u;
+        shift = l;
+    }
+    __device__ __forceinline__ int operator()(int n) const {
+        return static_cast<int>((__umulhi(static_cast<unsigned>(n), mul) + static_cast<unsigned>(n)) >> shift);
+    }
+};
 
 struct NchwConvArgs {
     const half_t* x;
@@ -58,6 +74,7 @@ struct NchwConvArgs {
     float bn_eps;
     const half_t* residual;
     int relu;
+    FastDiv div_P, div_W, div_OW, div_H2, div_wchunks, div_percg;  // by P, W, OW, H + 2, W / NPX, nrow * (W / NPX)
     int out_ev;   // pixels per output store: the largest of 8, 4, 2, 1 that divides P (a run then stays inside one image)
 };
 
@@ -135,11 +152,22 @@ __device__ __forceinline__ void Transpose8(const PixVec<NPX> (&in)[8], Bytes16 (
     }
 }
 
+template <int I, int N, typename F>
+__device__ __forceinline__ void StaticFor(F&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        StaticFor<I + 1, N>(f);
+    }
+}
+
 // KSPLIT = 2: a second set of WPX * WCH waves works on the same tile and takes every other channel chunk through LDS stages of
 // its own; the two accumulator sets are added through LDS before the epilogue.  For grids with at most one tile per compute unit
 // (7x7 planes, small batches) this doubles the waves and the loads in flight per unit, which is what bounds those layers.
 template <int TAPS, int WPX, int WCH, int CK, int NPX, int MAXI, int KSPLIT = 1>
-__global__ __launch_bounds__(64 * WPX * WCH * KSPLIT) void NchwConvKernel(NchwConvArgs p) {
+// Eight-wave workgroups that do not split the reduction are meant to run two to a compute unit (four waves per SIMD): they
+// are kept within 128 registers.
+__global__ __launch_bounds__(64 * WPX * WCH * KSPLIT) __attribute__((amdgpu_waves_per_eu(WPX * WCH >= 8 && KSPLIT == 1 ? 4 : 1, 8)))
+void NchwConvKernel(NchwConvArgs p) {
     constexpr int PW = 2, CW = 2;  // wave tile: 64 pixels x 64 channels
     constexpr int NT = 64 * WPX * WCH;       // threads of one reduction group
     constexpr int NT_ALL = NT * KSPLIT;
@@ -179,8 +207,8 @@ __global__ __launch_bounds__(64 * WPX * WCH * KSPLIT) void NchwConvKernel(NchwCo
     int base_row = 0, last_row = 0;
     if constexpr (TAPS == 9) {
         int m_last = min(m0 + BM, p.M) - 1;
-        int nf = m0 / p.P, hf = (m0 - nf * p.P) / p.W;
-        int nl = m_last / p.P, hl = (m_last - nl * p.P) / p.W;
+        int nf = p.div_P(m0), hf = p.div_W(m0 - nf * p.P);
+        int nl = p.div_P(m_last), hl = p.div_W(m_last - nl * p.P);
         base_row = nf * (p.H + 2) + hf;          // one above the first output row
         last_row = nl * (p.H + 2) + hl + 2;      // one below the last output row
     }
@@ -196,12 +224,12 @@ __global__ __launch_bounds__(64 * WPX * WCH * KSPLIT) void NchwConvKernel(NchwCo
         if constexpr (TAPS == 9) {
             const int wchunks = p.W / NPX;
             const int per_cg = p.nrow * wchunks;
-            int cg = it / per_cg;
+            int cg = p.div_percg(it);
             int q = it - cg * per_cg;
-            int pr = q / wchunks;
+            int pr = p.div_wchunks(q);
             int wc = q - pr * wchunks;
             int grow = base_row + pr;
-            int n = grow / (p.H + 2);
+            int n = p.div_H2(grow);
             int hh = grow - n * (p.H + 2) - 1;
             valid = cg < CG && grow <= last_row && n < p.N && hh >= 0 && hh < p.H;
             voff = (((n * p.C + cg * 8) * p.H + hh) * p.W + wc * NPX) * 2;
@@ -212,9 +240,9 @@ __global__ __launch_bounds__(64 * WPX * WCH * KSPLIT) void NchwConvKernel(NchwCo
             int q = it - cg * per_cg;
             int m = m0 + q * NPX;
             valid = cg < CG && m < p.M;
-            int n = m / p.P;
+            int n = p.div_P(m);
             int pix = m - n * p.P;
-            int oh = pix / p.OW;
+            int oh = p.div_OW(pix);
             int ow = pix - oh * p.OW;
             voff = (((n * p.C + cg * 8) * p.H + oh * p.stride) * p.W + ow * p.stride) * 2;
             loff = (cg * p.nslot + q * NPX) * 16;
@@ -253,39 +281,57 @@ __global__ __launch_bounds__(64 * WPX * WCH * KSPLIT) void NchwConvKernel(NchwCo
 
     PixVec<NPX> xreg[MAXI][8];
     Bytes16 wreg[WPT];
-    auto load_chunk = [&](int gi) {  // gi: chunk number inside this group; the groups interleave chunks
-        const int ci = gi * KSPLIT + kg;
-        const int xs = ci * CK * HW * 2;
+    // Side work of one loop iteration, cut into single operations that the loop deals out between its MFMAs:
+    //   activation slot i: one operation that transposes the registers loaded an iteration ago and writes them to LDS,
+    //                      then eight operations that each load one channel plane of the chunk after the next;
+    //   filter slot i:     one LDS write, one load.
+    constexpr int XOPS = MAXI * 9;
+    constexpr int NOPS = XOPS + WPT * 2;
+    int xs_next = 0, ws_next = 0;  // scalar offsets of the chunk being loaded
+    auto side = [&](auto op_tag, char* stage) {
+        constexpr int op = decltype(op_tag)::value;
+        if constexpr (op < XOPS) {
+            constexpr int i = op / 9, r = op % 9;
+            if constexpr (r == 0) {
+                Bytes16 t[NPX];
+                Transpose8<NPX>(xreg[i], t);
+                char* dst = xlds[i] >= 0 ? stage + xlds[i] : lds + dump_off;
 #pragma unroll
-        for (int i = 0; i < MAXI; ++i) {
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
+                for (int e = 0; e < NPX; ++e) *reinterpret_cast<Bytes16*>(dst + e * 16) = t[e];
+            } else {
+                constexpr int j = r - 1;
                 if (NPX == 1 && p.pair_load) {
-                    // strided gather: read the aligned dword that holds the wanted pixel in its low half.  Neighbouring
-                    // lanes then read neighbouring dwords (coalesced), where 2-byte loads 4 bytes apart are handled lane by lane.
-                    xreg[i][j].d[0] = __builtin_amdgcn_raw_buffer_load_b32(xr, xvoff[i], xs + j * HW * 2, 0);
+                    xreg[i][j].d[0] = __builtin_amdgcn_raw_buffer_load_b32(xr, xvoff[i], xs_next + j * HW * 2, 0);
                 } else {
-                    xreg[i][j] = BufLoad<NPX>(xr, xvoff[i], xs + j * HW * 2);
+                    xreg[i][j] = BufLoad<NPX>(xr, xvoff[i], xs_next + j * HW * 2);
                 }
             }
+        } else {
+            constexpr int q = op - XOPS, i = q / 2;
+            if constexpr (q % 2 == 0) {
+                char* dst = wlds[i] >= 0 ? stage + wlds[i] : lds + dump_off;
+                *reinterpret_cast<Bytes16*>(dst) = wreg[i];
+            } else {
+                wreg[i] = __builtin_amdgcn_raw_buffer_load_b128(wr, wvoff[i], ws_next, 0);
+            }
         }
-        const int ws = (TAPS == 1 && p.w_direct) ? ci * CK * 2 : ci * (CG * TAPS) * p.K * 16;
-#pragma unroll
-        for (int i = 0; i < WPT; ++i) wreg[i] = __builtin_amdgcn_raw_buffer_load_b128(wr, wvoff[i], ws, 0);
     };
-    auto store_chunk = [&](char* stage) {
-#pragma unroll
-        for (int i = 0; i < MAXI; ++i) {
-            Bytes16 t[NPX];
-            Transpose8<NPX>(xreg[i], t);
-            char* dst = xlds[i] >= 0 ? stage + xlds[i] : lds + dump_off;
-#pragma unroll
-            for (int e = 0; e < NPX; ++e) *reinterpret_cast<Bytes16*>(dst + e * 16) = t[e];
-        }
-#pragma unroll
-        for (int i = 0; i < WPT; ++i) {
-            if (wlds[i] >= 0) *reinterpret_cast<Bytes16*>(stage + wlds[i]) = wreg[i];
-        }
+    auto set_chunk = [&](int gi) {  // gi: chunk number inside this group; the groups interleave chunks
+        const int ci = gi * KSPLIT + kg;
+        xs_next = ci * CK * HW * 2;
+        ws_next = (TAPS == 1 && p.w_direct) ? ci * CK * 2 : ci * (CG * TAPS) * p.K * 16;
+    };
+    auto load_all = [&]() {
+        StaticFor<0, NOPS>([&](auto t) {
+            constexpr int op = decltype(t)::value;
+            if constexpr ((op < XOPS && op % 9 != 0) || (op >= XOPS && (op - XOPS) % 2 == 1)) side(t, lds);
+        });
+    };
+    auto store_all = [&](char* stage) {
+        StaticFor<0, NOPS>([&](auto t) {
+            constexpr int op = decltype(t)::value;
+            if constexpr ((op < XOPS && op % 9 == 0) || (op >= XOPS && (op - XOPS) % 2 == 0)) side(t, stage);
+        });
     };
 
     // ---- fragment addresses ----
@@ -296,9 +342,9 @@ __global__ __launch_bounds__(64 * WPX * WCH * KSPLIT) void NchwConvKernel(NchwCo
         int slot;
         if constexpr (TAPS == 9) {
             int mm = m < p.M ? m : p.M - 1;
-            int n = mm / p.P;
+            int n = p.div_P(mm);
             int pix = mm - n * p.P;
-            int h = pix / p.W;
+            int h = p.div_W(pix);
             int w = pix - h * p.W;
             slot = (n * (p.H + 2) + h + 1 - base_row) * W2 + w + 1;
             slot -= W2 + 1;  // tap (r, s) adds r * W2 + s
@@ -320,57 +366,82 @@ __global__ __launch_bounds__(64 * WPX * WCH * KSPLIT) void NchwConvKernel(NchwCo
         }
     }
 
-    // One channel chunk out of a stage.  Fragments are double-buffered by hand: the reads of step i+1 are issued
-    // before the MFMAs of step i, and the scheduling groups keep that order in the instruction stream.
-    auto compute = [&](const char* stage) {
-        constexpr int NSTEP = TAPS * KS;
-        Bytes16 af[2][PW], bf[2][CW];
-        auto read_frags = [&](int st, Bytes16(&fa)[PW], Bytes16(&fb)[CW]) {
-            const int tap = st / KS, ks = st % KS;
-            const int toff = TAPS == 9 ? ((tap / 3) * W2 + (tap % 3)) * 16 : 0;
-#pragma unroll
-            for (int a = 0; a < PW; ++a) fa[a] = *reinterpret_cast<const Bytes16*>(stage + aoff[a] + toff + ks * a_ks);
-#pragma unroll
-            for (int b = 0; b < CW; ++b) {
-                fb[b] = *reinterpret_cast<const Bytes16*>(stage + boff + ks * 2 * WCGP + (tap * BN + b * 32) * 16);
-            }
-        };
-        read_frags(0, af[0], bf[0]);
-#pragma unroll
-        for (int st = 0; st < NSTEP; ++st) {
-            if (st + 1 < NSTEP) read_frags(st + 1, af[(st + 1) & 1], bf[(st + 1) & 1]);
-#pragma unroll
-            for (int a = 0; a < PW; ++a) {
-#pragma unroll
-                for (int b = 0; b < CW; ++b) MfmaTile<half_t>(af[st & 1][a], bf[st & 1][b], acc[a][b]);
-            }
-            if (st + 1 < NSTEP) __builtin_amdgcn_sched_group_barrier(0x100, PW + CW, 0);  // DS reads of the next step
-            __builtin_amdgcn_sched_group_barrier(0x008, PW * CW, 0);                      // MFMAs of this step
+    // One loop iteration: chunk ci is multiplied out of `cur` while the registers that hold chunk ci+1 go to `nxt` and are
+    // refilled with chunk ci+2.  The instruction stream is laid out by hand (every sched_barrier pins what precedes it):
+    // after each MFMA one fragment read of the step after the next (fragments live in three rotating register sets, so a
+    // read has two steps = 8 MFMAs to land) and this slot's share of the side operations.  The matrix pipe never waits for
+    // the load path: LDS writes and buffer loads issue in the shadow of the MFMAs.
+    constexpr int NSTEP = TAPS * KS;
+    constexpr int NSLOT = NSTEP * PW * CW;
+    Bytes16 af[3][PW], bf[3][CW];
+    auto read_frag = [&](const char* stage, auto st_tag, auto q_tag) {
+        constexpr int st = decltype(st_tag)::value, q = decltype(q_tag)::value;
+        constexpr int tap = st / KS, ks = st % KS;
+        const int toff = TAPS == 9 ? ((tap / 3) * W2 + (tap % 3)) * 16 : 0;
+        if constexpr (q < PW) {
+            af[st % 3][q] = *reinterpret_cast<const Bytes16*>(stage + aoff[q] + toff + ks * a_ks);
+        } else {
+            constexpr int b = q - PW;
+            bf[st % 3][b] = *reinterpret_cast<const Bytes16*>(stage + boff + ks * 2 * WCGP + (tap * BN + b * 32) * 16);
         }
+    };
+    auto iteration = [&](const char* cur, char* nxt, auto stores_tag, auto loads_tag) {
+        constexpr bool STORES = decltype(stores_tag)::value, LOADS = decltype(loads_tag)::value;
+        StaticFor<0, (NSTEP < 2 ? NSTEP : 2)>([&](auto st) { StaticFor<0, PW + CW>([&](auto q) { read_frag(cur, st, q); }); });
+        __builtin_amdgcn_sched_barrier(0);
+        StaticFor<0, NSTEP>([&](auto st_tag) {
+            constexpr int st = decltype(st_tag)::value;
+            StaticFor<0, PW * CW>([&](auto q_tag) {
+                constexpr int q = decltype(q_tag)::value;
+                constexpr int a = q / CW, b = q % CW;
+                constexpr int slot = st * PW * CW + q;
+                MfmaTile<half_t>(af[st % 3][a], bf[st % 3][b], acc[a][b]);
+                __builtin_amdgcn_sched_barrier(0);
+                if constexpr (st + 2 < NSTEP) {  // PW + CW reads over PW * CW slots
+                    StaticFor<q * (PW + CW) / (PW * CW), (q + 1) * (PW + CW) / (PW * CW)>(
+                            [&](auto f) { read_frag(cur, std::integral_constant<int, st + 2>{}, f); });
+                }
+                StaticFor<slot * NOPS / NSLOT, (slot + 1) * NOPS / NSLOT>([&](auto op_tag) {
+                    constexpr int op = decltype(op_tag)::value;
+                    constexpr bool is_load = (op < XOPS && op % 9 != 0) || (op >= XOPS && (op - XOPS) % 2 == 1);
+                    if constexpr (is_load ? LOADS : STORES) side(op_tag, nxt);
+                });
+                __builtin_amdgcn_sched_barrier(0);
+            });
+        });
     };
 
     // ---- pipeline ----
-    // Stage (ci & 1) holds chunk ci.  At the top of iteration ci the registers hold chunk ci+1, loaded one whole
-    // iteration ago: they go to the other stage (free since the barrier that ended iteration ci-1), the loads of chunk
-    // ci+2 are issued into the same registers, and only then chunk ci is multiplied.  No wave ever waits for a load it
-    // has just issued, and the LDS writes of one wave overlap the MFMAs of the others.
+    // Stage (ci & 1) holds chunk ci.  Loads run two chunks ahead of the multiplication, through registers.  The last two
+    // iterations are compiled without the loads (and the last one without the LDS writes) they would have no use for.
     const int nchunks = p.C / CK / KSPLIT;  // per group; the host only picks KSPLIT when it divides the chunk count
-    load_chunk(0);
+    using True = std::integral_constant<bool, true>;
+    using False = std::integral_constant<bool, false>;
+    set_chunk(0);
+    load_all();
     if constexpr (TAPS == 9) {  // borders of all patches must read as zero; nothing ever writes them
         for (int off = tid_all * 16; off < KSPLIT * 2 * stage_bytes; off += NT_ALL * 16) *reinterpret_cast<Bytes16*>(lds + off) = Bytes16(0);
         __syncthreads();
     }
-    store_chunk(glds);
-    if (nchunks > 1) load_chunk(1);
+    store_all(glds);
+    if (nchunks > 1) {
+        set_chunk(1);
+        load_all();
+    }
     __syncthreads();
-    for (int ci = 0; ci < nchunks; ++ci) {
-        char* cur = glds + (ci & 1) * stage_bytes;
-        char* nxt = glds + ((ci + 1) & 1) * stage_bytes;
-        if (ci + 1 < nchunks) store_chunk(nxt);
-        if (ci + 2 < nchunks) load_chunk(ci + 2);
-        compute(cur);
+    int ci = 0;
+    for (; ci + 2 < nchunks; ++ci) {
+        set_chunk(ci + 2);
+        iteration(glds + (ci & 1) * stage_bytes, glds + ((ci + 1) & 1) * stage_bytes, True{}, True{});
         __syncthreads();
     }
+    if (ci + 1 < nchunks) {
+        iteration(glds + (ci & 1) * stage_bytes, glds + ((ci + 1) & 1) * stage_bytes, True{}, False{});
+        __syncthreads();
+        ++ci;
+    }
+    iteration(glds + (ci & 1) * stage_bytes, glds + ((ci + 1) & 1) * stage_bytes, False{}, False{});
+    __syncthreads();
 
     // ---- the second group hands its sums over (the loop's last barrier has retired every stage read) ----
     if constexpr (KSPLIT > 1) {
@@ -439,8 +510,6 @@ __global__ __launch_bounds__(64 * WPX * WCH * KSPLIT) void NchwConvKernel(NchwCo
             }
         }
     };
-    using True = std::integral_constant<bool, true>;
-    using False = std::integral_constant<bool, false>;
     const bool has_bn = p.bn_gamma != nullptr;
     const bool relu_here = p.relu && p.residual == nullptr;  // with a residual, ReLU follows the addition
     if (kg == 0) {
@@ -466,7 +535,7 @@ __global__ __launch_bounds__(64 * WPX * WCH * KSPLIT) void NchwConvKernel(NchwCo
             const int cc = (tid_all % (CPR > NT_ALL ? NT_ALL : CPR)) + cj * NT_ALL;
             const int m = m0 + cc * EV;
             if (m >= p.M) continue;
-            const int img = m / p.P;
+            const int img = p.div_P(m);
             const int pix = m - img * p.P;
             const int64_t obase = static_cast<int64_t>(img) * p.K * p.P + pix;
             for (int row = (CPR > NT_ALL ? 0 : tid_all / CPR); row < BN; row += ROW_STEP) {
