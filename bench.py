@@ -81,9 +81,9 @@ def main():
     eager_ms = (time.perf_counter() - t0) / 3 * 1e3
     graph = None
     if not args.eager:
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            y = step()
+        from chainer_amd.graph import capture
+        graph = capture(step)
+        y = graph.result
         graph.replay()
         torch.cuda.synchronize()
         eager_out = step().get()
@@ -145,11 +145,8 @@ def main():
     if not args.eager:
         def fstep():
             return cfg.resnet50_forward_fused(chx, params, x)
-        yf = fstep()
-        torch.cuda.synchronize()
-        fgraph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(fgraph):
-            yf = fstep()
+        fgraph = capture(fstep)
+        yf = fgraph.result
         for _ in range(max(args.warmup, 1)):
             fgraph.replay()
         torch.cuda.synchronize()

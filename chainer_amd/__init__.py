@@ -5,9 +5,10 @@
 ``libhipcx.so``; every routine decomposes into kernel calls exactly as the reference routine does.
 """
 from chainer_amd import _lib
-from chainer_amd._lib import (ChainerxError, DimensionError, DtypeError, ChainerxNotImplementedError, ChainerxIndexError,
+from chainer_amd._lib import (OutOfMemoryError, ChainerxError, DimensionError, DtypeError, ChainerxNotImplementedError, ChainerxIndexError,
                               BackendError, DeviceError)
-from chainer_amd._array import ndarray, array, to_numpy, synchronize, device_available
+from chainer_amd._array import (ndarray, array, to_numpy, synchronize, device_available, memory_arena, pool_stats,
+                                free_unused_blocks)
 from chainer_amd.routines import *  # noqa: F401,F403
 from chainer_amd import routines
 

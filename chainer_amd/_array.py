@@ -2,8 +2,10 @@
 
 It plays the role of ``chainerx.ndarray`` for the harness and the tests: a (buffer, offset, shape,
 byte-strides, dtype) tuple, with views made on the host and every arithmetic operation forwarded
-to one C-ABI kernel call.  PyTorch only owns the device buffer (its caching allocator stands in
-for the plugin's memory pool) and the stream.
+to one C-ABI kernel call.  Device memory comes from the library's own pool (``hipcx_malloc`` /
+``hipcx_free``) and crosses the host boundary through its copy entry points
+(``hipcx_from_host_memory``, ``hipcx_memcpy_to_host``): the Device interface of the backend.
+PyTorch is only asked for the current stream (and captures HIP graphs in the benchmarks).
 """
 import ctypes
 
@@ -70,9 +72,80 @@ def contiguous_strides(shape, itemsize):
     return tuple(reversed(st))
 
 
+DEVICE_INDEX = 0
+
+
+class DeviceBuffer(object):
+    """One allocation of the backend's memory pool (Device::Allocate, CX/device.h:33); returned to the pool when the last
+    array that refers to it goes away, like the deleter of the reference's ``shared_ptr<void>``."""
+
+    __slots__ = ('ptr', 'nbytes', '__weakref__')
+
+    def __init__(self, nbytes):
+        _require_device()
+        self.nbytes = int(nbytes)
+        out = ctypes.c_void_p()
+        _lib.call('hipcx_malloc', DEVICE_INDEX, max(self.nbytes, 1), ctypes.byref(out))
+        self.ptr = out.value or 0
+
+    @classmethod
+    def adopt(cls, ptr, nbytes):
+        """Takes ownership of a pointer the pool has already handed out (hipcx_from_host_memory)."""
+        self = cls.__new__(cls)
+        self.ptr = int(ptr or 0)
+        self.nbytes = int(nbytes)
+        return self
+
+    def data_ptr(self):
+        return self.ptr
+
+    def __del__(self):
+        ptr, self.ptr = self.ptr, 0
+        if ptr:
+            try:
+                _lib.load().hipcx_free(DEVICE_INDEX, ctypes.c_void_p(ptr))
+            except Exception:  # interpreter shutdown: the library may be gone already
+                pass
+
+
 def alloc_bytes(nbytes):
-    _require_device()
-    return torch().empty(max(int(nbytes), 1), dtype=torch().uint8, device='cuda:0')
+    return DeviceBuffer(nbytes)
+
+
+def pool_stats():
+    """Counters of the device memory pool (hipcx_pool_stats)."""
+    st = _lib.CPoolStats()
+    _lib.call('hipcx_pool_stats', DEVICE_INDEX, ctypes.byref(st))
+    return {name: int(getattr(st, name)) for name, _ in _lib.CPoolStats._fields_}
+
+
+def free_unused_blocks():
+    """MemoryPool::FreeUnusedBlocks (CX/cuda/memory_pool.cc:172-203)."""
+    _lib.call('hipcx_pool_free_unused', DEVICE_INDEX)
+
+
+_next_arena = [1]
+
+
+class memory_arena(object):
+    """Allocations made inside the ``with`` block come from, and return to, free lists of their own.  A HIP graph is
+    captured inside one (after an eager pass in the same arena has filled its free lists, so that the capture itself never
+    reaches the driver): the addresses baked into the graph are then not handed to anybody else until ``release()``."""
+
+    def __init__(self):
+        self.id = _next_arena[0]
+        _next_arena[0] += 1
+
+    def __enter__(self):
+        _lib.call('hipcx_pool_set_arena', DEVICE_INDEX, self.id)
+        return self
+
+    def __exit__(self, *exc):
+        _lib.call('hipcx_pool_set_arena', DEVICE_INDEX, 0)
+        return False
+
+    def release(self):
+        _lib.call('hipcx_pool_release_arena', DEVICE_INDEX, self.id)
 
 
 class ndarray(object):
@@ -295,10 +368,11 @@ class ndarray(object):
         """Device -> host (numpy) copy; synchronises like Array::ToNative (CX/array.cc:399-444)."""
         a = self.as_contiguous()
         n = a.size * a.itemsize
+        host = numpy.empty(a.shape, a.dtype)
         if n == 0:
-            return numpy.empty(a.shape, a.dtype)
-        host = a._buf[a._offset:a._offset + n].cpu().numpy()
-        return host.view(a.dtype).reshape(a.shape).copy()
+            return host
+        _lib.call('hipcx_memcpy_to_host', DEVICE_INDEX, ctypes.c_void_p(host.ctypes.data), ctypes.c_void_p(a._ptr), n, current_stream())
+        return host
 
     def __array__(self, dtype=None, copy=None):
         a = self.get()
@@ -395,8 +469,9 @@ def array(obj, dtype=None):
     _require_device()
     if a.size == 0:
         return ndarray.empty(a.shape, a.dtype)
-    host = torch().from_numpy(a.reshape(-1).view(numpy.uint8))
-    buf = host.to('cuda:0')
+    out = ctypes.c_void_p()
+    _lib.call('hipcx_from_host_memory', DEVICE_INDEX, ctypes.c_void_p(a.ctypes.data), a.nbytes, ctypes.byref(out), current_stream())
+    buf = DeviceBuffer.adopt(out.value, a.nbytes)
     return ndarray(buf, 0, a.shape, contiguous_strides(a.shape, a.dtype.itemsize), a.dtype)
 
 

@@ -40,6 +40,10 @@ class DeviceError(ChainerxError):
     pass
 
 
+class OutOfMemoryError(ChainerxError, MemoryError):
+    """chainerx::cuda::OutOfMemoryError (CX/cuda/memory_pool.h:34-37)."""
+
+
 _STATUS_TO_EXC = {
     1: ChainerxError,
     2: DimensionError,
@@ -48,6 +52,7 @@ _STATUS_TO_EXC = {
     5: ChainerxIndexError,
     6: BackendError,
     7: DeviceError,
+    8: OutOfMemoryError,
 }
 
 
@@ -59,6 +64,11 @@ class CArray(ctypes.Structure):
         ('shape', ctypes.c_int64 * MAX_NDIM),
         ('strides', ctypes.c_int64 * MAX_NDIM),
     ]
+
+
+class CPoolStats(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_uint64) for n in ('in_use_bytes', 'cached_bytes', 'in_use_blocks', 'cached_blocks',
+                                               'device_allocations', 'retries')]
 
 
 class CScalar(ctypes.Structure):
@@ -104,6 +114,18 @@ SIGNATURES = {
     'hipcx_device_count': (_INT, [ctypes.POINTER(ctypes.c_int)]),
     'hipcx_synchronize': (_INT, [_INT]),
     'hipcx_device_name': (_INT, [_INT, ctypes.c_char_p, _SZ]),
+    'hipcx_malloc': (_INT, [_INT, _SZ, ctypes.POINTER(ctypes.c_void_p)]),
+    'hipcx_free': (_INT, [_INT, _V]),
+    'hipcx_pool_free_unused': (_INT, [_INT]),
+    'hipcx_pool_stats': (_INT, [_INT, ctypes.POINTER(CPoolStats)]),
+    'hipcx_pool_set_arena': (_INT, [_INT, _INT]),
+    'hipcx_pool_release_arena': (_INT, [_INT, _INT]),
+    'hipcx_pool_destroy': (_INT, [_INT]),
+    'hipcx_memcpy_from_host': (_INT, [_INT, _V, _V, _SZ, _V]),
+    'hipcx_memcpy_to_host': (_INT, [_INT, _V, _V, _SZ, _V]),
+    'hipcx_memcpy_device': (_INT, [_INT, _V, _INT, _V, _SZ, _V]),
+    'hipcx_from_host_memory': (_INT, [_INT, _V, _SZ, ctypes.POINTER(ctypes.c_void_p), _V]),
+    'hipcx_check_device_pointer': (_INT, [_INT, _V]),
     'hipcx_add': (_INT, [_A, _A, _A, _V]),
     'hipcx_add_as': (_INT, [_A, _S, _A, _V]),
     'hipcx_subtract': (_INT, [_A, _A, _A, _V]),

@@ -50,14 +50,13 @@ def device_time(fn, iters=20, warmup=5, rounds=3):
 def graph_time(fn, iters=20):
     """Seconds per replay of `fn` captured into a HIP graph (launch overhead of its kernels removed)."""
     import torch
-    fn()
-    torch.cuda.synchronize()
-    g = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(g):
-        fn()
+    from chainer_amd.graph import capture
+    g = capture(fn)
     g.replay()
     torch.cuda.synchronize()
-    return device_time(g.replay, iters, 3)
+    seconds = device_time(g.replay, iters, 3)
+    g.release()
+    return seconds
 
 
 def cpu_time(fn, min_s=0.2):

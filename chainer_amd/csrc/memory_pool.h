@@ -1,0 +1,215 @@
+// Device / pinned-host memory pool of the hip backend (host code only: no HIP headers, so that the class can be
+// built and exercised with a fake allocator on a machine without a GPU).
+//
+// Role in the reference: chainerx::cuda::MemoryPool (CX/cuda/memory_pool.{h,cc}) behind CudaDevice::Allocate
+// (CX/cuda/cuda_device/memory.cc:17-26).  Kept from it: the 512-byte allocation unit (memory_pool.h:29), Malloc(0) ==
+// nullptr (memory_pool.cc:209-211), "release every cached block and try once more" before an allocation is reported as
+// out of memory (memory_pool.cc:236-243), Free of a pointer the pool does not know is an error (memory_pool.cc:262-264),
+// a noexcept free for deleters (memory_pool.cc:296-302) and deleters that outlive the pool (weak_ptr,
+// cuda_device/memory.cc:19-24).
+//
+// Different by design (sized for one process owning a 288 GB device, launches on HIP streams and graphs):
+//  * no splitting and merging of chunks: requests are rounded to size classes (512-byte units up to 4 KiB, then steps of
+//    1/8 of the size, then whole 2 MiB pages from 16 MiB on) and a freed block serves later requests of its class only --
+//    O(log classes) per call, no neighbour bookkeeping, at most 12.5 % of slack per block;
+//  * arenas: a block remembers the arena it was allocated in and returns to that arena's free lists.  A HIP graph is
+//    captured inside an arena of its own, so the addresses baked into the graph are never handed to anybody else
+//    until the arena is released (the graph destroyed);
+//  * when the device allocator reports failure only the general arena's cache is released: the blocks of a graph's
+//    arena stay where the graph expects them.
+#pragma once
+
+#include <atomic>
+#include <cstddef>
+#include <cstdint>
+#include <functional>
+#include <map>
+#include <memory>
+#include <mutex>
+#include <stdexcept>
+#include <string>
+#include <unordered_map>
+#include <utility>
+#include <vector>
+
+namespace hipcx {
+
+constexpr size_t kAllocationUnit = 512;  // CX/cuda/memory_pool.h:29 kAllocationUnitSize
+
+// What the pool allocates from (CX/cuda/memory_pool.h:48-78: Allocator, DeviceMemoryAllocator, PinnedMemoryAllocator).
+class Allocator {
+public:
+    virtual ~Allocator() = default;
+    virtual bool Malloc(void** ptr, size_t bytes) = 0;  // false: out of memory (any other failure throws)
+    virtual void Free(void* ptr) noexcept = 0;
+};
+
+class OutOfMemoryError : public std::runtime_error {  // CX/cuda/memory_pool.h:34-37
+public:
+    explicit OutOfMemoryError(size_t bytes) : std::runtime_error("Out of memory allocating " + std::to_string(bytes) + " bytes.") {}
+};
+
+struct PoolStats {
+    size_t in_use_bytes = 0;     // handed out and not yet freed (rounded sizes)
+    size_t cached_bytes = 0;     // free blocks held for reuse, all arenas
+    size_t in_use_blocks = 0;
+    size_t cached_blocks = 0;
+    size_t allocator_calls = 0;  // successful Allocator::Malloc calls so far
+    size_t retries = 0;          // allocations that only succeeded after the cache was released
+};
+
+class MemoryPool {
+public:
+    explicit MemoryPool(std::unique_ptr<Allocator> allocator) : allocator_(std::move(allocator)) {}
+    // Gives everything back to the allocator, blocks still in use included (CX/cuda/memory_pool.cc:160-170): once the pool
+    // is gone the memory is gone; deleters made by MakeShared notice and do nothing.
+    ~MemoryPool() {
+        for (auto& kv : in_use_) allocator_->Free(kv.first);
+        for (auto& arena : free_) {
+            for (auto& bin : arena.second) {
+                for (void* p : bin.second) allocator_->Free(p);
+            }
+        }
+    }
+    MemoryPool(const MemoryPool&) = delete;
+    MemoryPool& operator=(const MemoryPool&) = delete;
+
+    static size_t RoundSize(size_t bytes) {
+        size_t units = (bytes + kAllocationUnit - 1) / kAllocationUnit;
+        if (bytes >= (16u << 20)) {  // whole 2 MiB pages
+            constexpr size_t kPage = 2u << 20;
+            return (bytes + kPage - 1) / kPage * kPage;
+        }
+        if (units <= 8) return units * kAllocationUnit;
+        // steps of 1/8 of the power of two below: 8, 9, ..., 16, 18, ..., 32, 36, ...
+        size_t p = 8;
+        while (p * 2 <= units) p *= 2;
+        size_t step = p / 8;
+        return (units + step - 1) / step * step * kAllocationUnit;
+    }
+
+    // nullptr for 0 bytes; throws OutOfMemoryError when the allocator fails twice.  `arena`: see SetArena().
+    void* Malloc(size_t bytes) { return Malloc(bytes, current_arena_.load()); }
+    void* Malloc(size_t bytes, int arena) {
+        if (bytes == 0) return nullptr;
+        const size_t size = RoundSize(bytes);
+        std::lock_guard<std::mutex> lock(mutex_);
+        void* ptr = nullptr;
+        auto a = free_.find(arena);
+        if (a != free_.end()) {
+            auto bin = a->second.find(size);
+            if (bin != a->second.end() && !bin->second.empty()) {
+                ptr = bin->second.back();
+                bin->second.pop_back();
+                stats_.cached_bytes -= size;
+                --stats_.cached_blocks;
+            }
+        }
+        if (ptr == nullptr) {
+            if (!allocator_->Malloc(&ptr, size)) {
+                ReleaseCachedLocked();
+                ++stats_.retries;
+                if (!allocator_->Malloc(&ptr, size)) {
+                    --stats_.retries;
+                    throw OutOfMemoryError(bytes);
+                }
+            }
+            ++stats_.allocator_calls;
+        }
+        in_use_.emplace(ptr, Block{size, arena});
+        stats_.in_use_bytes += size;
+        ++stats_.in_use_blocks;
+        return ptr;
+    }
+
+    // Returns the block to the free lists of the arena it came from.  Throws for a pointer that is not in use.
+    void Free(void* ptr) {
+        if (ptr == nullptr) return;
+        std::lock_guard<std::mutex> lock(mutex_);
+        auto it = in_use_.find(ptr);
+        if (it == in_use_.end()) throw std::runtime_error("Cannot free out-of-pool memory");
+        const Block b = it->second;
+        in_use_.erase(it);
+        stats_.in_use_bytes -= b.size;
+        --stats_.in_use_blocks;
+        free_[b.arena][b.size].push_back(ptr);
+        stats_.cached_bytes += b.size;
+        ++stats_.cached_blocks;
+    }
+    void FreeNoExcept(void* ptr) noexcept {
+        try {
+            Free(ptr);
+        } catch (...) {
+        }
+    }
+
+    // Gives the cached blocks of the general arena back to the allocator (MemoryPool::FreeUnusedBlocks, memory_pool.cc:172-203).
+    void FreeUnusedBlocks() {
+        std::lock_guard<std::mutex> lock(mutex_);
+        ReleaseCachedLocked();
+    }
+
+    // Allocations made through Malloc(bytes) from now on belong to `arena` (0 is the general arena).  One setting for the
+    // pool, not per thread: a HIP graph is captured by one thread while the others are idle.
+    void SetArena(int arena) { current_arena_.store(arena); }
+    int arena() const { return current_arena_.load(); }
+    // The cached blocks of `arena` join the general arena; blocks of it still in use will follow when they are freed.
+    void ReleaseArena(int arena) {
+        if (arena == 0) return;
+        std::lock_guard<std::mutex> lock(mutex_);
+        auto a = free_.find(arena);
+        if (a != free_.end()) {
+            for (auto& bin : a->second) {
+                auto& dst = free_[0][bin.first];
+                dst.insert(dst.end(), bin.second.begin(), bin.second.end());
+            }
+            free_.erase(a);
+        }
+        for (auto& kv : in_use_) {
+            if (kv.second.arena == arena) kv.second.arena = 0;
+        }
+        int expected = arena;
+        current_arena_.compare_exchange_strong(expected, 0);
+    }
+
+    PoolStats stats() const {
+        std::lock_guard<std::mutex> lock(mutex_);
+        return stats_;
+    }
+
+    // shared_ptr whose deleter returns the block if the pool is still alive and does nothing otherwise
+    // (the ownership rule of Device::Allocate results, CX/cuda/cuda_device/memory.cc:17-26).
+    static std::shared_ptr<void> MakeShared(const std::shared_ptr<MemoryPool>& pool, size_t bytes) {
+        std::weak_ptr<MemoryPool> weak = pool;
+        return std::shared_ptr<void>(pool->Malloc(bytes), [weak](void* p) noexcept {
+            if (std::shared_ptr<MemoryPool> alive = weak.lock()) alive->FreeNoExcept(p);
+        });
+    }
+
+private:
+    struct Block {
+        size_t size;
+        int arena;
+    };
+    void ReleaseCachedLocked() {
+        auto a = free_.find(0);
+        if (a == free_.end()) return;
+        for (auto& bin : a->second) {
+            for (void* p : bin.second) {
+                allocator_->Free(p);
+                stats_.cached_bytes -= bin.first;
+                --stats_.cached_blocks;
+            }
+        }
+        free_.erase(a);
+    }
+
+    std::unique_ptr<Allocator> allocator_;
+    mutable std::mutex mutex_;
+    std::unordered_map<void*, Block> in_use_;
+    std::map<int, std::map<size_t, std::vector<void*>>> free_;  // arena -> rounded size -> blocks
+    std::atomic<int> current_arena_{0};
+    PoolStats stats_;
+};
+
+}  // namespace hipcx

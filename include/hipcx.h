@@ -17,7 +17,8 @@
  *  - Return value: 0 on success, otherwise a `hipcx_status` naming the ChainerX exception type
  *    (CX/error.h:48-95) the plugin must throw; `hipcx_last_error()` gives the message.
  *  - Kernels that need device scratch memory take `workspace`/`workspace_bytes`; the matching
- *    `*_workspace_size` function tells how much.  The library itself never allocates.
+ *    `*_workspace_size` function tells how much.  No kernel entry point allocates; device memory
+ *    comes from the caller, who may get it from the pool below (hipcx_malloc).
  */
 #ifndef HIPCX_H_
 #define HIPCX_H_
@@ -51,7 +52,8 @@ typedef enum hipcx_status { /* CX/error.h:48-95 */
     HIPCX_NOT_IMPLEMENTED_ERROR = 4,
     HIPCX_INDEX_ERROR = 5,
     HIPCX_BACKEND_ERROR = 6,
-    HIPCX_DEVICE_ERROR = 7
+    HIPCX_DEVICE_ERROR = 7,
+    HIPCX_OUT_OF_MEMORY_ERROR = 8 /* chainerx::cuda::OutOfMemoryError, CX/cuda/memory_pool.h:34-37 */
 } hipcx_status;
 
 typedef enum hipcx_scalar_kind { /* CX/dtype.h DtypeKind */
@@ -93,6 +95,49 @@ int hipcx_version(void);
 int hipcx_device_count(int* count);          /* Backend::GetDeviceCount, CX/backend.h:29 */
 int hipcx_synchronize(int device_index);     /* Device::Synchronize, CX/device.h:71 */
 int hipcx_device_name(int device_index, char* buf, size_t buf_len);
+
+/* ---- device memory: chainerx::Device (CX/device.h:24-71) as the CUDA backend implements it (CX/cuda/cuda_device/memory.cc) ----
+ * Allocation goes through a pool per device (role of chainerx::cuda::MemoryPool, CX/cuda/memory_pool.{h,cc}): 512-byte
+ * allocation units, freed blocks are cached and reused, and when the driver reports out of memory the cached blocks are
+ * released and the allocation is tried once more before HIPCX_OUT_OF_MEMORY_ERROR is returned (memory_pool.cc:236-243).
+ *   hipcx_malloc            Device::Allocate, device.h:33 (0 bytes -> NULL, CX/native/native_device/memory.cc:14-19)
+ *   hipcx_free              the deleter of an allocation (cuda_device/memory.cc:19-24): returns the block to the pool; a pointer
+ *                           the pool does not hold is HIPCX_CHAINERX_ERROR (memory_pool.cc:262-264); after hipcx_pool_destroy
+ *                           it does nothing (the pool took its memory with it)
+ *   hipcx_pool_free_unused  MemoryPool::FreeUnusedBlocks, memory_pool.cc:172-203
+ *   hipcx_pool_destroy      ~MemoryPool (memory_pool.cc:160-170): waits for the device, then gives every block back to the driver
+ *   hipcx_memcpy_from_host  Device::MemoryCopyFrom with a native source = MemoryCopyFromHostAsync (cuda_device/memory.cc:37-51): the
+ *                           bytes are staged in pooled page-locked memory and copied asynchronously on `stream`; `src` may be
+ *                           reused as soon as the call returns
+ *   hipcx_memcpy_to_host    Device::MemoryCopyTo with a native destination (cuda_device/memory.cc:104-122): ordered behind the work
+ *                           queued on `stream`, complete when the call returns
+ *   hipcx_memcpy_device     MemoryCopyFrom / MemoryCopyTo between hip devices (cuda_device/memory.cc:84-91,110-113), asynchronous
+ *   hipcx_from_host_memory  Device::FromHostMemory, device.h:64 = Allocate + MemoryCopyFromHostAsync (cuda_device/memory.cc:146-150);
+ *                           TransferDataFrom / TransferDataTo (device.h:49-60) are hipcx_malloc + one of the copies above
+ *   hipcx_check_device_pointer  the check of Device::MakeDataFromForeignPointer (cuda_device/memory.cc:53-75)
+ * Arenas have no counterpart in the reference: allocations made after hipcx_pool_set_arena(device, a) with a > 0 come from, and
+ * return to, free lists of their own, so the addresses a HIP graph captured in arena a refers to are not handed to anybody else
+ * until hipcx_pool_release_arena(device, a).  Arena 0 is the general one.  The setting is per device, not per thread. */
+typedef struct hipcx_pool_stats_t {
+    uint64_t in_use_bytes;       /* handed out, rounded sizes */
+    uint64_t cached_bytes;       /* free blocks held for reuse */
+    uint64_t in_use_blocks;
+    uint64_t cached_blocks;
+    uint64_t device_allocations; /* hipMalloc calls that succeeded so far */
+    uint64_t retries;            /* allocations that only succeeded after the cache was released */
+} hipcx_pool_stats_t;
+int hipcx_malloc(int device, size_t bytes, void** ptr);
+int hipcx_free(int device, void* ptr);
+int hipcx_pool_free_unused(int device);
+int hipcx_pool_stats(int device, hipcx_pool_stats_t* stats);
+int hipcx_pool_set_arena(int device, int arena);
+int hipcx_pool_release_arena(int device, int arena);
+int hipcx_pool_destroy(int device);
+int hipcx_memcpy_from_host(int device, void* dst, const void* src, size_t bytes, void* stream);
+int hipcx_memcpy_to_host(int device, void* dst, const void* src, size_t bytes, void* stream);
+int hipcx_memcpy_device(int dst_device, void* dst, int src_device, const void* src, size_t bytes, void* stream);
+int hipcx_from_host_memory(int device, const void* src, size_t bytes, void** out, void* stream);
+int hipcx_check_device_pointer(int device, const void* ptr);
 
 /* ---- elementwise arithmetic: CX/kernels/arithmetic.h ---- */
 /* Inputs must already have out's dtype (the plugin applies AsType as CX/native/kernel_regist.h:55-56 does). */
