@@ -82,10 +82,11 @@ class DeviceBuffer(object):
     __slots__ = ('ptr', 'nbytes', '__weakref__')
 
     def __init__(self, nbytes):
+        self.ptr = 0
         _require_device()
         self.nbytes = int(nbytes)
         out = ctypes.c_void_p()
-        _lib.call('hipcx_malloc', DEVICE_INDEX, max(self.nbytes, 1), ctypes.byref(out))
+        _lib.call('hipcx_malloc_on_stream', DEVICE_INDEX, max(self.nbytes, 1), current_stream(), ctypes.byref(out))
         self.ptr = out.value or 0
 
     @classmethod

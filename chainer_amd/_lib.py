@@ -115,6 +115,7 @@ SIGNATURES = {
     'hipcx_synchronize': (_INT, [_INT]),
     'hipcx_device_name': (_INT, [_INT, ctypes.c_char_p, _SZ]),
     'hipcx_malloc': (_INT, [_INT, _SZ, ctypes.POINTER(ctypes.c_void_p)]),
+    'hipcx_malloc_on_stream': (_INT, [_INT, _SZ, _V, ctypes.POINTER(ctypes.c_void_p)]),
     'hipcx_free': (_INT, [_INT, _V]),
     'hipcx_pool_free_unused': (_INT, [_INT]),
     'hipcx_pool_stats': (_INT, [_INT, ctypes.POINTER(CPoolStats)]),

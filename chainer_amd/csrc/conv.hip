@@ -4,6 +4,7 @@
 // (CX/native/native_device/dot.cc:181-227, conv.cc:41-89).
 #include <algorithm>
 #include <cstdlib>
+#include <mutex>
 #include <utility>
 #include <vector>
 
@@ -27,11 +28,13 @@ struct ProfileState {
     double bytes = 0.0;
 };
 ProfileState g_profile;
+std::mutex g_profile_mutex;  // launches from several host threads may record into one profiling window
 
 struct ProfileScope {
     hipStream_t stream;
     hipEvent_t stop = nullptr;
     ProfileScope(hipStream_t s, double flops, double bytes) : stream(s) {
+        std::lock_guard<std::mutex> lock(g_profile_mutex);
         if (!g_profile.on) return;
         hipEvent_t start = nullptr;
         HIPCX_CHECK_HIP(hipEventCreate(&start));
@@ -45,6 +48,24 @@ struct ProfileScope {
         if (stop != nullptr) (void)hipEventRecord(stop, stream);
     }
 };
+
+// Raises a kernel's dynamic LDS limit when a launch needs more than it has been given so far.  The limit is a property of the
+// function on one device; several host threads may launch the same kernel, so the bookkeeping is per kernel instantiation
+// (the Tag type), per device, and serialised (the reference serialises its launchers on a mutex too, CX/cuda/elementwise.cuh:38).
+template <typename Tag>
+void EnsureDynamicLds(const void* kernel, int lds_bytes) {
+    constexpr int kMaxDevices = 64;
+    static std::mutex mu;
+    static int configured[kMaxDevices] = {};
+    int dev = 0;
+    HIPCX_CHECK_HIP(hipGetDevice(&dev));
+    HIPCX_REQUIRE(dev >= 0 && dev < kMaxDevices, HIPCX_DEVICE_ERROR, "device index out of range");
+    std::lock_guard<std::mutex> lock(mu);
+    if (lds_bytes > configured[dev]) {
+        HIPCX_CHECK_HIP(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes));
+        configured[dev] = lds_bytes;
+    }
+}
 
 template <typename T, int WM, int WN, bool PM>
 void LaunchShape(IGemmArgs<T> p, bool fast16, bool fast8, hipStream_t stream) {
@@ -73,19 +94,13 @@ void LaunchShape(IGemmArgs<T> p, bool fast16, bool fast8, hipStream_t stream) {
         constexpr int lds_bytes = PipeLdsBytes<T, WM, WN, PM>();
         if (fast16) {
             auto kern = IGemmPipeKernel<T, WM, WN, 16, PM>;
-            static bool configured = false;
-            if (!configured) {
-                HIPCX_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes));
-                configured = true;
-            }
+            struct Tag16 {};
+            EnsureDynamicLds<Tag16>(reinterpret_cast<const void*>(kern), lds_bytes);
             hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, p);
         } else {
             auto kern = IGemmPipeKernel<T, WM, WN, 8, PM>;
-            static bool configured = false;
-            if (!configured) {
-                HIPCX_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes));
-                configured = true;
-            }
+            struct Tag8 {};
+            EnsureDynamicLds<Tag8>(reinterpret_cast<const void*>(kern), lds_bytes);
             hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, p);
         }
     } else if (fast16) {
@@ -223,12 +238,8 @@ bool TrySmallDot(const hipcx_array* a, const hipcx_array* b, const hipcx_array* 
         }
         p.nw = best_nw;
         const int lds_bytes = best_nw * 2 * 32 * 144;
-        static const bool configured = [] {
-            HIPCX_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(SmallDotRowsKernel<T>), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                8 * 2 * 32 * 144));
-            return true;
-        }();
-        (void)configured;
+        struct RowsTag {};
+        EnsureDynamicLds<RowsTag>(reinterpret_cast<const void*>(SmallDotRowsKernel<T>), 8 * 2 * 32 * 144);
         hipLaunchKernelGGL((SmallDotRowsKernel<T>), dim3(static_cast<unsigned>(blocks)), dim3(64 * best_nw), lds_bytes, stream, p);
         CheckLaunch("small_dot_rows");
         return true;
@@ -367,11 +378,8 @@ NchwPlan PlanNchw(const hipcx_array* x, const hipcx_array* w, const hipcx_array*
 template <int TAPS, int WPX, int WCH, int CK, int NPX, int MAXI, int KSPLIT = 1>
 void LaunchNchwKernel(const NchwConvArgs& a, int lds_bytes, hipStream_t stream) {
     auto kern = NchwConvKernel<TAPS, WPX, WCH, CK, NPX, MAXI, KSPLIT>;
-    static int configured = 0;
-    if (lds_bytes > configured) {
-        HIPCX_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes));
-        configured = lds_bytes;
-    }
+    struct Tag {};  // a type of its own for every instantiation of this launcher
+    EnsureDynamicLds<Tag>(reinterpret_cast<const void*>(kern), lds_bytes);
     int64_t total = static_cast<int64_t>(a.tiles_m) * a.tiles_n;
     dim3 grid(static_cast<unsigned>((total + 7) / 8 * 8)), block(64 * WPX * WCH * KSPLIT);
     hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, a);
@@ -542,11 +550,8 @@ void RunStem(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, c
     ProfileScope prof(stream, 2.0 * M * 64 * 3 * 49,
                       2.0 * (static_cast<double>(a.N) * 3 * a.H * a.W + 64.0 * 3 * 49 + M * 64));
     auto kern = StemConv7x7s2Kernel<3>;
-    static int configured = 0;
-    if (pl.lds_bytes > configured) {
-        HIPCX_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, pl.lds_bytes));
-        configured = pl.lds_bytes;
-    }
+    struct StemTag {};
+    EnsureDynamicLds<StemTag>(reinterpret_cast<const void*>(kern), pl.lds_bytes);
     int blocks = a.N * ((a.OH + 1) / 2);
     hipLaunchKernelGGL(kern, dim3(blocks), dim3(256), pl.lds_bytes, stream, a);
     CheckLaunch("stem_conv");
@@ -759,6 +764,7 @@ extern "C" {
 
 int hipcx_profile_start(void) {
     return Guard([&] {
+        std::lock_guard<std::mutex> lock(g_profile_mutex);
         HIPCX_REQUIRE(!g_profile.on, HIPCX_CHAINERX_ERROR, "profiling is already on");
         g_profile = ProfileState{};
         g_profile.on = true;
@@ -767,6 +773,7 @@ int hipcx_profile_start(void) {
 
 int hipcx_profile_stop(int64_t* launches, double* total_ms, double* flops, double* bytes) {
     return Guard([&] {
+        std::lock_guard<std::mutex> lock(g_profile_mutex);
         HIPCX_REQUIRE(g_profile.on, HIPCX_CHAINERX_ERROR, "profiling is not on");
         g_profile.on = false;
         double ms = 0.0;

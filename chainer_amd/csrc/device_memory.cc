@@ -4,6 +4,7 @@
 #include <array>
 #include <cstring>
 #include <deque>
+#include <map>
 
 #include "common.h"
 #include "memory_pool.h"
@@ -77,6 +78,16 @@ struct DeviceState {
     std::shared_ptr<MemoryPool> pinned_pool;
     std::mutex keeper_mutex;
     std::deque<std::pair<hipEvent_t, std::shared_ptr<void>>> keeper;
+    std::mutex partition_mutex;
+    std::map<hipStream_t, uint32_t> partitions;  // stream -> partition of the device pool (the null stream is partition 0)
+
+    uint32_t PartitionOf(hipStream_t stream) {
+        if (stream == nullptr) return 0;
+        std::lock_guard<std::mutex> lock(partition_mutex);
+        auto it = partitions.find(stream);
+        if (it == partitions.end()) it = partitions.emplace(stream, static_cast<uint32_t>(partitions.size() + 1)).first;
+        return it->second;
+    }
 
     void Collect() {
         std::lock_guard<std::mutex> lock(keeper_mutex);
@@ -170,14 +181,17 @@ using namespace hipcx;
 
 extern "C" {
 
-int hipcx_malloc(int device, size_t bytes, void** ptr) {
+int hipcx_malloc_on_stream(int device, size_t bytes, void* stream, void** ptr) {
     return GuardMemory([&] {
         HIPCX_REQUIRE(ptr != nullptr, HIPCX_CHAINERX_ERROR, "ptr is null");
         *ptr = nullptr;
         if (bytes == 0) return;  // Allocate(0) is a null pointer (CX/native/native_device/memory.cc:14-19)
-        *ptr = StateOf(device)->device_pool->Malloc(bytes);
+        std::shared_ptr<DeviceState> st = StateOf(device);
+        *ptr = st->device_pool->Malloc(bytes, st->PartitionOf(AsStream(stream)));
     });
 }
+
+int hipcx_malloc(int device, size_t bytes, void** ptr) { return hipcx_malloc_on_stream(device, bytes, nullptr, ptr); }
 
 int hipcx_free(int device, void* ptr) {
     return GuardMemory([&] {
@@ -285,7 +299,7 @@ int hipcx_from_host_memory(int device, const void* src, size_t bytes, void** out
         if (bytes == 0) return;
         HIPCX_REQUIRE(src != nullptr, HIPCX_CHAINERX_ERROR, "from_host_memory: src is null");
         std::shared_ptr<DeviceState> st = StateOf(device);
-        void* dst = st->device_pool->Malloc(bytes);
+        void* dst = st->device_pool->Malloc(bytes, st->PartitionOf(AsStream(stream)));
         try {
             UploadAsync(*st, device, dst, src, bytes, AsStream(stream));
         } catch (...) {

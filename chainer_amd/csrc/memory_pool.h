@@ -15,6 +15,10 @@
 //  * arenas: a block remembers the arena it was allocated in and returns to that arena's free lists.  A HIP graph is
 //    captured inside an arena of its own, so the addresses baked into the graph are never handed to anybody else
 //    until the arena is released (the graph destroyed);
+//  * partitions: inside an arena, a freed block is only reused by allocations of the same partition.  The device layer
+//    uses one partition per HIP stream: work queued on a stream runs in order, so a block freed and reallocated on one
+//    stream needs no synchronisation, while another stream never gets it (the reference launches everything on one
+//    stream and has no such problem);
 //  * when the device allocator reports failure only the general arena's cache is released: the blocks of a graph's
 //    arena stay where the graph expects them.
 #pragma once
@@ -89,10 +93,11 @@ public:
     }
 
     // nullptr for 0 bytes; throws OutOfMemoryError when the allocator fails twice.  `arena`: see SetArena().
-    void* Malloc(size_t bytes) { return Malloc(bytes, current_arena_.load()); }
-    void* Malloc(size_t bytes, int arena) {
+    void* Malloc(size_t bytes, uint32_t partition = 0) { return Malloc(bytes, current_arena_.load(), partition); }
+    void* Malloc(size_t bytes, int arena_number, uint32_t partition) {
         if (bytes == 0) return nullptr;
         const size_t size = RoundSize(bytes);
+        const uint64_t arena = Key(arena_number, partition);
         std::lock_guard<std::mutex> lock(mutex_);
         void* ptr = nullptr;
         auto a = free_.find(arena);
@@ -153,20 +158,25 @@ public:
     // pool, not per thread: a HIP graph is captured by one thread while the others are idle.
     void SetArena(int arena) { current_arena_.store(arena); }
     int arena() const { return current_arena_.load(); }
-    // The cached blocks of `arena` join the general arena; blocks of it still in use will follow when they are freed.
+    // The cached blocks of `arena` join the general arena (each in its partition); blocks of it still in use will follow
+    // when they are freed.
     void ReleaseArena(int arena) {
         if (arena == 0) return;
         std::lock_guard<std::mutex> lock(mutex_);
-        auto a = free_.find(arena);
-        if (a != free_.end()) {
+        for (auto a = free_.begin(); a != free_.end();) {
+            if (ArenaOf(a->first) != arena) {
+                ++a;
+                continue;
+            }
+            auto& general = free_[Key(0, PartitionOf(a->first))];
             for (auto& bin : a->second) {
-                auto& dst = free_[0][bin.first];
+                auto& dst = general[bin.first];
                 dst.insert(dst.end(), bin.second.begin(), bin.second.end());
             }
-            free_.erase(a);
+            a = free_.erase(a);
         }
         for (auto& kv : in_use_) {
-            if (kv.second.arena == arena) kv.second.arena = 0;
+            if (ArenaOf(kv.second.arena) == arena) kv.second.arena = Key(0, PartitionOf(kv.second.arena));
         }
         int expected = arena;
         current_arena_.compare_exchange_strong(expected, 0);
@@ -179,9 +189,9 @@ public:
 
     // shared_ptr whose deleter returns the block if the pool is still alive and does nothing otherwise
     // (the ownership rule of Device::Allocate results, CX/cuda/cuda_device/memory.cc:17-26).
-    static std::shared_ptr<void> MakeShared(const std::shared_ptr<MemoryPool>& pool, size_t bytes) {
+    static std::shared_ptr<void> MakeShared(const std::shared_ptr<MemoryPool>& pool, size_t bytes, uint32_t partition = 0) {
         std::weak_ptr<MemoryPool> weak = pool;
-        return std::shared_ptr<void>(pool->Malloc(bytes), [weak](void* p) noexcept {
+        return std::shared_ptr<void>(pool->Malloc(bytes, partition), [weak](void* p) noexcept {
             if (std::shared_ptr<MemoryPool> alive = weak.lock()) alive->FreeNoExcept(p);
         });
     }
@@ -189,25 +199,32 @@ public:
 private:
     struct Block {
         size_t size;
-        int arena;
+        uint64_t arena;  // Key(arena, partition)
     };
-    void ReleaseCachedLocked() {
-        auto a = free_.find(0);
-        if (a == free_.end()) return;
-        for (auto& bin : a->second) {
-            for (void* p : bin.second) {
-                allocator_->Free(p);
-                stats_.cached_bytes -= bin.first;
-                --stats_.cached_blocks;
+    static uint64_t Key(int arena, uint32_t partition) { return (static_cast<uint64_t>(static_cast<uint32_t>(arena)) << 32) | partition; }
+    static int ArenaOf(uint64_t key) { return static_cast<int>(key >> 32); }
+    static uint32_t PartitionOf(uint64_t key) { return static_cast<uint32_t>(key & 0xffffffffu); }
+    void ReleaseCachedLocked() {  // every partition of the general arena
+        for (auto a = free_.begin(); a != free_.end();) {
+            if (ArenaOf(a->first) != 0) {
+                ++a;
+                continue;
             }
+            for (auto& bin : a->second) {
+                for (void* p : bin.second) {
+                    allocator_->Free(p);
+                    stats_.cached_bytes -= bin.first;
+                    --stats_.cached_blocks;
+                }
+            }
+            a = free_.erase(a);
         }
-        free_.erase(a);
     }
 
     std::unique_ptr<Allocator> allocator_;
     mutable std::mutex mutex_;
     std::unordered_map<void*, Block> in_use_;
-    std::map<int, std::map<size_t, std::vector<void*>>> free_;  // arena -> rounded size -> blocks
+    std::map<uint64_t, std::map<size_t, std::vector<void*>>> free_;  // (arena, partition) -> rounded size -> blocks
     std::atomic<int> current_arena_{0};
     PoolStats stats_;
 };

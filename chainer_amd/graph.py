@@ -28,11 +28,15 @@ def capture(fn):
     """Runs ``fn()`` once eagerly and once under capture; returns a CapturedGraph."""
     t = torch()
     arena = memory_arena()
+    # both passes run on one side stream: the pool keeps the blocks of different streams apart
+    stream = t.cuda.Stream()
+    stream.wait_stream(t.cuda.current_stream())
     with arena:
-        out = fn()
-        t.cuda.synchronize()
+        with t.cuda.stream(stream):
+            out = fn()
+        stream.synchronize()
         del out
         graph = t.cuda.CUDAGraph()
-        with t.cuda.graph(graph):
+        with t.cuda.graph(graph, stream=stream):
             out = fn()
     return CapturedGraph(graph, out, arena)

@@ -14,6 +14,9 @@
  *  - Scalars follow `chainerx::Scalar` (CX/scalar.h): a kind tag plus an int64 or a double.
  *  - Every call is asynchronous on `stream` (a `hipStream_t`, may be NULL for the default
  *    stream), like the CUDA backend (CX/cuda/elementwise.cuh:41-47).
+ *  - Every entry point may be called from several host threads at once (CX/testing/threading.h:34-60 is how the
+ *    reference tests that); state shared between calls is guarded inside the library.  The exceptions say so:
+ *    hipcx_sum_static_scratch (one scratch array per device) and the profiling window (one per process).
  *  - Return value: 0 on success, otherwise a `hipcx_status` naming the ChainerX exception type
  *    (CX/error.h:48-95) the plugin must throw; `hipcx_last_error()` gives the message.
  *  - Kernels that need device scratch memory take `workspace`/`workspace_bytes`; the matching
@@ -115,6 +118,10 @@ int hipcx_device_name(int device_index, char* buf, size_t buf_len);
  *   hipcx_from_host_memory  Device::FromHostMemory, device.h:64 = Allocate + MemoryCopyFromHostAsync (cuda_device/memory.cc:146-150);
  *                           TransferDataFrom / TransferDataTo (device.h:49-60) are hipcx_malloc + one of the copies above
  *   hipcx_check_device_pointer  the check of Device::MakeDataFromForeignPointer (cuda_device/memory.cc:53-75)
+ * hipcx_malloc_on_stream has no counterpart either (the reference launches everything on one stream): a block allocated for
+ * `stream` is, once freed, only handed to later allocations for the same stream, so work queued on different streams (e.g. by
+ * different host threads) never shares a block that may still be in use; hipcx_malloc is the null stream's variant, and
+ * hipcx_from_host_memory allocates for the stream it copies on.  hipcx_free needs no stream: a block remembers where it belongs.
  * Arenas have no counterpart in the reference: allocations made after hipcx_pool_set_arena(device, a) with a > 0 come from, and
  * return to, free lists of their own, so the addresses a HIP graph captured in arena a refers to are not handed to anybody else
  * until hipcx_pool_release_arena(device, a).  Arena 0 is the general one.  The setting is per device, not per thread. */
@@ -127,6 +134,7 @@ typedef struct hipcx_pool_stats_t {
     uint64_t retries;            /* allocations that only succeeded after the cache was released */
 } hipcx_pool_stats_t;
 int hipcx_malloc(int device, size_t bytes, void** ptr);
+int hipcx_malloc_on_stream(int device, size_t bytes, void* stream, void** ptr);
 int hipcx_free(int device, void* ptr);
 int hipcx_pool_free_unused(int device);
 int hipcx_pool_stats(int device, hipcx_pool_stats_t* stats);
@@ -315,7 +323,7 @@ int hipcx_lstm_cell(const hipcx_array* c, const hipcx_array* x, const hipcx_arra
 /* Measurement aid (no counterpart in the reference): between start and stop every implicit-GEMM launch made by
  * hipcx_dot / hipcx_conv from the calling process is bracketed by a pair of HIP events on its stream.  stop waits for them
  * and returns the number of launches, the sum of their durations, and their algorithmic flops (2 per multiply-add) and
- * bytes (each operand once).  Not thread-safe; one profiling window at a time. */
+ * bytes (each operand once).  One profiling window per process at a time; launches from any thread are recorded into it. */
 int hipcx_profile_start(void);
 int hipcx_profile_stop(int64_t* launches, double* total_ms, double* flops, double* bytes);
 

@@ -179,6 +179,37 @@ static void TestArenas() {
     pool.Free(r);
 }
 
+static void TestPartitions() {
+    auto fs = std::make_shared<FakeState>();
+    fs->capacity = 64 * 1024;
+    MemoryPool pool(std::unique_ptr<Allocator>(new FakeAllocator(fs)));
+    void* a = pool.Malloc(4096, 1u);  // "stream 1"
+    pool.Free(a);
+    void* b = pool.Malloc(4096, 2u);  // "stream 2" must not get stream 1's block
+    CHECK(b != a);
+    void* c = pool.Malloc(4096, 1u);  // stream 1 does
+    CHECK(c == a);
+    pool.Free(b);
+    pool.Free(c);
+    // arenas and partitions combine: a graph arena's block stays in its partition when the arena is released
+    pool.SetArena(3);
+    void* g = pool.Malloc(8192, 2u);
+    pool.Free(g);
+    pool.SetArena(0);
+    CHECK(pool.Malloc(8192, 2u) != g);
+    pool.ReleaseArena(3);
+    void* h1 = pool.Malloc(8192, 1u);
+    CHECK(h1 != g);
+    void* h2 = pool.Malloc(8192, 2u);
+    CHECK(h2 == g);
+    // out of memory releases every partition of the general arena
+    size_t cached_before = pool.stats().cached_blocks;
+    CHECK(cached_before >= 2);
+    void* big = pool.Malloc(40 * 1024, 5u);
+    CHECK(big != nullptr);
+    CHECK(pool.stats().cached_blocks == 0);
+}
+
 static void TestThreads() {
     auto fs = std::make_shared<FakeState>();
     fs->capacity = size_t{1} << 26;
@@ -209,6 +240,7 @@ int main() {
     TestRetryThenOutOfMemory();
     TestDeleterOutlivesPool();
     TestArenas();
+    TestPartitions();
     TestThreads();
     if (g_failures != 0) {
         std::printf("%d check(s) failed\n", g_failures);

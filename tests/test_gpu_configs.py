@@ -21,8 +21,8 @@ def test_mlp_full_size():
     x, t = cfg.mlp_input()
     y1, l1 = cfg.mlp_forward(chx, to_dev(chx, cfg, p), chx.array(x), chx.array(t))
     y2, l2 = cfg.mlp_forward(O, p, x, t)
-    assert_close(y1.get(), y2, 1e-5, 'logits')
-    assert_close(l1.get(), l2, 1e-5, 'loss')
+    assert_close(y1.get(), y2, 1e-5, 'logits', elementwise=True)
+    assert_close(l1.get(), l2, 1e-5, 'loss', elementwise=True)
     assert_exact(chx.argmax(y1, 1).get(), O.argmax(y2, 1), 'predictions')
 
 
@@ -32,7 +32,7 @@ def test_cifar_convnet():
     from chainer_amd import configs as cfg
     p = cfg.cifar_params()
     x = cfg.cifar_input(batch=4)
-    assert_close(cfg.cifar_forward(chx, to_dev(chx, cfg, p), chx.array(x)).get(), cfg.cifar_forward(O, p, x), 1e-5)
+    assert_close(cfg.cifar_forward(chx, to_dev(chx, cfg, p), chx.array(x)).get(), cfg.cifar_forward(O, p, x), 1e-5, 'cifar logits', elementwise=True)
 
 
 def test_resnet50_fp16_against_oracle_and_batch_invariance():
@@ -46,7 +46,7 @@ def test_resnet50_fp16_against_oracle_and_batch_invariance():
     ref = cfg.resnet50_forward(O, p, x[:2])
     y2 = cfg.resnet50_forward(chx, pd, chx.array(x[:2])).get()
     assert np.isfinite(ref.astype(np.float32)).all()
-    assert_close(y2, ref, 2e-2, 'batch 2 vs oracle')
+    assert_close(y2, ref, 2e-2, 'batch 2 vs oracle', elementwise=True)
     assert np.array_equal(y2.argmax(1), ref.argmax(1))
     y128 = cfg.resnet50_forward(chx, pd, chx.array(x)).get()
     assert y128.shape == (128, 1000) and np.isfinite(y128.astype(np.float32)).all()
@@ -63,7 +63,7 @@ def test_lstm_language_model():
     ids = cfg.lstm_lm_input(batch=8, seq=5, vocab=1000)
     o1, h1, c1 = cfg.lstm_lm_forward(chx, to_dev(chx, cfg, p), chx.array(ids), chx.zeros)
     o2, h2, c2 = cfg.lstm_lm_forward(O, p, ids, np.zeros)
-    assert_close(o1.get(), o2, 1e-5, 'log-probabilities')
+    assert_close(o1.get(), o2, 1e-5, 'log-probabilities', elementwise=True)
     assert_close(h1[1].get(), h2[1], 1e-5, 'h')
     assert_close(c1[0].get(), c2[0], 1e-5, 'c')
     # full-size model, two time steps (the oracle's 650x10000 projection takes about a second per step)
@@ -71,5 +71,5 @@ def test_lstm_language_model():
     ids = cfg.lstm_lm_input(seq=2)
     o1, h1, _ = cfg.lstm_lm_forward(chx, to_dev(chx, cfg, p), chx.array(ids), chx.zeros)
     o2, h2, _ = cfg.lstm_lm_forward(O, p, ids, np.zeros)
-    assert_close(o1.get(), o2, 1e-5, 'full-size log-probabilities')
+    assert_close(o1.get(), o2, 1e-5, 'full-size log-probabilities', elementwise=True)
     assert_exact(chx.argmax(o1, 1).get(), O.argmax(o2, 1), 'full-size predictions')

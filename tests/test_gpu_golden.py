@@ -2,7 +2,7 @@
 import numpy as np
 import pytest
 
-from test_oracle_pins import GOLDEN, run_golden, SORTING_LITERALS
+from test_oracle_pins import GOLDEN, run_golden, SORTING_LITERALS, block_tie_rows
 from helpers import upload_view
 
 pytestmark = pytest.mark.gpu
@@ -33,3 +33,28 @@ def test_argmax_reference_literals(x, axis):
         got = chx.argmax(upload_view(chx, x.astype(dt)) if x.ndim else chx.array(xa), axis).get()
         assert got.dtype == np.int64
         assert np.array_equal(got, np.argmax(xa, axis))
+
+
+def test_argmax_block_tie_literals():
+    """The hand-traced tie cases of tests/golden/argmax_block_ties.json (the later 32-element block wins; traces in
+    tests/golden/README.md) through the hip ArgMax / ArgMin kernels: as a 1-D array (row kernel), as rows of a matrix, as a
+    strided column (column kernels), and spread over a long row that is split across workgroups."""
+    import chainer_amd as chx
+    for dt in (np.float32, np.float16, np.float64, np.int32, np.int8):
+        for name, row, expected, mirrored in block_tie_rows(dt):
+            what = '%s %s' % (name, np.dtype(dt))
+            assert int(chx.argmax(chx.array(row), 0).get()) == expected, what
+            assert int(chx.argmin(chx.array(mirrored), 0).get()) == expected, what
+            m = np.stack([row, row[::-1].copy(), row])
+            got = chx.argmax(chx.array(m), 1).get()
+            assert got[0] == expected and got[2] == expected, what
+            assert int(chx.argmax(chx.array(np.ascontiguousarray(m.T)), 0).get()[0]) == expected, what
+    # the same rule far out in a long row (blocks merged by the binary counter across workgroup boundaries): the oracle, itself
+    # held to the literals above, is the reference here
+    from oracle import native as O
+    rng = np.random.default_rng(3)
+    x = rng.integers(-100, 100, (3, 300000)).astype(np.float32)
+    for r, positions in enumerate([(5, 40, 299999), (70000, 131072, 131073), (31, 32, 262144)]):
+        x[r, list(positions)] = 1000
+    assert np.array_equal(chx.argmax(chx.array(x), 1).get(), O.argmax(x, 1))
+    assert np.array_equal(chx.argmin(chx.array(-x), 1).get(), O.argmin(-x, 1))

@@ -278,7 +278,7 @@ def test_argmax_reference_literals(x, axis):
 
 def test_argmax_tie_free_and_in_block_ties():
     """C: without ties the answer is unique (= numpy.argmax); ties inside one 32-element block and in the <=3-element
-    tail resolve to the first index like numpy (reduce.h:28-31,65,69-72).  The rule between blocks is unpinned."""
+    tail resolve to the first index like numpy (reduce.h:28-31,65,69-72).  The rule between blocks: test_argmax_block_tie_literals."""
     rng = np.random.default_rng(6)
     for n in (1, 5, 31, 32, 33, 100, 4096, 70001):
         x = rng.permutation(n * 3).reshape(3, n).astype(np.float32)
@@ -289,6 +289,36 @@ def test_argmax_tie_free_and_in_block_ties():
     x = rng.integers(0, 3, (200, 35)).astype(np.float32)
     x[:, :32] -= 10  # maximum lives in the 3-element tail
     assert np.array_equal(O.argmax(x, 1), x.argmax(1))
+
+
+def block_tie_rows(dtype, lo=-50, hi=40):
+    """(name, row, expected argmax, mirrored row whose argmin is the same index) for every hand-traced case of
+    tests/golden/argmax_block_ties.json: the maximum at the listed positions, distinct smaller values elsewhere."""
+    cases = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), 'golden', 'argmax_block_ties.json')))['cases']
+    rows = []
+    for c in cases:
+        n = c['length']
+        rng = np.random.default_rng(n * 7 + len(c['max_at']))
+        row = rng.integers(lo, hi, n).astype(np.float64)
+        row[c['max_at']] = hi + 3
+        rows.append((c['name'], row.astype(dtype), c['expected'], (-row).astype(dtype)))
+    return rows
+
+
+def test_argmax_block_tie_literals():
+    """R-by-hand: the tie rule between 32-element blocks (the later block wins), traced through the reference's
+    PairwiseReduction in tests/golden/README.md; a first-index-wins (numpy) or last-index-wins rule fails several cases."""
+    numpy_rule = last_rule = 0
+    for dt in (np.float32, np.float16, np.float64, np.int32, np.int8):
+        for name, row, expected, mirrored in block_tie_rows(dt):
+            assert int(O.argmax(row, 0)) == expected, (name, dt)
+            assert int(O.argmin(mirrored, 0)) == expected, (name, dt)
+            m = np.stack([row, row[::-1].copy(), row])  # as rows of a matrix, and as a column of its transpose
+            assert int(O.argmax(m, 1)[0]) == expected and int(O.argmax(m, 1)[2]) == expected, (name, dt)
+            assert int(O.argmax(np.ascontiguousarray(m.T), 0)[0]) == expected, (name, dt)
+            numpy_rule += int(np.argmax(row)) != expected
+            last_rule += (len(row) - 1 - int(np.argmax(row[::-1]))) != expected
+    assert numpy_rule > 0 and last_rule > 0  # the fixture tells the rule apart from both simple ones
 
 
 def test_argmax_nan_rule():
