@@ -48,6 +48,8 @@ struct SumImpl {
     using In = In_;
     using Out = Out_;
     using Acc = std::conditional_t<std::is_same<Out_, half_t>::value, float, Out_>;
+    using Row = SumImpl;
+    __device__ static Acc FromRow(Acc a, int64_t) { return a; }
     static constexpr bool kSerialFold = true;
     static constexpr bool kHasIndex = false;
     __device__ static Acc Identity() { return Acc(0); }
@@ -117,6 +119,8 @@ struct AMaxImpl {
     using Out = T;
     // half values are compared as floats (exact and order preserving); bool as int
     using Acc = std::conditional_t<std::is_same<T, half_t>::value, float, std::conditional_t<std::is_same<T, bool>::value, int, T>>;
+    using Row = AMaxImpl;
+    __device__ static Acc FromRow(Acc a, int64_t) { return a; }
     static constexpr bool kSerialFold = false;
     static constexpr bool kHasIndex = false;
     __device__ static Acc Identity() { return static_cast<Acc>(MIN ? MaxOrInf<T>() : LowestOrInf<T>()); }
@@ -130,24 +134,28 @@ struct AMaxImpl {
     __device__ static Acc Shfl(Acc a, int src) { return __shfl(a, src); }
 };
 
-template <typename V>
+template <typename V, typename I = int64_t>
 struct MaxIdx {
     V v;
-    int64_t i;  // < 0: empty / identity
+    I i;  // < 0: empty / identity
 };
 
 // MIN: ArgMin (`accum.min > next.min`), the mirror image of ArgMax (native/native_device/reduction.cc:34-92).
-template <typename T, bool MIN = false>
+// I: type of the index that travels with the value.  The row kernel counts from the first element of its block (at most
+// 65536 + 3 elements, Row below) and widens when it hands the result on (FromRow); every other kernel uses int64_t.
+template <typename T, bool MIN = false, typename I = int64_t>
 struct ArgMaxImpl {
     using In = T;
     using Out = int64_t;
     using V = std::conditional_t<std::is_same<T, half_t>::value, float, std::conditional_t<std::is_same<T, bool>::value, int, T>>;
-    using Acc = MaxIdx<V>;
+    using Acc = MaxIdx<V, I>;
+    using Row = ArgMaxImpl<T, MIN, int32_t>;
+    __device__ static Acc FromRow(typename Row::Acc a, int64_t base) { return Acc{a.v, a.i < 0 ? I(-1) : static_cast<I>(base + a.i)}; }
     static constexpr bool kSerialFold = false;
     static constexpr bool kHasIndex = true;
     __device__ static Acc Identity() { return Acc{V(0), -1}; }
     __device__ static Acc Empty() { return Acc{V(0), -1}; }
-    __device__ static Acc Map(In v, int64_t index) { return Acc{static_cast<V>(v), index}; }
+    __device__ static Acc Map(In v, int64_t index) { return Acc{static_cast<V>(v), static_cast<I>(index)}; }
     __device__ static void Reduce(Acc next, Acc& acc) {
         if (next.i < 0) return;
         if (acc.i < 0 || (MIN ? acc.v > next.v : acc.v < next.v)) acc = next;
@@ -172,6 +180,8 @@ struct AllAnyImpl {
     using In = bool;
     using Out = bool;
     using Acc = int;
+    using Row = AllAnyImpl;
+    __device__ static Acc FromRow(Acc a, int64_t) { return a; }
     static constexpr bool kSerialFold = false;
     static constexpr bool kHasIndex = false;
     __device__ static Acc Identity() { return ALL ? 1 : 0; }
@@ -207,26 +217,78 @@ struct ReduceGeom {
 __device__ __forceinline__ void OutOffsets(const ReduceGeom& g, int64_t o, int64_t& in_off, int64_t& out_off) {
     in_off = 0;
     out_off = 0;
-    for (int d = g.n_keep - 1; d >= 0; --d) {
+    for (int d = g.n_keep - 1; d >= 1; --d) {
         int64_t q = o / g.keep_shape[d];
         int64_t r = o - q * g.keep_shape[d];
         o = q;
         in_off += r * g.keep_in_stride[d];
         out_off += r * g.keep_out_stride[d];
     }
+    if (g.n_keep > 0) {  // what is left of `o` is the coordinate on the outermost kept axis: no division
+        in_off += o * g.keep_in_stride[0];
+        out_off += o * g.keep_out_stride[0];
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
 // Row kernel
 // ---------------------------------------------------------------------------------------------
+// The value that lane + N of the same row of 16 lanes holds (N < 16; a data-parallel-primitive move: no trip through the
+// LDS crossbar).  Lanes whose partner would lie in another row keep their own value.
+template <int N, typename T>
+__device__ __forceinline__ T FromLaneAbove(T v) {
+    constexpr int kWords = (sizeof(T) + 3) / 4;
+    int w[kWords] = {};
+    __builtin_memcpy(w, &v, sizeof(T));
+#pragma unroll
+    for (int i = 0; i < kWords; ++i) w[i] = __builtin_amdgcn_update_dpp(w[i], w[i], 0x100 + N /* row_shl:N */, 0xf, 0xf, false);
+    T r;
+    __builtin_memcpy(&r, w, sizeof(T));
+    return r;
+}
+
+template <typename In>
+struct alignas(sizeof(In) * 4) Group4 {
+    In v[4];
+};
+
+template <bool ALIGNED, typename In>
+__device__ __forceinline__ Group4<In> LoadGroup(const In* p) {
+    if (ALIGNED) return *reinterpret_cast<const Group4<In>*>(p);
+    Group4<In> q;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) q.v[j] = p[j];
+    return q;
+}
+
+// One step of the balanced tree over values held by lanes S apart: the lane takes the value of lane + S as the later
+// operand (the accumulator of the merge) and its own as the earlier one.  Valid in the lanes that are multiples of 2 * S.
+template <typename R, int S>
+__device__ __forceinline__ void MergeLaneAbove(typename R::Acc& acc, int lane) {
+    typename R::Acc later;
+    if constexpr (S < 16) {
+        later = FromLaneAbove<S>(acc);
+    } else {
+        later = R::Shfl(acc, lane + S);
+    }
+    R::Reduce(acc, later);
+    acc = later;
+}
+
 template <typename Impl, bool ALIGNED>
 __global__ __launch_bounds__(kRowThreads) void RowReduceKernel(ReduceGeom g, int64_t span, int blocks_per_row, void* partials) {
-    using In = typename Impl::In;
-    using Acc = typename Impl::Acc;
+    using R = typename Impl::Row;  // the same reduction with indices counted from the block's first element
+    using In = typename R::In;
+    using Acc = typename R::Acc;
     __shared__ Acc nodes[kMaxNodes];
+    __shared__ Acc wave_nodes[kRowThreads / 64];
 
-    const int64_t row = blockIdx.x / blocks_per_row;
-    const int blk = blockIdx.x - static_cast<int>(row * blocks_per_row);
+    int64_t row = blockIdx.x;
+    int blk = 0;
+    if (blocks_per_row != 1) {
+        row = blockIdx.x / static_cast<unsigned>(blocks_per_row);
+        blk = static_cast<int>(blockIdx.x - static_cast<unsigned>(row) * static_cast<unsigned>(blocks_per_row));
+    }
     int64_t in_off, out_off;
     OutOffsets(g, row, in_off, out_off);
     const char* xbase = g.in + in_off;
@@ -247,82 +309,148 @@ __global__ __launch_bounds__(kRowThreads) void RowReduceKernel(ReduceGeom g, int
     const int seg_lane = lane & 7;
     const int iters = static_cast<int>(span / kElemsPerIter);
 
-    for (int it = 0; it < iters; ++it) {
+    // The iterations of a block that lie wholly before the chunk with the leftover elements (all of them when the row is a
+    // whole number of groups) need no bounds checks; with one dense run they need no address arithmetic either.
+    const int64_t plain_len = L % 4 == 0 ? L : k_last * 32;
+    int plain_iters = 0;
+    if (g.seg_stride == 0 && plain_len > e_begin) {
+        const int64_t n = (plain_len - e_begin) / kElemsPerIter;
+        plain_iters = n < iters ? static_cast<int>(n) : iters;
+    }
+
+    // ---- a plain iteration: group of four -> chunk (8 lanes) -> node (wave) ----
+    auto plain = [&](int it, const Group4<In>& q) {
+        const int local = it * kElemsPerIter + tid * 4;  // index of the group's first element, counted from e_begin
+        // (e0 . e1) . (e2 . e3): the later element is `next`
+        Acc gv = R::Map(q.v[0], local);
+        R::Reduce(R::Map(q.v[1], local + 1), gv);
+        Acc p1 = R::Map(q.v[2], local + 2);
+        R::Reduce(R::Map(q.v[3], local + 3), p1);
+        R::Reduce(p1, gv);
+        Acc acc = R::Identity();
+        if (R::kSerialFold) {  // Identity . g0 . g1 ... g7, strictly in order; only the chunk's first lane needs it
+            R::Reduce(gv, acc);
+            R::Reduce(FromLaneAbove<1>(gv), acc);
+            R::Reduce(FromLaneAbove<2>(gv), acc);
+            R::Reduce(FromLaneAbove<3>(gv), acc);
+            R::Reduce(FromLaneAbove<4>(gv), acc);
+            R::Reduce(FromLaneAbove<5>(gv), acc);
+            R::Reduce(FromLaneAbove<6>(gv), acc);
+            R::Reduce(FromLaneAbove<7>(gv), acc);
+        } else {
+            R::MaskLaterNan(gv, seg_lane == 0);
+            R::Reduce(gv, acc);  // lane-local start: Identity . group
+            R::Reduce(FromLaneAbove<1>(acc), acc);  // the later operand is `next`
+            R::Reduce(FromLaneAbove<2>(acc), acc);
+            R::Reduce(FromLaneAbove<4>(acc), acc);
+        }
+        // 8 chunk results per wave -> one node: balanced tree, the later operand is the accumulator
+        MergeLaneAbove<R, 8>(acc, lane);
+        MergeLaneAbove<R, 16>(acc, lane);
+        MergeLaneAbove<R, 32>(acc, lane);
+        if (lane == 0) nodes[it * 4 + wave] = acc;
+    };
+
+    // ---- an iteration that may hold the end of the row: every step checked ----
+    auto guarded = [&](int it) {
         const int64_t grp = e_begin / 4 + static_cast<int64_t>(it) * kRowThreads + tid;
         const int64_t chunk = grp >> 3;
-        Acc gv = Impl::Empty();
+        const int local = it * kElemsPerIter + tid * 4;
+        Acc gv = R::Empty();
         if (grp < G) {
-            In e[4];
-            if (ALIGNED) {
-                struct alignas(sizeof(In) * 4) In4 {
-                    In v[4];
-                };
-                In4 q = *reinterpret_cast<const In4*>(at(grp * 4));
-#pragma unroll
-                for (int j = 0; j < 4; ++j) e[j] = q.v[j];
-            } else {
-                const In* xp = at(grp * 4);
-#pragma unroll
-                for (int j = 0; j < 4; ++j) e[j] = xp[j];
-            }
-            // (e0 . e1) . (e2 . e3): the later element is `next`
-            Acc p0 = Impl::Map(e[0], grp * 4);
-            Impl::Reduce(Impl::Map(e[1], grp * 4 + 1), p0);
-            Acc p1 = Impl::Map(e[2], grp * 4 + 2);
-            Impl::Reduce(Impl::Map(e[3], grp * 4 + 3), p1);
-            Impl::Reduce(p1, p0);
+            const Group4<In> q = LoadGroup<ALIGNED>(at(grp * 4));
+            Acc p0 = R::Map(q.v[0], local);
+            R::Reduce(R::Map(q.v[1], local + 1), p0);
+            Acc p1 = R::Map(q.v[2], local + 2);
+            R::Reduce(R::Map(q.v[3], local + 3), p1);
+            R::Reduce(p1, p0);
             gv = p0;
         }
         // ---- fold the 8 groups of a chunk into the segment leader ----
         Acc acc;
-        if (Impl::kSerialFold) {
-            acc = Impl::Identity();
-            Impl::Reduce(gv, acc);
+        if (R::kSerialFold) {
+            acc = R::Identity();
+            R::Reduce(gv, acc);
 #pragma unroll
             for (int j = 1; j < 8; ++j) {
-                Acc o = Impl::Shfl(gv, (lane & ~7) + j);
-                Impl::Reduce(o, acc);
+                Acc o = R::Shfl(gv, (lane & ~7) + j);
+                R::Reduce(o, acc);
             }
         } else {
-            Impl::MaskLaterNan(gv, seg_lane == 0);
-            acc = Impl::Identity();
-            Impl::Reduce(gv, acc);  // lane-local start: Identity . group
+            R::MaskLaterNan(gv, seg_lane == 0);
+            acc = R::Identity();
+            R::Reduce(gv, acc);  // lane-local start: Identity . group
 #pragma unroll
             for (int s = 1; s < 8; s <<= 1) {
-                Acc o = Impl::Shfl(acc, lane + s);  // the later operand
-                Impl::Reduce(o, acc);
+                Acc o = R::Shfl(acc, lane + s);  // the later operand
+                R::Reduce(o, acc);
             }
         }
         // ---- the last chunk also folds the leftover elements, in order ----
         if (seg_lane == 0 && chunk == k_last) {
-            for (int64_t i = G * 4; i < L; ++i) Impl::Reduce(Impl::Map(*at(i), i), acc);
+            for (int64_t i = G * 4; i < L; ++i) R::Reduce(R::Map(*at(i), i - e_begin), acc);
         }
-        if (chunk > k_last) acc = Impl::Empty();
+        if (chunk > k_last) acc = R::Empty();
         // ---- 8 chunk results per wave -> one node: balanced tree, the later operand is the accumulator ----
 #pragma unroll
         for (int s = 8; s < 64; s <<= 1) {
-            Acc later = Impl::Shfl(acc, lane + s);
-            Impl::Reduce(acc, later);
+            Acc later = R::Shfl(acc, lane + s);
+            R::Reduce(acc, later);
             acc = later;
         }
         if (lane == 0) nodes[it * 4 + wave] = acc;
+    };
+
+    // The loads of kLoadBatch plain iterations are issued together, ahead of the arithmetic of the first of them.
+    constexpr int kLoadBatch = 4;
+    const In* xrow = reinterpret_cast<const In*>(xbase) + e_begin + tid * 4;
+    int it = 0;
+    for (; it + kLoadBatch <= plain_iters; it += kLoadBatch) {
+        Group4<In> q[kLoadBatch];
+#pragma unroll
+        for (int u = 0; u < kLoadBatch; ++u) q[u] = LoadGroup<ALIGNED>(xrow + static_cast<int64_t>(it + u) * kElemsPerIter);
+        __builtin_amdgcn_sched_barrier(0);  // all loads in flight before anything waits for the first
+#pragma unroll
+        for (int u = 0; u < kLoadBatch; ++u) plain(it + u, q[u]);
     }
+    for (; it < plain_iters; ++it) plain(it, LoadGroup<ALIGNED>(xrow + static_cast<int64_t>(it) * kElemsPerIter));
+    for (; it < iters; ++it) guarded(it);
     __syncthreads();
-    const int n_nodes = iters * 4;  // a power of two
-    for (int s = 1; s < n_nodes; s <<= 1) {
-        for (int i = tid; (2 * i + 1) * s < n_nodes; i += kRowThreads) {
-            Acc earlier = nodes[2 * i * s];
-            Acc later = nodes[2 * i * s + s];
-            Impl::Reduce(earlier, later);
-            nodes[2 * i * s] = later;
-        }
+
+    // ---- tree over the block's nodes (a power of two, at least 4): each wave folds up to 64 consecutive ones ----
+    const int n_nodes = iters * 4;
+    Acc acc = R::Empty();
+    if (wave * 64 < n_nodes) {
+        if (wave * 64 + lane < n_nodes) acc = nodes[wave * 64 + lane];  // lanes past the end hold padding
+        MergeLaneAbove<R, 1>(acc, lane);
+        MergeLaneAbove<R, 2>(acc, lane);
+        MergeLaneAbove<R, 4>(acc, lane);
+        MergeLaneAbove<R, 8>(acc, lane);
+        MergeLaneAbove<R, 16>(acc, lane);
+        MergeLaneAbove<R, 32>(acc, lane);
+    }
+    if (n_nodes > 64) {  // 128 or 256 nodes: two or four waves hold a result each
+        if (lane == 0) wave_nodes[wave] = acc;
         __syncthreads();
+        if (tid == 0) {
+            Acc b = wave_nodes[1];
+            R::Reduce(acc, b);
+            if (n_nodes > 128) {
+                Acc c = wave_nodes[2];
+                Acc d = wave_nodes[3];
+                R::Reduce(c, d);
+                R::Reduce(b, d);
+                b = d;
+            }
+            acc = b;
+        }
     }
     if (tid == 0) {
+        const typename Impl::Acc result = Impl::FromRow(acc, e_begin);
         if (blocks_per_row == 1) {
-            *reinterpret_cast<typename Impl::Out*>(g.out + out_off) = Impl::MapOut(nodes[0]);
+            *reinterpret_cast<typename Impl::Out*>(g.out + out_off) = Impl::MapOut(result);
         } else {
-            reinterpret_cast<Acc*>(partials)[row * blocks_per_row + blk] = nodes[0];
+            reinterpret_cast<typename Impl::Acc*>(partials)[row * blocks_per_row + blk] = result;
         }
     }
 }
