@@ -42,6 +42,8 @@ constexpr int kMaxPartials = 1024;              // blocks per row handled by the
 //   Map(in, index)        impl.MapIn
 //   Reduce(next, acc)     impl.Reduce(next, accum), additionally a no-op when `next` is the padding value Empty()
 //   kSerialFold           whether the 8 groups of a chunk must be folded strictly in order (floating point addition)
+//   kFast, ReduceFast     a shorter Reduce for operands known to be neither padding (kFast >= 1) nor NaN (kFast == 2);
+//                         Probe(in) is a float that is NaN when `in` is
 // ---------------------------------------------------------------------------------------------
 template <typename In_, typename Out_>
 struct SumImpl {
@@ -52,6 +54,9 @@ struct SumImpl {
     __device__ static Acc FromRow(Acc a, int64_t) { return a; }
     static constexpr bool kSerialFold = true;
     static constexpr bool kHasIndex = false;
+    static constexpr int kFast = 0;
+    __device__ static void ReduceFast(Acc next, Acc& acc) { Reduce(next, acc); }
+    __device__ static float Probe(In) { return 0.f; }
     __device__ static Acc Identity() { return Acc(0); }
     __device__ static Acc Empty() { return Acc(0); }  // x + 0 == x for every x a chunk can produce (never -0)
     __device__ static Acc Map(In v, int64_t) {
@@ -123,6 +128,11 @@ struct AMaxImpl {
     __device__ static Acc FromRow(Acc a, int64_t) { return a; }
     static constexpr bool kSerialFold = false;
     static constexpr bool kHasIndex = false;
+    static constexpr int kFast = (std::is_same<T, half_t>::value || std::is_floating_point<T>::value) ? 2 : 0;
+    __device__ static void ReduceFast(Acc next, Acc& acc) {
+        if (MIN ? acc > next : acc < next) acc = next;
+    }
+    __device__ static float Probe(In v) { return static_cast<float>(v); }
     __device__ static Acc Identity() { return static_cast<Acc>(MIN ? MaxOrInf<T>() : LowestOrInf<T>()); }
     __device__ static Acc Empty() { return Identity(); }
     __device__ static Acc Map(In v, int64_t) { return static_cast<Acc>(v); }
@@ -153,6 +163,11 @@ struct ArgMaxImpl {
     __device__ static Acc FromRow(typename Row::Acc a, int64_t base) { return Acc{a.v, a.i < 0 ? I(-1) : static_cast<I>(base + a.i)}; }
     static constexpr bool kSerialFold = false;
     static constexpr bool kHasIndex = true;
+    static constexpr int kFast = (std::is_same<T, half_t>::value || std::is_floating_point<T>::value) ? 2 : 1;
+    __device__ static void ReduceFast(Acc next, Acc& acc) {
+        if (MIN ? acc.v > next.v : acc.v < next.v) acc = next;
+    }
+    __device__ static float Probe(In v) { return static_cast<float>(v); }
     __device__ static Acc Identity() { return Acc{V(0), -1}; }
     __device__ static Acc Empty() { return Acc{V(0), -1}; }
     __device__ static Acc Map(In v, int64_t index) { return Acc{static_cast<V>(v), static_cast<I>(index)}; }
@@ -184,6 +199,9 @@ struct AllAnyImpl {
     __device__ static Acc FromRow(Acc a, int64_t) { return a; }
     static constexpr bool kSerialFold = false;
     static constexpr bool kHasIndex = false;
+    static constexpr int kFast = 0;
+    __device__ static void ReduceFast(Acc next, Acc& acc) { Reduce(next, acc); }
+    __device__ static float Probe(In) { return 0.f; }
     __device__ static Acc Identity() { return ALL ? 1 : 0; }
     __device__ static Acc Empty() { return Identity(); }
     __device__ static Acc Map(In v, int64_t) { return v ? 1 : 0; }
@@ -234,14 +252,15 @@ __device__ __forceinline__ void OutOffsets(const ReduceGeom& g, int64_t o, int64
 // Row kernel
 // ---------------------------------------------------------------------------------------------
 // The value that lane + N of the same row of 16 lanes holds (N < 16; a data-parallel-primitive move: no trip through the
-// LDS crossbar).  Lanes whose partner would lie in another row keep their own value.
+// LDS crossbar).  Lanes whose partner would lie in another row get zero bits (and nobody reads their results); written this
+// way the compiler can fold the move into the instruction that consumes it.
 template <int N, typename T>
 __device__ __forceinline__ T FromLaneAbove(T v) {
     constexpr int kWords = (sizeof(T) + 3) / 4;
     int w[kWords] = {};
     __builtin_memcpy(w, &v, sizeof(T));
 #pragma unroll
-    for (int i = 0; i < kWords; ++i) w[i] = __builtin_amdgcn_update_dpp(w[i], w[i], 0x100 + N /* row_shl:N */, 0xf, 0xf, false);
+    for (int i = 0; i < kWords; ++i) w[i] = __builtin_amdgcn_update_dpp(0, w[i], 0x100 + N /* row_shl:N */, 0xf, 0xf, true);
     T r;
     __builtin_memcpy(&r, w, sizeof(T));
     return r;
@@ -261,18 +280,53 @@ __device__ __forceinline__ Group4<In> LoadGroup(const In* p) {
     return q;
 }
 
-// One step of the balanced tree over values held by lanes S apart: the lane takes the value of lane + S as the later
-// operand (the accumulator of the merge) and its own as the earlier one.  Valid in the lanes that are multiples of 2 * S.
-template <typename R, int S>
-__device__ __forceinline__ void MergeLaneAbove(typename R::Acc& acc, int lane) {
-    typename R::Acc later;
-    if constexpr (S < 16) {
-        later = FromLaneAbove<S>(acc);
-    } else {
-        later = R::Shfl(acc, lane + S);
+// Reduce of R, or its shorter form for operands known to be neither padding nor NaN.
+template <typename R, bool FAST>
+struct ReduceOp {
+    using Acc = typename R::Acc;
+    __device__ static __forceinline__ void Reduce(Acc next, Acc& acc) {
+        if constexpr (FAST) {
+            R::ReduceFast(next, acc);
+        } else {
+            R::Reduce(next, acc);
+        }
     }
-    R::Reduce(acc, later);
+};
+
+// One step of the balanced tree over values held by lanes S apart (S < 16): the lane takes the value of lane + S as the
+// later operand (the accumulator of the merge) and its own as the earlier one.  Valid in the lanes that are multiples of
+// 2 * S.
+template <typename Op, int S>
+__device__ __forceinline__ void MergeLaneAbove(typename Op::Acc& acc) {
+    typename Op::Acc later = FromLaneAbove<S>(acc);
+    Op::Reduce(acc, later);
     acc = later;
+}
+
+template <int LANE, typename T>
+__device__ __forceinline__ T ReadLane(T v) {  // the value held by lane LANE, in every lane (through scalar registers)
+    constexpr int kWords = (sizeof(T) + 3) / 4;
+    int w[kWords] = {};
+    __builtin_memcpy(w, &v, sizeof(T));
+#pragma unroll
+    for (int i = 0; i < kWords; ++i) w[i] = __builtin_amdgcn_readlane(w[i], LANE);
+    T r;
+    __builtin_memcpy(&r, w, sizeof(T));
+    return r;
+}
+
+// The last two levels of the tree over a wave: the values of lanes 0, 16, 32 and 48 (the first lane of each row of 16)
+// merged as (l0 . l16) . (l32 . l48), the later operand being the accumulator.  Every lane gets the result.
+template <typename Op>
+__device__ __forceinline__ typename Op::Acc MergeRows(typename Op::Acc acc) {
+    typename Op::Acc a = ReadLane<0>(acc);
+    typename Op::Acc b = ReadLane<16>(acc);
+    typename Op::Acc c = ReadLane<32>(acc);
+    typename Op::Acc d = ReadLane<48>(acc);
+    Op::Reduce(a, b);
+    Op::Reduce(c, d);
+    Op::Reduce(b, d);
+    return d;
 }
 
 template <typename Impl, bool ALIGNED>
@@ -318,37 +372,91 @@ __global__ __launch_bounds__(kRowThreads) void RowReduceKernel(ReduceGeom g, int
         plain_iters = n < iters ? static_cast<int>(n) : iters;
     }
 
-    // ---- a plain iteration: group of four -> chunk (8 lanes) -> node (wave) ----
-    auto plain = [&](int it, const Group4<In>& q) {
-        const int local = it * kElemsPerIter + tid * 4;  // index of the group's first element, counted from e_begin
-        // (e0 . e1) . (e2 . e3): the later element is `next`
-        Acc gv = R::Map(q.v[0], local);
-        R::Reduce(R::Map(q.v[1], local + 1), gv);
-        Acc p1 = R::Map(q.v[2], local + 2);
-        R::Reduce(R::Map(q.v[3], local + 3), p1);
-        R::Reduce(p1, gv);
-        Acc acc = R::Identity();
+    // ---- N plain iterations, stage by stage so that their instructions interleave: group of four -> chunk (8 lanes) ->
+    // node (wave).  FAST: no operand is padding or NaN, so the shorter Reduce applies and gives the same result. ----
+    auto plain_stages = [&](int it0, const Group4<In>* q, auto count, auto fast) {
+        constexpr int N = decltype(count)::value;
+        constexpr bool FAST = decltype(fast)::value;
+        using Op = ReduceOp<R, FAST>;
+        Acc acc[N];
+#pragma unroll
+        for (int u = 0; u < N; ++u) {
+            const int local = (it0 + u) * kElemsPerIter + tid * 4;  // index of the group's first element, counted from e_begin
+            // (e0 . e1) . (e2 . e3): the later element is `next`
+            Acc gv = R::Map(q[u].v[0], local);
+            Op::Reduce(R::Map(q[u].v[1], local + 1), gv);
+            Acc p1 = R::Map(q[u].v[2], local + 2);
+            Op::Reduce(R::Map(q[u].v[3], local + 3), p1);
+            Op::Reduce(p1, gv);
+            acc[u] = gv;
+        }
         if (R::kSerialFold) {  // Identity . g0 . g1 ... g7, strictly in order; only the chunk's first lane needs it
-            R::Reduce(gv, acc);
-            R::Reduce(FromLaneAbove<1>(gv), acc);
-            R::Reduce(FromLaneAbove<2>(gv), acc);
-            R::Reduce(FromLaneAbove<3>(gv), acc);
-            R::Reduce(FromLaneAbove<4>(gv), acc);
-            R::Reduce(FromLaneAbove<5>(gv), acc);
-            R::Reduce(FromLaneAbove<6>(gv), acc);
-            R::Reduce(FromLaneAbove<7>(gv), acc);
+            Acc gv[N];
+#pragma unroll
+            for (int u = 0; u < N; ++u) {
+                gv[u] = acc[u];
+                acc[u] = R::Identity();
+                Op::Reduce(gv[u], acc[u]);
+            }
+            auto step = [&](auto j) {
+#pragma unroll
+                for (int u = 0; u < N; ++u) Op::Reduce(FromLaneAbove<decltype(j)::value>(gv[u]), acc[u]);
+            };
+            step(std::integral_constant<int, 1>());
+            step(std::integral_constant<int, 2>());
+            step(std::integral_constant<int, 3>());
+            step(std::integral_constant<int, 4>());
+            step(std::integral_constant<int, 5>());
+            step(std::integral_constant<int, 6>());
+            step(std::integral_constant<int, 7>());
         } else {
-            R::MaskLaterNan(gv, seg_lane == 0);
-            R::Reduce(gv, acc);  // lane-local start: Identity . group
-            R::Reduce(FromLaneAbove<1>(acc), acc);  // the later operand is `next`
-            R::Reduce(FromLaneAbove<2>(acc), acc);
-            R::Reduce(FromLaneAbove<4>(acc), acc);
+            if (!FAST) {  // (with FAST, Identity . group == group and there is no NaN to mask)
+#pragma unroll
+                for (int u = 0; u < N; ++u) {
+                    Acc m = acc[u];
+                    R::MaskLaterNan(m, seg_lane == 0);
+                    acc[u] = R::Identity();
+                    R::Reduce(m, acc[u]);  // lane-local start: Identity . group
+                }
+            }
+            auto step = [&](auto s) {  // the later operand is `next`
+#pragma unroll
+                for (int u = 0; u < N; ++u) Op::Reduce(FromLaneAbove<decltype(s)::value>(acc[u]), acc[u]);
+            };
+            step(std::integral_constant<int, 1>());
+            step(std::integral_constant<int, 2>());
+            step(std::integral_constant<int, 4>());
         }
         // 8 chunk results per wave -> one node: balanced tree, the later operand is the accumulator
-        MergeLaneAbove<R, 8>(acc, lane);
-        MergeLaneAbove<R, 16>(acc, lane);
-        MergeLaneAbove<R, 32>(acc, lane);
-        if (lane == 0) nodes[it * 4 + wave] = acc;
+#pragma unroll
+        for (int u = 0; u < N; ++u) MergeLaneAbove<Op, 8>(acc[u]);
+#pragma unroll
+        for (int u = 0; u < N; ++u) acc[u] = MergeRows<Op>(acc[u]);
+        if (lane == 0) {
+#pragma unroll
+            for (int u = 0; u < N; ++u) nodes[(it0 + u) * 4 + wave] = acc[u];
+        }
+    };
+    auto plain = [&](int it0, const Group4<In>* q, auto count) {
+        constexpr int N = decltype(count)::value;
+        if constexpr (R::kFast == 0) {
+            plain_stages(it0, q, count, std::false_type());
+        } else if constexpr (R::kFast == 1) {
+            plain_stages(it0, q, count, std::true_type());
+        } else {
+            // Is a NaN among the wave's N * 256 elements?  A sum is NaN when an addend is (inf - inf also is: that only
+            // costs the longer path).
+            float t[N];
+#pragma unroll
+            for (int u = 0; u < N; ++u) t[u] = (R::Probe(q[u].v[0]) + R::Probe(q[u].v[1])) + (R::Probe(q[u].v[2]) + R::Probe(q[u].v[3]));
+#pragma unroll
+            for (int u = 1; u < N; ++u) t[0] += t[u];
+            if (__ballot(t[0] != t[0]) == 0) {
+                plain_stages(it0, q, count, std::true_type());
+            } else {
+                plain_stages(it0, q, count, std::false_type());
+            }
+        }
     };
 
     // ---- an iteration that may hold the end of the row: every step checked ----
@@ -410,10 +518,12 @@ __global__ __launch_bounds__(kRowThreads) void RowReduceKernel(ReduceGeom g, int
 #pragma unroll
         for (int u = 0; u < kLoadBatch; ++u) q[u] = LoadGroup<ALIGNED>(xrow + static_cast<int64_t>(it + u) * kElemsPerIter);
         __builtin_amdgcn_sched_barrier(0);  // all loads in flight before anything waits for the first
-#pragma unroll
-        for (int u = 0; u < kLoadBatch; ++u) plain(it + u, q[u]);
+        plain(it, q, std::integral_constant<int, kLoadBatch>());
     }
-    for (; it < plain_iters; ++it) plain(it, LoadGroup<ALIGNED>(xrow + static_cast<int64_t>(it) * kElemsPerIter));
+    for (; it < plain_iters; ++it) {
+        const Group4<In> q = LoadGroup<ALIGNED>(xrow + static_cast<int64_t>(it) * kElemsPerIter);
+        plain(it, &q, std::integral_constant<int, 1>());
+    }
     for (; it < iters; ++it) guarded(it);
     __syncthreads();
 
@@ -422,12 +532,12 @@ __global__ __launch_bounds__(kRowThreads) void RowReduceKernel(ReduceGeom g, int
     Acc acc = R::Empty();
     if (wave * 64 < n_nodes) {
         if (wave * 64 + lane < n_nodes) acc = nodes[wave * 64 + lane];  // lanes past the end hold padding
-        MergeLaneAbove<R, 1>(acc, lane);
-        MergeLaneAbove<R, 2>(acc, lane);
-        MergeLaneAbove<R, 4>(acc, lane);
-        MergeLaneAbove<R, 8>(acc, lane);
-        MergeLaneAbove<R, 16>(acc, lane);
-        MergeLaneAbove<R, 32>(acc, lane);
+        using Op = ReduceOp<R, false>;
+        MergeLaneAbove<Op, 1>(acc);
+        MergeLaneAbove<Op, 2>(acc);
+        MergeLaneAbove<Op, 4>(acc);
+        MergeLaneAbove<Op, 8>(acc);
+        acc = MergeRows<Op>(acc);
     }
     if (n_nodes > 64) {  // 128 or 256 nodes: two or four waves hold a result each
         if (lane == 0) wave_nodes[wave] = acc;

@@ -66,6 +66,33 @@ def test_argmax_ties_and_nans_bit_exact(length):
     assert_exact(chx.argmax(chx.array(xz), 1).get(), O.argmax(xz, 1), 'signed zeros')
 
 
+@pytest.mark.parametrize('dt', ['float16', 'float32', 'float64'])
+def test_long_rows_with_few_nans_infinities_and_signed_zeros(dt):
+    """The row kernel folds a wave's elements with a shorter comparison when none of them is NaN and with the full rule
+    otherwise: rows in which only a few waves hold a NaN take both routes and must still give the native backend's answer
+    bit for bit -- the index, which NaN-free maximum, and the sign of a zero maximum (the first of equal values wins)."""
+    import chainer_amd as chx
+    rng = np.random.default_rng(17)
+    rows, length = 12, 9000
+    x = rng.integers(-3, 1, (rows, length)).astype(dt)      # maximum 0, many ties
+    x[x == 0] = np.where(rng.random(int((x == 0).sum())) < 0.5, 0.0, -0.0).astype(dt)  # zeros of both signs
+    x[1, 5000] = np.nan                      # one NaN, one wave
+    x[2, [17, 4100, 8999]] = np.nan          # the last one among the leftover groups
+    x[3, 0] = np.nan                         # a leading NaN is never replaced
+    x[4, 100] = np.inf
+    x[4, 101] = -np.inf                      # inf - inf: the probe says NaN although there is none
+    x[5, 2000:2300] = np.inf
+    x[6, :] = -np.inf
+    x[7, 1024:2048] = np.nan                 # a whole iteration of NaNs
+    x[8, :] = np.where(rng.random(length) < 0.5, 0.0, -0.0).astype(dt)
+    X = chx.array(x)
+    for name in ('amax', 'amin', 'argmax', 'argmin'):
+        assert_exact(getattr(chx, name)(X, 1).get(), getattr(O, name)(x, 1), '%s %s' % (name, dt))
+    flat = chx.array(x.reshape(-1))           # one row split over several blocks
+    for name in ('amax', 'amin', 'argmax', 'argmin'):
+        assert_exact(getattr(chx, name)(flat, 0).get(), getattr(O, name)(x.reshape(-1), 0), '%s flat %s' % (name, dt))
+
+
 @pytest.mark.parametrize('dt,tol', [('float32', 1e-5), ('float64', 1e-12), ('float16', 2e-2)])
 def test_log_softmax_mean_softmax(dt, tol):
     import chainer_amd as chx
