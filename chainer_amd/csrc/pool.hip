@@ -216,31 +216,62 @@ __global__ __launch_bounds__(256) void MaxPoolRowsS2Kernel(PoolArgs p, int64_t t
 }
 
 // Global average pooling over dense NCHW planes (window = whole plane, no padding): a workgroup copies 256 consecutive
-// planes (one contiguous run) into LDS with 16-byte loads, then each thread sums one plane.  Sum in the compute type,
-// rounded to T, then divided in T arithmetic, like Sum followed by Divide.
+// planes (one contiguous run) into LDS with 16-byte loads -- eight per thread in flight at a time --, then each thread
+// sums one plane in order.  Sum in the compute type, rounded to T, then divided in T arithmetic, like Sum followed by
+// Divide.  Two-byte elements are read back from LDS as dwords (a plane may start in the upper half of one).
 template <typename T>
 __global__ __launch_bounds__(256) void GlobalAvgPoolKernel(const T* x, T* out, int64_t planes, int hw) {
     using C = compute_t<T>;
     extern __shared__ __align__(16) char lds[];
+    constexpr int kBatch = 8;
+    constexpr int kStep = 256 * 16;  // bytes the workgroup moves per load instruction
+    const int tid = threadIdx.x;
     const int64_t p0 = static_cast<int64_t>(blockIdx.x) * 256;
-    const int64_t np = planes - p0 < 256 ? planes - p0 : 256;
-    const int64_t bytes = np * hw * static_cast<int64_t>(sizeof(T));
+    const int np = static_cast<int>(planes - p0 < 256 ? planes - p0 : 256);
+    const int bytes = np * hw * static_cast<int>(sizeof(T));  // at most 64 KiB
     const char* src = reinterpret_cast<const char*>(x + p0 * hw);
-    for (int64_t off = static_cast<int64_t>(threadIdx.x) * 16; off < bytes; off += 256 * 16) {
-        if (off + 16 <= bytes) {
-            *reinterpret_cast<PVec<unsigned, 4>*>(lds + off) = *reinterpret_cast<const PVec<unsigned, 4>*>(src + off);
-        } else {
-            for (int64_t b = off; b < bytes; ++b) lds[b] = src[b];
+    if (bytes >= 16) {
+        const int last = (bytes - 16) & ~15;  // offset of the last whole 16 bytes
+        for (int base = tid * 16; base < bytes; base += kBatch * kStep) {
+            PVec<unsigned, 4> v[kBatch];
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u) {  // loads past the end are redirected, not skipped: no branch between the loads
+                const int off = base + u * kStep;
+                v[u] = *reinterpret_cast<const PVec<unsigned, 4>*>(src + (off < last ? off : last));
+            }
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u) {
+                const int off = base + u * kStep;
+                if (off + 16 <= bytes) *reinterpret_cast<PVec<unsigned, 4>*>(lds + off) = v[u];
+            }
         }
     }
+    for (int b = (bytes & ~15) + tid; b < bytes; b += 256) lds[b] = src[b];  // the last few bytes of the run
     __syncthreads();
-    if (threadIdx.x < np) {
-        const T* pl = reinterpret_cast<const T*>(lds) + threadIdx.x * hw;
+    if (tid < np) {
         C acc = C(0);
-        for (int i = 0; i < hw; ++i) acc += static_cast<C>(pl[i]);
+        if constexpr (sizeof(T) == 2) {
+            const unsigned* w = reinterpret_cast<const unsigned*>(lds);
+            auto lower = [](unsigned u) { return static_cast<C>(__builtin_bit_cast(T, static_cast<unsigned short>(u & 0xffffu))); };
+            auto upper = [](unsigned u) { return static_cast<C>(__builtin_bit_cast(T, static_cast<unsigned short>(u >> 16))); };
+            const int first = tid * hw;  // index of the plane's first element among the workgroup's two-byte elements
+            const int odd = first & 1;
+            const unsigned* pw = w + (first >> 1);
+            const int nwords = (hw + 2) / 2;  // the same trip count for every lane; halves outside the plane are skipped
+#pragma unroll 8
+            for (int j = 0; j < nwords; ++j) {
+                const unsigned u = pw[j];
+                const int e = 2 * j - odd;  // element held by the lower half
+                if (e >= 0 && e < hw) acc += lower(u);
+                if (e + 1 < hw) acc += upper(u);
+            }
+        } else {
+            const T* pl = reinterpret_cast<const T*>(lds) + tid * hw;
+            for (int i = 0; i < hw; ++i) acc += static_cast<C>(pl[i]);
+        }
         T s = static_cast<T>(acc);
         C div = static_cast<C>(static_cast<T>(static_cast<C>(hw)));
-        out[p0 + threadIdx.x] = static_cast<T>(static_cast<C>(s) / div);
+        out[p0 + tid] = static_cast<T>(static_cast<C>(s) / div);
     }
 }
 

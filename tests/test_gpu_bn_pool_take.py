@@ -53,6 +53,8 @@ def test_pooling(dt, tol):
     cases = [((2, 16, 9, 8), 3, 2, 1, False), ((2, 16, 9, 8), 3, 2, 1, True), ((2, 3, 7, 7), 2, 2, 0, False), ((1, 8, 7, 7), 7, 1, 0, False),
              ((2, 64, 12, 12), (3, 2), (2, 1), (1, 0), True), ((2, 8, 112, 112), 3, 2, 1, False), ((2, 8, 32, 32), 2, 2, 0, False),
              ((1, 4, 16, 24), 3, 2, 1, True), ((1, 4, 16, 16), (2, 3), 2, (0, 1), False)]
+    # whole-plane windows (global pooling) over more planes than one workgroup takes, odd and even plane sizes
+    cases += [((3, 200, 7, 7), 7, 1, 0, False), ((2, 301, 5, 5), 5, 1, 0, False), ((2, 130, 6, 6), 6, 1, 0, False), ((1, 257, 3, 5), (3, 5), 1, 0, False)]
     cases += [(xs, k, s, p, cv) for (xs, k, s, p) in POOL_GRID for cv in (False, True)]
     for shape, k, s, p, cv in cases:
         x = rng.standard_normal(shape).astype(dt)
