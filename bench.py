@@ -11,7 +11,12 @@ One JSON line is printed; besides the contract keys it carries
   roofline      the implicit-GEMM convolution kernel (the dominant one): algorithmic flops of its
                 launches in one step / their summed duration, measured with HIP events recorded on
                 the launch stream around each launch (hipcx_profile_start/stop) in extra steps run
-                after the timed region, against the dense fp16 MFMA peak.
+                after the timed region, against the dense fp16 MFMA peak.  `by_bound` splits the
+                same launches by what bounds each one on paper (flops / 2.5 PFLOP/s against bytes /
+                8 TB/s): the MFMA-bound launches against the MFMA peak, the HBM-bound ones against
+                the HBM peak, and `max_bound_frac` = sum of each launch's larger bound time / sum
+                of the measured durations.  `stream_copy` is a plain device copy timed in the same
+                run: the HBM rate this box actually reaches.
   cpu_baseline  the CPU oracle (a single-threaded restatement of the ChainerX native backend) on a
                 small batch of the same network, timed on this host.
 """
@@ -27,6 +32,7 @@ import numpy as np
 sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
 
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 matrix peak
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E peak
 # HBM bytes per convolution launch (fetch + write, averaged over the 53 convolutions of one step), from two rocprofv3
 # --pmc runs (FETCH_SIZE, WRITE_SIZE) scaled by what the same counters read for a 128 MiB copy kernel (x1.999, x1.000):
 # profiles/resnet50_conv_hbm_traffic.txt.  The algorithmic figure is 101 MB per launch.
@@ -121,6 +127,42 @@ def main():
     flops = ctypes.c_double()
     nbytes = ctypes.c_double()
     _lib.check(lib.hipcx_profile_stop(ctypes.byref(n), ctypes.byref(ms), ctypes.byref(flops), ctypes.byref(nbytes)))
+    rec_n = ctypes.c_int64()
+    rec_ms = (ctypes.c_double * n.value)()
+    rec_flops = (ctypes.c_double * n.value)()
+    rec_bytes = (ctypes.c_double * n.value)()
+    _lib.check(lib.hipcx_profile_records(n.value, rec_ms, rec_flops, rec_bytes, ctypes.byref(rec_n)))
+    groups = {'mfma': [0, 0.0, 0.0, 0.0], 'hbm': [0, 0.0, 0.0, 0.0]}  # launches, ms, flops, bytes
+    bound_ms = 0.0
+    for i in range(min(n.value, rec_n.value)):
+        t_mfma = rec_flops[i] / (MFMA_F16_PEAK_TFLOPS * 1e12) * 1e3
+        t_hbm = rec_bytes[i] / (HBM_PEAK_GBS * 1e9) * 1e3
+        g = groups['mfma' if t_mfma >= t_hbm else 'hbm']
+        g[0] += 1
+        g[1] += rec_ms[i]
+        g[2] += rec_flops[i]
+        g[3] += rec_bytes[i]
+        bound_ms += max(t_mfma, t_hbm)
+    gm, gh = groups['mfma'], groups['hbm']
+    by_bound = {
+        'mfma_bound': {'launches_per_step': gm[0] // prof_steps, 'kernel_ms_per_step': round(gm[1] / prof_steps, 3),
+                       'achieved_tflops': round(gm[2] / (gm[1] * 1e-3) / 1e12, 1) if gm[1] > 0 else 0.0,
+                       'frac_of_mfma_peak': round(gm[2] / (gm[1] * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS, 4) if gm[1] > 0 else None},
+        'hbm_bound': {'launches_per_step': gh[0] // prof_steps, 'kernel_ms_per_step': round(gh[1] / prof_steps, 3),
+                      'achieved_gbs': round(gh[3] / (gh[1] * 1e-3) / 1e9, 1) if gh[1] > 0 else 0.0,
+                      'frac_of_hbm_peak': round(gh[3] / (gh[1] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4) if gh[1] > 0 else None},
+        'max_bound_ms_per_step': round(bound_ms / prof_steps, 3),
+        'max_bound_frac': round(bound_ms / ms.value, 4) if ms.value > 0 else None,
+    }
+
+    # ---- a plain device copy (1 GiB read + 1 GiB written), ten per graph replay: what this box's HBM delivers ----
+    big = chx.array(np.zeros(512 * 1024 * 1024, np.float16))
+    from chainer_amd.bench_ops import kernel_time
+    copy_s = kernel_time(lambda: chx.copy(big))
+    stream_copy = {'bytes': 2 * big.nbytes, 'us': round(copy_s * 1e6, 1), 'gbs': round(2 * big.nbytes / copy_s / 1e9, 1),
+                   'frac_of_hbm_peak': round(2 * big.nbytes / copy_s / 1e9 / HBM_PEAK_GBS, 4)}
+    del big
+
     launches_per_step = n.value // prof_steps
     avg_launch_ms = ms.value / max(n.value, 1)
     achieved_tflops = flops.value / (ms.value * 1e-3) / 1e12 if ms.value > 0 else 0.0
@@ -138,6 +180,8 @@ def main():
         'algorithmic_gflop_per_step': round(flops.value / prof_steps / 1e9, 2),
         'algorithmic_gb_per_step': round(nbytes.value / prof_steps / 1e9, 3),
         'achieved_gbs': round(nbytes.value / (ms.value * 1e-3) / 1e9, 1) if ms.value > 0 else 0.0,
+        'by_bound': by_bound,
+        'stream_copy': stream_copy,
     }
 
     # ---- opt-in fused path (reported beside the headline, never as `value`): conv+bn(+add)+relu groups as one call ----

@@ -193,6 +193,8 @@ SIGNATURES = {
     'hipcx_profile_start': (_INT, []),
     'hipcx_profile_stop': (_INT, [_I64P, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double),
                                   ctypes.POINTER(ctypes.c_double)]),
+    'hipcx_profile_records': (_INT, [ctypes.c_int64, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double),
+                                     ctypes.POINTER(ctypes.c_double), _I64P]),
     'hipcx_fixed_batch_norm': (_INT, [_A, _A, _A, _A, _A, _S, _I8P, _INT, _A, _V]),
     'hipcx_batch_norm_workspace_size': (_SZ, [_A, _I8P, _INT]),
     'hipcx_batch_norm': (_INT, [_A, _A, _A, _A, _A, _S, _S, _I8P, _INT, _A, _A, _A, _V, _SZ, _V]),

@@ -21,9 +21,13 @@ namespace {
 // Optional event bracketing of every implicit-GEMM launch (hipcx_profile_start/stop): the events are
 // recorded on the launch stream right before and after the kernel, so their elapsed time is the
 // kernel's own duration and excludes the filter repack and any host work.
+struct ProfileRecord {  // one bracketed launch
+    double ms, flops, bytes;
+};
 struct ProfileState {
     bool on = false;
     std::vector<std::pair<hipEvent_t, hipEvent_t>> events;
+    std::vector<ProfileRecord> records;  // flops and bytes at launch; ms filled in by stop
     double flops = 0.0;
     double bytes = 0.0;
 };
@@ -40,6 +44,7 @@ struct ProfileScope {
         HIPCX_CHECK_HIP(hipEventCreate(&start));
         HIPCX_CHECK_HIP(hipEventCreate(&stop));
         g_profile.events.emplace_back(start, stop);
+        g_profile.records.push_back(ProfileRecord{0.0, flops, bytes});
         g_profile.flops += flops;
         g_profile.bytes += bytes;
         HIPCX_CHECK_HIP(hipEventRecord(start, stream));
@@ -777,11 +782,13 @@ int hipcx_profile_stop(int64_t* launches, double* total_ms, double* flops, doubl
         HIPCX_REQUIRE(g_profile.on, HIPCX_CHAINERX_ERROR, "profiling is not on");
         g_profile.on = false;
         double ms = 0.0;
-        for (auto& ev : g_profile.events) {
+        for (size_t i = 0; i < g_profile.events.size(); ++i) {
+            auto& ev = g_profile.events[i];
             HIPCX_CHECK_HIP(hipEventSynchronize(ev.second));
             float t = 0.f;
             HIPCX_CHECK_HIP(hipEventElapsedTime(&t, ev.first, ev.second));
             ms += t;
+            g_profile.records[i].ms = t;
             (void)hipEventDestroy(ev.first);
             (void)hipEventDestroy(ev.second);
         }
@@ -790,6 +797,20 @@ int hipcx_profile_stop(int64_t* launches, double* total_ms, double* flops, doubl
         if (flops) *flops = g_profile.flops;
         if (bytes) *bytes = g_profile.bytes;
         g_profile.events.clear();
+    });
+}
+
+int hipcx_profile_records(int64_t capacity, double* ms, double* flops, double* bytes, int64_t* count) {
+    return Guard([&] {
+        std::lock_guard<std::mutex> lock(g_profile_mutex);
+        HIPCX_REQUIRE(!g_profile.on, HIPCX_CHAINERX_ERROR, "profiling is still on: call hipcx_profile_stop first");
+        const int64_t n = static_cast<int64_t>(g_profile.records.size());
+        if (count) *count = n;
+        for (int64_t i = 0; i < n && i < capacity; ++i) {
+            if (ms) ms[i] = g_profile.records[i].ms;
+            if (flops) flops[i] = g_profile.records[i].flops;
+            if (bytes) bytes[i] = g_profile.records[i].bytes;
+        }
     });
 }
 

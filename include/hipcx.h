@@ -326,6 +326,9 @@ int hipcx_lstm_cell(const hipcx_array* c, const hipcx_array* x, const hipcx_arra
  * bytes (each operand once).  One profiling window per process at a time; launches from any thread are recorded into it. */
 int hipcx_profile_start(void);
 int hipcx_profile_stop(int64_t* launches, double* total_ms, double* flops, double* bytes);
+/* The launches of the last closed profiling window one by one, in launch order: duration, algorithmic flops and bytes of the
+ * first min(capacity, *count) of them; *count is the number recorded.  Valid until the next hipcx_profile_start. */
+int hipcx_profile_records(int64_t capacity, double* ms, double* flops, double* bytes, int64_t* count);
 
 /* ---- normalization: FixedBatchNormKernel CX/kernels/normalization.h:107 ----
  * gamma/beta/mean/var have the keep-dims reduced shape of x over `axis`
