@@ -193,6 +193,11 @@ SIGNATURES = {
     'hipcx_profile_start': (_INT, []),
     'hipcx_profile_stop': (_INT, [_I64P, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double),
                                   ctypes.POINTER(ctypes.c_double)]),
+    'hipcx_im2col': (_INT, [_A, _I64P, _I64P, _INT, _S, _A, _V]),
+    'hipcx_col2im': (_INT, [_A, _I64P, _I64P, _A, _V]),
+    'hipcx_conv_transpose_workspace_size': (_SZ, [_A, _A, _I64P, _I64P, _A]),
+    'hipcx_conv_transpose': (_INT, [_A, _A, _A, _I64P, _I64P, _A, _V, _SZ, _V]),
+    'hipcx_batch_norm_supported': (_INT, [_A, _I8P, _INT, ctypes.POINTER(_A), _INT]),
     'hipcx_profile_records': (_INT, [ctypes.c_int64, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double),
                                      ctypes.POINTER(ctypes.c_double), _I64P]),
     'hipcx_fixed_batch_norm': (_INT, [_A, _A, _A, _A, _A, _S, _I8P, _INT, _A, _V]),

@@ -370,6 +370,22 @@ using namespace hipcx;
 
 extern "C" {
 
+int hipcx_batch_norm_supported(const hipcx_array* x, const int8_t* axis, int naxis, const hipcx_array* const* params, int nparams) {
+    try {
+        if (x == nullptr || (nparams > 0 && params == nullptr)) return 0;
+        const BnTrainGeom g = MakeGeom(x, axis, naxis);
+        const int64_t total = static_cast<int64_t>(g.N) * g.C * g.L;
+        if (total == 0 || total >= (int64_t{1} << 31)) return 0;
+        for (int i = 0; i < nparams; ++i) {
+            if (params[i] == nullptr) return 0;
+            (void)ChannelStride(params[i], x, "parameter");
+        }
+        return 1;
+    } catch (...) {
+        return 0;
+    }
+}
+
 size_t hipcx_batch_norm_workspace_size(const hipcx_array* x, const int8_t* axis, int naxis) {
     try {
         if (x == nullptr) return 0;

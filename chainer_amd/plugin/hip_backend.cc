@@ -77,11 +77,19 @@ void CheckHip(hipError_t e, const char* what) {
     if (e != hipSuccess) throw BackendError{what, ": ", hipGetErrorString(e)};
 }
 
+// The error of a device allocation that fails even after the pool has released its cache (the CUDA backend's class of the
+// same name, chainerx/cuda/memory_pool.h:34-37, lives in that backend's namespace and is not visible to a plugin).
+class OutOfMemoryError : public ChainerxError {
+public:
+    using ChainerxError::ChainerxError;
+};
+
 // hipcx_status -> the ChainerX exception class named by it (chainerx/error.h:48-95).
 void Check(int status) {
     if (status == HIPCX_OK) return;
     std::string msg = hipcx_last_error();
     switch (status) {
+        case HIPCX_OUT_OF_MEMORY_ERROR: throw OutOfMemoryError{msg};
         case HIPCX_DIMENSION_ERROR: throw DimensionError{msg};
         case HIPCX_DTYPE_ERROR: throw DtypeError{msg};
         case HIPCX_NOT_IMPLEMENTED_ERROR: throw NotImplementedError{msg};
@@ -145,106 +153,63 @@ hipcx_scalar ToC(Scalar s) {
 
 std::vector<int8_t> ToC(const Axes& axes) { return std::vector<int8_t>(axes.begin(), axes.end()); }
 
-// Caching device allocator: power-of-two-ish size classes of 512-byte units, free blocks kept per
-// class, everything released and the request retried once when hipMalloc fails.  Buffers are
-// shared_ptr<void> whose deleter hands the block back; the pool outlives its buffers through a
-// shared_ptr held by each deleter, and the deleter never throws.
-class MemoryPool : public std::enable_shared_from_this<MemoryPool> {
-public:
-    explicit MemoryPool(int device_index) : device_index_{device_index} {}
-    ~MemoryPool() { FreeAll(); }
-
-    std::shared_ptr<void> Allocate(size_t bytesize) {
-        if (bytesize == 0) return nullptr;  // native does the same (native_device/memory.cc:14-19)
-        size_t size = RoundUp(bytesize);
-        void* ptr = nullptr;
-        {
-            std::lock_guard<std::mutex> lock{mutex_};
-            auto it = free_.find(size);
-            if (it != free_.end() && !it->second.empty()) {
-                ptr = it->second.back();
-                it->second.pop_back();
-            }
-        }
-        if (ptr == nullptr) {
-            SetDeviceScope scope{device_index_};
-            hipError_t e = hipMalloc(&ptr, size);
-            if (e != hipSuccess) {
-                (void)hipGetLastError();
-                FreeAll();
-                CheckHip(hipMalloc(&ptr, size), "hipMalloc");
-            }
-        }
-        std::shared_ptr<MemoryPool> self = shared_from_this();
-        return std::shared_ptr<void>{ptr, [self, size](void* p) noexcept { self->Release(p, size); }};
-    }
-
-private:
-    static size_t RoundUp(size_t n) {
-        constexpr size_t kUnit = 512;
-        size_t units = (n + kUnit - 1) / kUnit;
-        size_t cls = 1;
-        while (cls < units) cls += (cls < 8 ? 1 : cls / 8);  // 12.5 % steps above 4 KiB
-        return cls * kUnit;
-    }
-    void Release(void* p, size_t size) noexcept {
-        try {
-            std::lock_guard<std::mutex> lock{mutex_};
-            free_[size].push_back(p);
-        } catch (...) {
-            (void)hipFree(p);
-        }
-    }
-    void FreeAll() noexcept {
-        std::lock_guard<std::mutex> lock{mutex_};
-        for (auto& kv : free_) {
-            for (void* p : kv.second) (void)hipFree(p);
-        }
-        free_.clear();
-    }
-
-    int device_index_;
-    std::mutex mutex_;
-    std::map<size_t, std::vector<void*>> free_;
-};
+// A device int32 that a kernel raises (index out of range, LAPACK-style info): zeroed with a fill kernel, read back with the
+// library's blocking device-to-host copy.
+std::shared_ptr<void> NewDeviceFlag(Device& device) {
+    std::shared_ptr<void> flag = device.Allocate(sizeof(int32_t));
+    hipcx_array d{};
+    d.data = flag.get();
+    d.dtype = HIPCX_INT32;
+    d.ndim = 1;
+    d.shape[0] = 1;
+    d.strides[0] = sizeof(int32_t);
+    hipcx_scalar zero{};
+    zero.kind = HIPCX_KIND_INT;
+    Check(hipcx_fill(&d, zero, nullptr));
+    return flag;
+}
+int32_t ReadDeviceFlag(Device& device, const std::shared_ptr<void>& flag) {
+    int32_t host = 0;
+    Check(hipcx_memcpy_to_host(device.index(), &host, flag.get(), sizeof(int32_t), nullptr));
+    return host;
+}
 
 class HipBackend;
 
+// The Device interface (chainerx/device.h:24-71) over the library's device layer: every allocation comes from the pool behind
+// hipcx_malloc and goes back through hipcx_free (the deleter never throws and outlives the pool: a free after
+// hipcx_pool_destroy is a no-op inside the library), copies are the library's.
 class HipDevice : public Device {
 public:
-    HipDevice(Backend& backend, int index) : Device{backend, index}, pool_{std::make_shared<MemoryPool>(index)} {}
+    HipDevice(Backend& backend, int index) : Device{backend, index} {}
 
-    std::shared_ptr<void> Allocate(size_t bytesize) override { return pool_->Allocate(bytesize); }
+    std::shared_ptr<void> Allocate(size_t bytesize) override {
+        void* ptr = nullptr;
+        Check(hipcx_malloc(index(), bytesize, &ptr));  // 0 bytes -> nullptr; HIPCX_OUT_OF_MEMORY_ERROR -> OutOfMemoryError
+        return Wrap(ptr);
+    }
 
     std::shared_ptr<void> MakeDataFromForeignPointer(const std::shared_ptr<void>& data) override {
         if (data == nullptr) return data;
-        hipPointerAttribute_t attr{};
-        SetDeviceScope scope{index()};
-        hipError_t e = hipPointerGetAttributes(&attr, data.get());
-        if (e != hipSuccess || attr.device != index()) {
-            (void)hipGetLastError();
-            throw ChainerxError{"Memory is not a HIP allocation of device ", name()};
-        }
+        Check(hipcx_check_device_pointer(index(), data.get()));
         return data;
     }
 
     void MemoryCopyFrom(void* dst, const void* src, size_t bytesize, Device& src_device) override {
         if (bytesize == 0) return;
-        SetDeviceScope scope{index()};
-        if (&src_device == this || dynamic_cast<HipDevice*>(&src_device) != nullptr) {
-            CheckHip(hipMemcpyAsync(dst, src, bytesize, hipMemcpyDeviceToDevice, nullptr), "hipMemcpyAsync");
-        } else {  // native (host) source: blocking, like the CUDA backend (cuda/cuda_device/memory.cc:94-110)
-            CheckHip(hipMemcpy(dst, src, bytesize, hipMemcpyHostToDevice), "hipMemcpy");
+        if (auto* other = dynamic_cast<HipDevice*>(&src_device)) {
+            Check(hipcx_memcpy_device(index(), dst, other->index(), src, bytesize, nullptr));
+        } else {  // native (host) source
+            Check(hipcx_memcpy_from_host(index(), dst, src, bytesize, nullptr));
         }
     }
 
     void MemoryCopyTo(void* dst, const void* src, size_t bytesize, Device& dst_device) override {
         if (bytesize == 0) return;
-        SetDeviceScope scope{index()};
-        if (&dst_device == this || dynamic_cast<HipDevice*>(&dst_device) != nullptr) {
-            CheckHip(hipMemcpyAsync(dst, src, bytesize, hipMemcpyDeviceToDevice, nullptr), "hipMemcpyAsync");
+        if (auto* other = dynamic_cast<HipDevice*>(&dst_device)) {
+            Check(hipcx_memcpy_device(other->index(), dst, index(), src, bytesize, nullptr));
         } else {
-            CheckHip(hipMemcpy(dst, src, bytesize, hipMemcpyDeviceToHost), "hipMemcpy");
+            Check(hipcx_memcpy_to_host(index(), dst, src, bytesize, nullptr));
         }
     }
 
@@ -261,18 +226,19 @@ public:
     }
 
     std::shared_ptr<void> FromHostMemory(const std::shared_ptr<void>& src_ptr, size_t bytesize) override {
-        std::shared_ptr<void> dst = Allocate(bytesize);
-        if (bytesize != 0) {
-            SetDeviceScope scope{index()};
-            CheckHip(hipMemcpy(dst.get(), src_ptr.get(), bytesize, hipMemcpyHostToDevice), "hipMemcpy");
-        }
-        return dst;
+        void* ptr = nullptr;
+        Check(hipcx_from_host_memory(index(), src_ptr.get(), bytesize, &ptr, nullptr));
+        return Wrap(ptr);
     }
 
     void Synchronize() override { Check(hipcx_synchronize(index())); }
 
 private:
-    std::shared_ptr<MemoryPool> pool_;
+    std::shared_ptr<void> Wrap(void* ptr) {
+        if (ptr == nullptr) return nullptr;
+        const int device = index();
+        return std::shared_ptr<void>{ptr, [device](void* p) noexcept { (void)hipcx_free(device, p); }};
+    }
 };
 
 }  // namespace
@@ -870,40 +836,28 @@ public:
 };
 HIPCX_REGISTER_KERNEL(AveragePoolKernel, HipAveragePoolKernel)
 
-// ---- backward / training kernels: compositions over the kernels above, the way the native backend composes them ----
-// Im2Col (CX/native/im2col.cc:82-149) with the gather done by one strided Copy kernel per kernel offset.
+// ---- backward / training kernels ----
+// Im2Col (CX/native/im2col.cc:82-149) and Col2Im (CX/native/col2im.cc:76-122): one library call each.
 Array HipIm2Col(const Array& x, const Dims& k, const Dims& s, const Dims& p, bool cover_all, Scalar pad_value) {
     if (x.ndim() != 4) throw NotImplementedError{"hip backward kernels support 2 spatial dimensions."};
     Device& device = x.device();
+    SetDeviceScope scope{device.index()};
     int64_t oh = OutDim(x.shape()[2], k[0], s[0], p[0], cover_all), ow = OutDim(x.shape()[3], k[1], s[1], p[1], cover_all);
-    Shape padded_shape{x.shape()[0], x.shape()[1], x.shape()[2] + 2 * p[0] + (cover_all ? s[0] - 1 : 0),
-                       x.shape()[3] + 2 * p[1] + (cover_all ? s[1] - 1 : 0)};
-    Array padded = Full(padded_shape, pad_value, x.dtype(), device);
-    device.backend().CallKernel<CopyKernel>(x, padded.At({Slice{}, Slice{}, Slice{p[0], p[0] + x.shape()[2]}, Slice{p[1], p[1] + x.shape()[3]}}));
     Array col = Empty(Shape{x.shape()[0], x.shape()[1], k[0], k[1], oh, ow}, x.dtype(), device);
-    for (int64_t r = 0; r < k[0]; ++r) {
-        for (int64_t q = 0; q < k[1]; ++q) {
-            device.backend().CallKernel<CopyKernel>(
-                    padded.At({Slice{}, Slice{}, Slice{r, r + s[0] * oh, s[0]}, Slice{q, q + s[1] * ow, s[1]}}),
-                    col.At({Slice{}, Slice{}, ArrayIndex{r}, ArrayIndex{q}}));
-        }
-    }
+    hipcx_array cx = ToC(x), cc = ToC(col);
+    int64_t st[2] = {s[0], s[1]}, pd[2] = {p[0], p[1]};
+    Check(hipcx_im2col(&cx, st, pd, cover_all ? 1 : 0, ToC(pad_value), &cc, nullptr));
     return col;
 }
 
-// Col2Im (CX/native/col2im.cc:76-122): in-place strided Add kernels in the reference's (r, s) order.
 Array HipCol2Im(const Array& col, const Dims& s, const Dims& p, const Dims& out_size) {
     Device& device = col.device();
-    int64_t kh = col.shape()[2], kw = col.shape()[3], h = col.shape()[4], w = col.shape()[5];
-    Array padded = Zeros(Shape{col.shape()[0], col.shape()[1], out_size[0] + 2 * p[0] + s[0] - 1, out_size[1] + 2 * p[1] + s[1] - 1},
-                         col.dtype(), device);
-    for (int64_t r = 0; r < kh; ++r) {
-        for (int64_t q = 0; q < kw; ++q) {
-            Array view = padded.At({Slice{}, Slice{}, Slice{r, r + s[0] * h, s[0]}, Slice{q, q + s[1] * w, s[1]}});
-            device.backend().CallKernel<AddKernel>(view, col.At({Slice{}, Slice{}, ArrayIndex{r}, ArrayIndex{q}}), view);
-        }
-    }
-    return padded.At({Slice{}, Slice{}, Slice{p[0], p[0] + out_size[0]}, Slice{p[1], p[1] + out_size[1]}});
+    SetDeviceScope scope{device.index()};
+    Array out = Empty(Shape{col.shape()[0], col.shape()[1], out_size[0], out_size[1]}, col.dtype(), device);
+    hipcx_array cc = ToC(col), co = ToC(out);
+    int64_t st[2] = {s[0], s[1]}, pd[2] = {p[0], p[1]};
+    Check(hipcx_col2im(&cc, st, pd, &co, nullptr));
+    return out;
 }
 
 class HipConvGradWeightKernel : public ConvGradWeightKernel {
@@ -938,31 +892,26 @@ public:
                Dtype out_dtype, const absl::optional<Array>& out) override {
         if (out.has_value()) throw NotImplementedError{"Passing out as an argument is not yet supported."};
         if (x.ndim() != 4) throw NotImplementedError{"hip convolution supports 2 spatial dimensions."};
-        SetDeviceScope scope{x.device().index()};
-        const int64_t kh = w.shape()[2], kw = w.shape()[3];
-        if (stride[0] == 1 && stride[1] == 1 && pad[0] <= kh - 1 && pad[1] <= kw - 1 && GetKind(out_dtype) == DtypeKind::kFloat &&
-            out_size[0] == x.shape()[2] - 1 + kh - 2 * pad[0] && out_size[1] == x.shape()[3] - 1 + kw - 2 * pad[1]) {
-            // stride 1: a forward convolution with the filters flipped in both spatial axes, channel axes swapped, padding k - 1 - p
-            Array w_flipped = Flip(w, Axes{2, 3}).Transpose(Axes{1, 0, 2, 3}).Copy();
-            return x.device().backend().CallKernel<ConvKernel>(x, w_flipped, b, Dims{1, 1}, Dims{kh - 1 - pad[0], kw - 1 - pad[1]}, false,
-                                                               out_dtype, absl::nullopt);
-        }
-        if (kh == 1 && kw == 1 && pad[0] == 0 && pad[1] == 0 && GetKind(out_dtype) == DtypeKind::kFloat && x.GetTotalSize() > 0) {
-            // a 1x1 filter at any stride: every input pixel lands on one output pixel, so the result is a 1x1 forward convolution
-            // (channel axes of w swapped) scattered to every stride-th pixel of a zero-filled output
-            Array y1 = x.device().backend().CallKernel<ConvKernel>(x, w.Transpose(Axes{1, 0, 2, 3}).Copy(), absl::nullopt, Dims{1, 1},
-                                                                   Dims{0, 0}, false, out_dtype, absl::nullopt);
-            Array actual_out = Zeros(Shape{x.shape()[0], w.shape()[1], out_size[0], out_size[1]}, out_dtype, x.device());
-            // cover_all sizes: the last input row / column may fall outside the output
-            const int64_t hh = std::min(x.shape()[2], (out_size[0] + stride[0] - 1) / stride[0]);
-            const int64_t ww = std::min(x.shape()[3], (out_size[1] + stride[1] - 1) / stride[1]);
-            Array view = actual_out.At({Slice{}, Slice{}, Slice{0, hh * stride[0], stride[0]}, Slice{0, ww * stride[1], stride[1]}});
-            x.device().backend().CallKernel<CopyKernel>(y1.At({Slice{}, Slice{}, Slice{0, hh}, Slice{0, ww}}), view);
-            if (b.has_value()) {
-                actual_out += b->AsType(out_dtype, false).Reshape(Shape{1, b->shape()[0], 1, 1});
-            }
+        Device& device = x.device();
+        device.CheckDevicesCompatible(x, w);
+        if (b.has_value()) device.CheckDevicesCompatible(x, *b);
+        SetDeviceScope scope{device.index()};
+        if (GetKind(out_dtype) == DtypeKind::kFloat) {
+            // one entry: it picks the flipped forward convolution (stride 1), the scattered 1x1 convolution or the native
+            // composition (matrix product over the input channels, col2im, bias) by itself
+            Array xc = x.dtype() == out_dtype ? x : x.AsType(out_dtype);
+            Array wc = w.dtype() == out_dtype ? w : w.AsType(out_dtype);
+            absl::optional<Array> bc = b.has_value() ? absl::optional<Array>{b->dtype() == out_dtype ? *b : b->AsType(out_dtype)} : absl::nullopt;
+            Array actual_out = Empty(Shape{x.shape()[0], w.shape()[1], out_size[0], out_size[1]}, out_dtype, device);
+            hipcx_array cx = ToC(xc), cw = ToC(wc), co = ToC(actual_out), cb{};
+            if (bc.has_value()) cb = ToC(*bc);
+            int64_t st[2] = {stride[0], stride[1]}, pd[2] = {pad[0], pad[1]};
+            size_t ws_bytes = hipcx_conv_transpose_workspace_size(&cx, &cw, st, pd, &co);
+            std::shared_ptr<void> ws = device.Allocate(ws_bytes);
+            Check(hipcx_conv_transpose(&cx, &cw, bc.has_value() ? &cb : nullptr, st, pd, &co, ws.get(), ws_bytes, nullptr));
             return actual_out;
         }
+        // other dtypes: the native composition on this backend's kernels (TensorDot dispatches DotKernel here)
         Array col = native::TensorDot(w, x, Axes{0}, Axes{1}, out_dtype);  // [C_out, kh, kw, N, H, W]
         Array actual_out = HipCol2Im(col.Transpose(Axes{3, 0, 1, 2, 4, 5}), stride, pad, out_size);
         if (b.has_value()) {
@@ -978,16 +927,15 @@ HIPCX_REGISTER_KERNEL(ConvTransposeKernel, HipConvTransposeKernel)
 // dedicated kernels do not take (a non-contiguous x, mixed dtypes, other axis sets).  The state handed to the gradient is the
 // generic one (batch mean, 1 / sqrt(var + eps), dtype of beta), so either gradient kernel can consume either forward's state.
 namespace {
+// Whether hipcx_batch_norm / hipcx_batch_norm_grad take this case: the library decides (hipcx_batch_norm_supported).
 bool HipBatchNormApplies(const Array& x, const Axes& axis, std::initializer_list<const Array*> others) {
-    if (x.ndim() < 2 || !x.IsContiguous() || x.GetTotalSize() == 0 || x.GetTotalSize() >= (int64_t{1} << 31)) return false;
-    if (static_cast<int8_t>(axis.size()) != x.ndim() - 1) return false;
-    for (int8_t i = 0; i < static_cast<int8_t>(axis.size()); ++i) {
-        if (axis[i] != (i == 0 ? 0 : i + 1)) return false;
-    }
-    for (const Array* a : others) {
-        if (a->dtype() != x.dtype()) return false;
-    }
-    return true;
+    hipcx_array cx = ToC(x);
+    std::vector<int8_t> ax = ToC(axis);
+    std::vector<hipcx_array> descs;
+    for (const Array* a : others) descs.push_back(ToC(*a));
+    std::vector<const hipcx_array*> ptrs;
+    for (const hipcx_array& d : descs) ptrs.push_back(&d);
+    return hipcx_batch_norm_supported(&cx, ax.data(), static_cast<int>(ax.size()), ptrs.data(), static_cast<int>(ptrs.size())) == 1;
 }
 }  // namespace
 
@@ -1117,14 +1065,9 @@ HIPCX_REGISTER_KERNEL(AveragePoolGradKernel, HipAveragePoolGradKernel)
 // ---- linear algebra: Solve, Inverse, Cholesky, Syevd, Qr, Svd (the LAPACK-backed kernels of the native backend, native_device/linalg.cc) ----
 namespace {
 // A zeroed device int32 for LAPACK's `info`, and the check that turns a non-zero value into the reference's ChainerxError.
-std::shared_ptr<void> NewInfoFlag(Device& device) {
-    std::shared_ptr<void> flag = device.Allocate(sizeof(int32_t));
-    CheckHip(hipMemsetAsync(flag.get(), 0, sizeof(int32_t), nullptr), "hipMemsetAsync");
-    return flag;
-}
-void ThrowIfInfo(const std::shared_ptr<void>& flag, const char* what) {
-    int32_t host = 0;
-    CheckHip(hipMemcpy(&host, flag.get(), sizeof(int32_t), hipMemcpyDeviceToHost), "hipMemcpy");
+std::shared_ptr<void> NewInfoFlag(Device& device) { return NewDeviceFlag(device); }
+void ThrowIfInfo(Device& device, const std::shared_ptr<void>& flag, const char* what) {
+    const int32_t host = ReadDeviceFlag(device, flag);
     if (host != 0) throw ChainerxError{"Unsuccessful ", what, " execution. Info = ", host};
 }
 }  // namespace
@@ -1141,7 +1084,7 @@ public:
         std::shared_ptr<void> ws = device.Allocate(ws_bytes);
         std::shared_ptr<void> flag = NewInfoFlag(device);
         Check(hipcx_solve(&ca, &cb, &co, ws.get(), ws_bytes, static_cast<int32_t*>(flag.get()), nullptr));
-        ThrowIfInfo(flag, "gesv (Solve)");
+        ThrowIfInfo(device, flag, "gesv (Solve)");
     }
 };
 HIPCX_REGISTER_KERNEL(SolveKernel, HipSolveKernel)
@@ -1158,7 +1101,7 @@ public:
         std::shared_ptr<void> ws = device.Allocate(ws_bytes);
         std::shared_ptr<void> flag = NewInfoFlag(device);
         Check(hipcx_inverse(&ca, &co, ws.get(), ws_bytes, static_cast<int32_t*>(flag.get()), nullptr));
-        ThrowIfInfo(flag, "getrf (LU)");
+        ThrowIfInfo(device, flag, "getrf (LU)");
     }
 };
 HIPCX_REGISTER_KERNEL(InverseKernel, HipInverseKernel)
@@ -1173,7 +1116,7 @@ public:
         hipcx_array ca = ToC(a), co = ToC(out);
         std::shared_ptr<void> flag = NewInfoFlag(device);
         Check(hipcx_cholesky(&ca, &co, static_cast<int32_t*>(flag.get()), nullptr));
-        ThrowIfInfo(flag, "potrf (Cholesky)");
+        ThrowIfInfo(device, flag, "potrf (Cholesky)");
     }
 };
 HIPCX_REGISTER_KERNEL(CholeskyKernel, HipCholeskyKernel)
@@ -1250,12 +1193,10 @@ public:
             default: break;
         }
         bool checks = m == HIPCX_BOUNDS_DEFAULT || m == HIPCX_BOUNDS_RAISE;
-        std::shared_ptr<void> flag = checks ? device.Allocate(sizeof(int32_t)) : nullptr;
-        if (checks) CheckHip(hipMemsetAsync(flag.get(), 0, sizeof(int32_t), nullptr), "hipMemsetAsync");
+        std::shared_ptr<void> flag = checks ? NewDeviceFlag(device) : nullptr;
         Check(hipcx_take(&ca, &ci, axis, &co, m, static_cast<int32_t*>(flag.get()), nullptr));
         if (checks) {  // native raises IndexError on an out-of-range index (native_device/indexing.cc:68-74)
-            int32_t host = 0;
-            CheckHip(hipMemcpy(&host, flag.get(), sizeof(int32_t), hipMemcpyDeviceToHost), "hipMemcpy");
+            const int32_t host = ReadDeviceFlag(device, flag);
             if (host != 0) throw IndexError{"Index is out of bounds for axis ", static_cast<int>(axis), " with size ", a.shape()[axis]};
         }
     }
@@ -1280,12 +1221,10 @@ public:
         hipcx_array ca = ToC(a), ci = ToC(indices), cb = ToC(Cast(b, a.dtype())), co = ToC(out);
         int m = ToC(mode);
         bool checks = m == HIPCX_BOUNDS_DEFAULT || m == HIPCX_BOUNDS_RAISE;
-        std::shared_ptr<void> flag = checks ? device.Allocate(sizeof(int32_t)) : nullptr;
-        if (checks) CheckHip(hipMemsetAsync(flag.get(), 0, sizeof(int32_t), nullptr), "hipMemsetAsync");
+        std::shared_ptr<void> flag = checks ? NewDeviceFlag(device) : nullptr;
         Check(hipcx_add_at(&ca, &ci, axis, &cb, &co, m, static_cast<int32_t*>(flag.get()), nullptr));
         if (checks) {
-            int32_t host = 0;
-            CheckHip(hipMemcpy(&host, flag.get(), sizeof(int32_t), hipMemcpyDeviceToHost), "hipMemcpy");
+            const int32_t host = ReadDeviceFlag(device, flag);
             if (host != 0) throw IndexError{"Index is out of bounds for axis ", static_cast<int>(axis), " with size ", a.shape()[axis]};
         }
     }

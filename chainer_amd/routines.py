@@ -1420,15 +1420,24 @@ def _copy_into(dst_view, src):
     _lib.call('hipcx_copy', src.desc(), dst_view.desc(), current_stream())
 
 
+# True: Im2Col / Col2Im run as the native backend's chains of strided Copy / Add kernel calls instead of one launch each.
+COMPOSE_IM2COL = False
+
+
 def im2col(x, ksize, stride, pad, cover_all=False, pad_value=0):
-    """native_internal::Im2Col (CX/native/im2col.cc:82-149): a padded copy of x, then one strided Copy per kernel offset into
-    col[N, C, kh, kw, oh, ow]."""
+    """native_internal::Im2Col (CX/native/im2col.cc:82-149): col[N, C, kh, kw, oh, ow] -- one hipcx_im2col launch, or (COMPOSE_IM2COL)
+    a padded copy of x and one strided Copy per kernel offset as the native backend does it."""
     n, c, h, w = x.shape
     kh, kw = ksize
     sh, sw = stride
     ph, pw = pad
     oh = conv_out_dim(h, kh, sh, ph, cover_all)
     ow = conv_out_dim(w, kw, sw, pw, cover_all)
+    if not COMPOSE_IM2COL:
+        col = ndarray.empty((n, c, kh, kw, oh, ow), x.dtype)
+        _lib.call('hipcx_im2col', x.desc(), _i64((sh, sw)), _i64((ph, pw)), int(bool(cover_all)), _lib.make_scalar(pad_value), col.desc(),
+                  current_stream())
+        return col
     hp = h + 2 * ph + (sh - 1 if cover_all else 0)
     wp = w + 2 * pw + (sw - 1 if cover_all else 0)
     xp = full((n, c, hp, wp), pad_value, x.dtype)
@@ -1447,6 +1456,10 @@ def col2im(col, stride, pad, out_size):
     sh, sw = stride
     ph, pw = pad
     oh, ow = out_size
+    if not COMPOSE_IM2COL:  # one launch: every image position sums its contributions in the same order, with the same roundings
+        out = ndarray.empty((n, c, oh, ow), col.dtype)
+        _lib.call('hipcx_col2im', col.desc(), _i64((sh, sw)), _i64((ph, pw)), out.desc(), current_stream())
+        return out
     padded = zeros((n, c, oh + 2 * ph + sh - 1, ow + 2 * pw + sw - 1), col.dtype)
     for r in range(kh):
         for q in range(kw):
@@ -1508,6 +1521,9 @@ def conv_grad_weight(w_dtype, w_shape, x, gy, stride=1, pad=0, cover_all=False):
 
 # True: ConvTranspose always runs as the native backend's TensorDot + Col2Im composition.
 COMPOSE_CONV_TRANSPOSE = False
+# True: the route (flipped convolution / scattered 1x1 convolution / composition) is chosen and issued from here, kernel call by
+# kernel call, instead of inside hipcx_conv_transpose.
+ROUTE_CONV_TRANSPOSE_HERE = False
 
 
 def conv_transpose(x, w, b=None, stride=1, pad=0, out_size=None, out_dtype=None):
@@ -1527,6 +1543,17 @@ def conv_transpose(x, w, b=None, stride=1, pad=0, out_size=None, out_dtype=None)
             if d != conv_out_dim(o, k, st, p, False) and d != conv_out_dim(o, k, st, p, True):
                 raise _lib.DimensionError('Output dims %r is incosistent.' % (out_size,))
     dt = numpy.dtype(out_dtype) if out_dtype is not None else (result_type(x, w, b) if b is not None else result_type(x, w))
+    if not COMPOSE_CONV_TRANSPOSE and not ROUTE_CONV_TRANSPOSE_HERE and _kind(dt) == 3:
+        # one entry: it picks the flipped forward convolution, the scattered 1x1 convolution or the native composition itself
+        xc, wc = x.astype(dt, False), w.astype(dt, False)
+        bc = b.astype(dt, False) if b is not None else None
+        out = ndarray.empty((x.shape[0], w.shape[1]) + tuple(out_size), dt)
+        st, pd = _i64(stride), _i64(pad)
+        nbytes = _lib.load().hipcx_conv_transpose_workspace_size(xc.desc(), wc.desc(), st, pd, out.desc())
+        ws, wsp = _workspace(nbytes)
+        _lib.call('hipcx_conv_transpose', xc.desc(), wc.desc(), bc.desc() if bc is not None else None, st, pd, out.desc(), wsp, nbytes,
+                  current_stream())
+        return out
     if (not COMPOSE_CONV_TRANSPOSE and stride == (1, 1) and pad[0] <= kh - 1 and pad[1] <= kw - 1 and _kind(dt) == 3
             and tuple(out_size) == tuple(d - 1 + k - 2 * p for d, k, p in zip(x.shape[2:], (kh, kw), pad))):
         # At stride 1 the transposed convolution is a forward convolution with the filters flipped in both spatial axes, their

@@ -291,6 +291,26 @@ size_t hipcx_conv_workspace_size(const hipcx_array* x, const hipcx_array* w, con
 int hipcx_conv(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, const int64_t* stride, const int64_t* pad,
                int cover_all, const hipcx_array* out, void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---- Im2Col / Col2Im (CX/native/im2col.cc:82-149, col2im.cc:76-122) and ConvTransposeKernel (CX/kernels/connection.h:51-66) ----
+ * Two spatial axes; arrays of any strides (multiples of the item size).
+ * hipcx_im2col: col[N, C, kh, kw, oh, ow] (kernel and window extents are read from col's shape; oh / ow must be
+ *   hipcx_conv_out_dim of x's) gathered from x[N, C, H, W]; positions in the padding hold pad_value.  Any dtype.
+ * hipcx_col2im: out[N, C, H, W] = for every image position the sum of the col elements that cover it, added in ascending
+ *   (r, s) order from zero with one rounding to the dtype per addition: bit-identical to the native backend's chain of in-place
+ *   strided Add kernels on a zero-filled padded image, cropped.  Any dtype but bool.
+ * hipcx_conv_transpose: x[N, C_in, H, W], w[C_in, C_out, kh, kw], optional b[C_out], out[N, C_out, OH, OW] with OH / OW any size
+ *   consistent with x's (CX/routines/connection.cc:268-279); all of one floating point dtype.  Stride 1 runs as one forward
+ *   convolution with flipped filters, a 1x1 unpadded filter as a 1x1 convolution scattered into zeros, everything else as the
+ *   native composition (matrix product over the input channels, col2im, bias).  `workspace`: 256-byte aligned device memory of
+ *   hipcx_conv_transpose_workspace_size bytes. */
+int hipcx_im2col(const hipcx_array* x, const int64_t* stride, const int64_t* pad, int cover_all, hipcx_scalar pad_value,
+                 const hipcx_array* col, void* stream);
+int hipcx_col2im(const hipcx_array* col, const int64_t* stride, const int64_t* pad, const hipcx_array* out, void* stream);
+size_t hipcx_conv_transpose_workspace_size(const hipcx_array* x, const hipcx_array* w, const int64_t* stride, const int64_t* pad,
+                                           const hipcx_array* out);
+int hipcx_conv_transpose(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, const int64_t* stride, const int64_t* pad,
+                         const hipcx_array* out, void* workspace, size_t workspace_bytes, void* stream);
+
 /* Opt-in fused entry.  No single kernel of the reference corresponds to it: it is the composition
  *   ConvKernel -> FixedBatchNormKernel over the output channels (axis (0,2,3), CX/routines/normalization.cc:113-153)
  *   -> AddKernel with `residual` -> IfLessElseASSAKernel(x, 0, 0, x) (ReLU, CX/routines/misc.cc:210-216)
@@ -394,6 +414,9 @@ int hipcx_svd(const hipcx_array* a, const hipcx_array* u, const hipcx_array* s, 
  * hipcx_batch_norm writes out, the batch mean and 1 / sqrt(var + eps) (the state the gradient needs) and updates running_mean /
  * running_var in place (decay, and n / max(n - 1, 1) on the variance).  Both need hipcx_batch_norm_workspace_size bytes. */
 size_t hipcx_batch_norm_workspace_size(const hipcx_array* x, const int8_t* axis, int naxis);
+/* 1 when hipcx_batch_norm / hipcx_batch_norm_grad take this case (x, the axis set, and `nparams` per-channel arrays: gamma,
+ * beta, running statistics, or gout's state), 0 when the caller has to run the routine composition.  Sets no error. */
+int hipcx_batch_norm_supported(const hipcx_array* x, const int8_t* axis, int naxis, const hipcx_array* const* params, int nparams);
 int hipcx_batch_norm(const hipcx_array* x, const hipcx_array* gamma, const hipcx_array* beta, const hipcx_array* running_mean,
                      const hipcx_array* running_var, hipcx_scalar eps, hipcx_scalar decay, const int8_t* axis, int naxis,
                      const hipcx_array* out, const hipcx_array* mean_out, const hipcx_array* inv_std_out, void* workspace,

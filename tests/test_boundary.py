@@ -40,6 +40,26 @@ def test_library_exports_every_declared_symbol():
     assert sorted(s for s in exported if s.startswith('hipcx_')) == names
 
 
+def test_plugin_glue_only_forwards_to_declared_entry_points():
+    """The ChainerX plugin source cannot be built here (it needs a ChainerX checkout); what can be checked is that every
+    hipcx_* name it uses is declared in the header, and that it reaches device memory only through those entry points."""
+    import re
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    src = open(os.path.join(root, 'chainer_amd', 'plugin', 'hip_backend.cc')).read()
+    header = open(os.path.join(root, 'include', 'hipcx.h')).read()
+    declared = set(re.findall(r'\b(hipcx_[a-z0-9_]+)\s*\(', header))
+    code = re.sub(r'//[^\n]*', '', src)
+    used = set(re.findall(r'\b(hipcx_[a-z0-9_]+)\s*\(', code))
+    assert used, 'no entry point found in the plugin source'
+    assert not (used - declared), 'the plugin calls undeclared entry points: %r' % sorted(used - declared)
+    for name in ('hipcx_malloc', 'hipcx_free', 'hipcx_from_host_memory', 'hipcx_memcpy_to_host', 'hipcx_memcpy_from_host',
+                 'hipcx_memcpy_device', 'hipcx_check_device_pointer', 'hipcx_im2col', 'hipcx_col2im', 'hipcx_conv_transpose',
+                 'hipcx_batch_norm_supported'):
+        assert name in used, name
+    for forbidden in ('hipMalloc', 'hipFree', 'hipMemcpy', 'hipMemset', 'hipLaunchKernelGGL', '__global__'):
+        assert forbidden not in code, 'the plugin glue must not call %s itself' % forbidden
+
+
 def test_struct_layouts_match_header():
     from chainer_amd import _lib
     assert ctypes.sizeof(_lib.CArray) == 8 + 4 + 4 + 8 * 10 + 8 * 10
