@@ -282,13 +282,160 @@ __global__ void ConvNaiveF64Kernel(IGemmArgs<double> p) {
     p.out[img * p.osN + n * p.osC + oh * p.osH + ow * p.osW] = acc;
 }
 
-void LaunchF64(const IGemmArgs<double>& p, hipStream_t stream) {
+// float64 on the matrix cores: implicit GEMM with v_mfma_f64_16x16x4f64, any strides (operands are gathered).
+// A workgroup (4 waves, 2 x 2) computes a 64 (output positions) x 64 (filters) tile; the reduction index k = (c, r, s) advances
+// in chunks of 16 that are gathered into registers one chunk ahead and staged through LDS (two buffers, one barrier per chunk):
+//   As[k][m]  k-major, written with consecutive lanes along m (consecutive pixels: contiguous for NCHW at stride 1)
+//   Bs[n][k]  n-major, written with consecutive lanes along k (contiguous for dense filters)
+// MFMA operands: A lane l <-> (m = l % 16, k = l / 16), B lane l <-> (k = l / 16, n = l % 16); the accumulator register i of lane l
+// is D[m = 4 * i + l / 16][n = l % 16].  Products are summed in k order chunk by chunk, in double: equal to the sequential
+// loop to rounding (tests: 1e-12).
+constexpr int kF64TileM = 64, kF64TileN = 64, kF64Chunk = 16;
+using double4_t = __attribute__((ext_vector_type(4))) double;
+
+__global__ __launch_bounds__(256) void ConvMfmaF64Kernel(IGemmArgs<double> p) {
+    __shared__ double As[2][kF64Chunk][kF64TileM + 2];
+    __shared__ double Bs[2][kF64TileN][kF64Chunk + 1];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = (wave & 1) * 32, wn = (wave >> 1) * 32;
+    const int64_t bm = static_cast<int64_t>(blockIdx.x % p.tiles_m) * kF64TileM;
+    const int bn = static_cast<int>(blockIdx.x / p.tiles_m) * kF64TileN;
+    const int RS = p.R * p.S;
+
+    // ---- A gather: this thread's output position, and k = k0 + a_kk + 4 * i ----
+    const int a_m = tid & 63, a_kk = tid >> 6;
+    const int64_t m = bm + a_m;
+    const bool m_ok = m < p.M;
+    int ih0 = 0, iw0 = 0;
+    const double* xb = p.x;
+    if (m_ok) {
+        const int ow = static_cast<int>(m % p.OW);
+        const int64_t t = m / p.OW;
+        const int oh = static_cast<int>(t % p.OH);
+        const int64_t img = t / p.OH;
+        ih0 = oh * p.stride_h - p.pad_h;
+        iw0 = ow * p.stride_w - p.pad_w;
+        xb = p.x + img * p.xsN + ih0 * p.xsH + iw0 * p.xsW;
+    }
+    // ---- B gather: k = k0 + b_kk, filters n = bn + b_n + 16 * i ----
+    const int b_kk = tid & 15, b_n = tid >> 4;
+    double ra[4], rb[4];
+    auto gather = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int k = k0 + a_kk + 4 * i;
+            double v = 0.0;
+            if (m_ok && k < p.Kg) {
+                int c = k, r = 0, s2 = 0;
+                if (RS != 1) {  // (uniform) a matrix product or a 1x1 filter needs no division
+                    c = k / RS;
+                    const int rs = k - c * RS;
+                    r = rs / p.S;
+                    s2 = rs - r * p.S;
+                }
+                const int ih = ih0 + r, iw = iw0 + s2;
+                if (ih >= 0 && ih < p.H && iw >= 0 && iw < p.W) v = xb[c * p.xsC + r * p.xsH + s2 * p.xsW];
+            }
+            ra[i] = v;
+        }
+        const int k = k0 + b_kk;
+        int64_t woff = 0;
+        if (k < p.Kg) {
+            int c = k, r = 0, s2 = 0;
+            if (RS != 1) {
+                c = k / RS;
+                const int rs = k - c * RS;
+                r = rs / p.S;
+                s2 = rs - r * p.S;
+            }
+            woff = c * p.wsC + r * p.wsR + s2 * p.wsS;
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int n = bn + b_n + 16 * i;
+            rb[i] = (k < p.Kg && n < p.K) ? p.w[static_cast<int64_t>(n) * p.wsK + woff] : 0.0;
+        }
+    };
+    auto stage = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            As[buf][a_kk + 4 * i][a_m] = ra[i];
+            Bs[buf][b_n + 16 * i][b_kk] = rb[i];
+        }
+    };
+
+    double4_t acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = double4_t{0.0, 0.0, 0.0, 0.0};
+    }
+    const int nchunks = (p.Kg + kF64Chunk - 1) / kF64Chunk;
+    gather(0);
+    stage(0);
+    __syncthreads();
+    for (int ch = 0; ch < nchunks; ++ch) {
+        const int cur = ch & 1;
+        if (ch + 1 < nchunks) gather((ch + 1) * kF64Chunk);
+#pragma unroll
+        for (int ks = 0; ks < kF64Chunk / 4; ++ks) {
+            double a[2], b[2];
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                a[t] = As[cur][ks * 4 + (lane >> 4)][wm + t * 16 + (lane & 15)];
+                b[t] = Bs[cur][wn + t * 16 + (lane & 15)][ks * 4 + (lane >> 4)];
+            }
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+#pragma unroll
+                for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[i], b[j], acc[i][j], 0, 0, 0);
+            }
+        }
+        if (ch + 1 < nchunks) stage(cur ^ 1);  // the other buffer: its readers passed the barrier of the previous chunk
+        __syncthreads();
+    }
+
+    // ---- epilogue: bias, scatter through out's strides ----
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int64_t mo = bm + wm + i * 16 + 4 * e + (lane >> 4);
+            if (mo >= p.M) continue;
+            const int ow = static_cast<int>(mo % p.OW);
+            const int64_t t = mo / p.OW;
+            const int oh = static_cast<int>(t % p.OH);
+            const int64_t img = t / p.OH;
+            double* ob = p.out + img * p.osN + oh * p.osH + ow * p.osW;
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int n = bn + wn + j * 16 + (lane & 15);
+                if (n >= p.K) continue;
+                double v = acc[i][j][e];
+                if (p.bias != nullptr) v += p.bias[n * p.bias_stride];
+                ob[n * p.osC] = v;
+            }
+        }
+    }
+}
+
+void LaunchF64(IGemmArgs<double> p, hipStream_t stream) {
     int64_t total = p.M * p.K;
     if (total == 0) return;
-    int64_t blocks = (total + 255) / 256;
-    HIPCX_REQUIRE(blocks < (1LL << 31), HIPCX_NOT_IMPLEMENTED_ERROR, "problem too large for one launch");
-    hipLaunchKernelGGL(ConvNaiveF64Kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, p);
-    CheckLaunch("conv_f64");
+    if (total * p.Kg < (1 << 16) || p.Kg == 0) {  // a few thousand multiply-adds: not worth mostly empty tiles
+        int64_t blocks = (total + 255) / 256;
+        hipLaunchKernelGGL(ConvNaiveF64Kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, p);
+        CheckLaunch("conv_f64");
+        return;
+    }
+    const int64_t tiles_m = (p.M + kF64TileM - 1) / kF64TileM, tiles_n = (p.K + kF64TileN - 1) / kF64TileN;
+    HIPCX_REQUIRE(tiles_m * tiles_n < (1LL << 31) && tiles_m < (1LL << 31), HIPCX_NOT_IMPLEMENTED_ERROR, "problem too large for one launch");
+    p.tiles_m = static_cast<int>(tiles_m);
+    p.tiles_n = static_cast<int>(tiles_n);
+    ProfileScope prof(stream, 2.0 * static_cast<double>(p.M) * p.K * p.Kg,
+                      8.0 * (static_cast<double>(p.N) * p.C * p.H * p.W + static_cast<double>(p.K) * p.Kg + static_cast<double>(p.M) * p.K));
+    hipLaunchKernelGGL(ConvMfmaF64Kernel, dim3(static_cast<unsigned>(tiles_m * tiles_n)), dim3(256), 0, stream, p);
+    CheckLaunch("conv_mfma_f64");
 }
 
 int64_t ElemStride(const hipcx_array* a, int axis, const char* name) {
