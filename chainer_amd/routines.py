@@ -2009,9 +2009,36 @@ def _n_step_rnn_impl(impl, n_layers, hx, cx, ws, bs, xs, bidirectional, activati
     return stack(hy, 0), xs_next
 
 
-def n_step_lstm(n_layers, hx, cx, ws, bs, xs, fused=False):
+def _descriptor_pointers(arrays):
+    """A C array of hipcx_array pointers for `arrays` (the arrays must stay alive while it is used)."""
+    for a in arrays:
+        a.desc()  # builds and caches the descriptor
+    return (ctypes.POINTER(_lib.CArray) * len(arrays))(*[ctypes.pointer(a._desc) for a in arrays])
+
+
+def _n_step_lstm_kernel(n_layers, hx, cx, ws, bs, xs):
+    """The RnnKernel entry (hipcx_n_step_lstm): weights packed once, one launch per wavefront stage."""
+    if len(ws) != n_layers or len(bs) != n_layers or _py.any(len(w) != 8 for w in ws) or _py.any(len(b) != 8 for b in bs):
+        raise _lib.DimensionError('n_step_lstm needs eight matrices and eight biases per layer')
+    flat_w = [w for layer in ws for w in layer]
+    flat_b = [b for layer in bs for b in layer]
+    xs = list(xs)
+    hy = ndarray.empty(hx.shape, hx.dtype)
+    cy = ndarray.empty(cx.shape, cx.dtype)
+    ys = [ndarray.empty((x.shape[0], hx.shape[2]), hx.dtype) for x in xs]
+    pw, pb, px, py = (_descriptor_pointers(v) for v in (flat_w, flat_b, xs, ys))
+    nbytes = _lib.load().hipcx_n_step_lstm_workspace_size(n_layers, hx.desc(), px, len(xs))
+    wsb, wsp = _workspace(nbytes)
+    _lib.call('hipcx_n_step_lstm', n_layers, hx.desc(), cx.desc(), pw, pb, px, len(xs), hy.desc(), cy.desc(), py, wsp, nbytes, current_stream())
+    return hy, cy, ys
+
+
+def n_step_lstm(n_layers, hx, cx, ws, bs, xs, fused=False, kernel=False):
     """NStepLstm (CX/routines/n_step_rnn.cc:434-443) -> (hy, cy, ys).  ws[layer] / bs[layer] hold the eight matrices / vectors in
-    cuDNN order: input, forget, cell, output for x, then the same for h.  `fused` (opt-in) runs each cell through hipcx_lstm_cell."""
+    cuDNN order: input, forget, cell, output for x, then the same for h.  `fused` (opt-in) runs each cell through hipcx_lstm_cell;
+    `kernel` (opt-in, float32) runs the whole routine through hipcx_n_step_lstm, the RnnKernel the reference gives its cuda backend."""
+    if kernel and hx.dtype == numpy.dtype('float32'):
+        return _n_step_lstm_kernel(n_layers, hx, cx, ws, bs, xs)
     return _n_step_rnn_impl(_lstm_impl_fused if fused else _lstm_impl, n_layers, hx, cx, ws, bs, xs, False)
 
 

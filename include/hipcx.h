@@ -336,6 +336,19 @@ int hipcx_conv_bn_act(const hipcx_array* x, const hipcx_array* w, const hipcx_ar
  *   4j+k of x[B,4H]; a = tanh(g0), i, f, o = 1/(1+exp(-g)) (CX/routines/activation.cc:74-78); c_out = a*i + f*c;
  *   h_out = o*tanh(c_out).  Same operations in the same order as the ~25 separate kernels: bit-identical for float32/float64
  *   (float16 rounds once instead of after every kernel).  Errors as the routine raises them (DimensionError, DtypeError). */
+/* hipcx_n_step_lstm: RnnKernel (CX/kernels/rnn.h:34-49) in LSTM mode, one direction, float32 -- what NStepLstm
+ *   (CX/routines/n_step_rnn.cc:434-443) computes.  The reference hands this kernel only to its "cuda" backend (n_step_rnn.cc:210)
+ *   and composes the routine elsewhere, so a hip plugin reaches it after that test is widened; until then it is opt-in.
+ *   hx, cx, hy, cy: [n_layers, B, H]; ws / bs: n_layers * 8 matrices [H, in] / vectors [H] in cuDNN order (input, forget, cell,
+ *   output for x, then for h; in = xs' columns for layer 0, H above); xs[t]: [B_t, in] with B_t <= B; ys[t]: [B_t, H].  State rows
+ *   beyond a step's batch keep their values.  The eight matrices of a layer are packed once per call, every launch advances all
+ *   layers by one step (a wavefront: n_steps + n_layers - 1 launches), the gates never reach memory.  Equal to the composition
+ *   within float32 tolerance (the sums run in another order).  Other dtypes: HIPCX_NOT_IMPLEMENTED_ERROR (compose the routine).
+ *   `workspace`: 256-byte aligned, hipcx_n_step_lstm_workspace_size bytes (packed weights, padded state, layer outputs). */
+size_t hipcx_n_step_lstm_workspace_size(int n_layers, const hipcx_array* hx, const hipcx_array* const* xs, int n_steps);
+int hipcx_n_step_lstm(int n_layers, const hipcx_array* hx, const hipcx_array* cx, const hipcx_array* const* ws, const hipcx_array* const* bs,
+                      const hipcx_array* const* xs, int n_steps, const hipcx_array* hy, const hipcx_array* cy, const hipcx_array* const* ys,
+                      void* workspace, size_t workspace_bytes, void* stream);
 size_t hipcx_log_softmax_workspace_size(const hipcx_array* x);
 int hipcx_log_softmax(const hipcx_array* x, const hipcx_array* out, void* workspace, size_t workspace_bytes, void* stream);
 int hipcx_lstm_cell(const hipcx_array* c, const hipcx_array* x, const hipcx_array* h_out, const hipcx_array* c_out, void* stream);

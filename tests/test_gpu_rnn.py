@@ -97,3 +97,64 @@ def test_n_step_lstm_float16_and_errors():
         assert_close(y.get(), r, what='ys float16')
     with pytest.raises(chx.DimensionError):  # a batch larger than the state
         chx.n_step_lstm(2, HX[:, :3], CX[:, :3], W, B, X)
+
+
+@pytest.mark.parametrize('n_layers', [1, 2, 3, 5])
+def test_n_step_lstm_kernel_entry_matches_oracle(n_layers):
+    """hipcx_n_step_lstm (weights packed once, one launch per wavefront stage) against the oracle's routine composition: odd sizes
+    (reduction tails, partial unit and row tiles), ragged and non-monotonic step batches, more layers than one launch takes, and
+    the workload's own size."""
+    import chainer_amd as chx
+    rng = np.random.default_rng(13 + n_layers)
+    # (input size, units, sequence lengths): the batch is the number of sequences, step t holds the sequences longer than t
+    problems = [(4, 3, (5, 3, 3, 1)), (40, 64, (6,) * 8), (17, 33, (4, 2)), (50, 70, (3,) * 100 + (2,) * 20 + (1,) * 10),
+                (23, 9, (7,) * 66 + (2,) * 5)]
+    if n_layers == 2:
+        problems.append((650, 650, (2,) * 128))
+    for in_size, units, lengths in problems:
+        ws, bs, seqs, xs, hx, cx = _rnn_problem(rng, 'lstm', n_layers, False, in_size, units, lengths)
+        if units == 9:  # step batches that grow again (the routine only asks for batch <= state rows)
+            xs = [xs[0][:5], xs[1], xs[2][:1], xs[3]]
+        if units == 650:  # the workload's weight range (+-0.05): with +-0.6 the 1300-term sums reach ~12 and their rounding alone 2e-5
+            ws = [[m / np.float32(12) for m in layer] for layer in ws]
+        W, B, X, HX, CX = _upload(chx, ws, bs, xs, hx, cx)
+        ref = O.n_step_lstm(n_layers, hx, cx, ws, bs, xs)
+        got = chx.n_step_lstm(n_layers, HX, CX, W, B, X, kernel=True)
+        what = 'layers=%d in=%d units=%d lengths=%r' % (n_layers, in_size, units, lengths)
+        assert_close(got[0].get(), ref[0], what='hy ' + what)
+        assert_close(got[1].get(), ref[1], what='cy ' + what)
+        assert len(got[2]) == len(ref[2])
+        for t, (y, r) in enumerate(zip(got[2], ref[2])):
+            assert y.shape == r.shape
+            assert_close(y.get(), r, what='ys[%d] %s' % (t, what))
+        np.testing.assert_array_equal(HX.get(), hx)  # the inputs are left alone
+        np.testing.assert_array_equal(CX.get(), cx)
+
+
+def test_n_step_lstm_kernel_entry_views_and_errors():
+    import ctypes
+    import chainer_amd as chx
+    from chainer_amd import _lib, routines
+    rng = np.random.default_rng(14)
+    ws, bs, seqs, xs, hx, cx = _rnn_problem(rng, 'lstm', 2, False, 12, 20, (6, 6, 4))
+    W, B, X, HX, CX = _upload(chx, ws, bs, xs, hx, cx)
+    ref = O.n_step_lstm(2, hx, cx, ws, bs, xs)
+    # transposed weight storage and inputs that are column slices of a wider array (rows not 16-byte aligned)
+    Wt = [[chx.array(np.ascontiguousarray(m.T)).transpose((1, 0)) for m in layer] for layer in ws]
+    wide = [chx.array(np.concatenate([np.zeros((x.shape[0], 1), np.float32), x], 1)) for x in xs]
+    Xv = [w[:, 1:] for w in wide]
+    got = chx.n_step_lstm(2, HX, CX, Wt, B, Xv, kernel=True)
+    assert_close(got[0].get(), ref[0], what='hy, operands that are views')
+    for y, r in zip(got[2], ref[2]):
+        assert_close(y.get(), r, what='ys, operands that are views')
+    with pytest.raises(chx.DimensionError):  # a batch larger than the state
+        chx.n_step_lstm(2, HX[:, :2], CX[:, :2], W, B, X, kernel=True)
+    with pytest.raises(chx.DimensionError):  # a weight matrix of the wrong shape
+        bad = [list(layer) for layer in W]
+        bad[1][2] = bad[0][0]
+        chx.n_step_lstm(2, HX, CX, bad, B, X, kernel=True)
+    # other dtypes are not taken by the entry: the routine composes them
+    px = routines._descriptor_pointers(X)
+    h16 = chx.array(hx.astype(np.float16))
+    assert _lib.load().hipcx_n_step_lstm_workspace_size(2, h16.desc(), px, len(X)) == 0
+    assert _lib.load().hipcx_n_step_lstm_workspace_size(2, HX.desc(), px, len(X)) > 0
