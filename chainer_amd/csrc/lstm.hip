@@ -40,7 +40,7 @@ struct LstmJob {
     float* h_next;
     float* c;  // [B][H], updated in place
     int64_t c_stride;
-    const float* w;  // packed [4H][Xp + Hp]
+    const float* w;  // packed [4H][Xp + Hp rounded up to whole chunks], zero beyond the two segments
     const float* bias;  // [4H]
     float* y;  // [Bt][..]: this step's output rows
     int64_t y_stride;
@@ -86,6 +86,7 @@ __global__ __launch_bounds__(256) void LstmStepKernel(LstmStepArgs args) {
 
     const int Kp = job.Xp + Hp;
     const int nchunks = (Kp + kChunk - 1) / kChunk;
+    const int Kw = nchunks * kChunk;  // length of a packed weight row: zero beyond Kp, so that no block needs a bounds check
     const int a_row = r0 + wave * 16 + lm;
     const bool a_ok = a_row < Bt;
     const float* xrow = job.x + static_cast<int64_t>(a_ok ? a_row : 0) * job.Xp;
@@ -98,10 +99,9 @@ __global__ __launch_bounds__(256) void LstmStepKernel(LstmStepArgs args) {
         for (int i = 0; i < 4; ++i) {
             const int piece = tid + 256 * i;
             const int col = piece >> 5, k = kc + 4 * (piece & 31);
-            const int n = u0 * 4 + col;
-            float4_t v = {0.f, 0.f, 0.f, 0.f};
-            if (n < 4 * H && k < Kp) v = *reinterpret_cast<const float4_t*>(job.w + static_cast<int64_t>(n) * Kp + k);
-            wreg[i] = v;
+            int n = u0 * 4 + col;
+            if (n > 4 * H - 1) n = 4 * H - 1;  // columns past the last unit repeat the last row: their results are never stored
+            wreg[i] = *reinterpret_cast<const float4_t*>(job.w + static_cast<int64_t>(n) * Kw + k);
         }
     };
     auto store_w = [&](int buf) {
@@ -125,36 +125,38 @@ __global__ __launch_bounds__(256) void LstmStepKernel(LstmStepArgs args) {
     };
 
     float4_t acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
-    float4_t a_cur[kBlocks], a_next[kBlocks];
-    load_w(0);
-    load_a(0, a_cur);
-    store_w(0);
-    __syncthreads();
-    for (int ch = 0; ch < nchunks; ++ch) {
-        const int cur = ch & 1, kc = ch * kChunk;
-        if (ch + 1 < nchunks) {  // the next chunk's operands travel while this chunk's products run
-            load_w(kc + kChunk);
-            load_a(kc + kChunk, a_next);
-        }
+    // Two operand register sets used in turn (the chunk loop is unrolled by two, so no set is ever copied into the other: a copy
+    // would wait for the loads it copies and put the memory latency back in front of the products).
+    float4_t a_even[kBlocks], a_odd[kBlocks];
+    // No branch inside: the chunk after the last is the last one read again (into buffers nobody uses any more).
+    auto chunk = [&](int ch, const float4_t* a_now, float4_t* a_later) {
+        const int cur = ch & 1;
+        const int kc_next = (ch + 1 < nchunks ? ch + 1 : ch) * kChunk;
+        load_w(kc_next);  // the next chunk's operands travel while this chunk's products run
+        load_a(kc_next, a_later);
 #pragma unroll
         for (int kb = 0; kb < kBlocks; ++kb) {
-            if (kc + kb * 16 < Kp) {  // (uniform)
-                const float4_t b0 = *reinterpret_cast<const float4_t*>(&Bs[cur][lm][kb * 16 + 4 * lq]);
-                const float4_t b1 = *reinterpret_cast<const float4_t*>(&Bs[cur][16 + lm][kb * 16 + 4 * lq]);
+            const float4_t b0 = *reinterpret_cast<const float4_t*>(&Bs[cur][lm][kb * 16 + 4 * lq]);
+            const float4_t b1 = *reinterpret_cast<const float4_t*>(&Bs[cur][16 + lm][kb * 16 + 4 * lq]);
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a_cur[kb][j], b0[j], acc[0], 0, 0, 0);
-                    acc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a_cur[kb][j], b1[j], acc[1], 0, 0, 0);
-                }
+            for (int j = 0; j < 4; ++j) {
+                acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a_now[kb][j], b0[j], acc[0], 0, 0, 0);
+                acc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a_now[kb][j], b1[j], acc[1], 0, 0, 0);
             }
         }
-        if (ch + 1 < nchunks) {
-            store_w(cur ^ 1);  // the other buffer: its readers passed the barrier of the previous chunk
-#pragma unroll
-            for (int kb = 0; kb < kBlocks; ++kb) a_cur[kb] = a_next[kb];
-        }
+        store_w(cur ^ 1);  // the other buffer: its readers passed the barrier of the previous chunk
         __syncthreads();
+    };
+    load_w(0);
+    load_a(0, a_even);
+    store_w(0);
+    __syncthreads();
+    int ch = 0;
+    for (; ch + 1 < nchunks; ch += 2) {
+        chunk(ch, a_even, a_odd);
+        chunk(ch + 1, a_odd, a_even);
     }
+    if (ch < nchunks) chunk(ch, a_even, a_odd);
 
     // ---- the cell: accumulator register i of a lane is (row 4 * lq + i, column lm); the four lanes of a group of four hold the four
     // gates of one unit, so lane r of the group collects the gates of row 4 * lq + r ----
@@ -196,13 +198,13 @@ struct LstmPackArgs {
     int64_t w_row[8], w_col[8];  // element strides
     const float* b[8];
     int64_t b_stride[8];
-    float* w_out;  // [4H][Xp + Hp]
+    float* w_out;  // [4H][Xp + Hp rounded up to whole chunks]
     float* b_out;  // [4H]
     int H, I, Xp, Hp;
 };
 
 __global__ __launch_bounds__(256) void LstmPackKernel(LstmPackArgs p) {
-    const int Kp = p.Xp + p.Hp;
+    const int Kp = (p.Xp + p.Hp + kChunk - 1) / kChunk * kChunk;  // rows are padded to whole chunks with zeros
     const int64_t total = static_cast<int64_t>(4) * p.H * Kp;
     for (int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; idx < total; idx += static_cast<int64_t>(gridDim.x) * 256) {
         const int n = static_cast<int>(idx / Kp), k = static_cast<int>(idx - static_cast<int64_t>(n) * Kp);
@@ -244,6 +246,7 @@ __global__ __launch_bounds__(256) void LstmPadKernel(LstmPadArgs p) {
 
 size_t Round256(size_t v) { return (v + 255) / 256 * 256; }
 int RoundUp16(int64_t v) { return static_cast<int>((v + 15) / 16 * 16); }
+int64_t PackedRow(int64_t k) { return (k + kChunk - 1) / kChunk * kChunk; }
 
 void CheckStatus(int status) {
     if (status != HIPCX_OK) throw Error(status, hipcx_last_error());
@@ -289,7 +292,7 @@ LstmPlan PlanLstm(int n_layers, const hipcx_array* hx, const hipcx_array* const*
     for (int l = 0; l < n_layers; ++l) {
         const int64_t Xp = RoundUp16(l == 0 ? pl.I : pl.H);
         pl.w_off.push_back(off);
-        off += Round256(static_cast<size_t>(4 * pl.H * (Xp + pl.Hp)) * 4);
+        off += Round256(static_cast<size_t>(4 * pl.H * PackedRow(Xp + pl.Hp)) * 4);
         pl.b_off.push_back(off);
         off += Round256(static_cast<size_t>(4 * pl.H) * 4);
         pl.h_off.push_back(off);
@@ -419,7 +422,7 @@ int hipcx_n_step_lstm(int n_layers, const hipcx_array* hx, const hipcx_array* cx
             pa.I = static_cast<int>(in);
             pa.Xp = RoundUp16(in);
             pa.Hp = static_cast<int>(Hp);
-            const int64_t total = 4 * H * (pa.Xp + Hp);
+            const int64_t total = 4 * H * PackedRow(pa.Xp + Hp);
             int64_t blocks = (total + 255) / 256;
             const int64_t cap = static_cast<int64_t>(NumCUs()) * 16;
             hipLaunchKernelGGL(LstmPackKernel, dim3(static_cast<unsigned>(blocks > cap ? cap : blocks)), dim3(256), 0, st, pa);
