@@ -257,6 +257,12 @@ def section_lstm(chx, oracle, with_cpu):
          note='the composition restacks the eight gate matrices at every time step')
     emit(section='lstm', op='n_step_lstm 2 layers x 35 steps, opt-in: weights stacked once, one input Dot per layer, fused cell', batch=128,
          units=u, graph_replay_ms=round(hoisted * 1e3, 2), TFLOPs_graph=round(nflops / hoisted / 1e12, 2))
+    entry = graph_time(lambda: chx.n_step_lstm(2, hx, cx, ws, bs, xs, kernel=True), 5)
+    emit(section='lstm', op='n_step_lstm 2 layers x 35 steps, hipcx_n_step_lstm (the RnnKernel entry)', batch=128, units=u,
+         graph_replay_ms=round(entry * 1e3, 2), TFLOPs_graph=round(nflops / entry / 1e12, 2), fp32_mfma_frac=round(nflops / entry / 157.3e12, 4),
+         kernel_launches=36 + 12,
+         note='weights packed once per call, one launch per wavefront stage (36), gates stay in the MFMA accumulators; the reference '
+              'hands RnnKernel to its cuda backend only (routines/n_step_rnn.cc:210), so this entry is opt-in for a hip plugin')
     W = pd['embed']
     t = op_time(lambda: chx.take(W, I, 0, 'wrap'))
     bw_row('lstm', 'take [10000,650] rows by [128,35] ids', (128, 35, 650), t, 2 * 128 * 35 * 650 * 4 + ids.nbytes)

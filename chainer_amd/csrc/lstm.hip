@@ -93,8 +93,7 @@ __global__ __launch_bounds__(256) void LstmStepKernel(LstmStepArgs args) {
     const float* hrow = job.h_prev + static_cast<int64_t>(a_ok ? a_row : 0) * Hp;
 
     // weights: 32 columns x 128 k = 1024 16-byte pieces per chunk, four per thread
-    float4_t wreg[4];
-    auto load_w = [&](int kc) {
+    auto load_w = [&](int kc, float4_t* wreg) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int piece = tid + 256 * i;
@@ -104,7 +103,7 @@ __global__ __launch_bounds__(256) void LstmStepKernel(LstmStepArgs args) {
             wreg[i] = *reinterpret_cast<const float4_t*>(job.w + static_cast<int64_t>(n) * Kw + k);
         }
     };
-    auto store_w = [&](int buf) {
+    auto store_w = [&](int buf, const float4_t* wreg) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int piece = tid + 256 * i;
@@ -128,12 +127,15 @@ __global__ __launch_bounds__(256) void LstmStepKernel(LstmStepArgs args) {
     // Two operand register sets used in turn (the chunk loop is unrolled by two, so no set is ever copied into the other: a copy
     // would wait for the loads it copies and put the memory latency back in front of the products).
     float4_t a_even[kBlocks], a_odd[kBlocks];
-    // No branch inside: the chunk after the last is the last one read again (into buffers nobody uses any more).
-    auto chunk = [&](int ch, const float4_t* a_now, float4_t* a_later) {
+    // No branch inside: chunks after the last are the last one read again (into buffers nobody uses any more).  Activations
+    // (shared by every workgroup, so near) are fetched one chunk ahead; a workgroup's weight slice is its own and comes from
+    // farther away: two chunks ahead, held in registers for one chunk before it goes to LDS.
+    float4_t w_even[4], w_odd[4];
+    auto chunk = [&](int ch, const float4_t* a_now, float4_t* a_later, const float4_t* w_next, float4_t* w_after) {
         const int cur = ch & 1;
-        const int kc_next = (ch + 1 < nchunks ? ch + 1 : ch) * kChunk;
-        load_w(kc_next);  // the next chunk's operands travel while this chunk's products run
-        load_a(kc_next, a_later);
+        const int last = nchunks - 1;
+        load_w((ch + 2 < last ? ch + 2 : last) * kChunk, w_after);
+        load_a((ch + 1 < last ? ch + 1 : last) * kChunk, a_later);
 #pragma unroll
         for (int kb = 0; kb < kBlocks; ++kb) {
             const float4_t b0 = *reinterpret_cast<const float4_t*>(&Bs[cur][lm][kb * 16 + 4 * lq]);
@@ -144,19 +146,20 @@ __global__ __launch_bounds__(256) void LstmStepKernel(LstmStepArgs args) {
                 acc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a_now[kb][j], b1[j], acc[1], 0, 0, 0);
             }
         }
-        store_w(cur ^ 1);  // the other buffer: its readers passed the barrier of the previous chunk
+        store_w(cur ^ 1, w_next);  // chunk ch + 1, loaded during chunk ch - 1; the buffer's readers passed the previous barrier
         __syncthreads();
     };
-    load_w(0);
+    load_w(0, w_even);
     load_a(0, a_even);
-    store_w(0);
+    load_w((nchunks > 1 ? 1 : 0) * kChunk, w_odd);
+    store_w(0, w_even);
     __syncthreads();
     int ch = 0;
     for (; ch + 1 < nchunks; ch += 2) {
-        chunk(ch, a_even, a_odd);
-        chunk(ch + 1, a_odd, a_even);
+        chunk(ch, a_even, a_odd, w_odd, w_even);      // stores chunk ch + 1 (w_odd), fetches chunk ch + 2 into w_even
+        chunk(ch + 1, a_odd, a_even, w_even, w_odd);  // stores chunk ch + 2 (w_even), fetches chunk ch + 3 into w_odd
     }
-    if (ch < nchunks) chunk(ch, a_even, a_odd);
+    if (ch < nchunks) chunk(ch, a_even, a_odd, w_odd, w_even);
 
     // ---- the cell: accumulator register i of a lane is (row 4 * lq + i, column lm); the four lanes of a group of four hold the four
     // gates of one unit, so lane r of the group collects the gates of row 4 * lq + r ----
