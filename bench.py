@@ -46,7 +46,7 @@ def main():
     ap.add_argument('--warmup', type=int, default=5)
     ap.add_argument('--batch', type=int, default=128)
     ap.add_argument('--eager', action='store_true', help='time eager launches instead of a HIP graph replay')
-    ap.add_argument('--ops', nargs='?', const='sweep,mlp,cifar,resnet_layers,lstm,backward,train,linalg', default=None,
+    ap.add_argument('--ops', nargs='?', const='copy,sweep,mlp,cifar,resnet_layers,lstm,backward,train,linalg', default=None,
                     help='instead of the headline step, print per-operation roofline lines (chainer_amd.bench_ops) with a CPU baseline column')
     ap.add_argument('--cpu-batch', type=int, default=8, help='images for the CPU baseline (0 = skip)')
     args = ap.parse_args()
@@ -155,10 +155,11 @@ def main():
         'max_bound_frac': round(bound_ms / ms.value, 4) if ms.value > 0 else None,
     }
 
-    # ---- a plain device copy (1 GiB read + 1 GiB written), ten per graph replay: what this box's HBM delivers ----
+    # ---- a plain device copy (1 GiB read + 1 GiB written), ten back-to-back launches between two events (a launch lasts ~0.4 ms,
+    # far longer than the host needs to issue it): what this box's HBM delivers ----
     big = chx.array(np.zeros(512 * 1024 * 1024, np.float16))
-    from chainer_amd.bench_ops import kernel_time
-    copy_s = kernel_time(lambda: chx.copy(big))
+    from chainer_amd.bench_ops import device_time
+    copy_s = device_time(lambda: chx.copy(big), iters=10, warmup=2, rounds=2)
     stream_copy = {'bytes': 2 * big.nbytes, 'us': round(copy_s * 1e6, 1), 'gbs': round(2 * big.nbytes / copy_s / 1e9, 1),
                    'frac_of_hbm_peak': round(2 * big.nbytes / copy_s / 1e9 / HBM_PEAK_GBS, 4)}
     del big

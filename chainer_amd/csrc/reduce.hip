@@ -14,8 +14,9 @@
 //   * AMax propagates NaN (statistics.cc:38-42).
 //
 // RowReduceKernel: the reduced axes form one contiguous run (a "row").  Lane <-> group of four
-// (one 16-byte load), 8 lanes <-> chunk, then wave shuffles, an LDS tree and, for rows split
-// over several blocks, a second pass over per-block partials in the workspace.
+// (one 16-byte load), 8 lanes <-> chunk, 16 lanes <-> two chunks merged (one LDS node), then a tree
+// over the block's nodes and, for rows split over several blocks, a second pass over per-block
+// partials in the workspace.
 // GenericReduceKernel: any strides; one thread per output element runs the reference loop
 // literally.  Consecutive threads take consecutive outputs, so reducing over outer axes of a
 // dense array (a "column" reduction) is coalesced.
@@ -33,7 +34,8 @@ namespace {
 constexpr int kMaxDims = HIPCX_MAX_NDIM;
 constexpr int kRowThreads = 256;
 constexpr int kElemsPerIter = kRowThreads * 4;  // 1024 elements = 32 chunks = 4 nodes (one per wave)
-constexpr int kMaxNodes = 256;                  // LDS nodes per block -> span <= 65536 elements
+constexpr int kMaxIters = 64;                   // iterations per block -> span <= 65536 elements
+constexpr int kMaxNodes = kMaxIters * 16;       // LDS nodes per block: one per row of 16 lanes (two chunks) and iteration
 constexpr int kMaxPartials = 1024;              // blocks per row handled by the finalize pass
 
 // ---------------------------------------------------------------------------------------------
@@ -335,7 +337,7 @@ __global__ __launch_bounds__(kRowThreads) void RowReduceKernel(ReduceGeom g, int
     using In = typename R::In;
     using Acc = typename R::Acc;
     __shared__ Acc nodes[kMaxNodes];
-    __shared__ Acc wave_nodes[kRowThreads / 64];
+    __shared__ Acc wave_nodes[kMaxNodes / 64];
 
     int64_t row = blockIdx.x;
     int blk = 0;
@@ -427,14 +429,13 @@ __global__ __launch_bounds__(kRowThreads) void RowReduceKernel(ReduceGeom g, int
             step(std::integral_constant<int, 2>());
             step(std::integral_constant<int, 4>());
         }
-        // 8 chunk results per wave -> one node: balanced tree, the later operand is the accumulator
+        // the two chunks of a row of 16 lanes -> one node (the later operand is the accumulator); the tree above that level
+        // runs once per block, over the nodes
 #pragma unroll
         for (int u = 0; u < N; ++u) MergeLaneAbove<Op, 8>(acc[u]);
+        if ((lane & 15) == 0) {
 #pragma unroll
-        for (int u = 0; u < N; ++u) acc[u] = MergeRows<Op>(acc[u]);
-        if (lane == 0) {
-#pragma unroll
-            for (int u = 0; u < N; ++u) nodes[(it0 + u) * 4 + wave] = acc[u];
+            for (int u = 0; u < N; ++u) nodes[((it0 + u) * 4 + wave) * 4 + (lane >> 4)] = acc[u];
         }
     };
     auto plain = [&](int it0, const Group4<In>* q, auto count) {
@@ -499,14 +500,10 @@ __global__ __launch_bounds__(kRowThreads) void RowReduceKernel(ReduceGeom g, int
             for (int64_t i = G * 4; i < L; ++i) R::Reduce(R::Map(*at(i), i - e_begin), acc);
         }
         if (chunk > k_last) acc = R::Empty();
-        // ---- 8 chunk results per wave -> one node: balanced tree, the later operand is the accumulator ----
-#pragma unroll
-        for (int s = 8; s < 64; s <<= 1) {
-            Acc later = R::Shfl(acc, lane + s);
-            R::Reduce(acc, later);
-            acc = later;
-        }
-        if (lane == 0) nodes[it * 4 + wave] = acc;
+        // ---- the two chunks of a row of 16 lanes -> one node, the later operand is the accumulator ----
+        Acc later = R::Shfl(acc, lane + 8);
+        R::Reduce(acc, later);
+        if ((lane & 15) == 0) nodes[(it * 4 + wave) * 4 + (lane >> 4)] = later;
     };
 
     // The loads of kLoadBatch plain iterations are issued together, ahead of the arithmetic of the first of them.
@@ -527,32 +524,28 @@ __global__ __launch_bounds__(kRowThreads) void RowReduceKernel(ReduceGeom g, int
     for (; it < iters; ++it) guarded(it);
     __syncthreads();
 
-    // ---- tree over the block's nodes (a power of two, at least 4): each wave folds up to 64 consecutive ones ----
-    const int n_nodes = iters * 4;
+    // ---- tree over the block's nodes (a power of two, 16 to 1024): a wave folds 64 consecutive ones at a time, wave 0 then
+    // folds those results (at most 16) ----
+    using Op = ReduceOp<R, false>;
+    const int n_nodes = iters * 16;
     Acc acc = R::Empty();
-    if (wave * 64 < n_nodes) {
-        if (wave * 64 + lane < n_nodes) acc = nodes[wave * 64 + lane];  // lanes past the end hold padding
-        using Op = ReduceOp<R, false>;
+    for (int base = wave * 64; base < n_nodes; base += kRowThreads) {
+        acc = base + lane < n_nodes ? nodes[base + lane] : R::Empty();  // lanes past the end hold padding
         MergeLaneAbove<Op, 1>(acc);
         MergeLaneAbove<Op, 2>(acc);
         MergeLaneAbove<Op, 4>(acc);
         MergeLaneAbove<Op, 8>(acc);
         acc = MergeRows<Op>(acc);
+        if (lane == 0) wave_nodes[base >> 6] = acc;
     }
-    if (n_nodes > 64) {  // 128 or 256 nodes: two or four waves hold a result each
-        if (lane == 0) wave_nodes[wave] = acc;
+    if (n_nodes > 64) {
         __syncthreads();
-        if (tid == 0) {
-            Acc b = wave_nodes[1];
-            R::Reduce(acc, b);
-            if (n_nodes > 128) {
-                Acc c = wave_nodes[2];
-                Acc d = wave_nodes[3];
-                R::Reduce(c, d);
-                R::Reduce(b, d);
-                b = d;
-            }
-            acc = b;
+        if (wave == 0) {
+            acc = lane < (n_nodes >> 6) ? wave_nodes[lane] : R::Empty();
+            MergeLaneAbove<Op, 1>(acc);
+            MergeLaneAbove<Op, 2>(acc);
+            MergeLaneAbove<Op, 4>(acc);
+            MergeLaneAbove<Op, 8>(acc);
         }
     }
     if (tid == 0) {
@@ -847,7 +840,7 @@ ReducePlan MakePlan(const hipcx_array* a, const int8_t* axis, int naxis, const h
         pl.row_path = true;
         int64_t L = g.red_len;
         int64_t span = kElemsPerIter;
-        while (span < L && span < static_cast<int64_t>(kMaxNodes) * 256) span <<= 1;
+        while (span < L && span < static_cast<int64_t>(kMaxIters) * kElemsPerIter) span <<= 1;
         // few long rows: split rows over more blocks so that the whole chip is busy
         int64_t target_blocks = static_cast<int64_t>(NumCUs()) * 8;
         while (span > 4 * kElemsPerIter && g.n_out * ((L + span - 1) / span) < target_blocks && (L + span / 2 - 1) / (span / 2) <= kMaxPartials) {

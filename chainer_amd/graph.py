@@ -1,11 +1,15 @@
 """HIP graph capture of a sequence of kernel calls (launch-bound inner loops are replayed with one host call).
 
-The capture runs inside a memory arena of its own: an eager pass first fills the arena's free lists, the captured pass then
+The capture runs inside a memory arena of its own: eager passes first fill the arena's free lists, the captured pass then
 finds every block it asks for there (the capture never reaches the driver's allocator, which is not allowed while a stream
-is capturing), and afterwards nobody else is handed the addresses the graph has baked in.  PyTorch provides the capture
-itself (``torch.cuda.CUDAGraph``) and the stream.
+is capturing), and afterwards nobody else is handed the addresses the graph has baked in.  A function that keeps results of
+one call alive into the next (a training step that replaces its parameters) needs more than one eager pass before a pass
+allocates nothing new; the passes are repeated until that is the case.  PyTorch provides the capture itself
+(``torch.cuda.CUDAGraph``) and the stream.
 """
-from chainer_amd._array import memory_arena, torch
+from chainer_amd._array import memory_arena, pool_stats, torch
+
+MAX_WARM_PASSES = 4
 
 
 class CapturedGraph(object):
@@ -25,17 +29,22 @@ class CapturedGraph(object):
 
 
 def capture(fn):
-    """Runs ``fn()`` once eagerly and once under capture; returns a CapturedGraph."""
+    """Runs ``fn()`` eagerly until a pass gets all its memory from the arena's free lists, then once under capture; returns a
+    CapturedGraph."""
     t = torch()
     arena = memory_arena()
     # both passes run on one side stream: the pool keeps the blocks of different streams apart
     stream = t.cuda.Stream()
     stream.wait_stream(t.cuda.current_stream())
     with arena:
-        with t.cuda.stream(stream):
-            out = fn()
-        stream.synchronize()
-        del out
+        for _ in range(MAX_WARM_PASSES):
+            before = pool_stats()['device_allocations']
+            with t.cuda.stream(stream):
+                out = fn()
+            stream.synchronize()
+            del out
+            if pool_stats()['device_allocations'] == before:
+                break
         graph = t.cuda.CUDAGraph()
         with t.cuda.graph(graph, stream=stream):
             out = fn()

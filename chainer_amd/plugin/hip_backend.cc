@@ -51,6 +51,7 @@
 #include "chainerx/kernels/normalization.h"
 #include "chainerx/kernels/pooling.h"
 #include "chainerx/kernels/reduction.h"
+#include "chainerx/kernels/rnn.h"
 #include "chainerx/kernels/rounding.h"
 #include "chainerx/kernels/sorting.h"
 #include "chainerx/kernels/statistics.h"
@@ -1061,6 +1062,62 @@ public:
     }
 };
 HIPCX_REGISTER_KERNEL(AveragePoolGradKernel, HipAveragePoolGradKernel)
+
+// ---- RnnKernel (chainerx/kernels/rnn.h:34-49): the forward pass of a one-directional float32 LSTM in one library call.
+// The reference's NStepRnnImpl hands this kernel to the backend named "cuda" only (chainerx/routines/n_step_rnn.cc:210) and
+// composes the routine for every other backend, so the registration takes effect once that test also admits "hip".  Modes the
+// library does not take (GRU, plain RNN, both directions, other dtypes) raise NotImplementedError; no gradient state is kept.
+class HipRnnKernel : public RnnKernel {
+public:
+    std::tuple<std::vector<std::vector<Array>>, std::unique_ptr<RnnGradState>> Call(
+            int64_t n_layers, Array hx, absl::optional<Array> cx, const std::vector<std::vector<Array>>& ws, const std::vector<std::vector<Array>>& bs,
+            const std::vector<Array>& xs, int8_t bidirectional, int8_t mode, absl::optional<std::string> /*activation*/) override {
+        if (mode != 1 || bidirectional != 0 || !cx.has_value() || hx.dtype() != Dtype::kFloat32) {
+            throw NotImplementedError{"hip RnnKernel: one-directional float32 LSTM only."};
+        }
+        Device& device = hx.device();
+        SetDeviceScope scope{device.index()};
+        std::vector<Array> keep;  // contiguous float32 copies where the caller's arrays are something else
+        auto prepared = [&](const Array& a) {
+            device.CheckDevicesCompatible(hx, a);
+            keep.emplace_back(a.dtype() == Dtype::kFloat32 && a.IsContiguous() ? a : AsContiguous(a.AsType(Dtype::kFloat32)));
+            return ToC(keep.back());
+        };
+        hipcx_array chx_ = prepared(hx), ccx = prepared(*cx);
+        std::vector<hipcx_array> dw, db, dx, dy;
+        for (int64_t l = 0; l < n_layers; ++l) {
+            for (size_t i = 0; i < 8; ++i) {
+                dw.push_back(prepared(ws.at(l).at(i)));
+                db.push_back(prepared(bs.at(l).at(i)));
+            }
+        }
+        for (const Array& x : xs) dx.push_back(prepared(x));
+        Array hy = Empty(hx.shape(), Dtype::kFloat32, device);
+        Array cy = Empty(hx.shape(), Dtype::kFloat32, device);
+        std::vector<Array> ys;
+        for (const Array& x : xs) {
+            ys.emplace_back(Empty(Shape{x.shape()[0], hx.shape()[2]}, Dtype::kFloat32, device));
+            dy.push_back(ToC(ys.back()));
+        }
+        auto pointers = [](const std::vector<hipcx_array>& v) {
+            std::vector<const hipcx_array*> p;
+            for (const hipcx_array& d : v) p.push_back(&d);
+            return p;
+        };
+        std::vector<const hipcx_array*> pw = pointers(dw), pb = pointers(db), px = pointers(dx), py = pointers(dy);
+        hipcx_array chy = ToC(hy), ccy = ToC(cy);
+        const int n_steps = static_cast<int>(xs.size());
+        size_t ws_bytes = hipcx_n_step_lstm_workspace_size(static_cast<int>(n_layers), &chx_, px.data(), n_steps);
+        std::shared_ptr<void> wsp = device.Allocate(ws_bytes);
+        Check(hipcx_n_step_lstm(static_cast<int>(n_layers), &chx_, &ccx, pw.data(), pb.data(), px.data(), n_steps, &chy, &ccy, py.data(), wsp.get(),
+                                ws_bytes, nullptr));
+        std::vector<std::vector<Array>> ret;
+        ret.emplace_back(std::vector<Array>{std::move(hy), std::move(cy)});
+        ret.emplace_back(std::move(ys));
+        return std::make_tuple(std::move(ret), std::unique_ptr<RnnGradState>{});
+    }
+};
+HIPCX_REGISTER_KERNEL(RnnKernel, HipRnnKernel)
 
 // ---- linear algebra: Solve, Inverse, Cholesky, Syevd, Qr, Svd (the LAPACK-backed kernels of the native backend, native_device/linalg.cc) ----
 namespace {

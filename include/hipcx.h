@@ -285,8 +285,9 @@ int hipcx_dot(const hipcx_array* a, const hipcx_array* b, const hipcx_array* out
 /* Output extent of a convolution/pooling window (CX/routines/connection.cc:37-49). Returns -1 if not positive. */
 int64_t hipcx_conv_out_dim(int64_t in_dim, int64_t kernel_size, int64_t stride, int64_t pad, int cover_all);
 /* 2-D convolution forward, x[N,C,H,W] (any strides), w[K,C,kh,kw], optional b[K] (NULL = none),
- * out[N,K,OH,OW] with any strides: the plugin allocates it channels-last (an NCHW *view* of NHWC
- * memory, as the native backend's own result is: CX/native/native_device/conv.cc:78-84). */
+ * out[N,K,OH,OW] with any strides.  The plugin and the Python mirror allocate out C-contiguous (NCHW memory), like the CUDA
+ * backend (CX/cuda/cuda_conv.cc:311); the native backend's own result is an NCHW view of NHWC memory
+ * (CX/native/native_device/conv.cc:78-84), which this entry also accepts as `out`. */
 size_t hipcx_conv_workspace_size(const hipcx_array* x, const hipcx_array* w, const hipcx_array* out);
 int hipcx_conv(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, const int64_t* stride, const int64_t* pad,
                int cover_all, const hipcx_array* out, void* workspace, size_t workspace_bytes, void* stream);
