@@ -304,16 +304,21 @@ def resnet50_train_step(F, p, x, t, lr=0.01):
         else:
             container[key] = F.subtract(container[key], F.scale(g.reshape(container[key].shape), lr))
 
-    def swap(tree):  # filters are values of dicts: replace them where they live
-        for k, v in (tree.items() if isinstance(tree, dict) else enumerate(tree)):
-            if isinstance(v, (dict, list)):
-                swap(v)
-            elif id(v) in updates:
-                tree[k] = updates[id(v)]
-    swap(p)
+    _replace_leaves(p, updates)  # filters are values of dicts: replace them where they live
     p['fc_w'] = F.subtract(p['fc_w'], F.scale(g_fc_w, lr))
     p['fc_b'] = F.subtract(p['fc_b'], F.scale(g_fc_b, lr))
     return loss
+
+
+def _replace_leaves(tree, updates):
+    """tree[k] = updates[id(tree[k])] for every leaf that has an update.  A module-level function on purpose: a recursive closure
+    inside the step would form a reference cycle that keeps a whole generation of device arrays alive until the garbage
+    collector happens to run."""
+    for k, v in (tree.items() if isinstance(tree, dict) else enumerate(tree)):
+        if isinstance(v, (dict, list)):
+            _replace_leaves(v, updates)
+        elif id(v) in updates:
+            tree[k] = updates[id(v)]
 
 
 def resnet50_flops(batch=128, size=224):

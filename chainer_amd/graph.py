@@ -7,6 +7,8 @@ one call alive into the next (a training step that replaces its parameters) need
 allocates nothing new; the passes are repeated until that is the case.  PyTorch provides the capture itself
 (``torch.cuda.CUDAGraph``) and the stream.
 """
+import gc
+
 from chainer_amd._array import memory_arena, pool_stats, torch
 
 MAX_WARM_PASSES = 4
@@ -38,6 +40,7 @@ def capture(fn):
     stream.wait_stream(t.cuda.current_stream())
     with arena:
         for _ in range(MAX_WARM_PASSES):
+            gc.collect()  # arrays held only by garbage cycles would otherwise be freed at some later, arbitrary moment
             before = pool_stats()['device_allocations']
             with t.cuda.stream(stream):
                 out = fn()
@@ -45,6 +48,7 @@ def capture(fn):
             del out
             if pool_stats()['device_allocations'] == before:
                 break
+        gc.collect()
         graph = t.cuda.CUDAGraph()
         with t.cuda.graph(graph, stream=stream):
             out = fn()
