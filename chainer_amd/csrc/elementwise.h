@@ -101,7 +101,7 @@ struct EwArgs {
     int64_t cols;   // elements
     int64_t cvecs;  // cols / VEC
     int64_t nvec;   // rows * cvecs
-    int stream_in;  // inputs are too large to stay in the last-level cache: load them without allocating there
+    int stream_in;  // bit i + 1: input i is too large to stay in the last-level cache and is loaded without allocating there
 };
 
 // A 16-byte vector load that does not allocate in the caches (other sizes: a plain load).  A tensor larger than the memory-side
@@ -199,9 +199,10 @@ __global__ __launch_bounds__(kEwThreads) void EwKernel(EwArgs<Op::kNumIn + 1> ar
 #pragma unroll
             for (int i = 0; i < NIN; ++i) {
                 const char* p = args.ptr[i + 1] + off[u][i + 1];
+                const bool streamed = STREAM && ((args.stream_in >> (i + 1)) & 1);  // (uniform) a broadcast operand stays cached
                 if (i == 0) {
                     if (VEC > 1 && args.col_stride[NOPS > 1 ? 1 : 0] != 0) {
-                        in0[u] = STREAM ? LoadStreaming<Vec<In0, VEC>>(p) : *reinterpret_cast<const Vec<In0, VEC>*>(p);
+                        in0[u] = streamed ? LoadStreaming<Vec<In0, VEC>>(p) : *reinterpret_cast<const Vec<In0, VEC>*>(p);
                     } else {
                         In0 s = *reinterpret_cast<const In0*>(p);
 #pragma unroll
@@ -209,7 +210,7 @@ __global__ __launch_bounds__(kEwThreads) void EwKernel(EwArgs<Op::kNumIn + 1> ar
                     }
                 } else if (VEC > 1) {
                     if (args.col_stride[i + 1] != 0) {
-                        in[u][i] = STREAM ? LoadStreaming<Vec<In, VEC>>(p) : *reinterpret_cast<const Vec<In, VEC>*>(p);
+                        in[u][i] = streamed ? LoadStreaming<Vec<In, VEC>>(p) : *reinterpret_cast<const Vec<In, VEC>*>(p);
                     } else {
                         In s = *reinterpret_cast<const In*>(p);
 #pragma unroll
@@ -283,7 +284,16 @@ inline void LaunchEwVec(const EwPlan& p, const Op& op, hipStream_t stream) {
     a.cols = cols;
     a.cvecs = cols / VEC;
     a.nvec = rows * a.cvecs;
-    a.stream_in = a.nvec * VEC * static_cast<int64_t>(sizeof(typename Op::In)) > StreamingThresholdBytes() ? 1 : 0;
+    // an input streams when its own footprint (the axes it is not broadcast along) exceeds the threshold: a bias row added to a
+    // large matrix is read once per matrix row and has to stay in the cache
+    a.stream_in = 0;
+    for (int i = 1; i < NOPS; ++i) {
+        int64_t footprint = static_cast<int64_t>(sizeof(typename Op::In));
+        for (int d = 0; d < nd; ++d) {
+            if (p.strides[i][d] != 0) footprint *= p.shape[d];
+        }
+        if (footprint > StreamingThresholdBytes()) a.stream_in |= 1 << i;
+    }
     int64_t per_block = static_cast<int64_t>(kEwThreads) * kEwUnroll;
     int64_t blocks = (a.nvec + per_block - 1) / per_block;
     HIPCX_REQUIRE(blocks <= 0x7fffffffLL, HIPCX_NOT_IMPLEMENTED_ERROR, "array too large for one launch");
