@@ -336,10 +336,10 @@ def section_train(chx, oracle, with_cpu):
 
 
 def section_linalg(chx, oracle, with_cpu):
-    """Dense decompositions (float32; one workgroup per matrix: functional kernels, latency-bound).  The CPU column is LAPACK through
-    numpy, which is what the native backend calls."""
+    """Dense decompositions (float32).  Solve, inverse and Cholesky are blocked over many workgroups; QR, eigh and svd run in one
+    workgroup per matrix.  The CPU column is LAPACK through numpy, which is what the native backend calls."""
     rng = np.random.default_rng(8)
-    for n in (64, 256):
+    for n in (64, 256, 1024):
         a = (rng.standard_normal((n, n)) + np.sqrt(n) * np.eye(n)).astype(np.float32)
         sym = ((a + a.T) / 2).astype(np.float32)
         spd = (a @ a.T).astype(np.float32)
@@ -352,7 +352,7 @@ def section_linalg(chx, oracle, with_cpu):
                  ('eigh', lambda: chx.eigh(S), lambda: oracle.eigh(sym), None),
                  ('svd full', lambda: chx.svd(A), lambda: oracle.svd(a), None))
         for name, fn, cpu_fn, flops in cases:
-            t = device_time(fn, 3, 1)
+            t = device_time(fn, 3 if n <= 256 else 1, 1)
             row = dict(section='linalg', op=name, shape=[n, n], dtype='float32', us=round(t * 1e6, 1))
             if flops is not None:
                 row['GFLOPs'] = round(flops / t / 1e9, 2)

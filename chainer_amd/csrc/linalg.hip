@@ -1,13 +1,17 @@
 // Solve, Inverse and Cholesky (SolveKernel / InverseKernel / CholeskyKernel, CX/kernels/linalg.h:20-43) for float32 / float64
 // matrices.  The native backend hands these to LAPACK (gesv, getrf + getri, potrf: CX/native/native_device/linalg.cc:280-347,
-// 560-600); here each is one workgroup that factorises a dense row-major copy in place:
-//   * LU with partial pivoting (the first row of largest magnitude, as idamax picks it), the row operations applied to the right-hand
-//     sides as they happen, then back substitution -- Inverse is the same kernel on the identity;
-//   * right-looking Cholesky on the lower triangle, the strict upper triangle of the result zeroed.
+// 560-600); here they are blocked factorisations of a dense row-major copy, 32 columns at a time:
+//   * LU with partial pivoting (the first row of largest magnitude, as idamax picks it): one workgroup factors a panel with its rows
+//     in registers, then one workgroup per 64 columns of the rest of the matrix and of the right-hand sides applies the panel's row
+//     exchanges, solves for the panel's rows of U and subtracts L21 U12; back substitution runs per 64 right-hand sides, block row
+//     by block row -- Inverse is the same on the identity;
+//   * left-looking Cholesky on the lower triangle, one workgroup per 32 rows of a block column, the strict upper triangle of the
+//     result zeroed.
+// Triangular 32 x 32 blocks are inverted once (doubling levels of small products) and applied as products instead of substitutions.
 // Results agree with LAPACK's to rounding (the operation order differs), not to the bit.  A zero pivot / a non-positive diagonal
 // stores its 1-based position in the caller's flag, LAPACK's `info`, for the caller to raise on.
-// Functional kernels: one workgroup walks the whole matrix, which is adequate for the few-hundred-row systems these routines see
-// in the reference's callers (Gaussian-process and whitening layers), not for large factorizations.
+// Matrices above 8192 rows fall back to an LU kernel in which one workgroup walks the whole matrix.  QR, the symmetric
+// eigendecomposition and the SVD further down are one-workgroup kernels.
 #include "common.h"
 
 namespace hipcx {
@@ -20,7 +24,9 @@ __device__ __forceinline__ T AbsT(T v) {
     return v < T(0) ? -v : v;
 }
 
-// a: [n, n] row-major, destroyed.  b: [n, m] row-major, overwritten with the solution.
+// LU with partial pivoting and both substitutions in one workgroup that walks the whole matrix: the fallback for matrices too tall
+// for the panel kernel of the blocked factorisation.  a: [n, n] row-major, destroyed.  b: [n, m] row-major, overwritten with the
+// solution.
 template <typename T>
 __global__ __launch_bounds__(kLinalgThreads) void LuSolveKernel(T* a, T* b, int n, int m, int* info) {
     __shared__ T best_val[kLinalgThreads / 64];
@@ -107,40 +113,534 @@ __global__ __launch_bounds__(kLinalgThreads) void LuSolveKernel(T* a, T* b, int 
     }
 }
 
-// l: [n, n] row-major; on entry its lower triangle holds the matrix, on exit the factor with a zero strict upper triangle.
+constexpr int kNb = 32;  // width of a block column
+
+// the value of v in lane `lane` of the wavefront (lane is a constant once the caller's loop is unrolled)
+__device__ __forceinline__ float ReadLaneT(float v, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+__device__ __forceinline__ double ReadLaneT(double v, int lane) {
+    const uint64_t bits = __builtin_bit_cast(uint64_t, v);
+    const uint32_t lo = __builtin_amdgcn_readlane(static_cast<int>(bits), lane);
+    const uint32_t hi = __builtin_amdgcn_readlane(static_cast<int>(bits >> 32), lane);
+    return __builtin_bit_cast(double, (static_cast<uint64_t>(hi) << 32) | lo);
+}
+
 template <typename T>
-__global__ __launch_bounds__(kLinalgThreads) void CholeskyKernel(T* l, int n, int* info) {
+__device__ __forceinline__ T SqrtT(T v) {
+    if constexpr (std::is_same<T, float>::value) {
+        return sqrtf(v);
+    } else {
+        return sqrt(v);
+    }
+}
+
+// entry (i, j) of a kNb x kNb block in LDS, or of its transpose
+template <int TRANS, typename T>
+__device__ __forceinline__ T& BlockAt(T (&m)[kNb][kNb + 1], int i, int j) {
+    return TRANS ? m[j][i] : m[i][j];
+}
+
+// One level of the triangular inversion below: the diagonal blocks of size S are inverted already, and each pair of neighbours
+// (A over B, with C below A) gains the off-diagonal block -B^-1 C A^-1 of its 2S x 2S inverse.  16 * S entries, one per thread.
+template <int TRANS, int S, typename T>
+__device__ __forceinline__ void InvertTriangularLevels(T (&tri)[kNb][kNb + 1], T (&inv)[kNb][kNb + 1], T (&tmp)[kNb][kNb + 1], int tid) {
+    if constexpr (S < kNb) {
+        const int pair = tid / (S * S), i = tid / S % S, j = tid % S;
+        const int base = pair * 2 * S;
+        const bool active = tid < 16 * S;
+        if (active) {
+            T sum = T(0);
+#pragma unroll
+            for (int k = 0; k < S; ++k) sum += BlockAt<TRANS>(tri, base + S + i, base + k) * BlockAt<TRANS>(inv, base + k, base + j);
+            BlockAt<TRANS>(tmp, base + S + i, base + j) = sum;
+        }
+        __syncthreads();
+        if (active) {
+            T sum = T(0);
+#pragma unroll
+            for (int k = 0; k < S; ++k) sum -= BlockAt<TRANS>(inv, base + S + i, base + S + k) * BlockAt<TRANS>(tmp, base + S + k, base + j);
+            BlockAt<TRANS>(inv, base + S + i, base + j) = sum;
+        }
+        __syncthreads();
+        InvertTriangularLevels<TRANS, 2 * S>(tri, inv, tmp, tid);
+    }
+}
+
+// Inverse of the kNb x kNb triangular block `tri` (LDS; lower with UPPER = 0, upper with UPPER = 1; UNIT: the diagonal is taken as 1
+// and not read; the other triangle is not read) into `inv` (the other triangle zero-filled), by all 256 threads of the workgroup:
+// the reciprocals of the diagonal first, then five doubling levels of small products.  `tmp` is scratch.  Contains barriers; the
+// caller puts one before the call (tri complete) and finds inv complete on return.
+template <int UPPER, int UNIT, typename T>
+__device__ __forceinline__ void InvertTriangularBlock(T (&tri)[kNb][kNb + 1], T (&inv)[kNb][kNb + 1], T (&tmp)[kNb][kNb + 1], int tid) {
+    for (int e = tid; e < kNb * kNb; e += 256) {
+        const int r = e >> 5, c = e & (kNb - 1);
+        inv[r][c] = r != c ? T(0) : (UNIT ? T(1) : T(1) / tri[r][r]);
+    }
+    __syncthreads();
+    InvertTriangularLevels<UPPER, 1>(tri, inv, tmp, tid);
+}
+
+// What the row exchanges of one panel amount to: entry e says that row `row[e]` now holds what row `source[e]` held before the panel.
+struct LuExchanges {
+    int count;
+    int row[2 * kNb];
+    int source[2 * kNb];
+};
+
+// Device-side state of a blocked LU factorisation, kept behind the matrix copy in the workspace.
+struct LuState {
+    int info;  // LAPACK's info: 1-based position of the first zero pivot, 0 while there is none
+    LuExchanges exchanges;
+};
+
+template <typename T, int NB>
+struct LuPanelShared {
+    T candidate[2][16][NB];  // per column parity and wavefront: the row that wavefront proposes as the pivot row
+    T value[2][16];          // its magnitude in the column
+    int position[2][16];     // and its current position in the row order
+    int listed;
+};
+
+// v from the lane N places above in the same row of 16 lanes (DPP row_shl); lanes without such a neighbour keep their own value.
+template <int N, typename T>
+__device__ __forceinline__ T FromLaneAboveOrSelf(T v) {
+    constexpr int kWords = (sizeof(T) + 3) / 4;
+    int w[kWords] = {};
+    __builtin_memcpy(w, &v, sizeof(T));
+#pragma unroll
+    for (int i = 0; i < kWords; ++i) w[i] = __builtin_amdgcn_update_dpp(w[i], w[i], 0x100 + N /* row_shl:N */, 0xf, 0xf, false);
+    T r;
+    __builtin_memcpy(&r, w, sizeof(T));
+    return r;
+}
+
+// (v, p) <- the better of (v, p) and (ov, op): the larger magnitude, the earlier position among equals
+template <typename T>
+__device__ __forceinline__ void BetterPivot(T& v, int& p, T ov, int op) {
+    if (ov > v || (ov == v && op < p)) v = ov, p = op;
+}
+
+// Column steps K .. NB - 1 of the panel kernel below; a template recursion, so that K indexes registers.
+template <typename T, int ROWS, int NB, int K>
+__device__ __forceinline__ void LuPanelSteps(T (&row)[ROWS][NB], int (&pos)[ROWS], LuPanelShared<T, NB>& sh, int n, int j0, int w, LuState* state,
+                                             int* user_info) {
+    if constexpr (K < NB) {
+        if (K < w) {  // the same for every thread
+            const int tid = threadIdx.x;
+            const int nthreads = blockDim.x;
+            const int nwaves = nthreads >> 6;
+            const int wave = tid >> 6;
+            const int kk = j0 + K;
+            constexpr int par = K & 1;
+            // this thread's candidate: among its rows that are not pivot rows yet
+            T v = T(-1);
+            int p = 0x7fffffff;
+#pragma unroll
+            for (int r = 0; r < ROWS; ++r) {
+                const int gi = j0 + tid + r * nthreads;
+                if (pos[r] >= kk && gi < n) BetterPivot(v, p, AbsT(row[r][K]), pos[r]);
+            }
+            // the wavefront's candidate: within rows of 16 lanes by DPP, across the four rows through scalar registers
+            BetterPivot(v, p, FromLaneAboveOrSelf<8>(v), FromLaneAboveOrSelf<8>(p));
+            BetterPivot(v, p, FromLaneAboveOrSelf<4>(v), FromLaneAboveOrSelf<4>(p));
+            BetterPivot(v, p, FromLaneAboveOrSelf<2>(v), FromLaneAboveOrSelf<2>(p));
+            BetterPivot(v, p, FromLaneAboveOrSelf<1>(v), FromLaneAboveOrSelf<1>(p));
+            T wv = ReadLaneT(v, 0);
+            int wp = __builtin_amdgcn_readlane(p, 0);
+            BetterPivot(wv, wp, ReadLaneT(v, 16), __builtin_amdgcn_readlane(p, 16));
+            BetterPivot(wv, wp, ReadLaneT(v, 32), __builtin_amdgcn_readlane(p, 32));
+            BetterPivot(wv, wp, ReadLaneT(v, 48), __builtin_amdgcn_readlane(p, 48));
+#pragma unroll
+            for (int r = 0; r < ROWS; ++r) {
+                if (pos[r] == wp) {  // positions are distinct: one lane of the wavefront at most
+#pragma unroll
+                    for (int j = 0; j < NB; ++j) sh.candidate[par][wave][j] = row[r][j];
+                    sh.value[par][wave] = wv;
+                    sh.position[par][wave] = wp;
+                }
+            }
+            if (wp == 0x7fffffff && (tid & 63) == 0) sh.value[par][wave] = T(-1), sh.position[par][wave] = wp;  // no candidate here
+            __syncthreads();
+            T bv = sh.value[par][0];
+            int bp = sh.position[par][0];
+            int bw = 0;
+            for (int q = 1; q < nwaves; ++q) {
+                const T ov = sh.value[par][q];
+                const int op = sh.position[par][q];
+                if (ov > bv || (ov == bv && op < bp)) bv = ov, bp = op, bw = q;
+            }
+            if (bv > T(0)) {
+                // the rows at positions bp and kk change places, then the pivot row leaves every row after it
+#pragma unroll
+                for (int r = 0; r < ROWS; ++r) {
+                    const int was = pos[r];
+                    if (was == bp) pos[r] = kk;
+                    if (was == kk) pos[r] = bp;
+                }
+                const T scale = T(1) / sh.candidate[par][bw][K];  // getf2 scales the column by the reciprocal of the pivot
+#pragma unroll
+                for (int r = 0; r < ROWS; ++r) {
+                    const int gi = j0 + tid + r * nthreads;
+                    if (pos[r] > kk && gi < n) {
+                        const T m = row[r][K] * scale;
+                        row[r][K] = m;
+#pragma unroll
+                        for (int j = K + 1; j < NB; ++j) row[r][j] -= m * sh.candidate[par][bw][j];
+                    }
+                }
+            } else if (tid == 0 && state->info == 0) {  // a zero (or all-NaN) column is left as it is, as getrf leaves it
+                state->info = kk + 1;
+                if (user_info != nullptr) *user_info = kk + 1;
+            }
+        }
+        LuPanelSteps<T, ROWS, NB, K + 1>(row, pos, sh, n, j0, w, state, user_info);
+    }
+}
+
+// The panel of a right-looking blocked LU factorisation with partial pivoting: columns [j0, j0 + w) of a ([n, n] row-major, w <= NB),
+// rows j0 and below, one workgroup.  Every thread keeps ROWS rows of the panel in registers (row j0 + t + r * blockDim.x) together
+// with the position each of them has in the row order; an exchange of two rows only exchanges their positions, and the rows go
+// to their final positions when the panel is written back.  A column step: every wavefront proposes its row of largest magnitude
+// (the earliest in the current row order among equals, as idamax picks it) and leaves it in LDS, one barrier, every thread picks
+// the best proposal and subtracts it from its rows.  Rows that end somewhere else than they started are listed for the kernel
+// that updates the other columns.
+template <typename T, int ROWS, int NB>
+__global__ __launch_bounds__(1024) void LuPanelKernel(T* a, int n, int j0, int w, LuState* state, int* user_info) {
+    __shared__ LuPanelShared<T, NB> sh;
     const int tid = threadIdx.x;
-    for (int j = 0; j < n; ++j) {
-        const T d = l[static_cast<int64_t>(j) * n + j];
-        if (!(d > T(0))) {  // the same value for every thread: a uniform exit
-            if (tid == 0 && info != nullptr) *info = j + 1;
-            return;
+    const int nthreads = blockDim.x;
+    if (tid == 0) {
+        sh.listed = 0;
+        if (j0 == 0) state->info = 0;
+    }
+    T row[ROWS][NB];
+    int pos[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+        const int gi = j0 + tid + r * nthreads;
+        pos[r] = gi;
+#pragma unroll
+        for (int j = 0; j < NB; ++j) row[r][j] = gi < n && j < w ? a[static_cast<int64_t>(gi) * n + j0 + j] : T(0);
+    }
+    __syncthreads();  // every row is in registers before a row is written back to another row's place
+    LuPanelSteps<T, ROWS, NB, 0>(row, pos, sh, n, j0, w, state, user_info);
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+        const int gi = j0 + tid + r * nthreads;
+        if (gi < n) {
+#pragma unroll
+            for (int j = 0; j < NB; ++j) {
+                if (j < w) a[static_cast<int64_t>(pos[r]) * n + j0 + j] = row[r][j];
+            }
+            if (pos[r] != gi) {  // at most two rows per column step end up somewhere else
+                const int e = atomicAdd(&sh.listed, 1);
+                state->exchanges.row[e] = pos[r];
+                state->exchanges.source[e] = gi;
+            }
         }
-        T root;
-        if constexpr (std::is_same<T, float>::value) {
-            root = sqrtf(d);
-        } else {
-            root = sqrt(d);
+    }
+    __syncthreads();
+    if (tid == 0) state->exchanges.count = sh.listed;
+}
+
+// The columns right of a finished panel (columns [j0 + w, n) of a, and all m columns of the right-hand sides b), 64 columns per
+// workgroup: the panel's row exchanges, then U12 = L11^-1 A12 for the panel's rows (one thread per column), then
+// A22 -= L21 U12 for the rows below (64-row tiles through LDS, 4 x 4 outputs per thread).
+template <typename T>
+__global__ __launch_bounds__(256) void LuUpdateKernel(T* a, T* b, int n, int m, int j0, int w, const LuState* state) {
+    __shared__ T stage[64][65];  // exchanged rows, then tiles of L21
+    __shared__ T U[kNb][64];
+    __shared__ T L11[kNb][kNb + 1];
+    __shared__ T Linv[kNb][kNb + 1];
+    __shared__ T Ltmp[kNb][kNb + 1];
+    const int tid = threadIdx.x;
+    const int c = tid & 63, g = tid >> 6;
+    const int strips_a = (n - j0 - w + 63) / 64;
+    T* base;
+    int ld, col0;
+    if (static_cast<int>(blockIdx.x) < strips_a) {
+        base = a, ld = n, col0 = j0 + w + static_cast<int>(blockIdx.x) * 64;
+    } else {
+        base = b, ld = m, col0 = (static_cast<int>(blockIdx.x) - strips_a) * 64;
+    }
+    const int col = col0 + c;
+    const bool ok = col < ld;
+    const int count = state->exchanges.count;
+    for (int e = g; e < count; e += 4) stage[e][c] = ok ? base[static_cast<int64_t>(state->exchanges.source[e]) * ld + col] : T(0);
+    __syncthreads();
+    for (int e = g; e < count; e += 4) {
+        if (ok) base[static_cast<int64_t>(state->exchanges.row[e]) * ld + col] = stage[e][c];
+    }
+    for (int e = tid; e < kNb * kNb; e += 256) {
+        const int r = e >> 5, k = e & (kNb - 1);
+        L11[r][k] = r < w && k < w ? a[static_cast<int64_t>(j0 + r) * n + j0 + k] : T(0);
+    }
+    __syncthreads();  // the exchanged rows are in place for every thread of the workgroup
+    for (int r = g; r < kNb; r += 4) U[r][c] = ok && r < w ? base[static_cast<int64_t>(j0 + r) * ld + col] : T(0);
+    __syncthreads();
+    // U12 = L11^-1 A12: the inverse of the unit lower triangle once, then a product (8 rows per thread)
+    InvertTriangularBlock<0, 1>(L11, Linv, Ltmp, tid);
+    {
+        T u[kNb / 4];
+#pragma unroll
+        for (int i = 0; i < kNb / 4; ++i) {
+            const int r = g * (kNb / 4) + i;
+            T sum = T(0);
+            for (int k = 0; k <= r; ++k) sum += Linv[r][k] * U[k][c];
+            u[i] = sum;
         }
-        __syncthreads();  // every thread has read the diagonal before it is overwritten
-        if (tid == 0) l[static_cast<int64_t>(j) * n + j] = root;
-        for (int i = j + 1 + tid; i < n; i += kLinalgThreads) l[static_cast<int64_t>(i) * n + j] /= root;
         __syncthreads();
-        // trailing update of the lower triangle: l[i][k] -= l[i][j] * l[k][j] for j < k <= i
-        const int rows = n - j - 1;
-        const int64_t work = static_cast<int64_t>(rows) * rows;
-        for (int64_t e = tid; e < work; e += kLinalgThreads) {
-            const int i = j + 1 + static_cast<int>(e / rows);
-            const int k = j + 1 + static_cast<int>(e % rows);
-            if (k <= i) l[static_cast<int64_t>(i) * n + k] -= l[static_cast<int64_t>(i) * n + j] * l[static_cast<int64_t>(k) * n + j];
+#pragma unroll
+        for (int i = 0; i < kNb / 4; ++i) {
+            const int r = g * (kNb / 4) + i;
+            U[r][c] = u[i];
+            if (ok && r < w) base[static_cast<int64_t>(j0 + r) * ld + col] = u[i];
+        }
+    }
+    __syncthreads();
+    const int ty = tid >> 4, tx = tid & 15;
+    for (int i0 = j0 + w; i0 < n; i0 += 64) {
+        for (int e = tid; e < 64 * kNb; e += 256) {
+            const int r = e >> 5, k = e & (kNb - 1);
+            stage[r][k] = i0 + r < n && k < w ? a[static_cast<int64_t>(i0 + r) * n + j0 + k] : T(0);
+        }
+        __syncthreads();
+        T acc[4][4] = {};
+#pragma unroll 4
+        for (int k = 0; k < kNb; ++k) {
+            T lv[4], uv[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) lv[i] = stage[ty * 4 + i][k], uv[i] = U[k][tx * 4 + i];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] += lv[i] * uv[j];
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int gi = i0 + ty * 4 + i;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int cc = col0 + tx * 4 + j;
+                if (gi < n && cc < ld) base[static_cast<int64_t>(gi) * ld + cc] -= acc[i][j];
+            }
         }
         __syncthreads();
     }
-    for (int64_t e = tid; e < static_cast<int64_t>(n) * n; e += kLinalgThreads) {
-        const int i = static_cast<int>(e / n), k = static_cast<int>(e % n);
-        if (k > i) l[e] = T(0);
+}
+
+// Back substitution with the upper triangle of a factored matrix: b ([n, m] row-major, holding L^-1 P b) becomes the solution.
+// One workgroup per 64 columns of b walks the block rows upwards: y = b_j - U[j, below] x[below] (64-deep tiles through LDS), then
+// U_jj x_j = y with one thread per column.  Nothing happens when the factorisation met a zero pivot.
+template <typename T>
+__global__ __launch_bounds__(256) void LuBackKernel(const T* a, T* b, int n, int m, const LuState* state) {
+    __shared__ T Ut[kNb][65];
+    __shared__ T Xs[64][64];
+    __shared__ T Y[kNb][64];
+    __shared__ T Ujj[kNb][kNb + 1];
+    __shared__ T Uinv[kNb][kNb + 1];
+    __shared__ T Utmp[kNb][kNb + 1];
+    if (state->info != 0) return;
+    const int tid = threadIdx.x;
+    const int c = tid & 63, g = tid >> 6;
+    const int col0 = static_cast<int>(blockIdx.x) * 64;
+    const int ty = tid >> 4, tx = tid & 15;  // outputs: rows ty * 2 .. + 1, columns tx * 4 .. + 3
+    for (int j0 = (n - 1) / kNb * kNb; j0 >= 0; j0 -= kNb) {
+        const int w = min(kNb, n - j0);
+        T acc[2][4] = {};
+        for (int k0 = j0 + w; k0 < n; k0 += 64) {
+            for (int e = tid; e < kNb * 64; e += 256) {
+                const int r = e >> 6, k = e & 63;
+                Ut[r][k] = r < w && k0 + k < n ? a[static_cast<int64_t>(j0 + r) * n + k0 + k] : T(0);
+            }
+            for (int e = tid; e < 64 * 64; e += 256) {
+                const int k = e >> 6, cc = e & 63;
+                Xs[k][cc] = k0 + k < n && col0 + cc < m ? b[static_cast<int64_t>(k0 + k) * m + col0 + cc] : T(0);
+            }
+            __syncthreads();
+#pragma unroll 4
+            for (int k = 0; k < 64; ++k) {
+                T uv[2], xv[4];
+#pragma unroll
+                for (int i = 0; i < 2; ++i) uv[i] = Ut[ty * 2 + i][k];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) xv[j] = Xs[k][tx * 4 + j];
+#pragma unroll
+                for (int i = 0; i < 2; ++i) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) acc[i][j] += uv[i] * xv[j];
+                }
+            }
+            __syncthreads();
+        }
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int r = ty * 2 + i;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int cc = tx * 4 + j;
+                Y[r][cc] = r < w && col0 + cc < m ? b[static_cast<int64_t>(j0 + r) * m + col0 + cc] - acc[i][j] : T(0);
+            }
+        }
+        for (int e = tid; e < kNb * kNb; e += 256) {
+            const int r = e >> 5, k = e & (kNb - 1);
+            Ujj[r][k] = r < w && k < w ? a[static_cast<int64_t>(j0 + r) * n + j0 + k] : (r == k ? T(1) : T(0));
+        }
+        __syncthreads();
+        // x_j = U_jj^-1 y: the inverse of the upper triangle once, then a product (8 rows per thread)
+        InvertTriangularBlock<1, 0>(Ujj, Uinv, Utmp, tid);
+#pragma unroll
+        for (int i = 0; i < kNb / 4; ++i) {
+            const int r = g * (kNb / 4) + i;
+            T sum = T(0);
+            for (int k = r; k < kNb; ++k) sum += Uinv[r][k] * Y[k][c];
+            if (r < w && col0 + c < m) b[static_cast<int64_t>(j0 + r) * m + col0 + c] = sum;
+        }
+        __syncthreads();  // the block row's solution is in b before the next block row reads it
     }
+}
+
+// Cholesky factor of the kNb x kNb block D (lower triangle read, rows / columns past the matrix continued as the identity), in place, by
+// the first wavefront of the workgroup: lane i keeps row i in registers and the values of other rows arrive through v_readlane.
+// Returns the 1-based position of the first non-positive diagonal in every lane of that wavefront, 0 when there is none.
+template <typename T>
+__device__ __forceinline__ int FactorDiagonalBlock(T (&D)[kNb][kNb + 1], int tid) {
+    int failed = 0;
+    if (tid < 64) {
+        const int row = tid & (kNb - 1);
+        T d[kNb];
+#pragma unroll
+        for (int k = 0; k < kNb; ++k) d[k] = D[row][k];
+#pragma unroll
+        for (int k = 0; k < kNb; ++k) {
+            const T dk = ReadLaneT(d[k], k);
+            if (!(dk > T(0)) && failed == 0) failed = k + 1;
+            const T root = SqrtT(dk);
+            const T lik = row == k ? root : d[k] / root;
+            d[k] = lik;
+#pragma unroll
+            for (int j = k + 1; j < kNb; ++j) d[j] -= lik * ReadLaneT(lik, j);  // only columns j <= row are meaningful
+        }
+        if (tid < kNb) {
+#pragma unroll
+            for (int k = 0; k < kNb; ++k) D[row][k] = d[k];
+        }
+    }
+    return failed;
+}
+
+// Stores the factored diagonal block D at (i0, i0) of l and clears the strict upper triangle of its w rows.
+template <typename T>
+__device__ __forceinline__ void StoreDiagonalBlock(T* l, int n, int i0, int w, const T (&D)[kNb][kNb + 1], int tid) {
+    for (int e = tid; e < kNb * kNb; e += 256) {
+        const int r = e >> 5, c = e & (kNb - 1);
+        if (r < w && c < w) l[static_cast<int64_t>(i0 + r) * n + i0 + c] = c <= r ? D[r][c] : T(0);
+    }
+    const int right = n - (i0 + w);
+    for (int e = tid; e < w * right; e += 256) l[static_cast<int64_t>(i0 + e / right) * n + i0 + w + e % right] = T(0);
+}
+
+// One step of a left-looking blocked Cholesky factorisation of the lower triangle of l ([n, n] row-major).  With `first` set, one
+// workgroup factors the leading diagonal block.  Otherwise the diagonal block at j0 is already factored, and workgroup r owns the
+// kNb rows from i0 = j0 + (r + 1) * kNb: it subtracts the contribution of the finished columns [0, j0) from its rows of the block
+// column [j0, j0 + kNb) and solves them against the diagonal block's factor.  The workgroup right below the diagonal block (r = 0)
+// then holds everything the next diagonal block needs: it updates and factors that block as well, so that the next step finds it
+// ready and no workgroup ever reads a block that another one of the same launch writes.  A non-positive diagonal stores its 1-based
+// position in *info, once; later steps then leave the matrix alone.
+template <typename T>
+__global__ __launch_bounds__(256) void CholeskyBlockKernel(T* l, int n, int j0, int first, int* info) {
+    __shared__ T P[kNb][kNb + 1];  // 32 finished columns of the diagonal block's rows
+    __shared__ T Q[kNb][kNb + 1];  // the same columns of this workgroup's rows
+    __shared__ T D[kNb][kNb + 1];  // the diagonal block's factor, later the next diagonal block
+    __shared__ T R[kNb][kNb + 1];  // this workgroup's rows of the block column
+    if (info != nullptr && *info != 0) return;  // the same value for every thread of the grid: earlier launches wrote it
+    const int tid = threadIdx.x;
+    const int tr = tid >> 3, tc = (tid & 7) << 2;  // this thread's four outputs: row tr, columns tc .. tc + 3
+    if (first) {
+        const int w = min(kNb, n);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int col = tc + c;
+            D[tr][col] = tr < w && col < w ? l[static_cast<int64_t>(tr) * n + col] : (tr == col ? T(1) : T(0));
+        }
+        __syncthreads();
+        const int failed = FactorDiagonalBlock(D, tid);
+        if (tid == 0 && failed != 0 && info != nullptr) *info = failed;
+        __syncthreads();
+        StoreDiagonalBlock(l, n, 0, w, D, tid);
+        return;
+    }
+    const int i0 = j0 + (static_cast<int>(blockIdx.x) + 1) * kNb;
+    const int w = min(kNb, n - i0);  // rows of this workgroup
+    const bool next = blockIdx.x == 0;
+    T acc_r[4] = {T(0), T(0), T(0), T(0)};
+    T acc_d[4] = {T(0), T(0), T(0), T(0)};
+    for (int k0 = 0; k0 < j0; k0 += kNb) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            P[tr][tc + c] = l[static_cast<int64_t>(j0 + tr) * n + k0 + tc + c];
+            Q[tr][tc + c] = tr < w ? l[static_cast<int64_t>(i0 + tr) * n + k0 + tc + c] : T(0);
+        }
+        __syncthreads();
+#pragma unroll 8
+        for (int k = 0; k < kNb; ++k) {
+            const T qd = Q[tr][k];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) acc_r[c] += qd * P[tc + c][k];
+        }
+        if (next) {
+#pragma unroll 8
+            for (int k = 0; k < kNb; ++k) {
+                const T qd = Q[tr][k];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) acc_d[c] += qd * Q[tc + c][k];
+            }
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        const int col = tc + c;
+        D[tr][col] = l[static_cast<int64_t>(j0 + tr) * n + j0 + col];
+        R[tr][col] = tr < w ? l[static_cast<int64_t>(i0 + tr) * n + j0 + col] - acc_r[c] : T(0);
+    }
+    __syncthreads();
+    // x L^T = r for every row: the inverse of the factor once, then x = r L^-T (four entries per thread)
+    InvertTriangularBlock<0, 0>(D, P, Q, tid);
+    {
+        T x[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int col = tc + c;
+            T sum = T(0);
+            for (int k = 0; k <= col; ++k) sum += R[tr][k] * P[col][k];
+            x[c] = sum;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            R[tr][tc + c] = x[c];
+            if (tr < w) l[static_cast<int64_t>(i0 + tr) * n + j0 + tc + c] = x[c];
+        }
+    }
+    __syncthreads();
+    if (!next) return;
+    // the next diagonal block: its entries minus the products of these rows over all columns up to j0 + kNb
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        const int col = tc + c;
+        T s = acc_d[c];
+#pragma unroll 8
+        for (int k = 0; k < kNb; ++k) s += R[tr][k] * R[col][k];
+        D[tr][col] = tr < w && col < w ? l[static_cast<int64_t>(i0 + tr) * n + i0 + col] - s : (tr == col ? T(1) : T(0));
+    }
+    __syncthreads();
+    const int failed = FactorDiagonalBlock(D, tid);
+    if (tid == 0 && failed != 0 && info != nullptr) *info = i0 + failed;
+    __syncthreads();
+    StoreDiagonalBlock(l, n, i0, w, D, tid);
 }
 
 template <typename T>
@@ -306,11 +806,6 @@ __device__ void ApplyReflector(const T* w, int n, int j, int m, T tau, T* y, int
         }
         __syncthreads();
     }
-}
-
-template <typename T>
-__device__ inline T SqrtT(T x) {
-    return std::is_same<T, float>::value ? T(sqrtf(static_cast<float>(x))) : T(sqrt(static_cast<double>(x)));
 }
 
 // Householder QR in place, LAPACK geqrf's result: R on and above the diagonal of w ([m, n] row-major), the reflector vectors below
@@ -613,6 +1108,72 @@ void CopyInto(const hipcx_array* src, const hipcx_array* dst, void* stream, cons
     HIPCX_REQUIRE(rc == HIPCX_OK, HIPCX_CHAINERX_ERROR, std::string(what) + ": " + hipcx_last_error());
 }
 
+// Largest matrix the blocked LU takes: its panel kernel keeps all rows of a panel in the registers of one workgroup.
+constexpr int64_t kLuBlockedMaxN = 8192;
+
+size_t LuStateOffset(int64_t n) { return (static_cast<size_t>(n) * static_cast<size_t>(n) * 8 + 255) / 256 * 256; }
+
+template <typename T, int ROWS>
+void LaunchLuPanel(T* a, int n, int j0, int w, unsigned threads, LuState* state, int32_t* user_info, hipStream_t stream) {
+    constexpr int kBudget = sizeof(T) == 4 ? 64 : 32;  // panel values per thread
+    constexpr int NB = kBudget / ROWS < kNb ? kBudget / ROWS : kNb;
+    hipLaunchKernelGGL((LuPanelKernel<T, ROWS, NB>), dim3(1), dim3(threads), 0, stream, a, n, j0, w, state, user_info);
+}
+
+// Factors a ([n, n], destroyed) and solves for the m columns of b in place.  `state` lives in device memory.
+template <typename T>
+void LuSolveBlocked(T* a, T* b, int64_t n, int64_t m, LuState* state, int32_t* user_info, hipStream_t stream) {
+    constexpr int kBudget = sizeof(T) == 4 ? 64 : 32;
+    const unsigned strips_b = static_cast<unsigned>((m + 63) / 64);
+    for (int64_t j0 = 0; j0 < n;) {
+        const int64_t rows = n - j0;
+        int per_thread = 1;
+        while (rows > 1024 * per_thread) per_thread *= 2;
+        const int nb = std::min(kNb, kBudget / per_thread);
+        const int w = static_cast<int>(std::min<int64_t>(nb, rows));
+        const unsigned threads = static_cast<unsigned>(((rows + per_thread - 1) / per_thread + 63) / 64 * 64);
+        switch (per_thread) {
+            case 1:
+                LaunchLuPanel<T, 1>(a, static_cast<int>(n), static_cast<int>(j0), w, threads, state, user_info, stream);
+                break;
+            case 2:
+                LaunchLuPanel<T, 2>(a, static_cast<int>(n), static_cast<int>(j0), w, threads, state, user_info, stream);
+                break;
+            case 4:
+                LaunchLuPanel<T, 4>(a, static_cast<int>(n), static_cast<int>(j0), w, threads, state, user_info, stream);
+                break;
+            default:
+                LaunchLuPanel<T, 8>(a, static_cast<int>(n), static_cast<int>(j0), w, threads, state, user_info, stream);
+                break;
+        }
+        const unsigned strips_a = static_cast<unsigned>((n - j0 - w + 63) / 64);
+        hipLaunchKernelGGL(LuUpdateKernel<T>, dim3(strips_a + strips_b), dim3(256), 0, stream, a, b, static_cast<int>(n), static_cast<int>(m),
+                           static_cast<int>(j0), w, state);
+        j0 += w;
+    }
+    hipLaunchKernelGGL(LuBackKernel<T>, dim3(strips_b), dim3(256), 0, stream, a, b, static_cast<int>(n), static_cast<int>(m), state);
+}
+
+// a (already copied into the workspace) and b (already in out) -> the solution in out
+void LaunchLuSolve(int dtype, void* workspace, void* out, int64_t n, int64_t m, int32_t* error_flag, void* stream) {
+    if (n > kLuBlockedMaxN) {
+        if (dtype == HIPCX_FLOAT32) {
+            hipLaunchKernelGGL(LuSolveKernel<float>, dim3(1), dim3(kLinalgThreads), 0, AsStream(stream), static_cast<float*>(workspace),
+                               static_cast<float*>(out), static_cast<int>(n), static_cast<int>(m), error_flag);
+        } else {
+            hipLaunchKernelGGL(LuSolveKernel<double>, dim3(1), dim3(kLinalgThreads), 0, AsStream(stream), static_cast<double*>(workspace),
+                               static_cast<double*>(out), static_cast<int>(n), static_cast<int>(m), error_flag);
+        }
+        return;
+    }
+    LuState* state = reinterpret_cast<LuState*>(static_cast<char*>(workspace) + LuStateOffset(n));
+    if (dtype == HIPCX_FLOAT32) {
+        LuSolveBlocked<float>(static_cast<float*>(workspace), static_cast<float*>(out), n, m, state, error_flag, AsStream(stream));
+    } else {
+        LuSolveBlocked<double>(static_cast<double*>(workspace), static_cast<double*>(out), n, m, state, error_flag, AsStream(stream));
+    }
+}
+
 }  // namespace
 }  // namespace hipcx
 
@@ -622,7 +1183,7 @@ extern "C" {
 
 size_t hipcx_solve_workspace_size(const hipcx_array* a) {
     if (a == nullptr || a->ndim != 2 || a->shape[0] < 0) return 0;
-    return static_cast<size_t>(a->shape[0]) * static_cast<size_t>(a->shape[0]) * 8;
+    return LuStateOffset(a->shape[0]) + sizeof(LuState);  // the working copy of a (up to 8 bytes per element) and the pivoting state
 }
 
 int hipcx_solve(const hipcx_array* a, const hipcx_array* b, const hipcx_array* out, void* workspace, size_t workspace_bytes,
@@ -638,19 +1199,13 @@ int hipcx_solve(const hipcx_array* a, const hipcx_array* b, const hipcx_array* o
         const int64_t n = a->shape[0], m = b->ndim == 2 ? b->shape[1] : 1;
         if (n == 0 || m == 0) return;
         HIPCX_REQUIRE(m < (1LL << 20), HIPCX_NOT_IMPLEMENTED_ERROR, "solve: too many right-hand sides");
-        HIPCX_REQUIRE(workspace != nullptr && workspace_bytes >= static_cast<size_t>(n * n * ItemSize(out->dtype)), HIPCX_CHAINERX_ERROR,
+        HIPCX_REQUIRE(workspace != nullptr && workspace_bytes >= hipcx_solve_workspace_size(a), HIPCX_CHAINERX_ERROR,
                       "solve workspace too small");
         HIPCX_REQUIRE(reinterpret_cast<uintptr_t>(workspace) % 16 == 0, HIPCX_CHAINERX_ERROR, "workspace must be 16-byte aligned");
         hipcx_array lu = Dense2D(workspace, out->dtype, n, n);
         CopyInto(a, &lu, stream, "solve: copying a");
         CopyInto(b, out, stream, "solve: copying b");
-        if (out->dtype == HIPCX_FLOAT32) {
-            hipLaunchKernelGGL(LuSolveKernel<float>, dim3(1), dim3(kLinalgThreads), 0, AsStream(stream), static_cast<float*>(workspace),
-                               static_cast<float*>(out->data), static_cast<int>(n), static_cast<int>(m), error_flag);
-        } else {
-            hipLaunchKernelGGL(LuSolveKernel<double>, dim3(1), dim3(kLinalgThreads), 0, AsStream(stream), static_cast<double*>(workspace),
-                               static_cast<double*>(out->data), static_cast<int>(n), static_cast<int>(m), error_flag);
-        }
+        LaunchLuSolve(out->dtype, workspace, out->data, n, m, error_flag, stream);
         CheckLaunch("solve");
     });
 }
@@ -663,7 +1218,7 @@ int hipcx_inverse(const hipcx_array* a, const hipcx_array* out, void* workspace,
         HIPCX_REQUIRE(SameShape(a, out) && IsContiguous(out), HIPCX_DIMENSION_ERROR, "inverse: out must be C-contiguous with a's shape");
         const int64_t n = a->shape[0];
         if (n == 0) return;
-        HIPCX_REQUIRE(workspace != nullptr && workspace_bytes >= static_cast<size_t>(n * n * ItemSize(out->dtype)), HIPCX_CHAINERX_ERROR,
+        HIPCX_REQUIRE(workspace != nullptr && workspace_bytes >= hipcx_solve_workspace_size(a), HIPCX_CHAINERX_ERROR,
                       "inverse workspace too small");
         HIPCX_REQUIRE(reinterpret_cast<uintptr_t>(workspace) % 16 == 0, HIPCX_CHAINERX_ERROR, "workspace must be 16-byte aligned");
         hipcx_array lu = Dense2D(workspace, out->dtype, n, n);
@@ -671,13 +1226,10 @@ int hipcx_inverse(const hipcx_array* a, const hipcx_array* out, void* workspace,
         const unsigned blocks = static_cast<unsigned>((n * n + 255) / 256);
         if (out->dtype == HIPCX_FLOAT32) {
             hipLaunchKernelGGL(IdentityFillKernel<float>, dim3(blocks), dim3(256), 0, AsStream(stream), static_cast<float*>(out->data), static_cast<int>(n));
-            hipLaunchKernelGGL(LuSolveKernel<float>, dim3(1), dim3(kLinalgThreads), 0, AsStream(stream), static_cast<float*>(workspace),
-                               static_cast<float*>(out->data), static_cast<int>(n), static_cast<int>(n), error_flag);
         } else {
             hipLaunchKernelGGL(IdentityFillKernel<double>, dim3(blocks), dim3(256), 0, AsStream(stream), static_cast<double*>(out->data), static_cast<int>(n));
-            hipLaunchKernelGGL(LuSolveKernel<double>, dim3(1), dim3(kLinalgThreads), 0, AsStream(stream), static_cast<double*>(workspace),
-                               static_cast<double*>(out->data), static_cast<int>(n), static_cast<int>(n), error_flag);
         }
+        LaunchLuSolve(out->dtype, workspace, out->data, n, n, error_flag, stream);
         CheckLaunch("inverse");
     });
 }
@@ -691,12 +1243,17 @@ int hipcx_cholesky(const hipcx_array* a, const hipcx_array* out, int32_t* error_
         const int64_t n = a->shape[0];
         if (n == 0) return;
         CopyInto(a, out, stream, "cholesky: copying a");
-        if (out->dtype == HIPCX_FLOAT32) {
-            hipLaunchKernelGGL(CholeskyKernel<float>, dim3(1), dim3(kLinalgThreads), 0, AsStream(stream), static_cast<float*>(out->data),
-                               static_cast<int>(n), error_flag);
-        } else {
-            hipLaunchKernelGGL(CholeskyKernel<double>, dim3(1), dim3(kLinalgThreads), 0, AsStream(stream), static_cast<double*>(out->data),
-                               static_cast<int>(n), error_flag);
+        // the leading diagonal block, then one launch per block column that has rows below its diagonal block
+        for (int64_t j0 = -kNb; j0 + kNb < n; j0 += kNb) {
+            const int first = j0 < 0;
+            const unsigned blocks = first ? 1u : static_cast<unsigned>((n - j0 - 1) / kNb);
+            if (out->dtype == HIPCX_FLOAT32) {
+                hipLaunchKernelGGL(CholeskyBlockKernel<float>, dim3(blocks), dim3(256), 0, AsStream(stream), static_cast<float*>(out->data),
+                                   static_cast<int>(n), static_cast<int>(first ? 0 : j0), first, error_flag);
+            } else {
+                hipLaunchKernelGGL(CholeskyBlockKernel<double>, dim3(blocks), dim3(256), 0, AsStream(stream), static_cast<double*>(out->data),
+                                   static_cast<int>(n), static_cast<int>(first ? 0 : j0), first, error_flag);
+            }
         }
         CheckLaunch("cholesky");
     });

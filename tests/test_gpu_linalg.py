@@ -44,6 +44,50 @@ def test_solve_inverse_cholesky(dt, tol):
     assert x.dtype == np.float64
 
 
+@pytest.mark.parametrize('dt,tol', [('float32', 1e-4), ('float64', 1e-11)])
+def test_blocked_factorisations_at_block_edges_and_many_columns(dt, tol):
+    """Sizes around the 32-wide block columns and the 64-wide column strips, more right-hand sides than one strip holds, and
+    matrices whose panels need several rows per thread (above 1024 and above 2048 rows)."""
+    import chainer_amd as chx
+    rng = np.random.default_rng(11)
+    for n, m in ((31, 3), (32, 64), (33, 65), (63, 1), (64, 130), (65, 7), (96, 200), (257, 5), (1100, 9), (2100, 2)):
+        a = (rng.standard_normal((n, n)) + 3 * np.sqrt(n) * np.eye(n)).astype(dt)  # singular values stay well away from zero
+        a = a[rng.permutation(n)]  # every column's pivot sits somewhere else
+        b = rng.standard_normal((n, m)).astype(dt)
+        x = chx.solve(chx.array(a), chx.array(b)).get()
+        assert_close(x, O.solve(a, b), tol * n, 'solve n=%d m=%d' % (n, m))
+        assert np.abs(a.astype(np.float64) @ x.astype(np.float64) - b).max() <= tol * n
+        if n <= 1100:
+            inv = chx.inv(chx.array(a)).get()
+            assert_close(inv, O.inv(a), tol * n, 'inv n=%d' % n)
+        spd = (a.astype(np.float64) @ a.T.astype(np.float64)).astype(dt)
+        low = chx.cholesky(chx.array(spd)).get()
+        assert_close(low, O.cholesky(spd), tol * n, 'cholesky n=%d' % n)
+        assert np.array_equal(low, np.tril(low))
+
+
+def test_pivot_choice_among_equal_magnitudes_and_late_failures():
+    """Columns with several entries of the same largest magnitude (the first one in the current row order is the pivot, as
+    LAPACK's idamax picks it), a matrix that becomes singular only in a later block column, and a Cholesky input that stops
+    being positive definite there: the flag carries LAPACK's 1-based position."""
+    import chainer_amd as chx
+    rng = np.random.default_rng(12)
+    n = 70
+    a = rng.integers(-2, 3, (n, n)).astype('float64') + 3 * np.eye(n)
+    b = rng.standard_normal((n, 2))
+    assert_close(chx.solve(chx.array(a), chx.array(b)).get(), O.solve(a, b), 1e-9, 'integer-valued matrix')
+    sing = (rng.standard_normal((n, n)) + 8 * np.eye(n)).astype('float64')
+    sing[:, 50] = 0  # a zero column stays zero under elimination: the first zero pivot is at position 51
+    with pytest.raises(chx.ChainerxError, match='Info = 51'):
+        chx.solve(chx.array(sing), chx.array(b))
+    with pytest.raises(chx.ChainerxError, match='Info = 51'):
+        chx.inv(chx.array(sing))
+    spd = np.eye(n) * 4.0
+    spd[40, 40] = -1.0
+    with pytest.raises(chx.ChainerxError, match='Info = 41'):
+        chx.cholesky(chx.array(spd))
+
+
 def test_linalg_errors_and_empty():
     import chainer_amd as chx
     singular = np.array([[1., 2., 3.], [2., 4., 6.], [1., 0., 1.]], 'float32')
