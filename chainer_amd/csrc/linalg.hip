@@ -874,6 +874,147 @@ __global__ __launch_bounds__(kLinalgThreads) void FormQKernel(const T* w, int m,
     }
 }
 
+// Tallest matrix the multi-workgroup QR kernels take: a reflector (one column) sits in LDS, within the 64 KiB a launch gets unasked.
+constexpr int64_t kQrStripMaxRows = 4096;
+
+// Step j of the Householder QR above, spread over workgroups: every workgroup reads column j (rows j and below), forms the same
+// reflector from it (larfg's, as in HouseholderQrKernel) and applies it to its own 32 columns right of column j (8 row groups
+// whose partial sums meet in LDS).  Nobody may overwrite column j while others still read it: its final content (the scaled
+// reflector below the diagonal, beta on it) is written one launch later by workgroup 0, from the two scalars it leaves in
+// scal[(j & 1) * 2 ..]; a last launch with j = k only does that for column k - 1.
+template <typename T>
+__global__ __launch_bounds__(256) void QrColumnKernel(T* w, int m, int n, int j, int k, T* tau, int64_t tau_stride, T* scal) {
+    extern __shared__ __align__(16) char qr_column_lds[];
+    T* v = reinterpret_cast<T*>(qr_column_lds);  // the reflector: v[0] = 1, v[i] for row j + i
+    __shared__ T red[256];
+    __shared__ T sh_tau, sh_scale;
+    const int tid = threadIdx.x;
+    if (blockIdx.x == 0 && j > 0) {
+        const T scale = scal[((j - 1) & 1) * 2], beta = scal[((j - 1) & 1) * 2 + 1];
+        for (int i = j + tid; i < m; i += 256) w[static_cast<int64_t>(i) * n + j - 1] *= scale;
+        if (tid == 0) w[static_cast<int64_t>(j - 1) * n + j - 1] = beta;
+    }
+    if (j >= k) return;
+    const int rows = m - j;
+    T acc = T(0);
+    for (int i = tid; i < rows; i += 256) {
+        const T x = w[static_cast<int64_t>(j + i) * n + j];
+        v[i] = x;
+        if (i > 0) acc += x * x;
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) acc += __shfl_down(acc, o);
+    if ((tid & 63) == 0) red[tid >> 6] = acc;
+    __syncthreads();
+    if (tid == 0) {
+        const T xnorm2 = (red[0] + red[1]) + (red[2] + red[3]);
+        const T alpha = v[0];
+        T t = T(0), scale = T(1), beta = alpha;
+        if (xnorm2 != T(0)) {
+            const T norm = SqrtT(alpha * alpha + xnorm2);
+            beta = alpha >= T(0) ? -norm : norm;
+            t = (beta - alpha) / beta;
+            scale = T(1) / (alpha - beta);
+        }
+        sh_tau = t, sh_scale = scale;
+        if (blockIdx.x == 0) {
+            tau[j * tau_stride] = t;
+            scal[(j & 1) * 2] = scale;
+            scal[(j & 1) * 2 + 1] = beta;
+        }
+    }
+    __syncthreads();
+    const T t = sh_tau;
+    const int tx = tid & 31, ty = tid >> 5;
+    const int c0 = j + 1 + static_cast<int>(blockIdx.x) * 32;
+    if (t == T(0) || c0 >= n) return;  // the same for every thread of the workgroup
+    const T scale = sh_scale;
+    for (int i = tid; i < rows; i += 256) v[i] = i == 0 ? T(1) : v[i] * scale;
+    __syncthreads();
+    const int c = c0 + tx;
+    T dot = T(0);
+    if (c < n) {
+#pragma unroll 4
+        for (int i = ty; i < rows; i += 8) dot += v[i] * w[static_cast<int64_t>(j + i) * n + c];
+    }
+    red[tid] = dot;
+    __syncthreads();
+    T total = T(0);
+#pragma unroll
+    for (int g = 0; g < 8; ++g) total += red[g * 32 + tx];
+    total *= t;
+    if (c < n) {
+#pragma unroll 4
+        for (int i = ty; i < rows; i += 8) w[static_cast<int64_t>(j + i) * n + c] -= v[i] * total;
+    }
+}
+
+// q[m, mc] = H_0 H_1 ... H_{k-1} applied to the first mc columns of the identity (LAPACK orgqr), one workgroup per 32 columns of q.
+// Reflector j only touches columns j and beyond (the ones before it are still columns of the identity when it is applied), so
+// a workgroup starts at the last reflector that reaches its columns and walks down to reflector 0; the next reflector is fetched
+// into registers while the current one is applied.  LDS_STRIP: the workgroup's columns of q stay in LDS until the end (matrices
+// short enough for that), otherwise they are updated in place in memory.
+template <typename T, bool LDS_STRIP>
+__global__ __launch_bounds__(256) void FormQStripKernel(const T* w, int m, int n, int k, const T* tau, int64_t tau_stride, T* q, int64_t q_row,
+                                                        int64_t q_col, int mc) {
+    extern __shared__ __align__(16) char form_q_lds[];
+    T* v = reinterpret_cast<T*>(form_q_lds);
+    T* strip = v + m;  // [m][33], LDS_STRIP only
+    __shared__ T red[256];
+    constexpr int kFetch = static_cast<int>(kQrStripMaxRows / 256);  // rows of a reflector per thread
+    const int tid = threadIdx.x;
+    const int tx = tid & 31, ty = tid >> 5;
+    const int c0 = static_cast<int>(blockIdx.x) * 32;
+    const int c = c0 + tx;
+    auto at = [&](int i) -> T& { return LDS_STRIP ? strip[i * 33 + tx] : q[i * q_row + c * q_col]; };
+    if (LDS_STRIP || c < mc) {
+        for (int i = ty; i < m; i += 8) at(i) = i == c ? T(1) : T(0);
+    }
+    T next[kFetch];
+    auto fetch = [&](int j) {
+#pragma unroll
+        for (int u = 0; u < kFetch; ++u) {
+            const int i = tid + u * 256;
+            next[u] = i > 0 && i < m - j ? w[static_cast<int64_t>(j + i) * n + j] : T(1);
+        }
+    };
+    const int j_first = min(k - 1, c0 + 31);
+    fetch(j_first);
+    for (int j = j_first; j >= 0; --j) {
+        const int rows = m - j;
+        const T t = tau[j * tau_stride];
+#pragma unroll
+        for (int u = 0; u < kFetch; ++u) {
+            const int i = tid + u * 256;
+            if (i < rows) v[i] = next[u];
+        }
+        if (j > 0) fetch(j - 1);
+        __syncthreads();  // also: the identity (or the previous reflector's update) is complete
+        if (t != T(0)) {  // the same for every thread
+            const bool active = c < mc && c >= j;
+            T dot = T(0);
+            if (active) {
+#pragma unroll 4
+                for (int i = ty; i < rows; i += 8) dot += v[i] * at(j + i);
+            }
+            red[tid] = dot;
+            __syncthreads();
+            T total = T(0);
+#pragma unroll
+            for (int g = 0; g < 8; ++g) total += red[g * 32 + tx];
+            total *= t;
+            if (active) {
+#pragma unroll 4
+                for (int i = ty; i < rows; i += 8) at(j + i) -= v[i] * total;
+            }
+        }
+        __syncthreads();  // v and red are rewritten by the next reflector
+    }
+    if (LDS_STRIP && c < mc) {
+        for (int i = ty; i < m; i += 8) q[i * q_row + c * q_col] = strip[i * 33 + tx];
+    }
+}
+
 // r[i][c] = w[i][c] on and above the diagonal, 0 below (rows i < r_rows); or, raw, r[c][i] = w[i][c] (the column-major factored matrix)
 template <typename T>
 __global__ __launch_bounds__(256) void ExtractRKernel(const T* w, int m, int n, T* r, int64_t r_row, int64_t r_col, int r_rows, int raw) {
@@ -1305,7 +1446,7 @@ int hipcx_syevd(const hipcx_array* a, const hipcx_array* w, const hipcx_array* v
 
 size_t hipcx_qr_workspace_size(const hipcx_array* a) {
     if (a == nullptr || a->ndim != 2 || a->shape[0] < 0 || a->shape[1] < 0) return 0;
-    return static_cast<size_t>(a->shape[0]) * static_cast<size_t>(a->shape[1]) * 8 + 256;  // the factored copy
+    return static_cast<size_t>(a->shape[0]) * static_cast<size_t>(a->shape[1]) * 8 + 256;  // the factored copy, four scalars behind it
 }
 
 int hipcx_qr(const hipcx_array* a, const hipcx_array* q, const hipcx_array* r, const hipcx_array* tau, int mode, void* workspace,
@@ -1348,7 +1489,7 @@ int hipcx_qr(const hipcx_array* a, const hipcx_array* q, const hipcx_array* r, c
             return;
         }
         const size_t need = static_cast<size_t>(m * n * it);
-        HIPCX_REQUIRE(workspace != nullptr && workspace_bytes >= need, HIPCX_CHAINERX_ERROR, "qr workspace too small");
+        HIPCX_REQUIRE(workspace != nullptr && workspace_bytes >= need + 64, HIPCX_CHAINERX_ERROR, "qr workspace too small");
         HIPCX_REQUIRE(reinterpret_cast<uintptr_t>(workspace) % 16 == 0, HIPCX_CHAINERX_ERROR, "workspace must be 16-byte aligned");
         hipcx_array w_desc = Dense2D(workspace, dtype, m, n);
         CopyInto(a, &w_desc, stream, "qr");  // cast + gather into the dense working copy
@@ -1357,10 +1498,35 @@ int hipcx_qr(const hipcx_array* a, const hipcx_array* q, const hipcx_array* r, c
             T* w = static_cast<T*>(workspace);
             T* tau_p = static_cast<T*>(tau->data);
             const int64_t tau_stride = k > 1 ? tau->strides[0] / it : 1;
-            hipLaunchKernelGGL(HouseholderQrKernel<T>, dim3(1), dim3(kLinalgThreads), 0, st, w, static_cast<int>(m), static_cast<int>(n), tau_p, tau_stride);
-            if (want_q) {
-                hipLaunchKernelGGL(FormQKernel<T>, dim3(1), dim3(kLinalgThreads), 0, st, w, static_cast<int>(m), static_cast<int>(n), tau_p, tau_stride,
-                                   static_cast<T*>(q->data), q->strides[0] / it, q->strides[1] / it, static_cast<int>(mc));
+            if (m <= kQrStripMaxRows && m * n > 96 * 96) {
+                // one launch per column, the trailing columns spread over workgroups (below about a hundred rows the launches cost
+                // more than the one-workgroup kernel); the scalars a column leaves for the next launch live behind the factored copy
+                T* scal = reinterpret_cast<T*>(static_cast<char*>(workspace) + (need + 15) / 16 * 16);
+                for (int64_t j = 0; j <= k; ++j) {
+                    const unsigned strips = j < k ? static_cast<unsigned>(std::max<int64_t>(1, (n - j - 1 + 31) / 32)) : 1u;
+                    hipLaunchKernelGGL(QrColumnKernel<T>, dim3(strips), dim3(256), static_cast<size_t>(m * it), st, w, static_cast<int>(m),
+                                       static_cast<int>(n), static_cast<int>(j), static_cast<int>(k), tau_p, tau_stride, scal);
+                }
+                if (want_q) {
+                    const dim3 grid(static_cast<unsigned>((mc + 31) / 32));
+                    const size_t strip_bytes = static_cast<size_t>(m * 34 * it);  // the reflector and [m][33] of q
+                    if (strip_bytes <= 60 * 1024) {
+                        hipLaunchKernelGGL((FormQStripKernel<T, true>), grid, dim3(256), strip_bytes, st, w, static_cast<int>(m), static_cast<int>(n),
+                                           static_cast<int>(k), tau_p, tau_stride, static_cast<T*>(q->data), q->strides[0] / it, q->strides[1] / it,
+                                           static_cast<int>(mc));
+                    } else {
+                        hipLaunchKernelGGL((FormQStripKernel<T, false>), grid, dim3(256), static_cast<size_t>(m * it), st, w, static_cast<int>(m),
+                                           static_cast<int>(n), static_cast<int>(k), tau_p, tau_stride, static_cast<T*>(q->data), q->strides[0] / it,
+                                           q->strides[1] / it, static_cast<int>(mc));
+                    }
+                }
+            } else {
+                hipLaunchKernelGGL(HouseholderQrKernel<T>, dim3(1), dim3(kLinalgThreads), 0, st, w, static_cast<int>(m), static_cast<int>(n), tau_p,
+                                   tau_stride);
+                if (want_q) {
+                    hipLaunchKernelGGL(FormQKernel<T>, dim3(1), dim3(kLinalgThreads), 0, st, w, static_cast<int>(m), static_cast<int>(n), tau_p,
+                                       tau_stride, static_cast<T*>(q->data), q->strides[0] / it, q->strides[1] / it, static_cast<int>(mc));
+                }
             }
             const int raw = mode == HIPCX_QR_RAW ? 1 : 0;
             const int64_t total = (raw ? m : r_rows) * n;
