@@ -336,8 +336,8 @@ def section_train(chx, oracle, with_cpu):
 
 
 def section_linalg(chx, oracle, with_cpu):
-    """Dense decompositions (float32).  Solve, inverse and Cholesky are blocked over many workgroups; QR, eigh and svd run in one
-    workgroup per matrix.  The CPU column is LAPACK through numpy, which is what the native backend calls."""
+    """Dense decompositions (float32): blocked LU / Cholesky, QR by columns and Jacobi rounds, all spread over many workgroups above
+    about 64 to 100 rows.  The CPU column is LAPACK through numpy, which is what the native backend calls."""
     rng = np.random.default_rng(8)
     for n in (64, 256, 1024):
         a = (rng.standard_normal((n, n)) + np.sqrt(n) * np.eye(n)).astype(np.float32)

@@ -12,6 +12,8 @@
 // stores its 1-based position in the caller's flag, LAPACK's `info`, for the caller to raise on.
 // Matrices above 8192 rows fall back to an LU kernel in which one workgroup walks the whole matrix.  QR, the symmetric
 // eigendecomposition and the SVD further down are one-workgroup kernels.
+#include <vector>
+
 #include "common.h"
 
 namespace hipcx {
@@ -650,14 +652,128 @@ __global__ __launch_bounds__(256) void IdentityFillKernel(T* out, int n) {
     out[e] = (e / n == e % n) ? T(1) : T(0);
 }
 
+// The columns p and q of the round-robin pairing: player idx of `round` (np = N rounded up to even players, the last of them fixed).
+// q = -1 for the pair that holds the dummy player of an odd N.
+__device__ __forceinline__ void JacobiPair(int idx, int round, int N, int& p, int& q) {
+    const int rounds = N + (N & 1) - 1;
+    p = idx == 0 ? rounds : (round + idx) % rounds;
+    q = idx == 0 ? round % rounds : (round - idx + rounds) % rounds;
+    if (p > q) { const int t2 = p; p = q; q = t2; }
+    if (q >= N) q = -1;
+}
+
+constexpr int kEighMaxSweeps = 60;
+constexpr int kEighNormBlocks = 128;
+// up to this many rows the sweeps stay inside the one-workgroup kernel (two launches per round would cost more)
+constexpr int kEighOneWorkgroupMaxN = 64;
+
+// Sums of squares of s ([n, n]): partial[2 b] over the off-diagonal entries and partial[2 b + 1] over all entries that workgroup b
+// visits; the host adds the kEighNormBlocks pairs up.
+template <typename T>
+__global__ __launch_bounds__(256) void EighNormsKernel(const T* s, int n, T* partial) {
+    __shared__ T red[2][4];
+    const int tid = threadIdx.x;
+    T off = T(0), all = T(0);
+    const int64_t total = static_cast<int64_t>(n) * n;
+    for (int64_t e = static_cast<int64_t>(blockIdx.x) * 256 + tid; e < total; e += static_cast<int64_t>(kEighNormBlocks) * 256) {
+        const T x = s[e];
+        all += x * x;
+        if (e / n != e % n) off += x * x;
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) off += __shfl_down(off, o), all += __shfl_down(all, o);
+    if ((tid & 63) == 0) red[0][tid >> 6] = off, red[1][tid >> 6] = all;
+    __syncthreads();
+    if (tid == 0) {
+        partial[2 * blockIdx.x] = (red[0][0] + red[0][1]) + (red[0][2] + red[0][3]);
+        partial[2 * blockIdx.x + 1] = (red[1][0] + red[1][1]) + (red[1][2] + red[1][3]);
+    }
+}
+
+// First half of a round of the two-sided Jacobi sweeps of JacobiEighKernel below, spread over workgroups: one wavefront per pair
+// (p, q) of the round computes the rotation that annihilates s[p][q], leaves (cosine, sine) in cs[2 idx ..] and applies it from
+// the left: rows p and q of s, and rows p and q of vt (the accumulated rotations, transposed: row i is eigenvector i).
+template <typename T>
+__global__ __launch_bounds__(256) void EighRowsKernel(T* s, T* vt, int n, int round, int compute_v, T* cs) {
+    const int lane = threadIdx.x & 63;
+    const int idx = static_cast<int>(blockIdx.x) * 4 + static_cast<int>(threadIdx.x >> 6);
+    if (idx >= (n + 1) / 2) return;  // whole wavefronts
+    int p, q;
+    JacobiPair(idx, round, n, p, q);
+    T c = T(1), sn = T(0);
+    if (q >= 0) {
+        const T apq = s[static_cast<int64_t>(p) * n + q];
+        if (apq != T(0)) {
+            const T app = s[static_cast<int64_t>(p) * n + p], aqq = s[static_cast<int64_t>(q) * n + q];
+            const T tau = (aqq - app) / (T(2) * apq);
+            const T tt = (tau >= T(0) ? T(1) : T(-1)) / ((tau >= T(0) ? tau : -tau) + SqrtT(T(1) + tau * tau));
+            c = T(1) / SqrtT(T(1) + tt * tt);
+            sn = tt * c;
+        }
+    }
+    if (lane == 0) cs[2 * idx] = c, cs[2 * idx + 1] = sn;
+    if (sn == T(0)) return;  // the same in every lane
+    T* sp = s + static_cast<int64_t>(p) * n;
+    T* sq = s + static_cast<int64_t>(q) * n;
+#pragma unroll 4
+    for (int i = lane; i < n; i += 64) {
+        const T a = sp[i], b = sq[i];
+        sp[i] = c * a - sn * b;
+        sq[i] = sn * a + c * b;
+    }
+    if (compute_v) {
+        T* vp = vt + static_cast<int64_t>(p) * n;
+        T* vq = vt + static_cast<int64_t>(q) * n;
+#pragma unroll 4
+        for (int i = lane; i < n; i += 64) {
+            const T a = vp[i], b = vq[i];
+            vp[i] = c * a - sn * b;
+            vq[i] = sn * a + c * b;
+        }
+    }
+}
+
+// Second half of the round: the same rotations from the right.  Columns p and q of s change, but a workgroup walks rows: each of
+// its four wavefronts takes one row of s into LDS, rotates the entries (p, q) of every pair there and writes the row back.  The
+// entry a rotation annihilates is stored as an exact zero (see JacobiEighKernel).
+template <typename T>
+__global__ __launch_bounds__(256) void EighColumnsKernel(T* s, int n, int round, const T* cs) {
+    extern __shared__ __align__(16) char eigh_rows_lds[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    T* row = reinterpret_cast<T*>(eigh_rows_lds) + static_cast<int64_t>(wave) * n;
+    const int r = static_cast<int>(blockIdx.x) * 4 + wave;
+    const bool valid = r < n;
+    if (valid) {
+        for (int i = lane; i < n; i += 64) row[i] = s[static_cast<int64_t>(r) * n + i];
+    }
+    __syncthreads();
+    if (valid) {
+        for (int idx = lane; idx < (n + 1) / 2; idx += 64) {
+            int p, q;
+            JacobiPair(idx, round, n, p, q);
+            if (q < 0) continue;
+            const T c = cs[2 * idx], sn = cs[2 * idx + 1];
+            if (sn == T(0)) continue;
+            const T a = row[p], b = row[q];
+            row[p] = r == q ? T(0) : c * a - sn * b;
+            row[q] = r == p ? T(0) : sn * a + c * b;
+        }
+    }
+    __syncthreads();
+    if (valid) {
+        for (int i = lane; i < n; i += 64) s[static_cast<int64_t>(r) * n + i] = row[i];
+    }
+}
+
 // Symmetric eigendecomposition by cyclic Jacobi rotations, one workgroup.  s: [n, n] row-major, symmetric on entry, destroyed
 // (its diagonal converges to the eigenvalues); v: [n, n] accumulates the rotations (eigenvectors as columns); w: the eigenvalues in
 // ascending order, with the columns of v permuted to match (LAPACK syevd's order, CX/native/native_device/linalg.cc:602-660).
 // A sweep visits all pairs in n - 1 rounds of n / 2 disjoint pairs (round-robin pairing), so the rotations of a round apply in
-// parallel: first to the columns of s and v, then to the rows of s.
+// parallel: first to the columns of s and v, then to the rows of s.  With do_sweeps = 0 the sweeps have been done already
+// (EighRowsKernel / EighColumnsKernel, which keep the rotations transposed in v_scratch) and only the order and the outputs are produced.
 template <typename T>
 __global__ __launch_bounds__(kLinalgThreads) void JacobiEighKernel(T* s, T* v, T* w, int n, int compute_v, int64_t v_row, int64_t v_col,
-                                                                   int64_t w_stride, T* v_scratch) {
+                                                                   int64_t w_stride, T* v_scratch, int do_sweeps) {
     extern __shared__ __align__(16) char eigh_lds[];
     T* cs = reinterpret_cast<T*>(eigh_lds);             // [half][2]: cosine, sine of the round's rotations
     int* pq = reinterpret_cast<int*>(cs + 2 * ((n + 1) / 2));  // [half][2]: the pairs
@@ -667,7 +783,9 @@ __global__ __launch_bounds__(kLinalgThreads) void JacobiEighKernel(T* s, T* v, T
     const int np = n + (n & 1);  // players of the round-robin schedule (one dummy when n is odd)
     const int half = np / 2;
     const int m = np - 1;
-    for (int64_t e = tid; e < static_cast<int64_t>(n) * n; e += kLinalgThreads) v_scratch[e] = (e / n == e % n) ? T(1) : T(0);
+    if (do_sweeps) {
+        for (int64_t e = tid; e < static_cast<int64_t>(n) * n; e += kLinalgThreads) v_scratch[e] = (e / n == e % n) ? T(1) : T(0);
+    }
     __syncthreads();
     auto block_sum = [&](T x) -> T {
 #pragma unroll
@@ -687,7 +805,7 @@ __global__ __launch_bounds__(kLinalgThreads) void JacobiEighKernel(T* s, T* v, T
         __syncthreads();
     }
     const T eps = std::is_same<T, float>::value ? T(4e-7) : T(1e-15);  // relative off-diagonal norm at which rounding dominates
-    for (int sweep = 0; sweep < 60; ++sweep) {
+    for (int sweep = 0; sweep < (do_sweeps ? kEighMaxSweeps : 0); ++sweep) {
         T acc = T(0);
         for (int64_t e = tid; e < static_cast<int64_t>(n) * n; e += kLinalgThreads) {
             if (e / n != e % n) acc += s[e] * s[e];
@@ -761,7 +879,10 @@ __global__ __launch_bounds__(kLinalgThreads) void JacobiEighKernel(T* s, T* v, T
         }
         w[rank * w_stride] = wi;
         if (compute_v) {
-            for (int r = 0; r < n; ++r) v[r * v_row + rank * v_col] = v_scratch[static_cast<int64_t>(r) * n + i];
+            // the rotations were accumulated as columns by the sweeps above, as rows (transposed) by the spread-out sweeps
+            for (int r = 0; r < n; ++r) {
+                v[r * v_row + rank * v_col] = do_sweeps ? v_scratch[static_cast<int64_t>(r) * n + i] : v_scratch[static_cast<int64_t>(i) * n + r];
+            }
         }
     }
 }
@@ -1026,90 +1147,105 @@ __global__ __launch_bounds__(256) void ExtractRKernel(const T* w, int m, int n, 
     else r[i * r_row + c * r_col] = (c >= i && i < m) ? w[i * n + c] : T(0);
 }
 
-// Singular value decomposition by one-sided Jacobi rotations (Hestenes), one workgroup.  g: [M, N] row-major with M >= N, destroyed:
+constexpr int kSvdMaxSweeps = 60;
+// up to this many columns the sweeps stay inside the one-workgroup kernel (a launch per round would cost more)
+constexpr int kSvdOneWorkgroupMaxColumns = 64;
+
+// a pair of columns counts as orthogonal when |a_p . a_q| <= SvdTolerance(M) * |a_p| |a_q|
+template <typename T>
+__device__ __forceinline__ T SvdTolerance(int M) {
+    return SqrtT(static_cast<T>(M)) * (std::is_same<T, float>::value ? T(1.2e-7) : T(2.3e-16));
+}
+
+// One wavefront makes the columns p and q of g orthogonal (one-sided Jacobi, Hestenes) and applies the same rotation to v.  Columns
+// are contiguous in memory (g: [N][M], v: [N][N], both column by column), so the wavefront streams its two columns: three dot
+// products, a butterfly reduction that leaves the sums in every lane, the rotation, and the same two columns of g and v again.
+// Returns whether the pair needed a rotation (the same in every lane).
+template <typename T>
+__device__ __forceinline__ bool SvdRotatePair(T* g, int M, int N, T* v, int p, int q, int compute_uv, int lane) {
+    T* gp = g + static_cast<int64_t>(p) * M;
+    T* gq = g + static_cast<int64_t>(q) * M;
+    T alpha = T(0), beta = T(0), gamma = T(0);
+#pragma unroll 4
+    for (int i = lane; i < M; i += 64) {
+        const T a = gp[i], b = gq[i];
+        alpha += a * a, beta += b * b, gamma += a * b;
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        alpha += __shfl_xor(alpha, o);
+        beta += __shfl_xor(beta, o);
+        gamma += __shfl_xor(gamma, o);
+    }
+    const T abs_gamma = gamma >= T(0) ? gamma : -gamma;
+    if (!(abs_gamma > SvdTolerance<T>(M) * SqrtT(alpha * beta) && abs_gamma > T(0))) return false;
+    const T zeta = (beta - alpha) / (T(2) * gamma);
+    const T tt = (zeta >= T(0) ? T(1) : T(-1)) / ((zeta >= T(0) ? zeta : -zeta) + SqrtT(T(1) + zeta * zeta));
+    const T c = T(1) / SqrtT(T(1) + tt * tt);
+    const T sn = c * tt;
+#pragma unroll 4
+    for (int i = lane; i < M; i += 64) {
+        const T a = gp[i], b = gq[i];
+        gp[i] = c * a - sn * b;
+        gq[i] = sn * a + c * b;
+    }
+    if (compute_uv) {
+        T* vp = v + static_cast<int64_t>(p) * N;
+        T* vq = v + static_cast<int64_t>(q) * N;
+#pragma unroll 4
+        for (int i = lane; i < N; i += 64) {
+            const T a = vp[i], b = vq[i];
+            vp[i] = c * a - sn * b;
+            vq[i] = sn * a + c * b;
+        }
+    }
+    return true;
+}
+
+// One round of the one-sided Jacobi sweeps of JacobiSvdKernel below, spread over workgroups: the round's disjoint column pairs go
+// one to a wavefront.  *rotated becomes 1 when any pair of the sweep needed a rotation.
+template <typename T>
+__global__ __launch_bounds__(256) void SvdRoundKernel(T* g, int M, int N, T* v, int round, int compute_uv, int* rotated) {
+    const int lane = threadIdx.x & 63;
+    const int idx = static_cast<int>(blockIdx.x) * 4 + static_cast<int>(threadIdx.x >> 6);
+    if (idx >= (N + 1) / 2) return;  // whole wavefronts
+    int p, q;
+    JacobiPair(idx, round, N, p, q);
+    if (q < 0) return;
+    if (SvdRotatePair(g, M, N, v, p, q, compute_uv, lane) && lane == 0) *rotated = 1;  // every writer stores the same value
+}
+
+// Singular value decomposition by one-sided Jacobi rotations (Hestenes), one workgroup.  g: the [M, N] matrix (M >= N) stored column
+// by column ([N][M]: a column is contiguous), destroyed:
 // its columns are rotated in pairs until they are mutually orthogonal, then their norms are the singular values and the normalised
-// columns the left vectors; v: [N, N] accumulates the rotations (right vectors as columns).  Results leave in descending order of
-// the singular value: s[rank], tall(i, rank) = g[i][j] / sigma_j, sq(i, rank) = v[i][j], both addressed through (row, col)
-// element strides so that the caller decides which of u / vt each one is and how it is transposed.  Columns whose singular value
-// is zero are left for the completion kernel; *first_fill receives the number of columns that are final.
+// columns the left vectors; v: [N, N] accumulates the rotations (right vectors as columns, stored column by column as well).
+// Results leave in descending order of the singular value: s[rank], tall(i, rank) = g(i, j) / sigma_j, sq(i, rank) = v(i, j), both
+// addressed through (row, col) element strides so that the caller decides which of u / vt each one is and how it is transposed.
+// Columns whose singular value is zero are left for the completion kernel; *first_fill receives the number of columns that are
+// final.  With do_sweeps = 0 the rotations have been applied already (SvdRoundKernel) and only the singular values, their order
+// and the outputs are produced.
 template <typename T>
 __global__ __launch_bounds__(kLinalgThreads) void JacobiSvdKernel(T* g, int M, int N, T* v, T* sigma, int* rank, T* s_out, int64_t s_stride,
                                                                   T* tall, int64_t tall_row, int64_t tall_col, T* sq, int64_t sq_row,
-                                                                  int64_t sq_col, int compute_uv, int* first_fill) {
+                                                                  int64_t sq_col, int compute_uv, int* first_fill, int do_sweeps) {
     constexpr int kGroups = kLinalgThreads / 64;
-    __shared__ T part[3 * kLinalgThreads];
-    __shared__ T cs[2 * 64];
     __shared__ int rotated, zeros;
-    const int tid = threadIdx.x, tx = tid & 63, ty = tid >> 6;
+    const int tid = threadIdx.x;
     const int np = N + (N & 1), half = np / 2, rounds = np - 1;
-    if (compute_uv) {
+    if (compute_uv && do_sweeps) {
         for (int64_t e = tid; e < static_cast<int64_t>(N) * N; e += kLinalgThreads) v[e] = (e / N == e % N) ? T(1) : T(0);
     }
-    const T tol = SqrtT(static_cast<T>(M)) * (std::is_same<T, float>::value ? T(1.2e-7) : T(2.3e-16));
     __syncthreads();
-    for (int sweep = 0; sweep < 60; ++sweep) {
+    for (int sweep = 0; sweep < (do_sweeps ? kSvdMaxSweeps : 0); ++sweep) {
         if (tid == 0) rotated = 0;
         __syncthreads();
         for (int round = 0; round < rounds; ++round) {
-            for (int c0 = 0; c0 < half; c0 += 64) {  // uniform bounds
-                const int idx = c0 + tx;
-                int p = 0, q = -1;
-                if (idx < half) {
-                    p = idx == 0 ? rounds : (round + idx) % rounds;
-                    q = idx == 0 ? round % rounds : (round - idx + rounds) % rounds;
-                    if (p > q) { const int t2 = p; p = q; q = t2; }
-                    if (q >= N) q = -1;  // the dummy player of an odd N
-                }
-                T alpha = T(0), beta = T(0), gamma = T(0);
-                if (q >= 0) {
-                    for (int i = ty; i < M; i += kGroups) {
-                        const T a = g[static_cast<int64_t>(i) * N + p], b = g[static_cast<int64_t>(i) * N + q];
-                        alpha += a * a, beta += b * b, gamma += a * b;
-                    }
-                }
-                part[ty * 64 + tx] = alpha;
-                part[kLinalgThreads + ty * 64 + tx] = beta;
-                part[2 * kLinalgThreads + ty * 64 + tx] = gamma;
-                __syncthreads();
-                if (ty == 0) {
-                    alpha = beta = gamma = T(0);
-#pragma unroll
-                    for (int k2 = 0; k2 < kGroups; ++k2) {
-                        alpha += part[k2 * 64 + tx];
-                        beta += part[kLinalgThreads + k2 * 64 + tx];
-                        gamma += part[2 * kLinalgThreads + k2 * 64 + tx];
-                    }
-                    T c = T(1), sn = T(0);
-                    const T abs_gamma = gamma >= T(0) ? gamma : -gamma;
-                    if (q >= 0 && abs_gamma > tol * SqrtT(alpha * beta) && abs_gamma > T(0)) {
-                        const T zeta = (beta - alpha) / (T(2) * gamma);
-                        const T tt = (zeta >= T(0) ? T(1) : T(-1)) / ((zeta >= T(0) ? zeta : -zeta) + SqrtT(T(1) + zeta * zeta));
-                        c = T(1) / SqrtT(T(1) + tt * tt);
-                        sn = c * tt;
-                        rotated = 1;  // every writer stores the same value
-                    }
-                    cs[2 * tx] = c, cs[2 * tx + 1] = sn;
-                }
-                __syncthreads();
-                const T c = cs[2 * tx], sn = cs[2 * tx + 1];
-                if (q >= 0 && sn != T(0)) {
-                    for (int i = ty; i < M; i += kGroups) {
-                        T* row = g + static_cast<int64_t>(i) * N;
-                        const T a = row[p], b = row[q];
-                        row[p] = c * a - sn * b;
-                        row[q] = sn * a + c * b;
-                    }
-                    if (compute_uv) {
-                        for (int i = ty; i < N; i += kGroups) {
-                            T* row = v + static_cast<int64_t>(i) * N;
-                            const T a = row[p], b = row[q];
-                            row[p] = c * a - sn * b;
-                            row[q] = sn * a + c * b;
-                        }
-                    }
-                }
-                __syncthreads();
+            for (int idx = tid >> 6; idx < half; idx += kGroups) {  // a pair per wavefront
+                int p, q;
+                JacobiPair(idx, round, N, p, q);
+                if (q >= 0 && SvdRotatePair(g, M, N, v, p, q, compute_uv, tid & 63)) rotated = 1;  // every writer stores the same value
             }
+            __syncthreads();  // the pairs of a round are disjoint; the next round pairs the columns anew
         }
         const int any = rotated;
         __syncthreads();
@@ -1119,7 +1255,7 @@ __global__ __launch_bounds__(kLinalgThreads) void JacobiSvdKernel(T* g, int M, i
     for (int j = tid; j < N; j += kLinalgThreads) {
         T acc = T(0);
         for (int i = 0; i < M; ++i) {
-            const T x = g[static_cast<int64_t>(i) * N + j];
+            const T x = g[static_cast<int64_t>(j) * M + i];
             acc += x * x;
         }
         sigma[j] = SqrtT(acc);
@@ -1144,12 +1280,12 @@ __global__ __launch_bounds__(kLinalgThreads) void JacobiSvdKernel(T* g, int M, i
     if (tid == 0) *first_fill = N - zeros;
     if (!compute_uv) return;
     for (int64_t e = tid; e < static_cast<int64_t>(M) * N; e += kLinalgThreads) {
-        const int64_t i = e / N, j = e % N;
+        const int64_t j = e / M, i = e % M;
         const T sj = sigma[j];
         tall[i * tall_row + rank[j] * tall_col] = sj > floor_value ? g[e] / sj : T(0);
     }
     for (int64_t e = tid; e < static_cast<int64_t>(N) * N; e += kLinalgThreads) {
-        const int64_t i = e / N, j = e % N;
+        const int64_t j = e / N, i = e % N;
         sq[i * sq_row + rank[j] * sq_col] = v[e];
     }
 }
@@ -1402,7 +1538,8 @@ int hipcx_cholesky(const hipcx_array* a, const hipcx_array* out, int32_t* error_
 
 size_t hipcx_syevd_workspace_size(const hipcx_array* a) {
     if (a == nullptr || a->ndim != 2 || a->shape[0] < 0) return 0;
-    return static_cast<size_t>(a->shape[0]) * static_cast<size_t>(a->shape[0]) * 8 * 2;  // the working copy and the rotations
+    // the working copy and the rotations; a round's (cosine, sine) pairs and the partial norms of a sweep
+    return static_cast<size_t>(a->shape[0]) * static_cast<size_t>(a->shape[0]) * 8 * 2 + (static_cast<size_t>(a->shape[0]) + 2 + 2 * kEighNormBlocks) * 8;
 }
 
 int hipcx_syevd(const hipcx_array* a, const hipcx_array* w, const hipcx_array* v, char uplo, int compute_v, void* workspace,
@@ -1420,8 +1557,7 @@ int hipcx_syevd(const hipcx_array* a, const hipcx_array* w, const hipcx_array* v
         if (n == 0) return;
         HIPCX_REQUIRE(n <= 4096, HIPCX_NOT_IMPLEMENTED_ERROR, "hip eigh: matrix too large for the one-workgroup Jacobi kernel");
         const int64_t it = ItemSize(a->dtype);
-        const size_t need = static_cast<size_t>(n * n * it) * 2;
-        HIPCX_REQUIRE(workspace != nullptr && workspace_bytes >= need, HIPCX_CHAINERX_ERROR, "eigh workspace too small");
+        HIPCX_REQUIRE(workspace != nullptr && workspace_bytes >= hipcx_syevd_workspace_size(a), HIPCX_CHAINERX_ERROR, "eigh workspace too small");
         HIPCX_REQUIRE(reinterpret_cast<uintptr_t>(workspace) % 16 == 0, HIPCX_CHAINERX_ERROR, "workspace must be 16-byte aligned");
         const int upper = (uplo == 'U' || uplo == 'u') ? 1 : 0;
         const unsigned blocks = static_cast<unsigned>((n * n + 255) / 256);
@@ -1434,9 +1570,36 @@ int hipcx_syevd(const hipcx_array* a, const hipcx_array* w, const hipcx_array* v
             T* vs = reinterpret_cast<T*>(ws + n * n * it);
             hipLaunchKernelGGL(SymmetrizeKernel<T>, dim3(blocks), dim3(256), 0, st, static_cast<const T*>(a->data), a->strides[0] / it,
                                a->strides[1] / it, s, static_cast<int>(n), upper);
+            const bool spread = n > kEighOneWorkgroupMaxN;
+            if (spread) {
+                // the sweeps as two launches per round over many workgroups; before every sweep the host reads how much is left
+                // off the diagonal
+                T* cs = reinterpret_cast<T*>(ws + 2 * n * n * it);
+                T* partial = cs + 2 * ((n + 1) / 2);
+                std::vector<T> sums(2 * kEighNormBlocks);
+                if (compute_v) hipLaunchKernelGGL(IdentityFillKernel<T>, dim3(blocks), dim3(256), 0, st, vs, static_cast<int>(n));
+                const unsigned pair_blocks = static_cast<unsigned>(((n + 1) / 2 + 3) / 4), row_blocks = static_cast<unsigned>((n + 3) / 4);
+                const double eps = std::is_same<T, float>::value ? 4e-7 : 1e-15;  // as in JacobiEighKernel
+                double total_norm = 0.0;
+                for (int sweep = 0; sweep < kEighMaxSweeps; ++sweep) {
+                    hipLaunchKernelGGL(EighNormsKernel<T>, dim3(kEighNormBlocks), dim3(256), 0, st, s, static_cast<int>(n), partial);
+                    HIPCX_CHECK_HIP(hipMemcpyAsync(sums.data(), partial, sums.size() * sizeof(T), hipMemcpyDeviceToHost, st));
+                    HIPCX_CHECK_HIP(hipStreamSynchronize(st));
+                    double off = 0.0, all = 0.0;
+                    for (int b2 = 0; b2 < kEighNormBlocks; ++b2) off += static_cast<double>(sums[2 * b2]), all += static_cast<double>(sums[2 * b2 + 1]);
+                    if (sweep == 0) total_norm = all;
+                    if (!(off > eps * eps * total_norm)) break;
+                    const int rounds = static_cast<int>(n + (n & 1)) - 1;
+                    for (int round = 0; round < rounds; ++round) {
+                        hipLaunchKernelGGL(EighRowsKernel<T>, dim3(pair_blocks), dim3(256), 0, st, s, vs, static_cast<int>(n), round, compute_v ? 1 : 0, cs);
+                        hipLaunchKernelGGL(EighColumnsKernel<T>, dim3(row_blocks), dim3(256), static_cast<size_t>(4 * n * it), st, s,
+                                           static_cast<int>(n), round, cs);
+                    }
+                }
+            }
             hipLaunchKernelGGL(JacobiEighKernel<T>, dim3(1), dim3(kLinalgThreads), lds, st, s, static_cast<T*>(v->data),
                                static_cast<T*>(w->data), static_cast<int>(n), compute_v ? 1 : 0, compute_v ? v->strides[0] / it : 0,
-                               compute_v ? v->strides[1] / it : 0, w->strides[0] / it, vs);
+                               compute_v ? v->strides[1] / it : 0, w->strides[0] / it, vs, spread ? 0 : 1);
         };
         if (a->dtype == HIPCX_FLOAT32) run(float{});
         else run(double{});
@@ -1543,7 +1706,7 @@ size_t hipcx_svd_workspace_size(const hipcx_array* a) {
     if (a == nullptr || a->ndim != 2 || a->shape[0] < 0 || a->shape[1] < 0) return 0;
     const size_t big = static_cast<size_t>(std::max(a->shape[0], a->shape[1])), small = static_cast<size_t>(std::min(a->shape[0], a->shape[1]));
     // the working copy, the accumulated rotations, singular values + ranks + projections, the count of final columns
-    return (big * small + small * small + 2 * small + big) * 8 + 8 * 256;
+    return (big * small + small * small + 2 * small + big) * 8 + 8 * 256;  // the slack also holds one flag per sweep
 }
 
 int hipcx_svd(const hipcx_array* a, const hipcx_array* u, const hipcx_array* s, const hipcx_array* vt, int full_matrices, int compute_uv,
@@ -1598,10 +1761,12 @@ int hipcx_svd(const hipcx_array* a, const hipcx_array* u, const hipcx_array* s, 
         char* sigma_mem = take(static_cast<size_t>(N) * it);
         char* dots_mem = take(static_cast<size_t>(M) * it);
         char* rank_mem = take(static_cast<size_t>(N) * sizeof(int) + sizeof(int));
+        char* flags_mem = take(kSvdMaxSweeps * sizeof(int));
         HIPCX_REQUIRE(off <= workspace_bytes, HIPCX_CHAINERX_ERROR, "svd workspace too small");
-        hipcx_array g_desc = Dense2D(g_mem, dtype, M, N);
+        // the working copy holds the tall matrix column by column: [N][M]
+        hipcx_array g_desc = Dense2D(g_mem, dtype, N, M);
         hipcx_array src = *a;
-        if (transposed) {
+        if (!transposed) {
             std::swap(src.shape[0], src.shape[1]);
             std::swap(src.strides[0], src.strides[1]);
         }
@@ -1622,9 +1787,32 @@ int hipcx_svd(const hipcx_array* a, const hipcx_array* u, const hipcx_array* s, 
             }
             int* rank = reinterpret_cast<int*>(rank_mem);
             int* first_fill = rank + N;
+            const bool spread = N > kSvdOneWorkgroupMaxColumns;
+            if (spread) {
+                // the sweeps as one launch per round over many workgroups; the host reads after every sweep whether it rotated anything
+                int* rotated = reinterpret_cast<int*>(flags_mem);
+                HIPCX_CHECK_HIP(hipMemsetAsync(rotated, 0, kSvdMaxSweeps * sizeof(int), st));
+                if (compute_uv) {
+                    hipLaunchKernelGGL(IdentityFillKernel<T>, dim3(static_cast<unsigned>((N * N + 255) / 256)), dim3(256), 0, st,
+                                       reinterpret_cast<T*>(v_mem), static_cast<int>(N));
+                }
+                const int np = static_cast<int>(N + (N & 1));
+                const unsigned blocks = static_cast<unsigned>((np / 2 + 3) / 4);
+                for (int sweep = 0; sweep < kSvdMaxSweeps; ++sweep) {
+                    for (int round = 0; round < np - 1; ++round) {
+                        hipLaunchKernelGGL(SvdRoundKernel<T>, dim3(blocks), dim3(256), 0, st, reinterpret_cast<T*>(g_mem), static_cast<int>(M),
+                                           static_cast<int>(N), reinterpret_cast<T*>(v_mem), round, compute_uv ? 1 : 0, rotated + sweep);
+                    }
+                    int any = 0;
+                    HIPCX_CHECK_HIP(hipMemcpyAsync(&any, rotated + sweep, sizeof(int), hipMemcpyDeviceToHost, st));
+                    HIPCX_CHECK_HIP(hipStreamSynchronize(st));
+                    if (!any) break;
+                }
+            }
             hipLaunchKernelGGL(JacobiSvdKernel<T>, dim3(1), dim3(kLinalgThreads), 0, st, reinterpret_cast<T*>(g_mem), static_cast<int>(M),
                                static_cast<int>(N), reinterpret_cast<T*>(v_mem), reinterpret_cast<T*>(sigma_mem), rank, static_cast<T*>(s->data),
-                               k > 1 ? s->strides[0] / it : 1, tall, tall_row, tall_col, sq, sq_row, sq_col, compute_uv ? 1 : 0, first_fill);
+                               k > 1 ? s->strides[0] / it : 1, tall, tall_row, tall_col, sq, sq_row, sq_col, compute_uv ? 1 : 0, first_fill,
+                               spread ? 0 : 1);
             if (compute_uv) {
                 hipLaunchKernelGGL(CompleteBasisKernel<T>, dim3(1), dim3(kLinalgThreads), 0, st, tall, tall_row, tall_col, static_cast<int>(M),
                                    static_cast<int>(tall_cols), first_fill, reinterpret_cast<T*>(dots_mem));

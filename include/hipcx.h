@@ -381,9 +381,10 @@ int hipcx_conv_grad_weight(const hipcx_array* x, const hipcx_array* gy, const in
 
 /* ---- linear algebra: SolveKernel, InverseKernel, CholeskyKernel CX/kernels/linalg.h:20-43 (float32 / float64, 2-D) ----
  * The native backend calls LAPACK gesv / getrf + getri / potrf (CX/native/native_device/linalg.cc:280-347, 560-600); these entries
- * agree with it to rounding.  `out` is C-contiguous; a (and b) are cast to out's dtype.  `error_flag`: a device int32 the caller
- * zeroes; a singular / not positive definite matrix stores LAPACK's `info` (1-based position) there and the reference's
- * ChainerxError is the caller's to raise.  Workspace: hipcx_solve_workspace_size(a) bytes for solve and inverse. */
+ * agree with it to rounding (blocked factorisations, 32 columns at a time, spread over many workgroups).  `out` is C-contiguous;
+ * a (and b) are cast to out's dtype.  `error_flag`: a device int32 the caller zeroes; a singular / not positive definite matrix
+ * stores LAPACK's `info` (1-based position) there and the reference's ChainerxError is the caller's to raise.  Workspace:
+ * hipcx_solve_workspace_size(a) bytes for solve and inverse. */
 size_t hipcx_solve_workspace_size(const hipcx_array* a);
 int hipcx_solve(const hipcx_array* a, const hipcx_array* b, const hipcx_array* out, void* workspace, size_t workspace_bytes,
                 int32_t* error_flag, void* stream);
@@ -393,8 +394,10 @@ int hipcx_cholesky(const hipcx_array* a, const hipcx_array* out, int32_t* error_
 /* ---- SyevdKernel CX/kernels/linalg.h:45-48 (float32 / float64, a 2-D and square) ----
  * Eigenvalues w (ascending) and, when compute_v, eigenvectors v (as columns) of the symmetric matrix held in a's `uplo` triangle
  * ('U' / 'L', either case; the other triangle is never read), as LAPACK syevd gives them to the native backend
- * (CX/native/native_device/linalg.cc:602-660).  Cyclic Jacobi rotations in one workgroup: eigenvalues agree with LAPACK's to
- * rounding, eigenvectors up to the sign of each column (and up to a rotation inside an eigenspace of a repeated eigenvalue).
+ * (CX/native/native_device/linalg.cc:602-660).  Cyclic Jacobi rotations: eigenvalues agree with LAPACK's to rounding, eigenvectors
+ * up to the sign of each column (and up to a rotation inside an eigenspace of a repeated eigenvalue).  Up to 64 rows everything
+ * runs in one workgroup; beyond that a round of rotations is two launches over many workgroups and the call waits for the stream
+ * once per sweep to read how much is left off the diagonal (so it cannot be captured into a graph).
  * w: [n], v: [n, n], any strides, a's dtype.  Workspace: hipcx_syevd_workspace_size(a) bytes.  n <= 4096. */
 size_t hipcx_syevd_workspace_size(const hipcx_array* a);
 int hipcx_syevd(const hipcx_array* a, const hipcx_array* w, const hipcx_array* v, char uplo, int compute_v, void* workspace,
@@ -402,7 +405,9 @@ int hipcx_syevd(const hipcx_array* a, const hipcx_array* w, const hipcx_array* v
 
 /* ---- QrKernel CX/kernels/linalg.h:38-41, modes CX/routines/linalg.h:22-28 (float32 / float64; a 2-D [m, n], cast to r's dtype) ----
  * Householder QR with LAPACK geqrf's reflectors (beta = -sign(alpha) * norm) and orgqr's Q, as the native backend calls them
- * (CX/native/native_device/linalg.cc:349-430): values and signs agree with it to rounding.  k = min(m, n).
+ * (CX/native/native_device/linalg.cc:349-430): values and signs agree with it to rounding.  k = min(m, n).  Matrices of about a
+ * hundred rows and more run as one launch per column with the trailing columns spread over workgroups, smaller ones (and those
+ * above 4096 rows) in one workgroup.
  *   HIPCX_QR_REDUCED : q [m, k], r [k, n] upper triangular          HIPCX_QR_COMPLETE : q [m, m], r [m, n]
  *   HIPCX_QR_R       : r [k, n] alone (q ignored)                   HIPCX_QR_RAW      : r [n, m] = the factored matrix in column-major
  * order (R and the reflector vectors), q ignored.  tau [k] receives the reflector scalars in every mode. */
@@ -414,9 +419,11 @@ int hipcx_qr(const hipcx_array* a, const hipcx_array* q, const hipcx_array* r, c
 /* ---- SvdKernel CX/kernels/linalg.h:33-36 (float32 / float64; a 2-D [m, n]; k = min(m, n)) ----
  * a = u @ diag(s) @ vt with s descending, as LAPACK gesdd gives it to the native backend (CX/native/native_device/linalg.cc:432-503):
  * u [m, k] and vt [k, n], or, full_matrices, u [m, m] and vt [n, n]; without compute_uv only s [k] is written (u, vt ignored).
- * One-sided Jacobi rotations in one workgroup: singular values agree with LAPACK's to rounding; singular vectors up to a common
+ * One-sided Jacobi rotations: singular values agree with LAPACK's to rounding; singular vectors up to a common
  * sign of u[:, i] and vt[i, :] (and a rotation inside the space of a repeated value; the columns that complete a full u / vt, or
- * that belong to zero singular values, are some orthonormal basis of the same space).  max(m, n) <= 4096. */
+ * that belong to zero singular values, are some orthonormal basis of the same space).  Up to k = 64 the sweeps run in one
+ * workgroup; beyond that a round of rotations is one launch with a wavefront per column pair, and the call waits for the stream
+ * once per sweep to read whether anything was rotated (so it cannot be captured into a graph).  max(m, n) <= 4096. */
 size_t hipcx_svd_workspace_size(const hipcx_array* a);
 int hipcx_svd(const hipcx_array* a, const hipcx_array* u, const hipcx_array* s, const hipcx_array* vt, int full_matrices, int compute_uv,
               void* workspace, size_t workspace_bytes, void* stream);

@@ -311,6 +311,40 @@ def test_svd_errors_and_empty():
         chx.pinv(chx.zeros((2, 2), 'int64'))
 
 
+def test_decompositions_spread_over_workgroups_at_larger_sizes():
+    """eigh, qr and svd at sizes where their sweeps / column steps run as many launches over many workgroups (odd sizes: the
+    round-robin pairing has a dummy player; more columns than one strip; a matrix above 1024 rows), float32, through what
+    defines the factors and against the oracle's values."""
+    import chainer_amd as chx
+    rng = np.random.default_rng(21)
+    tol = 1e-4
+    n = 513
+    a = rng.standard_normal((n, n)).astype('float32')
+    a = ((a + a.T) / 2).astype('float32')
+    w, v = chx.eigh(chx.array(a))
+    w, v = w.get(), v.get().astype(np.float64)
+    scale = np.abs(a).max() * n ** 0.5
+    assert np.all(np.diff(w) >= 0)
+    assert np.abs(w - O.eigh(a)[0]).max() <= tol * scale * n ** 0.5
+    assert np.abs(a.astype(np.float64) @ v - v * w).max() <= tol * scale * n ** 0.5
+    assert np.abs(v.T @ v - np.eye(n)).max() <= tol * n
+    for m, n in ((1030, 333), (333, 1030)):
+        a = rng.standard_normal((m, n)).astype('float32')
+        k = min(m, n)
+        q, r = chx.qr(chx.array(a))
+        q, r = q.get().astype(np.float64), r.get().astype(np.float64)
+        assert q.shape == (m, k) and r.shape == (k, n)
+        assert np.abs(q @ r - a).max() <= tol * max(m, n) and np.abs(q.T @ q - np.eye(k)).max() <= tol * max(m, n)
+        assert np.array_equal(r, np.triu(r))
+        q_ref, r_ref = O.qr(a)
+        assert np.abs(np.abs(np.diag(r)) - np.abs(np.diag(r_ref))).max() <= tol * max(m, n)
+        u, sv, vt = chx.svd(chx.array(a), full_matrices=False)
+        u, sv, vt = u.get().astype(np.float64), sv.get(), vt.get().astype(np.float64)
+        assert np.abs(sv - O.svd(a, compute_uv=False)).max() <= tol * max(m, n) * 4
+        assert np.abs((u * sv) @ vt - a).max() <= tol * max(m, n) * 4
+        assert np.abs(u.T @ u - np.eye(k)).max() <= tol * max(m, n) * 4 and np.abs(vt @ vt.T - np.eye(k)).max() <= tol * max(m, n) * 4
+
+
 def test_one_workgroup_limits():
     """Matrices beyond what the one-workgroup kernels take are refused before anything is launched."""
     import chainer_amd as chx
