@@ -690,34 +690,75 @@ __global__ __launch_bounds__(256) void EighNormsKernel(const T* s, int n, T* par
     }
 }
 
-// First half of a round of the two-sided Jacobi sweeps of JacobiEighKernel below, spread over workgroups: one wavefront per pair
-// (p, q) of the round computes the rotation that annihilates s[p][q], leaves (cosine, sine) in cs[2 idx ..] and applies it from
-// the left: rows p and q of s, and rows p and q of vt (the accumulated rotations, transposed: row i is eigenvector i).
+// The rotations of `round` from the right, applied to one row of s held in LDS (entries p and q of every pair of that round); the
+// entry a rotation annihilates is stored as an exact zero (see JacobiEighKernel).  r is the row's index; the `lanes` threads that
+// share the row each take every lanes-th pair.
 template <typename T>
-__global__ __launch_bounds__(256) void EighRowsKernel(T* s, T* vt, int n, int round, int compute_v, T* cs) {
-    const int lane = threadIdx.x & 63;
-    const int idx = static_cast<int>(blockIdx.x) * 4 + static_cast<int>(threadIdx.x >> 6);
-    if (idx >= (n + 1) / 2) return;  // whole wavefronts
+__device__ __forceinline__ void EighRotateRowEntries(T* row, int r, int n, int round, const T* cs, int lane, int lanes) {
+    for (int idx = lane; idx < (n + 1) / 2; idx += lanes) {
+        int p, q;
+        JacobiPair(idx, round, n, p, q);
+        if (q < 0) continue;
+        const T c = cs[2 * idx], sn = cs[2 * idx + 1];
+        if (sn == T(0)) continue;
+        const T a = row[p], b = row[q];
+        row[p] = r == q ? T(0) : c * a - sn * b;
+        row[q] = r == p ? T(0) : sn * a + c * b;
+    }
+}
+
+// A round of the two-sided Jacobi sweeps of JacobiEighKernel below, spread over workgroups, one per pair (p, q).
+// Rotations from the left change rows p and q; rotations from the right change columns, but every row can apply them to itself
+// once the round's (cosine, sine) pairs are known.  So a workgroup takes rows p and q of s into LDS, first applies the previous
+// round's rotations from the right to them (prev_round >= 0, from cs_prev), then has everything it needs for its own rotation
+// (s[p][p], s[q][q], s[p][q] lie in these rows): it leaves (cosine, sine) in cs_next[2 idx ..] and applies the rotation from the
+// left to the two rows of s and of vt (the accumulated rotations, transposed: row i is eigenvector i).  The rotations of the last
+// round from the right are EighColumnsKernel's.
+template <typename T>
+__global__ __launch_bounds__(256) void EighRoundKernel(T* s, T* vt, int n, int prev_round, int round, int compute_v, const T* cs_prev, T* cs_next) {
+    extern __shared__ __align__(16) char eigh_round_lds[];
+    T* row_p = reinterpret_cast<T*>(eigh_round_lds);
+    T* row_q = row_p + n;
+    const int lane = threadIdx.x;
+    constexpr int kLanes = 256;
+    const int idx = static_cast<int>(blockIdx.x);
     int p, q;
-    JacobiPair(idx, round, n, p, q);
+    JacobiPair(idx, round, n, p, q);  // q = -1: p sits out this round, but still owes the previous round's rotations
+    T* sp = s + static_cast<int64_t>(p) * n;
+    T* sq = s + static_cast<int64_t>(q < 0 ? p : q) * n;
+    for (int i = lane; i < n; i += kLanes) {
+        row_p[i] = sp[i];
+        if (q >= 0) row_q[i] = sq[i];
+    }
+    __syncthreads();
+    if (prev_round >= 0) {
+        EighRotateRowEntries(row_p, p, n, prev_round, cs_prev, lane, kLanes);
+        if (q >= 0) EighRotateRowEntries(row_q, q, n, prev_round, cs_prev, lane, kLanes);
+        __syncthreads();
+    }
     T c = T(1), sn = T(0);
     if (q >= 0) {
-        const T apq = s[static_cast<int64_t>(p) * n + q];
+        const T apq = row_p[q];
         if (apq != T(0)) {
-            const T app = s[static_cast<int64_t>(p) * n + p], aqq = s[static_cast<int64_t>(q) * n + q];
+            const T app = row_p[p], aqq = row_q[q];
             const T tau = (aqq - app) / (T(2) * apq);
             const T tt = (tau >= T(0) ? T(1) : T(-1)) / ((tau >= T(0) ? tau : -tau) + SqrtT(T(1) + tau * tau));
             c = T(1) / SqrtT(T(1) + tt * tt);
             sn = tt * c;
         }
     }
-    if (lane == 0) cs[2 * idx] = c, cs[2 * idx + 1] = sn;
-    if (sn == T(0)) return;  // the same in every lane
-    T* sp = s + static_cast<int64_t>(p) * n;
-    T* sq = s + static_cast<int64_t>(q) * n;
-#pragma unroll 4
-    for (int i = lane; i < n; i += 64) {
-        const T a = sp[i], b = sq[i];
+    if (lane == 0) cs_next[2 * idx] = c, cs_next[2 * idx + 1] = sn;
+    if (sn == T(0)) {  // the same in every thread
+        if (prev_round >= 0) {
+            for (int i = lane; i < n; i += kLanes) {
+                sp[i] = row_p[i];
+                if (q >= 0) sq[i] = row_q[i];
+            }
+        }
+        return;
+    }
+    for (int i = lane; i < n; i += kLanes) {
+        const T a = row_p[i], b = row_q[i];
         sp[i] = c * a - sn * b;
         sq[i] = sn * a + c * b;
     }
@@ -725,7 +766,7 @@ __global__ __launch_bounds__(256) void EighRowsKernel(T* s, T* vt, int n, int ro
         T* vp = vt + static_cast<int64_t>(p) * n;
         T* vq = vt + static_cast<int64_t>(q) * n;
 #pragma unroll 4
-        for (int i = lane; i < n; i += 64) {
+        for (int i = lane; i < n; i += kLanes) {
             const T a = vp[i], b = vq[i];
             vp[i] = c * a - sn * b;
             vq[i] = sn * a + c * b;
@@ -733,32 +774,21 @@ __global__ __launch_bounds__(256) void EighRowsKernel(T* s, T* vt, int n, int ro
     }
 }
 
-// Second half of the round: the same rotations from the right.  Columns p and q of s change, but a workgroup walks rows: each of
-// its four wavefronts takes one row of s into LDS, rotates the entries (p, q) of every pair there and writes the row back.  The
-// entry a rotation annihilates is stored as an exact zero (see JacobiEighKernel).
+// The rotations of `round` from the right for the whole matrix (after the last round of a sweep): each of a workgroup's
+// wavefronts (up to four: as many rows as fit in 64 KiB of LDS) takes one row of s into LDS, rotates the entries (p, q) of every
+// pair there and writes the row back.
 template <typename T>
 __global__ __launch_bounds__(256) void EighColumnsKernel(T* s, int n, int round, const T* cs) {
     extern __shared__ __align__(16) char eigh_rows_lds[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     T* row = reinterpret_cast<T*>(eigh_rows_lds) + static_cast<int64_t>(wave) * n;
-    const int r = static_cast<int>(blockIdx.x) * 4 + wave;
+    const int r = static_cast<int>(blockIdx.x * (blockDim.x >> 6)) + wave;
     const bool valid = r < n;
     if (valid) {
         for (int i = lane; i < n; i += 64) row[i] = s[static_cast<int64_t>(r) * n + i];
     }
     __syncthreads();
-    if (valid) {
-        for (int idx = lane; idx < (n + 1) / 2; idx += 64) {
-            int p, q;
-            JacobiPair(idx, round, n, p, q);
-            if (q < 0) continue;
-            const T c = cs[2 * idx], sn = cs[2 * idx + 1];
-            if (sn == T(0)) continue;
-            const T a = row[p], b = row[q];
-            row[p] = r == q ? T(0) : c * a - sn * b;
-            row[q] = r == p ? T(0) : sn * a + c * b;
-        }
-    }
+    if (valid) EighRotateRowEntries(row, r, n, round, cs, lane, 64);
     __syncthreads();
     if (valid) {
         for (int i = lane; i < n; i += 64) s[static_cast<int64_t>(r) * n + i] = row[i];
@@ -1157,17 +1187,18 @@ __device__ __forceinline__ T SvdTolerance(int M) {
     return SqrtT(static_cast<T>(M)) * (std::is_same<T, float>::value ? T(1.2e-7) : T(2.3e-16));
 }
 
-// One wavefront makes the columns p and q of g orthogonal (one-sided Jacobi, Hestenes) and applies the same rotation to v.  Columns
-// are contiguous in memory (g: [N][M], v: [N][N], both column by column), so the wavefront streams its two columns: three dot
-// products, a butterfly reduction that leaves the sums in every lane, the rotation, and the same two columns of g and v again.
-// Returns whether the pair needed a rotation (the same in every lane).
-template <typename T>
-__device__ __forceinline__ bool SvdRotatePair(T* g, int M, int N, T* v, int p, int q, int compute_uv, int lane) {
+// WAVES wavefronts (one, or a whole workgroup of four with `sums` in LDS) make the columns p and q of g orthogonal (one-sided
+// Jacobi, Hestenes) and apply the same rotation to v.  Columns are contiguous in memory (g: [N][M], v: [N][N], both column by
+// column), so the threads stream the two columns: three dot products, a butterfly reduction that leaves the sums in every lane,
+// the rotation, and the same two columns of g and v again.  Returns whether the pair needed a rotation (the same in every thread).
+template <int WAVES, typename T>
+__device__ __forceinline__ bool SvdRotatePair(T* g, int M, int N, T* v, int p, int q, int compute_uv, int lane, T (*sums)[3]) {
+    constexpr int kLanes = 64 * WAVES;
     T* gp = g + static_cast<int64_t>(p) * M;
     T* gq = g + static_cast<int64_t>(q) * M;
     T alpha = T(0), beta = T(0), gamma = T(0);
 #pragma unroll 4
-    for (int i = lane; i < M; i += 64) {
+    for (int i = lane; i < M; i += kLanes) {
         const T a = gp[i], b = gq[i];
         alpha += a * a, beta += b * b, gamma += a * b;
     }
@@ -1177,6 +1208,13 @@ __device__ __forceinline__ bool SvdRotatePair(T* g, int M, int N, T* v, int p, i
         beta += __shfl_xor(beta, o);
         gamma += __shfl_xor(gamma, o);
     }
+    if constexpr (WAVES > 1) {  // the wavefronts' sums meet in LDS; every thread adds them in the same order
+        if ((lane & 63) == 0) sums[lane >> 6][0] = alpha, sums[lane >> 6][1] = beta, sums[lane >> 6][2] = gamma;
+        __syncthreads();
+        alpha = beta = gamma = T(0);
+#pragma unroll
+        for (int w2 = 0; w2 < WAVES; ++w2) alpha += sums[w2][0], beta += sums[w2][1], gamma += sums[w2][2];
+    }
     const T abs_gamma = gamma >= T(0) ? gamma : -gamma;
     if (!(abs_gamma > SvdTolerance<T>(M) * SqrtT(alpha * beta) && abs_gamma > T(0))) return false;
     const T zeta = (beta - alpha) / (T(2) * gamma);
@@ -1184,7 +1222,7 @@ __device__ __forceinline__ bool SvdRotatePair(T* g, int M, int N, T* v, int p, i
     const T c = T(1) / SqrtT(T(1) + tt * tt);
     const T sn = c * tt;
 #pragma unroll 4
-    for (int i = lane; i < M; i += 64) {
+    for (int i = lane; i < M; i += kLanes) {
         const T a = gp[i], b = gq[i];
         gp[i] = c * a - sn * b;
         gq[i] = sn * a + c * b;
@@ -1193,7 +1231,7 @@ __device__ __forceinline__ bool SvdRotatePair(T* g, int M, int N, T* v, int p, i
         T* vp = v + static_cast<int64_t>(p) * N;
         T* vq = v + static_cast<int64_t>(q) * N;
 #pragma unroll 4
-        for (int i = lane; i < N; i += 64) {
+        for (int i = lane; i < N; i += kLanes) {
             const T a = vp[i], b = vq[i];
             vp[i] = c * a - sn * b;
             vq[i] = sn * a + c * b;
@@ -1202,17 +1240,15 @@ __device__ __forceinline__ bool SvdRotatePair(T* g, int M, int N, T* v, int p, i
     return true;
 }
 
-// One round of the one-sided Jacobi sweeps of JacobiSvdKernel below, spread over workgroups: the round's disjoint column pairs go
-// one to a wavefront.  *rotated becomes 1 when any pair of the sweep needed a rotation.
+// One round of the one-sided Jacobi sweeps of JacobiSvdKernel below, spread over workgroups: one per disjoint column pair of the
+// round.  *rotated becomes 1 when any pair of the sweep needed a rotation.
 template <typename T>
 __global__ __launch_bounds__(256) void SvdRoundKernel(T* g, int M, int N, T* v, int round, int compute_uv, int* rotated) {
-    const int lane = threadIdx.x & 63;
-    const int idx = static_cast<int>(blockIdx.x) * 4 + static_cast<int>(threadIdx.x >> 6);
-    if (idx >= (N + 1) / 2) return;  // whole wavefronts
+    __shared__ T sums[4][3];
     int p, q;
-    JacobiPair(idx, round, N, p, q);
+    JacobiPair(static_cast<int>(blockIdx.x), round, N, p, q);
     if (q < 0) return;
-    if (SvdRotatePair(g, M, N, v, p, q, compute_uv, lane) && lane == 0) *rotated = 1;  // every writer stores the same value
+    if (SvdRotatePair<4>(g, M, N, v, p, q, compute_uv, static_cast<int>(threadIdx.x), sums) && threadIdx.x == 0) *rotated = 1;
 }
 
 // Singular value decomposition by one-sided Jacobi rotations (Hestenes), one workgroup.  g: the [M, N] matrix (M >= N) stored column
@@ -1243,7 +1279,7 @@ __global__ __launch_bounds__(kLinalgThreads) void JacobiSvdKernel(T* g, int M, i
             for (int idx = tid >> 6; idx < half; idx += kGroups) {  // a pair per wavefront
                 int p, q;
                 JacobiPair(idx, round, N, p, q);
-                if (q >= 0 && SvdRotatePair(g, M, N, v, p, q, compute_uv, tid & 63)) rotated = 1;  // every writer stores the same value
+                if (q >= 0 && SvdRotatePair<1>(g, M, N, v, p, q, compute_uv, tid & 63, static_cast<T(*)[3]>(nullptr))) rotated = 1;  // every writer stores the same value
             }
             __syncthreads();  // the pairs of a round are disjoint; the next round pairs the columns anew
         }
@@ -1538,8 +1574,8 @@ int hipcx_cholesky(const hipcx_array* a, const hipcx_array* out, int32_t* error_
 
 size_t hipcx_syevd_workspace_size(const hipcx_array* a) {
     if (a == nullptr || a->ndim != 2 || a->shape[0] < 0) return 0;
-    // the working copy and the rotations; a round's (cosine, sine) pairs and the partial norms of a sweep
-    return static_cast<size_t>(a->shape[0]) * static_cast<size_t>(a->shape[0]) * 8 * 2 + (static_cast<size_t>(a->shape[0]) + 2 + 2 * kEighNormBlocks) * 8;
+    // the working copy and the rotations; the (cosine, sine) pairs of two rounds and the partial norms of a sweep
+    return static_cast<size_t>(a->shape[0]) * static_cast<size_t>(a->shape[0]) * 8 * 2 + (2 * static_cast<size_t>(a->shape[0]) + 4 + 2 * kEighNormBlocks) * 8;
 }
 
 int hipcx_syevd(const hipcx_array* a, const hipcx_array* w, const hipcx_array* v, char uplo, int compute_v, void* workspace,
@@ -1572,13 +1608,14 @@ int hipcx_syevd(const hipcx_array* a, const hipcx_array* w, const hipcx_array* v
                                a->strides[1] / it, s, static_cast<int>(n), upper);
             const bool spread = n > kEighOneWorkgroupMaxN;
             if (spread) {
-                // the sweeps as two launches per round over many workgroups; before every sweep the host reads how much is left
-                // off the diagonal
-                T* cs = reinterpret_cast<T*>(ws + 2 * n * n * it);
-                T* partial = cs + 2 * ((n + 1) / 2);
+                // the sweeps as one launch per round over many workgroups (and one more per sweep for the last round's rotations
+                // from the right); before every sweep the host reads how much is left off the diagonal
+                const int64_t half = (n + 1) / 2;
+                T* cs = reinterpret_cast<T*>(ws + 2 * n * n * it);  // two sets of (cosine, sine) pairs, used in turn
+                T* partial = cs + 4 * half;
                 std::vector<T> sums(2 * kEighNormBlocks);
                 if (compute_v) hipLaunchKernelGGL(IdentityFillKernel<T>, dim3(blocks), dim3(256), 0, st, vs, static_cast<int>(n));
-                const unsigned pair_blocks = static_cast<unsigned>(((n + 1) / 2 + 3) / 4), row_blocks = static_cast<unsigned>((n + 3) / 4);
+                const int64_t rows_per_block = std::max<int64_t>(1, std::min<int64_t>(4, 65536 / (n * it)));
                 const double eps = std::is_same<T, float>::value ? 4e-7 : 1e-15;  // as in JacobiEighKernel
                 double total_norm = 0.0;
                 for (int sweep = 0; sweep < kEighMaxSweeps; ++sweep) {
@@ -1591,10 +1628,13 @@ int hipcx_syevd(const hipcx_array* a, const hipcx_array* w, const hipcx_array* v
                     if (!(off > eps * eps * total_norm)) break;
                     const int rounds = static_cast<int>(n + (n & 1)) - 1;
                     for (int round = 0; round < rounds; ++round) {
-                        hipLaunchKernelGGL(EighRowsKernel<T>, dim3(pair_blocks), dim3(256), 0, st, s, vs, static_cast<int>(n), round, compute_v ? 1 : 0, cs);
-                        hipLaunchKernelGGL(EighColumnsKernel<T>, dim3(row_blocks), dim3(256), static_cast<size_t>(4 * n * it), st, s,
-                                           static_cast<int>(n), round, cs);
+                        hipLaunchKernelGGL(EighRoundKernel<T>, dim3(static_cast<unsigned>(half)), dim3(256), static_cast<size_t>(2 * n * it), st, s, vs,
+                                           static_cast<int>(n), round - 1, round, compute_v ? 1 : 0, cs + ((round + 1) & 1) * 2 * half,
+                                           cs + (round & 1) * 2 * half);
                     }
+                    hipLaunchKernelGGL(EighColumnsKernel<T>, dim3(static_cast<unsigned>((n + rows_per_block - 1) / rows_per_block)),
+                                       dim3(static_cast<unsigned>(64 * rows_per_block)), static_cast<size_t>(rows_per_block * n * it), st, s,
+                                       static_cast<int>(n), rounds - 1, cs + ((rounds - 1) & 1) * 2 * half);
                 }
             }
             hipLaunchKernelGGL(JacobiEighKernel<T>, dim3(1), dim3(kLinalgThreads), lds, st, s, static_cast<T*>(v->data),
@@ -1797,7 +1837,7 @@ int hipcx_svd(const hipcx_array* a, const hipcx_array* u, const hipcx_array* s, 
                                        reinterpret_cast<T*>(v_mem), static_cast<int>(N));
                 }
                 const int np = static_cast<int>(N + (N & 1));
-                const unsigned blocks = static_cast<unsigned>((np / 2 + 3) / 4);
+                const unsigned blocks = static_cast<unsigned>(np / 2);
                 for (int sweep = 0; sweep < kSvdMaxSweeps; ++sweep) {
                     for (int round = 0; round < np - 1; ++round) {
                         hipLaunchKernelGGL(SvdRoundKernel<T>, dim3(blocks), dim3(256), 0, st, reinterpret_cast<T*>(g_mem), static_cast<int>(M),
