@@ -274,8 +274,8 @@ def section_lstm(chx, oracle, with_cpu):
 def section_backward(chx, oracle, with_cpu):
     """Backward / training kernels at ResNet-50 layer shapes (float16, batch 32).  The convolution gradients are compositions of
     the forward kernels (Im2Col / Col2Im copies plus one matrix product) -- functional, not tuned; batch normalisation, its
-    gradient and the pooling gradients have kernels of their own.  Timed as HIP-graph replays (a composition is 10-25
-    kernel launches; issued eagerly from Python it would be host-bound)."""
+    gradient and the pooling gradients have kernels of their own.  Timed as bursts of ten calls in one HIP-graph replay (issued
+    eagerly from Python the short ones would be host-bound, and a graph of a single kernel measures the replay's own latency)."""
     rng = np.random.default_rng(6)
     n, c, k, hw = 32, 256, 256, 14
     x = chx.array(rng.standard_normal((n, c, hw, hw)).astype(np.float16))
@@ -285,7 +285,7 @@ def section_backward(chx, oracle, with_cpu):
     for name, fn in (('conv_grad_weight 3x3', lambda: chx.conv_grad_weight('float16', w.shape, x, gy, 1, 1)),
                      ('conv_transpose 3x3', lambda: chx.conv_transpose(gy, w, None, 1, 1, (hw, hw))),
                      ('conv 3x3 (forward, for scale)', lambda: chx.conv(x, w, None, 1, 1))):
-        t = graph_time(fn, 5)
+        t = op_time(fn)
         emit(section='backward', op=name, shape=[n, c, hw, hw, k], us=round(t * 1e6, 1), TFLOPs=round(flops / t / 1e12, 2),
              fp16_mfma_frac=round(flops / t / 1e12 / MFMA_PEAK['float16'], 4))
     shape = (32, 256, 56, 56)
@@ -296,21 +296,21 @@ def section_backward(chx, oracle, with_cpu):
     nbytes = xb.nbytes
     out_state = []
     out_state[:] = [chx.batch_norm(xb, prm[0], prm[1], rm, rv)]
-    t = graph_time(lambda: chx.batch_norm(xb, prm[0], prm[1], rm, rv), 5)
+    t = op_time(lambda: chx.batch_norm(xb, prm[0], prm[1], rm, rv))
     bw_row('backward', 'batch_norm (training forward)', shape, t, 4 * nbytes, 5,
            note='algorithmic bytes: three reads (sum, centred sum of squares, normalise) and one write')
     state = out_state[0][1]
-    t = graph_time(lambda: chx.batch_norm_grad(xb, prm[0], gb, state), 5)
+    t = op_time(lambda: chx.batch_norm_grad(xb, prm[0], gb, state))
     bw_row('backward', 'batch_norm_grad', shape, t, 5 * nbytes, 3,
            note='algorithmic bytes: x and gout read twice, gx written')
     xp = chx.array(rng.standard_normal((32, 64, 112, 112)).astype(np.float16))
     gp = chx.array(rng.standard_normal((32, 64, 56, 56)).astype(np.float16))
-    t = graph_time(lambda: chx.max_pool_grad(xp, gp, 3, 2, 1), 5)
+    t = op_time(lambda: chx.max_pool_grad(xp, gp, 3, 2, 1))
     bw_row('backward', 'max_pool_grad 3x3/2 pad 1', (32, 64, 112, 112), t, 2 * xp.nbytes + gp.nbytes, 2,
            note='window ArgMax kernel + gather kernel; bits of the Im2Col / ArgMax / Col2Im composition')
     xa = chx.array(rng.standard_normal((128, 2048, 7, 7)).astype(np.float16))
     ga = chx.array(rng.standard_normal((128, 2048, 1, 1)).astype(np.float16))
-    t = graph_time(lambda: chx.average_pool_grad(xa, ga, 7, 1, 0, 'zero'), 5)
+    t = op_time(lambda: chx.average_pool_grad(xa, ga, 7, 1, 0, 'zero'))
     bw_row('backward', 'average_pool_grad 7x7 (global)', (128, 2048, 7, 7), t, xa.nbytes + ga.nbytes)
 
 

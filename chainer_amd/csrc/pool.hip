@@ -650,6 +650,71 @@ PoolGradArgs MakeGradArgs(const hipcx_array* x, const hipcx_array* gout, const i
     return p;
 }
 
+// AveragePoolGrad of a window that is the whole, unpadded plane: every position of plane (n, c) receives the one gradient of that
+// plane divided by the window size, with PoolGradKernel's roundings (the quotient in T, added to a zero of T).  gx is dense NCHW;
+// a thread writes 16 bytes, which may run over into the following planes.
+template <typename T, typename IdxT>
+__global__ __launch_bounds__(256) void GlobalAvgPoolGradKernel(PoolGradArgs p, IdxT total) {
+    using C = compute_t<T>;
+    constexpr int V = 16 / sizeof(T);
+    const T* gout = static_cast<const T*>(p.gout);
+    T* gx = static_cast<T*>(p.gx);
+    const IdxT hw = static_cast<IdxT>(p.H * p.W);
+    const bool dense_gout = p.gsC == 1 && p.gsN == p.C;  // one gradient per plane, in plane order
+    auto plane_value = [&](IdxT plane) {
+        int64_t at = static_cast<int64_t>(plane);
+        if (!dense_gout) {
+            const IdxT n = plane / static_cast<IdxT>(p.C);
+            at = static_cast<int64_t>(n) * p.gsN + static_cast<int64_t>(plane - n * static_cast<IdxT>(p.C)) * p.gsC;
+        }
+        T g = gout[at];
+        if (p.pad_mode == HIPCX_PAD_IGNORE) {
+            const T width = static_cast<T>(static_cast<C>(static_cast<T>(static_cast<C>(p.H))) * static_cast<C>(static_cast<T>(static_cast<C>(p.W))));
+            g = static_cast<T>(static_cast<C>(g) / static_cast<C>(width));
+        }
+        T acc = static_cast<T>(static_cast<C>(T(0)) + static_cast<C>(g));
+        if (p.pad_mode == HIPCX_PAD_ZERO) acc = static_cast<T>(static_cast<C>(acc) / static_cast<C>(static_cast<T>(static_cast<C>(p.kh * p.kw))));
+        return acc;
+    };
+    const IdxT e0 = (static_cast<IdxT>(blockIdx.x) * 256 + threadIdx.x) * V;
+    if (e0 >= total) return;
+    IdxT plane = e0 / hw;
+    IdxT rem = e0 - plane * hw;
+    T value = plane_value(plane);
+    if (hw >= static_cast<IdxT>(V) && e0 + V <= total) {
+        // at most one plane boundary inside the 16 bytes: both values are fetched up front, and the vector is put together in
+        // registers (sizeof(T)-sized lanes of four dwords)
+        const bool crosses = rem + V > hw;
+        const T later = crosses ? plane_value(plane + 1) : value;
+        using Bits = std::conditional_t<sizeof(T) == 2, uint16_t, std::conditional_t<sizeof(T) == 4, uint32_t, uint64_t>>;
+        const uint64_t first = __builtin_bit_cast(Bits, value), second = __builtin_bit_cast(Bits, later);
+        PVec<unsigned, 4> out;
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            uint64_t word = 0;  // the elements that overlap dword d (for 8-byte elements: one half of an element)
+            if constexpr (sizeof(T) == 8) {
+                const uint64_t e = rem + d / 2 < hw ? first : second;
+                word = (d & 1) ? e >> 32 : e & 0xffffffffu;
+            } else {
+                constexpr int per = 4 / sizeof(T);
+#pragma unroll
+                for (int k = 0; k < per; ++k) word |= (rem + d * per + k < hw ? first : second) << (8 * sizeof(T) * k);
+            }
+            out.v[d] = static_cast<unsigned>(word);
+        }
+        *reinterpret_cast<PVec<unsigned, 4>*>(gx + e0) = out;
+        return;
+    }
+    for (int k = 0; k < V && e0 + k < total; ++k) {
+        if (rem == hw) {
+            rem = 0;
+            value = plane_value(++plane);
+        }
+        gx[e0 + k] = value;
+        ++rem;
+    }
+}
+
 template <typename T, bool IS_MAX>
 void RunPoolGrad(const PoolGradArgs& p, hipStream_t stream) {
     const int64_t total = static_cast<int64_t>(p.N) * p.C * p.H * p.W;
@@ -666,6 +731,22 @@ void RunPoolGrad(const PoolGradArgs& p, hipStream_t stream) {
                 hipLaunchKernelGGL((WindowArgMaxKernel<T, int64_t>), grid_for(windows), dim3(256), 0, stream, p, windows);
             }
             CheckLaunch("window_argmax");
+        }
+    }
+    if constexpr (!IS_MAX) {
+        const bool whole_plane = p.OH == 1 && p.OW == 1 && p.kh == p.H && p.kw == p.W && p.ph == 0 && p.pw == 0;
+        const bool dense = p.dsW == 1 && p.dsH == p.W && p.dsC == static_cast<int64_t>(p.H) * p.W && p.dsN == p.dsC * p.C;
+        if (whole_plane && dense && reinterpret_cast<uintptr_t>(p.gx) % 16 == 0) {
+            constexpr int V = 16 / sizeof(T);
+            const int64_t threads = (total + V - 1) / V;
+            const dim3 blocks(static_cast<unsigned>((threads + 255) / 256));
+            if (total + 16 < (1LL << 31)) {
+                hipLaunchKernelGGL((GlobalAvgPoolGradKernel<T, unsigned>), blocks, dim3(256), 0, stream, p, static_cast<unsigned>(total));
+            } else {
+                hipLaunchKernelGGL((GlobalAvgPoolGradKernel<T, int64_t>), blocks, dim3(256), 0, stream, p, total);
+            }
+            CheckLaunch("pool_grad");
+            return;
         }
     }
     const bool small = p.kh <= 2 * p.sh && p.kw <= 2 * p.sw && p.OH > 0 && p.OW > 0;

@@ -177,7 +177,9 @@ def test_pool_gradient_kernels_have_the_bits_of_the_composition(dt):
     from chainer_amd import routines
     rng = np.random.default_rng(61)
     cases = POOL_CASES + [((2, 3, 20, 20), 7, 3, 3, False), ((1, 2, 15, 15), 7, 1, 0, False), ((2, 4, 9, 11), (3, 2), (1, 2), (1, 0), True),
-                          ((3, 5, 12, 12), 3, 2, 1, False), ((2, 8, 56, 56), 3, 2, 1, False)]
+                          ((3, 5, 12, 12), 3, 2, 1, False), ((2, 8, 56, 56), 3, 2, 1, False),
+                          # windows that are the whole plane (the global pooling of a classifier head): planes of 49, 30 and 9 elements
+                          ((3, 5, 7, 7), 7, 1, 0, False), ((2, 3, 6, 5), (6, 5), 1, 0, False), ((1, 1, 3, 3), 3, 3, 0, False)]
     for (shape, k, s, p, cv) in cases:
         x = rng.integers(-3, 4, shape).astype(dt)
         if np.dtype(dt).kind == 'f':
