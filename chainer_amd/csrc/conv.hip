@@ -527,9 +527,9 @@ NchwPlan PlanNchw(const hipcx_array* x, const hipcx_array* w, const hipcx_array*
     return pl;
 }
 
-template <int TAPS, int WPX, int WCH, int CK, int NPX, int MAXI, int KSPLIT = 1>
+template <int TAPS, int WPX, int WCH, int CK, int NPX, int MAXI, int KSPLIT = 1, bool PAIR = false>
 void LaunchNchwKernel(const NchwConvArgs& a, int lds_bytes, hipStream_t stream) {
-    auto kern = NchwConvKernel<TAPS, WPX, WCH, CK, NPX, MAXI, KSPLIT>;
+    auto kern = NchwConvKernel<TAPS, WPX, WCH, CK, NPX, MAXI, KSPLIT, PAIR>;
     struct Tag {};  // a type of its own for every instantiation of this launcher
     EnsureDynamicLds<Tag>(reinterpret_cast<const void*>(kern), lds_bytes);
     int64_t total = static_cast<int64_t>(a.tiles_m) * a.tiles_n;
@@ -592,7 +592,8 @@ void RunNchw(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, c
         a.div_wchunks = FastDiv(a.W / pl.npx);
         a.div_percg = FastDiv(pl.nrow * (a.W / pl.npx));
     }
-    a.pair_load = (pl.taps == 1 && pl.npx == 1 && a.stride == 2 && a.W % 2 == 0) ? 1 : 0;
+    // single-pixel loads of a stride-2 layer over an even width fetch whole dwords (the wanted pixel and its odd neighbour)
+    const bool pair_load = pl.taps == 1 && pl.npx == 1 && a.stride == 2 && a.W % 2 == 0;
     a.out_ev = a.P % 8 == 0 ? 8 : a.P % 4 == 0 ? 4 : a.P % 2 == 0 ? 2 : 1;
     const bool w_dense = w->strides[1] == 2 && w->strides[0] == static_cast<int64_t>(a.C) * 2 && reinterpret_cast<uintptr_t>(w->data) % 16 == 0;
     static const bool direct_ok = [] { const char* e = getenv("HIPCX_W_DIRECT"); return e == nullptr || e[0] != '0'; }();
@@ -611,8 +612,16 @@ void RunNchw(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, c
     double bytes = 2.0 * (static_cast<double>(a.N) * a.C * a.H * a.W + static_cast<double>(a.K) * RS * a.C + static_cast<double>(a.M) * a.K);
     ProfileScope prof(stream, flops, bytes);
     const int key = (pl.ksplit - 1) * 1000000 + (pl.ck / 16) * 100000 + pl.taps * 10000 + pl.wpx * 1000 + pl.wch * 100 + pl.npx * 10 + pl.maxi;
+    // single-pixel 1x1 kernels exist with and without dword loads
+#define HIPCX_NCHW_LAUNCH(TAPS, WPX, WCH, CK, NPX, MAXI, KSPLIT)                                          \
+    if constexpr (TAPS == 1 && NPX == 1) {                                                                \
+        if (pair_load) LaunchNchwKernel<TAPS, WPX, WCH, CK, NPX, MAXI, KSPLIT, true>(a, pl.lds_bytes, stream); \
+        else LaunchNchwKernel<TAPS, WPX, WCH, CK, NPX, MAXI, KSPLIT, false>(a, pl.lds_bytes, stream);     \
+    } else {                                                                                              \
+        LaunchNchwKernel<TAPS, WPX, WCH, CK, NPX, MAXI, KSPLIT>(a, pl.lds_bytes, stream);                 \
+    }
 #define HIPCX_NCHW_CASE(TAPS, WPX, WCH, CK, NPX, MAXI) \
-    case (CK / 16) * 100000 + TAPS * 10000 + WPX * 1000 + WCH * 100 + NPX * 10 + MAXI: LaunchNchwKernel<TAPS, WPX, WCH, CK, NPX, MAXI>(a, pl.lds_bytes, stream); break;
+    case (CK / 16) * 100000 + TAPS * 10000 + WPX * 1000 + WCH * 100 + NPX * 10 + MAXI: { HIPCX_NCHW_LAUNCH(TAPS, WPX, WCH, CK, NPX, MAXI, 1) } break;
     switch (key) {
         HIPCX_NCHW_CASE(1, 4, 1, 32, 2, 2)
         HIPCX_NCHW_CASE(1, 4, 1, 32, 1, 4)
@@ -625,7 +634,7 @@ void RunNchw(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, c
         HIPCX_NCHW_CASE(9, 4, 1, 16, 1, 2)
         HIPCX_NCHW_CASE(9, 4, 1, 16, 1, 4)
 #define HIPCX_NCHW_SPLIT_CASE(TAPS, WPX, WCH, CK, NPX, MAXI) \
-    case 1000000 + (CK / 16) * 100000 + TAPS * 10000 + WPX * 1000 + WCH * 100 + NPX * 10 + MAXI: LaunchNchwKernel<TAPS, WPX, WCH, CK, NPX, MAXI, 2>(a, pl.lds_bytes, stream); break;
+    case 1000000 + (CK / 16) * 100000 + TAPS * 10000 + WPX * 1000 + WCH * 100 + NPX * 10 + MAXI: { HIPCX_NCHW_LAUNCH(TAPS, WPX, WCH, CK, NPX, MAXI, 2) } break;
         HIPCX_NCHW_SPLIT_CASE(1, 2, 2, 32, 2, 1)
         HIPCX_NCHW_SPLIT_CASE(1, 2, 2, 32, 1, 2)
         HIPCX_NCHW_SPLIT_CASE(1, 1, 4, 32, 1, 1)
@@ -637,6 +646,7 @@ void RunNchw(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, c
         default: throw Error(HIPCX_CHAINERX_ERROR, "nchw conv: no kernel for plan " + std::to_string(key));
     }
 #undef HIPCX_NCHW_CASE
+#undef HIPCX_NCHW_LAUNCH
 }
 
 

@@ -62,7 +62,6 @@ struct NchwConvArgs {
     int nslot;  // slots per channel group in the LDS patch
     int64_t bias_stride;
     unsigned x_bytes, wp_bytes;
-    int pair_load;  // NPX == 1 only: every wanted pixel sits at an even element offset with a readable odd neighbour (stride 2, even W)
     int w_direct;  // 1x1 only: read the filter bank in place (a row's 8 consecutive channels are one 16-byte group already)
     // Optional fused tail (all null / 0 for a plain convolution): fixed batch normalisation over the output channels,
     // a residual addend of out's shape (dense NCHW) and ReLU.
@@ -163,7 +162,10 @@ __device__ __forceinline__ void StaticFor(F&& f) {
 // KSPLIT = 2: a second set of WPX * WCH waves works on the same tile and takes every other channel chunk through LDS stages of
 // its own; the two accumulator sets are added through LDS before the epilogue.  For grids with at most one tile per compute unit
 // (7x7 planes, small batches) this doubles the waves and the loads in flight per unit, which is what bounds those layers.
-template <int TAPS, int WPX, int WCH, int CK, int NPX, int MAXI, int KSPLIT = 1>
+// PAIR (single-pixel loads only): every wanted pixel sits at an even element offset with a readable odd neighbour (stride 2, even
+// width), so a pixel is fetched as a whole dword; a template parameter because a run-time choice would put a branch after every
+// load of the hand-scheduled loop.
+template <int TAPS, int WPX, int WCH, int CK, int NPX, int MAXI, int KSPLIT = 1, bool PAIR = false>
 // Eight-wave workgroups that do not split the reduction are meant to run two to a compute unit (four waves per SIMD): they
 // are kept within 128 registers.
 __global__ __launch_bounds__(64 * WPX * WCH * KSPLIT) __attribute__((amdgpu_waves_per_eu(WPX * WCH >= 8 && KSPLIT == 1 ? 4 : 1, 8)))
@@ -300,7 +302,7 @@ void NchwConvKernel(NchwConvArgs p) {
                 for (int e = 0; e < NPX; ++e) *reinterpret_cast<Bytes16*>(dst + e * 16) = t[e];
             } else {
                 constexpr int j = r - 1;
-                if (NPX == 1 && p.pair_load) {
+                if constexpr (NPX == 1 && PAIR) {
                     xreg[i][j].d[0] = __builtin_amdgcn_raw_buffer_load_b32(xr, xvoff[i], xs_next + j * HW * 2, 0);
                 } else {
                     xreg[i][j] = BufLoad<NPX>(xr, xvoff[i], xs_next + j * HW * 2);
