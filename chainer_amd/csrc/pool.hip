@@ -650,6 +650,160 @@ PoolGradArgs MakeGradArgs(const hipcx_array* x, const hipcx_array* gout, const i
     return p;
 }
 
+// ---- MaxPoolGrad of K x K windows (K = 2 or 3) at horizontal stride 2 with padding PW = 0 or 1 over dense NCHW planes whose
+// width W is a multiple of 8, OW = W / 2: the usual down-sampling pooling.  Two passes like the general path (the ArgMax of every
+// window, then a gather per input position), but a thread takes four neighbouring windows / eight neighbouring positions, so
+// that every input row is one aligned vector load plus at most one extra element instead of a load per tap. ----
+
+// ArgMax of N <= 32 values in the order of the native reduction loop (CX/native/reduce.h:46-83): groups of four, then the tail.
+template <int N, typename V>
+__device__ __forceinline__ int TreeArgMax(const V (&e)[N]) {
+    using B = WinBest<V>;
+    static_assert(N <= 32, "one block of the reduction tree");
+    B accum{V(0), -1};
+    constexpr int kMain = N - N % 4;
+#pragma unroll
+    for (int i = 0; i < kMain; i += 4) {
+        B p0{e[i], i};
+        WinReduce(B{e[i + 1], i + 1}, p0);
+        B p1{e[i + 2], i + 2};
+        WinReduce(B{e[i + 3], i + 3}, p1);
+        WinReduce(p1, p0);
+        WinReduce(p0, accum);
+    }
+#pragma unroll
+    for (int i = kMain; i < N; ++i) WinReduce(B{e[i], i}, accum);
+    return accum.i;
+}
+
+// win[((n * C + c) * OH + oh) * OW + ow] = ArgMax of the window, one byte each; a thread writes the four windows ow = 4 kk .. 4 kk + 3.
+template <typename T, int K, int PW>
+__global__ __launch_bounds__(256) void WindowArgMaxStride2Kernel(PoolGradArgs p, uint32_t* win, unsigned total) {
+    using V = std::conditional_t<std::is_same<T, half_t>::value, float, std::conditional_t<std::is_same<T, bool>::value, int, T>>;
+    const unsigned idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx >= total) return;
+    const unsigned quads = static_cast<unsigned>(p.OW) / 4;
+    unsigned t = idx;
+    const int kk = static_cast<int>(t % quads);
+    t /= quads;
+    const int oh = static_cast<int>(t % p.OH);
+    t /= p.OH;
+    const int c = static_cast<int>(t % p.C);
+    const int64_t n = t / p.C;
+    const T* xb = static_cast<const T*>(p.x) + n * p.xsN + static_cast<int64_t>(c) * p.xsC;
+    V e[4][K * K];
+#pragma unroll
+    for (int r = 0; r < K; ++r) {
+        const int ih = oh * p.sh - p.ph + r;
+        const bool row_ok = ih >= 0 && ih < p.H;
+        const T* row = xb + static_cast<int64_t>(row_ok ? ih : 0) * p.W + 8 * kk;
+        PVec<T, 8> vec = *reinterpret_cast<const PVec<T, 8>*>(row);
+        T left = Lowest<T>(), right = Lowest<T>();
+        if (PW == 1 && row_ok && kk > 0) left = row[-1];
+        if (PW == 0 && K == 3 && row_ok && 8 * kk + 8 < p.W) right = row[8];
+#pragma unroll
+        for (int w4 = 0; w4 < 4; ++w4) {
+#pragma unroll
+            for (int q = 0; q < K; ++q) {
+                const int col = 2 * w4 - PW + q;  // a constant after unrolling: -1 .. 8
+                T v = col < 0 ? left : (col > 7 ? right : vec.v[col < 0 ? 0 : (col > 7 ? 7 : col)]);
+                if (!row_ok) v = Lowest<T>();
+                e[w4][r * K + q] = static_cast<V>(v);
+            }
+        }
+    }
+    uint32_t packed = 0;
+#pragma unroll
+    for (int w4 = 0; w4 < 4; ++w4) packed |= static_cast<uint32_t>(TreeArgMax(e[w4])) << (8 * w4);
+    win[idx] = packed;
+}
+
+// gx over eight neighbouring positions w = 8 kk .. 8 kk + 7 of a row: the windows that cover them are two window rows at most
+// (K <= 2 * sh) times the five windows j = 4 kk - 1 + PW .. 4 kk + 3 + PW; their ArgMax bytes and gradients are loaded up front (an
+// aligned group of four plus one), and every position adds the gradients of the windows whose ArgMax it is, in the order of the
+// general kernel (window row descending, then window column descending).
+template <typename T, int K, int PW>
+__global__ __launch_bounds__(256) void MaxPoolGradStride2Kernel(PoolGradArgs p, const uint8_t* win, unsigned total) {
+    using C = compute_t<T>;
+    const unsigned idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx >= total) return;
+    const unsigned octets = static_cast<unsigned>(p.W) / 8;
+    unsigned t = idx;
+    const int kk = static_cast<int>(t % octets);
+    t /= octets;
+    const int h = static_cast<int>(t % p.H);
+    t /= p.H;
+    const int c = static_cast<int>(t % p.C);
+    const int64_t n = t / p.C;
+    const T* gb = static_cast<const T*>(p.gout) + n * p.gsN + static_cast<int64_t>(c) * p.gsC;
+    const uint8_t* wb = win + (n * p.C + c) * (static_cast<int64_t>(p.OH) * p.OW);
+    const int y = h + p.ph;
+    int i_hi = y / p.sh;
+    if (i_hi > p.OH - 1) i_hi = p.OH - 1;
+    // slot s of a window row holds window j = 4 kk - 1 + s, s = 0 .. 5
+    T g[2][6];
+    int ix[2][6];
+    bool row_ok[2];
+    int row_r[2];
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {
+        const int i = i_hi - a;
+        const int r = y - i * p.sh;
+        row_ok[a] = i >= 0 && r < K;
+        row_r[a] = r;
+        const int ic = row_ok[a] ? i : 0;
+        const T* grow = gb + static_cast<int64_t>(ic) * p.OW + 4 * kk;
+        const uint8_t* wrow = wb + static_cast<int64_t>(ic) * p.OW + 4 * kk;
+        const PVec<T, 4> g4 = *reinterpret_cast<const PVec<T, 4>*>(grow);
+        const uint32_t w4 = *reinterpret_cast<const uint32_t*>(wrow);
+#pragma unroll
+        for (int s = 0; s < 6; ++s) g[a][s] = T(0), ix[a][s] = -1;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) g[a][1 + s] = g4.v[s], ix[a][1 + s] = row_ok[a] ? static_cast<int>((w4 >> (8 * s)) & 0xffu) : -1;
+        if (PW == 0 && K == 3 && row_ok[a] && kk > 0) g[a][0] = grow[-1], ix[a][0] = wrow[-1];
+        if (PW == 1 && row_ok[a] && 4 * kk + 4 < p.OW) g[a][5] = grow[4], ix[a][5] = wrow[4];
+    }
+    PVec<T, 8> out;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        const int q_hi = (PW + k) & 1;
+        const int slot = ((PW + k) >> 1) + 1;  // of window j_hi = (8 kk + PW + k) / 2
+        T acc = T(0);
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+            if (ix[a][slot] == row_r[a] * K + q_hi) acc = static_cast<T>(static_cast<C>(acc) + static_cast<C>(g[a][slot]));
+            if (K == 3 && q_hi == 0 && ix[a][slot - 1] == row_r[a] * K + 2) acc = static_cast<T>(static_cast<C>(acc) + static_cast<C>(g[a][slot - 1]));
+        }
+        out.v[k] = acc;
+    }
+    T* dst = static_cast<T*>(p.gx) + n * p.dsN + static_cast<int64_t>(c) * p.dsC + static_cast<int64_t>(h) * p.W + 8 * kk;
+    *reinterpret_cast<PVec<T, 8>*>(dst) = out;
+}
+
+// Whether the two kernels above take this MaxPoolGrad.
+inline bool Stride2MaxPoolGradApplies(const PoolGradArgs& p, size_t item) {
+    // (2 x 2 windows with padding never give OW = W / 2)
+    const bool window = p.kh == p.kw && ((p.kh == 2 && p.pw == 0) || (p.kh == 3 && (p.pw == 0 || p.pw == 1))) && p.sw == 2 && p.kh <= 2 * p.sh;
+    const bool planes = p.W % 8 == 0 && p.OW * 2 == p.W && p.OH > 0;
+    const bool dense = p.xsW == 1 && p.xsH == p.W && p.dsW == 1 && p.dsH == p.W && p.gsW == 1 && p.gsH == p.OW && p.xsC % 8 == 0 &&
+                       p.xsN % 8 == 0 && p.dsC % 8 == 0 && p.dsN % 8 == 0 && p.gsC % 4 == 0 && p.gsN % 4 == 0;
+    const bool aligned = reinterpret_cast<uintptr_t>(p.x) % (8 * item) == 0 && reinterpret_cast<uintptr_t>(p.gx) % (8 * item) == 0 &&
+                         reinterpret_cast<uintptr_t>(p.gout) % (4 * item) == 0 && reinterpret_cast<uintptr_t>(p.win_index) % 4 == 0;
+    return window && planes && dense && aligned;
+}
+
+template <typename T, int K, int PW>
+void LaunchStride2MaxPoolGrad(const PoolGradArgs& p, hipStream_t stream) {
+    const unsigned quads = static_cast<unsigned>(static_cast<int64_t>(p.N) * p.C * p.OH * (p.OW / 4));
+    const unsigned octets = static_cast<unsigned>(static_cast<int64_t>(p.N) * p.C * p.H * (p.W / 8));
+    hipLaunchKernelGGL((WindowArgMaxStride2Kernel<T, K, PW>), dim3((quads + 255) / 256), dim3(256), 0, stream, p,
+                       reinterpret_cast<uint32_t*>(p.win_index), quads);
+    CheckLaunch("window_argmax");
+    hipLaunchKernelGGL((MaxPoolGradStride2Kernel<T, K, PW>), dim3((octets + 255) / 256), dim3(256), 0, stream, p,
+                       reinterpret_cast<const uint8_t*>(p.win_index), octets);
+    CheckLaunch("pool_grad");
+}
+
 // AveragePoolGrad of a window that is the whole, unpadded plane: every position of plane (n, c) receives the one gradient of that
 // plane divided by the window size, with PoolGradKernel's roundings (the quotient in T, added to a zero of T).  gx is dense NCHW;
 // a thread writes 16 bytes, which may run over into the following planes.
@@ -723,6 +877,14 @@ void RunPoolGrad(const PoolGradArgs& p, hipStream_t stream) {
     const int64_t cap = static_cast<int64_t>(NumCUs()) * 64;
     auto grid_for = [&](int64_t n) { int64_t b = (n + 255) / 256; return dim3(static_cast<unsigned>(b > cap ? cap : (b < 1 ? 1 : b))); };
     const bool narrow = total + cap * 256 < (1LL << 31) && windows + cap * 256 < (1LL << 31);  // 32-bit index arithmetic
+    if constexpr (IS_MAX && !std::is_same<T, bool>::value) {
+        if (narrow && windows > 0 && Stride2MaxPoolGradApplies(p, sizeof(T))) {
+            if (p.kh == 2) LaunchStride2MaxPoolGrad<T, 2, 0>(p, stream);
+            else if (p.pw == 0) LaunchStride2MaxPoolGrad<T, 3, 0>(p, stream);
+            else LaunchStride2MaxPoolGrad<T, 3, 1>(p, stream);
+            return;
+        }
+    }
     if constexpr (IS_MAX) {
         if (windows > 0) {
             if (narrow) {

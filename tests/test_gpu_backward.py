@@ -178,6 +178,10 @@ def test_pool_gradient_kernels_have_the_bits_of_the_composition(dt):
     rng = np.random.default_rng(61)
     cases = POOL_CASES + [((2, 3, 20, 20), 7, 3, 3, False), ((1, 2, 15, 15), 7, 1, 0, False), ((2, 4, 9, 11), (3, 2), (1, 2), (1, 0), True),
                           ((3, 5, 12, 12), 3, 2, 1, False), ((2, 8, 56, 56), 3, 2, 1, False),
+                          # stride-2 windows over planes whose width is a multiple of 8 with OW = W / 2 (vector kernels): 3x3 without
+                          # padding (cover_all), 2x2, a vertical stride of 3, several octets per row
+                          ((2, 3, 16, 16), 3, 2, 0, True), ((2, 3, 16, 24), 2, 2, 0, False), ((1, 2, 12, 16), 3, (3, 2), (1, 1), False),
+                          ((2, 2, 14, 40), 3, 2, 1, False),
                           # windows that are the whole plane (the global pooling of a classifier head): planes of 49, 30 and 9 elements
                           ((3, 5, 7, 7), 7, 1, 0, False), ((2, 3, 6, 5), (6, 5), 1, 0, False), ((1, 1, 3, 3), 3, 3, 0, False)]
     for (shape, k, s, p, cv) in cases:
