@@ -99,6 +99,26 @@ __global__ __launch_bounds__(256) void TakeKernel(TakeArgs t) {
     }
 }
 
+// Embedding-style rows (no left axes, the right part dense on both sides): a wavefront per index, which it resolves once; its lanes
+// then stream the row in BYTES-sized pieces.
+template <int BYTES>
+__global__ __launch_bounds__(256) void TakeRowsKernel(TakeArgs t) {
+    struct alignas(BYTES) Elem {
+        char b[BYTES];
+    };
+    const int lane = threadIdx.x & 63;
+    const int64_t waves = static_cast<int64_t>(gridDim.x) * (blockDim.x >> 6);
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6); i < t.index.total; i += waves) {
+        int64_t ioff = 0, unused = 0;
+        Decompose(t.index, i, ioff, unused);
+        const int64_t index = ResolveIndex(LoadIndex(t.idx + ioff, t.idx_dtype), t.axis_dim, t.mode, t.error_flag);
+        const Elem* src = reinterpret_cast<const Elem*>(t.a + index * t.axis_stride);
+        Elem* dst = reinterpret_cast<Elem*>(t.out + i * t.right_vecs * BYTES);
+#pragma unroll 4
+        for (int64_t v = lane; v < t.right_vecs; v += 64) dst[v] = src[v];
+    }
+}
+
 // AddAt: out[l..., index[i...], r...] += b[l..., i..., r...] on top of a copy of `a` (indexing.cc:107-190).  One thread
 // owns one (l, r) position and walks the indices in C order, so contributions to the same element are added in the
 // reference's order (float results are bit-identical; float16 rounds after every addition, as Float16::operator+= does).
@@ -203,12 +223,26 @@ extern "C" int hipcx_take(const hipcx_array* a, const hipcx_array* indices, int8
         hipStream_t st = AsStream(stream);
         int64_t cap = static_cast<int64_t>(NumCUs()) * 32;
 
-        // embedding-style rows
-        int64_t row_bytes = t.right.total * it;
-        bool rows = t.left.total == 1 && row_bytes % 16 == 0 && row_bytes > 0 && DenseGroup(t.right, t.right.stride_a, it) &&
-                    DenseGroup(t.right, t.right.stride_o, it) && t.axis_stride % 16 == 0 && reinterpret_cast<uintptr_t>(t.a) % 16 == 0 &&
-                    reinterpret_cast<uintptr_t>(t.out) % 16 == 0 && IsContiguous(out);
-        if (rows) {
+        // embedding-style rows, in the widest pieces their size and alignment allow
+        const int64_t row_bytes = t.right.total * it;
+        const uintptr_t misalign = static_cast<uintptr_t>(row_bytes) | static_cast<uintptr_t>(t.axis_stride < 0 ? -t.axis_stride : t.axis_stride) |
+                                   reinterpret_cast<uintptr_t>(t.a) | reinterpret_cast<uintptr_t>(t.out);
+        const int piece = misalign % 16 == 0 ? 16 : (misalign % 8 == 0 ? 8 : (misalign % 4 == 0 ? 4 : 0));
+        const bool rows = t.left.total == 1 && piece != 0 && row_bytes > 0 && DenseGroup(t.right, t.right.stride_a, it) &&
+                          DenseGroup(t.right, t.right.stride_o, it) && IsContiguous(out);
+        if (rows && row_bytes / piece >= 16) {
+            t.right_vecs = row_bytes / piece;
+            t.total = t.index.total * t.right_vecs;
+            int64_t blocks = (t.index.total + 3) / 4;
+            if (blocks > cap * 4) blocks = cap * 4;
+            const dim3 grid(static_cast<unsigned>(blocks)), block(256);
+            if (piece == 16) hipLaunchKernelGGL(TakeRowsKernel<16>, grid, block, 0, st, t);
+            else if (piece == 8) hipLaunchKernelGGL(TakeRowsKernel<8>, grid, block, 0, st, t);
+            else hipLaunchKernelGGL(TakeRowsKernel<4>, grid, block, 0, st, t);
+            CheckLaunch("take(rows)");
+            return;
+        }
+        if (rows && piece == 16) {  // short rows: a thread per 16-byte piece
             t.right_vecs = row_bytes / 16;
             t.total = t.index.total * t.right_vecs;
             int64_t blocks = (t.total + 255) / 256;

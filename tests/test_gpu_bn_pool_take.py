@@ -116,6 +116,15 @@ def test_take_bounds_and_embedding_shape():
     Wd, Id = chx.array(W), chx.array(ids)
     assert_exact(chx.take(Wd, Id[:, 3], 0).get(), W[ids[:, 3]], 'embedding rows, strided ids')
     assert_exact(chx.take(Wd, Id, 0).get(), W[ids], 'embedding rows, the whole [128,35] batch')
+    with pytest.raises(IndexError):
+        chx.take(Wd, chx.array(np.array([3, 10000], 'int64')), 0)
+    # long rows in 4-byte pieces (68 bytes) and in 16-byte pieces (2048 bytes), negative and wrapped indices
+    for shape, dt in (((300, 17), 'float32'), ((90, 1024), 'float16'), ((40, 33), 'int32')):
+        a = (rng.standard_normal(shape) * 100).astype(dt)
+        idx = rng.integers(-shape[0], shape[0], (9, 11)).astype('int64')
+        assert_exact(chx.take(chx.array(a), chx.array(idx), 0).get(), O.take(a, idx, 0), 'rows %r' % (shape,))
+        far = rng.integers(-5 * shape[0], 5 * shape[0], (70,)).astype('int64')
+        assert_exact(chx.take(chx.array(a), chx.array(far), 0, 'wrap').get(), O.take(a, far, 0, 'wrap'), 'wrapped rows %r' % (shape,))
 
 
 @pytest.mark.parametrize('dt,tol', [('float32', 1e-5), ('float64', 1e-12), ('float16', 2e-2)])
