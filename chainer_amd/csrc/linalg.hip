@@ -12,6 +12,7 @@
 // stores its 1-based position in the caller's flag, LAPACK's `info`, for the caller to raise on.
 // Matrices above 8192 rows fall back to an LU kernel in which one workgroup walks the whole matrix.  QR, the symmetric
 // eigendecomposition and the SVD further down are one-workgroup kernels.
+#include <mutex>
 #include <vector>
 
 #include "common.h"
@@ -1421,6 +1422,22 @@ void CopyInto(const hipcx_array* src, const hipcx_array* dst, void* stream, cons
     HIPCX_REQUIRE(rc == HIPCX_OK, HIPCX_CHAINERX_ERROR, std::string(what) + ": " + hipcx_last_error());
 }
 
+// Raises a kernel's limit of dynamic LDS to 150 KiB, once per device and kernel (`slot` tells the kernels that share this function
+// apart); several host threads may get here at once.
+void AllowLargeLds(const void* kernel, int slot) {
+    constexpr int kMaxDevices = 64, kSlots = 2;
+    static std::mutex mu;
+    static bool done[kSlots][kMaxDevices] = {};
+    int dev = 0;
+    HIPCX_CHECK_HIP(hipGetDevice(&dev));
+    HIPCX_REQUIRE(dev >= 0 && dev < kMaxDevices && slot >= 0 && slot < kSlots, HIPCX_DEVICE_ERROR, "device index out of range");
+    std::lock_guard<std::mutex> lock(mu);
+    if (!done[slot][dev]) {
+        HIPCX_CHECK_HIP(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024));
+        done[slot][dev] = true;
+    }
+}
+
 // Largest matrix the blocked LU takes: its panel kernel keeps all rows of a panel in the registers of one workgroup.
 constexpr int64_t kLuBlockedMaxN = 8192;
 
@@ -1713,7 +1730,9 @@ int hipcx_qr(const hipcx_array* a, const hipcx_array* q, const hipcx_array* r, c
                 if (want_q) {
                     const dim3 grid(static_cast<unsigned>((mc + 31) / 32));
                     const size_t strip_bytes = static_cast<size_t>(m * 34 * it);  // the reflector and [m][33] of q
-                    if (strip_bytes <= 60 * 1024) {
+                    if (strip_bytes <= 150 * 1024) {
+                        // beyond the 64 KiB a launch gets unasked, the kernel is told once per device that it may have more
+                        if (strip_bytes > 60 * 1024) AllowLargeLds(reinterpret_cast<const void*>(FormQStripKernel<T, true>), std::is_same<T, float>::value ? 0 : 1);
                         hipLaunchKernelGGL((FormQStripKernel<T, true>), grid, dim3(256), strip_bytes, st, w, static_cast<int>(m), static_cast<int>(n),
                                            static_cast<int>(k), tau_p, tau_stride, static_cast<T*>(q->data), q->strides[0] / it, q->strides[1] / it,
                                            static_cast<int>(mc));
