@@ -3,8 +3,8 @@
 // 560-600); here they are blocked factorisations of a dense row-major copy, 32 columns at a time:
 //   * LU with partial pivoting (the first row of largest magnitude, as idamax picks it): one workgroup factors a panel with its rows
 //     in registers, then one workgroup per 64 columns of the rest of the matrix and of the right-hand sides applies the panel's row
-//     exchanges, solves for the panel's rows of U and subtracts L21 U12; back substitution runs per 64 right-hand sides, block row
-//     by block row -- Inverse is the same on the identity;
+//     exchanges, solves for the panel's rows of U and subtracts L21 U12; back substitution is two launches per block row (solve the
+//     block row, take it out of the rows above) -- Inverse is the same on the identity;
 //   * left-looking Cholesky on the lower triangle, one workgroup per 32 rows of a block column, the strict upper triangle of the
 //     result zeroed.
 // Triangular 32 x 32 blocks are inverted once (doubling levels of small products) and applied as products instead of substitutions.
@@ -434,13 +434,12 @@ __global__ __launch_bounds__(256) void LuUpdateKernel(T* a, T* b, int n, int m, 
     }
 }
 
-// Back substitution with the upper triangle of a factored matrix: b ([n, m] row-major, holding L^-1 P b) becomes the solution.
-// One workgroup per 64 columns of b walks the block rows upwards: y = b_j - U[j, below] x[below] (64-deep tiles through LDS), then
-// U_jj x_j = y with one thread per column.  Nothing happens when the factorisation met a zero pivot.
+// Back substitution with the upper triangle of a factored matrix: b ([n, m] row-major, holding L^-1 P b) becomes the solution, block
+// row by block row from the bottom, two launches per block row.  This one solves U_jj x_j = b_j in place for the kNb rows from j0
+// (64 columns of b per workgroup): the inverse of the triangular block once, then a product.  Nothing happens when the
+// factorisation met a zero pivot.
 template <typename T>
-__global__ __launch_bounds__(256) void LuBackKernel(const T* a, T* b, int n, int m, const LuState* state) {
-    __shared__ T Ut[kNb][65];
-    __shared__ T Xs[64][64];
+__global__ __launch_bounds__(256) void LuBackSolveKernel(const T* a, T* b, int n, int m, int j0, const LuState* state) {
     __shared__ T Y[kNb][64];
     __shared__ T Ujj[kNb][kNb + 1];
     __shared__ T Uinv[kNb][kNb + 1];
@@ -448,60 +447,64 @@ __global__ __launch_bounds__(256) void LuBackKernel(const T* a, T* b, int n, int
     if (state->info != 0) return;
     const int tid = threadIdx.x;
     const int c = tid & 63, g = tid >> 6;
-    const int col0 = static_cast<int>(blockIdx.x) * 64;
-    const int ty = tid >> 4, tx = tid & 15;  // outputs: rows ty * 2 .. + 1, columns tx * 4 .. + 3
-    for (int j0 = (n - 1) / kNb * kNb; j0 >= 0; j0 -= kNb) {
-        const int w = min(kNb, n - j0);
-        T acc[2][4] = {};
-        for (int k0 = j0 + w; k0 < n; k0 += 64) {
-            for (int e = tid; e < kNb * 64; e += 256) {
-                const int r = e >> 6, k = e & 63;
-                Ut[r][k] = r < w && k0 + k < n ? a[static_cast<int64_t>(j0 + r) * n + k0 + k] : T(0);
-            }
-            for (int e = tid; e < 64 * 64; e += 256) {
-                const int k = e >> 6, cc = e & 63;
-                Xs[k][cc] = k0 + k < n && col0 + cc < m ? b[static_cast<int64_t>(k0 + k) * m + col0 + cc] : T(0);
-            }
-            __syncthreads();
+    const int col = static_cast<int>(blockIdx.x) * 64 + c;
+    const int w = min(kNb, n - j0);
+    for (int r = g; r < kNb; r += 4) Y[r][c] = r < w && col < m ? b[static_cast<int64_t>(j0 + r) * m + col] : T(0);
+    for (int e = tid; e < kNb * kNb; e += 256) {
+        const int r = e >> 5, k = e & (kNb - 1);
+        Ujj[r][k] = r < w && k < w ? a[static_cast<int64_t>(j0 + r) * n + j0 + k] : (r == k ? T(1) : T(0));
+    }
+    __syncthreads();
+    InvertTriangularBlock<1, 0>(Ujj, Uinv, Utmp, tid);
+#pragma unroll
+    for (int i = 0; i < kNb / 4; ++i) {
+        const int r = g * (kNb / 4) + i;
+        T sum = T(0);
+        for (int k = r; k < kNb; ++k) sum += Uinv[r][k] * Y[k][c];
+        if (r < w && col < m) b[static_cast<int64_t>(j0 + r) * m + col] = sum;
+    }
+}
+
+// ... and this one takes the solved block row out of the rows above it: b[r0 .. r0 + 63] -= U[r0 .. r0 + 63, j0 .. j0 + w) x_j for the
+// 64 rows of workgroup (x, .) and the 64 columns of workgroup (., y), 4 x 4 entries per thread.
+template <typename T>
+__global__ __launch_bounds__(256) void LuBackUpdateKernel(const T* a, T* b, int n, int m, int j0, const LuState* state) {
+    __shared__ T Us[64][kNb + 1];
+    __shared__ T Xs[kNb][64];
+    if (state->info != 0) return;
+    const int tid = threadIdx.x;
+    const int r0 = static_cast<int>(blockIdx.x) * 64, col0 = static_cast<int>(blockIdx.y) * 64;
+    const int w = min(kNb, n - j0);
+    for (int e = tid; e < 64 * kNb; e += 256) {
+        const int r = e >> 5, k = e & (kNb - 1);
+        Us[r][k] = r0 + r < j0 && k < w ? a[static_cast<int64_t>(r0 + r) * n + j0 + k] : T(0);
+    }
+    for (int e = tid; e < kNb * 64; e += 256) {
+        const int k = e >> 6, cc = e & 63;
+        Xs[k][cc] = k < w && col0 + cc < m ? b[static_cast<int64_t>(j0 + k) * m + col0 + cc] : T(0);
+    }
+    __syncthreads();
+    const int ty = tid >> 4, tx = tid & 15;
+    T acc[4][4] = {};
 #pragma unroll 4
-            for (int k = 0; k < 64; ++k) {
-                T uv[2], xv[4];
+    for (int k = 0; k < kNb; ++k) {
+        T uv[4], xv[4];
 #pragma unroll
-                for (int i = 0; i < 2; ++i) uv[i] = Ut[ty * 2 + i][k];
+        for (int i = 0; i < 4; ++i) uv[i] = Us[ty * 4 + i][k], xv[i] = Xs[k][tx * 4 + i];
 #pragma unroll
-                for (int j = 0; j < 4; ++j) xv[j] = Xs[k][tx * 4 + j];
+        for (int i = 0; i < 4; ++i) {
 #pragma unroll
-                for (int i = 0; i < 2; ++i) {
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) acc[i][j] += uv[i] * xv[j];
-                }
-            }
-            __syncthreads();
+            for (int j = 0; j < 4; ++j) acc[i][j] += uv[i] * xv[j];
         }
+    }
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const int r = ty * 2 + i;
+    for (int i = 0; i < 4; ++i) {
+        const int r = r0 + ty * 4 + i;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int cc = tx * 4 + j;
-                Y[r][cc] = r < w && col0 + cc < m ? b[static_cast<int64_t>(j0 + r) * m + col0 + cc] - acc[i][j] : T(0);
-            }
+        for (int j = 0; j < 4; ++j) {
+            const int cc = col0 + tx * 4 + j;
+            if (r < j0 && cc < m) b[static_cast<int64_t>(r) * m + cc] -= acc[i][j];
         }
-        for (int e = tid; e < kNb * kNb; e += 256) {
-            const int r = e >> 5, k = e & (kNb - 1);
-            Ujj[r][k] = r < w && k < w ? a[static_cast<int64_t>(j0 + r) * n + j0 + k] : (r == k ? T(1) : T(0));
-        }
-        __syncthreads();
-        // x_j = U_jj^-1 y: the inverse of the upper triangle once, then a product (8 rows per thread)
-        InvertTriangularBlock<1, 0>(Ujj, Uinv, Utmp, tid);
-#pragma unroll
-        for (int i = 0; i < kNb / 4; ++i) {
-            const int r = g * (kNb / 4) + i;
-            T sum = T(0);
-            for (int k = r; k < kNb; ++k) sum += Uinv[r][k] * Y[k][c];
-            if (r < w && col0 + c < m) b[static_cast<int64_t>(j0 + r) * m + col0 + c] = sum;
-        }
-        __syncthreads();  // the block row's solution is in b before the next block row reads it
     }
 }
 
@@ -1481,7 +1484,14 @@ void LuSolveBlocked(T* a, T* b, int64_t n, int64_t m, LuState* state, int32_t* u
                            static_cast<int>(j0), w, state);
         j0 += w;
     }
-    hipLaunchKernelGGL(LuBackKernel<T>, dim3(strips_b), dim3(256), 0, stream, a, b, static_cast<int>(n), static_cast<int>(m), state);
+    for (int64_t j0 = (n - 1) / kNb * kNb; j0 >= 0; j0 -= kNb) {
+        hipLaunchKernelGGL(LuBackSolveKernel<T>, dim3(strips_b), dim3(256), 0, stream, a, b, static_cast<int>(n), static_cast<int>(m),
+                           static_cast<int>(j0), state);
+        if (j0 > 0) {
+            hipLaunchKernelGGL(LuBackUpdateKernel<T>, dim3(static_cast<unsigned>((j0 + 63) / 64), strips_b), dim3(256), 0, stream, a, b,
+                               static_cast<int>(n), static_cast<int>(m), static_cast<int>(j0), state);
+        }
+    }
 }
 
 // a (already copied into the workspace) and b (already in out) -> the solution in out
