@@ -659,9 +659,10 @@ __global__ __launch_bounds__(256) void IdentityFillKernel(T* out, int n) {
 // The columns p and q of the round-robin pairing: player idx of `round` (np = N rounded up to even players, the last of them fixed).
 // q = -1 for the pair that holds the dummy player of an odd N.
 __device__ __forceinline__ void JacobiPair(int idx, int round, int N, int& p, int& q) {
-    const int rounds = N + (N & 1) - 1;
-    p = idx == 0 ? rounds : (round + idx) % rounds;
-    q = idx == 0 ? round % rounds : (round - idx + rounds) % rounds;
+    const int rounds = N + (N & 1) - 1;  // round < rounds and idx <= rounds / 2: the sums below stay under 2 * rounds
+    const int up = round + idx, down = round - idx + rounds;
+    p = idx == 0 ? rounds : (up >= rounds ? up - rounds : up);
+    q = idx == 0 ? round : (down >= rounds ? down - rounds : down);
     if (p > q) { const int t2 = p; p = q; q = t2; }
     if (q >= N) q = -1;
 }
@@ -694,21 +695,30 @@ __global__ __launch_bounds__(256) void EighNormsKernel(const T* s, int n, T* par
     }
 }
 
-// The rotations of `round` from the right, applied to one row of s held in LDS (entries p and q of every pair of that round); the
-// entry a rotation annihilates is stored as an exact zero (see JacobiEighKernel).  r is the row's index; the `lanes` threads that
-// share the row each take every lanes-th pair.
+// The rotation (c, sn) of pair `idx` of `round` from the right, applied to one or two rows of s held in LDS (entries p and q of that
+// pair; row_b may be null); the entry a rotation annihilates is stored as an exact zero (see JacobiEighKernel).  ra / rb are the rows'
+// indices.
 template <typename T>
-__device__ __forceinline__ void EighRotateRowEntries(T* row, int r, int n, int round, const T* cs, int lane, int lanes) {
-    for (int idx = lane; idx < (n + 1) / 2; idx += lanes) {
-        int p, q;
-        JacobiPair(idx, round, n, p, q);
-        if (q < 0) continue;
-        const T c = cs[2 * idx], sn = cs[2 * idx + 1];
-        if (sn == T(0)) continue;
-        const T a = row[p], b = row[q];
-        row[p] = r == q ? T(0) : c * a - sn * b;
-        row[q] = r == p ? T(0) : sn * a + c * b;
+__device__ __forceinline__ void EighRotateRowEntry(T* row_a, int ra, T* row_b, int rb, int n, int round, int idx, T c, T sn) {
+    int p, q;
+    JacobiPair(idx, round, n, p, q);
+    if (q < 0 || sn == T(0)) return;
+    {
+        const T a = row_a[p], b = row_a[q];
+        row_a[p] = ra == q ? T(0) : c * a - sn * b;
+        row_a[q] = ra == p ? T(0) : sn * a + c * b;
     }
+    if (row_b != nullptr) {
+        const T a = row_b[p], b = row_b[q];
+        row_b[p] = rb == q ? T(0) : c * a - sn * b;
+        row_b[q] = rb == p ? T(0) : sn * a + c * b;
+    }
+}
+
+// ... of every pair of the round; the `lanes` threads that share the rows each take every lanes-th pair.
+template <typename T>
+__device__ __forceinline__ void EighRotateRowEntries(T* row_a, int ra, T* row_b, int rb, int n, int round, const T* cs, int lane, int lanes) {
+    for (int idx = lane; idx < (n + 1) / 2; idx += lanes) EighRotateRowEntry(row_a, ra, row_b, rb, n, round, idx, cs[2 * idx], cs[2 * idx + 1]);
 }
 
 // A round of the two-sided Jacobi sweeps of JacobiEighKernel below, spread over workgroups, one per pair (p, q).
@@ -730,14 +740,39 @@ __global__ __launch_bounds__(256) void EighRoundKernel(T* s, T* vt, int n, int p
     JacobiPair(idx, round, n, p, q);  // q = -1: p sits out this round, but still owes the previous round's rotations
     T* sp = s + static_cast<int64_t>(p) * n;
     T* sq = s + static_cast<int64_t>(q < 0 ? p : q) * n;
+    // Everything this workgroup reads from memory is asked for up front, so that the loads travel together: its two rows of s, the
+    // previous round's rotations its threads will apply (the first kAhead pairs of each thread) and its two rows of vt (the first
+    // kAhead entries of each thread); longer rows fetch the rest when they get there.
+    constexpr int kAhead = 4;
+    const int half = (n + 1) / 2;
+    T ahead_c[kAhead], ahead_s[kAhead], ahead_vp[kAhead], ahead_vq[kAhead];
+    T* vp = vt + static_cast<int64_t>(p) * n;
+    T* vq = vt + static_cast<int64_t>(q < 0 ? p : q) * n;
+#pragma unroll
+    for (int u = 0; u < kAhead; ++u) {
+        const int other = lane + u * kLanes;
+        const bool have_pair = prev_round >= 0 && other < half;
+        ahead_c[u] = have_pair ? cs_prev[2 * other] : T(1);
+        ahead_s[u] = have_pair ? cs_prev[2 * other + 1] : T(0);
+        const bool have_v = compute_v && q >= 0 && other < n;
+        ahead_vp[u] = have_v ? vp[other] : T(0);
+        ahead_vq[u] = have_v ? vq[other] : T(0);
+    }
     for (int i = lane; i < n; i += kLanes) {
         row_p[i] = sp[i];
         if (q >= 0) row_q[i] = sq[i];
     }
     __syncthreads();
     if (prev_round >= 0) {
-        EighRotateRowEntries(row_p, p, n, prev_round, cs_prev, lane, kLanes);
-        if (q >= 0) EighRotateRowEntries(row_q, q, n, prev_round, cs_prev, lane, kLanes);
+        T* second = q >= 0 ? row_q : static_cast<T*>(nullptr);
+#pragma unroll
+        for (int u = 0; u < kAhead; ++u) {
+            const int other = lane + u * kLanes;
+            if (other < half) EighRotateRowEntry(row_p, p, second, q, n, prev_round, other, ahead_c[u], ahead_s[u]);
+        }
+        for (int other = lane + kAhead * kLanes; other < half; other += kLanes) {
+            EighRotateRowEntry(row_p, p, second, q, n, prev_round, other, cs_prev[2 * other], cs_prev[2 * other + 1]);
+        }
         __syncthreads();
     }
     T c = T(1), sn = T(0);
@@ -767,10 +802,15 @@ __global__ __launch_bounds__(256) void EighRoundKernel(T* s, T* vt, int n, int p
         sq[i] = sn * a + c * b;
     }
     if (compute_v) {
-        T* vp = vt + static_cast<int64_t>(p) * n;
-        T* vq = vt + static_cast<int64_t>(q) * n;
-#pragma unroll 4
-        for (int i = lane; i < n; i += kLanes) {
+#pragma unroll
+        for (int u = 0; u < kAhead; ++u) {
+            const int i = lane + u * kLanes;
+            if (i < n) {
+                vp[i] = c * ahead_vp[u] - sn * ahead_vq[u];
+                vq[i] = sn * ahead_vp[u] + c * ahead_vq[u];
+            }
+        }
+        for (int i = lane + kAhead * kLanes; i < n; i += kLanes) {
             const T a = vp[i], b = vq[i];
             vp[i] = c * a - sn * b;
             vq[i] = sn * a + c * b;
@@ -792,7 +832,7 @@ __global__ __launch_bounds__(256) void EighColumnsKernel(T* s, int n, int round,
         for (int i = lane; i < n; i += 64) row[i] = s[static_cast<int64_t>(r) * n + i];
     }
     __syncthreads();
-    if (valid) EighRotateRowEntries(row, r, n, round, cs, lane, 64);
+    if (valid) EighRotateRowEntries(row, r, static_cast<T*>(nullptr), -1, n, round, cs, lane, 64);
     __syncthreads();
     if (valid) {
         for (int i = lane; i < n; i += 64) s[static_cast<int64_t>(r) * n + i] = row[i];
