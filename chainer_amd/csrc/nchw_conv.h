@@ -218,6 +218,11 @@ void NchwConvKernel(NchwConvArgs p) {
     // ---- activation load slots of this thread ----
     int xvoff[MAXI];  // byte offset of (n, channel group base, first pixel) in x; out of range for idle slots
     int xlds[MAXI];   // byte offset of the first pixel's group inside a stage
+    // Two-pixel loads of the 1x1 kernels: a lane's two 16-byte groups are neighbours, so the lanes of a wave write with a stride
+    // of 32 bytes and would use only half of the LDS banks.  Every other run of 8 lanes therefore stores its two groups in
+    // swapped order (slot s lives at s ^ ((s >> 4) & 1)); the fragment reads below apply the same exchange.
+    constexpr bool kSwapPairs = TAPS == 1 && NPX == 2;
+    int xflip[MAXI];  // 16 where the two groups are swapped, else 0
 #pragma unroll
     for (int i = 0; i < MAXI; ++i) {
         int it = tid + i * NT;
@@ -236,6 +241,7 @@ void NchwConvKernel(NchwConvArgs p) {
             valid = cg < CG && grow <= last_row && n < p.N && hh >= 0 && hh < p.H;
             voff = (((n * p.C + cg * 8) * p.H + hh) * p.W + wc * NPX) * 2;
             loff = (cg * p.nslot + pr * W2 + wc * NPX + 1) * 16;
+            xflip[i] = 0;
         } else {
             constexpr int per_cg = BM / NPX;
             int cg = it / per_cg;
@@ -248,6 +254,7 @@ void NchwConvKernel(NchwConvArgs p) {
             int ow = pix - oh * p.OW;
             voff = (((n * p.C + cg * 8) * p.H + oh * p.stride) * p.W + ow * p.stride) * 2;
             loff = (cg * p.nslot + q * NPX) * 16;
+            xflip[i] = kSwapPairs ? ((q >> 3) & 1) * 16 : 0;
         }
         xvoff[i] = valid ? voff : 0x7fffffff;  // beyond the buffer: the load returns zeros
         xlds[i] = valid ? loff : -1;           // idle slots write into the dump area
@@ -299,7 +306,7 @@ void NchwConvKernel(NchwConvArgs p) {
                 Transpose8<NPX>(xreg[i], t);
                 char* dst = xlds[i] >= 0 ? stage + xlds[i] : lds + dump_off;
 #pragma unroll
-                for (int e = 0; e < NPX; ++e) *reinterpret_cast<Bytes16*>(dst + e * 16) = t[e];
+                for (int e = 0; e < NPX; ++e) *reinterpret_cast<Bytes16*>(dst + (kSwapPairs ? (e * 16) ^ xflip[i] : e * 16)) = t[e];
             } else {
                 constexpr int j = r - 1;
                 if constexpr (NPX == 1 && PAIR) {
@@ -352,6 +359,7 @@ void NchwConvKernel(NchwConvArgs p) {
             slot -= W2 + 1;  // tap (r, s) adds r * W2 + s
         } else {
             slot = (wpx * PW + a) * 32 + lr;
+            if constexpr (kSwapPairs) slot ^= (slot >> 4) & 1;
         }
         aoff[a] = (g * p.nslot + slot) * 16;
     }
