@@ -527,6 +527,27 @@ NchwPlan PlanNchw(const hipcx_array* x, const hipcx_array* w, const hipcx_array*
     return pl;
 }
 
+// How many workgroups of `kernel` the device holds at once (for the launch shape given); asked once per kernel instantiation (the
+// Tag type), device and LDS size, from any thread.
+template <typename Tag>
+int ResidentWorkgroups(const void* kernel, int block_threads, int lds_bytes) {
+    constexpr int kMaxDevices = 64;
+    static std::mutex mu;
+    static int resident[kMaxDevices] = {};
+    static int asked_lds[kMaxDevices] = {};
+    int dev = 0;
+    HIPCX_CHECK_HIP(hipGetDevice(&dev));
+    HIPCX_REQUIRE(dev >= 0 && dev < kMaxDevices, HIPCX_DEVICE_ERROR, "device index out of range");
+    std::lock_guard<std::mutex> lock(mu);
+    if (resident[dev] == 0 || asked_lds[dev] != lds_bytes) {
+        int per_cu = 0;
+        HIPCX_CHECK_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, block_threads, static_cast<size_t>(lds_bytes)));
+        resident[dev] = std::max(1, per_cu) * NumCUs();
+        asked_lds[dev] = lds_bytes;
+    }
+    return resident[dev];
+}
+
 template <int TAPS, int WPX, int WCH, int CK, int NPX, int MAXI, int KSPLIT = 1, bool PAIR = false>
 void LaunchNchwKernel(const NchwConvArgs& a, int lds_bytes, hipStream_t stream) {
     auto kern = NchwConvKernel<TAPS, WPX, WCH, CK, NPX, MAXI, KSPLIT, PAIR>;
@@ -534,6 +555,14 @@ void LaunchNchwKernel(const NchwConvArgs& a, int lds_bytes, hipStream_t stream) 
     EnsureDynamicLds<Tag>(reinterpret_cast<const void*>(kern), lds_bytes);
     int64_t total = static_cast<int64_t>(a.tiles_m) * a.tiles_n;
     dim3 grid(static_cast<unsigned>((total + 7) / 8 * 8)), block(64 * WPX * WCH * KSPLIT);
+    if constexpr (NchwWalksTiles(TAPS, WPX * WCH, NPX, KSPLIT)) {
+        // these kernels walk tiles: no more workgroups than the chip holds at once (a multiple of 8, one share per XCD)
+        static const bool walk = [] { const char* e = getenv("HIPCX_CONV_WALK"); return e == nullptr || e[0] != '0'; }();
+        if (walk) {
+            const int resident = ResidentWorkgroups<Tag>(reinterpret_cast<const void*>(kern), static_cast<int>(block.x), lds_bytes);
+            grid.x = std::min(grid.x, static_cast<unsigned>(std::max(8, resident / 8 * 8)));
+        }
+    }
     hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, a);
     CheckLaunch("nchw_conv");
 }

@@ -74,15 +74,18 @@ struct BytesOf<8> {
 // XCD-aware tile order: hardware deals consecutive workgroup ids round-robin to the 8 XCDs, each
 // with its own L2.  Remap so that every XCD walks a contiguous range of tiles; with the channel
 // tile as the fast index, blocks that share an activation tile then share an L2.
-__device__ __forceinline__ bool TileOf(int tiles_m, int tiles_n, int& tile_m, int& tile_n) {
+__device__ __forceinline__ bool TileOf(int tiles_m, int tiles_n, int b, int& tile_m, int& tile_n) {
     int total = tiles_m * tiles_n;
     int per = (total + 7) / 8;
-    int b = blockIdx.x;
+    if (b >= per * 8) return false;
     int logical = (b % 8) * per + b / 8;
     if (logical >= total) return false;
     tile_n = logical % tiles_n;
     tile_m = logical / tiles_n;
     return true;
+}
+__device__ __forceinline__ bool TileOf(int tiles_m, int tiles_n, int& tile_m, int& tile_n) {
+    return TileOf(tiles_m, tiles_n, static_cast<int>(blockIdx.x), tile_m, tile_n);
 }
 
 template <typename T>

@@ -159,6 +159,10 @@ __device__ __forceinline__ void StaticFor(F&& f) {
     }
 }
 
+// Which instantiations walk several tiles per workgroup: the four-wave 1x1 kernels with two-pixel loads.  (The single-pixel and
+// eight-wave variants have no registers to spare for the next tile's loads during the epilogue and measured slower.)
+constexpr bool NchwWalksTiles(int taps, int waves, int npx, int ksplit) { return taps == 1 && ksplit == 1 && npx == 2 && waves == 4; }
+
 // KSPLIT = 2: a second set of WPX * WCH waves works on the same tile and takes every other channel chunk through LDS stages of
 // its own; the two accumulator sets are added through LDS before the epilogue.  For grids with at most one tile per compute unit
 // (7x7 planes, small batches) this doubles the waves and the loads in flight per unit, which is what bounds those layers.
@@ -168,7 +172,7 @@ __device__ __forceinline__ void StaticFor(F&& f) {
 template <int TAPS, int WPX, int WCH, int CK, int NPX, int MAXI, int KSPLIT = 1, bool PAIR = false>
 // Eight-wave workgroups that do not split the reduction are meant to run two to a compute unit (four waves per SIMD): they
 // are kept within 128 registers.
-__global__ __launch_bounds__(64 * WPX * WCH * KSPLIT) __attribute__((amdgpu_waves_per_eu(WPX * WCH >= 8 && KSPLIT == 1 ? 4 : 1, 8)))
+__global__ __launch_bounds__(64 * WPX * WCH * KSPLIT) __attribute__((amdgpu_waves_per_eu(WPX * WCH >= 8 && KSPLIT == 1 ? 4 : (NchwWalksTiles(TAPS, WPX * WCH, NPX, KSPLIT) ? 3 : 1), 8)))
 void NchwConvKernel(NchwConvArgs p) {
     constexpr int PW = 2, CW = 2;  // wave tile: 64 pixels x 64 channels
     constexpr int NT = 64 * WPX * WCH;       // threads of one reduction group
@@ -188,10 +192,15 @@ void NchwConvKernel(NchwConvArgs p) {
     const int stage_bytes = patch_bytes + CG * WCGP;
     const int dump_off = KSPLIT * 2 * stage_bytes;  // NPX * 16 bytes that absorb the writes of idle load slots
 
+    // Some 1x1 kernels (NchwWalksTiles) walk several tiles per workgroup when the grid is smaller than the tile count (the
+    // host launches as many workgroups as fit on the chip at once): the first loads of the next tile are issued before the
+    // current tile is written out, so that their latency and the tile's set-up hide behind the epilogue.
+    constexpr bool kWalk = NchwWalksTiles(TAPS, WPX * WCH, NPX, KSPLIT);
+    int vblock = blockIdx.x;  // the virtual workgroup index of the current tile
     int tile_m, tile_n;
-    if (!TileOf(p.tiles_m, p.tiles_n, tile_m, tile_n)) return;
-    const int m0 = tile_m * BM;
-    const int n0 = tile_n * BN;
+    if (!TileOf(p.tiles_m, p.tiles_n, vblock, tile_m, tile_n)) return;
+    int m0 = tile_m * BM;
+    int n0 = tile_n * BN;
     const int tid_all = threadIdx.x;
     const int kg = KSPLIT > 1 ? __builtin_amdgcn_readfirstlane(tid_all / NT) : 0;  // reduction group of this wave
     const int tid = tid_all - kg * NT;                                             // thread index inside the group
@@ -223,6 +232,7 @@ void NchwConvKernel(NchwConvArgs p) {
     // swapped order (slot s lives at s ^ ((s >> 4) & 1)); the fragment reads below apply the same exchange.
     constexpr bool kSwapPairs = TAPS == 1 && NPX == 2;
     int xflip[MAXI];  // 16 where the two groups are swapped, else 0
+    auto place_x_slots = [&](int m_first) {
 #pragma unroll
     for (int i = 0; i < MAXI; ++i) {
         int it = tid + i * NT;
@@ -246,7 +256,7 @@ void NchwConvKernel(NchwConvArgs p) {
             constexpr int per_cg = BM / NPX;
             int cg = it / per_cg;
             int q = it - cg * per_cg;
-            int m = m0 + q * NPX;
+            int m = m_first + q * NPX;
             valid = cg < CG && m < p.M;
             int n = p.div_P(m);
             int pix = m - n * p.P;
@@ -259,9 +269,12 @@ void NchwConvKernel(NchwConvArgs p) {
         xvoff[i] = valid ? voff : 0x7fffffff;  // beyond the buffer: the load returns zeros
         xlds[i] = valid ? loff : -1;           // idle slots write into the dump area
     }
+    };
+    place_x_slots(m0);
     // ---- filter load slots ----
     int wvoff[WPT];
     int wlds[WPT];
+    auto place_w_slots = [&](int n_first) {
 #pragma unroll
     for (int i = 0; i < WPT; ++i) {
         int wi = tid + i * NT;
@@ -276,14 +289,16 @@ void NchwConvKernel(NchwConvArgs p) {
             tap = rest / BN;
             kl = rest - tap * BN;
         }
-        bool valid = wi < WITEMS && n0 + kl < p.K;
+        bool valid = wi < WITEMS && n_first + kl < p.K;
         if (TAPS == 1 && p.w_direct) {
-            wvoff[i] = valid ? ((n0 + kl) * p.C + cg * 8) * 2 : 0x7fffffff;
+            wvoff[i] = valid ? ((n_first + kl) * p.C + cg * 8) * 2 : 0x7fffffff;
         } else {
-            wvoff[i] = valid ? ((cg * TAPS + tap) * p.K + n0 + kl) * 16 : 0x7fffffff;
+            wvoff[i] = valid ? ((cg * TAPS + tap) * p.K + n_first + kl) * 16 : 0x7fffffff;
         }
         wlds[i] = wi < WITEMS ? patch_bytes + cg * WCGP + (tap * BN + kl) * 16 : -1;
     }
+    };
+    place_w_slots(n0);
 
     const __amdgpu_buffer_rsrc_t xr = MakeRsrc(p.x, p.x_bytes);
     const __amdgpu_buffer_rsrc_t wr = MakeRsrc(p.wp, p.wp_bytes);
@@ -433,6 +448,7 @@ void NchwConvKernel(NchwConvArgs p) {
         for (int off = tid_all * 16; off < KSPLIT * 2 * stage_bytes; off += NT_ALL * 16) *reinterpret_cast<Bytes16*>(lds + off) = Bytes16(0);
         __syncthreads();
     }
+    for (;;) {  // one pass per tile; a single pass unless this workgroup walks several tiles
     store_all(glds);
     if (nchunks > 1) {
         set_chunk(1);
@@ -478,6 +494,23 @@ void NchwConvKernel(NchwConvArgs p) {
             }
         }
         __syncthreads();  // the staging tile below reuses this memory
+    }
+
+    // ---- the next tile of this workgroup: its load slots, and its first chunk on the way before this tile is written out ----
+    bool more = false;
+    int m0_next = 0, n0_next = 0;
+    if constexpr (kWalk) {
+        vblock += static_cast<int>(gridDim.x);
+        int tm, tn;
+        more = TileOf(p.tiles_m, p.tiles_n, vblock, tm, tn);
+        if (more) {
+            m0_next = tm * BM;
+            n0_next = tn * BN;
+            place_x_slots(m0_next);
+            place_w_slots(n0_next);
+            set_chunk(0);
+            load_all();
+        }
     }
 
     // ---- epilogue ----
@@ -578,6 +611,19 @@ void NchwConvKernel(NchwConvArgs p) {
         case 4: store_ev(std::integral_constant<int, 4>{}); break;
         case 2: store_ev(std::integral_constant<int, 2>{}); break;
         default: store_ev(std::integral_constant<int, 1>{}); break;
+    }
+    if (!more) break;  // the same for every thread of the workgroup
+    __syncthreads();   // the output tile has left LDS before the next tile's operands are written there
+    m0 = m0_next;
+    n0 = n0_next;
+#pragma unroll
+    for (int a = 0; a < PW; ++a) {
+#pragma unroll
+        for (int b = 0; b < CW; ++b) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.f;
+        }
+    }
     }
 }
 

@@ -140,6 +140,23 @@ def test_conv_linearity_at_resnet_layer_size():
     assert np.array_equal(chx.conv(X, chx.array(delta), None, 1, 1).get(), x)
 
 
+def test_pointwise_conv_with_more_tiles_than_resident_workgroups():
+    """A 1x1 convolution whose tile count (1568 tiles of 128 x 128) exceeds what the device holds at once, so that every
+    workgroup walks several tiles: against the oracle, with a bias, and an identity filter bank reproduces the input bit for bit
+    (each output tile lands where it belongs)."""
+    import chainer_amd as chx
+    rng = np.random.default_rng(14)
+    x = rng.standard_normal((32, 64, 56, 56)).astype('float16')
+    w = (rng.standard_normal((256, 64, 1, 1)) / 8).astype('float16')
+    b = rng.standard_normal(256).astype('float16')
+    got = chx.conv(chx.array(x), chx.array(w), chx.array(b)).get()
+    assert_close(got, O.conv(x, w, b), 2e-2, 'conv 1x1, 1568 tiles')
+    eye = np.zeros((256, 64, 1, 1), 'float16')
+    eye[np.arange(256), np.arange(256) % 64, 0, 0] = 1
+    out = chx.conv(chx.array(x), chx.array(eye)).get()
+    assert np.array_equal(out, np.tile(x, (1, 4, 1, 1)))
+
+
 @pytest.mark.parametrize('dt,tol', DT)
 def test_dot_operand_layouts_large(dt, tol):
     """Products large enough for the tiled MFMA kernel with every operand layout Dot accepts without a copy in the reference
