@@ -1231,8 +1231,11 @@ bool BatchedProductApplies(const void* a, int64_t a_row, int64_t a_slice, const 
            Aligned(bt, 16) && Aligned(out, 16);
 }
 
+// With taps_s > 0 row j of bt_b is a window of a larger array: j = (c, r, s) with c = j / (taps_r * taps_s) starts at
+// bt_b + c * bt_row + r * r_stride + s * s_stride (elements; 16-byte granules like the other strides).
 void LaunchBatchedProduct(int dtype, const void* a, int64_t a_row, int64_t a_slice, const void* bt, int64_t bt_row, int64_t bt_slice, int64_t m,
-                          int64_t n, int64_t depth, int batch, void* out, float* partial, hipStream_t stream) {
+                          int64_t n, int64_t depth, int batch, void* out, float* partial, hipStream_t stream, int taps_r, int taps_s,
+                          int64_t r_stride, int64_t s_stride) {
     auto run = [&](auto tag) {
         using T = decltype(tag);
         IGemmArgs<T> p{};
@@ -1254,6 +1257,8 @@ void LaunchBatchedProduct(int dtype, const void* a, int64_t a_row, int64_t a_sli
         p.Kg = static_cast<int>(depth);
         p.batch = batch;
         p.x_slice = a_slice, p.w_slice = bt_slice;
+        p.w_taps_r = taps_r, p.w_taps_s = taps_s;
+        p.w_r_stride = r_stride, p.w_s_stride = s_stride;
         p.ksplit = partial != nullptr ? BatchedProductSlices(m, n, depth, batch, dtype) : 1;
         p.partial = p.ksplit > 1 ? partial : nullptr;
         // the work accounting of the launch sees the whole reduction

@@ -7,6 +7,14 @@
 //     col_t[c][r][s][n][oh][ow]     (Im2Col in one launch instead of kh*kw strided copies of a padded image)
 // and then gw[k][(c, r, s)] = Dot(gy_t, col_t^T), which for these shapes (few output tiles, long reduction) runs with the
 // reduction split over workgroups.
+//
+// Filters larger than 1x1 at stride 1 (float16 / float32) avoid the kh*kw-fold Im2Col: x is written kw times as zero-padded planes
+// whose rows are Wp = W + 2*pw rounded up to a 16-byte granule, copy s shifted left by s elements, and gy once with its rows
+// padded to Wp with zeros.  On that common grid tap (r, s) of channel c is the window of copy s that starts r rows down, so
+//     gw[k][c][r][s] = sum_n sum_q gy_p[n][k][q] * x_s[s][n][c][q + r*Wp],   q over OH*Wp
+// is one accumulated matrix product per image whose right-hand rows alias windows of the copies; the zero columns of gy_p cancel
+// the products that wrap around a row end.  (A non-finite x value therefore meets a zero of gy_p in windows the reference never
+// multiplies it into: inf or NaN in x can turn up as NaN in more filter taps than in the reference.)
 #include "common.h"
 
 namespace hipcx {
@@ -103,6 +111,59 @@ __global__ __launch_bounds__(256) void TransposeNKKernel(GradWeightArgs p, int64
         const int k = static_cast<int>(t / p.N);
         *reinterpret_cast<GVec<T, VEC>*>(gt + idx * VEC) =
                 *reinterpret_cast<const GVec<T, VEC>*>(gy + ((static_cast<int64_t>(n) * p.K + k) * pv + v) * VEC);
+    }
+}
+
+struct ShiftedArgs {
+    const void* x;
+    const void* gy;
+    void* xs;   // [kw][N*C][Hp*Wp]
+    void* gyp;  // [N*K][OH*Wp]
+    int planes_x, planes_gy;  // N*C, N*K
+    int H, W, OH, OW, Hp, Wp, ph, pw, kw;
+};
+
+// xs[s][plane][q] = padded x[plane][q + s]; one thread writes VEC consecutive q.
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void ShiftedPlanesKernel(ShiftedArgs p, unsigned total) {
+    const T* x = static_cast<const T*>(p.x);
+    T* xs = static_cast<T*>(p.xs);
+    const unsigned per_plane = static_cast<unsigned>(p.Hp * p.Wp / VEC);
+    for (unsigned idx = blockIdx.x * 256u + threadIdx.x; idx < total; idx += gridDim.x * 256u) {
+        unsigned t = idx / per_plane;
+        const unsigned qv = idx - t * per_plane;
+        const unsigned s = t / static_cast<unsigned>(p.planes_x);
+        const unsigned plane = t - s * static_cast<unsigned>(p.planes_x);
+        const T* src = x + static_cast<int64_t>(plane) * p.H * p.W;
+        GVec<T, VEC> out;
+        int q = static_cast<int>(qv) * VEC + static_cast<int>(s);
+        int hp = q / p.Wp, wp = q - hp * p.Wp;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            const int ih = hp - p.ph, iw = wp - p.pw;
+            out.v[e] = (ih >= 0 && ih < p.H && iw >= 0 && iw < p.W) ? src[ih * p.W + iw] : T(0);  // rows past Hp fail ih < H
+            if (++wp == p.Wp) wp = 0, ++hp;
+        }
+        *reinterpret_cast<GVec<T, VEC>*>(xs + static_cast<int64_t>(idx) * VEC) = out;
+        if (idx + gridDim.x * 256u < idx) break;  // the next index would wrap
+    }
+}
+
+// gyp[plane][oh][w] = gy[plane][oh][w] for w < OW, 0 up to Wp.
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void PaddedRowsKernel(ShiftedArgs p, unsigned total) {
+    const T* gy = static_cast<const T*>(p.gy);
+    T* gyp = static_cast<T*>(p.gyp);
+    const unsigned per_row = static_cast<unsigned>(p.Wp / VEC);
+    for (unsigned idx = blockIdx.x * 256u + threadIdx.x; idx < total; idx += gridDim.x * 256u) {
+        const unsigned row = idx / per_row;  // plane * OH + oh: rows of gy are OW apart
+        const int w0 = static_cast<int>(idx - row * per_row) * VEC;
+        const T* src = gy + static_cast<int64_t>(row) * p.OW;
+        GVec<T, VEC> out;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) out.v[e] = w0 + e < p.OW ? src[w0 + e] : T(0);
+        *reinterpret_cast<GVec<T, VEC>*>(gyp + static_cast<int64_t>(idx) * VEC) = out;
+        if (idx + gridDim.x * 256u < idx) break;
     }
 }
 
@@ -211,7 +272,8 @@ size_t BatchedProductPartialBytes(int64_t m, int64_t n, int64_t depth, int batch
 bool BatchedProductApplies(const void* a, int64_t a_row, int64_t a_slice, const void* bt, int64_t bt_row, int64_t bt_slice, int64_t depth,
                            const void* out, int dtype);
 void LaunchBatchedProduct(int dtype, const void* a, int64_t a_row, int64_t a_slice, const void* bt, int64_t bt_row, int64_t bt_slice, int64_t m,
-                          int64_t n, int64_t depth, int batch, void* out, float* partial, hipStream_t stream);
+                          int64_t n, int64_t depth, int batch, void* out, float* partial, hipStream_t stream, int taps_r = 0, int taps_s = 0,
+                          int64_t r_stride = 0, int64_t s_stride = 0);
 
 namespace {
 // A 1x1 filter at stride 1 without padding: gw[k][c] = sum over images of gy_n [K, pixels] @ x_n [C, pixels]^T, which the MFMA kernel
@@ -227,6 +289,52 @@ bool DirectPointwise(const GradWeightPlan& pl, const hipcx_array* x, const hipcx
     return BatchedProductApplies(gy->data, pixels, static_cast<int64_t>(a.K) * pixels, x->data, pixels, static_cast<int64_t>(a.C) * pixels, pixels,
                                  gw->data, gw->dtype);
 }
+
+// Filters larger than 1x1 at stride 1: shifted zero-padded copies of x instead of Im2Col (see the top of the file).
+struct ShiftedPlan {
+    bool ok = false;
+    ShiftedArgs a{};
+    int64_t depth = 0, plane = 0;  // OH*Wp; Hp*Wp
+    size_t xs_bytes = 0, gyp_bytes = 0, partial_bytes = 0;
+};
+
+ShiftedPlan PlanShifted(const GradWeightPlan& pl, int dtype) {
+    ShiftedPlan sp;
+    static const bool enabled = [] { const char* e = getenv("HIPCX_GRAD_WEIGHT_SHIFTED"); return e == nullptr || e[0] != '0'; }();
+    const GradWeightArgs& g = pl.a;
+    if (!enabled || (dtype != HIPCX_FLOAT16 && dtype != HIPCX_FLOAT32)) return sp;
+    if (g.sh != 1 || g.sw != 1 || g.kh * g.kw == 1) return sp;
+    if (g.OH != g.H + 2 * g.ph - g.kh + 1 || g.OW != g.W + 2 * g.pw - g.kw + 1) return sp;  // cover_all adds nothing at stride 1
+    const int64_t it = ItemSize(dtype), epc = 16 / it;
+    const int64_t Wp = (g.W + 2 * g.pw + epc - 1) / epc * epc, Hp = g.H + 2 * g.ph;
+    // worth it when the kw copies are smaller than the kh*kw-fold Im2Col
+    if (g.kw * Hp * Wp * g.C >= static_cast<int64_t>(g.kh) * g.kw * g.OH * g.OW * g.C) return sp;
+    const int64_t xs_elems = static_cast<int64_t>(g.kw) * g.N * g.C * Hp * Wp, gyp_elems = static_cast<int64_t>(g.N) * g.K * g.OH * Wp;
+    if (xs_elems / epc >= (1LL << 32) || gyp_elems / epc >= (1LL << 32)) return sp;  // 32-bit vector indices in the copy kernels
+    sp.a.planes_x = g.N * g.C, sp.a.planes_gy = g.N * g.K;
+    sp.a.H = g.H, sp.a.W = g.W, sp.a.OH = g.OH, sp.a.OW = g.OW, sp.a.Hp = static_cast<int>(Hp), sp.a.Wp = static_cast<int>(Wp);
+    sp.a.ph = g.ph, sp.a.pw = g.pw, sp.a.kw = g.kw;
+    sp.depth = g.OH * Wp;
+    sp.plane = Hp * Wp;
+    sp.xs_bytes = RoundUp256(static_cast<size_t>(xs_elems * it));
+    sp.gyp_bytes = RoundUp256(static_cast<size_t>(gyp_elems * it));
+    sp.partial_bytes = BatchedProductPartialBytes(g.K, static_cast<int64_t>(g.C) * g.kh * g.kw, sp.depth, g.N, dtype);
+    sp.ok = true;
+    return sp;
+}
+
+template <typename T>
+void RunShiftedCopies(const ShiftedArgs& a, hipStream_t stream) {
+    constexpr int VEC = 16 / sizeof(T);
+    const int64_t cap = static_cast<int64_t>(NumCUs()) * 32;
+    auto grid = [&](int64_t n) { int64_t b = (n + 255) / 256; return dim3(static_cast<unsigned>(b > cap ? cap : (b < 1 ? 1 : b))); };
+    const int64_t total_x = static_cast<int64_t>(a.kw) * a.planes_x * (a.Hp * a.Wp / VEC);
+    hipLaunchKernelGGL((ShiftedPlanesKernel<T, VEC>), grid(total_x), dim3(256), 0, stream, a, static_cast<unsigned>(total_x));
+    CheckLaunch("shifted planes (weight gradient)");
+    const int64_t total_gy = static_cast<int64_t>(a.planes_gy) * a.OH * (a.Wp / VEC);
+    hipLaunchKernelGGL((PaddedRowsKernel<T, VEC>), grid(total_gy), dim3(256), 0, stream, a, static_cast<unsigned>(total_gy));
+    CheckLaunch("padded rows (weight gradient)");
+}
 }  // namespace
 
 extern "C" {
@@ -241,7 +349,9 @@ size_t hipcx_conv_grad_weight_workspace_size(const hipcx_array* x, const hipcx_a
         // descriptors alone may not have yet: the answer covers both.
         const size_t direct = BatchedProductPartialBytes(pl.a.K, pl.a.C, static_cast<int64_t>(pl.a.H) * pl.a.W, pl.a.N, gw->dtype) + 256;
         const size_t staged = pl.col_bytes + pl.gyt_bytes + hipcx_dot_workspace_size(&pl.gy_t, &pl.col_view, &out);
-        return std::max(direct, staged);
+        const ShiftedPlan sp = PlanShifted(pl, gw->dtype);
+        const size_t shifted = sp.ok ? sp.xs_bytes + sp.gyp_bytes + sp.partial_bytes + 256 : 0;
+        return std::max(std::max(direct, staged), shifted);
     } catch (...) {
         return 0;
     }
@@ -268,6 +378,24 @@ int hipcx_conv_grad_weight(const hipcx_array* x, const hipcx_array* gy, const in
             LaunchBatchedProduct(gw->dtype, gy->data, pixels, static_cast<int64_t>(pl.a.K) * pixels, x->data, pixels,
                                  static_cast<int64_t>(pl.a.C) * pixels, pl.a.K, pl.a.C, pixels, pl.a.N, gw->data,
                                  partial_bytes ? static_cast<float*>(workspace) : nullptr, AsStream(stream));
+            return;
+        }
+        ShiftedPlan sp = PlanShifted(pl, gw->dtype);
+        if (sp.ok && reinterpret_cast<uintptr_t>(workspace) % 16 == 0 && reinterpret_cast<uintptr_t>(gw->data) % 16 == 0) {
+            const size_t need = sp.xs_bytes + sp.gyp_bytes + sp.partial_bytes;
+            HIPCX_REQUIRE(workspace != nullptr && workspace_bytes >= need, HIPCX_CHAINERX_ERROR,
+                          "conv_grad_weight workspace too small: need " + std::to_string(need) + " bytes");
+            char* ws = static_cast<char*>(workspace);
+            sp.a.x = x->data, sp.a.gy = gy->data;
+            sp.a.xs = ws, sp.a.gyp = ws + sp.xs_bytes;
+            hipStream_t st = AsStream(stream);
+            if (gw->dtype == HIPCX_FLOAT16) RunShiftedCopies<half_t>(sp.a, st);
+            else RunShiftedCopies<float>(sp.a, st);
+            const GradWeightArgs& g = pl.a;
+            LaunchBatchedProduct(gw->dtype, sp.a.gyp, sp.depth, static_cast<int64_t>(g.K) * sp.depth, sp.a.xs, sp.plane,
+                                 static_cast<int64_t>(g.C) * sp.plane, g.K, static_cast<int64_t>(g.C) * g.kh * g.kw, sp.depth, g.N, gw->data,
+                                 sp.partial_bytes ? reinterpret_cast<float*>(ws + sp.xs_bytes + sp.gyp_bytes) : nullptr, st, g.kh, g.kw, sp.a.Wp,
+                                 static_cast<int64_t>(g.N) * g.C * sp.plane);
             return;
         }
         const size_t dot_bytes = hipcx_dot_workspace_size(&pl.gy_t, &pl.col_view, &out);

@@ -48,6 +48,10 @@ struct IGemmArgs {
     // 0: off.  Weight gradients of 1x1 convolutions read gy and x in place this way (one [channels, pixels] matrix per image).
     int batch;
     int64_t x_slice, w_slice;
+    // Filter rows that alias shifted windows of one array (fast kernel; weight gradients of filters larger than 1x1 at stride 1):
+    // row n = (c, r, s), c = n / (w_taps_r * w_taps_s), starts at w + c * wsK + r * w_r_stride + s * w_s_stride.  w_taps_s == 0: off.
+    int w_taps_r, w_taps_s;
+    int64_t w_r_stride, w_s_stride;
 };
 
 constexpr int kRowBytes = 128;           // bytes of the reduction axis per tile row
@@ -360,7 +364,15 @@ __global__ __launch_bounds__(64 * WM * WN) void IGemmFastKernel(IGemmArgs<T> p) 
     for (int i = 0; i < WCH; ++i) {
         int n = n0 + row0 + i * (NT / CPR);
         wvalid[i] = n < p.K;
-        wrow[i] = p.w + static_cast<int64_t>(wvalid[i] ? n : 0) * p.wsK;
+        if (!wvalid[i]) n = 0;
+        if (p.w_taps_s > 0) {
+            const int taps = p.w_taps_r * p.w_taps_s;
+            const int c = n / taps, t = n - c * taps;
+            const int r = t / p.w_taps_s, s = t - r * p.w_taps_s;
+            wrow[i] = p.w + static_cast<int64_t>(c) * p.wsK + r * p.w_r_stride + s * p.w_s_stride;
+        } else {
+            wrow[i] = p.w + static_cast<int64_t>(n) * p.wsK;
+        }
     }
 
     const bool uniform_rs = (p.C % BKE) == 0;

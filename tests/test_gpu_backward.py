@@ -25,6 +25,11 @@ CONV_CASES = [  # N, C, H, W, K, kh, kw, stride, pad, cover_all
     # stride 1: ConvTranspose runs as a forward convolution with flipped filters (padding k - 1 - p)
     (2, 6, 7, 9, 10, 2, 3, 1, (0, 1), False), (2, 8, 9, 9, 12, 5, 5, 1, 2, False), (2, 16, 6, 6, 16, 3, 3, 1, 0, False),
     (4, 64, 14, 14, 128, 3, 3, 1, 1, False), (2, 128, 7, 7, 256, 1, 1, 1, 0, False), (2, 5, 6, 6, 7, 3, 3, 1, 2, False),
+    # filters larger than 1x1 at stride 1 in float16 / float32: ConvGradWeight multiplies gy with windows of shifted zero-padded
+    # copies of x (planes wider than the padded row granule, non-square planes and filters, one-sided padding, a reduction
+    # split over many slices, channel counts that are no multiple of a tile)
+    (2, 64, 28, 28, 64, 3, 3, 1, 1, False), (3, 16, 12, 20, 24, 3, 3, 1, 1, False), (2, 8, 10, 12, 8, 3, 5, 1, (1, 2), False),
+    (16, 64, 14, 14, 64, 3, 3, 1, 1, False), (2, 13, 15, 17, 21, 3, 3, 1, (1, 0), False), (1, 8, 30, 30, 8, 2, 2, 1, 0, False),
 ]
 
 
