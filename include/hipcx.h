@@ -373,7 +373,9 @@ int hipcx_fixed_batch_norm(const hipcx_array* x, const hipcx_array* gamma, const
 
 /* ---- ConvGradWeightKernel CX/kernels/connection.h:34-49 (2-D, C-contiguous NCHW x and gy in gw's float dtype) ----
  * gw[k, c, r, s] = sum over n, oh, ow of gy[n, k, oh, ow] * x[n, c, oh*stride - pad + r, ow*stride - pad + s]: the native
- * backend's TensorDot(gy, Im2Col(x)) (CX/native/native_device/conv.cc:91-124), equal to tolerance (float accumulation). */
+ * backend's TensorDot(gy, Im2Col(x)) (CX/native/native_device/conv.cc:91-124), equal to tolerance (float accumulation).
+ * For filters larger than 1x1 at stride 1 (float16 / float32) the sum runs over zero-padded rows, in which every x value is
+ * also multiplied by zeros of a padded gy: an inf or NaN in x may appear as NaN in filter taps the reference leaves finite. */
 size_t hipcx_conv_grad_weight_workspace_size(const hipcx_array* x, const hipcx_array* gy, const hipcx_array* gw, const int64_t* stride,
                                              const int64_t* pad, int cover_all);
 int hipcx_conv_grad_weight(const hipcx_array* x, const hipcx_array* gy, const int64_t* stride, const int64_t* pad, int cover_all,
