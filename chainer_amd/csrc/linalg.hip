@@ -218,6 +218,29 @@ __device__ __forceinline__ T FromLaneAboveOrSelf(T v) {
     return r;
 }
 
+// v of the lane N places further down in the lane's row of 16, wrapping around inside the row (DPP row_ror)
+template <int N, typename T>
+__device__ __forceinline__ T FromLaneRotated(T v) {
+    constexpr int kWords = (sizeof(T) + 3) / 4;
+    int w[kWords] = {};
+    __builtin_memcpy(w, &v, sizeof(T));
+#pragma unroll
+    for (int i = 0; i < kWords; ++i) w[i] = __builtin_amdgcn_update_dpp(w[i], w[i], 0x120 + N /* row_ror:N */, 0xf, 0xf, false);
+    T r;
+    __builtin_memcpy(&r, w, sizeof(T));
+    return r;
+}
+
+// The sum of v over the wavefront, the same bits in every lane: four rotations inside the rows of 16, then the four row sums.
+template <typename T>
+__device__ __forceinline__ T WaveSum(T v) {
+    v += FromLaneRotated<8>(v);
+    v += FromLaneRotated<4>(v);
+    v += FromLaneRotated<2>(v);
+    v += FromLaneRotated<1>(v);
+    return (ReadLaneT(v, 0) + ReadLaneT(v, 16)) + (ReadLaneT(v, 32) + ReadLaneT(v, 48));
+}
+
 // (v, p) <- the better of (v, p) and (ov, op): the larger magnitude, the earlier position among equals
 template <typename T>
 __device__ __forceinline__ void BetterPivot(T& v, int& p, T ov, int op) {
@@ -1231,13 +1254,13 @@ __device__ __forceinline__ T SvdTolerance(int M) {
     return SqrtT(static_cast<T>(M)) * (std::is_same<T, float>::value ? T(1.2e-7) : T(2.3e-16));
 }
 
-// WAVES wavefronts (one, or a whole workgroup of four with `sums` in LDS) make the columns p and q of g orthogonal (one-sided
-// Jacobi, Hestenes) and apply the same rotation to v.  Columns are contiguous in memory (g: [N][M], v: [N][N], both column by
-// column), so the threads stream the two columns: three dot products, a butterfly reduction that leaves the sums in every lane,
-// the rotation, and the same two columns of g and v again.  Returns whether the pair needed a rotation (the same in every thread).
-template <int WAVES, typename T>
-__device__ __forceinline__ bool SvdRotatePair(T* g, int M, int N, T* v, int p, int q, int compute_uv, int lane, T (*sums)[3]) {
-    constexpr int kLanes = 64 * WAVES;
+// One wavefront makes the columns p and q of g orthogonal (one-sided Jacobi, Hestenes) and applies the same rotation to v.
+// Columns are contiguous in memory (g: [N][M], v: [N][N], both column by column), so the lanes stream the two columns: three dot
+// products, their sums over the wavefront, the rotation, and the same two columns of g and v again.  Returns whether the pair
+// needed a rotation (the same in every lane).
+template <typename T>
+__device__ __forceinline__ bool SvdRotatePair(T* g, int M, int N, T* v, int p, int q, int compute_uv, int lane) {
+    constexpr int kLanes = 64;
     T* gp = g + static_cast<int64_t>(p) * M;
     T* gq = g + static_cast<int64_t>(q) * M;
     T alpha = T(0), beta = T(0), gamma = T(0);
@@ -1246,19 +1269,7 @@ __device__ __forceinline__ bool SvdRotatePair(T* g, int M, int N, T* v, int p, i
         const T a = gp[i], b = gq[i];
         alpha += a * a, beta += b * b, gamma += a * b;
     }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        alpha += __shfl_xor(alpha, o);
-        beta += __shfl_xor(beta, o);
-        gamma += __shfl_xor(gamma, o);
-    }
-    if constexpr (WAVES > 1) {  // the wavefronts' sums meet in LDS; every thread adds them in the same order
-        if ((lane & 63) == 0) sums[lane >> 6][0] = alpha, sums[lane >> 6][1] = beta, sums[lane >> 6][2] = gamma;
-        __syncthreads();
-        alpha = beta = gamma = T(0);
-#pragma unroll
-        for (int w2 = 0; w2 < WAVES; ++w2) alpha += sums[w2][0], beta += sums[w2][1], gamma += sums[w2][2];
-    }
+    alpha = WaveSum(alpha), beta = WaveSum(beta), gamma = WaveSum(gamma);
     const T abs_gamma = gamma >= T(0) ? gamma : -gamma;
     if (!(abs_gamma > SvdTolerance<T>(M) * SqrtT(alpha * beta) && abs_gamma > T(0))) return false;
     const T zeta = (beta - alpha) / (T(2) * gamma);
@@ -1284,15 +1295,161 @@ __device__ __forceinline__ bool SvdRotatePair(T* g, int M, int N, T* v, int p, i
     return true;
 }
 
-// One round of the one-sided Jacobi sweeps of JacobiSvdKernel below, spread over workgroups: one per disjoint column pair of the
-// round.  *rotated becomes 1 when any pair of the sweep needed a rotation.
+// The one-sided Jacobi sweeps of JacobiSvdKernel below, spread over workgroups by blocks of kSvdBlock columns.  A sweep visits
+// every column pair once: one launch with block_round < 0, in which workgroup b runs a round-robin over the pairs inside block b,
+// then one launch per round of a round-robin over the blocks, in which a workgroup owns a pair of blocks (P, Q) and rotates
+// column i of P against column (i + r) mod kSvdBlock of Q in its inner round r -- kSvdBlock disjoint pairs, one per wavefront,
+// with a barrier between inner rounds (the columns stay in global memory; the workgroup's own stores are visible to it after the
+// barrier).  *rotated becomes 1 when any pair of the sweep needed a rotation.
+constexpr int kSvdBlock = 16;
+constexpr int kSvdBlockThreads = 64 * kSvdBlock;
 template <typename T>
-__global__ __launch_bounds__(256) void SvdRoundKernel(T* g, int M, int N, T* v, int round, int compute_uv, int* rotated) {
-    __shared__ T sums[4][3];
-    int p, q;
-    JacobiPair(static_cast<int>(blockIdx.x), round, N, p, q);
-    if (q < 0) return;
-    if (SvdRotatePair<4>(g, M, N, v, p, q, compute_uv, static_cast<int>(threadIdx.x), sums) && threadIdx.x == 0) *rotated = 1;
+__global__ __launch_bounds__(kSvdBlockThreads) void SvdBlockRoundKernel(T* g, int M, int N, T* v, int blocks, int block_round, int compute_uv,
+                                                                        int* rotated) {
+    const int wave = static_cast<int>(threadIdx.x) >> 6, lane = static_cast<int>(threadIdx.x) & 63;
+    bool any = false;
+    if (block_round < 0) {
+        const int base = static_cast<int>(blockIdx.x) * kSvdBlock;
+        const int cols = N - base < kSvdBlock ? N - base : kSvdBlock;
+        const int np = cols + (cols & 1);
+        for (int r = 0; r < np - 1; ++r) {
+            for (int idx = wave; idx < np / 2; idx += kSvdBlock) {
+                int p, q;
+                JacobiPair(idx, r, cols, p, q);
+                if (q >= 0 && SvdRotatePair(g, M, N, v, base + p, base + q, compute_uv, lane)) any = true;
+            }
+            __syncthreads();
+        }
+    } else {
+        int P, Q;
+        JacobiPair(static_cast<int>(blockIdx.x), block_round, blocks, P, Q);
+        if (Q < 0) return;  // the whole workgroup: the dummy block of an odd count
+        const int pb = P * kSvdBlock, qb = Q * kSvdBlock;
+        const int qc = N - qb < kSvdBlock ? N - qb : kSvdBlock;  // P < Q: only Q can be the short last block
+        for (int r = 0; r < kSvdBlock; ++r) {
+            const int j = (wave + r) & (kSvdBlock - 1);
+            if (j < qc && SvdRotatePair(g, M, N, v, pb + wave, qb + j, compute_uv, lane)) any = true;
+            __syncthreads();
+        }
+    }
+    if (any && lane == 0) *rotated = 1;
+}
+
+// The same launch as SvdBlockRoundKernel for matrices short enough that the columns of a block pair fit into LDS
+// (SvdBlockLdsBytes): the workgroup copies its (up to) 2 * kSvdBlock columns of g in, rotates them there -- an inner round then
+// costs LDS traffic and a barrier instead of two trips to memory -- and writes them back.  The rotations are also applied to the
+// columns of a 2 * kSvdBlock square matrix jm that starts as the identity; at the end V's columns of the block pair are replaced
+// by their products with jm (one pass over them: a thread per row keeps the row's entries in registers and reads jm's columns
+// as LDS broadcasts), which is what applying every rotation to V in turn amounts to.
+constexpr int kSvdPair = 2 * kSvdBlock;
+template <typename T>
+size_t SvdBlockLdsBytes(int64_t M) {
+    return static_cast<size_t>(kSvdPair * M + kSvdPair * kSvdPair) * sizeof(T);
+}
+constexpr size_t kSvdBlockLdsMax = 144 * 1024;
+
+// One wavefront makes the LDS columns gp, gq orthogonal and rotates the columns jp, jq of jm with them.
+template <typename T>
+__device__ __forceinline__ bool SvdRotateLdsPair(T* gp, T* gq, int M, T* jp, T* jq, int compute_uv, int lane) {
+    T alpha = T(0), beta = T(0), gamma = T(0);
+#pragma unroll 4
+    for (int i = lane; i < M; i += 64) {
+        const T a = gp[i], b = gq[i];
+        alpha += a * a, beta += b * b, gamma += a * b;
+    }
+    alpha = WaveSum(alpha), beta = WaveSum(beta), gamma = WaveSum(gamma);
+    const T abs_gamma = gamma >= T(0) ? gamma : -gamma;
+    if (!(abs_gamma > SvdTolerance<T>(M) * SqrtT(alpha * beta) && abs_gamma > T(0))) return false;
+    const T zeta = (beta - alpha) / (T(2) * gamma);
+    const T tt = (zeta >= T(0) ? T(1) : T(-1)) / ((zeta >= T(0) ? zeta : -zeta) + SqrtT(T(1) + zeta * zeta));
+    const T c = T(1) / SqrtT(T(1) + tt * tt);
+    const T sn = c * tt;
+#pragma unroll 4
+    for (int i = lane; i < M; i += 64) {
+        const T a = gp[i], b = gq[i];
+        gp[i] = c * a - sn * b;
+        gq[i] = sn * a + c * b;
+    }
+    if (compute_uv && lane < kSvdPair) {
+        const T a = jp[lane], b = jq[lane];
+        jp[lane] = c * a - sn * b;
+        jq[lane] = sn * a + c * b;
+    }
+    return true;
+}
+
+template <typename T>
+__global__ __launch_bounds__(kSvdBlockThreads) void SvdBlockLdsRoundKernel(T* g, int M, int N, T* v, int blocks, int block_round, int compute_uv,
+                                                                           int* rotated) {
+    extern __shared__ __align__(16) char svd_lds[];
+    T* cols = reinterpret_cast<T*>(svd_lds);  // [kSvdPair][M]: local column l is column l of block P, or l - kSvdBlock of block Q
+    T* jm = cols + static_cast<size_t>(kSvdPair) * M;  // [kSvdPair][kSvdPair], column by column
+    const int tid = static_cast<int>(threadIdx.x), wave = tid >> 6, lane = tid & 63;
+    int P = static_cast<int>(blockIdx.x), Q = -1;
+    if (block_round >= 0) {
+        JacobiPair(static_cast<int>(blockIdx.x), block_round, blocks, P, Q);
+        if (Q < 0) return;  // the whole workgroup: the dummy block of an odd count
+    }
+    const int pb = P * kSvdBlock, qb = Q * kSvdBlock;
+    const int pc = N - pb < kSvdBlock ? N - pb : kSvdBlock;
+    const int qc = Q < 0 ? 0 : (N - qb < kSvdBlock ? N - qb : kSvdBlock);
+    auto present = [&](int l) { return l < kSvdBlock ? l < pc : l - kSvdBlock < qc; };
+    auto column = [&](int l) { return static_cast<int64_t>(l < kSvdBlock ? pb + l : qb + l - kSvdBlock); };
+    for (int l = wave; l < kSvdPair; l += kSvdBlock) {
+        if (!present(l)) continue;
+        const T* src = g + column(l) * M;
+        for (int i = lane; i < M; i += 64) cols[static_cast<size_t>(l) * M + i] = src[i];
+    }
+    for (int e = tid; e < kSvdPair * kSvdPair; e += kSvdBlockThreads) jm[e] = (e / kSvdPair == e % kSvdPair) ? T(1) : T(0);
+    __syncthreads();
+    bool any = false;
+    const int players = pc + (pc & 1);
+    const int rounds = block_round < 0 ? players - 1 : kSvdBlock;
+    for (int r = 0; r < rounds; ++r) {
+        int a = -1, b = -1;
+        if (block_round < 0) {
+            if (wave < players / 2) {
+                JacobiPair(wave, r, pc, a, b);
+                if (b < 0) a = -1;
+            }
+        } else {
+            const int j = (wave + r) & (kSvdBlock - 1);
+            if (j < qc) a = wave, b = kSvdBlock + j;
+        }
+        if (a >= 0 && SvdRotateLdsPair(cols + static_cast<size_t>(a) * M, cols + static_cast<size_t>(b) * M, M, jm + a * kSvdPair, jm + b * kSvdPair,
+                                       compute_uv, lane)) {
+            any = true;
+        }
+        __syncthreads();
+    }
+    for (int l = wave; l < kSvdPair; l += kSvdBlock) {
+        if (!present(l)) continue;
+        T* dst = g + column(l) * M;
+        for (int i = lane; i < M; i += 64) dst[i] = cols[static_cast<size_t>(l) * M + i];
+    }
+    if (compute_uv) {
+        struct alignas(16) Quad {
+            T e[4];
+        };
+        for (int row = tid; row < N; row += kSvdBlockThreads) {
+            T vin[kSvdPair];
+#pragma unroll
+            for (int l = 0; l < kSvdPair; ++l) vin[l] = present(l) ? v[column(l) * N + row] : T(0);
+            for (int c = 0; c < kSvdPair; ++c) {
+                if (!present(c)) continue;
+                const Quad* jc = reinterpret_cast<const Quad*>(jm + c * kSvdPair);
+                T acc[4] = {T(0), T(0), T(0), T(0)};
+#pragma unroll
+                for (int l4 = 0; l4 < kSvdPair / 4; ++l4) {
+                    const Quad w4 = jc[l4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc[e] += vin[4 * l4 + e] * w4.e[e];
+                }
+                v[column(c) * N + row] = (acc[0] + acc[1]) + (acc[2] + acc[3]);
+            }
+        }
+    }
+    if (any && lane == 0) *rotated = 1;
 }
 
 // Singular value decomposition by one-sided Jacobi rotations (Hestenes), one workgroup.  g: the [M, N] matrix (M >= N) stored column
@@ -1302,7 +1459,7 @@ __global__ __launch_bounds__(256) void SvdRoundKernel(T* g, int M, int N, T* v, 
 // Results leave in descending order of the singular value: s[rank], tall(i, rank) = g(i, j) / sigma_j, sq(i, rank) = v(i, j), both
 // addressed through (row, col) element strides so that the caller decides which of u / vt each one is and how it is transposed.
 // Columns whose singular value is zero are left for the completion kernel; *first_fill receives the number of columns that are
-// final.  With do_sweeps = 0 the rotations have been applied already (SvdRoundKernel) and only the singular values, their order
+// final.  With do_sweeps = 0 the rotations have been applied already (SvdBlockRoundKernel) and only the singular values, their order
 // and the outputs are produced.
 template <typename T>
 __global__ __launch_bounds__(kLinalgThreads) void JacobiSvdKernel(T* g, int M, int N, T* v, T* sigma, int* rank, T* s_out, int64_t s_stride,
@@ -1323,7 +1480,7 @@ __global__ __launch_bounds__(kLinalgThreads) void JacobiSvdKernel(T* g, int M, i
             for (int idx = tid >> 6; idx < half; idx += kGroups) {  // a pair per wavefront
                 int p, q;
                 JacobiPair(idx, round, N, p, q);
-                if (q >= 0 && SvdRotatePair<1>(g, M, N, v, p, q, compute_uv, tid & 63, static_cast<T(*)[3]>(nullptr))) rotated = 1;  // every writer stores the same value
+                if (q >= 0 && SvdRotatePair(g, M, N, v, p, q, compute_uv, tid & 63)) rotated = 1;  // every writer stores the same value
             }
             __syncthreads();  // the pairs of a round are disjoint; the next round pairs the columns anew
         }
@@ -1468,7 +1625,7 @@ void CopyInto(const hipcx_array* src, const hipcx_array* dst, void* stream, cons
 // Raises a kernel's limit of dynamic LDS to 150 KiB, once per device and kernel (`slot` tells the kernels that share this function
 // apart); several host threads may get here at once.
 void AllowLargeLds(const void* kernel, int slot) {
-    constexpr int kMaxDevices = 64, kSlots = 2;
+    constexpr int kMaxDevices = 64, kSlots = 4;
     static std::mutex mu;
     static bool done[kSlots][kMaxDevices] = {};
     int dev = 0;
@@ -1898,19 +2055,31 @@ int hipcx_svd(const hipcx_array* a, const hipcx_array* u, const hipcx_array* s, 
             int* first_fill = rank + N;
             const bool spread = N > kSvdOneWorkgroupMaxColumns;
             if (spread) {
-                // the sweeps as one launch per round over many workgroups; the host reads after every sweep whether it rotated anything
+                // the sweeps as one launch per round of column blocks; the host reads after every sweep whether it rotated anything
                 int* rotated = reinterpret_cast<int*>(flags_mem);
                 HIPCX_CHECK_HIP(hipMemsetAsync(rotated, 0, kSvdMaxSweeps * sizeof(int), st));
                 if (compute_uv) {
                     hipLaunchKernelGGL(IdentityFillKernel<T>, dim3(static_cast<unsigned>((N * N + 255) / 256)), dim3(256), 0, st,
                                        reinterpret_cast<T*>(v_mem), static_cast<int>(N));
                 }
-                const int np = static_cast<int>(N + (N & 1));
-                const unsigned blocks = static_cast<unsigned>(np / 2);
+                const int blocks = static_cast<int>((N + kSvdBlock - 1) / kSvdBlock);
+                const int players = blocks + (blocks & 1);
+                const size_t lds_bytes = SvdBlockLdsBytes<T>(M);
+                const bool in_lds = lds_bytes <= kSvdBlockLdsMax;
+                // beyond the 64 KiB a launch gets unasked, the kernel is told once per device that it may have more
+                if (in_lds && lds_bytes > 60 * 1024) AllowLargeLds(reinterpret_cast<const void*>(SvdBlockLdsRoundKernel<T>), std::is_same<T, float>::value ? 2 : 3);
                 for (int sweep = 0; sweep < kSvdMaxSweeps; ++sweep) {
-                    for (int round = 0; round < np - 1; ++round) {
-                        hipLaunchKernelGGL(SvdRoundKernel<T>, dim3(blocks), dim3(256), 0, st, reinterpret_cast<T*>(g_mem), static_cast<int>(M),
-                                           static_cast<int>(N), reinterpret_cast<T*>(v_mem), round, compute_uv ? 1 : 0, rotated + sweep);
+                    for (int round = -1; round < players - 1; ++round) {  // -1: the pairs inside every block
+                        const dim3 grid(static_cast<unsigned>(round < 0 ? blocks : players / 2));
+                        if (in_lds) {
+                            hipLaunchKernelGGL(SvdBlockLdsRoundKernel<T>, grid, dim3(kSvdBlockThreads), lds_bytes, st, reinterpret_cast<T*>(g_mem),
+                                               static_cast<int>(M), static_cast<int>(N), reinterpret_cast<T*>(v_mem), blocks, round, compute_uv ? 1 : 0,
+                                               rotated + sweep);
+                        } else {
+                            hipLaunchKernelGGL(SvdBlockRoundKernel<T>, grid, dim3(kSvdBlockThreads), 0, st, reinterpret_cast<T*>(g_mem),
+                                               static_cast<int>(M), static_cast<int>(N), reinterpret_cast<T*>(v_mem), blocks, round, compute_uv ? 1 : 0,
+                                               rotated + sweep);
+                        }
                     }
                     int any = 0;
                     HIPCX_CHECK_HIP(hipMemcpyAsync(&any, rotated + sweep, sizeof(int), hipMemcpyDeviceToHost, st));
