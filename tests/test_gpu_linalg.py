@@ -343,6 +343,20 @@ def test_decompositions_spread_over_workgroups_at_larger_sizes():
         assert np.abs(sv - O.svd(a, compute_uv=False)).max() <= tol * max(m, n) * 4
         assert np.abs((u * sv) @ vt - a).max() <= tol * max(m, n) * 4
         assert np.abs(u.T @ u - np.eye(k)).max() <= tol * max(m, n) * 4 and np.abs(vt @ vt.T - np.eye(k)).max() <= tol * max(m, n) * 4
+    # svd of matrices whose column-block pairs do not fit into LDS (the rotations then run on the columns in memory), a short last
+    # block of columns and an odd number of blocks; wide input (the transposed problem) and singular values only as well
+    for dt, (m, n), rtol in (('float32', (1300, 70), 1e-4), ('float64', (700, 90), 1e-12), ('float64', (90, 700), 1e-12)):
+        a = rng.standard_normal((m, n)).astype(dt)
+        k = min(m, n)
+        u, sv, vt = chx.svd(chx.array(a), full_matrices=False)
+        u, sv, vt = u.get().astype(np.float64), sv.get().astype(np.float64), vt.get().astype(np.float64)
+        bound = rtol * max(m, n) * 4
+        assert np.abs(sv - O.svd(a, compute_uv=False)).max() <= bound and np.all(np.diff(sv) <= 0)
+        assert np.abs((u * sv) @ vt - a).max() <= bound
+        assert np.abs(u.T @ u - np.eye(k)).max() <= bound and np.abs(vt @ vt.T - np.eye(k)).max() <= bound
+        only = chx.svd(chx.array(a), compute_uv=False)
+        only = only[1] if isinstance(only, (tuple, list)) else only
+        assert np.abs(only.get().astype(np.float64) - sv).max() <= bound
 
 
 def test_one_workgroup_limits():
