@@ -718,156 +718,13 @@ __global__ __launch_bounds__(256) void EighNormsKernel(const T* s, int n, T* par
     }
 }
 
-// The rotation (c, sn) of pair `idx` of `round` from the right, applied to one or two rows of s held in LDS (entries p and q of that
-// pair; row_b may be null); the entry a rotation annihilates is stored as an exact zero (see JacobiEighKernel).  ra / rb are the rows'
-// indices.
-template <typename T>
-__device__ __forceinline__ void EighRotateRowEntry(T* row_a, int ra, T* row_b, int rb, int n, int round, int idx, T c, T sn) {
-    int p, q;
-    JacobiPair(idx, round, n, p, q);
-    if (q < 0 || sn == T(0)) return;
-    {
-        const T a = row_a[p], b = row_a[q];
-        row_a[p] = ra == q ? T(0) : c * a - sn * b;
-        row_a[q] = ra == p ? T(0) : sn * a + c * b;
-    }
-    if (row_b != nullptr) {
-        const T a = row_b[p], b = row_b[q];
-        row_b[p] = rb == q ? T(0) : c * a - sn * b;
-        row_b[q] = rb == p ? T(0) : sn * a + c * b;
-    }
-}
-
-// ... of every pair of the round; the `lanes` threads that share the rows each take every lanes-th pair.
-template <typename T>
-__device__ __forceinline__ void EighRotateRowEntries(T* row_a, int ra, T* row_b, int rb, int n, int round, const T* cs, int lane, int lanes) {
-    for (int idx = lane; idx < (n + 1) / 2; idx += lanes) EighRotateRowEntry(row_a, ra, row_b, rb, n, round, idx, cs[2 * idx], cs[2 * idx + 1]);
-}
-
-// A round of the two-sided Jacobi sweeps of JacobiEighKernel below, spread over workgroups, one per pair (p, q).
-// Rotations from the left change rows p and q; rotations from the right change columns, but every row can apply them to itself
-// once the round's (cosine, sine) pairs are known.  So a workgroup takes rows p and q of s into LDS, first applies the previous
-// round's rotations from the right to them (prev_round >= 0, from cs_prev), then has everything it needs for its own rotation
-// (s[p][p], s[q][q], s[p][q] lie in these rows): it leaves (cosine, sine) in cs_next[2 idx ..] and applies the rotation from the
-// left to the two rows of s and of vt (the accumulated rotations, transposed: row i is eigenvector i).  The rotations of the last
-// round from the right are EighColumnsKernel's.
-template <typename T>
-__global__ __launch_bounds__(256) void EighRoundKernel(T* s, T* vt, int n, int prev_round, int round, int compute_v, const T* cs_prev, T* cs_next) {
-    extern __shared__ __align__(16) char eigh_round_lds[];
-    T* row_p = reinterpret_cast<T*>(eigh_round_lds);
-    T* row_q = row_p + n;
-    const int lane = threadIdx.x;
-    constexpr int kLanes = 256;
-    const int idx = static_cast<int>(blockIdx.x);
-    int p, q;
-    JacobiPair(idx, round, n, p, q);  // q = -1: p sits out this round, but still owes the previous round's rotations
-    T* sp = s + static_cast<int64_t>(p) * n;
-    T* sq = s + static_cast<int64_t>(q < 0 ? p : q) * n;
-    // Everything this workgroup reads from memory is asked for up front, so that the loads travel together: its two rows of s, the
-    // previous round's rotations its threads will apply (the first kAhead pairs of each thread) and its two rows of vt (the first
-    // kAhead entries of each thread); longer rows fetch the rest when they get there.
-    constexpr int kAhead = 4;
-    const int half = (n + 1) / 2;
-    T ahead_c[kAhead], ahead_s[kAhead], ahead_vp[kAhead], ahead_vq[kAhead];
-    T* vp = vt + static_cast<int64_t>(p) * n;
-    T* vq = vt + static_cast<int64_t>(q < 0 ? p : q) * n;
-#pragma unroll
-    for (int u = 0; u < kAhead; ++u) {
-        const int other = lane + u * kLanes;
-        const bool have_pair = prev_round >= 0 && other < half;
-        ahead_c[u] = have_pair ? cs_prev[2 * other] : T(1);
-        ahead_s[u] = have_pair ? cs_prev[2 * other + 1] : T(0);
-        const bool have_v = compute_v && q >= 0 && other < n;
-        ahead_vp[u] = have_v ? vp[other] : T(0);
-        ahead_vq[u] = have_v ? vq[other] : T(0);
-    }
-    for (int i = lane; i < n; i += kLanes) {
-        row_p[i] = sp[i];
-        if (q >= 0) row_q[i] = sq[i];
-    }
-    __syncthreads();
-    if (prev_round >= 0) {
-        T* second = q >= 0 ? row_q : static_cast<T*>(nullptr);
-#pragma unroll
-        for (int u = 0; u < kAhead; ++u) {
-            const int other = lane + u * kLanes;
-            if (other < half) EighRotateRowEntry(row_p, p, second, q, n, prev_round, other, ahead_c[u], ahead_s[u]);
-        }
-        for (int other = lane + kAhead * kLanes; other < half; other += kLanes) {
-            EighRotateRowEntry(row_p, p, second, q, n, prev_round, other, cs_prev[2 * other], cs_prev[2 * other + 1]);
-        }
-        __syncthreads();
-    }
-    T c = T(1), sn = T(0);
-    if (q >= 0) {
-        const T apq = row_p[q];
-        if (apq != T(0)) {
-            const T app = row_p[p], aqq = row_q[q];
-            const T tau = (aqq - app) / (T(2) * apq);
-            const T tt = (tau >= T(0) ? T(1) : T(-1)) / ((tau >= T(0) ? tau : -tau) + SqrtT(T(1) + tau * tau));
-            c = T(1) / SqrtT(T(1) + tt * tt);
-            sn = tt * c;
-        }
-    }
-    if (lane == 0) cs_next[2 * idx] = c, cs_next[2 * idx + 1] = sn;
-    if (sn == T(0)) {  // the same in every thread
-        if (prev_round >= 0) {
-            for (int i = lane; i < n; i += kLanes) {
-                sp[i] = row_p[i];
-                if (q >= 0) sq[i] = row_q[i];
-            }
-        }
-        return;
-    }
-    for (int i = lane; i < n; i += kLanes) {
-        const T a = row_p[i], b = row_q[i];
-        sp[i] = c * a - sn * b;
-        sq[i] = sn * a + c * b;
-    }
-    if (compute_v) {
-#pragma unroll
-        for (int u = 0; u < kAhead; ++u) {
-            const int i = lane + u * kLanes;
-            if (i < n) {
-                vp[i] = c * ahead_vp[u] - sn * ahead_vq[u];
-                vq[i] = sn * ahead_vp[u] + c * ahead_vq[u];
-            }
-        }
-        for (int i = lane + kAhead * kLanes; i < n; i += kLanes) {
-            const T a = vp[i], b = vq[i];
-            vp[i] = c * a - sn * b;
-            vq[i] = sn * a + c * b;
-        }
-    }
-}
-
-// The rotations of `round` from the right for the whole matrix (after the last round of a sweep): each of a workgroup's
-// wavefronts (up to four: as many rows as fit in 64 KiB of LDS) takes one row of s into LDS, rotates the entries (p, q) of every
-// pair there and writes the row back.
-template <typename T>
-__global__ __launch_bounds__(256) void EighColumnsKernel(T* s, int n, int round, const T* cs) {
-    extern __shared__ __align__(16) char eigh_rows_lds[];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    T* row = reinterpret_cast<T*>(eigh_rows_lds) + static_cast<int64_t>(wave) * n;
-    const int r = static_cast<int>(blockIdx.x * (blockDim.x >> 6)) + wave;
-    const bool valid = r < n;
-    if (valid) {
-        for (int i = lane; i < n; i += 64) row[i] = s[static_cast<int64_t>(r) * n + i];
-    }
-    __syncthreads();
-    if (valid) EighRotateRowEntries(row, r, static_cast<T*>(nullptr), -1, n, round, cs, lane, 64);
-    __syncthreads();
-    if (valid) {
-        for (int i = lane; i < n; i += 64) s[static_cast<int64_t>(r) * n + i] = row[i];
-    }
-}
-
 // Symmetric eigendecomposition by cyclic Jacobi rotations, one workgroup.  s: [n, n] row-major, symmetric on entry, destroyed
 // (its diagonal converges to the eigenvalues); v: [n, n] accumulates the rotations (eigenvectors as columns); w: the eigenvalues in
 // ascending order, with the columns of v permuted to match (LAPACK syevd's order, CX/native/native_device/linalg.cc:602-660).
 // A sweep visits all pairs in n - 1 rounds of n / 2 disjoint pairs (round-robin pairing), so the rotations of a round apply in
-// parallel: first to the columns of s and v, then to the rows of s.  With do_sweeps = 0 the sweeps have been done already
-// (EighRowsKernel / EighColumnsKernel, which keep the rotations transposed in v_scratch) and only the order and the outputs are produced.
+// parallel: first to the columns of s and v, then to the rows of s.  With do_sweeps = 0 the decomposition has been done already
+// (one-sided block sweeps, which leave the eigenvalues on the diagonal of s and the eigenvectors transposed in v_scratch) and only the
+// order and the outputs are produced.
 template <typename T>
 __global__ __launch_bounds__(kLinalgThreads) void JacobiEighKernel(T* s, T* v, T* w, int n, int compute_v, int64_t v_row, int64_t v_col,
                                                                    int64_t w_stride, T* v_scratch, int do_sweeps) {
@@ -981,6 +838,43 @@ __global__ __launch_bounds__(kLinalgThreads) void JacobiEighKernel(T* s, T* v, T
                 v[r * v_row + rank * v_col] = do_sweeps ? v_scratch[static_cast<int64_t>(r) * n + i] : v_scratch[static_cast<int64_t>(i) * n + r];
             }
         }
+    }
+}
+
+// s[i][i] += shift
+template <typename T>
+__global__ __launch_bounds__(256) void EighShiftKernel(T* s, int n, T shift) {
+    const int i = static_cast<int>(blockIdx.x) * 256 + static_cast<int>(threadIdx.x);
+    if (i < n) s[static_cast<int64_t>(i) * n + i] += shift;
+}
+
+// Eigenvalue j as the Rayleigh quotient of the original matrix a0 ([n, n], symmetric) with row j of vt (the eigenvector, as the
+// one-sided sweeps leave it): lambda_j = (v . a0 v) / (v . v), stored at s[j][j] where the output pass of JacobiEighKernel looks for
+// it.  Its error is of second order in the eigenvector's, and the norm that thousands of rotations leave slightly off one cancels.
+// A workgroup per eigenvector, a wavefront per row of a0.
+template <typename T>
+__global__ __launch_bounds__(256) void EighRayleighKernel(const T* a0, const T* vt, int n, T* s) {
+    extern __shared__ __align__(16) char rayleigh_lds[];
+    T* vj = reinterpret_cast<T*>(rayleigh_lds);  // [n]
+    __shared__ T part[4][2];
+    const int j = static_cast<int>(blockIdx.x), tid = static_cast<int>(threadIdx.x), wave = tid >> 6, lane = tid & 63;
+    for (int i = tid; i < n; i += 256) vj[i] = vt[static_cast<int64_t>(j) * n + i];
+    __syncthreads();
+    T num = T(0), den = T(0);
+    for (int i = wave; i < n; i += 4) {
+        const T* row = a0 + static_cast<int64_t>(i) * n;
+        T dot = T(0);
+        for (int c = lane; c < n; c += 64) dot += row[c] * vj[c];
+        dot = WaveSum(dot);
+        num += vj[i] * dot;
+        den += vj[i] * vj[i];
+    }
+    if (lane == 0) part[wave][0] = num, part[wave][1] = den;
+    __syncthreads();
+    if (tid == 0) {
+        const T nn = (part[0][0] + part[1][0]) + (part[2][0] + part[3][0]);
+        const T dd = (part[0][1] + part[1][1]) + (part[2][1] + part[3][1]);
+        s[static_cast<int64_t>(j) * n + j] = nn / dd;
     }
 }
 
@@ -1638,6 +1532,37 @@ void AllowLargeLds(const void* kernel, int slot) {
     }
 }
 
+// The one-sided Jacobi sweeps over g ([N][M], column by column) as launches of column-block rounds, until a sweep rotates nothing:
+// the host reads one flag per sweep (a stream wait).  v ([N][N], column by column) starts as the identity and takes the rotations
+// when compute_uv is set.  rotated: kSvdMaxSweeps ints of device memory.
+template <typename T>
+void RunBlockJacobiSweeps(T* g, int64_t M, int64_t N, T* v, bool compute_uv, int* rotated, hipStream_t st) {
+    HIPCX_CHECK_HIP(hipMemsetAsync(rotated, 0, kSvdMaxSweeps * sizeof(int), st));
+    if (compute_uv) hipLaunchKernelGGL(IdentityFillKernel<T>, dim3(static_cast<unsigned>((N * N + 255) / 256)), dim3(256), 0, st, v, static_cast<int>(N));
+    const int blocks = static_cast<int>((N + kSvdBlock - 1) / kSvdBlock);
+    const int players = blocks + (blocks & 1);
+    const size_t lds_bytes = SvdBlockLdsBytes<T>(M);
+    const bool in_lds = lds_bytes <= kSvdBlockLdsMax;
+    // beyond the 64 KiB a launch gets unasked, the kernel is told once per device that it may have more
+    if (in_lds && lds_bytes > 60 * 1024) AllowLargeLds(reinterpret_cast<const void*>(SvdBlockLdsRoundKernel<T>), std::is_same<T, float>::value ? 2 : 3);
+    for (int sweep = 0; sweep < kSvdMaxSweeps; ++sweep) {
+        for (int round = -1; round < players - 1; ++round) {  // -1: the pairs inside every block
+            const dim3 grid(static_cast<unsigned>(round < 0 ? blocks : players / 2));
+            if (in_lds) {
+                hipLaunchKernelGGL(SvdBlockLdsRoundKernel<T>, grid, dim3(kSvdBlockThreads), lds_bytes, st, g, static_cast<int>(M), static_cast<int>(N), v,
+                                   blocks, round, compute_uv ? 1 : 0, rotated + sweep);
+            } else {
+                hipLaunchKernelGGL(SvdBlockRoundKernel<T>, grid, dim3(kSvdBlockThreads), 0, st, g, static_cast<int>(M), static_cast<int>(N), v, blocks,
+                                   round, compute_uv ? 1 : 0, rotated + sweep);
+            }
+        }
+        int any = 0;
+        HIPCX_CHECK_HIP(hipMemcpyAsync(&any, rotated + sweep, sizeof(int), hipMemcpyDeviceToHost, st));
+        HIPCX_CHECK_HIP(hipStreamSynchronize(st));
+        if (!any) break;
+    }
+}
+
 // Largest matrix the blocked LU takes: its panel kernel keeps all rows of a panel in the registers of one workgroup.
 constexpr int64_t kLuBlockedMaxN = 8192;
 
@@ -1796,10 +1721,18 @@ int hipcx_cholesky(const hipcx_array* a, const hipcx_array* out, int32_t* error_
     });
 }
 
+namespace {
+// where the one-sided method keeps the matrix itself: behind the working copy, the rotations, the (cosine, sine) pairs of two rounds
+// and the partial norms of a sweep
+size_t EighOriginalOffset(int64_t n) {
+    const size_t front = static_cast<size_t>(n) * static_cast<size_t>(n) * 8 * 2 + (2 * static_cast<size_t>(n) + 4 + 2 * kEighNormBlocks) * 8;
+    return (front + 255) / 256 * 256;
+}
+}  // namespace
+
 size_t hipcx_syevd_workspace_size(const hipcx_array* a) {
     if (a == nullptr || a->ndim != 2 || a->shape[0] < 0) return 0;
-    // the working copy and the rotations; the (cosine, sine) pairs of two rounds and the partial norms of a sweep
-    return static_cast<size_t>(a->shape[0]) * static_cast<size_t>(a->shape[0]) * 8 * 2 + (2 * static_cast<size_t>(a->shape[0]) + 4 + 2 * kEighNormBlocks) * 8;
+    return EighOriginalOffset(a->shape[0]) + static_cast<size_t>(a->shape[0]) * static_cast<size_t>(a->shape[0]) * 8;
 }
 
 int hipcx_syevd(const hipcx_array* a, const hipcx_array* w, const hipcx_array* v, char uplo, int compute_v, void* workspace,
@@ -1832,33 +1765,31 @@ int hipcx_syevd(const hipcx_array* a, const hipcx_array* w, const hipcx_array* v
                                a->strides[1] / it, s, static_cast<int>(n), upper);
             const bool spread = n > kEighOneWorkgroupMaxN;
             if (spread) {
-                // the sweeps as one launch per round over many workgroups (and one more per sweep for the last round's rotations
-                // from the right); before every sweep the host reads how much is left off the diagonal
-                const int64_t half = (n + 1) / 2;
-                T* cs = reinterpret_cast<T*>(ws + 2 * n * n * it);  // two sets of (cosine, sine) pairs, used in turn
-                T* partial = cs + 4 * half;
+                // Above kEighOneWorkgroupMaxN rows: one-sided sweeps on the shifted matrix.  With shift = |A|_F >= |A|_2 the matrix
+                // A + shift I is positive semidefinite, so making its columns orthogonal by rotations from the right (the SVD's block
+                // rounds) gives (A + shift I) V = V diag(lambda + shift) with the rotations' product V orthogonal by construction --
+                // the eigenvectors; pairs +-lambda, which have equal singular values in A itself, are apart after the shift.  The
+                // eigenvalues are then taken as Rayleigh quotients of the original matrix with those vectors.  A symmetric matrix is
+                // its own column-by-column copy, and the product of the rotations comes out transposed, as the output pass expects
+                // it from sweeps run outside JacobiEighKernel.
+                T* cs = reinterpret_cast<T*>(ws + 2 * n * n * it);  // the sweeps' flags
+                T* partial = cs + 4 * ((n + 1) / 2);
                 std::vector<T> sums(2 * kEighNormBlocks);
-                if (compute_v) hipLaunchKernelGGL(IdentityFillKernel<T>, dim3(blocks), dim3(256), 0, st, vs, static_cast<int>(n));
-                const int64_t rows_per_block = std::max<int64_t>(1, std::min<int64_t>(4, 65536 / (n * it)));
-                const double eps = std::is_same<T, float>::value ? 4e-7 : 1e-15;  // as in JacobiEighKernel
-                double total_norm = 0.0;
-                for (int sweep = 0; sweep < kEighMaxSweeps; ++sweep) {
-                    hipLaunchKernelGGL(EighNormsKernel<T>, dim3(kEighNormBlocks), dim3(256), 0, st, s, static_cast<int>(n), partial);
-                    HIPCX_CHECK_HIP(hipMemcpyAsync(sums.data(), partial, sums.size() * sizeof(T), hipMemcpyDeviceToHost, st));
-                    HIPCX_CHECK_HIP(hipStreamSynchronize(st));
-                    double off = 0.0, all = 0.0;
-                    for (int b2 = 0; b2 < kEighNormBlocks; ++b2) off += static_cast<double>(sums[2 * b2]), all += static_cast<double>(sums[2 * b2 + 1]);
-                    if (sweep == 0) total_norm = all;
-                    if (!(off > eps * eps * total_norm)) break;
-                    const int rounds = static_cast<int>(n + (n & 1)) - 1;
-                    for (int round = 0; round < rounds; ++round) {
-                        hipLaunchKernelGGL(EighRoundKernel<T>, dim3(static_cast<unsigned>(half)), dim3(256), static_cast<size_t>(2 * n * it), st, s, vs,
-                                           static_cast<int>(n), round - 1, round, compute_v ? 1 : 0, cs + ((round + 1) & 1) * 2 * half,
-                                           cs + (round & 1) * 2 * half);
-                    }
-                    hipLaunchKernelGGL(EighColumnsKernel<T>, dim3(static_cast<unsigned>((n + rows_per_block - 1) / rows_per_block)),
-                                       dim3(static_cast<unsigned>(64 * rows_per_block)), static_cast<size_t>(rows_per_block * n * it), st, s,
-                                       static_cast<int>(n), rounds - 1, cs + ((rounds - 1) & 1) * 2 * half);
+                hipLaunchKernelGGL(EighNormsKernel<T>, dim3(kEighNormBlocks), dim3(256), 0, st, s, static_cast<int>(n), partial);
+                HIPCX_CHECK_HIP(hipMemcpyAsync(sums.data(), partial, sums.size() * sizeof(T), hipMemcpyDeviceToHost, st));
+                HIPCX_CHECK_HIP(hipStreamSynchronize(st));
+                double all = 0.0;
+                for (int b2 = 0; b2 < kEighNormBlocks; ++b2) all += static_cast<double>(sums[2 * b2 + 1]);
+                const T shift = static_cast<T>(std::sqrt(all));
+                if (shift > T(0) && std::isfinite(static_cast<double>(shift))) {
+                    T* a0 = reinterpret_cast<T*>(ws + EighOriginalOffset(n));  // the matrix itself, for the eigenvalues
+                    HIPCX_CHECK_HIP(hipMemcpyAsync(a0, s, static_cast<size_t>(n * n * it), hipMemcpyDeviceToDevice, st));
+                    hipLaunchKernelGGL(EighShiftKernel<T>, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, st, s, static_cast<int>(n), shift);
+                    RunBlockJacobiSweeps(s, n, n, vs, true, reinterpret_cast<int*>(cs), st);
+                    hipLaunchKernelGGL(EighRayleighKernel<T>, dim3(static_cast<unsigned>(n)), dim3(256), static_cast<size_t>(n * it), st, a0, vs,
+                                       static_cast<int>(n), s);
+                } else if (compute_v) {  // the zero matrix (or a non-finite one, whose values pass through): every vector is an eigenvector
+                    hipLaunchKernelGGL(IdentityFillKernel<T>, dim3(blocks), dim3(256), 0, st, vs, static_cast<int>(n));
                 }
             }
             hipLaunchKernelGGL(JacobiEighKernel<T>, dim3(1), dim3(kLinalgThreads), lds, st, s, static_cast<T*>(v->data),
@@ -2055,37 +1986,7 @@ int hipcx_svd(const hipcx_array* a, const hipcx_array* u, const hipcx_array* s, 
             int* first_fill = rank + N;
             const bool spread = N > kSvdOneWorkgroupMaxColumns;
             if (spread) {
-                // the sweeps as one launch per round of column blocks; the host reads after every sweep whether it rotated anything
-                int* rotated = reinterpret_cast<int*>(flags_mem);
-                HIPCX_CHECK_HIP(hipMemsetAsync(rotated, 0, kSvdMaxSweeps * sizeof(int), st));
-                if (compute_uv) {
-                    hipLaunchKernelGGL(IdentityFillKernel<T>, dim3(static_cast<unsigned>((N * N + 255) / 256)), dim3(256), 0, st,
-                                       reinterpret_cast<T*>(v_mem), static_cast<int>(N));
-                }
-                const int blocks = static_cast<int>((N + kSvdBlock - 1) / kSvdBlock);
-                const int players = blocks + (blocks & 1);
-                const size_t lds_bytes = SvdBlockLdsBytes<T>(M);
-                const bool in_lds = lds_bytes <= kSvdBlockLdsMax;
-                // beyond the 64 KiB a launch gets unasked, the kernel is told once per device that it may have more
-                if (in_lds && lds_bytes > 60 * 1024) AllowLargeLds(reinterpret_cast<const void*>(SvdBlockLdsRoundKernel<T>), std::is_same<T, float>::value ? 2 : 3);
-                for (int sweep = 0; sweep < kSvdMaxSweeps; ++sweep) {
-                    for (int round = -1; round < players - 1; ++round) {  // -1: the pairs inside every block
-                        const dim3 grid(static_cast<unsigned>(round < 0 ? blocks : players / 2));
-                        if (in_lds) {
-                            hipLaunchKernelGGL(SvdBlockLdsRoundKernel<T>, grid, dim3(kSvdBlockThreads), lds_bytes, st, reinterpret_cast<T*>(g_mem),
-                                               static_cast<int>(M), static_cast<int>(N), reinterpret_cast<T*>(v_mem), blocks, round, compute_uv ? 1 : 0,
-                                               rotated + sweep);
-                        } else {
-                            hipLaunchKernelGGL(SvdBlockRoundKernel<T>, grid, dim3(kSvdBlockThreads), 0, st, reinterpret_cast<T*>(g_mem),
-                                               static_cast<int>(M), static_cast<int>(N), reinterpret_cast<T*>(v_mem), blocks, round, compute_uv ? 1 : 0,
-                                               rotated + sweep);
-                        }
-                    }
-                    int any = 0;
-                    HIPCX_CHECK_HIP(hipMemcpyAsync(&any, rotated + sweep, sizeof(int), hipMemcpyDeviceToHost, st));
-                    HIPCX_CHECK_HIP(hipStreamSynchronize(st));
-                    if (!any) break;
-                }
+                RunBlockJacobiSweeps(reinterpret_cast<T*>(g_mem), M, N, reinterpret_cast<T*>(v_mem), compute_uv != 0, reinterpret_cast<int*>(flags_mem), st);
             }
             hipLaunchKernelGGL(JacobiSvdKernel<T>, dim3(1), dim3(kLinalgThreads), 0, st, reinterpret_cast<T*>(g_mem), static_cast<int>(M),
                                static_cast<int>(N), reinterpret_cast<T*>(v_mem), reinterpret_cast<T*>(sigma_mem), rank, static_cast<T*>(s->data),

@@ -396,10 +396,12 @@ int hipcx_cholesky(const hipcx_array* a, const hipcx_array* out, int32_t* error_
 /* ---- SyevdKernel CX/kernels/linalg.h:45-48 (float32 / float64, a 2-D and square) ----
  * Eigenvalues w (ascending) and, when compute_v, eigenvectors v (as columns) of the symmetric matrix held in a's `uplo` triangle
  * ('U' / 'L', either case; the other triangle is never read), as LAPACK syevd gives them to the native backend
- * (CX/native/native_device/linalg.cc:602-660).  Cyclic Jacobi rotations: eigenvalues agree with LAPACK's to rounding, eigenvectors
- * up to the sign of each column (and up to a rotation inside an eigenspace of a repeated eigenvalue).  Up to 64 rows everything
- * runs in one workgroup; beyond that a round of rotations is two launches over many workgroups and the call waits for the stream
- * once per sweep to read how much is left off the diagonal (so it cannot be captured into a graph).
+ * (CX/native/native_device/linalg.cc:602-660).  Jacobi rotations: eigenvalues agree with LAPACK's to rounding, eigenvectors
+ * up to the sign of each column (and up to a rotation inside an eigenspace of a repeated eigenvalue).  Up to 64 rows a two-sided
+ * cyclic Jacobi runs in one workgroup; beyond that the columns of A + |A|_F I are made orthogonal by the one-sided block sweeps
+ * of hipcx_svd (the rotations' product holds the eigenvectors, the eigenvalues are their Rayleigh quotients with A), and the
+ * call waits for the stream once for the norm and once per sweep to read whether anything was rotated (so it cannot be captured
+ * into a graph).
  * w: [n], v: [n, n], any strides, a's dtype.  Workspace: hipcx_syevd_workspace_size(a) bytes.  n <= 4096. */
 size_t hipcx_syevd_workspace_size(const hipcx_array* a);
 int hipcx_syevd(const hipcx_array* a, const hipcx_array* w, const hipcx_array* v, char uplo, int compute_v, void* workspace,

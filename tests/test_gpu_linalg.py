@@ -359,6 +359,39 @@ def test_decompositions_spread_over_workgroups_at_larger_sizes():
         assert np.abs(only.get().astype(np.float64) - sv).max() <= bound
 
 
+def test_eigh_above_one_workgroup_on_hard_spectra():
+    """eigh above 64 rows runs the SVD's one-sided block sweeps on A + |A|_F I and takes the eigenvalues as Rayleigh quotients:
+    spectra that would defeat one-sided rotations without the shift (pairs +-lambda, repeated and zero eigenvalues, a matrix
+    whose columns are orthogonal as they stand), through what defines an eigendecomposition.
+    Bar: 20 eps sqrt(n) |A|_2 for eigenvalues, 40 eps sqrt(n) |A|_2 for residuals, 20 eps n for orthogonality."""
+    import chainer_amd as chx
+    rng = np.random.default_rng(22)
+    for dt, eps in (('float32', 1.2e-7), ('float64', 2.3e-16)):
+        n = 200
+        q, _ = np.linalg.qr(rng.standard_normal((n, n)))
+        half = np.logspace(-6, 0, n // 2)
+        cases = {
+            'random': (lambda g: (g + g.T) / 2)(rng.standard_normal((333, 333))),
+            'pairs': (q * np.concatenate([half, -half])) @ q.T,
+            'repeated': (q * np.repeat([1.0, -1.0, 0.5, 0.0], n // 4)) @ q.T,
+            'antidiagonal': np.fliplr(np.eye(96)),  # eigenvalues +-1 only
+            'zero': np.zeros((70, 70)),
+        }
+        for name, a in cases.items():
+            a = ((a + a.T) / 2).astype(dt)
+            m = a.shape[0]
+            w, v = chx.eigh(chx.array(a))
+            w, v = w.get().astype(np.float64), v.get().astype(np.float64)
+            a64 = a.astype(np.float64)
+            scale = eps * np.sqrt(m) * max(np.abs(np.linalg.eigvalsh(a64)).max(), 0.0)
+            assert np.all(np.diff(w) >= 0), (dt, name)
+            assert np.abs(w - np.linalg.eigvalsh(a64)).max() <= 20 * scale, (dt, name)
+            assert np.abs(a64 @ v - v * w).max() <= 40 * scale, (dt, name)
+            assert np.abs(v.T @ v - np.eye(m)).max() <= 20 * eps * m, (dt, name)
+            only = chx.eigvalsh(chx.array(a)).get().astype(np.float64)
+            assert np.abs(only - w).max() <= 20 * scale, (dt, name)
+
+
 def test_one_workgroup_limits():
     """Matrices beyond what the one-workgroup kernels take are refused before anything is launched."""
     import chainer_amd as chx
