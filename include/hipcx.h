@@ -426,8 +426,9 @@ int hipcx_qr(const hipcx_array* a, const hipcx_array* q, const hipcx_array* r, c
  * One-sided Jacobi rotations: singular values agree with LAPACK's to rounding; singular vectors up to a common
  * sign of u[:, i] and vt[i, :] (and a rotation inside the space of a repeated value; the columns that complete a full u / vt, or
  * that belong to zero singular values, are some orthonormal basis of the same space).  Up to k = 64 the sweeps run in one
- * workgroup; beyond that a round of rotations is one launch with a wavefront per column pair, and the call waits for the stream
- * once per sweep to read whether anything was rotated (so it cannot be captured into a graph).  max(m, n) <= 4096. */
+ * workgroup; beyond that a sweep is k / 16 launches over blocks of 16 columns (a workgroup per pair of blocks, a wavefront per
+ * column pair), and the call waits for the stream once per sweep to read whether anything was rotated (so it cannot be captured
+ * into a graph).  max(m, n) <= 4096. */
 size_t hipcx_svd_workspace_size(const hipcx_array* a);
 int hipcx_svd(const hipcx_array* a, const hipcx_array* u, const hipcx_array* s, const hipcx_array* vt, int full_matrices, int compute_uv,
               void* workspace, size_t workspace_bytes, void* stream);
