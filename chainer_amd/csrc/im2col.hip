@@ -164,6 +164,15 @@ size_t RoundUp(size_t v) { return (v + 255) / 256 * 256; }
 
 enum Route { kFlippedConv, kPointwiseScatter, kProductCol2Im };
 
+// w[ci, co, kh - 1 - r, kw - 1 - q] read as [co, ci, r, q]: a view (swapped channel axes, negative spatial strides)
+hipcx_array FlippedFilters(const hipcx_array& w) {
+    hipcx_array wv = Permuted(w, {1, 0, 2, 3});
+    wv.data = static_cast<char*>(w.data) + (w.shape[2] - 1) * w.strides[2] + (w.shape[3] - 1) * w.strides[3];
+    wv.strides[2] = -w.strides[2];
+    wv.strides[3] = -w.strides[3];
+    return wv;
+}
+
 struct TransposePlan {
     Route route;
     int64_t N, Ci, Co, H, W, kh, kw, OH, OW;
@@ -211,12 +220,10 @@ TransposePlan PlanTranspose(const hipcx_array* x, const hipcx_array* w, const hi
     const size_t it = static_cast<size_t>(ItemSize(dt));
     if (stride[0] == 1 && stride[1] == 1 && pad[0] <= pl.kh - 1 && pad[1] <= pl.kw - 1 && pl.OH == pl.H - 1 + pl.kh - 2 * pad[0] &&
         pl.OW == pl.W - 1 + pl.kw - 2 * pad[1]) {
-        pl.route = kFlippedConv;
-        pl.w_copy = Dense(nullptr, dt, {pl.Co, pl.Ci, pl.kh, pl.kw});
-        pl.x_off = pl.mid_off = pl.inner_off = RoundUp(static_cast<size_t>(TotalSize(&pl.w_copy)) * it);
-        hipcx_array wc = pl.w_copy;
-        wc.data = base + pl.w_off;
-        pl.inner_bytes = hipcx_conv_workspace_size(x, &wc, out);
+        pl.route = kFlippedConv;  // on a view of w: the convolution reads its filters through their strides, no copy
+        pl.x_off = pl.mid_off = pl.inner_off = 0;
+        const hipcx_array wv = FlippedFilters(*w);
+        pl.inner_bytes = hipcx_conv_workspace_size(x, &wv, out);
     } else if (pl.kh == 1 && pl.kw == 1 && pad[0] == 0 && pad[1] == 0 && TotalSize(x) > 0) {
         pl.route = kPointwiseScatter;
         pl.w_copy = Dense(nullptr, dt, {pl.Co, pl.Ci, 1, 1});
@@ -321,14 +328,9 @@ int hipcx_conv_transpose(const hipcx_array* x, const hipcx_array* w, const hipcx
         const int64_t one[2] = {1, 1}, zero[2] = {0, 0};
         const int64_t it = ItemSize(out->dtype);
         if (pl.route == kFlippedConv) {
-            // w[ci, co, kh - 1 - r, kw - 1 - q] read as [co, ci, r, q]
-            hipcx_array wv = Permuted(*w, {1, 0, 2, 3});
-            wv.data = static_cast<char*>(w->data) + (pl.kh - 1) * w->strides[2] + (pl.kw - 1) * w->strides[3];
-            wv.strides[2] = -w->strides[2];
-            wv.strides[3] = -w->strides[3];
-            Check(hipcx_copy(&wv, &pl.w_copy, stream));
+            const hipcx_array wv = FlippedFilters(*w);
             const int64_t fpad[2] = {pl.kh - 1 - pad[0], pl.kw - 1 - pad[1]};
-            Check(hipcx_conv(x, &pl.w_copy, b, one, fpad, 0, out, inner, pl.inner_bytes, stream));
+            Check(hipcx_conv(x, &wv, b, one, fpad, 0, out, inner, pl.inner_bytes, stream));
             return;
         }
         if (pl.route == kPointwiseScatter) {
