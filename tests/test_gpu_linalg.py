@@ -377,6 +377,8 @@ def test_eigh_above_one_workgroup_on_hard_spectra():
             'antidiagonal': np.fliplr(np.eye(96)),  # eigenvalues +-1 only
             'zero': np.zeros((70, 70)),
         }
+        if dt == 'float64':  # too many rows for the block pairs to sit in LDS: the sweeps rotate the columns in memory
+            cases['random, in memory'] = (lambda g: (g + g.T) / 2)(rng.standard_normal((600, 600)))
         for name, a in cases.items():
             a = ((a + a.T) / 2).astype(dt)
             m = a.shape[0]
