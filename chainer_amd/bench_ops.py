@@ -361,6 +361,34 @@ def section_linalg(chx, oracle, with_cpu):
             emit(**row)
 
 
+def section_dot(chx, oracle, with_cpu):
+    """Dot: the matrix products of the five workloads (as the Linear link hands them over: x row-major, W^T a view of the
+    [out, in] weights) and a calibration product with both operands stored along the reduction axis."""
+    rng = np.random.default_rng(5)
+    cases = [
+        ('MLP layer 1 (config 1)', 'float32', 100, 784, 1000),
+        ('LSTM gates (config 5)', 'float32', 128, 650, 2600),
+        ('LSTM output layer, 35 steps (config 5)', 'float32', 4480, 650, 10000),
+        ('ResNet-50 classifier (config 4)', 'float16', 128, 2048, 1000),
+        ('calibration', 'float16', 4096, 4096, 4096),
+        ('calibration', 'float16', 8192, 8192, 8192),
+    ]
+    for name, dt, m, k, n in cases:
+        a = rng.standard_normal((m, k)).astype(dt)
+        wt = (rng.standard_normal((n, k)) / np.sqrt(k)).astype(dt)
+        A, B = chx.array(a), chx.array(wt).T
+        t = op_time(lambda: chx.dot(A, B))
+        flops = 2.0 * m * n * k
+        nbytes = (m * k + n * k + m * n) * a.dtype.itemsize
+        peak = MFMA_PEAK[dt]
+        row = dict(section='dot', op='dot %s [%d,%d] . [%d,%d]^T (%s)' % (dt, m, k, n, k, name), us=round(t * 1e6, 2), TFLOPs=round(flops / t / 1e12, 2),
+                   mfma_frac=round(flops / t / 1e12 / peak, 4), GBps=round(nbytes / t / 1e9, 1), hbm_frac=round(nbytes / t / 1e9 / HBM_PEAK, 4),
+                   bound='mfma' if flops / (peak * 1e12) >= nbytes / (HBM_PEAK * 1e9) else 'hbm')
+        if with_cpu and m * n * k <= 4e8:
+            row['cpu_native_1core_us'] = round(cpu_time(lambda: oracle.dot(a, np.ascontiguousarray(wt.T))) * 1e6, 1)
+        emit(**row)
+
+
 def section_copy(chx, oracle, with_cpu):
     """A plain copy of known size (128 MiB read + 128 MiB written): the calibration point for HBM traffic counters."""
     x = chx.array(np.zeros(64 * 1024 * 1024, np.float16))
@@ -368,7 +396,7 @@ def section_copy(chx, oracle, with_cpu):
     bw_row('copy', 'copy float16 [67108864]', (64 * 1024 * 1024,), t, 2 * x.nbytes)
 
 
-SECTIONS = {'copy': section_copy, 'sweep': section_sweep, 'mlp': section_mlp, 'cifar': section_cifar, 'resnet_layers': section_resnet_layers, 'lstm': section_lstm, 'backward': section_backward, 'train': section_train, 'linalg': section_linalg}
+SECTIONS = {'copy': section_copy, 'sweep': section_sweep, 'dot': section_dot, 'mlp': section_mlp, 'cifar': section_cifar, 'resnet_layers': section_resnet_layers, 'lstm': section_lstm, 'backward': section_backward, 'train': section_train, 'linalg': section_linalg}
 
 
 def run(sections, cpu=None):

@@ -8,6 +8,7 @@
 #include <utility>
 #include <vector>
 
+#include "gemm_pp.h"
 #include "igemm.h"
 #include "igemm_pipe.h"
 #include "layout_kernels.h"
@@ -190,6 +191,45 @@ void LaunchIGemmImpl(IGemmArgs<T> p, hipStream_t stream) {
     }
 }
 
+
+// Large float16 products with both operands' reduction index at unit stride (gemm_pp.h).  Returns false when the problem does
+// not qualify: the 128 x 128 kernels below then take it.
+bool TryGemmPp(const hipcx_array* a, const hipcx_array* b, const hipcx_array* out, hipStream_t stream) {
+    static const bool enabled = [] { const char* e = getenv("HIPCX_DOT_PP"); return e == nullptr || e[0] != '0'; }();
+    static const int band = [] { const char* e = getenv("HIPCX_DOT_PP_BAND"); return e != nullptr && atoi(e) > 0 ? atoi(e) : 8; }();
+    if (!enabled) return false;
+    const int64_t M = a->shape[0], K = a->shape[1], N = b->shape[1];
+    if (K % 32 != 0 || K < gemm_pp::kMinK || N % 4 != 0) return false;
+    // a: rows of K contiguous halves; b: columns of K contiguous halves (the view Linear hands over, or a staged copy)
+    if (a->strides[1] != 2 || b->strides[0] != 2 || out->strides[1] != 2) return false;
+    const int64_t lda = a->strides[0] / 2, ldb = b->strides[1] / 2, ldc = out->strides[0] / 2;
+    if (a->strides[0] % 16 != 0 || b->strides[1] % 16 != 0 || out->strides[0] % 8 != 0 || lda < K || ldb < K || ldc < N) return false;
+    if (reinterpret_cast<uintptr_t>(a->data) % 16 != 0 || reinterpret_cast<uintptr_t>(b->data) % 16 != 0 || reinterpret_cast<uintptr_t>(out->data) % 8 != 0) return false;
+    if (256 * lda * 2 >= (1LL << 31) || 256 * ldb * 2 >= (1LL << 31)) return false;  // 32-bit offsets inside a tile's rows
+    const int64_t tiles_m = (M + 255) / 256, tiles_n = (N + 255) / 256;
+    // enough 256 x 256 tiles to occupy most of the chip; smaller products fill it better with 128 x 128 tiles
+    if (tiles_m * tiles_n < (NumCUs() * 3) / 4 || tiles_m * tiles_n >= (1LL << 24)) return false;
+    gemm_pp::GemmArgs p{};
+    p.a = static_cast<const half_t*>(a->data);
+    p.b = static_cast<const half_t*>(b->data);
+    p.c = static_cast<half_t*>(out->data);
+    p.M = static_cast<int>(M);
+    p.N = static_cast<int>(N);
+    p.K = static_cast<int>(K);
+    p.lda = static_cast<int>(lda);
+    p.ldb = static_cast<int>(ldb);
+    p.ldc = static_cast<int>(ldc);
+    p.tiles_m = static_cast<int>(tiles_m);
+    p.tiles_n = static_cast<int>(tiles_n);
+    p.band = band;
+    ProfileScope prof(stream, 2.0 * static_cast<double>(M) * N * K, 2.0 * (static_cast<double>(M) * K + static_cast<double>(N) * K + static_cast<double>(M) * N));
+    struct GemmPpTag {};
+    EnsureDynamicLds<GemmPpTag>(reinterpret_cast<const void*>(gemm_pp::GemmPpKernel), gemm_pp::kLdsBytes);
+    const unsigned grid = static_cast<unsigned>((tiles_m * tiles_n + 7) / 8 * 8);
+    hipLaunchKernelGGL(gemm_pp::GemmPpKernel, dim3(grid), dim3(512), gemm_pp::kLdsBytes, stream, p);
+    CheckLaunch("gemm_pp");
+    return true;
+}
 
 // Small-output matrix products (small_dot.h).  Returns false when the problem does not qualify.
 template <typename T>
@@ -1388,6 +1428,7 @@ int hipcx_dot(const hipcx_array* a, const hipcx_array* b, const hipcx_array* out
             }
         }
         if (out->dtype == HIPCX_FLOAT16) {
+            if (slices == 1 && TryGemmPp(a, b, out, st)) return;
             if (slices == 1 && TrySmallDot<half_t>(a, b, out, st)) return;
             IGemmArgs<half_t> p{};
             fill(p);

@@ -227,3 +227,33 @@ def test_dot_staged_operands_with_split_reduction(dt, tol):
         for la, A in (('a row-major', A_row), ('a transposed view', A_t)):
             for lb, B in (('b row-major', B_row), ('b transposed view', B_t)):
                 assert_close(chx.dot(A, B).get(), ref, tol, 'dot %s %r, %s, %s' % (dt, (m, k, n), la, lb))
+
+
+def test_dot_float16_256_tiles():
+    """float16 products large enough for the 256 x 256 tile kernel (at least 192 such tiles, reduction a multiple of 32): exact on
+    integer-valued data (float accumulation of small integers has no rounding), partial tiles on both edges, padded pitches, and
+    every operand layout (row-major operands are staged into the layout the kernel reads).  Too large for the serial oracle
+    loop: random data is checked against the float64 product of the stored values."""
+    import chainer_amd as chx
+    rng = np.random.default_rng(31)
+    for (m, k, n) in [(4096, 96, 4096), (3600, 160, 3700), (2304, 1024, 6148)]:
+        a = rng.integers(-3, 4, (m, k)).astype('float16')
+        bt = rng.integers(-3, 4, (n, k)).astype('float16')
+        ref = (a.astype(np.int64) @ bt.astype(np.int64).T)
+        assert np.abs(ref).max() < 2048  # every result is a float16 value
+        got = chx.dot(chx.array(a), chx.array(bt).T).get()
+        assert np.array_equal(got.astype(np.int64), ref), 'integer-valued dot %r' % ((m, k, n),)
+    m, k, n = 3840, 512, 4104
+    a = rng.standard_normal((m, k)).astype('float16')
+    b = (rng.standard_normal((k, n)) / np.sqrt(k)).astype('float16')
+    ref = (a.astype(np.float64) @ b.astype(np.float64)).astype('float16')
+    A_row, B_row = chx.array(a), chx.array(b)
+    A_t = chx.array(np.ascontiguousarray(a.T)).T
+    B_t = chx.array(np.ascontiguousarray(b.T)).T
+    for la, A in (('a row-major', A_row), ('a transposed view', A_t)):
+        for lb, B in (('b row-major', B_row), ('b transposed view', B_t)):
+            assert_close(chx.dot(A, B).get(), ref, 2e-2, 'dot %r, %s, %s' % ((m, k, n), la, lb))
+    ap = padded((m, k), a, (8, 0), 'float16')        # row pitch k + 8 halves: 16-byte aligned rows
+    btp = padded((n, k), np.ascontiguousarray(b.T), (24, 0), 'float16')
+    got = chx.dot(upload_view(chx, ap), upload_view(chx, btp).T).get()
+    assert_close(got, ref, 2e-2, 'dot of operands with padded pitches')
