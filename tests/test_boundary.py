@@ -41,8 +41,8 @@ def test_library_exports_every_declared_symbol():
 
 
 def test_plugin_glue_only_forwards_to_declared_entry_points():
-    """The ChainerX plugin source cannot be built here (it needs a ChainerX checkout); what can be checked is that every
-    hipcx_* name it uses is declared in the header, and that it reaches device memory only through those entry points."""
+    """Checks of the plugin source that need no ChainerX checkout (test_plugin_signatures.py compiles it against one): every
+    hipcx_* name it uses is declared in the header, and it reaches device memory only through those entry points."""
     import re
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     src = open(os.path.join(root, 'chainer_amd', 'plugin', 'hip_backend.cc')).read()
