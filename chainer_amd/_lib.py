@@ -160,6 +160,7 @@ SIGNATURES = {
     'hipcx_conv_out_dim': (ctypes.c_int64, [ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, _INT]),
     'hipcx_conv_workspace_size': (_SZ, [_A, _A, _A]),
     'hipcx_conv': (_INT, [_A, _A, _A, _I64P, _I64P, _INT, _A, _V, _SZ, _V]),
+    'hipcx_conv_route': (_INT, [_A, _A, _A, _I64P, _I64P, _A]),
     'hipcx_conv_bn_act': (_INT, [_A, _A, _A, _I64P, _I64P, _INT, _A, _A, _A, _A, _S, _A, _INT, _A, _V, _SZ, _V]),
     'hipcx_amin': (_INT, [_A, _I8P, _INT, _A, _V, _SZ, _V]),
     'hipcx_argmin': (_INT, [_A, _I8P, _INT, _A, _V, _SZ, _V]),

@@ -13,6 +13,7 @@
 #include "igemm_pipe.h"
 #include "layout_kernels.h"
 #include "nchw_conv.h"
+#include "pw_conv.h"
 #include "stem_conv.h"
 #include "small_dot.h"
 
@@ -719,6 +720,87 @@ void RunNchw(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, c
 }
 
 
+// ---- float16 1x1 / stride 1 layers on the LDS-direct ring (pw_conv.h) ----
+struct PwPlan {
+    bool ok = false;
+    int wm = 2, wn = 4;
+};
+
+PwPlan PlanPw(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, const hipcx_array* out, const int64_t* stride, const int64_t* pad) {
+    PwPlan pl;
+    static const bool enabled = [] { const char* e = getenv("HIPCX_CONV_PW"); return e == nullptr || e[0] != '0'; }();
+    if (!enabled || x->dtype != HIPCX_FLOAT16 || !IsContiguous(x) || !IsContiguous(out)) return pl;
+    const int64_t N = x->shape[0], C = x->shape[1], P = x->shape[2] * x->shape[3], K = w->shape[0];
+    if (w->shape[2] != 1 || w->shape[3] != 1 || stride[0] != 1 || stride[1] != 1 || pad[0] != 0 || pad[1] != 0) return pl;
+    if (C % 32 != 0 || P % 4 != 0 || K > kPwMaxBiasK) return pl;
+    if (w->strides[1] != 2 || w->strides[0] != C * 2 || reinterpret_cast<uintptr_t>(w->data) % 16 != 0) return pl;  // dense [K][C] rows
+    if (reinterpret_cast<uintptr_t>(x->data) % 16 != 0 || reinterpret_cast<uintptr_t>(out->data) % 16 != 0) return pl;
+    if (b != nullptr && b->strides[0] % 2 != 0) return pl;
+    if (N * C * P * 2 >= (1LL << 31) || N * K * P * 2 >= (1LL << 31) || K * C * 2 >= (1LL << 31)) return pl;
+    const int64_t PS = (P + 7) / 8 * 8;
+    // Where these kernels measured faster than the 128 x 128 tiles on ResNet-50's layers at batch 128: very wide outputs over a
+    // short reduction (256 x 256 tiles: the layer streams, and an activation tile is fetched once per 256 output channels
+    // instead of once per 128) and 128 output channels (512 x 128 tiles).  Elsewhere the smaller tiles, three workgroups to a
+    // compute unit, overlap their load, multiply and store phases better than one workgroup of eight waves does.
+    if ((K >= 1024 && C <= 256) || (K >= 256 && C <= 64)) {
+        pl.wm = 2, pl.wn = 4;
+    } else if (K > 64 && K <= 128) {
+        pl.wm = 4, pl.wn = 2;
+    } else {
+        return pl;
+    }
+    const int64_t tiles = ((N * PS + 128 * pl.wm - 1) / (128 * pl.wm)) * ((K + 64 * pl.wn - 1) / (64 * pl.wn));
+    if (tiles < (NumCUs() * 3) / 4 || tiles >= (1LL << 24)) return pl;
+    pl.ok = true;
+    return pl;
+}
+
+template <int WM, int WN>
+void LaunchPw(PwConvArgs a, hipStream_t stream) {
+    constexpr int BM = 128 * WM, BN = 64 * WN;
+    a.tiles_m = (a.MS + BM - 1) / BM;
+    a.tiles_n = (a.K + BN - 1) / BN;
+    a.total_tiles = a.tiles_m * a.tiles_n;
+    constexpr int lds_bytes = PwLdsBytes<WM, WN>();
+    // workgroups walk tiles: one per compute unit (a multiple of 8, one share per XCD)
+    const unsigned grid = static_cast<unsigned>(std::min((a.total_tiles + 7) / 8 * 8, std::max(8, NumCUs() / 8 * 8)));
+    if (a.P % 8 != 0) {
+        auto kern = PwConvKernel<WM, WN, true>;
+        struct Tag {};
+        EnsureDynamicLds<Tag>(reinterpret_cast<const void*>(kern), lds_bytes);
+        hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds_bytes, stream, a);
+    } else {
+        auto kern = PwConvKernel<WM, WN, false>;
+        struct Tag {};
+        EnsureDynamicLds<Tag>(reinterpret_cast<const void*>(kern), lds_bytes);
+        hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds_bytes, stream, a);
+    }
+    CheckLaunch("pw_conv");
+}
+
+void RunPw(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, const PwPlan& pl, const hipcx_array* out, hipStream_t stream) {
+    PwConvArgs a{};
+    a.x = static_cast<const half_t*>(x->data);
+    a.w = static_cast<const half_t*>(w->data);
+    a.bias = b ? static_cast<const half_t*>(b->data) : nullptr;
+    a.bias_stride = b ? b->strides[0] / 2 : 0;
+    a.out = static_cast<half_t*>(out->data);
+    a.N = static_cast<int>(x->shape[0]);
+    a.C = static_cast<int>(x->shape[1]);
+    a.K = static_cast<int>(w->shape[0]);
+    a.P = static_cast<int>(x->shape[2] * x->shape[3]);
+    a.PS = (a.P + 7) / 8 * 8;
+    a.MS = a.N * a.PS;
+    a.div_PS = FastDiv(a.PS);
+    a.x_bytes = static_cast<unsigned>(static_cast<int64_t>(a.N) * a.C * a.P * 2);
+    a.w_bytes = static_cast<unsigned>(static_cast<int64_t>(a.K) * a.C * 2);
+    a.out_bytes = static_cast<unsigned>(static_cast<int64_t>(a.N) * a.K * a.P * 2);
+    const double M = static_cast<double>(a.N) * a.P;
+    ProfileScope prof(stream, 2.0 * M * a.K * a.C, 2.0 * (M * a.C + static_cast<double>(a.K) * a.C + M * a.K));
+    if (pl.wm == 2) LaunchPw<2, 4>(a, stream);
+    else LaunchPw<4, 2>(a, stream);
+}
+
 // ---- float16 7x7/2 stem path (stem_conv.h) ----
 struct StemPlan {
     bool ok = false;
@@ -1057,12 +1139,31 @@ size_t hipcx_conv_workspace_size(const hipcx_array* x, const hipcx_array* w, con
     }
 }
 
+int hipcx_conv_route(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, const int64_t* stride, const int64_t* pad,
+                     const hipcx_array* out) {
+    try {
+        if (x == nullptr || w == nullptr || out == nullptr || stride == nullptr || pad == nullptr) return -1;
+        if (x->ndim != 4 || w->ndim != 4 || out->ndim != 4) return -1;
+        if (PlanPw(x, w, b, out, stride, pad).ok) return 3;
+        if (PlanNchw(x, w, out, stride, pad).ok) return 1;
+        if (PlanStem(x, w, out, stride, pad).ok) return 2;
+        return 0;
+    } catch (...) {
+        return -1;
+    }
+}
+
 int hipcx_conv(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, const int64_t* stride, const int64_t* pad,
                int cover_all, const hipcx_array* out, void* workspace, size_t workspace_bytes, void* stream) {
     return Guard([&] {
         CheckConv(x, w, b, stride, pad, cover_all, out);
         if (TotalSize(out) == 0) return;
         hipStream_t st = AsStream(stream);
+        PwPlan ppl = PlanPw(x, w, b, out, stride, pad);
+        if (ppl.ok) {
+            RunPw(x, w, b, ppl, out, st);
+            return;
+        }
         NchwPlan npl = PlanNchw(x, w, out, stride, pad);
         if (npl.ok) {
             HIPCX_REQUIRE(workspace != nullptr && workspace_bytes >= npl.wp_bytes, HIPCX_CHAINERX_ERROR,

@@ -1112,6 +1112,20 @@ def conv(x, w, b=None, stride=1, pad=0, cover_all=False, out_dtype=None):
     return out
 
 
+def conv_route(x, w, b=None, stride=1, pad=0, cover_all=False):
+    """Which kernel family `conv` runs for these arguments (hipcx_conv_route): 0 general implicit GEMM, 1 float16 NCHW kernels
+    with 128-wide tiles, 2 the 7x7 / 2 stem kernel, 3 the float16 1x1 kernel with LDS-direct operand loads.  For tests and
+    benchmarks; not part of the ChainerX routine surface."""
+    stride, pad = _pair(stride), _pair(pad)
+    dt = result_type(x, w, b) if b is not None else result_type(x, w)
+    oh = conv_out_dim(x.shape[2], w.shape[2], stride[0], pad[0], cover_all)
+    ow = conv_out_dim(x.shape[3], w.shape[3], stride[1], pad[1], cover_all)
+    out = _spatial_out(x, x.shape[0], w.shape[0], oh, ow, dt)
+    xc, wc = x.astype(dt, False), w.astype(dt, False)
+    bc = b.astype(dt, False) if b is not None else None
+    return int(_lib.load().hipcx_conv_route(xc.desc(), wc.desc(), bc.desc() if bc is not None else None, _i64(stride), _i64(pad), out.desc()))
+
+
 def conv_bn_act(x, w, b=None, stride=1, pad=0, cover_all=False, bn=None, eps=2e-5, residual=None, relu=False):
     """Opt-in fused block: relu(fixed_batch_norm(conv(x, w, b), *bn, eps, axis=(0, 2, 3)) + residual) in one kernel call.
     `bn` is None or (gamma, beta, mean, var), one value per output channel.  Not part of the ChainerX routine surface:

@@ -289,6 +289,12 @@ int64_t hipcx_conv_out_dim(int64_t in_dim, int64_t kernel_size, int64_t stride, 
  * backend (CX/cuda/cuda_conv.cc:311); the native backend's own result is an NCHW view of NHWC memory
  * (CX/native/native_device/conv.cc:78-84), which this entry also accepts as `out`. */
 size_t hipcx_conv_workspace_size(const hipcx_array* x, const hipcx_array* w, const hipcx_array* out);
+/* Which kernel family hipcx_conv runs for these arguments (no counterpart in the reference: for tests and benchmarks that must
+ * know that a specialised kernel, not the general one, produced a result).  0: general implicit GEMM (any dtype / layout);
+ * 1: float16 NCHW kernels with 128-wide tiles; 2: float16 7x7 / 2 stem kernel; 3: float16 1x1 / stride 1 kernel that loads its
+ * operands straight into LDS and walks 256 x 256 or 512 x 128 tiles; -1: invalid arguments. */
+int hipcx_conv_route(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, const int64_t* stride, const int64_t* pad,
+                     const hipcx_array* out);
 int hipcx_conv(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, const int64_t* stride, const int64_t* pad,
                int cover_all, const hipcx_array* out, void* workspace, size_t workspace_bytes, void* stream);
 

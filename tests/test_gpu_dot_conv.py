@@ -257,3 +257,41 @@ def test_dot_float16_256_tiles():
     btp = padded((n, k), np.ascontiguousarray(b.T), (24, 0), 'float16')
     got = chx.dot(upload_view(chx, ap), upload_view(chx, btp).T).get()
     assert_close(got, ref, 2e-2, 'dot of operands with padded pitches')
+
+
+def test_conv1x1_float16_lds_direct_ring():
+    """1x1 / stride 1 float16 layers on the kernel that loads its operands straight into LDS (route 3): 256 x 256 tiles for wide
+    outputs over a short reduction, 512 x 128 tiles for 128 output channels; planes whose pixel count is a multiple of 8 and of 4
+    only (the last 16-byte piece of a plane is then half empty), workgroups that walk more than one tile, partial channel tiles,
+    bias.  Integer-valued data: float accumulation has no rounding, so results are exact and the rounding of the bias sum is the
+    only one.  Too large for the serial oracle loop: the reference is the same sum of products in float64."""
+    import chainer_amd as chx
+    from chainer_amd import routines
+    rng = np.random.default_rng(41)
+    cases = [(128, 64, 28, 256, True), (128, 64, 14, 1024, True), (96, 96, 14, 1320, False), (256, 32, 28, 128, True), (340, 160, 20, 100, True),
+             (128, 512, 28, 128, False)]
+    for (n, c, hw, k, with_bias) in cases:
+        x = rng.integers(-3, 4, (n, c, hw, hw)).astype('float16')
+        w = rng.integers(-2, 3, (k, c, 1, 1)).astype('float16')
+        b = rng.integers(-8, 9, k).astype('float16') if with_bias else None
+        X, W, B = chx.array(x), chx.array(w), (chx.array(b) if with_bias else None)
+        assert routines.conv_route(X, W, B) == 3, 'expected the LDS-direct 1x1 kernel for %r' % ((n, c, hw, k),)
+        got = chx.conv(X, W, B).get()
+        ref = np.einsum('nchw,kc->nkhw', x.astype(np.float32), w[:, :, 0, 0].astype(np.float32))
+        if with_bias:
+            ref = ref + b.astype(np.float32)[None, :, None, None]
+        assert np.abs(ref).max() <= 2048
+        assert np.array_equal(got.astype(np.float32), ref), 'conv 1x1 %r' % ((n, c, hw, k),)
+    # random data against the float64 sum of products
+    n, c, hw, k = 128, 256, 14, 1024
+    x = rng.standard_normal((n, c, hw, hw)).astype('float16')
+    w = (rng.standard_normal((k, c, 1, 1)) / np.sqrt(c)).astype('float16')
+    b = rng.standard_normal(k).astype('float16')
+    X, W, B = chx.array(x), chx.array(w), chx.array(b)
+    assert routines.conv_route(X, W, B) == 3
+    got = chx.conv(X, W, B).get()
+    ref = (np.einsum('nchw,kc->nkhw', x.astype(np.float64), w[:, :, 0, 0].astype(np.float64)) + b.astype(np.float64)[None, :, None, None]).astype('float16')
+    assert_close(got, ref, 2e-2, 'conv 1x1 %r' % ((n, c, hw, k),))
+    # the general kernels keep the shapes the plan leaves out
+    small = chx.array(rng.standard_normal((2, 64, 14, 14)).astype('float16'))
+    assert routines.conv_route(small, chx.array(w[:256, :64])) != 3
