@@ -46,7 +46,7 @@ def main():
     ap.add_argument('--warmup', type=int, default=5)
     ap.add_argument('--batch', type=int, default=128)
     ap.add_argument('--eager', action='store_true', help='time eager launches instead of a HIP graph replay')
-    ap.add_argument('--ops', nargs='?', const='copy,sweep,mlp,cifar,resnet_layers,lstm,backward,train,linalg', default=None,
+    ap.add_argument('--ops', nargs='?', const='copy,sweep,dot,mlp,cifar,resnet_layers,lstm,backward,train,linalg', default=None,
                     help='instead of the headline step, print per-operation roofline lines (chainer_amd.bench_ops) with a CPU baseline column')
     ap.add_argument('--cpu-batch', type=int, default=8, help='images for the CPU baseline (0 = skip)')
     args = ap.parse_args()

@@ -51,8 +51,10 @@ def current_stream():
 
 
 def synchronize():
-    """Device::Synchronize (CX/device.h:71)."""
+    """Device::Synchronize (CX/device.h:71).  Raises the IndexError of an earlier take / add_at (default bounds mode) whose indices
+    were out of range."""
     torch().cuda.synchronize()
+    _lib.call('hipcx_synchronize', DEVICE_INDEX)
 
 
 def dtype_code(dtype):
@@ -99,6 +101,13 @@ class DeviceBuffer(object):
 
     def data_ptr(self):
         return self.ptr
+
+    def record_stream(self, stream=None):
+        """Announces that work on this block is queued on ``stream`` (a raw stream handle; default: the current stream), which is
+        not the stream it was allocated on: the pool then holds the block back after its release until that work has run
+        (hipcx_record_stream)."""
+        if self.ptr:
+            _lib.call('hipcx_record_stream', DEVICE_INDEX, ctypes.c_void_p(self.ptr), current_stream() if stream is None else stream)
 
     def __del__(self):
         ptr, self.ptr = self.ptr, 0
@@ -194,6 +203,11 @@ class ndarray(object):
     @property
     def nbytes(self):
         return self.size * self.itemsize
+
+    def record_stream(self, stream=None):
+        """See DeviceBuffer.record_stream: call it when the array is used on a stream other than the one it was created on and may
+        be dropped before that stream is waited for."""
+        self._buf.record_stream(stream)
 
     @property
     def data_ptr(self):

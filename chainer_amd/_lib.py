@@ -113,6 +113,7 @@ SIGNATURES = {
     'hipcx_version': (_INT, []),
     'hipcx_device_count': (_INT, [ctypes.POINTER(ctypes.c_int)]),
     'hipcx_synchronize': (_INT, [_INT]),
+    'hipcx_record_stream': (_INT, [_INT, _V, _V]),
     'hipcx_device_name': (_INT, [_INT, ctypes.c_char_p, _SZ]),
     'hipcx_malloc': (_INT, [_INT, _SZ, ctypes.POINTER(ctypes.c_void_p)]),
     'hipcx_malloc_on_stream': (_INT, [_INT, _SZ, _V, ctypes.POINTER(ctypes.c_void_p)]),

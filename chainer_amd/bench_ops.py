@@ -26,6 +26,7 @@ import numpy as np
 
 HBM_PEAK = 8000.0  # GB/s
 MFMA_PEAK = {'float16': 2500.0, 'float32': 157.3}  # TFLOP/s
+FAMILY_REPS = 4  # calls per operation in the `families` section (after one warm-up call)
 
 
 def device_time(fn, iters=20, warmup=5, rounds=3):
@@ -229,15 +230,14 @@ def section_lstm(chx, oracle, with_cpu):
     I = chx.array(ids)
     fn = lambda: cfg.lstm_lm_forward(chx, pd, I, chx.zeros)
     eager = device_time(fn, 3, 1)
-    graph = graph_time(lambda: cfg.lstm_lm_forward(chx, pd, I, chx.zeros, 'wrap'), 5)
+    graph = graph_time(fn, 5)
     flops = 60.57e9 + 58.24e9
     row = dict(section='lstm', op='35-step forward', batch=128, eager_ms=round(eager * 1e3, 2), graph_replay_ms=round(graph * 1e3, 2),
                TFLOPs_graph=round(flops / graph / 1e12, 2), tokens_per_s_graph=round(128 * 35 / graph, 0), kernel_launches=35 * 86 + 7,
-               note='eager time is host launch overhead (~3000 kernel calls); the graph replay uses take(mode="wrap") because the default '
-                    'bounds mode reads an error flag back every step (the native backend raises IndexError) and cannot be captured; '
-                    'results are identical for in-range ids')
+               note='eager time is host launch overhead (~3000 kernel calls); take runs in the default bounds mode (mode=None, what the '
+                    'reference caller passes): an out-of-range id is recorded on the device and raised by the next get / synchronize')
     emit(**row)
-    fused = graph_time(lambda: cfg.lstm_lm_forward(chx, pd, I, chx.zeros, 'wrap', True), 5)
+    fused = graph_time(lambda: cfg.lstm_lm_forward(chx, pd, I, chx.zeros, None, True), 5)
     emit(section='lstm', op='35-step forward, fused opt-in Lstm cell and LogSoftmax', batch=128, graph_replay_ms=round(fused * 1e3, 2),
          TFLOPs_graph=round(flops / fused / 1e12, 2), tokens_per_s_graph=round(128 * 35 / fused, 0), kernel_launches=35 * 14 + 1,
          note='hipcx_lstm_cell and hipcx_log_softmax replace the ~25-kernel cell and the 7-kernel LogSoftmax chains; not the drop-in kernel boundary')
@@ -264,7 +264,7 @@ def section_lstm(chx, oracle, with_cpu):
          note='weights packed once per call, one launch per wavefront stage (36), gates stay in the MFMA accumulators; the reference '
               'hands RnnKernel to its cuda backend only (routines/n_step_rnn.cc:210), so this entry is opt-in for a hip plugin')
     W = pd['embed']
-    t = op_time(lambda: chx.take(W, I, 0, 'wrap'))
+    t = op_time(lambda: chx.take(W, I, 0))
     bw_row('lstm', 'take [10000,650] rows by [128,35] ids', (128, 35, 650), t, 2 * 128 * 35 * 650 * 4 + ids.nbytes)
     if with_cpu:
         ids2 = ids[:, :1]
@@ -389,6 +389,65 @@ def section_dot(chx, oracle, with_cpu):
         emit(**row)
 
 
+def section_families(chx, oracle, with_cpu):
+    """One operation per hot-path kernel family, each called FAMILY_REPS times in a row (eagerly, nothing else in between), with
+    its algorithmic bytes and flops: the run a counter profile (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE /
+    SQ_VALU_MFMA_BUSY_CYCLES) is taken of, so that counters per dispatch can be set against what the operation has to move or
+    compute.  `kernel` is a pattern the dispatched kernel's name matches; operations follow each other in the order printed."""
+    rng = np.random.default_rng(8)
+    reps = FAMILY_REPS
+    f16, f32 = np.float16, np.float32
+    act = chx.array(rng.standard_normal((128, 256, 56, 56)).astype(f16))
+    act2 = chx.array(rng.standard_normal((128, 256, 56, 56)).astype(f16))
+    n_act = 128 * 256 * 56 * 56
+    bn = [chx.array(v.astype(f16)) for v in (rng.uniform(0.5, 1.5, 256), rng.normal(0, 0.1, 256), rng.normal(0, 0.1, 256), rng.uniform(0.5, 1.5, 256))]
+    pool_in = chx.array(rng.standard_normal((128, 64, 112, 112)).astype(f16))
+    x32 = chx.array(rng.standard_normal((4096, 4096)).astype(f32))
+    table = chx.array(rng.standard_normal((10000, 650)).astype(f32))
+    ids = chx.array(rng.integers(0, 10000, (128, 35)).astype(np.int32))
+    a1, w1 = chx.array(rng.random((100, 784)).astype(f32)), chx.array((rng.standard_normal((1000, 784)) / 28).astype(f32))
+    a5, w5 = chx.array(rng.standard_normal((128, 650)).astype(f32)), chx.array(rng.uniform(-0.05, 0.05, (2600, 650)).astype(f32))
+    a5o, w5o = chx.array(rng.standard_normal((4480, 650)).astype(f32)), chx.array(rng.uniform(-0.05, 0.05, (10000, 650)).astype(f32))
+    a4, w4 = chx.array(rng.standard_normal((128, 2048)).astype(f16)), chx.array((rng.standard_normal((1000, 2048)) / 45).astype(f16))
+    ag, wg = chx.array(rng.standard_normal((4096, 4096)).astype(f16)), chx.array((rng.standard_normal((4096, 4096)) / 64).astype(f16))
+    cx, cw = chx.array(rng.standard_normal((256, 64, 32, 32)).astype(f32)), chx.array((rng.standard_normal((64, 64, 3, 3)) / 24).astype(f32))
+    px = chx.array(rng.standard_normal((128, 512, 28, 28)).astype(f16))
+    pw = chx.array((rng.standard_normal((128, 512, 1, 1)) / 23).astype(f16))
+    u = 650
+    ws = [[chx.array(rng.uniform(-0.05, 0.05, (u, u)).astype(f32)) for _ in range(8)] for _ in range(2)]
+    bs = [[chx.array(rng.uniform(-0.05, 0.05, (u,)).astype(f32)) for _ in range(8)] for _ in range(2)]
+    xs = [chx.array(rng.standard_normal((128, u)).astype(f32)) for _ in range(35)]
+    hx, cxs = chx.array(np.zeros((2, 128, u), f32)), chx.array(np.zeros((2, 128, u), f32))
+    ops = [
+        # name, kernel pattern, call, algorithmic bytes per dispatch, flops per dispatch, dispatches of that kernel per call
+        ('residual add float16 [128,256,56,56]', r'EwKernel.*(Add|BinaryAA)', lambda: chx.add(act, act2), 3 * n_act * 2, 0, 1),
+        ('relu float16 [128,256,56,56]', r'EwKernel.*(IfLess|Select|Relu)', lambda: chx.relu(act), 2 * n_act * 2, 0, 1),
+        ('exp float32 [4096,4096]', r'EwKernel.*UnaryOp', lambda: chx.exp(x32), 2 * 4096 * 4096 * 4, 0, 1),
+        ('fixed_batch_norm float16 [128,256,56,56]', r'BnChannelsFirstKernel', lambda: chx.fixed_batch_norm(act, *bn, axis=(0, 2, 3)), 2 * n_act * 2, 0, 1),
+        ('max_pool 3x3/2 pad 1 float16 [128,64,112,112]', r'MaxPoolRowsS2Kernel', lambda: chx.max_pool(pool_in, 3, 2, 1, False),
+         (128 * 64 * 112 * 112 + 128 * 64 * 56 * 56) * 2, 0, 1),
+        ('take float32 [10000,650] by [128,35]', r'TakeRowsKernel', lambda: chx.take(table, ids, 0), 2 * 128 * 35 * 650 * 4 + 128 * 35 * 4, 0, 1),
+        ('dot float32 [100,784].[784,1000] (config 1)', r'SmallDot', lambda: chx.dot(a1, w1.T), (100 * 784 + 784 * 1000 + 100 * 1000) * 4, 2.0 * 100 * 784 * 1000, 1),
+        ('dot float32 [128,650].[650,2600] (config 5 gates)', r'SmallDot', lambda: chx.dot(a5, w5.T), (128 * 650 + 650 * 2600 + 128 * 2600) * 4, 2.0 * 128 * 650 * 2600, 1),
+        ('dot float32 [4480,650].[650,10000] (config 5 output layer)', r'IGemmFastKernel<float', lambda: chx.dot(a5o, w5o.T),
+         (4480 * 650 + 650 * 10000 + 4480 * 10000) * 4, 2.0 * 4480 * 650 * 10000, 1),
+        ('dot float16 [128,2048].[2048,1000] (config 4 classifier)', r'SmallDot', lambda: chx.dot(a4, w4.T), (128 * 2048 + 2048 * 1000 + 128 * 1000) * 2, 2.0 * 128 * 2048 * 1000, 1),
+        ('dot float16 [4096,4096].[4096,4096] (calibration)', r'GemmPpKernel', lambda: chx.dot(ag, wg.T), 3 * 4096 * 4096 * 2, 2.0 * 4096 ** 3, 1),
+        ('conv float32 3x3 [256,64,32,32] -> 64 (config 3)', r'IGemmFastKernel<float', lambda: chx.conv(cx, cw, None, 1, 1),
+         (2 * 256 * 64 * 32 * 32 + 64 * 64 * 9) * 4, 2.0 * 256 * 32 * 32 * 64 * 64 * 9, 1),
+        ('conv float16 1x1 [128,512,28,28] -> 128', r'PwConvKernel', lambda: chx.conv(px, pw), (128 * 512 * 784 + 128 * 512 + 128 * 128 * 784) * 2, 2.0 * 128 * 784 * 128 * 512, 1),
+        ('n_step_lstm float32 2 layers x 35 steps, batch 128, 650 units (RnnKernel entry)', r'LstmStepKernel',
+         lambda: chx.n_step_lstm(2, hx, cxs, ws, bs, xs, kernel=True), 0, 2.0 * 128 * 4 * u * 2 * u * 2 * 35 / 36, 36),
+    ]
+    for name, pattern, fn, nbytes, flops, per_call in ops:
+        fn()
+        chx.synchronize()
+        for _ in range(reps):
+            fn()
+        chx.synchronize()
+        emit(section='families', op=name, kernel=pattern, calls=reps + 1, dispatches_per_call=per_call, algorithmic_bytes=int(nbytes), flops=float(flops))
+
+
 def section_copy(chx, oracle, with_cpu):
     """A plain copy of known size (128 MiB read + 128 MiB written): the calibration point for HBM traffic counters."""
     x = chx.array(np.zeros(64 * 1024 * 1024, np.float16))
@@ -396,7 +455,7 @@ def section_copy(chx, oracle, with_cpu):
     bw_row('copy', 'copy float16 [67108864]', (64 * 1024 * 1024,), t, 2 * x.nbytes)
 
 
-SECTIONS = {'copy': section_copy, 'sweep': section_sweep, 'dot': section_dot, 'mlp': section_mlp, 'cifar': section_cifar, 'resnet_layers': section_resnet_layers, 'lstm': section_lstm, 'backward': section_backward, 'train': section_train, 'linalg': section_linalg}
+SECTIONS = {'copy': section_copy, 'sweep': section_sweep, 'dot': section_dot, 'families': section_families, 'mlp': section_mlp, 'cifar': section_cifar, 'resnet_layers': section_resnet_layers, 'lstm': section_lstm, 'backward': section_backward, 'train': section_train, 'linalg': section_linalg}
 
 
 def run(sections, cpu=None):
@@ -409,7 +468,7 @@ def run(sections, cpu=None):
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument('--section', default=','.join(k for k in SECTIONS if k != 'copy'))
+    ap.add_argument('--section', default=','.join(k for k in SECTIONS if k not in ('copy', 'families')))
     args = ap.parse_args()
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     if root not in sys.path:

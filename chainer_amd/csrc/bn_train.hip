@@ -5,9 +5,10 @@
 // The reference's generic kernels are routine compositions (CX/routines/normalization.cc:155-250): Mean, Var = Mean((x - mean)^2),
 // 1 / sqrt(var + eps), five elementwise passes, four in-place updates of the running statistics -- about twenty launches that read
 // or write the tensor a dozen times.  Here: two statistics passes (sum, then centred sum of squares: the two-pass variance of the
-// reference, not E[x^2] - mean^2), one per-channel finish, one normalising pass.  Arithmetic runs in float (double for float64)
-// with one rounding per stored value, so float16 results are at least as accurate as the composition's; agreement with it is to
-// tolerance, not to the bit.
+// reference, not E[x^2] - mean^2), one per-channel finish, one normalising pass.  Arithmetic runs in float (double for float64).
+// float16 values are rounded to float16 at every point where the composition holds an array (see Rnd), so the special values of the
+// reference's float16 arithmetic come out the same -- a sum past 65504 is inf, the statistics and the output that follow from it
+// are inf / NaN -- and finite results differ from the composition's only by the order of the float additions inside a sum.
 //
 // Statistics: grid (C, S).  Block (c, s) walks images s, s + S, ... of channel c with 16-byte loads, reduces over the block and
 // stores one partial; the finish kernel adds a channel's S partials in order (deterministic).
@@ -33,6 +34,20 @@ __device__ __forceinline__ C BlockSum(C v, C* lds) {
         for (int w = 0; w < kBnTrainThreads / 64; ++w) r += lds[w];
     }
     return r;  // valid in thread 0
+}
+
+// float16 arrays: the reference composes BatchNorm from routines that each round their result to float16 (and its float16 Sum
+// accumulates in float but hands out a float16, CX/native/native_device/reduction.cc:105-110), so a sum past 65504 is inf there,
+// (x - mean)^2 past 65504 is inf, 1 / count is a float16 subnormal, and so on.  Rnd applies that rounding wherever the composition
+// has an array in between; arithmetic between two roundings runs in float as the reference's Float16 operators do.  For float32
+// and float64 it is the identity.
+template <typename T>
+__device__ __forceinline__ compute_t<T> Rnd(compute_t<T> v) {
+    if constexpr (sizeof(T) == 2) {
+        return static_cast<compute_t<T>>(static_cast<T>(v));
+    } else {
+        return v;
+    }
 }
 
 // The per-channel state (mean, 1 / std): compute-type vectors in the workspace (forward), or the caller's arrays in the array dtype
@@ -85,12 +100,12 @@ __global__ __launch_bounds__(kBnTrainThreads) void BnStatKernel(BnStatArgs p) {
             if (MODE == 0) {
                 a0 += xe;
             } else if (MODE == 1) {
-                C d = xe - m;
-                a0 += d * d;
+                C d = Rnd<T>(xe - m);
+                a0 += Rnd<T>(d * d);
             } else {
                 C ge = static_cast<C>(gv.v[e]);
                 a0 += ge;
-                a1 += ge * ((xe - m) * is);
+                a1 += Rnd<T>(ge * Rnd<T>(Rnd<T>(xe - m) * is));
             }
         }
     }
@@ -127,28 +142,31 @@ __global__ __launch_bounds__(256) void BnFinishKernel(BnFinishArgs p) {
     C sum = C(0);
     for (int s = 0; s < p.S; ++s) sum += part[s * 2];
     const C n = static_cast<C>(p.count);
+    // Mean = Sum (handed out in the array dtype) / count (CX/routines/statistics.cc:113-123)
     if (STEP == 0) {
-        static_cast<C*>(p.mean)[c] = sum / n;
+        static_cast<C*>(p.mean)[c] = Rnd<T>(Rnd<T>(sum) / n);
         return;
     }
     const C mean = static_cast<const C*>(p.mean)[c];
-    const C var = sum / n;
+    const C var = Rnd<T>(Rnd<T>(sum) / n);
+    // Reciprocal(Sqrt(var + eps)) with eps as a scalar of the array dtype (CX/routines/normalization.cc:141)
     C inv_std;
     if constexpr (std::is_same<C, float>::value) {
-        inv_std = 1.0f / sqrtf(var + static_cast<float>(p.eps));
+        inv_std = Rnd<T>(1.0f / Rnd<T>(sqrtf(Rnd<T>(var + Rnd<T>(static_cast<float>(p.eps))))));
     } else {
         inv_std = 1.0 / sqrt(var + p.eps);
     }
     static_cast<C*>(p.inv_std)[c] = inv_std;
     static_cast<T*>(p.mean_out)[c * p.mo_stride] = static_cast<T>(mean);
     static_cast<T*>(p.inv_std_out)[c * p.io_stride] = static_cast<T>(inv_std);
-    const C decay = static_cast<C>(p.decay);
-    const C inv_decay = static_cast<C>(1.0 - p.decay);
-    const C adjust = static_cast<C>(p.count / (p.count - 1.0 > 1.0 ? p.count - 1.0 : 1.0));
+    // running *= decay; running += (inv_decay [* count / (count - 1)]) * statistic, scalars in the array dtype (CX/routines/normalization.cc:185-190)
+    const C decay = Rnd<T>(static_cast<C>(p.decay));
+    const C inv_decay = Rnd<T>(static_cast<C>(1.0 - p.decay));
+    const C inv_decay_adjusted = Rnd<T>(static_cast<C>((1.0 - p.decay) * (p.count / (p.count - 1.0 > 1.0 ? p.count - 1.0 : 1.0))));
     T* rm = static_cast<T*>(p.running_mean) + c * p.rm_stride;
     T* rv = static_cast<T*>(p.running_var) + c * p.rv_stride;
-    *rm = static_cast<T>(static_cast<C>(*rm) * decay + inv_decay * mean);
-    *rv = static_cast<T>(static_cast<C>(*rv) * decay + inv_decay * adjust * var);
+    *rm = static_cast<T>(Rnd<T>(static_cast<C>(*rm) * decay) + Rnd<T>(inv_decay * mean));
+    *rv = static_cast<T>(Rnd<T>(static_cast<C>(*rv) * decay) + Rnd<T>(inv_decay_adjusted * var));
 }
 
 struct BnApplyArgs {
@@ -182,8 +200,8 @@ __global__ __launch_bounds__(256) void BnGradFinishKernel(BnApplyArgs p) {
         sg += part[s * 2];
         sgx += part[s * 2 + 1];
     }
-    part[0] = sg;
-    part[1] = sgx;
+    part[0] = Rnd<T>(sg);  // what the gradient pass reads back is the array-dtype sum, as in the reference
+    part[1] = Rnd<T>(sgx);
     static_cast<T*>(p.gbeta)[c * p.gb_stride] = static_cast<T>(sg);
     static_cast<T*>(p.ggamma)[c * p.gg_stride] = static_cast<T>(sgx);
 }
@@ -197,7 +215,7 @@ __global__ __launch_bounds__(256) void BnApplyKernel(BnApplyArgs p) {
     const T* g = static_cast<const T*>(p.g);
     T* out = static_cast<T*>(p.out);
     const int64_t nvec = p.total / VEC;
-    const C inv_n = static_cast<C>(1.0 / p.count);
+    const C inv_n = Rnd<T>(static_cast<C>(1.0 / p.count));  // a scalar of the array dtype
     // The array is one contiguous run of [N][C] planes of L elements, cut into vectors without regard to the planes: when VEC does
     // not divide L a vector can hold the end of one plane and the start of the next (never more: the host keeps VEC <= L), and
     // its elements pick the constants of their own channel.  32-bit index arithmetic: the host checks total < 2^31.
@@ -231,13 +249,13 @@ __global__ __launch_bounds__(256) void BnApplyKernel(BnApplyArgs p) {
                 gbeta2 = part2[0], ggamma2 = part2[1];
             }
             Vec<T, VEC> gv = *reinterpret_cast<const Vec<T, VEC>*>(g + v * VEC);
-            const C scale = ga * is, scale2 = ga2 * is2;
+            const C scale = Rnd<T>(ga * is), scale2 = Rnd<T>(ga2 * is2);
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
                 const bool second = e >= split_at;
-                C x_hat = (static_cast<C>(xv.v[e]) - (second ? m2 : m)) * (second ? is2 : is);
-                o.v[e] = static_cast<T>((second ? scale2 : scale) *
-                                        (static_cast<C>(gv.v[e]) - (x_hat * (second ? ggamma2 : ggamma) + (second ? gbeta2 : gbeta)) * inv_n));
+                C x_hat = Rnd<T>(Rnd<T>(static_cast<C>(xv.v[e]) - (second ? m2 : m)) * (second ? is2 : is));
+                C t = Rnd<T>(Rnd<T>(Rnd<T>(x_hat * (second ? ggamma2 : ggamma)) + (second ? gbeta2 : gbeta)) * inv_n);
+                o.v[e] = static_cast<T>((second ? scale2 : scale) * Rnd<T>(static_cast<C>(gv.v[e]) - t));
             }
         } else {
             const C be = static_cast<C>(static_cast<const T*>(p.beta)[c * p.beta_stride]);
@@ -245,7 +263,8 @@ __global__ __launch_bounds__(256) void BnApplyKernel(BnApplyArgs p) {
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
                 const bool second = e >= split_at;
-                o.v[e] = static_cast<T>(((static_cast<C>(xv.v[e]) - (second ? m2 : m)) * (second ? is2 : is)) * (second ? ga2 : ga) + (second ? be2 : be));
+                C t = Rnd<T>(Rnd<T>(static_cast<C>(xv.v[e]) - (second ? m2 : m)) * (second ? is2 : is));
+                o.v[e] = static_cast<T>(Rnd<T>(t * (second ? ga2 : ga)) + (second ? be2 : be));
             }
         }
         *reinterpret_cast<Vec<T, VEC>*>(out + v * VEC) = o;

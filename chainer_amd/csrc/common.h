@@ -25,6 +25,17 @@ struct Error : std::runtime_error {
 
 void SetLastError(const std::string& msg);
 
+// Out-of-range indices of Take / AddAt in the default bounds mode, reported late: the native backend throws IndexError from
+// inside the kernel call (CX/native/native_device/indexing.cc:68-74), which on a device would cost a read-back and a host wait
+// per call.  Instead each device has one sticky record of four int64 {set, index, extent, axis} in page-locked host memory that
+// kernels write through its device address, and the calls at which the host waits for the device anyway -- hipcx_synchronize and
+// hipcx_memcpy_to_host, the only points where results become visible (CX/cuda/cuda_device/memory.cc:94-122) -- look at it after
+// their wait: a set record is cleared and becomes their HIPCX_INDEX_ERROR.
+// DeferredIndexErrorRecord: the current device's record as a kernel argument (allocated on first use).
+// CheckDeferredIndexError: throws Error(HIPCX_INDEX_ERROR) if `device`'s record is set; the caller has just waited for the work.
+int64_t* DeferredIndexErrorRecord();
+void CheckDeferredIndexError(int device);
+
 #define HIPCX_CHECK_HIP(expr)                                                                           \
     do {                                                                                                \
         hipError_t e_ = (expr);                                                                         \

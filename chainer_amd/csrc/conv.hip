@@ -82,6 +82,9 @@ void LaunchShape(IGemmArgs<T> p, bool fast16, bool fast8, hipStream_t stream) {
     int64_t total = static_cast<int64_t>(p.tiles_m) * p.tiles_n;
     HIPCX_REQUIRE(total < (1LL << 30), HIPCX_NOT_IMPLEMENTED_ERROR, "problem too large for one launch");
     int per = static_cast<int>((total + 7) / 8);
+    // wide products: a row of concurrent tiles would read more second-operand panels than an XCD's L2 holds
+    static const int band_env = [] { const char* e = getenv("HIPCX_IGEMM_BAND"); return e != nullptr ? atoi(e) : 8; }();
+    p.band = p.tiles_n > 16 ? band_env : 0;
     static const bool pipe_env = [] { const char* e = getenv("HIPCX_IGEMM_PIPE"); return e != nullptr && e[0] == '1'; }();
     if (PM || pipe_env || !(fast16 || fast8) || p.partial == nullptr) p.ksplit = 1;  // only the simple fast kernel splits the reduction
     dim3 grid(per * 8, 1), block(64 * WM * WN);

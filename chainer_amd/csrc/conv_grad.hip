@@ -13,8 +13,11 @@
 // padded to Wp with zeros.  On that common grid tap (r, s) of channel c is the window of copy s that starts r rows down, so
 //     gw[k][c][r][s] = sum_n sum_q gy_p[n][k][q] * x_s[s][n][c][q + r*Wp],   q over OH*Wp
 // is one accumulated matrix product per image whose right-hand rows alias windows of the copies; the zero columns of gy_p cancel
-// the products that wrap around a row end.  (A non-finite x value therefore meets a zero of gy_p in windows the reference never
-// multiplies it into: inf or NaN in x can turn up as NaN in more filter taps than in the reference.)
+// the products that wrap around a row end.  A non-finite x value would meet a zero of gy_p in windows the reference never
+// multiplies it into (0 * inf = NaN in filter taps that stay finite there), so the copy kernel flags every input channel that holds
+// an inf or NaN and, after the product, GradWeightChannelFixupKernel computes the flagged channels' filter taps again the
+// reference's way (the sum over the Im2Col windows, padding multiplied as zeros).  With finite data that kernel's workgroups read
+// one flag each and exit.
 #include "common.h"
 
 namespace hipcx {
@@ -119,9 +122,20 @@ struct ShiftedArgs {
     const void* gy;
     void* xs;   // [kw][N*C][Hp*Wp]
     void* gyp;  // [N*K][OH*Wp]
+    int* nonfinite;  // [C]: set to 1 for channels of x that hold an inf or NaN (cleared by PaddedRowsKernel, which runs first)
     int planes_x, planes_gy;  // N*C, N*K
+    int C;
     int H, W, OH, OW, Hp, Wp, ph, pw, kw;
 };
+
+template <typename T>
+__device__ __forceinline__ bool NonFinite(T v) {
+    if constexpr (sizeof(T) == 2) {
+        return (__builtin_bit_cast(unsigned short, v) & 0x7c00u) == 0x7c00u;
+    } else {
+        return (__builtin_bit_cast(unsigned, v) & 0x7f800000u) == 0x7f800000u;
+    }
+}
 
 // xs[s][plane][q] = padded x[plane][q + s]; one thread writes VEC consecutive q.
 template <typename T, int VEC>
@@ -145,6 +159,12 @@ __global__ __launch_bounds__(256) void ShiftedPlanesKernel(ShiftedArgs p, unsign
             if (++wp == p.Wp) wp = 0, ++hp;
         }
         *reinterpret_cast<GVec<T, VEC>*>(xs + static_cast<int64_t>(idx) * VEC) = out;
+        if (s == 0) {  // copy 0 holds every element of x
+            bool bad = false;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) bad |= NonFinite<T>(out.v[e]);
+            if (bad) p.nonfinite[plane % static_cast<unsigned>(p.C)] = 1;
+        }
         if (idx + gridDim.x * 256u < idx) break;  // the next index would wrap
     }
 }
@@ -155,6 +175,9 @@ __global__ __launch_bounds__(256) void PaddedRowsKernel(ShiftedArgs p, unsigned 
     const T* gy = static_cast<const T*>(p.gy);
     T* gyp = static_cast<T*>(p.gyp);
     const unsigned per_row = static_cast<unsigned>(p.Wp / VEC);
+    if (blockIdx.x == 0) {
+        for (int c = threadIdx.x; c < p.C; c += 256) p.nonfinite[c] = 0;
+    }
     for (unsigned idx = blockIdx.x * 256u + threadIdx.x; idx < total; idx += gridDim.x * 256u) {
         const unsigned row = idx / per_row;  // plane * OH + oh: rows of gy are OW apart
         const int w0 = static_cast<int>(idx - row * per_row) * VEC;
@@ -164,6 +187,36 @@ __global__ __launch_bounds__(256) void PaddedRowsKernel(ShiftedArgs p, unsigned 
         for (int e = 0; e < VEC; ++e) out.v[e] = w0 + e < p.OW ? src[w0 + e] : T(0);
         *reinterpret_cast<GVec<T, VEC>*>(gyp + static_cast<int64_t>(idx) * VEC) = out;
         if (idx + gridDim.x * 256u < idx) break;
+    }
+}
+
+// Filter taps of the input channels flagged in `nonfinite`, summed the reference's way: gw[k][c][r][s] = sum over (n, oh, ow) of
+// gy[n][k][oh][ow] * col, col = x[n][c][oh*sh - ph + r][ow*sw - pw + s] or the padding's zero (still multiplied, as TensorDot
+// multiplies Im2Col's zeros: CX/native/native_device/conv.cc:91-124).  Grid (C, slices); a wave per output, lanes over the sum.
+template <typename T>
+__global__ __launch_bounds__(256) void GradWeightChannelFixupKernel(GradWeightArgs p, const int* nonfinite, T* gw) {
+    const int c = blockIdx.x;
+    if (nonfinite[c] == 0) return;
+    const T* x = static_cast<const T*>(p.x);
+    const T* gy = static_cast<const T*>(p.gy);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int taps = p.kh * p.kw, outputs = p.K * taps;
+    const int64_t plane = static_cast<int64_t>(p.OH) * p.OW, total = plane * p.N;
+    for (int o = blockIdx.y * 4 + wave; o < outputs; o += gridDim.y * 4) {
+        const int k = o / taps, r = (o - k * taps) / p.kw, s = o % p.kw;
+        float acc = 0.0f;
+        for (int64_t i = lane; i < total; i += 64) {
+            const int n = static_cast<int>(i / plane);
+            const int pix = static_cast<int>(i - n * plane);
+            const int oh = pix / p.OW, ow = pix - oh * p.OW;
+            const int ih = oh * p.sh - p.ph + r, iw = ow * p.sw - p.pw + s;
+            const float xv = (ih >= 0 && ih < p.H && iw >= 0 && iw < p.W)
+                                     ? static_cast<float>(x[((static_cast<int64_t>(n) * p.C + c) * p.H + ih) * p.W + iw]) : 0.0f;
+            acc += static_cast<float>(gy[(static_cast<int64_t>(n) * p.K + k) * plane + pix]) * xv;
+        }
+#pragma unroll
+        for (int d = 32; d > 0; d >>= 1) acc += __shfl_down(acc, d);
+        if (lane == 0) gw[(static_cast<int64_t>(k) * p.C + c) * taps + (o - k * taps)] = static_cast<T>(acc);
     }
 }
 
@@ -295,7 +348,7 @@ struct ShiftedPlan {
     bool ok = false;
     ShiftedArgs a{};
     int64_t depth = 0, plane = 0;  // OH*Wp; Hp*Wp
-    size_t xs_bytes = 0, gyp_bytes = 0, partial_bytes = 0;
+    size_t xs_bytes = 0, gyp_bytes = 0, partial_bytes = 0, flag_bytes = 0;
 };
 
 ShiftedPlan PlanShifted(const GradWeightPlan& pl, int dtype) {
@@ -313,7 +366,8 @@ ShiftedPlan PlanShifted(const GradWeightPlan& pl, int dtype) {
     if (xs_elems / epc >= (1LL << 32) || gyp_elems / epc >= (1LL << 32)) return sp;  // 32-bit vector indices in the copy kernels
     sp.a.planes_x = g.N * g.C, sp.a.planes_gy = g.N * g.K;
     sp.a.H = g.H, sp.a.W = g.W, sp.a.OH = g.OH, sp.a.OW = g.OW, sp.a.Hp = static_cast<int>(Hp), sp.a.Wp = static_cast<int>(Wp);
-    sp.a.ph = g.ph, sp.a.pw = g.pw, sp.a.kw = g.kw;
+    sp.a.ph = g.ph, sp.a.pw = g.pw, sp.a.kw = g.kw, sp.a.C = g.C;
+    sp.flag_bytes = RoundUp256(static_cast<size_t>(g.C) * sizeof(int));
     sp.depth = g.OH * Wp;
     sp.plane = Hp * Wp;
     sp.xs_bytes = RoundUp256(static_cast<size_t>(xs_elems * it));
@@ -328,12 +382,21 @@ void RunShiftedCopies(const ShiftedArgs& a, hipStream_t stream) {
     constexpr int VEC = 16 / sizeof(T);
     const int64_t cap = static_cast<int64_t>(NumCUs()) * 32;
     auto grid = [&](int64_t n) { int64_t b = (n + 255) / 256; return dim3(static_cast<unsigned>(b > cap ? cap : (b < 1 ? 1 : b))); };
-    const int64_t total_x = static_cast<int64_t>(a.kw) * a.planes_x * (a.Hp * a.Wp / VEC);
-    hipLaunchKernelGGL((ShiftedPlanesKernel<T, VEC>), grid(total_x), dim3(256), 0, stream, a, static_cast<unsigned>(total_x));
-    CheckLaunch("shifted planes (weight gradient)");
     const int64_t total_gy = static_cast<int64_t>(a.planes_gy) * a.OH * (a.Wp / VEC);
-    hipLaunchKernelGGL((PaddedRowsKernel<T, VEC>), grid(total_gy), dim3(256), 0, stream, a, static_cast<unsigned>(total_gy));
+    hipLaunchKernelGGL((PaddedRowsKernel<T, VEC>), grid(total_gy), dim3(256), 0, stream, a, static_cast<unsigned>(total_gy));  // clears the flags
     CheckLaunch("padded rows (weight gradient)");
+    const int64_t total_x = static_cast<int64_t>(a.kw) * a.planes_x * (a.Hp * a.Wp / VEC);
+    hipLaunchKernelGGL((ShiftedPlanesKernel<T, VEC>), grid(total_x), dim3(256), 0, stream, a, static_cast<unsigned>(total_x));  // sets them
+    CheckLaunch("shifted planes (weight gradient)");
+}
+
+template <typename T>
+void RunChannelFixup(const GradWeightArgs& g, const int* nonfinite, void* gw, hipStream_t stream) {
+    const int outputs = g.K * g.kh * g.kw;
+    const int slices = std::max(1, std::min(outputs / 4, 16));
+    hipLaunchKernelGGL((GradWeightChannelFixupKernel<T>), dim3(static_cast<unsigned>(g.C), static_cast<unsigned>(slices)), dim3(256), 0, stream, g,
+                       nonfinite, static_cast<T*>(gw));
+    CheckLaunch("non-finite channels (weight gradient)");
 }
 }  // namespace
 
@@ -350,7 +413,7 @@ size_t hipcx_conv_grad_weight_workspace_size(const hipcx_array* x, const hipcx_a
         const size_t direct = BatchedProductPartialBytes(pl.a.K, pl.a.C, static_cast<int64_t>(pl.a.H) * pl.a.W, pl.a.N, gw->dtype) + 256;
         const size_t staged = pl.col_bytes + pl.gyt_bytes + hipcx_dot_workspace_size(&pl.gy_t, &pl.col_view, &out);
         const ShiftedPlan sp = PlanShifted(pl, gw->dtype);
-        const size_t shifted = sp.ok ? sp.xs_bytes + sp.gyp_bytes + sp.partial_bytes + 256 : 0;
+        const size_t shifted = sp.ok ? sp.xs_bytes + sp.gyp_bytes + sp.partial_bytes + sp.flag_bytes + 256 : 0;
         return std::max(std::max(direct, staged), shifted);
     } catch (...) {
         return 0;
@@ -382,12 +445,13 @@ int hipcx_conv_grad_weight(const hipcx_array* x, const hipcx_array* gy, const in
         }
         ShiftedPlan sp = PlanShifted(pl, gw->dtype);
         if (sp.ok && reinterpret_cast<uintptr_t>(workspace) % 16 == 0 && reinterpret_cast<uintptr_t>(gw->data) % 16 == 0) {
-            const size_t need = sp.xs_bytes + sp.gyp_bytes + sp.partial_bytes;
+            const size_t need = sp.xs_bytes + sp.gyp_bytes + sp.partial_bytes + sp.flag_bytes;
             HIPCX_REQUIRE(workspace != nullptr && workspace_bytes >= need, HIPCX_CHAINERX_ERROR,
                           "conv_grad_weight workspace too small: need " + std::to_string(need) + " bytes");
             char* ws = static_cast<char*>(workspace);
             sp.a.x = x->data, sp.a.gy = gy->data;
             sp.a.xs = ws, sp.a.gyp = ws + sp.xs_bytes;
+            sp.a.nonfinite = reinterpret_cast<int*>(ws + sp.xs_bytes + sp.gyp_bytes + sp.partial_bytes);
             hipStream_t st = AsStream(stream);
             if (gw->dtype == HIPCX_FLOAT16) RunShiftedCopies<half_t>(sp.a, st);
             else RunShiftedCopies<float>(sp.a, st);
@@ -396,6 +460,8 @@ int hipcx_conv_grad_weight(const hipcx_array* x, const hipcx_array* gy, const in
                                  static_cast<int64_t>(g.C) * sp.plane, g.K, static_cast<int64_t>(g.C) * g.kh * g.kw, sp.depth, g.N, gw->data,
                                  sp.partial_bytes ? reinterpret_cast<float*>(ws + sp.xs_bytes + sp.gyp_bytes) : nullptr, st, g.kh, g.kw, sp.a.Wp,
                                  static_cast<int64_t>(g.N) * g.C * sp.plane);
+            if (gw->dtype == HIPCX_FLOAT16) RunChannelFixup<half_t>(g, sp.a.nonfinite, gw->data, st);
+            else RunChannelFixup<float>(g, sp.a.nonfinite, gw->data, st);
             return;
         }
         const size_t dot_bytes = hipcx_dot_workspace_size(&pl.gy_t, &pl.col_view, &out);

@@ -1,6 +1,7 @@
 // Library-wide state: last-error string, device queries.
 #include <cstdlib>
 #include <cstdint>
+#include <mutex>
 #include "common.h"
 
 namespace hipcx {
@@ -18,6 +19,44 @@ int64_t StreamingThresholdBytes() {
         return mb <= 0 ? INT64_MAX : mb * 1000000;
     }();
     return bytes;
+}
+
+namespace {
+constexpr int kMaxRecordDevices = 64;
+std::mutex g_record_mu;
+volatile int64_t* g_record_host[kMaxRecordDevices] = {};  // page-locked, four int64 per device
+int64_t* g_record_dev[kMaxRecordDevices] = {};            // the same memory as the device addresses it
+}  // namespace
+
+int64_t* DeferredIndexErrorRecord() {
+    int dev = 0;
+    HIPCX_CHECK_HIP(hipGetDevice(&dev));
+    HIPCX_REQUIRE(dev >= 0 && dev < kMaxRecordDevices, HIPCX_DEVICE_ERROR, "device index out of range");
+    std::lock_guard<std::mutex> lock(g_record_mu);
+    if (g_record_dev[dev] == nullptr) {
+        void* host = nullptr;
+        HIPCX_CHECK_HIP(hipHostMalloc(&host, 4 * sizeof(int64_t), hipHostMallocMapped | hipHostMallocCoherent));
+        for (int i = 0; i < 4; ++i) static_cast<volatile int64_t*>(host)[i] = 0;
+        void* devptr = nullptr;
+        HIPCX_CHECK_HIP(hipHostGetDevicePointer(&devptr, host, 0));
+        g_record_host[dev] = static_cast<volatile int64_t*>(host);
+        g_record_dev[dev] = static_cast<int64_t*>(devptr);
+    }
+    return g_record_dev[dev];
+}
+
+void CheckDeferredIndexError(int device) {
+    if (device < 0 || device >= kMaxRecordDevices) return;
+    int64_t index = 0, dim = 0, axis = 0;
+    {
+        std::lock_guard<std::mutex> lock(g_record_mu);
+        volatile int64_t* rec = g_record_host[device];
+        if (rec == nullptr || rec[0] == 0) return;
+        index = rec[1], dim = rec[2], axis = rec[3];
+        rec[0] = 0;
+    }
+    throw Error(HIPCX_INDEX_ERROR, "Index " + std::to_string(index) + " is out of bounds for axis " + std::to_string(axis) + " with size " +
+                                           std::to_string(dim) + " (an earlier take / add_at in the default bounds mode)");
 }
 
 int NumCUs() {
@@ -66,6 +105,7 @@ int hipcx_synchronize(int device_index) {
         hipError_t e = hipDeviceSynchronize();
         (void)hipSetDevice(prev);
         HIPCX_CHECK_HIP(e);
+        CheckDeferredIndexError(device_index);
     });
 }
 

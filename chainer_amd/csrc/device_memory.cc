@@ -46,6 +46,15 @@ public:
         return true;
     }
     void Free(void* ptr) noexcept override { (void)hipFree(ptr); }
+    // An event recorded behind the work `stream` holds now; the predicate polls it.  The event lives as long as the predicate.
+    std::function<bool()> Fence(void* stream) override {
+        SetDeviceScope scope(device_);
+        hipEvent_t ev = nullptr;
+        HIPCX_CHECK_HIP(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
+        std::shared_ptr<void> holder(ev, [](void* e) { (void)hipEventDestroy(static_cast<hipEvent_t>(e)); });
+        HIPCX_CHECK_HIP(hipEventRecord(ev, static_cast<hipStream_t>(stream)));
+        return [holder] { return hipEventQuery(static_cast<hipEvent_t>(holder.get())) == hipSuccess; };
+    }
 
 private:
     int device_;
@@ -128,6 +137,12 @@ std::array<std::shared_ptr<DeviceState>, kMaxDevices>& States() {
     return *states;
 }
 
+// Blocks that were in use when hipcx_pool_destroy took their pool away: see OrphanSet.
+OrphanSet& OrphansOf(int device) {
+    static auto* sets = new std::array<OrphanSet, kMaxDevices>();
+    return (*sets)[device];
+}
+
 std::shared_ptr<DeviceState> StateOf(int device, bool create = true) {
     HIPCX_REQUIRE(device >= 0 && device < kMaxDevices, HIPCX_DEVICE_ERROR, "invalid device index " + std::to_string(device));
     std::lock_guard<std::mutex> lock(StatesMutex());
@@ -196,9 +211,25 @@ int hipcx_malloc(int device, size_t bytes, void** ptr) { return hipcx_malloc_on_
 int hipcx_free(int device, void* ptr) {
     return GuardMemory([&] {
         if (ptr == nullptr) return;
+        HIPCX_REQUIRE(device >= 0 && device < kMaxDevices, HIPCX_DEVICE_ERROR, "invalid device index " + std::to_string(device));
+        // a block of a pool that hipcx_pool_destroy took away: its memory went with the pool (deleters outlive the pool), and the
+        // pool that may exist by now must not see this pointer
+        if (OrphansOf(device).Take(ptr)) return;
         std::shared_ptr<DeviceState> st = StateOf(device, false);
-        if (st == nullptr) return;  // the pool is gone and took its memory with it: nothing to do (deleters outlive the pool)
+        if (st == nullptr) return;
         st->device_pool->Free(ptr);
+    });
+}
+
+int hipcx_record_stream(int device, void* ptr, void* stream) {
+    return GuardMemory([&] {
+        if (ptr == nullptr) return;
+        std::shared_ptr<DeviceState> st = StateOf(device, false);
+        HIPCX_REQUIRE(st != nullptr, HIPCX_CHAINERX_ERROR, "record_stream: the device has no pool");
+        uint32_t partition = 0;
+        HIPCX_REQUIRE(st->device_pool->BlockPartition(ptr, &partition), HIPCX_CHAINERX_ERROR, "record_stream: not a block in use");
+        if (st->PartitionOf(AsStream(stream)) == partition) return;  // its own stream: ordered anyway
+        st->device_pool->RecordStream(ptr, stream);
     });
 }
 
@@ -254,6 +285,7 @@ int hipcx_pool_destroy(int device) {
         SetDeviceScope scope(device);
         (void)hipDeviceSynchronize();  // nothing may still run on memory that is about to go back to the driver
         st->DrainKeeper();
+        OrphansOf(device).Add(st->device_pool->InUsePointers());  // their frees are still to come: see hipcx_free
     });
 }
 
@@ -276,6 +308,7 @@ int hipcx_memcpy_to_host(int device, void* dst, const void* src, size_t bytes, v
         hipStream_t s = AsStream(stream);
         HIPCX_CHECK_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, s));
         HIPCX_CHECK_HIP(hipStreamSynchronize(s));
+        CheckDeferredIndexError(device);  // the bytes may come from a Take whose indices were out of range
     });
 }
 

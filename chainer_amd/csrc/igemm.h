@@ -37,6 +37,7 @@ struct IGemmArgs {
     int64_t M;                   // N*OH*OW
     int Kg;                      // R*S*C
     int tiles_m, tiles_n;
+    int band;                    // fast kernel: tile columns per band of the tile order (0: columns fast over the whole row)
     int out_vec;                 // 1 if the 4 accumulators a lane holds per group can be stored as one vector
     int out_wide;                // 1 if 16-byte runs along the output's contiguous axis can be stored (pipelined kernel)
     // Split reduction (matrix products with few output tiles and a long reduction axis, e.g. weight gradients): grid.x slices of
@@ -90,6 +91,26 @@ __device__ __forceinline__ bool TileOf(int tiles_m, int tiles_n, int b, int& til
 }
 __device__ __forceinline__ bool TileOf(int tiles_m, int tiles_n, int& tile_m, int& tile_n) {
     return TileOf(tiles_m, tiles_n, static_cast<int>(blockIdx.x), tile_m, tile_n);
+}
+// The same with the tile columns cut into bands of `band`: inside a band the column is still the fast index, and the rows are
+// walked before the next band starts.  The 32 tiles an XCD runs at a time then cover band columns x 32 / band rows and read
+// band + 32 / band operand panels instead of 33, and a band's filter panels stay in that XCD's L2 while its rows go by: for
+// products with many tile columns (wide matrix products) this is what keeps the second operand from being fetched once per tile row.
+__device__ __forceinline__ bool TileOfBanded(int tiles_m, int tiles_n, int band, int& tile_m, int& tile_n) {
+    if (band <= 0) return TileOf(tiles_m, tiles_n, tile_m, tile_n);
+    int total = tiles_m * tiles_n;
+    int per = (total + 7) / 8;
+    int b = static_cast<int>(blockIdx.x);
+    if (b >= per * 8) return false;
+    int logical = (b % 8) * per + b / 8;
+    if (logical >= total) return false;
+    int band_tiles = band * tiles_m;
+    int bi = logical / band_tiles;
+    int rem = logical - bi * band_tiles;
+    int cols = min(band, tiles_n - bi * band);
+    tile_n = bi * band + rem % cols;
+    tile_m = rem / cols;
+    return true;
 }
 
 template <typename T>
@@ -325,7 +346,7 @@ __global__ __launch_bounds__(64 * WM * WN) void IGemmFastKernel(IGemmArgs<T> p) 
         slice = blockIdx.x;
         tile_n = static_cast<int>(blockIdx.y) % p.tiles_n;
         tile_m = static_cast<int>(blockIdx.y) / p.tiles_n;
-    } else if (!TileOf(p.tiles_m, p.tiles_n, tile_m, tile_n)) {
+    } else if (!TileOfBanded(p.tiles_m, p.tiles_n, p.band, tile_m, tile_n)) {
         return;
     }
     const int m0 = tile_m * BM;

@@ -111,7 +111,8 @@ __global__ __launch_bounds__(256) void LstmStepKernel(LstmStepArgs args) {
         }
     };
     // Activations: a lane's operand for block kb of a chunk is four consecutive k of its row, one 16-byte load; the eight loads of
-    // a chunk are issued together.  Blocks past the end re-read the row's first block (their weights are zero).  Rows past the
+    // a chunk are issued together.  Blocks past the end load the row's first block (a valid address) and are then replaced by
+    // zeros: their weights are zero as well, but 0 * inf would be NaN where the reference forms no product at all.  Rows past the
     // step's batch read row 0: their products stay in accumulator rows that are never stored.
     constexpr int kBlocks = kChunk / 16;
     auto load_a = [&](int kc, float4_t* a) {
@@ -119,7 +120,8 @@ __global__ __launch_bounds__(256) void LstmStepKernel(LstmStepArgs args) {
         for (int kb = 0; kb < kBlocks; ++kb) {
             const int kglob = kc + kb * 16;
             const float* p = kglob < job.Xp ? xrow + kglob : (kglob < Kp ? hrow + (kglob - job.Xp) : hrow);  // (uniform selects)
-            a[kb] = *reinterpret_cast<const float4_t*>(p + 4 * lq);
+            const float4_t v = *reinterpret_cast<const float4_t*>(p + 4 * lq);
+            a[kb] = kglob < Kp ? v : float4_t{0.f, 0.f, 0.f, 0.f};
         }
     };
 

@@ -18,7 +18,9 @@
 //  * partitions: inside an arena, a freed block is only reused by allocations of the same partition.  The device layer
 //    uses one partition per HIP stream: work queued on a stream runs in order, so a block freed and reallocated on one
 //    stream needs no synchronisation, while another stream never gets it (the reference launches everything on one
-//    stream and has no such problem);
+//    stream and has no such problem).  That covers a block used on the stream it was allocated for.  A block that is also
+//    used on another stream is announced with RecordStream; its Free then holds it back until that stream has caught up.
+//    Without the announcement the owner must not free the block before the foreign stream's work on it was waited for;
 //  * when the device allocator reports failure only the general arena's cache is released: the blocks of a graph's
 //    arena stay where the graph expects them.
 #pragma once
@@ -33,6 +35,7 @@
 #include <stdexcept>
 #include <string>
 #include <unordered_map>
+#include <unordered_set>
 #include <utility>
 #include <vector>
 
@@ -46,6 +49,12 @@ public:
     virtual ~Allocator() = default;
     virtual bool Malloc(void** ptr, size_t bytes) = 0;  // false: out of memory (any other failure throws)
     virtual void Free(void* ptr) noexcept = 0;
+    // A predicate that turns true once the work queued on `stream` up to now has run (device memory: an event recorded on the
+    // stream).  An empty function: nothing to wait for.  Used for blocks that were announced with MemoryPool::RecordStream.
+    virtual std::function<bool()> Fence(void* stream) {
+        (void)stream;
+        return {};
+    }
 };
 
 class OutOfMemoryError : public std::runtime_error {  // CX/cuda/memory_pool.h:34-37
@@ -99,6 +108,7 @@ public:
         const size_t size = RoundSize(bytes);
         const uint64_t arena = Key(arena_number, partition);
         std::lock_guard<std::mutex> lock(mutex_);
+        CollectPendingLocked();
         void* ptr = nullptr;
         auto a = free_.find(arena);
         if (a != free_.end()) {
@@ -121,25 +131,67 @@ public:
             }
             ++stats_.allocator_calls;
         }
-        in_use_.emplace(ptr, Block{size, arena});
+        in_use_.emplace(ptr, Block{size, arena, {}});
         stats_.in_use_bytes += size;
         ++stats_.in_use_blocks;
         return ptr;
     }
 
     // Returns the block to the free lists of the arena it came from.  Throws for a pointer that is not in use.
+    // A block with recorded streams (RecordStream) is held back -- still counted as in use -- until the work those streams had
+    // queued at this moment has run; Malloc and FreeUnusedBlocks move such blocks on.
     void Free(void* ptr) {
         if (ptr == nullptr) return;
         std::lock_guard<std::mutex> lock(mutex_);
         auto it = in_use_.find(ptr);
         if (it == in_use_.end()) throw std::runtime_error("Cannot free out-of-pool memory");
-        const Block b = it->second;
-        in_use_.erase(it);
-        stats_.in_use_bytes -= b.size;
-        --stats_.in_use_blocks;
-        free_[b.arena][b.size].push_back(ptr);
-        stats_.cached_bytes += b.size;
-        ++stats_.cached_blocks;
+        if (pending_.count(ptr) != 0) throw std::runtime_error("Cannot free out-of-pool memory");  // freed twice
+        if (!it->second.streams.empty()) {
+            std::vector<std::function<bool()>> fences;
+            for (void* stream : it->second.streams) {
+                std::function<bool()> f = allocator_->Fence(stream);
+                if (f) fences.push_back(std::move(f));
+            }
+            it->second.streams.clear();
+            if (!fences.empty()) {
+                pending_.emplace(ptr, std::move(fences));
+                return;
+            }
+        }
+        ReleaseLocked(it);
+    }
+    // `ptr` (in use) has work queued on `stream`, which is not the stream it was allocated for: its Free must not hand the block
+    // to a new owner before that work has run.  The caller filters out the block's own stream (BlockPartition).
+    void RecordStream(void* ptr, void* stream) {
+        std::lock_guard<std::mutex> lock(mutex_);
+        auto it = in_use_.find(ptr);
+        if (it == in_use_.end() || pending_.count(ptr) != 0) throw std::runtime_error("record_stream: not a block in use");
+        for (void* s : it->second.streams) {
+            if (s == stream) return;
+        }
+        it->second.streams.push_back(stream);
+    }
+    // The partition (stream) the block was allocated for; false if `ptr` is not in use.
+    bool BlockPartition(void* ptr, uint32_t* partition) const {
+        std::lock_guard<std::mutex> lock(mutex_);
+        auto it = in_use_.find(ptr);
+        if (it == in_use_.end()) return false;
+        *partition = PartitionOf(it->second.arena);
+        return true;
+    }
+    // Pointers handed out and not yet freed (blocks held back by Free included).
+    std::vector<void*> InUsePointers() const {
+        std::lock_guard<std::mutex> lock(mutex_);
+        std::vector<void*> v;
+        v.reserve(in_use_.size());
+        for (auto& kv : in_use_) {
+            if (pending_.count(kv.first) == 0) v.push_back(kv.first);
+        }
+        return v;
+    }
+    size_t pending_blocks() const {
+        std::lock_guard<std::mutex> lock(mutex_);
+        return pending_.size();
     }
     void FreeNoExcept(void* ptr) noexcept {
         try {
@@ -151,6 +203,7 @@ public:
     // Gives the cached blocks of the general arena back to the allocator (MemoryPool::FreeUnusedBlocks, memory_pool.cc:172-203).
     void FreeUnusedBlocks() {
         std::lock_guard<std::mutex> lock(mutex_);
+        CollectPendingLocked();
         ReleaseCachedLocked();
     }
 
@@ -200,7 +253,31 @@ private:
     struct Block {
         size_t size;
         uint64_t arena;  // Key(arena, partition)
+        std::vector<void*> streams;  // RecordStream
     };
+    void ReleaseLocked(std::unordered_map<void*, Block>::iterator it) {
+        void* ptr = it->first;
+        const size_t size = it->second.size;
+        const uint64_t arena = it->second.arena;
+        in_use_.erase(it);
+        stats_.in_use_bytes -= size;
+        --stats_.in_use_blocks;
+        free_[arena][size].push_back(ptr);
+        stats_.cached_bytes += size;
+        ++stats_.cached_blocks;
+    }
+    void CollectPendingLocked() {
+        for (auto p = pending_.begin(); p != pending_.end();) {
+            bool done = true;
+            for (auto& fence : p->second) done = done && fence();
+            if (!done) {
+                ++p;
+                continue;
+            }
+            ReleaseLocked(in_use_.find(p->first));
+            p = pending_.erase(p);
+        }
+    }
     static uint64_t Key(int arena, uint32_t partition) { return (static_cast<uint64_t>(static_cast<uint32_t>(arena)) << 32) | partition; }
     static int ArenaOf(uint64_t key) { return static_cast<int>(key >> 32); }
     static uint32_t PartitionOf(uint64_t key) { return static_cast<uint32_t>(key & 0xffffffffu); }
@@ -224,9 +301,39 @@ private:
     std::unique_ptr<Allocator> allocator_;
     mutable std::mutex mutex_;
     std::unordered_map<void*, Block> in_use_;
+    std::unordered_map<void*, std::vector<std::function<bool()>>> pending_;  // freed, waiting for foreign streams (still in in_use_)
     std::map<uint64_t, std::map<size_t, std::vector<void*>>> free_;  // (arena, partition) -> rounded size -> blocks
     std::atomic<int> current_arena_{0};
     PoolStats stats_;
+};
+
+// Pointers that were still in use when a device's pool was destroyed (the pool takes their memory with it).  Their owners'
+// deleters run later, perhaps after a new pool exists on the device -- which may even have been given the same address again.
+// Such a free must not reach the new pool: the first Free of an orphaned address is swallowed here.  (If the new pool did hand
+// the address out again and its new owner frees first, that free is the one swallowed and the block stays allocated until the
+// stale free arrives: late, never wrong.)  The reference ties each deleter to its pool object with a weak_ptr instead
+// (CX/cuda/cuda_device/memory.cc:19-24); a C ABI that frees by (device, pointer) needs the bookkeeping on this side.
+class OrphanSet {
+public:
+    void Add(const std::vector<void*>& ptrs) {
+        std::lock_guard<std::mutex> lock(mutex_);
+        for (void* p : ptrs) orphans_.insert(p);
+    }
+    bool Take(void* ptr) {  // true: ptr was an orphan and is now forgotten
+        std::lock_guard<std::mutex> lock(mutex_);
+        auto it = orphans_.find(ptr);
+        if (it == orphans_.end()) return false;
+        orphans_.erase(it);
+        return true;
+    }
+    size_t size() const {
+        std::lock_guard<std::mutex> lock(mutex_);
+        return orphans_.size();
+    }
+
+private:
+    mutable std::mutex mutex_;
+    std::unordered_multiset<void*> orphans_;
 };
 
 }  // namespace hipcx

@@ -260,8 +260,9 @@ __global__ __launch_bounds__(256) void GlobalAvgPoolKernel(const T* x, T* out, i
             const int nwords = (hw + 2) / 2;  // the same trip count for every lane; halves outside the plane are skipped
 #pragma unroll 8
             for (int j = 0; j < nwords; ++j) {
-                const unsigned u = pw[j];
                 const int e = 2 * j - odd;  // element held by the lower half
+                const unsigned u = e < hw ? pw[j] : 0u;  // the last trip of a plane that starts on a word boundary holds nothing of it: no read
+                                                         // (for the workgroup's last plane that word would lie past the end of the LDS)
                 if (e >= 0 && e < hw) acc += lower(u);
                 if (e + 1 < hw) acc += upper(u);
             }

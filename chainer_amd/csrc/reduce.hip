@@ -938,23 +938,38 @@ void Run(const hipcx_array* a, const int8_t* axis, int naxis, const hipcx_array*
     CheckLaunch("generic_reduce");
 }
 
-// The device address of `scratch` on the current device.  In host code the array's name is only a handle for this lookup,
-// never an address a kernel may be given.  Looked up once per device, with that device current.
-void* StaticScratchAddress() {
+// What a device needs for hipcx_sum_static_scratch, set up on the first call there with that device current:
+//   address   the device address of `scratch`.  In host code the array's name is only a handle for this lookup, never an address a
+//             kernel may be given.
+//   done      an event recorded behind each call's kernels.  The array is one per device, so a call on another stream than the
+//             previous one first makes its stream wait for that event: calls from different streams or host threads take turns on
+//             the array instead of racing.  (Calls issued into a stream that is being captured are not chained: a graph replays at
+//             times of its owner's choosing, who then orders it against other users of the array.)
+struct StaticScratchSlot {
+    std::mutex mu;  // host threads issue their calls one at a time
+    void* address = nullptr;
+    hipEvent_t done = nullptr;
+    hipStream_t last = nullptr;
+    bool pending = false;
+};
+
+StaticScratchSlot& StaticScratchOfCurrentDevice() {
     constexpr int kMaxDevices = 64;
     static std::mutex mu;
-    static void* address[kMaxDevices] = {};
+    static StaticScratchSlot slots[kMaxDevices];
     int dev = 0;
     HIPCX_CHECK_HIP(hipGetDevice(&dev));
     HIPCX_REQUIRE(dev >= 0 && dev < kMaxDevices, HIPCX_DEVICE_ERROR, "device index beyond the static scratch table");
     std::lock_guard<std::mutex> lock(mu);
-    if (address[dev] == nullptr) {
+    StaticScratchSlot& slot = slots[dev];
+    if (slot.address == nullptr) {
         void* ptr = nullptr;
         HIPCX_CHECK_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
         HIPCX_REQUIRE(ptr != nullptr, HIPCX_BACKEND_ERROR, "hipGetSymbolAddress returned a null address for the static scratch");
-        address[dev] = ptr;
+        HIPCX_CHECK_HIP(hipEventCreateWithFlags(&slot.done, hipEventDisableTiming));
+        slot.address = ptr;
     }
-    return address[dev];
+    return slot;
 }
 
 }  // namespace
@@ -1001,8 +1016,8 @@ int hipcx_sum(const hipcx_array* a, const int8_t* axis, int naxis, const hipcx_a
 
 // hipcx_sum for callers that can neither allocate a workspace nor have one allocated for them: the per-block / per-slice
 // partial results go to the library's own static device array.  Same kernels and launch plan as hipcx_sum, hence the same bits.
-// Every partial is written before it is read, so nothing has to be cleared between calls; calls that overlap on one device
-// (different streams or threads) share the array and race.
+// Every partial is written before it is read, so nothing has to be cleared between calls; calls from different streams or host
+// threads on one device share the array and are chained through an event (see StaticScratchSlot) -- except under stream capture.
 int hipcx_sum_static_scratch(const hipcx_array* a, const int8_t* axis, int naxis, const hipcx_array* out, void* stream) {
     int status = Guard([&] {
         ValidateArray(a, "a");
@@ -1013,10 +1028,32 @@ int hipcx_sum_static_scratch(const hipcx_array* a, const int8_t* axis, int naxis
                               std::to_string(static_cast<size_t>(HIPCX_STATIC_SCRATCH_BYTES)) + "; use hipcx_sum with a workspace");
     });
     if (status != HIPCX_OK) return status;
-    void* ptr = nullptr;
-    status = Guard([&] { ptr = StaticScratchAddress(); });
+    StaticScratchSlot* slot = nullptr;
+    status = Guard([&] { slot = &StaticScratchOfCurrentDevice(); });
     if (status != HIPCX_OK) return status;
-    return hipcx_sum(a, axis, naxis, out, ptr, HIPCX_STATIC_SCRATCH_BYTES, stream);
+    std::lock_guard<std::mutex> lock(slot->mu);
+    hipStream_t s = AsStream(stream);
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &capture) != hipSuccess) {
+        (void)hipGetLastError();
+        capture = hipStreamCaptureStatusActive;  // cannot tell: leave the stream alone
+    }
+    const bool chained = capture == hipStreamCaptureStatusNone;
+    if (chained && slot->pending && slot->last != s) {
+        status = Guard([&] { HIPCX_CHECK_HIP(hipStreamWaitEvent(s, slot->done, 0)); });
+        if (status != HIPCX_OK) return status;
+    }
+    status = hipcx_sum(a, axis, naxis, out, slot->address, HIPCX_STATIC_SCRATCH_BYTES, stream);
+    if (chained) {
+        int recorded = Guard([&] { HIPCX_CHECK_HIP(hipEventRecord(slot->done, s)); });
+        if (recorded == HIPCX_OK) {
+            slot->last = s;
+            slot->pending = true;
+        } else if (status == HIPCX_OK) {
+            status = recorded;
+        }
+    }
+    return status;
 }
 
 int hipcx_amax(const hipcx_array* a, const int8_t* axis, int naxis, const hipcx_array* out, void* workspace, size_t workspace_bytes,

@@ -29,7 +29,9 @@ struct TakeArgs {
     int64_t axis_stride;  // bytes
     int idx_dtype;
     int mode;
+    int axis;
     int32_t* error_flag;
+    int64_t* deferred;  // used when error_flag is null (DEFAULT mode)
     int64_t total;  // work items: elements, or 16-byte vectors on the row path
     int64_t right_vecs;  // row path: 16-byte vectors per row
 };
@@ -54,7 +56,10 @@ __device__ __forceinline__ int64_t LoadIndex(const char* p, int dtype) {
     }
 }
 
-__device__ __forceinline__ int64_t ResolveIndex(int64_t index, int64_t dim, int mode, int32_t* error_flag) {
+// An out-of-range index in the DEFAULT / RAISE modes is reported and replaced by 0 (the access stays in bounds; the caller discards
+// the result).  Reported where: the caller's flag, or -- deferred -- the device's sticky record {set, index, extent, axis} in
+// page-locked host memory, which the next synchronising call turns into the IndexError (see DeferredIndexErrorRecord).
+__device__ __forceinline__ int64_t ResolveIndex(int64_t index, int64_t dim, int mode, int32_t* error_flag, int64_t* deferred, int axis) {
     if (mode == HIPCX_BOUNDS_CLIP) {
         return index < 0 ? 0 : (index >= dim ? dim - 1 : index);
     }
@@ -63,8 +68,13 @@ __device__ __forceinline__ int64_t ResolveIndex(int64_t index, int64_t dim, int 
         return index % dim;
     }
     if (index < -dim || index >= dim) {
-        *error_flag = 1;
-        return 0;  // stay in bounds; the caller discards the result
+        if (error_flag != nullptr) {
+            *error_flag = 1;
+        } else {
+            deferred[1] = index, deferred[2] = dim, deferred[3] = axis;
+            deferred[0] = 1;
+        }
+        return 0;
     }
     return index < 0 ? index + dim : index;
 }
@@ -82,7 +92,7 @@ __global__ __launch_bounds__(256) void TakeKernel(TakeArgs t) {
             int64_t v = w - i * t.right_vecs;
             int64_t ioff = 0, unused = 0;
             Decompose(t.index, i, ioff, unused);
-            int64_t index = ResolveIndex(LoadIndex(t.idx + ioff, t.idx_dtype), t.axis_dim, t.mode, t.error_flag);
+            int64_t index = ResolveIndex(LoadIndex(t.idx + ioff, t.idx_dtype), t.axis_dim, t.mode, t.error_flag, t.deferred, t.axis);
             *reinterpret_cast<Elem*>(t.out + w * BYTES) = *reinterpret_cast<const Elem*>(t.a + index * t.axis_stride + v * BYTES);
         } else {
             int64_t r = w % t.right.total;
@@ -93,7 +103,7 @@ __global__ __launch_bounds__(256) void TakeKernel(TakeArgs t) {
             Decompose(t.left, l, a_off, o_off);
             Decompose(t.right, r, a_off, o_off);
             Decompose(t.index, i, ioff, o_off);
-            int64_t index = ResolveIndex(LoadIndex(t.idx + ioff, t.idx_dtype), t.axis_dim, t.mode, t.error_flag);
+            int64_t index = ResolveIndex(LoadIndex(t.idx + ioff, t.idx_dtype), t.axis_dim, t.mode, t.error_flag, t.deferred, t.axis);
             *reinterpret_cast<Elem*>(t.out + o_off) = *reinterpret_cast<const Elem*>(t.a + a_off + index * t.axis_stride);
         }
     }
@@ -111,7 +121,7 @@ __global__ __launch_bounds__(256) void TakeRowsKernel(TakeArgs t) {
     for (int64_t i = static_cast<int64_t>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6); i < t.index.total; i += waves) {
         int64_t ioff = 0, unused = 0;
         Decompose(t.index, i, ioff, unused);
-        const int64_t index = ResolveIndex(LoadIndex(t.idx + ioff, t.idx_dtype), t.axis_dim, t.mode, t.error_flag);
+        const int64_t index = ResolveIndex(LoadIndex(t.idx + ioff, t.idx_dtype), t.axis_dim, t.mode, t.error_flag, t.deferred, t.axis);
         const Elem* src = reinterpret_cast<const Elem*>(t.a + index * t.axis_stride);
         Elem* dst = reinterpret_cast<Elem*>(t.out + i * t.right_vecs * BYTES);
 #pragma unroll 4
@@ -136,7 +146,7 @@ __global__ __launch_bounds__(256) void AddAtKernel(TakeArgs t) {
     for (int64_t i = 0; i < t.index.total; ++i) {
         int64_t ioff = 0, bo = b_off;
         Decompose(t.index, i, ioff, bo);
-        const int64_t index = ResolveIndex(LoadIndex(t.idx + ioff, t.idx_dtype), t.axis_dim, t.mode, t.error_flag);
+        const int64_t index = ResolveIndex(LoadIndex(t.idx + ioff, t.idx_dtype), t.axis_dim, t.mode, t.error_flag, t.deferred, t.axis);
         T* dst = reinterpret_cast<T*>(acc_base + index * t.axis_stride);
         const T bv = *reinterpret_cast<const T*>(t.out + bo);
         if constexpr (std::is_same<T, bool>::value) {
@@ -178,8 +188,8 @@ extern "C" int hipcx_take(const hipcx_array* a, const hipcx_array* indices, int8
                       HIPCX_DTYPE_ERROR, "Only arrays of integer dtype can be used as indices.");
         HIPCX_REQUIRE(out->dtype == a->dtype, HIPCX_DTYPE_ERROR, "take: out must have a's dtype");
         HIPCX_REQUIRE(mode >= HIPCX_BOUNDS_DEFAULT && mode <= HIPCX_BOUNDS_CLIP, HIPCX_CHAINERX_ERROR, "take: invalid bounds mode");
-        HIPCX_REQUIRE(error_flag != nullptr || mode == HIPCX_BOUNDS_WRAP || mode == HIPCX_BOUNDS_CLIP, HIPCX_CHAINERX_ERROR,
-                      "take: the default and raise bounds modes report out-of-range indices through error_flag, which is null");
+        HIPCX_REQUIRE(error_flag != nullptr || mode != HIPCX_BOUNDS_RAISE, HIPCX_CHAINERX_ERROR,
+                      "take: the raise bounds mode reports out-of-range indices through error_flag, which is null");
         HIPCX_REQUIRE(out->ndim == a->ndim - 1 + indices->ndim, HIPCX_DIMENSION_ERROR, "take: out has the wrong number of dimensions");
         TakeArgs t{};
         t.a = static_cast<const char*>(a->data);
@@ -189,7 +199,9 @@ extern "C" int hipcx_take(const hipcx_array* a, const hipcx_array* indices, int8
         t.axis_stride = a->strides[axis];
         t.idx_dtype = indices->dtype;
         t.mode = mode;
+        t.axis = axis;
         t.error_flag = error_flag;
+        if (error_flag == nullptr && mode == HIPCX_BOUNDS_DEFAULT) t.deferred = DeferredIndexErrorRecord();
         t.left.total = t.index.total = t.right.total = 1;
         int o = 0;
         for (int d = 0; d < axis; ++d, ++o) {
@@ -281,8 +293,8 @@ extern "C" int hipcx_add_at(const hipcx_array* a, const hipcx_array* indices, in
                       HIPCX_DTYPE_ERROR, "Only arrays of integer dtype can be used as indices.");
         HIPCX_REQUIRE(out->dtype == a->dtype && b->dtype == a->dtype, HIPCX_DTYPE_ERROR, "add_at: a, b and out must share a dtype");
         HIPCX_REQUIRE(mode >= HIPCX_BOUNDS_DEFAULT && mode <= HIPCX_BOUNDS_CLIP, HIPCX_CHAINERX_ERROR, "add_at: invalid bounds mode");
-        HIPCX_REQUIRE(error_flag != nullptr || mode == HIPCX_BOUNDS_WRAP || mode == HIPCX_BOUNDS_CLIP, HIPCX_CHAINERX_ERROR,
-                      "add_at: the default and raise bounds modes report out-of-range indices through error_flag, which is null");
+        HIPCX_REQUIRE(error_flag != nullptr || mode != HIPCX_BOUNDS_RAISE, HIPCX_CHAINERX_ERROR,
+                      "add_at: the raise bounds mode reports out-of-range indices through error_flag, which is null");
         HIPCX_REQUIRE(SameShape(a, out), HIPCX_DIMENSION_ERROR, "add_at: out must have a's shape");
         HIPCX_REQUIRE(b->ndim == a->ndim - 1 + indices->ndim, HIPCX_DIMENSION_ERROR, "add_at: b has the wrong number of dimensions");
         TakeArgs t{};
@@ -293,7 +305,9 @@ extern "C" int hipcx_add_at(const hipcx_array* a, const hipcx_array* indices, in
         t.axis_stride = out->strides[axis];
         t.idx_dtype = indices->dtype;
         t.mode = mode;
+        t.axis = axis;
         t.error_flag = error_flag;
+        if (error_flag == nullptr && mode == HIPCX_BOUNDS_DEFAULT) t.deferred = DeferredIndexErrorRecord();
         t.left.total = t.index.total = t.right.total = 1;
         int o = 0;
         for (int d = 0; d < axis; ++d, ++o) {

@@ -48,6 +48,10 @@ def capture(fn):
             del out
             if pool_stats()['device_allocations'] == before:
                 break
+        else:
+            raise RuntimeError('capture: fn() still took new memory from the driver in each of its %d warm passes (it allocates more '
+                               'from pass to pass, e.g. by keeping its results alive); a pass that allocates cannot be captured'
+                               % MAX_WARM_PASSES)
         gc.collect()
         graph = t.cuda.CUDAGraph()
         with t.cuda.graph(graph, stream=stream):

@@ -1249,10 +1249,13 @@ public:
             case IndexBoundsMode::kClip: m = HIPCX_BOUNDS_CLIP; break;
             default: break;
         }
-        bool checks = m == HIPCX_BOUNDS_DEFAULT || m == HIPCX_BOUNDS_RAISE;
+        // kRaise: checked here, at the cost of a read-back (native_device/indexing.cc:68-74).  kDefault, what the routine passes
+        // for mode=None: no flag -- the library records an out-of-range index on the device and HipDevice::Synchronize /
+        // MemoryCopyTo, the calls that wait for the device, throw the IndexError before any result can be read.
+        bool checks = m == HIPCX_BOUNDS_RAISE;
         std::shared_ptr<void> flag = checks ? NewDeviceFlag(device) : nullptr;
         Check(hipcx_take(&ca, &ci, axis, &co, m, static_cast<int32_t*>(flag.get()), nullptr));
-        if (checks) {  // native raises IndexError on an out-of-range index (native_device/indexing.cc:68-74)
+        if (checks) {
             const int32_t host = ReadDeviceFlag(device, flag);
             if (host != 0) throw IndexError{"Index is out of bounds for axis ", static_cast<int>(axis), " with size ", a.shape()[axis]};
         }
@@ -1277,7 +1280,7 @@ public:
         SetDeviceScope scope{device.index()};
         hipcx_array ca = ToC(a), ci = ToC(indices), cb = ToC(Cast(b, a.dtype())), co = ToC(out);
         int m = ToC(mode);
-        bool checks = m == HIPCX_BOUNDS_DEFAULT || m == HIPCX_BOUNDS_RAISE;
+        bool checks = m == HIPCX_BOUNDS_RAISE;  // kDefault: deferred, as in HipTakeKernel
         std::shared_ptr<void> flag = checks ? NewDeviceFlag(device) : nullptr;
         Check(hipcx_add_at(&ca, &ci, axis, &cb, &co, m, static_cast<int32_t*>(flag.get()), nullptr));
         if (checks) {

@@ -1386,8 +1386,10 @@ _BOUNDS = {None: 0, 'raise': 1, 'wrap': 2, 'clip': 3}
 
 
 def take(a, indices, axis, mode=None):
-    """Take (CX/routines/indexing.cc:171-205). mode None / 'raise' raise IndexError on out-of-range ids like the
-    native backend; checking that costs one 4-byte read-back after the kernel."""
+    """Take (CX/routines/indexing.cc:171-205).  mode 'raise' raises IndexError on out-of-range ids from this call, like the native
+    backend (one 4-byte read-back after the kernel).  mode None -- what the reference's callers pass -- raises it too, but late: the
+    kernel records the bad index on the device and the next call that waits for the device (``get`` / ``synchronize``) raises, so
+    a loop of take calls never waits for the host and can be captured into a graph."""
     if _kind(indices.dtype) not in (1, 2):
         raise _lib.DtypeError('Only arrays of integer dtype can be used as indices.')
     axis = _normalize_axis(axis, a.ndim)
@@ -1396,7 +1398,7 @@ def take(a, indices, axis, mode=None):
     m = _BOUNDS[mode]
     flag = None
     flag_ptr = None
-    if m in (0, 1):
+    if m == 1:
         flag = zeros((1,), 'int32')
         flag_ptr = ctypes.cast(ctypes.c_void_p(flag.data_ptr), ctypes.POINTER(ctypes.c_int32))
     _lib.call('hipcx_take', a.desc(), indices.desc(), axis, out.desc(), m, flag_ptr, current_stream())
@@ -1417,7 +1419,7 @@ def add_at(a, indices, axis, b, mode=None):
     m = _BOUNDS[mode]
     flag = None
     flag_ptr = None
-    if m in (0, 1):
+    if m == 1:
         flag = zeros((1,), 'int32')
         flag_ptr = ctypes.cast(ctypes.c_void_p(flag.data_ptr), ctypes.POINTER(ctypes.c_int32))
     _lib.call('hipcx_add_at', a.desc(), indices.desc(), axis, b.astype(a.dtype, False).desc(), out.desc(), m, flag_ptr, current_stream())

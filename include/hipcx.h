@@ -106,7 +106,13 @@ int hipcx_device_name(int device_index, char* buf, size_t buf_len);
  *   hipcx_malloc            Device::Allocate, device.h:33 (0 bytes -> NULL, CX/native/native_device/memory.cc:14-19)
  *   hipcx_free              the deleter of an allocation (cuda_device/memory.cc:19-24): returns the block to the pool; a pointer
  *                           the pool does not hold is HIPCX_CHAINERX_ERROR (memory_pool.cc:262-264); after hipcx_pool_destroy
- *                           it does nothing (the pool took its memory with it)
+ *                           it does nothing (the pool took its memory with it), also when a new pool exists on the device by then
+ *   hipcx_record_stream     no counterpart in the reference (it launches everything on one stream): announces that `ptr`, a block
+ *                           in use, has work queued on `stream`, a stream other than the one it was allocated for
+ *                           (hipcx_malloc: the null stream).  hipcx_free then keeps the block out of the free lists until the work
+ *                           that stream holds at the time of the free has run.  Without the announcement a block must not be
+ *                           freed before its last use on a foreign stream was waited for: a block goes back to the free list of
+ *                           its own stream at once and the next allocation there may overwrite it
  *   hipcx_pool_free_unused  MemoryPool::FreeUnusedBlocks, memory_pool.cc:172-203
  *   hipcx_pool_destroy      ~MemoryPool (memory_pool.cc:160-170): waits for the device, then gives every block back to the driver
  *   hipcx_memcpy_from_host  Device::MemoryCopyFrom with a native source = MemoryCopyFromHostAsync (cuda_device/memory.cc:37-51): the
@@ -136,6 +142,7 @@ typedef struct hipcx_pool_stats_t {
 int hipcx_malloc(int device, size_t bytes, void** ptr);
 int hipcx_malloc_on_stream(int device, size_t bytes, void* stream, void** ptr);
 int hipcx_free(int device, void* ptr);
+int hipcx_record_stream(int device, void* ptr, void* stream);
 int hipcx_pool_free_unused(int device);
 int hipcx_pool_stats(int device, hipcx_pool_stats_t* stats);
 int hipcx_pool_set_arena(int device, int arena);
@@ -380,8 +387,9 @@ int hipcx_fixed_batch_norm(const hipcx_array* x, const hipcx_array* gamma, const
 /* ---- ConvGradWeightKernel CX/kernels/connection.h:34-49 (2-D, C-contiguous NCHW x and gy in gw's float dtype) ----
  * gw[k, c, r, s] = sum over n, oh, ow of gy[n, k, oh, ow] * x[n, c, oh*stride - pad + r, ow*stride - pad + s]: the native
  * backend's TensorDot(gy, Im2Col(x)) (CX/native/native_device/conv.cc:91-124), equal to tolerance (float accumulation).
- * For filters larger than 1x1 at stride 1 (float16 / float32) the sum runs over zero-padded rows, in which every x value is
- * also multiplied by zeros of a padded gy: an inf or NaN in x may appear as NaN in filter taps the reference leaves finite. */
+ * inf / NaN in x or gy give the reference's inf / NaN in the reference's filter taps: the route for filters larger than 1x1 at
+ * stride 1 (float16 / float32), whose sum runs over zero-padded rows in which an x value also meets zeros of a padded gy, notes
+ * the input channels that hold a non-finite value and sums their taps again over the reference's windows. */
 size_t hipcx_conv_grad_weight_workspace_size(const hipcx_array* x, const hipcx_array* gy, const hipcx_array* gw, const int64_t* stride,
                                              const int64_t* pad, int cover_all);
 int hipcx_conv_grad_weight(const hipcx_array* x, const hipcx_array* gy, const int64_t* stride, const int64_t* pad, int cover_all,
@@ -479,11 +487,18 @@ int hipcx_average_pool_grad(const hipcx_array* gout, const int64_t* kernel_size,
                             const hipcx_array* gx, void* stream);
 
 /* ---- indexing: TakeKernel CX/kernels/indexing.h:17 ----
- * `error_flag` is a device int32 the caller zeroes before the call; with mode DEFAULT/RAISE the
- * kernel stores 1 there when an index is out of range (the native backend raises IndexError,
- * CX/native/native_device/indexing.cc:68-74); the plugin reads it back and throws.  It may be NULL
- * only for the WRAP and CLIP modes; DEFAULT/RAISE without it is refused with HIPCX_CHAINERX_ERROR
- * (no silent wrapping).  Nothing is written to `out` by a call that is refused. */
+ * Out-of-range indices in the DEFAULT and RAISE modes (the native backend throws IndexError from the kernel call,
+ * CX/native/native_device/indexing.cc:68-74):
+ *   `error_flag` not NULL: a device int32 the caller zeroes before the call; the kernel stores 1 there when an index is out of
+ *       range; the caller reads it back and throws (one host wait per call).
+ *   `error_flag` NULL, mode DEFAULT (what the routine passes for mode=None): the kernel records {index, extent, axis} in a sticky
+ *       per-device record and the next hipcx_synchronize / hipcx_memcpy_to_host on the device -- the calls that wait for the
+ *       device, and the only way results reach the host (CX/cuda/cuda_device/memory.cc:94-122) -- returns HIPCX_INDEX_ERROR
+ *       with the reference's message and clears the record.  The take call itself never waits and can be captured into a graph.
+ *       (A wait on a stream that the faulty kernel is not ordered before may miss it; the next wait reports it.)
+ *   `error_flag` NULL, mode RAISE: refused with HIPCX_CHAINERX_ERROR.
+ * WRAP and CLIP never report.  No mode ever reads or writes out of bounds: a faulty index is treated as 0 after it was reported.
+ * Nothing is written to `out` by a call that is refused. */
 int hipcx_take(const hipcx_array* a, const hipcx_array* indices, int8_t axis, const hipcx_array* out, int mode, int32_t* error_flag,
                void* stream);
 

@@ -5,6 +5,7 @@
 //   deleter after pool    Device::Allocate results may outlive the pool (CX/cuda/cuda_device/memory.cc:19-24)
 #include <cstdio>
 #include <cstdlib>
+#include <functional>
 #include <set>
 #include <thread>
 #include <vector>
@@ -59,6 +60,14 @@ public:
         s_->live.erase(it);
         ++s_->frees;
     }
+
+    // a fake stream is a pointer to a bool that says whether the stream has caught up
+    std::function<bool()> Fence(void* stream) override {
+        const bool* idle = static_cast<const bool*>(stream);
+        ++fences_;
+        return [idle] { return *idle; };
+    }
+    int fences_ = 0;
 
 private:
     std::shared_ptr<FakeState> s_;
@@ -234,7 +243,91 @@ static void TestThreads() {
     CHECK(fs->outstanding == 0);
 }
 
+// A block used on a stream other than its own: after RecordStream its Free holds it back until that stream has caught up; without
+// the announcement it is handed out again at once (the documented rule: the owner waits before freeing).
+static void TestRecordStream() {
+    auto fs = std::make_shared<FakeState>();
+    MemoryPool pool(std::unique_ptr<Allocator>(new FakeAllocator(fs)));
+    bool stream_b_idle = false, stream_c_idle = false;
+    void* a = pool.Malloc(1000, 1);
+    pool.RecordStream(a, &stream_b_idle);
+    pool.RecordStream(a, &stream_b_idle);  // recorded once
+    pool.RecordStream(a, &stream_c_idle);
+    pool.Free(a);
+    CHECK(pool.pending_blocks() == 1);
+    CHECK(pool.stats().in_use_blocks == 1 && pool.stats().cached_blocks == 0);  // held back: still counted as in use
+    void* b = pool.Malloc(1000, 1);
+    CHECK(b != a);  // a new block: the kernel on the other stream may still read a
+    bool threw = false;
+    try {
+        pool.Free(a);  // freed twice
+    } catch (const std::runtime_error&) {
+        threw = true;
+    }
+    CHECK(threw);
+    threw = false;
+    try {
+        pool.RecordStream(a, &stream_b_idle);  // no longer the caller's
+    } catch (const std::runtime_error&) {
+        threw = true;
+    }
+    CHECK(threw);
+    stream_b_idle = true;
+    void* c = pool.Malloc(1000, 1);
+    CHECK(c != a);  // one of the two streams is still busy
+    stream_c_idle = true;
+    void* d = pool.Malloc(1000, 1);
+    CHECK(d == a && pool.pending_blocks() == 0);
+    CHECK(pool.InUsePointers().size() == 3);
+    pool.Free(b), pool.Free(c), pool.Free(d);
+    // the same sequence without the announcement: immediate reuse
+    void* e = pool.Malloc(5000, 1);
+    pool.Free(e);
+    CHECK(pool.Malloc(5000, 1) == e);
+    // a held-back block is not among the pointers whose frees are still to come, and goes back to the allocator with the pool
+    bool never = false;
+    void* f = pool.Malloc(70000, 2);
+    pool.RecordStream(f, &never);
+    pool.Free(f);
+    for (void* p : pool.InUsePointers()) CHECK(p != f);
+    pool.FreeUnusedBlocks();
+    CHECK(pool.pending_blocks() == 1);
+}
+
+// hipcx_pool_destroy, then a new pool on the device, then the stale frees of the first pool's blocks: swallowed, whatever address
+// the new pool hands out.
+static void TestOrphans() {
+    auto fs = std::make_shared<FakeState>();
+    OrphanSet orphans;
+    void* stale = nullptr;
+    {
+        MemoryPool first(std::unique_ptr<Allocator>(new FakeAllocator(fs)));
+        stale = first.Malloc(3000);
+        void* freed = first.Malloc(3000);
+        first.Free(freed);
+        std::vector<void*> in_use = first.InUsePointers();
+        CHECK(in_use.size() == 1 && in_use[0] == stale);
+        orphans.Add(in_use);
+    }  // the pool takes its memory with it
+    CHECK(fs->outstanding == 0);
+    fs->next = reinterpret_cast<uintptr_t>(stale);  // the driver hands the same address out again
+    MemoryPool second(std::unique_ptr<Allocator>(new FakeAllocator(fs)));
+    void* fresh = second.Malloc(3000);
+    CHECK(fresh == stale);
+    auto free_like_the_entry_point = [&](void* p) {
+        if (orphans.Take(p)) return;
+        second.Free(p);
+    };
+    free_like_the_entry_point(stale);  // the first pool's owner lets go: must not free the second pool's live block
+    CHECK(second.stats().in_use_blocks == 1 && orphans.size() == 0);
+    free_like_the_entry_point(fresh);  // the real free
+    CHECK(second.stats().in_use_blocks == 0 && second.stats().cached_blocks == 1);
+    CHECK(!orphans.Take(fresh));
+}
+
 int main() {
+    TestRecordStream();
+    TestOrphans();
     TestRounding();
     TestReuseAndZero();
     TestRetryThenOutOfMemory();

@@ -239,7 +239,7 @@ def test_batch_norm_kernels_against_the_composition(dt, tol):
               (5, 7, 3, 3)]
     if dt != 'float16':
         # 50176 elements per channel: the float16 composition (like the native backend) overflows its Sum of squares there and
-        # returns inf statistics, while the kernel accumulates in float -- a case where the two differ on purpose
+        # returns inf statistics; test_batch_norm_float16_overflow covers that case
         shapes.append((64, 32, 28, 28))
     for shape in shapes:
         C = shape[1]
@@ -286,3 +286,91 @@ def test_batch_norm_kernels_against_the_composition(dt, tol):
     g1, b1 = np.ones(8, dt), np.zeros(8, dt)
     out, _ = chx.batch_norm(X, chx.array(g1), chx.array(b1), chx.array(b1.copy()), chx.array(g1.copy()))
     assert_close(out.get(), O.batch_norm(x, g1, b1, b1.copy(), g1.copy(), 2e-5, 0.9)[0], tol, 'channels-last input')
+
+
+@pytest.mark.parametrize('case', ['sum of squares', 'sum', 'square', 'finite'])
+def test_batch_norm_float16_overflow(case):
+    """The reference's float16 BatchNorm is a composition of float16 routines (CX/routines/normalization.cc:155-193): its Sum hands
+    out a float16 (inf past 65504), (x - mean)^2 is a float16 array, and everything after an inf follows IEEE rules.  The kernels
+    give the same special values in the same places as the oracle and as the composition run on the device: a variance of inf
+    (inv_std 0, out == beta), a mean of inf (out NaN), one squared deviation of inf in an otherwise small channel, and -- as the
+    control -- the same shape with finite statistics."""
+    import chainer_amd as chx
+    from chainer_amd import routines
+    rng = np.random.default_rng(171)
+    shape = (64, 6, 28, 28)  # 50176 elements per channel
+    x = rng.standard_normal(shape)
+    if case == 'sum of squares':
+        x = x * 2                      # sum (x - mean)^2 is about 2e5
+    elif case == 'sum':
+        x = x * 0.25 + 3               # sum x is about 1.5e5
+    elif case == 'square':
+        x = x * 0.05
+        x[3, 2, 5, 7] = 300.0          # (x - mean)^2 = 9e4 rounds to inf in channel 2 only
+    else:
+        x = x * 0.05 + 0.01
+    x = x.astype(np.float16)
+    C = shape[1]
+    gamma, beta = rng.uniform(0.5, 1.5, C).astype(np.float16), rng.standard_normal(C).astype(np.float16)
+    rm0, rv0 = rng.standard_normal(C).astype(np.float16), rng.uniform(0.5, 1.5, C).astype(np.float16)
+    gout = (rng.standard_normal(shape) * 0.1).astype(np.float16)
+    res = {}
+    for mode in ('kernel', 'composition'):
+        routines.COMPOSE_BATCH_NORM = mode == 'composition'
+        try:
+            RM, RV = chx.array(rm0), chx.array(rv0)
+            out, state = chx.batch_norm(chx.array(x), chx.array(gamma), chx.array(beta), RM, RV, 2e-5, 0.9)
+            gx, gg, gb = chx.batch_norm_grad(chx.array(x), chx.array(gamma), chx.array(gout), state)
+            res[mode] = [out.get(), RM.get(), RV.get(), state[0].get(), state[1].get(), gx.get(), gg.get(), gb.get()]
+        finally:
+            routines.COMPOSE_BATCH_NORM = False
+    o_ref, rm_ref, rv_ref, st_ref = O.batch_norm(x, gamma, beta, rm0.copy(), rv0.copy(), 2e-5, 0.9)
+    gx_ref, gg_ref, gb_ref = O.batch_norm_grad(x, gamma, gout, st_ref)
+    ref = [o_ref, rm_ref, rv_ref, st_ref[0].reshape(C), st_ref[1].reshape(C), gx_ref, gg_ref.reshape(C), gb_ref.reshape(C)]
+    names = ['out', 'running_mean', 'running_var', 'mean', 'inv_std', 'gx', 'ggamma', 'gbeta']
+    # the case is what its name says
+    if case == 'sum of squares':
+        assert np.all(ref[4] == 0) and np.all(np.isinf(rv_ref)) and np.all(np.isfinite(o_ref))
+    elif case == 'sum':
+        assert np.all(np.isinf(ref[3])) and np.all(np.isnan(o_ref))
+    elif case == 'square':
+        assert ref[4][2] == 0 and np.all(ref[4][[0, 1, 3, 4, 5]] > 0)
+    else:
+        assert all(np.all(np.isfinite(r)) for r in ref)
+    for name, k, c, r in zip(names, res['kernel'], res['composition'], ref):
+        k, c = k.reshape(r.shape), c.reshape(r.shape)
+        # assert_close demands the same NaN pattern and the same infinities before it compares the finite values
+        tol = 5e-2 if name in ('gx', 'ggamma', 'gbeta') else 2e-2
+        assert_close(k, r, tol, 'float16 batch_norm (%s) %s: kernel vs oracle' % (case, name))
+        assert_close(k, c, tol, 'float16 batch_norm (%s) %s: kernel vs composition on the device' % (case, name))
+
+
+@pytest.mark.parametrize('dt,tol', [('float16', 2e-2), ('float32', 1e-4)])
+def test_conv_grad_weight_special_values(dt, tol):
+    """inf / NaN in x on the route that reads shifted zero-padded copies of x (filters larger than 1x1 at stride 1): the filter
+    taps that the reference's TensorDot(gy, Im2Col(x)) leaves finite stay finite, the others carry the same inf / NaN
+    (CX/native/native_device/conv.cc:91-124).  Values planted in a corner, on an edge column (where a shifted window wraps around
+    a row end) and in the interior, one channel each; an inf in gy meets the padding's zeros in both implementations."""
+    import chainer_amd as chx
+    rng = np.random.default_rng(190)
+    for (N, C, H, W, K, kh, kw, pd) in [(4, 12, 14, 14, 16, 3, 3, 1), (2, 6, 9, 13, 8, 3, 5, (1, 2)), (3, 8, 12, 12, 8, 2, 2, 0)]:
+        x = rng.standard_normal((N, C, H, W)).astype(dt)
+        gy_shape = O.conv(x.astype('float32'), np.zeros((K, C, kh, kw), 'float32'), None, 1, pd).shape
+        gy = np.abs(rng.standard_normal(gy_shape)).astype(dt) + np.asarray(0.25, dt)  # no zeros, one sign: inf * gy sums to inf, not NaN
+        x[0, 1, 0, 0] = np.inf
+        x[1, 3, 4, W - 1] = -np.inf
+        x[N - 1, 4, H - 1, 0] = np.inf
+        x[1, 5, H // 2, W // 2] = np.nan
+        ref = O.conv_grad_weight((K, C, kh, kw), x, gy, 1, pd)
+        what = '%s %r' % (dt, (N, C, H, W, K, kh, kw, pd))
+        assert np.isfinite(ref[:, [0, 2]]).all() and not np.isfinite(ref[:, 1]).all(), what
+        if kh == 3 and pd != 0:
+            # the corner value is outside some taps' windows: those taps are finite in the reference
+            assert np.isfinite(ref[:, 1]).any() and np.isinf(ref[:, 1]).any(), what
+        got = chx.conv_grad_weight(dt, (K, C, kh, kw), chx.array(x), chx.array(gy), 1, pd).get()
+        assert_close(got, ref, tol, 'conv_grad_weight with inf / NaN in x ' + what)  # same NaN pattern, same infinities, finite values close
+        gy2 = gy.copy()
+        gy2[0, 2, 0, 1] = np.inf
+        x2 = rng.standard_normal((N, C, H, W)).astype(dt)
+        assert_close(chx.conv_grad_weight(dt, (K, C, kh, kw), chx.array(x2), chx.array(gy2), 1, pd).get(),
+                     O.conv_grad_weight((K, C, kh, kw), x2, gy2, 1, pd), tol, 'conv_grad_weight with inf in gy ' + what)

@@ -54,7 +54,8 @@ def test_pooling(dt, tol):
              ((2, 64, 12, 12), (3, 2), (2, 1), (1, 0), True), ((2, 8, 112, 112), 3, 2, 1, False), ((2, 8, 32, 32), 2, 2, 0, False),
              ((1, 4, 16, 24), 3, 2, 1, True), ((1, 4, 16, 16), (2, 3), 2, (0, 1), False)]
     # whole-plane windows (global pooling) over more planes than one workgroup takes, odd and even plane sizes
-    cases += [((3, 200, 7, 7), 7, 1, 0, False), ((2, 301, 5, 5), 5, 1, 0, False), ((2, 130, 6, 6), 6, 1, 0, False), ((1, 257, 3, 5), (3, 5), 1, 0, False)]
+    cases += [((3, 200, 7, 7), 7, 1, 0, False), ((2, 301, 5, 5), 5, 1, 0, False), ((2, 130, 6, 6), 6, 1, 0, False), ((1, 257, 3, 5), (3, 5), 1, 0, False),
+              ((2, 150, 8, 8), 8, 1, 0, False), ((1, 512, 2, 2), 2, 1, 0, False)]  # full workgroups of even planes
     cases += [(xs, k, s, p, cv) for (xs, k, s, p) in POOL_GRID for cv in (False, True)]
     for shape, k, s, p, cv in cases:
         x = rng.standard_normal(shape).astype(dt)
@@ -105,10 +106,21 @@ def test_take(dt):
 def test_take_bounds_and_embedding_shape():
     import chainer_amd as chx
     rng = np.random.default_rng(5)
-    with pytest.raises(IndexError):  # native raises in the default mode (CX/native/native_device/indexing.cc:68-74)
-        chx.take(chx.zeros((4, 3), 'float32'), chx.array(np.array([5], 'int64')), 0)
+    # native raises in the default mode (CX/native/native_device/indexing.cc:68-74); here the call itself returns (no wait for the
+    # device) and the error surfaces at the first point where the result could be read
+    bad = chx.take(chx.zeros((4, 3), 'float32'), chx.array(np.array([5], 'int64')), 0)
+    with pytest.raises(IndexError, match='Index 5 is out of bounds for axis 0 with size 4'):
+        bad.get()
+    assert bad.get().shape == (1, 3)  # reported once: the record is cleared
+    bad = chx.take(chx.zeros((4, 3), 'float32'), chx.array(np.array([[0, -5]], 'int32')), 0)
+    good = chx.take(chx.ones((4, 3), 'float32'), chx.array(np.array([1], 'int64')), 0)  # later, valid work does not clear it
     with pytest.raises(IndexError):
+        chx.synchronize()
+    chx.synchronize()
+    assert_exact(good.get(), np.ones((1, 3), 'float32'), 'a valid take after a bad one')
+    with pytest.raises(IndexError):  # 'raise' checks inside the call
         chx.take(chx.zeros((4, 3), 'float32'), chx.array(np.array([-5], 'int64')), 0, 'raise')
+    chx.synchronize()  # ... and leaves nothing behind
     with pytest.raises(chx.DtypeError):
         chx.take(chx.zeros((4, 3), 'float32'), chx.zeros((2,), 'float32'), 0)
     ids = rng.integers(0, 10000, (128, 35)).astype('int32')
@@ -117,7 +129,7 @@ def test_take_bounds_and_embedding_shape():
     assert_exact(chx.take(Wd, Id[:, 3], 0).get(), W[ids[:, 3]], 'embedding rows, strided ids')
     assert_exact(chx.take(Wd, Id, 0).get(), W[ids], 'embedding rows, the whole [128,35] batch')
     with pytest.raises(IndexError):
-        chx.take(Wd, chx.array(np.array([3, 10000], 'int64')), 0)
+        chx.take(Wd, chx.array(np.array([3, 10000], 'int64')), 0).get()
     # long rows in 4-byte pieces (68 bytes) and in 16-byte pieces (2048 bytes), negative and wrapped indices
     for shape, dt in (((300, 17), 'float32'), ((90, 1024), 'float16'), ((40, 33), 'int32')):
         a = (rng.standard_normal(shape) * 100).astype(dt)

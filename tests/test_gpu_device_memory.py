@@ -133,3 +133,71 @@ def test_graph_capture_in_an_arena_survives_other_allocations():
         assert np.array_equal(g.result.get(), eager), 'replay %d' % i
         del junk
     g.release()
+
+
+def test_record_stream_holds_a_freed_block_back():
+    """A block allocated for one stream and used on another: after hipcx_record_stream its free waits for that stream, so the next
+    allocation of its size class gets other memory while the foreign stream is busy and the block itself once it has caught up.
+    Recording the block's own stream changes nothing."""
+    import torch
+    L = _lib()
+    import chainer_amd as chx
+    chx.synchronize()
+    nbytes = 3 << 20
+    p = ctypes.c_void_p()
+    L.call('hipcx_malloc', 0, nbytes, ctypes.byref(p))  # the null stream's partition
+    first = p.value
+    L.call('hipcx_record_stream', 0, ctypes.c_void_p(first), ctypes.c_void_p(None))  # its own stream: immediate reuse
+    L.call('hipcx_free', 0, ctypes.c_void_p(first))
+    L.call('hipcx_malloc', 0, nbytes, ctypes.byref(p))
+    assert p.value == first
+    side = torch.cuda.Stream()
+    a = torch.randn(8192, 8192, device='cuda')
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        for _ in range(24):  # a few hundred milliseconds of work queued on the side stream
+            a = torch.mm(a, a) * 1e-4
+    L.call('hipcx_record_stream', 0, ctypes.c_void_p(first), ctypes.c_void_p(side.cuda_stream))
+    L.call('hipcx_free', 0, ctypes.c_void_p(first))
+    busy = not side.query()
+    L.call('hipcx_malloc', 0, nbytes, ctypes.byref(p))
+    second = p.value
+    if busy:
+        assert second != first, 'the block was handed out again while the side stream could still use it'
+    side.synchronize()
+    L.call('hipcx_free', 0, ctypes.c_void_p(second))
+    got = []
+    for _ in range(2):  # both blocks of the class are free now
+        L.call('hipcx_malloc', 0, nbytes, ctypes.byref(p))
+        got.append(p.value)
+    assert first in got
+    for g in got:
+        L.call('hipcx_free', 0, ctypes.c_void_p(g))
+    with pytest.raises(chx.ChainerxError, match='not a block in use'):
+        L.call('hipcx_record_stream', 0, ctypes.c_void_p(first), ctypes.c_void_p(side.cuda_stream))
+    assert busy, 'the side stream finished before the free: the test did not exercise the hold-back'
+
+
+def test_take_default_mode_is_captured_and_still_raises():
+    """Take in the default bounds mode (mode=None, what the reference's callers pass) neither waits for the device nor reads a flag
+    back, so a captured graph can hold it; an id that is out of range at replay time raises IndexError when the result is read."""
+    import torch
+    import chainer_amd as chx
+    from chainer_amd.graph import capture
+    rng = np.random.default_rng(9)
+    table = rng.standard_normal((100, 64)).astype(np.float32)
+    ids = rng.integers(0, 100, (32,)).astype(np.int32)
+    T, I = chx.array(table), chx.array(ids)
+    g = capture(lambda: chx.take(T, I, 0) * 2.0)
+    g.replay()
+    torch.cuda.synchronize()
+    assert np.array_equal(g.result.get(), table[ids] * 2.0)
+    I[5:6].fill(100)  # one past the end, written on the device
+    g.replay()
+    with pytest.raises(IndexError, match='Index 100 is out of bounds for axis 0 with size 100'):
+        g.result.get()
+    I[5:6].fill(-100)  # the lowest valid index
+    g.replay()
+    ids[5] = 0
+    assert np.array_equal(g.result.get(), table[ids] * 2.0)
+    g.release()

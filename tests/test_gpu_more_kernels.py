@@ -341,8 +341,10 @@ def test_add_at(dt):
     b = rand(rng, (5, 4, 7), dt)
     got = chx.add_at(chx.array(a)[:, ::-1], chx.array(idx), 1, chx.array(b)[::-1]).get()
     assert_exact(got, O.add_at(a[:, ::-1], idx, 1, b[::-1]), 'add_at views')
+    with pytest.raises(chx.ChainerxIndexError):  # default mode: raised where the result would be read
+        chx.add_at(chx.array(a), chx.array(np.array([6])), 1, chx.array(rand(rng, (5, 1, 7), dt))).get()
     with pytest.raises(chx.ChainerxIndexError):
-        chx.add_at(chx.array(a), chx.array(np.array([6])), 1, chx.array(rand(rng, (5, 1, 7), dt)))
+        chx.add_at(chx.array(a), chx.array(np.array([6])), 1, chx.array(rand(rng, (5, 1, 7), dt)), 'raise')
     # the embedding gradient: many rows scattered into a table
     if dt == 'float32':
         table = np.zeros((50, 16), dt)

@@ -131,6 +131,29 @@ def test_n_step_lstm_kernel_entry_matches_oracle(n_layers):
         np.testing.assert_array_equal(CX.get(), cx)
 
 
+def test_n_step_lstm_kernel_entry_special_values():
+    """An inf in the initial hidden state or in an input row reaches the gates as +-inf (saturated sigmoids, tanh +-1), as in the
+    routine composition -- the kernel's zero-weight blocks past the end of a row's reduction form no 0 * inf products.  Sizes whose
+    reduction ends inside a chunk, so that such blocks exist."""
+    import chainer_amd as chx
+    rng = np.random.default_rng(77)
+    for in_size, units, lengths in [(17, 33, (4, 4, 2)), (40, 70, (3,) * 20)]:
+        ws, bs, seqs, xs, hx, cx = _rnn_problem(rng, 'lstm', 1, False, in_size, units, lengths)
+        ws = [[np.abs(m) + np.float32(0.01) for m in layer] for layer in ws]  # one sign: inf * w sums to inf, never inf - inf
+        hx[0, 0, :3] = np.inf
+        hx[0, 1, 0] = -np.inf
+        xs[0][2, 1] = np.inf
+        W, B, X, HX, CX = _upload(chx, ws, bs, xs, hx, cx)
+        ref = O.n_step_lstm(1, hx, cx, ws, bs, xs)
+        got = chx.n_step_lstm(1, HX, CX, W, B, X, kernel=True)
+        what = 'in=%d units=%d' % (in_size, units)
+        assert np.isfinite(ref[0]).all() and np.isfinite(ref[2][0]).all(), what  # saturated gates, finite states
+        assert_close(got[0].get(), ref[0], what='hy ' + what)
+        assert_close(got[1].get(), ref[1], what='cy ' + what)
+        for t, (y, r) in enumerate(zip(got[2], ref[2])):
+            assert_close(y.get(), r, what='ys[%d] %s' % (t, what))
+
+
 def test_n_step_lstm_kernel_entry_views_and_errors():
     import ctypes
     import chainer_amd as chx

@@ -53,3 +53,27 @@ def test_static_scratch_sum_refuses_reductions_beyond_its_size():
         pytest.skip('this launch plan fits the static scratch (%d bytes)' % need)
     with pytest.raises(chx.ChainerxError, match='static scratch'):
         _lib.call('hipcx_sum_static_scratch', X.desc(), ax, 1, out.desc(), current_stream())
+
+
+def test_static_scratch_sum_calls_on_two_streams_take_turns():
+    """Calls from different streams share the one static array of the device: each waits for the previous call's kernels, so
+    interleaved calls on two streams give the results of hipcx_sum."""
+    import torch
+    import chainer_amd as chx
+    from chainer_amd import _lib
+    rng = np.random.default_rng(78)
+    xs = [rng.standard_normal((64, 262144)).astype('float32'), rng.standard_normal((48, 200000)).astype('float32')]
+    X = [chx.array(x) for x in xs]
+    refs = [chx.sum(a, axis=1).get() for a in X]
+    outs = [chx.ndarray.empty((a.shape[0],), 'float32') for a in X]
+    for o in outs:
+        o.fill(0)
+    chx.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    ax = (ctypes.c_int8 * 1)(1)
+    for rep in range(6):
+        for i in (0, 1):
+            _lib.call('hipcx_sum_static_scratch', X[i].desc(), ax, 1, outs[i].desc(), ctypes.c_void_p(streams[i].cuda_stream))
+    torch.cuda.synchronize()
+    for i in (0, 1):
+        assert_exact(outs[i].get(), refs[i], 'sum_static_scratch on stream %d' % i)
