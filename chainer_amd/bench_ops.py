@@ -291,8 +291,10 @@ def section_backward(chx, oracle, with_cpu):
     shape = (32, 256, 56, 56)
     xb = chx.array(rng.standard_normal(shape).astype(np.float16))
     gb = chx.array(rng.standard_normal(shape).astype(np.float16))
-    prm = [chx.array(rng.uniform(0.5, 1.5, 256).astype(np.float16)) for _ in range(2)]
-    rm, rv = chx.array(np.zeros(256, np.float16)), chx.array(np.ones(256, np.float16))
+    # float16 activations with float32 parameters and statistics (the mixed-precision call: the reference then computes in float32;
+    # with float16 parameters its float16 sums over 100352 elements per channel overflow to inf, and so do this library's)
+    prm = [chx.array(rng.uniform(0.5, 1.5, 256).astype(np.float32)) for _ in range(2)]
+    rm, rv = chx.array(np.zeros(256, np.float32)), chx.array(np.ones(256, np.float32))
     nbytes = xb.nbytes
     out_state = []
     out_state[:] = [chx.batch_norm(xb, prm[0], prm[1], rm, rv)]
@@ -315,12 +317,12 @@ def section_backward(chx, oracle, with_cpu):
 
 
 def section_train(chx, oracle, with_cpu):
-    """ResNet-50 training step (forward with batch statistics, hand-written backward, SGD) in float16 -- the kernel sequence of the
-    reference's ImageNet example without its autograd bookkeeping.  Not the headline metric: it shows the backward set end to end."""
+    """ResNet-50 training step (forward with batch statistics, hand-written backward, SGD) with float16 filters and activations and
+    float32 batch normalisation parameters -- the kernel sequence of the reference's ImageNet example without its autograd bookkeeping.  Not the headline metric: it shows the backward set end to end."""
     import copy
     from chainer_amd import configs as cfg
     F = cfg.DeviceTrainOps(chx)
-    p0 = cfg.resnet50_params()
+    p0 = cfg.resnet50_params_mixed()
     for batch in (32, 128):
         x = chx.array(cfg.resnet50_input(batch=batch))
         t = chx.array(np.random.default_rng(8).integers(0, 1000, batch).astype(np.int32))
@@ -329,7 +331,7 @@ def section_train(chx, oracle, with_cpu):
         eager = device_time(step, 2, 1, 1)
         graph = graph_time(step, 3)
         flops = 3.0 * cfg.resnet50_flops(batch)
-        emit(section='train', op='ResNet-50 training step, float16', batch=batch, eager_ms=round(eager * 1e3, 2),
+        emit(section='train', op='ResNet-50 training step, float16 (batch norm parameters float32)', batch=batch, eager_ms=round(eager * 1e3, 2),
              graph_replay_ms=round(graph * 1e3, 2), img_per_s_graph=round(batch / graph, 1), TFLOPs_graph=round(flops / graph / 1e12, 1),
              note='3x the forward flops (forward, data gradient, weight gradient); eager time includes ~1500 Python-issued kernel calls')
         del pd

@@ -153,6 +153,23 @@ def resnet50_params(seed=4, dtype=np.float16, n_out=1000, residual_gamma_scale=R
     return p
 
 
+def resnet50_params_mixed(**kwargs):
+    """resnet50_params with the batch normalisation parameters and running statistics in float32: how a float16 network is trained
+    (Chainer's mixed16 keeps them in float32, chainer/links/normalization/batch_normalization.py:213-268).  BatchNorm then computes
+    in float32 (ResultType(x, gamma, beta), CX/routines/normalization.cc:176-180); an all-float16 call sums its statistics into
+    float16 arrays, which overflow beyond a few thousand elements per channel."""
+    p = resnet50_params(**kwargs)
+
+    def widen(tree):
+        for k, v in (tree.items() if isinstance(tree, dict) else enumerate(tree)):
+            if isinstance(v, dict) and 'gamma' in v:
+                tree[k] = {name: a.astype(np.float32) for name, a in v.items()}
+            elif isinstance(v, (dict, list)):
+                widen(v)
+    widen(p)
+    return p
+
+
 def resnet50_input(seed=4, batch=128, dtype=np.float16, size=224):
     return _rng(seed + 1000).standard_normal((batch, 3, size, size)).astype(np.float32).astype(dtype)
 

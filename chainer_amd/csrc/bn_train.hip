@@ -41,10 +41,10 @@ __device__ __forceinline__ C BlockSum(C v, C* lds) {
 // (x - mean)^2 past 65504 is inf, 1 / count is a float16 subnormal, and so on.  Rnd applies that rounding wherever the composition
 // has an array in between; arithmetic between two roundings runs in float as the reference's Float16 operators do.  For float32
 // and float64 it is the identity.
-template <typename T>
-__device__ __forceinline__ compute_t<T> Rnd(compute_t<T> v) {
-    if constexpr (sizeof(T) == 2) {
-        return static_cast<compute_t<T>>(static_cast<T>(v));
+template <typename P, typename C>
+__device__ __forceinline__ C Rnd(C v) {
+    if constexpr (sizeof(P) == 2) {
+        return static_cast<C>(static_cast<P>(v));
     } else {
         return v;
     }
@@ -52,10 +52,10 @@ __device__ __forceinline__ compute_t<T> Rnd(compute_t<T> v) {
 
 // The per-channel state (mean, 1 / std): compute-type vectors in the workspace (forward), or the caller's arrays in the array dtype
 // with an element stride (gradient: the state BatchNorm handed out) -- read in place, so the gradient needs no widening copies.
-template <typename T>
+template <typename T, typename P>
 __device__ __forceinline__ compute_t<T> LoadState(const void* ptr, int c, int in_array_dtype, int64_t stride) {
     using C = compute_t<T>;
-    return in_array_dtype ? static_cast<C>(static_cast<const T*>(ptr)[c * stride]) : static_cast<const C*>(ptr)[c];
+    return in_array_dtype ? static_cast<C>(static_cast<const P*>(ptr)[c * stride]) : static_cast<const C*>(ptr)[c];
 }
 
 struct BnStatArgs {
@@ -72,7 +72,7 @@ struct BnStatArgs {
 };
 
 // MODE 0: sum x.  MODE 1: sum (x - mean)^2.  MODE 2: sum g and sum g * (x - mean) * inv_std.
-template <typename T, int MODE, int VEC>
+template <typename T, typename P, int MODE, int VEC>
 __global__ __launch_bounds__(kBnTrainThreads) void BnStatKernel(BnStatArgs p) {
     using C = compute_t<T>;
     __shared__ C lds[kBnTrainThreads / 64];
@@ -80,8 +80,8 @@ __global__ __launch_bounds__(kBnTrainThreads) void BnStatKernel(BnStatArgs p) {
     const T* x = static_cast<const T*>(p.x);
     const T* g = static_cast<const T*>(p.g);
     C m = C(0), is = C(1);
-    if (MODE >= 1) m = LoadState<T>(p.mean, c, p.state_in_array_dtype, p.mean_stride);
-    if (MODE == 2) is = LoadState<T>(p.inv_std, c, p.state_in_array_dtype, p.inv_stride);
+    if (MODE >= 1) m = LoadState<T, P>(p.mean, c, p.state_in_array_dtype, p.mean_stride);
+    if (MODE == 2) is = LoadState<T, P>(p.inv_std, c, p.state_in_array_dtype, p.inv_stride);
     C a0 = C(0), a1 = C(0);
     // The slice's images n = s, s + S, ... times the plane's vectors form one index space shared out over the threads, so that
     // planes shorter than the workgroup (14x14, 7x7) keep every lane busy.  32-bit index arithmetic: the host checks N * L < 2^31.
@@ -100,12 +100,12 @@ __global__ __launch_bounds__(kBnTrainThreads) void BnStatKernel(BnStatArgs p) {
             if (MODE == 0) {
                 a0 += xe;
             } else if (MODE == 1) {
-                C d = Rnd<T>(xe - m);
-                a0 += Rnd<T>(d * d);
+                C d = Rnd<P>(xe - m);
+                a0 += Rnd<P>(d * d);
             } else {
                 C ge = static_cast<C>(gv.v[e]);
                 a0 += ge;
-                a1 += Rnd<T>(ge * Rnd<T>(Rnd<T>(xe - m) * is));
+                a1 += Rnd<P>(ge * Rnd<P>(Rnd<P>(xe - m) * is));
             }
         }
     }
@@ -133,7 +133,7 @@ struct BnFinishArgs {
 };
 
 // STEP 0: mean from the sums.  STEP 1: variance -> inv_std, state outputs, running statistics (CX/routines/normalization.cc:176-191).
-template <typename T, int STEP>
+template <typename T, typename P, int STEP>
 __global__ __launch_bounds__(256) void BnFinishKernel(BnFinishArgs p) {
     using C = compute_t<T>;
     const int c = blockIdx.x * blockDim.x + threadIdx.x;
@@ -144,29 +144,29 @@ __global__ __launch_bounds__(256) void BnFinishKernel(BnFinishArgs p) {
     const C n = static_cast<C>(p.count);
     // Mean = Sum (handed out in the array dtype) / count (CX/routines/statistics.cc:113-123)
     if (STEP == 0) {
-        static_cast<C*>(p.mean)[c] = Rnd<T>(Rnd<T>(sum) / n);
+        static_cast<C*>(p.mean)[c] = Rnd<P>(Rnd<P>(sum) / n);
         return;
     }
     const C mean = static_cast<const C*>(p.mean)[c];
-    const C var = Rnd<T>(Rnd<T>(sum) / n);
+    const C var = Rnd<P>(Rnd<P>(sum) / n);
     // Reciprocal(Sqrt(var + eps)) with eps as a scalar of the array dtype (CX/routines/normalization.cc:141)
     C inv_std;
     if constexpr (std::is_same<C, float>::value) {
-        inv_std = Rnd<T>(1.0f / Rnd<T>(sqrtf(Rnd<T>(var + Rnd<T>(static_cast<float>(p.eps))))));
+        inv_std = Rnd<P>(1.0f / Rnd<P>(sqrtf(Rnd<P>(var + Rnd<P>(static_cast<float>(p.eps))))));
     } else {
         inv_std = 1.0 / sqrt(var + p.eps);
     }
     static_cast<C*>(p.inv_std)[c] = inv_std;
-    static_cast<T*>(p.mean_out)[c * p.mo_stride] = static_cast<T>(mean);
-    static_cast<T*>(p.inv_std_out)[c * p.io_stride] = static_cast<T>(inv_std);
+    static_cast<P*>(p.mean_out)[c * p.mo_stride] = static_cast<P>(mean);
+    static_cast<P*>(p.inv_std_out)[c * p.io_stride] = static_cast<P>(inv_std);
     // running *= decay; running += (inv_decay [* count / (count - 1)]) * statistic, scalars in the array dtype (CX/routines/normalization.cc:185-190)
-    const C decay = Rnd<T>(static_cast<C>(p.decay));
-    const C inv_decay = Rnd<T>(static_cast<C>(1.0 - p.decay));
-    const C inv_decay_adjusted = Rnd<T>(static_cast<C>((1.0 - p.decay) * (p.count / (p.count - 1.0 > 1.0 ? p.count - 1.0 : 1.0))));
-    T* rm = static_cast<T*>(p.running_mean) + c * p.rm_stride;
-    T* rv = static_cast<T*>(p.running_var) + c * p.rv_stride;
-    *rm = static_cast<T>(Rnd<T>(static_cast<C>(*rm) * decay) + Rnd<T>(inv_decay * mean));
-    *rv = static_cast<T>(Rnd<T>(static_cast<C>(*rv) * decay) + Rnd<T>(inv_decay_adjusted * var));
+    const C decay = Rnd<P>(static_cast<C>(p.decay));
+    const C inv_decay = Rnd<P>(static_cast<C>(1.0 - p.decay));
+    const C inv_decay_adjusted = Rnd<P>(static_cast<C>((1.0 - p.decay) * (p.count / (p.count - 1.0 > 1.0 ? p.count - 1.0 : 1.0))));
+    P* rm = static_cast<P*>(p.running_mean) + c * p.rm_stride;
+    P* rv = static_cast<P*>(p.running_var) + c * p.rv_stride;
+    *rm = static_cast<P>(Rnd<P>(static_cast<C>(*rm) * decay) + Rnd<P>(inv_decay * mean));
+    *rv = static_cast<P>(Rnd<P>(static_cast<C>(*rv) * decay) + Rnd<P>(inv_decay_adjusted * var));
 }
 
 struct BnApplyArgs {
@@ -189,7 +189,7 @@ struct BnApplyArgs {
 };
 
 // Gradient finish: ggamma = sum g * x_hat, gbeta = sum g, one thread per channel; leaves both as compute-type values at partial[c][0].
-template <typename T>
+template <typename T, typename P>
 __global__ __launch_bounds__(256) void BnGradFinishKernel(BnApplyArgs p) {
     using C = compute_t<T>;
     const int c = blockIdx.x * blockDim.x + threadIdx.x;
@@ -200,22 +200,22 @@ __global__ __launch_bounds__(256) void BnGradFinishKernel(BnApplyArgs p) {
         sg += part[s * 2];
         sgx += part[s * 2 + 1];
     }
-    part[0] = Rnd<T>(sg);  // what the gradient pass reads back is the array-dtype sum, as in the reference
-    part[1] = Rnd<T>(sgx);
-    static_cast<T*>(p.gbeta)[c * p.gb_stride] = static_cast<T>(sg);
-    static_cast<T*>(p.ggamma)[c * p.gg_stride] = static_cast<T>(sgx);
+    part[0] = Rnd<P>(sg);  // what the gradient pass reads back is the array-dtype sum, as in the reference
+    part[1] = Rnd<P>(sgx);
+    static_cast<P*>(p.gbeta)[c * p.gb_stride] = static_cast<P>(sg);
+    static_cast<P*>(p.ggamma)[c * p.gg_stride] = static_cast<P>(sgx);
 }
 
 // GRAD false: out = ((x - mean) * inv_std) * gamma + beta.
 // GRAD true:  gx = (gamma * inv_std) * (g - (x_hat * ggamma + gbeta) / count)   (CX/routines/normalization.cc:232-246).
-template <typename T, bool GRAD, int VEC>
+template <typename T, typename P, bool GRAD, int VEC>
 __global__ __launch_bounds__(256) void BnApplyKernel(BnApplyArgs p) {
     using C = compute_t<T>;
     const T* x = static_cast<const T*>(p.x);
     const T* g = static_cast<const T*>(p.g);
     T* out = static_cast<T*>(p.out);
     const int64_t nvec = p.total / VEC;
-    const C inv_n = Rnd<T>(static_cast<C>(1.0 / p.count));  // a scalar of the array dtype
+    const C inv_n = Rnd<P>(static_cast<C>(1.0 / p.count));  // a scalar of the array dtype
     // The array is one contiguous run of [N][C] planes of L elements, cut into vectors without regard to the planes: when VEC does
     // not divide L a vector can hold the end of one plane and the start of the next (never more: the host keeps VEC <= L), and
     // its elements pick the constants of their own channel.  32-bit index arithmetic: the host checks total < 2^31.
@@ -229,14 +229,14 @@ __global__ __launch_bounds__(256) void BnApplyKernel(BnApplyArgs p) {
         const int c2 = c + 1 == p.C ? 0 : c + 1;
         const bool split = planes_split && within + VEC > L;
         const int split_at = split ? static_cast<int>(L - within) : VEC;  // elements from split_at on belong to channel c2
-        const C m = LoadState<T>(p.mean, c, p.state_in_array_dtype, p.mean_stride);
-        const C is = LoadState<T>(p.inv_std, c, p.state_in_array_dtype, p.inv_stride);
-        const C ga = static_cast<C>(static_cast<const T*>(p.gamma)[c * p.gamma_stride]);
+        const C m = LoadState<T, P>(p.mean, c, p.state_in_array_dtype, p.mean_stride);
+        const C is = LoadState<T, P>(p.inv_std, c, p.state_in_array_dtype, p.inv_stride);
+        const C ga = static_cast<C>(static_cast<const P*>(p.gamma)[c * p.gamma_stride]);
         C m2 = m, is2 = is, ga2 = ga;
         if (split) {
-            m2 = LoadState<T>(p.mean, c2, p.state_in_array_dtype, p.mean_stride);
-            is2 = LoadState<T>(p.inv_std, c2, p.state_in_array_dtype, p.inv_stride);
-            ga2 = static_cast<C>(static_cast<const T*>(p.gamma)[c2 * p.gamma_stride]);
+            m2 = LoadState<T, P>(p.mean, c2, p.state_in_array_dtype, p.mean_stride);
+            is2 = LoadState<T, P>(p.inv_std, c2, p.state_in_array_dtype, p.inv_stride);
+            ga2 = static_cast<C>(static_cast<const P*>(p.gamma)[c2 * p.gamma_stride]);
         }
         Vec<T, VEC> xv = *reinterpret_cast<const Vec<T, VEC>*>(x + v * VEC);
         Vec<T, VEC> o;
@@ -249,22 +249,22 @@ __global__ __launch_bounds__(256) void BnApplyKernel(BnApplyArgs p) {
                 gbeta2 = part2[0], ggamma2 = part2[1];
             }
             Vec<T, VEC> gv = *reinterpret_cast<const Vec<T, VEC>*>(g + v * VEC);
-            const C scale = Rnd<T>(ga * is), scale2 = Rnd<T>(ga2 * is2);
+            const C scale = Rnd<P>(ga * is), scale2 = Rnd<P>(ga2 * is2);
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
                 const bool second = e >= split_at;
-                C x_hat = Rnd<T>(Rnd<T>(static_cast<C>(xv.v[e]) - (second ? m2 : m)) * (second ? is2 : is));
-                C t = Rnd<T>(Rnd<T>(Rnd<T>(x_hat * (second ? ggamma2 : ggamma)) + (second ? gbeta2 : gbeta)) * inv_n);
-                o.v[e] = static_cast<T>((second ? scale2 : scale) * Rnd<T>(static_cast<C>(gv.v[e]) - t));
+                C x_hat = Rnd<P>(Rnd<P>(static_cast<C>(xv.v[e]) - (second ? m2 : m)) * (second ? is2 : is));
+                C t = Rnd<P>(Rnd<P>(Rnd<P>(x_hat * (second ? ggamma2 : ggamma)) + (second ? gbeta2 : gbeta)) * inv_n);
+                o.v[e] = static_cast<T>((second ? scale2 : scale) * Rnd<P>(static_cast<C>(gv.v[e]) - t));
             }
         } else {
-            const C be = static_cast<C>(static_cast<const T*>(p.beta)[c * p.beta_stride]);
-            const C be2 = split ? static_cast<C>(static_cast<const T*>(p.beta)[c2 * p.beta_stride]) : be;
+            const C be = static_cast<C>(static_cast<const P*>(p.beta)[c * p.beta_stride]);
+            const C be2 = split ? static_cast<C>(static_cast<const P*>(p.beta)[c2 * p.beta_stride]) : be;
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
                 const bool second = e >= split_at;
-                C t = Rnd<T>(Rnd<T>(static_cast<C>(xv.v[e]) - (second ? m2 : m)) * (second ? is2 : is));
-                o.v[e] = static_cast<T>(Rnd<T>(t * (second ? ga2 : ga)) + (second ? be2 : be));
+                C t = Rnd<P>(Rnd<P>(static_cast<C>(xv.v[e]) - (second ? m2 : m)) * (second ? is2 : is));
+                o.v[e] = static_cast<T>(Rnd<P>(t * (second ? ga2 : ga)) + (second ? be2 : be));
             }
         }
         *reinterpret_cast<Vec<T, VEC>*>(out + v * VEC) = o;
@@ -308,9 +308,11 @@ size_t TrainWorkspace(const BnTrainGeom& g) {
 }
 
 // A per-channel vector: shape [C] or the keep-dims shape of x; returns its element stride along the channel axis.
-int64_t ChannelStride(const hipcx_array* a, const hipcx_array* x, const char* name) {
+// `param_dtype`: the dtype the per-channel arrays of the call share (see ParamDtype).
+int64_t ChannelStride(const hipcx_array* a, const hipcx_array* x, const char* name, int param_dtype) {
     ValidateArray(a, name);
-    HIPCX_REQUIRE(a->dtype == x->dtype, HIPCX_NOT_IMPLEMENTED_ERROR, std::string(name) + ": must have x's dtype on the hip backend");
+    HIPCX_REQUIRE(a->dtype == param_dtype, HIPCX_NOT_IMPLEMENTED_ERROR,
+                  std::string(name) + ": the per-channel arrays must share one dtype, x's or (for float16 x) float32, on the hip backend");
     const int64_t it = ItemSize(a->dtype);
     if (a->ndim == 1) {
         HIPCX_REQUIRE(a->shape[0] == x->shape[1], HIPCX_DIMENSION_ERROR, std::string(name) + " must have one value per channel");
@@ -321,6 +323,27 @@ int64_t ChannelStride(const hipcx_array* a, const hipcx_array* x, const char* na
         HIPCX_REQUIRE(a->shape[d] == (d == 1 ? x->shape[1] : 1), HIPCX_DIMENSION_ERROR, std::string(name) + " must have the keep-dims reduced shape of x");
     }
     return a->strides[1] / it;
+}
+
+// The dtype of the per-channel arrays, taken from `first` (gamma): x's dtype, or float32 with a float16 x -- the mixed-precision
+// call of a float16 network whose normalisation parameters stay in float32.  The reference computes in ResultType(x, gamma, beta)
+// (CX/routines/normalization.cc:176-180): float32 then, with one rounding of the output to float16 and none of the float16
+// overflow of an all-float16 call.
+int ParamDtype(const hipcx_array* x, const hipcx_array* first) {
+    ValidateArray(first, "gamma");
+    HIPCX_REQUIRE(first->dtype == x->dtype || (x->dtype == HIPCX_FLOAT16 && first->dtype == HIPCX_FLOAT32), HIPCX_NOT_IMPLEMENTED_ERROR,
+                  "hip batch_norm: the per-channel arrays must have x's dtype, or float32 for a float16 x");
+    return first->dtype;
+}
+
+// Calls f with (tag of x's type, tag of the per-channel arrays' type).
+template <typename F>
+void VisitBnDtypes(int x_dtype, int param_dtype, F&& f) {
+    if (x_dtype == HIPCX_FLOAT16 && param_dtype == HIPCX_FLOAT32) {
+        f(Tag<half_t>{}, Tag<float>{});
+        return;
+    }
+    VisitFloatDtype(x_dtype, [&](auto tag) { f(tag, tag); });
 }
 
 // Widths of the two kernel families.  The statistics kernels read whole planes of one channel, so their vectors must divide the
@@ -346,21 +369,21 @@ BnWidths PickWidths(int64_t L, int64_t total, int64_t item, std::initializer_lis
     return w;
 }
 
-template <typename T, int MODE>
+template <typename T, typename P, int MODE>
 void LaunchStat(const BnStatArgs& a, int width, hipStream_t stream) {
     constexpr int VEC = 16 / sizeof(T);
     dim3 grid(static_cast<unsigned>(a.C), static_cast<unsigned>(a.S));
     if (width == VEC) {
-        hipLaunchKernelGGL((BnStatKernel<T, MODE, VEC>), grid, dim3(kBnTrainThreads), 0, stream, a);
+        hipLaunchKernelGGL((BnStatKernel<T, P, MODE, VEC>), grid, dim3(kBnTrainThreads), 0, stream, a);
     } else if (VEC >= 4 && width == VEC / 2) {
-        hipLaunchKernelGGL((BnStatKernel<T, MODE, (VEC >= 4 ? VEC / 2 : 1)>), grid, dim3(kBnTrainThreads), 0, stream, a);
+        hipLaunchKernelGGL((BnStatKernel<T, P, MODE, (VEC >= 4 ? VEC / 2 : 1)>), grid, dim3(kBnTrainThreads), 0, stream, a);
     } else {
-        hipLaunchKernelGGL((BnStatKernel<T, MODE, 1>), grid, dim3(kBnTrainThreads), 0, stream, a);
+        hipLaunchKernelGGL((BnStatKernel<T, P, MODE, 1>), grid, dim3(kBnTrainThreads), 0, stream, a);
     }
     CheckLaunch("batch_norm statistics");
 }
 
-template <typename T, bool GRAD>
+template <typename T, typename P, bool GRAD>
 void LaunchApply(const BnApplyArgs& a, bool vec, hipStream_t stream) {
     constexpr int VEC = 16 / sizeof(T);
     int64_t nvec = a.total / (vec ? VEC : 1);
@@ -369,9 +392,9 @@ void LaunchApply(const BnApplyArgs& a, bool vec, hipStream_t stream) {
     if (blocks > cap) blocks = cap;
     if (blocks < 1) blocks = 1;
     if (vec) {
-        hipLaunchKernelGGL((BnApplyKernel<T, GRAD, VEC>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, a);
+        hipLaunchKernelGGL((BnApplyKernel<T, P, GRAD, VEC>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, a);
     } else {
-        hipLaunchKernelGGL((BnApplyKernel<T, GRAD, 1>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, a);
+        hipLaunchKernelGGL((BnApplyKernel<T, P, GRAD, 1>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, a);
     }
     CheckLaunch("batch_norm apply");
 }
@@ -397,7 +420,7 @@ int hipcx_batch_norm_supported(const hipcx_array* x, const int8_t* axis, int nax
         if (total == 0 || total >= (int64_t{1} << 31)) return 0;
         for (int i = 0; i < nparams; ++i) {
             if (params[i] == nullptr) return 0;
-            (void)ChannelStride(params[i], x, "parameter");
+            (void)ChannelStride(params[i], x, "parameter", ParamDtype(x, params[0]));
         }
         return 1;
     } catch (...) {
@@ -425,12 +448,13 @@ int hipcx_batch_norm(const hipcx_array* x, const hipcx_array* gamma, const hipcx
                       "hip batch_norm: out must be C-contiguous with x's shape and dtype");
         BnFinishArgs f{};
         BnApplyArgs a{};
-        a.gamma_stride = ChannelStride(gamma, x, "gamma");
-        a.beta_stride = ChannelStride(beta, x, "beta");
-        f.rm_stride = ChannelStride(running_mean, x, "running_mean");
-        f.rv_stride = ChannelStride(running_var, x, "running_var");
-        f.mo_stride = ChannelStride(mean_out, x, "mean_out");
-        f.io_stride = ChannelStride(inv_std_out, x, "inv_std_out");
+        const int pd = ParamDtype(x, gamma);
+        a.gamma_stride = ChannelStride(gamma, x, "gamma", pd);
+        a.beta_stride = ChannelStride(beta, x, "beta", pd);
+        f.rm_stride = ChannelStride(running_mean, x, "running_mean", pd);
+        f.rv_stride = ChannelStride(running_var, x, "running_var", pd);
+        f.mo_stride = ChannelStride(mean_out, x, "mean_out", pd);
+        f.io_stride = ChannelStride(inv_std_out, x, "inv_std_out", pd);
         const int64_t total = static_cast<int64_t>(g.N) * g.C * g.L;
         if (total == 0) return;
         CheckWorkspace(workspace, workspace_bytes, TrainWorkspace(g));
@@ -468,14 +492,15 @@ int hipcx_batch_norm(const hipcx_array* x, const hipcx_array* gamma, const hipcx
         a.C = g.C, a.S = g.S, a.L = g.L, a.total = total;
         a.count = f.count;
         const unsigned cblocks = static_cast<unsigned>((g.C + 255) / 256);
-        VisitFloatDtype(x->dtype, [&](auto tag) {
+        VisitBnDtypes(x->dtype, pd, [&](auto tag, auto ptag) {
             using T = typename decltype(tag)::type;
-            LaunchStat<T, 0>(s, widths.stat, st);
-            hipLaunchKernelGGL((BnFinishKernel<T, 0>), dim3(cblocks), dim3(256), 0, st, f);
-            LaunchStat<T, 1>(s, widths.stat, st);
-            hipLaunchKernelGGL((BnFinishKernel<T, 1>), dim3(cblocks), dim3(256), 0, st, f);
+            using P = typename decltype(ptag)::type;
+            LaunchStat<T, P, 0>(s, widths.stat, st);
+            hipLaunchKernelGGL((BnFinishKernel<T, P, 0>), dim3(cblocks), dim3(256), 0, st, f);
+            LaunchStat<T, P, 1>(s, widths.stat, st);
+            hipLaunchKernelGGL((BnFinishKernel<T, P, 1>), dim3(cblocks), dim3(256), 0, st, f);
             CheckLaunch("batch_norm finish");
-            LaunchApply<T, false>(a, widths.apply, st);
+            LaunchApply<T, P, false>(a, widths.apply, st);
         });
     });
 }
@@ -492,11 +517,12 @@ int hipcx_batch_norm_grad(const hipcx_array* x, const hipcx_array* gamma, const 
         HIPCX_REQUIRE(gx->dtype == x->dtype && SameShape(x, gx) && IsContiguous(gx), HIPCX_NOT_IMPLEMENTED_ERROR,
                       "hip batch_norm_grad: gx must be C-contiguous with x's shape and dtype");
         BnApplyArgs a{};
-        a.gamma_stride = ChannelStride(gamma, x, "gamma");
-        a.gg_stride = ChannelStride(ggamma, x, "ggamma");
-        a.gb_stride = ChannelStride(gbeta, x, "gbeta");
-        const int64_t mean_stride = ChannelStride(mean, x, "mean");
-        const int64_t inv_stride = ChannelStride(inv_std, x, "inv_std");
+        const int pd = ParamDtype(x, gamma);
+        a.gamma_stride = ChannelStride(gamma, x, "gamma", pd);
+        a.gg_stride = ChannelStride(ggamma, x, "ggamma", pd);
+        a.gb_stride = ChannelStride(gbeta, x, "gbeta", pd);
+        const int64_t mean_stride = ChannelStride(mean, x, "mean", pd);
+        const int64_t inv_stride = ChannelStride(inv_std, x, "inv_std", pd);
         const int64_t total = static_cast<int64_t>(g.N) * g.C * g.L;
         if (total == 0) return;
         CheckWorkspace(workspace, workspace_bytes, TrainWorkspace(g));
@@ -506,8 +532,6 @@ int hipcx_batch_norm_grad(const hipcx_array* x, const hipcx_array* gamma, const 
         hipStream_t st = AsStream(stream);
         HIPCX_REQUIRE(total < (int64_t{1} << 31), HIPCX_NOT_IMPLEMENTED_ERROR, "hip batch_norm_grad: array too large for the dedicated kernels");
         const BnWidths widths = PickWidths(g.L, total, ItemSize(x->dtype), {x->data, gout->data, gx->data});
-        HIPCX_REQUIRE(mean->dtype == x->dtype && inv_std->dtype == x->dtype, HIPCX_NOT_IMPLEMENTED_ERROR,
-                      "hip batch_norm_grad: the state must have x's dtype");
         BnStatArgs s{};
         s.x = x->data;
         s.g = gout->data;
@@ -531,12 +555,13 @@ int hipcx_batch_norm_grad(const hipcx_array* x, const hipcx_array* gamma, const 
         a.C = g.C, a.S = g.S, a.L = g.L, a.total = total;
         a.count = static_cast<double>(g.N) * static_cast<double>(g.L);
         const unsigned cblocks = static_cast<unsigned>((g.C + 255) / 256);
-        VisitFloatDtype(x->dtype, [&](auto tag) {
+        VisitBnDtypes(x->dtype, pd, [&](auto tag, auto ptag) {
             using T = typename decltype(tag)::type;
-            LaunchStat<T, 2>(s, widths.stat, st);
-            hipLaunchKernelGGL((BnGradFinishKernel<T>), dim3(cblocks), dim3(256), 0, st, a);
+            using P = typename decltype(ptag)::type;
+            LaunchStat<T, P, 2>(s, widths.stat, st);
+            hipLaunchKernelGGL((BnGradFinishKernel<T, P>), dim3(cblocks), dim3(256), 0, st, a);
             CheckLaunch("batch_norm_grad finish");
-            LaunchApply<T, true>(a, widths.apply, st);
+            LaunchApply<T, P, true>(a, widths.apply, st);
         });
     });
 }

@@ -1616,11 +1616,14 @@ def var(a, axis=None, keepdims=False):
 COMPOSE_BATCH_NORM = False
 
 
-def _bn_kernel_applies(x, axes, others):
-    """The dedicated kernels take a C-contiguous x of fewer than 2^31 elements reduced over every axis but 1, with every other array
-    in x's dtype."""
+def _bn_kernel_applies(x, axes, params, same=()):
+    """The dedicated kernels take a C-contiguous x of fewer than 2^31 elements reduced over every axis but 1; the per-channel arrays
+    ``params`` share one dtype, x's or -- for a float16 x -- float32 (the mixed-precision call: parameters and statistics of a
+    float16 network kept in float32); the arrays in ``same`` have x's dtype."""
+    pd = params[0].dtype
     return (not COMPOSE_BATCH_NORM and x.ndim >= 2 and tuple(axes) == (0,) + tuple(range(2, x.ndim)) and x.is_contiguous and x.size < 2 ** 31
-            and _py.all(a.dtype == x.dtype for a in others))
+            and (pd == x.dtype or (x.dtype == numpy.dtype('float16') and pd == numpy.dtype('float32')))
+            and _py.all(a.dtype == pd for a in params) and _py.all(a.dtype == x.dtype for a in same))
 
 
 def batch_norm(x, gamma, beta, running_mean, running_var, eps=2e-5, decay=0.9, axis=None):
@@ -1635,8 +1638,8 @@ def batch_norm(x, gamma, beta, running_mean, running_var, eps=2e-5, decay=0.9, a
     if _bn_kernel_applies(x, axes, (gamma, beta, running_mean, running_var)) and x.size > 0:
         # the dedicated kernels: two statistics passes, a per-channel finish, one normalising pass
         out = ndarray.empty(x.shape, x.dtype)
-        x_mean = ndarray.empty(red_shape, x.dtype)
-        inv_std = ndarray.empty(red_shape, x.dtype)
+        x_mean = ndarray.empty(red_shape, interm)  # the state has the promoted dtype (CX/routines/normalization.cc:141-150)
+        inv_std = ndarray.empty(red_shape, interm)
         ax = (ctypes.c_int8 * len(axes))(*axes)
         nbytes = _lib.load().hipcx_batch_norm_workspace_size(x.desc(), ax, len(axes))
         ws, wsp = _workspace(nbytes)
@@ -1666,11 +1669,11 @@ def batch_norm_grad(x, gamma, gout, state, axis=None):
     axes = _sorted_axes((0,) + tuple(range(2, x.ndim)) if axis is None else axis, x.ndim)
     red_shape = tuple(1 if i in axes else d for i, d in enumerate(x.shape))
     interm = x_mean.dtype
-    if (_bn_kernel_applies(x, axes, (gamma, gout, x_mean, x_inv_std)) and gout.shape == x.shape and gout.is_contiguous
-            and numpy.dtype(beta_dtype) == x.dtype and x.size > 0):
+    if (_bn_kernel_applies(x, axes, (gamma, x_mean, x_inv_std), (gout,)) and gout.shape == x.shape and gout.is_contiguous
+            and numpy.dtype(beta_dtype) == gamma.dtype and x.size > 0):
         gx = ndarray.empty(x.shape, x.dtype)
-        ggamma = ndarray.empty(gamma.shape, x.dtype)
-        gbeta = ndarray.empty(gamma.shape, x.dtype)
+        ggamma = ndarray.empty(gamma.shape, gamma.dtype)
+        gbeta = ndarray.empty(gamma.shape, gamma.dtype)
         ax = (ctypes.c_int8 * len(axes))(*axes)
         nbytes = _lib.load().hipcx_batch_norm_workspace_size(x.desc(), ax, len(axes))
         ws, wsp = _workspace(nbytes)

@@ -864,10 +864,13 @@ def var(a, axis=None, keepdims=False):
 
 
 def batch_norm(x, gamma, beta, running_mean, running_var, eps=2e-5, decay=0.9, axis=None):
-    """GenericBatchNormKernel (CX/routines/normalization.cc:155-193), operands of one float dtype.  Returns
-    (out, new_running_mean, new_running_var, (x_mean, x_inv_std))."""
-    x = np.asarray(x)
-    dt = x.dtype
+    """GenericBatchNormKernel (CX/routines/normalization.cc:155-193).  Returns (out, new_running_mean, new_running_var,
+    (x_mean, x_inv_std)).  The statistics and the normalisation run in ResultType(x, gamma, beta) (:176-180) -- float32 for a
+    float16 x with float32 parameters -- and out is cast back to x's dtype (:143); the state keeps the promoted dtype."""
+    x_in = np.asarray(x)
+    dt = np.result_type(x_in.dtype, np.asarray(gamma).dtype, np.asarray(beta).dtype)
+    x = x_in.astype(dt, copy=False)
+    gamma, beta = np.asarray(gamma).astype(dt, copy=False), np.asarray(beta).astype(dt, copy=False)
     axes = tuple(sorted(a % x.ndim for a in ((0,) + tuple(range(2, x.ndim)) if axis is None else axis)))
     red = tuple(1 if i in axes else d for i, d in enumerate(x.shape))
     x_mean = mean(x, axes, True)
@@ -878,18 +881,23 @@ def batch_norm(x, gamma, beta, running_mean, running_var, eps=2e-5, decay=0.9, a
     out = add(multiply(multiply(subtract(x, B(x_mean)), B(inv_std)), B(g)), B(bt))
     n = x.size // max(1, np.asarray(gamma).size)
     inv_decay = 1.0 - float(decay)
-    rm = add(multiply(np.asarray(running_mean).reshape(red), _scalar_as(decay, dt)), multiply(x_mean, _scalar_as(inv_decay, dt)))
-    rv = add(multiply(np.asarray(running_var).reshape(red), _scalar_as(decay, dt)),
-             multiply(x_var, _scalar_as(inv_decay * (float(n) / max(n - 1, 1)), dt)))
+    rdt = np.asarray(running_mean).dtype  # running *= decay; running += (...).AsType(running dtype) (:185-190)
+    rm = add(multiply(np.asarray(running_mean).reshape(red), _scalar_as(decay, rdt)), multiply(x_mean, _scalar_as(inv_decay, dt)).astype(rdt, copy=False))
+    rv = add(multiply(np.asarray(running_var).reshape(red), _scalar_as(decay, rdt)),
+             multiply(x_var, _scalar_as(inv_decay * (float(n) / max(n - 1, 1)), dt)).astype(rdt, copy=False))
     shp = np.asarray(gamma).shape
-    return out, rm.reshape(shp), rv.reshape(shp), (x_mean, inv_std)
+    return out.astype(x_in.dtype, copy=False), rm.reshape(shp), rv.reshape(shp), (x_mean, inv_std)
 
 
 def batch_norm_grad(x, gamma, gout, state, axis=None):
-    """GenericBatchNormGradKernel (CX/routines/normalization.cc:195-250): (gx, ggamma, gbeta)."""
-    x, gout = np.asarray(x), np.asarray(gout)
-    dt = x.dtype
+    """GenericBatchNormGradKernel (CX/routines/normalization.cc:195-250): (gx, ggamma, gbeta).  Computed in the state's dtype
+    (:224-232); gx is cast to x's dtype, ggamma to gamma's, gbeta to the state's beta dtype -- taken to be gamma's here (:234-246)."""
+    x_in, gout = np.asarray(x), np.asarray(gout)
     x_mean, x_inv_std = state
+    dt = np.asarray(x_mean).dtype
+    x, gout = x_in.astype(dt, copy=False), gout.astype(dt, copy=False)
+    gamma_dtype = np.asarray(gamma).dtype
+    gamma = np.asarray(gamma).astype(dt, copy=False)
     axes = tuple(sorted(a % x.ndim for a in ((0,) + tuple(range(2, x.ndim)) if axis is None else axis)))
     red = tuple(1 if i in axes else d for i, d in enumerate(x.shape))
     B = lambda v: np.broadcast_to(v, x.shape)
@@ -901,7 +909,7 @@ def batch_norm_grad(x, gamma, gout, state, axis=None):
     inner = multiply(add(multiply(x_hat, B(ggamma)), B(gbeta)), _scalar_as(1.0 / n, dt))
     gx = multiply(B(multiply(g, x_inv_std)), subtract(gout, inner))
     shp = np.asarray(gamma).shape
-    return gx, ggamma.reshape(shp), gbeta.reshape(shp)
+    return gx.astype(x_in.dtype, copy=False), ggamma.reshape(shp).astype(gamma_dtype, copy=False), gbeta.reshape(shp).astype(gamma_dtype, copy=False)
 
 
 def max_pool_grad(x, gout, ksize, stride=None, pad=0, cover_all=False):

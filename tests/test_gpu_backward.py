@@ -374,3 +374,40 @@ def test_conv_grad_weight_special_values(dt, tol):
         x2 = rng.standard_normal((N, C, H, W)).astype(dt)
         assert_close(chx.conv_grad_weight(dt, (K, C, kh, kw), chx.array(x2), chx.array(gy2), 1, pd).get(),
                      O.conv_grad_weight((K, C, kh, kw), x2, gy2, 1, pd), tol, 'conv_grad_weight with inf in gy ' + what)
+
+
+def test_batch_norm_float16_with_float32_parameters():
+    """The mixed-precision call (float16 x and gout; float32 gamma, beta, running statistics): the reference computes in float32
+    (CX/routines/normalization.cc:176-180) and so do the kernels -- no float16 overflow at 50176 elements per channel, state and
+    parameter gradients in float32, out and gx in float16.  Against the oracle and against the composition on the device."""
+    import chainer_amd as chx
+    from chainer_amd import routines
+    rng = np.random.default_rng(172)
+    for shape in [(64, 6, 28, 28), (4, 5, 7, 7), (16, 8)]:
+        C = shape[1]
+        x = (rng.standard_normal(shape) * 2 + 0.5).astype(np.float16)
+        gamma, beta = rng.uniform(0.5, 1.5, C).astype(np.float32), rng.standard_normal(C).astype(np.float32)
+        rm0, rv0 = rng.standard_normal(C).astype(np.float32), rng.uniform(0.5, 1.5, C).astype(np.float32)
+        gout = rng.standard_normal(shape).astype(np.float16)
+        axis = (0,) if len(shape) == 2 else None
+        res = {}
+        for mode in ('kernel', 'composition'):
+            routines.COMPOSE_BATCH_NORM = mode == 'composition'
+            try:
+                RM, RV = chx.array(rm0), chx.array(rv0)
+                out, state = chx.batch_norm(chx.array(x), chx.array(gamma), chx.array(beta), RM, RV, 2e-5, 0.9, axis)
+                gx, gg, gb = chx.batch_norm_grad(chx.array(x), chx.array(gamma), chx.array(gout), state, axis)
+                res[mode] = [out.get(), RM.get(), RV.get(), state[0].get(), state[1].get(), gx.get(), gg.get(), gb.get()]
+            finally:
+                routines.COMPOSE_BATCH_NORM = False
+        o_ref, rm_ref, rv_ref, st_ref = O.batch_norm(x, gamma, beta, rm0.copy(), rv0.copy(), 2e-5, 0.9, axis)
+        gx_ref, gg_ref, gb_ref = O.batch_norm_grad(x, gamma, gout, st_ref, axis)
+        ref = [o_ref, rm_ref, rv_ref, st_ref[0], st_ref[1], gx_ref, gg_ref, gb_ref]
+        names = ['out', 'running_mean', 'running_var', 'mean', 'inv_std', 'gx', 'ggamma', 'gbeta']
+        dtypes = ['float16', 'float32', 'float32', 'float32', 'float32', 'float16', 'float32', 'float32']
+        for name, dt, k, c, r in zip(names, dtypes, res['kernel'], res['composition'], ref):
+            assert k.dtype == np.dtype(dt) and c.dtype == np.dtype(dt), (name, k.dtype, c.dtype)
+            assert np.isfinite(k).all(), name
+            tol = {'out': 2e-3, 'gx': 4e-3, 'ggamma': 2e-4, 'gbeta': 2e-4}.get(name, 2e-5)
+            assert_close(k.reshape(r.shape), r, tol, 'mixed batch_norm %s %r: kernel vs oracle' % (name, shape))
+            assert_close(k.reshape(r.shape), c.reshape(r.shape), tol, 'mixed batch_norm %s %r: kernel vs composition' % (name, shape))

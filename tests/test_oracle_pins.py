@@ -732,6 +732,43 @@ def test_batch_norm_training_closed_forms():
         assert abs((loss(x, gamma, beta + e) - loss(x, gamma, beta - e)) / (2 * h) - gb[c]) <= 1e-6
 
 
+def test_batch_norm_dtypes():
+    """The dtype rules of GenericBatchNormKernel (CX/routines/normalization.cc:176-193, 224-246).  float16 x with float32 parameters:
+    computed in float32 -- statistics, state and running values are float32 and agree with the float64 closed form to float32
+    accuracy, out / gx are float16 and within half a float16 ulp of it, and 50176 elements per channel are no problem.  All float16:
+    the same size overflows the float16 Sum of (x - mean)^2 (native Sum hands out a float16, CX/native/native_device/reduction.cc:105-110):
+    variance inf, inv_std 0, out == beta exactly."""
+    rng = np.random.default_rng(44)
+    shape = (64, 3, 28, 28)
+    x = (rng.standard_normal(shape) * 2 + 0.5).astype(np.float16)
+    gamma, beta = rng.uniform(0.5, 1.5, 3).astype(np.float32), rng.standard_normal(3).astype(np.float32)
+    rm, rv = rng.standard_normal(3).astype(np.float32), rng.uniform(0.5, 1.5, 3).astype(np.float32)
+    out, nrm, nrv, (mean, inv_std) = O.batch_norm(x, gamma, beta, rm, rv, 2e-5, 0.9)
+    assert out.dtype == np.float16 and nrm.dtype == nrv.dtype == mean.dtype == inv_std.dtype == np.float32
+    x64 = x.astype(np.float64)
+    m, v = x64.mean(axis=(0, 2, 3)), x64.var(axis=(0, 2, 3))
+    bc = lambda a: a.reshape(1, 3, 1, 1)
+    assert np.allclose(mean.ravel(), m, rtol=1e-5, atol=1e-6) and np.allclose(inv_std.ravel(), 1 / np.sqrt(v + 2e-5), rtol=1e-5)
+    want = (x64 - bc(m)) / np.sqrt(bc(v) + 2e-5) * bc(gamma.astype(np.float64)) + bc(beta.astype(np.float64))
+    assert np.abs(out.astype(np.float64) - want).max() <= np.abs(want).max() * 2.0 ** -11 * 1.01  # one rounding to float16
+    n = x.size // 3
+    assert np.allclose(nrm, 0.9 * rm + 0.1 * m, rtol=1e-5, atol=1e-6) and np.allclose(nrv, 0.9 * rv + 0.1 * v * n / (n - 1), rtol=1e-5)
+    gout = rng.standard_normal(shape).astype(np.float16)
+    gx, gg, gb = O.batch_norm_grad(x, gamma, gout, (mean, inv_std))
+    assert gx.dtype == np.float16 and gg.dtype == gb.dtype == np.float32
+    g64 = gout.astype(np.float64)
+    xh = (x64 - bc(m)) / np.sqrt(bc(v) + 2e-5)
+    assert np.allclose(gb, g64.sum(axis=(0, 2, 3)), rtol=1e-4, atol=1e-3) and np.allclose(gg, (g64 * xh).sum(axis=(0, 2, 3)), rtol=1e-4, atol=1e-3)
+    gx64 = bc(gamma.astype(np.float64)) / np.sqrt(bc(v) + 2e-5) * (g64 - (xh * bc((g64 * xh).sum(axis=(0, 2, 3))) + bc(g64.sum(axis=(0, 2, 3)))) / n)
+    assert np.abs(gx.astype(np.float64) - gx64).max() <= np.abs(gx64).max() * 2.0 ** -10
+    # all float16
+    g16, b16 = gamma.astype(np.float16), beta.astype(np.float16)
+    out, nrm, nrv, (mean, inv_std) = O.batch_norm(x, g16, b16, rm.astype(np.float16), rv.astype(np.float16), 2e-5, 0.9)
+    assert out.dtype == nrm.dtype == mean.dtype == inv_std.dtype == np.float16
+    assert np.all(inv_std == 0) and np.all(np.isinf(nrv)) and np.all(np.isfinite(mean))
+    assert np.array_equal(out, np.broadcast_to(bc(b16), shape))
+
+
 # ---------------------------------------------------------------------------------------------
 # activations built from other routines, and the n-step recurrent family: textbook formulas in float64
 # ---------------------------------------------------------------------------------------------
