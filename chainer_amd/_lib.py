@@ -203,6 +203,13 @@ SIGNATURES = {
     'hipcx_n_step_lstm_workspace_size': (_SZ, [_INT, _A, ctypes.POINTER(_A), _INT]),
     'hipcx_n_step_lstm': (_INT, [_INT, _A, _A, ctypes.POINTER(_A), ctypes.POINTER(_A), ctypes.POINTER(_A), _INT, _A, _A, ctypes.POINTER(_A),
                                  _V, _SZ, _V]),
+    'hipcx_n_step_rnn_reserve_size': (_SZ, [_INT, _INT, _INT, _A, ctypes.POINTER(_A), _INT]),
+    'hipcx_n_step_rnn_workspace_size': (_SZ, [_INT, _INT, _INT, _INT, _A, ctypes.POINTER(_A), _INT]),
+    'hipcx_n_step_rnn': (_INT, [_INT, _INT, _INT, _INT, _A, _A, ctypes.POINTER(_A), ctypes.POINTER(_A), ctypes.POINTER(_A), _INT, _A, _A,
+                                ctypes.POINTER(_A), _V, _SZ, _V, _SZ, _V]),
+    'hipcx_n_step_rnn_backward': (_INT, [_INT, _INT, _INT, _INT, _A, ctypes.POINTER(_A), ctypes.POINTER(_A), ctypes.POINTER(_A), _INT, _A, _A,
+                                         ctypes.POINTER(_A), _V, _SZ, _A, _A, ctypes.POINTER(_A), ctypes.POINTER(_A), ctypes.POINTER(_A),
+                                         _V, _SZ, _V]),
     'hipcx_profile_records': (_INT, [ctypes.c_int64, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double),
                                      ctypes.POINTER(ctypes.c_double), _I64P]),
     'hipcx_fixed_batch_norm': (_INT, [_A, _A, _A, _A, _A, _S, _I8P, _INT, _A, _V]),

@@ -1063,61 +1063,182 @@ public:
 };
 HIPCX_REGISTER_KERNEL(AveragePoolGradKernel, HipAveragePoolGradKernel)
 
-// ---- RnnKernel (chainerx/kernels/rnn.h:34-49): the forward pass of a one-directional float32 LSTM in one library call.
-// The reference's NStepRnnImpl hands this kernel to the backend named "cuda" only (chainerx/routines/n_step_rnn.cc:210) and
-// composes the routine for every other backend, so the registration takes effect once that test also admits "hip".  Modes the
-// library does not take (GRU, plain RNN, both directions, other dtypes) raise NotImplementedError; no gradient state is kept.
+// ---- RnnKernel / RnnBackwardKernel (chainerx/kernels/rnn.h:34-66): float32 LSTM, GRU and tanh / relu RNN, one or both directions,
+// through hipcx_n_step_rnn / hipcx_n_step_rnn_backward.  The reference's NStepRnnImpl hands these kernels to the backend named "cuda"
+// only (chainerx/routines/n_step_rnn.cc:210,330) and composes the routine for every other backend, so the registrations take effect
+// once that test also admits "hip".  Other dtypes raise NotImplementedError.
+namespace {
+// What the forward pass leaves for the backward pass: the library's reserve (gate activations, states before each step, outputs of
+// the lower layers) and the call's mode.
+class HipRnnGradState : public RnnGradState {
+public:
+    std::shared_ptr<void> reserve;
+    size_t reserve_bytes = 0;
+    int8_t mode = 0;
+    int activation = 0;
+};
+
+struct RnnOperands {
+    std::vector<Array> keep;  // contiguous float32 copies where the caller's arrays are something else
+    std::vector<hipcx_array> w, b, x;
+    std::vector<const hipcx_array*> pw, pb, px;
+};
+
+hipcx_array PrepareRnnOperand(RnnOperands& ops, Device& device, const Array& reference, const Array& a) {
+    device.CheckDevicesCompatible(reference, a);
+    ops.keep.emplace_back(a.dtype() == Dtype::kFloat32 && a.IsContiguous() ? a : AsContiguous(a.AsType(Dtype::kFloat32)));
+    return ToC(ops.keep.back());
+}
+
+std::vector<const hipcx_array*> PointersTo(const std::vector<hipcx_array>& v) {
+    std::vector<const hipcx_array*> p;
+    p.reserve(v.size());
+    for (const hipcx_array& d : v) p.push_back(&d);
+    return p;
+}
+
+void PrepareRnnOperands(RnnOperands& ops, Device& device, const Array& hx, const std::vector<std::vector<Array>>& ws,
+                        const std::vector<std::vector<Array>>& bs, const std::vector<Array>& xs) {
+    size_t n = 0;
+    for (const std::vector<Array>& group : ws) n += 2 * group.size();
+    ops.keep.reserve(n + xs.size() + 8);
+    for (size_t i = 0; i < ws.size(); ++i) {
+        for (size_t j = 0; j < ws[i].size(); ++j) {
+            ops.w.push_back(PrepareRnnOperand(ops, device, hx, ws[i][j]));
+            ops.b.push_back(PrepareRnnOperand(ops, device, hx, bs.at(i).at(j)));
+        }
+    }
+    for (const Array& x : xs) ops.x.push_back(PrepareRnnOperand(ops, device, hx, x));
+    ops.pw = PointersTo(ops.w), ops.pb = PointersTo(ops.b), ops.px = PointersTo(ops.x);
+}
+
+int RnnActivation(const absl::optional<std::string>& activation) { return activation.has_value() && *activation == "relu" ? 1 : 0; }
+}  // namespace
+
 class HipRnnKernel : public RnnKernel {
 public:
     std::tuple<std::vector<std::vector<Array>>, std::unique_ptr<RnnGradState>> Call(
             int64_t n_layers, Array hx, absl::optional<Array> cx, const std::vector<std::vector<Array>>& ws, const std::vector<std::vector<Array>>& bs,
-            const std::vector<Array>& xs, int8_t bidirectional, int8_t mode, absl::optional<std::string> /*activation*/) override {
-        if (mode != 1 || bidirectional != 0 || !cx.has_value() || hx.dtype() != Dtype::kFloat32) {
-            throw NotImplementedError{"hip RnnKernel: one-directional float32 LSTM only."};
-        }
+            const std::vector<Array>& xs, int8_t bidirectional, int8_t mode, absl::optional<std::string> activation) override {
+        if (hx.dtype() != Dtype::kFloat32) throw NotImplementedError{"hip RnnKernel: float32 only."};
+        if (mode == 1 && !cx.has_value()) throw ChainerxError{"hip RnnKernel: the LSTM mode needs cx."};
         Device& device = hx.device();
         SetDeviceScope scope{device.index()};
-        std::vector<Array> keep;  // contiguous float32 copies where the caller's arrays are something else
-        auto prepared = [&](const Array& a) {
-            device.CheckDevicesCompatible(hx, a);
-            keep.emplace_back(a.dtype() == Dtype::kFloat32 && a.IsContiguous() ? a : AsContiguous(a.AsType(Dtype::kFloat32)));
-            return ToC(keep.back());
-        };
-        hipcx_array chx_ = prepared(hx), ccx = prepared(*cx);
-        std::vector<hipcx_array> dw, db, dx, dy;
-        for (int64_t l = 0; l < n_layers; ++l) {
-            for (size_t i = 0; i < 8; ++i) {
-                dw.push_back(prepared(ws.at(l).at(i)));
-                db.push_back(prepared(bs.at(l).at(i)));
-            }
-        }
-        for (const Array& x : xs) dx.push_back(prepared(x));
+        RnnOperands ops;
+        PrepareRnnOperands(ops, device, hx, ws, bs, xs);
+        hipcx_array chx_ = PrepareRnnOperand(ops, device, hx, hx);
+        hipcx_array ccx{};
+        if (mode == 1) ccx = PrepareRnnOperand(ops, device, hx, *cx);
+        const int64_t directions = bidirectional ? 2 : 1;
         Array hy = Empty(hx.shape(), Dtype::kFloat32, device);
-        Array cy = Empty(hx.shape(), Dtype::kFloat32, device);
+        Array cy = mode == 1 ? Empty(hx.shape(), Dtype::kFloat32, device) : Array{};
         std::vector<Array> ys;
+        std::vector<hipcx_array> dy;
         for (const Array& x : xs) {
-            ys.emplace_back(Empty(Shape{x.shape()[0], hx.shape()[2]}, Dtype::kFloat32, device));
+            ys.emplace_back(Empty(Shape{x.shape()[0], directions * hx.shape()[2]}, Dtype::kFloat32, device));
             dy.push_back(ToC(ys.back()));
         }
-        auto pointers = [](const std::vector<hipcx_array>& v) {
-            std::vector<const hipcx_array*> p;
-            for (const hipcx_array& d : v) p.push_back(&d);
-            return p;
-        };
-        std::vector<const hipcx_array*> pw = pointers(dw), pb = pointers(db), px = pointers(dx), py = pointers(dy);
-        hipcx_array chy = ToC(hy), ccy = ToC(cy);
+        std::vector<const hipcx_array*> py = PointersTo(dy);
+        hipcx_array chy = ToC(hy), ccy{};
+        if (mode == 1) ccy = ToC(cy);
         const int n_steps = static_cast<int>(xs.size());
-        size_t ws_bytes = hipcx_n_step_lstm_workspace_size(static_cast<int>(n_layers), &chx_, px.data(), n_steps);
+        // A gradient may be asked for later if any input belongs to a graph; then the forward pass keeps its reserve.
+        bool training = !internal::GetArrayBody(hx)->nodes().empty() || (cx.has_value() && !internal::GetArrayBody(*cx)->nodes().empty());
+        for (const Array& x : xs) training = training || !internal::GetArrayBody(x)->nodes().empty();
+        for (const std::vector<Array>& group : ws) {
+            for (const Array& w : group) training = training || !internal::GetArrayBody(w)->nodes().empty();
+        }
+        for (const std::vector<Array>& group : bs) {
+            for (const Array& b : group) training = training || !internal::GetArrayBody(b)->nodes().empty();
+        }
+        std::unique_ptr<HipRnnGradState> state;
+        void* reserve = nullptr;
+        size_t reserve_bytes = 0;
+        if (training) {
+            state = std::make_unique<HipRnnGradState>();
+            reserve_bytes = hipcx_n_step_rnn_reserve_size(static_cast<int>(n_layers), bidirectional, mode, &chx_, ops.px.data(), n_steps);
+            state->reserve = device.Allocate(reserve_bytes);
+            state->reserve_bytes = reserve_bytes;
+            state->mode = mode;
+            state->activation = RnnActivation(activation);
+            reserve = state->reserve.get();
+        }
+        size_t ws_bytes = hipcx_n_step_rnn_workspace_size(static_cast<int>(n_layers), bidirectional, mode, 0, &chx_, ops.px.data(), n_steps);
+        if (training) ws_bytes = hipcx_n_step_rnn_workspace_size(static_cast<int>(n_layers), bidirectional, mode, 1, &chx_, ops.px.data(), n_steps);
         std::shared_ptr<void> wsp = device.Allocate(ws_bytes);
-        Check(hipcx_n_step_lstm(static_cast<int>(n_layers), &chx_, &ccx, pw.data(), pb.data(), px.data(), n_steps, &chy, &ccy, py.data(), wsp.get(),
-                                ws_bytes, nullptr));
+        Check(hipcx_n_step_rnn(static_cast<int>(n_layers), bidirectional, mode, RnnActivation(activation), &chx_, mode == 1 ? &ccx : nullptr,
+                               ops.pw.data(), ops.pb.data(), ops.px.data(), n_steps, &chy, mode == 1 ? &ccy : nullptr, py.data(), reserve,
+                               reserve_bytes, wsp.get(), ws_bytes, nullptr));
         std::vector<std::vector<Array>> ret;
-        ret.emplace_back(std::vector<Array>{std::move(hy), std::move(cy)});
+        std::vector<Array> states{std::move(hy)};
+        if (mode == 1) states.emplace_back(std::move(cy));
+        ret.emplace_back(std::move(states));
         ret.emplace_back(std::move(ys));
-        return std::make_tuple(std::move(ret), std::unique_ptr<RnnGradState>{});
+        return std::make_tuple(std::move(ret), std::unique_ptr<RnnGradState>{std::move(state)});
     }
 };
 HIPCX_REGISTER_KERNEL(RnnKernel, HipRnnKernel)
+
+class HipRnnBackwardKernel : public RnnBackwardKernel {
+public:
+    // Returns {{dhx[, dcx]}, {dw, db for every matrix in ws' order}, {dxs}} as NStepRnnImpl's backward reads it
+    // (chainerx/routines/n_step_rnn.cc:330-354).
+    std::vector<std::vector<Array>> Call(
+            int64_t n_layers, Array hx, absl::optional<Array> cx, const std::vector<std::vector<Array>>& ws, const std::vector<std::vector<Array>>& bs,
+            const std::vector<Array>& xs, Array dhy, absl::optional<Array> dcy, std::vector<Array> /*ys*/, std::vector<Array> dys,
+            int8_t bidirectional, const std::shared_ptr<chainerx::RnnGradState>& state) override {
+        auto* st = dynamic_cast<HipRnnGradState*>(state.get());
+        if (st == nullptr) throw ChainerxError{"hip RnnBackwardKernel: the forward pass kept no state (no input required a gradient)."};
+        Device& device = hx.device();
+        SetDeviceScope scope{device.index()};
+        const int8_t mode = st->mode;
+        RnnOperands ops;
+        PrepareRnnOperands(ops, device, hx, ws, bs, xs);
+        hipcx_array chx_ = PrepareRnnOperand(ops, device, hx, hx);
+        hipcx_array cdhy = PrepareRnnOperand(ops, device, hx, dhy);
+        hipcx_array cdcy{};
+        const bool has_dcy = mode == 1 && dcy.has_value();
+        if (has_dcy) cdcy = PrepareRnnOperand(ops, device, hx, *dcy);
+        std::vector<hipcx_array> cdys;
+        for (const Array& g : dys) cdys.push_back(PrepareRnnOperand(ops, device, hx, g));
+        std::vector<const hipcx_array*> pdys = PointersTo(cdys);
+        Array dhx = Empty(hx.shape(), Dtype::kFloat32, device);
+        Array dcx = mode == 1 ? Empty(hx.shape(), Dtype::kFloat32, device) : Array{};
+        std::vector<Array> dws, dbs, dxs, params;
+        std::vector<hipcx_array> cdw, cdb, cdx;
+        for (size_t i = 0; i < ws.size(); ++i) {
+            for (size_t j = 0; j < ws[i].size(); ++j) {
+                dws.emplace_back(Empty(ws[i][j].shape(), Dtype::kFloat32, device));
+                dbs.emplace_back(Empty(bs.at(i).at(j).shape(), Dtype::kFloat32, device));
+            }
+        }
+        for (const Array& x : xs) dxs.emplace_back(Empty(x.shape(), Dtype::kFloat32, device));
+        for (const Array& a : dws) cdw.push_back(ToC(a));
+        for (const Array& a : dbs) cdb.push_back(ToC(a));
+        for (const Array& a : dxs) cdx.push_back(ToC(a));
+        std::vector<const hipcx_array*> pdw = PointersTo(cdw), pdb = PointersTo(cdb), pdx = PointersTo(cdx);
+        hipcx_array cdhx = ToC(dhx), cdcx{};
+        if (mode == 1) cdcx = ToC(dcx);
+        const int n_steps = static_cast<int>(xs.size());
+        size_t ws_bytes = hipcx_n_step_rnn_workspace_size(static_cast<int>(n_layers), bidirectional, mode, 1, &chx_, ops.px.data(), n_steps);
+        std::shared_ptr<void> wsp = device.Allocate(ws_bytes);
+        Check(hipcx_n_step_rnn_backward(static_cast<int>(n_layers), bidirectional, mode, st->activation, &chx_, ops.pw.data(), ops.pb.data(),
+                                        ops.px.data(), n_steps, &cdhy, has_dcy ? &cdcy : nullptr, pdys.data(), st->reserve.get(), st->reserve_bytes,
+                                        &cdhx, mode == 1 ? &cdcx : nullptr, pdw.data(), pdb.data(), pdx.data(), wsp.get(), ws_bytes, nullptr));
+        std::vector<Array> states{std::move(dhx)};
+        if (mode == 1) states.emplace_back(std::move(dcx));
+        for (size_t i = 0; i < dws.size(); ++i) {  // interleaved: w0, b0, w1, b1, ...
+            params.emplace_back(std::move(dws[i]));
+            params.emplace_back(std::move(dbs[i]));
+        }
+        std::vector<std::vector<Array>> ret;
+        ret.emplace_back(std::move(states));
+        ret.emplace_back(std::move(params));
+        ret.emplace_back(std::move(dxs));
+        return ret;
+    }
+};
+HIPCX_REGISTER_KERNEL(RnnBackwardKernel, HipRnnBackwardKernel)
 
 // ---- linear algebra: Solve, Inverse, Cholesky, Syevd, Qr, Svd (the LAPACK-backed kernels of the native backend, native_device/linalg.cc) ----
 namespace {

@@ -2035,6 +2035,70 @@ def _descriptor_pointers(arrays):
     return (ctypes.POINTER(_lib.CArray) * len(arrays))(*[ctypes.pointer(a._desc) for a in arrays])
 
 
+class RnnGradState(object):
+    """What RnnKernel hands to RnnBackwardKernel (chainerx::RnnGradState, CX/kernels/rnn.h:22-32): the reserve the forward pass
+    filled and the call's arguments."""
+
+    def __init__(self, **kw):
+        self.__dict__.update(kw)
+
+
+_RNN_MODES = {'gru': 0, 'lstm': 1, 'rnn': 2}
+
+
+def rnn(n_layers, hx, cx, ws, bs, xs, bidirectional, mode, activation=None, training=False):
+    """RnnKernel::Call (CX/kernels/rnn.h:34-49) through hipcx_n_step_rnn, float32: ``mode`` 'gru' / 'lstm' / 'rnn' (or the
+    reference's 0 / 1 / 2), ``activation`` 'tanh' / 'relu' for 'rnn'.  ws[layer * directions + direction] / bs[...] hold the 6 / 8 / 2
+    matrices / vectors of that layer and direction.  Returns ((hy, cy or None), ys, state); ``state`` is None unless ``training``."""
+    m = _RNN_MODES.get(mode, mode)
+    if m not in (0, 1, 2):
+        raise _lib.ChainerxError('rnn: unknown mode %r' % (mode,))
+    act = {None: 0, 'tanh': 0, 'relu': 1}[activation]
+    d = 2 if bidirectional else 1
+    flat_w = [w for group in ws for w in group]
+    flat_b = [b for group in bs for b in group]
+    xs = list(xs)
+    hy = ndarray.empty(hx.shape, hx.dtype)
+    cy = ndarray.empty(cx.shape, cx.dtype) if m == 1 else None
+    ys = [ndarray.empty((x.shape[0], d * hx.shape[2]), hx.dtype) for x in xs]
+    pw, pb, px, py = (_descriptor_pointers(v) for v in (flat_w, flat_b, xs, ys))
+    L = _lib.load()
+    rbytes = L.hipcx_n_step_rnn_reserve_size(n_layers, d - 1, m, hx.desc(), px, len(xs)) if training else 0
+    reserve, rp = _workspace(rbytes) if training else (None, None)
+    nbytes = L.hipcx_n_step_rnn_workspace_size(n_layers, d - 1, m, int(bool(training)), hx.desc(), px, len(xs))
+    wsb, wsp = _workspace(nbytes)
+    _lib.call('hipcx_n_step_rnn', n_layers, d - 1, m, act, hx.desc(), cx.desc() if m == 1 else None, pw, pb, px, len(xs), hy.desc(),
+              cy.desc() if m == 1 else None, py, rp, rbytes, wsp, nbytes, current_stream())
+    state = None
+    if training:
+        state = RnnGradState(reserve=reserve, reserve_ptr=rp, reserve_bytes=rbytes, n_layers=n_layers, directions=d, mode=m, activation=act,
+                             hx=hx, ws=flat_w, bs=flat_b, xs=xs)
+    return (hy, cy), ys, state
+
+
+def rnn_backward(state, dhy, dcy, dys):
+    """RnnBackwardKernel::Call (CX/kernels/rnn.h:51-66) through hipcx_n_step_rnn_backward: the gradients of the forward pass that
+    produced ``state``.  ``dcy`` and entries of ``dys`` may be None (zeros).  Returns ((dhx, dcx or None), dws, dbs, dxs) with dws / dbs
+    flat in the order of the forward call's matrices."""
+    st = state
+    dhx = ndarray.empty(st.hx.shape, st.hx.dtype)
+    dcx = ndarray.empty(st.hx.shape, st.hx.dtype) if st.mode == 1 else None
+    dws = [ndarray.empty(w.shape, w.dtype) for w in st.ws]
+    dbs = [ndarray.empty(b.shape, b.dtype) for b in st.bs]
+    dxs = [ndarray.empty(x.shape, x.dtype) for x in st.xs]
+    pw, pb, px, pdw, pdb, pdx = (_descriptor_pointers(v) for v in (st.ws, st.bs, st.xs, dws, dbs, dxs))
+    for a in dys:
+        if a is not None:
+            a.desc()
+    pdy = (ctypes.POINTER(_lib.CArray) * len(dys))(*[ctypes.pointer(a._desc) if a is not None else None for a in dys])
+    nbytes = _lib.load().hipcx_n_step_rnn_workspace_size(st.n_layers, st.directions - 1, st.mode, 1, st.hx.desc(), px, len(st.xs))
+    wsb, wsp = _workspace(nbytes)
+    _lib.call('hipcx_n_step_rnn_backward', st.n_layers, st.directions - 1, st.mode, st.activation, st.hx.desc(), pw, pb, px, len(st.xs),
+              dhy.desc(), dcy.desc() if (dcy is not None and st.mode == 1) else None, pdy, st.reserve_ptr, st.reserve_bytes, dhx.desc(),
+              dcx.desc() if st.mode == 1 else None, pdw, pdb, pdx, wsp, nbytes, current_stream())
+    return (dhx, dcx), dws, dbs, dxs
+
+
 def _n_step_lstm_kernel(n_layers, hx, cx, ws, bs, xs):
     """The RnnKernel entry (hipcx_n_step_lstm): weights packed once, one launch per wavefront stage."""
     if len(ws) != n_layers or len(bs) != n_layers or _py.any(len(w) != 8 for w in ws) or _py.any(len(b) != 8 for b in bs):
@@ -2061,28 +2125,49 @@ def n_step_lstm(n_layers, hx, cx, ws, bs, xs, fused=False, kernel=False):
     return _n_step_rnn_impl(_lstm_impl_fused if fused else _lstm_impl, n_layers, hx, cx, ws, bs, xs, False)
 
 
-def n_step_bilstm(n_layers, hx, cx, ws, bs, xs, fused=False):
+def _rnn_kernel_route(kernel, hx):
+    """`kernel` (opt-in) runs a whole n-step routine through hipcx_n_step_rnn, the RnnKernel the reference gives its cuda backend
+    (CX/routines/n_step_rnn.cc:210); float32 only, other dtypes take the composition."""
+    return kernel and hx.dtype == numpy.dtype('float32')
+
+
+def n_step_bilstm(n_layers, hx, cx, ws, bs, xs, fused=False, kernel=False):
     """NStepBiLstm (CX/routines/n_step_rnn.cc:445-454): ws[2*layer + direction]."""
+    if _rnn_kernel_route(kernel, hx):
+        (hy, cy), ys, _ = rnn(n_layers, hx, cx, ws, bs, xs, True, 'lstm')
+        return hy, cy, ys
     return _n_step_rnn_impl(_lstm_impl_fused if fused else _lstm_impl, n_layers, hx, cx, ws, bs, xs, True)
 
 
-def n_step_gru(n_layers, hx, ws, bs, xs):
+def n_step_gru(n_layers, hx, ws, bs, xs, kernel=False):
     """NStepGru (CX/routines/n_step_rnn.cc:456-465) -> (hy, ys); six matrices per layer: reset, update, candidate for x, then h."""
+    if _rnn_kernel_route(kernel, hx):
+        (hy, _), ys, _ = rnn(n_layers, hx, None, ws, bs, xs, False, 'gru')
+        return hy, ys
     return _n_step_rnn_impl(_gru_impl, n_layers, hx, None, ws, bs, xs, False)
 
 
-def n_step_bigru(n_layers, hx, ws, bs, xs):
+def n_step_bigru(n_layers, hx, ws, bs, xs, kernel=False):
     """NStepBiGru (CX/routines/n_step_rnn.cc:467-476)."""
+    if _rnn_kernel_route(kernel, hx):
+        (hy, _), ys, _ = rnn(n_layers, hx, None, ws, bs, xs, True, 'gru')
+        return hy, ys
     return _n_step_rnn_impl(_gru_impl, n_layers, hx, None, ws, bs, xs, True)
 
 
-def n_step_rnn(n_layers, hx, ws, bs, xs, activation='tanh'):
+def n_step_rnn(n_layers, hx, ws, bs, xs, activation='tanh', kernel=False):
     """NStepRnn (CX/routines/n_step_rnn.cc:478-487) -> (hy, ys); activation 'tanh' or 'relu'."""
+    if _rnn_kernel_route(kernel, hx):
+        (hy, _), ys, _ = rnn(n_layers, hx, None, ws, bs, xs, False, 'rnn', activation)
+        return hy, ys
     return _n_step_rnn_impl(_rnn_impl, n_layers, hx, None, ws, bs, xs, False, activation)
 
 
-def n_step_birnn(n_layers, hx, ws, bs, xs, activation='tanh'):
+def n_step_birnn(n_layers, hx, ws, bs, xs, activation='tanh', kernel=False):
     """NStepBiRnn (CX/routines/n_step_rnn.cc:489-498)."""
+    if _rnn_kernel_route(kernel, hx):
+        (hy, _), ys, _ = rnn(n_layers, hx, None, ws, bs, xs, True, 'rnn', activation)
+        return hy, ys
     return _n_step_rnn_impl(_rnn_impl, n_layers, hx, None, ws, bs, xs, True, activation)
 
 

@@ -363,6 +363,32 @@ size_t hipcx_n_step_lstm_workspace_size(int n_layers, const hipcx_array* hx, con
 int hipcx_n_step_lstm(int n_layers, const hipcx_array* hx, const hipcx_array* cx, const hipcx_array* const* ws, const hipcx_array* const* bs,
                       const hipcx_array* const* xs, int n_steps, const hipcx_array* hy, const hipcx_array* cy, const hipcx_array* const* ys,
                       void* workspace, size_t workspace_bytes, void* stream);
+/* hipcx_n_step_rnn / hipcx_n_step_rnn_backward: RnnKernel and RnnBackwardKernel (CX/kernels/rnn.h:34-66) for float32, every mode
+ *   NStepRnnImpl passes (CX/routines/n_step_rnn.cc:434-497): `mode` 0 GRU, 1 LSTM, 2 RNN (`activation` 0 tanh, 1 relu; ignored for
+ *   the other modes), `bidirectional` 0 / 1.  D = directions, G = 3 / 4 / 1 gates.
+ *   hx, hy (cx, cy: LSTM only, else NULL): [n_layers * D, B, H], index layer * D + direction.  ws / bs: for every layer-direction
+ *   2 * G matrices [H, in] ([H, H] for the second G) / vectors [H] in the reference's (cuDNN's) order, in = xs' columns for layer 0
+ *   and D * H above.  xs[t]: [B_t, in] with B_t <= B; ys[t]: [B_t, D * H] (unit stride along the last axis).  Rows of the state beyond
+ *   B_t keep their values (OneDirectionalLoop, n_step_rnn.cc:133-175).
+ *   `reserve`: NULL for inference; for training hipcx_n_step_rnn_reserve_size bytes (256-byte aligned) that the forward pass fills
+ *   (gate activations, the states before each step, the lower layers' outputs: the role of RnnGradState) and the backward pass reads.
+ *   `workspace`: 256-byte aligned, hipcx_n_step_rnn_workspace_size bytes (`training` 1 covers both passes).
+ *   Backward (RnnBackwardKernel::Call's grad lists): dhy (dcy: LSTM, may be NULL = zeros), dys[t] [B_t, D * H] (an entry may be NULL =
+ *   zeros) -> dhx (dcx), dws / dbs shaped and ordered like ws / bs (C-contiguous), dxs[t] [B_t, in].
+ *   Equal to the routine composition / its autograd gradients to float32 tolerance (sums in another order).  One-direction LSTM
+ *   inference runs hipcx_n_step_lstm. */
+size_t hipcx_n_step_rnn_reserve_size(int n_layers, int bidirectional, int mode, const hipcx_array* hx, const hipcx_array* const* xs, int n_steps);
+size_t hipcx_n_step_rnn_workspace_size(int n_layers, int bidirectional, int mode, int training, const hipcx_array* hx, const hipcx_array* const* xs,
+                                       int n_steps);
+int hipcx_n_step_rnn(int n_layers, int bidirectional, int mode, int activation, const hipcx_array* hx, const hipcx_array* cx,
+                     const hipcx_array* const* ws, const hipcx_array* const* bs, const hipcx_array* const* xs, int n_steps, const hipcx_array* hy,
+                     const hipcx_array* cy, const hipcx_array* const* ys, void* reserve, size_t reserve_bytes, void* workspace,
+                     size_t workspace_bytes, void* stream);
+int hipcx_n_step_rnn_backward(int n_layers, int bidirectional, int mode, int activation, const hipcx_array* hx, const hipcx_array* const* ws,
+                              const hipcx_array* const* bs, const hipcx_array* const* xs, int n_steps, const hipcx_array* dhy,
+                              const hipcx_array* dcy, const hipcx_array* const* dys, const void* reserve, size_t reserve_bytes,
+                              const hipcx_array* dhx, const hipcx_array* dcx, const hipcx_array* const* dws, const hipcx_array* const* dbs,
+                              const hipcx_array* const* dxs, void* workspace, size_t workspace_bytes, void* stream);
 size_t hipcx_log_softmax_workspace_size(const hipcx_array* x);
 int hipcx_log_softmax(const hipcx_array* x, const hipcx_array* out, void* workspace, size_t workspace_bytes, void* stream);
 int hipcx_lstm_cell(const hipcx_array* c, const hipcx_array* x, const hipcx_array* h_out, const hipcx_array* c_out, void* stream);

@@ -181,3 +181,112 @@ def test_n_step_lstm_kernel_entry_views_and_errors():
     h16 = chx.array(hx.astype(np.float16))
     assert _lib.load().hipcx_n_step_lstm_workspace_size(2, h16.desc(), px, len(X)) == 0
     assert _lib.load().hipcx_n_step_lstm_workspace_size(2, HX.desc(), px, len(X)) > 0
+
+
+def _oracle_forward(kind, n_layers, bidirectional, activation, hx, cx, ws, bs, xs):
+    """(hy, cy or None, ys) of the oracle's routine composition for one family member."""
+    if kind == 'lstm':
+        return (O.n_step_bilstm if bidirectional else O.n_step_lstm)(n_layers, hx, cx, ws, bs, xs)
+    if kind == 'gru':
+        hy, ys = (O.n_step_bigru if bidirectional else O.n_step_gru)(n_layers, hx, ws, bs, xs)
+    else:
+        hy, ys = (O.n_step_birnn if bidirectional else O.n_step_rnn)(n_layers, hx, ws, bs, xs, activation)
+    return hy, None, ys
+
+
+@pytest.mark.parametrize('kind,n_layers,bidirectional,activation', CASES + [('gru', 3, False, None), ('rnn', 3, True, 'relu')])
+def test_rnn_kernel_forward_matches_oracle(kind, n_layers, bidirectional, activation):
+    """hipcx_n_step_rnn (RnnKernel, CX/kernels/rnn.h:34-49) in every mode and direction against the oracle's routine composition:
+    inference and training (reserve kept) give the same outputs; ragged and non-monotonic step batches; odd sizes."""
+    import chainer_amd as chx
+    rng = np.random.default_rng(21)
+    for in_size, units, lengths in [(4, 3, (5, 3, 3, 1)), (40, 64, (6,) * 8), (17, 33, (4, 2)), (23, 9, (7,) * 66 + (2,) * 5)]:
+        ws, bs, seqs, xs, hx, cx = _rnn_problem(rng, kind, n_layers, bidirectional, in_size, units, lengths)
+        if units == 9 and not bidirectional:  # step batches that grow again (the routine only asks for batch <= state rows)
+            xs = [xs[0][:5], xs[1], xs[2][:1], xs[3]]
+        W, B, X, HX, CX = _upload(chx, ws, bs, xs, hx, cx)
+        hy_ref, cy_ref, ys_ref = _oracle_forward(kind, n_layers, bidirectional, activation, hx, cx, ws, bs, xs)
+        what = '%s layers=%d bi=%s act=%s in=%d units=%d' % (kind, n_layers, bidirectional, activation, in_size, units)
+        for training in (False, True):
+            (hy, cy), ys, state = chx.rnn(n_layers, HX, CX if kind == 'lstm' else None, W, B, X, bidirectional, kind, activation, training)
+            assert (state is not None) == training
+            assert_close(hy.get(), hy_ref, 2e-5, 'hy %s training=%s' % (what, training))
+            if kind == 'lstm':
+                assert_close(cy.get(), cy_ref, 2e-5, 'cy ' + what)
+            else:
+                assert cy is None
+            assert len(ys) == len(ys_ref)
+            for t, (y, r) in enumerate(zip(ys, ys_ref)):
+                assert_close(y.get(), r, 2e-5, 'ys[%d] %s' % (t, what))
+        np.testing.assert_array_equal(HX.get(), hx)  # the inputs are left alone
+
+
+@pytest.mark.parametrize('kind,n_layers,bidirectional,activation', CASES)
+def test_rnn_backward_kernel_matches_finite_differences(kind, n_layers, bidirectional, activation):
+    """hipcx_n_step_rnn_backward (RnnBackwardKernel, CX/kernels/rnn.h:51-66) against central differences of the oracle's forward
+    composition in float64: with loss = <hy, dhy> + <cy, dcy> + sum_t <ys[t], dys[t]>, every entry of dhx, dcx, dws, dbs and dxs is
+    the derivative of the loss by the matching input entry.  Ragged batches (rows whose sequence has ended carry their state and its
+    gradient), one dys entry and dcy absent (zeros)."""
+    import chainer_amd as chx
+    rng = np.random.default_rng(31 + n_layers)
+    in_size, units, lengths = 4, 3, (5, 3, 3, 1)
+    ws, bs, seqs, xs, hx, cx = _rnn_problem(rng, kind, n_layers, bidirectional, in_size, units, lengths)
+    if activation == 'relu':  # keep the pre-activations away from the kink, where a central difference is not the derivative
+        bs = [[b + np.float32(0.5) * np.sign(b) for b in group] for group in bs]
+    d = 2 if bidirectional else 1
+    dhy = rng.standard_normal(hx.shape).astype(np.float32)
+    dcy = rng.standard_normal(hx.shape).astype(np.float32) if n_layers == 1 else None
+    dys = [rng.standard_normal((x.shape[0], d * units)).astype(np.float32) for x in xs]
+    dys[1] = None
+    W, B, X, HX, CX = _upload(chx, ws, bs, xs, hx, cx)
+    _, _, state = chx.rnn(n_layers, HX, CX if kind == 'lstm' else None, W, B, X, bidirectional, kind, activation, True)
+    (dhx, dcx), dws, dbs, dxs = chx.rnn_backward(state, chx.array(dhy), chx.array(dcy) if dcy is not None else None,
+                                                 [chx.array(g) if g is not None else None for g in dys])
+
+    f64 = lambda a: np.asarray(a, np.float64)
+    p_hx, p_cx = f64(hx), f64(cx)
+    p_ws, p_bs = [[f64(m) for m in g] for g in ws], [[f64(v) for v in g] for g in bs]
+    p_xs = [f64(x) for x in xs]
+
+    def loss():
+        hy, cy, ys = _oracle_forward(kind, n_layers, bidirectional, activation, p_hx, p_cx, p_ws, p_bs, p_xs)
+        total = float((hy * dhy).sum())
+        if kind == 'lstm' and dcy is not None:
+            total += float((cy * dcy).sum())
+        return total + sum(float((y * g).sum()) for y, g in zip(ys, dys) if g is not None)
+
+    def numeric(a):
+        g = np.zeros(a.shape)
+        eps = 1e-6
+        for i in np.ndindex(*a.shape):
+            keep = a[i]
+            a[i] = keep + eps
+            up = loss()
+            a[i] = keep - eps
+            down = loss()
+            a[i] = keep
+            g[i] = (up - down) / (2 * eps)
+        return g
+
+    what = '%s layers=%d bi=%s act=%s' % (kind, n_layers, bidirectional, activation)
+
+    def check(got, want, name):
+        got = got.get().astype(np.float64)
+        assert got.shape == want.shape, name
+        scale = max(np.abs(want).max(), 1.0)
+        assert np.abs(got - want).max() <= 2e-4 * scale, '%s %s: max error %.3g (scale %.3g)' % (name, what, np.abs(got - want).max(), scale)
+
+    check(dhx, numeric(p_hx), 'dhx')
+    if kind == 'lstm':
+        check(dcx, numeric(p_cx), 'dcx')
+    else:
+        assert dcx is None
+    flat_w = [m for g in p_ws for m in g]
+    flat_b = [v for g in p_bs for v in g]
+    assert len(dws) == len(flat_w) and len(dbs) == len(flat_b)
+    for i, (g, a) in enumerate(zip(dws, flat_w)):
+        check(g, numeric(a), 'dws[%d]' % i)
+    for i, (g, a) in enumerate(zip(dbs, flat_b)):
+        check(g, numeric(a), 'dbs[%d]' % i)
+    for t, (g, a) in enumerate(zip(dxs, p_xs)):
+        check(g, numeric(a), 'dxs[%d]' % t)
