@@ -1074,6 +1074,13 @@ void CheckConv(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b,
 }  // namespace
 }  // namespace hipcx
 
+namespace hipcx {
+// nd_ops.hip: arrays without exactly two spatial axes
+size_t ConvNdWorkspaceSize(const hipcx_array* x, const hipcx_array* w, const hipcx_array* out);
+void ConvNd(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, const int64_t* stride, const int64_t* pad, int cover_all,
+            const hipcx_array* out, void* workspace, size_t workspace_bytes, void* stream);
+}  // namespace hipcx
+
 using namespace hipcx;
 
 extern "C" {
@@ -1126,8 +1133,14 @@ int hipcx_profile_records(int64_t capacity, double* ms, double* flops, double* b
 }
 
 size_t hipcx_conv_workspace_size(const hipcx_array* x, const hipcx_array* w, const hipcx_array* out) {
-    (void)out;
-    if (x == nullptr || w == nullptr || x->ndim != 4 || w->ndim != 4) return 0;
+    if (x == nullptr || w == nullptr) return 0;
+    if (x->ndim != 4 || w->ndim != 4) {
+        try {
+            return x->ndim >= 2 ? ConvNdWorkspaceSize(x, w, out) : 0;
+        } catch (...) {
+            return 0;
+        }
+    }
     try {
         // the staging decision does not depend on stride/pad except for the sub-sampled 1x1 case, which needs less;
         // report the full-plane size
@@ -1159,6 +1172,10 @@ int hipcx_conv_route(const hipcx_array* x, const hipcx_array* w, const hipcx_arr
 int hipcx_conv(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, const int64_t* stride, const int64_t* pad,
                int cover_all, const hipcx_array* out, void* workspace, size_t workspace_bytes, void* stream) {
     return Guard([&] {
+        if (x != nullptr && x->ndim != 4) {  // not two spatial axes: nd_ops.hip
+            ConvNd(x, w, b, stride, pad, cover_all, out, workspace, workspace_bytes, stream);
+            return;
+        }
         CheckConv(x, w, b, stride, pad, cover_all, out);
         if (TotalSize(out) == 0) return;
         hipStream_t st = AsStream(stream);

@@ -927,6 +927,12 @@ void RunPoolGrad(const PoolGradArgs& p, hipStream_t stream) {
 }  // namespace
 }  // namespace hipcx
 
+namespace hipcx {
+// nd_ops.hip: arrays without exactly two spatial axes
+void PoolNd(bool is_max, const hipcx_array* x, const int64_t* ksize, const int64_t* stride, const int64_t* pad, int cover_all, int pad_mode,
+            const hipcx_array* out, void* stream);
+}  // namespace hipcx
+
 using namespace hipcx;
 
 extern "C" {
@@ -934,6 +940,10 @@ extern "C" {
 int hipcx_max_pool(const hipcx_array* x, const int64_t* kernel_size, const int64_t* stride, const int64_t* pad, int cover_all,
                    const hipcx_array* out, void* stream) {
     return Guard([&] {
+        if (x != nullptr && x->ndim != 4) {
+            PoolNd(true, x, kernel_size, stride, pad, cover_all, HIPCX_PAD_ZERO, out, stream);
+            return;
+        }
         PoolArgs p = MakeArgs(x, kernel_size, stride, pad, cover_all, out);
         VisitDtype(x->dtype, [&](auto tag) {
             using T = typename decltype(tag)::type;
@@ -947,6 +957,10 @@ int hipcx_average_pool(const hipcx_array* x, const int64_t* kernel_size, const i
     return Guard([&] {
         HIPCX_REQUIRE(pad_mode == HIPCX_PAD_ZERO || pad_mode == HIPCX_PAD_IGNORE, HIPCX_CHAINERX_ERROR, "invalid pad mode");
         HIPCX_REQUIRE(x != nullptr && IsFloatDtype(x->dtype), HIPCX_DTYPE_ERROR, "cannot apply average pooling to non-float arrays");
+        if (x->ndim != 4) {
+            PoolNd(false, x, kernel_size, stride, pad, 0, pad_mode, out, stream);
+            return;
+        }
         PoolArgs p = MakeArgs(x, kernel_size, stride, pad, 0, out);
         p.pad_mode = pad_mode;
         VisitFloatDtype(x->dtype, [&](auto tag) {

@@ -730,21 +730,27 @@ public:
     Array Call(const Array& x, const Array& w, const absl::optional<Array>& b, const Dims& stride, const Dims& pad, bool cover_all,
                Dtype out_dtype, const absl::optional<Array>& out) override {
         if (out.has_value()) throw NotImplementedError{"Passing out as an argument is not yet supported."};  // like native conv.cc:52-55
-        if (x.ndim() != 4) throw NotImplementedError{"hip conv supports 2 spatial dimensions."};
+        // any number of spatial axes, like the native kernel (native_device/conv.cc:57-61); the library's dedicated kernels are 2-D
+        if (x.ndim() < 2 || w.ndim() != x.ndim()) throw DimensionError{"Mismatched number of dimensions in input and weights."};
         Device& device = x.device();
         device.CheckDevicesCompatible(x, w);
         if (b.has_value()) device.CheckDevicesCompatible(*b);
         SetDeviceScope scope{device.index()};
-        Shape out_shape{x.shape()[0], w.shape()[0], OutDim(x.shape()[2], w.shape()[2], stride[0], pad[0], cover_all),
-                        OutDim(x.shape()[3], w.shape()[3], stride[1], pad[1], cover_all)};
+        const int8_t n = x.ndim() - 2;
+        Shape out_shape{x.shape()[0], w.shape()[0]};
+        std::vector<int64_t> st, pd;
+        for (int8_t d = 0; d < n; ++d) {
+            out_shape.emplace_back(OutDim(x.shape()[2 + d], w.shape()[2 + d], stride[d], pad[d], cover_all));
+            st.push_back(stride[d]);
+            pd.push_back(pad[d]);
+        }
         Array y = Empty(out_shape, out_dtype, device);  // C-contiguous NCHW, like cuda/cuda_conv.cc:311
         Array xc = Cast(x, out_dtype), wc = Cast(w, out_dtype);
         hipcx_array cx = ToC(xc), cw = ToC(wc), cy = ToC(y), cb{};
         if (b.has_value()) cb = ToC(Cast(*b, out_dtype));
-        int64_t st[2] = {stride[0], stride[1]}, pd[2] = {pad[0], pad[1]};
         size_t ws_bytes = hipcx_conv_workspace_size(&cx, &cw, &cy);
         std::shared_ptr<void> ws = device.Allocate(ws_bytes);
-        Check(hipcx_conv(&cx, &cw, b.has_value() ? &cb : nullptr, st, pd, cover_all ? 1 : 0, &cy, ws.get(), ws_bytes, nullptr));
+        Check(hipcx_conv(&cx, &cw, b.has_value() ? &cb : nullptr, st.data(), pd.data(), cover_all ? 1 : 0, &cy, ws.get(), ws_bytes, nullptr));
         return y;
     }
 };
@@ -797,9 +803,13 @@ private:
 };
 
 Shape PoolOutShape(const Array& x, const Dims& k, const Dims& s, const Dims& p, bool cover_all) {
-    if (x.ndim() != 4) throw NotImplementedError{"hip pooling supports 2 spatial dimensions."};
-    return Shape{x.shape()[0], x.shape()[1], OutDim(x.shape()[2], k[0], s[0], p[0], cover_all), OutDim(x.shape()[3], k[1], s[1], p[1], cover_all)};
+    if (x.ndim() < 3) throw DimensionError{"pooling needs at least one spatial axis."};
+    Shape out_shape{x.shape()[0], x.shape()[1]};
+    for (int8_t d = 0; d < x.ndim() - 2; ++d) out_shape.emplace_back(OutDim(x.shape()[2 + d], k[d], s[d], p[d], cover_all));
+    return out_shape;
 }
+
+std::vector<int64_t> ToVector(const Dims& dims) { return std::vector<int64_t>(dims.begin(), dims.end()); }
 
 class HipMaxPoolKernel : public MaxPoolKernel {
 public:
@@ -810,8 +820,8 @@ public:
         SetDeviceScope scope{device.index()};
         Array y = Empty(PoolOutShape(x, kernel_size, stride, pad, cover_all), x.dtype(), device);
         hipcx_array cx = ToC(x), cy = ToC(y);
-        int64_t k[2] = {kernel_size[0], kernel_size[1]}, s[2] = {stride[0], stride[1]}, p[2] = {pad[0], pad[1]};
-        Check(hipcx_max_pool(&cx, k, s, p, cover_all ? 1 : 0, &cy, nullptr));
+        std::vector<int64_t> k = ToVector(kernel_size), s = ToVector(stride), p = ToVector(pad);
+        Check(hipcx_max_pool(&cx, k.data(), s.data(), p.data(), cover_all ? 1 : 0, &cy, nullptr));
         std::unique_ptr<MaxPoolGradState> state = return_state ? std::make_unique<HipMaxPoolGradState>(x, cover_all) : nullptr;
         return std::make_tuple(std::move(y), std::move(state));
     }
@@ -828,9 +838,9 @@ public:
         SetDeviceScope scope{device.index()};
         Array y = Empty(PoolOutShape(x, kernel_size, stride, pad, false), x.dtype(), device);
         hipcx_array cx = ToC(x), cy = ToC(y);
-        int64_t k[2] = {kernel_size[0], kernel_size[1]}, s[2] = {stride[0], stride[1]}, p[2] = {pad[0], pad[1]};
+        std::vector<int64_t> k = ToVector(kernel_size), s = ToVector(stride), p = ToVector(pad);
         int mode = pad_mode == AveragePoolPadMode::kZero ? HIPCX_PAD_ZERO : HIPCX_PAD_IGNORE;
-        Check(hipcx_average_pool(&cx, k, s, p, mode, &cy, nullptr));
+        Check(hipcx_average_pool(&cx, k.data(), s.data(), p.data(), mode, &cy, nullptr));
         std::unique_ptr<AveragePoolGradState> state = return_state ? std::make_unique<HipAveragePoolGradState>(x) : nullptr;
         return std::make_tuple(std::move(y), std::move(state));
     }

@@ -1091,18 +1091,19 @@ def _spatial_out(x, n, c, h, w, dtype):
 
 
 def conv(x, w, b=None, stride=1, pad=0, cover_all=False, out_dtype=None):
-    """Conv (CX/routines/connection.cc:140-208), 2-D only: one ConvKernel call with the bias inside."""
-    if x.ndim != 4 or w.ndim != 4:
-        raise _lib.ChainerxNotImplementedError('only 2-D convolution is on the supported path')
-    stride, pad = _pair(stride), _pair(pad)
+    """Conv (CX/routines/connection.cc:140-208): one ConvKernel call with the bias inside.  Any number of spatial axes; the
+    dedicated kernels are the 2-D ones (0 and 1 axes run through them as extents of one, 3 and more through a plain kernel)."""
+    if x.ndim < 2 or w.ndim != x.ndim:
+        raise _lib.DimensionError('Mismatched number of dimensions in input %r and weights %r.' % (x.shape, w.shape))
+    n = x.ndim - 2
+    stride, pad = _pair(stride, n), _pair(pad, n)
     if w.shape[1] != x.shape[1]:
         raise _lib.DimensionError('Mismatched number of input channels in input %r and weights %r.' % (x.shape, w.shape))
     if b is not None and (b.ndim != 1 or b.shape[0] != w.shape[0]):
         raise _lib.DimensionError('Mismatched bias shape %r for weights %r.' % (b.shape, w.shape))
     dt = numpy.dtype(out_dtype) if out_dtype is not None else (result_type(x, w, b) if b is not None else result_type(x, w))
-    oh = conv_out_dim(x.shape[2], w.shape[2], stride[0], pad[0], cover_all)
-    ow = conv_out_dim(x.shape[3], w.shape[3], stride[1], pad[1], cover_all)
-    out = _spatial_out(x, x.shape[0], w.shape[0], oh, ow, dt)
+    dims = tuple(conv_out_dim(x.shape[2 + d], w.shape[2 + d], stride[d], pad[d], cover_all) for d in range(n))
+    out = _spatial_out(x, x.shape[0], w.shape[0], dims[0], dims[1], dt) if n == 2 else ndarray.empty((x.shape[0], w.shape[0]) + dims, dt)
     xc, wc = x.astype(dt, False), w.astype(dt, False)
     bc = b.astype(dt, False) if b is not None else None
     nbytes = _lib.load().hipcx_conv_workspace_size(xc.desc(), wc.desc(), out.desc())
@@ -1183,32 +1184,32 @@ def _dense_strides_like(x):
 
 
 def max_pool(x, ksize, stride=None, pad=0, cover_all=False):
-    """MaxPool (CX/routines/pooling.cc:52-123), 2-D."""
-    if x.ndim != 4:
-        raise _lib.ChainerxNotImplementedError('only 2-D pooling is on the supported path')
-    ksize = _pair(ksize)
-    stride = ksize if stride is None else _pair(stride)
-    pad = _pair(pad)
-    oh = conv_out_dim(x.shape[2], ksize[0], stride[0], pad[0], cover_all)
-    ow = conv_out_dim(x.shape[3], ksize[1], stride[1], pad[1], cover_all)
-    out = _spatial_out(x, x.shape[0], x.shape[1], oh, ow, x.dtype)
+    """MaxPool (CX/routines/pooling.cc:52-123); one or more spatial axes (the dedicated kernels are the 2-D ones)."""
+    if x.ndim < 3:
+        raise _lib.DimensionError('pooling needs at least one spatial axis, got the shape %r' % (x.shape,))
+    n = x.ndim - 2
+    ksize = _pair(ksize, n)
+    stride = ksize if stride is None else _pair(stride, n)
+    pad = _pair(pad, n)
+    dims = tuple(conv_out_dim(x.shape[2 + d], ksize[d], stride[d], pad[d], cover_all) for d in range(n))
+    out = _spatial_out(x, x.shape[0], x.shape[1], dims[0], dims[1], x.dtype) if n == 2 else ndarray.empty(x.shape[:2] + dims, x.dtype)
     _lib.call('hipcx_max_pool', x.desc(), _i64(ksize), _i64(stride), _i64(pad), int(bool(cover_all)), out.desc(), current_stream())
     return out
 
 
 def average_pool(x, ksize, stride=None, pad=0, pad_mode='ignore'):
-    """AveragePool (CX/routines/pooling.cc:125-169), 2-D, float dtypes only."""
+    """AveragePool (CX/routines/pooling.cc:125-169), float dtypes only; one or more spatial axes."""
     if _kind(x.dtype) != 3:
         raise _lib.DtypeError('cannot apply average pooling to non-float arrays')
-    if x.ndim != 4:
-        raise _lib.ChainerxNotImplementedError('only 2-D pooling is on the supported path')
-    ksize = _pair(ksize)
-    stride = ksize if stride is None else _pair(stride)
-    pad = _pair(pad)
+    if x.ndim < 3:
+        raise _lib.DimensionError('pooling needs at least one spatial axis, got the shape %r' % (x.shape,))
+    n = x.ndim - 2
+    ksize = _pair(ksize, n)
+    stride = ksize if stride is None else _pair(stride, n)
+    pad = _pair(pad, n)
     mode = {'zero': 1, 'ignore': 2}[pad_mode]
-    oh = conv_out_dim(x.shape[2], ksize[0], stride[0], pad[0], False)
-    ow = conv_out_dim(x.shape[3], ksize[1], stride[1], pad[1], False)
-    out = _spatial_out(x, x.shape[0], x.shape[1], oh, ow, x.dtype)
+    dims = tuple(conv_out_dim(x.shape[2 + d], ksize[d], stride[d], pad[d], False) for d in range(n))
+    out = _spatial_out(x, x.shape[0], x.shape[1], dims[0], dims[1], x.dtype) if n == 2 else ndarray.empty(x.shape[:2] + dims, x.dtype)
     _lib.call('hipcx_average_pool', x.desc(), _i64(ksize), _i64(stride), _i64(pad), mode, out.desc(), current_stream())
     return out
 

@@ -291,8 +291,10 @@ int hipcx_dot(const hipcx_array* a, const hipcx_array* b, const hipcx_array* out
               void* stream);
 /* Output extent of a convolution/pooling window (CX/routines/connection.cc:37-49). Returns -1 if not positive. */
 int64_t hipcx_conv_out_dim(int64_t in_dim, int64_t kernel_size, int64_t stride, int64_t pad, int cover_all);
-/* 2-D convolution forward, x[N,C,H,W] (any strides), w[K,C,kh,kw], optional b[K] (NULL = none),
- * out[N,K,OH,OW] with any strides.  The plugin and the Python mirror allocate out C-contiguous (NCHW memory), like the CUDA
+/* Convolution forward (ConvKernel CX/kernels/connection.h:14-32), x[N,C,H,W] (any strides), w[K,C,kh,kw], optional b[K] (NULL = none),
+ * out[N,K,OH,OW] with any strides.  Other ranks, like the native kernel (CX/native/native_device/conv.cc:57-89): x[N,C,d_1..d_n] with
+ * w[K,C,k_1..k_n], `stride` and `pad` holding n values; n = 0 and 1 run the 2-D kernels over extents of one, n >= 3 a plain
+ * one-thread-per-output kernel (a correctness path: float accumulation for float16, bias added after rounding, as the native backend).  The plugin and the Python mirror allocate out C-contiguous (NCHW memory), like the CUDA
  * backend (CX/cuda/cuda_conv.cc:311); the native backend's own result is an NCHW view of NHWC memory
  * (CX/native/native_device/conv.cc:78-84), which this entry also accepts as `out`. */
 size_t hipcx_conv_workspace_size(const hipcx_array* x, const hipcx_array* w, const hipcx_array* out);
@@ -491,7 +493,9 @@ int hipcx_batch_norm_grad(const hipcx_array* x, const hipcx_array* gamma, const 
                           const hipcx_array* inv_std, const int8_t* axis, int naxis, const hipcx_array* gx, const hipcx_array* ggamma,
                           const hipcx_array* gbeta, void* workspace, size_t workspace_bytes, void* stream);
 
-/* ---- pooling: CX/kernels/pooling.h:29,83 (2-D, NCHW logical layout, any strides) ---- */
+/* ---- pooling: CX/kernels/pooling.h:29,83 (NCHW logical layout, any strides; x[N,C,d_1..d_n] with n values per window parameter:
+ * the dedicated kernels are the 2-D ones, n = 1 runs them over an extent of one, n >= 3 a plain one-thread-per-output kernel with
+ * the native backend's arithmetic, CX/native/native_device/pool.cc:69-94,191-302) ---- */
 int hipcx_max_pool(const hipcx_array* x, const int64_t* kernel_size, const int64_t* stride, const int64_t* pad, int cover_all,
                    const hipcx_array* out, void* stream);
 int hipcx_average_pool(const hipcx_array* x, const int64_t* kernel_size, const int64_t* stride, const int64_t* pad, int pad_mode,

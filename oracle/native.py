@@ -746,6 +746,80 @@ def fixed_batch_norm(x, gamma, beta, mean, var, eps=2e-5, axis=None):
     return out.astype(x.dtype)
 
 
+def _tuple_n(v, n):
+    if isinstance(v, (int, np.integer)):
+        return (int(v),) * n
+    v = tuple(int(i) for i in v)
+    assert len(v) == n, (v, n)
+    return v
+
+
+def _windows_nd(x, ksize, stride, pad, cover_all, pad_value):
+    """Im2Col over n spatial axes (CX/native/im2col.cc:82-149): [N, C, k_1..k_n, o_1..o_n]; the padded copy of x is filled with
+    `pad_value` (cover_all adds stride - 1 more on the high side) and one strided view per kernel offset is copied out."""
+    n = x.ndim - 2
+    out_dims = tuple(conv_out_dim(x.shape[2 + d], ksize[d], stride[d], pad[d], cover_all) for d in range(n))
+    padded_shape = x.shape[:2] + tuple(x.shape[2 + d] + 2 * pad[d] + (stride[d] - 1 if cover_all else 0) for d in range(n))
+    padded = np.full(padded_shape, pad_value, x.dtype)
+    padded[(slice(None), slice(None)) + tuple(slice(pad[d], pad[d] + x.shape[2 + d]) for d in range(n))] = x
+    col = np.empty(x.shape[:2] + tuple(ksize) + out_dims, x.dtype)
+    for kidx in np.ndindex(*ksize):
+        src = (slice(None), slice(None)) + tuple(slice(kidx[d], kidx[d] + stride[d] * out_dims[d], stride[d]) for d in range(n))
+        col[(slice(None), slice(None)) + kidx] = padded[src]
+    return col
+
+
+def conv_nd(x, w, b=None, stride=1, pad=0, cover_all=False):
+    """NativeConvKernel for any number of spatial axes (conv.cc:41-89): Im2Col, TensorDot(col, w) over (channel, k_1..k_n) --
+    native Dot, float16 accumulating in float -- then `y += b` in the array dtype, then the channel axis moved to position 1."""
+    x, w = np.asarray(x), np.asarray(w)
+    assert x.dtype == w.dtype and x.ndim == w.ndim and x.shape[1] == w.shape[1]
+    n = x.ndim - 2
+    stride, pad = _tuple_n(stride, n), _tuple_n(pad, n)
+    col = _windows_nd(x, w.shape[2:], stride, pad, cover_all, 0)
+    axes = tuple(range(1, n + 2))
+    y = _tensordot(col, w, axes, axes)  # [N, o_1..o_n, K]
+    if b is not None:
+        y = add(y, np.broadcast_to(np.asarray(b).astype(y.dtype), y.shape))
+    return np.ascontiguousarray(np.moveaxis(y, -1, 1))
+
+
+def max_pool_nd(x, ksize, stride=None, pad=0, cover_all=False):
+    """NativeMaxPoolKernel over n spatial axes (pool.cc:69-94): Im2Col padded with the lowest value, AMax over the kernel axes."""
+    x = np.asarray(x)
+    n = x.ndim - 2
+    ksize = _tuple_n(ksize, n)
+    stride = ksize if stride is None else _tuple_n(stride, n)
+    col = _windows_nd(x, ksize, stride, _tuple_n(pad, n), cover_all, _lowest(x.dtype))
+    return amax(col, tuple(range(2, 2 + n)))
+
+
+def average_pool_nd(x, ksize, stride=None, pad=0, pad_mode='ignore'):
+    """NativeAveragePoolKernel over n spatial axes (pool.cc:191-302): zero-padded Im2Col, Sum over the kernel axes (an array of the
+    input dtype), divided by the window size ('zero') or by the number of window positions inside the array ('ignore'): the outer
+    product of the per-axis widths, built in the array dtype."""
+    x = np.asarray(x)
+    n = x.ndim - 2
+    ksize = _tuple_n(ksize, n)
+    stride = ksize if stride is None else _tuple_n(stride, n)
+    pad = _tuple_n(pad, n)
+    col = _windows_nd(x, ksize, stride, pad, False, 0)
+    s = sum(col, tuple(range(2, 2 + n)))
+    if pad_mode == 'zero':
+        with np.errstate(all='ignore'):
+            return (s / _scalar_as(int(np.prod(ksize)), x.dtype)).astype(x.dtype)
+    widths = None
+    for i in range(n):
+        d, k, st, p = x.shape[2 + i], ksize[i], stride[i], pad[i]
+        n_out = conv_out_dim(d, k, st, p, False)
+        start = np.arange(n_out).astype(x.dtype) * _scalar_as(st, x.dtype) - _scalar_as(p, x.dtype)
+        end = start + _scalar_as(k, x.dtype)
+        w = (np.minimum(end, _scalar_as(d, x.dtype)) - np.maximum(start, _scalar_as(0, x.dtype))).astype(x.dtype)
+        widths = w if widths is None else (widths[..., None] * w).astype(x.dtype)
+    with np.errstate(all='ignore'):
+        return (s / widths).astype(x.dtype)
+
+
 def _windows(x, ksize, stride, pad, cover_all, pad_value):
     """Im2Col (CX/native/im2col.cc:82-149): [N,C,kh,kw,OH,OW] with `pad_value` outside the image."""
     N, C, H, W = x.shape

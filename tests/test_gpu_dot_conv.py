@@ -295,3 +295,53 @@ def test_conv1x1_float16_lds_direct_ring():
     # the general kernels keep the shapes the plan leaves out
     small = chx.array(rng.standard_normal((2, 64, 14, 14)).astype('float16'))
     assert routines.conv_route(small, chx.array(w[:256, :64])) != 3
+
+
+@pytest.mark.parametrize('cover_all', [False, True])
+def test_conv_and_pooling_over_n_axes_reference_grid(cover_all):
+    """The rows of the reference's grids that are not 2-D (test_connection.py:178-203: 0, 1 and 3 spatial axes; test_pooling.py:15-27:
+    1, 3 and 4) and the 2-D ones through the same entry points, against the oracle's n-axis restatements; dense and padded
+    (non-contiguous) inputs, with and without bias, both pad modes, NaN / inf in pooling windows, larger 3-D cases."""
+    import chainer_amd as chx
+    from test_oracle_pins import CONV_ND_GRID, POOL_ND_GRID
+    rng = np.random.default_rng(17)
+    conv_cases = CONV_ND_GRID + [((2, 8, 5, 9, 7), (6, 8, 3, 3, 3), 1, 1), ((3, 4, 6, 6, 6), (5, 4, 2, 3, 1), (2, 1, 2), (0, 1, 0)),
+                                 ((4, 16, 40), (8, 16, 5), 2, 2), ((5, 32), (7, 32), 1, 0)]
+    for dt, tol in DT:
+        for xs, ws, stride, pad in conv_cases:
+            x = rng.standard_normal(xs).astype(dt)
+            w = (rng.standard_normal(ws) / np.sqrt(np.prod(ws[1:]))).astype(dt)
+            b = rng.standard_normal(ws[0]).astype(dt)
+            what = 'conv %s %r' % (dt, (xs, ws, stride, pad, cover_all))
+            for bias in (None, b):
+                ref = O.conv_nd(x, w, bias, stride, pad, cover_all)
+                y = chx.conv(chx.array(x), chx.array(w), chx.array(bias) if bias is not None else None, stride, pad, cover_all)
+                assert y.shape == ref.shape and y.dtype == ref.dtype, what
+                assert_close(y.get(), ref, tol, what)
+            if len(xs) > 2:
+                xp = padded(xs, x, 1, dt)
+                y = chx.conv(upload_view(chx, xp), chx.array(w), chx.array(b), stride, pad, cover_all)
+                assert_close(y.get(), O.conv_nd(x, w, b, stride, pad, cover_all), tol, what + ' (padded x)')
+        pool_cases = POOL_ND_GRID + [((2, 5, 6, 7, 8), (3, 2, 3), (2, 1, 2), (1, 0, 1)), ((3, 4, 33), (4,), 3, 1)]
+        for xs, ks, stride, pad in pool_cases:
+            x = rng.standard_normal(xs).astype(dt)
+            what = 'pool %s %r' % (dt, (xs, ks, stride, pad, cover_all))
+            got = chx.max_pool(chx.array(x), ks, stride, pad, cover_all).get()
+            assert np.array_equal(got, O.max_pool_nd(x, ks, stride, pad, cover_all)), 'max_' + what
+            xn = x.copy()
+            xn.reshape(-1)[::7] = np.nan
+            xn.reshape(-1)[3::11] = np.inf
+            got = chx.max_pool(chx.array(xn), ks, stride, pad, cover_all).get()
+            assert np.array_equal(got, O.max_pool_nd(xn, ks, stride, pad, cover_all), equal_nan=True), 'max_' + what + ' with NaN / inf'
+            if not cover_all:
+                for mode in ('zero', 'ignore'):
+                    got, ref = chx.average_pool(chx.array(x), ks, stride, pad, mode).get(), O.average_pool_nd(x, ks, stride, pad, mode)
+                    fin = np.isfinite(ref)
+                    assert got.shape == ref.shape and np.array_equal(np.isnan(got), np.isnan(ref)), 'average_%s %s' % (what, mode)
+                    assert_close(np.where(fin, got, 0), np.where(fin, ref, 0), tol * 2, 'average_%s %s' % (what, mode))
+        xi = rng.integers(-50, 50, (2, 3, 4, 5, 6)).astype('int32')
+        assert np.array_equal(chx.max_pool(chx.array(xi), (2, 2, 3), 2, 1, cover_all).get(), O.max_pool_nd(xi, (2, 2, 3), 2, 1, cover_all))
+    with pytest.raises(chx.DimensionError):
+        chx.conv(chx.zeros((1, 3, 4, 4, 4), 'float32'), chx.zeros((2, 4, 1, 1, 1), 'float32'))
+    with pytest.raises(chx.DimensionError):
+        chx.max_pool(chx.zeros((1, 3, 2, 2, 2), 'float32'), 3, 1, 0)

@@ -732,6 +732,93 @@ def test_batch_norm_training_closed_forms():
         assert abs((loss(x, gamma, beta + e) - loss(x, gamma, beta - e)) / (2 * h) - gb[c]) <= 1e-6
 
 
+def _brute_conv_nd(x, w, b, stride, pad, cover_all):
+    """Definition of the cross-correlation, one output element at a time, float64."""
+    n = x.ndim - 2
+    od = [O.conv_out_dim(x.shape[2 + d], w.shape[2 + d], stride[d], pad[d], cover_all) for d in range(n)]
+    out = np.zeros((x.shape[0], w.shape[0]) + tuple(od))
+    for idx in np.ndindex(*out.shape):
+        nb, k, o = idx[0], idx[1], idx[2:]
+        acc = 0.0
+        for c in range(x.shape[1]):
+            for kidx in np.ndindex(*w.shape[2:]):
+                i = tuple(o[d] * stride[d] - pad[d] + kidx[d] for d in range(n))
+                if all(0 <= i[d] < x.shape[2 + d] for d in range(n)):
+                    acc += float(x[(nb, c) + i]) * float(w[(k, c) + kidx])
+        out[idx] = acc + (float(b[k]) if b is not None else 0.0)
+    return out
+
+
+def _brute_pool_nd(x, ksize, stride, pad, cover_all, kind):
+    n = x.ndim - 2
+    od = [O.conv_out_dim(x.shape[2 + d], ksize[d], stride[d], pad[d], cover_all) for d in range(n)]
+    out = np.zeros(x.shape[:2] + tuple(od))
+    for idx in np.ndindex(*out.shape):
+        vals = []
+        for kidx in np.ndindex(*ksize):
+            i = tuple(idx[2 + d] * stride[d] - pad[d] + kidx[d] for d in range(n))
+            if all(0 <= i[d] < x.shape[2 + d] for d in range(n)):
+                vals.append(float(x[idx[:2] + i]))
+        if kind == 'max':
+            out[idx] = max(vals) if vals else -np.inf
+        elif kind == 'zero':
+            out[idx] = np.sum(vals) / np.prod(ksize)
+        else:
+            # the divisor is the product of the per-axis overlaps min(start + k, extent) - max(start, 0), which the reference does not
+            # clamp at zero (CX/native/native_device/pool.cc:197-225): a window wholly outside an axis gives a negative factor
+            div = 1.0
+            for d in range(n):
+                start = idx[2 + d] * stride[d] - pad[d]
+                div *= min(start + ksize[d], x.shape[2 + d]) - max(start, 0)
+            with np.errstate(all='ignore'):
+                out[idx] = np.float64(np.sum(vals)) / div
+    return out
+
+
+# the reference's own grids: tests/chainerx_tests/unit_tests/routines_tests/test_connection.py:178-203, test_pooling.py:15-27
+CONV_ND_GRID = [((1, 3), (5, 3), 1, 0), ((1, 3, 4), (5, 3, 2), 3, 2), ((2, 3, 4), (5, 3, 1), 1, 0), ((2, 3, 4, 4), (2, 3, 3, 3), 2, (2, 0)),
+                ((1, 3, 4, 4), (2, 3, 3, 3), (1, 2), 1), ((2, 3, 2, 6, 3), (2, 3, 1, 3, 2), (1, 2, 3), (2, 0, 1)),
+                ((1, 3, 2, 6, 3), (2, 3, 1, 3, 2), 2, (2, 0, 1))]
+POOL_ND_GRID = [((2, 3, 4), (1,), 1, 0), ((1, 3, 4), (2,), 3, 2), ((2, 3, 4, 4), (3, 3), 1, 0), ((1, 3, 4, 4), (3, 3), (1, 2), 1),
+                ((1, 3, 4, 4), (3, 3), 2, (2, 0)), ((1, 3, 2, 6, 3), (1, 3, 2), 2, (2, 0, 1)), ((2, 3, 2, 6, 3), (1, 3, 2), (1, 2, 3), (2, 0, 1)),
+                ((1, 3, 2, 6, 3, 2), (1, 3, 2, 2), 2, 2)]
+
+
+def test_conv_and_pooling_over_n_axes():
+    """The restatements for any number of spatial axes: equal to the 2-D ones (pinned above) bit for bit on 2-D input, and equal to
+    the definition evaluated element by element on the reference's grids of 0-, 1-, 3- and 4-D cases (a wrong axis order in the
+    window copy, a missing cover_all row or a divisor taken over the wrong axes fails)."""
+    rng = np.random.default_rng(61)
+    tup = lambda v, n: (v,) * n if isinstance(v, int) else tuple(v)
+    for dt in ('float32', 'float16'):
+        x = rng.standard_normal((2, 3, 7, 6)).astype(dt)
+        w = rng.standard_normal((4, 3, 3, 2)).astype(dt)
+        b = rng.standard_normal(4).astype(dt)
+        for cv in (False, True):
+            assert np.array_equal(O.conv_nd(x, w, b, (2, 1), (1, 0), cv), O.conv(x, w, b, (2, 1), (1, 0), cv))
+            assert np.array_equal(O.max_pool_nd(x, (3, 2), (2, 1), (1, 0), cv), O.max_pool(x, (3, 2), (2, 1), (1, 0), cv))
+        for mode in ('zero', 'ignore'):
+            assert np.array_equal(O.average_pool_nd(x, (3, 2), (2, 1), (1, 0), mode), O.average_pool(x, (3, 2), (2, 1), (1, 0), mode), equal_nan=True)
+    for xs, ws, stride, pad in CONV_ND_GRID:
+        n = len(xs) - 2
+        x, w, b = rng.standard_normal(xs), rng.standard_normal(ws), rng.standard_normal(ws[0])
+        for cv in (False, True):
+            for bias in (None, b):
+                got = O.conv_nd(x, w, bias, stride, pad, cv)
+                want = _brute_conv_nd(x, w, bias, tup(stride, n), tup(pad, n), cv)
+                assert got.shape == want.shape and np.allclose(got, want, rtol=1e-12, atol=1e-12), (xs, ws, stride, pad, cv)
+    for xs, ks, stride, pad in POOL_ND_GRID:
+        n = len(xs) - 2
+        x = rng.standard_normal(xs)
+        for cv in (False, True):
+            got = O.max_pool_nd(x, ks, stride, pad, cv)
+            assert np.array_equal(got, _brute_pool_nd(x, ks, tup(stride, n), tup(pad, n), cv, 'max')), (xs, ks, stride, pad, cv)
+        for mode in ('zero', 'ignore'):
+            got = O.average_pool_nd(x, ks, stride, pad, mode)
+            want = _brute_pool_nd(x, ks, tup(stride, n), tup(pad, n), False, mode)
+            assert got.shape == want.shape and np.allclose(got, want, rtol=1e-12, atol=1e-12, equal_nan=True), (xs, ks, stride, pad, mode)
+
+
 def test_batch_norm_dtypes():
     """The dtype rules of GenericBatchNormKernel (CX/routines/normalization.cc:176-193, 224-246).  float16 x with float32 parameters:
     computed in float32 -- statistics, state and running values are float32 and agree with the float64 closed form to float32
