@@ -726,7 +726,7 @@ void RunNchw(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, c
 // ---- float16 1x1 / stride 1 layers on the LDS-direct ring (pw_conv.h) ----
 struct PwPlan {
     bool ok = false;
-    int wm = 2, wn = 4;
+    int wm = 2, wn = 2;  // wave grid of the workgroup: 256 pixels x 128 channels
 };
 
 PwPlan PlanPw(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, const hipcx_array* out, const int64_t* stride, const int64_t* pad) {
@@ -741,19 +741,17 @@ PwPlan PlanPw(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, 
     if (b != nullptr && b->strides[0] % 2 != 0) return pl;
     if (N * C * P * 2 >= (1LL << 31) || N * K * P * 2 >= (1LL << 31) || K * C * 2 >= (1LL << 31)) return pl;
     const int64_t PS = (P + 7) / 8 * 8;
-    // Where these kernels measured faster than the 128 x 128 tiles on ResNet-50's layers at batch 128: very wide outputs over a
-    // short reduction (256 x 256 tiles: the layer streams, and an activation tile is fetched once per 256 output channels
-    // instead of once per 128) and 128 output channels (512 x 128 tiles).  Elsewhere the smaller tiles, three workgroups to a
-    // compute unit, overlap their load, multiply and store phases better than one workgroup of eight waves does.
-    if ((K >= 1024 && C <= 256) || (K >= 256 && C <= 64)) {
-        pl.wm = 2, pl.wn = 4;
-    } else if (K > 64 && K <= 128) {
-        pl.wm = 4, pl.wn = 2;
-    } else {
-        return pl;
-    }
+    // Where these kernels measured faster than the 128 x 128 tiles on ResNet-50's layers at batch 128 (microseconds, the 128 x 128
+    // kernels first): 256 -> 1024 at 14x14 29.6 / 26.0, 128 -> 512 at 28x28 33.5 / 26.8, 512 -> 128 at 28x28 29.8 / 22.4,
+    // 64 -> 256 at 56x56 45.3 / 40.6, 512 -> 2048 at 7x7 29.9 / 25.1 -- all with four-wave workgroups on 256-pixel x 128-channel
+    // tiles, two to a compute unit, which overlap each other's load, multiply and store phases.  Deep reductions into few
+    // channels (1024 -> 256: 26.5 either way; 2048 -> 512 and 256 -> 64: slower) stay with the 128 x 128 tiles and their split
+    // reduction.  The eight-wave variants (one workgroup per unit, 256 x 256 or 512 x 128 tiles) measured between the two.
+    if (!((K >= 256 && C <= 512) || (K > 64 && K <= 128))) return pl;
+    pl.wm = 2, pl.wn = 2;
     const int64_t tiles = ((N * PS + 128 * pl.wm - 1) / (128 * pl.wm)) * ((K + 64 * pl.wn - 1) / (64 * pl.wn));
-    if (tiles < (NumCUs() * 3) / 4 || tiles >= (1LL << 24)) return pl;
+    const int64_t slots = pl.wm * pl.wn == 4 ? 2 * NumCUs() : NumCUs();  // workgroups resident at a time
+    if (tiles < (slots * 3) / 4 || tiles >= (1LL << 24)) return pl;
     pl.ok = true;
     return pl;
 }
@@ -765,18 +763,19 @@ void LaunchPw(PwConvArgs a, hipStream_t stream) {
     a.tiles_n = (a.K + BN - 1) / BN;
     a.total_tiles = a.tiles_m * a.tiles_n;
     constexpr int lds_bytes = PwLdsBytes<WM, WN>();
-    // workgroups walk tiles: one per compute unit (a multiple of 8, one share per XCD)
-    const unsigned grid = static_cast<unsigned>(std::min((a.total_tiles + 7) / 8 * 8, std::max(8, NumCUs() / 8 * 8)));
+    constexpr int kPerUnit = WM * WN == 4 ? 2 : 1;  // four-wave workgroups run two to a compute unit
+    // workgroups walk tiles: as many as the device holds at a time (a multiple of 8, one share per XCD)
+    const unsigned grid = static_cast<unsigned>(std::min((a.total_tiles + 7) / 8 * 8, std::max(8, kPerUnit * NumCUs() / 8 * 8)));
     if (a.P % 8 != 0) {
         auto kern = PwConvKernel<WM, WN, true>;
         struct Tag {};
         EnsureDynamicLds<Tag>(reinterpret_cast<const void*>(kern), lds_bytes);
-        hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds_bytes, stream, a);
+        hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * WM * WN), lds_bytes, stream, a);
     } else {
         auto kern = PwConvKernel<WM, WN, false>;
         struct Tag {};
         EnsureDynamicLds<Tag>(reinterpret_cast<const void*>(kern), lds_bytes);
-        hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds_bytes, stream, a);
+        hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * WM * WN), lds_bytes, stream, a);
     }
     CheckLaunch("pw_conv");
 }
@@ -800,8 +799,7 @@ void RunPw(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, con
     a.out_bytes = static_cast<unsigned>(static_cast<int64_t>(a.N) * a.K * a.P * 2);
     const double M = static_cast<double>(a.N) * a.P;
     ProfileScope prof(stream, 2.0 * M * a.K * a.C, 2.0 * (M * a.C + static_cast<double>(a.K) * a.C + M * a.K));
-    if (pl.wm == 2) LaunchPw<2, 4>(a, stream);
-    else LaunchPw<4, 2>(a, stream);
+    LaunchPw<2, 2>(a, stream);
 }
 
 // ---- float16 7x7/2 stem path (stem_conv.h) ----

@@ -5,12 +5,13 @@
 // i.e. per image the matrix product out_n [K, P] = w [K, C] . x_n [C, P] with the pixels contiguous in x and out.
 //
 // Work decomposition.  Pixels are numbered in "slots": image n owns slots [n * PS, n * PS + P) with PS = P rounded up to a
-// multiple of 8, so that a 16-byte piece of 8 consecutive slots never straddles two images.  A workgroup of eight wavefronts
-// owns a tile of BM = 128 * WM slots x BN = 64 * WN output channels (WM * WN = 8; a wave multiplies 128 slots x 64 channels
-// = 4 x 2 MFMA 32x32x16 blocks, 128 accumulator registers) and walks the input channels in chunks of 32.
+// multiple of 8, so that a 16-byte piece of 8 consecutive slots never straddles two images.  A workgroup of four wavefronts
+// owns a tile of BM = 128 * WM slots x BN = 64 * WN output channels (WM * WN = 4; a wave multiplies 128 slots x 64 channels
+// = 4 x 2 MFMA 32x32x16 blocks, 128 accumulator registers) and walks the input channels in chunks of 32.  Two workgroups run
+// on a compute unit, each on tiles of its own: while one writes a tile out, the other one loads and multiplies.
 //
 // Operands reach LDS without passing through registers: buffer loads with the LDS modifier write 16 bytes per lane,
-// 1 KiB per instruction, into a ring of three stages.
+// 1 KiB per instruction, into a ring of two stages.
 //   * activations stay as they lie in memory -- rows of pixels, one row per channel: stage[c][slot].  The MFMA operand (8
 //     consecutive channels of one pixel per lane) is gathered by transposing LDS reads (ds_read_b64_tr_b16: sixteen lanes read
 //     a 4-channel x 16-pixel block and each receives the four channels of its pixel).  16-byte piece i of channel row c is
@@ -18,11 +19,13 @@
 //     64-byte bank groups (the loading lane picks the global piece that belongs at its LDS position).
 //   * filters are read in place from the dense [K][C] bank: stage[k][4 pieces of 8 channels], piece g of row k at position
 //     g ^ ((k >> 2) & 3), read as whole MFMA operands with ds_read_b128.
-// The wavefronts form two groups of four (one wave of each group on every SIMD) that alternate between a memory phase (issue
-// the loads of the chunk after next, read the fragments of the current chunk into registers) and an MFMA phase (16 MFMAs),
-// half a period apart, separated by workgroup barriers: while one wave of a SIMD multiplies, the other one feeds.
+// Per chunk a wave issues its share of the loads of the next chunk, reads the fragments of the current chunk into
+// registers, multiplies (16 MFMAs), waits for the loads of the next chunk and meets the others at one barrier.
 // A workgroup walks several tiles (the host launches no more workgroups than the device holds): the chunk ring runs across
 // tile boundaries, so the first chunks of the next tile are on their way while the current tile is written out.
+// (An eight-wave variant -- one workgroup per compute unit on 256 x 256 or 512 x 128 tiles, its two groups of four waves
+// alternating between a memory and an MFMA phase half a period apart -- measured 2 to 7 microseconds slower per layer: all of
+// a tile's phases then run inside one workgroup.)
 //
 // Epilogue: accumulators (a lane holds 4 consecutive pixels of one channel) are rounded to float16 and regrouped through a
 // wave-private LDS area into 16-byte pieces of 8 pixels, stored with buffer stores whose out-of-range offsets drop the
@@ -33,10 +36,6 @@
 #include "common.h"
 #include "igemm.h"
 #include "nchw_conv.h"
-
-#ifndef PW_ABL
-#define PW_ABL 0
-#endif
 
 namespace hipcx {
 
@@ -79,36 +78,39 @@ __device__ __forceinline__ void PwWaitVmcnt() {
 
 constexpr int kPwStagePitch = 136;                // bytes per channel row of the epilogue's staging area (64 pixels + 8)
 constexpr int kPwStageBytes = 32 * kPwStagePitch;  // per wave: 32 channels x 64 pixels
-constexpr int kPwStages = 3;
+constexpr int kPwStages = 2;  // a ring of three measured 1 us slower per layer: two workgroups per unit already keep loads in flight
 
 constexpr int kPwMaxBiasK = 2048;                 // output channels whose bias values fit the LDS copy
 
+// The ring, the epilogue's staging areas of the four waves and the bias copy: 69 KiB for 256 x 128 tiles, two workgroups to a unit.
 template <int WM, int WN>
 constexpr int PwLdsBytes() {
-    return kPwStages * (32 * 128 * WM * 2 + 64 * WN * 64) + 8 * kPwStageBytes + kPwMaxBiasK * 2;
+    return kPwStages * (32 * 128 * WM * 2 + 64 * WN * 64) + 4 * kPwStageBytes + kPwMaxBiasK * 2;
 }
 
 // PART: P is not a multiple of 8 (the last piece of a plane is incomplete and goes out as one 8-byte store; P % 4 == 0).
 template <int WM, int WN, bool PART>
-__global__ __launch_bounds__(512) void PwConvKernel(PwConvArgs p) {
-    static_assert(WM * WN == 8, "eight wavefronts");
+__global__ __launch_bounds__(64 * WM * WN) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void PwConvKernel(PwConvArgs p) {
+    constexpr int NW = WM * WN;
+    static_assert(NW == 4, "four wavefronts");
     constexpr int BM = 128 * WM, BN = 64 * WN;
     constexpr int NSTAGE = kPwStages, AHEAD = NSTAGE - 1;
+    static_assert(AHEAD == 1, "the wait below counts no younger chunk in flight");
     constexpr int ROWX = BM * 2;          // bytes per channel row of the activation tile
     constexpr int XT_B = 32 * ROWX;       // activation tile of one chunk
     constexpr int WT_B = BN * 64;         // filter tile of one chunk
     constexpr int STAGE_B = XT_B + WT_B;
-    constexpr int LX = BM / 128, LW = BN / 128;  // load instructions per wave and chunk
+    constexpr int LX = BM / (16 * NW), LW = BN / (16 * NW);  // load instructions per wave and chunk (1 KiB each)
     constexpr int LPC = LX + LW;
     constexpr int RING_B = NSTAGE * STAGE_B;
     constexpr int NST = PART ? 32 : 16;  // store instructions per wave and tile
-    static_assert((AHEAD - 1) * LPC + NST < 64, "vmcnt range");
+    static_assert(NST < 64, "vmcnt range");
     extern __shared__ __align__(16) char lds[];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int grp = wave >> 2;
     const int wm = wave % WM, wn = wave / WM;
     const int nc = p.C / 32;
 
@@ -128,9 +130,9 @@ __global__ __launch_bounds__(512) void PwConvKernel(PwConvArgs p) {
 
     // The bias vector goes to LDS once, before the first operand load is issued: a global load in the epilogue would make the
     // compiler wait for every outstanding memory operation, the next tile's operand loads and this tile's stores included.
-    half_t* const bias_lds = reinterpret_cast<half_t*>(lds + RING_B + 8 * kPwStageBytes);
+    half_t* const bias_lds = reinterpret_cast<half_t*>(lds + RING_B + NW * kPwStageBytes);
     if (p.bias != nullptr) {
-        for (int k = tid; k < p.K; k += 512) bias_lds[k] = p.bias[k * p.bias_stride];
+        for (int k = tid; k < p.K; k += 64 * NW) bias_lds[k] = p.bias[k * p.bias_stride];
     }
 
     const pw_int4_t xr = PwRsrc(p.x, p.x_bytes);
@@ -294,13 +296,13 @@ __global__ __launch_bounds__(512) void PwConvKernel(PwConvArgs p) {
                     }
                     // the wave reads what its own lanes wrote: no barrier, the compiler's wait for the LDS writes suffices
 #pragma unroll
-                    for (int it = 0; it < ((PW_ABL & 32) ? 0 : 4); ++it) {
+                    for (int it = 0; it < 4; ++it) {
                         const int row = it * 8 + (lane >> 3);
                         const Bytes8 lo = *reinterpret_cast<const Bytes8*>(stg + row * kPwStagePitch + (lane & 7) * 16);
                         const Bytes8 hi = *reinterpret_cast<const Bytes8*>(stg + row * kPwStagePitch + (lane & 7) * 16 + 8);
                         const bool kok = k0 + j * 32 + row < p.K;
                         const int off = obase[ip] + (j * 32 + it * 8) * p.P * 2;
-                        __builtin_amdgcn_raw_buffer_store_b128(Bytes16{lo.x, lo.y, hi.x, hi.y}, orsrc, (!(PW_ABL & 1) && kok && nvalid[ip] >= 8) ? off : 0x7fffffff, 0, 0);
+                        __builtin_amdgcn_raw_buffer_store_b128(Bytes16{lo.x, lo.y, hi.x, hi.y}, orsrc, (kok && nvalid[ip] >= 8) ? off : 0x7fffffff, 0, 0);
                         if constexpr (PART) {
                             __builtin_amdgcn_raw_buffer_store_b64(lo, orsrc, (kok && nvalid[ip] >= 4 && nvalid[ip] < 8) ? off : 0x7fffffff, 0, 0);
                         }
@@ -317,64 +319,33 @@ __global__ __launch_bounds__(512) void PwConvKernel(PwConvArgs p) {
     if (!c_valid) return;  // the same for every wave of the workgroup
 #pragma unroll
     for (int a = 0; a < AHEAD; ++a) issue_next();
-    // the first chunk has landed when at most the chunks issued after it are outstanding
-    if (g_issue >= AHEAD) PwWaitVmcnt<(AHEAD - 1) * LPC>(); else PwWaitVmcnt<0>();
+    // the first chunk has landed
+    PwWaitVmcnt<0>();
     __builtin_amdgcn_s_barrier();
-    if (grp == 1) __builtin_amdgcn_s_barrier();
     int g = 0;
-    bool stores_behind = false;  // an epilogue's stores were issued after the loads of chunk g + 1
-    // The first group is half a period ahead: it keeps a finished tile in its accumulators through the memory phase of the next
-    // tile's first chunk and writes it out at the start of the following MFMA phase, when the second group writes out its part
-    // (two epilogues one after the other would leave the matrix pipes idle twice as long).
-    bool epi_pending = false;
-    int e_tm = 0, e_tn = 0;
+    // Per chunk: load the next chunk, read and multiply the current one, then wait for the next chunk and meet at one barrier.
+    // The latency this leaves exposed is covered by the second workgroup on the compute unit.
     while (c_valid) {
         __builtin_amdgcn_sched_barrier(0);
-        const bool issued = (PW_ABL & 16) ? false : issue_next();
-        if constexpr (!(PW_ABL & 8)) read_frags(g % NSTAGE);
-        // chunk g + 1 (this wave's share) must have landed before the barrier behind which it is read
-        if constexpr (!(PW_ABL & 16)) {
-        if (issued && g_issue - g == AHEAD + 1) {
-            if (stores_behind) PwWaitVmcnt<(AHEAD - 1) * LPC + NST>(); else PwWaitVmcnt<(AHEAD - 1) * LPC>();
-        } else {
-            PwWaitVmcnt<0>();
-        }
-        }
-        stores_behind = false;
-        __builtin_amdgcn_sched_barrier(0);
-        __builtin_amdgcn_s_barrier();
-        __builtin_amdgcn_sched_barrier(0);
-        if (epi_pending) {
-            if constexpr (!(PW_ABL & 2)) {
-                epilogue(e_tm, e_tn);
-                stores_behind = true;
-            }
-            zero_acc();
-            epi_pending = false;
-        }
-        if constexpr (!(PW_ABL & 4)) compute();
-        __builtin_amdgcn_sched_barrier(0);
-        __builtin_amdgcn_s_barrier();
-        __builtin_amdgcn_sched_barrier(0);
+        issue_next();  // chunk g + 1 into the stage chunk g - 1 was read from (everybody passed the barrier)
+        read_frags(g % NSTAGE);
+        compute();
         ++g;
+        bool stored = false;
         if (++c_cb == nc) {
             c_cb = 0;
             ++c_i;
-            e_tm = c_tm;
-            e_tn = c_tn;
+            const int e_tm = c_tm, e_tn = c_tn;
             c_valid = tile_at(c_i, c_tm, c_tn);
-            if (grp == 1 || !c_valid) {
-                if constexpr (!(PW_ABL & 2)) {
-                    epilogue(e_tm, e_tn);
-                    stores_behind = true;
-                }
-                zero_acc();
-            } else {
-                epi_pending = true;
-            }
+            epilogue(e_tm, e_tn);
+            zero_acc();
+            stored = true;
         }
+        // the chunk issued above must have landed; the tile's stores, if any, were issued after it
+        __builtin_amdgcn_sched_barrier(0);
+        if (stored) PwWaitVmcnt<NST>(); else PwWaitVmcnt<0>();
+        __builtin_amdgcn_s_barrier();
     }
-    if (grp == 0) __builtin_amdgcn_s_barrier();
 }
 
 }  // namespace hipcx

@@ -260,8 +260,8 @@ def test_dot_float16_256_tiles():
 
 
 def test_conv1x1_float16_lds_direct_ring():
-    """1x1 / stride 1 float16 layers on the kernel that loads its operands straight into LDS (route 3): 256 x 256 tiles for wide
-    outputs over a short reduction, 512 x 128 tiles for 128 output channels; planes whose pixel count is a multiple of 8 and of 4
+    """1x1 / stride 1 float16 layers on the kernel that loads its operands straight into LDS (route 3; four-wave workgroups on
+    256-pixel x 128-channel tiles, two to a compute unit): planes whose pixel count is a multiple of 8 and of 4
     only (the last 16-byte piece of a plane is then half empty), workgroups that walk more than one tile, partial channel tiles,
     bias.  Integer-valued data: float accumulation has no rounding, so results are exact and the rounding of the bias sum is the
     only one.  Too large for the serial oracle loop: the reference is the same sum of products in float64."""
@@ -269,7 +269,7 @@ def test_conv1x1_float16_lds_direct_ring():
     from chainer_amd import routines
     rng = np.random.default_rng(41)
     cases = [(128, 64, 28, 256, True), (128, 64, 14, 1024, True), (96, 96, 14, 1320, False), (256, 32, 28, 128, True), (340, 160, 20, 100, True),
-             (128, 512, 28, 128, False)]
+             (128, 512, 28, 128, False), (1600, 64, 6, 300, True)]
     for (n, c, hw, k, with_bias) in cases:
         x = rng.integers(-3, 4, (n, c, hw, hw)).astype('float16')
         w = rng.integers(-2, 3, (k, c, 1, 1)).astype('float16')
