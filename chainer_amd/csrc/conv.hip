@@ -866,7 +866,9 @@ void RunStem(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, c
     auto kern = StemConv7x7s2Kernel<3>;
     struct StemTag {};
     EnsureDynamicLds<StemTag>(reinterpret_cast<const void*>(kern), pl.lds_bytes);
-    int blocks = a.N * ((a.OH + 1) / 2);
+    // workgroups walk tiles (two output rows of one image each): as many as the device holds at a time, two per compute unit
+    static const int per_unit = [] { const char* e = getenv("HIPCX_STEM_PER_UNIT"); return e != nullptr && atoi(e) > 0 ? atoi(e) : 2; }();
+    const int blocks = std::min(a.N * ((a.OH + 1) / 2), per_unit * NumCUs());
     hipLaunchKernelGGL(kern, dim3(blocks), dim3(256), pl.lds_bytes, stream, a);
     CheckLaunch("stem_conv");
 }

@@ -13,6 +13,9 @@
 // built in registers from aligned global loads with v_alignbit.  Filters stay in registers for the whole workgroup
 // (waves 0-1 own output channels 0-31, waves 2-3 channels 32-63).  The output tile leaves through LDS as
 // [channel][pixel] so that stores are whole cache lines, with the optional batch-norm / ReLU tail applied on the way.
+// A workgroup walks tiles (the host launches as many workgroups as the device holds at a time): filters are loaded once, and
+// the global loads of the next tile's rows are issued before the current tile is multiplied and written out, so that their
+// latency runs under that work instead of in front of the next tile.
 #pragma once
 
 #include "nchw_conv.h"
@@ -39,7 +42,7 @@ struct StemConvArgs {
 };
 
 template <int C>
-__global__ __launch_bounds__(256) void StemConv7x7s2Kernel(StemConvArgs p) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void StemConv7x7s2Kernel(StemConvArgs p) {
     constexpr int K = 64;
     constexpr int NPAIR = C * 7;
     constexpr int KSTEPS = (NPAIR + 1) / 2;
@@ -55,9 +58,7 @@ __global__ __launch_bounds__(256) void StemConv7x7s2Kernel(StemConvArgs p) {
     const int chalf = wave >> 1;  // which 32 output channels
     const int sub0 = wave & 1;    // first pixel sub-tile; the wave takes every second one
     const int tiles_per_img = (p.OH + 1) / 2;
-    const int n = blockIdx.x / tiles_per_img;
-    const int oh0 = 2 * (blockIdx.x - n * tiles_per_img);
-    const int npix = min(2, p.OH - oh0) * p.OW;  // valid pixels of this tile
+    const int total_tiles = p.N * tiles_per_img;
     const int nsub = (2 * p.OW + 31) / 32;
     const int ch = p.W / 8;  // 16-byte chunks per input row
 
@@ -71,38 +72,42 @@ __global__ __launch_bounds__(256) void StemConv7x7s2Kernel(StemConvArgs p) {
         wf[ks] = __builtin_amdgcn_raw_buffer_load_b128(wr, ((ks * 2 + g) * K + chalf * 32 + lr) * 16, 0, 0);
     }
 
-    // ---- zero rows, then stage the input rows as four shifted copies ----
-    for (int off = tid * 16; off < 3 * p.rowp; off += 256 * 16) {
-#pragma unroll
-        for (int k = 0; k < 4; ++k) *reinterpret_cast<Bytes16*>(lds + k * p.copyb + NROW * p.rowp + off) = Bytes16(0);
-    }
-    // Thread (tr, tj) stages 16-byte chunk tj (+32 per pass) of rows tr, tr + 8, ...: no divisions by run-time values, and all
-    // loads of a pass are issued before the first is used.
+    // Thread (tr, tj) stages 16-byte chunk tj of rows tr, tr + 8, ... (W <= 256: one chunk per thread and row): no divisions by
+    // run-time values, and all loads of a tile are issued before the first is used.
     constexpr int kRowsPerThread = (NROW + 7) / 8;
     const int tj = tid & 31, tr = tid >> 5;
-    for (int j = tj; j < ch; j += 32) {
-        Bytes16 g1[kRowsPerThread];
-        Bytes8 g0[kRowsPerThread], g2[kRowsPerThread];
+    Bytes16 g1[kRowsPerThread];
+    Bytes8 g0[kRowsPerThread], g2[kRowsPerThread];
+    auto issue_rows = [&](int tile) {  // global loads of the tile's input rows into registers
+        const int n = tile / tiles_per_img;
+        const int oh0 = 2 * (tile - n * tiles_per_img);
 #pragma unroll
         for (int u = 0; u < kRowsPerThread; ++u) {
             const int rr = tr + 8 * u;
             const int c = rr / 9;
             const int ih = 2 * oh0 - 3 + (rr - c * 9);
-            const bool row_ok = rr < NROW && ih >= 0 && ih < p.H;
-            const int base = (((n * C + c) * p.H + ih) * p.W + j * 8) * 2;
+            const bool row_ok = tj < ch && rr < NROW && ih >= 0 && ih < p.H;
+            const int base = (((n * C + c) * p.H + ih) * p.W + tj * 8) * 2;
             g1[u] = __builtin_amdgcn_raw_buffer_load_b128(xr, row_ok ? base : 0x7fffffff, 0, 0);
-            g0[u] = __builtin_amdgcn_raw_buffer_load_b64(xr, (row_ok && j > 0) ? base - 8 : 0x7fffffff, 0, 0);
-            g2[u] = __builtin_amdgcn_raw_buffer_load_b64(xr, (row_ok && j + 1 < ch) ? base + 16 : 0x7fffffff, 0, 0);
+            g0[u] = __builtin_amdgcn_raw_buffer_load_b64(xr, (row_ok && tj > 0) ? base - 8 : 0x7fffffff, 0, 0);
+            g2[u] = __builtin_amdgcn_raw_buffer_load_b64(xr, (row_ok && tj + 1 < ch) ? base + 16 : 0x7fffffff, 0, 0);
         }
+    };
+    auto stage_rows = [&]() {  // zero rows, then the loaded rows as four shifted copies
+        for (int off = tid * 16; off < 3 * p.rowp; off += 256 * 16) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) *reinterpret_cast<Bytes16*>(lds + k * p.copyb + NROW * p.rowp + off) = Bytes16(0);
+        }
+        if (tj >= ch) return;
 #pragma unroll
         for (int u = 0; u < kRowsPerThread; ++u) {
             const int rr = tr + 8 * u;
             if (rr >= NROW) continue;
-            // d[i] holds input pixels 8*j - 8 + 2*i, +1 of this row (i = 2 .. 9)
+            // d[i] holds input pixels 8*tj - 8 + 2*i, +1 of this row (i = 2 .. 9)
             unsigned d[10] = {0, 0, g0[u].x, g0[u].y, g1[u].x, g1[u].y, g1[u].z, g1[u].w, g2[u].x, g2[u].y};
-            char* dst = lds + rr * p.rowp + j * 16;
+            char* dst = lds + rr * p.rowp + tj * 16;
 #pragma unroll
-            for (int k = 0; k < 4; ++k) {  // copy k, chunk j = padded pixels 8*j + 2*k .. +7 = input pixels 8*j + 2*k - 3 .. +4
+            for (int k = 0; k < 4; ++k) {  // copy k, chunk tj = padded pixels 8*tj + 2*k .. +7 = input pixels 8*tj + 2*k - 3 .. +4
                 Bytes16 v;
                 v.x = __builtin_amdgcn_alignbit(d[3 + k], d[2 + k], 16);
                 v.y = __builtin_amdgcn_alignbit(d[4 + k], d[3 + k], 16);
@@ -111,7 +116,36 @@ __global__ __launch_bounds__(256) void StemConv7x7s2Kernel(StemConvArgs p) {
                 *reinterpret_cast<Bytes16*>(dst + k * p.copyb) = v;
             }
         }
+    };
+
+    int poff[KSTEPS];  // staged row of this lane's filter row (c, r) in each step
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+        int pair = 2 * ks + g;
+        int c = pair / 7, r = pair - c * 7;
+        poff[ks] = (pair < NPAIR ? c * 9 + r : NROW) * p.rowp;
     }
+    // per-channel constants of the epilogue
+    const int nch = chalf * 32 + lr;
+    const float bias = p.bias != nullptr ? static_cast<float>(p.bias[nch * p.bias_stride]) : 0.f;
+    const bool has_bn = p.bn_gamma != nullptr;
+    float bn_mean = 0.f, bn_inv = 1.f, bn_gamma = 1.f, bn_beta = 0.f;
+    if (has_bn) {
+        bn_mean = static_cast<float>(p.bn_mean[nch * p.bn_stride]);
+        bn_inv = 1.0f / sqrtf(static_cast<float>(p.bn_var[nch * p.bn_stride]) + p.bn_eps);
+        bn_gamma = static_cast<float>(p.bn_gamma[nch * p.bn_stride]);
+        bn_beta = static_cast<float>(p.bn_beta[nch * p.bn_stride]);
+    }
+
+    int tile = blockIdx.x;
+    if (tile >= total_tiles) return;
+    issue_rows(tile);
+    for (; tile < total_tiles; tile += gridDim.x) {
+    const int n = tile / tiles_per_img;
+    const int oh0 = 2 * (tile - n * tiles_per_img);
+    const int npix = min(2, p.OH - oh0) * p.OW;  // valid pixels of this tile
+    stage_rows();
+    if (tile + static_cast<int>(gridDim.x) < total_tiles) issue_rows(tile + gridDim.x);  // in flight during the rest of this tile
 
     // ---- operand addresses ----
     int abase[MAXSUB];
@@ -123,14 +157,6 @@ __global__ __launch_bounds__(256) void StemConv7x7s2Kernel(StemConvArgs p) {
         int ow = q - (orow ? p.OW : 0);
         abase[s] = (ow & 3) * p.copyb + 2 * orow * p.rowp + (ow >> 2) * 16;
     }
-    int poff[KSTEPS];  // staged row of this lane's filter row (c, r) in each step
-#pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) {
-        int pair = 2 * ks + g;
-        int c = pair / 7, r = pair - c * 7;
-        poff[ks] = (pair < NPAIR ? c * 9 + r : NROW) * p.rowp;
-    }
-
     float16_t acc[MAXSUB];
 #pragma unroll
     for (int s = 0; s < MAXSUB; ++s) {
@@ -154,16 +180,6 @@ __global__ __launch_bounds__(256) void StemConv7x7s2Kernel(StemConvArgs p) {
     // ---- epilogue: [channel][pixel] tile, then coalesced rows ----
     const int opitch = 2 * p.OW * 2 + 16;
     {
-        const int nch = chalf * 32 + lr;
-        float bias = p.bias != nullptr ? static_cast<float>(p.bias[nch * p.bias_stride]) : 0.f;
-        const bool has_bn = p.bn_gamma != nullptr;
-        float bn_mean = 0.f, bn_inv = 1.f, bn_gamma = 1.f, bn_beta = 0.f;
-        if (has_bn) {
-            bn_mean = static_cast<float>(p.bn_mean[nch * p.bn_stride]);
-            bn_inv = 1.0f / sqrtf(static_cast<float>(p.bn_var[nch * p.bn_stride]) + p.bn_eps);
-            bn_gamma = static_cast<float>(p.bn_gamma[nch * p.bn_stride]);
-            bn_beta = static_cast<float>(p.bn_beta[nch * p.bn_stride]);
-        }
 #pragma unroll
         for (int s = 0; s < MAXSUB; ++s) {
             if (sub0 + 2 * s >= nsub) continue;
@@ -193,6 +209,8 @@ __global__ __launch_bounds__(256) void StemConv7x7s2Kernel(StemConvArgs p) {
             *reinterpret_cast<Bytes16*>(dst + static_cast<int64_t>(row) * p.OH * p.OW) = v;
         }
     }
+    __syncthreads();  // the output tile has been read: the next tile's rows may be staged over it
+    }  // tiles
 }
 
 // w[64][C][7][7] (element strides) -> wp[ksteps][2][64][8] with zero padding.
