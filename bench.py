@@ -168,7 +168,7 @@ def main():
     avg_launch_ms = ms.value / max(n.value, 1)
     achieved_tflops = flops.value / (ms.value * 1e-3) / 1e12 if ms.value > 0 else 0.0
     roofline = {
-        'kernel': 'NchwConvKernel / IGemmFastKernel (convolution + linear, MFMA implicit GEMM)',
+        'kernel': 'NchwConvKernel / PwConvKernel / StemConv7x7s2Kernel / SmallDotKernel (every convolution and the linear layer of a pass, MFMA implicit GEMM)',
         'bound': 'mfma',
         'achieved': round(achieved_tflops, 2),
         'peak': MFMA_F16_PEAK_TFLOPS,

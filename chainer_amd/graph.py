@@ -38,22 +38,26 @@ def capture(fn):
     # both passes run on one side stream: the pool keeps the blocks of different streams apart
     stream = t.cuda.Stream()
     stream.wait_stream(t.cuda.current_stream())
-    with arena:
-        for _ in range(MAX_WARM_PASSES):
-            gc.collect()  # arrays held only by garbage cycles would otherwise be freed at some later, arbitrary moment
-            before = pool_stats()['device_allocations']
-            with t.cuda.stream(stream):
+    try:
+        with arena:
+            for _ in range(MAX_WARM_PASSES):
+                gc.collect()  # arrays held only by garbage cycles would otherwise be freed at some later, arbitrary moment
+                before = pool_stats()['device_allocations']
+                with t.cuda.stream(stream):
+                    out = fn()
+                stream.synchronize()
+                del out
+                if pool_stats()['device_allocations'] == before:
+                    break
+            else:
+                raise RuntimeError('capture: fn() still took new memory from the driver in each of its %d warm passes (it allocates more '
+                                   'from pass to pass, e.g. by keeping its results alive); a pass that allocates cannot be captured'
+                                   % MAX_WARM_PASSES)
+            gc.collect()
+            graph = t.cuda.CUDAGraph()
+            with t.cuda.graph(graph, stream=stream):
                 out = fn()
-            stream.synchronize()
-            del out
-            if pool_stats()['device_allocations'] == before:
-                break
-        else:
-            raise RuntimeError('capture: fn() still took new memory from the driver in each of its %d warm passes (it allocates more '
-                               'from pass to pass, e.g. by keeping its results alive); a pass that allocates cannot be captured'
-                               % MAX_WARM_PASSES)
-        gc.collect()
-        graph = t.cuda.CUDAGraph()
-        with t.cuda.graph(graph, stream=stream):
-            out = fn()
+    except BaseException:
+        arena.release()  # its cached blocks join the general pool again
+        raise
     return CapturedGraph(graph, out, arena)

@@ -178,8 +178,9 @@ int32_t ReadDeviceFlag(Device& device, const std::shared_ptr<void>& flag) {
 class HipBackend;
 
 // The Device interface (chainerx/device.h:24-71) over the library's device layer: every allocation comes from the pool behind
-// hipcx_malloc and goes back through hipcx_free (the deleter never throws and outlives the pool: a free after
-// hipcx_pool_destroy is a no-op inside the library), copies are the library's.
+// hipcx_malloc and goes back through hipcx_free (the deleter never throws and outlives the pool: the library remembers the blocks
+// that were in use when hipcx_pool_destroy took their pool away and swallows their frees, also when a new pool exists on the
+// device by then), copies are the library's.
 class HipDevice : public Device {
 public:
     HipDevice(Backend& backend, int index) : Device{backend, index} {}

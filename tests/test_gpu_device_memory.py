@@ -201,3 +201,28 @@ def test_take_default_mode_is_captured_and_still_raises():
     ids[5] = 0
     assert np.array_equal(g.result.get(), table[ids] * 2.0)
     g.release()
+
+
+def test_graph_capture_refuses_a_function_that_keeps_allocating():
+    """capture() warms a function up until one pass takes all its memory from the arena's free lists.  A function that keeps its
+    results alive allocates new blocks in every pass: capture raises a clear error instead of calling the driver's allocator under
+    stream capture."""
+    import chainer_amd as chx
+    from chainer_amd import graph
+    hoard = []
+
+    def grows():
+        hoard.append(chx.zeros((256, 1024), 'float32') + 1.0)
+        return hoard[-1]
+
+    with pytest.raises(RuntimeError, match='warm passes'):
+        graph.capture(grows)
+    assert len(hoard) == graph.MAX_WARM_PASSES
+    del hoard[:]
+    # a function that settles after its first pass is captured as before
+    x = chx.ones((64, 64), 'float32')
+    g = graph.capture(lambda: x + x)
+    g.replay()
+    chx.synchronize()
+    assert np.array_equal(g.result.get(), np.full((64, 64), 2, np.float32))
+    g.release()
