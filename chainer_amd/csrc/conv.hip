@@ -1075,7 +1075,9 @@ void CheckConv(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b,
 }  // namespace hipcx
 
 namespace hipcx {
-// nd_ops.hip: arrays without exactly two spatial axes
+// int_dot.hip: Dot for the integer dtypes and bool
+void IntDot(const hipcx_array* a, const hipcx_array* b, const hipcx_array* out, hipStream_t stream);
+// nd_ops.hip: arrays without exactly two spatial axes, and the integer dtypes
 size_t ConvNdWorkspaceSize(const hipcx_array* x, const hipcx_array* w, const hipcx_array* out);
 void ConvNd(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, const int64_t* stride, const int64_t* pad, int cover_all,
             const hipcx_array* out, void* workspace, size_t workspace_bytes, void* stream);
@@ -1134,6 +1136,7 @@ int hipcx_profile_records(int64_t capacity, double* ms, double* flops, double* b
 
 size_t hipcx_conv_workspace_size(const hipcx_array* x, const hipcx_array* w, const hipcx_array* out) {
     if (x == nullptr || w == nullptr) return 0;
+    if (!IsFloatDtype(x->dtype)) return 0;
     if (x->ndim != 4 || w->ndim != 4) {
         try {
             return x->ndim >= 2 ? ConvNdWorkspaceSize(x, w, out) : 0;
@@ -1172,7 +1175,7 @@ int hipcx_conv_route(const hipcx_array* x, const hipcx_array* w, const hipcx_arr
 int hipcx_conv(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, const int64_t* stride, const int64_t* pad,
                int cover_all, const hipcx_array* out, void* workspace, size_t workspace_bytes, void* stream) {
     return Guard([&] {
-        if (x != nullptr && x->ndim != 4) {  // not two spatial axes: nd_ops.hip
+        if (x != nullptr && out != nullptr && (x->ndim != 4 || !IsFloatDtype(out->dtype))) {  // not two spatial axes, or integers: nd_ops.hip
             ConvNd(x, w, b, stride, pad, cover_all, out, workspace, workspace_bytes, stream);
             return;
         }
@@ -1435,6 +1438,7 @@ extern "C" {
 
 size_t hipcx_dot_workspace_size(const hipcx_array* a, const hipcx_array* b, const hipcx_array* out) {
     try {
+        if (out != nullptr && !IsFloatDtype(out->dtype)) return 0;
         DotStaging st = PlanDotStaging(a, b, out);
         size_t split = 0;
         if (a != nullptr && b != nullptr && out != nullptr && a->ndim == 2 && b->ndim == 2) {
@@ -1456,7 +1460,6 @@ int hipcx_dot(const hipcx_array* a, const hipcx_array* b, const hipcx_array* out
                       "ChainerX dot supports only 2-dimensional arrays.");
         int64_t m = a->shape[0], k = a->shape[1], n = b->shape[1];
         HIPCX_REQUIRE(b->shape[0] == k && out->shape[0] == m && out->shape[1] == n, HIPCX_DIMENSION_ERROR, "dot: shape mismatch");
-        HIPCX_REQUIRE(IsFloatDtype(out->dtype), HIPCX_NOT_IMPLEMENTED_ERROR, "hip dot supports floating point dtypes only");
         HIPCX_REQUIRE(a->dtype == out->dtype && b->dtype == out->dtype, HIPCX_DTYPE_ERROR,
                       "a and b must have out's dtype (cast with hipcx_copy first)");
         HIPCX_REQUIRE(m < (1LL << 31) && n < (1LL << 31) && k < (1LL << 31), HIPCX_NOT_IMPLEMENTED_ERROR, "extent too large");
@@ -1466,6 +1469,10 @@ int hipcx_dot(const hipcx_array* a, const hipcx_array* b, const hipcx_array* out
             hipcx_scalar zero{HIPCX_KIND_INT, 0, 0, 0.0};
             int s = hipcx_fill(out, zero, stream);
             if (s != HIPCX_OK) throw Error(s, hipcx_last_error());
+            return;
+        }
+        if (!IsFloatDtype(out->dtype)) {  // integers and bool: int_dot.hip
+            IntDot(a, b, out, st);
             return;
         }
         auto fill = [&](auto& p) {

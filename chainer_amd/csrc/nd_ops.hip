@@ -1,9 +1,11 @@
 // Convolution and pooling over any number of spatial axes (ConvKernel CX/kernels/connection.h:14-32, MaxPoolKernel / AveragePoolKernel
 // CX/kernels/pooling.h:20-64): the correctness path for what is not 2-D.  The native backend handles every rank with one algorithm,
 // Im2Col over n axes followed by TensorDot (conv.cc:52-89) or by a reduction over the kernel axes (pool.cc:68-95, 191-250); the
-// dedicated kernels of this library are 2-D.  Here
+// dedicated kernels of this library are 2-D and floating point.  Here
 //   * 0 and 1 spatial axes are 2-D problems with extents of one and run through the 2-D entry points (same kernels, same results);
-//   * 3 and more spatial axes run the plain kernels below: one thread per output element, a loop over the window (and the input
+//   * 3 and more spatial axes, and convolutions of the integer dtypes and bool over any number of axes (the native backend
+//     multiplies those like any other dtype, in the array dtype: arithmetic modulo 2^bits, which no order changes), run the plain
+//     kernels below: one thread per output element, a loop over the window (and the input
 //     channels).  They follow the reference's arithmetic -- float accumulation for float16, the bias added after the sum was rounded
 //     to the array dtype, max pooling that keeps a NaN once it met one and pads with the lowest value, average pooling that rounds
 //     the window sum to the array dtype before the division -- and make no attempt at speed.
@@ -65,9 +67,22 @@ __device__ __forceinline__ int64_t DecodeOutput(const NdArgs& p, int64_t idx, in
     return off + n * p.os[0] + c * p.os[1];
 }
 
+// Accumulator of the convolution: float for float16, an unsigned type at least as wide for integers (sums modulo 2^bits without
+// signed overflow, truncated on store), 32 bits for bool (a count of products that cannot wrap, stored as "any").
+template <typename T>
+struct NdAcc {
+    using type = compute_t<T>;
+};
+template <> struct NdAcc<bool> { using type = uint32_t; };
+template <> struct NdAcc<int8_t> { using type = uint32_t; };
+template <> struct NdAcc<uint8_t> { using type = uint32_t; };
+template <> struct NdAcc<int16_t> { using type = uint32_t; };
+template <> struct NdAcc<int32_t> { using type = uint32_t; };
+template <> struct NdAcc<int64_t> { using type = uint64_t; };
+
 template <typename T>
 __global__ __launch_bounds__(256) void ConvNdKernel(NdArgs p, int64_t total) {
-    using A = compute_t<T>;
+    using A = typename NdAcc<T>::type;
     const T* x = static_cast<const T*>(p.x);
     const T* w = static_cast<const T*>(p.w);
     T* out = static_cast<T*>(p.out);
@@ -225,15 +240,15 @@ void ConvNd(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, co
     ValidateArray(out, "out");
     HIPCX_REQUIRE(x->ndim >= 2 && w->ndim == x->ndim && out->ndim == x->ndim, HIPCX_DIMENSION_ERROR,
                   "conv: x, w and out need the same rank, at least 2 (batch / output channels and input channels)");
-    HIPCX_REQUIRE(IsFloatDtype(out->dtype) && x->dtype == out->dtype && w->dtype == out->dtype && (b == nullptr || b->dtype == out->dtype),
-                  HIPCX_DTYPE_ERROR, "conv: x, w and b must have out's floating point dtype (cast with hipcx_copy first)");
+    HIPCX_REQUIRE(x->dtype == out->dtype && w->dtype == out->dtype && (b == nullptr || b->dtype == out->dtype), HIPCX_DTYPE_ERROR,
+                  "conv: x, w and b must have out's dtype (cast with hipcx_copy first)");
     HIPCX_REQUIRE(w->shape[1] == x->shape[1], HIPCX_DIMENSION_ERROR, "Mismatched number of input channels in input and weights.");
     if (b != nullptr) {
         ValidateArray(b, "b");
         HIPCX_REQUIRE(b->ndim == 1 && b->shape[0] == w->shape[0], HIPCX_DIMENSION_ERROR, "Mismatched bias shape for weights.");
     }
     const int n = x->ndim - 2;
-    if (n <= 1) {
+    if (n <= 1 && IsFloatDtype(out->dtype)) {
         hipcx_array x4 = AsFourAxes(x), w4 = AsFourAxes(w), o4 = AsFourAxes(out);
         int64_t s4[2], p4[2];
         FourAxisWindow(n, stride, 1, s4);
@@ -253,7 +268,7 @@ void ConvNd(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, co
     }
     const int64_t total = TotalSize(out);
     if (total == 0) return;
-    VisitFloatDtype(out->dtype, [&](auto tag) {
+    VisitDtype(out->dtype, [&](auto tag) {
         using T = typename decltype(tag)::type;
         hipLaunchKernelGGL((ConvNdKernel<T>), dim3(NdBlocks(total)), dim3(256), 0, AsStream(stream), p, total);
     });

@@ -285,7 +285,10 @@ int hipcx_any(const hipcx_array* a, const int8_t* axis, int naxis, const hipcx_a
 int hipcx_sum_static_scratch(const hipcx_array* a, const int8_t* axis, int naxis, const hipcx_array* out, void* stream);
 
 /* ---- linear algebra / connection: CX/kernels/linalg.h:15, connection.h:21 ---- */
-/* out[M,N] = a[M,K] . b[K,N]; float16/32/64; fp16 accumulates in fp32 (CX/native/native_device/dot.cc:181-227). */
+/* out[M,N] = a[M,K] . b[K,N], all three of one dtype.  float16/32/64 run on the matrix pipes; fp16 accumulates in fp32.  The
+ * integer dtypes and bool are multiplied as the native backend does (CX/native/native_device/dot.cc:130-134, 181-227: one
+ * accumulator of the array dtype, i.e. sums modulo 2^bits; bool is "any of the conjunctions") by a plain tiled kernel -- the cuda
+ * backend raises for them (CX/cuda/cuda_device/dot.cu:74-76). */
 size_t hipcx_dot_workspace_size(const hipcx_array* a, const hipcx_array* b, const hipcx_array* out);
 int hipcx_dot(const hipcx_array* a, const hipcx_array* b, const hipcx_array* out, void* workspace, size_t workspace_bytes,
               void* stream);
@@ -294,14 +297,16 @@ int64_t hipcx_conv_out_dim(int64_t in_dim, int64_t kernel_size, int64_t stride, 
 /* Convolution forward (ConvKernel CX/kernels/connection.h:14-32), x[N,C,H,W] (any strides), w[K,C,kh,kw], optional b[K] (NULL = none),
  * out[N,K,OH,OW] with any strides.  Other ranks, like the native kernel (CX/native/native_device/conv.cc:57-89): x[N,C,d_1..d_n] with
  * w[K,C,k_1..k_n], `stride` and `pad` holding n values; n = 0 and 1 run the 2-D kernels over extents of one, n >= 3 a plain
- * one-thread-per-output kernel (a correctness path: float accumulation for float16, bias added after rounding, as the native backend).  The plugin and the Python mirror allocate out C-contiguous (NCHW memory), like the CUDA
+ * one-thread-per-output kernel (a correctness path: float accumulation for float16, bias added after rounding, as the native backend).
+ * Integer dtypes and bool, which the native backend's Im2Col + TensorDot accepts like any other, run that plain kernel at every
+ * rank (sums modulo 2^bits, equal bit for bit).  The plugin and the Python mirror allocate out C-contiguous (NCHW memory), like the CUDA
  * backend (CX/cuda/cuda_conv.cc:311); the native backend's own result is an NCHW view of NHWC memory
  * (CX/native/native_device/conv.cc:78-84), which this entry also accepts as `out`. */
 size_t hipcx_conv_workspace_size(const hipcx_array* x, const hipcx_array* w, const hipcx_array* out);
 /* Which kernel family hipcx_conv runs for these arguments (no counterpart in the reference: for tests and benchmarks that must
  * know that a specialised kernel, not the general one, produced a result).  0: general implicit GEMM (any dtype / layout);
  * 1: float16 NCHW kernels with 128-wide tiles; 2: float16 7x7 / 2 stem kernel; 3: float16 1x1 / stride 1 kernel that loads its
- * operands straight into LDS and walks 256 x 256 or 512 x 128 tiles; -1: invalid arguments. */
+ * operands straight into LDS and walks 256 x 128 tiles; -1: invalid arguments. */
 int hipcx_conv_route(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, const int64_t* stride, const int64_t* pad,
                      const hipcx_array* out);
 int hipcx_conv(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, const int64_t* stride, const int64_t* pad,

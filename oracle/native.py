@@ -668,6 +668,14 @@ def dot(a, b):
         rc = L.oracle_dot_f16(_ptr(ac.view(np.uint16), _u16p), _ptr(bc.view(np.uint16), _u16p), _ptr(ob, _u16p), _i64(m), _i64(k), _i64(n))
         assert rc == 0
         out = ob.view(np.float16)
+    elif a.dtype == np.bool_:
+        # MultiplyAdd(bool, bool, bool) = (x && y) || z (dot.cc:134)
+        out = (ac.astype(np.int64) @ bc.astype(np.int64)) != 0
+    elif a.dtype.kind in 'iu':
+        # one accumulator of the array dtype per element, acc = a*b + acc (dot.cc:130-132, 200-214): the sum modulo 2^bits,
+        # whatever the order; computed modulo 2^64 (numpy's integer matmul wraps) and truncated
+        with np.errstate(over='ignore'):
+            out = (ac.astype(np.uint64) @ bc.astype(np.uint64)).astype(a.dtype)
     else:
         raise TypeError(a.dtype)
     return out

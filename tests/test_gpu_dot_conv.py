@@ -106,6 +106,70 @@ def test_dot_integer_valued_is_exact():
         assert np.array_equal(got.astype(np.int64), a.astype(np.int64) @ b.astype(np.int64))
 
 
+INT_DTYPES = ('int8', 'uint8', 'int16', 'int32', 'int64')
+
+
+def test_dot_and_linear_of_integers_and_bool():
+    """The native backend multiplies every dtype (dot.cc:177-227); integer sums are arithmetic modulo 2^bits, so the results
+    are equal bit for bit over the full value range, whatever the layout of the operands."""
+    import chainer_amd as chx
+    rng = np.random.default_rng(31)
+    for dt in INT_DTYPES:
+        info = np.iinfo(dt)
+        for (m, k, n) in [(7, 33, 5), (64, 64, 64), (130, 100, 70), (1, 1, 1), (3, 2000, 3), (100, 17, 129)]:
+            a = rng.integers(info.min, info.max, (m, k), dtype=dt, endpoint=True)
+            b = rng.integers(info.min, info.max, (k, n), dtype=dt, endpoint=True)
+            ref = O.dot(a, b)
+            what = '%s %s' % (dt, (m, k, n))
+            got = chx.dot(chx.array(a), chx.array(b))
+            assert got.dtype == ref.dtype and np.array_equal(got.get(), ref), what
+            at = chx.array(np.ascontiguousarray(a.T)).T
+            bt = chx.array(np.ascontiguousarray(b.T)).T
+            assert np.array_equal(chx.dot(at, bt).get(), ref), 'transposed views ' + what
+            bias = rng.integers(info.min, info.max, n, dtype=dt, endpoint=True)
+            wt = np.ascontiguousarray(b.T)
+            assert np.array_equal(chx.linear(chx.array(a), chx.array(wt), chx.array(bias)).get(), O.linear(a, wt, bias)), 'linear ' + what
+        ap = padded((5, 9), rng.integers(-100, 100, (5, 9)), 1, dt)
+        bp = padded((9, 4), rng.integers(-100, 100, (9, 4)), 2, dt)
+        assert np.array_equal(chx.dot(upload_view(chx, ap), upload_view(chx, bp)).get(), O.dot(np.ascontiguousarray(ap), np.ascontiguousarray(bp)))
+    a = rng.integers(0, 3, (70, 90)) == 0
+    b = rng.integers(0, 20, (90, 50)) == 0
+    got = chx.dot(chx.array(a), chx.array(b))
+    assert got.dtype == np.bool_ and np.array_equal(got.get(), O.dot(a, b))
+    # mixed operand dtypes are cast to the result dtype first (dot.cc:177-178)
+    a8 = rng.integers(-128, 127, (9, 11), dtype='int8')
+    b32 = rng.integers(-2 ** 31, 2 ** 31 - 1, (11, 6), dtype='int32')
+    assert np.array_equal(chx.dot(chx.array(a8), chx.array(b32)).get(), O.dot(a8.astype('int32'), b32))
+    z = chx.dot(chx.zeros((3, 0), 'int32'), chx.zeros((0, 4), 'int32'))
+    assert z.dtype == np.int32 and z.shape == (3, 4) and not z.get().any()
+
+
+def test_conv_of_integers_over_any_number_of_axes():
+    """Integer convolutions (the native backend's Im2Col + TensorDot takes every dtype): equal to the oracle bit for bit, values
+    large enough to wrap, 0 to 3 spatial axes, dense and permuted input."""
+    import chainer_amd as chx
+    rng = np.random.default_rng(32)
+    cases = [((2, 3), (4, 3), 1, 0), ((2, 3, 9), (4, 3, 3), 2, 1), ((2, 3, 7, 6), (5, 3, 3, 2), (2, 1), (1, 0)),
+             ((3, 16, 8, 8), (32, 16, 3, 3), 1, 1), ((2, 2, 5, 4, 6), (3, 2, 2, 3, 2), (1, 2, 1), (1, 0, 1))]
+    for dt in INT_DTYPES + ('bool',):
+        for xs, ws, stride, pad in cases:
+            if dt == 'bool':
+                x, w, b = (rng.integers(0, 4, xs) == 0), (rng.integers(0, 4, ws) == 0), (rng.integers(0, 4, ws[0]) == 0)
+            else:
+                info = np.iinfo(dt)
+                lo, hi = max(info.min, -2 ** 20), min(info.max, 2 ** 20)
+                x, w, b = (rng.integers(lo, hi, s).astype(dt) for s in (xs, ws, ws[0]))
+            for cv in (False, True):
+                for bias in (None, b):
+                    ref = O.conv_nd(x, w, bias, stride, pad, cv)
+                    got = chx.conv(chx.array(x), chx.array(w), chx.array(bias) if bias is not None else None, stride, pad, cv)
+                    assert got.dtype == ref.dtype and got.shape == ref.shape, (dt, xs, ws)
+                    assert np.array_equal(got.get(), ref), (dt, xs, ws, stride, pad, cv, bias is not None)
+            if len(xs) == 4:
+                got = chx.conv(channels_last(chx, x), chx.array(w), chx.array(b), stride, pad)
+                assert np.array_equal(got.get(), O.conv_nd(x, w, b, stride, pad)), ('permuted', dt, xs)
+
+
 def test_dot_conv_edge_cases_and_errors():
     import chainer_amd as chx
     z = chx.dot(chx.zeros((3, 0), 'float32'), chx.zeros((0, 4), 'float32')).get()

@@ -367,6 +367,39 @@ def test_dot_matches_float64_matmul(dtype, tol):
         assert np.array_equal(O.dot(ai, bi).astype(np.int64), ai.astype(np.int64) @ bi.astype(np.int64))
 
 
+INT_DTYPES = ('int8', 'uint8', 'int16', 'int32', 'int64')
+
+
+def wrap_to(value, dtype):
+    """A Python integer reduced to the two's-complement range of `dtype`."""
+    info = np.iinfo(dtype)
+    value &= (1 << info.bits) - 1
+    return value - (1 << info.bits) if info.min < 0 and value >= 1 << (info.bits - 1) else value
+
+
+def test_dot_of_integers_and_bool_wraps_like_one_accumulator():
+    """L: the native loop acc = a*b + acc with an accumulator of the array dtype (dot.cc:130-134, 200-214), evaluated with Python's
+    unbounded integers and reduced modulo 2^bits, over the full value range of every integer dtype (a sum kept in a wider type
+    or saturated fails); bool is "any of the conjunctions"."""
+    rng = np.random.default_rng(12)
+    for dtype in INT_DTYPES:
+        info = np.iinfo(dtype)
+        a = rng.integers(info.min, info.max, (5, 9), dtype=dtype, endpoint=True)
+        b = rng.integers(info.min, info.max, (9, 4), dtype=dtype, endpoint=True)
+        got = O.dot(a, b)
+        assert got.dtype == np.dtype(dtype)
+        for i in range(5):
+            for j in range(4):
+                acc = sum(int(a[i, l]) * int(b[l, j]) for l in range(9))
+                assert int(got[i, j]) == wrap_to(acc, dtype), (dtype, i, j)
+    a = rng.integers(0, 2, (6, 7)).astype(bool)
+    b = rng.integers(0, 4, (7, 5)) == 0
+    got = O.dot(a, b)
+    assert got.dtype == np.bool_
+    want = [[any(a[i, l] and b[l, j] for l in range(7)) for j in range(5)] for i in range(6)]
+    assert np.array_equal(got, np.array(want))
+
+
 def brute_conv(x, w, b, stride, pad, cover_all):
     """Definition of the cross-correlation (float64), out extent from the definition of cover_all: the last window must
     cover the last padded input element (chainer.utils.conv.get_conv_outsize)."""
@@ -732,20 +765,21 @@ def test_batch_norm_training_closed_forms():
         assert abs((loss(x, gamma, beta + e) - loss(x, gamma, beta - e)) / (2 * h) - gb[c]) <= 1e-6
 
 
-def _brute_conv_nd(x, w, b, stride, pad, cover_all):
-    """Definition of the cross-correlation, one output element at a time, float64."""
+def _brute_conv_nd(x, w, b, stride, pad, cover_all, number=float):
+    """Definition of the cross-correlation, one output element at a time, in float64 (or, with number=int, in Python's
+    unbounded integers)."""
     n = x.ndim - 2
     od = [O.conv_out_dim(x.shape[2 + d], w.shape[2 + d], stride[d], pad[d], cover_all) for d in range(n)]
-    out = np.zeros((x.shape[0], w.shape[0]) + tuple(od))
+    out = np.zeros((x.shape[0], w.shape[0]) + tuple(od), dtype=np.float64 if number is float else object)
     for idx in np.ndindex(*out.shape):
         nb, k, o = idx[0], idx[1], idx[2:]
-        acc = 0.0
+        acc = number(0)
         for c in range(x.shape[1]):
             for kidx in np.ndindex(*w.shape[2:]):
                 i = tuple(o[d] * stride[d] - pad[d] + kidx[d] for d in range(n))
                 if all(0 <= i[d] < x.shape[2 + d] for d in range(n)):
-                    acc += float(x[(nb, c) + i]) * float(w[(k, c) + kidx])
-        out[idx] = acc + (float(b[k]) if b is not None else 0.0)
+                    acc += number(x[(nb, c) + i]) * number(w[(k, c) + kidx])
+        out[idx] = acc + (number(b[k]) if b is not None else number(0))
     return out
 
 
@@ -807,6 +841,19 @@ def test_conv_and_pooling_over_n_axes():
                 got = O.conv_nd(x, w, bias, stride, pad, cv)
                 want = _brute_conv_nd(x, w, bias, tup(stride, n), tup(pad, n), cv)
                 assert got.shape == want.shape and np.allclose(got, want, rtol=1e-12, atol=1e-12), (xs, ws, stride, pad, cv)
+    # integer dtypes: the definition in exact integer arithmetic, reduced modulo 2^bits (values large enough to wrap)
+    for dtype in INT_DTYPES:
+        info = np.iinfo(dtype)
+        lo, hi = max(info.min, -2 ** 20), min(info.max, 2 ** 20)
+        for xs, ws, stride, pad in CONV_ND_GRID[::3]:
+            n = len(xs) - 2
+            x = rng.integers(lo, hi, xs).astype(dtype)
+            w = rng.integers(lo, hi, ws).astype(dtype)
+            b = rng.integers(lo, hi, ws[0]).astype(dtype)
+            got = O.conv_nd(x, w, b, stride, pad, False)
+            want = _brute_conv_nd(x, w, b, tup(stride, n), tup(pad, n), False, number=int)
+            assert got.dtype == np.dtype(dtype) and got.shape == want.shape
+            assert all(int(g) == wrap_to(int(v), dtype) for g, v in zip(got.ravel(), want.ravel())), (dtype, xs, ws)
     for xs, ks, stride, pad in POOL_ND_GRID:
         n = len(xs) - 2
         x = rng.standard_normal(xs)
