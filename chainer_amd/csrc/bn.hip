@@ -95,14 +95,7 @@ __global__ __launch_bounds__(kBnFlatThreads) void BnChannelsFirstKernel(const T*
     C* prm = reinterpret_cast<C*>(bn_lds);  // [max_rows][4]
     const int64_t e0 = static_cast<int64_t>(blockIdx.x) * kSpan;
     const int64_t row_first = e0 / L;
-    for (int r = threadIdx.x; r < max_rows; r += kBnFlatThreads) {
-        int ch = static_cast<int>((row_first + r) % C_);
-        prm[r * 4 + 0] = static_cast<C>(mean[ch * pstride]);
-        prm[r * 4 + 1] = InvStd<C>(static_cast<C>(var[ch * pstride]), eps);
-        prm[r * 4 + 2] = static_cast<C>(gamma[ch * pstride]);
-        prm[r * 4 + 3] = static_cast<C>(beta[ch * pstride]);
-    }
-    __syncthreads();
+    // the elements first: their loads are in flight while the parameters are fetched and staged
     const bool rows_hold_whole_vectors = L % VEC == 0;
     Vec<T, VEC> in[kBnFlatUnroll];
     int64_t idx[kBnFlatUnroll];
@@ -114,6 +107,14 @@ __global__ __launch_bounds__(kBnFlatThreads) void BnChannelsFirstKernel(const T*
             in[u] = stream_in ? LoadStreaming<Vec<T, VEC>>(src) : *reinterpret_cast<const Vec<T, VEC>*>(src);
         }
     }
+    for (int r = threadIdx.x; r < max_rows; r += kBnFlatThreads) {
+        int ch = static_cast<int>((row_first + r) % C_);
+        prm[r * 4 + 0] = static_cast<C>(mean[ch * pstride]);
+        prm[r * 4 + 1] = InvStd<C>(static_cast<C>(var[ch * pstride]), eps);
+        prm[r * 4 + 2] = static_cast<C>(gamma[ch * pstride]);
+        prm[r * 4 + 3] = static_cast<C>(beta[ch * pstride]);
+    }
+    __syncthreads();
 #pragma unroll
     for (int u = 0; u < kBnFlatUnroll; ++u) {
         if (idx[u] >= total) continue;
@@ -129,6 +130,20 @@ __global__ __launch_bounds__(kBnFlatThreads) void BnChannelsFirstKernel(const T*
                 t = t * q1;
                 t = t * q2;
                 t = t + q3;
+                o.v[e] = static_cast<T>(t);
+            }
+        } else if (L >= VEC) {  // the vector lies in one row or crosses into the next one: two parameter sets, chosen per element
+            const int here = static_cast<int>(L) - col;  // elements of this vector that belong to row r
+            const int r2 = r + 1 < max_rows ? r + 1 : r;
+            const C p0 = prm[r * 4 + 0], p1 = prm[r * 4 + 1], p2 = prm[r * 4 + 2], p3 = prm[r * 4 + 3];
+            const C n0 = prm[r2 * 4 + 0], n1 = prm[r2 * 4 + 1], n2 = prm[r2 * 4 + 2], n3 = prm[r2 * 4 + 3];
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                const bool first = e < here;
+                C t = static_cast<C>(in[u].v[e]) - (first ? p0 : n0);
+                t = t * (first ? p1 : n1);
+                t = t * (first ? p2 : n2);
+                t = t + (first ? p3 : n3);
                 o.v[e] = static_cast<T>(t);
             }
         } else {
