@@ -848,6 +848,18 @@ __global__ __launch_bounds__(256) void EighShiftKernel(T* s, int n, T shift) {
     if (i < n) s[static_cast<int64_t>(i) * n + i] += shift;
 }
 
+// The same with the shift |A|_F taken from EighNormsKernel's partial sums on the device (the arithmetic of the host path: a double
+// sum of the partials, its root rounded to T); a zero or non-finite norm shifts by nothing.
+template <typename T>
+__global__ __launch_bounds__(256) void EighShiftFromNormsKernel(T* s, int n, const T* partial) {
+    double all = 0.0;
+    for (int b = 0; b < kEighNormBlocks; ++b) all += static_cast<double>(partial[2 * b + 1]);
+    T shift = static_cast<T>(sqrt(all));
+    if (!(shift > T(0)) || !isfinite(static_cast<double>(shift))) shift = T(0);
+    const int i = static_cast<int>(blockIdx.x) * 256 + static_cast<int>(threadIdx.x);
+    if (i < n) s[static_cast<int64_t>(i) * n + i] += shift;
+}
+
 // Eigenvalue j as the Rayleigh quotient of the original matrix a0 ([n, n], symmetric) with row j of vt (the eigenvector, as the
 // one-sided sweeps leave it): lambda_j = (v . a0 v) / (v . v), stored at s[j][j] where the output pass of JacobiEighKernel looks for
 // it.  Its error is of second order in the eigenvector's, and the norm that thousands of rotations leave slightly off one cancels.
@@ -1194,12 +1206,14 @@ __device__ __forceinline__ bool SvdRotatePair(T* g, int M, int N, T* v, int p, i
 // then one launch per round of a round-robin over the blocks, in which a workgroup owns a pair of blocks (P, Q) and rotates
 // column i of P against column (i + r) mod kSvdBlock of Q in its inner round r -- kSvdBlock disjoint pairs, one per wavefront,
 // with a barrier between inner rounds (the columns stay in global memory; the workgroup's own stores are visible to it after the
-// barrier).  *rotated becomes 1 when any pair of the sweep needed a rotation.
+// barrier).  *rotated becomes 1 when any pair of the sweep needed a rotation; a launch whose `gate` points at a zero (the flag of the
+// sweep before) does nothing, which is how sweeps end without the host looking.
 constexpr int kSvdBlock = 16;
 constexpr int kSvdBlockThreads = 64 * kSvdBlock;
 template <typename T>
 __global__ __launch_bounds__(kSvdBlockThreads) void SvdBlockRoundKernel(T* g, int M, int N, T* v, int blocks, int block_round, int compute_uv,
-                                                                        int* rotated) {
+                                                                        int* rotated, const int* gate) {
+    if (gate != nullptr && *gate == 0) return;  // the previous sweep rotated nothing: the decomposition has converged
     const int wave = static_cast<int>(threadIdx.x) >> 6, lane = static_cast<int>(threadIdx.x) & 63;
     bool any = false;
     if (block_round < 0) {
@@ -1274,7 +1288,8 @@ __device__ __forceinline__ bool SvdRotateLdsPair(T* gp, T* gq, int M, T* jp, T* 
 
 template <typename T>
 __global__ __launch_bounds__(kSvdBlockThreads) void SvdBlockLdsRoundKernel(T* g, int M, int N, T* v, int blocks, int block_round, int compute_uv,
-                                                                           int* rotated) {
+                                                                           int* rotated, const int* gate) {
+    if (gate != nullptr && *gate == 0) return;  // the previous sweep rotated nothing: the decomposition has converged
     extern __shared__ __align__(16) char svd_lds[];
     T* cols = reinterpret_cast<T*>(svd_lds);  // [kSvdPair][M]: local column l is column l of block P, or l - kSvdBlock of block Q
     T* jm = cols + static_cast<size_t>(kSvdPair) * M;  // [kSvdPair][kSvdPair], column by column
@@ -1532,12 +1547,32 @@ void AllowLargeLds(const void* kernel, int slot) {
     }
 }
 
-// The one-sided Jacobi sweeps over g ([N][M], column by column) as launches of column-block rounds, until a sweep rotates nothing:
-// the host reads one flag per sweep (a stream wait).  v ([N][N], column by column) starts as the identity and takes the rotations
-// when compute_uv is set.  rotated: kSvdMaxSweeps ints of device memory.
+__global__ __launch_bounds__(64) void ClearFlagsKernel(int* flags, int n) {
+    const int i = static_cast<int>(threadIdx.x);
+    if (i < n) flags[i] = 0;
+}
+
+inline bool StreamIsCapturing(hipStream_t st) {
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    HIPCX_CHECK_HIP(hipStreamIsCapturing(st, &status));
+    return status != hipStreamCaptureStatusNone;
+}
+
+// Sweeps issued on a stream that is being captured into a graph: the host cannot look at a flag there, so a fixed number of sweeps is
+// recorded and every launch is gated on the flag of the sweep before it (one-sided Jacobi in float32 / float64 needs 6-12 sweeps on
+// the matrices of the tests, about 15 on graded ones).
+constexpr int kSvdCapturedSweeps = 30;
+static_assert(kSvdCapturedSweeps <= kSvdMaxSweeps && kSvdMaxSweeps <= 64, "one flag per sweep, cleared by one wavefront");
+
+// The one-sided Jacobi sweeps over g ([N][M], column by column) as launches of column-block rounds, until a sweep rotates nothing.
+// Outside graph capture the host reads one flag per sweep (a stream wait) and stops launching; under capture it launches
+// kSvdCapturedSweeps gated sweeps and never waits, with the same results (a gated-off launch is the launch the host would not have
+// made).  v ([N][N], column by column) starts as the identity and takes the rotations when compute_uv is set.  rotated:
+// kSvdMaxSweeps ints of device memory.
 template <typename T>
 void RunBlockJacobiSweeps(T* g, int64_t M, int64_t N, T* v, bool compute_uv, int* rotated, hipStream_t st) {
-    HIPCX_CHECK_HIP(hipMemsetAsync(rotated, 0, kSvdMaxSweeps * sizeof(int), st));
+    const bool captured = StreamIsCapturing(st);
+    hipLaunchKernelGGL(ClearFlagsKernel, dim3(1), dim3(64), 0, st, rotated, kSvdMaxSweeps);  // a kernel, not a memset node
     if (compute_uv) hipLaunchKernelGGL(IdentityFillKernel<T>, dim3(static_cast<unsigned>((N * N + 255) / 256)), dim3(256), 0, st, v, static_cast<int>(N));
     const int blocks = static_cast<int>((N + kSvdBlock - 1) / kSvdBlock);
     const int players = blocks + (blocks & 1);
@@ -1545,17 +1580,20 @@ void RunBlockJacobiSweeps(T* g, int64_t M, int64_t N, T* v, bool compute_uv, int
     const bool in_lds = lds_bytes <= kSvdBlockLdsMax;
     // beyond the 64 KiB a launch gets unasked, the kernel is told once per device that it may have more
     if (in_lds && lds_bytes > 60 * 1024) AllowLargeLds(reinterpret_cast<const void*>(SvdBlockLdsRoundKernel<T>), std::is_same<T, float>::value ? 2 : 3);
-    for (int sweep = 0; sweep < kSvdMaxSweeps; ++sweep) {
+    const int max_sweeps = captured ? kSvdCapturedSweeps : kSvdMaxSweeps;
+    for (int sweep = 0; sweep < max_sweeps; ++sweep) {
+        const int* gate = captured && sweep > 0 ? rotated + sweep - 1 : nullptr;
         for (int round = -1; round < players - 1; ++round) {  // -1: the pairs inside every block
             const dim3 grid(static_cast<unsigned>(round < 0 ? blocks : players / 2));
             if (in_lds) {
                 hipLaunchKernelGGL(SvdBlockLdsRoundKernel<T>, grid, dim3(kSvdBlockThreads), lds_bytes, st, g, static_cast<int>(M), static_cast<int>(N), v,
-                                   blocks, round, compute_uv ? 1 : 0, rotated + sweep);
+                                   blocks, round, compute_uv ? 1 : 0, rotated + sweep, gate);
             } else {
                 hipLaunchKernelGGL(SvdBlockRoundKernel<T>, grid, dim3(kSvdBlockThreads), 0, st, g, static_cast<int>(M), static_cast<int>(N), v, blocks,
-                                   round, compute_uv ? 1 : 0, rotated + sweep);
+                                   round, compute_uv ? 1 : 0, rotated + sweep, gate);
             }
         }
+        if (captured) continue;
         int any = 0;
         HIPCX_CHECK_HIP(hipMemcpyAsync(&any, rotated + sweep, sizeof(int), hipMemcpyDeviceToHost, st));
         HIPCX_CHECK_HIP(hipStreamSynchronize(st));
@@ -1776,6 +1814,21 @@ int hipcx_syevd(const hipcx_array* a, const hipcx_array* w, const hipcx_array* v
                 T* partial = cs + 4 * ((n + 1) / 2);
                 std::vector<T> sums(2 * kEighNormBlocks);
                 hipLaunchKernelGGL(EighNormsKernel<T>, dim3(kEighNormBlocks), dim3(256), 0, st, s, static_cast<int>(n), partial);
+                if (StreamIsCapturing(st)) {
+                    // no host wait under graph capture: the shift is taken on the device and the sweeps are gated launches.  A zero
+                    // matrix goes the same way (nothing rotates, every Rayleigh quotient is zero).
+                    T* a0 = reinterpret_cast<T*>(ws + EighOriginalOffset(n));
+                    HIPCX_CHECK_HIP(hipMemcpyAsync(a0, s, static_cast<size_t>(n * n * it), hipMemcpyDeviceToDevice, st));
+                    hipLaunchKernelGGL(EighShiftFromNormsKernel<T>, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, st, s, static_cast<int>(n),
+                                       partial);
+                    RunBlockJacobiSweeps(s, n, n, vs, true, reinterpret_cast<int*>(cs), st);
+                    hipLaunchKernelGGL(EighRayleighKernel<T>, dim3(static_cast<unsigned>(n)), dim3(256), static_cast<size_t>(n * it), st, a0, vs,
+                                       static_cast<int>(n), s);
+                    hipLaunchKernelGGL(JacobiEighKernel<T>, dim3(1), dim3(kLinalgThreads), lds, st, s, static_cast<T*>(v->data),
+                                       static_cast<T*>(w->data), static_cast<int>(n), compute_v ? 1 : 0, compute_v ? v->strides[0] / it : 0,
+                                       compute_v ? v->strides[1] / it : 0, w->strides[0] / it, vs, 0);
+                    return;
+                }
                 HIPCX_CHECK_HIP(hipMemcpyAsync(sums.data(), partial, sums.size() * sizeof(T), hipMemcpyDeviceToHost, st));
                 HIPCX_CHECK_HIP(hipStreamSynchronize(st));
                 double all = 0.0;

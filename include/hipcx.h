@@ -447,8 +447,10 @@ int hipcx_cholesky(const hipcx_array* a, const hipcx_array* out, int32_t* error_
  * up to the sign of each column (and up to a rotation inside an eigenspace of a repeated eigenvalue).  Up to 64 rows a two-sided
  * cyclic Jacobi runs in one workgroup; beyond that the columns of A + |A|_F I are made orthogonal by the one-sided block sweeps
  * of hipcx_svd (the rotations' product holds the eigenvectors, the eigenvalues are their Rayleigh quotients with A), and the
- * call waits for the stream once for the norm and once per sweep to read whether anything was rotated (so it cannot be captured
- * into a graph).
+ * call waits for the stream once for the norm and once per sweep to read whether anything was rotated.  On a stream that is being
+ * captured into a graph it waits for nothing: the norm stays on the device and 30 sweeps are recorded, each launch gated on the
+ * flag of the sweep before it (the same rotations, the same results bit for bit; a matrix that needs more than 30 sweeps would be
+ * left short of convergence there, against 60 with the host in the loop).
  * w: [n], v: [n, n], any strides, a's dtype.  Workspace: hipcx_syevd_workspace_size(a) bytes.  n <= 4096. */
 size_t hipcx_syevd_workspace_size(const hipcx_array* a);
 int hipcx_syevd(const hipcx_array* a, const hipcx_array* w, const hipcx_array* v, char uplo, int compute_v, void* workspace,
@@ -474,8 +476,9 @@ int hipcx_qr(const hipcx_array* a, const hipcx_array* q, const hipcx_array* r, c
  * sign of u[:, i] and vt[i, :] (and a rotation inside the space of a repeated value; the columns that complete a full u / vt, or
  * that belong to zero singular values, are some orthonormal basis of the same space).  Up to k = 64 the sweeps run in one
  * workgroup; beyond that a sweep is k / 16 launches over blocks of 16 columns (a workgroup per pair of blocks, a wavefront per
- * column pair), and the call waits for the stream once per sweep to read whether anything was rotated (so it cannot be captured
- * into a graph).  max(m, n) <= 4096. */
+ * column pair), and the call waits for the stream once per sweep to read whether anything was rotated -- except on a stream that
+ * is being captured into a graph, where 30 sweeps are recorded, each launch gated on the flag of the sweep before it (same
+ * rotations, same results; see hipcx_syevd).  max(m, n) <= 4096. */
 size_t hipcx_svd_workspace_size(const hipcx_array* a);
 int hipcx_svd(const hipcx_array* a, const hipcx_array* u, const hipcx_array* s, const hipcx_array* vt, int full_matrices, int compute_uv,
               void* workspace, size_t workspace_bytes, void* stream);

@@ -403,3 +403,39 @@ def test_one_workgroup_limits():
     with pytest.raises(chx.ChainerxNotImplementedError):
         chx.svd(big)
 
+
+
+def test_svd_and_eigh_are_captured_into_a_graph_without_host_waits():
+    """Above one workgroup's size the Jacobi sweeps are separate launches that end when a sweep rotates nothing.  Outside capture the
+    host reads that flag; on a capturing stream (where it cannot) a fixed number of sweeps is recorded, each gated on the flag of the
+    sweep before it.  Both run the same rotations: the replays equal the eager results bit for bit, also after the input changed."""
+    import torch
+    import chainer_amd as chx
+    from chainer_amd import routines
+    from chainer_amd.graph import capture
+    rng = np.random.default_rng(77)
+    n = 150
+    a0 = rng.standard_normal((n, n)).astype(np.float32)
+    a1 = (rng.standard_normal((n, n)) * np.linspace(1e-3, 1.0, n)).astype(np.float32)  # graded columns: more sweeps
+    A = chx.array(a0)
+    S = chx.array(((a0 + a0.T) / 2).astype(np.float32))
+    g_svd = capture(lambda: chx.svd(A, full_matrices=False))
+    g_eig = capture(lambda: chx.eigh(S))
+    for a in (a0, a1, np.zeros((n, n), np.float32), a0):
+        sym = ((a + a.T) / 2).astype(np.float32)
+        routines._copy_into(A, chx.array(a))  # new values in the buffers the graphs read
+        routines._copy_into(S, chx.array(sym))
+        u, s, vt = (t.get() for t in chx.svd(A, full_matrices=False))
+        w, v = (t.get() for t in chx.eigh(S))
+        g_svd.replay()
+        g_eig.replay()
+        torch.cuda.synchronize()
+        ur, sr, vtr = (t.get() for t in g_svd.result)
+        wr, vr = (t.get() for t in g_eig.result)
+        assert np.array_equal(sr, s) and np.array_equal(ur, u) and np.array_equal(vtr, vt)
+        assert np.array_equal(wr, w) and np.array_equal(vr, v)
+        if a.any():
+            assert np.abs((ur.astype(np.float64) * sr) @ vtr - a).max() <= 1e-4 * np.abs(a).max() * n
+            assert np.abs(sym.astype(np.float64) @ vr - vr.astype(np.float64) * wr).max() <= 1e-4 * np.abs(sym).max() * n
+    g_svd.release()
+    g_eig.release()
