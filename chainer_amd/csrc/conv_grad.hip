@@ -317,6 +317,12 @@ void RunLayouts(const GradWeightArgs& a, hipStream_t stream) {
 }  // namespace
 }  // namespace hipcx
 
+namespace hipcx {
+// nd_ops.hip: arrays without exactly two spatial axes
+void ConvGradWeightNd(const hipcx_array* x, const hipcx_array* gy, const int64_t* stride, const int64_t* pad, int cover_all, const hipcx_array* gw,
+                      void* stream);
+}  // namespace hipcx
+
 using namespace hipcx;
 
 // conv.hip: accumulated batch of matrix products on the MFMA kernel
@@ -406,6 +412,7 @@ size_t hipcx_conv_grad_weight_workspace_size(const hipcx_array* x, const hipcx_a
                                              const int64_t* pad, int cover_all) {
     try {
         if (x == nullptr || gy == nullptr || gw == nullptr) return 0;
+        if (x->ndim != 4) return 0;  // the n-axis kernel needs none
         GradWeightPlan pl = PlanGradWeight(x, gy, gw, stride, pad, cover_all);
         hipcx_array out = GwAsMatrix(gw);
         // Which path the call takes depends on the alignment of the data pointers, which a caller sizing its workspace from
@@ -423,6 +430,10 @@ size_t hipcx_conv_grad_weight_workspace_size(const hipcx_array* x, const hipcx_a
 int hipcx_conv_grad_weight(const hipcx_array* x, const hipcx_array* gy, const int64_t* stride, const int64_t* pad, int cover_all,
                            const hipcx_array* gw, void* workspace, size_t workspace_bytes, void* stream) {
     return Guard([&] {
+        if (x != nullptr && x->ndim != 4) {  // not two spatial axes: nd_ops.hip
+            ConvGradWeightNd(x, gy, stride, pad, cover_all, gw, stream);
+            return;
+        }
         GradWeightPlan pl = PlanGradWeight(x, gy, gw, stride, pad, cover_all);
         hipcx_array out = GwAsMatrix(gw);
         if (out.shape[0] == 0 || out.shape[1] == 0) return;

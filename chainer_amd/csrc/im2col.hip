@@ -264,6 +264,12 @@ void AddBias(const hipcx_array* b, const hipcx_array* out, void* stream) {
 }  // namespace
 }  // namespace hipcx
 
+namespace hipcx {
+// nd_ops.hip: arrays without exactly two spatial axes
+void ConvTransposeNd(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, const int64_t* stride, const int64_t* pad,
+                     const hipcx_array* out, void* stream);
+}  // namespace hipcx
+
 using namespace hipcx;
 
 extern "C" {
@@ -305,6 +311,7 @@ int hipcx_col2im(const hipcx_array* col, const int64_t* stride, const int64_t* p
 
 size_t hipcx_conv_transpose_workspace_size(const hipcx_array* x, const hipcx_array* w, const int64_t* stride, const int64_t* pad,
                                            const hipcx_array* out) {
+    if (x != nullptr && x->ndim != 4) return 0;  // the n-axis kernel needs none
     try {
         return PlanTranspose(x, w, nullptr, stride, pad, out, reinterpret_cast<char*>(uintptr_t{1} << 20)).total;
     } catch (...) {
@@ -315,6 +322,10 @@ size_t hipcx_conv_transpose_workspace_size(const hipcx_array* x, const hipcx_arr
 int hipcx_conv_transpose(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b, const int64_t* stride, const int64_t* pad,
                          const hipcx_array* out, void* workspace, size_t workspace_bytes, void* stream) {
     return Guard([&] {
+        if (x != nullptr && x->ndim != 4) {  // not two spatial axes: nd_ops.hip
+            ConvTransposeNd(x, w, b, stride, pad, out, stream);
+            return;
+        }
         char* base = static_cast<char*>(workspace);
         TransposePlan pl = PlanTranspose(x, w, b, stride, pad, out, base != nullptr ? base : reinterpret_cast<char*>(uintptr_t{1} << 20));
         if (TotalSize(out) == 0) return;

@@ -11,6 +11,7 @@
 // Channels-last data is processed VEC channels per thread with 16-byte accesses; any other
 // layout one element per thread, with the thread order following the output's fastest axis.
 #include "common.h"
+#include "window_argmax.h"
 
 namespace hipcx {
 namespace {
@@ -406,70 +407,19 @@ struct PoolGradArgs {
     int* win_index;  // max only: ArgMax of every window, dense [N, C, OH, OW]
 };
 
-template <typename V>
-struct WinBest {
-    V v;
-    int i;  // < 0: empty
-};
-
-template <typename V>
-__device__ __forceinline__ void WinReduce(WinBest<V> next, WinBest<V>& acc) {  // ArgMax's rule: a later element must be strictly larger
-    if (next.i < 0) return;
-    if (acc.i < 0 || acc.v < next.v) acc = next;
-}
-
-// ArgMax over the kh x kw window of output (oh, ow) as the native backend computes it: the reduction loop of CX/native/reduce.h:46-83
-// over the Im2Col'ed window, whose out-of-image taps hold the lowest value (CX/native/native_device/pool.cc:97-113).
+// ArgMax over the kh x kw window of output (oh, ow) as the native backend computes it: the reduction order of window_argmax.h over the
+// Im2Col'ed window, whose out-of-image taps hold the lowest value (CX/native/native_device/pool.cc:97-113).
 template <typename T>
 __device__ int WindowArgMax(const PoolGradArgs& p, const T* xb, int oh, int ow) {
-    using V = std::conditional_t<std::is_same<T, half_t>::value, float, std::conditional_t<std::is_same<T, bool>::value, int, T>>;
-    using B = WinBest<V>;
+    using V = win_value_t<T>;
     const int h0 = oh * p.sh - p.ph, w0 = ow * p.sw - p.pw;
-    const int len = p.kh * p.kw;
-    int i = 0, r = 0, q = 0;
-    auto next_elem = [&]() -> B {
+    int r = 0, q = 0;
+    return NativeOrderArgMax<V>(p.kh * p.kw, [&](int) -> V {
         const int ih = h0 + r, iw = w0 + q;
-        T v = (ih >= 0 && ih < p.H && iw >= 0 && iw < p.W) ? xb[ih * p.xsH + iw * p.xsW] : Lowest<T>();
-        B b{static_cast<V>(v), i};
-        ++i;
+        const T v = (ih >= 0 && ih < p.H && iw >= 0 && iw < p.W) ? xb[ih * p.xsH + iw * p.xsW] : Lowest<T>();
         if (++q == p.kw) q = 0, ++r;
-        return b;
-    };
-    const int main_len = len - (len % 4);
-    B accum{V(0), -1};
-    if (main_len <= 32) {  // one block of the tree: groups of four, then the tail (every usual window)
-        while (i < main_len) {
-            B p0 = next_elem();
-            WinReduce(next_elem(), p0);
-            B p1 = next_elem();
-            WinReduce(next_elem(), p1);
-            WinReduce(p1, p0);
-            WinReduce(p0, accum);
-        }
-        while (i < len) WinReduce(next_elem(), accum);
-        return accum.i;
-    }
-    B tree[26];
-    while (i < main_len) {
-        if (i != 0 && i % 32 == 0) {
-            int lvl = 0;
-            for (int k = i >> 1; k % 32 == 0; k >>= 1, ++lvl) WinReduce(tree[lvl], accum);
-            tree[lvl] = accum;
-            accum = B{V(0), -1};
-        }
-        B p0 = next_elem();
-        WinReduce(next_elem(), p0);
-        B p1 = next_elem();
-        WinReduce(next_elem(), p1);
-        WinReduce(p1, p0);
-        WinReduce(p0, accum);
-    }
-    while (i < len) WinReduce(next_elem(), accum);
-    int lvl = 0;
-    for (int k = (len / 4 - 1) / 8; k > 0; k >>= 1, ++lvl) {
-        if (k & 1) WinReduce(tree[lvl], accum);
-    }
-    return accum.i;
+        return static_cast<V>(v);
+    });
 }
 
 template <typename T, typename IdxT>
@@ -929,6 +879,10 @@ void RunPoolGrad(const PoolGradArgs& p, hipStream_t stream) {
 
 namespace hipcx {
 // nd_ops.hip: arrays without exactly two spatial axes
+void PoolGradNd(bool is_max, const hipcx_array* x, const hipcx_array* gout, const int64_t* ksize, const int64_t* stride, const int64_t* pad,
+                int cover_all, int pad_mode, const hipcx_array* gx, void* stream);
+void MaxPoolGradGradNd(const hipcx_array* x, const hipcx_array* ggx, const int64_t* ksize, const int64_t* stride, const int64_t* pad, int cover_all,
+                       const hipcx_array* ggout, void* stream);
 void PoolNd(bool is_max, const hipcx_array* x, const int64_t* ksize, const int64_t* stride, const int64_t* pad, int cover_all, int pad_mode,
             const hipcx_array* out, void* stream);
 }  // namespace hipcx
@@ -980,7 +934,11 @@ size_t hipcx_max_pool_grad_workspace_size(const hipcx_array* gout) {
 int hipcx_max_pool_grad(const hipcx_array* x, const hipcx_array* gout, const int64_t* kernel_size, const int64_t* stride,
                         const int64_t* pad, int cover_all, const hipcx_array* gx, void* workspace, size_t workspace_bytes, void* stream) {
     return Guard([&] {
-        HIPCX_REQUIRE(x != nullptr, HIPCX_CHAINERX_ERROR, "null array x");
+        HIPCX_REQUIRE(x != nullptr && gx != nullptr, HIPCX_CHAINERX_ERROR, "null array");
+        if (x->ndim != 4) {  // not two spatial axes: nd_ops.hip
+            PoolGradNd(true, x, gout, kernel_size, stride, pad, cover_all, HIPCX_PAD_ZERO, gx, stream);
+            return;
+        }
         PoolGradArgs p = MakeGradArgs(x, gout, kernel_size, stride, pad, cover_all, gx);
         const size_t need = hipcx_max_pool_grad_workspace_size(gout);
         HIPCX_REQUIRE(need == 0 || (workspace != nullptr && workspace_bytes >= need), HIPCX_CHAINERX_ERROR,
@@ -1003,6 +961,10 @@ int hipcx_average_pool_grad(const hipcx_array* gout, const int64_t* kernel_size,
     return Guard([&] {
         HIPCX_REQUIRE(pad_mode == HIPCX_PAD_ZERO || pad_mode == HIPCX_PAD_IGNORE, HIPCX_CHAINERX_ERROR, "invalid pad mode");
         HIPCX_REQUIRE(gx != nullptr && IsFloatDtype(gx->dtype), HIPCX_DTYPE_ERROR, "cannot apply average pooling to non-float arrays");
+        if (gx->ndim != 4) {  // not two spatial axes: nd_ops.hip
+            PoolGradNd(false, nullptr, gout, kernel_size, stride, pad, 0, pad_mode, gx, stream);
+            return;
+        }
         PoolGradArgs p = MakeGradArgs(nullptr, gout, kernel_size, stride, pad, 0, gx);
         p.pad_mode = pad_mode;
         VisitFloatDtype(gx->dtype, [&](auto tag) {
@@ -1016,6 +978,10 @@ int hipcx_max_pool_grad_grad(const hipcx_array* x, const hipcx_array* ggx, const
                              const int64_t* pad, int cover_all, const hipcx_array* ggout, void* stream) {
     return Guard([&] {
         HIPCX_REQUIRE(x != nullptr && ggx != nullptr, HIPCX_CHAINERX_ERROR, "null array");
+        if (x->ndim != 4) {  // not two spatial axes: nd_ops.hip
+            MaxPoolGradGradNd(x, ggx, kernel_size, stride, pad, cover_all, ggout, stream);
+            return;
+        }
         // the geometry helper wants (x, window-shaped array, image-shaped array): here the image-shaped one is ggx
         PoolGradArgs p = MakeGradArgs(x, ggout, kernel_size, stride, pad, cover_all, ggx);
         // swap roles: gout/gs* <- ggx (image), gx/ds* <- ggout (windows)

@@ -880,18 +880,20 @@ public:
         Device& device = x.device();
         device.CheckDevicesCompatible(x, gy);
         SetDeviceScope scope{device.index()};
-        if (x.ndim() == 4 && GetKind(w_dtype) == DtypeKind::kFloat) {
-            // one entry: Im2Col and the gy transpose as one kernel each, then the matrix product (split over the reduction)
+        if (GetKind(w_dtype) == DtypeKind::kFloat) {
+            // one entry, any number of spatial axes (native_device/conv.cc:91-124).  Two axes: Im2Col and the gy transpose as one
+            // kernel each, then the matrix product (split over the reduction); otherwise a plain kernel with the native arithmetic
             Array xc = AsContiguous(x.dtype() == w_dtype ? x : x.AsType(w_dtype));
             Array gc = AsContiguous(gy.dtype() == w_dtype ? gy : gy.AsType(w_dtype));
             Array gw = Empty(w_shape, w_dtype, device);
             hipcx_array cx = ToC(xc), cg = ToC(gc), cw = ToC(gw);
-            int64_t st[2] = {stride[0], stride[1]}, pd[2] = {pad[0], pad[1]};
-            size_t ws_bytes = hipcx_conv_grad_weight_workspace_size(&cx, &cg, &cw, st, pd, cover_all ? 1 : 0);
+            std::vector<int64_t> st(stride.begin(), stride.end()), pd(pad.begin(), pad.end());
+            size_t ws_bytes = hipcx_conv_grad_weight_workspace_size(&cx, &cg, &cw, st.data(), pd.data(), cover_all ? 1 : 0);
             std::shared_ptr<void> ws = device.Allocate(ws_bytes);
-            Check(hipcx_conv_grad_weight(&cx, &cg, st, pd, cover_all ? 1 : 0, &cw, ws.get(), ws_bytes, nullptr));
+            Check(hipcx_conv_grad_weight(&cx, &cg, st.data(), pd.data(), cover_all ? 1 : 0, &cw, ws.get(), ws_bytes, nullptr));
             return gw;
         }
+        if (x.ndim() != 4) throw NotImplementedError{"hip convolution of non-floating dtypes supports 2 spatial dimensions."};
         Array col = HipIm2Col(x, Dims{w_shape[2], w_shape[3]}, stride, pad, cover_all, 0);
         return native::TensorDot(gy, col, Axes{0, 2, 3}, Axes{0, 4, 5}, w_dtype);  // dispatches DotKernel on this backend
     }
@@ -903,26 +905,29 @@ public:
     Array Call(const Array& x, const Array& w, const absl::optional<Array>& b, const Dims& stride, const Dims& pad, const Dims& out_size,
                Dtype out_dtype, const absl::optional<Array>& out) override {
         if (out.has_value()) throw NotImplementedError{"Passing out as an argument is not yet supported."};
-        if (x.ndim() != 4) throw NotImplementedError{"hip convolution supports 2 spatial dimensions."};
         Device& device = x.device();
         device.CheckDevicesCompatible(x, w);
         if (b.has_value()) device.CheckDevicesCompatible(x, *b);
         SetDeviceScope scope{device.index()};
         if (GetKind(out_dtype) == DtypeKind::kFloat) {
-            // one entry: it picks the flipped forward convolution (stride 1), the scattered 1x1 convolution or the native
-            // composition (matrix product over the input channels, col2im, bias) by itself
+            // one entry, any number of spatial axes (native_device/conv.cc:126-160).  Two axes: it picks the flipped forward
+            // convolution (stride 1), the scattered 1x1 convolution or the native composition (matrix product over the input
+            // channels, col2im, bias) by itself; otherwise a plain kernel with the native arithmetic
             Array xc = x.dtype() == out_dtype ? x : x.AsType(out_dtype);
             Array wc = w.dtype() == out_dtype ? w : w.AsType(out_dtype);
             absl::optional<Array> bc = b.has_value() ? absl::optional<Array>{b->dtype() == out_dtype ? *b : b->AsType(out_dtype)} : absl::nullopt;
-            Array actual_out = Empty(Shape{x.shape()[0], w.shape()[1], out_size[0], out_size[1]}, out_dtype, device);
+            Shape out_shape{x.shape()[0], w.shape()[1]};
+            std::copy(out_size.begin(), out_size.end(), std::back_inserter(out_shape));
+            Array actual_out = Empty(out_shape, out_dtype, device);
             hipcx_array cx = ToC(xc), cw = ToC(wc), co = ToC(actual_out), cb{};
             if (bc.has_value()) cb = ToC(*bc);
-            int64_t st[2] = {stride[0], stride[1]}, pd[2] = {pad[0], pad[1]};
-            size_t ws_bytes = hipcx_conv_transpose_workspace_size(&cx, &cw, st, pd, &co);
+            std::vector<int64_t> st(stride.begin(), stride.end()), pd(pad.begin(), pad.end());
+            size_t ws_bytes = hipcx_conv_transpose_workspace_size(&cx, &cw, st.data(), pd.data(), &co);
             std::shared_ptr<void> ws = device.Allocate(ws_bytes);
-            Check(hipcx_conv_transpose(&cx, &cw, bc.has_value() ? &cb : nullptr, st, pd, &co, ws.get(), ws_bytes, nullptr));
+            Check(hipcx_conv_transpose(&cx, &cw, bc.has_value() ? &cb : nullptr, st.data(), pd.data(), &co, ws.get(), ws_bytes, nullptr));
             return actual_out;
         }
+        if (x.ndim() != 4) throw NotImplementedError{"hip convolution of non-floating dtypes supports 2 spatial dimensions."};
         // other dtypes: the native composition on this backend's kernels (TensorDot dispatches DotKernel here)
         Array col = native::TensorDot(w, x, Axes{0}, Axes{1}, out_dtype);  // [C_out, kh, kw, N, H, W]
         Array actual_out = HipCol2Im(col.Transpose(Axes{3, 0, 1, 2, 4, 5}), stride, pad, out_size);
@@ -1022,10 +1027,10 @@ public:
         Array actual_gx = Empty(x.shape(), x.dtype(), device);
         const Array& g = gout.dtype() == x.dtype() ? gout : gout.AsType(x.dtype());
         hipcx_array cx = ToC(x), cg = ToC(g), cgx = ToC(actual_gx);
-        int64_t k[2] = {kernel_size[0], kernel_size[1]}, s[2] = {stride[0], stride[1]}, p[2] = {pad[0], pad[1]};
+        std::vector<int64_t> k(kernel_size.begin(), kernel_size.end()), s(stride.begin(), stride.end()), p(pad.begin(), pad.end());  // any rank
         size_t ws_bytes = hipcx_max_pool_grad_workspace_size(&cg);
         std::shared_ptr<void> ws = device.Allocate(ws_bytes);
-        Check(hipcx_max_pool_grad(&cx, &cg, k, s, p, st.cover_all() ? 1 : 0, &cgx, ws.get(), ws_bytes, nullptr));
+        Check(hipcx_max_pool_grad(&cx, &cg, k.data(), s.data(), p.data(), st.cover_all() ? 1 : 0, &cgx, ws.get(), ws_bytes, nullptr));
         std::unique_ptr<MaxPoolGradGradState> grad_grad_state = return_state ? std::make_unique<HipMaxPoolGradGradState>(x) : nullptr;
         return std::make_tuple(std::move(actual_gx), std::move(grad_grad_state));
     }
@@ -1045,8 +1050,8 @@ public:
         Array actual_ggout = Empty(PoolOutShape(x, kernel_size, stride, pad, cover_all), x.dtype(), device);
         const Array& g = ggx.dtype() == x.dtype() ? ggx : ggx.AsType(x.dtype());
         hipcx_array cx = ToC(x), cg = ToC(g), co = ToC(actual_ggout);
-        int64_t k[2] = {kernel_size[0], kernel_size[1]}, s[2] = {stride[0], stride[1]}, p[2] = {pad[0], pad[1]};
-        Check(hipcx_max_pool_grad_grad(&cx, &cg, k, s, p, cover_all ? 1 : 0, &co, nullptr));
+        std::vector<int64_t> k(kernel_size.begin(), kernel_size.end()), s(stride.begin(), stride.end()), p(pad.begin(), pad.end());  // any rank
+        Check(hipcx_max_pool_grad_grad(&cx, &cg, k.data(), s.data(), p.data(), cover_all ? 1 : 0, &co, nullptr));
         return actual_ggout;
     }
 };
@@ -1066,9 +1071,9 @@ public:
         Array actual_gx = Empty(x.shape(), x.dtype(), device);
         const Array& g = gout.dtype() == x.dtype() ? gout : gout.AsType(x.dtype());
         hipcx_array cg = ToC(g), cgx = ToC(actual_gx);
-        int64_t k[2] = {kernel_size[0], kernel_size[1]}, s[2] = {stride[0], stride[1]}, p[2] = {pad[0], pad[1]};
+        std::vector<int64_t> k(kernel_size.begin(), kernel_size.end()), s(stride.begin(), stride.end()), p(pad.begin(), pad.end());  // any rank
         int mode = pad_mode == AveragePoolPadMode::kZero ? HIPCX_PAD_ZERO : HIPCX_PAD_IGNORE;
-        Check(hipcx_average_pool_grad(&cg, k, s, p, mode, &cgx, nullptr));
+        Check(hipcx_average_pool_grad(&cg, k.data(), s.data(), p.data(), mode, &cgx, nullptr));
         return actual_gx;
     }
 };

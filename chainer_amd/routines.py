@@ -1502,13 +1502,31 @@ def tensordot(a, b, a_axes, b_axes, out_dtype=None):
 COMPOSE_CONV_GRAD_WEIGHT = False
 
 
+def _conv_grad_weight_nd(w_dtype, w_shape, x, gy, stride, pad, cover_all):
+    """ConvGradWeight with other than two spatial axes: one plain kernel with the native composition's arithmetic."""
+    n = x.ndim - 2
+    if x.ndim < 2 or gy.ndim != x.ndim or len(w_shape) != x.ndim:
+        raise _lib.DimensionError('x, gy and w need the same number of dimensions')
+    stride, pad = _pair(stride, n), _pair(pad, n)
+    dims = tuple(conv_out_dim(x.shape[2 + d], w_shape[2 + d], stride[d], pad[d], cover_all) for d in range(n))
+    if gy.shape != (x.shape[0], w_shape[0]) + dims or w_shape[1] != x.shape[1]:
+        raise _lib.DimensionError('gy has the wrong shape')
+    wdt = numpy.dtype(w_dtype)
+    if _kind(wdt) != 3:
+        raise _lib.DtypeError('the gradient with respect to the filters needs a floating point dtype')
+    gw = ndarray.empty(tuple(w_shape), wdt)
+    _lib.call('hipcx_conv_grad_weight', x.astype(wdt, False).desc(), gy.astype(wdt, False).desc(), _i64(stride), _i64(pad),
+              int(bool(cover_all)), gw.desc(), ctypes.c_void_p(0), 0, current_stream())
+    return gw
+
+
 def conv_grad_weight(w_dtype, w_shape, x, gy, stride=1, pad=0, cover_all=False):
     """ConvGradWeightKernel after the native backend (CX/native/native_device/conv.cc:91-124): Im2Col(x), then TensorDot(gy, col)
     over the batch and the output positions -> gw[K, C, kh, kw].  The same two matrices meet in the same Dot; only the col is
     laid out [C, kh, kw, N, oh, ow] so that both Dot operands have the reduction index (n, oh, ow) as their unit-stride axis
     (the MFMA kernel's layout) and no transposed copy of the col is needed (134 against 246 us for a 3x3 layer of 256 channels)."""
     if x.ndim != 4:
-        raise _lib.ChainerxNotImplementedError('only 2-D convolution is on the supported path')
+        return _conv_grad_weight_nd(w_dtype, w_shape, x, gy, stride, pad, cover_all)
     (kh, kw), (sh, sw), (ph, pw) = tuple(w_shape[2:]), _pair(stride), _pair(pad)
     n, c, h, w = x.shape
     oh = conv_out_dim(h, kh, sh, ph, cover_all)
@@ -1543,11 +1561,40 @@ COMPOSE_CONV_TRANSPOSE = False
 ROUTE_CONV_TRANSPOSE_HERE = False
 
 
+def _conv_transpose_nd(x, w, b, stride, pad, out_size, out_dtype):
+    """ConvTranspose with other than two spatial axes (the native kernel takes any number, CX/native/native_device/conv.cc:126-160):
+    one plain kernel that adds up, per output position, what Col2Im would add there, in its order."""
+    n = x.ndim - 2
+    if x.ndim < 2 or w.ndim != x.ndim:
+        raise _lib.DimensionError('Mismatched number of dimensions in input %r and weights %r.' % (x.shape, w.shape))
+    stride, pad = _pair(stride, n), _pair(pad, n)
+    if w.shape[0] != x.shape[1]:
+        raise _lib.DimensionError('Mismatched number of input channels in input of shape %r and filter of shape %r' % (x.shape, w.shape))
+    ksize = tuple(w.shape[2:])
+    if out_size is None:
+        out_size = tuple(st * (d - 1) + k - 2 * p for d, k, st, p in zip(x.shape[2:], ksize, stride, pad))
+    else:
+        out_size = _pair(out_size, n)
+        for d, o, k, st, p in zip(x.shape[2:], out_size, ksize, stride, pad):
+            if d != conv_out_dim(o, k, st, p, False) and d != conv_out_dim(o, k, st, p, True):
+                raise _lib.DimensionError('Output dims %r is incosistent.' % (out_size,))
+    if b is not None and (b.ndim != 1 or b.shape[0] != w.shape[1]):
+        raise _lib.DimensionError('Mismatched bias shape %r for weights %r.' % (b.shape, w.shape))
+    dt = numpy.dtype(out_dtype) if out_dtype is not None else (result_type(x, w, b) if b is not None else result_type(x, w))
+    if _kind(dt) != 3:
+        raise _lib.DtypeError('conv_transpose over %d spatial axes needs a floating point dtype' % n)
+    out = ndarray.empty((x.shape[0], w.shape[1]) + tuple(out_size), dt)
+    bc = b.astype(dt, False) if b is not None else None
+    _lib.call('hipcx_conv_transpose', x.astype(dt, False).desc(), w.astype(dt, False).desc(), bc.desc() if bc is not None else None,
+              _i64(stride), _i64(pad), out.desc(), ctypes.c_void_p(0), 0, current_stream())
+    return out
+
+
 def conv_transpose(x, w, b=None, stride=1, pad=0, out_size=None, out_dtype=None):
     """ConvTranspose (CX/routines/connection.cc:214-320) over the native kernel (CX/native/native_device/conv.cc:126-160):
     col = TensorDot(w, x) over the input channels, batch axis rolled first, Col2Im, bias added in place.  w: [C_in, C_out, kh, kw]."""
     if x.ndim != 4:
-        raise _lib.ChainerxNotImplementedError('only 2-D convolution is on the supported path')
+        return _conv_transpose_nd(x, w, b, stride, pad, out_size, out_dtype)
     stride, pad = _pair(stride), _pair(pad)
     if w.shape[0] != x.shape[1]:
         raise _lib.DimensionError('Mismatched number of input channels in input of shape %r and filter of shape %r' % (x.shape, w.shape))
@@ -1699,9 +1746,34 @@ def batch_norm_grad(x, gamma, gout, state, axis=None):
 COMPOSE_POOL_GRADIENTS = False
 
 
+def _pool_grad_nd(entry, x, gout, ksize, stride, pad, flag):
+    """MaxPoolGrad / AveragePoolGrad with other than two spatial axes: one plain kernel per call, the bits of the native composition.
+    `flag`: cover_all for max pooling, the pad mode for average pooling (whose output extents never use cover_all)."""
+    n = x.ndim - 2
+    is_max = entry == 'hipcx_max_pool_grad'
+    if n < 1 or gout.ndim != x.ndim or gout.dtype != x.dtype:
+        raise _lib.DimensionError('gout needs the rank and dtype of x (at least one spatial axis)')
+    if x.dtype == numpy.dtype('bool') or (not is_max and _kind(x.dtype) != 3):
+        raise _lib.DtypeError('pooling gradient: unsupported dtype %s' % x.dtype)
+    ksize = _pair(ksize, n)
+    stride = ksize if stride is None else _pair(stride, n)
+    pad = _pair(pad, n)
+    dims = tuple(conv_out_dim(x.shape[2 + d], ksize[d], stride[d], pad[d], bool(flag) if is_max else False) for d in range(n))
+    if gout.shape != tuple(x.shape[:2]) + dims:
+        raise _lib.DimensionError('gout has the wrong shape')
+    gx = ndarray.empty(x.shape, x.dtype)
+    if is_max:
+        _lib.call(entry, x.desc(), gout.desc(), _i64(ksize), _i64(stride), _i64(pad), flag, gx.desc(), ctypes.c_void_p(0), 0, current_stream())
+    else:
+        _lib.call(entry, gout.desc(), _i64(ksize), _i64(stride), _i64(pad), flag, gx.desc(), current_stream())
+    return gx
+
+
 def max_pool_grad(x, gout, ksize, stride=None, pad=0, cover_all=False):
     """MaxPoolGradKernel after the native backend (CX/native/native_device/pool.cc:97-143): Im2Col with -inf padding, ArgMax over
     the kernel axes (its tie rule picks the position), gout placed at that kernel offset of an otherwise zero col, Col2Im."""
+    if x.ndim != 4:
+        return _pool_grad_nd('hipcx_max_pool_grad', x, gout, ksize, stride, pad, int(bool(cover_all)))
     ksize = _pair(ksize)
     stride = ksize if stride is None else _pair(stride)
     pad = _pair(pad)
@@ -1736,6 +1808,18 @@ def max_pool_grad(x, gout, ksize, stride=None, pad=0, cover_all=False):
 def max_pool_grad_grad(x, ggx, ksize, stride=None, pad=0, cover_all=False):
     """MaxPoolGradGradKernel after the native backend (CX/native/native_device/pool.cc:147-177): the element of every window
     of ggx at the position where x had its maximum -- Im2Col(ggx) with the kernel axes last, flattened, Take at index + offset."""
+    if x.ndim != 4:
+        n = x.ndim - 2
+        if n < 1 or ggx.shape != x.shape or ggx.dtype != x.dtype or x.dtype == numpy.dtype('bool'):
+            raise _lib.DimensionError('ggx needs the shape and dtype of x (at least one spatial axis, not bool)')
+        ksize = _pair(ksize, n)
+        stride = ksize if stride is None else _pair(stride, n)
+        pad = _pair(pad, n)
+        dims = tuple(conv_out_dim(x.shape[2 + d], ksize[d], stride[d], pad[d], cover_all) for d in range(n))
+        ggout = ndarray.empty(tuple(x.shape[:2]) + dims, x.dtype)
+        _lib.call('hipcx_max_pool_grad_grad', x.desc(), ggx.desc(), _i64(ksize), _i64(stride), _i64(pad), int(bool(cover_all)),
+                  ggout.desc(), current_stream())
+        return ggout
     ksize = _pair(ksize)
     stride = ksize if stride is None else _pair(stride)
     pad = _pair(pad)
@@ -1759,6 +1843,8 @@ def average_pool_grad(x, gout, ksize, stride=None, pad=0, pad_mode='ignore'):
     """AveragePoolGradKernel as the native backend runs it (CX/native/native_device/pool.cc:304-346): gout (divided by the
     per-window width first in 'ignore' mode) broadcast over the kernel axes, Col2Im, and in 'zero' mode a division by the
     window size afterwards."""
+    if x.ndim != 4:
+        return _pool_grad_nd('hipcx_average_pool_grad', x, gout, ksize, stride, pad, {'zero': 1, 'ignore': 2}[pad_mode])
     ksize = _pair(ksize)
     stride = ksize if stride is None else _pair(stride)
     pad = _pair(pad)

@@ -323,7 +323,9 @@ int hipcx_conv(const hipcx_array* x, const hipcx_array* w, const hipcx_array* b,
  *   consistent with x's (CX/routines/connection.cc:268-279); all of one floating point dtype.  Stride 1 runs as one forward
  *   convolution with flipped filters, a 1x1 unpadded filter as a 1x1 convolution scattered into zeros, everything else as the
  *   native composition (matrix product over the input channels, col2im, bias).  `workspace`: 256-byte aligned device memory of
- *   hipcx_conv_transpose_workspace_size bytes. */
+ *   hipcx_conv_transpose_workspace_size bytes.  Other ranks (x[N, C_in, d_1..d_n], w[C_in, C_out, k_1..k_n], n values in `stride`
+ *   and `pad`, as the native kernel takes them, CX/native/native_device/conv.cc:126-160) run a plain one-thread-per-output kernel
+ *   that follows the native composition's order of operations (bit-identical to it); no workspace. */
 int hipcx_im2col(const hipcx_array* x, const int64_t* stride, const int64_t* pad, int cover_all, hipcx_scalar pad_value,
                  const hipcx_array* col, void* stream);
 int hipcx_col2im(const hipcx_array* col, const int64_t* stride, const int64_t* pad, const hipcx_array* out, void* stream);
@@ -422,7 +424,9 @@ int hipcx_fixed_batch_norm(const hipcx_array* x, const hipcx_array* gamma, const
  * backend's TensorDot(gy, Im2Col(x)) (CX/native/native_device/conv.cc:91-124), equal to tolerance (float accumulation).
  * inf / NaN in x or gy give the reference's inf / NaN in the reference's filter taps: the route for filters larger than 1x1 at
  * stride 1 (float16 / float32), whose sum runs over zero-padded rows in which an x value also meets zeros of a padded gy, notes
- * the input channels that hold a non-finite value and sums their taps again over the reference's windows. */
+ * the input channels that hold a non-finite value and sums their taps again over the reference's windows.
+ * Other ranks (x[N, C, d_1..d_n], gy[N, K, o_1..o_n], gw[K, C, k_1..k_n], any strides) run a plain kernel, one thread per filter
+ * element with the native Dot's order of fused multiply-adds (bit-identical to the composition); no workspace. */
 size_t hipcx_conv_grad_weight_workspace_size(const hipcx_array* x, const hipcx_array* gy, const hipcx_array* gw, const int64_t* stride,
                                              const int64_t* pad, int cover_all);
 int hipcx_conv_grad_weight(const hipcx_array* x, const hipcx_array* gy, const int64_t* stride, const int64_t* pad, int cover_all,
@@ -513,7 +517,9 @@ int hipcx_average_pool(const hipcx_array* x, const int64_t* kernel_size, const i
  * x is the forward input the reference keeps in its grad state; gx has x's shape.  Results carry the bits of the native
  * backend's Im2Col / ArgMax / Col2Im composition (CX/native/native_device/pool.cc:97-143, 304-346): contributions are added in
  * kernel-offset order with one rounding per addition, and the window maximum is chosen by ArgMax's tie and NaN rule.
- * `workspace`: device memory of hipcx_max_pool_grad_workspace_size(gout) bytes (the ArgMax of every window, one int each). */
+ * `workspace`: device memory of hipcx_max_pool_grad_workspace_size(gout) bytes (the ArgMax of every window, one int each).
+ * The three entries take any number of spatial axes like the forward ones (n values per window parameter); other than two run
+ * plain kernels with the same bits and need no workspace. */
 size_t hipcx_max_pool_grad_workspace_size(const hipcx_array* gout);
 int hipcx_max_pool_grad(const hipcx_array* x, const hipcx_array* gout, const int64_t* kernel_size, const int64_t* stride,
                         const int64_t* pad, int cover_all, const hipcx_array* gx, void* workspace, size_t workspace_bytes, void* stream);

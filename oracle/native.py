@@ -1044,6 +1044,104 @@ def average_pool_grad(x, gout, ksize, stride=None, pad=0, pad_mode='ignore'):
     return gx
 
 
+def _col2im_nd(col, stride, pad, out_size):
+    """native_internal::Col2Im over n spatial axes (CX/native/col2im.cc:22-122): col [N, C, k_1..k_n, o_1..o_n]; a zero array of the
+    padded size (stride - 1 more on the high side) receives one strided in-place `+=` per kernel offset in C order, every addition
+    rounded to the array dtype; the padding is cut off."""
+    n = len(out_size)
+    ksize, odims = col.shape[2:2 + n], col.shape[2 + n:]
+    padded = np.zeros(col.shape[:2] + tuple(out_size[d] + 2 * pad[d] + stride[d] - 1 for d in range(n)), col.dtype)
+    with np.errstate(all='ignore'):
+        for kidx in np.ndindex(*ksize):
+            sel = (slice(None), slice(None)) + tuple(slice(kidx[d], kidx[d] + stride[d] * odims[d], stride[d]) for d in range(n))
+            view = padded[sel]
+            view[...] = add(view, col[(slice(None), slice(None)) + kidx])
+    return padded[(slice(None), slice(None)) + tuple(slice(pad[d], pad[d] + out_size[d]) for d in range(n))]
+
+
+def conv_grad_weight_nd(w_shape, x, gy, stride=1, pad=0, cover_all=False):
+    """NativeConvGradWeightKernel for any number of spatial axes (conv.cc:91-124): Im2Col(x), TensorDot(gy, col) over the batch axis
+    and the output positions."""
+    x, gy = np.asarray(x), np.asarray(gy)
+    n = x.ndim - 2
+    col = _windows_nd(x, tuple(w_shape[2:]), _tuple_n(stride, n), _tuple_n(pad, n), cover_all, 0)
+    out_axes = tuple(range(2, 2 + n))
+    return _tensordot(gy, col, (0,) + out_axes, (0,) + tuple(a + n for a in out_axes))
+
+
+def conv_transpose_nd(x, w, b=None, stride=1, pad=0, out_size=None):
+    """NativeConvTransposeKernel for any number of spatial axes (conv.cc:126-160): TensorDot(w, x) over the input channels gives
+    [C_out, k_1..k_n, N, i_1..i_n], the batch axis is moved first, Col2Im, then the bias."""
+    x, w = np.asarray(x), np.asarray(w)
+    n = x.ndim - 2
+    stride, pad = _tuple_n(stride, n), _tuple_n(pad, n)
+    ksize = w.shape[2:]
+    if out_size is None:
+        out_size = tuple(st * (d - 1) + k - 2 * p for d, k, st, p in zip(x.shape[2:], ksize, stride, pad))
+    col = np.moveaxis(_tensordot(w, x, (0,), (1,)), n + 1, 0)
+    out = np.ascontiguousarray(_col2im_nd(np.ascontiguousarray(col), stride, pad, _tuple_n(out_size, n)))
+    if b is not None:
+        out = add(out, np.broadcast_to(np.asarray(b).reshape((1, -1) + (1,) * n), out.shape))
+    return out
+
+
+def max_pool_grad_nd(x, gout, ksize, stride=None, pad=0, cover_all=False):
+    """NativeMaxPoolGradKernel over n spatial axes (pool.cc:97-143): ArgMax of the windows (padding holds the lowest value; native tie
+    rule), gout placed at that kernel offset of a zero col, Col2Im."""
+    x, gout = np.asarray(x), np.asarray(gout)
+    n = x.ndim - 2
+    ksize = _tuple_n(ksize, n)
+    stride = ksize if stride is None else _tuple_n(stride, n)
+    pad = _tuple_n(pad, n)
+    col = _windows_nd(x, ksize, stride, pad, cover_all, _lowest(x.dtype))
+    idx = argmax(col, tuple(range(2, 2 + n)))
+    taps = np.arange(int(np.prod(ksize))).reshape((1, 1) + ksize + (1,) * n)
+    lift = (slice(None), slice(None)) + (None,) * n
+    gcol = np.where(idx[lift] == taps, gout[lift], np.zeros((), x.dtype)).astype(x.dtype)
+    return np.ascontiguousarray(_col2im_nd(gcol, stride, pad, x.shape[2:]))
+
+
+def max_pool_grad_grad_nd(x, ggx, ksize, stride=None, pad=0, cover_all=False):
+    """NativeMaxPoolGradGradKernel over n spatial axes (pool.cc:147-177): the element of every window of ggx at the ArgMax position
+    of x's window (a position in the padding reads the lowest value)."""
+    x, ggx = np.asarray(x), np.asarray(ggx)
+    n = x.ndim - 2
+    ksize = _tuple_n(ksize, n)
+    stride = ksize if stride is None else _tuple_n(stride, n)
+    pad = _tuple_n(pad, n)
+    idx = argmax(_windows_nd(x, ksize, stride, pad, cover_all, _lowest(x.dtype)), tuple(range(2, 2 + n)))
+    col = _windows_nd(ggx, ksize, stride, pad, cover_all, _lowest(x.dtype))
+    col = np.moveaxis(col, tuple(range(2, 2 + n)), tuple(range(2 + n, 2 + 2 * n)))  # kernel axes last
+    flat = col.reshape(col.shape[:2 + n] + (-1,))
+    return np.take_along_axis(flat, idx[..., None], axis=-1)[..., 0]
+
+
+def average_pool_grad_nd(x, gout, ksize, stride=None, pad=0, pad_mode='ignore'):
+    """NativeAveragePoolGradKernel over n spatial axes (pool.cc:304-346): gout (divided by the windows' widths first in 'ignore'
+    mode) broadcast over the kernel axes, Col2Im, divided by the window size afterwards in 'zero' mode."""
+    x, gout = np.asarray(x), np.asarray(gout)
+    n = x.ndim - 2
+    ksize = _tuple_n(ksize, n)
+    stride = ksize if stride is None else _tuple_n(stride, n)
+    pad = _tuple_n(pad, n)
+    g = gout
+    if pad_mode == 'ignore':
+        widths = None
+        for i in range(n):
+            d, k, st, p = x.shape[2 + i], ksize[i], stride[i], pad[i]
+            start = np.arange(gout.shape[2 + i]).astype(x.dtype) * _scalar_as(st, x.dtype) - _scalar_as(p, x.dtype)
+            end = start + _scalar_as(k, x.dtype)
+            w = (np.minimum(end, _scalar_as(d, x.dtype)) - np.maximum(start, _scalar_as(0, x.dtype))).astype(x.dtype)
+            widths = w if widths is None else (widths[..., None] * w).astype(x.dtype)
+        g = divide(gout, np.broadcast_to(widths, gout.shape))
+    lift = (slice(None), slice(None)) + (None,) * n
+    gcol = np.broadcast_to(g[lift], gout.shape[:2] + ksize + gout.shape[2:])
+    gx = np.ascontiguousarray(_col2im_nd(gcol, stride, pad, x.shape[2:]))
+    if pad_mode == 'zero':
+        gx = divide(gx, _scalar_as(int(np.prod(ksize)), x.dtype))
+    return gx
+
+
 def take(a, indices, axis, mode=None):
     """NativeTakeKernel (indexing.cc:31-103): mode None/'raise' raise IndexError when out of range."""
     a = np.asarray(a)

@@ -411,3 +411,55 @@ def test_batch_norm_float16_with_float32_parameters():
             tol = {'out': 2e-3, 'gx': 4e-3, 'ggamma': 2e-4, 'gbeta': 2e-4}.get(name, 2e-5)
             assert_close(k.reshape(r.shape), r, tol, 'mixed batch_norm %s %r: kernel vs oracle' % (name, shape))
             assert_close(k.reshape(r.shape), c.reshape(r.shape), tol, 'mixed batch_norm %s %r: kernel vs composition' % (name, shape))
+
+
+@pytest.mark.parametrize('dt', ['float32', 'float16', 'float64'])
+def test_gradients_over_n_axes_have_the_bits_of_the_composition(dt):
+    """ConvGradWeight, ConvTranspose and the pooling gradients with 0, 1, 3 and 4 spatial axes (the native kernels take any number,
+    conv.cc:91-160, pool.cc:97-177, 304-346; the reference's test grids): plain kernels that follow the order of the native Dot loop
+    and of Col2Im's additions, so the results equal the oracle's compositions bit for bit."""
+    import chainer_amd as chx
+    from test_oracle_pins import CONV_ND_GRID, POOL_ND_GRID
+    rng = np.random.default_rng(91)
+    for xs, ws, stride, pad in CONV_ND_GRID:
+        if len(xs) == 4:
+            continue  # two spatial axes: the dedicated kernels, tested above
+        n = len(xs) - 2
+        x = rng.standard_normal(xs).astype(dt)
+        w = rng.standard_normal(ws).astype(dt)
+        for cv in (False, True):
+            gy = rng.standard_normal(O.conv_nd(x, w, None, stride, pad, cv).shape).astype(dt)
+            what = '%s %s' % (dt, (xs, ws, stride, pad, cv))
+            gw = chx.conv_grad_weight(dt, ws, chx.array(x), chx.array(gy), stride, pad, cv)
+            assert_exact(gw.get(), O.conv_grad_weight_nd(ws, x, gy, stride, pad, cv), 'conv_grad_weight ' + what)
+            gx = chx.conv_transpose(chx.array(gy), chx.array(w), None, stride, pad, xs[2:])
+            assert_exact(gx.get(), O.conv_transpose_nd(gy, w, None, stride, pad, xs[2:]), 'conv_transpose as the data gradient ' + what)
+        wt = rng.standard_normal((xs[1], 4) + tuple(ws[2:])).astype(dt)
+        b = rng.standard_normal(4).astype(dt)
+        ref = None
+        try:
+            ref = O.conv_transpose_nd(x, wt, b, stride, pad)
+        except ValueError:
+            pass  # the default output size is not positive for this case
+        if ref is not None and ref.size:
+            got = chx.conv_transpose(chx.array(x), chx.array(wt), chx.array(b), stride, pad)
+            assert_exact(got.get(), ref, 'conv_transpose with bias %s %s' % (dt, (xs, ws, stride, pad)))
+    for xs, ks, stride, pad in POOL_ND_GRID:
+        if len(xs) == 4:
+            continue
+        x = rng.standard_normal(xs).astype(dt)
+        x.flat[::3] = x.flat[1::3][:x.flat[::3].size]  # ties inside windows: the ArgMax rule decides
+        X = chx.array(x)
+        for cv in (False, True):
+            g = rng.standard_normal(O.max_pool_nd(x, ks, stride, pad, cv).shape).astype(dt)
+            what = '%s %s' % (dt, (xs, ks, stride, pad, cv))
+            assert_exact(chx.max_pool_grad(X, chx.array(g), ks, stride, pad, cv).get(), O.max_pool_grad_nd(x, g, ks, stride, pad, cv),
+                         'max_pool_grad ' + what)
+            gg = rng.standard_normal(xs).astype(dt)
+            assert_exact(chx.max_pool_grad_grad(X, chx.array(gg), ks, stride, pad, cv).get(), O.max_pool_grad_grad_nd(x, gg, ks, stride, pad, cv),
+                         'max_pool_grad_grad ' + what)
+        for mode in ('zero', 'ignore'):
+            g = rng.standard_normal(O.average_pool_nd(x, ks, stride, pad, mode).shape).astype(dt)
+            got = chx.average_pool_grad(X, chx.array(g), ks, stride, pad, mode).get()
+            ref = O.average_pool_grad_nd(x, g, ks, stride, pad, mode)
+            assert np.array_equal(got, ref, equal_nan=True), 'average_pool_grad %s %s' % (dt, (xs, ks, stride, pad, mode))

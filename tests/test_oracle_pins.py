@@ -866,6 +866,92 @@ def test_conv_and_pooling_over_n_axes():
             assert got.shape == want.shape and np.allclose(got, want, rtol=1e-12, atol=1e-12, equal_nan=True), (xs, ks, stride, pad, mode)
 
 
+def test_gradients_over_n_axes():
+    """The backward restatements for any number of spatial axes: equal to the 2-D ones (pinned above) bit for bit on 2-D input; on
+    the reference's 0-, 1-, 3- and 4-D grids the convolution gradients are the adjoints of the forward restatement in float64
+    (<conv(x, w), gy> = <w, grad_weight> = <x, conv_transpose(gy, w)>: a transposed operand or a wrong stride / pad axis breaks the
+    identity), average-pool gradients the adjoint of average pooling, and the max-pool gradients the definition on tie-free data
+    (gx collects the gradient of every window whose largest element it is; the double backward reads ggx there)."""
+    rng = np.random.default_rng(67)
+    tup = lambda v, n: (v,) * n if isinstance(v, int) else tuple(v)
+    for dt in ('float32', 'float16', 'float64'):
+        x = rng.standard_normal((2, 3, 7, 6)).astype(dt)
+        w = rng.standard_normal((4, 3, 3, 2)).astype(dt)
+        wt = rng.standard_normal((3, 4, 3, 2)).astype(dt)
+        b = rng.standard_normal(4).astype(dt)
+        gy = rng.standard_normal(O.conv(x, w, None, (2, 1), (1, 0)).shape).astype(dt)
+        assert np.array_equal(O.conv_grad_weight_nd(w.shape, x, gy, (2, 1), (1, 0)), O.conv_grad_weight(w.shape, x, gy, (2, 1), (1, 0)))
+        assert np.array_equal(O.conv_transpose_nd(x, wt, b, (2, 1), (1, 0)), O.conv_transpose(x, wt, b, (2, 1), (1, 0)))
+        for cv in (False, True):
+            g = rng.standard_normal(O.max_pool(x, (3, 2), (2, 1), (1, 0), cv).shape).astype(dt)
+            assert np.array_equal(O.max_pool_grad_nd(x, g, (3, 2), (2, 1), (1, 0), cv), O.max_pool_grad(x, g, (3, 2), (2, 1), (1, 0), cv))
+            gg = rng.standard_normal(x.shape).astype(dt)
+            assert np.array_equal(O.max_pool_grad_grad_nd(x, gg, (3, 2), (2, 1), (1, 0), cv), O.max_pool_grad_grad(x, gg, (3, 2), (2, 1), (1, 0), cv))
+        for mode in ('zero', 'ignore'):
+            g = rng.standard_normal(O.average_pool(x, (3, 2), (2, 1), (1, 0), mode).shape).astype(dt)
+            assert np.array_equal(O.average_pool_grad_nd(x, g, (3, 2), (2, 1), (1, 0), mode), O.average_pool_grad(x, g, (3, 2), (2, 1), (1, 0), mode),
+                                  equal_nan=True)
+    for xs, ws, stride, pad in CONV_ND_GRID:
+        n = len(xs) - 2
+        x, w = rng.standard_normal(xs), rng.standard_normal(ws)
+        for cv in (False, True):
+            y = O.conv_nd(x, w, None, stride, pad, cv)
+            gy = rng.standard_normal(y.shape)
+            lhs = float((y * gy).sum())
+            gw = O.conv_grad_weight_nd(ws, x, gy, stride, pad, cv)
+            assert gw.shape == tuple(ws) and abs(float((gw * w).sum()) - lhs) <= 1e-10 * max(1.0, abs(lhs)), (xs, ws, stride, pad, cv)
+            gx = O.conv_transpose_nd(gy, w, None, stride, pad, out_size=xs[2:])
+            assert gx.shape == tuple(xs) and abs(float((gx * x).sum()) - lhs) <= 1e-10 * max(1.0, abs(lhs)), (xs, ws, stride, pad, cv)
+        # the default output size and the bias of ConvTranspose: w read as [C_in, C_out, k...]
+        wt = rng.standard_normal((xs[1], 4) + tuple(ws[2:]))
+        st, pd = tup(stride, n), tup(pad, n)
+        dims = tuple(s_ * (d - 1) + k - 2 * p_ for d, k, s_, p_ in zip(xs[2:], ws[2:], st, pd))
+        if all(d > 0 for d in dims):
+            bias = rng.standard_normal(4)
+            out = O.conv_transpose_nd(x, wt, bias, stride, pad)
+            assert out.shape == (xs[0], 4) + dims
+            z = rng.standard_normal(out.shape)
+            back = O.conv_nd(z, wt, None, stride, pad)  # the convolution whose adjoint this is
+            lhs = float(((out - bias.reshape((1, 4) + (1,) * n)) * z).sum())
+            assert back.shape == tuple(xs) and abs(float((back * x).sum()) - lhs) <= 1e-10 * max(1.0, abs(lhs)), (xs, ws, stride, pad)
+    for xs, ks, stride, pad in POOL_ND_GRID:
+        n = len(xs) - 2
+        st, pd = tup(stride, n), tup(pad, n)
+        x = rng.permutation(int(np.prod(xs))).reshape(xs).astype(np.float64)  # no ties
+        for cv in (False, True):
+            y = O.max_pool_nd(x, ks, stride, pad, cv)
+            g = rng.standard_normal(y.shape)
+            want = np.zeros(xs)
+            ggx = rng.standard_normal(xs)
+            want_gg = np.zeros(y.shape)
+            for idx in np.ndindex(*y.shape):
+                best = None
+                for kidx in np.ndindex(*ks):
+                    i = tuple(idx[2 + d] * st[d] - pd[d] + kidx[d] for d in range(n))
+                    if all(0 <= i[d] < xs[2 + d] for d in range(n)):
+                        pos = idx[:2] + i
+                        if best is None or x[pos] > x[best]:
+                            best = pos
+                if best is None:  # a window entirely in the padding: its ArgMax is its first position, which lies outside x
+                    want_gg[idx] = -np.inf
+                    continue
+                want[best] += g[idx]
+                want_gg[idx] = ggx[best]
+            got = O.max_pool_grad_nd(x, g, ks, stride, pad, cv)
+            assert got.shape == tuple(xs) and np.allclose(got, want, rtol=1e-12, atol=1e-12), (xs, ks, stride, pad, cv)
+            assert np.array_equal(O.max_pool_grad_grad_nd(x, ggx, ks, stride, pad, cv), want_gg), (xs, ks, stride, pad, cv)
+        xr = rng.standard_normal(xs)
+        for mode in ('zero', 'ignore'):
+            y = O.average_pool_nd(xr, ks, stride, pad, mode)
+            if not np.isfinite(y).all():
+                continue  # windows that lie in the padding altogether divide by a width of zero
+            g = rng.standard_normal(y.shape)
+            gx = O.average_pool_grad_nd(xr, g, ks, stride, pad, mode)
+            assert gx.shape == tuple(xs)
+            lhs = float((y * g).sum())
+            assert abs(float((gx * xr).sum()) - lhs) <= 1e-10 * max(1.0, abs(lhs)), (xs, ks, stride, pad, mode)
+
+
 def test_batch_norm_dtypes():
     """The dtype rules of GenericBatchNormKernel (CX/routines/normalization.cc:176-193, 224-246).  float16 x with float32 parameters:
     computed in float32 -- statistics, state and running values are float32 and agree with the float64 closed form to float32
