@@ -36,7 +36,7 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E peak
 # HBM bytes per launch of the dominant kernels (fetch + write, averaged over the 53 convolutions and the linear layer of one
 # step), from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) scaled by what the same counters read for a 128 MiB copy
 # kernel (x1.999, x1.000): profiles/resnet50_conv_hbm_traffic.txt.  The algorithmic figure is 99.2 MB per launch.
-CONV_HBM_TRAFFIC_BYTES_PER_LAUNCH = 109.9e6
+CONV_HBM_TRAFFIC_BYTES_PER_LAUNCH = 111.4e6
 
 
 def main():
